@@ -1,0 +1,626 @@
+/*
+ * CPU ORACLE - TEST INFRASTRUCTURE, NOT PRODUCT CODE.  See oracle.h.
+ *
+ * Plain C restatement of the reference's quantized-decode arithmetic.
+ * Pinning status of each function (what fixes it besides this text) is listed
+ * in the comment above it; the tests under tests/ run those checks.
+ */
+#include "oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------ */
+/* scalar codecs                                                       */
+/* ------------------------------------------------------------------ */
+
+/* neural/neuralsafetensors.pas:294-329 (DecodeF16).
+ * Pinned by: 21 known answers + Inf/NaN table of tests/TestNeuralVolume.pas:3223-3294,
+ * and an exhaustive 65536-value sweep against the compiler's _Float16. */
+float orc_f16_to_f32(uint16_t bits)
+{
+  uint32_t sign = (bits >> 15) & 1u, exponent = (bits >> 10) & 0x1Fu, mant = bits & 0x3FFu, o;
+  float r;
+  if (exponent == 0) {
+    if (mant == 0) { o = sign << 31; memcpy(&r, &o, 4); return r; }
+    r = (float)mant * 5.9604644775390625e-8f; /* m * 2^-24, exact */
+    return sign ? -r : r;
+  }
+  if (exponent == 0x1F) o = (sign << 31) | (0xFFu << 23) | (mant << 13);
+  else                  o = (sign << 31) | ((exponent + 112u) << 23) | (mant << 13);
+  memcpy(&r, &o, 4);
+  return r;
+}
+
+/* neural/neuralsafetensors.pas:338-396 (EncodeF16). Normal range rounds to nearest even;
+ * the subnormal branch rounds on the single bit shifted out, as the reference does.
+ * Pinned by: decode(encode(h)) == h for every finite half; normal range vs _Float16. */
+uint16_t orc_f32_to_f16(float v)
+{
+  uint32_t bits, sign, ex, mant, half;
+  int e;
+  memcpy(&bits, &v, 4);
+  sign = (bits >> 16) & 0x8000u; ex = (bits >> 23) & 0xFFu; mant = bits & 0x7FFFFFu;
+  if (ex == 0xFF) return (uint16_t)(sign | (mant ? 0x7E00u : 0x7C00u));
+  e = (int)ex - 127 + 15;
+  if (e >= 0x1F) return (uint16_t)(sign | 0x7C00u);
+  if (e <= 0) {
+    if (e < -10) return (uint16_t)sign;
+    mant |= 0x800000u;
+    half = mant >> (14 - e);
+    if ((mant >> (13 - e)) & 1u) half++;
+    return (uint16_t)(sign | half);
+  }
+  half = ((uint32_t)e << 10) | (mant >> 13);
+  if (mant & 0x1000u) { if ((mant & 0xFFFu) || (half & 1u)) half++; }
+  return (uint16_t)(sign | half);
+}
+
+/* neural/neuralgguf.pas:448-464 (DequantizeQ4KScaleMin == ggml get_scale_min_k4).
+ * Pinned by: tiny_kquant golden vectors (through orc_dequant_q4_k) and a brute-force
+ * check against the 6-bit field definition (tests build the 12 bytes from known sc/mn). */
+void orc_q4k_scale_min(const uint8_t* p, uint8_t* sc, uint8_t* mn)
+{
+  for (int j = 0; j < 4; j++) {
+    uint8_t d = p[j], m = p[j + 4], md = p[j + 8];
+    sc[j]     = d & 0x3F;
+    sc[j + 4] = (uint8_t)((md & 0x0F) | ((d >> 2) & 0x30));
+    mn[j]     = m & 0x3F;
+    mn[j + 4] = (uint8_t)((md >> 4) | ((m >> 2) & 0x30));
+  }
+}
+
+/* ------------------------------------------------------------------ */
+/* block geometry: neural/neuralgguf.pas:100-138                       */
+/* ------------------------------------------------------------------ */
+int64_t orc_block_elems(int type)
+{
+  switch (type) {
+    case ORC_F32: case ORC_F16: case ORC_I8ROW: return 1;
+    case ORC_Q4_0: case ORC_Q8_0: return 32;
+    case ORC_Q4_K: return 256;
+  }
+  return -1;
+}
+int64_t orc_block_bytes(int type)
+{
+  switch (type) {
+    case ORC_F32: return 4; case ORC_F16: return 2; case ORC_I8ROW: return 1;
+    case ORC_Q4_0: return 18; case ORC_Q8_0: return 34; case ORC_Q4_K: return 144;
+  }
+  return -1;
+}
+int64_t orc_row_bytes(int type, int64_t cols)
+{
+  int64_t be = orc_block_elems(type);
+  if (be <= 0 || cols % be) return -1;
+  return cols / be * orc_block_bytes(type);
+}
+
+/* ------------------------------------------------------------------ */
+/* dequantizers                                                        */
+/* ------------------------------------------------------------------ */
+
+/* neural/neuralgguf.pas:1487-1503 -> TNNetVolume.DequantizeInt8 (neuralvolume.pas:12564-12582):
+ * x = d * q, one single-precision multiply (exact: 11-bit x 7-bit significands).
+ * Pinned by: closed form on hand-built blocks; tiny_llama_q8.gguf vs its fp32 twin. */
+void orc_dequant_q8_0(const uint8_t* raw, int64_t nb, float* out)
+{
+  for (int64_t b = 0; b < nb; b++, raw += 34, out += 32) {
+    uint16_t h; memcpy(&h, raw, 2);
+    float d = orc_f16_to_f32(h);
+    const int8_t* q = (const int8_t*)(raw + 2);
+    for (int i = 0; i < 32; i++) out[i] = d * (float)q[i];
+  }
+}
+
+/* neural/neuralgguf.pas:811-845 (LegacyNibble, DequantizeQ4_0): element e<16 is the low
+ * nibble of byte e, e>=16 the high nibble of byte e-16; x = d * (nibble - 8).
+ * Pinned by: the hand-built block of tests/TestNeuralPretrained.pas:6116-6143. */
+void orc_dequant_q4_0(const uint8_t* raw, int64_t nb, float* out)
+{
+  for (int64_t b = 0; b < nb; b++, raw += 18, out += 32) {
+    uint16_t h; memcpy(&h, raw, 2);
+    float d = orc_f16_to_f32(h);
+    const uint8_t* q = raw + 2;
+    for (int e = 0; e < 32; e++) {
+      int nib = (e < 16) ? (q[e] & 0x0F) : ((q[e - 16] >> 4) & 0x0F);
+      out[e] = d * (float)(nib - 8);
+    }
+  }
+}
+
+/* neural/neuralgguf.pas:472-514 (DequantizeQ4K): x = (d*sc)*q - dmin*mn, evaluated as two
+ * separate roundings-free products and one subtraction (see the exactness note in the
+ * header of tests/test_oracle_dequant.py).
+ * Pinned by: bit-exact against tests/fixtures/tiny_kquant_ref.json (1024 gguf-py values). */
+void orc_dequant_q4_k(const uint8_t* raw, int64_t nb, float* out)
+{
+  uint8_t sc[8], mn[8];
+  for (int64_t b = 0; b < nb; b++, raw += 144, out += 256) {
+    uint16_t h0, h1; memcpy(&h0, raw, 2); memcpy(&h1, raw + 2, 2);
+    float d = orc_f16_to_f32(h0), dmin = orc_f16_to_f32(h1);
+    orc_q4k_scale_min(raw + 4, sc, mn);
+    for (int c = 0; c < 4; c++) {
+      volatile float dscLo = d * (float)sc[2 * c], dmLo = dmin * (float)mn[2 * c];
+      volatile float dscHi = d * (float)sc[2 * c + 1], dmHi = dmin * (float)mn[2 * c + 1];
+      const uint8_t* chunk = raw + 16 + 32 * c;
+      float* lo = out + 64 * c; float* hi = lo + 32;
+      for (int i = 0; i < 32; i++) {
+        uint8_t pb = chunk[i];
+        /* Exact result either way (the two products are exact and share a 2^-24 grid), so
+         * fma contraction cannot change a bit; done in double to make that explicit. */
+        lo[i] = (float)((double)dscLo * (double)(pb & 0x0F) - (double)dmLo);
+        hi[i] = (float)((double)dscHi * (double)(pb >> 4) - (double)dmHi);
+      }
+    }
+  }
+}
+
+/* neural/neuralgguf.pas:1471-1523 (DecodeGGMLSpan) */
+int orc_dequant(int type, const void* raw, int64_t n, float* out)
+{
+  const uint8_t* p = (const uint8_t*)raw;
+  switch (type) {
+    case ORC_F32: memcpy(out, raw, (size_t)n * 4); return 0;
+    case ORC_F16: for (int64_t i = 0; i < n; i++) { uint16_t h; memcpy(&h, p + 2 * i, 2); out[i] = orc_f16_to_f32(h); } return 0;
+    case ORC_Q8_0: if (n % 32) return -1; orc_dequant_q8_0(p, n / 32, out); return 0;
+    case ORC_Q4_0: if (n % 32) return -1; orc_dequant_q4_0(p, n / 32, out); return 0;
+    case ORC_Q4_K: if (n % 256) return -1; orc_dequant_q4_k(p, n / 256, out); return 0;
+  }
+  return -2;
+}
+
+/* ------------------------------------------------------------------ */
+/* quantizers                                                          */
+/* ------------------------------------------------------------------ */
+
+/* neural/neuralgguf.pas:1966-1989: d = amax/127, q = round-half-away(x/d) clamped to +-127.
+ * Pinned by: |x - dequant(quant(x))| <= d/2 round trip; the reference writer's recipe. */
+void orc_quant_q8_0(const float* x, int64_t n, uint8_t* out)
+{
+  for (int64_t b = 0; b < n / 32; b++, x += 32, out += 34) {
+    float amax = 0;
+    for (int i = 0; i < 32; i++) { float v = fabsf(x[i]); if (v > amax) amax = v; }
+    float scale = amax / 127.0f, inv = scale == 0 ? 0 : 1.0f / scale;
+    uint16_t h = orc_f32_to_f16(scale); memcpy(out, &h, 2);
+    for (int i = 0; i < 32; i++) {
+      float q = x[i] * inv;
+      int e = q >= 0 ? (int)(q + 0.5f) : (int)(q - 0.5f);
+      if (e > 127) e = 127; if (e < -127) e = -127;
+      out[2 + i] = (uint8_t)(int8_t)e;
+    }
+  }
+}
+
+/* ggml quantize_row_q4_0_ref behaviour (not in the reference; this build's own definition):
+ * d = (signed element of largest magnitude) / -8, q = min(15, (int)(x/d + 8.5)). */
+void orc_quant_q4_0(const float* x, int64_t n, uint8_t* out)
+{
+  for (int64_t b = 0; b < n / 32; b++, x += 32, out += 18) {
+    float amax = 0, mx = 0;
+    for (int i = 0; i < 32; i++) { float v = fabsf(x[i]); if (v > amax) { amax = v; mx = x[i]; } }
+    float d = mx / -8.0f, id = d == 0 ? 0 : 1.0f / d;
+    uint16_t h = orc_f32_to_f16(d); memcpy(out, &h, 2);
+    for (int e = 0; e < 16; e++) {
+      int q0 = (int)(x[e] * id + 8.5f), q1 = (int)(x[e + 16] * id + 8.5f);
+      if (q0 > 15) q0 = 15; if (q1 > 15) q1 = 15; if (q0 < 0) q0 = 0; if (q1 < 0) q1 = 0;
+      out[2 + e] = (uint8_t)(q0 | (q1 << 4));
+    }
+  }
+}
+
+/* Simple affine Q4_K packer (this build's own; any valid packer is acceptable because the
+ * dequantized values are the contract).  Per 32-sub-block: lo = min(0, min x), step =
+ * (max-lo)/15; super-block d = max step / 63, dmin = max(-lo) / 63 (both stored as half);
+ * sc = round(step/d), mn = round(-lo/dmin); q = round((x + dmin*mn)/(d*sc)) in 0..15.
+ * Byte layout: neural/neuralgguf.pas:440-447 (6-bit packing) and 472-514 (nibbles). */
+void orc_quant_q4_k(const float* x, int64_t n, uint8_t* out)
+{
+  for (int64_t b = 0; b < n / 256; b++, x += 256, out += 144) {
+    float step[8], lo[8], maxstep = 0, maxneg = 0;
+    for (int j = 0; j < 8; j++) {
+      float mn_ = 0, mx_ = -INFINITY;
+      for (int i = 0; i < 32; i++) { float v = x[32 * j + i]; if (v < mn_) mn_ = v; if (v > mx_) mx_ = v; }
+      if (mx_ < mn_) mx_ = mn_;
+      lo[j] = mn_; step[j] = (mx_ - mn_) / 15.0f;
+      if (step[j] > maxstep) maxstep = step[j];
+      if (-mn_ > maxneg) maxneg = -mn_;
+    }
+    uint16_t hd = orc_f32_to_f16(maxstep / 63.0f), hm = orc_f32_to_f16(maxneg / 63.0f);
+    float d = orc_f16_to_f32(hd), dmin = orc_f16_to_f32(hm);
+    uint8_t sc[8], mn[8];
+    for (int j = 0; j < 8; j++) {
+      int s = d > 0 ? (int)lrintf(step[j] / d) : 0, m = dmin > 0 ? (int)lrintf(-lo[j] / dmin) : 0;
+      if (s > 63) s = 63; if (m > 63) m = 63; if (s < 0) s = 0; if (m < 0) m = 0;
+      sc[j] = (uint8_t)s; mn[j] = (uint8_t)m;
+    }
+    memcpy(out, &hd, 2); memcpy(out + 2, &hm, 2);
+    uint8_t* p = out + 4;
+    for (int j = 0; j < 4; j++) {
+      p[j]     = (uint8_t)((sc[j] & 63) | ((sc[j + 4] >> 4) << 6));
+      p[j + 4] = (uint8_t)((mn[j] & 63) | ((mn[j + 4] >> 4) << 6));
+      p[j + 8] = (uint8_t)((sc[j + 4] & 15) | ((mn[j + 4] & 15) << 4));
+    }
+    for (int c = 0; c < 4; c++) {
+      for (int i = 0; i < 32; i++) {
+        int q[2];
+        for (int hlf = 0; hlf < 2; hlf++) {
+          int j = 2 * c + hlf;
+          float ds = d * (float)sc[j], off = dmin * (float)mn[j];
+          int v = ds > 0 ? (int)lrintf((x[32 * j + i] + off) / ds) : 0;
+          if (v < 0) v = 0; if (v > 15) v = 15;
+          q[hlf] = v;
+        }
+        out[16 + 32 * c + i] = (uint8_t)(q[0] | (q[1] << 4));
+      }
+    }
+  }
+}
+
+/* neural/neuralvolume.pas:12501-12562 scalar twin: codes = round(v * (1/max) * 127) clamped
+ * to +-127, scale = max/127 (callers: neural/neuralvolume.pas:926-987).  Round is
+ * round-half-even (FPC Round / vcvtps2dq).  PARITY NOTE: the reference documents the tie
+ * behaviour on boundary products as not bit-stable across its own builds
+ * (neuralvolume.pas:728-735); pinned here by the round trip |x - scale*code| <= scale/2. */
+void orc_quant_int8_row(const float* x, int64_t n, int8_t* codes, float* scale)
+{
+  float mx = 0;
+  for (int64_t i = 0; i < n; i++) { float v = fabsf(x[i]); if (v > mx) mx = v; }
+  *scale = mx / 127.0f;
+  if (mx <= 0) { memset(codes, 0, (size_t)n); return; }
+  float recip = 1.0f / mx;
+  for (int64_t i = 0; i < n; i++) {
+    float s = x[i] * recip * 127.0f;
+    if (s > 127) s = 127; else if (s < -127) s = -127;
+    codes[i] = (int8_t)lrintf(s);
+  }
+}
+
+/* ------------------------------------------------------------------ */
+/* row permutations                                                    */
+/* ------------------------------------------------------------------ */
+
+/* neural/neuralgguf.pas:428-438 */
+int64_t orc_gguf_deinterleaved_src_row(int64_t hf_row, int head_dim)
+{
+  int64_t half = head_dim >> 1, r = hf_row % head_dim;
+  if (r < half) return (hf_row - r) + 2 * r;
+  return (hf_row - r) + 2 * (r - half) + 1;
+}
+
+/* neural/neuralpretrained.pas:14792-14812 (full-rotary case): HF row -> neuron index so that
+ * interleaved-pair RoPE equals HF rotate_half. */
+int64_t orc_map_target_neuron(int64_t row, int head_dim)
+{
+  int64_t half = head_dim >> 1, head = row / head_dim, r = row % head_dim;
+  int64_t t = (r < half) ? 2 * r : 2 * (r - half) + 1;
+  return head * head_dim + t;
+}
+
+/* ------------------------------------------------------------------ */
+/* linear layer                                                        */
+/* ------------------------------------------------------------------ */
+
+/* neural.cl:114-146 activation tail (two-branch sigmoid, clamped tanh). */
+static float apply_act(float v, int act)
+{
+  if (act == 1) return v < 0 ? 0 : v;
+  if (act == 2) { if (v > 0) return 1.0f / (1.0f + expf(-v)); float s = expf(v); return s / (1.0f + s); }
+  if (act == 3) { float xc = v > 10 ? 10 : (v < -10 ? -10 : v); float e = expf(-2.0f * xc); return (1.0f - e) / (1.0f + e); }
+  return v;
+}
+
+/* Definition of the block-fused GEMV: dequantize the row exactly as the reference's loader
+ * would (neuralgguf.pas:1471-1523), then Out[b*NumAs+a] = dot(W[a], X[b]) + bias[a]
+ * (neuralvolume.pas:12127-12423 result layout; bias before activation, neural.cl:111-146).
+ * ORC_I8ROW: scale applied once to the raw code sum (neuralvolume.pas:12693-12745).
+ * Pinned by: definition (dequant is pinned above); fp32 vs double accumulation agree. */
+int orc_gemv(int type, const void* raw, const float* scales, int64_t rows, int64_t cols,
+             const float* x, int n_b, const float* bias, int act, int acc64, float* y)
+{
+  int64_t rb = orc_row_bytes(type, cols);
+  if (rb < 0) return -1;
+  int err = 0;
+#pragma omp parallel
+  {
+    float* w = (float*)malloc((size_t)cols * sizeof(float));
+#pragma omp for schedule(static)
+    for (int64_t a = 0; a < rows; a++) {
+      const uint8_t* rp = (const uint8_t*)raw + a * rb;
+      if (type == ORC_I8ROW) { const int8_t* c = (const int8_t*)rp; for (int64_t i = 0; i < cols; i++) w[i] = (float)c[i]; }
+      else if (orc_dequant(type, rp, cols, w)) { err = -2; continue; }
+      for (int b = 0; b < n_b; b++) {
+        const float* xb = x + (int64_t)b * cols;
+        float r;
+        if (acc64) { double s = 0; for (int64_t i = 0; i < cols; i++) s += (double)w[i] * (double)xb[i]; if (type == ORC_I8ROW) s *= (double)scales[a]; r = (float)s; }
+        else       { float s = 0;  for (int64_t i = 0; i < cols; i++) s += w[i] * xb[i]; if (type == ORC_I8ROW) s *= scales[a]; r = s; }
+        if (bias) r += bias[a];
+        y[(int64_t)b * rows + a] = apply_act(r, act);
+      }
+    }
+    free(w);
+  }
+  return err;
+}
+
+/* ------------------------------------------------------------------ */
+/* elementwise layer math                                              */
+/* ------------------------------------------------------------------ */
+
+/* neural.cl:1047-1085 with FUseMean == 0: inv = 1/sqrt(mean(x^2)+eps); y = g*(x*inv). */
+void orc_rmsnorm(const float* x, const float* gain, int n, float eps, float* y)
+{
+  float ss = 0;
+  for (int c = 0; c < n; c++) ss = fmaf(x[c], x[c], ss);
+  float inv = 1.0f / sqrtf(ss / (float)n + eps);
+  for (int c = 0; c < n; c++) y[c] = gain[c] * (x[c] * inv);
+}
+
+/* Host-side frequency table the device kernel receives (neural.cl:1510-1515): theta_k =
+ * base^(-2k/head_dim), computed in double and rounded once. */
+void orc_rope_thetas(float base, int head_dim, float* th)
+{
+  for (int k = 0; k < head_dim / 2; k++) th[k] = (float)pow((double)base, -2.0 * k / head_dim);
+}
+
+/* neural.cl:1517-1542: pairs (2k,2k+1) per head, angle = (float)pos * theta_k (fp32 product). */
+void orc_rope_interleaved(float* x, int n_heads, int head_dim, int pos, const float* th)
+{
+  for (int h = 0; h < n_heads; h++)
+    for (int k = 0; k < head_dim / 2; k++) {
+      float angle = (float)pos * th[k];
+      float s = (float)sin((double)angle), c = (float)cos((double)angle);
+      float* p = x + h * head_dim + 2 * k;
+      float x0 = p[0], x1 = p[1];
+      p[0] = c * x0 - s * x1;
+      p[1] = s * x0 + c * x1;
+    }
+}
+
+/* neural.cl:1213-1263 flag 1: y = A * (B * sigmoid(B)), A = first half (up), B = second (gate). */
+void orc_swiglu(const float* ug, int half, float* y)
+{
+  for (int d = 0; d < half; d++) {
+    float a = ug[d], b = ug[half + d], sig;
+    if (b > 0) sig = 1.0f / (1.0f + expf(-b)); else { float s = expf(b); sig = s / (1.0f + s); }
+    y[d] = a * (b * sig);
+  }
+}
+
+/* neural.cl:1594-1647 with FApplyMinScale == 0 (TNNetPointwiseSoftMax). */
+void orc_softmax(const float* x, int n, float* y)
+{
+  float mx = x[0];
+  for (int c = 1; c < n; c++) if (x[c] > mx) mx = x[c];
+  float tot = 0;
+  for (int c = 0; c < n; c++) {
+    float a = x[c] - mx; if (a > 4000) a = 4000; else if (a < -4000) a = -4000;
+    y[c] = expf(a); tot += y[c];
+  }
+  if (tot > 0) { float inv = 1.0f / tot; for (int c = 0; c < n; c++) y[c] *= inv; }
+}
+
+/* TNNetTopKGate (source unavailable; known answer tests/TestNeuralNumerical.pas:74997-75042):
+ * keep the k largest, zero the rest, optionally renormalise survivors to sum 1.  Ties: the
+ * lower index is kept first (PARITY NOTE: tie rule not visible in the reference checkout).
+ * idx_out lists survivors in descending value order. */
+void orc_topk_gate(const float* p, int n, int k, int renorm, float* g, int* idx)
+{
+  char* used = (char*)calloc((size_t)n, 1);
+  float sum = 0;
+  for (int c = 0; c < n; c++) g[c] = 0;
+  for (int j = 0; j < k; j++) {
+    int best = -1;
+    for (int c = 0; c < n; c++) if (!used[c] && (best < 0 || p[c] > p[best])) best = c;
+    used[best] = 1; idx[j] = best; sum += p[best];
+  }
+  for (int j = 0; j < k; j++) g[idx[j]] = renorm ? (sum > 0 ? p[idx[j]] / sum : 0) : p[idx[j]];
+  free(used);
+}
+
+/* neuralchatengine.pas:683-697 (ArgMaxRow): strict > from index 0, lowest index wins ties. */
+int orc_argmax(const float* x, int n)
+{
+  int b = 0;
+  for (int i = 1; i < n; i++) if (x[i] > x[b]) b = i;
+  return b;
+}
+
+/* ------------------------------------------------------------------ */
+/* attention                                                           */
+/* ------------------------------------------------------------------ */
+
+static float round_half(float v) { return orc_f16_to_f32(orc_f32_to_f16(v)); }
+
+/* neural.cl:2354-2379 (append) + 2406-2499 (decode): scores q.K_j/sqrt(dk) (+softcap), max,
+ * exp-shift, normaliser, out = (sum_j e_j V_j) * (1/sum).
+ * Pinned by: tiny_*_logits.json through orc_model_step; brute-force softmax identity. */
+void orc_attn_decode(const float* qkv, int hq, int hkv, int dk, float* kc, float* vc, int max_ctx,
+                     int cache_len, int window, float softcap, int kv_f16, float* out)
+{
+  const int qw = hq * dk, kw = hkv * dk, group = hq / hkv;
+  for (int g = 0; g < hkv; g++)
+    for (int d = 0; d < dk; d++) {
+      float k = qkv[qw + g * dk + d], v = qkv[qw + kw + g * dk + d];
+      if (kv_f16) { k = round_half(k); v = round_half(v); }
+      kc[((int64_t)g * max_ctx + cache_len) * dk + d] = k;
+      vc[((int64_t)g * max_ctx + cache_len) * dk + d] = v;
+    }
+  const int len = cache_len + 1;
+  const int j0 = (window > 0 && len > window) ? len - window : 0;
+  const float inv_sqrt = 1.0f / sqrtf((float)dk);
+  float* sc = (float*)malloc((size_t)len * sizeof(float));
+  for (int h = 0; h < hq; h++) {
+    const int g = h / group;
+    const float* q = qkv + h * dk;
+    float m = -1e30f;
+    for (int j = j0; j < len; j++) {
+      const float* kr = kc + ((int64_t)g * max_ctx + j) * dk;
+      float acc = 0;
+      for (int d = 0; d < dk; d++) acc = fmaf(q[d], kr[d], acc);
+      float s = acc * inv_sqrt;
+      if (softcap > 0) s = softcap * tanhf(s / softcap);
+      sc[j] = s; if (s > m) m = s;
+    }
+    float sum = 0;
+    for (int j = j0; j < len; j++) { sc[j] = expf(sc[j] - m); sum += sc[j]; }
+    const float inv = sum > 0 ? 1.0f / sum : 0;
+    for (int d = 0; d < dk; d++) {
+      float acc = 0;
+      for (int j = j0; j < len; j++) acc = fmaf(sc[j], vc[((int64_t)g * max_ctx + j) * dk + d], acc);
+      out[h * dk + d] = acc * inv;
+    }
+  }
+  free(sc);
+}
+
+/* ------------------------------------------------------------------ */
+/* whole decoder                                                       */
+/* ------------------------------------------------------------------ */
+
+typedef struct { int type; int64_t rows, cols; const void* raw; const float* scales; const float* bias; } orc_tensor;
+
+typedef struct {
+  orc_tensor w[9];
+  const float* v[5];
+  float *kc, *vc;
+} orc_layer;
+
+struct orc_model {
+  orc_config cfg;
+  orc_tensor embed, head;
+  const float* final_norm;
+  orc_layer* layers;
+  float* theta;
+  int len;
+  float *x, *h, *qkv, *att, *gu, *mid, *tmp, *probs, *gates, *logits;
+  int* sel;
+};
+
+orc_model* orc_model_new(const orc_config* cfg)
+{
+  orc_model* m = (orc_model*)calloc(1, sizeof(*m));
+  m->cfg = *cfg;
+  const int L = cfg->n_layers, d = cfg->d_model, qw = cfg->n_q_heads * cfg->head_dim, kw = cfg->n_kv_heads * cfg->head_dim;
+  m->layers = (orc_layer*)calloc((size_t)L, sizeof(orc_layer));
+  for (int l = 0; l < L; l++) {
+    m->layers[l].kc = (float*)calloc((size_t)kw * cfg->max_ctx, sizeof(float));
+    m->layers[l].vc = (float*)calloc((size_t)kw * cfg->max_ctx, sizeof(float));
+  }
+  m->theta = (float*)malloc(sizeof(float) * (size_t)(cfg->head_dim / 2));
+  orc_rope_thetas(cfg->rope_theta, cfg->head_dim, m->theta);
+  int wide = d; if (qw > wide) wide = qw;
+  m->x = (float*)calloc((size_t)d, 4); m->h = (float*)calloc((size_t)wide, 4);
+  m->qkv = (float*)calloc((size_t)(qw + 2 * kw), 4); m->att = (float*)calloc((size_t)qw, 4);
+  m->gu = (float*)calloc((size_t)2 * cfg->ffn, 4); m->mid = (float*)calloc((size_t)cfg->ffn, 4);
+  m->tmp = (float*)calloc((size_t)wide, 4);
+  int ne = cfg->n_experts > 0 ? cfg->n_experts : 1;
+  m->probs = (float*)calloc((size_t)ne, 4); m->gates = (float*)calloc((size_t)ne, 4); m->sel = (int*)calloc((size_t)ne, sizeof(int));
+  m->logits = (float*)calloc((size_t)cfg->vocab, 4);
+  return m;
+}
+
+void orc_model_free(orc_model* m)
+{
+  if (!m) return;
+  for (int l = 0; l < m->cfg.n_layers; l++) { free(m->layers[l].kc); free(m->layers[l].vc); }
+  free(m->layers); free(m->theta); free(m->x); free(m->h); free(m->qkv); free(m->att); free(m->gu); free(m->mid);
+  free(m->tmp); free(m->probs); free(m->gates); free(m->sel); free(m->logits); free(m);
+}
+
+int orc_model_set_tensor(orc_model* m, int layer, int slot, int type, int64_t rows, int64_t cols,
+                         const void* raw, const float* scales, const float* bias)
+{
+  orc_tensor t = { type, rows, cols, raw, scales, bias };
+  if (slot == ORC_W_EMBED) { m->embed = t; return 0; }
+  if (slot == ORC_W_HEAD) { m->head = t; return 0; }
+  if (layer < 0 || layer >= m->cfg.n_layers || slot < 2 || slot > 8) return -1;
+  m->layers[layer].w[slot] = t;
+  return 0;
+}
+
+int orc_model_set_vec(orc_model* m, int layer, int slot, const float* v, int n)
+{
+  (void)n;
+  if (slot == ORC_V_FINAL_NORM) { m->final_norm = v; return 0; }
+  if (layer < 0 || layer >= m->cfg.n_layers || slot < 0 || slot > 4) return -1;
+  m->layers[layer].v[slot] = v;
+  return 0;
+}
+
+void orc_model_reset(orc_model* m) { m->len = 0; }
+void orc_model_truncate(orc_model* m, int n) { if (n < m->len) m->len = n < 0 ? 0 : n; }
+int  orc_model_len(const orc_model* m) { return m->len; }
+
+static void lin(const orc_model* m, const orc_tensor* t, int64_t row0, int64_t rows, const float* x, float* y)
+{
+  int64_t rb = orc_row_bytes(t->type, t->cols);
+  orc_gemv(t->type, (const uint8_t*)t->raw + row0 * rb, t->scales ? t->scales + row0 : 0, rows, t->cols, x, 1,
+           t->bias ? t->bias + row0 : 0, 0, m->cfg.acc64, y);
+}
+
+/* One decode step in the reference's graph order (neuralpretrained.pas:16384-16882 builds it;
+ * neuraldecode.pas:5696-5712 StepForward runs it): embedding row -> per block { RMSNorm ->
+ * q,k,v (+bias) -> [full-width q/k RMSNorm] -> interleaved RoPE -> cached GQA -> o -> +res ->
+ * RMSNorm -> gate|up -> SwiGLU -> down -> +res } -> final RMSNorm -> head -> argmax.
+ * MoE FFN (neuralpretrained.pas:15331-15388): router -> softmax over all experts -> top-k
+ * (renorm iff norm_topk) -> sum_e g_e * down_e(SwiGLU(gateup_e(h))).
+ * Pinned by: tests/fixtures/tiny_{llama,smollm2,qwen2,mistral,olmoe}_logits.json (< 1e-4). */
+int orc_model_step(orc_model* m, int token, int pos, float* logits)
+{
+  const orc_config* c = &m->cfg;
+  const int d = c->d_model, hd = c->head_dim, qw = c->n_q_heads * hd, kw = c->n_kv_heads * hd, I = c->ffn;
+  if (pos != m->len || pos >= c->max_ctx || token < 0 || token >= c->vocab) return -1;
+  {
+    int64_t rb = orc_row_bytes(m->embed.type, m->embed.cols);
+    if (m->embed.type == ORC_I8ROW) {
+      const int8_t* cd = (const int8_t*)m->embed.raw + (int64_t)token * rb;
+      for (int i = 0; i < d; i++) m->x[i] = (float)cd[i] * m->embed.scales[token]; /* neural.cl:1447-1470 */
+    } else orc_dequant(m->embed.type, (const uint8_t*)m->embed.raw + (int64_t)token * rb, d, m->x);
+  }
+  for (int l = 0; l < c->n_layers; l++) {
+    orc_layer* ly = &m->layers[l];
+    orc_rmsnorm(m->x, ly->v[ORC_V_ATTN_NORM], d, c->eps, m->h);
+    lin(m, &ly->w[ORC_W_Q], 0, qw, m->h, m->qkv);
+    lin(m, &ly->w[ORC_W_K], 0, kw, m->h, m->qkv + qw);
+    lin(m, &ly->w[ORC_W_V], 0, kw, m->h, m->qkv + qw + kw);
+    if (c->qk_norm_full) {
+      orc_rmsnorm(m->qkv, ly->v[ORC_V_Q_NORM], qw, c->eps, m->tmp); memcpy(m->qkv, m->tmp, (size_t)qw * 4);
+      orc_rmsnorm(m->qkv + qw, ly->v[ORC_V_K_NORM], kw, c->eps, m->tmp); memcpy(m->qkv + qw, m->tmp, (size_t)kw * 4);
+    }
+    orc_rope_interleaved(m->qkv, c->n_q_heads, hd, pos, m->theta);
+    orc_rope_interleaved(m->qkv + qw, c->n_kv_heads, hd, pos, m->theta);
+    orc_attn_decode(m->qkv, c->n_q_heads, c->n_kv_heads, hd, ly->kc, ly->vc, c->max_ctx, pos, c->window, 0.0f, c->kv_f16, m->att);
+    lin(m, &ly->w[ORC_W_O], 0, d, m->att, m->tmp);
+    for (int i = 0; i < d; i++) m->x[i] += m->tmp[i];
+    orc_rmsnorm(m->x, ly->v[ORC_V_MLP_NORM], d, c->eps, m->h);
+    if (c->n_experts > 0) {
+      lin(m, &ly->w[ORC_W_ROUTER], 0, c->n_experts, m->h, m->tmp);
+      orc_softmax(m->tmp, c->n_experts, m->probs);
+      orc_topk_gate(m->probs, c->n_experts, c->top_k, c->norm_topk, m->gates, m->sel);
+      float* acc = (float*)calloc((size_t)d, 4);
+      for (int j = 0; j < c->top_k; j++) {
+        int e = m->sel[j];
+        lin(m, &ly->w[ORC_W_GATEUP], (int64_t)e * 2 * I, 2 * I, m->h, m->gu);
+        orc_swiglu(m->gu, I, m->mid);
+        lin(m, &ly->w[ORC_W_DOWN], (int64_t)e * d, d, m->mid, m->tmp);
+        for (int i = 0; i < d; i++) acc[i] = fmaf(m->gates[e], m->tmp[i], acc[i]); /* neural.cl:2738-2748 */
+      }
+      for (int i = 0; i < d; i++) m->x[i] += acc[i];
+      free(acc);
+    } else {
+      lin(m, &ly->w[ORC_W_GATEUP], 0, 2 * I, m->h, m->gu);
+      orc_swiglu(m->gu, I, m->mid);
+      lin(m, &ly->w[ORC_W_DOWN], 0, d, m->mid, m->tmp);
+      for (int i = 0; i < d; i++) m->x[i] += m->tmp[i];
+    }
+  }
+  orc_rmsnorm(m->x, m->final_norm, d, c->eps, m->h);
+  const orc_tensor* hw = m->head.raw ? &m->head : &m->embed; /* tied head: neuralpretrained.pas:15555- */
+  lin(m, hw, 0, c->vocab, m->h, m->logits);
+  if (logits) memcpy(logits, m->logits, (size_t)c->vocab * 4);
+  m->len = pos + 1;
+  return orc_argmax(m->logits, c->vocab);
+}
