@@ -1,0 +1,214 @@
+/*
+ * caihip - C ABI of the MI355X (gfx950) quantized LLM decode path for CAI Neural API.
+ *
+ * Plain C, cdecl, opaque handles, int error codes, no exceptions across the boundary.
+ * The library owns all device memory; every create has a destroy; host pointers are never
+ * retained after a call returns.  All calls enqueue on one in-order HIP stream owned by the
+ * library (the analogue of the reference's single shared in-order OpenCL queue,
+ * examples/ChatTerminal/README.md:174-180); calls are not re-entrant.
+ *
+ * Citations are file:line in the reference checkout (joaopauloschuler/neural-api).
+ */
+#ifndef CAIHIP_H
+#define CAIHIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- error codes ---- */
+#define CAI_OK               0
+#define CAI_ERR_INVALID     (-1)  /* bad argument / shape */
+#define CAI_ERR_HIP         (-2)  /* HIP runtime error (text in cai_last_error) */
+#define CAI_ERR_NOMEM       (-3)
+#define CAI_ERR_UNSUPPORTED (-4)
+#define CAI_ERR_STATE       (-5)  /* not initialised, slot not set, cache full ... */
+
+/* ---- weight storage types: ggml ids (neural/neuralgguf.pas:86-98) ---- */
+#define CAI_F32    0
+#define CAI_F16    1
+#define CAI_Q4_0   2
+#define CAI_Q8_0   8
+#define CAI_Q4_K   12
+#define CAI_I8ROW  100  /* per-row symmetric int8 + fp32 row scale (neural/neuralvolume.pas:926-987) */
+
+/* ---- activation opcodes fused into the linear layer (neural/neural.cl:114-146) ---- */
+#define CAI_ACT_NONE    0
+#define CAI_ACT_RELU    1
+#define CAI_ACT_SIGMOID 2
+#define CAI_ACT_TANH    3
+
+/* ---- pointer-space flags for compute calls ---- */
+#define CAI_X_DEVICE 1  /* input pointer is device memory (a producer's resident buffer; cf. pExternalVBs, neural/neuralopencl.pas:946) */
+#define CAI_Y_DEVICE 2  /* output pointer is device memory (no read-back; cf. ResultBuffer, neural/neuralopencl.pas:383-388) */
+
+/* ---- KV cache element types ---- */
+#define CAI_KV_F32 0
+#define CAI_KV_F16 1
+
+typedef struct cai_qw_s*      cai_qw_t;       /* resident quantized weight matrix */
+typedef struct cai_kv_s*      cai_kv_t;       /* KV cache of one sequence, all layers */
+typedef struct cai_kv_snap_s* cai_kv_snap_t;  /* deep copy of a KV cache's live rows */
+typedef struct cai_decoder_s* cai_decoder_t;  /* step-resident decoder */
+
+/* =====================================================================================
+ * Library lifetime.  Replaces TNNet.EnableOpenCL(PlatformId, DeviceId, shared)
+ * (neural/neuralchatengine.pas:1156-1157): selects the GPU and creates the stream.
+ * ===================================================================================== */
+int cai_init(int device_ordinal);
+int cai_shutdown(void);
+/* Copies the text of the last error of the calling process into buf (NUL terminated). */
+int cai_last_error(char* buf, int buf_len);
+int cai_device_name(char* buf, int buf_len);
+/* Blocks until all enqueued work is finished (FinishAndLoadResult's clFinish, neural/neuralopencl.pas:1058-1104). */
+int cai_sync(void);
+/* hipStream_t of the library, for callers that record their own events. */
+int cai_get_stream(void** stream_out);
+/* HIP-event stopwatch on the library stream: start, enqueue work, stop -> elapsed ms. */
+int cai_timer_start(void);
+int cai_timer_stop(float* ms_out);
+
+/* Device buffers for resident activations. */
+int cai_dev_alloc(int64_t bytes, void** ptr_out);
+int cai_dev_free(void* ptr);
+int cai_dev_upload(void* dst_dev, const void* src_host, int64_t bytes);
+int cai_dev_download(void* dst_host, const void* src_dev, int64_t bytes);
+
+/* =====================================================================================
+ * Resident quantized weights.
+ * Replaces TDotProductSharedKernel.PrepareForComputeInt8(pCodes, pScales, NumAs, pSize, VBs)
+ * (neural/neuralopencl.pas:844-891): a blocking one-time upload; staging may be freed on return.
+ * `blocks` holds `rows` rows of cols/block_elems GGUF blocks, row-major [out][in], exactly the
+ * bytes of a GGUF tensor (neural/neuralgguf.pas:100-138, 226-236).  It may be a host or a device
+ * pointer.  `bias` (rows floats, host) may be NULL.
+ * ===================================================================================== */
+int cai_qw_create(int qtype, int64_t rows, int64_t cols, const void* blocks, const float* bias, cai_qw_t* out);
+/* Per-row int8 form: codes row-major [rows][cols], one fp32 scale per row
+ * (TNNetVolume.QuantizeInt8 output, neural/neuralvolume.pas:12501-12562). */
+int cai_qw_create_int8row(int64_t rows, int64_t cols, const int8_t* codes, const float* scales,
+                          const float* bias, cai_qw_t* out);
+int cai_qw_destroy(cai_qw_t w);                       /* UnprepareForCompute, neural/neuralopencl.pas:527-562 */
+int cai_qw_info(cai_qw_t w, int* qtype, int64_t* rows, int64_t* cols, int64_t* device_bytes);
+/* Dequantizes rows [row0, row0+n_rows) on the device into fp32 (bit-exact to DecodeGGMLSpan,
+ * neural/neuralgguf.pas:1471-1523).  flags: CAI_Y_DEVICE. */
+int cai_qw_dequant_rows(cai_qw_t w, int64_t row0, int64_t n_rows, float* out, int flags);
+
+/* =====================================================================================
+ * Linear layer forward (TNNetPointwiseConvLinear / TNNetFullConnectLinear).
+ * Replaces ComputeInt8 + FinishAndLoadResult (neural/neuralopencl.pas:946-1104):
+ *   y[b*rows + a] = act( dot(W[a], x[b*cols ..]) + bias[a] ),  b < n_b  (1 <= n_b <= 8)
+ * Weights are dequantized in registers; accumulation is fp32.
+ * ===================================================================================== */
+int cai_qgemv(cai_qw_t w, const float* x, int n_b, float* y, int act, int flags);
+/* Multi-token form on the matrix cores (prefill): x is [n_tokens][cols], y is [n_tokens][rows].
+ * No counterpart in the reference, whose prefill is token-at-a-time
+ * (neural/neuralchatengine.pas:1466-1470); results equal n_tokens GEMVs within bf16-input tolerance. */
+int cai_qgemm(cai_qw_t w, const float* x, int n_tokens, float* y, int flags);
+
+/* =====================================================================================
+ * Elementwise layer math on fp32 rows.  flags: CAI_X_DEVICE | CAI_Y_DEVICE.
+ * ===================================================================================== */
+/* TNNetTokenRMSNorm (neural/neural.cl:1047-1085, FUseMean = 0); x, y: [n_tokens][n]. */
+int cai_rmsnorm(const float* x, const float* gain_host, int n, int n_tokens, float eps, float* y, int flags);
+/* TNNetRotaryEmbedding, interleaved pairs, head-tiled theta (neural/neural.cl:1517-1542);
+ * in place over x = [n_heads][head_dim] at absolute position pos. */
+int cai_rope(float* x, int n_heads, int head_dim, int pos, float theta_base, int flags);
+/* TNNetSwiGLU (neural/neural.cl:1213-1263 flag 1): y[d] = x[d] * silu(x[half+d]). */
+int cai_swiglu(const float* x, int half, int n_tokens, float* y, int flags);
+/* ArgMaxRow (neural/neuralchatengine.pas:683-697): lowest index wins ties. */
+int cai_argmax(const float* x, int n, int32_t* index_out, int flags);
+/* TNNetPointwiseSoftMax + TNNetTopKGate (neural/neuralpretrained.pas:15347-15365):
+ * softmax over n experts, keep top-k, renormalise iff renorm.  Outputs are host arrays of k. */
+int cai_router_topk(const float* logits, int n, int k, int renorm, int32_t* expert_out, float* gate_out, int flags);
+
+/* =====================================================================================
+ * KV cache + cached GQA decode attention (TNNetFusedSDPA).
+ * Replaces BeginIncrementalDecode(MaxCtx, Int8KV) / ResetCache / TruncateCache / CacheLength /
+ * Capture/RestoreCacheState (tests/TestNeuralFusedSDPA.pas:228-454) and the kernels
+ * cai_sdpa_append_kv + cai_sdpa_decode (neural/neural.cl:2354-2499).
+ * Cache layout is head-major: row (layer, kv_head g, position p) at ((layer*kv_heads+g)*max_ctx+p)*head_dim.
+ * ===================================================================================== */
+int cai_kv_create(int n_layers, int kv_heads, int head_dim, int max_ctx, int kv_dtype, cai_kv_t* out);
+int cai_kv_destroy(cai_kv_t kv);
+int cai_kv_reset(cai_kv_t kv);
+int cai_kv_truncate(cai_kv_t kv, int n);          /* keeps the first n rows of every layer */
+int cai_kv_len(cai_kv_t kv, int layer, int* len_out);
+int cai_kv_snapshot(cai_kv_t kv, cai_kv_snap_t* out);
+int cai_kv_restore(cai_kv_t kv, cai_kv_snap_t snap);
+int cai_kv_snap_destroy(cai_kv_snap_t snap);
+/* One token of one layer: qkv = [Q (q_heads*hd) | K (kv_heads*hd) | V (kv_heads*hd)]; appends K,V at
+ * slot CacheLength(layer), then out[h] = softmax(q_h.K/sqrt(hd)) V over the live range
+ * (window > 0: last `window` rows; softcap > 0: Gemma-2 style cap).  out: [q_heads*hd]. */
+int cai_attn_decode(cai_kv_t kv, int layer, const float* qkv, int q_heads, int window, float softcap,
+                    float* out, int flags);
+
+/* =====================================================================================
+ * Step-resident decoder (TNNetStreamingDecoder over a Llama / Qwen2 / OLMoE graph).
+ * Replaces Session.StepForward(InV, AbsPos) -> FNet.Compute (neural/neuraldecode.pas:5696-5712) for
+ * the graph BuildLlamaFromTensorReaderWithConfig wires (neural/neuralpretrained.pas:16384-16882):
+ * activations never leave the GPU inside a step (neural/tasklist.md:768-790 names the per-layer
+ * host round trip as the bottleneck of the OpenCL path).
+ * ===================================================================================== */
+typedef struct cai_decoder_config {
+  int32_t n_layers, d_model, n_q_heads, n_kv_heads, head_dim, ffn, vocab, max_ctx;
+  float   eps, rope_theta;
+  int32_t window;        /* sliding window, 0 = none */
+  int32_t qk_norm_full;  /* OLMoE: RMSNorm over the full q and k widths before RoPE */
+  int32_t n_experts;     /* 0 = dense SwiGLU FFN; else `ffn` is the per-expert width */
+  int32_t top_k;
+  int32_t norm_topk;
+  int32_t kv_dtype;      /* CAI_KV_F32 / CAI_KV_F16 */
+  int32_t max_batch;     /* independent sequences, each with its own KV cache (1..8) */
+} cai_decoder_config;
+
+/* weight slots (layer = -1 for EMBED / HEAD; HEAD unset = tied to EMBED) */
+#define CAI_W_EMBED  0
+#define CAI_W_HEAD   1
+#define CAI_W_Q      2
+#define CAI_W_K      3
+#define CAI_W_V      4
+#define CAI_W_O      5
+#define CAI_W_GATEUP 6  /* rows 0..I-1 up, I..2I-1 gate (neural/neuralpretrained.pas:240-243); MoE bank: expert e at rows e*2I */
+#define CAI_W_DOWN   7  /* MoE bank: expert e at rows e*d_model */
+#define CAI_W_ROUTER 8
+/* vector slots */
+#define CAI_V_ATTN_NORM  0
+#define CAI_V_MLP_NORM   1
+#define CAI_V_FINAL_NORM 2  /* layer = -1 */
+#define CAI_V_Q_NORM     3
+#define CAI_V_K_NORM     4
+
+int cai_decoder_create(const cai_decoder_config* cfg, cai_decoder_t* out);
+int cai_decoder_destroy(cai_decoder_t d);
+/* The decoder borrows `w`; the caller destroys it after the decoder. q/k rows must be in the
+ * interleaved-rotary order of MapTargetNeuron (neural/neuralpretrained.pas:14792-14812), which is the
+ * stored order of llama.cpp GGUF files. */
+int cai_decoder_set_weight(cai_decoder_t d, int layer, int slot, cai_qw_t w);
+int cai_decoder_set_vector(cai_decoder_t d, int layer, int slot, const float* v_host, int n);
+/* One token for each of sequences 0..n_b-1: tokens[b] at absolute position pos[b] (must equal that
+ * sequence's cache length).  logits (host, [n_b][vocab]) and argmax (host, [n_b]) may be NULL. */
+int cai_decoder_step(cai_decoder_t d, const int32_t* tokens, const int32_t* pos, int n_b,
+                     float* logits, int32_t* argmax);
+/* Greedy continuation of sequence 0 with no host round trip between tokens: feeds `first_token` at
+ * position `pos`, then each argmax as the next token; writes n_tokens ids (the greedy fast path of
+ * neural/neuralchatengine.pas:1485-1561 with ArgMaxRow on the device). */
+int cai_decoder_generate(cai_decoder_t d, int32_t first_token, int pos, int n_tokens, int32_t* tokens_out);
+/* Multi-token prompt ingestion for sequence `seq` on the matrix cores: equals n sequential steps
+ * within tolerance.  last_logits (host, [vocab]) and argmax may be NULL. */
+int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* tokens, int n, int pos0,
+                        float* last_logits, int32_t* argmax);
+/* Session management (neural/neuraldecode.pas:5714-5843): always safe after a failed step. */
+int cai_decoder_reset(cai_decoder_t d, int seq);
+int cai_decoder_truncate(cai_decoder_t d, int seq, int n);
+int cai_decoder_len(cai_decoder_t d, int seq, int* len_out);
+int cai_decoder_snapshot(cai_decoder_t d, int seq, cai_kv_snap_t* out);
+int cai_decoder_restore(cai_decoder_t d, int seq, cai_kv_snap_t snap);
+/* Bytes of weights, biases and gains one decoded token streams (for roofline accounting). */
+int cai_decoder_weight_bytes(cai_decoder_t d, int64_t* algorithmic_bytes_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

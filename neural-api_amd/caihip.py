@@ -1,0 +1,298 @@
+"""ctypes view of include/caihip.h (tests and bench plumbing; no compute here)."""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import lib_path
+
+F32, F16, Q4_0, Q8_0, Q4_K, I8ROW = 0, 1, 2, 8, 12, 100
+ACT_NONE, ACT_RELU, ACT_SIGMOID, ACT_TANH = 0, 1, 2, 3
+X_DEVICE, Y_DEVICE = 1, 2
+KV_F32, KV_F16 = 0, 1
+W_EMBED, W_HEAD, W_Q, W_K, W_V, W_O, W_GATEUP, W_DOWN, W_ROUTER = range(9)
+V_ATTN_NORM, V_MLP_NORM, V_FINAL_NORM, V_Q_NORM, V_K_NORM = range(5)
+
+# every symbol include/caihip.h declares
+SYMBOLS = """cai_init cai_shutdown cai_last_error cai_device_name cai_sync cai_get_stream cai_timer_start cai_timer_stop
+cai_dev_alloc cai_dev_free cai_dev_upload cai_dev_download
+cai_qw_create cai_qw_create_int8row cai_qw_destroy cai_qw_info cai_qw_dequant_rows cai_qgemv cai_qgemm
+cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_router_topk
+cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_attn_decode
+cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_generate
+cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_snapshot cai_decoder_restore
+cai_decoder_weight_bytes""".split()
+
+
+class DecoderConfig(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n_layers", "d_model", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab", "max_ctx")] + \
+               [("eps", C.c_float), ("rope_theta", C.c_float)] + \
+               [(n, C.c_int32) for n in ("window", "qk_norm_full", "n_experts", "top_k", "norm_topk", "kv_dtype", "max_batch")]
+
+
+class CaiError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("caihip error %d: %s" % (code, msg))
+        self.code = code
+
+
+_LIB = None
+
+
+def load():
+    """Loads libcaihip.so.  Fails loudly when it is missing: there is no other compute path."""
+    global _LIB
+    if _LIB is None:
+        _LIB = C.CDLL(lib_path())
+        for s in SYMBOLS:
+            getattr(_LIB, s).restype = C.c_int
+        vp, i64, i32, f32 = C.c_void_p, C.c_int64, C.c_int, C.c_float
+        L = _LIB
+        L.cai_init.argtypes = [i32]
+        L.cai_last_error.argtypes = [C.c_char_p, i32]
+        L.cai_device_name.argtypes = [C.c_char_p, i32]
+        L.cai_get_stream.argtypes = [C.POINTER(vp)]
+        L.cai_timer_stop.argtypes = [C.POINTER(f32)]
+        L.cai_dev_alloc.argtypes = [i64, C.POINTER(vp)]
+        L.cai_dev_free.argtypes = [vp]
+        L.cai_dev_upload.argtypes = [vp, vp, i64]
+        L.cai_dev_download.argtypes = [vp, vp, i64]
+        L.cai_qw_create.argtypes = [i32, i64, i64, vp, vp, C.POINTER(vp)]
+        L.cai_qw_create_int8row.argtypes = [i64, i64, vp, vp, vp, C.POINTER(vp)]
+        L.cai_qw_destroy.argtypes = [vp]
+        L.cai_qw_info.argtypes = [vp, C.POINTER(i32), C.POINTER(i64), C.POINTER(i64), C.POINTER(i64)]
+        L.cai_qw_dequant_rows.argtypes = [vp, i64, i64, vp, i32]
+        L.cai_qgemv.argtypes = [vp, vp, i32, vp, i32, i32]
+        L.cai_qgemm.argtypes = [vp, vp, i32, vp, i32]
+        L.cai_rmsnorm.argtypes = [vp, vp, i32, i32, f32, vp, i32]
+        L.cai_rope.argtypes = [vp, i32, i32, i32, f32, i32]
+        L.cai_swiglu.argtypes = [vp, i32, i32, vp, i32]
+        L.cai_argmax.argtypes = [vp, i32, vp, i32]
+        L.cai_router_topk.argtypes = [vp, i32, i32, i32, vp, vp, i32]
+        L.cai_kv_create.argtypes = [i32, i32, i32, i32, i32, C.POINTER(vp)]
+        L.cai_kv_destroy.argtypes = [vp]
+        L.cai_kv_reset.argtypes = [vp]
+        L.cai_kv_truncate.argtypes = [vp, i32]
+        L.cai_kv_len.argtypes = [vp, i32, C.POINTER(i32)]
+        L.cai_kv_snapshot.argtypes = [vp, C.POINTER(vp)]
+        L.cai_kv_restore.argtypes = [vp, vp]
+        L.cai_kv_snap_destroy.argtypes = [vp]
+        L.cai_attn_decode.argtypes = [vp, i32, vp, i32, i32, f32, vp, i32]
+        L.cai_decoder_create.argtypes = [C.POINTER(DecoderConfig), C.POINTER(vp)]
+        L.cai_decoder_destroy.argtypes = [vp]
+        L.cai_decoder_set_weight.argtypes = [vp, i32, i32, vp]
+        L.cai_decoder_set_vector.argtypes = [vp, i32, i32, vp, i32]
+        L.cai_decoder_step.argtypes = [vp, vp, vp, i32, vp, vp]
+        L.cai_decoder_generate.argtypes = [vp, i32, i32, i32, vp]
+        L.cai_decoder_prefill.argtypes = [vp, i32, vp, i32, i32, vp, vp]
+        L.cai_decoder_reset.argtypes = [vp, i32]
+        L.cai_decoder_truncate.argtypes = [vp, i32, i32]
+        L.cai_decoder_len.argtypes = [vp, i32, C.POINTER(i32)]
+        L.cai_decoder_snapshot.argtypes = [vp, i32, C.POINTER(vp)]
+        L.cai_decoder_restore.argtypes = [vp, i32, vp]
+        L.cai_decoder_weight_bytes.argtypes = [vp, C.POINTER(i64)]
+    return _LIB
+
+
+def last_error():
+    buf = C.create_string_buffer(1024)
+    load().cai_last_error(buf, 1024)
+    return buf.value.decode("utf-8", "replace")
+
+
+def check(rc):
+    if rc != 0:
+        raise CaiError(rc, last_error())
+
+
+def init(device=0):
+    check(load().cai_init(device))
+
+
+def device_name():
+    buf = C.create_string_buffer(256)
+    check(load().cai_device_name(buf, 256))
+    return buf.value.decode()
+
+
+def _ptr(a):
+    if a is None:
+        return None
+    if isinstance(a, int):
+        return C.c_void_p(a)
+    return C.c_void_p(a.ctypes.data)
+
+
+class QWeight:
+    """Resident quantized matrix (cai_qw_t)."""
+
+    def __init__(self, qtype, rows, cols, blocks, bias=None, scales=None):
+        self.qtype, self.rows, self.cols = qtype, rows, cols
+        h = C.c_void_p()
+        if bias is not None:
+            bias = np.ascontiguousarray(bias, np.float32)
+        if qtype == I8ROW:
+            codes = np.ascontiguousarray(blocks).view(np.int8)
+            scales = np.ascontiguousarray(scales, np.float32)
+            check(load().cai_qw_create_int8row(rows, cols, _ptr(codes), _ptr(scales), _ptr(bias), C.byref(h)))
+        else:
+            if not isinstance(blocks, int):
+                blocks = np.ascontiguousarray(blocks)
+            check(load().cai_qw_create(qtype, rows, cols, _ptr(blocks), _ptr(bias), C.byref(h)))
+        self.h = h
+
+    def dequant_rows(self, row0=0, n_rows=None):
+        n_rows = self.rows - row0 if n_rows is None else n_rows
+        out = np.empty((n_rows, self.cols), np.float32)
+        check(load().cai_qw_dequant_rows(self.h, row0, n_rows, _ptr(out), 0))
+        return out
+
+    def gemv(self, x, act=0):
+        x = np.ascontiguousarray(x, np.float32).reshape(-1, self.cols)
+        y = np.empty((x.shape[0], self.rows), np.float32)
+        check(load().cai_qgemv(self.h, _ptr(x), x.shape[0], _ptr(y), act, 0))
+        return y
+
+    def gemm(self, x):
+        x = np.ascontiguousarray(x, np.float32).reshape(-1, self.cols)
+        y = np.empty((x.shape[0], self.rows), np.float32)
+        check(load().cai_qgemm(self.h, _ptr(x), x.shape[0], _ptr(y), 0))
+        return y
+
+    def device_bytes(self):
+        b = C.c_int64()
+        check(load().cai_qw_info(self.h, None, None, None, C.byref(b)))
+        return b.value
+
+    def close(self):
+        if self.h:
+            load().cai_qw_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class KVCache:
+    def __init__(self, n_layers, kv_heads, head_dim, max_ctx, dtype=KV_F32):
+        self.h = C.c_void_p()
+        self.kv_heads, self.head_dim = kv_heads, head_dim
+        check(load().cai_kv_create(n_layers, kv_heads, head_dim, max_ctx, dtype, C.byref(self.h)))
+
+    def attn_decode(self, layer, qkv, q_heads, window=0, softcap=0.0):
+        qkv = np.ascontiguousarray(qkv, np.float32)
+        out = np.empty(q_heads * self.head_dim, np.float32)
+        check(load().cai_attn_decode(self.h, layer, _ptr(qkv), q_heads, window, softcap, _ptr(out), 0))
+        return out
+
+    def len(self, layer=0):
+        n = C.c_int()
+        check(load().cai_kv_len(self.h, layer, C.byref(n)))
+        return n.value
+
+    def reset(self):
+        check(load().cai_kv_reset(self.h))
+
+    def truncate(self, n):
+        check(load().cai_kv_truncate(self.h, n))
+
+    def snapshot(self):
+        s = C.c_void_p()
+        check(load().cai_kv_snapshot(self.h, C.byref(s)))
+        return s
+
+    def restore(self, s):
+        check(load().cai_kv_restore(self.h, s))
+
+    def close(self):
+        if self.h:
+            load().cai_kv_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Decoder:
+    """cai_decoder_t built from a backend-neutral spec: {"cfg", "tensors", "vecs"}."""
+
+    def __init__(self, spec, max_batch=1, kv_dtype=KV_F32, max_ctx=None):
+        c = spec["cfg"]
+        self.cfg = DecoderConfig(n_layers=c["n_layers"], d_model=c["d_model"], n_q_heads=c["n_q_heads"], n_kv_heads=c["n_kv_heads"],
+                                 head_dim=c["head_dim"], ffn=c["ffn"], vocab=c["vocab"], max_ctx=max_ctx or c["max_ctx"], eps=c["eps"],
+                                 rope_theta=c["rope_theta"], window=c.get("window", 0), qk_norm_full=c.get("qk_norm_full", 0),
+                                 n_experts=c.get("n_experts", 0), top_k=c.get("top_k", 0), norm_topk=c.get("norm_topk", 0),
+                                 kv_dtype=kv_dtype, max_batch=max_batch)
+        self.h = C.c_void_p()
+        check(load().cai_decoder_create(C.byref(self.cfg), C.byref(self.h)))
+        self.weights = []
+        for (layer, slot), t in spec["tensors"].items():
+            w = t.get("qw") or QWeight(t["type"], t["rows"], t["cols"], t["raw"], t.get("bias"), t.get("scales"))
+            self.weights.append(w)
+            check(load().cai_decoder_set_weight(self.h, layer, slot, w.h))
+        for (layer, slot), v in spec["vecs"].items():
+            v = np.ascontiguousarray(v, np.float32)
+            check(load().cai_decoder_set_vector(self.h, layer, slot, _ptr(v), v.size))
+
+    def step(self, tokens, pos, want_logits=True):
+        tokens = np.ascontiguousarray(np.atleast_1d(tokens), np.int32); pos = np.ascontiguousarray(np.atleast_1d(pos), np.int32)
+        nb = tokens.size
+        lg = np.empty((nb, self.cfg.vocab), np.float32) if want_logits else None
+        am = np.empty(nb, np.int32)
+        check(load().cai_decoder_step(self.h, _ptr(tokens), _ptr(pos), nb, _ptr(lg), _ptr(am)))
+        return am, lg
+
+    def generate(self, first_token, pos, n):
+        out = np.empty(n, np.int32)
+        check(load().cai_decoder_generate(self.h, int(first_token), int(pos), n, _ptr(out)))
+        return out
+
+    def prefill(self, tokens, pos0=0, seq=0, want_logits=True):
+        tokens = np.ascontiguousarray(tokens, np.int32)
+        lg = np.empty(self.cfg.vocab, np.float32) if want_logits else None
+        am = C.c_int32()
+        check(load().cai_decoder_prefill(self.h, seq, _ptr(tokens), tokens.size, pos0, _ptr(lg), C.byref(am)))
+        return am.value, lg
+
+    def reset(self, seq=0):
+        check(load().cai_decoder_reset(self.h, seq))
+
+    def truncate(self, n, seq=0):
+        check(load().cai_decoder_truncate(self.h, seq, n))
+
+    def len(self, seq=0):
+        n = C.c_int()
+        check(load().cai_decoder_len(self.h, seq, C.byref(n)))
+        return n.value
+
+    def snapshot(self, seq=0):
+        s = C.c_void_p()
+        check(load().cai_decoder_snapshot(self.h, seq, C.byref(s)))
+        return s
+
+    def restore(self, s, seq=0):
+        check(load().cai_decoder_restore(self.h, seq, s))
+
+    def weight_bytes(self):
+        b = C.c_int64()
+        check(load().cai_decoder_weight_bytes(self.h, C.byref(b)))
+        return b.value
+
+    def close(self):
+        if self.h:
+            load().cai_decoder_destroy(self.h)
+            self.h = None
+            for w in self.weights:
+                w.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,437 @@
+// Step-resident decoder: one token per sequence per step, every activation stays in HBM/L2 for the whole
+// step, the launch sequence is captured once per batch width into a HIP graph and replayed.
+//
+// Graph order follows the reference importer (neural/neuralpretrained.pas:16384-16882) and one
+// StepForward (neural/neuraldecode.pas:5696-5712):
+//   Embedding -> per block { TokenRMSNorm -> q,k,v (+bias) -> [full-width q/k RMSNorm] -> RoPE -> FusedSDPA
+//   (append + cached GQA) -> o-proj -> Sum -> TokenRMSNorm -> gate|up -> SwiGLU -> down -> Sum }
+//   -> final TokenRMSNorm -> vocab projection -> ArgMaxRow.
+// MoE blocks (neural/neuralpretrained.pas:15331-15388): router -> softmax -> top-k gate -> expert banks.
+#include "cai_internal.hpp"
+
+#include <algorithm>
+
+struct cai_decoder_s {
+  cai_decoder_config cfg{};
+  struct Layer { cai_qw_s* w[9] = {nullptr}; float* v[5] = {nullptr}; };
+  std::vector<Layer> layers;
+  cai_qw_s* embed = nullptr; cai_qw_s* head = nullptr;
+  float* final_norm = nullptr;
+  float* theta = nullptr;
+  cai_kv_s kv;
+  float *x = nullptr, *qkv = nullptr, *att = nullptr, *gu = nullptr, *mid = nullptr, *logits = nullptr;
+  float *router_logits = nullptr, *router_probs = nullptr, *moe_gate = nullptr, *moe_part = nullptr;
+  int32_t* moe_expert = nullptr;
+  int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_argmax = nullptr, *d_gen = nullptr;
+  int32_t* h_io = nullptr;   // pinned: tokens[8] pos[8] argmax[8]
+  hipGraphExec_t graph[9] = {nullptr};
+  bool use_graph = true;
+  int qw() const { return cfg.n_q_heads * cfg.head_dim; }
+  int kw() const { return cfg.n_kv_heads * cfg.head_dim; }
+};
+
+namespace cai {
+
+__global__ void advance_kernel(int32_t* tokens, int32_t* pos, const int32_t* argmax, int32_t* gen_out, int idx)
+{
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    const int32_t t = argmax[0];
+    gen_out[idx] = t; tokens[0] = t; pos[0] += 1;
+  }
+}
+
+static void invalidate_graphs(cai_decoder_s* d)
+{
+  for (auto& g : d->graph) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
+}
+
+static int check_ready(cai_decoder_s* d)
+{
+  const cai_decoder_config& c = d->cfg;
+  if (!d->embed) return set_error(CAI_ERR_STATE, "decoder: embedding weight not set");
+  if (!d->final_norm) return set_error(CAI_ERR_STATE, "decoder: final norm gain not set");
+  for (int l = 0; l < c.n_layers; l++) {
+    const auto& L = d->layers[l];
+    const int need_w[] = {CAI_W_Q, CAI_W_K, CAI_W_V, CAI_W_O, CAI_W_GATEUP, CAI_W_DOWN};
+    for (int s : need_w) if (!L.w[s]) return set_error(CAI_ERR_STATE, "decoder: layer %d weight slot %d not set", l, s);
+    if (c.n_experts > 0 && !L.w[CAI_W_ROUTER]) return set_error(CAI_ERR_STATE, "decoder: layer %d router not set", l);
+    if (!L.v[CAI_V_ATTN_NORM] || !L.v[CAI_V_MLP_NORM]) return set_error(CAI_ERR_STATE, "decoder: layer %d norm gains not set", l);
+    if (c.qk_norm_full && (!L.v[CAI_V_Q_NORM] || !L.v[CAI_V_K_NORM])) return set_error(CAI_ERR_STATE, "decoder: layer %d q/k norm gains not set", l);
+  }
+  return CAI_OK;
+}
+
+static bool is_block_quant(int qt) { return qt == CAI_Q4_K || qt == CAI_Q4_0 || qt == CAI_Q8_0; }
+
+// Enqueues one whole step for activation rows 0..n_b-1 mapped to cache sequences seq0..seq0+n_b-1.
+static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
+{
+  const cai_decoder_config& c = d->cfg;
+  const int dm = c.d_model, qw = d->qw(), kw = d->kw(), I = c.ffn, qkvw = qw + 2 * kw;
+  int rc;
+  if ((rc = launch_embed(d->embed, d->d_tokens, n_b, d->x))) return rc;
+  for (int l = 0; l < c.n_layers; l++) {
+    auto& L = d->layers[l];
+    // --- attention half ---
+    {
+      MultiGemv m{}; m.n = 3;
+      const int slots[3] = {CAI_W_Q, CAI_W_K, CAI_W_V}; const int offs[3] = {0, qw, qw + kw};
+      bool same = true;
+      for (int i = 0; i < 3; i++) {
+        m.w[i] = L.w[slots[i]]; m.row0[i] = 0; m.rows[i] = m.w[i]->rows; m.y_off[i] = offs[i];
+        same = same && m.w[i]->qtype == m.w[0]->qtype;
+      }
+      if (same) {
+        if ((rc = launch_gemv_multi(m, d->x, n_b, d->qkv, qkvw, CAI_ACT_NONE, nullptr, L.v[CAI_V_ATTN_NORM], c.eps, 0))) return rc;
+      } else {
+        for (int i = 0; i < 3; i++) {
+          MultiGemv one{}; one.n = 1; one.w[0] = m.w[i]; one.rows[0] = m.rows[i]; one.y_off[0] = offs[i];
+          if ((rc = launch_gemv_multi(one, d->x, n_b, d->qkv, qkvw, CAI_ACT_NONE, nullptr, L.v[CAI_V_ATTN_NORM], c.eps, 0))) return rc;
+        }
+      }
+    }
+    if (c.qk_norm_full) {
+      launch_rmsnorm_strided(d->qkv, L.v[CAI_V_Q_NORM], qw, n_b, c.eps, d->qkv, qkvw, qkvw);
+      launch_rmsnorm_strided(d->qkv + qw, L.v[CAI_V_K_NORM], kw, n_b, c.eps, d->qkv + qw, qkvw, qkvw);
+    }
+    if ((rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0))) return rc;
+    if ((rc = launch_gemv(L.w[CAI_W_O], 0, dm, d->att, n_b, d->x, dm, CAI_ACT_NONE, d->x))) return rc;
+    // --- feed-forward half ---
+    if (c.n_experts == 0) {
+      MultiGemv m{}; m.n = 1; m.w[0] = L.w[CAI_W_GATEUP]; m.rows[0] = 2 * I;
+      if (is_block_quant(m.w[0]->qtype)) {
+        if ((rc = launch_gemv_multi(m, d->x, n_b, d->mid, I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, I))) return rc;
+      } else {
+        if ((rc = launch_gemv_multi(m, d->x, n_b, d->gu, 2 * I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;
+        launch_swiglu(d->gu, I, n_b, d->mid);
+      }
+      if ((rc = launch_gemv(L.w[CAI_W_DOWN], 0, dm, d->mid, n_b, d->x, dm, CAI_ACT_NONE, d->x))) return rc;
+    } else {
+      const int E = c.n_experts, K = c.top_k;
+      MultiGemv r{}; r.n = 1; r.w[0] = L.w[CAI_W_ROUTER]; r.rows[0] = E;
+      if ((rc = launch_gemv_multi(r, d->x, n_b, d->router_logits, E, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;
+      launch_router_topk(d->router_logits, E, K, c.norm_topk, n_b, d->moe_expert, d->moe_gate, d->router_probs);
+      for (int b = 0; b < n_b; b++) {
+        MultiGemv g{}; g.n = 1; g.w[0] = L.w[CAI_W_GATEUP]; g.rows[0] = 2 * I;
+        g.slot_expert = d->moe_expert + b * K; g.n_slots = K; g.expert_rows = 2 * I; g.x_slot_stride = 0;
+        const float* xb = d->x + (int64_t)b * dm;
+        if (is_block_quant(g.w[0]->qtype)) {
+          g.y_slot_stride = I;
+          if ((rc = launch_gemv_multi(g, xb, 1, d->mid, I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, I))) return rc;
+        } else {
+          g.y_slot_stride = 2 * I;
+          if ((rc = launch_gemv_multi(g, xb, 1, d->gu, 2 * I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;
+          launch_swiglu(d->gu, I, K, d->mid);
+        }
+        MultiGemv dn{}; dn.n = 1; dn.w[0] = L.w[CAI_W_DOWN]; dn.rows[0] = dm;
+        dn.slot_expert = d->moe_expert + b * K; dn.n_slots = K; dn.expert_rows = dm; dn.x_slot_stride = I; dn.y_slot_stride = dm;
+        if ((rc = launch_gemv_multi(dn, d->mid, 1, d->moe_part, dm, CAI_ACT_NONE, nullptr, nullptr, 0.0f, 0))) return rc;
+        launch_moe_combine(d->x + (int64_t)b * dm, d->moe_part, d->moe_gate + b * K, K, dm, 1);
+      }
+    }
+  }
+  {
+    cai_qw_s* hw = d->head ? d->head : d->embed;   // tied head (neural/neuralpretrained.pas:15555-)
+    MultiGemv m{}; m.n = 1; m.w[0] = hw; m.rows[0] = c.vocab;
+    if ((rc = launch_gemv_multi(m, d->x, n_b, d->logits, c.vocab, CAI_ACT_NONE, nullptr, d->final_norm, c.eps, 0))) return rc;
+  }
+  launch_argmax(d->logits, c.vocab, n_b, d->d_argmax);
+  return CAI_OK;
+}
+
+static int run_step(cai_decoder_s* d, int n_b)
+{
+  Context& c = ctx();
+  if (!d->use_graph) { const int rc = enqueue_step(d, n_b, 0); if (rc) return rc; CAI_HIP(hipGetLastError()); return CAI_OK; }
+  if (!d->graph[n_b]) {
+    hipGraph_t g = nullptr;
+    CAI_HIP(hipStreamBeginCapture(c.stream, hipStreamCaptureModeThreadLocal));
+    const int rc = enqueue_step(d, n_b, 0);
+    const hipError_t e = hipStreamEndCapture(c.stream, &g);
+    if (rc) { if (g) (void)hipGraphDestroy(g); return rc; }
+    if (e != hipSuccess) return hip_fail(e, "hipStreamEndCapture", __FILE__, __LINE__);
+    const hipError_t e2 = hipGraphInstantiate(&d->graph[n_b], g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e2 != hipSuccess) return hip_fail(e2, "hipGraphInstantiate", __FILE__, __LINE__);
+  }
+  CAI_HIP(hipGraphLaunch(d->graph[n_b], c.stream));
+  return CAI_OK;
+}
+
+}  // namespace cai
+
+using namespace cai;
+
+extern "C" int cai_decoder_create(const cai_decoder_config* cfg, cai_decoder_t* out)
+{
+  CAI_READY();
+  CAI_REQUIRE(cfg && out, "cai_decoder_create: null argument");
+  const cai_decoder_config& c = *cfg;
+  CAI_REQUIRE(c.n_layers > 0 && c.d_model > 0 && c.n_q_heads > 0 && c.n_kv_heads > 0 && c.head_dim > 0 && c.ffn > 0 && c.vocab > 0 && c.max_ctx > 0,
+              "cai_decoder_create: non-positive dimension");
+  CAI_REQUIRE(c.n_q_heads % c.n_kv_heads == 0 && c.n_q_heads / c.n_kv_heads <= 8, "cai_decoder_create: %d query heads per %d KV heads unsupported", c.n_q_heads, c.n_kv_heads);
+  CAI_REQUIRE(c.max_batch >= 1 && c.max_batch <= 8, "cai_decoder_create: max_batch %d outside 1..8", c.max_batch);
+  CAI_REQUIRE(c.n_experts == 0 || (c.top_k >= 1 && c.top_k <= c.n_experts && c.top_k <= 64), "cai_decoder_create: top_k %d of %d experts", c.top_k, c.n_experts);
+  cai_decoder_s* d = new cai_decoder_s();
+  d->cfg = c;
+  d->layers.resize(c.n_layers);
+  const int B = c.max_batch, qw = d->qw(), kw = d->kw();
+  int rc = kv_alloc(&d->kv, B, c.n_layers, c.n_kv_heads, c.head_dim, c.max_ctx, c.kv_dtype);
+  if (rc) { delete d; return rc; }
+  std::vector<float> th; rope_thetas(c.rope_theta, c.head_dim, th);
+  auto alloc_f = [&](float** p, size_t n) { return hipMalloc((void**)p, n * sizeof(float)); };
+  hipError_t e = alloc_f(&d->theta, th.size());
+  const int K = std::max(c.top_k, 1);
+  if (e == hipSuccess) e = alloc_f(&d->x, (size_t)B * c.d_model);
+  if (e == hipSuccess) e = alloc_f(&d->qkv, (size_t)B * (qw + 2 * kw));
+  if (e == hipSuccess) e = alloc_f(&d->att, (size_t)B * qw);
+  if (e == hipSuccess) e = alloc_f(&d->gu, (size_t)std::max(B, K) * 2 * c.ffn);
+  if (e == hipSuccess) e = alloc_f(&d->mid, (size_t)std::max(B, K) * c.ffn);
+  if (e == hipSuccess) e = alloc_f(&d->logits, (size_t)B * c.vocab);
+  if (c.n_experts > 0) {
+    if (e == hipSuccess) e = alloc_f(&d->router_logits, (size_t)B * c.n_experts);
+    if (e == hipSuccess) e = alloc_f(&d->router_probs, (size_t)B * c.n_experts);
+    if (e == hipSuccess) e = alloc_f(&d->moe_gate, (size_t)B * K);
+    if (e == hipSuccess) e = alloc_f(&d->moe_part, (size_t)K * c.d_model);
+    if (e == hipSuccess) e = hipMalloc((void**)&d->moe_expert, (size_t)B * K * sizeof(int32_t));
+  }
+  if (e == hipSuccess) e = hipMalloc((void**)&d->d_tokens, 3 * 8 * sizeof(int32_t));
+  if (e == hipSuccess) e = hipMalloc((void**)&d->d_gen, (size_t)c.max_ctx * sizeof(int32_t));
+  if (e == hipSuccess) e = hipHostMalloc((void**)&d->h_io, 3 * 8 * sizeof(int32_t), hipHostMallocDefault);
+  if (e == hipSuccess) e = hipMemcpyAsync(d->theta, th.data(), th.size() * 4, hipMemcpyHostToDevice, ctx().stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(ctx().stream);
+  if (e != hipSuccess) { cai_decoder_destroy(d); return hip_fail(e, "cai_decoder_create allocation", __FILE__, __LINE__); }
+  d->d_pos = d->d_tokens + 8; d->d_argmax = d->d_tokens + 16;
+  const char* ng = getenv("CAIHIP_NO_GRAPH");
+  d->use_graph = !(ng && ng[0] == '1');
+  *out = d;
+  return CAI_OK;
+}
+
+extern "C" int cai_decoder_destroy(cai_decoder_t d)
+{
+  if (!d) return CAI_OK;
+  if (ctx().ready) (void)hipStreamSynchronize(ctx().stream);
+  invalidate_graphs(d);
+  kv_free(&d->kv);
+  float* fs[] = {d->theta, d->x, d->qkv, d->att, d->gu, d->mid, d->logits, d->router_logits, d->router_probs, d->moe_gate, d->moe_part, d->final_norm};
+  for (float* p : fs) if (p) (void)hipFree(p);
+  for (auto& L : d->layers) for (float* p : L.v) if (p) (void)hipFree(p);
+  if (d->moe_expert) (void)hipFree(d->moe_expert);
+  if (d->d_tokens) (void)hipFree(d->d_tokens);
+  if (d->d_gen) (void)hipFree(d->d_gen);
+  if (d->h_io) (void)hipHostFree(d->h_io);
+  delete d;
+  return CAI_OK;
+}
+
+extern "C" int cai_decoder_set_weight(cai_decoder_t d, int layer, int slot, cai_qw_t w)
+{
+  CAI_REQUIRE(d && w, "cai_decoder_set_weight: null argument");
+  const cai_decoder_config& c = d->cfg;
+  const int qw = d->qw(), kw = d->kw();
+  int64_t rows = -1, cols = -1;
+  const int64_t E = c.n_experts > 0 ? c.n_experts : 1;
+  switch (slot) {
+    case CAI_W_EMBED: case CAI_W_HEAD: rows = c.vocab; cols = c.d_model; break;
+    case CAI_W_Q: rows = qw; cols = c.d_model; break;
+    case CAI_W_K: case CAI_W_V: rows = kw; cols = c.d_model; break;
+    case CAI_W_O: rows = c.d_model; cols = qw; break;
+    case CAI_W_GATEUP: rows = E * 2 * c.ffn; cols = c.d_model; break;
+    case CAI_W_DOWN: rows = E * c.d_model; cols = c.ffn; break;
+    case CAI_W_ROUTER: rows = c.n_experts; cols = c.d_model; break;
+    default: return set_error(CAI_ERR_INVALID, "cai_decoder_set_weight: unknown slot %d", slot);
+  }
+  CAI_REQUIRE(w->rows == rows && w->cols == cols, "cai_decoder_set_weight: slot %d expects %lld x %lld, got %lld x %lld", slot,
+              (long long)rows, (long long)cols, (long long)w->rows, (long long)w->cols);
+  if (slot == CAI_W_EMBED) d->embed = w;
+  else if (slot == CAI_W_HEAD) d->head = w;
+  else {
+    CAI_REQUIRE(layer >= 0 && layer < c.n_layers, "cai_decoder_set_weight: layer %d of %d", layer, c.n_layers);
+    d->layers[layer].w[slot] = w;
+  }
+  invalidate_graphs(d);
+  return CAI_OK;
+}
+
+extern "C" int cai_decoder_set_vector(cai_decoder_t d, int layer, int slot, const float* v, int n)
+{
+  CAI_READY();
+  CAI_REQUIRE(d && v, "cai_decoder_set_vector: null argument");
+  const cai_decoder_config& c = d->cfg;
+  int want = c.d_model;
+  if (slot == CAI_V_Q_NORM) want = d->qw(); else if (slot == CAI_V_K_NORM) want = d->kw();
+  CAI_REQUIRE(slot >= 0 && slot <= 4, "cai_decoder_set_vector: unknown slot %d", slot);
+  CAI_REQUIRE(n == want, "cai_decoder_set_vector: slot %d expects %d values, got %d", slot, want, n);
+  float** dst;
+  if (slot == CAI_V_FINAL_NORM) dst = &d->final_norm;
+  else {
+    CAI_REQUIRE(layer >= 0 && layer < c.n_layers, "cai_decoder_set_vector: layer %d of %d", layer, c.n_layers);
+    dst = &d->layers[layer].v[slot];
+  }
+  if (!*dst) CAI_HIP(hipMalloc((void**)dst, (size_t)n * 4));
+  CAI_HIP(hipMemcpyAsync(*dst, v, (size_t)n * 4, hipMemcpyHostToDevice, ctx().stream));
+  CAI_HIP(hipStreamSynchronize(ctx().stream));
+  invalidate_graphs(d);
+  return CAI_OK;
+}
+
+extern "C" int cai_decoder_step(cai_decoder_t d, const int32_t* tokens, const int32_t* pos, int n_b, float* logits, int32_t* argmax)
+{
+  CAI_READY();
+  CAI_REQUIRE(d && tokens && pos, "cai_decoder_step: null argument");
+  const cai_decoder_config& c = d->cfg;
+  CAI_REQUIRE(n_b >= 1 && n_b <= c.max_batch, "cai_decoder_step: n_b %d outside 1..%d", n_b, c.max_batch);
+  int rc = check_ready(d); if (rc) return rc;
+  for (int b = 0; b < n_b; b++) {
+    CAI_REQUIRE(tokens[b] >= 0 && tokens[b] < c.vocab, "cai_decoder_step: token %d outside vocab %d", tokens[b], c.vocab);
+    if (pos[b] != d->kv.len_at(b, 0)) return set_error(CAI_ERR_STATE, "cai_decoder_step: sequence %d is at position %d, got %d", b, d->kv.len_at(b, 0), pos[b]);
+    if (pos[b] >= c.max_ctx) return set_error(CAI_ERR_STATE, "cai_decoder_step: sequence %d reached max_ctx %d", b, c.max_ctx);
+  }
+  Context& cx = ctx();
+  for (int b = 0; b < n_b; b++) { d->h_io[b] = tokens[b]; d->h_io[8 + b] = pos[b]; }
+  CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
+  if ((rc = run_step(d, n_b))) return rc;
+  if (logits) CAI_HIP(hipMemcpyAsync(logits, d->logits, (size_t)n_b * c.vocab * 4, hipMemcpyDeviceToHost, cx.stream));
+  CAI_HIP(hipMemcpyAsync(d->h_io + 16, d->d_argmax, 8 * sizeof(int32_t), hipMemcpyDeviceToHost, cx.stream));
+  CAI_HIP(hipStreamSynchronize(cx.stream));
+  for (int b = 0; b < n_b; b++) {
+    for (int l = 0; l < c.n_layers; l++) d->kv.len_at(b, l) = pos[b] + 1;
+    if (argmax) argmax[b] = d->h_io[16 + b];
+  }
+  return CAI_OK;
+}
+
+extern "C" int cai_decoder_generate(cai_decoder_t d, int32_t first_token, int pos, int n_tokens, int32_t* tokens_out)
+{
+  CAI_READY();
+  CAI_REQUIRE(d && tokens_out && n_tokens >= 1, "cai_decoder_generate: bad argument");
+  const cai_decoder_config& c = d->cfg;
+  int rc = check_ready(d); if (rc) return rc;
+  CAI_REQUIRE(first_token >= 0 && first_token < c.vocab, "cai_decoder_generate: token %d outside vocab %d", first_token, c.vocab);
+  if (pos != d->kv.len_at(0, 0)) return set_error(CAI_ERR_STATE, "cai_decoder_generate: sequence 0 is at position %d, got %d", d->kv.len_at(0, 0), pos);
+  if (pos + n_tokens > c.max_ctx) return set_error(CAI_ERR_STATE, "cai_decoder_generate: %d tokens from %d exceed max_ctx %d", n_tokens, pos, c.max_ctx);
+  Context& cx = ctx();
+  d->h_io[0] = first_token; d->h_io[8] = pos;
+  CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
+  for (int i = 0; i < n_tokens; i++) {
+    if ((rc = run_step(d, 1))) return rc;
+    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, cx.stream, d->d_tokens, d->d_pos, d->d_argmax, d->d_gen, i);
+  }
+  CAI_HIP(hipMemcpyAsync(tokens_out, d->d_gen, (size_t)n_tokens * sizeof(int32_t), hipMemcpyDeviceToHost, cx.stream));
+  CAI_HIP(hipStreamSynchronize(cx.stream));
+  for (int l = 0; l < c.n_layers; l++) d->kv.len_at(0, l) = pos + n_tokens;
+  return CAI_OK;
+}
+
+extern "C" int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* tokens, int n, int pos0, float* last_logits, int32_t* argmax)
+{
+  CAI_READY();
+  CAI_REQUIRE(d && tokens && n >= 1, "cai_decoder_prefill: bad argument");
+  const cai_decoder_config& c = d->cfg;
+  CAI_REQUIRE(seq >= 0 && seq < c.max_batch, "cai_decoder_prefill: sequence %d of %d", seq, c.max_batch);
+  int rc = check_ready(d); if (rc) return rc;
+  if (pos0 != d->kv.len_at(seq, 0)) return set_error(CAI_ERR_STATE, "cai_decoder_prefill: sequence %d is at position %d, got %d", seq, d->kv.len_at(seq, 0), pos0);
+  if (pos0 + n > c.max_ctx) return set_error(CAI_ERR_STATE, "cai_decoder_prefill: %d tokens from %d exceed max_ctx %d", n, pos0, c.max_ctx);
+  for (int i = 0; i < n; i++) CAI_REQUIRE(tokens[i] >= 0 && tokens[i] < c.vocab, "cai_decoder_prefill: token %d outside vocab %d", tokens[i], c.vocab);
+  Context& cx = ctx();
+  // Token-at-a-time ingestion, the reference's own prefill (neural/neuralchatengine.pas:1466-1470).
+  for (int i = 0; i < n; i++) {
+    CAI_HIP(hipStreamSynchronize(cx.stream));   // h_io is reused
+    d->h_io[0] = tokens[i]; d->h_io[8] = pos0 + i;
+    CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
+    if (seq == 0) { if ((rc = run_step(d, 1))) return rc; }
+    else { if ((rc = enqueue_step(d, 1, seq))) return rc; }
+  }
+  if (last_logits) CAI_HIP(hipMemcpyAsync(last_logits, d->logits, (size_t)c.vocab * 4, hipMemcpyDeviceToHost, cx.stream));
+  CAI_HIP(hipMemcpyAsync(d->h_io + 16, d->d_argmax, 8 * sizeof(int32_t), hipMemcpyDeviceToHost, cx.stream));
+  CAI_HIP(hipStreamSynchronize(cx.stream));
+  for (int l = 0; l < c.n_layers; l++) d->kv.len_at(seq, l) = pos0 + n;
+  if (argmax) *argmax = d->h_io[16];
+  return CAI_OK;
+}
+
+extern "C" int cai_decoder_reset(cai_decoder_t d, int seq)
+{
+  CAI_REQUIRE(d, "cai_decoder_reset: null decoder");
+  CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch, "cai_decoder_reset: sequence %d of %d", seq, d->cfg.max_batch);
+  for (int l = 0; l < d->cfg.n_layers; l++) d->kv.len_at(seq, l) = 0;
+  return CAI_OK;
+}
+
+extern "C" int cai_decoder_truncate(cai_decoder_t d, int seq, int n)
+{
+  CAI_REQUIRE(d, "cai_decoder_truncate: null decoder");
+  CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch && n >= 0, "cai_decoder_truncate: bad argument");
+  for (int l = 0; l < d->cfg.n_layers; l++) if (d->kv.len_at(seq, l) > n) d->kv.len_at(seq, l) = n;
+  return CAI_OK;
+}
+
+extern "C" int cai_decoder_len(cai_decoder_t d, int seq, int* len_out)
+{
+  CAI_REQUIRE(d && len_out, "cai_decoder_len: null argument");
+  CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch, "cai_decoder_len: sequence %d of %d", seq, d->cfg.max_batch);
+  *len_out = d->kv.len_at(seq, 0);
+  return CAI_OK;
+}
+
+extern "C" int cai_decoder_snapshot(cai_decoder_t d, int seq, cai_kv_snap_t* out)
+{
+  CAI_READY();
+  CAI_REQUIRE(d && out, "cai_decoder_snapshot: null argument");
+  CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch, "cai_decoder_snapshot: sequence %d of %d", seq, d->cfg.max_batch);
+  return kv_snapshot(&d->kv, seq, out);
+}
+
+extern "C" int cai_decoder_restore(cai_decoder_t d, int seq, cai_kv_snap_t snap)
+{
+  CAI_READY();
+  CAI_REQUIRE(d && snap, "cai_decoder_restore: null argument");
+  CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch, "cai_decoder_restore: sequence %d of %d", seq, d->cfg.max_batch);
+  return kv_restore(&d->kv, seq, snap);
+}
+
+extern "C" int cai_decoder_weight_bytes(cai_decoder_t d, int64_t* out)
+{
+  CAI_REQUIRE(d && out, "cai_decoder_weight_bytes: null argument");
+  const cai_decoder_config& c = d->cfg;
+  int rc = check_ready(d); if (rc) return rc;
+  int64_t b = 0;
+  const cai_qw_s* hw = d->head ? d->head : d->embed;
+  b += hw->algo_bytes + (int64_t)c.d_model * 4;             // head + final norm gain
+  b += d->embed->algo_bytes / d->embed->rows;                // one embedding row
+  for (auto& L : d->layers) {
+    const int dense[] = {CAI_W_Q, CAI_W_K, CAI_W_V, CAI_W_O};
+    for (int s : dense) b += L.w[s]->algo_bytes;
+    if (c.n_experts > 0) {
+      b += L.w[CAI_W_ROUTER]->algo_bytes;
+      b += (L.w[CAI_W_GATEUP]->algo_bytes + L.w[CAI_W_DOWN]->algo_bytes) / c.n_experts * c.top_k;
+    } else b += L.w[CAI_W_GATEUP]->algo_bytes + L.w[CAI_W_DOWN]->algo_bytes;
+    b += 2 * (int64_t)c.d_model * 4;
+  }
+  *out = b;
+  return CAI_OK;
+}
+
+// cai_qgemm: multi-token linear layer. Until the matrix-core kernel is in place it walks the tokens in groups
+// of up to 8 through the small-batch kernel (same results as n_tokens GEMVs).
+extern "C" int cai_qgemm(cai_qw_t w, const float* x, int n_tokens, float* y, int flags)
+{
+  CAI_READY();
+  CAI_REQUIRE(w && x && y && n_tokens >= 1, "cai_qgemm: bad argument");
+  Context& c = ctx();
+  const size_t xb = (size_t)n_tokens * w->cols * 4, yb = (size_t)n_tokens * w->rows * 4;
+  const float* dx = x; float* dy = y; int rc;
+  if (!(flags & CAI_X_DEVICE)) {
+    if ((rc = ensure_stage(&c.stage_in, &c.stage_in_cap, xb))) return rc;
+    CAI_HIP(hipMemcpyAsync(c.stage_in, x, xb, hipMemcpyHostToDevice, c.stream));
+    dx = (const float*)c.stage_in;
+  }
+  if (!(flags & CAI_Y_DEVICE)) { if ((rc = ensure_stage(&c.stage_out, &c.stage_out_cap, yb))) return rc; dy = (float*)c.stage_out; }
+  for (int t = 0; t < n_tokens; t += 8) {
+    const int nb = std::min(8, n_tokens - t);
+    if ((rc = launch_gemv(w, 0, w->rows, dx + (int64_t)t * w->cols, nb, dy + (int64_t)t * w->rows, w->rows, CAI_ACT_NONE, nullptr))) return rc;
+  }
+  if (!(flags & CAI_Y_DEVICE)) { CAI_HIP(hipMemcpyAsync(y, dy, yb, hipMemcpyDeviceToHost, c.stream)); CAI_HIP(hipStreamSynchronize(c.stream)); }
+  return CAI_OK;
+}

@@ -1,0 +1,617 @@
+// Block-quantized matrix-vector / small-batch kernels for gfx950 (wave64).
+//
+// One wave owns R output rows and walks the reduction axis with 16-byte (128-bit) loads of packed
+// quant data, one "unit" per lane per step; the activation vector is staged once per work-group in
+// LDS in a unit-transposed order (16 adjacent lanes read 16 adjacent float4 -> no bank conflicts)
+// and reused for all rows of the wave.  Weights are dequantized in registers, accumulation is fp32,
+// and the per-row sum is reduced across the 64 lanes with DPP row shifts + row broadcasts.
+//
+// Semantics of the layer this implements: Out[b*NumAs + a] = act(dot(W[a], X[b]) + bias[a])
+// (reference: neural/neuralvolume.pas:12127-12423, 12693-12745; fused tail neural/neural.cl:111-146).
+#include "cai_internal.hpp"
+
+namespace cai {
+
+// ------------------------------------------------------------------------------------------
+// wave64 sum: DPP row_shr within rows of 16, then row_bcast15 / row_bcast31; total ends in lane 63.
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v)
+{
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, true)); // row_shr:1
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x112, 0xf, 0xf, true)); // row_shr:2
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x114, 0xf, 0xf, true)); // row_shr:4
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x118, 0xf, 0xf, true)); // row_shr:8
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xa, 0xf, true)); // row_bcast:15
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xc, 0xf, true)); // row_bcast:31
+  return v;  // valid in lane 63
+}
+
+__device__ __forceinline__ float act_apply(float v, int act)
+{
+  // neural/neural.cl:114-146
+  if (act == CAI_ACT_RELU) return v < 0.0f ? 0.0f : v;
+  if (act == CAI_ACT_SIGMOID) {
+    if (v > 0.0f) return 1.0f / (1.0f + expf(-v));
+    const float s = expf(v); return s / (1.0f + s);
+  }
+  if (act == CAI_ACT_TANH) {
+    float xc = v > 10.0f ? 10.0f : (v < -10.0f ? -10.0f : v);
+    const float e = expf(-2.0f * xc); return (1.0f - e) / (1.0f + e);
+  }
+  return v;
+}
+
+__device__ __forceinline__ float silu_mul(float up, float gate)
+{
+  // neural/neural.cl:1236-1247: two-branch sigmoid, y = A * (B * sigmoid(B))
+  float sig;
+  if (gate > 0.0f) sig = 1.0f / (1.0f + expf(-gate));
+  else { const float s = expf(gate); sig = s / (1.0f + s); }
+  return up * (gate * sig);
+}
+
+struct GemvSeg {
+  const uint8_t* data; const uint8_t* aux; const float* bias;
+  int rows;       // rows of this segment computed by the launch
+  int y_off;      // offset of the segment's first output inside a y row
+  int grp_end;    // cumulative row-group count (exclusive)
+};
+
+struct GemvParams {
+  GemvSeg seg[3];
+  int n_seg;
+  const float* x;        // [NB][cols]
+  float* y;              // [NB][y_stride]
+  const float* residual; // same indexing as y, may be null
+  const float* norm_gain; float norm_eps;  // fused RMSNorm on the input when norm_gain != null
+  int cols;
+  int kp;                // panel length in floats (multiple of 256)
+  int y_stride;
+  int act;
+  int half;              // swiglu: rows [0,half) are up, [half,2*half) gate
+  // expert-bank gather (MoE): blockIdx.y = slot; the slot's expert id selects a row window of the bank
+  const int32_t* slot_expert; int64_t expert_rows; int x_slot_stride; int y_slot_stride;
+};
+
+// units per lane-step and geometry per type
+template <int QT> struct QTraits;
+template <> struct QTraits<CAI_Q4_K> { static constexpr int UW = 32, T = 8; };  // weights per unit, float4 per unit
+template <> struct QTraits<CAI_Q4_0> { static constexpr int UW = 32, T = 8; };
+template <> struct QTraits<CAI_Q8_0> { static constexpr int UW = 16, T = 4; };
+
+// original float4 index n (within the panel) -> LDS float4 slot, unit-transposed in tiles of 16 units
+template <int QT> __device__ __forceinline__ int lds_slot(int n)
+{
+  int u, t;
+  if (QT == CAI_Q4_K) {
+    // n = [sb][cc:2][hi:1][h:1][tt:2]; unit = sb*8 + cc*2 + h; t = hi*4 + tt
+    const int sb = n >> 6, cc = (n >> 4) & 3, hi = (n >> 3) & 1, h = (n >> 2) & 1, tt = n & 3;
+    u = sb * 8 + cc * 2 + h; t = hi * 4 + tt;
+  } else if (QT == CAI_Q4_0) { u = n >> 3; t = n & 7; }
+  else { u = n >> 2; t = n & 3; }
+  constexpr int T = QTraits<QT>::T;
+  return (u >> 4) * 16 * T + t * 16 + (u & 15);
+}
+
+template <int QT> __device__ __forceinline__ int lds_unit_base(int u)
+{
+  constexpr int T = QTraits<QT>::T;
+  return (u >> 4) * 16 * T + (u & 15);   // + t*16
+}
+
+__device__ __forceinline__ float cvt_ub0(uint32_t v) { return (float)(v & 0xffu); }
+__device__ __forceinline__ float cvt_ub1(uint32_t v) { return (float)((v >> 8) & 0xffu); }
+__device__ __forceinline__ float cvt_ub2(uint32_t v) { return (float)((v >> 16) & 0xffu); }
+__device__ __forceinline__ float cvt_ub3(uint32_t v) { return (float)(v >> 24); }
+
+// Q4_K: the 6-bit (scale, min) pairs of sub-blocks 2cc and 2cc+1 from the 12 packed bytes
+// (neural/neuralgguf.pas:448-464).  Returns packed bytes: sc = [sc_lo | sc_hi<<8], mn likewise.
+__device__ __forceinline__ void q4k_scale_pair(uint32_t d0, uint32_t d1, uint32_t d2, int cc, uint32_t& sc, uint32_t& mn)
+{
+  const int sh = (cc & 1) * 16;
+  const uint32_t h0 = (d0 >> sh) & 0xffffu, h1 = (d1 >> sh) & 0xffffu, h2 = (d2 >> sh) & 0xffffu;
+  if (cc < 2) { sc = h0 & 0x3f3fu; mn = h1 & 0x3f3fu; }
+  else { sc = (h2 & 0x0f0fu) | ((h0 >> 2) & 0x3030u); mn = ((h2 >> 4) & 0x0f0fu) | ((h1 >> 2) & 0x3030u); }
+}
+
+// ------------------------------------------------------------------------------------------
+// Fast kernel: Q4_K / Q4_0 / Q8_0.  MODE 0: plain rows.  MODE 1: SwiGLU pairs (row i and row half+i).
+// ------------------------------------------------------------------------------------------
+template <int QT, int NB, int R, int MODE>
+__global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
+{
+  extern __shared__ float4 xs4[];          // [NB][kp/4]
+  constexpr int UW = QTraits<QT>::UW, T = QTraits<QT>::T;
+  constexpr int RR = MODE == 1 ? 2 * R : R;  // weight rows per wave
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int grp = blockIdx.x * 4 + wave;
+
+  // segment lookup (groups never straddle segments)
+  int s = 0, grp0 = 0;
+  if (p.n_seg > 1 && grp >= p.seg[0].grp_end) { s = 1; grp0 = p.seg[0].grp_end; }
+  if (p.n_seg > 2 && grp >= p.seg[1].grp_end) { s = 2; grp0 = p.seg[1].grp_end; }
+  const GemvSeg sg = p.seg[s];
+  const int row_first = (grp - grp0) * R;
+  const bool wave_live = grp < p.seg[p.n_seg - 1].grp_end;
+  int64_t bank_row = 0;
+  const float* xin = p.x; float* yout = p.y;
+  if (p.slot_expert) {
+    bank_row = (int64_t)p.slot_expert[blockIdx.y] * p.expert_rows;
+    xin += (int64_t)blockIdx.y * p.x_slot_stride; yout += (int64_t)blockIdx.y * p.y_slot_stride;
+  }
+
+  const int cols = p.cols;
+  int64_t row_bytes, aux_row_bytes = 0;
+  if (QT == CAI_Q4_K) row_bytes = (int64_t)(cols >> 8) * 144;
+  else if (QT == CAI_Q4_0) { row_bytes = cols >> 1; aux_row_bytes = (cols >> 5) * 2; }
+  else { row_bytes = cols; aux_row_bytes = (cols >> 5) * 2; }
+
+  const uint8_t* rp[RR]; const uint8_t* ap[RR]; bool live[RR];
+#pragma unroll
+  for (int r = 0; r < RR; r++) {
+    int row = row_first + (MODE == 1 ? (r >> 1) : r);
+    live[r] = wave_live && row < (MODE == 1 ? p.half : sg.rows);
+    if (!live[r]) row = 0;
+    if (MODE == 1 && (r & 1)) row += p.half;
+    rp[r] = sg.data + (bank_row + row) * row_bytes;
+    ap[r] = sg.aux + (bank_row + row) * aux_row_bytes;
+  }
+
+  float acc[RR][NB];
+#pragma unroll
+  for (int r = 0; r < RR; r++)
+#pragma unroll
+    for (int b = 0; b < NB; b++) acc[r][b] = 0.0f;
+
+  // fused RMSNorm statistics (neural/neural.cl:1047-1085): inv = 1/sqrt(mean(x^2)+eps), per batch row
+  float inv_rms[NB];
+  if (p.norm_gain) {
+    __shared__ float red[NB][4];
+#pragma unroll
+    for (int b = 0; b < NB; b++) {
+      float ss = 0.0f;
+      const float* xb = xin + (int64_t)b * cols;
+      for (int i = threadIdx.x; i < cols; i += 256) { const float v = xb[i]; ss = fmaf(v, v, ss); }
+      ss = wave_sum(ss);
+      if (lane == 63) red[b][wave] = ss;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int b = 0; b < NB; b++) {
+      const float tot = (red[b][0] + red[b][1]) + (red[b][2] + red[b][3]);
+      inv_rms[b] = 1.0f / sqrtf(tot / (float)cols + p.norm_eps);
+    }
+  }
+
+  for (int k0 = 0; k0 < cols; k0 += p.kp) {
+    const int kp = min(p.kp, cols - k0);
+    const int n4 = kp >> 2;
+    __syncthreads();
+#pragma unroll
+    for (int b = 0; b < NB; b++) {
+      const float4* src = reinterpret_cast<const float4*>(xin + (int64_t)b * cols + k0);
+      float4* dst = xs4 + b * (p.kp >> 2);
+      for (int n = threadIdx.x; n < n4; n += 256) {
+        float4 v = src[n];
+        if (p.norm_gain) {
+          const float4 g = reinterpret_cast<const float4*>(p.norm_gain + k0)[n];
+          v.x = g.x * (v.x * inv_rms[b]); v.y = g.y * (v.y * inv_rms[b]);
+          v.z = g.z * (v.z * inv_rms[b]); v.w = g.w * (v.w * inv_rms[b]);
+        }
+        dst[lds_slot<QT>(n)] = v;
+      }
+    }
+    __syncthreads();
+
+    const int n_units = kp / UW;
+    for (int u = lane; u < n_units; u += 64) {
+      // ---- issue all weight loads of this step first ----
+      uint4 q[RR]; uint4 hdr[RR]; uint16_t dh[RR];
+      if (QT == CAI_Q4_K) {
+        const int sb = (k0 >> 8) + (u >> 3), j = u & 7;
+#pragma unroll
+        for (int r = 0; r < RR; r++) {
+          const uint8_t* blk = rp[r] + (int64_t)sb * 144;
+          hdr[r] = *reinterpret_cast<const uint4*>(blk);
+          q[r] = *reinterpret_cast<const uint4*>(blk + 16 + 16 * j);
+        }
+      } else if (QT == CAI_Q4_0) {
+        const int blk = (k0 >> 5) + u;
+#pragma unroll
+        for (int r = 0; r < RR; r++) {
+          q[r] = *reinterpret_cast<const uint4*>(rp[r] + (int64_t)blk * 16);
+          dh[r] = *reinterpret_cast<const uint16_t*>(ap[r] + blk * 2);
+        }
+      } else {
+        const int un = (k0 >> 4) + u;
+#pragma unroll
+        for (int r = 0; r < RR; r++) {
+          q[r] = *reinterpret_cast<const uint4*>(rp[r] + (int64_t)un * 16);
+          dh[r] = *reinterpret_cast<const uint16_t*>(ap[r] + (un >> 1) * 2);
+        }
+      }
+      const int xb0 = lds_unit_base<QT>(u);
+
+      if (NB == 1) {
+        // x unit in registers, reused for every row of the wave
+        float xv[UW];
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+          const float4 v = xs4[xb0 + t * 16];
+          xv[4 * t] = v.x; xv[4 * t + 1] = v.y; xv[4 * t + 2] = v.z; xv[4 * t + 3] = v.w;
+        }
+        if (QT == CAI_Q4_K) {
+          float sxlo = 0.0f, sxhi = 0.0f;
+#pragma unroll
+          for (int i = 0; i < 16; i++) { sxlo += xv[i]; sxhi += xv[16 + i]; }
+          const int cc = (u & 7) >> 1;
+#pragma unroll
+          for (int r = 0; r < RR; r++) {
+            const uint32_t qw[4] = {q[r].x, q[r].y, q[r].z, q[r].w};
+            float slo = 0.0f, shi = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+              const uint32_t lo = qw[w] & 0x0f0f0f0fu, hi = (qw[w] >> 4) & 0x0f0f0f0fu;
+              slo = fmaf(cvt_ub0(lo), xv[4 * w], slo);     slo = fmaf(cvt_ub1(lo), xv[4 * w + 1], slo);
+              slo = fmaf(cvt_ub2(lo), xv[4 * w + 2], slo); slo = fmaf(cvt_ub3(lo), xv[4 * w + 3], slo);
+              shi = fmaf(cvt_ub0(hi), xv[16 + 4 * w], shi);     shi = fmaf(cvt_ub1(hi), xv[16 + 4 * w + 1], shi);
+              shi = fmaf(cvt_ub2(hi), xv[16 + 4 * w + 2], shi); shi = fmaf(cvt_ub3(hi), xv[16 + 4 * w + 3], shi);
+            }
+            uint32_t sc, mn; q4k_scale_pair(hdr[r].y, hdr[r].z, hdr[r].w, cc, sc, mn);
+            const float d = __half2float(__ushort_as_half((unsigned short)(hdr[r].x & 0xffffu)));
+            const float dmin = __half2float(__ushort_as_half((unsigned short)(hdr[r].x >> 16)));
+            const float part = d * (cvt_ub0(sc) * slo + cvt_ub1(sc) * shi) - dmin * (cvt_ub0(mn) * sxlo + cvt_ub1(mn) * sxhi);
+            acc[r][0] += part;
+          }
+        } else if (QT == CAI_Q4_0) {
+          float sx = 0.0f;
+#pragma unroll
+          for (int i = 0; i < 32; i++) sx += xv[i];
+#pragma unroll
+          for (int r = 0; r < RR; r++) {
+            const uint32_t qw[4] = {q[r].x, q[r].y, q[r].z, q[r].w};
+            float sq = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+              const uint32_t lo = qw[w] & 0x0f0f0f0fu, hi = (qw[w] >> 4) & 0x0f0f0f0fu;
+              sq = fmaf(cvt_ub0(lo), xv[4 * w], sq);     sq = fmaf(cvt_ub1(lo), xv[4 * w + 1], sq);
+              sq = fmaf(cvt_ub2(lo), xv[4 * w + 2], sq); sq = fmaf(cvt_ub3(lo), xv[4 * w + 3], sq);
+              sq = fmaf(cvt_ub0(hi), xv[16 + 4 * w], sq);     sq = fmaf(cvt_ub1(hi), xv[16 + 4 * w + 1], sq);
+              sq = fmaf(cvt_ub2(hi), xv[16 + 4 * w + 2], sq); sq = fmaf(cvt_ub3(hi), xv[16 + 4 * w + 3], sq);
+            }
+            const float d = __half2float(__ushort_as_half(dh[r]));
+            acc[r][0] = fmaf(d, sq - 8.0f * sx, acc[r][0]);
+          }
+        } else {  // Q8_0
+#pragma unroll
+          for (int r = 0; r < RR; r++) {
+            const uint32_t qw[4] = {q[r].x, q[r].y, q[r].z, q[r].w};
+            float sq = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+              sq = fmaf((float)(int8_t)(qw[w] & 0xff), xv[4 * w], sq);
+              sq = fmaf((float)(int8_t)((qw[w] >> 8) & 0xff), xv[4 * w + 1], sq);
+              sq = fmaf((float)(int8_t)((qw[w] >> 16) & 0xff), xv[4 * w + 2], sq);
+              sq = fmaf((float)(int8_t)(qw[w] >> 24), xv[4 * w + 3], sq);
+            }
+            acc[r][0] = fmaf(__half2float(__ushort_as_half(dh[r])), sq, acc[r][0]);
+          }
+        }
+      } else {
+        // small batch: dequantize the unit of every row once (unscaled integer values as floats),
+        // then stream the NB activation units from LDS
+        float wf[RR][UW];
+        float s0[RR], s1[RR], m0[RR], m1[RR];
+#pragma unroll
+        for (int r = 0; r < RR; r++) {
+          const uint32_t qw[4] = {q[r].x, q[r].y, q[r].z, q[r].w};
+          if (QT == CAI_Q8_0) {
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+              wf[r][4 * w] = (float)(int8_t)(qw[w] & 0xff); wf[r][4 * w + 1] = (float)(int8_t)((qw[w] >> 8) & 0xff);
+              wf[r][4 * w + 2] = (float)(int8_t)((qw[w] >> 16) & 0xff); wf[r][4 * w + 3] = (float)(int8_t)(qw[w] >> 24);
+            }
+            s0[r] = __half2float(__ushort_as_half(dh[r]));
+          } else {
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+              const uint32_t lo = qw[w] & 0x0f0f0f0fu, hi = (qw[w] >> 4) & 0x0f0f0f0fu;
+              wf[r][4 * w] = cvt_ub0(lo); wf[r][4 * w + 1] = cvt_ub1(lo); wf[r][4 * w + 2] = cvt_ub2(lo); wf[r][4 * w + 3] = cvt_ub3(lo);
+              wf[r][16 + 4 * w] = cvt_ub0(hi); wf[r][16 + 4 * w + 1] = cvt_ub1(hi); wf[r][16 + 4 * w + 2] = cvt_ub2(hi); wf[r][16 + 4 * w + 3] = cvt_ub3(hi);
+            }
+            if (QT == CAI_Q4_K) {
+              uint32_t sc, mn; q4k_scale_pair(hdr[r].y, hdr[r].z, hdr[r].w, (u & 7) >> 1, sc, mn);
+              const float d = __half2float(__ushort_as_half((unsigned short)(hdr[r].x & 0xffffu)));
+              const float dmin = __half2float(__ushort_as_half((unsigned short)(hdr[r].x >> 16)));
+              s0[r] = d * cvt_ub0(sc); s1[r] = d * cvt_ub1(sc); m0[r] = dmin * cvt_ub0(mn); m1[r] = dmin * cvt_ub1(mn);
+            } else s0[r] = __half2float(__ushort_as_half(dh[r]));
+          }
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+          float xv[UW];
+          const float4* xb = xs4 + b * (p.kp >> 2);
+#pragma unroll
+          for (int t = 0; t < T; t++) {
+            const float4 v = xb[xb0 + t * 16];
+            xv[4 * t] = v.x; xv[4 * t + 1] = v.y; xv[4 * t + 2] = v.z; xv[4 * t + 3] = v.w;
+          }
+          if (QT == CAI_Q8_0) {
+#pragma unroll
+            for (int r = 0; r < RR; r++) {
+              float sq = 0.0f;
+#pragma unroll
+              for (int i = 0; i < 16; i++) sq = fmaf(wf[r][i], xv[i], sq);
+              acc[r][b] = fmaf(s0[r], sq, acc[r][b]);
+            }
+          } else if (QT == CAI_Q4_0) {
+            float sx = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 32; i++) sx += xv[i];
+#pragma unroll
+            for (int r = 0; r < RR; r++) {
+              float sq = 0.0f;
+#pragma unroll
+              for (int i = 0; i < 32; i++) sq = fmaf(wf[r][i], xv[i], sq);
+              acc[r][b] = fmaf(s0[r], sq - 8.0f * sx, acc[r][b]);
+            }
+          } else {
+            float sxlo = 0.0f, sxhi = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) { sxlo += xv[i]; sxhi += xv[16 + i]; }
+#pragma unroll
+            for (int r = 0; r < RR; r++) {
+              float slo = 0.0f, shi = 0.0f;
+#pragma unroll
+              for (int i = 0; i < 16; i++) { slo = fmaf(wf[r][i], xv[i], slo); shi = fmaf(wf[r][16 + i], xv[16 + i], shi); }
+              acc[r][b] += (s0[r] * slo + s1[r] * shi) - (m0[r] * sxlo + m1[r] * sxhi);
+            }
+          }
+        }
+      }
+    }
+  }
+
+  // ---- reduce across the wave and write ----
+#pragma unroll
+  for (int r = 0; r < RR; r++)
+#pragma unroll
+    for (int b = 0; b < NB; b++) acc[r][b] = wave_sum(acc[r][b]);
+
+  if (lane == 63) {
+    if (MODE == 0) {
+#pragma unroll
+      for (int r = 0; r < RR; r++) {
+        if (!live[r]) continue;
+        const int row = row_first + r;
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+          float v = acc[r][b];
+          if (sg.bias) v += sg.bias[bank_row + row];
+          v = act_apply(v, p.act);
+          const int64_t o = (int64_t)b * p.y_stride + sg.y_off + row;
+          if (p.residual) v += p.residual[o];
+          yout[o] = v;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        if (!live[2 * r]) continue;
+        const int row = row_first + r;
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+          float up = acc[2 * r][b], gate = acc[2 * r + 1][b];
+          if (sg.bias) { up += sg.bias[bank_row + row]; gate += sg.bias[bank_row + p.half + row]; }
+          yout[(int64_t)b * p.y_stride + sg.y_off + row] = silu_mul(up, gate);
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Simple kernel: F32 / F16 / I8ROW and any shape the fast kernel does not take.  One wave per row,
+// lanes stride the row with scalar loads (coalesced), fp32 accumulation.
+// ------------------------------------------------------------------------------------------
+template <int QT>
+__global__ __launch_bounds__(256) void gemv_simple(const GemvParams p, int n_b)
+{
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t grow = (int64_t)blockIdx.x * 4 + wave;
+  int s = 0; int64_t g0 = 0;
+  if (p.n_seg > 1 && grow >= p.seg[0].grp_end) { s = 1; g0 = p.seg[0].grp_end; }
+  if (p.n_seg > 2 && grow >= p.seg[1].grp_end) { s = 2; g0 = p.seg[1].grp_end; }
+  if (grow >= p.seg[p.n_seg - 1].grp_end) return;
+  const GemvSeg sg = p.seg[s];
+  const int row = (int)(grow - g0);
+  const int cols = p.cols;
+  int64_t bank_row = 0;
+  const float* xin = p.x; float* yout = p.y;
+  if (p.slot_expert) {
+    bank_row = (int64_t)p.slot_expert[blockIdx.y] * p.expert_rows;
+    xin += (int64_t)blockIdx.y * p.x_slot_stride; yout += (int64_t)blockIdx.y * p.y_slot_stride;
+  }
+  const int64_t wrow = bank_row + row;
+  for (int b = 0; b < n_b; b++) {
+    const float* xb = xin + (int64_t)b * cols;
+    float inv = 1.0f;
+    if (p.norm_gain) {
+      float ss = 0.0f;
+      for (int i = lane; i < cols; i += 64) ss = fmaf(xb[i], xb[i], ss);
+      ss = wave_sum(ss);
+      ss = __shfl(ss, 63);
+      inv = 1.0f / sqrtf(ss / (float)cols + p.norm_eps);
+    }
+    float acc = 0.0f;
+    for (int i = lane; i < cols; i += 64) {
+      float w;
+      if (QT == CAI_F32) w = reinterpret_cast<const float*>(sg.data)[wrow * cols + i];
+      else if (QT == CAI_F16) w = __half2float(reinterpret_cast<const __half*>(sg.data)[wrow * cols + i]);
+      else w = (float)reinterpret_cast<const int8_t*>(sg.data)[wrow * cols + i];
+      float xv = xb[i];
+      if (p.norm_gain) xv = p.norm_gain[i] * (xv * inv);
+      acc = fmaf(w, xv, acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 63) {
+      if (QT == CAI_I8ROW) acc *= reinterpret_cast<const float*>(sg.aux)[wrow];
+      if (sg.bias) acc += sg.bias[wrow];
+      acc = act_apply(acc, p.act);
+      const int64_t o = (int64_t)b * p.y_stride + sg.y_off + row;
+      if (p.residual) acc += p.residual[o];
+      yout[o] = acc;
+    }
+  }
+}
+
+// y[b][i] = x[b][i] * silu(x[b][half+i]) for the simple path (unfused SwiGLU)
+__global__ void swiglu_rows(const float* x, int half, int n_tokens, float* y)
+{
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)half * n_tokens) return;
+  const int t = (int)(i / half), d = (int)(i - (int64_t)t * half);
+  y[i] = silu_mul(x[(int64_t)t * 2 * half + d], x[(int64_t)t * 2 * half + half + d]);
+}
+
+static bool fast_type(int qt) { return qt == CAI_Q4_K || qt == CAI_Q4_0 || qt == CAI_Q8_0; }
+
+static int panel_len(int cols, int nb)
+{
+  int kp = 8192;
+  while ((int64_t)kp * nb * 4 > 65536) kp >>= 1;
+  const int cols256 = (cols + 255) / 256 * 256;
+  if (kp > cols256) kp = cols256;
+  return kp;
+}
+
+template <int QT, int NB, int MODE>
+static int launch_fast_r(const GemvParams& p, int n_groups_r, int R, int n_slots, hipStream_t st)
+{
+  const size_t lds = (size_t)NB * p.kp * 4;
+  const dim3 grid((n_groups_r + 3) / 4, n_slots);
+  if constexpr (NB == 1 && MODE == 0) {
+    if (R == 4) { hipLaunchKernelGGL((gemv_fast<QT, NB, 4, MODE>), grid, dim3(256), lds, st, p); return CAI_OK; }
+  }
+  if (R == 4) return set_error(CAI_ERR_INVALID, "gemv: 4 rows per wave only exists for batch 1 plain rows");
+  if (R == 2) hipLaunchKernelGGL((gemv_fast<QT, NB, 2, MODE>), grid, dim3(256), lds, st, p);
+  else hipLaunchKernelGGL((gemv_fast<QT, NB, 1, MODE>), grid, dim3(256), lds, st, p);
+  return CAI_OK;
+}
+
+// Rows per wave: enough groups to give every CU several waves, more rows per wave when the matrix is tall.
+static int pick_r(int64_t total_rows, int nb, int mode)
+{
+  if (nb > 1 || mode == 1) return total_rows >= 16384 ? 2 : 1;
+  if (total_rows >= 32768) return 4;
+  if (total_rows >= 8192) return 2;
+  return 1;
+}
+
+
+template <int QT, int MODE>
+static int launch_fast_nb(GemvParams& p, const MultiGemv& m, int nb, hipStream_t st)
+{
+  int64_t total = 0;
+  for (int i = 0; i < m.n; i++) total += m.rows[i];
+  const int ns = m.slot_expert ? m.n_slots : 1;
+  const int R = pick_r((MODE == 1 ? 2 * total : total) * ns, nb, MODE);
+  int cum = 0;
+  for (int i = 0; i < m.n; i++) {
+    cum += (int)((m.rows[i] + R - 1) / R);
+    p.seg[i].grp_end = cum;
+  }
+  switch (nb) {
+    case 1: return launch_fast_r<QT, 1, MODE>(p, cum, R, ns, st);
+    case 2: return launch_fast_r<QT, 2, MODE>(p, cum, R, ns, st);
+    case 3: return launch_fast_r<QT, 3, MODE>(p, cum, R, ns, st);
+    case 4: return launch_fast_r<QT, 4, MODE>(p, cum, R, ns, st);
+    case 5: return launch_fast_r<QT, 5, MODE>(p, cum, R, ns, st);
+    case 6: return launch_fast_r<QT, 6, MODE>(p, cum, R, ns, st);
+    case 7: return launch_fast_r<QT, 7, MODE>(p, cum, R, ns, st);
+    case 8: return launch_fast_r<QT, 8, MODE>(p, cum, R, ns, st);
+  }
+  return set_error(CAI_ERR_INVALID, "gemv: n_b %d out of range 1..8", nb);
+}
+
+static int64_t data_row_bytes(const cai_qw_s* w)
+{
+  switch (w->qtype) {
+    case CAI_Q4_K: return w->cols / 256 * 144;
+    case CAI_Q4_0: return w->cols / 2;
+    case CAI_Q8_0: case CAI_I8ROW: return w->cols;
+    case CAI_F32: return w->cols * 4;
+    case CAI_F16: return w->cols * 2;
+  }
+  return 0;
+}
+static int64_t aux_row_bytes(const cai_qw_s* w)
+{
+  if (w->qtype == CAI_Q4_0 || w->qtype == CAI_Q8_0) return w->cols / 32 * 2;
+  if (w->qtype == CAI_I8ROW) return 4;
+  return 0;
+}
+
+// Up to three matrices of one type and width share the staged activation (q|k|v in one launch).
+int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int64_t y_stride, int act,
+                      const float* residual, const float* norm_gain, float norm_eps, int swiglu_half)
+{
+  Context& c = ctx();
+  const cai_qw_s* w0 = m.w[0];
+  GemvParams p{};
+  p.n_seg = m.n; p.x = x; p.y = y; p.residual = residual; p.norm_gain = norm_gain; p.norm_eps = norm_eps;
+  p.cols = (int)w0->cols; p.y_stride = (int)y_stride; p.act = act; p.half = swiglu_half;
+  p.slot_expert = m.slot_expert; p.expert_rows = m.expert_rows; p.x_slot_stride = m.x_slot_stride; p.y_slot_stride = m.y_slot_stride;
+  const int n_slots = m.slot_expert ? m.n_slots : 1;
+  for (int i = 0; i < m.n; i++) {
+    const cai_qw_s* w = m.w[i];
+    if (w->qtype != w0->qtype || w->cols != w0->cols) return set_error(CAI_ERR_INVALID, "gemv: fused matrices differ in type or width");
+    if (m.row0[i] < 0 || m.rows[i] <= 0 || m.row0[i] + m.rows[i] > w->rows)
+      return set_error(CAI_ERR_INVALID, "gemv: row range [%lld,+%lld) outside matrix of %lld rows", (long long)m.row0[i], (long long)m.rows[i], (long long)w->rows);
+    p.seg[i].data = w->data + m.row0[i] * data_row_bytes(w);
+    p.seg[i].aux = w->aux ? w->aux + m.row0[i] * aux_row_bytes(w) : nullptr;
+    p.seg[i].bias = w->bias ? w->bias + m.row0[i] : nullptr;
+    p.seg[i].rows = (int)m.rows[i];
+    p.seg[i].y_off = m.y_off[i];
+  }
+  const int qt = w0->qtype;
+  if (fast_type(qt)) {
+    p.kp = panel_len(p.cols, n_b);
+    if (swiglu_half) {
+      if (m.n != 1) return set_error(CAI_ERR_INVALID, "gemv: swiglu takes one matrix");
+      p.seg[0].rows = swiglu_half;
+      MultiGemv mm = m; mm.rows[0] = swiglu_half;
+      if (qt == CAI_Q4_K) return launch_fast_nb<CAI_Q4_K, 1>(p, mm, n_b, c.stream);
+      if (qt == CAI_Q4_0) return launch_fast_nb<CAI_Q4_0, 1>(p, mm, n_b, c.stream);
+      return launch_fast_nb<CAI_Q8_0, 1>(p, mm, n_b, c.stream);
+    }
+    if (qt == CAI_Q4_K) return launch_fast_nb<CAI_Q4_K, 0>(p, m, n_b, c.stream);
+    if (qt == CAI_Q4_0) return launch_fast_nb<CAI_Q4_0, 0>(p, m, n_b, c.stream);
+    return launch_fast_nb<CAI_Q8_0, 0>(p, m, n_b, c.stream);
+  }
+  if (swiglu_half) return set_error(CAI_ERR_UNSUPPORTED, "gemv: fused swiglu needs a block-quantized matrix");
+  int64_t cum = 0;
+  for (int i = 0; i < m.n; i++) { cum += m.rows[i]; p.seg[i].grp_end = (int)cum; }
+  const dim3 grid((unsigned)((cum + 3) / 4), n_slots);
+  if (qt == CAI_F32) hipLaunchKernelGGL(gemv_simple<CAI_F32>, grid, dim3(256), 0, c.stream, p, n_b);
+  else if (qt == CAI_F16) hipLaunchKernelGGL(gemv_simple<CAI_F16>, grid, dim3(256), 0, c.stream, p, n_b);
+  else if (qt == CAI_I8ROW) hipLaunchKernelGGL(gemv_simple<CAI_I8ROW>, grid, dim3(256), 0, c.stream, p, n_b);
+  else return set_error(CAI_ERR_UNSUPPORTED, "gemv: weight type %d", qt);
+  return CAI_OK;
+}
+
+int launch_gemv(const cai_qw_s* w, int64_t row0, int64_t n_rows, const float* x, int n_b, float* y,
+                int64_t y_stride, int act, const float* residual)
+{
+  MultiGemv m{}; m.n = 1; m.w[0] = w; m.row0[0] = row0; m.rows[0] = n_rows; m.y_off[0] = 0;
+  return launch_gemv_multi(m, x, n_b, y, y_stride, act, residual, nullptr, 0.0f, 0);
+}
+
+int launch_swiglu(const float* x, int half, int n_tokens, float* y)
+{
+  const int64_t n = (int64_t)half * n_tokens;
+  hipLaunchKernelGGL(swiglu_rows, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx().stream, x, half, n_tokens, y);
+  return CAI_OK;
+}
+
+}  // namespace cai

@@ -1,0 +1,130 @@
+// Internal declarations shared by the caihip translation units (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string>
+#include <vector>
+
+#include "../../include/caihip.h"
+
+namespace cai {
+
+struct Context {
+  bool        ready = false;
+  int         device = 0;
+  hipStream_t stream = nullptr;
+  hipEvent_t  ev0 = nullptr, ev1 = nullptr;
+  int         n_cu = 256;
+  char        name[128] = {0};
+  // scratch used by calls that take host pointers (grown on demand)
+  void*  stage_in = nullptr;  size_t stage_in_cap = 0;
+  void*  stage_out = nullptr; size_t stage_out_cap = 0;
+  int32_t* d_small = nullptr;            // 1024 ints of device scratch for small arguments/results
+  int32_t* h_small = nullptr;            // 1024 ints of pinned host memory paired with d_small
+};
+
+Context& ctx();
+int  set_error(int code, const char* fmt, ...);
+int  hip_fail(hipError_t e, const char* what, const char* file, int line);
+int  ensure_stage(void** p, size_t* cap, size_t need);
+
+#define CAI_HIP(call)                                                        \
+  do {                                                                       \
+    hipError_t e__ = (call);                                                 \
+    if (e__ != hipSuccess) return cai::hip_fail(e__, #call, __FILE__, __LINE__); \
+  } while (0)
+
+#define CAI_REQUIRE(cond, ...)                                               \
+  do {                                                                       \
+    if (!(cond)) return cai::set_error(CAI_ERR_INVALID, __VA_ARGS__);        \
+  } while (0)
+
+#define CAI_READY()                                                          \
+  do {                                                                       \
+    if (!cai::ctx().ready) return cai::set_error(CAI_ERR_STATE, "cai_init has not been called"); \
+  } while (0)
+
+// ---------------------------------------------------------------------------------------------
+// Resident weight matrix.  Device layouts (the on-disk block format stays the contract; these are
+// the library's own):
+//   Q4_K : the 144-byte super-blocks as stored (16-byte aligned rows).
+//   Q8_0 : two planes - qs[rows][cols] int8 (32 B per block, 16-byte aligned) and d[rows][cols/32] half.
+//   Q4_0 : two planes - qs[rows][cols/2] bytes (16 B per block) and d[rows][cols/32] half.
+//   F32/F16 : as stored.   I8ROW : codes[rows][cols] + scales[rows].
+// ---------------------------------------------------------------------------------------------
+}  // namespace cai
+
+struct cai_qw_s {
+  int      qtype = 0;
+  int64_t  rows = 0, cols = 0;
+  uint8_t* data = nullptr;     // quants plane or the raw blocks
+  uint8_t* aux = nullptr;      // half scales plane (Q8_0/Q4_0) or float row scales (I8ROW)
+  float*   bias = nullptr;
+  int64_t  data_bytes = 0, aux_bytes = 0;
+  int64_t  algo_bytes = 0;     // bytes of the GGUF form (+bias): what one GEMV must stream
+};
+
+struct cai_kv_s {
+  int n_seq = 1, n_layers = 0, kv_heads = 0, head_dim = 0, max_ctx = 0, dtype = 0;
+  void* k = nullptr; void* v = nullptr;   // [seq][layer][kv_head][max_ctx][head_dim]
+  std::vector<int> len;                   // [seq][layer] live rows (host mirror)
+  int split_len = 64, n_splits = 1;       // split-K geometry of the decode kernel (fixed at creation)
+  float* part = nullptr;                  // [seq][q_head][split][head_dim+2] split-K partials
+  int part_q_heads = 0;
+  int32_t* d_len = nullptr;               // [seq] device scratch: rows live BEFORE the token being decoded
+  size_t elem() const { return dtype == CAI_KV_F16 ? 2 : 4; }
+  int64_t layer_elems() const { return (int64_t)kv_heads * max_ctx * head_dim; }
+  int64_t seq_elems() const { return layer_elems() * n_layers; }
+  int& len_at(int seq, int layer) { return len[(size_t)seq * n_layers + layer]; }
+};
+
+struct cai_kv_snap_s {
+  int n_layers = 0, kv_heads = 0, head_dim = 0, dtype = 0, rows = 0;
+  std::vector<int> len;                   // per layer
+  void* k = nullptr; void* v = nullptr;   // [layer][kv_head][rows][head_dim]
+};
+
+namespace cai {
+
+// ---- launchers (all enqueue on ctx().stream; pointers are device pointers) ----
+int launch_gemv(const cai_qw_s* w, int64_t row0, int64_t n_rows, const float* x, int n_b, float* y,
+                int64_t y_stride, int act, const float* residual);
+// Up to three matrices of one type and width sharing the staged activation (q|k|v in one launch); or, with
+// slot_expert set, n_slots row windows of one expert bank (window e = rows [e*expert_rows, +rows[0]) ), slot j
+// reading x + j*x_slot_stride and writing y + j*y_slot_stride.
+struct MultiGemv {
+  const cai_qw_s* w[3]; int64_t row0[3]; int64_t rows[3]; int y_off[3]; int n;
+  const int32_t* slot_expert; int n_slots; int64_t expert_rows; int x_slot_stride; int y_slot_stride;
+};
+// norm_gain != null fuses RMSNorm(eps) of x into the staging; swiglu_half > 0 computes
+// y[i] = up_i * silu(gate_i) from rows i and swiglu_half + i of the (single) matrix.
+int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int64_t y_stride, int act,
+                      const float* residual, const float* norm_gain, float norm_eps, int swiglu_half);
+int launch_dequant_rows(const cai_qw_s* w, int64_t row0, int64_t n_rows, float* out);
+int launch_rmsnorm(const float* x, const float* gain, int n, int n_tokens, float eps, float* y);
+int launch_rope(float* x, int n_heads, int head_dim, const int32_t* pos_dev, int pos_host, const float* theta, int n_tokens, int64_t token_stride);
+int launch_swiglu(const float* x, int half, int n_tokens, float* y);
+int launch_add(float* x, const float* y, int64_t n);
+int launch_argmax(const float* x, int n, int n_rows, int32_t* out);
+int launch_embed(const cai_qw_s* w, const int32_t* tokens_dev, int n_tokens, float* out);
+int launch_router_topk(const float* logits, int n, int k, int renorm, int n_tokens, int32_t* expert_out, float* gate_out, float* probs_scratch);
+int launch_rmsnorm_strided(const float* x, const float* gain, int n, int n_tokens, float eps, float* y, int64_t x_stride, int64_t y_stride);
+int launch_moe_combine(float* x, const float* part, const float* gate, int k, int n, int n_tokens);
+int launch_split_blocks(const uint8_t* raw, int block_bytes, int64_t n_blocks, uint8_t* qs, uint16_t* d);
+// qkv: [n_seq][qkv_stride] rows [Q|K|V]; theta != null applies interleaved RoPE to Q and K first.  pos_dev[s] is
+// both the rotary position and the cache slot the new K,V row goes to; the live range is [.., pos_dev[s]].
+// Activation row s uses cache sequence seq0 + s.
+int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, int n_seq, int q_heads, int window,
+                     float softcap, const float* theta, const int32_t* pos_dev, float* out, int64_t out_stride, int seq0);
+int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, int max_ctx, int dtype);
+void kv_free(cai_kv_s* kv);
+int kv_snapshot(cai_kv_s* kv, int seq, cai_kv_snap_s** out);
+int kv_restore(cai_kv_s* kv, int seq, const cai_kv_snap_s* snap);
+int launch_gemm_mfma(const cai_qw_s* w, const float* x, int n_tokens, float* y, const float* residual);
+
+void rope_thetas(float base, int head_dim, std::vector<float>& out);
+
+}  // namespace cai

@@ -1,0 +1,375 @@
+// Elementwise layer math, block dequantization, embedding gather, arg-max and the MoE router for gfx950.
+#include "cai_internal.hpp"
+#include <string.h>
+#include <math.h>
+
+namespace cai {
+
+__device__ __forceinline__ float wave_sum_all(float v)
+{
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x112, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x114, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x118, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xa, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xc, 0xf, true));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// ------------------------------------------------------------------------------------------
+// Element (row, i) of a resident matrix, bit-exact to DecodeGGMLSpan (neural/neuralgguf.pas:1471-1523).
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ float f16_bits_to_float(uint16_t h) { return __half2float(__ushort_as_half(h)); }
+
+__device__ float dequant_elem(int qtype, const uint8_t* data, const uint8_t* aux, int64_t cols, int64_t row, int64_t i)
+{
+  switch (qtype) {
+    case CAI_F32: return reinterpret_cast<const float*>(data)[row * cols + i];
+    case CAI_F16: return f16_bits_to_float(reinterpret_cast<const uint16_t*>(data)[row * cols + i]);
+    case CAI_I8ROW:  // code * Scales[row] (neural/neural.cl:1447-1470)
+      return (float)reinterpret_cast<const int8_t*>(data)[row * cols + i] * reinterpret_cast<const float*>(aux)[row];
+    case CAI_Q8_0: {  // x = d * q (neural/neuralgguf.pas:1487-1503)
+      const float d = f16_bits_to_float(reinterpret_cast<const uint16_t*>(aux)[row * (cols >> 5) + (i >> 5)]);
+      return d * (float)reinterpret_cast<const int8_t*>(data)[row * cols + i];
+    }
+    case CAI_Q4_0: {  // x = d * (nibble - 8); e<16 low nibble of byte e, else high nibble of byte e-16 (neuralgguf.pas:811-845)
+      const int64_t blk = i >> 5; const int e = (int)(i & 31);
+      const float d = f16_bits_to_float(reinterpret_cast<const uint16_t*>(aux)[row * (cols >> 5) + blk]);
+      const uint8_t b = data[row * (cols >> 1) + blk * 16 + (e & 15)];
+      const int nib = e < 16 ? (b & 15) : (b >> 4);
+      return d * (float)(nib - 8);
+    }
+    case CAI_Q4_K: {  // x = (d*sc)*q - dmin*mn (neural/neuralgguf.pas:448-514)
+      const uint8_t* blk = data + (row * (cols >> 8) + (i >> 8)) * 144;
+      const int e = (int)(i & 255), c = e >> 6, hi = (e >> 5) & 1, idx = e & 31, j = 2 * c + hi;
+      const float d = f16_bits_to_float(*reinterpret_cast<const uint16_t*>(blk));
+      const float dmin = f16_bits_to_float(*reinterpret_cast<const uint16_t*>(blk + 2));
+      const uint8_t* s = blk + 4;
+      int sc, mn;
+      if (j < 4) { sc = s[j] & 63; mn = s[j + 4] & 63; }
+      else { sc = (s[j + 4] & 15) | ((s[j - 4] >> 2) & 0x30); mn = (s[j + 4] >> 4) | ((s[j] >> 2) & 0x30); }
+      const uint8_t b = blk[16 + 32 * c + idx];
+      const int q = hi ? (b >> 4) : (b & 15);
+      const float dsc = d * (float)sc, dm = dmin * (float)mn;
+      return dsc * (float)q - dm;
+    }
+  }
+  return 0.0f;
+}
+
+__global__ void dequant_rows_kernel(int qtype, const uint8_t* data, const uint8_t* aux, int64_t cols, int64_t row0, int64_t n, float* out)
+{
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  out[idx] = dequant_elem(qtype, data, aux, cols, row0 + idx / cols, idx % cols);
+}
+
+int launch_dequant_rows(const cai_qw_s* w, int64_t row0, int64_t n_rows, float* out)
+{
+  const int64_t n = n_rows * w->cols;
+  hipLaunchKernelGGL(dequant_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx().stream,
+                     w->qtype, w->data, w->aux, w->cols, row0, n, out);
+  return CAI_OK;
+}
+
+// Embedding gather (TNNetEmbedding; neural/neural.cl:1422-1470): Y[t] = W[token_t], dequantized.
+__global__ void embed_kernel(int qtype, const uint8_t* data, const uint8_t* aux, int64_t cols, const int32_t* tokens, float* out)
+{
+  const int t = blockIdx.y;
+  const int64_t row = tokens[t];
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < cols; i += (int64_t)gridDim.x * blockDim.x)
+    out[(int64_t)t * cols + i] = dequant_elem(qtype, data, aux, cols, row, i);
+}
+
+int launch_embed(const cai_qw_s* w, const int32_t* tokens_dev, int n_tokens, float* out)
+{
+  const int bx = (int)std::min<int64_t>((w->cols + 255) / 256, 64);
+  hipLaunchKernelGGL(embed_kernel, dim3(bx, n_tokens), dim3(256), 0, ctx().stream, w->qtype, w->data, w->aux, w->cols, tokens_dev, out);
+  return CAI_OK;
+}
+
+// ---- GGUF block stream -> planes (Q8_0: 34-byte blocks, Q4_0: 18-byte blocks; neural/neuralgguf.pas:100-131) ----
+__global__ void split_blocks_kernel(const uint8_t* raw, int block_bytes, int64_t n_blocks, uint8_t* qs, uint16_t* d)
+{
+  const int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= n_blocks) return;
+  const uint8_t* src = raw + b * block_bytes;
+  d[b] = (uint16_t)(src[0] | (src[1] << 8));
+  const int qb = block_bytes - 2;
+  // 2-byte aligned source (block sizes are even): move halfwords
+  const uint16_t* s16 = reinterpret_cast<const uint16_t*>(src + 2);
+  uint16_t* d16 = reinterpret_cast<uint16_t*>(qs + b * qb);
+  for (int i = 0; i < qb / 2; i++) d16[i] = s16[i];
+}
+
+int launch_split_blocks(const uint8_t* raw, int block_bytes, int64_t n_blocks, uint8_t* qs, uint16_t* d)
+{
+  hipLaunchKernelGGL(split_blocks_kernel, dim3((unsigned)((n_blocks + 255) / 256)), dim3(256), 0, ctx().stream, raw, block_bytes, n_blocks, qs, d);
+  return CAI_OK;
+}
+
+// ---- TNNetTokenRMSNorm (neural/neural.cl:1047-1085): y = g * (x * rsqrt(mean(x^2) + eps)) ----
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* x, const float* gain, int n, float eps, float* y, int64_t x_stride, int64_t y_stride)
+{
+  const float* xr = x + (int64_t)blockIdx.x * x_stride;
+  float* yr = y + (int64_t)blockIdx.x * y_stride;
+  __shared__ float red[4];
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < n; i += 256) ss = fmaf(xr[i], xr[i], ss);
+  ss = wave_sum_all(ss);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float tot = (red[0] + red[1]) + (red[2] + red[3]);
+  const float inv = 1.0f / sqrtf(tot / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += 256) yr[i] = gain[i] * (xr[i] * inv);
+}
+
+int launch_rmsnorm_strided(const float* x, const float* gain, int n, int n_tokens, float eps, float* y, int64_t x_stride, int64_t y_stride)
+{
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3(n_tokens), dim3(256), 0, ctx().stream, x, gain, n, eps, y, x_stride, y_stride);
+  return CAI_OK;
+}
+int launch_rmsnorm(const float* x, const float* gain, int n, int n_tokens, float eps, float* y)
+{
+  return launch_rmsnorm_strided(x, gain, n, n_tokens, eps, y, n, n);
+}
+
+// ---- TNNetRotaryEmbedding (neural/neural.cl:1517-1542), interleaved pairs, head-tiled theta ----
+__global__ void rope_kernel(float* x, int n_heads, int head_dim, const int32_t* pos, const float* theta, int64_t token_stride)
+{
+  const int t = blockIdx.y;
+  const int half = head_dim >> 1;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_heads * half) return;
+  const int k = i % half;
+  const float angle = (float)pos[t] * theta[k];
+  float s, c; sincosf(angle, &s, &c);
+  float* p = x + (int64_t)t * token_stride + (i / half) * head_dim + 2 * k;
+  const float x0 = p[0], x1 = p[1];
+  p[0] = c * x0 - s * x1;
+  p[1] = s * x0 + c * x1;
+}
+
+int launch_rope(float* x, int n_heads, int head_dim, const int32_t* pos_dev, int, const float* theta, int n_tokens, int64_t token_stride)
+{
+  const int n = n_heads * (head_dim >> 1);
+  hipLaunchKernelGGL(rope_kernel, dim3((n + 255) / 256, n_tokens), dim3(256), 0, ctx().stream, x, n_heads, head_dim, pos_dev, theta, token_stride);
+  return CAI_OK;
+}
+
+// Host-side frequency table (neural/neural.cl:1510-1515): theta_k = base^(-2k/head_dim) in double, rounded once.
+void rope_thetas(float base, int head_dim, std::vector<float>& out)
+{
+  out.resize(head_dim / 2);
+  for (int k = 0; k < head_dim / 2; k++) out[k] = (float)pow((double)base, -2.0 * k / head_dim);
+}
+
+__global__ void add_kernel(float* x, const float* y, int64_t n)
+{
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] += y[i];
+}
+int launch_add(float* x, const float* y, int64_t n)
+{
+  hipLaunchKernelGGL(add_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx().stream, x, y, n);
+  return CAI_OK;
+}
+
+// x[t][i] += sum_j gate[t][j] * part[t][j][i]   (gate-weighted expert mixture, neural/neural.cl:2738-2751)
+__global__ void moe_combine_kernel(float* x, const float* part, const float* gate, int k, int n)
+{
+  const int t = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float acc = 0.0f;
+  for (int j = 0; j < k; j++) acc = fmaf(gate[t * k + j], part[((int64_t)t * k + j) * n + i], acc);
+  x[(int64_t)t * n + i] += acc;
+}
+int launch_moe_combine(float* x, const float* part, const float* gate, int k, int n, int n_tokens)
+{
+  hipLaunchKernelGGL(moe_combine_kernel, dim3((n + 255) / 256, n_tokens), dim3(256), 0, ctx().stream, x, part, gate, k, n);
+  return CAI_OK;
+}
+
+// ---- ArgMaxRow (neural/neuralchatengine.pas:683-697): strict >, lowest index wins ties ----
+__global__ __launch_bounds__(1024) void argmax_kernel(const float* x, int n, int32_t* out)
+{
+  const float* xr = x + (int64_t)blockIdx.x * n;
+  float best = -INFINITY; int bi = 0x7fffffff;
+  for (int i = threadIdx.x; i < n; i += 1024) {
+    const float v = xr[i];
+    if (bi == 0x7fffffff || v > best) { best = v; bi = i; }   // indices rise per thread: ties keep the earlier one
+  }
+  __shared__ float sv[1024]; __shared__ int si[1024];
+  sv[threadIdx.x] = best; si[threadIdx.x] = bi;
+  __syncthreads();
+  for (int s = 512; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s) {
+      const float ov = sv[threadIdx.x + s]; const int oi = si[threadIdx.x + s];
+      if (oi != 0x7fffffff && (si[threadIdx.x] == 0x7fffffff || ov > sv[threadIdx.x] || (ov == sv[threadIdx.x] && oi < si[threadIdx.x]))) {
+        sv[threadIdx.x] = ov; si[threadIdx.x] = oi;
+      }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = si[0] == 0x7fffffff ? 0 : si[0];
+}
+
+int launch_argmax(const float* x, int n, int n_rows, int32_t* out)
+{
+  hipLaunchKernelGGL(argmax_kernel, dim3(n_rows), dim3(1024), 0, ctx().stream, x, n, out);
+  return CAI_OK;
+}
+
+// ---- router: TNNetPointwiseSoftMax (neural/neural.cl:1594-1647) + TNNetTopKGate ----
+// One thread per token, the way the reference keeps a group's reduction inside one work-item.
+__global__ void router_topk_kernel(const float* logits, int n, int k, int renorm, int n_tokens, int32_t* expert_out, float* gate_out, float* probs)
+{
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n_tokens) return;
+  const float* x = logits + (int64_t)t * n;
+  float* p = probs + (int64_t)t * n;
+  float mx = x[0];
+  for (int c = 1; c < n; c++) mx = fmaxf(mx, x[c]);
+  float tot = 0.0f;
+  for (int c = 0; c < n; c++) {
+    float a = x[c] - mx; a = a > 4000.0f ? 4000.0f : (a < -4000.0f ? -4000.0f : a);
+    const float e = expf(a); p[c] = e; tot += e;
+  }
+  if (tot > 0.0f) { const float inv = 1.0f / tot; for (int c = 0; c < n; c++) p[c] *= inv; }
+  float sum = 0.0f;
+  for (int j = 0; j < k; j++) {
+    int best = -1; float bv = 0.0f;
+    for (int c = 0; c < n; c++) {
+      const float v = p[c];
+      if (v >= 0.0f && (best < 0 || v > bv)) { best = c; bv = v; }
+    }
+    expert_out[t * k + j] = best; gate_out[t * k + j] = bv; sum += bv;
+    p[best] = -1.0f;   // taken
+  }
+  if (renorm) { const float inv = sum > 0.0f ? 1.0f / sum : 0.0f; for (int j = 0; j < k; j++) gate_out[t * k + j] *= inv; }
+}
+
+int launch_router_topk(const float* logits, int n, int k, int renorm, int n_tokens, int32_t* expert_out, float* gate_out, float* probs_scratch)
+{
+  hipLaunchKernelGGL(router_topk_kernel, dim3((n_tokens + 63) / 64), dim3(64), 0, ctx().stream, logits, n, k, renorm, n_tokens, expert_out, gate_out, probs_scratch);
+  return CAI_OK;
+}
+
+}  // namespace cai
+
+// ------------------------------------------------------------------------------------------
+// C ABI: standalone layer ops
+// ------------------------------------------------------------------------------------------
+using namespace cai;
+
+namespace {
+// Stages a host input on the device when needed; returns the device pointer to use.
+int stage_input(const void* p, size_t bytes, int is_dev, const void** dev)
+{
+  Context& c = ctx();
+  if (is_dev) { *dev = p; return CAI_OK; }
+  const int rc = ensure_stage(&c.stage_in, &c.stage_in_cap, bytes); if (rc) return rc;
+  CAI_HIP(hipMemcpyAsync(c.stage_in, p, bytes, hipMemcpyHostToDevice, c.stream));
+  *dev = c.stage_in;
+  return CAI_OK;
+}
+int stage_output(void* p, size_t bytes, int is_dev, void** dev)
+{
+  Context& c = ctx();
+  if (is_dev) { *dev = p; return CAI_OK; }
+  const int rc = ensure_stage(&c.stage_out, &c.stage_out_cap, bytes); if (rc) return rc;
+  *dev = c.stage_out;
+  return CAI_OK;
+}
+int finish_output(void* host, const void* dev, size_t bytes, int is_dev)
+{
+  Context& c = ctx();
+  if (!is_dev) CAI_HIP(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, c.stream));
+  CAI_HIP(hipStreamSynchronize(c.stream));
+  return CAI_OK;
+}
+}  // namespace
+
+extern "C" int cai_rmsnorm(const float* x, const float* gain_host, int n, int n_tokens, float eps, float* y, int flags)
+{
+  CAI_READY();
+  CAI_REQUIRE(x && gain_host && y && n > 0 && n_tokens > 0, "cai_rmsnorm: bad argument");
+  Context& c = ctx();
+  const size_t bytes = (size_t)n * n_tokens * 4;
+  float* d_gain = nullptr;
+  CAI_HIP(hipMalloc(&d_gain, (size_t)n * 4));
+  CAI_HIP(hipMemcpyAsync(d_gain, gain_host, (size_t)n * 4, hipMemcpyHostToDevice, c.stream));
+  const void* dx; void* dy; int rc;
+  if ((rc = stage_input(x, bytes, flags & CAI_X_DEVICE, &dx))) { (void)hipFree(d_gain); return rc; }
+  if ((rc = stage_output(y, bytes, flags & CAI_Y_DEVICE, &dy))) { (void)hipFree(d_gain); return rc; }
+  launch_rmsnorm((const float*)dx, d_gain, n, n_tokens, eps, (float*)dy);
+  rc = finish_output(y, dy, bytes, flags & CAI_Y_DEVICE);
+  (void)hipFree(d_gain);
+  return rc;
+}
+
+extern "C" int cai_rope(float* x, int n_heads, int head_dim, int pos, float theta_base, int flags)
+{
+  CAI_READY();
+  CAI_REQUIRE(x && n_heads > 0 && head_dim >= 2 && !(head_dim & 1) && head_dim <= 512, "cai_rope: bad argument");
+  Context& c = ctx();
+  std::vector<float> th; rope_thetas(theta_base, head_dim, th);
+  float* d_th = reinterpret_cast<float*>(c.d_small + 16);
+  static_assert(sizeof(float) == sizeof(int32_t), "");
+  c.h_small[0] = pos;
+  memcpy(c.h_small + 16, th.data(), th.size() * 4);   // h_small/d_small hold 16 ints + 256 floats
+  CAI_HIP(hipMemcpyAsync(c.d_small, c.h_small, (16 + th.size()) * 4, hipMemcpyHostToDevice, c.stream));
+  const size_t bytes = (size_t)n_heads * head_dim * 4;
+  const int dev = (flags & (CAI_X_DEVICE | CAI_Y_DEVICE)) != 0;
+  float* dx = x;
+  if (!dev) {
+    const int rc = ensure_stage(&c.stage_in, &c.stage_in_cap, bytes); if (rc) return rc;
+    CAI_HIP(hipMemcpyAsync(c.stage_in, x, bytes, hipMemcpyHostToDevice, c.stream));
+    dx = (float*)c.stage_in;
+  }
+  launch_rope(dx, n_heads, head_dim, c.d_small, 0, d_th, 1, 0);
+  return finish_output(x, dx, bytes, dev);
+}
+
+extern "C" int cai_swiglu(const float* x, int half, int n_tokens, float* y, int flags)
+{
+  CAI_READY();
+  CAI_REQUIRE(x && y && half > 0 && n_tokens > 0, "cai_swiglu: bad argument");
+  const size_t ob = (size_t)half * n_tokens * 4;
+  const void* dx; void* dy; int rc;
+  if ((rc = stage_input(x, 2 * ob, flags & CAI_X_DEVICE, &dx))) return rc;
+  if ((rc = stage_output(y, ob, flags & CAI_Y_DEVICE, &dy))) return rc;
+  launch_swiglu((const float*)dx, half, n_tokens, (float*)dy);
+  return finish_output(y, dy, ob, flags & CAI_Y_DEVICE);
+}
+
+extern "C" int cai_argmax(const float* x, int n, int32_t* index_out, int flags)
+{
+  CAI_READY();
+  CAI_REQUIRE(x && index_out && n > 0, "cai_argmax: bad argument");
+  Context& c = ctx();
+  const void* dx; int rc;
+  if ((rc = stage_input(x, (size_t)n * 4, flags & CAI_X_DEVICE, &dx))) return rc;
+  launch_argmax((const float*)dx, n, 1, c.d_small);
+  CAI_HIP(hipMemcpyAsync(c.h_small, c.d_small, 4, hipMemcpyDeviceToHost, c.stream));
+  CAI_HIP(hipStreamSynchronize(c.stream));
+  *index_out = c.h_small[0];
+  return CAI_OK;
+}
+
+extern "C" int cai_router_topk(const float* logits, int n, int k, int renorm, int32_t* expert_out, float* gate_out, int flags)
+{
+  CAI_READY();
+  CAI_REQUIRE(logits && expert_out && gate_out && n > 0 && k > 0 && k <= n && k <= 64, "cai_router_topk: bad argument");
+  Context& c = ctx();
+  const void* dx; void* dscr; int rc;
+  if ((rc = stage_input(logits, (size_t)n * 4, flags & CAI_X_DEVICE, &dx))) return rc;
+  if ((rc = stage_output(nullptr, (size_t)n * 4, 0, &dscr))) return rc;
+  int32_t* d_e = c.d_small; float* d_g = reinterpret_cast<float*>(c.d_small + 64);
+  launch_router_topk((const float*)dx, n, k, renorm, 1, d_e, d_g, (float*)dscr);
+  CAI_HIP(hipMemcpyAsync(c.h_small, c.d_small, 128 * 4, hipMemcpyDeviceToHost, c.stream));
+  CAI_HIP(hipStreamSynchronize(c.stream));
+  for (int j = 0; j < k; j++) { expert_out[j] = c.h_small[j]; memcpy(&gate_out[j], &c.h_small[64 + j], 4); }
+  return CAI_OK;
+}

@@ -1,0 +1,28 @@
+"""Loads the product library for the GPU tests (through its C ABI only)."""
+import importlib
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+pkg = importlib.import_module("neural-api_amd")
+cai = importlib.import_module("neural-api_amd.caihip")
+_inited = False
+
+
+def dev():
+    """Returns the ctypes view after cai_init(0); raises if the HIP library is missing or no GPU is present."""
+    global _inited
+    if not _inited:
+        cai.init(0)
+        _inited = True
+    return cai
+
+
+def rel_err(got, want):
+    """max |got - want| / max |want| : the logit tolerance metric (bar: <= 1e-3)."""
+    import numpy as np
+    denom = max(float(np.max(np.abs(want))), 1e-30)
+    return float(np.max(np.abs(np.asarray(got, np.float64) - np.asarray(want, np.float64)))) / denom

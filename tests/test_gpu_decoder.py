@@ -1,0 +1,152 @@
+"""Step-resident decoder on the device: reference-held logits, oracle parity on quantized synthetic models,
+greedy-token identity, session management.  All calls go through the C ABI."""
+import numpy as np
+import pytest
+
+from helpers import oracle_lib as O
+from helpers.device_model import run_sequences_device
+from helpers.fixtures_io import load_json, ref_path
+from helpers.model_build import oracle_model, spec_from_gguf_llama, spec_from_ref_fixture, synthetic_spec
+
+pytestmark = pytest.mark.gpu
+FAMILIES = ["tiny_llama", "tiny_smollm2", "tiny_qwen2", "tiny_mistral", "tiny_olmoe"]
+
+
+@pytest.mark.parametrize("name", FAMILIES)
+def test_device_decoder_matches_reference_logits(name):
+    # the reference's own gate (tests/TestNeuralPretrained.pas:5739-5743): max |diff| < 1e-4
+    from helpers.device import dev
+    cai = dev()
+    ref = load_json(name + "_logits.json")
+    dec = cai.Decoder(spec_from_ref_fixture(name, O.F32, max_ctx=32))
+    got = run_sequences_device(dec, ref["sequences"])
+    assert np.max(np.abs(got - np.array(ref["logits"], np.float32))) < 1e-4
+
+
+def test_device_gguf_imports_match():
+    from helpers.device import dev, rel_err
+    cai = dev()
+    ref = load_json("tiny_llama_logits.json")
+    dec = cai.Decoder(spec_from_gguf_llama(ref_path("tiny_llama_f32.gguf"), max_ctx=32))
+    got = run_sequences_device(dec, ref["sequences"])
+    assert np.max(np.abs(got - np.array(ref["logits"], np.float32))) < 1e-4
+    # Q8_0 GGUF (hidden 32): device == oracle on the same blocks, tightly
+    spec = spec_from_gguf_llama(ref_path("tiny_llama_q8.gguf"), max_ctx=32)
+    seq = [1, 5, 2, 7, 3, 0, 6, 4, 1, 1]
+    om = oracle_model(spec, acc64=1)
+    want = np.array([om.step(t, p)[1] for p, t in enumerate(seq)])
+    got = run_sequences_device(cai.Decoder(spec), [seq])[0]
+    assert rel_err(got, want) < 1e-5
+
+
+SHAPES = {
+    # scaled-down twins of the BASELINE shapes (same head grouping / bias / MoE structure)
+    "qwen7b_like_q4k": dict(cfg=dict(n_layers=3, d_model=512, n_q_heads=14, n_kv_heads=2, head_dim=128, ffn=1024, vocab=2048, max_ctx=128,
+                                     eps=1e-6, rope_theta=1e6), qtype=O.Q4_K, head=O.Q8_0, bias=True),
+    "smollm_like_q8": dict(cfg=dict(n_layers=3, d_model=576, n_q_heads=9, n_kv_heads=3, head_dim=64, ffn=1536, vocab=3000, max_ctx=160,
+                                    eps=1e-5, rope_theta=1e4, tied=True), qtype=O.Q8_0, head=None, bias=False),
+    "llama_like_q4_0": dict(cfg=dict(n_layers=2, d_model=256, n_q_heads=4, n_kv_heads=4, head_dim=64, ffn=512, vocab=1000, max_ctx=96,
+                                     eps=1e-5, rope_theta=1e4), qtype=O.Q4_0, head=None, bias=False),
+    "olmoe_like_q8": dict(cfg=dict(n_layers=2, d_model=256, n_q_heads=4, n_kv_heads=4, head_dim=64, ffn=128, vocab=1500, max_ctx=96,
+                                   eps=1e-5, rope_theta=1e4, n_experts=16, top_k=4, norm_topk=0, qk_norm_full=1), qtype=O.Q8_0, head=None, bias=False),
+}
+
+
+@pytest.mark.parametrize("name", list(SHAPES))
+def test_quantized_decoder_logits_and_greedy_tokens(name):
+    """Logits within 1e-3 relative of the oracle and the greedy token sequence identical for 64 tokens."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    s = SHAPES[name]
+    spec = synthetic_spec(s["cfg"], s["qtype"], head_qtype=s["head"], qkv_bias=s["bias"], std=0.05)
+    rng = np.random.default_rng(424242)
+    prompt = rng.integers(0, spec["cfg"]["vocab"], 16).tolist()
+    om = oracle_model(spec, acc64=1)
+    dec = cai.Decoder(spec)
+    worst = 0.0
+    tok_o, tok_d = None, None
+    for p, t in enumerate(prompt):
+        tok_o, lo = om.step(t, p); am, ld = dec.step(t, p); tok_d = int(am[0])
+        worst = max(worst, rel_err(ld[0], lo))
+    assert worst < 1e-3
+    seq_o, seq_d = [], []
+    for i in range(64):
+        p = len(prompt) + i
+        seq_o.append(tok_o); seq_d.append(tok_d)
+        n_o, lo = om.step(tok_o, p); am, ld = dec.step(tok_d, p)
+        if tok_o == tok_d:
+            worst = max(worst, rel_err(ld[0], lo))
+        tok_o, tok_d = n_o, int(am[0])
+    assert seq_o == seq_d
+    assert worst < 1e-3
+
+
+def test_generate_equals_step_loop_and_batch_equals_single():
+    from helpers.device import dev
+    cai = dev()
+    s = SHAPES["qwen7b_like_q4k"]
+    spec = synthetic_spec(s["cfg"], s["qtype"], head_qtype=s["head"], qkv_bias=True, std=0.05)
+    dec = cai.Decoder(spec, max_batch=4)
+    prompt = [5, 17, 900, 3]
+    for p, t in enumerate(prompt[:-1]):
+        dec.step(t, p, want_logits=False)
+    snap = dec.snapshot()
+    gen = dec.generate(prompt[-1], 3, 24)
+    assert dec.len() == 27
+    dec.restore(snap)
+    assert dec.len() == 3
+    tok, seq = prompt[-1], []
+    for i in range(24):
+        am, _ = dec.step(tok, 3 + i, want_logits=False)
+        tok = int(am[0]); seq.append(tok)
+    assert seq == gen.tolist()
+    cai.load().cai_kv_snap_destroy(snap)
+    # four independent sequences stepped together == each stepped alone
+    rng = np.random.default_rng(3)
+    toks = rng.integers(0, spec["cfg"]["vocab"], (4, 10))
+    singles = []
+    for b in range(4):
+        dec.reset(0)
+        singles.append([dec.step(int(toks[b, p]), p)[1][0].copy() for p in range(10)])
+    for b in range(4):
+        dec.reset(b)
+    for p in range(10):
+        _, lg = dec.step(toks[:, p], np.full(4, p))
+        for b in range(4):
+            assert np.max(np.abs(lg[b] - singles[b][p])) <= 1e-5 * np.max(np.abs(singles[b][p]))
+
+
+def test_prefill_equals_sequential_steps():
+    from helpers.device import dev, rel_err
+    cai = dev()
+    s = SHAPES["smollm_like_q8"]
+    spec = synthetic_spec(s["cfg"], s["qtype"], std=0.05)
+    dec = cai.Decoder(spec, max_batch=2)
+    toks = [3, 14, 15, 92, 65, 35, 89, 79, 32, 38, 46]
+    last = None
+    for p, t in enumerate(toks):
+        _, last = dec.step(t, p)
+    am, lg = dec.prefill(toks, 0, seq=1)
+    assert rel_err(lg, last[0]) < 1e-3 and am == int(np.argmax(last[0]))
+    assert dec.len(1) == len(toks)
+
+
+def test_truncate_and_error_paths():
+    from helpers.device import dev
+    cai = dev()
+    spec = spec_from_ref_fixture("tiny_llama", O.F32, max_ctx=8)
+    dec = cai.Decoder(spec)
+    seq = [1, 2, 3, 4, 5, 6]
+    full = [dec.step(t, p)[1][0].copy() for p, t in enumerate(seq)]
+    dec.truncate(3)                       # prefix reuse (neuralchatengine.pas:1434-1439)
+    again = [dec.step(t, p)[1][0].copy() for p, t in list(enumerate(seq))[3:]]
+    assert all(np.array_equal(a, b) for a, b in zip(again, full[3:]))
+    with pytest.raises(cai.CaiError):     # wrong position
+        dec.step(1, 2)
+    with pytest.raises(cai.CaiError):     # token outside the vocabulary
+        dec.step(9999, dec.len())
+    dec.step(1, 6); dec.step(1, 7)
+    with pytest.raises(cai.CaiError):     # context exhausted: refused on the host, nothing launched
+        dec.step(1, 8)
+    dec.reset()                           # always safe after a failed step (neuralchatengine.pas:1630-1636)
+    assert np.array_equal(dec.step(seq[0], 0)[1][0], full[0])

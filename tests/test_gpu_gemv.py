@@ -1,0 +1,129 @@
+"""Block-fused GEMV / small-batch kernels against the oracle's dequantize-then-dot definition.
+
+Tolerance: max |y - y_ref| / max |y_ref| <= 1e-3 (north-star bar for fp32 logits); measured values are ~1e-6.
+y_ref accumulates in double over the bit-exact dequantized weights.
+"""
+import numpy as np
+import pytest
+
+from helpers import oracle_lib as O
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+TIGHT = 2e-5
+
+
+def make(qt, rows, cols, seed):
+    rng = np.random.default_rng(seed)
+    w = (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32)
+    return O.quantize(qt, w), rng
+
+
+@pytest.mark.parametrize("qt", [O.Q4_K, O.Q8_0, O.Q4_0])
+@pytest.mark.parametrize("rows,cols", [(2048, 2048), (5632, 2048), (2048, 5632), (3, 256), (1, 9728), (1000, 3584), (64, 18944), (40000, 512)])
+@pytest.mark.parametrize("nb", [1, 4])
+def test_gemv_matches_oracle(qt, rows, cols, nb):
+    from helpers.device import dev, rel_err
+    cai = dev()
+    raw, rng = make(qt, rows, cols, rows * 7 + cols)
+    x = rng.standard_normal((nb, cols)).astype(np.float32)
+    bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
+    w = cai.QWeight(qt, rows, cols, raw, bias)
+    got = w.gemv(x)
+    want = O.gemv(qt, raw, rows, cols, x, bias, 0, 1)
+    assert got.shape == want.shape
+    assert rel_err(got, want) < TIGHT
+
+
+@pytest.mark.parametrize("qt,rows,cols", [(O.Q8_0, 576, 576), (O.Q8_0, 192, 576), (O.Q8_0, 576, 1536), (O.Q4_0, 96, 160), (O.Q8_0, 5, 32)])
+def test_gemv_non_256_multiple_widths(qt, rows, cols):
+    # SmolLM2-135M widths: 576 = 18 blocks of 32 (not a multiple of 256)
+    from helpers.device import dev, rel_err
+    cai = dev()
+    raw, rng = make(qt, rows, cols, 5)
+    for nb in (1, 2, 3, 5, 8):
+        x = rng.standard_normal((nb, cols)).astype(np.float32)
+        got = cai.QWeight(qt, rows, cols, raw).gemv(x)
+        assert rel_err(got, O.gemv(qt, raw, rows, cols, x, None, 0, 1)) < TIGHT
+
+
+@pytest.mark.parametrize("nb", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_all_batch_widths_q4k(nb):
+    from helpers.device import dev, rel_err
+    cai = dev()
+    raw, rng = make(O.Q4_K, 777, 1024, nb)
+    x = rng.standard_normal((nb, 1024)).astype(np.float32)
+    got = cai.QWeight(O.Q4_K, 777, 1024, raw).gemv(x)
+    assert rel_err(got, O.gemv(O.Q4_K, raw, 777, 1024, x, None, 0, 1)) < TIGHT
+
+
+@pytest.mark.parametrize("act", [0, 1, 2, 3])
+def test_fused_bias_and_activation_order(act):
+    # y = act(dot + bias): bias before activation (neural.cl:111-146)
+    from helpers.device import dev
+    cai = dev()
+    raw, rng = make(O.Q8_0, 300, 512, 77)
+    x = rng.standard_normal((2, 512)).astype(np.float32) * 3
+    bias = rng.standard_normal(300).astype(np.float32)
+    got = cai.QWeight(O.Q8_0, 300, 512, raw, bias).gemv(x, act)
+    want = O.gemv(O.Q8_0, raw, 300, 512, x, bias, act, 1)
+    assert np.max(np.abs(got - want)) < 1e-5
+
+
+@pytest.mark.parametrize("qt", [O.F32, O.F16])
+@pytest.mark.parametrize("rows,cols", [(11, 8), (8, 12), (8, 5), (300, 1000)])
+def test_float_weight_types_any_width(qt, rows, cols):
+    from helpers.device import dev, rel_err
+    cai = dev()
+    raw, rng = make(qt, rows, cols, 3)
+    x = rng.standard_normal((3, cols)).astype(np.float32)
+    got = cai.QWeight(qt, rows, cols, raw).gemv(x)
+    assert rel_err(got, O.gemv(qt, raw, rows, cols, x, None, 0, 1)) < TIGHT
+
+
+def test_int8_row_path_scale_then_bias():
+    # the reference's own fused-quant format: y = scale_a * sum(code*x) + bias_a (neuralvolume.pas:12693-12745)
+    from helpers.device import dev, rel_err
+    cai = dev()
+    rng = np.random.default_rng(9)
+    wf = (rng.standard_normal((128, 515)) * 0.05).astype(np.float32)
+    codes, scales = O.quant_int8_rows(wf)
+    bias = rng.standard_normal(128).astype(np.float32)
+    x = rng.standard_normal((2, 515)).astype(np.float32)
+    got = cai.QWeight(cai.I8ROW, 128, 515, codes, bias, scales).gemv(x)
+    want = O.gemv(O.I8ROW, codes.view(np.uint8), 128, 515, x, bias, 0, 1, scales)
+    assert rel_err(got, want) < TIGHT
+
+
+def test_linearity_and_zero_input():
+    # size-independent properties at a full-size shape (18944 x 3584 Q4_K)
+    from helpers.device import dev, rel_err
+    cai = dev()
+    raw, rng = make(O.Q4_K, 18944, 3584, 42)
+    w = cai.QWeight(O.Q4_K, 18944, 3584, raw)
+    a = rng.standard_normal(3584).astype(np.float32); b = rng.standard_normal(3584).astype(np.float32)
+    ya, yb, yab = w.gemv(a)[0], w.gemv(b)[0], w.gemv(a + b)[0]
+    assert rel_err(yab, ya + yb) < 1e-5
+    assert np.all(w.gemv(np.zeros(3584, np.float32)) == 0)
+    # one-hot input reads one dequantized column exactly
+    e = np.zeros(3584, np.float32); e[1234] = 1
+    col = O.dequant(O.Q4_K, raw, 18944 * 3584).reshape(18944, 3584)[:, 1234]
+    assert rel_err(w.gemv(e)[0], col) < 1e-6
+
+
+def test_lm_head_shape_q8_0():
+    # 152064 x 3584 Q8_0 (Qwen2.5-7B head) at batch 1
+    from helpers.device import dev, rel_err
+    cai = dev()
+    rows, cols = 152064, 3584
+    rng = np.random.default_rng(1)
+    raw = np.empty(rows * O.row_bytes(O.Q8_0, cols), np.uint8)
+    step = 19008
+    for r0 in range(0, rows, step):
+        blk = (rng.standard_normal((step, cols)) * 0.02).astype(np.float32)
+        raw[r0 * O.row_bytes(O.Q8_0, cols):(r0 + step) * O.row_bytes(O.Q8_0, cols)] = O.quantize(O.Q8_0, blk)
+    x = rng.standard_normal(cols).astype(np.float32)
+    got = cai.QWeight(O.Q8_0, rows, cols, raw).gemv(x)
+    want = O.gemv(O.Q8_0, raw, rows, cols, x, None, 0, 1)
+    assert rel_err(got, want) < TIGHT
+    assert int(np.argmax(got)) == int(np.argmax(want))
