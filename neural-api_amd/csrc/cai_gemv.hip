@@ -66,6 +66,7 @@ struct GemvParams {
   const float* norm_gain; float norm_eps;  // fused RMSNorm on the input when norm_gain != null
   int cols;
   int kp;                // panel length in floats (multiple of 256)
+  int kp_lds;            // LDS floats reserved per batch row: kp rounded up to whole 16-unit tiles
   int y_stride;
   int act;
   int half;              // swiglu: rows [0,half) are up, [half,2*half) gate
@@ -190,7 +191,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
 #pragma unroll
     for (int b = 0; b < NB; b++) {
       const float4* src = reinterpret_cast<const float4*>(xin + (int64_t)b * cols + k0);
-      float4* dst = xs4 + b * (p.kp >> 2);
+      float4* dst = xs4 + b * (p.kp_lds >> 2);
       for (int n = threadIdx.x; n < n4; n += 256) {
         float4 v = src[n];
         if (p.norm_gain) {
@@ -330,7 +331,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
 #pragma unroll
         for (int b = 0; b < NB; b++) {
           float xv[UW];
-          const float4* xb = xs4 + b * (p.kp >> 2);
+          const float4* xb = xs4 + b * (p.kp_lds >> 2);
 #pragma unroll
           for (int t = 0; t < T; t++) {
             const float4 v = xb[xb0 + t * 16];
@@ -488,7 +489,7 @@ static int panel_len(int cols, int nb)
 template <int QT, int NB, int MODE>
 static int launch_fast_r(const GemvParams& p, int n_groups_r, int R, int n_slots, hipStream_t st)
 {
-  const size_t lds = (size_t)NB * p.kp * 4;
+  const size_t lds = (size_t)NB * p.kp_lds * 4;
   const dim3 grid((n_groups_r + 3) / 4, n_slots);
   if constexpr (NB == 1 && MODE == 0) {
     if (R == 4) { hipLaunchKernelGGL((gemv_fast<QT, NB, 4, MODE>), grid, dim3(256), lds, st, p); return CAI_OK; }
@@ -577,6 +578,7 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
   const int qt = w0->qtype;
   if (fast_type(qt)) {
     p.kp = panel_len(p.cols, n_b);
+    p.kp_lds = (p.kp + 511) / 512 * 512;
     if (swiglu_half) {
       if (m.n != 1) return set_error(CAI_ERR_INVALID, "gemv: swiglu takes one matrix");
       p.seg[0].rows = swiglu_half;

@@ -21,8 +21,9 @@ def dev():
     return cai
 
 
-def rel_err(got, want):
-    """max |got - want| / max |want| : the logit tolerance metric (bar: <= 1e-3)."""
+def rel_err(got, want, floor=0.0):
+    """max |got - want| / max(max |want|, floor): the logit tolerance metric (bar: <= 1e-3).
+    `floor` is the typical magnitude of a result (for a lone output that happens to cancel to ~0)."""
     import numpy as np
-    denom = max(float(np.max(np.abs(want))), 1e-30)
+    denom = max(float(np.max(np.abs(want))), floor, 1e-30)
     return float(np.max(np.abs(np.asarray(got, np.float64) - np.asarray(want, np.float64)))) / denom

@@ -32,7 +32,7 @@ def test_gemv_matches_oracle(qt, rows, cols, nb):
     got = w.gemv(x)
     want = O.gemv(qt, raw, rows, cols, x, bias, 0, 1)
     assert got.shape == want.shape
-    assert rel_err(got, want) < TIGHT
+    assert rel_err(got, want, floor=0.02 * cols ** 0.5) < TIGHT
 
 
 @pytest.mark.parametrize("qt,rows,cols", [(O.Q8_0, 576, 576), (O.Q8_0, 192, 576), (O.Q8_0, 576, 1536), (O.Q4_0, 96, 160), (O.Q8_0, 5, 32)])
