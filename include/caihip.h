@@ -102,6 +102,12 @@ int cai_qw_dequant_rows(cai_qw_t w, int64_t row0, int64_t n_rows, float* out, in
  * Weights are dequantized in registers; accumulation is fp32.
  * ===================================================================================== */
 int cai_qgemv(cai_qw_t w, const float* x, int n_b, float* y, int act, int flags);
+/* Fused feed-forward front half: TokenRMSNorm(gain, eps) -> gate|up projection -> SwiGLU in one kernel
+ * (TNNetTokenRMSNorm + TNNetPointwiseConvLinear(2I) + TNNetSwiGLU, neural/neuralpretrained.pas:16815-16862;
+ * row layout up = rows 0..I-1, gate = rows I..2I-1, neural/neuralpretrained.pas:240-243).
+ *   y[b*I + i] = up_i(h_b) * silu(gate_i(h_b)),  h_b = rmsnorm(x_b) (gain == NULL: h_b = x_b)
+ * `gain` lives where x lives (host, or device with CAI_X_DEVICE).  Block-quantized weights only. */
+int cai_ffn_gateup(cai_qw_t gateup, const float* x, const float* gain, float eps, int n_b, float* y, int flags);
 /* Multi-token form on the matrix cores (prefill): x is [n_tokens][cols], y is [n_tokens][rows].
  * No counterpart in the reference, whose prefill is token-at-a-time
  * (neural/neuralchatengine.pas:1466-1470); results equal n_tokens GEMVs within bf16-input tolerance. */

@@ -16,7 +16,7 @@ V_ATTN_NORM, V_MLP_NORM, V_FINAL_NORM, V_Q_NORM, V_K_NORM = range(5)
 # every symbol include/caihip.h declares
 SYMBOLS = """cai_init cai_shutdown cai_last_error cai_device_name cai_sync cai_get_stream cai_timer_start cai_timer_stop
 cai_dev_alloc cai_dev_free cai_dev_upload cai_dev_download
-cai_qw_create cai_qw_create_int8row cai_qw_destroy cai_qw_info cai_qw_dequant_rows cai_qgemv cai_qgemm
+cai_qw_create cai_qw_create_int8row cai_qw_destroy cai_qw_info cai_qw_dequant_rows cai_qgemv cai_ffn_gateup cai_qgemm
 cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_router_topk
 cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_attn_decode
 cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_generate
@@ -64,6 +64,7 @@ def load():
         L.cai_qw_dequant_rows.argtypes = [vp, i64, i64, vp, i32]
         L.cai_qgemv.argtypes = [vp, vp, i32, vp, i32, i32]
         L.cai_qgemm.argtypes = [vp, vp, i32, vp, i32]
+        L.cai_ffn_gateup.argtypes = [vp, vp, vp, f32, i32, vp, i32]
         L.cai_rmsnorm.argtypes = [vp, vp, i32, i32, f32, vp, i32]
         L.cai_rope.argtypes = [vp, i32, i32, i32, f32, i32]
         L.cai_swiglu.argtypes = [vp, i32, i32, vp, i32]
@@ -151,6 +152,13 @@ class QWeight:
         x = np.ascontiguousarray(x, np.float32).reshape(-1, self.cols)
         y = np.empty((x.shape[0], self.rows), np.float32)
         check(load().cai_qgemv(self.h, _ptr(x), x.shape[0], _ptr(y), act, 0))
+        return y
+
+    def ffn_gateup(self, x, gain=None, eps=1e-6):
+        x = np.ascontiguousarray(x, np.float32).reshape(-1, self.cols)
+        y = np.empty((x.shape[0], self.rows // 2), np.float32)
+        g = None if gain is None else np.ascontiguousarray(gain, np.float32)
+        check(load().cai_ffn_gateup(self.h, _ptr(x), _ptr(g), eps, x.shape[0], _ptr(y), 0))
         return y
 
     def gemm(self, x):

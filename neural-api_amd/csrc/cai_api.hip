@@ -282,3 +282,32 @@ extern "C" int cai_qgemv(cai_qw_t w, const float* x, int n_b, float* y, int act,
   }
   return CAI_OK;
 }
+
+extern "C" int cai_ffn_gateup(cai_qw_t w, const float* x, const float* gain, float eps, int n_b, float* y, int flags)
+{
+  CAI_READY();
+  CAI_REQUIRE(w && x && y, "cai_ffn_gateup: null argument");
+  CAI_REQUIRE(n_b >= 1 && n_b <= 8, "cai_ffn_gateup: n_b %d outside 1..8", n_b);
+  CAI_REQUIRE(w->rows % 2 == 0, "cai_ffn_gateup: %lld rows is not an up|gate pair", (long long)w->rows);
+  Context& c = ctx();
+  const int64_t I = w->rows / 2;
+  const size_t xb = (size_t)n_b * w->cols * 4, gb = gain ? (size_t)w->cols * 4 : 0, yb = (size_t)n_b * I * 4;
+  const float* dx = x; const float* dg = gain; float* dy = y; int rc;
+  if (!(flags & CAI_X_DEVICE)) {
+    if ((rc = ensure_stage(&c.stage_in, &c.stage_in_cap, xb + gb))) return rc;
+    CAI_HIP(hipMemcpyAsync(c.stage_in, x, xb, hipMemcpyHostToDevice, c.stream));
+    dx = (const float*)c.stage_in;
+    if (gain) {
+      CAI_HIP(hipMemcpyAsync((char*)c.stage_in + xb, gain, gb, hipMemcpyHostToDevice, c.stream));
+      dg = (const float*)((char*)c.stage_in + xb);
+    }
+  }
+  if (!(flags & CAI_Y_DEVICE)) { if ((rc = ensure_stage(&c.stage_out, &c.stage_out_cap, yb))) return rc; dy = (float*)c.stage_out; }
+  MultiGemv m{}; m.n = 1; m.w[0] = w; m.rows[0] = w->rows;
+  if ((rc = launch_gemv_multi(m, dx, n_b, dy, I, CAI_ACT_NONE, nullptr, dg, eps, (int)I))) return rc;
+  if (!(flags & CAI_Y_DEVICE)) {
+    CAI_HIP(hipMemcpyAsync(y, dy, yb, hipMemcpyDeviceToHost, c.stream));
+    CAI_HIP(hipStreamSynchronize(c.stream));
+  }
+  return CAI_OK;
+}
