@@ -7,7 +7,9 @@
 // Device formulation: split-K over the key axis.  Work-group (split, kv_head, sequence) streams its slice
 // of K and V exactly once with coalesced row loads (32 lanes x 16 B cover one 128-wide row), serves all
 // `G` query heads of the group from that one pass, and keeps an online-softmax state (m, l, acc) per
-// head; the 8 half-waves of the group meet in LDS, and a second tiny kernel merges the splits.
+// head; the 8 half-waves of the group meet in LDS, and the last work-group of a (sequence, KV head) to finish merges
+// the splits (arrival counter + device-scope fence), so the whole layer step is one launch.  RoPE of q and of
+// the new k row and the cache append happen inside the same kernel.
 #include "cai_internal.hpp"
 
 namespace cai {
@@ -44,79 +46,95 @@ struct AttnParams {
   float* part;                 // [seq][q_head][split][hd+2]
   float* out; int64_t out_stride;
   int seq0;                    // cache sequence index of activation row 0
+  int* counters;               // [seq][kv_head] arrival counters of the split merge (zero between launches)
 };
 
-// ---- RoPE on q and k (interleaved pairs, neural/neural.cl:1517-1542) + KV append (2354-2379) ----
-template <typename KV_T>
-__global__ __launch_bounds__(256) void rope_append_kernel(const AttnParams p)
-{
-  const int seq = blockIdx.x;
-  float* row = p.qkv + (int64_t)seq * p.qkv_stride;
-  const int pos = p.pos[seq];
-  const int qw = p.q_heads * p.hd, kw = p.kv_heads * p.hd;
-  KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (seq + p.seq0) * p.seq_elems + p.layer_off;
-  KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (seq + p.seq0) * p.seq_elems + p.layer_off;
-  // q pairs then k pairs
-  const int n_pairs = (qw + kw) >> 1;
-  for (int i = threadIdx.x; i < n_pairs; i += 256) {
-    const int e = 2 * i;                  // element index inside [Q|K]
-    float x0 = row[e], x1 = row[e + 1];
-    if (p.theta) {
-      const int k = (e % p.hd) >> 1;
-      const float angle = (float)pos * p.theta[k];
-      float s, c; sincosf(angle, &s, &c);
-      const float y0 = c * x0 - s * x1, y1 = s * x0 + c * x1;
-      x0 = y0; x1 = y1;
-      if (e < qw) { row[e] = x0; row[e + 1] = x1; }
-    }
-    if (e >= qw) {
-      const int ke = e - qw, g = ke / p.hd, d = ke % p.hd;
-      KV_T* dst = kc + ((int64_t)g * p.max_ctx + pos) * p.hd + d;
-      dst[0] = kv_from_float<KV_T>(x0); dst[1] = kv_from_float<KV_T>(x1);
-    }
-  }
-  for (int i = threadIdx.x; i < kw; i += 256) {
-    const int g = i / p.hd, d = i % p.hd;
-    vc[((int64_t)g * p.max_ctx + pos) * p.hd + d] = kv_from_float<KV_T>(row[qw + kw + i]);
-  }
-}
-
-// ---- split-K decode ----
+// ---- one kernel per token and layer: RoPE (neural/neural.cl:1517-1542) + KV append (2354-2379) +
+//      split-K online-softmax decode (2406-2499) + merge of the splits by the last work-group to finish ----
 template <int G, int DS, typename KV_T>
-__global__ __launch_bounds__(256) void attn_split_kernel(const AttnParams p)
+__global__ __launch_bounds__(256) void attn_step_kernel(const AttnParams p)
 {
   const int split = blockIdx.x, g = blockIdx.y, seq = blockIdx.z;
-  const int len = p.pos[seq] + 1;
+  const int pos = p.pos[seq];
+  const int len = pos + 1;
   const int j_start = (p.window > 0 && len > p.window) ? len - p.window : 0;
   const int s_begin = max(j_start, split * p.split_len), s_end = min(len, (split + 1) * p.split_len);
-  if (s_begin >= s_end) return;   // whole work-group leaves together: no barrier was reached yet
+  if (s_begin >= s_end) return;   // whole work-group leaves together, before any barrier
+  const int s_first = j_start / p.split_len, s_last = pos / p.split_len;
+  const int n_active = s_last - s_first + 1;
 
   const int hw = threadIdx.x >> 5, l32 = threadIdx.x & 31;
-  const int hd = p.hd;
+  const int hd = p.hd, qw = p.q_heads * hd, kw = p.kv_heads * hd;
   const int d0 = l32 * DS;
-  const float* qrow = p.qkv + (int64_t)seq * p.qkv_stride;
+  const float* row = p.qkv + (int64_t)seq * p.qkv_stride;
+
+  // rotation of this lane's pairs at the token's position (DS even, or DS == 1 with the pair split over 2 lanes)
+  float rs[(DS + 1) / 2], rc[(DS + 1) / 2];
+#pragma unroll
+  for (int i = 0; i < (DS + 1) / 2; i++) {
+    rs[i] = 0.0f; rc[i] = 1.0f;
+    const int d = d0 + 2 * i;
+    if (p.theta && d < hd) { const float angle = (float)pos * p.theta[d >> 1]; sincosf(angle, &rs[i], &rc[i]); }
+  }
+  // loads DS elements of a head vector and rotates them (pairs (2k, 2k+1))
+  auto load_rot = [&](const float* v, float (&o)[DS], bool rotate) {
+    if (DS >= 2) {
+#pragma unroll
+      for (int i = 0; i < DS; i += 2) {
+        const int d = d0 + i;
+        const float x0 = d < hd ? v[d] : 0.0f, x1 = d + 1 < hd ? v[d + 1] : 0.0f;
+        if (rotate) { o[i] = rc[i / 2] * x0 - rs[i / 2] * x1; o[i + (DS > 1 ? 1 : 0)] = rs[i / 2] * x0 + rc[i / 2] * x1; }
+        else { o[i] = x0; o[i + (DS > 1 ? 1 : 0)] = x1; }
+      }
+    } else {
+      const int d = d0;
+      const float own = d < hd ? v[d] : 0.0f, mate = (d ^ 1) < hd ? v[d ^ 1] : 0.0f;
+      if (rotate) o[0] = (d & 1) ? (rs[0] * mate + rc[0] * own) : (rc[0] * own - rs[0] * mate);
+      else o[0] = own;
+    }
+  };
 
   float q[G][DS], acc[G][DS], m[G], l[G];
 #pragma unroll
   for (int h = 0; h < G; h++) {
     m[h] = -1e30f; l[h] = 0.0f;
+    load_rot(row + (g * G + h) * hd, q[h], p.theta != nullptr);
+#pragma unroll
+    for (int i = 0; i < DS; i++) acc[h][i] = 0.0f;
+  }
+  KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+
+  // the work-group whose slice holds `pos` appends the new row and keeps it in registers
+  float knew[DS], vnew[DS];
+  const bool owns_new = pos >= s_begin && pos < s_end;
+  if (owns_new) {
+    load_rot(row + qw + g * hd, knew, p.theta != nullptr);
+    float dummy[DS];
+    load_rot(row + qw + kw + g * hd, dummy, false);
 #pragma unroll
     for (int i = 0; i < DS; i++) {
-      const int d = d0 + i;
-      q[h][i] = d < hd ? qrow[(g * G + h) * hd + d] : 0.0f;
-      acc[h][i] = 0.0f;
+      vnew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(dummy[i]));
+      knew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(knew[i]));
+      if (hw == 0 && d0 + i < hd) {
+        kc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(knew[i]);
+        vc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(vnew[i]);
+      }
     }
   }
-  const KV_T* kc = reinterpret_cast<const KV_T*>(p.kc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
-  const KV_T* vc = reinterpret_cast<const KV_T*>(p.vc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
 
   for (int j = s_begin + hw; j < s_end; j += 8) {
     float kd[DS], vd[DS];
+    if (j == pos) {
 #pragma unroll
-    for (int i = 0; i < DS; i++) {
-      const int d = d0 + i;
-      kd[i] = d < hd ? kv_to_float<KV_T>(kc[(int64_t)j * hd + d]) : 0.0f;
-      vd[i] = d < hd ? kv_to_float<KV_T>(vc[(int64_t)j * hd + d]) : 0.0f;
+      for (int i = 0; i < DS; i++) { kd[i] = knew[i]; vd[i] = vnew[i]; }
+    } else {
+#pragma unroll
+      for (int i = 0; i < DS; i++) {
+        const int d = d0 + i;
+        kd[i] = d < hd ? kv_to_float<KV_T>(kc[(int64_t)j * hd + d]) : 0.0f;
+        vd[i] = d < hd ? kv_to_float<KV_T>(vc[(int64_t)j * hd + d]) : 0.0f;
+      }
     }
 #pragma unroll
     for (int h = 0; h < G; h++) {
@@ -137,6 +155,7 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const AttnParams p)
   // ---- merge the 8 half-waves through LDS ----
   __shared__ float sm[8][G], sl[8][G];
   __shared__ float sacc[8][G][32 * DS];
+  __shared__ int s_last_flag;
   if (l32 == 0) {
 #pragma unroll
     for (int h = 0; h < G; h++) { sm[hw][h] = m[h]; sl[hw][h] = l[h]; }
@@ -159,39 +178,62 @@ __global__ __launch_bounds__(256) void attn_split_kernel(const AttnParams p)
       L = fmaf(sl[w][h], e, L); A = fmaf(sacc[w][h][d], e, A);
     }
     const int qh = g * G + h;
-    if (p.n_splits == 1) {
+    if (n_active == 1) {
       p.out[(int64_t)seq * p.out_stride + qh * hd + d] = L > 0.0f ? A * (1.0f / L) : 0.0f;
     } else {
+      // device-coherent stores: the merging work-group may sit on another XCD (its own L2)
       float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + split) * (hd + 2);
-      pt[d] = A;
-      if (d == 0) { pt[hd] = M; pt[hd + 1] = L; }
+      __hip_atomic_store(&pt[d], A, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (d == 0) {
+        __hip_atomic_store(&pt[hd], M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&pt[hd + 1], L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
   }
-}
+  if (n_active == 1) return;
 
-__global__ void attn_merge_kernel(const AttnParams p)
-{
-  const int qh = blockIdx.x, seq = blockIdx.y;
-  const int hd = p.hd;
-  const int len = p.pos[seq] + 1;
-  const int j_start = (p.window > 0 && len > p.window) ? len - p.window : 0;
-  const int s_first = j_start / p.split_len, s_last = (len - 1) / p.split_len;
-  const float* pt = p.part + ((int64_t)seq * p.q_heads + qh) * p.n_splits * (hd + 2);
-  float M = -1e30f;
-  for (int s = s_first; s <= s_last; s++) M = fmaxf(M, pt[s * (hd + 2) + hd]);
-  float L = 0.0f;
-  for (int s = s_first; s <= s_last; s++) {
-    const float ls = pt[s * (hd + 2) + hd + 1];
-    if (ls > 0.0f) L = fmaf(ls, expf(pt[s * (hd + 2) + hd] - M), L);
+  // ---- the last work-group of this (sequence, KV head) to arrive merges the splits ----
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // every lane's stores have been acknowledged
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int* cnt = p.counters + seq * p.kv_heads + g;
+    const int prev = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    const int last = prev == n_active - 1;
+    if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+    s_last_flag = last;
   }
-  const float inv = L > 0.0f ? 1.0f / L : 0.0f;
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-    float A = 0.0f;
-    for (int s = s_first; s <= s_last; s++) {
-      const float ls = pt[s * (hd + 2) + hd + 1];
-      if (ls > 0.0f) A = fmaf(pt[s * (hd + 2) + d], expf(pt[s * (hd + 2) + hd] - M), A);
+  __syncthreads();
+  if (!s_last_flag) return;
+  // all (M, L) pairs of the group first (independent device-coherent loads), then the accumulators in batches
+  __shared__ float mM[G][64], mL[G][64];
+  for (int i = threadIdx.x; i < G * n_active; i += 256) {
+    const int h = i / n_active, s = s_first + i % n_active;
+    const float* pt = p.part + (((int64_t)seq * p.q_heads + g * G + h) * p.n_splits + s) * (hd + 2);
+    mM[h][s - s_first] = __hip_atomic_load(&pt[hd], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    mL[h][s - s_first] = __hip_atomic_load(&pt[hd + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  for (int o = threadIdx.x; o < G * hd; o += 256) {
+    const int h = o / hd, d = o % hd, qh = g * G + h;
+    const float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + s_first) * (hd + 2) + d;
+    float M = -1e30f;
+    for (int s = 0; s < n_active; s++) M = fmaxf(M, mM[h][s]);
+    float L = 0.0f, A = 0.0f;
+    for (int s0 = 0; s0 < n_active; s0 += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++)
+        v[u] = s0 + u < n_active ? __hip_atomic_load(&pt[(int64_t)(s0 + u) * (hd + 2)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        if (s0 + u < n_active) {
+          const float ls = mL[h][s0 + u];
+          const float e = ls > 0.0f ? expf(mM[h][s0 + u] - M) : 0.0f;
+          L = fmaf(ls, e, L); A = fmaf(v[u], e, A);
+        }
+      }
     }
-    p.out[(int64_t)seq * p.out_stride + qh * hd + d] = A * inv;
+    p.out[(int64_t)seq * p.out_stride + qh * hd + d] = L > 0.0f ? A * (1.0f / L) : 0.0f;
   }
 }
 
@@ -199,9 +241,9 @@ template <int G, typename KV_T>
 static int launch_split_ds(const AttnParams& p, int n_seq, hipStream_t st)
 {
   const dim3 grid(p.n_splits, p.kv_heads, n_seq);
-  if (p.hd <= 32) hipLaunchKernelGGL((attn_split_kernel<G, 1, KV_T>), grid, dim3(256), 0, st, p);
-  else if (p.hd <= 64) hipLaunchKernelGGL((attn_split_kernel<G, 2, KV_T>), grid, dim3(256), 0, st, p);
-  else if (p.hd <= 128) hipLaunchKernelGGL((attn_split_kernel<G, 4, KV_T>), grid, dim3(256), 0, st, p);
+  if (p.hd <= 32) hipLaunchKernelGGL((attn_step_kernel<G, 1, KV_T>), grid, dim3(256), 0, st, p);
+  else if (p.hd <= 64) hipLaunchKernelGGL((attn_step_kernel<G, 2, KV_T>), grid, dim3(256), 0, st, p);
+  else if (p.hd <= 128) hipLaunchKernelGGL((attn_step_kernel<G, 4, KV_T>), grid, dim3(256), 0, st, p);
   else return set_error(CAI_ERR_UNSUPPORTED, "attention: head_dim %d > 128", p.hd);
   return CAI_OK;
 }
@@ -237,18 +279,9 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   p.window = window; p.softcap = softcap; p.inv_sqrt = 1.0f / sqrtf((float)kv->head_dim);
   p.theta = theta; p.pos = pos_dev; p.split_len = kv->split_len; p.n_splits = kv->n_splits;
   p.part = kv->part; p.out = out; p.out_stride = out_stride; p.seq0 = seq0;
-  int rc;
-  if (kv->dtype == CAI_KV_F16) {
-    hipLaunchKernelGGL(rope_append_kernel<__half>, dim3(n_seq), dim3(256), 0, c.stream, p);
-    rc = launch_split_g<__half>(p, n_seq, c.stream);
-  } else {
-    hipLaunchKernelGGL(rope_append_kernel<float>, dim3(n_seq), dim3(256), 0, c.stream, p);
-    rc = launch_split_g<float>(p, n_seq, c.stream);
-  }
-  if (rc) return rc;
-  if (p.n_splits > 1)
-    hipLaunchKernelGGL(attn_merge_kernel, dim3(q_heads, n_seq), dim3(kv->head_dim >= 128 ? 128 : 64), 0, c.stream, p);
-  return CAI_OK;
+  p.counters = kv->d_counters;
+  if (kv->dtype == CAI_KV_F16) return launch_split_g<__half>(p, n_seq, c.stream);
+  return launch_split_g<float>(p, n_seq, c.stream);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -262,7 +295,7 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   kv->n_seq = n_seq; kv->n_layers = n_layers; kv->kv_heads = kv_heads; kv->head_dim = head_dim; kv->max_ctx = max_ctx; kv->dtype = dtype;
   kv->len.assign((size_t)n_seq * n_layers, 0);
   int sl = (max_ctx + 47) / 48; sl = (sl + 31) / 32 * 32; if (sl < 32) sl = 32;
-  kv->split_len = sl; kv->n_splits = (max_ctx + sl - 1) / sl;
+  kv->split_len = sl; kv->n_splits = (max_ctx + sl - 1) / sl;   // <= 48 by construction (the merge stage holds 64)
   const size_t bytes = (size_t)kv->seq_elems() * n_seq * kv->elem();
   CAI_HIP(hipMalloc(&kv->k, bytes));
   CAI_HIP(hipMalloc(&kv->v, bytes));
@@ -271,6 +304,8 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   kv->part_q_heads = kv_heads * 8;
   CAI_HIP(hipMalloc(&kv->part, (size_t)n_seq * kv->part_q_heads * kv->n_splits * (head_dim + 2) * sizeof(float)));
   CAI_HIP(hipMalloc(&kv->d_len, sizeof(int32_t) * n_seq));
+  CAI_HIP(hipMalloc(&kv->d_counters, sizeof(int) * n_seq * kv_heads));
+  CAI_HIP(hipMemsetAsync(kv->d_counters, 0, sizeof(int) * n_seq * kv_heads, ctx().stream));
   CAI_HIP(hipStreamSynchronize(ctx().stream));
   return CAI_OK;
 }
@@ -281,6 +316,8 @@ void kv_free(cai_kv_s* kv)
   if (kv->v) (void)hipFree(kv->v);
   if (kv->part) (void)hipFree(kv->part);
   if (kv->d_len) (void)hipFree(kv->d_len);
+  if (kv->d_counters) (void)hipFree(kv->d_counters);
+  kv->d_counters = nullptr;
   kv->k = kv->v = nullptr; kv->part = nullptr; kv->d_len = nullptr;
 }
 

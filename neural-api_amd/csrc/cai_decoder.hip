@@ -22,6 +22,7 @@ struct cai_decoder_s {
   float *x = nullptr, *qkv = nullptr, *att = nullptr, *gu = nullptr, *mid = nullptr, *logits = nullptr;
   float *router_logits = nullptr, *router_probs = nullptr, *moe_gate = nullptr, *moe_part = nullptr;
   int32_t* moe_expert = nullptr;
+  float* am_v = nullptr; int32_t* am_i = nullptr;   // arg-max slice winners
   int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_argmax = nullptr, *d_gen = nullptr;
   int32_t* h_io = nullptr;   // pinned: tokens[8] pos[8] argmax[8]
   hipGraphExec_t graph[9] = {nullptr};
@@ -135,7 +136,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
     MultiGemv m{}; m.n = 1; m.w[0] = hw; m.rows[0] = c.vocab;
     if ((rc = launch_gemv_multi(m, d->x, n_b, d->logits, c.vocab, CAI_ACT_NONE, nullptr, d->final_norm, c.eps, 0))) return rc;
   }
-  launch_argmax(d->logits, c.vocab, n_b, d->d_argmax);
+  launch_argmax(d->logits, c.vocab, n_b, d->d_argmax, d->am_v, d->am_i);
   return CAI_OK;
 }
 
@@ -195,6 +196,9 @@ extern "C" int cai_decoder_create(const cai_decoder_config* cfg, cai_decoder_t* 
     if (e == hipSuccess) e = alloc_f(&d->moe_part, (size_t)K * c.d_model);
     if (e == hipSuccess) e = hipMalloc((void**)&d->moe_expert, (size_t)B * K * sizeof(int32_t));
   }
+  const int ame = argmax_scratch_entries(c.vocab, B);
+  if (e == hipSuccess) e = alloc_f(&d->am_v, (size_t)ame);
+  if (e == hipSuccess) e = hipMalloc((void**)&d->am_i, (size_t)ame * sizeof(int32_t));
   if (e == hipSuccess) e = hipMalloc((void**)&d->d_tokens, 3 * 8 * sizeof(int32_t));
   if (e == hipSuccess) e = hipMalloc((void**)&d->d_gen, (size_t)c.max_ctx * sizeof(int32_t));
   if (e == hipSuccess) e = hipHostMalloc((void**)&d->h_io, 3 * 8 * sizeof(int32_t), hipHostMallocDefault);
@@ -218,6 +222,8 @@ extern "C" int cai_decoder_destroy(cai_decoder_t d)
   for (float* p : fs) if (p) (void)hipFree(p);
   for (auto& L : d->layers) for (float* p : L.v) if (p) (void)hipFree(p);
   if (d->moe_expert) (void)hipFree(d->moe_expert);
+  if (d->am_v) (void)hipFree(d->am_v);
+  if (d->am_i) (void)hipFree(d->am_i);
   if (d->d_tokens) (void)hipFree(d->d_tokens);
   if (d->d_gen) (void)hipFree(d->d_gen);
   if (d->h_io) (void)hipHostFree(d->h_io);

@@ -75,6 +75,7 @@ struct cai_kv_s {
   float* part = nullptr;                  // [seq][q_head][split][head_dim+2] split-K partials
   int part_q_heads = 0;
   int32_t* d_len = nullptr;               // [seq] device scratch: rows live BEFORE the token being decoded
+  int* d_counters = nullptr;              // [seq][kv_head] split-merge arrival counters
   size_t elem() const { return dtype == CAI_KV_F16 ? 2 : 4; }
   int64_t layer_elems() const { return (int64_t)kv_heads * max_ctx * head_dim; }
   int64_t seq_elems() const { return layer_elems() * n_layers; }
@@ -108,7 +109,8 @@ int launch_rmsnorm(const float* x, const float* gain, int n, int n_tokens, float
 int launch_rope(float* x, int n_heads, int head_dim, const int32_t* pos_dev, int pos_host, const float* theta, int n_tokens, int64_t token_stride);
 int launch_swiglu(const float* x, int half, int n_tokens, float* y);
 int launch_add(float* x, const float* y, int64_t n);
-int launch_argmax(const float* x, int n, int n_rows, int32_t* out);
+int launch_argmax(const float* x, int n, int n_rows, int32_t* out, float* scratch_v, int32_t* scratch_i);
+int argmax_scratch_entries(int n, int n_rows);
 int launch_embed(const cai_qw_s* w, const int32_t* tokens_dev, int n_tokens, float* out);
 int launch_router_topk(const float* logits, int n, int k, int renorm, int n_tokens, int32_t* expert_out, float* gate_out, float* probs_scratch);
 int launch_rmsnorm_strided(const float* x, const float* gain, int n, int n_tokens, float eps, float* y, int64_t x_stride, int64_t y_stride);

@@ -192,34 +192,52 @@ int launch_moe_combine(float* x, const float* part, const float* gate, int k, in
 }
 
 // ---- ArgMaxRow (neural/neuralchatengine.pas:683-697): strict >, lowest index wins ties ----
-__global__ __launch_bounds__(1024) void argmax_kernel(const float* x, int n, int32_t* out)
+// Two stages: work-groups scan 4096-element slices, then one work-group folds the slice winners.
+__device__ __forceinline__ bool argmax_better(float v, int i, float bv, int bi) { return bi < 0 || v > bv || (v == bv && i < bi); }
+
+__global__ __launch_bounds__(256) void argmax_stage1(const float* x, int n, float* pv, int32_t* pi, int n_slices)
 {
-  const float* xr = x + (int64_t)blockIdx.x * n;
-  float best = -INFINITY; int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < n; i += 1024) {
-    const float v = xr[i];
-    if (bi == 0x7fffffff || v > best) { best = v; bi = i; }   // indices rise per thread: ties keep the earlier one
-  }
-  __shared__ float sv[1024]; __shared__ int si[1024];
+  const int row = blockIdx.y, slice = blockIdx.x;
+  const float* xr = x + (int64_t)row * n;
+  float best = 0.0f; int bi = -1;
+  const int i0 = slice * 4096, i1 = min(n, i0 + 4096);
+  for (int i = i0 + threadIdx.x; i < i1; i += 256) { const float v = xr[i]; if (bi < 0 || v > best) { best = v; bi = i; } }
+  __shared__ float sv[256]; __shared__ int si[256];
   sv[threadIdx.x] = best; si[threadIdx.x] = bi;
   __syncthreads();
-  for (int s = 512; s > 0; s >>= 1) {
+  for (int s = 128; s > 0; s >>= 1) {
     if ((int)threadIdx.x < s) {
       const float ov = sv[threadIdx.x + s]; const int oi = si[threadIdx.x + s];
-      if (oi != 0x7fffffff && (si[threadIdx.x] == 0x7fffffff || ov > sv[threadIdx.x] || (ov == sv[threadIdx.x] && oi < si[threadIdx.x]))) {
-        sv[threadIdx.x] = ov; si[threadIdx.x] = oi;
-      }
+      if (oi >= 0 && argmax_better(ov, oi, sv[threadIdx.x], si[threadIdx.x])) { sv[threadIdx.x] = ov; si[threadIdx.x] = oi; }
     }
     __syncthreads();
   }
-  if (threadIdx.x == 0) out[blockIdx.x] = si[0] == 0x7fffffff ? 0 : si[0];
+  if (threadIdx.x == 0) { pv[row * n_slices + slice] = sv[0]; pi[row * n_slices + slice] = si[0]; }
 }
 
-int launch_argmax(const float* x, int n, int n_rows, int32_t* out)
+__global__ __launch_bounds__(64) void argmax_stage2(const float* pv, const int32_t* pi, int n_slices, int32_t* out)
 {
-  hipLaunchKernelGGL(argmax_kernel, dim3(n_rows), dim3(1024), 0, ctx().stream, x, n, out);
+  const int row = blockIdx.x;
+  float best = 0.0f; int bi = -1;
+  for (int s = threadIdx.x; s < n_slices; s += 64) {
+    const float v = pv[row * n_slices + s]; const int i = pi[row * n_slices + s];
+    if (i >= 0 && argmax_better(v, i, best, bi)) { best = v; bi = i; }
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off); const int oi = __shfl_xor(bi, off);
+    if (oi >= 0 && argmax_better(ov, oi, best, bi)) { best = ov; bi = oi; }
+  }
+  if (threadIdx.x == 0) out[row] = bi < 0 ? 0 : bi;
+}
+
+int launch_argmax(const float* x, int n, int n_rows, int32_t* out, float* scratch_v, int32_t* scratch_i)
+{
+  const int n_slices = (n + 4095) / 4096;
+  hipLaunchKernelGGL(argmax_stage1, dim3(n_slices, n_rows), dim3(256), 0, ctx().stream, x, n, scratch_v, scratch_i, n_slices);
+  hipLaunchKernelGGL(argmax_stage2, dim3(n_rows), dim3(64), 0, ctx().stream, scratch_v, scratch_i, n_slices, out);
   return CAI_OK;
 }
+int argmax_scratch_entries(int n, int n_rows) { return (n + 4095) / 4096 * n_rows; }
 
 // ---- router: TNNetPointwiseSoftMax (neural/neural.cl:1594-1647) + TNNetTopKGate ----
 // One thread per token, the way the reference keeps a group's reduction inside one work-item.
@@ -351,7 +369,9 @@ extern "C" int cai_argmax(const float* x, int n, int32_t* index_out, int flags)
   Context& c = ctx();
   const void* dx; int rc;
   if ((rc = stage_input(x, (size_t)n * 4, flags & CAI_X_DEVICE, &dx))) return rc;
-  launch_argmax((const float*)dx, n, 1, c.d_small);
+  const int ne = argmax_scratch_entries(n, 1);
+  void* scr; if ((rc = stage_output(nullptr, (size_t)ne * 8, 0, &scr))) return rc;
+  launch_argmax((const float*)dx, n, 1, c.d_small, (float*)scr, (int32_t*)scr + ne);
   CAI_HIP(hipMemcpyAsync(c.h_small, c.d_small, 4, hipMemcpyDeviceToHost, c.stream));
   CAI_HIP(hipStreamSynchronize(c.stream));
   *index_out = c.h_small[0];
