@@ -7,9 +7,10 @@
 // Device formulation: split-K over the key axis.  Work-group (split, kv_head, sequence) streams its slice
 // of K and V exactly once with coalesced row loads (32 lanes x 16 B cover one 128-wide row), serves all
 // `G` query heads of the group from that one pass, and keeps an online-softmax state (m, l, acc) per
-// head; the 8 half-waves of the group meet in LDS, and the last work-group of a (sequence, KV head) to finish merges
-// the splits (arrival counter + device-scope fence), so the whole layer step is one launch.  RoPE of q and of
-// the new k row and the cache append happen inside the same kernel.
+// head; the 8 half-waves of the group meet in LDS, and a second small kernel (one work-group per query head) merges
+// the splits.  (Merging inside the first kernel through an arrival counter was measured slower: every
+// device-coherent hand-off between work-groups costs a memory round trip of ~2.5 us.)  RoPE of q and of the new k
+// row and the cache append happen inside the split kernel.
 #include "cai_internal.hpp"
 
 namespace cai {
@@ -49,11 +50,14 @@ struct AttnParams {
   int* counters;               // [seq][kv_head] arrival counters of the split merge (zero between launches)
 };
 
-// ---- one kernel per token and layer: RoPE (neural/neural.cl:1517-1542) + KV append (2354-2379) +
-//      split-K online-softmax decode (2406-2499) + merge of the splits by the last work-group to finish ----
-template <int G, int DS, typename KV_T>
+// ---- split kernel: RoPE (neural/neural.cl:1517-1542) + KV append (2354-2379) + split-K online-softmax decode
+//      (2406-2499).  The loop over the group's query heads is NOT unrolled and the per-head running state lives in
+//      LDS: the kernel stays a few KB of code, which matters for a launch this short (a cold instruction cache is
+//      refilled from L2 on every CU at every launch). ----
+template <int DS, typename KV_T>
 __global__ __launch_bounds__(256) void attn_step_kernel(const AttnParams p)
 {
+  extern __shared__ float lds[];
   const int split = blockIdx.x, g = blockIdx.y, seq = blockIdx.z;
   const int pos = p.pos[seq];
   const int len = pos + 1;
@@ -63,10 +67,37 @@ __global__ __launch_bounds__(256) void attn_step_kernel(const AttnParams p)
   const int s_first = j_start / p.split_len, s_last = pos / p.split_len;
   const int n_active = s_last - s_first + 1;
 
-  const int hw = threadIdx.x >> 5, l32 = threadIdx.x & 31;
+  const int tid = threadIdx.x, hw = tid >> 5, l32 = tid & 31;
   const int hd = p.hd, qw = p.q_heads * hd, kw = p.kv_heads * hd;
+  const int G = p.q_heads / p.kv_heads;
   const int d0 = l32 * DS;
   const float* row = p.qkv + (int64_t)seq * p.qkv_stride;
+  KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+
+  // LDS: rotated q [G][32*DS] | state m,l [G][256] each | acc [G][DS][256]
+  float* sq = lds;
+  float* st_m = sq + G * 32 * DS;
+  float* st_l = st_m + G * 256;
+  float* st_a = st_l + G * 256;
+
+  constexpr int PCH = 4;
+  float kdA[PCH][DS], vdA[PCH][DS], kdB[PCH][DS], vdB[PCH][DS];
+  auto load_chunk = [&](float (&kd)[PCH][DS], float (&vd)[PCH][DS], int j0) {
+    if (j0 >= s_end) return;
+#pragma unroll
+    for (int c = 0; c < PCH; c++) {
+      const int j = min(j0 + 8 * c, s_end - 1);
+#pragma unroll
+      for (int i = 0; i < DS; i++) {
+        const int d = d0 + i;
+        const bool ok = d < hd && j != pos;   // the appended row comes from registers
+        kd[c][i] = ok ? kv_to_float<KV_T>(kc[(int64_t)j * hd + d]) : 0.0f;
+        vd[c][i] = ok ? kv_to_float<KV_T>(vc[(int64_t)j * hd + d]) : 0.0f;
+      }
+    }
+  };
+  load_chunk(kdA, vdA, s_begin + hw);      // cached rows are requested before the rotation math
 
   // rotation of this lane's pairs at the token's position (DS even, or DS == 1 with the pair split over 2 lanes)
   float rs[(DS + 1) / 2], rc[(DS + 1) / 2];
@@ -76,7 +107,6 @@ __global__ __launch_bounds__(256) void attn_step_kernel(const AttnParams p)
     const int d = d0 + 2 * i;
     if (p.theta && d < hd) { const float angle = (float)pos * p.theta[d >> 1]; sincosf(angle, &rs[i], &rc[i]); }
   }
-  // loads DS elements of a head vector and rotates them (pairs (2k, 2k+1))
   auto load_rot = [&](const float* v, float (&o)[DS], bool rotate) {
     if (DS >= 2) {
 #pragma unroll
@@ -93,28 +123,27 @@ __global__ __launch_bounds__(256) void attn_step_kernel(const AttnParams p)
       else o[0] = own;
     }
   };
-
-  float q[G][DS], acc[G][DS], m[G], l[G];
+  // rotated q of the group's heads -> LDS (half-wave hw takes heads hw, hw+8, ..); state reset
+  for (int h = hw; h < G; h += 8) {
+    float qr[DS];
+    load_rot(row + (g * G + h) * hd, qr, p.theta != nullptr);
 #pragma unroll
-  for (int h = 0; h < G; h++) {
-    m[h] = -1e30f; l[h] = 0.0f;
-    load_rot(row + (g * G + h) * hd, q[h], p.theta != nullptr);
-#pragma unroll
-    for (int i = 0; i < DS; i++) acc[h][i] = 0.0f;
+    for (int i = 0; i < DS; i++) sq[h * 32 * DS + d0 + i] = qr[i];
   }
-  KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
-  KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
-
+  for (int h = 0; h < G; h++) {
+    st_m[h * 256 + tid] = -1e30f; st_l[h * 256 + tid] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < DS; i++) st_a[(h * DS + i) * 256 + tid] = 0.0f;
+  }
   // the work-group whose slice holds `pos` appends the new row and keeps it in registers
   float knew[DS], vnew[DS];
   const bool owns_new = pos >= s_begin && pos < s_end;
   if (owns_new) {
     load_rot(row + qw + g * hd, knew, p.theta != nullptr);
-    float dummy[DS];
-    load_rot(row + qw + kw + g * hd, dummy, false);
+    load_rot(row + qw + kw + g * hd, vnew, false);
 #pragma unroll
     for (int i = 0; i < DS; i++) {
-      vnew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(dummy[i]));
+      vnew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(vnew[i]));
       knew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(knew[i]));
       if (hw == 0 && d0 + i < hd) {
         kc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(knew[i]);
@@ -122,113 +151,111 @@ __global__ __launch_bounds__(256) void attn_step_kernel(const AttnParams p)
       }
     }
   }
-
-  for (int j = s_begin + hw; j < s_end; j += 8) {
-    float kd[DS], vd[DS];
-    if (j == pos) {
-#pragma unroll
-      for (int i = 0; i < DS; i++) { kd[i] = knew[i]; vd[i] = vnew[i]; }
-    } else {
-#pragma unroll
-      for (int i = 0; i < DS; i++) {
-        const int d = d0 + i;
-        kd[i] = d < hd ? kv_to_float<KV_T>(kc[(int64_t)j * hd + d]) : 0.0f;
-        vd[i] = d < hd ? kv_to_float<KV_T>(vc[(int64_t)j * hd + d]) : 0.0f;
-      }
-    }
-#pragma unroll
-    for (int h = 0; h < G; h++) {
-      float s = 0.0f;
-#pragma unroll
-      for (int i = 0; i < DS; i++) s = fmaf(q[h][i], kd[i], s);
-      s = half_wave_allsum(s) * p.inv_sqrt;
-      if (p.softcap > 0.0f) s = p.softcap * tanhf(s / p.softcap);
-      const float mn = fmaxf(m[h], s);
-      const float corr = expf(m[h] - mn), pj = expf(s - mn);
-      l[h] = l[h] * corr + pj;
-#pragma unroll
-      for (int i = 0; i < DS; i++) acc[h][i] = acc[h][i] * corr + pj * vd[i];
-      m[h] = mn;
-    }
-  }
-
-  // ---- merge the 8 half-waves through LDS ----
-  __shared__ float sm[8][G], sl[8][G];
-  __shared__ float sacc[8][G][32 * DS];
-  __shared__ int s_last_flag;
-  if (l32 == 0) {
-#pragma unroll
-    for (int h = 0; h < G; h++) { sm[hw][h] = m[h]; sl[hw][h] = l[h]; }
-  }
-#pragma unroll
-  for (int h = 0; h < G; h++)
-#pragma unroll
-    for (int i = 0; i < DS; i++) sacc[hw][h][d0 + i] = acc[h][i];
   __syncthreads();
 
-  for (int o = threadIdx.x; o < G * hd; o += 256) {
-    const int h = o / hd, d = o % hd;
+  auto reduce_chunk = [&](float (&kd)[PCH][DS], float (&vd)[PCH][DS], int j0) {
+#pragma unroll
+    for (int c = 0; c < PCH; c++) {
+      if (owns_new && min(j0 + 8 * c, s_end - 1) == pos) {
+#pragma unroll
+        for (int i = 0; i < DS; i++) { kd[c][i] = knew[i]; vd[c][i] = vnew[i]; }
+      }
+    }
+#pragma unroll 1
+    for (int h = 0; h < G; h++) {
+      float qh[DS];
+#pragma unroll
+      for (int i = 0; i < DS; i++) qh[i] = sq[h * 32 * DS + d0 + i];
+      float sc[PCH], cmax = -1e30f;
+#pragma unroll
+      for (int c = 0; c < PCH; c++) {
+        float s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < DS; i++) s = fmaf(qh[i], kd[c][i], s);
+        s = half_wave_allsum(s) * p.inv_sqrt;
+        if (p.softcap > 0.0f) s = p.softcap * tanhf(s / p.softcap);
+        sc[c] = (j0 + 8 * c < s_end) ? s : -1e30f;
+        cmax = fmaxf(cmax, sc[c]);
+      }
+      const float mo = st_m[h * 256 + tid];
+      const float mn = fmaxf(mo, cmax);
+      const float corr = expf(mo - mn);
+      float lsum = 0.0f, a[DS];
+#pragma unroll
+      for (int i = 0; i < DS; i++) a[i] = st_a[(h * DS + i) * 256 + tid] * corr;
+#pragma unroll
+      for (int c = 0; c < PCH; c++) {
+        const float pj = (j0 + 8 * c < s_end) ? expf(sc[c] - mn) : 0.0f;
+        lsum += pj;
+#pragma unroll
+        for (int i = 0; i < DS; i++) a[i] = fmaf(pj, vd[c][i], a[i]);
+      }
+      st_l[h * 256 + tid] = st_l[h * 256 + tid] * corr + lsum;
+      st_m[h * 256 + tid] = mn;
+#pragma unroll
+      for (int i = 0; i < DS; i++) st_a[(h * DS + i) * 256 + tid] = a[i];
+    }
+  };
+  for (int j0 = s_begin + hw; j0 < s_end; j0 += 16 * PCH) {
+    load_chunk(kdB, vdB, j0 + 8 * PCH);
+    reduce_chunk(kdA, vdA, j0);
+    if (j0 + 8 * PCH < s_end) {
+      load_chunk(kdA, vdA, j0 + 16 * PCH);
+      reduce_chunk(kdB, vdB, j0 + 8 * PCH);
+    }
+  }
+  __syncthreads();
+
+  // ---- merge the 8 half-waves (their states sit in LDS) ----
+  for (int o = tid; o < G * hd; o += 256) {
+    const int h = o / hd, d = o % hd, src_l = d / DS, src_i = d % DS;
     float M = -1e30f;
 #pragma unroll
-    for (int w = 0; w < 8; w++) M = fmaxf(M, sm[w][h]);
+    for (int w = 0; w < 8; w++) M = fmaxf(M, st_m[h * 256 + w * 32 + src_l]);
     float L = 0.0f, A = 0.0f;
 #pragma unroll
     for (int w = 0; w < 8; w++) {
-      const float e = sl[w][h] > 0.0f ? expf(sm[w][h] - M) : 0.0f;
-      L = fmaf(sl[w][h], e, L); A = fmaf(sacc[w][h][d], e, A);
+      const float lw = st_l[h * 256 + w * 32 + src_l];
+      const float e = lw > 0.0f ? expf(st_m[h * 256 + w * 32 + src_l] - M) : 0.0f;
+      L = fmaf(lw, e, L); A = fmaf(st_a[(h * DS + src_i) * 256 + w * 32 + src_l], e, A);
     }
     const int qh = g * G + h;
     if (n_active == 1) {
       p.out[(int64_t)seq * p.out_stride + qh * hd + d] = L > 0.0f ? A * (1.0f / L) : 0.0f;
     } else {
-      // device-coherent stores: the merging work-group may sit on another XCD (its own L2)
       float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + split) * (hd + 2);
-      __hip_atomic_store(&pt[d], A, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (d == 0) {
-        __hip_atomic_store(&pt[hd], M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&pt[hd + 1], L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
+      pt[d] = A;
+      if (d == 0) { pt[hd] = M; pt[hd + 1] = L; }
     }
   }
-  if (n_active == 1) return;
+}
 
-  // ---- the last work-group of this (sequence, KV head) to arrive merges the splits ----
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // every lane's stores have been acknowledged
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int* cnt = p.counters + seq * p.kv_heads + g;
-    const int prev = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    const int last = prev == n_active - 1;
-    if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
-    s_last_flag = last;
-  }
-  __syncthreads();
-  if (!s_last_flag) return;
-  // all (M, L) pairs of the group first (independent device-coherent loads), then the accumulators in batches
-  __shared__ float mM[G][64], mL[G][64];
-  for (int i = threadIdx.x; i < G * n_active; i += 256) {
-    const int h = i / n_active, s = s_first + i % n_active;
-    const float* pt = p.part + (((int64_t)seq * p.q_heads + g * G + h) * p.n_splits + s) * (hd + 2);
-    mM[h][s - s_first] = __hip_atomic_load(&pt[hd], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    mL[h][s - s_first] = __hip_atomic_load(&pt[hd + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-  __syncthreads();
-  for (int o = threadIdx.x; o < G * hd; o += 256) {
-    const int h = o / hd, d = o % hd, qh = g * G + h;
-    const float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + s_first) * (hd + 2) + d;
-    float M = -1e30f;
-    for (int s = 0; s < n_active; s++) M = fmaxf(M, mM[h][s]);
-    float L = 0.0f, A = 0.0f;
-    for (int s0 = 0; s0 < n_active; s0 += 8) {
-      float v[8];
+// ---- merge of the split partials: one work-group per query head; all partial loads are issued together ----
+__global__ __launch_bounds__(128) void attn_merge_kernel(const AttnParams p)
+{
+  const int qh = blockIdx.x, seq = blockIdx.y;
+  const int hd = p.hd;
+  const int pos = p.pos[seq], len = pos + 1;
+  const int j_start = (p.window > 0 && len > p.window) ? len - p.window : 0;
+  const int s_first = j_start / p.split_len, s_last = pos / p.split_len;
+  const int n_active = s_last - s_first + 1;
+  if (n_active == 1) return;                       // the split kernel already wrote the final row
+  const float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + s_first) * (hd + 2);
+  __shared__ float mM[64], mL[64];
+  for (int s = threadIdx.x; s < n_active; s += blockDim.x) { mM[s] = pt[(int64_t)s * (hd + 2) + hd]; mL[s] = pt[(int64_t)s * (hd + 2) + hd + 1]; }
+  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    float A = 0.0f, L = 0.0f, M = -1e30f;
+    bool first = true;
+    for (int s0 = 0; s0 < n_active; s0 += 16) {
+      float v[16];
 #pragma unroll
-      for (int u = 0; u < 8; u++)
-        v[u] = s0 + u < n_active ? __hip_atomic_load(&pt[(int64_t)(s0 + u) * (hd + 2)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.0f;
+      for (int u = 0; u < 16; u++) v[u] = s0 + u < n_active ? pt[(int64_t)(s0 + u) * (hd + 2) + d] : 0.0f;
+      if (first) { __syncthreads(); for (int s = 0; s < n_active; s++) M = fmaxf(M, mM[s]); first = false; }
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
+      for (int u = 0; u < 16; u++) {
         if (s0 + u < n_active) {
-          const float ls = mL[h][s0 + u];
-          const float e = ls > 0.0f ? expf(mM[h][s0 + u] - M) : 0.0f;
+          const float ls = mL[s0 + u];
+          const float e = ls > 0.0f ? expf(mM[s0 + u] - M) : 0.0f;
           L = fmaf(ls, e, L); A = fmaf(v[u], e, A);
         }
       }
@@ -237,31 +264,153 @@ __global__ __launch_bounds__(256) void attn_step_kernel(const AttnParams p)
   }
 }
 
-template <int G, typename KV_T>
-static int launch_split_ds(const AttnParams& p, int n_seq, hipStream_t st)
+// ---- short contexts: one work-group of 32 half-waves per QUERY head walks the whole live range; no split,
+//      no cross-work-group merge (each extra device-coherent hand-off costs a memory round trip, ~2.5 us) ----
+template <int DS, typename KV_T>
+__global__ __launch_bounds__(1024) void attn_head_kernel(const AttnParams p)
 {
-  const dim3 grid(p.n_splits, p.kv_heads, n_seq);
-  if (p.hd <= 32) hipLaunchKernelGGL((attn_step_kernel<G, 1, KV_T>), grid, dim3(256), 0, st, p);
-  else if (p.hd <= 64) hipLaunchKernelGGL((attn_step_kernel<G, 2, KV_T>), grid, dim3(256), 0, st, p);
-  else if (p.hd <= 128) hipLaunchKernelGGL((attn_step_kernel<G, 4, KV_T>), grid, dim3(256), 0, st, p);
-  else return set_error(CAI_ERR_UNSUPPORTED, "attention: head_dim %d > 128", p.hd);
+  const int h = blockIdx.x, seq = blockIdx.y;
+  const int G = p.q_heads / p.kv_heads, g = h / G;
+  const int pos = p.pos[seq];
+  const int len = pos + 1;
+  const int j_start = (p.window > 0 && len > p.window) ? len - p.window : 0;
+  const int hw = threadIdx.x >> 5, l32 = threadIdx.x & 31;
+  const int hd = p.hd, qw = p.q_heads * hd, kw = p.kv_heads * hd;
+  const int d0 = l32 * DS;
+  const float* row = p.qkv + (int64_t)seq * p.qkv_stride;
+  KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+
+  constexpr int PCH = 4;
+  // cached rows of a chunk are all requested before any is used; the first chunk before the rotation math below
+  float kd[PCH][DS], vd[PCH][DS];
+  auto load_chunk = [&](int j0) {
+#pragma unroll
+    for (int c = 0; c < PCH; c++) {
+      const int j = min(j0 + 32 * c, len - 1);
+#pragma unroll
+      for (int i = 0; i < DS; i++) {
+        const int d = d0 + i;
+        const bool ok = d < hd && j != pos;      // the row being appended is taken from registers instead
+        kd[c][i] = ok ? kv_to_float<KV_T>(kc[(int64_t)j * hd + d]) : 0.0f;
+        vd[c][i] = ok ? kv_to_float<KV_T>(vc[(int64_t)j * hd + d]) : 0.0f;
+      }
+    }
+  };
+  load_chunk(j_start + hw);
+
+  float rs[(DS + 1) / 2], rc[(DS + 1) / 2];
+#pragma unroll
+  for (int i = 0; i < (DS + 1) / 2; i++) {
+    rs[i] = 0.0f; rc[i] = 1.0f;
+    const int d = d0 + 2 * i;
+    if (p.theta && d < hd) { const float angle = (float)pos * p.theta[d >> 1]; sincosf(angle, &rs[i], &rc[i]); }
+  }
+  auto load_rot = [&](const float* v, float (&o)[DS], bool rotate) {
+    if (DS >= 2) {
+#pragma unroll
+      for (int i = 0; i < DS; i += 2) {
+        const int d = d0 + i;
+        const float x0 = d < hd ? v[d] : 0.0f, x1 = d + 1 < hd ? v[d + 1] : 0.0f;
+        if (rotate) { o[i] = rc[i / 2] * x0 - rs[i / 2] * x1; o[i + (DS > 1 ? 1 : 0)] = rs[i / 2] * x0 + rc[i / 2] * x1; }
+        else { o[i] = x0; o[i + (DS > 1 ? 1 : 0)] = x1; }
+      }
+    } else {
+      const int d = d0;
+      const float own = d < hd ? v[d] : 0.0f, mate = (d ^ 1) < hd ? v[d ^ 1] : 0.0f;
+      if (rotate) o[0] = (d & 1) ? (rs[0] * mate + rc[0] * own) : (rc[0] * own - rs[0] * mate);
+      else o[0] = own;
+    }
+  };
+  float q[DS], knew[DS], vnew[DS], acc[DS];
+  load_rot(row + h * hd, q, p.theta != nullptr);
+  load_rot(row + qw + g * hd, knew, p.theta != nullptr);
+  load_rot(row + qw + kw + g * hd, vnew, false);
+#pragma unroll
+  for (int i = 0; i < DS; i++) {
+    knew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(knew[i]));
+    vnew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(vnew[i]));
+    acc[i] = 0.0f;
+    if (h == g * G && hw == 0 && d0 + i < hd) {   // the first query head of the group appends the row
+      kc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(knew[i]);
+      vc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(vnew[i]);
+    }
+  }
+  float m = -1e30f, l = 0.0f;
+  for (int j0 = j_start + hw; j0 < len; j0 += 32 * PCH) {
+    float sc[PCH], cmax = -1e30f;
+#pragma unroll
+    for (int c = 0; c < PCH; c++) {
+      if (min(j0 + 32 * c, len - 1) == pos) {
+#pragma unroll
+        for (int i = 0; i < DS; i++) { kd[c][i] = knew[i]; vd[c][i] = vnew[i]; }
+      }
+      float s = 0.0f;
+#pragma unroll
+      for (int i = 0; i < DS; i++) s = fmaf(q[i], kd[c][i], s);
+      s = half_wave_allsum(s) * p.inv_sqrt;
+      if (p.softcap > 0.0f) s = p.softcap * tanhf(s / p.softcap);
+      sc[c] = (j0 + 32 * c < len) ? s : -1e30f;
+      cmax = fmaxf(cmax, sc[c]);
+    }
+    const float mn = fmaxf(m, cmax), corr = expf(m - mn);
+    float lsum = 0.0f, a[DS];
+#pragma unroll
+    for (int i = 0; i < DS; i++) a[i] = acc[i] * corr;
+#pragma unroll
+    for (int c = 0; c < PCH; c++) {
+      const float pj = (j0 + 32 * c < len) ? expf(sc[c] - mn) : 0.0f;
+      lsum += pj;
+#pragma unroll
+      for (int i = 0; i < DS; i++) a[i] = fmaf(pj, vd[c][i], a[i]);
+    }
+    if (j0 + 32 * PCH < len) load_chunk(j0 + 32 * PCH);   // request the next chunk (this one is consumed)
+    l = l * corr + lsum; m = mn;
+#pragma unroll
+    for (int i = 0; i < DS; i++) acc[i] = a[i];
+  }
+  __shared__ float sm[32], sl[32];
+  __shared__ float sacc[32][32 * DS];
+  if (l32 == 0) { sm[hw] = m; sl[hw] = l; }
+#pragma unroll
+  for (int i = 0; i < DS; i++) sacc[hw][d0 + i] = acc[i];
+  __syncthreads();
+  for (int d = threadIdx.x; d < hd; d += 1024) {
+    float M = -1e30f;
+#pragma unroll
+    for (int w = 0; w < 32; w++) M = fmaxf(M, sm[w]);
+    float L = 0.0f, A = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 32; w++) {
+      const float e = sl[w] > 0.0f ? expf(sm[w] - M) : 0.0f;
+      L = fmaf(sl[w], e, L); A = fmaf(sacc[w][d], e, A);
+    }
+    p.out[(int64_t)seq * p.out_stride + h * hd + d] = L > 0.0f ? A * (1.0f / L) : 0.0f;
+  }
+}
+
+template <typename KV_T>
+static int launch_head_kernel(const AttnParams& p, int n_seq, hipStream_t st)
+{
+  const dim3 grid(p.q_heads, n_seq);
+  if (p.hd <= 32) hipLaunchKernelGGL((attn_head_kernel<1, KV_T>), grid, dim3(1024), 0, st, p);
+  else if (p.hd <= 64) hipLaunchKernelGGL((attn_head_kernel<2, KV_T>), grid, dim3(1024), 0, st, p);
+  else hipLaunchKernelGGL((attn_head_kernel<4, KV_T>), grid, dim3(1024), 0, st, p);
   return CAI_OK;
 }
 
 template <typename KV_T>
 static int launch_split_g(const AttnParams& p, int n_seq, hipStream_t st)
 {
-  switch (p.q_heads / p.kv_heads) {
-    case 1: return launch_split_ds<1, KV_T>(p, n_seq, st);
-    case 2: return launch_split_ds<2, KV_T>(p, n_seq, st);
-    case 3: return launch_split_ds<3, KV_T>(p, n_seq, st);
-    case 4: return launch_split_ds<4, KV_T>(p, n_seq, st);
-    case 5: return launch_split_ds<5, KV_T>(p, n_seq, st);
-    case 6: return launch_split_ds<6, KV_T>(p, n_seq, st);
-    case 7: return launch_split_ds<7, KV_T>(p, n_seq, st);
-    case 8: return launch_split_ds<8, KV_T>(p, n_seq, st);
-  }
-  return set_error(CAI_ERR_UNSUPPORTED, "attention: %d query heads per KV head (supported 1..8)", p.q_heads / p.kv_heads);
+  const int G = p.q_heads / p.kv_heads;
+  if (G < 1 || G > 8) return set_error(CAI_ERR_UNSUPPORTED, "attention: %d query heads per KV head (supported 1..8)", G);
+  const dim3 grid(p.n_splits, p.kv_heads, n_seq);
+  auto lds = [&](int ds) { return (size_t)(G * 32 * ds + G * 256 * (2 + ds)) * sizeof(float); };
+  if (p.hd <= 32) hipLaunchKernelGGL((attn_step_kernel<1, KV_T>), grid, dim3(256), lds(1), st, p);
+  else if (p.hd <= 64) hipLaunchKernelGGL((attn_step_kernel<2, KV_T>), grid, dim3(256), lds(2), st, p);
+  else if (p.hd <= 128) hipLaunchKernelGGL((attn_step_kernel<4, KV_T>), grid, dim3(256), lds(4), st, p);
+  else return set_error(CAI_ERR_UNSUPPORTED, "attention: head_dim %d > 128", p.hd);
+  return CAI_OK;
 }
 
 int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, int n_seq, int q_heads, int window,
@@ -280,8 +429,14 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   p.theta = theta; p.pos = pos_dev; p.split_len = kv->split_len; p.n_splits = kv->n_splits;
   p.part = kv->part; p.out = out; p.out_stride = out_stride; p.seq0 = seq0;
   p.counters = kv->d_counters;
-  if (kv->dtype == CAI_KV_F16) return launch_split_g<__half>(p, n_seq, c.stream);
-  return launch_split_g<float>(p, n_seq, c.stream);
+  if (kv->max_ctx <= kv->short_ctx_limit) {
+    if (kv->dtype == CAI_KV_F16) return launch_head_kernel<__half>(p, n_seq, c.stream);
+    return launch_head_kernel<float>(p, n_seq, c.stream);
+  }
+  const int rc = kv->dtype == CAI_KV_F16 ? launch_split_g<__half>(p, n_seq, c.stream) : launch_split_g<float>(p, n_seq, c.stream);
+  if (rc) return rc;
+  if (p.n_splits > 1) hipLaunchKernelGGL(attn_merge_kernel, dim3(q_heads, n_seq), dim3(128), 0, c.stream, p);
+  return CAI_OK;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -294,13 +449,20 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   if (dtype != CAI_KV_F32 && dtype != CAI_KV_F16) return set_error(CAI_ERR_INVALID, "kv cache: dtype %d", dtype);
   kv->n_seq = n_seq; kv->n_layers = n_layers; kv->kv_heads = kv_heads; kv->head_dim = head_dim; kv->max_ctx = max_ctx; kv->dtype = dtype;
   kv->len.assign((size_t)n_seq * n_layers, 0);
-  int sl = (max_ctx + 47) / 48; sl = (sl + 31) / 32 * 32; if (sl < 32) sl = 32;
-  kv->split_len = sl; kv->n_splits = (max_ctx + sl - 1) / sl;   // <= 48 by construction (the merge stage holds 64)
+  // few, fat splits: every extra split costs the merging work-group another device-coherent load round,
+  // while one CU sustains only ~20 GB/s, so a slice should stay under ~100 KB
+  int sl = (max_ctx + 15) / 16; sl = (sl + 31) / 32 * 32; if (sl < 32) sl = 32; if (sl > 256) sl = 256;
+  kv->split_len = sl; kv->n_splits = (max_ctx + sl - 1) / sl;   // the merge stage holds up to 64 splits
   const size_t bytes = (size_t)kv->seq_elems() * n_seq * kv->elem();
+  if (kv->n_splits > 64) return set_error(CAI_ERR_UNSUPPORTED, "kv cache: max_ctx %d needs %d splits (limit 64 x 256 rows)", max_ctx, kv->n_splits);
   CAI_HIP(hipMalloc(&kv->k, bytes));
   CAI_HIP(hipMalloc(&kv->v, bytes));
   CAI_HIP(hipMemsetAsync(kv->k, 0, bytes, ctx().stream));
   CAI_HIP(hipMemsetAsync(kv->v, 0, bytes, ctx().stream));
+  {
+    const char* e = getenv("CAIHIP_ATTN_SHORT_CTX");      // caches up to this length use the per-head kernel
+    kv->short_ctx_limit = e ? atoi(e) : 0;
+  }
   kv->part_q_heads = kv_heads * 8;
   CAI_HIP(hipMalloc(&kv->part, (size_t)n_seq * kv->part_q_heads * kv->n_splits * (head_dim + 2) * sizeof(float)));
   CAI_HIP(hipMalloc(&kv->d_len, sizeof(int32_t) * n_seq));

@@ -23,6 +23,7 @@ struct cai_decoder_s {
   float *router_logits = nullptr, *router_probs = nullptr, *moe_gate = nullptr, *moe_part = nullptr;
   int32_t* moe_expert = nullptr;
   float* am_v = nullptr; int32_t* am_i = nullptr;   // arg-max slice winners
+  float* ssq = nullptr;                              // 2 x 1024 sum-of-squares partials (RMSNorm hand-off)
   int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_argmax = nullptr, *d_gen = nullptr;
   int32_t* h_io = nullptr;   // pinned: tokens[8] pos[8] argmax[8]
   hipGraphExec_t graph[9] = {nullptr};
@@ -71,6 +72,9 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
   const int dm = c.d_model, qw = d->qw(), kw = d->kw(), I = c.ffn, qkvw = qw + 2 * kw;
   int rc;
   if ((rc = launch_embed(d->embed, d->d_tokens, n_b, d->x))) return rc;
+  float* ssq_o = d->ssq;          // written by the o-projection, read by gate|up
+  float* ssq_d = d->ssq + 1024;   // written by the down projection, read by the next block's q|k|v
+  bool have_ssq_d = false;
   for (int l = 0; l < c.n_layers; l++) {
     auto& L = d->layers[l];
     // --- attention half ---
@@ -82,6 +86,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
         m.w[i] = L.w[slots[i]]; m.row0[i] = 0; m.rows[i] = m.w[i]->rows; m.y_off[i] = offs[i];
         same = same && m.w[i]->qtype == m.w[0]->qtype;
       }
+      if (same && have_ssq_d && gemv_hands_off_ssq(m.w[0], n_b)) m.ssq_in = ssq_d;
       if (same) {
         if ((rc = launch_gemv_multi(m, d->x, n_b, d->qkv, qkvw, CAI_ACT_NONE, nullptr, L.v[CAI_V_ATTN_NORM], c.eps, 0))) return rc;
       } else {
@@ -96,17 +101,29 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
       launch_rmsnorm_strided(d->qkv + qw, L.v[CAI_V_K_NORM], kw, n_b, c.eps, d->qkv + qw, qkvw, qkvw);
     }
     if ((rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0))) return rc;
-    if ((rc = launch_gemv(L.w[CAI_W_O], 0, dm, d->att, n_b, d->x, dm, CAI_ACT_NONE, d->x))) return rc;
+    const bool o_hands = gemv_hands_off_ssq(L.w[CAI_W_O], n_b);
+    {
+      MultiGemv m{}; m.n = 1; m.w[0] = L.w[CAI_W_O]; m.rows[0] = dm;
+      if (o_hands) m.ssq_out = ssq_o;
+      if ((rc = launch_gemv_multi(m, d->att, n_b, d->x, dm, CAI_ACT_NONE, d->x, nullptr, 0.0f, 0))) return rc;
+    }
+    have_ssq_d = false;
     // --- feed-forward half ---
     if (c.n_experts == 0) {
       MultiGemv m{}; m.n = 1; m.w[0] = L.w[CAI_W_GATEUP]; m.rows[0] = 2 * I;
+      if (o_hands && gemv_hands_off_ssq(m.w[0], n_b)) m.ssq_in = ssq_o;
       if (is_block_quant(m.w[0]->qtype)) {
         if ((rc = launch_gemv_multi(m, d->x, n_b, d->mid, I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, I))) return rc;
       } else {
         if ((rc = launch_gemv_multi(m, d->x, n_b, d->gu, 2 * I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;
         launch_swiglu(d->gu, I, n_b, d->mid);
       }
-      if ((rc = launch_gemv(L.w[CAI_W_DOWN], 0, dm, d->mid, n_b, d->x, dm, CAI_ACT_NONE, d->x))) return rc;
+      {
+        MultiGemv dn{}; dn.n = 1; dn.w[0] = L.w[CAI_W_DOWN]; dn.rows[0] = dm;
+        have_ssq_d = gemv_hands_off_ssq(dn.w[0], n_b);
+        if (have_ssq_d) dn.ssq_out = ssq_d;
+        if ((rc = launch_gemv_multi(dn, d->mid, n_b, d->x, dm, CAI_ACT_NONE, d->x, nullptr, 0.0f, 0))) return rc;
+      }
     } else {
       const int E = c.n_experts, K = c.top_k;
       MultiGemv r{}; r.n = 1; r.w[0] = L.w[CAI_W_ROUTER]; r.rows[0] = E;
@@ -134,6 +151,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
   {
     cai_qw_s* hw = d->head ? d->head : d->embed;   // tied head (neural/neuralpretrained.pas:15555-)
     MultiGemv m{}; m.n = 1; m.w[0] = hw; m.rows[0] = c.vocab;
+    if (have_ssq_d && gemv_hands_off_ssq(hw, n_b)) m.ssq_in = ssq_d;
     if ((rc = launch_gemv_multi(m, d->x, n_b, d->logits, c.vocab, CAI_ACT_NONE, nullptr, d->final_norm, c.eps, 0))) return rc;
   }
   launch_argmax(d->logits, c.vocab, n_b, d->d_argmax, d->am_v, d->am_i);
@@ -199,6 +217,7 @@ extern "C" int cai_decoder_create(const cai_decoder_config* cfg, cai_decoder_t* 
   const int ame = argmax_scratch_entries(c.vocab, B);
   if (e == hipSuccess) e = alloc_f(&d->am_v, (size_t)ame);
   if (e == hipSuccess) e = hipMalloc((void**)&d->am_i, (size_t)ame * sizeof(int32_t));
+  if (e == hipSuccess) e = alloc_f(&d->ssq, 2 * 1024);
   if (e == hipSuccess) e = hipMalloc((void**)&d->d_tokens, 3 * 8 * sizeof(int32_t));
   if (e == hipSuccess) e = hipMalloc((void**)&d->d_gen, (size_t)c.max_ctx * sizeof(int32_t));
   if (e == hipSuccess) e = hipHostMalloc((void**)&d->h_io, 3 * 8 * sizeof(int32_t), hipHostMallocDefault);
@@ -218,7 +237,7 @@ extern "C" int cai_decoder_destroy(cai_decoder_t d)
   if (ctx().ready) (void)hipStreamSynchronize(ctx().stream);
   invalidate_graphs(d);
   kv_free(&d->kv);
-  float* fs[] = {d->theta, d->x, d->qkv, d->att, d->gu, d->mid, d->logits, d->router_logits, d->router_probs, d->moe_gate, d->moe_part, d->final_norm};
+  float* fs[] = {d->ssq, d->theta, d->x, d->qkv, d->att, d->gu, d->mid, d->logits, d->router_logits, d->router_probs, d->moe_gate, d->moe_part, d->final_norm};
   for (float* p : fs) if (p) (void)hipFree(p);
   for (auto& L : d->layers) for (float* p : L.v) if (p) (void)hipFree(p);
   if (d->moe_expert) (void)hipFree(d->moe_expert);

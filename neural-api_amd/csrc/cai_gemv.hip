@@ -405,6 +405,11 @@ static bool stream_kernel_enabled()
   static const int on = []() { const char* e = getenv("CAIHIP_GEMV_V1"); return (e && e[0] == '1') ? 0 : 1; }();
   return on != 0;
 }
+// True when a batch-1 launch on this matrix goes through the streaming kernel (which honours ssq_in / ssq_out).
+bool gemv_hands_off_ssq(const cai_qw_s* w, int n_b)
+{
+  return w->qtype == CAI_Q4_K && n_b == 1 && stream_kernel_enabled() && (((w->cols >> 8) + 15) >> 4) <= 8;
+}
 static bool fast_type(int qt) { return qt == CAI_Q4_K || qt == CAI_Q4_0 || qt == CAI_Q8_0; }
 
 static int panel_len(int cols, int nb)
@@ -492,6 +497,7 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
   GemvParams p{};
   p.n_seg = m.n; p.x = x; p.y = y; p.residual = residual; p.norm_gain = norm_gain; p.norm_eps = norm_eps;
   p.cols = (int)w0->cols; p.y_stride = (int)y_stride; p.act = act; p.half = swiglu_half;
+  p.ssq_in = nullptr; p.ssq_out = nullptr;
   p.slot_expert = m.slot_expert; p.expert_rows = m.expert_rows; p.x_slot_stride = m.x_slot_stride; p.y_slot_stride = m.y_slot_stride;
   const int n_slots = m.slot_expert ? m.n_slots : 1;
   for (int i = 0; i < m.n; i++) {
@@ -509,7 +515,9 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
   if (qt == CAI_Q4_K && n_b == 1 && !m.slot_expert && stream_kernel_enabled()) {
     MultiGemv mm = m;
     if (swiglu_half) { if (m.n != 1) return set_error(CAI_ERR_INVALID, "gemv: swiglu takes one matrix"); p.seg[0].rows = swiglu_half; }
+    p.ssq_in = m.ssq_in; p.ssq_out = m.ssq_out;
     const int rc = launch_q4k_stream(p, mm, swiglu_half, c.stream);
+    p.ssq_in = nullptr; p.ssq_out = nullptr;
     if (rc != CAI_ERR_UNSUPPORTED) return rc;
   }
   if (fast_type(qt)) {

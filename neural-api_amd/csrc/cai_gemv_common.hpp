@@ -42,6 +42,8 @@ __device__ __forceinline__ float silu_mul(float up, float gate)
   return up * (gate * sig);
 }
 
+constexpr int SSQ_PARTS = 1024;   // slots of a sum-of-squares partial array (>= any producer grid)
+
 struct GemvSeg {
   const uint8_t* data; const uint8_t* aux; const float* bias;
   int rows;       // rows of this segment computed by the launch
@@ -56,6 +58,8 @@ struct GemvParams {
   float* y;              // [NB][y_stride]
   const float* residual; // same indexing as y, may be null
   const float* norm_gain; float norm_eps;  // fused RMSNorm on the input when norm_gain != null
+  const float* ssq_in;   // optional: sum(x^2) as SSQ_PARTS partials written by the kernel that produced x
+  float* ssq_out;        // optional: this kernel's per-work-group partials of sum(y^2) (SSQ_PARTS slots)
   int cols;
   int kp;                // panel length in floats (multiple of 256)
   int kp_lds;            // LDS floats reserved per batch row: kp rounded up to whole 16-unit tiles

@@ -72,6 +72,7 @@ struct cai_kv_s {
   void* k = nullptr; void* v = nullptr;   // [seq][layer][kv_head][max_ctx][head_dim]
   std::vector<int> len;                   // [seq][layer] live rows (host mirror)
   int split_len = 64, n_splits = 1;       // split-K geometry of the decode kernel (fixed at creation)
+  int short_ctx_limit = 0;                // caches no longer than this use the per-query-head kernel (no split)
   float* part = nullptr;                  // [seq][q_head][split][head_dim+2] split-K partials
   int part_q_heads = 0;
   int32_t* d_len = nullptr;               // [seq] device scratch: rows live BEFORE the token being decoded
@@ -99,11 +100,15 @@ int launch_gemv(const cai_qw_s* w, int64_t row0, int64_t n_rows, const float* x,
 struct MultiGemv {
   const cai_qw_s* w[3]; int64_t row0[3]; int64_t rows[3]; int y_off[3]; int n;
   const int32_t* slot_expert; int n_slots; int64_t expert_rows; int x_slot_stride; int y_slot_stride;
+  // RMSNorm hand-off between consecutive batch-1 Q4_K layers: the producer leaves per-work-group partials of
+  // sum(y^2) (1024 floats) that the consumer sums instead of re-reducing its input.  Both optional.
+  const float* ssq_in; float* ssq_out;
 };
 // norm_gain != null fuses RMSNorm(eps) of x into the staging; swiglu_half > 0 computes
 // y[i] = up_i * silu(gate_i) from rows i and swiglu_half + i of the (single) matrix.
 int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int64_t y_stride, int act,
                       const float* residual, const float* norm_gain, float norm_eps, int swiglu_half);
+bool gemv_hands_off_ssq(const cai_qw_s* w, int n_b);
 int launch_dequant_rows(const cai_qw_s* w, int64_t row0, int64_t n_rows, float* out);
 int launch_rmsnorm(const float* x, const float* gain, int n, int n_tokens, float eps, float* y);
 int launch_rope(float* x, int n_heads, int head_dim, const int32_t* pos_dev, int pos_host, const float* theta, int n_tokens, int64_t token_stride);
