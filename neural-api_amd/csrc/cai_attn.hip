@@ -47,6 +47,9 @@ struct AttnParams {
   float* part;                 // [seq][q_head][split][hd+2]
   float* out; int64_t out_stride;
   int seq0;                    // cache sequence index of activation row 0
+  int seq_mul;                 // 1: activation row s uses cache sequence seq0 + s; 0: all rows share sequence seq0 (prompt)
+  int appended;                // 1: the K,V rows of this step are already in the cache (prompt ingestion)
+  float* part_override;        // split partials buffer when more rows than cache sequences are in flight
   int* counters;               // [seq][kv_head] arrival counters of the split merge (zero between launches)
 };
 
@@ -72,8 +75,8 @@ __global__ __launch_bounds__(256) void attn_step_kernel(const AttnParams p)
   const int G = p.q_heads / p.kv_heads;
   const int d0 = l32 * DS;
   const float* row = p.qkv + (int64_t)seq * p.qkv_stride;
-  KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
-  KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (seq * p.seq_mul + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (seq * p.seq_mul + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
 
   // LDS: rotated q [G][32*DS] | state m,l [G][256] each | acc [G][DS][256]
   float* sq = lds;
@@ -91,7 +94,7 @@ __global__ __launch_bounds__(256) void attn_step_kernel(const AttnParams p)
 #pragma unroll
       for (int i = 0; i < DS; i++) {
         const int d = d0 + i;
-        const bool ok = d < hd && j != pos;   // the appended row comes from registers
+        const bool ok = d < hd && (j != pos || p.appended);   // the row appended here comes from registers
         kd[c][i] = ok ? kv_to_float<KV_T>(kc[(int64_t)j * hd + d]) : 0.0f;
         vd[c][i] = ok ? kv_to_float<KV_T>(vc[(int64_t)j * hd + d]) : 0.0f;
       }
@@ -137,7 +140,7 @@ __global__ __launch_bounds__(256) void attn_step_kernel(const AttnParams p)
   }
   // the work-group whose slice holds `pos` appends the new row and keeps it in registers
   float knew[DS], vnew[DS];
-  const bool owns_new = pos >= s_begin && pos < s_end;
+  const bool owns_new = !p.appended && pos >= s_begin && pos < s_end;
   if (owns_new) {
     load_rot(row + qw + g * hd, knew, p.theta != nullptr);
     load_rot(row + qw + kw + g * hd, vnew, false);
@@ -413,12 +416,41 @@ static int launch_split_g(const AttnParams& p, int n_seq, hipStream_t st)
   return CAI_OK;
 }
 
+// Prompt ingestion: rotate the K rows of n_tok tokens at their positions and write K,V into sequence `seq`.
+template <typename KV_T>
+__global__ __launch_bounds__(256) void kv_append_rows_kernel(const AttnParams p)
+{
+  const int b = blockIdx.x;
+  const float* row = p.qkv + (int64_t)b * p.qkv_stride;
+  const int pos = p.pos[b];
+  const int hd = p.hd, qw = p.q_heads * hd, kw = p.kv_heads * hd;
+  KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (int64_t)p.seq0 * p.seq_elems + p.layer_off;
+  KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (int64_t)p.seq0 * p.seq_elems + p.layer_off;
+  for (int i = threadIdx.x; i < (kw >> 1); i += 256) {
+    const int e = 2 * i, g = e / hd, d = e % hd;
+    float x0 = row[qw + e], x1 = row[qw + e + 1];
+    if (p.theta) {
+      const float angle = (float)pos * p.theta[d >> 1];
+      float sn, cs; sincosf(angle, &sn, &cs);
+      const float y0 = cs * x0 - sn * x1, y1 = sn * x0 + cs * x1;
+      x0 = y0; x1 = y1;
+    }
+    KV_T* dst = kc + ((int64_t)g * p.max_ctx + pos) * hd + d;
+    dst[0] = kv_from_float<KV_T>(x0); dst[1] = kv_from_float<KV_T>(x1);
+  }
+  for (int i = threadIdx.x; i < kw; i += 256) {
+    const int g = i / hd, d = i % hd;
+    vc[((int64_t)g * p.max_ctx + pos) * hd + d] = kv_from_float<KV_T>(row[qw + kw + i]);
+  }
+}
+
 int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, int n_seq, int q_heads, int window,
-                     float softcap, const float* theta, const int32_t* pos_dev, float* out, int64_t out_stride, int seq0)
+                     float softcap, const float* theta, const int32_t* pos_dev, float* out, int64_t out_stride, int seq0,
+                     int prompt_rows, float* prompt_part)
 {
   Context& c = ctx();
   if (layer < 0 || layer >= kv->n_layers) return set_error(CAI_ERR_INVALID, "attention: layer %d of %d", layer, kv->n_layers);
-  if (n_seq < 1 || seq0 < 0 || seq0 + n_seq > kv->n_seq) return set_error(CAI_ERR_INVALID, "attention: %d sequences, cache holds %d", n_seq, kv->n_seq);
+  if (n_seq < 1 || seq0 < 0 || seq0 + (prompt_rows ? 1 : n_seq) > kv->n_seq) return set_error(CAI_ERR_INVALID, "attention: %d sequences, cache holds %d", n_seq, kv->n_seq);
   if (q_heads % kv->kv_heads) return set_error(CAI_ERR_INVALID, "attention: %d query heads not a multiple of %d KV heads", q_heads, kv->kv_heads);
   if (q_heads > kv->part_q_heads) return set_error(CAI_ERR_INVALID, "attention: %d query heads exceed the cache's scratch (%d)", q_heads, kv->part_q_heads);
   AttnParams p{};
@@ -427,9 +459,14 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   p.q_heads = q_heads; p.kv_heads = kv->kv_heads; p.hd = kv->head_dim; p.max_ctx = kv->max_ctx;
   p.window = window; p.softcap = softcap; p.inv_sqrt = 1.0f / sqrtf((float)kv->head_dim);
   p.theta = theta; p.pos = pos_dev; p.split_len = kv->split_len; p.n_splits = kv->n_splits;
-  p.part = kv->part; p.out = out; p.out_stride = out_stride; p.seq0 = seq0;
+  p.part = prompt_rows ? prompt_part : kv->part; p.out = out; p.out_stride = out_stride; p.seq0 = seq0;
+  p.seq_mul = prompt_rows ? 0 : 1; p.appended = prompt_rows ? 1 : 0;
+  if (prompt_rows) {
+    if (kv->dtype == CAI_KV_F16) hipLaunchKernelGGL(kv_append_rows_kernel<__half>, dim3(n_seq), dim3(256), 0, c.stream, p);
+    else hipLaunchKernelGGL(kv_append_rows_kernel<float>, dim3(n_seq), dim3(256), 0, c.stream, p);
+  }
   p.counters = kv->d_counters;
-  if (kv->max_ctx <= kv->short_ctx_limit) {
+  if (!prompt_rows && kv->max_ctx <= kv->short_ctx_limit) {
     if (kv->dtype == CAI_KV_F16) return launch_head_kernel<__half>(p, n_seq, c.stream);
     return launch_head_kernel<float>(p, n_seq, c.stream);
   }
@@ -623,7 +660,7 @@ extern "C" int cai_attn_decode(cai_kv_t kv, int layer, const float* qkv, int q_h
   if (!(flags & CAI_Y_DEVICE)) { rc = ensure_stage(&c.stage_out, &c.stage_out_cap, out_b); if (rc) return rc; d_out = (float*)c.stage_out; }
   c.h_small[0] = len;
   CAI_HIP(hipMemcpyAsync(kv->d_len, c.h_small, sizeof(int32_t), hipMemcpyHostToDevice, c.stream));
-  rc = launch_attn_step(kv, layer, (float*)c.stage_in, 0, 1, q_heads, window, softcap, nullptr, kv->d_len, d_out, 0, 0);
+  rc = launch_attn_step(kv, layer, (float*)c.stage_in, 0, 1, q_heads, window, softcap, nullptr, kv->d_len, d_out, 0, 0, 0, nullptr);
   if (rc) return rc;
   if (!(flags & CAI_Y_DEVICE)) CAI_HIP(hipMemcpyAsync(out, d_out, out_b, hipMemcpyDeviceToHost, c.stream));
   CAI_HIP(hipStreamSynchronize(c.stream));

@@ -24,6 +24,10 @@ struct cai_decoder_s {
   int32_t* moe_expert = nullptr;
   float* am_v = nullptr; int32_t* am_i = nullptr;   // arg-max slice winners
   float* ssq = nullptr;                              // 2 x 1024 sum-of-squares partials (RMSNorm hand-off)
+  // prompt ingestion (multi-token) buffers, allocated at the first prefill: rows of up to pf_cap tokens
+  int pf_cap = 0;
+  float *px = nullptr, *pqkv = nullptr, *patt = nullptr, *pgu = nullptr, *pmid = nullptr, *ppart = nullptr;
+  int32_t* ptokpos = nullptr;                        // [2][pf_cap]: tokens, positions
   int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_argmax = nullptr, *d_gen = nullptr;
   int32_t* h_io = nullptr;   // pinned: tokens[8] pos[8] argmax[8]
   hipGraphExec_t graph[9] = {nullptr};
@@ -158,6 +162,70 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
   return CAI_OK;
 }
 
+
+// Multi-token prompt ingestion of one chunk (n <= pf_cap tokens of sequence `seq` at positions pos0..): every linear
+// layer runs once for the whole chunk (matrix cores for Q4_K), K,V rows are appended, then each token attends up to
+// its own position.  Equals n sequential steps (the reference's prefill, neural/neuralchatengine.pas:1466-1470).
+static int ensure_prefill_buffers(cai_decoder_s* d, int n)
+{
+  if (d->pf_cap >= n) return CAI_OK;
+  const cai_decoder_config& c = d->cfg;
+  const int cap = std::max(n, 128);
+  CAI_HIP(hipStreamSynchronize(ctx().stream));
+  { float* pf[] = {d->px, d->pqkv, d->patt, d->pgu, d->pmid, d->ppart}; for (float* q : pf) if (q) (void)hipFree(q); }
+  if (d->ptokpos) (void)hipFree(d->ptokpos);
+  d->px = d->pqkv = d->patt = d->pgu = d->pmid = d->ppart = nullptr; d->ptokpos = nullptr; d->pf_cap = 0;
+  const size_t qkvw = d->qw() + 2 * d->kw();
+  CAI_HIP(hipMalloc((void**)&d->px, (size_t)cap * c.d_model * 4));
+  CAI_HIP(hipMalloc((void**)&d->pqkv, (size_t)cap * qkvw * 4));
+  CAI_HIP(hipMalloc((void**)&d->patt, (size_t)cap * d->qw() * 4));
+  CAI_HIP(hipMalloc((void**)&d->pgu, (size_t)cap * 2 * c.ffn * 4));
+  CAI_HIP(hipMalloc((void**)&d->pmid, (size_t)cap * c.ffn * 4));
+  CAI_HIP(hipMalloc((void**)&d->ppart, (size_t)cap * c.n_q_heads * d->kv.n_splits * (c.head_dim + 2) * 4));
+  CAI_HIP(hipMalloc((void**)&d->ptokpos, (size_t)cap * 2 * sizeof(int32_t)));
+  d->pf_cap = cap;
+  return CAI_OK;
+}
+
+static int linear_rows(const cai_qw_s* w, bool prepped, const float* x, int64_t x_stride, const float* gain, float eps, int n,
+                       float* y, int64_t y_stride, const float* residual)
+{
+  if (gemm_mfma_supported(w)) {
+    int rc;
+    if (!prepped && (rc = prefill_prep(x, x_stride, gain, eps, (int)w->cols, n))) return rc;
+    return prefill_gemm(w, n, y, y_stride, residual);
+  }
+  return prefill_linear(w, x, x_stride, gain, eps, n, y, y_stride, residual);
+}
+
+static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
+{
+  const cai_decoder_config& c = d->cfg;
+  const int dm = c.d_model, qw = d->qw(), kw = d->kw(), I = c.ffn, qkvw = qw + 2 * kw;
+  const int32_t* toks = d->ptokpos; const int32_t* poss = d->ptokpos + d->pf_cap;
+  int rc;
+  if ((rc = launch_embed(d->embed, toks, n, d->px))) return rc;
+  for (int l = 0; l < c.n_layers; l++) {
+    auto& L = d->layers[l];
+    const cai_qw_s* wq = L.w[CAI_W_Q]; const cai_qw_s* wk = L.w[CAI_W_K]; const cai_qw_s* wv = L.w[CAI_W_V];
+    const bool all_mfma = gemm_mfma_supported(wq) && gemm_mfma_supported(wk) && gemm_mfma_supported(wv);
+    if (all_mfma && (rc = prefill_prep(d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, dm, n))) return rc;
+    if ((rc = linear_rows(wq, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv, qkvw, nullptr))) return rc;
+    if ((rc = linear_rows(wk, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw, qkvw, nullptr))) return rc;
+    if ((rc = linear_rows(wv, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw + kw, qkvw, nullptr))) return rc;
+    if (c.qk_norm_full) {
+      launch_rmsnorm_strided(d->pqkv, L.v[CAI_V_Q_NORM], qw, n, c.eps, d->pqkv, qkvw, qkvw);
+      launch_rmsnorm_strided(d->pqkv + qw, L.v[CAI_V_K_NORM], kw, n, c.eps, d->pqkv + qw, qkvw, qkvw);
+    }
+    if ((rc = launch_attn_step(&d->kv, l, d->pqkv, qkvw, n, c.n_q_heads, c.window, 0.0f, d->theta, poss, d->patt, qw, seq, 1, d->ppart))) return rc;
+    if ((rc = linear_rows(L.w[CAI_W_O], false, d->patt, qw, nullptr, 0.0f, n, d->px, dm, d->px))) return rc;
+    if ((rc = linear_rows(L.w[CAI_W_GATEUP], false, d->px, dm, L.v[CAI_V_MLP_NORM], c.eps, n, d->pgu, 2 * I, nullptr))) return rc;
+    launch_swiglu(d->pgu, I, n, d->pmid);
+    if ((rc = linear_rows(L.w[CAI_W_DOWN], false, d->pmid, I, nullptr, 0.0f, n, d->px, dm, d->px))) return rc;
+  }
+  return CAI_OK;
+}
+
 static int run_step(cai_decoder_s* d, int n_b)
 {
   Context& c = ctx();
@@ -240,6 +308,8 @@ extern "C" int cai_decoder_destroy(cai_decoder_t d)
   float* fs[] = {d->ssq, d->theta, d->x, d->qkv, d->att, d->gu, d->mid, d->logits, d->router_logits, d->router_probs, d->moe_gate, d->moe_part, d->final_norm};
   for (float* p : fs) if (p) (void)hipFree(p);
   for (auto& L : d->layers) for (float* p : L.v) if (p) (void)hipFree(p);
+  { float* pf[] = {d->px, d->pqkv, d->patt, d->pgu, d->pmid, d->ppart}; for (float* q : pf) if (q) (void)hipFree(q); }
+  if (d->ptokpos) (void)hipFree(d->ptokpos);
   if (d->moe_expert) (void)hipFree(d->moe_expert);
   if (d->am_v) (void)hipFree(d->am_v);
   if (d->am_i) (void)hipFree(d->am_i);
@@ -360,13 +430,36 @@ extern "C" int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* toke
   if (pos0 + n > c.max_ctx) return set_error(CAI_ERR_STATE, "cai_decoder_prefill: %d tokens from %d exceed max_ctx %d", n, pos0, c.max_ctx);
   for (int i = 0; i < n; i++) CAI_REQUIRE(tokens[i] >= 0 && tokens[i] < c.vocab, "cai_decoder_prefill: token %d outside vocab %d", tokens[i], c.vocab);
   Context& cx = ctx();
-  // Token-at-a-time ingestion, the reference's own prefill (neural/neuralchatengine.pas:1466-1470).
-  for (int i = 0; i < n; i++) {
-    CAI_HIP(hipStreamSynchronize(cx.stream));   // h_io is reused
-    d->h_io[0] = tokens[i]; d->h_io[8] = pos0 + i;
-    CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
-    if (seq == 0) { if ((rc = run_step(d, 1))) return rc; }
-    else { if ((rc = enqueue_step(d, 1, seq))) return rc; }
+  const char* tok_env = getenv("CAIHIP_PREFILL_TOKENWISE");
+  const bool tokenwise = c.n_experts > 0 || n == 1 || (tok_env && tok_env[0] == '1');
+  if (tokenwise) {
+    // Token-at-a-time ingestion, the reference's own prefill (neural/neuralchatengine.pas:1466-1470).
+    for (int i = 0; i < n; i++) {
+      CAI_HIP(hipStreamSynchronize(cx.stream));   // h_io is reused
+      d->h_io[0] = tokens[i]; d->h_io[8] = pos0 + i;
+      CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
+      if (seq == 0) { if ((rc = run_step(d, 1))) return rc; }
+      else { if ((rc = enqueue_step(d, 1, seq))) return rc; }
+    }
+  } else {
+    const int chunk = 512;
+    if ((rc = ensure_prefill_buffers(d, std::min(n, chunk)))) return rc;
+    std::vector<int32_t> tp((size_t)2 * d->pf_cap);
+    for (int t0 = 0; t0 < n; t0 += chunk) {
+      const int m = std::min(chunk, n - t0);
+      for (int i = 0; i < m; i++) { tp[i] = tokens[t0 + i]; tp[d->pf_cap + i] = pos0 + t0 + i; }
+      CAI_HIP(hipMemcpyAsync(d->ptokpos, tp.data(), tp.size() * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
+      CAI_HIP(hipStreamSynchronize(cx.stream));
+      if ((rc = enqueue_prefill_chunk(d, seq, m))) return rc;
+      CAI_HIP(hipGetLastError());
+      if (t0 + chunk >= n) {
+        // logits of the last prompt token only: final RMSNorm + vocabulary projection + arg-max on its row
+        cai_qw_s* hw = d->head ? d->head : d->embed;
+        MultiGemv hm{}; hm.n = 1; hm.w[0] = hw; hm.rows[0] = c.vocab;
+        if ((rc = launch_gemv_multi(hm, d->px + (int64_t)(m - 1) * c.d_model, 1, d->logits, c.vocab, CAI_ACT_NONE, nullptr, d->final_norm, c.eps, 0))) return rc;
+        launch_argmax(d->logits, c.vocab, 1, d->d_argmax, d->am_v, d->am_i);
+      }
+    }
   }
   if (last_logits) CAI_HIP(hipMemcpyAsync(last_logits, d->logits, (size_t)c.vocab * 4, hipMemcpyDeviceToHost, cx.stream));
   CAI_HIP(hipMemcpyAsync(d->h_io + 16, d->d_argmax, 8 * sizeof(int32_t), hipMemcpyDeviceToHost, cx.stream));
@@ -438,25 +531,3 @@ extern "C" int cai_decoder_weight_bytes(cai_decoder_t d, int64_t* out)
   return CAI_OK;
 }
 
-// cai_qgemm: multi-token linear layer. Until the matrix-core kernel is in place it walks the tokens in groups
-// of up to 8 through the small-batch kernel (same results as n_tokens GEMVs).
-extern "C" int cai_qgemm(cai_qw_t w, const float* x, int n_tokens, float* y, int flags)
-{
-  CAI_READY();
-  CAI_REQUIRE(w && x && y && n_tokens >= 1, "cai_qgemm: bad argument");
-  Context& c = ctx();
-  const size_t xb = (size_t)n_tokens * w->cols * 4, yb = (size_t)n_tokens * w->rows * 4;
-  const float* dx = x; float* dy = y; int rc;
-  if (!(flags & CAI_X_DEVICE)) {
-    if ((rc = ensure_stage(&c.stage_in, &c.stage_in_cap, xb))) return rc;
-    CAI_HIP(hipMemcpyAsync(c.stage_in, x, xb, hipMemcpyHostToDevice, c.stream));
-    dx = (const float*)c.stage_in;
-  }
-  if (!(flags & CAI_Y_DEVICE)) { if ((rc = ensure_stage(&c.stage_out, &c.stage_out_cap, yb))) return rc; dy = (float*)c.stage_out; }
-  for (int t = 0; t < n_tokens; t += 8) {
-    const int nb = std::min(8, n_tokens - t);
-    if ((rc = launch_gemv(w, 0, w->rows, dx + (int64_t)t * w->cols, nb, dy + (int64_t)t * w->rows, w->rows, CAI_ACT_NONE, nullptr))) return rc;
-  }
-  if (!(flags & CAI_Y_DEVICE)) { CAI_HIP(hipMemcpyAsync(y, dy, yb, hipMemcpyDeviceToHost, c.stream)); CAI_HIP(hipStreamSynchronize(c.stream)); }
-  return CAI_OK;
-}

@@ -123,14 +123,23 @@ int launch_moe_combine(float* x, const float* part, const float* gate, int k, in
 int launch_split_blocks(const uint8_t* raw, int block_bytes, int64_t n_blocks, uint8_t* qs, uint16_t* d);
 // qkv: [n_seq][qkv_stride] rows [Q|K|V]; theta != null applies interleaved RoPE to Q and K first.  pos_dev[s] is
 // both the rotary position and the cache slot the new K,V row goes to; the live range is [.., pos_dev[s]].
-// Activation row s uses cache sequence seq0 + s.
+// Activation row s uses cache sequence seq0 + s.  prompt_rows != 0: the n_seq rows are consecutive tokens of ONE
+// sequence (seq0): their K,V rows are appended first, then every row attends up to its own position; prompt_part must
+// hold n_seq * q_heads * n_splits * (head_dim + 2) floats.
 int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, int n_seq, int q_heads, int window,
-                     float softcap, const float* theta, const int32_t* pos_dev, float* out, int64_t out_stride, int seq0);
+                     float softcap, const float* theta, const int32_t* pos_dev, float* out, int64_t out_stride, int seq0,
+                     int prompt_rows = 0, float* prompt_part = nullptr);
 int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, int max_ctx, int dtype);
 void kv_free(cai_kv_s* kv);
 int kv_snapshot(cai_kv_s* kv, int seq, cai_kv_snap_s** out);
 int kv_restore(cai_kv_s* kv, int seq, const cai_kv_snap_s* snap);
-int launch_gemm_mfma(const cai_qw_s* w, const float* x, int n_tokens, float* y, const float* residual);
+// multi-token linear layer (matrix cores for Q4_K, small-batch kernel otherwise); gain != null fuses RMSNorm
+int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok,
+                   float* y, int64_t y_stride, const float* residual);
+bool gemm_mfma_supported(const cai_qw_s* w);
+// split pre-pass / product form: prep once, then any number of matrices of that width
+int prefill_prep(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok);
+int prefill_gemm(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride, const float* residual);
 
 void rope_thetas(float base, int head_dim, std::vector<float>& out);
 

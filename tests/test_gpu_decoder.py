@@ -150,3 +150,35 @@ def test_truncate_and_error_paths():
         dec.step(1, 8)
     dec.reset()                           # always safe after a failed step (neuralchatengine.pas:1630-1636)
     assert np.array_equal(dec.step(seq[0], 0)[1][0], full[0])
+
+
+def test_matrix_core_prefill_equals_steps_and_feeds_decode():
+    """Q4_K decoder: multi-token prompt ingestion (MFMA GEMM + prompt attention) == token-at-a-time steps; a 600-token
+    prompt crosses the 512-token chunk boundary; decode continues identically from either cache."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    s = SHAPES["qwen7b_like_q4k"]
+    cfg = dict(s["cfg"]); cfg["max_ctx"] = 700
+    spec = synthetic_spec(cfg, s["qtype"], head_qtype=s["head"], qkv_bias=True, std=0.05)
+    dec = cai.Decoder(spec, max_batch=2)
+    rng = np.random.default_rng(5)
+    for n in (7, 130, 600):
+        toks = rng.integers(0, cfg["vocab"], n).astype(np.int32)
+        dec.reset(0); dec.reset(1)
+        last = None
+        for p, t in enumerate(toks):
+            am_s, last = dec.step(int(t), p)
+        am_p, lg = dec.prefill(toks, 0, seq=1)
+        assert rel_err(lg, last[0]) < 1e-4, n
+        assert am_p == int(am_s[0])
+        assert dec.len(1) == n
+    # continue decoding on sequence 0 after a prefill there: same tokens as after the stepped prompt
+    toks = rng.integers(0, cfg["vocab"], 40).astype(np.int32)
+    dec.reset(0)
+    for p, t in enumerate(toks[:-1]):
+        dec.step(int(t), p, want_logits=False)
+    a = dec.generate(int(toks[-1]), 39, 16)
+    dec.reset(0)
+    dec.prefill(toks[:-1], 0, seq=0, want_logits=False)
+    b = dec.generate(int(toks[-1]), 39, 16)
+    assert a.tolist() == b.tolist()

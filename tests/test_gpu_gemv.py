@@ -127,3 +127,28 @@ def test_lm_head_shape_q8_0():
     want = O.gemv(O.Q8_0, raw, rows, cols, x, None, 0, 1)
     assert rel_err(got, want) < TIGHT
     assert int(np.argmax(got)) == int(np.argmax(want))
+
+
+@pytest.mark.parametrize("rows,cols,T", [(128, 256, 1), (1000, 1024, 5), (300, 3584, 128), (777, 2048, 200), (4608, 3584, 64)])
+def test_multi_token_gemm_on_matrix_cores_equals_gemv(rows, cols, T):
+    """cai_qgemm (Q4_K: MFMA with exact integer blocks and hi/lo-split activations) == T single-token layers."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    raw, rng = make(O.Q4_K, rows, cols, T)
+    x = (rng.standard_normal((T, cols)) * rng.uniform(0.01, 30.0, (T, 1))).astype(np.float32)   # very different scales per token
+    bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
+    w = cai.QWeight(O.Q4_K, rows, cols, raw, bias)
+    got = w.gemm(x)
+    want = O.gemv(O.Q4_K, raw, rows, cols, x, bias, 0, 1)
+    for t in range(T):
+        assert rel_err(got[t], want[t], floor=0.02 * cols ** 0.5 * float(np.abs(x[t]).mean())) < TIGHT, t
+
+
+def test_multi_token_gemm_other_types_and_tokens_not_multiple_of_eight():
+    from helpers.device import dev, rel_err
+    cai = dev()
+    for qt in (O.Q8_0, O.Q4_0):
+        raw, rng = make(qt, 200, 576, 9)
+        x = rng.standard_normal((13, 576)).astype(np.float32)
+        got = cai.QWeight(qt, 200, 576, raw).gemm(x)
+        assert rel_err(got, O.gemv(qt, raw, 200, 576, x, None, 0, 1)) < TIGHT
