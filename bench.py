@@ -62,6 +62,12 @@ def cpu_baseline(cfg, seconds_budget=20.0):
                       "median of %d runs, extrapolated to a full token; attention/norms excluded" % (cfg["n_layers"], reps)}
 
 
+# HBM bytes per launch of the 7B-shape gate|up kernel from hardware counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000
+# KiB, factors from a 1 GiB copy kernel): profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt.  Not measurable from
+# inside this process; re-collect when the kernel changes.
+GATEUP_TRAFFIC_BYTES = int((37514.7 * 2.000 + 3220.3 * 1.000) * 1024)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -70,6 +76,7 @@ def main():
     ap.add_argument("--config", default="qwen2.5-7b-q4k", choices=list(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernel-reps", type=int, default=5)
+    ap.add_argument("--copy-calibration", action="store_true", help="only run the 1 GiB device copy kernel 5 times (reference for traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives are part of it)" % args.gpus, file=sys.stderr)
@@ -83,6 +90,14 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr); sys.exit(3)
     cai.init(0)
+    if args.copy_calibration:
+        a = torch.ones(1 << 28, dtype=torch.float32, device="cuda"); b = torch.empty_like(a)
+        torch.cuda.synchronize()
+        for _ in range(5):
+            cai.check(cai.load().cai_dev_copy(b.data_ptr(), a.data_ptr(), a.numel() * 4))
+        cai.check(cai.load().cai_sync())
+        print(json.dumps({"copy_calibration": {"bytes_read": a.numel() * 4, "bytes_written": a.numel() * 4, "launches": 5}}))
+        return
     conf = CONFIGS[args.config]
     cfg = dict(conf["cfg"])
     prompt_len = conf["prompt"]
@@ -96,14 +111,21 @@ def main():
     torch.cuda.empty_cache()
     t_build = time.time() - t0
     wbytes = dec.weight_bytes()
+    n_lin_weights = cfg["n_layers"] * (cfg["d_model"] * (cfg["n_q_heads"] + 2 * cfg["n_kv_heads"]) * cfg["head_dim"] + cfg["n_q_heads"] * cfg["head_dim"] * cfg["d_model"] + 3 * cfg["ffn"] * cfg["d_model"])
 
     rng = np.random.default_rng(424242)
     prompt = rng.integers(0, cfg["vocab"], prompt_len).astype(np.int32)
-    am, _ = dec.prefill(prompt[:-1], 0, want_logits=False) if prompt_len > 1 else (0, None)
+    lib = cai.load()
+    pf_ms = C.c_float(0)
+    if prompt_len > 1:
+        dec.prefill(prompt[:min(8, prompt_len - 1)], 0, want_logits=False)   # warm the prefill kernels and buffers
+        dec.reset()
+        cai.check(lib.cai_sync()); cai.check(lib.cai_timer_start())
+        dec.prefill(prompt[:-1], 0, want_logits=False)
+        cai.check(lib.cai_timer_stop(C.byref(pf_ms)))
     tok = int(prompt[-1]); pos = prompt_len - 1
     if W > 0:
         out = dec.generate(tok, pos, W); tok = int(out[-1]); pos += W
-    lib = cai.load()
     cai.check(lib.cai_sync()); torch.cuda.synchronize()
     ms = C.c_float()
     t1 = time.perf_counter()
@@ -148,10 +170,15 @@ def main():
                    "weights": "random N(0,0.02), %s body + %s head, fp32 KV cache" % (conf["qtype"], conf["head"]),
                    "algorithmic_bytes_per_token": int(algo_bytes), "hip_event_ms_per_step": round(ms.value / K, 4),
                    "whole_step_hbm_frac": round(algo_bytes / (wall / K) / 1e9 / HBM_PEAK_GBS, 4), "device": cai.device_name(),
-                   "build_s": round(t_build, 1)},
-        "roofline": {"bound": "hbm", "kernel": "gemv_fast<Q4_K,1,R,swiglu> (RMSNorm+gate|up+SwiGLU, %dx%d)" % (2 * I, d),
+                   "build_s": round(t_build, 1),
+                   "prefill": {"tokens": prompt_len - 1, "ms": round(pf_ms.value, 2),
+                               "tok_per_s": round((prompt_len - 1) / max(pf_ms.value, 1e-6) * 1e3, 1),
+                               "linear_tflops": round(2.0 * n_lin_weights * (prompt_len - 1) / max(pf_ms.value, 1e-6) / 1e9, 1),
+                               "note": "multi-token ingestion: f16 MFMA (exact block integers, hi/lo-split activations = 2 MFMA passes per useful FLOP) + prompt attention; MFMA f16 dense peak 2500 TFLOP/s"}},
+        "roofline": {"bound": "hbm", "kernel": "gemv_q4k_stream<1,1,false> (RMSNorm+gate|up+SwiGLU, %dx%d)" % (2 * I, d),
                      "achieved": round(k_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(k_gbs / HBM_PEAK_GBS, 4),
-                     "avg_launch_us": round(k_avg_us, 2), "algorithmic_bytes_per_launch": int(k_bytes), "traffic": None},
+                     "avg_launch_us": round(k_avg_us, 2), "algorithmic_bytes_per_launch": int(k_bytes),
+                     "traffic": GATEUP_TRAFFIC_BYTES if args.config == "qwen2.5-7b-q4k" else None, "traffic_unit": "bytes/launch"},
     }
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(cfg)

@@ -75,6 +75,9 @@ int cai_dev_alloc(int64_t bytes, void** ptr_out);
 int cai_dev_free(void* ptr);
 int cai_dev_upload(void* dst_dev, const void* src_host, int64_t bytes);
 int cai_dev_download(void* dst_host, const void* src_dev, int64_t bytes);
+/* Plain device-to-device copy kernel (16-byte loads/stores; bytes must be a multiple of 16).  Also the known-size
+ * reference against which hardware traffic counters are scaled. */
+int cai_dev_copy(void* dst_dev, const void* src_dev, int64_t bytes);
 
 /* =====================================================================================
  * Resident quantized weights.

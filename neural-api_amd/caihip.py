@@ -15,7 +15,7 @@ V_ATTN_NORM, V_MLP_NORM, V_FINAL_NORM, V_Q_NORM, V_K_NORM = range(5)
 
 # every symbol include/caihip.h declares
 SYMBOLS = """cai_init cai_shutdown cai_last_error cai_device_name cai_sync cai_get_stream cai_timer_start cai_timer_stop
-cai_dev_alloc cai_dev_free cai_dev_upload cai_dev_download
+cai_dev_alloc cai_dev_free cai_dev_upload cai_dev_download cai_dev_copy
 cai_qw_create cai_qw_create_int8row cai_qw_destroy cai_qw_info cai_qw_dequant_rows cai_qgemv cai_ffn_gateup cai_qgemm
 cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_router_topk
 cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_attn_decode
@@ -57,6 +57,7 @@ def load():
         L.cai_dev_free.argtypes = [vp]
         L.cai_dev_upload.argtypes = [vp, vp, i64]
         L.cai_dev_download.argtypes = [vp, vp, i64]
+        L.cai_dev_copy.argtypes = [vp, vp, i64]
         L.cai_qw_create.argtypes = [i32, i64, i64, vp, vp, C.POINTER(vp)]
         L.cai_qw_create_int8row.argtypes = [i64, i64, vp, vp, vp, C.POINTER(vp)]
         L.cai_qw_destroy.argtypes = [vp]

@@ -4,6 +4,7 @@
 #include <stdarg.h>
 #include <string.h>
 #include <mutex>
+#include <algorithm>
 
 namespace cai {
 
@@ -142,6 +143,24 @@ extern "C" int cai_dev_download(void* h, const void* d, int64_t bytes)
   CAI_READY(); CAI_REQUIRE(d && h && bytes >= 0, "cai_dev_download: bad argument");
   CAI_HIP(hipMemcpyAsync(h, d, (size_t)bytes, hipMemcpyDeviceToHost, ctx().stream));
   CAI_HIP(hipStreamSynchronize(ctx().stream));
+  return CAI_OK;
+}
+
+namespace cai {
+__global__ __launch_bounds__(256) void copy16_kernel(const uint4* src, uint4* dst, size_t n16)
+{
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; const size_t stride = (size_t)gridDim.x * 256;
+  for (; i < n16; i += stride) dst[i] = src[i];
+}
+}  // namespace cai
+
+extern "C" int cai_dev_copy(void* dst, const void* src, int64_t bytes)
+{
+  CAI_READY(); CAI_REQUIRE(dst && src && bytes > 0 && bytes % 16 == 0, "cai_dev_copy: bad argument");
+  const size_t n16 = (size_t)bytes / 16;
+  const int grid = (int)std::min<size_t>((n16 + 255) / 256, 8192);
+  hipLaunchKernelGGL(cai::copy16_kernel, dim3(grid), dim3(256), 0, ctx().stream, (const uint4*)src, (uint4*)dst, n16);
+  CAI_HIP(hipGetLastError());
   return CAI_OK;
 }
 

@@ -52,6 +52,7 @@ function cai_dev_alloc(bytes: Int64; ptr_out: PPointer): LongInt; cdecl; externa
 function cai_dev_free(ptr: Pointer): LongInt; cdecl; external CAIHIP_LIB;
 function cai_dev_upload(dst_dev, src_host: Pointer; bytes: Int64): LongInt; cdecl; external CAIHIP_LIB;
 function cai_dev_download(dst_host, src_dev: Pointer; bytes: Int64): LongInt; cdecl; external CAIHIP_LIB;
+function cai_dev_copy(dst_dev, src_dev: Pointer; bytes: Int64): LongInt; cdecl; external CAIHIP_LIB;
 
 function cai_qw_create(qtype: LongInt; rows, cols: Int64; blocks: Pointer; bias: PSingle; out_w: PCaiQW): LongInt; cdecl; external CAIHIP_LIB;
 function cai_qw_create_int8row(rows, cols: Int64; codes: PShortInt; scales, bias: PSingle; out_w: PCaiQW): LongInt; cdecl; external CAIHIP_LIB;
