@@ -267,40 +267,51 @@ __global__ __launch_bounds__(128) void attn_merge_kernel(const AttnParams p)
   }
 }
 
-// ---- short contexts: one work-group of 32 half-waves per QUERY head walks the whole live range; no split,
-//      no cross-work-group merge (each extra device-coherent hand-off costs a memory round trip, ~2.5 us) ----
+// ---- short caches: one work-group per (split, QUERY head).  The G heads of a group each re-read the slice (from
+//      L2: their work-groups are numbered so that they land on the same XCD), but no work-group loops over heads:
+//      with one wave per SIMD that loop is a chain of dependent DPP/exp/LDS latencies and dominated the step.
+//      Running state lives in registers; LDS is used once, for the meeting of the 8 half-waves. ----
 template <int DS, typename KV_T>
-__global__ __launch_bounds__(1024) void attn_head_kernel(const AttnParams p)
+__global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p)
 {
-  const int h = blockIdx.x, seq = blockIdx.y;
-  const int G = p.q_heads / p.kv_heads, g = h / G;
+  const int G = p.q_heads / p.kv_heads;
+  // linear id = item_lo + 8 * (h + G * item_hi), item = split + n_splits * kv_head: consecutive ids rotate over the XCDs
+  const int L = blockIdx.x, item = (L & 7) + 8 * ((L >> 3) / G), h = (L >> 3) % G;
+  if (item >= p.n_splits * p.kv_heads) return;
+  const int split = item % p.n_splits, g = item / p.n_splits, seq = blockIdx.y;
   const int pos = p.pos[seq];
   const int len = pos + 1;
   const int j_start = (p.window > 0 && len > p.window) ? len - p.window : 0;
-  const int hw = threadIdx.x >> 5, l32 = threadIdx.x & 31;
+  const int s_begin = max(j_start, split * p.split_len), s_end = min(len, (split + 1) * p.split_len);
+  if (s_begin >= s_end) return;   // whole work-group leaves together, before any barrier
+  const int s_first = j_start / p.split_len, s_last = pos / p.split_len;
+  const int n_active = s_last - s_first + 1;
+
+  const int tid = threadIdx.x, hw = tid >> 5, l32 = tid & 31;
   const int hd = p.hd, qw = p.q_heads * hd, kw = p.kv_heads * hd;
   const int d0 = l32 * DS;
   const float* row = p.qkv + (int64_t)seq * p.qkv_stride;
-  KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
-  KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (seq + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (seq * p.seq_mul + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (seq * p.seq_mul + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
 
   constexpr int PCH = 4;
-  // cached rows of a chunk are all requested before any is used; the first chunk before the rotation math below
-  float kd[PCH][DS], vd[PCH][DS];
-  auto load_chunk = [&](int j0) {
+  float kdA[PCH][DS], vdA[PCH][DS], kdB[PCH][DS], vdB[PCH][DS];
+  auto load_chunk = [&](float (&kd)[PCH][DS], float (&vd)[PCH][DS], int j0) {
+    if (j0 >= s_end) return;
 #pragma unroll
     for (int c = 0; c < PCH; c++) {
-      const int j = min(j0 + 32 * c, len - 1);
+      const int j = min(j0 + 8 * c, s_end - 1);
 #pragma unroll
       for (int i = 0; i < DS; i++) {
         const int d = d0 + i;
-        const bool ok = d < hd && j != pos;      // the row being appended is taken from registers instead
+        const bool ok = d < hd && (j != pos || p.appended);   // the row appended here comes from registers
         kd[c][i] = ok ? kv_to_float<KV_T>(kc[(int64_t)j * hd + d]) : 0.0f;
         vd[c][i] = ok ? kv_to_float<KV_T>(vc[(int64_t)j * hd + d]) : 0.0f;
       }
     }
   };
-  load_chunk(j_start + hw);
+  load_chunk(kdA, vdA, s_begin + hw);      // cached rows are requested before the rotation math
+  load_chunk(kdB, vdB, s_begin + hw + 8 * PCH);
 
   float rs[(DS + 1) / 2], rc[(DS + 1) / 2];
 #pragma unroll
@@ -326,25 +337,30 @@ __global__ __launch_bounds__(1024) void attn_head_kernel(const AttnParams p)
     }
   };
   float q[DS], knew[DS], vnew[DS], acc[DS];
-  load_rot(row + h * hd, q, p.theta != nullptr);
-  load_rot(row + qw + g * hd, knew, p.theta != nullptr);
-  load_rot(row + qw + kw + g * hd, vnew, false);
+  load_rot(row + (g * G + h) * hd, q, p.theta != nullptr);
 #pragma unroll
-  for (int i = 0; i < DS; i++) {
-    knew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(knew[i]));
-    vnew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(vnew[i]));
-    acc[i] = 0.0f;
-    if (h == g * G && hw == 0 && d0 + i < hd) {   // the first query head of the group appends the row
-      kc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(knew[i]);
-      vc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(vnew[i]);
+  for (int i = 0; i < DS; i++) { acc[i] = 0.0f; knew[i] = 0.0f; vnew[i] = 0.0f; }
+  // every work-group whose slice holds `pos` keeps the new row in registers; the group's first head appends it
+  const bool owns_new = !p.appended && pos >= s_begin && pos < s_end;
+  if (owns_new) {
+    load_rot(row + qw + g * hd, knew, p.theta != nullptr);
+    load_rot(row + qw + kw + g * hd, vnew, false);
+#pragma unroll
+    for (int i = 0; i < DS; i++) {
+      vnew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(vnew[i]));
+      knew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(knew[i]));
+      if (h == 0 && hw == 0 && d0 + i < hd) {
+        kc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(knew[i]);
+        vc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(vnew[i]);
+      }
     }
   }
   float m = -1e30f, l = 0.0f;
-  for (int j0 = j_start + hw; j0 < len; j0 += 32 * PCH) {
+  auto reduce_chunk = [&](float (&kd)[PCH][DS], float (&vd)[PCH][DS], int j0) {
     float sc[PCH], cmax = -1e30f;
 #pragma unroll
     for (int c = 0; c < PCH; c++) {
-      if (min(j0 + 32 * c, len - 1) == pos) {
+      if (owns_new && min(j0 + 8 * c, s_end - 1) == pos) {
 #pragma unroll
         for (int i = 0; i < DS; i++) { kd[c][i] = knew[i]; vd[c][i] = vnew[i]; }
       }
@@ -353,52 +369,70 @@ __global__ __launch_bounds__(1024) void attn_head_kernel(const AttnParams p)
       for (int i = 0; i < DS; i++) s = fmaf(q[i], kd[c][i], s);
       s = half_wave_allsum(s) * p.inv_sqrt;
       if (p.softcap > 0.0f) s = p.softcap * tanhf(s / p.softcap);
-      sc[c] = (j0 + 32 * c < len) ? s : -1e30f;
+      sc[c] = (j0 + 8 * c < s_end) ? s : -1e30f;
       cmax = fmaxf(cmax, sc[c]);
     }
     const float mn = fmaxf(m, cmax), corr = expf(m - mn);
-    float lsum = 0.0f, a[DS];
+    float lsum = 0.0f;
 #pragma unroll
-    for (int i = 0; i < DS; i++) a[i] = acc[i] * corr;
+    for (int i = 0; i < DS; i++) acc[i] *= corr;
 #pragma unroll
     for (int c = 0; c < PCH; c++) {
-      const float pj = (j0 + 32 * c < len) ? expf(sc[c] - mn) : 0.0f;
+      const float pj = (j0 + 8 * c < s_end) ? expf(sc[c] - mn) : 0.0f;
       lsum += pj;
 #pragma unroll
-      for (int i = 0; i < DS; i++) a[i] = fmaf(pj, vd[c][i], a[i]);
+      for (int i = 0; i < DS; i++) acc[i] = fmaf(pj, vd[c][i], acc[i]);
     }
-    if (j0 + 32 * PCH < len) load_chunk(j0 + 32 * PCH);   // request the next chunk (this one is consumed)
     l = l * corr + lsum; m = mn;
-#pragma unroll
-    for (int i = 0; i < DS; i++) acc[i] = a[i];
+  };
+  for (int j0 = s_begin + hw; j0 < s_end; j0 += 16 * PCH) {
+    reduce_chunk(kdA, vdA, j0);
+    if (j0 + 16 * PCH < s_end) load_chunk(kdA, vdA, j0 + 16 * PCH);
+    if (j0 + 8 * PCH < s_end) {
+      reduce_chunk(kdB, vdB, j0 + 8 * PCH);
+      if (j0 + 24 * PCH < s_end) load_chunk(kdB, vdB, j0 + 24 * PCH);
+    }
   }
-  __shared__ float sm[32], sl[32];
-  __shared__ float sacc[32][32 * DS];
+
+  // ---- meeting of the 8 half-waves ----
+  __shared__ float sm[8], sl[8];
+  __shared__ float sacc[8][32 * DS];
   if (l32 == 0) { sm[hw] = m; sl[hw] = l; }
 #pragma unroll
   for (int i = 0; i < DS; i++) sacc[hw][d0 + i] = acc[i];
   __syncthreads();
-  for (int d = threadIdx.x; d < hd; d += 1024) {
+  if (tid < hd) {
+    const int d = tid;
     float M = -1e30f;
 #pragma unroll
-    for (int w = 0; w < 32; w++) M = fmaxf(M, sm[w]);
-    float L = 0.0f, A = 0.0f;
+    for (int w = 0; w < 8; w++) M = fmaxf(M, sm[w]);
+    float Ls = 0.0f, A = 0.0f;
 #pragma unroll
-    for (int w = 0; w < 32; w++) {
+    for (int w = 0; w < 8; w++) {
       const float e = sl[w] > 0.0f ? expf(sm[w] - M) : 0.0f;
-      L = fmaf(sl[w], e, L); A = fmaf(sacc[w][d], e, A);
+      Ls = fmaf(sl[w], e, Ls); A = fmaf(sacc[w][d], e, A);
     }
-    p.out[(int64_t)seq * p.out_stride + h * hd + d] = L > 0.0f ? A * (1.0f / L) : 0.0f;
+    const int qh = g * G + h;
+    if (n_active == 1) {
+      p.out[(int64_t)seq * p.out_stride + qh * hd + d] = Ls > 0.0f ? A * (1.0f / Ls) : 0.0f;
+    } else {
+      float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + split) * (hd + 2);
+      pt[d] = A;
+      if (d == 0) { pt[hd] = M; pt[hd + 1] = Ls; }
+    }
   }
 }
 
 template <typename KV_T>
-static int launch_head_kernel(const AttnParams& p, int n_seq, hipStream_t st)
+static int launch_split_head(const AttnParams& p, int n_seq, hipStream_t st)
 {
-  const dim3 grid(p.q_heads, n_seq);
-  if (p.hd <= 32) hipLaunchKernelGGL((attn_head_kernel<1, KV_T>), grid, dim3(1024), 0, st, p);
-  else if (p.hd <= 64) hipLaunchKernelGGL((attn_head_kernel<2, KV_T>), grid, dim3(1024), 0, st, p);
-  else hipLaunchKernelGGL((attn_head_kernel<4, KV_T>), grid, dim3(1024), 0, st, p);
+  const int G = p.q_heads / p.kv_heads;
+  const int items = p.n_splits * p.kv_heads;
+  const dim3 grid(8 * G * ((items + 7) / 8), n_seq);
+  if (p.hd <= 32) hipLaunchKernelGGL((attn_split_head_kernel<1, KV_T>), grid, dim3(256), 0, st, p);
+  else if (p.hd <= 64) hipLaunchKernelGGL((attn_split_head_kernel<2, KV_T>), grid, dim3(256), 0, st, p);
+  else if (p.hd <= 128) hipLaunchKernelGGL((attn_split_head_kernel<4, KV_T>), grid, dim3(256), 0, st, p);
+  else return set_error(CAI_ERR_UNSUPPORTED, "attention: head_dim %d > 128", p.hd);
   return CAI_OK;
 }
 
@@ -466,11 +500,11 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
     else hipLaunchKernelGGL(kv_append_rows_kernel<float>, dim3(n_seq), dim3(256), 0, c.stream, p);
   }
   p.counters = kv->d_counters;
-  if (!prompt_rows && kv->max_ctx <= kv->short_ctx_limit) {
-    if (kv->dtype == CAI_KV_F16) return launch_head_kernel<__half>(p, n_seq, c.stream);
-    return launch_head_kernel<float>(p, n_seq, c.stream);
-  }
-  const int rc = kv->dtype == CAI_KV_F16 ? launch_split_g<__half>(p, n_seq, c.stream) : launch_split_g<float>(p, n_seq, c.stream);
+  int rc;
+  if (kv->max_ctx <= kv->short_ctx_limit)   // short caches: per-head work-groups (K,V re-read from L2 by the group's heads)
+    rc = kv->dtype == CAI_KV_F16 ? launch_split_head<__half>(p, n_seq, c.stream) : launch_split_head<float>(p, n_seq, c.stream);
+  else
+    rc = kv->dtype == CAI_KV_F16 ? launch_split_g<__half>(p, n_seq, c.stream) : launch_split_g<float>(p, n_seq, c.stream);
   if (rc) return rc;
   if (p.n_splits > 1) hipLaunchKernelGGL(attn_merge_kernel, dim3(q_heads, n_seq), dim3(128), 0, c.stream, p);
   return CAI_OK;
@@ -497,8 +531,8 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   CAI_HIP(hipMemsetAsync(kv->k, 0, bytes, ctx().stream));
   CAI_HIP(hipMemsetAsync(kv->v, 0, bytes, ctx().stream));
   {
-    const char* e = getenv("CAIHIP_ATTN_SHORT_CTX");      // caches up to this length use the per-head kernel
-    kv->short_ctx_limit = e ? atoi(e) : 0;
+    const char* e = getenv("CAIHIP_ATTN_SHORT_CTX");      // caches up to this capacity use the per-head split kernel
+    kv->short_ctx_limit = e ? atoi(e) : 4096;
   }
   kv->part_q_heads = kv_heads * 8;
   CAI_HIP(hipMalloc(&kv->part, (size_t)n_seq * kv->part_q_heads * kv->n_splits * (head_dim + 2) * sizeof(float)));

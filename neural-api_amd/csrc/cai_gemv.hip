@@ -400,6 +400,7 @@ __global__ void swiglu_rows(const float* x, int half, int n_tokens, float* y)
 }
 
 int launch_q4k_stream(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream_t st);
+int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream_t st);
 static bool stream_kernel_enabled()
 {
   static const int on = []() { const char* e = getenv("CAIHIP_GEMV_V1"); return (e && e[0] == '1') ? 0 : 1; }();
@@ -516,7 +517,8 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
     MultiGemv mm = m;
     if (swiglu_half) { if (m.n != 1) return set_error(CAI_ERR_INVALID, "gemv: swiglu takes one matrix"); p.seg[0].rows = swiglu_half; }
     p.ssq_in = m.ssq_in; p.ssq_out = m.ssq_out;
-    const int rc = launch_q4k_stream(p, mm, swiglu_half, c.stream);
+    static const bool float_x = []() { const char* e = getenv("CAIHIP_GEMV_FLOAT_X"); return e && e[0] == '1'; }();
+    const int rc = float_x ? launch_q4k_stream(p, mm, swiglu_half, c.stream) : launch_q4k_dot(p, mm, swiglu_half, c.stream);
     p.ssq_in = nullptr; p.ssq_out = nullptr;
     if (rc != CAI_ERR_UNSUPPORTED) return rc;
   }

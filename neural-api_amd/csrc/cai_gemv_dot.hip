@@ -1,0 +1,385 @@
+// Persistent streaming Q4_K matrix-vector kernel for batch-1 decode on gfx950, integer-dot form.
+//
+// The weights of a Q4_K sub-block are 4-bit integers with one float scale, so dot(W[a], X) splits into an exact
+// integer part and a handful of float operations per 32 weights once X is held as integers too.  Each
+// work-group turns the activation vector (token RMSNorm fused) into block-float form once: per 32 values one
+// float scale s = max|x| / (2^22 - 1) and 23-bit integers q = rint(x / s), stored as three balanced base-256
+// digits (each a signed byte).  The inner loop is then v_dot4_i32_i8 on nibbles widened to bytes: 3 mask/shift
+// operations and 6 dot4 per 8 weights instead of 16 conversions + 16 FMAs.  The integer sums are exact; the
+// only rounding beyond the float path is that of x itself, 2^-23 of its 32-block maximum.
+//
+// Work layout (as in the float kernel): a fixed number of work-groups stays resident and strides over the row
+// groups; one lane owns one pair of sub-blocks (64 weights = two 128-bit loads + the 16-byte super-block
+// header); rows longer than 4096 columns are split over `nsw` waves, each keeping its slice of the quantised
+// activation in registers (52 VGPRs).  Weights of the next NS-1 row groups are in flight while one is reduced.
+//
+// Semantics: Out[a] = act(dot(W[a], X) + bias[a]) (+ residual), or for the fused feed-forward front half
+// Out[i] = up_i * silu(gate_i) with up = row i and gate = row half + i
+// (reference: neural/neuralvolume.pas:12127-12423; neural/neural.cl:111-146, 1047-1085, 1213-1263).
+#include "cai_gemv_common.hpp"
+#include <set>
+#include <type_traits>
+
+namespace cai {
+
+namespace {
+
+struct Q4kRegs { uint4 h, q0, q1; };
+
+// LDS slot (in uint4) of the t-th uint4 (t = 0..15) of unit u (64 activations): tiles of 16 units, transposed
+__device__ __forceinline__ int xq_slot(int u, int t) { return (u >> 4) * 256 + t * 16 + (u & 15); }
+
+constexpr float XQ_MAX = 4194303.0f;          // 2^22 - 1
+constexpr int NL = 3;                         // balanced base-256 digits per activation
+
+__device__ __forceinline__ float quad_max(float v)
+{
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xb1, 0xf, 0xf, true)));  // quad_perm [1,0,3,2]
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4e, 0xf, 0xf, true)));  // quad_perm [2,3,0,1]
+  return v;
+}
+__device__ __forceinline__ float quad_poison(float v)   // v is 0 or NaN per lane; NaN if any lane of the quad has it
+{
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xb1, 0xf, 0xf, true));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4e, 0xf, 0xf, true));
+  return v;
+}
+__device__ __forceinline__ int quad_sum(int v)
+{
+  v += __builtin_amdgcn_update_dpp(0, v, 0xb1, 0xf, 0xf, true);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x4e, 0xf, 0xf, true);
+  return v;
+}
+
+// four rounded activations (as float bit patterns of x*inv + 1.5*2^23) -> one dword per digit
+__device__ __forceinline__ void pack_digits(const float (&f)[4], int (&d)[NL])
+{
+  uint32_t e[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)   // integer value + 0x808080, then flip the digit sign bits: bytes are balanced digits
+    e[i] = (__builtin_bit_cast(uint32_t, f[i]) + (0x00808080u - 0x4B400000u)) ^ 0x00808080u;
+  const uint32_t p01 = __builtin_amdgcn_perm(e[1], e[0], 0x05010400u), p23 = __builtin_amdgcn_perm(e[3], e[2], 0x05010400u);
+  const uint32_t h01 = __builtin_amdgcn_perm(e[1], e[0], 0x06020602u), h23 = __builtin_amdgcn_perm(e[3], e[2], 0x06020602u);
+  d[0] = (int)__builtin_amdgcn_perm(p23, p01, 0x05040100u);
+  d[1] = (int)__builtin_amdgcn_perm(p23, p01, 0x07060302u);
+  d[2] = (int)__builtin_amdgcn_perm(h23, h01, 0x05040100u);
+}
+
+}  // namespace
+
+template <int R, int MODE, bool MULTISEG, int NS>
+__global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
+{
+  extern __shared__ uint4 xq4[];
+  constexpr int RR = MODE == 1 ? 2 * R : R;
+  __shared__ float s_ss[16];
+  constexpr int CH = 4;                       // row groups between two meetings of the slice waves
+  __shared__ float s_part[2][16][CH][RR];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int step = wave % nsw, gslot = wave / nsw;
+  const int cols = p.cols, nsb = cols >> 8;
+  const int64_t row_bytes = (int64_t)nsb * 144;
+  const int sb = step * 16 + (lane >> 2), cc = lane & 3;
+  const bool act = sb < nsb;
+  const int g_first = blockIdx.x * gwv + gslot, g_stride = gridDim.x * gwv;
+  const int n_iters = (n_groups + g_stride - 1) / g_stride;
+  const int64_t lane_off = (int64_t)(act ? sb : 0) * 144;
+
+  // group -> segment, first row of the group inside the segment
+  auto locate = [&](int g, const GemvSeg*& sg, int& row0) {
+    int s = 0, g0 = 0;
+    if (MULTISEG) {
+      if (p.n_seg > 1 && g >= p.seg[0].grp_end) { s = 1; g0 = p.seg[0].grp_end; }
+      if (p.n_seg > 2 && g >= p.seg[1].grp_end) { s = 2; g0 = p.seg[1].grp_end; }
+    }
+    sg = &p.seg[s]; row0 = (g - g0) * R;
+  };
+  auto issue = [&](int g, Q4kRegs (&rg)[RR]) {
+    if (g < n_groups && act) {
+      const GemvSeg* sg; int row0; locate(g, sg, row0);
+      const int lim = MODE == 1 ? p.half : sg->rows;
+#pragma unroll
+      for (int r = 0; r < RR; r++) {
+        int row = row0 + (MODE == 1 ? (r >> 1) : r);
+        if (row >= lim) row = lim - 1;               // tail group: re-read the last row, result is not written
+        if (MODE == 1 && (r & 1)) row += p.half;
+        const uint8_t* blk = sg->data + (int64_t)row * row_bytes + lane_off;
+        rg[r].h = *reinterpret_cast<const uint4*>(blk);
+        rg[r].q0 = *reinterpret_cast<const uint4*>(blk + 16 + 32 * cc);
+        rg[r].q1 = *reinterpret_cast<const uint4*>(blk + 32 + 32 * cc);
+      }
+    }
+  };
+
+  Q4kRegs buf[NS][RR];
+  // weights do not depend on the activation: request the first row groups before anything else
+#pragma unroll
+  for (int k = 0; k < NS - 1; k++) issue(g_first + k * g_stride, buf[k]);
+
+  // ---- activation -> block-float integers, once per work-group, through LDS ----
+  {
+    float inv_rms = 1.0f;
+    const float4* src = reinterpret_cast<const float4*>(p.x);
+    const float4* gsrc = reinterpret_cast<const float4*>(p.norm_gain);
+    const int n8 = cols >> 3, nthr = blockDim.x;
+    // one thread = 8 consecutive activations (a quarter of a 32-block: the block's four threads are one DPP quad);
+    // the first eight are requested before the sum of squares is gathered, every later eight one turn ahead
+    int n = threadIdx.x;
+    float4 c0 = {0, 0, 0, 0}, c1 = c0, cg0 = c0, cg1 = c0;
+    if (n < n8) {
+      c0 = src[2 * n]; c1 = src[2 * n + 1];
+      if (p.norm_gain) { cg0 = gsrc[2 * n]; cg1 = gsrc[2 * n + 1]; }
+    }
+    if (p.norm_gain) {
+      float t = 0.0f;
+      if (p.ssq_in) {
+        // sum of squares of x delivered by the producing kernel as SSQ_PARTS per-work-group partials (fixed order)
+#pragma unroll
+        for (int i = 0; i < SSQ_PARTS / 64; i++) t += p.ssq_in[i * 64 + lane];
+        t = wave_sum(t);
+        t = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, t), 63));
+      } else {
+        for (int k = threadIdx.x; k < n8 * 2; k += nthr) {
+          const float4 v = src[k];
+          t = fmaf(v.x, v.x, t); t = fmaf(v.y, v.y, t); t = fmaf(v.z, v.z, t); t = fmaf(v.w, v.w, t);
+        }
+        t = wave_sum(t);
+        if (lane == 63) s_ss[wave] = t;
+        __syncthreads();
+        t = 0.0f;
+        for (int w = 0; w < (int)(blockDim.x >> 6); w++) t += s_ss[w];
+        __syncthreads();                                 // s_ss is reused by the output sum of squares
+      }
+      inv_rms = 1.0f / sqrtf(t / (float)cols + p.norm_eps);
+    }
+    while (n < n8) {
+      float4 v0 = c0, v1 = c1;
+      const float4 g0 = cg0, g1 = cg1;
+      const int nn = n + nthr;
+      if (nn < n8) {
+        c0 = src[2 * nn]; c1 = src[2 * nn + 1];
+        if (p.norm_gain) { cg0 = gsrc[2 * nn]; cg1 = gsrc[2 * nn + 1]; }
+      }
+      if (p.norm_gain) {
+        v0.x = g0.x * (v0.x * inv_rms); v0.y = g0.y * (v0.y * inv_rms); v0.z = g0.z * (v0.z * inv_rms); v0.w = g0.w * (v0.w * inv_rms);
+        v1.x = g1.x * (v1.x * inv_rms); v1.y = g1.y * (v1.y * inv_rms); v1.z = g1.z * (v1.z * inv_rms); v1.w = g1.w * (v1.w * inv_rms);
+      }
+      float m = fmaxf(fmaxf(fmaxf(fabsf(v0.x), fabsf(v0.y)), fmaxf(fabsf(v0.z), fabsf(v0.w))),
+                      fmaxf(fmaxf(fabsf(v1.x), fabsf(v1.y)), fmaxf(fabsf(v1.z), fabsf(v1.w))));
+      m = quad_max(m);
+      const bool ok = m > 0.0f && m < 3.0e38f;           // an all-zero block contributes 0
+      // 0 for finite values, NaN when the eight hold an inf or a NaN: carried into the scale so the outputs show it
+      const float poison = (((v0.x + v0.y) + (v0.z + v0.w)) + ((v1.x + v1.y) + (v1.z + v1.w))) * 0.0f;
+      const float inv = ok ? XQ_MAX / m : 0.0f, s = ok ? m * (1.0f / XQ_MAX) : 0.0f;
+      const float fa[4] = {fmaf(v0.x, inv, 12582912.0f), fmaf(v0.y, inv, 12582912.0f), fmaf(v0.z, inv, 12582912.0f), fmaf(v0.w, inv, 12582912.0f)};
+      const float fb[4] = {fmaf(v1.x, inv, 12582912.0f), fmaf(v1.y, inv, 12582912.0f), fmaf(v1.z, inv, 12582912.0f), fmaf(v1.w, inv, 12582912.0f)};
+      int da[NL], db[NL];
+      pack_digits(fa, da); pack_digits(fb, db);
+      int isum = 0;
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        isum += (int)(__builtin_bit_cast(uint32_t, fa[i]) - 0x4B400000u) + (int)(__builtin_bit_cast(uint32_t, fb[i]) - 0x4B400000u);
+      isum = quad_sum(isum);
+      // n = [unit][half:1][j:2]: the unit's record holds per digit 4 uint4 (2 per 32-block), then one uint4 of
+      // {scale A, scale B, s*sum A, s*sum B}
+      const int u = n >> 3, hb = (n >> 2) & 1, j = n & 3;
+      uint32_t* rec = reinterpret_cast<uint32_t*>(xq4);
+#pragma unroll
+      for (int L = 0; L < NL; L++) {
+        uint32_t* dst = rec + (size_t)xq_slot(u, L * 4 + hb * 2 + (j >> 1)) * 4 + (j & 1) * 2;
+        dst[0] = (uint32_t)da[L]; dst[1] = (uint32_t)db[L];
+      }
+      // the block's scale must be poisoned by any of its four threads
+      const float s_blk = s + quad_poison(poison);
+      if (j == 0) {
+        float* fr = reinterpret_cast<float*>(rec + (size_t)xq_slot(u, NL * 4) * 4);
+        fr[hb] = s_blk; fr[2 + hb] = s_blk * (float)isum;
+      }
+      n = nn;
+    }
+    __syncthreads();
+  }
+  int xq[NL][16];
+  float sA = 0.0f, sB = 0.0f, mA = 0.0f, mB = 0.0f;
+  if (act) {
+    const int u = sb * 4 + cc;
+#pragma unroll
+    for (int L = 0; L < NL; L++) {
+#pragma unroll
+      for (int t = 0; t < 4; t++) {
+        const uint4 v = xq4[xq_slot(u, L * 4 + t)];
+        xq[L][4 * t] = (int)v.x; xq[L][4 * t + 1] = (int)v.y; xq[L][4 * t + 2] = (int)v.z; xq[L][4 * t + 3] = (int)v.w;
+      }
+    }
+    const uint4 v = xq4[xq_slot(u, NL * 4)];
+    sA = __builtin_bit_cast(float, v.x); sB = __builtin_bit_cast(float, v.y);
+    mA = __builtin_bit_cast(float, v.z); mB = __builtin_bit_cast(float, v.w);
+  } else {
+#pragma unroll
+    for (int L = 0; L < NL; L++)
+#pragma unroll
+      for (int t = 0; t < 16; t++) xq[L][t] = 0;
+  }
+
+  float ssq_acc = 0.0f;   // squares of the outputs this thread wrote (for the consumer's RMSNorm)
+  auto process = [&](Q4kRegs (&cur)[RR], Q4kRegs (&nxt)[RR], int it) {
+    const int g = g_first + it * g_stride;
+    issue(g + (NS - 1) * g_stride, nxt);
+    float acc[RR];
+#pragma unroll
+    for (int r = 0; r < RR; r++) acc[r] = 0.0f;
+    if (g < n_groups && act) {
+#pragma unroll
+      for (int r = 0; r < RR; r++) {
+        const uint32_t qw[8] = {cur[r].q0.x, cur[r].q0.y, cur[r].q0.z, cur[r].q0.w, cur[r].q1.x, cur[r].q1.y, cur[r].q1.z, cur[r].q1.w};
+        int ia[NL], ib[NL];
+#pragma unroll
+        for (int L = 0; L < NL; L++) { ia[L] = 0; ib[L] = 0; }
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+          const int a = (int)(qw[w] & 0x0f0f0f0fu), b = (int)((qw[w] >> 4) & 0x0f0f0f0fu);
+#pragma unroll
+          for (int L = 0; L < NL; L++) {
+            ia[L] = __builtin_amdgcn_sdot4(a, xq[L][w], ia[L], false);
+            ib[L] = __builtin_amdgcn_sdot4(b, xq[L][8 + w], ib[L], false);
+          }
+        }
+        const float fa = (float)(ia[0] + (ia[1] << 8) + (ia[2] << 16)), fb = (float)(ib[0] + (ib[1] << 8) + (ib[2] << 16));
+        uint32_t sc, mn; q4k_scale_pair(cur[r].h.y, cur[r].h.z, cur[r].h.w, cc, sc, mn);
+        const float d = __half2float(__ushort_as_half((unsigned short)(cur[r].h.x & 0xffffu)));
+        const float dmin = __half2float(__ushort_as_half((unsigned short)(cur[r].h.x >> 16)));
+        acc[r] = d * (cvt_ub0(sc) * (sA * fa) + cvt_ub1(sc) * (sB * fb)) - dmin * (cvt_ub0(mn) * mA + cvt_ub1(mn) * mB);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < RR; r++) acc[r] = wave_sum(acc[r]);   // total in lane 63
+
+    if (nsw > 1) {
+      // Slice waves meet every CH row groups: partial sums are parked in LDS (double-buffered by chunk parity), one
+      // barrier per chunk, then the lanes of the slice-0 wave finish one output row each.
+      const int slot = it % CH, par = (it / CH) & 1;
+      if (lane == 63) {
+#pragma unroll
+        for (int r = 0; r < RR; r++) s_part[par][wave][slot][r] = acc[r];
+      }
+      if (slot != CH - 1 && it != n_iters - 1) return;
+      __syncthreads();
+      if (step != 0) return;
+      const int n_out = (slot + 1) * (MODE == 1 ? R : RR);
+      if (lane >= n_out) return;
+      const int sl = lane / (MODE == 1 ? R : RR), r = lane % (MODE == 1 ? R : RR);
+      const int gg = g_first + (it - slot + sl) * g_stride;
+      if (gg >= n_groups) return;
+      const GemvSeg* sg; int row0; locate(gg, sg, row0);
+      const int row = row0 + r;
+      if (MODE == 0) {
+        if (row >= sg->rows) return;
+        float v = 0.0f;
+        for (int s2 = 0; s2 < nsw; s2++) v += s_part[par][gslot * nsw + s2][sl][r];
+        if (sg->bias) v += sg->bias[row];
+        v = act_apply(v, p.act);
+        const int o = sg->y_off + row;
+        if (p.residual) v += p.residual[o];
+        p.y[o] = v; ssq_acc = fmaf(v, v, ssq_acc);
+      } else {
+        if (row >= p.half) return;
+        float up = 0.0f, gate = 0.0f;
+        for (int s2 = 0; s2 < nsw; s2++) { up += s_part[par][gslot * nsw + s2][sl][2 * r]; gate += s_part[par][gslot * nsw + s2][sl][2 * r + 1]; }
+        if (sg->bias) { up += sg->bias[row]; gate += sg->bias[p.half + row]; }
+        p.y[sg->y_off + row] = silu_mul(up, gate);
+      }
+      return;
+    }
+    if (lane != 63 || g >= n_groups) return;
+
+    const GemvSeg* sg; int row0; locate(g, sg, row0);
+    if (MODE == 0) {
+#pragma unroll
+      for (int r = 0; r < RR; r++) {
+        const int row = row0 + r;
+        if (row >= sg->rows) break;
+        float v = acc[r];
+        if (sg->bias) v += sg->bias[row];
+        v = act_apply(v, p.act);
+        const int o = sg->y_off + row;
+        if (p.residual) v += p.residual[o];
+        p.y[o] = v; ssq_acc = fmaf(v, v, ssq_acc);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        const int row = row0 + r;
+        if (row >= p.half) break;
+        float up = acc[2 * r], gate = acc[2 * r + 1];
+        if (sg->bias) { up += sg->bias[row]; gate += sg->bias[p.half + row]; }
+        p.y[sg->y_off + row] = silu_mul(up, gate);
+      }
+    }
+  };
+
+  for (int it = 0; it < n_iters; it += NS) {
+#pragma unroll
+    for (int k = 0; k < NS; k++)
+      if (it + k < n_iters) process(buf[k], buf[(k + NS - 1) % NS], it + k);
+  }
+
+  if (p.ssq_out) {   // per-work-group partial of sum(y^2), summed in a fixed order; unused slots are zeroed by group 0
+    __syncthreads();
+    const float t = wave_sum(ssq_acc);
+    if (lane == 63) s_ss[wave] = t;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float tot = 0.0f;
+      for (int w = 0; w < (int)(blockDim.x >> 6); w++) tot += s_ss[w];
+      p.ssq_out[blockIdx.x] = tot;
+    }
+    if (blockIdx.x == 0) for (int i = gridDim.x + threadIdx.x; i < SSQ_PARTS; i += blockDim.x) p.ssq_out[i] = 0.0f;
+  }
+}
+
+// Host launcher.  Returns CAI_ERR_UNSUPPORTED when the shape does not fit this kernel (caller falls back).
+int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream_t st)
+{
+  Context& c = ctx();
+  const int cols = p.cols, nsb = cols >> 8;
+  const int nsw = (nsb + 15) >> 4;          // waves along the columns
+  if (nsw > 8) return CAI_ERR_UNSUPPORTED;  // rows longer than 32768 columns
+  static const int ns_env = []() { const char* e = getenv("CAIHIP_DOT_NS"); return e ? atoi(e) : 2; }();
+  static const int W = []() { const char* e = getenv("CAIHIP_DOT_W"); return e ? atoi(e) : 12; }();   // resident waves per CU
+  // row groups in flight per work-group: short rows share one quantised activation among 4 waves; long rows
+  // fill the CU with a single work-group
+  const int gwv = nsw >= 3 ? std::max(1, W / nsw) : 4 / nsw;
+  int64_t total = 0;
+  for (int i = 0; i < m.n; i++) total += swiglu_half ? swiglu_half : m.rows[i];
+  const int waves_per_wg = nsw * gwv;
+  const size_t lds = (size_t)((cols + 1023) / 1024 * 1024) * 4;   // 16 uint4 per 64 activations
+  int wg_per_cu = W / waves_per_wg; if (wg_per_cu < 1) wg_per_cu = 1;
+  { const int lds_fit = (int)((160 * 1024 - 4096) / (lds + 1024)); if (wg_per_cu > lds_fit) wg_per_cu = lds_fit < 1 ? 1 : lds_fit; }
+  const int max_wgs = c.n_cu * wg_per_cu;
+  int R = 1;
+  if (!swiglu_half && total >= (int64_t)max_wgs * gwv * 4) R = 2;
+  int cum = 0;
+  for (int i = 0; i < m.n; i++) {
+    const int64_t rows = swiglu_half ? swiglu_half : m.rows[i];
+    cum += (int)((rows + R - 1) / R);
+    p.seg[i].grp_end = cum;
+  }
+  const int grid = std::min(std::min((cum + gwv - 1) / gwv, max_wgs), SSQ_PARTS);
+  const dim3 block(64 * waves_per_wg);
+  auto go = [&](auto kern) {
+    static std::set<const void*> raised;   // kernels whose dynamic-LDS limit has been raised
+    if (raised.insert((const void*)kern).second) (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 2048);
+    hipLaunchKernelGGL(kern, dim3(grid), block, lds, st, p, cum, nsw, gwv);
+  };
+  auto pick = [&](auto ns) {
+    constexpr int NSV = decltype(ns)::value;
+    if (swiglu_half) go(gemv_q4k_dot<1, 1, false, NSV>);
+    else if (m.n > 1) { if (R == 2) go(gemv_q4k_dot<2, 0, true, NSV>); else go(gemv_q4k_dot<1, 0, true, NSV>); }
+    else { if (R == 2) go(gemv_q4k_dot<2, 0, false, NSV>); else go(gemv_q4k_dot<1, 0, false, NSV>); }
+  };
+  if (ns_env == 3) pick(std::integral_constant<int, 3>());
+  else pick(std::integral_constant<int, 2>());
+  return CAI_OK;
+}
+
+}  // namespace cai
