@@ -21,6 +21,16 @@ CONFIGS = {
     # BASELINE.json configs[2]: Qwen2.5-7B shape, Q4_K body, Q8_0 untied head, QKV bias
     "qwen2.5-7b-q4k": dict(cfg=dict(n_layers=28, d_model=3584, n_q_heads=28, n_kv_heads=4, head_dim=128, ffn=18944, vocab=152064,
                                     max_ctx=768, eps=1e-6, rope_theta=1e6), qtype="Q4_K", head="Q8_0", bias=True, prompt=512),
+    # BASELINE.json configs[0] (the reference's own CPU-runnable case): SmolLM2-135M shape, Q8_0, tied head
+    "smollm2-135m-q8_0": dict(cfg=dict(n_layers=30, d_model=576, n_q_heads=9, n_kv_heads=3, head_dim=64, ffn=1536, vocab=49152,
+                                       max_ctx=256, eps=1e-5, rope_theta=1e5, tied=True), qtype="Q8_0", head="Q8_0", bias=False, prompt=16),
+    # configs[3]: OLMoE-1B-7B shape, Q8_0, 64 experts top-8, full-width QK norm
+    "olmoe-1b-7b-q8_0": dict(cfg=dict(n_layers=16, d_model=2048, n_q_heads=16, n_kv_heads=16, head_dim=128, ffn=1024, vocab=50304,
+                                      max_ctx=768, eps=1e-5, rope_theta=1e4, qk_norm_full=1, n_experts=64, top_k=8, norm_topk=0),
+                             qtype="Q8_0", head="Q8_0", bias=False, prompt=256),
+    # configs[4]: Qwen2.5-32B shape, Q4_K body and head, fp16 KV cache, 8192-token context (batch via --batch)
+    "qwen2.5-32b-q4k": dict(cfg=dict(n_layers=64, d_model=5120, n_q_heads=40, n_kv_heads=8, head_dim=128, ffn=27648, vocab=152064,
+                                     max_ctx=8448, eps=1e-6, rope_theta=1e6), qtype="Q4_K", head="Q4_K", bias=True, prompt=8192, kv="f16"),
     # reduced shapes for quick local runs of this script
     "tiny-q4k": dict(cfg=dict(n_layers=2, d_model=512, n_q_heads=4, n_kv_heads=2, head_dim=128, ffn=1024, vocab=4096,
                               max_ctx=256, eps=1e-6, rope_theta=1e6), qtype="Q4_K", head="Q8_0", bias=True, prompt=16),
@@ -76,6 +86,7 @@ def main():
     ap.add_argument("--config", default="qwen2.5-7b-q4k", choices=list(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernel-reps", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=1, help="independent sequences decoded together (1..8)")
     ap.add_argument("--copy-calibration", action="store_true", help="only run the 1 GiB device copy kernel 5 times (reference for traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -107,7 +118,8 @@ def main():
     QT = {"Q4_K": cai.Q4_K, "Q8_0": cai.Q8_0, "Q4_0": cai.Q4_0}
     t0 = time.time()
     spec = synth.random_decoder_spec(cfg, QT[conf["qtype"]], QT[conf["head"]], seed=424242, qkv_bias=conf["bias"])
-    dec = cai.Decoder(spec)
+    B = args.batch
+    dec = cai.Decoder(spec, max_batch=B, kv_dtype=cai.KV_F16 if conf.get("kv") == "f16" else cai.KV_F32)
     torch.cuda.empty_cache()
     t_build = time.time() - t0
     wbytes = dec.weight_bytes()
@@ -123,25 +135,45 @@ def main():
         cai.check(lib.cai_sync()); cai.check(lib.cai_timer_start())
         dec.prefill(prompt[:-1], 0, want_logits=False)
         cai.check(lib.cai_timer_stop(C.byref(pf_ms)))
+        for b in range(1, B):
+            dec.prefill(prompt[:-1], 0, seq=b, want_logits=False)
     tok = int(prompt[-1]); pos = prompt_len - 1
+
+    def decode(tok, pos, n):
+        """n greedy steps of all B sequences; batch 1 chains the steps on the device, a batch steps from the host"""
+        if B == 1:
+            out = dec.generate(tok, pos, n)
+            return int(out[-1])
+        toks = np.full(B, tok, np.int32) if np.isscalar(tok) else tok
+        for i in range(n):
+            toks, _ = dec.step(toks, np.full(B, pos + i, np.int32), want_logits=False)
+        return toks
+
     if W > 0:
-        out = dec.generate(tok, pos, W); tok = int(out[-1]); pos += W
+        tok = decode(tok, pos, W); pos += W
     cai.check(lib.cai_sync()); torch.cuda.synchronize()
     ms = C.c_float()
     t1 = time.perf_counter()
     cai.check(lib.cai_timer_start())
-    out = dec.generate(tok, pos, K)
+    decode(tok, pos, K)
     cai.check(lib.cai_timer_stop(C.byref(ms)))
     cai.check(lib.cai_sync()); torch.cuda.synchronize()
     wall = time.perf_counter() - t1
     ms_per_step = wall * 1e3 / K
-    tok_s = K / wall
+    tok_s = K * B / wall
     ctx_mid = pos + K // 2
-    kv_bytes = cfg["n_layers"] * 2 * cfg["n_kv_heads"] * cfg["head_dim"] * 4 * ctx_mid
+    kv_bytes = B * cfg["n_layers"] * 2 * cfg["n_kv_heads"] * cfg["head_dim"] * (2 if conf.get("kv") == "f16" else 4) * ctx_mid
+    ne = cfg.get("n_experts", 0)
     algo_bytes = wbytes + kv_bytes
 
-    # ---- dominant kernel: fused RMSNorm + gate|up Q4_K GEMV + SwiGLU (76.4 MB of blocks per launch) ----
+    # ---- dominant kernel: fused RMSNorm + gate|up GEMV + SwiGLU (76.4 MB of blocks per launch at the 7B shape) ----
     L = cfg["n_layers"]
+    if ne:
+        print(json.dumps({"metric": "decode tok/s (%s)" % args.config, "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
+                          "ms_per_step": round(ms_per_step, 4), "batch": B, "algorithmic_bytes_per_step": int(algo_bytes),
+                          "whole_step_hbm_frac": round(algo_bytes / (wall / K) / 1e9 / HBM_PEAK_GBS, 4),
+                          "prefill": {"tokens": prompt_len - 1, "ms": round(pf_ms.value, 2)}}))
+        return
     gu = [spec["tensors"][(l, cai.W_GATEUP)]["qw"] for l in range(L)]
     d, I = cfg["d_model"], cfg["ffn"]
     x = torch.randn(d, device="cuda"); g = torch.ones(d, device="cuda"); y = torch.empty(I, device="cuda")
@@ -161,21 +193,22 @@ def main():
     k_gbs = k_bytes / (k_avg_us * 1e-6) / 1e9
 
     res = {
-        "metric": "decode tok/s @bs1 (Qwen2.5-7B-shape Q4_K) + % of HBM-bandwidth roofline",
+        "metric": "decode tok/s @bs1 (Qwen2.5-7B-shape Q4_K) + % of HBM-bandwidth roofline" if args.config == "qwen2.5-7b-q4k" and B == 1
+                  else "decode tok/s (%s, batch %d)" % (args.config, B),
         "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "q4_k/q8_0 weights, f32 accumulate", "data": "synthetic",
-        "config": {"workload": "%s: %d-token random prompt (seed 424242), then greedy decode at batch 1; timed %d decode tokens at ctx %d..%d"
-                               % (args.config, prompt_len, K, pos + 1, pos + K),
-                   "weights": "random N(0,0.02), %s body + %s head, fp32 KV cache" % (conf["qtype"], conf["head"]),
-                   "algorithmic_bytes_per_token": int(algo_bytes), "hip_event_ms_per_step": round(ms.value / K, 4),
+        "config": {"workload": "%s: %d-token random prompt (seed 424242), then greedy decode at batch %d; timed %d decode steps at ctx %d..%d"
+                               % (args.config, prompt_len, B, K, pos + 1, pos + K),
+                   "weights": "random N(0,0.02), %s body + %s head, %s KV cache" % (conf["qtype"], conf["head"], conf.get("kv", "f32")),
+                   "algorithmic_bytes_per_step": int(algo_bytes), "hip_event_ms_per_step": round(ms.value / K, 4),
                    "whole_step_hbm_frac": round(algo_bytes / (wall / K) / 1e9 / HBM_PEAK_GBS, 4), "device": cai.device_name(),
                    "build_s": round(t_build, 1),
                    "prefill": {"tokens": prompt_len - 1, "ms": round(pf_ms.value, 2),
                                "tok_per_s": round((prompt_len - 1) / max(pf_ms.value, 1e-6) * 1e3, 1),
                                "linear_tflops": round(2.0 * n_lin_weights * (prompt_len - 1) / max(pf_ms.value, 1e-6) / 1e9, 1),
                                "note": "multi-token ingestion: f16 MFMA (exact block integers, hi/lo-split activations = 2 MFMA passes per useful FLOP) + prompt attention; MFMA f16 dense peak 2500 TFLOP/s"}},
-        "roofline": {"bound": "hbm", "kernel": "gemv_q4k_stream<1,1,false> (RMSNorm+gate|up+SwiGLU, %dx%d)" % (2 * I, d),
+        "roofline": {"bound": "hbm", "kernel": "%s (RMSNorm+gate|up+SwiGLU, %dx%d)" % ("gemv_q4k_dot<1,1,false,2>" if conf["qtype"] == "Q4_K" else "gemv_fast<%s>" % conf["qtype"], 2 * I, d),
                      "achieved": round(k_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(k_gbs / HBM_PEAK_GBS, 4),
                      "avg_launch_us": round(k_avg_us, 2), "algorithmic_bytes_per_launch": int(k_bytes),
                      "traffic": GATEUP_TRAFFIC_BYTES if args.config == "qwen2.5-7b-q4k" else None, "traffic_unit": "bytes/launch"},

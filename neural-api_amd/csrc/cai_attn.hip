@@ -35,6 +35,22 @@ template <typename T> __device__ __forceinline__ T kv_from_float(float v);
 template <> __device__ __forceinline__ float kv_from_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ __half kv_from_float<__half>(float v) { return __float2half_rn(v); }
 
+
+// DS consecutive cache elements as floats with ONE vector load (the head width is a multiple of DS, so a lane's
+// DS-wide slot is either wholly inside the row or wholly outside it)
+template <int DS, typename KV_T> __device__ __forceinline__ void load_row_vec(const KV_T* src, float (&o)[DS]);
+template <> __device__ __forceinline__ void load_row_vec<1, float>(const float* s, float (&o)[1]) { o[0] = s[0]; }
+template <> __device__ __forceinline__ void load_row_vec<2, float>(const float* s, float (&o)[2]) { const float2 v = *reinterpret_cast<const float2*>(s); o[0] = v.x; o[1] = v.y; }
+template <> __device__ __forceinline__ void load_row_vec<4, float>(const float* s, float (&o)[4]) { const float4 v = *reinterpret_cast<const float4*>(s); o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w; }
+template <> __device__ __forceinline__ void load_row_vec<1, __half>(const __half* s, float (&o)[1]) { o[0] = __half2float(s[0]); }
+template <> __device__ __forceinline__ void load_row_vec<2, __half>(const __half* s, float (&o)[2]) { const __half2 v = *reinterpret_cast<const __half2*>(s); o[0] = __low2float(v); o[1] = __high2float(v); }
+template <> __device__ __forceinline__ void load_row_vec<4, __half>(const __half* s, float (&o)[4])
+{
+  const uint2 r = *reinterpret_cast<const uint2*>(s);
+  const __half2 a = __builtin_bit_cast(__half2, r.x), b = __builtin_bit_cast(__half2, r.y);
+  o[0] = __low2float(a); o[1] = __high2float(a); o[2] = __low2float(b); o[3] = __high2float(b);
+}
+
 struct AttnParams {
   float* qkv; int64_t qkv_stride;
   void* kc; void* vc;          // base of [seq][layer][kv_head][max_ctx][hd]
@@ -85,19 +101,15 @@ __global__ __launch_bounds__(256) void attn_step_kernel(const AttnParams p)
   float* st_a = st_l + G * 256;
 
   constexpr int PCH = 4;
-  float kdA[PCH][DS], vdA[PCH][DS], kdB[PCH][DS], vdB[PCH][DS];
+  float kdA[PCH][DS] = {}, vdA[PCH][DS] = {}, kdB[PCH][DS] = {}, vdB[PCH][DS] = {};
   auto load_chunk = [&](float (&kd)[PCH][DS], float (&vd)[PCH][DS], int j0) {
-    if (j0 >= s_end) return;
+    if (j0 >= s_end || d0 >= hd) return;       // lanes beyond the head width keep their zeros
 #pragma unroll
     for (int c = 0; c < PCH; c++) {
       const int j = min(j0 + 8 * c, s_end - 1);
-#pragma unroll
-      for (int i = 0; i < DS; i++) {
-        const int d = d0 + i;
-        const bool ok = d < hd && (j != pos || p.appended);   // the row appended here comes from registers
-        kd[c][i] = ok ? kv_to_float<KV_T>(kc[(int64_t)j * hd + d]) : 0.0f;
-        vd[c][i] = ok ? kv_to_float<KV_T>(vc[(int64_t)j * hd + d]) : 0.0f;
-      }
+      // (the slot of the row being appended may hold stale values: reduce_chunk replaces it from registers)
+      load_row_vec<DS, KV_T>(kc + (int64_t)j * hd + d0, kd[c]);
+      load_row_vec<DS, KV_T>(vc + (int64_t)j * hd + d0, vd[c]);
     }
   };
   load_chunk(kdA, vdA, s_begin + hw);      // cached rows are requested before the rotation math
@@ -295,19 +307,15 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
   KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (seq * p.seq_mul + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
 
   constexpr int PCH = 4;
-  float kdA[PCH][DS], vdA[PCH][DS], kdB[PCH][DS], vdB[PCH][DS];
+  float kdA[PCH][DS] = {}, vdA[PCH][DS] = {}, kdB[PCH][DS] = {}, vdB[PCH][DS] = {};
   auto load_chunk = [&](float (&kd)[PCH][DS], float (&vd)[PCH][DS], int j0) {
-    if (j0 >= s_end) return;
+    if (j0 >= s_end || d0 >= hd) return;       // lanes beyond the head width keep their zeros
 #pragma unroll
     for (int c = 0; c < PCH; c++) {
       const int j = min(j0 + 8 * c, s_end - 1);
-#pragma unroll
-      for (int i = 0; i < DS; i++) {
-        const int d = d0 + i;
-        const bool ok = d < hd && (j != pos || p.appended);   // the row appended here comes from registers
-        kd[c][i] = ok ? kv_to_float<KV_T>(kc[(int64_t)j * hd + d]) : 0.0f;
-        vd[c][i] = ok ? kv_to_float<KV_T>(vc[(int64_t)j * hd + d]) : 0.0f;
-      }
+      // (the slot of the row being appended may hold stale values: reduce_chunk replaces it from registers)
+      load_row_vec<DS, KV_T>(kc + (int64_t)j * hd + d0, kd[c]);
+      load_row_vec<DS, KV_T>(vc + (int64_t)j * hd + d0, vd[c]);
     }
   };
   load_chunk(kdA, vdA, s_begin + hw);      // cached rows are requested before the rotation math
@@ -515,7 +523,7 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
 // ------------------------------------------------------------------------------------------
 int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, int max_ctx, int dtype)
 {
-  if (n_seq < 1 || n_layers < 1 || kv_heads < 1 || head_dim < 2 || (head_dim & 1) || head_dim > 128 || max_ctx < 1)
+  if (n_seq < 1 || n_layers < 1 || kv_heads < 1 || head_dim < 2 || (head_dim & 1) || (head_dim > 64 && (head_dim & 3)) || head_dim > 128 || max_ctx < 1)
     return set_error(CAI_ERR_INVALID, "kv cache: bad geometry seq=%d layers=%d kv_heads=%d head_dim=%d max_ctx=%d", n_seq, n_layers, kv_heads, head_dim, max_ctx);
   if (dtype != CAI_KV_F32 && dtype != CAI_KV_F16) return set_error(CAI_ERR_INVALID, "kv cache: dtype %d", dtype);
   kv->n_seq = n_seq; kv->n_layers = n_layers; kv->kv_heads = kv_heads; kv->head_dim = head_dim; kv->max_ctx = max_ctx; kv->dtype = dtype;
@@ -532,7 +540,7 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   CAI_HIP(hipMemsetAsync(kv->v, 0, bytes, ctx().stream));
   {
     const char* e = getenv("CAIHIP_ATTN_SHORT_CTX");      // caches up to this capacity use the per-head split kernel
-    kv->short_ctx_limit = e ? atoi(e) : 4096;
+    kv->short_ctx_limit = e ? atoi(e) : (1 << 30);
   }
   kv->part_q_heads = kv_heads * 8;
   CAI_HIP(hipMalloc(&kv->part, (size_t)n_seq * kv->part_q_heads * kv->n_splits * (head_dim + 2) * sizeof(float)));

@@ -101,8 +101,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
       }
     }
     if (c.qk_norm_full) {
-      launch_rmsnorm_strided(d->qkv, L.v[CAI_V_Q_NORM], qw, n_b, c.eps, d->qkv, qkvw, qkvw);
-      launch_rmsnorm_strided(d->qkv + qw, L.v[CAI_V_K_NORM], kw, n_b, c.eps, d->qkv + qw, qkvw, qkvw);
+      launch_rmsnorm_pair(d->qkv, L.v[CAI_V_Q_NORM], qw, L.v[CAI_V_K_NORM], kw, n_b, c.eps, qkvw);
     }
     if ((rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0))) return rc;
     const bool o_hands = gemv_hands_off_ssq(L.w[CAI_W_O], n_b);
@@ -214,8 +213,7 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
     if ((rc = linear_rows(wk, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw, qkvw, nullptr))) return rc;
     if ((rc = linear_rows(wv, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw + kw, qkvw, nullptr))) return rc;
     if (c.qk_norm_full) {
-      launch_rmsnorm_strided(d->pqkv, L.v[CAI_V_Q_NORM], qw, n, c.eps, d->pqkv, qkvw, qkvw);
-      launch_rmsnorm_strided(d->pqkv + qw, L.v[CAI_V_K_NORM], kw, n, c.eps, d->pqkv + qw, qkvw, qkvw);
+      launch_rmsnorm_pair(d->pqkv, L.v[CAI_V_Q_NORM], qw, L.v[CAI_V_K_NORM], kw, n, c.eps, qkvw);
     }
     if ((rc = launch_attn_step(&d->kv, l, d->pqkv, qkvw, n, c.n_q_heads, c.window, 0.0f, d->theta, poss, d->patt, qw, seq, 1, d->ppart))) return rc;
     if ((rc = linear_rows(L.w[CAI_W_O], false, d->patt, qw, nullptr, 0.0f, n, d->px, dm, d->px))) return rc;

@@ -129,6 +129,29 @@ int launch_rmsnorm_strided(const float* x, const float* gain, int n, int n_token
   hipLaunchKernelGGL(rmsnorm_kernel, dim3(n_tokens), dim3(256), 0, ctx().stream, x, gain, n, eps, y, x_stride, y_stride);
   return CAI_OK;
 }
+// Two adjacent segments of every token row normalised in place by one launch (full-width q and k norms of OLMoE,
+// neural/neuralpretrained.pas:16511-16530): work-group (t, 0) takes [0, n_a), (t, 1) takes [n_a, n_a + n_b).
+__global__ __launch_bounds__(256) void rmsnorm_pair_kernel(float* x, const float* gain_a, int n_a, const float* gain_b, int n_b, float eps, int64_t stride)
+{
+  float* xr = x + (int64_t)blockIdx.x * stride + (blockIdx.y ? n_a : 0);
+  const float* gain = blockIdx.y ? gain_b : gain_a;
+  const int n = blockIdx.y ? n_b : n_a;
+  __shared__ float red[4];
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < n; i += 256) ss = fmaf(xr[i], xr[i], ss);
+  ss = wave_sum_all(ss);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float tot = (red[0] + red[1]) + (red[2] + red[3]);
+  const float inv = 1.0f / sqrtf(tot / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += 256) xr[i] = gain[i] * (xr[i] * inv);
+}
+
+int launch_rmsnorm_pair(float* x, const float* gain_a, int n_a, const float* gain_b, int n_b, int n_tokens, float eps, int64_t stride)
+{
+  hipLaunchKernelGGL(rmsnorm_pair_kernel, dim3(n_tokens, 2), dim3(256), 0, ctx().stream, x, gain_a, n_a, gain_b, n_b, eps, stride);
+  return CAI_OK;
+}
 int launch_rmsnorm(const float* x, const float* gain, int n, int n_tokens, float eps, float* y)
 {
   return launch_rmsnorm_strided(x, gain, n, n_tokens, eps, y, n, n);
@@ -240,37 +263,62 @@ int launch_argmax(const float* x, int n, int n_rows, int32_t* out, float* scratc
 int argmax_scratch_entries(int n, int n_rows) { return (n + 4095) / 4096 * n_rows; }
 
 // ---- router: TNNetPointwiseSoftMax (neural/neural.cl:1594-1647) + TNNetTopKGate ----
-// One thread per token, the way the reference keeps a group's reduction inside one work-item.
-__global__ void router_topk_kernel(const float* logits, int n, int k, int renorm, int n_tokens, int32_t* expert_out, float* gate_out, float* probs)
+// One wave per token; lane i owns experts i, i+64, ...  Selection is k rounds of a wave-wide arg-max in which the
+// larger probability wins and, between equals, the lower expert index (the reference scans upwards with '>').
+constexpr int ROUTER_MAX_PER_LANE = 8;   // up to 512 experts
+__global__ __launch_bounds__(64) void router_topk_kernel(const float* logits, int n, int k, int renorm, int n_tokens, int32_t* expert_out, float* gate_out, float* probs)
 {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n_tokens) return;
+  const int t = blockIdx.x, lane = threadIdx.x;
   const float* x = logits + (int64_t)t * n;
-  float* p = probs + (int64_t)t * n;
-  float mx = x[0];
-  for (int c = 1; c < n; c++) mx = fmaxf(mx, x[c]);
+  float v[ROUTER_MAX_PER_LANE];
+  float mx = -3.0e38f;
+#pragma unroll
+  for (int i = 0; i < ROUTER_MAX_PER_LANE; i++) {
+    const int c = lane + 64 * i;
+    v[i] = c < n ? x[c] : -3.0e38f;
+    mx = fmaxf(mx, v[i]);
+  }
+  for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
   float tot = 0.0f;
-  for (int c = 0; c < n; c++) {
-    float a = x[c] - mx; a = a > 4000.0f ? 4000.0f : (a < -4000.0f ? -4000.0f : a);
-    const float e = expf(a); p[c] = e; tot += e;
+#pragma unroll
+  for (int i = 0; i < ROUTER_MAX_PER_LANE; i++) {
+    const int c = lane + 64 * i;
+    float a = v[i] - mx; a = a > 4000.0f ? 4000.0f : (a < -4000.0f ? -4000.0f : a);
+    v[i] = c < n ? expf(a) : 0.0f;
+    tot += v[i];
   }
-  if (tot > 0.0f) { const float inv = 1.0f / tot; for (int c = 0; c < n; c++) p[c] *= inv; }
-  float sum = 0.0f;
+  for (int m = 32; m >= 1; m >>= 1) tot += __shfl_xor(tot, m, 64);
+  const float inv = tot > 0.0f ? 1.0f / tot : 1.0f;
+#pragma unroll
+  for (int i = 0; i < ROUTER_MAX_PER_LANE; i++) {
+    const int c = lane + 64 * i;
+    v[i] *= inv;
+    if (c < n) probs[(int64_t)t * n + c] = v[i]; else v[i] = -1.0f;   // -1 marks "not a candidate"
+  }
+  float sum = 0.0f, mine = 0.0f;   // lane j keeps the j-th selected gate
   for (int j = 0; j < k; j++) {
-    int best = -1; float bv = 0.0f;
-    for (int c = 0; c < n; c++) {
-      const float v = p[c];
-      if (v >= 0.0f && (best < 0 || v > bv)) { best = c; bv = v; }
+    float bv = -1.0f; int bc = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < ROUTER_MAX_PER_LANE; i++)
+      if (v[i] > bv) { bv = v[i]; bc = lane + 64 * i; }   // ascending index inside the lane: '>' keeps the first
+    for (int m = 32; m >= 1; m >>= 1) {
+      const float ov = __shfl_xor(bv, m, 64); const int oc = __shfl_xor(bc, m, 64);
+      if (ov > bv || (ov == bv && oc < bc)) { bv = ov; bc = oc; }
     }
-    expert_out[t * k + j] = best; gate_out[t * k + j] = bv; sum += bv;
-    p[best] = -1.0f;   // taken
+    if ((bc & 63) == lane) {
+#pragma unroll
+      for (int i = 0; i < ROUTER_MAX_PER_LANE; i++) if (bc == lane + 64 * i) v[i] = -1.0f;   // taken
+    }
+    if (lane == (j & 63)) { mine = bv; expert_out[t * k + j] = bc; }
+    sum += bv;
   }
-  if (renorm) { const float inv = sum > 0.0f ? 1.0f / sum : 0.0f; for (int j = 0; j < k; j++) gate_out[t * k + j] *= inv; }
+  if (lane < k) gate_out[t * k + lane] = renorm ? (sum > 0.0f ? mine * (1.0f / sum) : 0.0f) : mine;
 }
 
 int launch_router_topk(const float* logits, int n, int k, int renorm, int n_tokens, int32_t* expert_out, float* gate_out, float* probs_scratch)
 {
-  hipLaunchKernelGGL(router_topk_kernel, dim3((n_tokens + 63) / 64), dim3(64), 0, ctx().stream, logits, n, k, renorm, n_tokens, expert_out, gate_out, probs_scratch);
+  if (n < 1 || n > 64 * ROUTER_MAX_PER_LANE || k < 1 || k > 64 || k > n) return set_error(CAI_ERR_UNSUPPORTED, "router: %d experts, top-%d (supported: up to %d experts, k <= 64)", n, k, 64 * ROUTER_MAX_PER_LANE);
+  hipLaunchKernelGGL(router_topk_kernel, dim3(n_tokens), dim3(64), 0, ctx().stream, logits, n, k, renorm, n_tokens, expert_out, gate_out, probs_scratch);
   return CAI_OK;
 }
 
