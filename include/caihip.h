@@ -215,7 +215,38 @@ int cai_decoder_len(cai_decoder_t d, int seq, int* len_out);
 int cai_decoder_snapshot(cai_decoder_t d, int seq, cai_kv_snap_t* out);
 int cai_decoder_restore(cai_decoder_t d, int seq, cai_kv_snap_t snap);
 /* Bytes of weights, biases and gains one decoded token streams (for roofline accounting). */
+/* the configuration the decoder was created with (a loader fills it from the file) */
+int cai_decoder_get_config(cai_decoder_t d, cai_decoder_config* out);
 int cai_decoder_weight_bytes(cai_decoder_t d, int64_t* algorithmic_bytes_out);
+
+/* ---------------------------------------------------------------------------------------------
+ * GGUF container (replaces TNNetGGUFReader, neural/neuralgguf.pas:1072-1220 ParseFile, 1525-1672 tensor reads)
+ * and the llama / qwen2 importer (BuildLlamaFromGGUFEx and the qwen2 branch, neural/neuralpretrained.pas:17484-17876).
+ * The file is mapped read-only.  Shapes are row-major (ggml's contiguous axis last): an HF [out, in] matrix reads
+ * [out, in].  Tokenizer metadata stays with the host application.
+ * ------------------------------------------------------------------------------------------- */
+typedef struct cai_gguf_s* cai_gguf_t;
+int cai_gguf_open(const char* path, cai_gguf_t* out);
+int cai_gguf_close(cai_gguf_t g);
+int cai_gguf_info(cai_gguf_t g, int* version, int* alignment, int64_t* n_tensors, int64_t* n_meta, int64_t* data_start);
+int cai_gguf_meta_int(cai_gguf_t g, const char* key, int64_t* out);      /* GetMetaInt: any integer or bool value */
+int cai_gguf_meta_float(cai_gguf_t g, const char* key, double* out);     /* GetMetaFloat */
+int cai_gguf_meta_str(cai_gguf_t g, const char* key, char* buf, int n);  /* GetMetaString */
+int cai_gguf_meta_array_count(cai_gguf_t g, const char* key, int64_t* out);
+int cai_gguf_meta_array_str(cai_gguf_t g, const char* key, int64_t index, char* buf, int n);  /* GetMetaArrayString */
+int cai_gguf_find_tensor(cai_gguf_t g, const char* name, int64_t* index);
+int cai_gguf_tensor_info(cai_gguf_t g, int64_t index, char* name_buf, int name_n, int* ggml_type, int* n_dims,
+                         int64_t* shape8, int64_t* data_offset, int64_t* nbytes);
+/* pointer into the mapping, valid until cai_gguf_close (the raw-bytes read of neural/neuralsafetensors.pas:1024) */
+int cai_gguf_tensor_data(cai_gguf_t g, int64_t index, const void** ptr);
+/* resident weight from a 2-D tensor in stored order and stored type (F32, F16, Q4_0, Q8_0, Q4_K); bias_name may be
+ * NULL or name a tensor that is absent */
+int cai_gguf_load_qw(cai_gguf_t g, const char* name, const char* bias_name, cai_qw_t* out);
+/* Whole decoder from a llama or qwen2 file; the decoder owns the weights it loads.  max_ctx <= 0 takes
+ * <arch>.context_length.  Blocks go up in stored order: llama.cpp's q/k row order is the interleaved-rotary order
+ * the decode kernels rotate (neural/neuralgguf.pas:428-438 composed with neural/neuralpretrained.pas:14792-14812
+ * is the identity). */
+int cai_decoder_load_gguf(const char* path, int max_ctx, int max_batch, int kv_dtype, cai_decoder_t* out);
 
 #ifdef __cplusplus
 }

@@ -21,7 +21,9 @@ cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_router_topk
 cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_attn_decode
 cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_generate
 cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_snapshot cai_decoder_restore
-cai_decoder_weight_bytes""".split()
+cai_decoder_weight_bytes cai_decoder_get_config cai_decoder_load_gguf
+cai_gguf_open cai_gguf_close cai_gguf_info cai_gguf_meta_int cai_gguf_meta_float cai_gguf_meta_str cai_gguf_meta_array_count
+cai_gguf_meta_array_str cai_gguf_find_tensor cai_gguf_tensor_info cai_gguf_tensor_data cai_gguf_load_qw""".split()
 
 
 class DecoderConfig(C.Structure):
@@ -93,6 +95,20 @@ def load():
         L.cai_decoder_snapshot.argtypes = [vp, i32, C.POINTER(vp)]
         L.cai_decoder_restore.argtypes = [vp, i32, vp]
         L.cai_decoder_weight_bytes.argtypes = [vp, C.POINTER(i64)]
+        L.cai_decoder_get_config.argtypes = [vp, C.POINTER(DecoderConfig)]
+        L.cai_decoder_load_gguf.argtypes = [C.c_char_p, i32, i32, i32, C.POINTER(vp)]
+        L.cai_gguf_open.argtypes = [C.c_char_p, C.POINTER(vp)]
+        L.cai_gguf_close.argtypes = [vp]
+        L.cai_gguf_info.argtypes = [vp, C.POINTER(i32), C.POINTER(i32), C.POINTER(i64), C.POINTER(i64), C.POINTER(i64)]
+        L.cai_gguf_meta_int.argtypes = [vp, C.c_char_p, C.POINTER(i64)]
+        L.cai_gguf_meta_float.argtypes = [vp, C.c_char_p, C.POINTER(C.c_double)]
+        L.cai_gguf_meta_str.argtypes = [vp, C.c_char_p, C.c_char_p, i32]
+        L.cai_gguf_meta_array_count.argtypes = [vp, C.c_char_p, C.POINTER(i64)]
+        L.cai_gguf_meta_array_str.argtypes = [vp, C.c_char_p, i64, C.c_char_p, i32]
+        L.cai_gguf_find_tensor.argtypes = [vp, C.c_char_p, C.POINTER(i64)]
+        L.cai_gguf_tensor_info.argtypes = [vp, i64, C.c_char_p, i32, C.POINTER(i32), C.POINTER(i32), C.POINTER(i64), C.POINTER(i64), C.POINTER(i64)]
+        L.cai_gguf_tensor_data.argtypes = [vp, i64, C.POINTER(vp)]
+        L.cai_gguf_load_qw.argtypes = [vp, C.c_char_p, C.c_char_p, C.POINTER(vp)]
     return _LIB
 
 
@@ -228,8 +244,94 @@ class KVCache:
             pass
 
 
+class GGUF:
+    """cai_gguf_t: the container reader (no GPU needed)."""
+
+    def __init__(self, path):
+        self.h = C.c_void_p()
+        check(load().cai_gguf_open(os.fsencode(path), C.byref(self.h)))
+
+    def info(self):
+        v, a = C.c_int(), C.c_int(); nt, nm, ds = C.c_int64(), C.c_int64(), C.c_int64()
+        check(load().cai_gguf_info(self.h, C.byref(v), C.byref(a), C.byref(nt), C.byref(nm), C.byref(ds)))
+        return dict(version=v.value, alignment=a.value, n_tensors=nt.value, n_meta=nm.value, data_start=ds.value)
+
+    def meta_int(self, key, default=None):
+        v = C.c_int64()
+        rc = load().cai_gguf_meta_int(self.h, key.encode(), C.byref(v))
+        if rc != 0 and default is not None:
+            return default
+        check(rc)
+        return v.value
+
+    def meta_float(self, key, default=None):
+        v = C.c_double()
+        rc = load().cai_gguf_meta_float(self.h, key.encode(), C.byref(v))
+        if rc != 0 and default is not None:
+            return default
+        check(rc)
+        return v.value
+
+    def meta_str(self, key, default=None):
+        buf = C.create_string_buffer(4096)
+        rc = load().cai_gguf_meta_str(self.h, key.encode(), buf, 4096)
+        if rc != 0 and default is not None:
+            return default
+        check(rc)
+        return buf.value.decode("utf-8", "replace")
+
+    def meta_array_count(self, key):
+        v = C.c_int64()
+        check(load().cai_gguf_meta_array_count(self.h, key.encode(), C.byref(v)))
+        return v.value
+
+    def meta_array_str(self, key, index):
+        buf = C.create_string_buffer(4096)
+        check(load().cai_gguf_meta_array_str(self.h, key.encode(), index, buf, 4096))
+        return buf.value.decode("utf-8", "replace")
+
+    def has_tensor(self, name):
+        i = C.c_int64()
+        return load().cai_gguf_find_tensor(self.h, name.encode(), C.byref(i)) == 0
+
+    def tensor(self, name_or_index):
+        i = C.c_int64(name_or_index) if isinstance(name_or_index, int) else C.c_int64()
+        if not isinstance(name_or_index, int):
+            check(load().cai_gguf_find_tensor(self.h, name_or_index.encode(), C.byref(i)))
+        nb = C.create_string_buffer(512); t, nd = C.c_int(), C.c_int(); sh = (C.c_int64 * 8)(); off, nbytes = C.c_int64(), C.c_int64()
+        check(load().cai_gguf_tensor_info(self.h, i.value, nb, 512, C.byref(t), C.byref(nd), sh, C.byref(off), C.byref(nbytes)))
+        return dict(index=i.value, name=nb.value.decode(), type=t.value, shape=list(sh[:nd.value]), offset=off.value, nbytes=nbytes.value)
+
+    def tensor_bytes(self, name):
+        t = self.tensor(name)
+        p = C.c_void_p()
+        check(load().cai_gguf_tensor_data(self.h, t["index"], C.byref(p)))
+        return np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_uint8)), shape=(t["nbytes"],)).copy()
+
+    def close(self):
+        if self.h:
+            load().cai_gguf_close(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class Decoder:
     """cai_decoder_t built from a backend-neutral spec: {"cfg", "tensors", "vecs"}."""
+
+    @classmethod
+    def from_gguf(cls, path, max_ctx=0, max_batch=1, kv_dtype=KV_F32):
+        """llama / qwen2 file loaded by the library itself (cai_decoder_load_gguf)."""
+        self = cls.__new__(cls)
+        self.h = C.c_void_p(); self.weights = []
+        check(load().cai_decoder_load_gguf(os.fsencode(path), max_ctx, max_batch, kv_dtype, C.byref(self.h)))
+        self.cfg = DecoderConfig()
+        check(load().cai_decoder_get_config(self.h, C.byref(self.cfg)))
+        return self
 
     def __init__(self, spec, max_batch=1, kv_dtype=KV_F32, max_ctx=None):
         c = spec["cfg"]

@@ -32,6 +32,7 @@ struct cai_decoder_s {
   int32_t* h_io = nullptr;   // pinned: tokens[8] pos[8] argmax[8]
   hipGraphExec_t graph[9] = {nullptr};
   bool use_graph = true;
+  std::vector<cai_qw_s*> owned;   // weights created by a loader on the decoder's behalf, destroyed with it
   int qw() const { return cfg.n_q_heads * cfg.head_dim; }
   int kw() const { return cfg.n_kv_heads * cfg.head_dim; }
 };
@@ -314,9 +315,14 @@ extern "C" int cai_decoder_destroy(cai_decoder_t d)
   if (d->d_tokens) (void)hipFree(d->d_tokens);
   if (d->d_gen) (void)hipFree(d->d_gen);
   if (d->h_io) (void)hipHostFree(d->h_io);
+  for (cai_qw_s* w : d->owned) (void)cai_qw_destroy(w);
   delete d;
   return CAI_OK;
 }
+
+namespace cai {
+void decoder_adopt_weight(cai_decoder_s* d, cai_qw_s* w) { d->owned.push_back(w); }
+}  // namespace cai
 
 extern "C" int cai_decoder_set_weight(cai_decoder_t d, int layer, int slot, cai_qw_t w)
 {
@@ -505,6 +511,13 @@ extern "C" int cai_decoder_restore(cai_decoder_t d, int seq, cai_kv_snap_t snap)
   CAI_REQUIRE(d && snap, "cai_decoder_restore: null argument");
   CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch, "cai_decoder_restore: sequence %d of %d", seq, d->cfg.max_batch);
   return kv_restore(&d->kv, seq, snap);
+}
+
+extern "C" int cai_decoder_get_config(cai_decoder_t d, cai_decoder_config* out)
+{
+  CAI_REQUIRE(d && out, "cai_decoder_get_config: null argument");
+  *out = d->cfg;
+  return CAI_OK;
 }
 
 extern "C" int cai_decoder_weight_bytes(cai_decoder_t d, int64_t* out)

@@ -119,6 +119,7 @@ int argmax_scratch_entries(int n, int n_rows);
 int launch_embed(const cai_qw_s* w, const int32_t* tokens_dev, int n_tokens, float* out);
 int launch_router_topk(const float* logits, int n, int k, int renorm, int n_tokens, int32_t* expert_out, float* gate_out, float* probs_scratch);
 int launch_rmsnorm_strided(const float* x, const float* gain, int n, int n_tokens, float eps, float* y, int64_t x_stride, int64_t y_stride);
+void decoder_adopt_weight(cai_decoder_s* d, cai_qw_s* w);   // the decoder destroys w with itself
 int launch_rmsnorm_pair(float* x, const float* gain_a, int n_a, const float* gain_b, int n_b, int n_tokens, float eps, int64_t stride);
 int launch_moe_combine(float* x, const float* part, const float* gate, int k, int n, int n_tokens);
 int launch_split_blocks(const uint8_t* raw, int block_bytes, int64_t n_blocks, uint8_t* qs, uint16_t* d);

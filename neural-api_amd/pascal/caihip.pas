@@ -30,8 +30,8 @@ const
   CAI_V_ATTN_NORM = 0; CAI_V_MLP_NORM = 1; CAI_V_FINAL_NORM = 2; CAI_V_Q_NORM = 3; CAI_V_K_NORM = 4;
 
 type
-  TCaiQW = Pointer; TCaiKV = Pointer; TCaiKVSnap = Pointer; TCaiDecoder = Pointer;
-  PCaiQW = ^TCaiQW; PCaiKV = ^TCaiKV; PCaiKVSnap = ^TCaiKVSnap; PCaiDecoder = ^TCaiDecoder;
+  TCaiQW = Pointer; TCaiKV = Pointer; TCaiKVSnap = Pointer; TCaiDecoder = Pointer; TCaiGGUF = Pointer;
+  PCaiQW = ^TCaiQW; PCaiKV = ^TCaiKV; PCaiKVSnap = ^TCaiKVSnap; PCaiDecoder = ^TCaiDecoder; PCaiGGUF = ^TCaiGGUF;
 
   TCaiDecoderConfig = packed record
     n_layers, d_model, n_q_heads, n_kv_heads, head_dim, ffn, vocab, max_ctx: LongInt;
@@ -92,6 +92,22 @@ function cai_decoder_len(d: TCaiDecoder; seq: LongInt; len_out: PLongInt): LongI
 function cai_decoder_snapshot(d: TCaiDecoder; seq: LongInt; out_snap: PCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_restore(d: TCaiDecoder; seq: LongInt; snap: TCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_weight_bytes(d: TCaiDecoder; algorithmic_bytes_out: PInt64): LongInt; cdecl; external CAIHIP_LIB;
+function cai_decoder_get_config(d: TCaiDecoder; out_cfg: Pointer): LongInt; cdecl; external CAIHIP_LIB;
+function cai_decoder_load_gguf(path: PChar; max_ctx, max_batch, kv_dtype: LongInt; out_decoder: PCaiDecoder): LongInt; cdecl; external CAIHIP_LIB;
+
+// GGUF container (TNNetGGUFReader, neural/neuralgguf.pas:1072-1220)
+function cai_gguf_open(path: PChar; out_gguf: PCaiGGUF): LongInt; cdecl; external CAIHIP_LIB;
+function cai_gguf_close(g: TCaiGGUF): LongInt; cdecl; external CAIHIP_LIB;
+function cai_gguf_info(g: TCaiGGUF; version, alignment: PLongInt; n_tensors, n_meta, data_start: PInt64): LongInt; cdecl; external CAIHIP_LIB;
+function cai_gguf_meta_int(g: TCaiGGUF; key: PChar; out_value: PInt64): LongInt; cdecl; external CAIHIP_LIB;
+function cai_gguf_meta_float(g: TCaiGGUF; key: PChar; out_value: PDouble): LongInt; cdecl; external CAIHIP_LIB;
+function cai_gguf_meta_str(g: TCaiGGUF; key: PChar; buf: PChar; n: LongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_gguf_meta_array_count(g: TCaiGGUF; key: PChar; out_count: PInt64): LongInt; cdecl; external CAIHIP_LIB;
+function cai_gguf_meta_array_str(g: TCaiGGUF; key: PChar; index: Int64; buf: PChar; n: LongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_gguf_find_tensor(g: TCaiGGUF; name: PChar; index: PInt64): LongInt; cdecl; external CAIHIP_LIB;
+function cai_gguf_tensor_info(g: TCaiGGUF; index: Int64; name_buf: PChar; name_n: LongInt; ggml_type, n_dims: PLongInt; shape8, data_offset, nbytes: PInt64): LongInt; cdecl; external CAIHIP_LIB;
+function cai_gguf_tensor_data(g: TCaiGGUF; index: Int64; ptr: PPointer): LongInt; cdecl; external CAIHIP_LIB;
+function cai_gguf_load_qw(g: TCaiGGUF; name, bias_name: PChar; out_qw: PCaiQW): LongInt; cdecl; external CAIHIP_LIB;
 
 implementation
 

@@ -1,0 +1,115 @@
+"""The library's GGUF container reader against the reference's fixtures and its parse-error rules
+(TNNetGGUFReader.ParseFile, neural/neuralgguf.pas:1072-1220; assertions of tests/TestNeuralPretrained.pas:5765-5817).
+Runs without a GPU: the container entry points touch no device."""
+import struct
+
+import numpy as np
+import pytest
+
+from helpers.device import cai
+from helpers.fixtures_io import GGUFFile, ref_path
+
+
+def test_tiny_llama_f32_metadata_and_tensor_table():
+    g = cai.GGUF(ref_path("tiny_llama_f32.gguf"))
+    info = g.info()
+    assert info["version"] == 3 and info["alignment"] == 32 and info["n_tensors"] == 21
+    assert g.meta_str("general.architecture") == "llama"
+    assert g.meta_int("llama.block_count") == 2
+    assert g.meta_int("llama.embedding_length") == 8
+    assert g.meta_int("llama.feed_forward_length") == 12
+    assert g.meta_int("llama.attention.head_count") == 2
+    assert g.meta_int("llama.attention.head_count_kv") == 1
+    assert g.meta_int("llama.context_length") == 16
+    assert g.meta_int("llama.vocab_size") == 11
+    assert abs(g.meta_float("llama.rope.freq_base") - 10000.0) < 1e-3
+    assert abs(g.meta_float("llama.attention.layer_norm_rms_epsilon") - 1e-5) < 1e-9
+    assert g.meta_int("no.such.key", 77) == 77 and g.meta_str("no.such.key", "dflt") == "dflt"
+    assert g.meta_str("tokenizer.ggml.model") == "llama"
+    assert g.meta_array_count("tokenizer.ggml.tokens") == 11
+    assert g.meta_array_str("tokenizer.ggml.tokens", 3) == "<tok_3>"
+    assert g.has_tensor("token_embd.weight") and g.has_tensor("output.weight") and not g.has_tensor("nope")
+    t = g.tensor("token_embd.weight")
+    assert t["shape"] == [11, 8] and t["type"] == cai.F32          # ggml stores [8, 11]; served row-major
+    assert g.tensor("blk.0.attn_k.weight")["shape"] == [4, 8]
+    assert g.tensor("output_norm.weight")["shape"] == [8]
+    with pytest.raises(cai.CaiError):
+        g.tensor("nope")
+    with pytest.raises(cai.CaiError):
+        g.meta_array_str("tokenizer.ggml.tokens", 11)
+
+
+@pytest.mark.parametrize("name", ["tiny_llama_f32.gguf", "tiny_llama_f16.gguf", "tiny_llama_q8.gguf", "tiny_kquant.gguf"])
+def test_every_tensor_matches_the_python_reader_byte_for_byte(name):
+    g = cai.GGUF(ref_path(name)); py = GGUFFile(ref_path(name))
+    assert g.info()["n_tensors"] == len(py.tensors) and g.info()["data_start"] == py.data_start
+    for i, (tname, t) in enumerate(py.tensors.items()):
+        got = g.tensor(i)
+        assert got["name"] == tname and got["type"] == t["type"] and got["shape"] == t["shape"] and got["offset"] == t["offset"]
+        _, _, raw = py.raw(tname)
+        assert np.array_equal(g.tensor_bytes(tname), raw)
+
+
+def test_kquant_fixture_layout_facts():
+    g = cai.GGUF(ref_path("tiny_kquant.gguf"))
+    assert g.info()["version"] == 3 and g.info()["n_tensors"] == 5
+    want = {"kq.Q4_K.weight": (12, 4096, 576), "kq.Q5_K.weight": (13, 4672, 704), "kq.Q6_K.weight": (14, 5376, 840), "kq.Q2_K.weight": (10, 6240, 336)}
+    for n, (ty, off, nb) in want.items():
+        t = g.tensor(n)
+        assert (t["type"], t["offset"], t["nbytes"], t["shape"]) == (ty, off, nb, [1024])   # offsets are relative to the data section
+
+
+def _gguf(version=3, meta=(), tensors=(), magic=b"GGUF", pad_to=None, data=b""):
+    def s(x):
+        return struct.pack("<Q", len(x)) + x
+    b = magic + struct.pack("<IQQ", version, len(tensors), len(meta))
+    for k, vt, payload in meta:
+        b += s(k) + struct.pack("<I", vt) + payload
+    for name, dims, ty, off in tensors:
+        b += s(name) + struct.pack("<I", len(dims)) + b"".join(struct.pack("<Q", d) for d in dims) + struct.pack("<IQ", ty, off)
+    if pad_to:
+        b += b"\0" * (-len(b) % pad_to)
+    return b + data
+
+
+CASES = {
+    "too small": (b"GGUF\3\0\0\0", "too small"),
+    "bad magic": (_gguf(magic=b"GGML"), "bad magic"),
+    "version 1": (_gguf(version=1), "unsupported version 1"),
+    "implausible counts": (b"GGUF" + struct.pack("<IQQ", 3, 1 << 40, 0), "implausible header counts"),
+    "empty key": (_gguf(meta=[(b"", 4, struct.pack("<I", 1))]), "empty metadata key"),
+    "duplicate key": (_gguf(meta=[(b"a", 4, struct.pack("<I", 1)), (b"a", 4, struct.pack("<I", 2))]), "duplicate metadata key"),
+    "truncated value": (_gguf(meta=[(b"a", 10, b"\1\2")]), "truncated"),
+    "unknown value type": (_gguf(meta=[(b"a", 99, b"")]), "bad or truncated value"),
+    "zero dims": (_gguf(tensors=[(b"t", [], 0, 0)]), "implausible n_dims 0"),
+    "zero dimension": (_gguf(tensors=[(b"t", [0], 0, 0)]), "implausible dimension"),
+    "duplicate tensor": (_gguf(tensors=[(b"t", [4], 0, 0), (b"t", [4], 0, 0)], pad_to=32, data=b"\0" * 64), "duplicate tensor name"),
+    "q8_0 not block multiple": (_gguf(tensors=[(b"t", [33, 2], 8, 0)], pad_to=32, data=b"\0" * 128), "not a multiple of the block size 32"),
+    "q4_k not block multiple": (_gguf(tensors=[(b"t", [128, 2], 12, 0)], pad_to=32, data=b"\0" * 512), "not a multiple of the block size 256"),
+    "bad alignment": (_gguf(meta=[(b"general.alignment", 4, struct.pack("<I", 24))]), "not a positive power of two"),
+    "tensor outside data": (_gguf(tensors=[(b"t", [64], 0, 0)], pad_to=32, data=b"\0" * 64), "falls outside the data section"),
+}
+
+
+@pytest.mark.parametrize("case", list(CASES))
+def test_malformed_files_are_refused_with_the_reference_reason(case, tmp_path):
+    blob, needle = CASES[case]
+    p = tmp_path / "bad.gguf"
+    p.write_bytes(blob)
+    with pytest.raises(cai.CaiError) as e:
+        cai.GGUF(str(p))
+    assert needle in str(e.value)
+
+
+def test_minimal_valid_file_and_missing_file(tmp_path):
+    p = tmp_path / "ok.gguf"
+    p.write_bytes(_gguf(meta=[(b"general.alignment", 4, struct.pack("<I", 64)), (b"x.flag", 7, b"\1"), (b"x.neg", 5, struct.pack("<i", -7)),
+                              (b"x.arr", 9, struct.pack("<IQ", 5, 3) + struct.pack("<3i", 1, 2, 3))],
+                        tensors=[(b"t", [4, 2], 0, 0)], pad_to=64, data=np.arange(8, dtype=np.float32).tobytes()))
+    g = cai.GGUF(str(p))
+    assert g.info()["alignment"] == 64 and g.info()["data_start"] % 64 == 0
+    assert g.meta_int("x.flag") == 1 and g.meta_int("x.neg") == -7 and g.meta_array_count("x.arr") == 3
+    assert g.tensor("t")["shape"] == [2, 4]
+    assert np.array_equal(g.tensor_bytes("t").view(np.float32), np.arange(8, dtype=np.float32))
+    with pytest.raises(cai.CaiError):
+        cai.GGUF(str(tmp_path / "absent.gguf"))
