@@ -1,0 +1,143 @@
+// C++ host-side mirror of the two reference objects that sit on the decode path, written over the C ABI of
+// include/caihip.h (this is the executable twin of the Free Pascal adapter described for maintainers; the
+// reference's own host language has no compiler in this build image):
+//
+//   TDotProductSharedKernel  (neural/neuralopencl.pas:245-388, 844-1104): per-layer offload object.
+//       PrepareForComputeInt8 -> blocking one-time upload of the weights; ComputeInt8 -> enqueue one product;
+//       FinishAndLoadResult -> block and write NumAs*NumBs floats laid out [b*NumAs + a].
+//       Errors are reported through ErrorProc and the call returns a code; nothing is thrown (957-969).
+//   TNNetStreamingDecoder    (neural/neuraldecode.pas:1210-1333, 5696-5843): session over a whole decoder.
+//       Reset, StepForward(window, AbsPos), TruncateTo, Snapshot / RestoreSnapshot, SDPACacheLength, Output.
+//       Importer-level failures raise (EPretrainedImportError / EGGUFError in the reference): here CaiError.
+#pragma once
+#include <caihip.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <functional>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace caihip {
+
+inline std::string LastError()
+{
+  char buf[1024];
+  cai_last_error(buf, (int)sizeof buf);
+  return std::string(buf);
+}
+
+struct CaiError : std::runtime_error {
+  int code;
+  CaiError(int c, const std::string& m) : std::runtime_error(m), code(c) {}
+};
+inline void Check(int rc) { if (rc != CAI_OK) throw CaiError(rc, LastError()); }
+
+// EnableOpenCL analogue (neural/neuralchatengine.pas:1156-1157): arm the device once per process.
+inline void EnableHIP(int device = 0) { Check(cai_init(device)); }
+
+class TDotProductSharedKernel {
+ public:
+  std::function<void(const std::string&)> ErrorProc = [](const std::string& m) { std::fprintf(stderr, "%s\n", m.c_str()); };
+
+  ~TDotProductSharedKernel() { UnprepareForCompute(); }
+
+  // per-row symmetric int8 codes + fp32 row scales (the reference's own resident format)
+  int PrepareForComputeInt8(const int8_t* pCodes, const float* pScales, int NumAs, int pSize, const float* pBias = nullptr)
+  {
+    UnprepareForCompute();
+    return Report(cai_qw_create_int8row(NumAs, pSize, pCodes, pScales, pBias, &w_), NumAs, pSize);
+  }
+  // GGUF blocks in stored order (CAI_Q8_0 / CAI_Q4_0 / CAI_Q4_K / CAI_F16 / CAI_F32): no dequantised copy is ever made
+  int PrepareForComputeBlocks(int qtype, const void* pBlocks, int NumAs, int pSize, const float* pBias = nullptr)
+  {
+    UnprepareForCompute();
+    return Report(cai_qw_create(qtype, NumAs, pSize, pBlocks, pBias, &w_), NumAs, pSize);
+  }
+  bool Int8Ready() const { return w_ != nullptr; }
+
+  // VBs: NumBs input vectors of pSize floats.  ActFN: 0 none, 1 ReLU, 2 sigmoid, 3 tanh (neural/neural.cl:114-146);
+  // bias is added before the activation.
+  int ComputeInt8(const float* VBs, int NumBs, int ActFN = 0)
+  {
+    if (!w_) return Fail(CAI_ERR_STATE, "ComputeInt8 before PrepareForComputeInt8");
+    result_.assign((size_t)NumBs * (size_t)num_as_, 0.0f);
+    const int rc = cai_qgemv(w_, VBs, NumBs, result_.data(), ActFN, 0);
+    if (rc) return Fail(rc, LastError());
+    pending_ = true;
+    return CAI_OK;
+  }
+  int FinishAndLoadResult(float* Results)
+  {
+    if (!pending_) return Fail(CAI_ERR_STATE, "FinishAndLoadResult without a ComputeInt8 in flight");
+    for (size_t i = 0; i < result_.size(); i++) Results[i] = result_[i];
+    pending_ = false;
+    return CAI_OK;
+  }
+  void UnprepareForCompute() { if (w_) { cai_qw_destroy(w_); w_ = nullptr; } pending_ = false; }
+
+ private:
+  int Report(int rc, int NumAs, int pSize) { if (rc) return Fail(rc, LastError()); num_as_ = NumAs; size_ = pSize; return CAI_OK; }
+  int Fail(int rc, const std::string& m) { if (ErrorProc) ErrorProc(m); return rc; }
+  cai_qw_t w_ = nullptr;
+  int num_as_ = 0, size_ = 0;
+  bool pending_ = false;
+  std::vector<float> result_;
+};
+
+class TNNetDecoderSessionSnapshot {
+ public:
+  explicit TNNetDecoderSessionSnapshot(cai_kv_snap_t s) : s_(s) {}
+  ~TNNetDecoderSessionSnapshot() { if (s_) cai_kv_snap_destroy(s_); }
+  TNNetDecoderSessionSnapshot(const TNNetDecoderSessionSnapshot&) = delete;
+  TNNetDecoderSessionSnapshot& operator=(const TNNetDecoderSessionSnapshot&) = delete;
+  cai_kv_snap_t handle() const { return s_; }
+ private:
+  cai_kv_snap_t s_;
+};
+
+class TNNetStreamingDecoder {
+ public:
+  // BuildLlamaFromGGUF + TNNetStreamingDecoder.Create(pNet, pMaxCacheLen): pMaxCacheLen <= 0 takes the file's context length
+  TNNetStreamingDecoder(const std::string& GGUFFileName, int pMaxCacheLen = 0, bool pF16KV = false)
+  {
+    Check(cai_decoder_load_gguf(GGUFFileName.c_str(), pMaxCacheLen, 1, pF16KV ? CAI_KV_F16 : CAI_KV_F32, &d_));
+    Check(cai_decoder_get_config(d_, &cfg_));
+    logits_.resize((size_t)cfg_.vocab);
+  }
+  ~TNNetStreamingDecoder() { if (d_) cai_decoder_destroy(d_); }
+  TNNetStreamingDecoder(const TNNetStreamingDecoder&) = delete;
+  TNNetStreamingDecoder& operator=(const TNNetStreamingDecoder&) = delete;
+
+  const cai_decoder_config& Config() const { return cfg_; }
+  void Reset() { Check(cai_decoder_reset(d_, 0)); }
+  // One streamed forward of a window of token ids; AbsPos is the absolute position of the FIRST token of the window.
+  // After it, Output() holds the logits of the window's last token and ArgMaxRow() their arg-max (lowest index on ties).
+  void StepForward(const int32_t* Tokens, int Count, int AbsPos)
+  {
+    if (Count == 1) { int32_t p = AbsPos; Check(cai_decoder_step(d_, Tokens, &p, 1, logits_.data(), &argmax_)); }
+    else Check(cai_decoder_prefill(d_, 0, Tokens, Count, AbsPos, logits_.data(), &argmax_));
+  }
+  void TruncateTo(int CommittedLen) { Check(cai_decoder_truncate(d_, 0, CommittedLen)); }
+  int SDPACacheLength(int /*Index*/ = 0) const { int n = 0; Check(cai_decoder_len(d_, 0, &n)); return n; }
+  TNNetDecoderSessionSnapshot* Snapshot() { cai_kv_snap_t s = nullptr; Check(cai_decoder_snapshot(d_, 0, &s)); return new TNNetDecoderSessionSnapshot(s); }
+  void RestoreSnapshot(const TNNetDecoderSessionSnapshot* Snap) { Check(cai_decoder_restore(d_, 0, Snap->handle())); }
+  const std::vector<float>& Output() const { return logits_; }
+  int ArgMaxRow() const { return argmax_; }
+  // Greedy fast path of the chat engine (neural/neuralchatengine.pas:1493-1494): n tokens chained on the device.
+  std::vector<int32_t> GenerateGreedy(int32_t FirstToken, int AbsPos, int n)
+  {
+    std::vector<int32_t> out((size_t)n);
+    Check(cai_decoder_generate(d_, FirstToken, AbsPos, n, out.data()));
+    return out;
+  }
+
+ private:
+  cai_decoder_t d_ = nullptr;
+  cai_decoder_config cfg_{};
+  std::vector<float> logits_;
+  int32_t argmax_ = -1;
+};
+
+}  // namespace caihip
