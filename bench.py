@@ -72,6 +72,62 @@ def cpu_baseline(cfg, seconds_budget=20.0):
                       "median of %d runs, extrapolated to a full token; attention/norms excluded" % (cfg["n_layers"], reps)}
 
 
+def gemv_sweep(cai, synth, torch, with_cpu):
+    """One JSON line per (type, shape, batch): resident blocks, x and y on the device, HIP-event time per launch while
+    rotating over enough copies of the matrix to exceed the 256 MB infinity cache (at most 24 copies: the small shapes stay
+    cache-resident and are labelled so)."""
+    lib = cai.load()
+    QT = {"Q8_0": (cai.Q8_0, 34 / 32), "Q4_0": (cai.Q4_0, 18 / 32), "Q4_K": (cai.Q4_K, 144 / 256)}
+    shapes = [(2048, 2048), (5632, 2048), (2048, 5632), (18944, 3584), (152064, 3584)]
+    gen = torch.Generator(device="cuda"); gen.manual_seed(424242)
+    cpu = None
+    if with_cpu:
+        import numpy as np
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        from helpers import oracle_lib as O
+        cpu = O.lib()
+    for name, (qt, bpw) in QT.items():
+        for rows, cols in shapes:
+            mat_bytes = rows * cols * bpw
+            copies = int(max(1, min(24, -(-320e6 // mat_bytes))))
+            ws = [synth.random_qweight(qt, rows, cols, gen)[0] for _ in range(copies)]
+            for nb in (1, 4):
+                x = torch.randn(nb, cols, device="cuda"); y = torch.empty(nb, rows, device="cuda")
+                torch.cuda.synchronize()
+                for w in ws:
+                    cai.check(lib.cai_qgemv(w.h, x.data_ptr(), nb, y.data_ptr(), 0, cai.X_DEVICE | cai.Y_DEVICE))
+                reps = max(2, int(200 // copies))
+                cai.check(lib.cai_sync()); cai.check(lib.cai_timer_start())
+                for _ in range(reps):
+                    for w in ws:
+                        cai.check(lib.cai_qgemv(w.h, x.data_ptr(), nb, y.data_ptr(), 0, cai.X_DEVICE | cai.Y_DEVICE))
+                ms = C.c_float(); cai.check(lib.cai_timer_stop(C.byref(ms)))
+                us = ms.value * 1e3 / (reps * copies)
+                algo = mat_bytes + 4 * cols * nb + 4 * rows * nb
+                line = {"gemv": name, "rows": rows, "cols": cols, "batch": nb, "us_per_launch": round(us, 2),
+                        "algorithmic_bytes": int(algo), "GB_per_s": round(algo / us / 1e3, 1), "frac_of_8TBps": round(algo / us / 1e3 / HBM_PEAK_GBS, 4),
+                        "working_set": "hbm" if copies * mat_bytes > 300e6 else "cache-resident (%d x %.1f MB)" % (copies, mat_bytes / 1e6)}
+                if cpu is not None and nb == 1 and name == "Q8_0":
+                    # restated reference AVX2 int8-per-row kernel on the same shape (1 B/weight), all host threads
+                    import numpy as np
+                    thr = min(cpu.cpu_max_threads(), 16)
+                    rng = np.random.default_rng(0)
+                    codes = rng.integers(-127, 128, (rows, cols), dtype=np.int8); sc = np.full(rows, 1e-3, np.float32)
+                    xv = rng.standard_normal(cols).astype(np.float32); yv = np.empty(rows, np.float32)
+                    ts = []
+                    for _ in range(5):
+                        t0 = time.perf_counter()
+                        cpu.cpu_linear_int8(codes.ctypes.data, sc.ctypes.data, rows, cols, xv.ctypes.data, 1, None, yv.ctypes.data, thr)
+                        ts.append(time.perf_counter() - t0)
+                    t = sorted(ts)[2]
+                    line["cpu_int8row_port"] = {"us": round(t * 1e6, 1), "GB_per_s": round(rows * cols / t / 1e9, 2), "cores": thr}
+                print(json.dumps(line), flush=True)
+            for w in ws:
+                w.close()
+            del ws
+            torch.cuda.empty_cache()
+
+
 # HBM bytes per launch of the 7B-shape gate|up kernel from hardware counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000
 # KiB, factors from a 1 GiB copy kernel): profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt.  Not measurable from
 # inside this process; re-collect when the kernel changes.
@@ -87,6 +143,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernel-reps", type=int, default=5)
     ap.add_argument("--batch", type=int, default=1, help="independent sequences decoded together (1..8)")
+    ap.add_argument("--gemv-sweep", action="store_true", help="isolated matrix-vector sweep (BASELINE configs[1]): Q8_0 / Q4_0 / Q4_K, five shapes, batch 1 and 4")
     ap.add_argument("--copy-calibration", action="store_true", help="only run the 1 GiB device copy kernel 5 times (reference for traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -108,6 +165,9 @@ def main():
             cai.check(cai.load().cai_dev_copy(b.data_ptr(), a.data_ptr(), a.numel() * 4))
         cai.check(cai.load().cai_sync())
         print(json.dumps({"copy_calibration": {"bytes_read": a.numel() * 4, "bytes_written": a.numel() * 4, "launches": 5}}))
+        return
+    if args.gemv_sweep:
+        gemv_sweep(cai, synth, torch, not args.no_cpu_baseline)
         return
     conf = CONFIGS[args.config]
     cfg = dict(conf["cfg"])

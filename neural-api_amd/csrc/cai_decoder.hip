@@ -32,6 +32,7 @@ struct cai_decoder_s {
   int32_t* h_io = nullptr;   // pinned: tokens[8] pos[8] argmax[8]
   hipGraphExec_t graph[9] = {nullptr};
   bool use_graph = true;
+  int ws_generation = -1;         // activation-workspace generation the captured batch graphs were built against
   std::vector<cai_qw_s*> owned;   // weights created by a loader on the decoder's behalf, destroyed with it
   int qw() const { return cfg.n_q_heads * cfg.head_dim; }
   int kw() const { return cfg.n_kv_heads * cfg.head_dim; }
@@ -80,8 +81,38 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
   float* ssq_o = d->ssq;          // written by the o-projection, read by gate|up
   float* ssq_d = d->ssq + 1024;   // written by the down projection, read by the next block's q|k|v
   bool have_ssq_d = false;
+  bool down_pending = false;      // small-batch path: the last down product has not been added to x yet
+  // 2..8 sequences on Q4_K weights: every linear layer goes to the matrix cores (weights streamed once for the batch)
+  auto mma_layer = [&](const cai_decoder_s::Layer& L) {
+    if (n_b < 2 || c.n_experts > 0) return false;
+    const int slots[6] = {CAI_W_Q, CAI_W_K, CAI_W_V, CAI_W_O, CAI_W_GATEUP, CAI_W_DOWN};
+    for (int sl : slots) if (!gemm_mfma_supported(L.w[sl])) return false;
+    return true;
+  };
   for (int l = 0; l < c.n_layers; l++) {
     auto& L = d->layers[l];
+    if (mma_layer(L)) {
+      // the down product of the previous block is still in slices: the pre-pass adds it to the residual stream
+      if (down_pending) rc = nb_prep_residual(d->x, dm, L.v[CAI_V_ATTN_NORM], c.eps, dm, n_b);
+      else rc = nb_prep_plain(d->x, dm, L.v[CAI_V_ATTN_NORM], c.eps, dm, n_b);
+      if (rc) return rc;
+      down_pending = false;
+      {
+        const cai_qw_s* qkv3[3] = {L.w[CAI_W_Q], L.w[CAI_W_K], L.w[CAI_W_V]}; const int off3[3] = {0, qw, qw + kw};
+        if ((rc = nb_gemm(qkv3, off3, 3, n_b)) || (rc = nb_reduce(d->qkv, qkvw, nullptr))) return rc;
+      }
+      if (c.qk_norm_full) launch_rmsnorm_pair(d->qkv, L.v[CAI_V_Q_NORM], qw, L.v[CAI_V_K_NORM], kw, n_b, c.eps, qkvw);
+      if ((rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0))) return rc;
+      const int zero = 0;
+      const cai_qw_s* wo = L.w[CAI_W_O]; const cai_qw_s* wgu = L.w[CAI_W_GATEUP]; const cai_qw_s* wdn = L.w[CAI_W_DOWN];
+      if ((rc = nb_prep_plain(d->att, qw, nullptr, 0.0f, qw, n_b)) || (rc = nb_gemm(&wo, &zero, 1, n_b))) return rc;
+      if ((rc = nb_prep_residual(d->x, dm, L.v[CAI_V_MLP_NORM], c.eps, dm, n_b)) || (rc = nb_gemm(&wgu, &zero, 1, n_b))) return rc;
+      if ((rc = nb_prep_swiglu(I, n_b)) || (rc = nb_gemm(&wdn, &zero, 1, n_b))) return rc;
+      down_pending = true;
+      have_ssq_d = false;
+      continue;
+    }
+    if (down_pending) { if ((rc = nb_prep_residual(d->x, dm, nullptr, 0.0f, dm, n_b))) return rc; down_pending = false; }
     // --- attention half ---
     {
       MultiGemv m{}; m.n = 3;
@@ -154,6 +185,15 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
   }
   {
     cai_qw_s* hw = d->head ? d->head : d->embed;   // tied head (neural/neuralpretrained.pas:15555-)
+    if (n_b >= 2 && gemm_mfma_supported(hw)) {
+      const int zero = 0; const cai_qw_s* hwc = hw;
+      if (down_pending) rc = nb_prep_residual(d->x, dm, d->final_norm, c.eps, dm, n_b);
+      else rc = nb_prep_plain(d->x, dm, d->final_norm, c.eps, dm, n_b);
+      if (rc || (rc = nb_gemm(&hwc, &zero, 1, n_b)) || (rc = nb_reduce(d->logits, c.vocab, nullptr))) return rc;
+      launch_argmax(d->logits, c.vocab, n_b, d->d_argmax, d->am_v, d->am_i);
+      return CAI_OK;
+    }
+    if (down_pending) { if ((rc = nb_prep_residual(d->x, dm, nullptr, 0.0f, dm, n_b))) return rc; down_pending = false; }
     MultiGemv m{}; m.n = 1; m.w[0] = hw; m.rows[0] = c.vocab;
     if (have_ssq_d && gemv_hands_off_ssq(hw, n_b)) m.ssq_in = ssq_d;
     if ((rc = launch_gemv_multi(m, d->x, n_b, d->logits, c.vocab, CAI_ACT_NONE, nullptr, d->final_norm, c.eps, 0))) return rc;
@@ -190,6 +230,7 @@ static int ensure_prefill_buffers(cai_decoder_s* d, int n)
 static int linear_rows(const cai_qw_s* w, bool prepped, const float* x, int64_t x_stride, const float* gain, float eps, int n,
                        float* y, int64_t y_stride, const float* residual)
 {
+  if (gemm_mfma_supported(w) && n <= 16) return nb_linear(w, x, x_stride, gain, eps, n, y, y_stride, residual);   // bandwidth-bound regime
   if (gemm_mfma_supported(w)) {
     int rc;
     if (!prepped && (rc = prefill_prep(x, x_stride, gain, eps, (int)w->cols, n))) return rc;
@@ -209,7 +250,7 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
     auto& L = d->layers[l];
     const cai_qw_s* wq = L.w[CAI_W_Q]; const cai_qw_s* wk = L.w[CAI_W_K]; const cai_qw_s* wv = L.w[CAI_W_V];
     const bool all_mfma = gemm_mfma_supported(wq) && gemm_mfma_supported(wk) && gemm_mfma_supported(wv);
-    if (all_mfma && (rc = prefill_prep(d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, dm, n))) return rc;
+    if (all_mfma && n > 16 && (rc = prefill_prep(d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, dm, n))) return rc;
     if ((rc = linear_rows(wq, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv, qkvw, nullptr))) return rc;
     if ((rc = linear_rows(wk, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw, qkvw, nullptr))) return rc;
     if ((rc = linear_rows(wv, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw + kw, qkvw, nullptr))) return rc;
@@ -228,6 +269,17 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
 static int run_step(cai_decoder_s* d, int n_b)
 {
   Context& c = ctx();
+  if (n_b >= 2) {   // the matrix-core path's activation workspace cannot grow inside a stream capture
+    const cai_decoder_config& cf = d->cfg;
+    const int dm = cf.d_model, qkvw = d->qw() + 2 * d->kw();
+    const int kmax = std::max(std::max(dm, d->qw()), cf.ffn);
+    auto al4 = [](int64_t v) { return (size_t)((v + 3) / 4 * 4); };
+    size_t part = std::max(std::max((size_t)nb_max_slices(dm) * al4(qkvw), (size_t)nb_max_slices(d->qw()) * al4(dm)),
+                           std::max((size_t)nb_max_slices(dm) * al4(2 * (int64_t)cf.ffn), (size_t)nb_max_slices(cf.ffn) * al4(dm)));
+    part = std::max(part, (size_t)nb_max_slices(dm) * al4(cf.vocab)) * 8;
+    const int rc = nb_reserve(kmax, part); if (rc) return rc;
+    if (d->ws_generation != nb_ws_generation()) { invalidate_graphs(d); d->ws_generation = nb_ws_generation(); }
+  }
   if (!d->use_graph) { const int rc = enqueue_step(d, n_b, 0); if (rc) return rc; CAI_HIP(hipGetLastError()); return CAI_OK; }
   if (!d->graph[n_b]) {
     hipGraph_t g = nullptr;

@@ -1,0 +1,487 @@
+// Small-batch (2..8 tokens per pass) Q4_K linear layer on the matrix cores of gfx950: the decode step of a few sequences.
+//
+// At batch 1 the layer is a matrix-vector product and the VALU keeps up with HBM; at batch b the same weights serve
+// b activations, so the contraction goes to v_mfma_f32_32x32x8_f16 while the weights are still streamed once.
+//   * A operand = sc_j * q, an integer <= 63 * 15 and therefore EXACT in f16: the 6-bit sub-block scale is folded into
+//     the nibble with one packed fma ((1024 + q) * sc - 1024 * sc, every term exact), so the matrix cores accumulate
+//     across a whole 256-weight super-block and the float scale d is applied once per super-block, not per 32 weights;
+//   * B operand = the activations of up to 8 tokens, scaled per (token, 256-block) by a power of two and split hi + lo
+//     into two f16 (22 significant bits): 8 hi + 8 lo columns of the MFMA tile (the other 16 stay zero);
+//   * the -dmin * mn_j * sum_{k in j} x_k term is one more MFMA step per super-block (k = the 8 sub-blocks).
+//   Y[t][r] = sum_sb sinv[t][sb] * ( d * P_main - 32 dmin * P_min )   (Q4_K: neural/neuralgguf.pas:472-514)
+//
+// Work layout: grid = (row groups, K slices).  A work-group stages ITS slice of the activations (up to 4 super-blocks)
+// in LDS once, then its 4 waves walk 32-row tiles independently - no barrier after the staging, weights of the next
+// two (tile, super-block) items always in flight.  Each slice writes a partial result; the consumer (next activation
+// pre-pass, SwiGLU, or a plain reduction) adds the slices in a fixed order.  Token RMSNorm factors out of the product:
+// the pre-pass stores g*x and per-block sums of squares, the consumer multiplies by 1/rms (neural/neural.cl:1047-1085).
+#include "cai_internal.hpp"
+#include "cai_gemv_common.hpp"
+#include <algorithm>
+
+namespace cai {
+
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+constexpr int NB_LDX = 260;      // halfs per staged activation column: 256 + pad (stride = 2 banks mod 64)
+constexpr int NB_SC = 16;        // staged columns: 8 tokens x {hi, lo}
+constexpr int NB_TK = 8;         // tokens per pass
+constexpr int NB_SMAX = 4;       // super-blocks per K slice (LDS: 4 x 8.6 KB, so three work-groups share a CU)
+
+struct NbSeg { const uint8_t* w; const float* bias; int rows; int y_off; int tile_end; };   // tile_end: cumulative 32-row tiles
+
+struct NbParams {
+  NbSeg seg[3]; int n_seg;                      // up to three matrices of equal width share one launch (q | k | v)
+  int n_tiles;
+  int cols;
+  const _Float16* xhi; const _Float16* xlo;     // [token][cols]
+  const _Float16* sxhi; const _Float16* sxlo;   // [token][cols/32]: (sum of the 32-block) * s / 32, split hi + lo
+  const float* sinvb;                           // [token][cols/256] 1 / s of the (token, 256-block)
+  int n_tok;
+  float* part; int64_t part_stride;             // part[(slice*n_tok + t)*part_stride + y_off + row]
+  int sb_per_slice;
+  int tile_stride;                              // tiles between two tiles of the same wave (= 4 * gridDim.x)
+};
+
+__device__ __forceinline__ half4_t bytes_to_half4(uint32_t t)
+{
+  // four bytes (0..255) -> four exact halfs 1024 + b (the byte becomes the low mantissa bits of 0x6400 = 1024.0)
+  const uint32_t p01 = __builtin_amdgcn_perm(0x64646464u, t, 0x04010400u);
+  const uint32_t p23 = __builtin_amdgcn_perm(0x64646464u, t, 0x04030402u);
+  const half2_t a = __builtin_bit_cast(half2_t, p01), b = __builtin_bit_cast(half2_t, p23);
+  return half4_t{a.x, a.y, b.x, b.y};
+}
+
+__global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
+{
+  extern __shared__ __align__(16) unsigned char nb_smem[];
+  const int S = p.sb_per_slice;
+  _Float16* xs = reinterpret_cast<_Float16*>(nb_smem);              // [S][16][NB_LDX]
+  _Float16* sxs = xs + S * NB_SC * NB_LDX;                           // [S][16][8]
+  float* sinv_s = reinterpret_cast<float*>(sxs + S * NB_SC * 8);     // [S][8]
+  float* s_d = sinv_s + S * NB_TK;                                   // [4 waves][2][32]: d, 32*dmin per row
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = lane & 31, kg = lane >> 5;
+  const int K = p.cols, nsb = K >> 8, nb32 = K >> 5;
+  const int slice = blockIdx.y, sb0 = slice * S, nS = min(S, nsb - sb0);
+  const int64_t row_bytes = (int64_t)nsb * 144;
+  const int tile0 = blockIdx.x * 4 + wave;
+  const int n_it = tile0 < p.n_tiles ? (p.n_tiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
+  const int nq = n_it * nS;                      // (tile, super-block) items of this wave
+
+  struct WRegs { uint4 h, q[4]; };
+  auto locate = [&](int tile, const NbSeg*& sg, int& R0) {
+    int sgi = 0, t0 = 0;
+    if (p.n_seg > 1 && tile >= p.seg[0].tile_end) { sgi = 1; t0 = p.seg[0].tile_end; }
+    if (p.n_seg > 2 && tile >= p.seg[1].tile_end) { sgi = 2; t0 = p.seg[1].tile_end; }
+    sg = &p.seg[sgi]; R0 = (tile - t0) * 32;
+  };
+  // weights of item q: header + this lane's 64 quant bytes (chunks 2kg, 2kg+1) of row R0 + n
+  auto load_w = [&](int q, WRegs& r) {
+    if (q < nq) {
+      const int tile = tile0 + (q / nS) * p.tile_stride, sb = sb0 + q % nS;
+      const NbSeg* sg; int R0; locate(tile, sg, R0);
+      const uint8_t* blk = sg->w + (int64_t)min(R0 + n, sg->rows - 1) * row_bytes + (int64_t)sb * 144;   // tail rows: re-read the last row
+      r.h = *reinterpret_cast<const uint4*>(blk);
+#pragma unroll
+      for (int i = 0; i < 4; i++) r.q[i] = *reinterpret_cast<const uint4*>(blk + 16 + 64 * kg + 16 * i);
+    }
+  };
+  WRegs wa, wb, wc;
+  load_w(0, wa); load_w(1, wb);                  // weights do not depend on the staging below
+
+  // ---- stage this slice of the activations: nS x 16 columns x 256 halfs, block sums, block scales ----
+  for (int idx = threadIdx.x; idx < nS * NB_SC * 32; idx += 256) {
+    const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC;
+    const int tok = col % NB_TK;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (tok < p.n_tok) v = *reinterpret_cast<const uint4*>(((col / NB_TK) ? p.xlo : p.xhi) + (int64_t)tok * K + (sb0 + s) * 256 + chunk * 8);
+    uint2* dst = reinterpret_cast<uint2*>(xs + (s * NB_SC + col) * NB_LDX + chunk * 8);   // columns are 8-byte aligned
+    dst[0] = make_uint2(v.x, v.y); dst[1] = make_uint2(v.z, v.w);
+  }
+  for (int idx = threadIdx.x; idx < nS * NB_SC; idx += 256) {
+    const int col = idx % NB_SC, s = idx / NB_SC, tok = col % NB_TK;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (tok < p.n_tok) v = *reinterpret_cast<const uint4*>(((col / NB_TK) ? p.sxlo : p.sxhi) + (int64_t)tok * nb32 + (sb0 + s) * 8);
+    *reinterpret_cast<uint4*>(sxs + idx * 8) = v;
+    if (col < NB_TK) sinv_s[s * NB_TK + tok] = tok < p.n_tok ? p.sinvb[(int64_t)tok * nsb + sb0 + s] : 0.0f;
+  }
+  __syncthreads();
+
+  float16_t acc;
+#pragma unroll
+  for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+  const bool col_on = n < NB_SC;                 // MFMA columns 16..31 multiply zeros
+  const half4_t zero4 = {(_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f};
+
+  auto compute = [&](const WRegs& r, int q) {
+    const int s = q % nS;
+    if (s == 0) {
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+    }
+    // 6-bit scales / mins of this lane's four sub-blocks 4kg .. 4kg+3 (neural/neuralgguf.pas:448-464), one per byte
+    const uint32_t sc4 = kg == 0 ? (r.h.y & 0x3f3f3f3fu) : ((r.h.w & 0x0f0f0f0fu) | ((r.h.y >> 2) & 0x30303030u));
+    const uint32_t mn4 = kg == 0 ? (r.h.z & 0x3f3f3f3fu) : (((r.h.w >> 4) & 0x0f0f0f0fu) | ((r.h.z >> 2) & 0x30303030u));
+    const _Float16 k1024 = (_Float16)1024.0f;
+    const half4_t sch = bytes_to_half4(sc4), mnh = bytes_to_half4(mn4);
+    const half4_t scv = half4_t{sch.x - k1024, sch.y - k1024, sch.z - k1024, sch.w - k1024};   // sc as halfs
+    const half4_t mnv = half4_t{mnh.x - k1024, mnh.y - k1024, mnh.z - k1024, mnh.w - k1024};
+    if (kg == 0) {
+      const float d = __half2float(__ushort_as_half((unsigned short)(r.h.x & 0xffffu)));
+      const float dmin = __half2float(__ushort_as_half((unsigned short)(r.h.x >> 16)));
+      s_d[(wave * 2 + 0) * 32 + n] = d; s_d[(wave * 2 + 1) * 32 + n] = dmin * 32.0f;
+    }
+    // two accumulators: consecutive MFMAs do not wait for each other
+    float16_t C0, C1, Cm;
+#pragma unroll
+    for (int v = 0; v < 16; v++) { C0[v] = 0.0f; C1[v] = 0.0f; Cm[v] = 0.0f; }
+    const _Float16* xcol = xs + (s * NB_SC + (col_on ? n : 0)) * NB_LDX + 128 * kg;
+#pragma unroll
+    for (int ccl = 0; ccl < 2; ccl++) {
+#pragma unroll
+      for (int hl = 0; hl < 2; hl++) {
+        const int j = 2 * ccl + hl;                                   // sub-block 4kg + j of the super-block
+        const _Float16 sj = j == 0 ? scv.x : (j == 1 ? scv.y : (j == 2 ? scv.z : scv.w));
+        const half2_t s2 = {sj, sj};
+        const half2_t c2 = {(_Float16)(-1024.0f) * sj, (_Float16)(-1024.0f) * sj};   // exact: a multiple of 1024 below 65504
+        const _Float16* xb = xcol + 32 * j;
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          const uint4& qq = r.q[2 * ccl + (t >> 2)];
+          const uint32_t qd = (t & 3) == 0 ? qq.x : ((t & 3) == 1 ? qq.y : ((t & 3) == 2 ? qq.z : qq.w));
+          const uint32_t nib = hl ? ((qd >> 4) & 0x0f0f0f0fu) : (qd & 0x0f0f0f0fu);
+          const uint32_t p01 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04010400u);
+          const uint32_t p23 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04030402u);
+          const half2_t a01 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, p01), s2, c2);   // (1024 + q) * sc - 1024 * sc = sc * q
+          const half2_t a23 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, p23), s2, c2);
+          const half4_t A = {a01.x, a01.y, a23.x, a23.y};
+          half4_t B = *reinterpret_cast<const half4_t*>(xb + 4 * t);
+          if (!col_on) B = zero4;
+          if (t & 1) C1 = __builtin_amdgcn_mfma_f32_32x32x8f16(A, B, C1, 0, 0, 0);
+          else C0 = __builtin_amdgcn_mfma_f32_32x32x8f16(A, B, C0, 0, 0, 0);
+        }
+      }
+    }
+    {
+      half4_t Bm = *reinterpret_cast<const half4_t*>(sxs + (s * NB_SC + (col_on ? n : 0)) * 8 + 4 * kg);
+      if (!col_on) Bm = zero4;
+      Cm = __builtin_amdgcn_mfma_f32_32x32x8f16(mnv, Bm, Cm, 0, 0, 0);
+    }
+    const float si = sinv_s[s * NB_TK + (n & (NB_TK - 1))];
+    __builtin_amdgcn_wave_barrier();   // s_d was written by this wave's own lanes above; LDS operations of a wave complete in order
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      const float4 d4 = *reinterpret_cast<const float4*>(&s_d[(wave * 2 + 0) * 32 + 8 * g + 4 * kg]);
+      const float4 m4 = *reinterpret_cast<const float4*>(&s_d[(wave * 2 + 1) * 32 + 8 * g + 4 * kg]);
+      acc[4 * g + 0] += si * (d4.x * (C0[4 * g + 0] + C1[4 * g + 0]) - m4.x * Cm[4 * g + 0]);
+      acc[4 * g + 1] += si * (d4.y * (C0[4 * g + 1] + C1[4 * g + 1]) - m4.y * Cm[4 * g + 1]);
+      acc[4 * g + 2] += si * (d4.z * (C0[4 * g + 2] + C1[4 * g + 2]) - m4.z * Cm[4 * g + 2]);
+      acc[4 * g + 3] += si * (d4.w * (C0[4 * g + 3] + C1[4 * g + 3]) - m4.w * Cm[4 * g + 3]);
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (s != nS - 1) return;
+    // ---- the slice's contribution of this tile: column t (hi) + column 8 + t (lo); lane t keeps 4 runs of 4 rows ----
+    const int tile = tile0 + (q / nS) * p.tile_stride;
+    const NbSeg* sg; int R0; locate(tile, sg, R0);
+    const int tok = n & (NB_TK - 1);
+    float tot[16];
+#pragma unroll
+    for (int v = 0; v < 16; v++) tot[v] = acc[v] + __shfl_xor(acc[v], NB_TK, 64);
+    if (n < NB_TK && tok < p.n_tok) {
+      float* dst = p.part + ((int64_t)slice * p.n_tok + tok) * p.part_stride + sg->y_off;
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const int row = R0 + 8 * g + 4 * kg;
+        if (row + 3 < sg->rows && ((sg->y_off + row) & 3) == 0) *reinterpret_cast<float4*>(dst + row) = make_float4(tot[4 * g], tot[4 * g + 1], tot[4 * g + 2], tot[4 * g + 3]);
+        else {
+#pragma unroll
+          for (int i = 0; i < 4; i++) if (row + i < sg->rows) dst[row + i] = tot[4 * g + i];
+        }
+      }
+    }
+  };
+
+  for (int q = 0; q < nq; q += 3) {
+    load_w(q + 2, wc); compute(wa, q);
+    if (q + 1 < nq) { load_w(q + 3, wa); compute(wb, q + 1); }
+    if (q + 2 < nq) { load_w(q + 4, wb); compute(wc, q + 2); }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Activation pre-pass: one work-group per (256-block, token).  Source of the block:
+//   SRC 0  x[t][k]                                                       (a plain activation row)
+//   SRC 1  res[t][k] + bias[k] + sum_s part[s][t][k], written back to res (a projection added to the residual stream)
+//   SRC 2  u * silu(g), u = inv_t * sum_s part[s][t][k] + bias[k], g likewise at column half + k   (SwiGLU of a product)
+// then v = gain[k] * value (gain optional), per-block power-of-two scale, hi/lo halfs, sub-block sums, and the block's
+// sum of squares of the un-gained value (for the RMSNorm the consumer of the product applies).
+// ------------------------------------------------------------------------------------------
+struct NbPrepParams {
+  const float* x; int64_t x_stride;             // SRC 0
+  float* res; int64_t res_stride;               // SRC 1 (in/out)
+  const float* part; int64_t part_stride; int n_slices; int n_tok;   // SRC 1, 2
+  const float* bias;                            // SRC 1: [K]; SRC 2: [2*half]
+  int half;                                     // SRC 2: column of the gate partner
+  const float* in_ssq; int in_nsb; int in_K; float in_eps;   // SRC 2: RMSNorm of the product's input (in_ssq null = none)
+  const float* gain;                            // optional, [K]
+  int K;
+  _Float16* hi; _Float16* lo; _Float16* sxhi; _Float16* sxlo; float* sinvb; float* ssq;
+};
+
+__device__ __forceinline__ float nb_inv_rms(const float* ssq, int nsb, int K, float eps, int tok)
+{
+  float t = 0.0f;
+  for (int i = 0; i < nsb; i++) t += ssq[(int64_t)tok * nsb + i];   // fixed order
+  return 1.0f / sqrtf(t / (float)K + eps);
+}
+
+template <int SRC>
+__global__ __launch_bounds__(256) void nb_prep_kernel(const NbPrepParams p)
+{
+  const int sb = blockIdx.x, tok = blockIdx.y, k = sb * 256 + threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float v;
+  if (SRC == 0) v = p.x[(int64_t)tok * p.x_stride + k];
+  else if (SRC == 1) {
+    v = p.res[(int64_t)tok * p.res_stride + k];
+    if (p.bias) v += p.bias[k];
+    for (int s = 0; s < p.n_slices; s++) v += p.part[((int64_t)s * p.n_tok + tok) * p.part_stride + k];
+    p.res[(int64_t)tok * p.res_stride + k] = v;
+  } else {
+    float up = 0.0f, gate = 0.0f;
+    for (int s = 0; s < p.n_slices; s++) {
+      const float* row = p.part + ((int64_t)s * p.n_tok + tok) * p.part_stride;
+      up += row[k]; gate += row[p.half + k];
+    }
+    if (p.in_ssq) { const float inv = nb_inv_rms(p.in_ssq, p.in_nsb, p.in_K, p.in_eps, tok); up *= inv; gate *= inv; }
+    if (p.bias) { up += p.bias[k]; gate += p.bias[p.half + k]; }
+    v = silu_mul(up, gate);
+  }
+  const float raw = v;
+  if (p.gain) v *= p.gain[k];
+  __shared__ float red[8];
+  float amax = fabsf(v), ss = raw * raw;
+  for (int off = 32; off > 0; off >>= 1) { amax = fmaxf(amax, __shfl_xor(amax, off, 64)); ss += __shfl_xor(ss, off, 64); }
+  if (lane == 0) { red[wave] = amax; red[4 + wave] = ss; }
+  __syncthreads();
+  const float a = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  int e = 0;
+  if (a > 0.0f && a < 3.0e38f) { int ex; frexpf(a, &ex); e = 14 - ex; }   // a * 2^e in [2^13, 2^14)
+  e = max(-60, min(60, e));
+  const float s = ldexpf(1.0f, e);
+  const float vs = v * s;
+  const _Float16 h = (_Float16)vs;
+  const int64_t o = (int64_t)tok * p.K + k;
+  p.hi[o] = h; p.lo[o] = (_Float16)(vs - (float)h);
+  float sum = vs;
+  for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);   // 32-lane groups = the 8 sub-blocks
+  if ((threadIdx.x & 31) == 0) {
+    const float q = sum * 0.03125f;
+    const _Float16 sh = (_Float16)q;
+    const int64_t b = (int64_t)tok * (p.K >> 5) + sb * 8 + (threadIdx.x >> 5);
+    p.sxhi[b] = sh; p.sxlo[b] = (_Float16)(q - (float)sh);
+  }
+  if (threadIdx.x == 0) {
+    p.sinvb[(int64_t)tok * (p.K >> 8) + sb] = ldexpf(1.0f, -e);
+    p.ssq[(int64_t)tok * (p.K >> 8) + sb] = (red[4] + red[5]) + (red[6] + red[7]);
+  }
+}
+
+// y[t][y_off + r] = inv_t * sum_s part[s][t][y_off + r] + bias[r] (+ residual): the plain consumer of a product
+struct NbReduceParams {
+  NbSeg seg[3]; int n_seg;
+  const float* part; int64_t part_stride; int n_slices; int n_tok;
+  const float* in_ssq; int in_nsb; int in_K; float in_eps;
+  float* y; int64_t y_stride; const float* residual;
+  int width;                                    // columns covered (sum of the segments)
+};
+__global__ __launch_bounds__(256) void nb_reduce_kernel(const NbReduceParams p)
+{
+  const int tok = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= p.width) return;
+  int sgi = 0;
+  if (p.n_seg > 1 && c >= p.seg[1].y_off) sgi = 1;
+  if (p.n_seg > 2 && c >= p.seg[2].y_off) sgi = 2;
+  float v = 0.0f;
+  for (int s = 0; s < p.n_slices; s++) v += p.part[((int64_t)s * p.n_tok + tok) * p.part_stride + c];
+  if (p.in_ssq) v *= nb_inv_rms(p.in_ssq, p.in_nsb, p.in_K, p.in_eps, tok);
+  if (p.seg[sgi].bias) v += p.seg[sgi].bias[c - p.seg[sgi].y_off];
+  const int64_t o = (int64_t)tok * p.y_stride + c;
+  if (p.residual) v += p.residual[o];
+  p.y[o] = v;
+}
+
+// ------------------------------------------------------------------------------------------
+// host side: workspace + the record of the product in flight (one stream, calls are sequential)
+// ------------------------------------------------------------------------------------------
+namespace {
+struct NbWs {
+  _Float16 *hi = nullptr, *lo = nullptr, *sxhi = nullptr, *sxlo = nullptr; float *sinvb = nullptr, *ssq[2] = {nullptr, nullptr}, *part = nullptr;
+  size_t cap_k = 0, cap_part = 0;
+  int generation = 0;
+  int cur = 0;                // ssq buffer the last pre-pass wrote
+};
+NbWs g_nb;
+struct NbProduct {            // what the last nb_gemm left in `part`
+  NbSeg seg[3]; int n_seg = 0; int n_slices = 0; int n_tok = 0; int64_t part_stride = 0; int width = 0;
+  const float* in_ssq = nullptr; int in_nsb = 0, in_K = 0; float in_eps = 0.0f;
+};
+NbProduct g_prod;
+const float* g_pending_ssq = nullptr; int g_pending_K = 0; float g_pending_eps = 0.0f;   // norm of the activations in the planes
+}  // namespace
+
+int nb_ws_generation() { return g_nb.generation; }
+
+// Reserves planes for k_max columns and a partial buffer of part_floats floats (never inside a stream capture).
+int nb_reserve(int k_max, size_t part_floats)
+{
+  const size_t need_k = (size_t)NB_TK * k_max;
+  if (need_k > g_nb.cap_k) {
+    CAI_HIP(hipStreamSynchronize(ctx().stream));
+    void* old[] = {g_nb.hi, g_nb.lo, g_nb.sxhi, g_nb.sxlo, g_nb.sinvb, g_nb.ssq[0], g_nb.ssq[1]};
+    for (void* q : old) if (q) (void)hipFree(q);
+    CAI_HIP(hipMalloc((void**)&g_nb.hi, need_k * 2)); CAI_HIP(hipMalloc((void**)&g_nb.lo, need_k * 2));
+    CAI_HIP(hipMalloc((void**)&g_nb.sxhi, need_k / 32 * 2 + 64)); CAI_HIP(hipMalloc((void**)&g_nb.sxlo, need_k / 32 * 2 + 64));
+    CAI_HIP(hipMalloc((void**)&g_nb.sinvb, need_k / 256 * 4 + 64));
+    CAI_HIP(hipMalloc((void**)&g_nb.ssq[0], need_k / 256 * 4 + 64)); CAI_HIP(hipMalloc((void**)&g_nb.ssq[1], need_k / 256 * 4 + 64));
+    g_nb.cap_k = need_k; g_nb.generation++;
+  }
+  if (part_floats > g_nb.cap_part) {
+    CAI_HIP(hipStreamSynchronize(ctx().stream));
+    if (g_nb.part) (void)hipFree(g_nb.part);
+    CAI_HIP(hipMalloc((void**)&g_nb.part, part_floats * 4));
+    g_nb.cap_part = part_floats; g_nb.generation++;
+  }
+  return CAI_OK;
+}
+
+// K slices a product over `cols` columns and `tiles` row tiles is cut into
+static void nb_geometry(int cols, int tiles, int& S, int& n_slices, int& gx, int& tile_stride)
+{
+  const int nsb = cols >> 8, n_cu = ctx().n_cu;
+  S = std::min(NB_SMAX, nsb);
+  { static const int force = []() { const char* e = getenv("CAIHIP_NB_S"); return e ? atoi(e) : 0; }(); if (force >= 1 && force <= 8) S = std::min(force, nsb); }
+  n_slices = (nsb + S - 1) / S;
+  gx = (tiles + 3) / 4;
+  // plenty of row groups: let a wave walk several tiles so the staged slice is reused
+  int per_wave = 1;
+  while (per_wave < 4 && (gx / (per_wave * 2)) * n_slices >= 3 * n_cu) per_wave *= 2;
+  gx = (gx + per_wave - 1) / per_wave;
+  tile_stride = gx * 4;
+}
+// upper bound of the slice count for a width (sizes the partial buffer): S never drops below min(4, blocks per row)
+int nb_max_slices(int cols) { const int nsb = cols >> 8; return (nsb + std::min(4, nsb) - 1) / std::min(4, std::max(nsb, 1)); }
+
+static int nb_prep_launch(int src, NbPrepParams& p, int n_tok)
+{
+  if (p.K % 256) return set_error(CAI_ERR_UNSUPPORTED, "small-batch pre-pass: width %d is not a multiple of 256", p.K);
+  if ((size_t)NB_TK * p.K > g_nb.cap_k || n_tok > NB_TK) return set_error(CAI_ERR_STATE, "small-batch pre-pass: workspace not reserved for %d x %d", n_tok, p.K);
+  g_nb.cur ^= 1;
+  p.hi = g_nb.hi; p.lo = g_nb.lo; p.sxhi = g_nb.sxhi; p.sxlo = g_nb.sxlo; p.sinvb = g_nb.sinvb; p.ssq = g_nb.ssq[g_nb.cur];
+  const dim3 grid(p.K >> 8, n_tok);
+  if (src == 0) hipLaunchKernelGGL(nb_prep_kernel<0>, grid, dim3(256), 0, ctx().stream, p);
+  else if (src == 1) hipLaunchKernelGGL(nb_prep_kernel<1>, grid, dim3(256), 0, ctx().stream, p);
+  else hipLaunchKernelGGL(nb_prep_kernel<2>, grid, dim3(256), 0, ctx().stream, p);
+  return CAI_OK;
+}
+static void nb_set_pending_norm(const float* gain, int K, float eps)
+{
+  g_pending_ssq = gain ? g_nb.ssq[g_nb.cur] : nullptr; g_pending_K = K; g_pending_eps = eps;
+}
+
+// planes <- x (RMSNorm with `gain` is completed by the consumer of the next product)
+int nb_prep_plain(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok)
+{
+  NbPrepParams p{}; p.x = x; p.x_stride = x_stride; p.gain = gain; p.K = K;
+  const int rc = nb_prep_launch(0, p, n_tok); if (rc) return rc;
+  nb_set_pending_norm(gain, K, eps);
+  return CAI_OK;
+}
+// res <- res + last product (+bias); planes <- res (norm as above).  The product must not itself carry a pending norm.
+int nb_prep_residual(float* res, int64_t res_stride, const float* gain, float eps, int K, int n_tok)
+{
+  if (g_prod.n_seg != 1 || g_prod.width != K || g_prod.n_tok != n_tok || g_prod.in_ssq)
+    return set_error(CAI_ERR_STATE, "small-batch residual pre-pass: no matching product in flight");
+  NbPrepParams p{}; p.res = res; p.res_stride = res_stride; p.part = g_nb.part; p.part_stride = g_prod.part_stride; p.n_slices = g_prod.n_slices; p.n_tok = n_tok;
+  p.bias = g_prod.seg[0].bias; p.gain = gain; p.K = K;
+  const int rc = nb_prep_launch(1, p, n_tok); if (rc) return rc;
+  nb_set_pending_norm(gain, K, eps);
+  g_prod.n_seg = 0;
+  return CAI_OK;
+}
+// planes <- SwiGLU of the last product (rows [0, half) up, [half, 2 half) gate)
+int nb_prep_swiglu(int half, int n_tok)
+{
+  if (g_prod.n_seg != 1 || g_prod.width != 2 * half || g_prod.n_tok != n_tok) return set_error(CAI_ERR_STATE, "small-batch SwiGLU pre-pass: no matching product in flight");
+  NbPrepParams p{}; p.part = g_nb.part; p.part_stride = g_prod.part_stride; p.n_slices = g_prod.n_slices; p.n_tok = n_tok;
+  p.bias = g_prod.seg[0].bias; p.half = half; p.in_ssq = g_prod.in_ssq; p.in_nsb = g_prod.in_nsb; p.in_K = g_prod.in_K; p.in_eps = g_prod.in_eps; p.K = half;
+  const int rc = nb_prep_launch(2, p, n_tok); if (rc) return rc;
+  nb_set_pending_norm(nullptr, half, 0.0f);
+  g_prod.n_seg = 0;
+  return CAI_OK;
+}
+
+// partials <- [W0; W1; W2] . planes
+int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok)
+{
+  if (n_w < 1 || n_w > 3 || n_tok < 1 || n_tok > NB_TK) return set_error(CAI_ERR_UNSUPPORTED, "small-batch gemm: %d matrices, %d tokens", n_w, n_tok);
+  NbParams p{};
+  p.n_seg = n_w; p.cols = (int)ws[0]->cols;
+  int tiles = 0, width = 0;
+  for (int i = 0; i < n_w; i++) {
+    if (ws[i]->qtype != CAI_Q4_K || ws[i]->cols != ws[0]->cols) return set_error(CAI_ERR_UNSUPPORTED, "small-batch gemm: matrix %d type %d width %lld", i, ws[i]->qtype, (long long)ws[i]->cols);
+    tiles += (int)((ws[i]->rows + 31) / 32);
+    p.seg[i].w = ws[i]->data; p.seg[i].bias = ws[i]->bias; p.seg[i].rows = (int)ws[i]->rows; p.seg[i].y_off = y_off[i]; p.seg[i].tile_end = tiles;
+    width = std::max(width, y_off[i] + (int)ws[i]->rows);
+  }
+  p.n_tiles = tiles;
+  int S, n_slices, gx, tile_stride;
+  nb_geometry(p.cols, tiles, S, n_slices, gx, tile_stride);
+  const int64_t stride = (width + 3) / 4 * 4;
+  if ((size_t)NB_TK * p.cols > g_nb.cap_k || (size_t)n_slices * n_tok * stride > g_nb.cap_part)
+    return set_error(CAI_ERR_STATE, "small-batch gemm: workspace not reserved (%d slices x %d tokens x %lld)", n_slices, n_tok, (long long)stride);
+  p.xhi = g_nb.hi; p.xlo = g_nb.lo; p.sxhi = g_nb.sxhi; p.sxlo = g_nb.sxlo; p.sinvb = g_nb.sinvb; p.n_tok = n_tok;
+  p.part = g_nb.part; p.part_stride = stride; p.sb_per_slice = S; p.tile_stride = tile_stride;
+  const size_t lds = (size_t)S * NB_SC * (NB_LDX + 8) * 2 + (size_t)S * NB_TK * 4 + 4 * 2 * 32 * 4;
+  static bool attr_done = false;
+  if (!attr_done) { (void)hipFuncSetAttribute((const void*)gemm_q4k_nb, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); attr_done = true; }
+  hipLaunchKernelGGL(gemm_q4k_nb, dim3(gx, n_slices), dim3(256), lds, ctx().stream, p);
+  for (int i = 0; i < 3; i++) g_prod.seg[i] = p.seg[i];
+  g_prod.n_seg = n_w; g_prod.n_slices = n_slices; g_prod.n_tok = n_tok; g_prod.part_stride = stride; g_prod.width = width;
+  g_prod.in_ssq = g_pending_ssq; g_prod.in_nsb = g_pending_K >> 8; g_prod.in_K = g_pending_K; g_prod.in_eps = g_pending_eps;
+  return CAI_OK;
+}
+
+// y <- last product (+bias, +residual), pending RMSNorm applied
+int nb_reduce(float* y, int64_t y_stride, const float* residual)
+{
+  if (g_prod.n_seg < 1) return set_error(CAI_ERR_STATE, "small-batch reduce: no product in flight");
+  NbReduceParams p{};
+  for (int i = 0; i < 3; i++) p.seg[i] = g_prod.seg[i];
+  p.n_seg = g_prod.n_seg; p.part = g_nb.part; p.part_stride = g_prod.part_stride; p.n_slices = g_prod.n_slices; p.n_tok = g_prod.n_tok;
+  p.in_ssq = g_prod.in_ssq; p.in_nsb = g_prod.in_nsb; p.in_K = g_prod.in_K; p.in_eps = g_prod.in_eps;
+  p.y = y; p.y_stride = y_stride; p.residual = residual; p.width = g_prod.width;
+  hipLaunchKernelGGL(nb_reduce_kernel, dim3((p.width + 255) / 256, p.n_tok), dim3(256), 0, ctx().stream, p);
+  g_prod.n_seg = 0;
+  return CAI_OK;
+}
+
+// Whole linear layer for up to 16 tokens (two passes above 8): y = W (gain . x / rms) + bias (+ residual)
+int nb_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok, float* y, int64_t y_stride, const float* residual)
+{
+  int rc;
+  if ((rc = nb_reserve((int)w->cols, (size_t)nb_max_slices((int)w->cols) * NB_TK * ((w->rows + 3) / 4 * 4)))) return rc;
+  for (int t0 = 0; t0 < n_tok; t0 += NB_TK) {
+    const int nt = std::min(NB_TK, n_tok - t0); const int zero = 0;
+    if ((rc = nb_prep_plain(x + (int64_t)t0 * x_stride, x_stride, gain, eps, (int)w->cols, nt))) return rc;
+    if ((rc = nb_gemm(&w, &zero, 1, nt))) return rc;
+    if ((rc = nb_reduce(y + (int64_t)t0 * y_stride, y_stride, residual ? residual + (int64_t)t0 * y_stride : nullptr))) return rc;
+  }
+  return CAI_OK;
+}
+
+}  // namespace cai

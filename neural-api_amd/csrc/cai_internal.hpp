@@ -140,8 +140,20 @@ int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const fl
                    float* y, int64_t y_stride, const float* residual);
 bool gemm_mfma_supported(const cai_qw_s* w);
 // split pre-pass / product form: prep once, then any number of matrices of that width
+int prefill_ws(int n_tok, int K, _Float16** hi, _Float16** lo, float** sx, float** sinv);   // grows the shared activation workspace
+// small-batch (<= 8 tokens per pass) matrix-core path: planes <- activations, partials <- product, consumer sums the slices
+int nb_ws_generation();                                        // changes whenever its workspace buffers are reallocated
+int nb_reserve(int k_max, size_t part_floats);                 // never inside a stream capture
+int nb_max_slices(int cols);
+int nb_prep_plain(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok);
+int nb_prep_residual(float* res, int64_t res_stride, const float* gain, float eps, int K, int n_tok);   // res += last product
+int nb_prep_swiglu(int half, int n_tok);                       // planes <- SwiGLU(last product)
+int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok);
+int nb_reduce(float* y, int64_t y_stride, const float* residual);
+int nb_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok, float* y, int64_t y_stride, const float* residual);
 int prefill_prep(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok);
 int prefill_gemm(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride, const float* residual);
+int prefill_gemm_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, float* y, int64_t y_stride);
 
 void rope_thetas(float base, int head_dim, std::vector<float>& out);
 

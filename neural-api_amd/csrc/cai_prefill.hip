@@ -307,6 +307,15 @@ int prefill_prep(const float* x, int64_t x_stride, const float* gain, float eps,
   if ((rc = prefill_ws(n_tok, K, &hi, &lo, &sx, &sinv))) return rc;
   return launch_xprep(x, x_stride, gain, eps, K, n_tok, hi, lo, sx, sinv);
 }
+// Several matrices of one width applied to the prepared activations (q | k | v).
+int prefill_gemm_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, float* y, int64_t y_stride)
+{
+  for (int i = 0; i < n_w; i++) {
+    const int rc = launch_gemm_q4k(ws[i], g_pws.hi, g_pws.lo, g_pws.sx, g_pws.sinv, n_tok, y + y_off[i], y_stride, nullptr, 0);
+    if (rc) return rc;
+  }
+  return CAI_OK;
+}
 int prefill_gemm(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride, const float* residual)
 {
   return launch_gemm_q4k(w, g_pws.hi, g_pws.lo, g_pws.sx, g_pws.sinv, n_tok, y, y_stride, residual, 0);
@@ -317,6 +326,7 @@ int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const fl
                    float* y, int64_t y_stride, const float* residual)
 {
   int rc;
+  if (gemm_mfma_supported(w) && n_tok <= 16) return nb_linear(w, x, x_stride, gain, eps, n_tok, y, y_stride, residual);   // bandwidth-bound regime
   if (gemm_mfma_supported(w)) {
     _Float16 *hi, *lo; float *sx, *sinv;
     if ((rc = prefill_ws(n_tok, (int)w->cols, &hi, &lo, &sx, &sinv))) return rc;

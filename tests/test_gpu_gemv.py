@@ -144,6 +144,23 @@ def test_multi_token_gemm_on_matrix_cores_equals_gemv(rows, cols, T):
         assert rel_err(got[t], want[t], floor=0.02 * cols ** 0.5 * float(np.abs(x[t]).mean())) < TIGHT, t
 
 
+@pytest.mark.parametrize("rows,cols,T", [(128, 256, 2), (33, 512, 3), (1000, 1024, 8), (3584, 3584, 8), (512, 18944, 4), (40000, 2048, 16), (5000, 768, 13)])
+def test_small_batch_gemm_on_matrix_cores_equals_gemv(rows, cols, T):
+    """2..16 tokens: the streaming matrix-core kernel (scales folded exactly into the f16 weight operand, block sums fed as one
+    more reduction step, 1/2/4 super-block slices per row tile) == T single-token layers, bias included."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    raw, rng = make(O.Q4_K, rows, cols, T + 100)
+    x = (rng.standard_normal((T, cols)) * rng.uniform(0.01, 30.0, (T, 1))).astype(np.float32)
+    x[0, : cols // 2] = 0.0                          # all-zero blocks
+    bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
+    w = cai.QWeight(O.Q4_K, rows, cols, raw, bias)
+    got = w.gemm(x)
+    want = O.gemv(O.Q4_K, raw, rows, cols, x, bias, 0, 1)
+    for t in range(T):
+        assert rel_err(got[t], want[t], floor=0.02 * cols ** 0.5 * float(np.abs(x[t]).mean())) < TIGHT, t
+
+
 def test_multi_token_gemm_other_types_and_tokens_not_multiple_of_eight():
     from helpers.device import dev, rel_err
     cai = dev()
