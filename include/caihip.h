@@ -32,6 +32,7 @@ extern "C" {
 #define CAI_Q4_0   2
 #define CAI_Q8_0   8
 #define CAI_Q4_K   12
+#define CAI_Q6_K   14  /* 210-byte super-blocks (neural/neuralgguf.pas:639-717); functional path, not bandwidth-tuned */
 #define CAI_I8ROW  100  /* per-row symmetric int8 + fp32 row scale (neural/neuralvolume.pas:926-987) */
 
 /* ---- activation opcodes fused into the linear layer (neural/neural.cl:114-146) ---- */
@@ -239,7 +240,7 @@ int cai_gguf_tensor_info(cai_gguf_t g, int64_t index, char* name_buf, int name_n
                          int64_t* shape8, int64_t* data_offset, int64_t* nbytes);
 /* pointer into the mapping, valid until cai_gguf_close (the raw-bytes read of neural/neuralsafetensors.pas:1024) */
 int cai_gguf_tensor_data(cai_gguf_t g, int64_t index, const void** ptr);
-/* resident weight from a 2-D tensor in stored order and stored type (F32, F16, Q4_0, Q8_0, Q4_K); bias_name may be
+/* resident weight from a 2-D tensor in stored order and stored type (F32, F16, Q4_0, Q8_0, Q4_K, Q6_K); bias_name may be
  * NULL or name a tensor that is absent */
 int cai_gguf_load_qw(cai_gguf_t g, const char* name, const char* bias_name, cai_qw_t* out);
 /* Whole decoder from a llama or qwen2 file; the decoder owns the weights it loads.  max_ctx <= 0 takes

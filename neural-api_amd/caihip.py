@@ -6,7 +6,7 @@ import numpy as np
 
 from . import lib_path
 
-F32, F16, Q4_0, Q8_0, Q4_K, I8ROW = 0, 1, 2, 8, 12, 100
+F32, F16, Q4_0, Q8_0, Q4_K, Q6_K, I8ROW = 0, 1, 2, 8, 12, 14, 100
 ACT_NONE, ACT_RELU, ACT_SIGMOID, ACT_TANH = 0, 1, 2, 3
 X_DEVICE, Y_DEVICE = 1, 2
 KV_F32, KV_F16 = 0, 1

@@ -530,7 +530,8 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   kv->len.assign((size_t)n_seq * n_layers, 0);
   // few, fat splits: every extra split costs the merging work-group another device-coherent load round,
   // while one CU sustains only ~20 GB/s, so a slice should stay under ~100 KB
-  int sl = (max_ctx + 15) / 16; sl = (sl + 31) / 32 * 32; if (sl < 32) sl = 32; if (sl > 256) sl = 256;
+  static const int sl_max = []() { const char* e = getenv("CAIHIP_ATTN_SPLIT_MAX"); const int v = e ? atoi(e) : 256; return v >= 32 ? v : 256; }();
+  int sl = (max_ctx + 15) / 16; sl = (sl + 31) / 32 * 32; if (sl < 32) sl = 32; if (sl > sl_max) sl = sl_max;
   kv->split_len = sl; kv->n_splits = (max_ctx + sl - 1) / sl;   // the merge stage holds up to 64 splits
   const size_t bytes = (size_t)kv->seq_elems() * n_seq * kv->elem();
   if (kv->n_splits > 64) return set_error(CAI_ERR_UNSUPPORTED, "kv cache: max_ctx %d needs %d splits (limit 64 x 256 rows)", max_ctx, kv->n_splits);

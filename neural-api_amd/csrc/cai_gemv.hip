@@ -369,6 +369,27 @@ __global__ __launch_bounds__(256) void gemv_simple(const GemvParams p, int n_b)
       inv = 1.0f / sqrtf(ss / (float)cols + p.norm_eps);
     }
     float acc = 0.0f;
+    if (QT == CAI_Q6_K) {
+      // one super-block (210 B) per pass of the wave: lane = (half n, position ll) owns elements 128n + ll + {0, 32, 64, 96},
+      // i.e. both nibbles of ql bytes 64n + ll and 64n + ll + 32 and the four 2-bit fields of qh byte 32n + ll
+      const uint8_t* rowp = sg.data + wrow * (int64_t)(cols >> 8) * 210;
+      const int n = lane >> 5, ll = lane & 31;
+      for (int sb = 0; sb < (cols >> 8); sb++) {
+        const uint8_t* blk = rowp + (int64_t)sb * 210;
+        const int l0 = blk[64 * n + ll], l1 = blk[64 * n + ll + 32], h = blk[128 + 32 * n + ll];
+        const int8_t* sc = reinterpret_cast<const int8_t*>(blk + 192) + 8 * n + (ll >> 4);
+        const float d = __half2float(__ushort_as_half((unsigned short)(blk[208] | (blk[209] << 8))));
+        const int q[4] = {((l0 & 15) | ((h & 3) << 4)) - 32, ((l1 & 15) | (((h >> 2) & 3) << 4)) - 32,
+                          ((l0 >> 4) | (((h >> 4) & 3) << 4)) - 32, ((l1 >> 4) | (((h >> 6) & 3) << 4)) - 32};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const int i = sb * 256 + 128 * n + ll + 32 * j;
+          float xv = xb[i];
+          if (p.norm_gain) xv = p.norm_gain[i] * (xv * inv);
+          acc = fmaf((d * (float)sc[2 * j]) * (float)q[j], xv, acc);
+        }
+      }
+    } else
     for (int i = lane; i < cols; i += 64) {
       float w;
       if (QT == CAI_F32) w = reinterpret_cast<const float*>(sg.data)[wrow * cols + i];
@@ -475,6 +496,7 @@ static int64_t data_row_bytes(const cai_qw_s* w)
 {
   switch (w->qtype) {
     case CAI_Q4_K: return w->cols / 256 * 144;
+    case CAI_Q6_K: return w->cols / 256 * 210;
     case CAI_Q4_0: return w->cols / 2;
     case CAI_Q8_0: case CAI_I8ROW: return w->cols;
     case CAI_F32: return w->cols * 4;
@@ -544,6 +566,7 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
   if (qt == CAI_F32) hipLaunchKernelGGL(gemv_simple<CAI_F32>, grid, dim3(256), 0, c.stream, p, n_b);
   else if (qt == CAI_F16) hipLaunchKernelGGL(gemv_simple<CAI_F16>, grid, dim3(256), 0, c.stream, p, n_b);
   else if (qt == CAI_I8ROW) hipLaunchKernelGGL(gemv_simple<CAI_I8ROW>, grid, dim3(256), 0, c.stream, p, n_b);
+  else if (qt == CAI_Q6_K) hipLaunchKernelGGL(gemv_simple<CAI_Q6_K>, grid, dim3(256), 0, c.stream, p, n_b);
   else return set_error(CAI_ERR_UNSUPPORTED, "gemv: weight type %d", qt);
   return CAI_OK;
 }

@@ -53,6 +53,16 @@ __device__ float dequant_elem(int qtype, const uint8_t* data, const uint8_t* aux
       const float dsc = d * (float)sc, dm = dmin * (float)mn;
       return dsc * (float)q - dm;
     }
+    case CAI_Q6_K: {  // x = (d*scale[i/16]) * ((ql | qh<<4) - 32) (neural/neuralgguf.pas:639-717)
+      const uint8_t* blk = data + (row * (cols >> 8) + (i >> 8)) * 210;
+      const int e = (int)(i & 255);
+      const float d = f16_bits_to_float((uint16_t)(blk[208] | (blk[209] << 8)));
+      const float dl = d * (float)reinterpret_cast<const int8_t*>(blk + 192)[e >> 4];
+      const int lo = blk[(e >> 7) * 64 + (e & 63)];
+      const int nib = (e & 127) < 64 ? (lo & 15) : (lo >> 4);
+      const int hi2 = (blk[128 + (e >> 7) * 32 + (e & 31)] >> (2 * ((e & 127) >> 5))) & 3;
+      return dl * (float)((nib | (hi2 << 4)) - 32);
+    }
   }
   return 0.0f;
 }

@@ -79,7 +79,7 @@ int64_t orc_block_elems(int type)
   switch (type) {
     case ORC_F32: case ORC_F16: case ORC_I8ROW: return 1;
     case ORC_Q4_0: case ORC_Q8_0: return 32;
-    case ORC_Q4_K: return 256;
+    case ORC_Q4_K: case ORC_Q6_K: return 256;
   }
   return -1;
 }
@@ -87,7 +87,7 @@ int64_t orc_block_bytes(int type)
 {
   switch (type) {
     case ORC_F32: return 4; case ORC_F16: return 2; case ORC_I8ROW: return 1;
-    case ORC_Q4_0: return 18; case ORC_Q8_0: return 34; case ORC_Q4_K: return 144;
+    case ORC_Q4_0: return 18; case ORC_Q8_0: return 34; case ORC_Q4_K: return 144; case ORC_Q6_K: return 210;
   }
   return -1;
 }
@@ -158,6 +158,60 @@ void orc_dequant_q4_k(const uint8_t* raw, int64_t nb, float* out)
   }
 }
 
+/* neural/neuralgguf.pas:639-717 (DequantizeQ6K): 210-byte super-block = 128 B ql (low 4 bits), 64 B qh (high 2 bits),
+ * 16 int8 group scales, f16 d.  Element i: ql byte (i/128)*64 + i%64, low nibble when i%128 < 64 else high; qh byte
+ * (i/128)*32 + i%32, 2-bit field at shift 2*((i%128)/32); q = (ql | qh<<4) - 32; x = (d * scale[i/16]) * q.
+ * d*scale has <= 18 significant bits and the product with q <= 24, so both roundings are exact. */
+void orc_dequant_q6_k(const uint8_t* raw, int64_t nb, float* out)
+{
+  for (int64_t b = 0; b < nb; b++, raw += 210, out += 256) {
+    const uint8_t* ql = raw; const uint8_t* qh = raw + 128; const int8_t* sc = (const int8_t*)(raw + 192);
+    uint16_t h; memcpy(&h, raw + 208, 2);
+    const float d = orc_f16_to_f32(h);
+    for (int i = 0; i < 256; i++) {
+      volatile float dl = d * (float)sc[i >> 4];
+      const int lo = ql[(i >> 7) * 64 + (i & 63)];
+      const int nib = (i & 127) < 64 ? (lo & 15) : (lo >> 4);
+      const int hi2 = (qh[(i >> 7) * 32 + (i & 31)] >> (2 * ((i & 127) >> 5))) & 3;
+      out[i] = dl * (float)((nib | (hi2 << 4)) - 32);
+    }
+  }
+}
+
+/* Packer for synthetic weights (the reference has none): per 16-group scale = max|x|/31 quantised to int8 against
+ * d = max scale / 127, q = round(x / (d*scale)) clamped to [-32, 31]. */
+void orc_quant_q6_k(const float* x, int64_t n, uint8_t* out)
+{
+  for (int64_t b = 0; b < n / 256; b++, x += 256, out += 210) {
+    float gs[16], smax = 0.0f;
+    for (int g = 0; g < 16; g++) {
+      float a = 0.0f;
+      for (int k = 0; k < 16; k++) { float v = fabsf(x[16 * g + k]); if (v > a) a = v; }
+      gs[g] = a / 31.0f; if (gs[g] > smax) smax = gs[g];
+    }
+    const uint16_t dh = orc_f32_to_f16(smax / 127.0f);
+    const float d = orc_f16_to_f32(dh);
+    memset(out, 0, 210);
+    memcpy(out + 208, &dh, 2);
+    int8_t* sc = (int8_t*)(out + 192);
+    for (int g = 0; g < 16; g++) {
+      int s = d > 0.0f ? (int)lrintf(gs[g] / d) : 0;
+      if (s > 127) s = 127;
+      if (s < 1 && gs[g] > 0.0f) s = 1;
+      sc[g] = (int8_t)s;
+    }
+    for (int i = 0; i < 256; i++) {
+      const float dl = d * (float)sc[i >> 4];
+      int q = dl > 0.0f ? (int)lrintf(x[i] / dl) : 0;
+      if (q < -32) q = -32; if (q > 31) q = 31;
+      const int u = q + 32;
+      uint8_t* pl = out + (i >> 7) * 64 + (i & 63);
+      if ((i & 127) < 64) *pl |= (uint8_t)(u & 15); else *pl |= (uint8_t)((u & 15) << 4);
+      out[128 + (i >> 7) * 32 + (i & 31)] |= (uint8_t)((u >> 4) << (2 * ((i & 127) >> 5)));
+    }
+  }
+}
+
 /* neural/neuralgguf.pas:1471-1523 (DecodeGGMLSpan) */
 int orc_dequant(int type, const void* raw, int64_t n, float* out)
 {
@@ -168,6 +222,7 @@ int orc_dequant(int type, const void* raw, int64_t n, float* out)
     case ORC_Q8_0: if (n % 32) return -1; orc_dequant_q8_0(p, n / 32, out); return 0;
     case ORC_Q4_0: if (n % 32) return -1; orc_dequant_q4_0(p, n / 32, out); return 0;
     case ORC_Q4_K: if (n % 256) return -1; orc_dequant_q4_k(p, n / 256, out); return 0;
+    case ORC_Q6_K: if (n % 256) return -1; orc_dequant_q6_k(p, n / 256, out); return 0;
   }
   return -2;
 }

@@ -20,7 +20,7 @@ extern "C" {
 
 /* ggml tensor type ids: neural/neuralgguf.pas:86-98 */
 enum {
-  ORC_F32 = 0, ORC_F16 = 1, ORC_Q4_0 = 2, ORC_Q8_0 = 8, ORC_Q4_K = 12,
+  ORC_F32 = 0, ORC_F16 = 1, ORC_Q4_0 = 2, ORC_Q8_0 = 8, ORC_Q4_K = 12, ORC_Q6_K = 14,
   ORC_I8ROW = 100 /* per-row symmetric int8 (neural/neuralvolume.pas:926-987) */
 };
 
@@ -38,6 +38,8 @@ int64_t  orc_row_bytes(int type, int64_t cols);     /* -1 if cols is not a whole
 void orc_dequant_q8_0(const uint8_t* raw, int64_t n_blocks, float* out);  /* neuralgguf.pas:1487-1503 + neuralvolume.pas:12564-12582 */
 void orc_dequant_q4_0(const uint8_t* raw, int64_t n_blocks, float* out);  /* neuralgguf.pas:811-845 */
 void orc_dequant_q4_k(const uint8_t* raw, int64_t n_blocks, float* out);  /* neuralgguf.pas:472-514 */
+void orc_dequant_q6_k(const uint8_t* raw, int64_t n_blocks, float* out);    /* neuralgguf.pas:639-717 (DequantizeQ6K) */
+void orc_quant_q6_k(const float* x, int64_t n_elems, uint8_t* out);        /* this build's packer; layout neuralgguf.pas:639-650 */
 int  orc_dequant(int type, const void* raw, int64_t n_elems, float* out); /* neuralgguf.pas:1471-1523 */
 
 /* ---- quantizers (make synthetic weights; only Q8_0 exists in the reference) ---- */

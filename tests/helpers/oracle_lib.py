@@ -9,7 +9,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 _LIB = None
 
-F32, F16, Q4_0, Q8_0, Q4_K, I8ROW = 0, 1, 2, 8, 12, 100
+F32, F16, Q4_0, Q8_0, Q4_K, Q6_K, I8ROW = 0, 1, 2, 8, 12, 14, 100
 W_EMBED, W_HEAD, W_Q, W_K, W_V, W_O, W_GATEUP, W_DOWN, W_ROUTER = range(9)
 V_ATTN_NORM, V_MLP_NORM, V_FINAL_NORM, V_Q_NORM, V_K_NORM = range(5)
 
@@ -35,7 +35,7 @@ def lib():
         L.orc_f32_to_f16.restype = C.c_uint16; L.orc_f32_to_f16.argtypes = [C.c_float]
         L.orc_row_bytes.restype = C.c_int64; L.orc_row_bytes.argtypes = [C.c_int, C.c_int64]
         L.orc_dequant.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_void_p]
-        for n in ("orc_quant_q8_0", "orc_quant_q4_0", "orc_quant_q4_k"):
+        for n in ("orc_quant_q8_0", "orc_quant_q4_0", "orc_quant_q4_k", "orc_quant_q6_k"):
             getattr(L, n).argtypes = [C.c_void_p, C.c_int64, C.c_void_p]; getattr(L, n).restype = None
         L.orc_quant_int8_row.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p]; L.orc_quant_int8_row.restype = None
         L.orc_gguf_deinterleaved_src_row.restype = C.c_int64; L.orc_gguf_deinterleaved_src_row.argtypes = [C.c_int64, C.c_int]
@@ -89,7 +89,7 @@ def quantize(t, x):
     rb = row_bytes(t, x.shape[-1])
     assert rb > 0
     out = np.empty(n // x.shape[-1] * rb, np.uint8)
-    fn = {Q8_0: lib().orc_quant_q8_0, Q4_0: lib().orc_quant_q4_0, Q4_K: lib().orc_quant_q4_k}[t]
+    fn = {Q8_0: lib().orc_quant_q8_0, Q4_0: lib().orc_quant_q4_0, Q4_K: lib().orc_quant_q4_k, Q6_K: lib().orc_quant_q6_k}[t]
     fn(_p(x), n, _p(out))
     return out
 

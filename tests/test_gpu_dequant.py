@@ -35,7 +35,17 @@ def test_q4k_reference_golden_bit_exact_on_device():
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-@pytest.mark.parametrize("qt", [O.Q8_0, O.Q4_0, O.Q4_K])
+def test_q6k_reference_golden_bit_exact_on_device():
+    from helpers.device import dev
+    cai = dev()
+    g = GGUFFile(ref_path("tiny_kquant.gguf"))
+    t, shape, raw = g.raw("kq.Q6_K.weight")
+    w = cai.QWeight(cai.Q6_K, 4, 256, raw)
+    want = np.array(load_json("tiny_kquant_ref.json")["dequant"]["Q6_K"], np.float32)
+    assert np.array_equal(w.dequant_rows().reshape(-1).view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("qt", [O.Q8_0, O.Q4_0, O.Q4_K, O.Q6_K])
 def test_random_bytes_bit_exact(qt):
     """Arbitrary block bytes (every scale/min/nibble pattern, subnormal and huge half scales)."""
     from helpers.device import dev
@@ -53,7 +63,7 @@ def test_random_bytes_bit_exact(qt):
     assert bits_equal(w.dequant_rows(5, 3), want[5:8])
 
 
-@pytest.mark.parametrize("qt", [O.Q8_0, O.Q4_0, O.Q4_K, O.F32, O.F16])
+@pytest.mark.parametrize("qt", [O.Q8_0, O.Q4_0, O.Q4_K, O.Q6_K, O.F32, O.F16])
 def test_quantized_weights_bit_exact(qt):
     from helpers.device import dev
     cai = dev()

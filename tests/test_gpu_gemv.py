@@ -81,6 +81,19 @@ def test_float_weight_types_any_width(qt, rows, cols):
     assert rel_err(got, O.gemv(qt, raw, rows, cols, x, None, 0, 1)) < TIGHT
 
 
+@pytest.mark.parametrize("rows,cols,nb", [(37, 256, 1), (512, 3584, 1), (300, 2048, 3)])
+def test_q6_k_gemv_matches_oracle(rows, cols, nb):
+    """Q6_K (the type real Q4_K_M files use for output.weight and part of ffn_down): functional path, same bar."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    raw, rng = make(O.Q6_K, rows, cols, rows + cols)
+    x = rng.standard_normal((nb, cols)).astype(np.float32)
+    bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
+    got = cai.QWeight(O.Q6_K, rows, cols, raw, bias).gemv(x)
+    want = O.gemv(O.Q6_K, raw, rows, cols, x, bias, 0, 1)
+    assert rel_err(got, want, floor=0.02 * cols ** 0.5) < TIGHT
+
+
 def test_int8_row_path_scale_then_bias():
     # the reference's own fused-quant format: y = scale_a * sum(code*x) + bias_a (neuralvolume.pas:12693-12745)
     from helpers.device import dev, rel_err

@@ -61,6 +61,28 @@ def test_qwen2_style_q4k_file_with_biases_and_untied_q8_head(tmp_path):
     assert np.array_equal(got.argmax(1), want.argmax(1))
 
 
+def test_mixed_q4k_q6k_file_like_a_q4_k_m_export(tmp_path):
+    """A Q4_K body whose output.weight, attn_v and ffn_down are Q6_K, the mix llama.cpp's Q4_K_M preset writes."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    cfg = dict(n_layers=2, d_model=256, n_q_heads=4, n_kv_heads=2, head_dim=64, ffn=512, vocab=300, max_ctx=48, eps=1e-5, rope_theta=1e4)
+    spec = synthetic_spec(cfg, O.Q4_K, head_qtype=O.Q6_K, seed=11)
+    rng = np.random.default_rng(3)
+    for l in range(cfg["n_layers"]):           # re-quantise attn_v and ffn_down as Q6_K
+        for slot in (O.W_V, O.W_DOWN):
+            t = spec["tensors"][(l, slot)]
+            w = (rng.standard_normal((t["rows"], t["cols"])) * 0.02).astype(np.float32)
+            t.update(type=O.Q6_K, raw=O.quantize(O.Q6_K, w))
+    path = str(tmp_path / "m.gguf")
+    spec_to_gguf(path, spec, "llama")
+    dec = cai.Decoder.from_gguf(path)
+    om = oracle_model(spec, acc64=1)
+    seq = [3, 299, 17, 17, 250, 9, 1, 0]
+    want = np.array([om.step(t, p)[1] for p, t in enumerate(seq)])
+    got = run(dec, [seq])[0]
+    assert rel_err(got, want) < 1e-3 and np.array_equal(got.argmax(1), want.argmax(1))
+
+
 def test_loader_refuses_what_it_cannot_run(tmp_path):
     from helpers.device import dev
     cai = dev()
@@ -73,9 +95,9 @@ def test_loader_refuses_what_it_cannot_run(tmp_path):
     m = dict(base); del m["llama.block_count"]; cases.append((m, tens, "llama.block_count"))
     cases.append((dict(base), tens, "missing tensor \"blk.0.attn_q.weight\""))
     m = dict(base); m["llama.rope.scaling.type"] = "yarn"; cases.append((m, tens, "rope.scaling.type"))
-    # a Q6_K embedding: listed by the container, refused by the loader
+    # a Q5_K embedding: listed by the container, refused by the loader
     m = dict(base); m["llama.embedding_length"] = 256
-    cases.append((m, [("token_embd.weight", [10, 256], 14, bytes(10 * 210))], "ggml type 14"))
+    cases.append((m, [("token_embd.weight", [10, 256], 13, bytes(10 * 176))], "ggml type 13"))
     for i, (meta, tensors, needle) in enumerate(cases):
         p = str(tmp_path / ("c%d.gguf" % i))
         write_gguf(p, meta, tensors)

@@ -180,3 +180,28 @@ def test_int8_row_roundtrip():
     codes, scales = O.quant_int8_rows(x)
     assert np.all(np.abs(codes.astype(np.float32) * scales[:, None] - x) <= scales[:, None] * 0.5 + 1e-7)
     assert np.all(np.abs(codes).max(1) == 127)
+
+
+def test_q6_k_dequant_matches_reference_vectors_bit_for_bit():
+    """tiny_kquant.gguf / tiny_kquant_ref.json (gguf-py values): d*scale and its product with q are exact in binary32."""
+    g = GGUFFile(ref_path("tiny_kquant.gguf"))
+    t, shape, raw = g.raw("kq.Q6_K.weight")
+    assert t == O.Q6_K and shape == [1024] and raw.size == 4 * 210
+    want = np.array(load_json("tiny_kquant_ref.json")["dequant"]["Q6_K"], np.float32)
+    got = O.dequant(O.Q6_K, raw, 1024)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_q6_k_closed_form_on_random_bytes_and_packer_round_trip():
+    rng = np.random.default_rng(5)
+    blk = rng.integers(0, 256, 210, dtype=np.uint8)
+    blk[208:210] = np.array([0.0123], np.float16).view(np.uint8)
+    got = O.dequant(O.Q6_K, blk, 256)
+    d = np.float32(np.array([0.0123], np.float16)[0]); sc = blk[192:208].view(np.int8)
+    for i in (0, 15, 16, 63, 64, 100, 127, 128, 191, 200, 255):
+        lo = int(blk[(i // 128) * 64 + i % 64]); nib = (lo & 15) if (i % 128) < 64 else (lo >> 4)
+        h2 = (int(blk[128 + (i // 128) * 32 + i % 32]) >> (2 * ((i % 128) // 32))) & 3
+        assert got[i] == np.float32(np.float32(d * np.float32(sc[i // 16])) * np.float32((nib | (h2 << 4)) - 32))
+    x = (rng.standard_normal(512) * 0.02).astype(np.float32)
+    back = O.dequant(O.Q6_K, O.quantize(O.Q6_K, x), 512)
+    assert np.max(np.abs(back - x)) < np.max(np.abs(x)) / 31 * 0.75      # half a step of the coarsest group, plus scale rounding
