@@ -267,7 +267,7 @@ def main():
                    "prefill": {"tokens": prompt_len - 1, "ms": round(pf_ms.value, 2),
                                "tok_per_s": round((prompt_len - 1) / max(pf_ms.value, 1e-6) * 1e3, 1),
                                "linear_tflops": round(2.0 * n_lin_weights * (prompt_len - 1) / max(pf_ms.value, 1e-6) / 1e9, 1),
-                               "note": "multi-token ingestion: f16 MFMA (exact block integers, hi/lo-split activations = 2 MFMA passes per useful FLOP) + prompt attention; MFMA f16 dense peak 2500 TFLOP/s"}},
+                               "note": "multi-token ingestion: f16 MFMA (exact scale*nibble weight operand, hi/lo-split activations = 2 MFMA passes per useful FLOP) + prompt attention; MFMA f16 dense peak 2500 TFLOP/s"}},
         "roofline": {"bound": "hbm", "kernel": "%s (RMSNorm+gate|up+SwiGLU, %dx%d)" % ("gemv_q4k_dot<1,1,false,2>" if conf["qtype"] == "Q4_K" else "gemv_fast<%s>" % conf["qtype"], 2 * I, d),
                      "achieved": round(k_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(k_gbs / HBM_PEAK_GBS, 4),
                      "avg_launch_us": round(k_avg_us, 2), "algorithmic_bytes_per_launch": int(k_bytes),

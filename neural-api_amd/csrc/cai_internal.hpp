@@ -140,7 +140,6 @@ int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const fl
                    float* y, int64_t y_stride, const float* residual);
 bool gemm_mfma_supported(const cai_qw_s* w);
 // split pre-pass / product form: prep once, then any number of matrices of that width
-int prefill_ws(int n_tok, int K, _Float16** hi, _Float16** lo, float** sx, float** sinv);   // grows the shared activation workspace
 // small-batch (<= 8 tokens per pass) matrix-core path: planes <- activations, partials <- product, consumer sums the slices
 int nb_ws_generation();                                        // changes whenever its workspace buffers are reallocated
 int nb_reserve(int k_max, size_t part_floats);                 // never inside a stream capture

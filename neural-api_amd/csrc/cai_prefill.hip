@@ -19,16 +19,14 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
-constexpr int PF_TOK = 128;   // tokens per work-group tile
-constexpr int PF_KC = 64;     // reduction chunk: one 32-byte Q4_K quant chunk = two sub-blocks
-constexpr int PF_LDK = PF_KC + 4;   // padded LDS row (halfs)
 
 // ------------------------------------------------------------------------------------------
 // Activation pre-pass (one work-group per token): optional RMSNorm (neural/neural.cl:1047-1085), then
-//   s = 2^e with max|x|*s in [2^13, 2^14),  hi = f16(x*s),  lo = f16(x*s - hi),  sx[b] = sum of x over 32-block b.
+//   s = 2^e with max|x|*s in [2^13, 2^14),  hi = f16(x*s),  lo = f16(x*s - hi),
+//   sxhi[b] + sxlo[b] = (sum of x over 32-block b) * s / 32 as two halfs (the block sums go to the matrix cores too).
 // ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void xprep_kernel(const float* x, int64_t x_stride, const float* gain, float eps, int K,
-                                                    _Float16* hi, _Float16* lo, float* sx, float* sinv)
+                                                    _Float16* hi, _Float16* lo, float* sinv, _Float16* sxhi, _Float16* sxlo)
 {
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const float* xr = x + (int64_t)t * x_stride;
@@ -75,205 +73,215 @@ __global__ __launch_bounds__(256) void xprep_kernel(const float* x, int64_t x_st
     hi[(int64_t)t * K + i] = h; lo[(int64_t)t * K + i] = l;
     float sum = v;
     for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
-    if (l32 == 0) sx[(int64_t)t * (K >> 5) + b] = sum;
+    if (l32 == 0) {   // the block sum in the scaled domain of hi/lo, divided by 32 so that it stays inside the half range
+      const float ss = sum * s * 0.03125f;
+      const _Float16 sh = (_Float16)ss;
+      sxhi[(int64_t)t * (K >> 5) + b] = sh; sxlo[(int64_t)t * (K >> 5) + b] = (_Float16)(ss - (float)sh);
+    }
   }
 }
 
 struct GemmParams {
   const uint8_t* w; const float* bias;
   int rows, cols;
-  const _Float16* xhi; const _Float16* xlo; const float* sx; const float* sinv;
+  const _Float16* xhi; const _Float16* xlo;     // [token][cols]
+  const _Float16* sxhi; const _Float16* sxlo;   // [token][cols/32]
+  const float* sinv;                            // [token]
   int n_tok;
   float* y; int64_t y_stride;       // y[t*y_stride + row]
   const float* residual;            // same indexing as y, may alias y
-  int swiglu_half;                  // > 0: rows [0,half) up, [half,2half) gate; y[t*y_stride + i] = up*silu(gate)
+  int n_row_groups, n_tok_tiles;
 };
 
-__device__ __forceinline__ half4_t nib_to_half4(uint32_t t)
+constexpr int PF_LDX = 260;       // halfs per staged token row: 256 + pad (stride = 2 banks mod 64)
+constexpr int PF_TT = 2;          // 32-token MFMA tiles per work-group pass
+
+__device__ __forceinline__ half4_t bytes_to_half4_pf(uint32_t t)
 {
-  // four integer bytes (0..15) -> four exact halfs: bytes become the low mantissa bits of 1024 + n, then -1024
+  // four bytes (0..255) -> four exact halfs 1024 + b (the byte becomes the low mantissa bits of 0x6400 = 1024.0)
   const uint32_t p01 = __builtin_amdgcn_perm(0x64646464u, t, 0x04010400u);
   const uint32_t p23 = __builtin_amdgcn_perm(0x64646464u, t, 0x04030402u);
-  const half2_t k = {(_Float16)1024.0f, (_Float16)1024.0f};
-  const half2_t a = __builtin_bit_cast(half2_t, p01) - k, b = __builtin_bit_cast(half2_t, p23) - k;
+  const half2_t a = __builtin_bit_cast(half2_t, p01), b = __builtin_bit_cast(half2_t, p23);
   return half4_t{a.x, a.y, b.x, b.y};
 }
 
-// One wave: 32 rows x 128 tokens.  MODE 0: plain rows (+bias, +residual).  MODE 1: SwiGLU pairs - the wave owns up rows
-// R0..R0+31 AND the matching gate rows, two accumulator sets.
-template <int MODE>
-__global__ __launch_bounds__(256) void gemm_q4k_mfma(const GemmParams p)
+// One work-group: 128 rows (wave = 32 rows) x 64 tokens, one super-block (256 columns) per step.
+//   * the weight operand sc_j * q (<= 63 * 15, exact in f16) is built once per super-block per wave and reused by both token
+//     tiles and by the hi and lo activation planes; the matrix cores accumulate across the whole super-block;
+//   * -dmin * mn_j * sum_{k in j} x_k is one more MFMA step per plane (k = the 8 sub-blocks);
+//   * d and dmin are applied once per super-block (32 FMAs per tile), the token scale once at the end.
+// Work-group ids are laid out so that the token tiles of one row group run on one XCD: the 8 re-reads of its weights (one
+// per 64 tokens) hit that XCD's L2.
+__global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
 {
-  __shared__ __align__(16) _Float16 xs_hi[PF_TOK * PF_LDK];
-  __shared__ __align__(16) _Float16 xs_lo[PF_TOK * PF_LDK];
-  __shared__ __align__(16) float s_ab[4][(MODE == 1 ? 2 : 1)][4][32];   // [wave][matrix][a_lo,b_lo,a_hi,b_hi][row]
-  constexpr int NM = MODE == 1 ? 2 : 1;
+  extern __shared__ __align__(16) unsigned char pf_smem[];
+  constexpr int NTOK = PF_TT * 32;
+  _Float16* xs_hi = reinterpret_cast<_Float16*>(pf_smem);            // [64][PF_LDX]
+  _Float16* xs_lo = xs_hi + NTOK * PF_LDX;
+  _Float16* sx_hi = xs_lo + NTOK * PF_LDX;                            // [64][8]
+  _Float16* sx_lo = sx_hi + NTOK * 8;
+  float* s_d = reinterpret_cast<float*>(sx_lo + NTOK * 8);            // [4 waves][2][32]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 31, kg = lane >> 5;
-  const int n_out = MODE == 1 ? p.swiglu_half : p.rows;
-  const int R0 = blockIdx.x * 128 + wave * 32;
-  const int T0 = blockIdx.y * PF_TOK;
-  const int K = p.cols, nsb = K >> 8;
+  // linear id = rg_lo + 8 * (tt + n_tok_tiles * rg_hi): a row group's token tiles share id mod 8
+  const int L = blockIdx.x, rg = (L & 7) + 8 * ((L >> 3) / p.n_tok_tiles), ttile = (L >> 3) % p.n_tok_tiles;
+  if (rg >= p.n_row_groups) return;
+  const int R0 = rg * 128 + wave * 32, T0 = ttile * NTOK;
+  const int K = p.cols, nsb = K >> 8, nb32 = K >> 5;
   const int64_t row_bytes = (int64_t)nsb * 144;
-  const uint8_t* wrow[NM];
-#pragma unroll
-  for (int mtx = 0; mtx < NM; mtx++) {
-    int r = min(R0 + n, n_out - 1);
-    if (MODE == 1 && mtx == 1) r += p.swiglu_half;
-    wrow[mtx] = p.w + (int64_t)r * row_bytes;
-  }
-  float16_t Y[NM][4];
-#pragma unroll
-  for (int mtx = 0; mtx < NM; mtx++)
-#pragma unroll
-    for (int tt = 0; tt < 4; tt++)
-#pragma unroll
-      for (int v = 0; v < 16; v++) Y[mtx][tt][v] = 0.0f;
-  float sinv_n[4];
-#pragma unroll
-  for (int tt = 0; tt < 4; tt++) { const int t = T0 + tt * 32 + n; sinv_n[tt] = t < p.n_tok ? p.sinv[t] : 0.0f; }
+  const uint8_t* wrow = p.w + (int64_t)min(R0 + n, p.rows - 1) * row_bytes;   // tail rows: re-read the last row, not written
 
-  uint4 hdr[NM];
-  for (int k0 = 0; k0 < K; k0 += PF_KC) {
-    const int sb = k0 >> 8, c = (k0 >> 6) & 3;
-    // ---- stage the activation chunk: 128 tokens x 64 k (hi and lo) ----
-    __syncthreads();
-    {
-      const int tok = threadIdx.x >> 1, half = threadIdx.x & 1;
-      const int t = T0 + tok;
-      uint4 h[4], l[4];
-      if (t < p.n_tok) {
-        const uint4* sh = reinterpret_cast<const uint4*>(p.xhi + (int64_t)t * K + k0 + half * 32);
-        const uint4* sl = reinterpret_cast<const uint4*>(p.xlo + (int64_t)t * K + k0 + half * 32);
+  struct WRegs { uint4 h, q[4]; };
+  auto load_w = [&](int sb, WRegs& r) {
+    if (sb < nsb) {
+      const uint8_t* blk = wrow + (int64_t)sb * 144;
+      r.h = *reinterpret_cast<const uint4*>(blk);
 #pragma unroll
-        for (int i = 0; i < 4; i++) { h[i] = sh[i]; l[i] = sl[i]; }
-      } else {
-#pragma unroll
-        for (int i = 0; i < 4; i++) { h[i] = make_uint4(0, 0, 0, 0); l[i] = make_uint4(0, 0, 0, 0); }
-      }
-      // padded rows are only 8-byte aligned: store as 64-bit pieces
-      uint2* dh = reinterpret_cast<uint2*>(xs_hi + tok * PF_LDK + half * 32);
-      uint2* dl = reinterpret_cast<uint2*>(xs_lo + tok * PF_LDK + half * 32);
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        dh[2 * i] = make_uint2(h[i].x, h[i].y); dh[2 * i + 1] = make_uint2(h[i].z, h[i].w);
-        dl[2 * i] = make_uint2(l[i].x, l[i].y); dl[2 * i + 1] = make_uint2(l[i].z, l[i].w);
-      }
+      for (int i = 0; i < 4; i++) r.q[i] = *reinterpret_cast<const uint4*>(blk + 16 + 64 * kg + 16 * i);
     }
-    // ---- weights of this chunk: 16 quant bytes per lane (elements 16kg .. 16kg+15 of both sub-blocks) ----
-    half4_t A[NM][2][4];
+  };
+  float16_t Y[PF_TT];
 #pragma unroll
-    for (int mtx = 0; mtx < NM; mtx++) {
-      const uint8_t* blk = wrow[mtx] + (int64_t)sb * 144;
-      if (c == 0) hdr[mtx] = *reinterpret_cast<const uint4*>(blk);
-      const uint4 q = *reinterpret_cast<const uint4*>(blk + 16 + 32 * c + 16 * kg);
-      const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+  for (int tt = 0; tt < PF_TT; tt++)
 #pragma unroll
-      for (int m = 0; m < 4; m++) {
-        A[mtx][0][m] = nib_to_half4(qw[m] & 0x0f0f0f0fu);
-        A[mtx][1][m] = nib_to_half4((qw[m] >> 4) & 0x0f0f0f0fu);
-      }
-      if (kg == 0) {   // block scales of row n for sub-blocks 2c and 2c+1
-        uint32_t sc, mn; q4k_scale_pair(hdr[mtx].y, hdr[mtx].z, hdr[mtx].w, c, sc, mn);
-        const float d = __half2float(__ushort_as_half((unsigned short)(hdr[mtx].x & 0xffffu)));
-        const float dmin = __half2float(__ushort_as_half((unsigned short)(hdr[mtx].x >> 16)));
-        s_ab[wave][mtx][0][n] = d * cvt_ub0(sc); s_ab[wave][mtx][1][n] = dmin * cvt_ub0(mn);
-        s_ab[wave][mtx][2][n] = d * cvt_ub1(sc); s_ab[wave][mtx][3][n] = dmin * cvt_ub1(mn);
-      }
+    for (int v = 0; v < 16; v++) Y[tt][v] = 0.0f;
+
+  WRegs wcur, wnxt;
+  load_w(0, wcur);
+  for (int sb = 0; sb < nsb; sb++) {
+    __syncthreads();                       // the previous step's LDS reads are done
+    // ---- stage 64 tokens x 256 columns of both planes, and the block sums ----
+    for (int idx = threadIdx.x; idx < NTOK * 32 * 2; idx += 256) {
+      const int chunk = idx & 31, tok = (idx >> 5) % NTOK, plane = (idx >> 5) / NTOK;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (T0 + tok < p.n_tok) v = *reinterpret_cast<const uint4*>((plane ? p.xlo : p.xhi) + (int64_t)(T0 + tok) * K + sb * 256 + chunk * 8);
+      uint2* dst = reinterpret_cast<uint2*>((plane ? xs_lo : xs_hi) + tok * PF_LDX + chunk * 8);
+      dst[0] = make_uint2(v.x, v.y); dst[1] = make_uint2(v.z, v.w);
     }
+    if (threadIdx.x < NTOK * 2) {
+      const int tok = threadIdx.x % NTOK, plane = threadIdx.x / NTOK;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (T0 + tok < p.n_tok) v = *reinterpret_cast<const uint4*>((plane ? p.sxlo : p.sxhi) + (int64_t)(T0 + tok) * nb32 + sb * 8);
+      *reinterpret_cast<uint4*>((plane ? sx_lo : sx_hi) + tok * 8) = v;
+    }
+    load_w(sb + 1, wnxt);
     __syncthreads();
 
-    // block sums of x for this lane's token column (two sub-blocks x four token tiles)
-    float sxv[4][2];
-#pragma unroll
-    for (int tt = 0; tt < 4; tt++) {
-      const int t = T0 + tt * 32 + n;
-#pragma unroll
-      for (int s2 = 0; s2 < 2; s2++) sxv[tt][s2] = t < p.n_tok ? p.sx[(int64_t)t * (K >> 5) + (k0 >> 5) + s2] : 0.0f;
+    // ---- weight operand of this super-block: 32 groups of four sc*q values ----
+    const WRegs& r = wcur;
+    const uint32_t sc4 = kg == 0 ? (r.h.y & 0x3f3f3f3fu) : ((r.h.w & 0x0f0f0f0fu) | ((r.h.y >> 2) & 0x30303030u));
+    const uint32_t mn4 = kg == 0 ? (r.h.z & 0x3f3f3f3fu) : (((r.h.w >> 4) & 0x0f0f0f0fu) | ((r.h.z >> 2) & 0x30303030u));
+    const _Float16 k1024 = (_Float16)1024.0f;
+    const half4_t sch = bytes_to_half4_pf(sc4), mnh = bytes_to_half4_pf(mn4);
+    const half4_t scv = half4_t{sch.x - k1024, sch.y - k1024, sch.z - k1024, sch.w - k1024};
+    const half4_t mnv = half4_t{mnh.x - k1024, mnh.y - k1024, mnh.z - k1024, mnh.w - k1024};
+    if (kg == 0) {
+      const float d = __half2float(__ushort_as_half((unsigned short)(r.h.x & 0xffffu)));
+      const float dmin = __half2float(__ushort_as_half((unsigned short)(r.h.x >> 16)));
+      s_d[(wave * 2 + 0) * 32 + n] = d; s_d[(wave * 2 + 1) * 32 + n] = dmin * 32.0f;
     }
+    half4_t A[4][8];
 #pragma unroll
-    for (int s2 = 0; s2 < 2; s2++) {
-      // per-row scales of this lane's 16 output rows: rows 8g + 4kg + (0..3)
-      float av[NM][16], bv[NM][16];
+    for (int j = 0; j < 4; j++) {                                      // sub-block 4kg + j
+      const int ccl = j >> 1, hl = j & 1;
+      const _Float16 sj = j == 0 ? scv.x : (j == 1 ? scv.y : (j == 2 ? scv.z : scv.w));
+      const half2_t s2 = {sj, sj};
+      const half2_t c2 = {(_Float16)(-1024.0f) * sj, (_Float16)(-1024.0f) * sj};   // exact: a multiple of 1024 below 65504
 #pragma unroll
-      for (int mtx = 0; mtx < NM; mtx++)
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-          const float4 a4 = *reinterpret_cast<const float4*>(&s_ab[wave][mtx][2 * s2][8 * g + 4 * kg]);
-          const float4 b4 = *reinterpret_cast<const float4*>(&s_ab[wave][mtx][2 * s2 + 1][8 * g + 4 * kg]);
-          av[mtx][4 * g] = a4.x; av[mtx][4 * g + 1] = a4.y; av[mtx][4 * g + 2] = a4.z; av[mtx][4 * g + 3] = a4.w;
-          bv[mtx][4 * g] = b4.x; bv[mtx][4 * g + 1] = b4.y; bv[mtx][4 * g + 2] = b4.z; bv[mtx][4 * g + 3] = b4.w;
-        }
-#pragma unroll
-      for (int tt = 0; tt < 4; tt++) {
-        const _Float16* bh = xs_hi + (tt * 32 + n) * PF_LDK + s2 * 32 + 16 * kg;
-        const _Float16* bl = xs_lo + (tt * 32 + n) * PF_LDK + s2 * 32 + 16 * kg;
-        half4_t Bh[4], Bl[4];
-#pragma unroll
-        for (int m = 0; m < 4; m++) { Bh[m] = *reinterpret_cast<const half4_t*>(bh + 4 * m); Bl[m] = *reinterpret_cast<const half4_t*>(bl + 4 * m); }
-#pragma unroll
-        for (int mtx = 0; mtx < NM; mtx++) {
-          float16_t P;
-#pragma unroll
-          for (int v = 0; v < 16; v++) P[v] = 0.0f;
-#pragma unroll
-          for (int m = 0; m < 4; m++) {
-            P = __builtin_amdgcn_mfma_f32_32x32x8f16(A[mtx][s2][m], Bh[m], P, 0, 0, 0);
-            P = __builtin_amdgcn_mfma_f32_32x32x8f16(A[mtx][s2][m], Bl[m], P, 0, 0, 0);
-          }
-          const float si = sinv_n[tt], sxn = sxv[tt][s2];
-#pragma unroll
-          for (int v = 0; v < 16; v++) Y[mtx][tt][v] += (av[mtx][v] * si) * P[v] - bv[mtx][v] * sxn;
-        }
+      for (int t = 0; t < 8; t++) {
+        const uint4& qq = r.q[2 * ccl + (t >> 2)];
+        const uint32_t qd = (t & 3) == 0 ? qq.x : ((t & 3) == 1 ? qq.y : ((t & 3) == 2 ? qq.z : qq.w));
+        const uint32_t nib = hl ? ((qd >> 4) & 0x0f0f0f0fu) : (qd & 0x0f0f0f0fu);
+        const uint32_t p01 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04010400u);
+        const uint32_t p23 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04030402u);
+        const half2_t a01 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, p01), s2, c2);   // (1024 + q) * sc - 1024 * sc = sc * q
+        const half2_t a23 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, p23), s2, c2);
+        A[j][t] = half4_t{a01.x, a01.y, a23.x, a23.y};
       }
     }
+    __builtin_amdgcn_wave_barrier();
+    float4 d4[4], m4[4];
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      d4[g] = *reinterpret_cast<const float4*>(&s_d[(wave * 2 + 0) * 32 + 8 * g + 4 * kg]);
+      m4[g] = *reinterpret_cast<const float4*>(&s_d[(wave * 2 + 1) * 32 + 8 * g + 4 * kg]);
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int tt = 0; tt < PF_TT; tt++) {
+      float16_t C0, C1, Cm;
+#pragma unroll
+      for (int v = 0; v < 16; v++) { C0[v] = 0.0f; C1[v] = 0.0f; Cm[v] = 0.0f; }
+      const _Float16* bh = xs_hi + (tt * 32 + n) * PF_LDX + 128 * kg;
+      const _Float16* bl = xs_lo + (tt * 32 + n) * PF_LDX + 128 * kg;
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+          const half4_t Bh = *reinterpret_cast<const half4_t*>(bh + 32 * j + 4 * t);
+          const half4_t Bl = *reinterpret_cast<const half4_t*>(bl + 32 * j + 4 * t);
+          C0 = __builtin_amdgcn_mfma_f32_32x32x8f16(A[j][t], Bh, C0, 0, 0, 0);
+          C1 = __builtin_amdgcn_mfma_f32_32x32x8f16(A[j][t], Bl, C1, 0, 0, 0);
+        }
+      {
+        const half4_t Bmh = *reinterpret_cast<const half4_t*>(sx_hi + (tt * 32 + n) * 8 + 4 * kg);
+        const half4_t Bml = *reinterpret_cast<const half4_t*>(sx_lo + (tt * 32 + n) * 8 + 4 * kg);
+        Cm = __builtin_amdgcn_mfma_f32_32x32x8f16(mnv, Bmh, Cm, 0, 0, 0);
+        Cm = __builtin_amdgcn_mfma_f32_32x32x8f16(mnv, Bml, Cm, 0, 0, 0);
+      }
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        Y[tt][4 * g + 0] += d4[g].x * (C0[4 * g + 0] + C1[4 * g + 0]) - m4[g].x * Cm[4 * g + 0];
+        Y[tt][4 * g + 1] += d4[g].y * (C0[4 * g + 1] + C1[4 * g + 1]) - m4[g].y * Cm[4 * g + 1];
+        Y[tt][4 * g + 2] += d4[g].z * (C0[4 * g + 2] + C1[4 * g + 2]) - m4[g].z * Cm[4 * g + 2];
+        Y[tt][4 * g + 3] += d4[g].w * (C0[4 * g + 3] + C1[4 * g + 3]) - m4[g].w * Cm[4 * g + 3];
+      }
+    }
+    wcur = wnxt;
   }
 
   // ---- write: lane holds column (token) n of each tile and rows 8g + 4kg + (0..3) ----
 #pragma unroll
-  for (int tt = 0; tt < 4; tt++) {
+  for (int tt = 0; tt < PF_TT; tt++) {
     const int t = T0 + tt * 32 + n;
     if (t >= p.n_tok) continue;
+    const float si = p.sinv[t];
 #pragma unroll
     for (int v = 0; v < 16; v++) {
       const int row = R0 + 8 * (v >> 2) + 4 * kg + (v & 3);
-      if (row >= n_out) continue;
+      if (row >= p.rows) continue;
       const int64_t o = (int64_t)t * p.y_stride + row;
-      if (MODE == 0) {
-        float r = Y[0][tt][v];
-        if (p.bias) r += p.bias[row];
-        if (p.residual) r += p.residual[o];
-        p.y[o] = r;
-      } else {
-        float up = Y[0][tt][v], gate = Y[NM - 1][tt][v];
-        if (p.bias) { up += p.bias[row]; gate += p.bias[p.swiglu_half + row]; }
-        p.y[o] = silu_mul(up, gate);
-      }
+      float r = Y[tt][v] * si;
+      if (p.bias) r += p.bias[row];
+      if (p.residual) r += p.residual[o];
+      p.y[o] = r;
     }
   }
 }
 
 int launch_xprep(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok,
-                 _Float16* hi, _Float16* lo, float* sx, float* sinv)
+                 _Float16* hi, _Float16* lo, float* sinv, _Float16* sxhi, _Float16* sxlo)
 {
-  hipLaunchKernelGGL(xprep_kernel, dim3(n_tok), dim3(256), 0, ctx().stream, x, x_stride, gain, eps, K, hi, lo, sx, sinv);
+  hipLaunchKernelGGL(xprep_kernel, dim3(n_tok), dim3(256), 0, ctx().stream, x, x_stride, gain, eps, K, hi, lo, sinv, sxhi, sxlo);
   return CAI_OK;
 }
 
 bool gemm_mfma_supported(const cai_qw_s* w) { return w->qtype == CAI_Q4_K; }
 
-int launch_gemm_q4k(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo, const float* sx, const float* sinv,
-                    int n_tok, float* y, int64_t y_stride, const float* residual, int swiglu_half)
+int launch_gemm_q4k(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo, const _Float16* sxhi, const _Float16* sxlo, const float* sinv,
+                    int n_tok, float* y, int64_t y_stride, const float* residual)
 {
   if (!gemm_mfma_supported(w)) return set_error(CAI_ERR_UNSUPPORTED, "prefill gemm: weight type %d", w->qtype);
   GemmParams p{};
   p.w = w->data; p.bias = w->bias; p.rows = (int)w->rows; p.cols = (int)w->cols;
-  p.xhi = xhi; p.xlo = xlo; p.sx = sx; p.sinv = sinv; p.n_tok = n_tok; p.y = y; p.y_stride = y_stride;
-  p.residual = residual; p.swiglu_half = swiglu_half;
-  const int n_out = swiglu_half ? swiglu_half : p.rows;
-  const dim3 grid((n_out + 127) / 128, (n_tok + PF_TOK - 1) / PF_TOK);
-  if (swiglu_half) return set_error(CAI_ERR_UNSUPPORTED, "prefill gemm: fused SwiGLU is not built (two accumulator sets exceed the register file)");
-  hipLaunchKernelGGL(gemm_q4k_mfma<0>, grid, dim3(256), 0, ctx().stream, p);
+  p.xhi = xhi; p.xlo = xlo; p.sxhi = sxhi; p.sxlo = sxlo; p.sinv = sinv; p.n_tok = n_tok; p.y = y; p.y_stride = y_stride;
+  p.residual = residual;
+  p.n_row_groups = (p.rows + 127) / 128; p.n_tok_tiles = (n_tok + PF_TT * 32 - 1) / (PF_TT * 32);
+  const size_t lds = (size_t)PF_TT * 32 * (PF_LDX + 8) * 2 * 2 + 4 * 2 * 32 * 4;
+  static bool attr_done = false;
+  if (!attr_done) { (void)hipFuncSetAttribute((const void*)gemm_q4k_pf, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); attr_done = true; }
+  const int grid = 8 * p.n_tok_tiles * ((p.n_row_groups + 7) / 8);
+  hipLaunchKernelGGL(gemm_q4k_pf, dim3(grid), dim3(256), lds, ctx().stream, p);
   return CAI_OK;
 }
 
@@ -283,42 +291,45 @@ int launch_gemm_q4k(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo,
 // workspace + C ABI
 // ------------------------------------------------------------------------------------------
 namespace cai {
-struct PrefillWs { _Float16* hi = nullptr; _Float16* lo = nullptr; float* sx = nullptr; float* sinv = nullptr; size_t cap_elems = 0; int cap_tok = 0; };
+struct PrefillWs { _Float16* hi = nullptr; _Float16* lo = nullptr; float* sinv = nullptr; _Float16* sxhi = nullptr; _Float16* sxlo = nullptr; size_t cap_elems = 0; int cap_tok = 0; };
 static PrefillWs g_pws;
 
-int prefill_ws(int n_tok, int K, _Float16** hi, _Float16** lo, float** sx, float** sinv)
+// Grows the shared activation workspace to n_tok x K (never inside a stream capture).
+static int prefill_reserve(int n_tok, int K)
 {
   const size_t need = (size_t)n_tok * K;
   if (need > g_pws.cap_elems || n_tok > g_pws.cap_tok) {
     CAI_HIP(hipStreamSynchronize(ctx().stream));
-    if (g_pws.hi) { (void)hipFree(g_pws.hi); (void)hipFree(g_pws.lo); (void)hipFree(g_pws.sx); (void)hipFree(g_pws.sinv); g_pws = PrefillWs(); }
+    void* old[] = {g_pws.hi, g_pws.lo, g_pws.sinv, g_pws.sxhi, g_pws.sxlo};
+    for (void* q : old) if (q) (void)hipFree(q);
     const size_t ce = std::max(need, g_pws.cap_elems); const int ct = std::max(n_tok, g_pws.cap_tok);
+    g_pws = PrefillWs();
     CAI_HIP(hipMalloc((void**)&g_pws.hi, ce * 2)); CAI_HIP(hipMalloc((void**)&g_pws.lo, ce * 2));
-    CAI_HIP(hipMalloc((void**)&g_pws.sx, ce / 32 * 4 + 64)); CAI_HIP(hipMalloc((void**)&g_pws.sinv, (size_t)ct * 4));
+    CAI_HIP(hipMalloc((void**)&g_pws.sxhi, ce / 32 * 2 + 64)); CAI_HIP(hipMalloc((void**)&g_pws.sxlo, ce / 32 * 2 + 64));
+    CAI_HIP(hipMalloc((void**)&g_pws.sinv, (size_t)ct * 4));
     g_pws.cap_elems = ce; g_pws.cap_tok = ct;
   }
-  *hi = g_pws.hi; *lo = g_pws.lo; *sx = g_pws.sx; *sinv = g_pws.sinv;
   return CAI_OK;
 }
 
 int prefill_prep(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok)
 {
-  _Float16 *hi, *lo; float *sx, *sinv; int rc;
-  if ((rc = prefill_ws(n_tok, K, &hi, &lo, &sx, &sinv))) return rc;
-  return launch_xprep(x, x_stride, gain, eps, K, n_tok, hi, lo, sx, sinv);
+  int rc;
+  if ((rc = prefill_reserve(n_tok, K))) return rc;
+  return launch_xprep(x, x_stride, gain, eps, K, n_tok, g_pws.hi, g_pws.lo, g_pws.sinv, g_pws.sxhi, g_pws.sxlo);
 }
 // Several matrices of one width applied to the prepared activations (q | k | v).
 int prefill_gemm_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, float* y, int64_t y_stride)
 {
   for (int i = 0; i < n_w; i++) {
-    const int rc = launch_gemm_q4k(ws[i], g_pws.hi, g_pws.lo, g_pws.sx, g_pws.sinv, n_tok, y + y_off[i], y_stride, nullptr, 0);
+    const int rc = launch_gemm_q4k(ws[i], g_pws.hi, g_pws.lo, g_pws.sxhi, g_pws.sxlo, g_pws.sinv, n_tok, y + y_off[i], y_stride, nullptr);
     if (rc) return rc;
   }
   return CAI_OK;
 }
 int prefill_gemm(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride, const float* residual)
 {
-  return launch_gemm_q4k(w, g_pws.hi, g_pws.lo, g_pws.sx, g_pws.sinv, n_tok, y, y_stride, residual, 0);
+  return launch_gemm_q4k(w, g_pws.hi, g_pws.lo, g_pws.sxhi, g_pws.sxlo, g_pws.sinv, n_tok, y, y_stride, residual);
 }
 
 // y[t][rows] = W x[t] (+bias) (+residual) for n_tok tokens; x rows are x_stride apart; gain != null fuses RMSNorm.
@@ -328,10 +339,8 @@ int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const fl
   int rc;
   if (gemm_mfma_supported(w) && n_tok <= 16) return nb_linear(w, x, x_stride, gain, eps, n_tok, y, y_stride, residual);   // bandwidth-bound regime
   if (gemm_mfma_supported(w)) {
-    _Float16 *hi, *lo; float *sx, *sinv;
-    if ((rc = prefill_ws(n_tok, (int)w->cols, &hi, &lo, &sx, &sinv))) return rc;
-    launch_xprep(x, x_stride, gain, eps, (int)w->cols, n_tok, hi, lo, sx, sinv);
-    return launch_gemm_q4k(w, hi, lo, sx, sinv, n_tok, y, y_stride, residual, 0);
+    if ((rc = prefill_prep(x, x_stride, gain, eps, (int)w->cols, n_tok))) return rc;
+    return prefill_gemm(w, n_tok, y, y_stride, residual);
   }
   // other weight types: groups of up to 8 tokens through the small-batch kernel (x must be contiguous)
   if (x_stride != w->cols) return set_error(CAI_ERR_UNSUPPORTED, "prefill linear: strided input needs a Q4_K matrix");
