@@ -142,6 +142,7 @@ def main():
     ap.add_argument("--config", default="qwen2.5-7b-q4k", choices=list(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernel-reps", type=int, default=5)
+    ap.add_argument("--kv", choices=["f32", "f16", "i8"], default=None, help="KV cache element type (default: the configuration's own)")
     ap.add_argument("--batch", type=int, default=1, help="independent sequences decoded together (1..8)")
     ap.add_argument("--gemv-sweep", action="store_true", help="isolated matrix-vector sweep (BASELINE configs[1]): Q8_0 / Q4_0 / Q4_K, five shapes, batch 1 and 4")
     ap.add_argument("--copy-calibration", action="store_true", help="only run the 1 GiB device copy kernel 5 times (reference for traffic counters)")
@@ -179,7 +180,8 @@ def main():
     t0 = time.time()
     spec = synth.random_decoder_spec(cfg, QT[conf["qtype"]], QT[conf["head"]], seed=424242, qkv_bias=conf["bias"])
     B = args.batch
-    dec = cai.Decoder(spec, max_batch=B, kv_dtype=cai.KV_F16 if conf.get("kv") == "f16" else cai.KV_F32)
+    kv_kind = args.kv or conf.get("kv", "f32")
+    dec = cai.Decoder(spec, max_batch=B, kv_dtype={"f32": cai.KV_F32, "f16": cai.KV_F16, "i8": cai.KV_I8}[kv_kind])
     torch.cuda.empty_cache()
     t_build = time.time() - t0
     wbytes = dec.weight_bytes()
@@ -222,7 +224,7 @@ def main():
     ms_per_step = wall * 1e3 / K
     tok_s = K * B / wall
     ctx_mid = pos + K // 2
-    kv_bytes = B * cfg["n_layers"] * 2 * cfg["n_kv_heads"] * cfg["head_dim"] * (2 if conf.get("kv") == "f16" else 4) * ctx_mid
+    kv_bytes = B * cfg["n_layers"] * 2 * cfg["n_kv_heads"] * cfg["head_dim"] * {"f32": 4, "f16": 2, "i8": 1}[kv_kind] * ctx_mid
     ne = cfg.get("n_experts", 0)
     algo_bytes = wbytes + kv_bytes
 
@@ -260,7 +262,7 @@ def main():
         "dtype": "q4_k/q8_0 weights, f32 accumulate", "data": "synthetic",
         "config": {"workload": "%s: %d-token random prompt (seed 424242), then greedy decode at batch %d; timed %d decode steps at ctx %d..%d"
                                % (args.config, prompt_len, B, K, pos + 1, pos + K),
-                   "weights": "random N(0,0.02), %s body + %s head, %s KV cache" % (conf["qtype"], conf["head"], conf.get("kv", "f32")),
+                   "weights": "random N(0,0.02), %s body + %s head, %s KV cache" % (conf["qtype"], conf["head"], kv_kind),
                    "algorithmic_bytes_per_step": int(algo_bytes), "hip_event_ms_per_step": round(ms.value / K, 4),
                    "whole_step_hbm_frac": round(algo_bytes / (wall / K) / 1e9 / HBM_PEAK_GBS, 4), "device": cai.device_name(),
                    "build_s": round(t_build, 1),

@@ -48,6 +48,8 @@ extern "C" {
 /* ---- KV cache element types ---- */
 #define CAI_KV_F32 0
 #define CAI_KV_F16 1
+#define CAI_KV_I8  2  /* codes in [-127,127] + one fp32 scale per cached row (scale = max|row|/127), the format of
+                         cai_sdpa_append_kv_int8 / QuantizeCacheRow, neural/neural.cl:2501-2580 */
 
 typedef struct cai_qw_s*      cai_qw_t;       /* resident quantized weight matrix */
 typedef struct cai_kv_s*      cai_kv_t;       /* KV cache of one sequence, all layers */
@@ -148,6 +150,13 @@ int cai_kv_len(cai_kv_t kv, int layer, int* len_out);
 int cai_kv_snapshot(cai_kv_t kv, cai_kv_snap_t* out);
 int cai_kv_restore(cai_kv_t kv, cai_kv_snap_t snap);
 int cai_kv_snap_destroy(cai_kv_snap_t snap);
+/* Host copy of one layer's live rows and its inverse (CaptureCacheState / CaptureCacheStateInt8 and RestoreCacheState /
+ * RestoreCacheStateInt8 as TNNetStreamingDecoder.Snapshot/Restore call them per layer, neural/neuraldecode.pas:5775-5790,
+ * 5828-5840; also the hand-off of a host-built prefix to the device).  k and v hold [kv_heads][len][head_dim] elements
+ * of the cache's type (float, IEEE half bits, or int8 codes); k_scales and v_scales hold [kv_heads][len] row scales and
+ * are used only by a CAI_KV_I8 cache (null otherwise).  Import sets the layer's length to len. */
+int cai_kv_export_layer(cai_kv_t kv, int layer, void* k, void* v, float* k_scales, float* v_scales);
+int cai_kv_import_layer(cai_kv_t kv, int layer, int len, const void* k, const void* v, const float* k_scales, const float* v_scales);
 /* One token of one layer: qkv = [Q (q_heads*hd) | K (kv_heads*hd) | V (kv_heads*hd)]; appends K,V at
  * slot CacheLength(layer), then out[h] = softmax(q_h.K/sqrt(hd)) V over the live range
  * (window > 0: last `window` rows; softcap > 0: Gemma-2 style cap).  out: [q_heads*hd]. */
@@ -169,7 +178,7 @@ typedef struct cai_decoder_config {
   int32_t n_experts;     /* 0 = dense SwiGLU FFN; else `ffn` is the per-expert width */
   int32_t top_k;
   int32_t norm_topk;
-  int32_t kv_dtype;      /* CAI_KV_F32 / CAI_KV_F16 */
+  int32_t kv_dtype;      /* CAI_KV_F32 / CAI_KV_F16 / CAI_KV_I8 */
   int32_t max_batch;     /* independent sequences, each with its own KV cache (1..8) */
 } cai_decoder_config;
 

@@ -9,7 +9,7 @@ from . import lib_path
 F32, F16, Q4_0, Q8_0, Q4_K, Q6_K, I8ROW = 0, 1, 2, 8, 12, 14, 100
 ACT_NONE, ACT_RELU, ACT_SIGMOID, ACT_TANH = 0, 1, 2, 3
 X_DEVICE, Y_DEVICE = 1, 2
-KV_F32, KV_F16 = 0, 1
+KV_F32, KV_F16, KV_I8 = 0, 1, 2
 W_EMBED, W_HEAD, W_Q, W_K, W_V, W_O, W_GATEUP, W_DOWN, W_ROUTER = range(9)
 V_ATTN_NORM, V_MLP_NORM, V_FINAL_NORM, V_Q_NORM, V_K_NORM = range(5)
 
@@ -18,7 +18,7 @@ SYMBOLS = """cai_init cai_shutdown cai_last_error cai_device_name cai_sync cai_g
 cai_dev_alloc cai_dev_free cai_dev_upload cai_dev_download cai_dev_copy
 cai_qw_create cai_qw_create_int8row cai_qw_destroy cai_qw_info cai_qw_dequant_rows cai_qgemv cai_ffn_gateup cai_qgemm
 cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_router_topk
-cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_attn_decode
+cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_kv_export_layer cai_kv_import_layer cai_attn_decode
 cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_generate
 cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_snapshot cai_decoder_restore
 cai_decoder_weight_bytes cai_decoder_get_config cai_decoder_load_gguf
@@ -81,6 +81,8 @@ def load():
         L.cai_kv_snapshot.argtypes = [vp, C.POINTER(vp)]
         L.cai_kv_restore.argtypes = [vp, vp]
         L.cai_kv_snap_destroy.argtypes = [vp]
+        L.cai_kv_export_layer.argtypes = [vp, C.c_int, vp, vp, vp, vp]
+        L.cai_kv_import_layer.argtypes = [vp, C.c_int, C.c_int, vp, vp, vp, vp]
         L.cai_attn_decode.argtypes = [vp, i32, vp, i32, i32, f32, vp, i32]
         L.cai_decoder_create.argtypes = [C.POINTER(DecoderConfig), C.POINTER(vp)]
         L.cai_decoder_destroy.argtypes = [vp]
@@ -204,7 +206,7 @@ class QWeight:
 class KVCache:
     def __init__(self, n_layers, kv_heads, head_dim, max_ctx, dtype=KV_F32):
         self.h = C.c_void_p()
-        self.kv_heads, self.head_dim = kv_heads, head_dim
+        self.kv_heads, self.head_dim, self.dtype = kv_heads, head_dim, dtype
         check(load().cai_kv_create(n_layers, kv_heads, head_dim, max_ctx, dtype, C.byref(self.h)))
 
     def attn_decode(self, layer, qkv, q_heads, window=0, softcap=0.0):
@@ -231,6 +233,22 @@ class KVCache:
 
     def restore(self, s):
         check(load().cai_kv_restore(self.h, s))
+
+    def export_layer(self, layer):
+        """(k, v, k_scales, v_scales): the live rows in the cache's element type; scales are None unless int8."""
+        n = self.len(layer)
+        et = {KV_F32: np.float32, KV_F16: np.float16, KV_I8: np.int8}[self.dtype]
+        k = np.zeros((self.kv_heads, n, self.head_dim), et); v = np.zeros_like(k)
+        ks = np.zeros((self.kv_heads, n), np.float32) if self.dtype == KV_I8 else None
+        vs = np.zeros_like(ks) if ks is not None else None
+        check(load().cai_kv_export_layer(self.h, layer, _ptr(k), _ptr(v), _ptr(ks) if ks is not None else None, _ptr(vs) if vs is not None else None))
+        return k, v, ks, vs
+
+    def import_layer(self, layer, k, v, ks=None, vs=None):
+        k = np.ascontiguousarray(k); v = np.ascontiguousarray(v)
+        if ks is not None:
+            ks = np.ascontiguousarray(ks, np.float32); vs = np.ascontiguousarray(vs, np.float32)
+        check(load().cai_kv_import_layer(self.h, layer, k.shape[1], _ptr(k), _ptr(v), _ptr(ks) if ks is not None else None, _ptr(vs) if vs is not None else None))
 
     def close(self):
         if self.h:

@@ -51,6 +51,49 @@ template <> __device__ __forceinline__ void load_row_vec<4, __half>(const __half
   o[0] = __low2float(a); o[1] = __high2float(a); o[2] = __low2float(b); o[3] = __high2float(b);
 }
 
+template <> __device__ __forceinline__ void load_row_vec<1, int8_t>(const int8_t* s, float (&o)[1]) { o[0] = (float)s[0]; }
+template <> __device__ __forceinline__ void load_row_vec<2, int8_t>(const int8_t* s, float (&o)[2])
+{
+  const int r = *reinterpret_cast<const short*>(s);
+  o[0] = (float)(int8_t)(r & 0xff); o[1] = (float)(int8_t)((r >> 8) & 0xff);
+}
+template <> __device__ __forceinline__ void load_row_vec<4, int8_t>(const int8_t* s, float (&o)[4])
+{
+  const int r = *reinterpret_cast<const int*>(s);
+  o[0] = (float)((r << 24) >> 24); o[1] = (float)((r << 16) >> 24); o[2] = (float)((r << 8) >> 24); o[3] = (float)(r >> 24);
+}
+
+// max over each half-wave (32 lanes), result in every lane of that half
+__device__ __forceinline__ float half_wave_allmax(float v)
+{
+  for (int o = 16; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// One cached row of an int8 cache from DS elements per lane of a half-wave (neural/neural.cl:2549-2578): the maximum
+// over FINITE magnitudes, zero codes and unit scale when that maximum is zero or denormal, else scale = max / 127 and
+// code = clamp(rint(v * (1/max) * 127)), NaN -> 0.  Lanes beyond the head width pass zeros.  On return v[] holds the
+// codes as floats.
+template <int DS> __device__ __forceinline__ float quantise_row_i8(float (&v)[DS])
+{
+  float m = 0.0f;
+#pragma unroll
+  for (int i = 0; i < DS; i++) {
+    const float a = fabsf(v[i]);
+    if (__builtin_bit_cast(uint32_t, a) <= 0x7F7FFFFFu) m = fmaxf(m, a);
+  }
+  m = half_wave_allmax(m);
+  const bool usable = __builtin_bit_cast(uint32_t, m) >= 0x00800000u;
+  const float recip = usable ? 1.0f / m : 0.0f;
+#pragma unroll
+  for (int i = 0; i < DS; i++) {
+    float scaled = v[i] * recip * 127.0f;
+    if (!usable || __builtin_bit_cast(uint32_t, fabsf(v[i])) > 0x7F800000u) scaled = 0.0f;
+    v[i] = fminf(fmaxf(rintf(scaled), -127.0f), 127.0f);
+  }
+  return usable ? m / 127.0f : 1.0f;
+}
+
 struct AttnParams {
   float* qkv; int64_t qkv_stride;
   void* kc; void* vc;          // base of [seq][layer][kv_head][max_ctx][hd]
@@ -67,6 +110,8 @@ struct AttnParams {
   int appended;                // 1: the K,V rows of this step are already in the cache (prompt ingestion)
   float* part_override;        // split partials buffer when more rows than cache sequences are in flight
   int* counters;               // [seq][kv_head] arrival counters of the split merge (zero between launches)
+  float* ksc; float* vsc;      // int8 caches: row scales [seq][layer][kv_head][max_ctx]
+  int64_t seq_rows, layer_row_off;
 };
 
 // ---- split kernel: RoPE (neural/neural.cl:1517-1542) + KV append (2354-2379) + split-K online-softmax decode
@@ -306,20 +351,31 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
   KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (seq * p.seq_mul + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
   KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (seq * p.seq_mul + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
 
+  // int8 cache: codes enter the dot products as they are; the K row scale multiplies the finished score and the V row
+  // scale the softmax weight (neural/neural.cl:2639-2640, 2683-2684), so nothing is dequantised per element
+  constexpr bool I8 = sizeof(KV_T) == 1;
+  const float* ksc = nullptr; const float* vsc = nullptr;
+  if (I8) {
+    const int64_t r0 = (seq * p.seq_mul + p.seq0) * p.seq_rows + p.layer_row_off + (int64_t)g * p.max_ctx;
+    ksc = p.ksc + r0; vsc = p.vsc + r0;
+  }
+
   constexpr int PCH = 4;
-  float kdA[PCH][DS] = {}, vdA[PCH][DS] = {}, kdB[PCH][DS] = {}, vdB[PCH][DS] = {};
-  auto load_chunk = [&](float (&kd)[PCH][DS], float (&vd)[PCH][DS], int j0) {
+  struct Chunk { float k[PCH][DS], v[PCH][DS], ks[PCH], vs[PCH]; };
+  Chunk cA = {}, cB = {};
+  auto load_chunk = [&](Chunk& ch, int j0) {
     if (j0 >= s_end || d0 >= hd) return;       // lanes beyond the head width keep their zeros
 #pragma unroll
     for (int c = 0; c < PCH; c++) {
       const int j = min(j0 + 8 * c, s_end - 1);
       // (the slot of the row being appended may hold stale values: reduce_chunk replaces it from registers)
-      load_row_vec<DS, KV_T>(kc + (int64_t)j * hd + d0, kd[c]);
-      load_row_vec<DS, KV_T>(vc + (int64_t)j * hd + d0, vd[c]);
+      load_row_vec<DS, KV_T>(kc + (int64_t)j * hd + d0, ch.k[c]);
+      load_row_vec<DS, KV_T>(vc + (int64_t)j * hd + d0, ch.v[c]);
+      if (I8) { ch.ks[c] = ksc[j]; ch.vs[c] = vsc[j]; }
     }
   };
-  load_chunk(kdA, vdA, s_begin + hw);      // cached rows are requested before the rotation math
-  load_chunk(kdB, vdB, s_begin + hw + 8 * PCH);
+  load_chunk(cA, s_begin + hw);      // cached rows are requested before the rotation math
+  load_chunk(cB, s_begin + hw + 8 * PCH);
 
   float rs[(DS + 1) / 2], rc[(DS + 1) / 2];
 #pragma unroll
@@ -350,32 +406,45 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
   for (int i = 0; i < DS; i++) { acc[i] = 0.0f; knew[i] = 0.0f; vnew[i] = 0.0f; }
   // every work-group whose slice holds `pos` keeps the new row in registers; the group's first head appends it
   const bool owns_new = !p.appended && pos >= s_begin && pos < s_end;
+  float knew_s = 1.0f, vnew_s = 1.0f;
   if (owns_new) {
     load_rot(row + qw + g * hd, knew, p.theta != nullptr);
     load_rot(row + qw + kw + g * hd, vnew, false);
+    if constexpr (I8) {
+      knew_s = quantise_row_i8<DS>(knew);
+      vnew_s = quantise_row_i8<DS>(vnew);
+      if (h == 0 && hw == 0) {
 #pragma unroll
-    for (int i = 0; i < DS; i++) {
-      vnew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(vnew[i]));
-      knew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(knew[i]));
-      if (h == 0 && hw == 0 && d0 + i < hd) {
-        kc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(knew[i]);
-        vc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(vnew[i]);
+        for (int i = 0; i < DS; i++)
+          if (d0 + i < hd) { kc[(int64_t)pos * hd + d0 + i] = (int8_t)knew[i]; vc[(int64_t)pos * hd + d0 + i] = (int8_t)vnew[i]; }
+        if (l32 == 0) { p.ksc[(ksc - p.ksc) + pos] = knew_s; p.vsc[(vsc - p.vsc) + pos] = vnew_s; }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < DS; i++) {
+        vnew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(vnew[i]));
+        knew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(knew[i]));
+        if (h == 0 && hw == 0 && d0 + i < hd) {
+          kc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(knew[i]);
+          vc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(vnew[i]);
+        }
       }
     }
   }
   float m = -1e30f, l = 0.0f;
-  auto reduce_chunk = [&](float (&kd)[PCH][DS], float (&vd)[PCH][DS], int j0) {
+  auto reduce_chunk = [&](Chunk& ch, int j0) {
     float sc[PCH], cmax = -1e30f;
 #pragma unroll
     for (int c = 0; c < PCH; c++) {
       if (owns_new && min(j0 + 8 * c, s_end - 1) == pos) {
 #pragma unroll
-        for (int i = 0; i < DS; i++) { kd[c][i] = knew[i]; vd[c][i] = vnew[i]; }
+        for (int i = 0; i < DS; i++) { ch.k[c][i] = knew[i]; ch.v[c][i] = vnew[i]; }
+        if (I8) { ch.ks[c] = knew_s; ch.vs[c] = vnew_s; }
       }
       float s = 0.0f;
 #pragma unroll
-      for (int i = 0; i < DS; i++) s = fmaf(q[i], kd[c][i], s);
-      s = half_wave_allsum(s) * p.inv_sqrt;
+      for (int i = 0; i < DS; i++) s = fmaf(q[i], ch.k[c][i], s);
+      s = half_wave_allsum(s) * (I8 ? ch.ks[c] * p.inv_sqrt : p.inv_sqrt);
       if (p.softcap > 0.0f) s = p.softcap * tanhf(s / p.softcap);
       sc[c] = (j0 + 8 * c < s_end) ? s : -1e30f;
       cmax = fmaxf(cmax, sc[c]);
@@ -388,17 +457,18 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
     for (int c = 0; c < PCH; c++) {
       const float pj = (j0 + 8 * c < s_end) ? expf(sc[c] - mn) : 0.0f;
       lsum += pj;
+      const float pv = I8 ? pj * ch.vs[c] : pj;
 #pragma unroll
-      for (int i = 0; i < DS; i++) acc[i] = fmaf(pj, vd[c][i], acc[i]);
+      for (int i = 0; i < DS; i++) acc[i] = fmaf(pv, ch.v[c][i], acc[i]);
     }
     l = l * corr + lsum; m = mn;
   };
   for (int j0 = s_begin + hw; j0 < s_end; j0 += 16 * PCH) {
-    reduce_chunk(kdA, vdA, j0);
-    if (j0 + 16 * PCH < s_end) load_chunk(kdA, vdA, j0 + 16 * PCH);
+    reduce_chunk(cA, j0);
+    if (j0 + 16 * PCH < s_end) load_chunk(cA, j0 + 16 * PCH);
     if (j0 + 8 * PCH < s_end) {
-      reduce_chunk(kdB, vdB, j0 + 8 * PCH);
-      if (j0 + 24 * PCH < s_end) load_chunk(kdB, vdB, j0 + 24 * PCH);
+      reduce_chunk(cB, j0 + 8 * PCH);
+      if (j0 + 24 * PCH < s_end) load_chunk(cB, j0 + 24 * PCH);
     }
   }
 
@@ -486,6 +556,49 @@ __global__ __launch_bounds__(256) void kv_append_rows_kernel(const AttnParams p)
   }
 }
 
+// The same for an int8 cache: one half-wave per (token, KV head, K|V) row, quantised with the decode step's rule.
+template <int DS>
+__global__ __launch_bounds__(256) void kv_append_rows_i8_kernel(const AttnParams p)
+{
+  const int b = blockIdx.x, hw = threadIdx.x >> 5, l32 = threadIdx.x & 31;
+  const float* row = p.qkv + (int64_t)b * p.qkv_stride;
+  const int pos = p.pos[b];
+  const int hd = p.hd, qw = p.q_heads * hd, kw = p.kv_heads * hd;
+  const int d0 = l32 * DS;
+  for (int item = hw; item < 2 * p.kv_heads; item += 8) {      // uniform per half-wave; both halves of a wave loop alike
+    const int g = item >> 1, is_v = item & 1;
+    const float* src = row + qw + (is_v ? kw : 0) + g * hd;
+    float v[DS];
+    if (DS >= 2) {
+#pragma unroll
+      for (int i = 0; i < DS; i += 2) {
+        const int d = d0 + i;
+        float x0 = d < hd ? src[d] : 0.0f, x1 = d + 1 < hd ? src[d + 1] : 0.0f;
+        if (p.theta && !is_v && d < hd) {
+          float sn, cs; sincosf((float)pos * p.theta[d >> 1], &sn, &cs);
+          const float y0 = cs * x0 - sn * x1, y1 = sn * x0 + cs * x1;
+          x0 = y0; x1 = y1;
+        }
+        v[i] = x0; v[i + (DS > 1 ? 1 : 0)] = x1;
+      }
+    } else {
+      const int d = d0;
+      const float own = d < hd ? src[d] : 0.0f, mate = (d ^ 1) < hd ? src[d ^ 1] : 0.0f;
+      v[0] = own;
+      if (p.theta && !is_v && d < hd) {
+        float sn, cs; sincosf((float)pos * p.theta[d >> 1], &sn, &cs);
+        v[0] = (d & 1) ? (sn * mate + cs * own) : (cs * own - sn * mate);
+      }
+    }
+    const float scale = quantise_row_i8<DS>(v);
+    const int64_t slot = (int64_t)p.seq0 * p.seq_rows + p.layer_row_off + (int64_t)g * p.max_ctx + pos;
+    int8_t* dst = reinterpret_cast<int8_t*>(is_v ? p.vc : p.kc) + (int64_t)p.seq0 * p.seq_elems + p.layer_off + ((int64_t)g * p.max_ctx + pos) * hd;
+#pragma unroll
+    for (int i = 0; i < DS; i++) if (d0 + i < hd) dst[d0 + i] = (int8_t)v[i];
+    if (l32 == 0) (is_v ? p.vsc : p.ksc)[slot] = scale;
+  }
+}
+
 int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, int n_seq, int q_heads, int window,
                      float softcap, const float* theta, const int32_t* pos_dev, float* out, int64_t out_stride, int seq0,
                      int prompt_rows, float* prompt_part)
@@ -503,13 +616,20 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   p.theta = theta; p.pos = pos_dev; p.split_len = kv->split_len; p.n_splits = kv->n_splits;
   p.part = prompt_rows ? prompt_part : kv->part; p.out = out; p.out_stride = out_stride; p.seq0 = seq0;
   p.seq_mul = prompt_rows ? 0 : 1; p.appended = prompt_rows ? 1 : 0;
-  if (prompt_rows) {
+  p.ksc = kv->ks; p.vsc = kv->vs; p.seq_rows = kv->seq_rows(); p.layer_row_off = (int64_t)layer * kv->layer_rows();
+  if (prompt_rows && kv->dtype == CAI_KV_I8) {
+    if (p.hd <= 32) hipLaunchKernelGGL(kv_append_rows_i8_kernel<1>, dim3(n_seq), dim3(256), 0, c.stream, p);
+    else if (p.hd <= 64) hipLaunchKernelGGL(kv_append_rows_i8_kernel<2>, dim3(n_seq), dim3(256), 0, c.stream, p);
+    else hipLaunchKernelGGL(kv_append_rows_i8_kernel<4>, dim3(n_seq), dim3(256), 0, c.stream, p);
+  } else if (prompt_rows) {
     if (kv->dtype == CAI_KV_F16) hipLaunchKernelGGL(kv_append_rows_kernel<__half>, dim3(n_seq), dim3(256), 0, c.stream, p);
     else hipLaunchKernelGGL(kv_append_rows_kernel<float>, dim3(n_seq), dim3(256), 0, c.stream, p);
   }
   p.counters = kv->d_counters;
   int rc;
-  if (kv->max_ctx <= kv->short_ctx_limit)   // short caches: per-head work-groups (K,V re-read from L2 by the group's heads)
+  if (kv->dtype == CAI_KV_I8)
+    rc = launch_split_head<int8_t>(p, n_seq, c.stream);
+  else if (kv->max_ctx <= kv->short_ctx_limit)   // short caches: per-head work-groups (K,V re-read from L2 by the group's heads)
     rc = kv->dtype == CAI_KV_F16 ? launch_split_head<__half>(p, n_seq, c.stream) : launch_split_head<float>(p, n_seq, c.stream);
   else
     rc = kv->dtype == CAI_KV_F16 ? launch_split_g<__half>(p, n_seq, c.stream) : launch_split_g<float>(p, n_seq, c.stream);
@@ -525,7 +645,7 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
 {
   if (n_seq < 1 || n_layers < 1 || kv_heads < 1 || head_dim < 2 || (head_dim & 1) || (head_dim > 64 && (head_dim & 3)) || head_dim > 128 || max_ctx < 1)
     return set_error(CAI_ERR_INVALID, "kv cache: bad geometry seq=%d layers=%d kv_heads=%d head_dim=%d max_ctx=%d", n_seq, n_layers, kv_heads, head_dim, max_ctx);
-  if (dtype != CAI_KV_F32 && dtype != CAI_KV_F16) return set_error(CAI_ERR_INVALID, "kv cache: dtype %d", dtype);
+  if (dtype != CAI_KV_F32 && dtype != CAI_KV_F16 && dtype != CAI_KV_I8) return set_error(CAI_ERR_INVALID, "kv cache: dtype %d", dtype);
   kv->n_seq = n_seq; kv->n_layers = n_layers; kv->kv_heads = kv_heads; kv->head_dim = head_dim; kv->max_ctx = max_ctx; kv->dtype = dtype;
   kv->len.assign((size_t)n_seq * n_layers, 0);
   // few, fat splits: every extra split costs the merging work-group another device-coherent load round,
@@ -539,6 +659,13 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   CAI_HIP(hipMalloc(&kv->v, bytes));
   CAI_HIP(hipMemsetAsync(kv->k, 0, bytes, ctx().stream));
   CAI_HIP(hipMemsetAsync(kv->v, 0, bytes, ctx().stream));
+  if (dtype == CAI_KV_I8) {
+    const size_t sb = (size_t)kv->seq_rows() * n_seq * sizeof(float);
+    CAI_HIP(hipMalloc(&kv->ks, sb));
+    CAI_HIP(hipMalloc(&kv->vs, sb));
+    CAI_HIP(hipMemsetAsync(kv->ks, 0, sb, ctx().stream));
+    CAI_HIP(hipMemsetAsync(kv->vs, 0, sb, ctx().stream));
+  }
   {
     const char* e = getenv("CAIHIP_ATTN_SHORT_CTX");      // caches up to this capacity use the per-head split kernel
     kv->short_ctx_limit = e ? atoi(e) : (1 << 30);
@@ -556,6 +683,9 @@ void kv_free(cai_kv_s* kv)
 {
   if (kv->k) (void)hipFree(kv->k);
   if (kv->v) (void)hipFree(kv->v);
+  if (kv->ks) (void)hipFree(kv->ks);
+  if (kv->vs) (void)hipFree(kv->vs);
+  kv->ks = kv->vs = nullptr;
   if (kv->part) (void)hipFree(kv->part);
   if (kv->d_len) (void)hipFree(kv->d_len);
   if (kv->d_counters) (void)hipFree(kv->d_counters);
@@ -586,6 +716,16 @@ int kv_snapshot(cai_kv_s* kv, int seq, cai_kv_snap_s** out)
       CAI_HIP(hipMemcpy2DAsync(dst, (size_t)rows * row_b, src, (size_t)kv->max_ctx * row_b, (size_t)rows * row_b,
                                (size_t)kv->n_layers * kv->kv_heads, hipMemcpyDeviceToDevice, ctx().stream));
     }
+    if (kv->dtype == CAI_KV_I8) {     // the row scales travel with the codes
+      const size_t sb = (size_t)kv->n_layers * kv->kv_heads * rows * sizeof(float);
+      if (hipMalloc(&s->ks, sb) != hipSuccess || hipMalloc(&s->vs, sb) != hipSuccess) {
+        (void)hipFree(s->k); (void)hipFree(s->v); if (s->ks) (void)hipFree(s->ks);
+        delete s; return set_error(CAI_ERR_NOMEM, "kv snapshot: out of device memory (%zu bytes)", 2 * sb);
+      }
+      for (int which = 0; which < 2; which++)
+        CAI_HIP(hipMemcpy2DAsync(which ? s->vs : s->ks, (size_t)rows * 4, (which ? kv->vs : kv->ks) + (size_t)seq * kv->seq_rows(), (size_t)kv->max_ctx * 4,
+                                 (size_t)rows * 4, (size_t)kv->n_layers * kv->kv_heads, hipMemcpyDeviceToDevice, ctx().stream));
+    }
     CAI_HIP(hipStreamSynchronize(ctx().stream));
   }
   *out = s;
@@ -606,6 +746,10 @@ int kv_restore(cai_kv_s* kv, int seq, const cai_kv_snap_s* s)
       CAI_HIP(hipMemcpy2DAsync(dst, (size_t)kv->max_ctx * row_b, src, (size_t)s->rows * row_b, (size_t)s->rows * row_b,
                                (size_t)kv->n_layers * kv->kv_heads, hipMemcpyDeviceToDevice, ctx().stream));
     }
+    if (kv->dtype == CAI_KV_I8)
+      for (int which = 0; which < 2; which++)
+        CAI_HIP(hipMemcpy2DAsync((which ? kv->vs : kv->ks) + (size_t)seq * kv->seq_rows(), (size_t)kv->max_ctx * 4, which ? s->vs : s->ks, (size_t)s->rows * 4,
+                                 (size_t)s->rows * 4, (size_t)kv->n_layers * kv->kv_heads, hipMemcpyDeviceToDevice, ctx().stream));
     CAI_HIP(hipStreamSynchronize(ctx().stream));
   }
   for (int l = 0; l < kv->n_layers; l++) kv->len_at(seq, l) = s->len[l];
@@ -680,7 +824,51 @@ extern "C" int cai_kv_snap_destroy(cai_kv_snap_t s)
   if (!s) return CAI_OK;
   if (s->k) (void)hipFree(s->k);
   if (s->v) (void)hipFree(s->v);
+  if (s->ks) (void)hipFree(s->ks);
+  if (s->vs) (void)hipFree(s->vs);
   delete s;
+  return CAI_OK;
+}
+
+// one layer of sequence 0 <-> packed host rows; dir 0 = device to host
+static int kv_layer_copy(cai_kv_s* kv, int layer, int len, void* k, void* v, float* ks, float* vs, int to_device)
+{
+  if (len == 0) return CAI_OK;
+  const size_t row_b = (size_t)kv->head_dim * kv->elem();
+  const hipMemcpyKind kind = to_device ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost;
+  auto copy2d = [&](char* dev, char* host, size_t unit) -> hipError_t {
+    return to_device ? hipMemcpy2DAsync(dev, (size_t)kv->max_ctx * unit, host, (size_t)len * unit, (size_t)len * unit, (size_t)kv->kv_heads, kind, ctx().stream)
+                     : hipMemcpy2DAsync(host, (size_t)len * unit, dev, (size_t)kv->max_ctx * unit, (size_t)len * unit, (size_t)kv->kv_heads, kind, ctx().stream);
+  };
+  CAI_HIP(copy2d((char*)kv->k + (size_t)layer * kv->layer_elems() * kv->elem(), (char*)k, row_b));
+  CAI_HIP(copy2d((char*)kv->v + (size_t)layer * kv->layer_elems() * kv->elem(), (char*)v, row_b));
+  if (kv->dtype == CAI_KV_I8) {
+    CAI_HIP(copy2d((char*)(kv->ks + (size_t)layer * kv->layer_rows()), (char*)ks, 4));
+    CAI_HIP(copy2d((char*)(kv->vs + (size_t)layer * kv->layer_rows()), (char*)vs, 4));
+  }
+  CAI_HIP(hipStreamSynchronize(ctx().stream));
+  return CAI_OK;
+}
+
+extern "C" int cai_kv_export_layer(cai_kv_t kv, int layer, void* k, void* v, float* k_scales, float* v_scales)
+{
+  CAI_READY();
+  CAI_REQUIRE(kv && k && v, "cai_kv_export_layer: null argument");
+  CAI_REQUIRE(layer >= 0 && layer < kv->n_layers, "cai_kv_export_layer: layer %d of %d", layer, kv->n_layers);
+  CAI_REQUIRE(kv->dtype != CAI_KV_I8 || (k_scales && v_scales), "cai_kv_export_layer: an int8 cache needs the scale outputs");
+  return kv_layer_copy(kv, layer, kv->len_at(0, layer), k, v, k_scales, v_scales, 0);
+}
+
+extern "C" int cai_kv_import_layer(cai_kv_t kv, int layer, int len, const void* k, const void* v, const float* k_scales, const float* v_scales)
+{
+  CAI_READY();
+  CAI_REQUIRE(kv && (len == 0 || (k && v)), "cai_kv_import_layer: null argument");
+  CAI_REQUIRE(layer >= 0 && layer < kv->n_layers, "cai_kv_import_layer: layer %d of %d", layer, kv->n_layers);
+  CAI_REQUIRE(len >= 0 && len <= kv->max_ctx, "cai_kv_import_layer: %d rows, cache holds %d", len, kv->max_ctx);
+  CAI_REQUIRE(kv->dtype != CAI_KV_I8 || len == 0 || (k_scales && v_scales), "cai_kv_import_layer: an int8 cache needs the row scales");
+  const int rc = kv_layer_copy(kv, layer, len, const_cast<void*>(k), const_cast<void*>(v), const_cast<float*>(k_scales), const_cast<float*>(v_scales), 1);
+  if (rc) return rc;
+  kv->len_at(0, layer) = len;
   return CAI_OK;
 }
 

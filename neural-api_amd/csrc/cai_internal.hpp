@@ -70,6 +70,7 @@ struct cai_qw_s {
 struct cai_kv_s {
   int n_seq = 1, n_layers = 0, kv_heads = 0, head_dim = 0, max_ctx = 0, dtype = 0;
   void* k = nullptr; void* v = nullptr;   // [seq][layer][kv_head][max_ctx][head_dim]
+  float* ks = nullptr; float* vs = nullptr;   // CAI_KV_I8 only: one scale per cached row, [seq][layer][kv_head][max_ctx]
   std::vector<int> len;                   // [seq][layer] live rows (host mirror)
   int split_len = 64, n_splits = 1;       // split-K geometry of the decode kernel (fixed at creation)
   int short_ctx_limit = 0;                // caches up to this capacity use the per-query-head split kernel
@@ -77,7 +78,9 @@ struct cai_kv_s {
   int part_q_heads = 0;
   int32_t* d_len = nullptr;               // [seq] device scratch: rows live BEFORE the token being decoded
   int* d_counters = nullptr;              // [seq][kv_head] split-merge arrival counters
-  size_t elem() const { return dtype == CAI_KV_F16 ? 2 : 4; }
+  size_t elem() const { return dtype == CAI_KV_F16 ? 2 : dtype == CAI_KV_I8 ? 1 : 4; }
+  int64_t layer_rows() const { return (int64_t)kv_heads * max_ctx; }
+  int64_t seq_rows() const { return layer_rows() * n_layers; }
   int64_t layer_elems() const { return (int64_t)kv_heads * max_ctx * head_dim; }
   int64_t seq_elems() const { return layer_elems() * n_layers; }
   int& len_at(int seq, int layer) { return len[(size_t)seq * n_layers + layer]; }
@@ -87,6 +90,7 @@ struct cai_kv_snap_s {
   int n_layers = 0, kv_heads = 0, head_dim = 0, dtype = 0, rows = 0;
   std::vector<int> len;                   // per layer
   void* k = nullptr; void* v = nullptr;   // [layer][kv_head][rows][head_dim]
+  float* ks = nullptr; float* vs = nullptr;   // [layer][kv_head][rows] row scales of an int8 cache
 };
 
 namespace cai {

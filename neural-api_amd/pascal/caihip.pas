@@ -24,7 +24,7 @@ const
   // fused activation opcodes = csAct* of the OpenCL kernels (neural/neural.cl:114-146)
   CAI_ACT_NONE = 0; CAI_ACT_RELU = 1; CAI_ACT_SIGMOID = 2; CAI_ACT_TANH = 3;
   CAI_X_DEVICE = 1; CAI_Y_DEVICE = 2;
-  CAI_KV_F32 = 0; CAI_KV_F16 = 1;
+  CAI_KV_F32 = 0; CAI_KV_F16 = 1; CAI_KV_I8 = 2;
   CAI_W_EMBED = 0; CAI_W_HEAD = 1; CAI_W_Q = 2; CAI_W_K = 3; CAI_W_V = 4; CAI_W_O = 5;
   CAI_W_GATEUP = 6; CAI_W_DOWN = 7; CAI_W_ROUTER = 8;
   CAI_V_ATTN_NORM = 0; CAI_V_MLP_NORM = 1; CAI_V_FINAL_NORM = 2; CAI_V_Q_NORM = 3; CAI_V_K_NORM = 4;
@@ -77,6 +77,8 @@ function cai_kv_len(kv: TCaiKV; layer: LongInt; len_out: PLongInt): LongInt; cde
 function cai_kv_snapshot(kv: TCaiKV; out_snap: PCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;
 function cai_kv_restore(kv: TCaiKV; snap: TCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;
 function cai_kv_snap_destroy(snap: TCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;
+function cai_kv_export_layer(kv: TCaiKV; layer: LongInt; k, v: Pointer; k_scales, v_scales: PSingle): LongInt; cdecl; external CAIHIP_LIB;
+function cai_kv_import_layer(kv: TCaiKV; layer, len: LongInt; k, v: Pointer; k_scales, v_scales: PSingle): LongInt; cdecl; external CAIHIP_LIB;
 function cai_attn_decode(kv: TCaiKV; layer: LongInt; qkv: PSingle; q_heads, window: LongInt; softcap: Single; out_f: PSingle; flags: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 
 function cai_decoder_create(cfg: PCaiDecoderConfig; out_d: PCaiDecoder): LongInt; cdecl; external CAIHIP_LIB;

@@ -499,7 +499,7 @@ void orc_attn_decode(const float* qkv, int hq, int hkv, int dk, float* kc, float
   for (int g = 0; g < hkv; g++)
     for (int d = 0; d < dk; d++) {
       float k = qkv[qw + g * dk + d], v = qkv[qw + kw + g * dk + d];
-      if (kv_f16) { k = round_half(k); v = round_half(v); }
+      if (kv_f16 == 1) { k = round_half(k); v = round_half(v); }
       kc[((int64_t)g * max_ctx + cache_len) * dk + d] = k;
       vc[((int64_t)g * max_ctx + cache_len) * dk + d] = v;
     }
@@ -531,6 +531,84 @@ void orc_attn_decode(const float* qkv, int hq, int hkv, int dk, float* kc, float
   free(sc);
 }
 
+/* neural.cl:2501-2580 (cai_sdpa_append_kv_int8), the device statement of the host's
+ * QuantizeCacheRow: max over FINITE magnitudes (neuralvolume.pas:12471 MaxAbsFinite), a row whose
+ * maximum is zero or denormal gets zero codes and unit scale, scale = max/127,
+ * code = clamp(rint(v * (1/max) * 127)) with NaN -> 0 and +/-Inf -> +/-127.
+ * Pinned by: the zero / one-outlier / flat / exact-midpoint rows of
+ * tests/TestNeuralNumerical.pas:69740-69800 and the MaxAbsFinite cases of
+ * tests/TestNeuralVolume.pas:2864-2903 (tests/test_oracle_kv_int8.py). */
+float orc_max_abs_finite(const float* x, int n)
+{
+  float m = 0.0f;
+  for (int i = 0; i < n; i++) {
+    float a = fabsf(x[i]); uint32_t b; memcpy(&b, &a, 4);
+    if (b <= 0x7F7FFFFFu && a > m) m = a;
+  }
+  return m;
+}
+
+void orc_kv_quant_row(const float* x, int n, int8_t* codes, float* scale)
+{
+  const float mx = orc_max_abs_finite(x, n);
+  uint32_t mb; memcpy(&mb, &mx, 4);
+  const int usable = mb >= 0x00800000u;
+  const float recip = usable ? 1.0f / mx : 0.0f;
+  *scale = usable ? mx / 127.0f : 1.0f;
+  for (int i = 0; i < n; i++) {
+    float a = fabsf(x[i]); uint32_t b; memcpy(&b, &a, 4);
+    float scaled = x[i] * recip * 127.0f;
+    if (b > 0x7F800000u || !usable) scaled = 0.0f;   /* an unusable row is all zero codes (neuralvolume.pas:725) */
+    float r = rintf(scaled);                 /* half-to-even under the default rounding mode */
+    if (r < -127.0f) r = -127.0f;
+    if (r > 127.0f) r = 127.0f;
+    codes[i] = (int8_t)r;
+  }
+}
+
+/* neural.cl:2582-2687 (cai_sdpa_decode_int8): same phases as the fp32 kernel; the K row scale
+ * multiplies the finished dot product together with 1/sqrt(dk), the V row scale multiplies the
+ * softmax weight, the codes enter the accumulators as integers-in-float.
+ * Pinned by: agreement with orc_attn_decode on caches whose rows quantise exactly
+ * (tests/test_oracle_kv_int8.py), plus orc_kv_quant_row's vectors for the append. */
+void orc_attn_decode_i8(const float* qkv, int hq, int hkv, int dk, int8_t* kq, float* ks, int8_t* vq, float* vs,
+                        int max_ctx, int cache_len, int window, float softcap, float* out)
+{
+  const int qw = hq * dk, kw = hkv * dk, group = hq / hkv;
+  for (int g = 0; g < hkv; g++) {
+    const int64_t slot = (int64_t)g * max_ctx + cache_len;
+    orc_kv_quant_row(qkv + qw + g * dk, dk, kq + slot * dk, ks + slot);
+    orc_kv_quant_row(qkv + qw + kw + g * dk, dk, vq + slot * dk, vs + slot);
+  }
+  const int len = cache_len + 1;
+  const int j0 = (window > 0 && len > window) ? len - window : 0;
+  const float inv_sqrt = 1.0f / sqrtf((float)dk);
+  float* sc = (float*)malloc((size_t)len * sizeof(float));
+  for (int h = 0; h < hq; h++) {
+    const int g = h / group;
+    const float* q = qkv + h * dk;
+    float m = -1e30f;
+    for (int j = j0; j < len; j++) {
+      const int8_t* kr = kq + ((int64_t)g * max_ctx + j) * dk;
+      float acc = 0;
+      for (int d = 0; d < dk; d++) acc = fmaf(q[d], (float)kr[d], acc);
+      float s = acc * (ks[(int64_t)g * max_ctx + j] * inv_sqrt);
+      if (softcap > 0) s = softcap * tanhf(s / softcap);
+      sc[j] = s; if (s > m) m = s;
+    }
+    float sum = 0;
+    for (int j = j0; j < len; j++) { sc[j] = expf(sc[j] - m); sum += sc[j]; }
+    const float inv = sum > 0 ? 1.0f / sum : 0;
+    for (int d = 0; d < dk; d++) {
+      float acc = 0;
+      for (int j = j0; j < len; j++)
+        acc = fmaf(sc[j] * vs[(int64_t)g * max_ctx + j], (float)vq[((int64_t)g * max_ctx + j) * dk + d], acc);
+      out[h * dk + d] = acc * inv;
+    }
+  }
+  free(sc);
+}
+
 /* ------------------------------------------------------------------ */
 /* whole decoder                                                       */
 /* ------------------------------------------------------------------ */
@@ -541,6 +619,7 @@ typedef struct {
   orc_tensor w[9];
   const float* v[5];
   float *kc, *vc;
+  int8_t *kq, *vq; float *ks, *vs;   /* int8 cache mode */
 } orc_layer;
 
 struct orc_model {
@@ -563,6 +642,10 @@ orc_model* orc_model_new(const orc_config* cfg)
   for (int l = 0; l < L; l++) {
     m->layers[l].kc = (float*)calloc((size_t)kw * cfg->max_ctx, sizeof(float));
     m->layers[l].vc = (float*)calloc((size_t)kw * cfg->max_ctx, sizeof(float));
+    if (cfg->kv_f16 == 2) {
+      m->layers[l].kq = (int8_t*)calloc((size_t)kw * cfg->max_ctx, 1); m->layers[l].vq = (int8_t*)calloc((size_t)kw * cfg->max_ctx, 1);
+      m->layers[l].ks = (float*)calloc((size_t)cfg->n_kv_heads * cfg->max_ctx, 4); m->layers[l].vs = (float*)calloc((size_t)cfg->n_kv_heads * cfg->max_ctx, 4);
+    }
   }
   m->theta = (float*)malloc(sizeof(float) * (size_t)(cfg->head_dim / 2));
   orc_rope_thetas(cfg->rope_theta, cfg->head_dim, m->theta);
@@ -580,7 +663,7 @@ orc_model* orc_model_new(const orc_config* cfg)
 void orc_model_free(orc_model* m)
 {
   if (!m) return;
-  for (int l = 0; l < m->cfg.n_layers; l++) { free(m->layers[l].kc); free(m->layers[l].vc); }
+  for (int l = 0; l < m->cfg.n_layers; l++) { orc_layer* y = &m->layers[l]; free(y->kc); free(y->vc); free(y->kq); free(y->vq); free(y->ks); free(y->vs); }
   free(m->layers); free(m->theta); free(m->x); free(m->h); free(m->qkv); free(m->att); free(m->gu); free(m->mid);
   free(m->tmp); free(m->probs); free(m->gates); free(m->sel); free(m->logits); free(m);
 }
@@ -647,7 +730,8 @@ int orc_model_step(orc_model* m, int token, int pos, float* logits)
     }
     orc_rope_interleaved(m->qkv, c->n_q_heads, hd, pos, m->theta);
     orc_rope_interleaved(m->qkv + qw, c->n_kv_heads, hd, pos, m->theta);
-    orc_attn_decode(m->qkv, c->n_q_heads, c->n_kv_heads, hd, ly->kc, ly->vc, c->max_ctx, pos, c->window, 0.0f, c->kv_f16, m->att);
+    if (c->kv_f16 == 2) orc_attn_decode_i8(m->qkv, c->n_q_heads, c->n_kv_heads, hd, ly->kq, ly->ks, ly->vq, ly->vs, c->max_ctx, pos, c->window, 0.0f, m->att);
+    else orc_attn_decode(m->qkv, c->n_q_heads, c->n_kv_heads, hd, ly->kc, ly->vc, c->max_ctx, pos, c->window, 0.0f, c->kv_f16, m->att);
     lin(m, &ly->w[ORC_W_O], 0, d, m->att, m->tmp);
     for (int i = 0; i < d; i++) m->x[i] += m->tmp[i];
     orc_rmsnorm(m->x, ly->v[ORC_V_MLP_NORM], d, c->eps, m->h);

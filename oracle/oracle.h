@@ -73,10 +73,18 @@ int  orc_argmax(const float* x, int n);                                         
 /* ---- cached GQA decode attention, fp32, head-major cache (neural.cl:2354-2499) ----
  * k_cache/v_cache: [kv_heads][max_ctx][head_dim]; qkv row = [Q | K | V]. Appends at slot
  * cache_len, then attends over [j_start .. cache_len] where window>0 limits the range.
- * kv_f16 != 0 rounds the appended K,V through IEEE half first (fp16 cache model). */
+ * kv_f16 == 1 rounds the appended K,V through IEEE half first (fp16 cache model). */
 void orc_attn_decode(const float* qkv, int q_heads, int kv_heads, int head_dim,
                      float* k_cache, float* v_cache, int max_ctx, int cache_len,
                      int window, float softcap, int kv_f16, float* out);
+
+/* ---- int8 KV cache: per-row symmetric codes + fp32 scale (neural.cl:2501-2687) ----
+ * codes [kv_heads][max_ctx][head_dim], scales [kv_heads][max_ctx]. */
+float orc_max_abs_finite(const float* x, int n);                                     /* neuralvolume.pas:12471 */
+void orc_kv_quant_row(const float* x, int n, int8_t* codes, float* scale);           /* neural.cl:2549-2578 */
+void orc_attn_decode_i8(const float* qkv, int q_heads, int kv_heads, int head_dim,
+                        int8_t* k_codes, float* k_scales, int8_t* v_codes, float* v_scales,
+                        int max_ctx, int cache_len, int window, float softcap, float* out);
 
 /* ---- whole decoder (Llama / Qwen2 / OLMoE families), one token at a time ---- */
 typedef struct orc_model orc_model;
@@ -87,7 +95,7 @@ typedef struct {
   int32_t window;         /* sliding window (0 = none) */
   int32_t qk_norm_full;   /* OLMoE: RMSNorm over full q / k width before RoPE */
   int32_t n_experts, top_k, norm_topk; /* n_experts == 0 -> dense SwiGLU FFN */
-  int32_t kv_f16;         /* store K,V rounded to half */
+  int32_t kv_f16;         /* cache element model: 0 fp32, 1 rounded to half, 2 int8 codes + row scale */
   int32_t acc64;          /* accumulate linear layers in double */
 } orc_config;
 

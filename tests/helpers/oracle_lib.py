@@ -51,6 +51,10 @@ def lib():
         L.orc_q4k_scale_min.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]; L.orc_q4k_scale_min.restype = None
         L.orc_attn_decode.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int, C.c_void_p]
         L.orc_attn_decode.restype = None
+        L.orc_max_abs_finite.restype = C.c_float; L.orc_max_abs_finite.argtypes = [C.c_void_p, C.c_int]
+        L.orc_kv_quant_row.restype = None; L.orc_kv_quant_row.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+        L.orc_attn_decode_i8.restype = None
+        L.orc_attn_decode_i8.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_void_p]
         L.orc_model_new.restype = C.c_void_p; L.orc_model_new.argtypes = [C.POINTER(OrcConfig)]
         L.orc_model_free.argtypes = [C.c_void_p]; L.orc_model_free.restype = None
         L.orc_model_set_tensor.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]

@@ -99,3 +99,122 @@ def test_cache_full_is_an_error_not_a_fault():
     with pytest.raises(cai.CaiError) as e:
         kv.attn_decode(0, row, 1)
     assert e.value.code == -5
+
+
+def oracle_run_i8(rows, hq, hkv, dk, ctx, window=0, softcap=0.0):
+    kq = np.zeros((hkv, ctx, dk), np.int8); vq = np.zeros_like(kq)
+    ks = np.zeros((hkv, ctx), np.float32); vs = np.zeros_like(ks)
+    outs = []
+    for pos in range(rows.shape[0]):
+        out = np.zeros(hq * dk, np.float32)
+        O.lib().orc_attn_decode_i8(rows[pos].ctypes.data, hq, hkv, dk, kq.ctypes.data, ks.ctypes.data, vq.ctypes.data, vs.ctypes.data,
+                                   ctx, pos, window, softcap, out.ctypes.data)
+        outs.append(out)
+    n = rows.shape[0]
+    return np.array(outs), (kq[:, :n], vq[:, :n], ks[:, :n], vs[:, :n])
+
+
+def stress_rows(rng, n, hq, hkv, dk):
+    """Random rows, with the quantiser stress rows of the reference's append test in the K and V slices of the first
+    steps (tests/TestNeuralNumerical.pas:69760-69800): all zeros, one outlier, flat, exact midpoints."""
+    rows = rng.standard_normal((n, (hq + 2 * hkv) * dk)).astype(np.float32)
+    kv = rows[:, hq * dk:].reshape(n, 2 * hkv, dk)
+    kv[1] = 0
+    kv[2] = 1e-4; kv[2, :, 0] = 100
+    kv[3] = 0.75
+    mid = np.full(dk, 0.5, np.float32); mid[dk - 1] = 1; d = 0
+    for cand in range(127):
+        v = np.float32(cand + 0.5) / np.float32(127)
+        if d < dk - 1 and np.float32(v * np.float32(127)) == np.float32(cand + 0.5):
+            mid[d] = v; d += 1
+    kv[4] = mid; kv[5] = -mid
+    return rows
+
+
+@pytest.mark.parametrize("hq,hkv,dk", [(2, 1, 4), (9, 3, 64), (28, 4, 128), (16, 16, 128), (8, 1, 32), (6, 2, 80)])
+@pytest.mark.parametrize("window", [0, 5])
+def test_int8_cache_codes_bit_exact_and_decode_matches_oracle(hq, hkv, dk, window):
+    """neural/neural.cl:2501-2687: the appended codes and row scales equal the oracle's bit for bit (the reference's own
+    OpenCL-vs-host test allows one step / one ulp); outputs within 1e-5 (the reference allows 1e-3)."""
+    from helpers.device import dev
+    cai = dev()
+    rng = np.random.default_rng(hq * 100 + dk + 7)
+    n, ctx = 45, 80
+    rows = stress_rows(rng, n, hq, hkv, dk)
+    want, (kq, vq, ks, vs) = oracle_run_i8(rows, hq, hkv, dk, ctx, window)
+    kv = cai.KVCache(2, hkv, dk, ctx, cai.KV_I8)
+    for pos in range(n):
+        got = kv.attn_decode(1, rows[pos], hq, window)
+        assert np.max(np.abs(got - want[pos])) < 1e-5 * max(1.0, np.max(np.abs(want[pos]))), pos
+    k, v, s_k, s_v = kv.export_layer(1)
+    np.testing.assert_array_equal(k, kq); np.testing.assert_array_equal(v, vq)
+    np.testing.assert_array_equal(s_k.view(np.uint32), ks.view(np.uint32))
+    np.testing.assert_array_equal(s_v.view(np.uint32), vs.view(np.uint32))
+    assert kv.len(0) == 0 and kv.export_layer(0)[0].shape == (hkv, 0, dk)
+
+
+def test_int8_cache_long_context_softcap_and_non_finite_rows():
+    from helpers.device import dev
+    cai = dev()
+    rng = np.random.default_rng(21)
+    hq, hkv, dk, n, ctx = 10, 2, 128, 600, 4096
+    rows = rng.standard_normal((n, (hq + 2 * hkv) * dk)).astype(np.float32)
+    want, (kq, vq, ks, vs) = oracle_run_i8(rows, hq, hkv, dk, ctx, 0, 20.0)
+    kv = cai.KVCache(1, hkv, dk, ctx, cai.KV_I8)
+    for pos in range(n):
+        got = kv.attn_decode(0, rows[pos], hq, 0, 20.0)
+        if pos % 97 == 0 or pos == n - 1:
+            assert np.max(np.abs(got - want[pos])) < 1e-5, pos
+    k, v, s_k, s_v = kv.export_layer(0)
+    np.testing.assert_array_equal(k, kq); np.testing.assert_array_equal(v, vq)
+    np.testing.assert_array_equal(s_k, ks); np.testing.assert_array_equal(s_v, vs)
+    # NaN -> code 0, +/-Inf -> +/-127, neither enters the row maximum; a denormal row is unusable (unit scale, zero codes)
+    kv2 = cai.KVCache(1, 1, 32, 8, cai.KV_I8)
+    row = np.zeros(3 * 32, np.float32); row[:32] = 0.1
+    row[32:64] = np.linspace(-1, 1, 32); row[33] = np.nan; row[34] = np.inf; row[35] = -np.inf
+    row[64:] = 1e-41
+    kv2.attn_decode(0, row, 1)
+    k, v, s_k, s_v = kv2.export_layer(0)
+    codes = np.zeros(32, np.int8); sc = np.zeros(1, np.float32)
+    kr = np.ascontiguousarray(row[32:64])
+    O.lib().orc_kv_quant_row(kr.ctypes.data, 32, codes.ctypes.data, sc.ctypes.data)
+    np.testing.assert_array_equal(k[0, 0], codes)
+    assert k[0, 0, 1] == 0 and k[0, 0, 2] == 127 and k[0, 0, 3] == -127 and s_k[0, 0] == sc[0] == np.float32(1) / np.float32(127)
+    assert not v.any() and s_v[0, 0] == 1.0
+
+
+def test_int8_cache_snapshot_restore_and_layer_import_export():
+    from helpers.device import dev
+    cai = dev()
+    rng = np.random.default_rng(33)
+    hq, hkv, dk, n = 6, 2, 64, 40
+    rows = rng.standard_normal((n, (hq + 2 * hkv) * dk)).astype(np.float32)
+    kv = cai.KVCache(2, hkv, dk, 64, cai.KV_I8)
+    first = [kv.attn_decode(1, rows[p], hq) for p in range(n)]
+    kv.truncate(10); snap = kv.snapshot()
+    for p in range(5):
+        kv.attn_decode(1, rows[30 + p], hq)
+    kv.restore(snap)
+    assert kv.len(1) == 10
+    again = [kv.attn_decode(1, rows[p], hq) for p in range(10, n)]
+    assert all(np.array_equal(a, b) for a, b in zip(again, first[10:]))
+    with pytest.raises(cai.CaiError):
+        cai.KVCache(2, hkv, dk, 64, cai.KV_F32).restore(snap)       # the element type must match
+    cai.load().cai_kv_snap_destroy(snap)
+    # a cache rebuilt from exported rows continues identically (the hand-off of a prefix built elsewhere)
+    kv.truncate(25)
+    state = kv.export_layer(1)
+    other = cai.KVCache(2, hkv, dk, 64, cai.KV_I8)
+    other.import_layer(1, *state)
+    assert other.len(1) == 25
+    for p in range(25, n):
+        assert np.array_equal(other.attn_decode(1, rows[p], hq), first[p])
+    # the float and half caches round-trip through the same two calls
+    for dtype in (cai.KV_F32, cai.KV_F16):
+        a = cai.KVCache(1, hkv, dk, 64, dtype)
+        ref = [a.attn_decode(0, rows[p], hq) for p in range(n)]
+        a.truncate(12)
+        b = cai.KVCache(1, hkv, dk, 64, dtype)
+        b.import_layer(0, *a.export_layer(0)[:2])
+        for p in range(12, 20):
+            assert np.array_equal(b.attn_decode(0, rows[p], hq), ref[p])

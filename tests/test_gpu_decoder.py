@@ -182,3 +182,34 @@ def test_matrix_core_prefill_equals_steps_and_feeds_decode():
     dec.prefill(toks[:-1], 0, seq=0, want_logits=False)
     b = dec.generate(int(toks[-1]), 39, 16)
     assert a.tolist() == b.tolist()
+
+
+def test_int8_kv_cache_decoder():
+    """Session over an int8 KV cache (TNNetStreamingDecoder with pInt8KV, neural/neuraldecode.pas:5775-5840): close to
+    the oracle run with the same cache model (codes may differ by one step where the two K,V rows differ in the last
+    bits), prompt ingestion and batch stepping agree with single steps, snapshot/restore replays exactly."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    s = SHAPES["qwen7b_like_q4k"]
+    spec = synthetic_spec(s["cfg"], s["qtype"], head_qtype=s["head"], qkv_bias=True, std=0.05)
+    rng = np.random.default_rng(77)
+    toks = rng.integers(0, spec["cfg"]["vocab"], 40).tolist()
+    om = oracle_model(spec, acc64=1, kv_f16=2)
+    of = oracle_model(spec, acc64=1)
+    dec = cai.Decoder(spec, max_batch=2, kv_dtype=cai.KV_I8)
+    worst, drift, steps = 0.0, 0.0, []
+    for p, t in enumerate(toks):
+        _, lo = om.step(t, p); _, lf = of.step(t, p); _, ld = dec.step(t, p)
+        steps.append(ld[0].copy())
+        worst = max(worst, rel_err(ld[0], lo)); drift = max(drift, rel_err(ld[0], lf))
+    assert worst < 5e-3, worst            # device int8 cache vs oracle int8 cache
+    assert drift < 5e-2, drift            # int8 cache vs fp32 cache: the quantisation itself
+    am, lg = dec.prefill(toks, 0, seq=1)  # prompt path: rows quantised by the append kernel, attention over codes
+    assert rel_err(lg, steps[-1]) < 2e-3 and dec.len(1) == len(toks)
+    dec.truncate(20); snap = dec.snapshot()
+    a = [dec.step(t, 20 + i)[1][0].copy() for i, t in enumerate(toks[20:30])]
+    dec.restore(snap)
+    b = [dec.step(t, 20 + i)[1][0].copy() for i, t in enumerate(toks[20:30])]
+    assert all(np.array_equal(x, y) for x, y in zip(a, b))
+    assert all(np.array_equal(x, y) for x, y in zip(a, steps[20:30]))
+    cai.load().cai_kv_snap_destroy(snap)
