@@ -4,13 +4,17 @@
 // appended to a head-major cache (row (g, p) at (g*MaxCtx + p)*Dk), then for each query head h (KV head
 // g = h / group) out_h = softmax(q_h . K_g / sqrt(Dk)) V_g over the live rows [jStart, len).
 //
-// Device formulation: split-K over the key axis.  Work-group (split, kv_head, sequence) streams its slice
-// of K and V exactly once with coalesced row loads (32 lanes x 16 B cover one 128-wide row), serves all
-// `G` query heads of the group from that one pass, and keeps an online-softmax state (m, l, acc) per
-// head; the 8 half-waves of the group meet in LDS, and a second small kernel (one work-group per query head) merges
-// the splits.  (Merging inside the first kernel through an arrival counter was measured slower: every
-// device-coherent hand-off between work-groups costs a memory round trip of ~2.5 us.)  RoPE of q and of the new k
-// row and the cache append happen inside the split kernel.
+// Device formulation: split-K over the key axis; a slice of the live rows per work-group, a small second kernel
+// (one work-group per query head) merges the slices.  (Merging inside the first kernel through an arrival counter was
+// measured slower: every device-coherent hand-off between work-groups costs a memory round trip of ~2.5 us.)  RoPE of
+// q and of the new k row and the cache append happen inside the split kernel.  Two split kernels:
+//   attn_group_kernel       one work-group per (slice, KV head) serves the whole group of query heads, so K and V are
+//                           fetched once; three phases per slice (scores -> LDS, softmax, value sum).  Used when the
+//                           grid fills the chip by itself (long caches, several sequences, prompt ingestion).
+//   attn_split_head_kernel  one work-group per (slice, QUERY head), online softmax in registers; the G heads of a
+//                           group re-read the slice from L2.  G times more work-groups: the better one for one
+//                           sequence with a short cache.
+// Cache element types: fp32, IEEE half, or int8 codes with one fp32 scale per cached row (neural/neural.cl:2501-2687).
 #include "cai_internal.hpp"
 
 namespace cai {
@@ -114,15 +118,62 @@ struct AttnParams {
   int64_t seq_rows, layer_row_off;
 };
 
-// ---- split kernel: RoPE (neural/neural.cl:1517-1542) + KV append (2354-2379) + split-K online-softmax decode
-//      (2406-2499).  The loop over the group's query heads is NOT unrolled and the per-head running state lives in
-//      LDS: the kernel stays a few KB of code, which matters for a launch this short (a cold instruction cache is
-//      refilled from L2 on every CU at every launch). ----
-template <int DS, typename KV_T>
-__global__ __launch_bounds__(256) void attn_step_kernel(const AttnParams p)
+// ---- split kernel: RoPE (neural/neural.cl:1517-1542) + KV append (2354-2379) + one slice of the cached decode
+//      (2406-2499), all query heads of a KV head in ONE work-group, so K and V are fetched once.
+//
+//      16 lanes x 8 elements cover a row, a wave holds 4 rows, the work-group 16 rows per pass; every load is 16
+//      contiguous bytes per lane and a wave's load is 4 whole rows.  Three phases like the reference kernel, but per
+//      slice: (1) scores of the slice into LDS (dot products reduced over 16 lanes with DPP), (2) slice maximum,
+//      exp-shift and sum per head, (3) the value sum.  The query heads are taken HC at a time (q and the accumulators
+//      live in registers: 8*HC each); a second chunk of heads re-reads the slice from cache.  The slice partial
+//      (sum_j e_j V_j, max, sum e_j) goes to the merge kernel, or straight to the output when the live range fits one
+//      slice. ----
+template <typename KV_T> struct Row8;
+template <> struct Row8<float>  { float4 a, b; };
+template <> struct Row8<__half> { uint4 a; };
+template <> struct Row8<int8_t> { uint2 a; };
+
+__device__ __forceinline__ void load8(const float* s, Row8<float>& r) { r.a = reinterpret_cast<const float4*>(s)[0]; r.b = reinterpret_cast<const float4*>(s)[1]; }
+__device__ __forceinline__ void load8(const __half* s, Row8<__half>& r) { r.a = *reinterpret_cast<const uint4*>(s); }
+__device__ __forceinline__ void load8(const int8_t* s, Row8<int8_t>& r) { r.a = *reinterpret_cast<const uint2*>(s); }
+__device__ __forceinline__ void unpack8(const Row8<float>& r, float (&v)[8])
+{
+  v[0] = r.a.x; v[1] = r.a.y; v[2] = r.a.z; v[3] = r.a.w; v[4] = r.b.x; v[5] = r.b.y; v[6] = r.b.z; v[7] = r.b.w;
+}
+__device__ __forceinline__ void unpack8(const Row8<__half>& r, float (&v)[8])
+{
+  const uint32_t w[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
+#pragma unroll
+  for (int i = 0; i < 4; i++) { const __half2 h = __builtin_bit_cast(__half2, w[i]); v[2 * i] = __low2float(h); v[2 * i + 1] = __high2float(h); }
+}
+__device__ __forceinline__ void unpack8(const Row8<int8_t>& r, float (&v)[8])
+{
+  const int w[2] = {(int)r.a.x, (int)r.a.y};
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    v[4 * i] = (float)((w[i] << 24) >> 24); v[4 * i + 1] = (float)((w[i] << 16) >> 24);
+    v[4 * i + 2] = (float)((w[i] << 8) >> 24); v[4 * i + 3] = (float)(w[i] >> 24);
+  }
+}
+
+// sum over each aligned group of 16 lanes, result in every lane of the group
+__device__ __forceinline__ float row16_allsum(float v)
+{
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xb1, 0xf, 0xf, true));   // lane ^ 1
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4e, 0xf, 0xf, true));   // lane ^ 2
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, true));  // 7 - lane within 8
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, true));  // 15 - lane within 16
+  return v;
+}
+
+template <int HC, typename KV_T>
+__global__ __launch_bounds__(256) void attn_group_kernel(const AttnParams p)
 {
   extern __shared__ float lds[];
-  const int split = blockIdx.x, g = blockIdx.y, seq = blockIdx.z;
+  constexpr bool I8 = sizeof(KV_T) == 1;
+  constexpr int NPF = sizeof(KV_T) == 4 ? 4 : 8;     // passes in flight per lane (32 registers either way)
+  const int G = p.q_heads / p.kv_heads, n_chunks = (G + HC - 1) / HC;
+  const int split = blockIdx.x % p.n_splits, g = blockIdx.x / p.n_splits, seq = blockIdx.y;
   const int pos = p.pos[seq];
   const int len = pos + 1;
   const int j_start = (p.window > 0 && len > p.window) ? len - p.window : 0;
@@ -130,163 +181,198 @@ __global__ __launch_bounds__(256) void attn_step_kernel(const AttnParams p)
   if (s_begin >= s_end) return;   // whole work-group leaves together, before any barrier
   const int s_first = j_start / p.split_len, s_last = pos / p.split_len;
   const int n_active = s_last - s_first + 1;
+  const int n_rows = s_end - s_begin, n_pass = (n_rows + 15) >> 4;
 
-  const int tid = threadIdx.x, hw = tid >> 5, l32 = tid & 31;
-  const int hd = p.hd, qw = p.q_heads * hd, kw = p.kv_heads * hd;
-  const int G = p.q_heads / p.kv_heads;
-  const int d0 = l32 * DS;
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r = lane >> 4, c = lane & 15, rr = 4 * w + r;
+  const int hd = p.hd, qw = p.q_heads * hd, kw = p.kv_heads * hd, SL = p.split_len;
+  const int d0 = 8 * c;
+  const bool lane_on = d0 < hd;
+  const int dl = lane_on ? d0 : 0;
   const float* row = p.qkv + (int64_t)seq * p.qkv_stride;
-  KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (seq * p.seq_mul + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
-  KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (seq * p.seq_mul + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  const int64_t cache_seq = seq * p.seq_mul + p.seq0;
+  KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + cache_seq * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + cache_seq * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  float* ksc = nullptr; float* vsc = nullptr;
+  if (I8) { const int64_t r0 = cache_seq * p.seq_rows + p.layer_row_off + (int64_t)g * p.max_ctx; ksc = p.ksc + r0; vsc = p.vsc + r0; }
 
-  // LDS: rotated q [G][32*DS] | state m,l [G][256] each | acc [G][DS][256]
-  float* sq = lds;
-  float* st_m = sq + G * 32 * DS;
-  float* st_l = st_m + G * 256;
-  float* st_a = st_l + G * 256;
+  float* sq = lds;                          // rotated q [G][128]
+  float* sS = sq + G * 128;                 // scores [G][SL]
+  constexpr int PW = HC > 4 ? 8 : 4;
+  float* sP = sS + G * SL;                  // softmax weights [chunk][SL][PW]
+  float* sred = sP + n_chunks * SL * PW;    // per-wave value sums [4][HC][128]
+  float* sML = sred + 4 * HC * 128;         // slice maximum [G], slice sum [G]
 
-  constexpr int PCH = 4;
-  float kdA[PCH][DS] = {}, vdA[PCH][DS] = {}, kdB[PCH][DS] = {}, vdB[PCH][DS] = {};
-  auto load_chunk = [&](float (&kd)[PCH][DS], float (&vd)[PCH][DS], int j0) {
-    if (j0 >= s_end || d0 >= hd) return;       // lanes beyond the head width keep their zeros
-#pragma unroll
-    for (int c = 0; c < PCH; c++) {
-      const int j = min(j0 + 8 * c, s_end - 1);
-      // (the slot of the row being appended may hold stale values: reduce_chunk replaces it from registers)
-      load_row_vec<DS, KV_T>(kc + (int64_t)j * hd + d0, kd[c]);
-      load_row_vec<DS, KV_T>(vc + (int64_t)j * hd + d0, vd[c]);
-    }
+  Row8<KV_T> ring[NPF];
+  float rsc[NPF];
+  auto issue = [&](const KV_T* base, const float* scales, int slot, int t) {
+    const int j = min(s_begin + 16 * t + rr, s_end - 1);
+    load8(base + (int64_t)j * hd + dl, ring[slot]);     // lanes beyond the head width re-read its start; q is zero there
+    if (I8) rsc[slot] = scales[j];
   };
-  load_chunk(kdA, vdA, s_begin + hw);      // cached rows are requested before the rotation math
-
-  // rotation of this lane's pairs at the token's position (DS even, or DS == 1 with the pair split over 2 lanes)
-  float rs[(DS + 1) / 2], rc[(DS + 1) / 2];
+  auto prime = [&](const KV_T* base, const float* scales) {
 #pragma unroll
-  for (int i = 0; i < (DS + 1) / 2; i++) {
-    rs[i] = 0.0f; rc[i] = 1.0f;
-    const int d = d0 + 2 * i;
-    if (p.theta && d < hd) { const float angle = (float)pos * p.theta[d >> 1]; sincosf(angle, &rs[i], &rc[i]); }
-  }
-  auto load_rot = [&](const float* v, float (&o)[DS], bool rotate) {
-    if (DS >= 2) {
-#pragma unroll
-      for (int i = 0; i < DS; i += 2) {
-        const int d = d0 + i;
-        const float x0 = d < hd ? v[d] : 0.0f, x1 = d + 1 < hd ? v[d + 1] : 0.0f;
-        if (rotate) { o[i] = rc[i / 2] * x0 - rs[i / 2] * x1; o[i + (DS > 1 ? 1 : 0)] = rs[i / 2] * x0 + rc[i / 2] * x1; }
-        else { o[i] = x0; o[i + (DS > 1 ? 1 : 0)] = x1; }
-      }
-    } else {
-      const int d = d0;
-      const float own = d < hd ? v[d] : 0.0f, mate = (d ^ 1) < hd ? v[d ^ 1] : 0.0f;
-      if (rotate) o[0] = (d & 1) ? (rs[0] * mate + rc[0] * own) : (rc[0] * own - rs[0] * mate);
-      else o[0] = own;
-    }
+    for (int u = 0; u < NPF; u++) { ring[u] = Row8<KV_T>{}; rsc[u] = 0.0f; if (u < n_pass) issue(base, scales, u, u); }
   };
-  // rotated q of the group's heads -> LDS (half-wave hw takes heads hw, hw+8, ..); state reset
-  for (int h = hw; h < G; h += 8) {
-    float qr[DS];
-    load_rot(row + (g * G + h) * hd, qr, p.theta != nullptr);
-#pragma unroll
-    for (int i = 0; i < DS; i++) sq[h * 32 * DS + d0 + i] = qr[i];
-  }
-  for (int h = 0; h < G; h++) {
-    st_m[h * 256 + tid] = -1e30f; st_l[h * 256 + tid] = 0.0f;
-#pragma unroll
-    for (int i = 0; i < DS; i++) st_a[(h * DS + i) * 256 + tid] = 0.0f;
-  }
-  // the work-group whose slice holds `pos` appends the new row and keeps it in registers
-  float knew[DS], vnew[DS];
   const bool owns_new = !p.appended && pos >= s_begin && pos < s_end;
-  if (owns_new) {
-    load_rot(row + qw + g * hd, knew, p.theta != nullptr);
-    load_rot(row + qw + kw + g * hd, vnew, false);
-#pragma unroll
-    for (int i = 0; i < DS; i++) {
-      vnew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(vnew[i]));
-      knew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(knew[i]));
-      if (hw == 0 && d0 + i < hd) {
-        kc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(knew[i]);
-        vc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(vnew[i]);
-      }
-    }
-  }
-  __syncthreads();
+  if (!owns_new) prime(kc, ksc);            // cached rows are requested before the rotation math
 
-  auto reduce_chunk = [&](float (&kd)[PCH][DS], float (&vd)[PCH][DS], int j0) {
-#pragma unroll
-    for (int c = 0; c < PCH; c++) {
-      if (owns_new && min(j0 + 8 * c, s_end - 1) == pos) {
-#pragma unroll
-        for (int i = 0; i < DS; i++) { kd[c][i] = knew[i]; vd[c][i] = vnew[i]; }
-      }
+  // rotated q of the group's heads -> LDS
+  for (int e = tid; e < G * (hd >> 1); e += 256) {
+    const int h = e / (hd >> 1), i = e % (hd >> 1);
+    const float* qh = row + (g * G + h) * hd;
+    float x0 = qh[2 * i], x1 = qh[2 * i + 1];
+    if (p.theta) {
+      float sn, cs; sincosf((float)pos * p.theta[i], &sn, &cs);
+      const float y0 = cs * x0 - sn * x1, y1 = sn * x0 + cs * x1;
+      x0 = y0; x1 = y1;
     }
-#pragma unroll 1
-    for (int h = 0; h < G; h++) {
-      float qh[DS];
-#pragma unroll
-      for (int i = 0; i < DS; i++) qh[i] = sq[h * 32 * DS + d0 + i];
-      float sc[PCH], cmax = -1e30f;
-#pragma unroll
-      for (int c = 0; c < PCH; c++) {
-        float s = 0.0f;
-#pragma unroll
-        for (int i = 0; i < DS; i++) s = fmaf(qh[i], kd[c][i], s);
-        s = half_wave_allsum(s) * p.inv_sqrt;
-        if (p.softcap > 0.0f) s = p.softcap * tanhf(s / p.softcap);
-        sc[c] = (j0 + 8 * c < s_end) ? s : -1e30f;
-        cmax = fmaxf(cmax, sc[c]);
-      }
-      const float mo = st_m[h * 256 + tid];
-      const float mn = fmaxf(mo, cmax);
-      const float corr = expf(mo - mn);
-      float lsum = 0.0f, a[DS];
-#pragma unroll
-      for (int i = 0; i < DS; i++) a[i] = st_a[(h * DS + i) * 256 + tid] * corr;
-#pragma unroll
-      for (int c = 0; c < PCH; c++) {
-        const float pj = (j0 + 8 * c < s_end) ? expf(sc[c] - mn) : 0.0f;
-        lsum += pj;
-#pragma unroll
-        for (int i = 0; i < DS; i++) a[i] = fmaf(pj, vd[c][i], a[i]);
-      }
-      st_l[h * 256 + tid] = st_l[h * 256 + tid] * corr + lsum;
-      st_m[h * 256 + tid] = mn;
-#pragma unroll
-      for (int i = 0; i < DS; i++) st_a[(h * DS + i) * 256 + tid] = a[i];
-    }
-  };
-  for (int j0 = s_begin + hw; j0 < s_end; j0 += 16 * PCH) {
-    load_chunk(kdB, vdB, j0 + 8 * PCH);
-    reduce_chunk(kdA, vdA, j0);
-    if (j0 + 8 * PCH < s_end) {
-      load_chunk(kdA, vdA, j0 + 16 * PCH);
-      reduce_chunk(kdB, vdB, j0 + 8 * PCH);
-    }
+    sq[h * 128 + 2 * i] = x0; sq[h * 128 + 2 * i + 1] = x1;
   }
-  __syncthreads();
-
-  // ---- merge the 8 half-waves (their states sit in LDS) ----
-  for (int o = tid; o < G * hd; o += 256) {
-    const int h = o / hd, d = o % hd, src_l = d / DS, src_i = d % DS;
-    float M = -1e30f;
+  // the work-group whose slice holds `pos` appends the new row: wave 0, one half-wave each for K and V
+  if (owns_new && w == 0) {
+    const int l32 = lane & 31, is_v = lane >> 5, e0 = 4 * l32;
+    const float* src = row + qw + (is_v ? kw : 0) + g * hd;
+    float v[4];
 #pragma unroll
-    for (int w = 0; w < 8; w++) M = fmaxf(M, st_m[h * 256 + w * 32 + src_l]);
-    float L = 0.0f, A = 0.0f;
-#pragma unroll
-    for (int w = 0; w < 8; w++) {
-      const float lw = st_l[h * 256 + w * 32 + src_l];
-      const float e = lw > 0.0f ? expf(st_m[h * 256 + w * 32 + src_l] - M) : 0.0f;
-      L = fmaf(lw, e, L); A = fmaf(st_a[(h * DS + src_i) * 256 + w * 32 + src_l], e, A);
+    for (int i = 0; i < 4; i += 2) {
+      const int d = e0 + i;
+      float x0 = d < hd ? src[d] : 0.0f, x1 = d + 1 < hd ? src[d + 1] : 0.0f;
+      if (p.theta && !is_v && d < hd) {
+        float sn, cs; sincosf((float)pos * p.theta[d >> 1], &sn, &cs);
+        const float y0 = cs * x0 - sn * x1, y1 = sn * x0 + cs * x1;
+        x0 = y0; x1 = y1;
+      }
+      v[i] = x0; v[i + 1] = x1;
     }
-    const int qh = g * G + h;
-    if (n_active == 1) {
-      p.out[(int64_t)seq * p.out_stride + qh * hd + d] = L > 0.0f ? A * (1.0f / L) : 0.0f;
+    KV_T* dst = (is_v ? vc : kc) + (int64_t)pos * hd;
+    if constexpr (I8) {
+      const float scale = quantise_row_i8<4>(v);
+#pragma unroll
+      for (int i = 0; i < 4; i++) if (e0 + i < hd) dst[e0 + i] = (int8_t)v[i];
+      if (l32 == 0) (is_v ? vsc : ksc)[pos] = scale;
     } else {
-      float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + split) * (hd + 2);
-      pt[d] = A;
-      if (d == 0) { pt[hd] = M; pt[hd + 1] = L; }
+#pragma unroll
+      for (int i = 0; i < 4; i++) if (e0 + i < hd) dst[e0 + i] = kv_from_float<KV_T>(v[i]);
     }
+  }
+  __syncthreads();      // q is staged; the appended row is visible to this work-group's loads
+  if (owns_new) prime(kc, ksc);
+
+  // ---- phase 1: scores of the slice ----
+  for (int ch = 0; ch < n_chunks; ch++) {
+    const int h0 = ch * HC;
+    if (ch > 0) prime(kc, ksc);
+    float q[HC][8];
+#pragma unroll
+    for (int hh = 0; hh < HC; hh++)
+#pragma unroll
+      for (int i = 0; i < 8; i++) q[hh][i] = (lane_on && h0 + hh < G) ? sq[(h0 + hh) * 128 + d0 + i] : 0.0f;
+    for (int t0 = 0; t0 < n_pass; t0 += NPF) {
+#pragma unroll
+      for (int u = 0; u < NPF; u++) {
+        const int t = t0 + u;
+        if (t < n_pass) {
+          float v[8];
+          unpack8(ring[u], v);
+          const float rs = rsc[u];
+          if (t + NPF < n_pass) issue(kc, ksc, u, t + NPF);
+          float sv = 0.0f;
+#pragma unroll
+          for (int hh = 0; hh < HC; hh++) {
+            float a = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) a = fmaf(q[hh][i], v[i], a);
+            a = row16_allsum(a);
+            if (c == hh) sv = a;
+          }
+          const int rl = 16 * t + rr;
+          if (rl < n_rows && c < HC && h0 + c < G) {
+            sS[(h0 + c) * SL + rl] = sv * (I8 ? rs * p.inv_sqrt : p.inv_sqrt);
+          }
+        }
+      }
+    }
+  }
+  prime(vc, vsc);        // the first value rows travel while the softmax runs
+  __syncthreads();
+
+  // ---- phase 2: slice maximum, exp-shift and sum per head (wave w takes heads w, w+4, ..) ----
+  for (int h = w; h < G; h += 4) {
+    float m = -1e30f;
+    if (p.softcap > 0.0f)
+      for (int rl = lane; rl < n_rows; rl += 64) sS[h * SL + rl] = p.softcap * tanhf(sS[h * SL + rl] / p.softcap);
+    for (int rl = lane; rl < n_rows; rl += 64) m = fmaxf(m, sS[h * SL + rl]);
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    float l = 0.0f;
+    for (int rl = lane; rl < n_rows; rl += 64) {
+      const float e = expf(sS[h * SL + rl] - m);
+      l += e;
+      sP[((h / HC) * SL + rl) * PW + h % HC] = I8 ? e * vsc[s_begin + rl] : e;
+    }
+    for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
+    if (lane == 0) { sML[h] = m; sML[G + h] = l; }
+  }
+  __syncthreads();
+
+  // ---- phase 3: value sums ----
+  for (int ch = 0; ch < n_chunks; ch++) {
+    const int h0 = ch * HC;
+    if (ch > 0) prime(vc, vsc);
+    float acc[HC][8];
+#pragma unroll
+    for (int hh = 0; hh < HC; hh++)
+#pragma unroll
+      for (int i = 0; i < 8; i++) acc[hh][i] = 0.0f;
+    for (int t0 = 0; t0 < n_pass; t0 += NPF) {
+#pragma unroll
+      for (int u = 0; u < NPF; u++) {
+        const int t = t0 + u;
+        if (t < n_pass) {
+          float v[8];
+          unpack8(ring[u], v);
+          if (t + NPF < n_pass) issue(vc, vsc, u, t + NPF);
+          const int rl = 16 * t + rr;
+          float pf[PW];
+#pragma unroll
+          for (int k4 = 0; k4 < PW; k4 += 4) {
+            float4 pw = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (rl < n_rows) pw = *reinterpret_cast<const float4*>(sP + ((int64_t)ch * SL + rl) * PW + k4);
+            pf[k4] = pw.x; pf[k4 + 1] = pw.y; pf[k4 + 2] = pw.z; pf[k4 + 3] = pw.w;
+          }
+#pragma unroll
+          for (int hh = 0; hh < HC; hh++)
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[hh][i] = fmaf(pf[hh], v[i], acc[hh][i]);
+        }
+      }
+    }
+    // the wave's 4 row groups, then the 4 waves
+#pragma unroll
+    for (int hh = 0; hh < HC; hh++)
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        float a = acc[hh][i];
+        a += __shfl_xor(a, 16, 64);
+        a += __shfl_xor(a, 32, 64);
+        if (r == 0 && lane_on) sred[(w * HC + hh) * 128 + d0 + i] = a;
+      }
+    __syncthreads();
+    for (int o = tid; o < HC * hd; o += 256) {
+      const int hh = o / hd, d = o % hd, h = h0 + hh;
+      if (h < G) {
+        const float A = (sred[(0 * HC + hh) * 128 + d] + sred[(1 * HC + hh) * 128 + d]) + (sred[(2 * HC + hh) * 128 + d] + sred[(3 * HC + hh) * 128 + d]);
+        const float M = sML[h], Ls = sML[G + h];
+        const int qh = g * G + h;
+        if (n_active == 1) {
+          p.out[(int64_t)seq * p.out_stride + qh * hd + d] = Ls > 0.0f ? A * (1.0f / Ls) : 0.0f;
+        } else {
+          float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + split) * (hd + 2);
+          pt[d] = A;
+          if (d == 0) { pt[hd] = M; pt[hd + 1] = Ls; }
+        }
+      }
+    }
+    __syncthreads();
   }
 }
 
@@ -515,16 +601,24 @@ static int launch_split_head(const AttnParams& p, int n_seq, hipStream_t st)
 }
 
 template <typename KV_T>
-static int launch_split_g(const AttnParams& p, int n_seq, hipStream_t st)
+static int launch_group(const AttnParams& p, int n_seq, hipStream_t st)
 {
   const int G = p.q_heads / p.kv_heads;
-  if (G < 1 || G > 8) return set_error(CAI_ERR_UNSUPPORTED, "attention: %d query heads per KV head (supported 1..8)", G);
-  const dim3 grid(p.n_splits, p.kv_heads, n_seq);
-  auto lds = [&](int ds) { return (size_t)(G * 32 * ds + G * 256 * (2 + ds)) * sizeof(float); };
-  if (p.hd <= 32) hipLaunchKernelGGL((attn_step_kernel<1, KV_T>), grid, dim3(256), lds(1), st, p);
-  else if (p.hd <= 64) hipLaunchKernelGGL((attn_step_kernel<2, KV_T>), grid, dim3(256), lds(2), st, p);
-  else if (p.hd <= 128) hipLaunchKernelGGL((attn_step_kernel<4, KV_T>), grid, dim3(256), lds(4), st, p);
-  else return set_error(CAI_ERR_UNSUPPORTED, "attention: head_dim %d > 128", p.hd);
+  static const int hc_max = []() { const char* e = getenv("CAIHIP_ATTN_HC"); const int v = e ? atoi(e) : 8; return v >= 1 && v <= 8 ? v : 8; }();
+  const int n_chunks = (G + hc_max - 1) / hc_max, hc = (G + n_chunks - 1) / n_chunks;
+  const dim3 grid(p.n_splits * p.kv_heads, n_seq);
+  const size_t lds = (size_t)(G * 128 + G * p.split_len + n_chunks * p.split_len * (hc > 4 ? 8 : 4) + 4 * hc * 128 + 2 * G) * sizeof(float);
+  if (lds > 64 * 1024) return set_error(CAI_ERR_UNSUPPORTED, "attention: %d query heads per KV head need %zu bytes of LDS", G, lds);
+  switch (hc) {
+    case 1: hipLaunchKernelGGL((attn_group_kernel<1, KV_T>), grid, dim3(256), lds, st, p); break;
+    case 2: hipLaunchKernelGGL((attn_group_kernel<2, KV_T>), grid, dim3(256), lds, st, p); break;
+    case 3: hipLaunchKernelGGL((attn_group_kernel<3, KV_T>), grid, dim3(256), lds, st, p); break;
+    case 4: hipLaunchKernelGGL((attn_group_kernel<4, KV_T>), grid, dim3(256), lds, st, p); break;
+    case 5: hipLaunchKernelGGL((attn_group_kernel<5, KV_T>), grid, dim3(256), lds, st, p); break;
+    case 6: hipLaunchKernelGGL((attn_group_kernel<6, KV_T>), grid, dim3(256), lds, st, p); break;
+    case 7: hipLaunchKernelGGL((attn_group_kernel<7, KV_T>), grid, dim3(256), lds, st, p); break;
+    default: hipLaunchKernelGGL((attn_group_kernel<8, KV_T>), grid, dim3(256), lds, st, p); break;
+  }
   return CAI_OK;
 }
 
@@ -627,12 +721,14 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   }
   p.counters = kv->d_counters;
   int rc;
-  if (kv->dtype == CAI_KV_I8)
-    rc = launch_split_head<int8_t>(p, n_seq, c.stream);
-  else if (kv->max_ctx <= kv->short_ctx_limit)   // short caches: per-head work-groups (K,V re-read from L2 by the group's heads)
-    rc = kv->dtype == CAI_KV_F16 ? launch_split_head<__half>(p, n_seq, c.stream) : launch_split_head<float>(p, n_seq, c.stream);
+  // one work-group per (slice, KV head) serving the whole group of query heads, or one per (slice, query head)
+  // (the first fetches K and V once but has G times fewer work-groups: it needs a grid that fills the chip by itself)
+  static const int group_min = []() { const char* e = getenv("CAIHIP_ATTN_GROUP_MIN"); return e ? atoi(e) : 256; }();
+  const bool grouped = (kv->head_dim & 7) == 0 && n_seq * kv->kv_heads * kv->n_splits >= group_min;
+  if (grouped)
+    rc = kv->dtype == CAI_KV_I8 ? launch_group<int8_t>(p, n_seq, c.stream) : kv->dtype == CAI_KV_F16 ? launch_group<__half>(p, n_seq, c.stream) : launch_group<float>(p, n_seq, c.stream);
   else
-    rc = kv->dtype == CAI_KV_F16 ? launch_split_g<__half>(p, n_seq, c.stream) : launch_split_g<float>(p, n_seq, c.stream);
+    rc = kv->dtype == CAI_KV_I8 ? launch_split_head<int8_t>(p, n_seq, c.stream) : kv->dtype == CAI_KV_F16 ? launch_split_head<__half>(p, n_seq, c.stream) : launch_split_head<float>(p, n_seq, c.stream);
   if (rc) return rc;
   if (p.n_splits > 1) hipLaunchKernelGGL(attn_merge_kernel, dim3(q_heads, n_seq), dim3(128), 0, c.stream, p);
   return CAI_OK;
@@ -665,10 +761,6 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
     CAI_HIP(hipMalloc(&kv->vs, sb));
     CAI_HIP(hipMemsetAsync(kv->ks, 0, sb, ctx().stream));
     CAI_HIP(hipMemsetAsync(kv->vs, 0, sb, ctx().stream));
-  }
-  {
-    const char* e = getenv("CAIHIP_ATTN_SHORT_CTX");      // caches up to this capacity use the per-head split kernel
-    kv->short_ctx_limit = e ? atoi(e) : (1 << 30);
   }
   kv->part_q_heads = kv_heads * 8;
   CAI_HIP(hipMalloc(&kv->part, (size_t)n_seq * kv->part_q_heads * kv->n_splits * (head_dim + 2) * sizeof(float)));

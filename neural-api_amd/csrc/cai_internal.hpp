@@ -73,7 +73,6 @@ struct cai_kv_s {
   float* ks = nullptr; float* vs = nullptr;   // CAI_KV_I8 only: one scale per cached row, [seq][layer][kv_head][max_ctx]
   std::vector<int> len;                   // [seq][layer] live rows (host mirror)
   int split_len = 64, n_splits = 1;       // split-K geometry of the decode kernel (fixed at creation)
-  int short_ctx_limit = 0;                // caches up to this capacity use the per-query-head split kernel
   float* part = nullptr;                  // [seq][q_head][split][head_dim+2] split-K partials
   int part_q_heads = 0;
   int32_t* d_len = nullptr;               // [seq] device scratch: rows live BEFORE the token being decoded
