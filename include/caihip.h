@@ -146,7 +146,14 @@ int cai_kv_create(int n_layers, int kv_heads, int head_dim, int max_ctx, int kv_
 int cai_kv_destroy(cai_kv_t kv);
 int cai_kv_reset(cai_kv_t kv);
 int cai_kv_truncate(cai_kv_t kv, int n);          /* keeps the first n rows of every layer */
-int cai_kv_len(cai_kv_t kv, int layer, int* len_out);
+int cai_kv_len(cai_kv_t kv, int layer, int* len_out);   /* tokens appended so far = the next position */
+/* StreamingLLM eviction (TNNetStreamingDecoder.EnableEviction / DisableEviction, neural/neuraldecode.pas:1257-1277,
+ * 5722-5735): the first sink_tokens positions and the latest recent_window positions stay cached, the middle is
+ * dropped, so a stream runs past max_ctx in constant memory.  Cached keys keep the rotation of their own position.
+ * sink_tokens + recent_window <= max_ctx; 0, 0 turns it off.  Until the stream passes the cap, results are
+ * bit-identical to the unbounded cache; the policy may only change while no sequence is past the smaller cap. */
+int cai_kv_set_eviction(cai_kv_t kv, int sink_tokens, int recent_window);
+int cai_kv_rows(cai_kv_t kv, int layer, int* rows_out);  /* rows held: min(len, cap) (SDPACacheLength, neural/neuraldecode.pas:1291-1294) */
 int cai_kv_snapshot(cai_kv_t kv, cai_kv_snap_t* out);
 int cai_kv_restore(cai_kv_t kv, cai_kv_snap_t snap);
 int cai_kv_snap_destroy(cai_kv_snap_t snap);
@@ -221,7 +228,14 @@ int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* tokens, int n, 
 /* Session management (neural/neuraldecode.pas:5714-5843): always safe after a failed step. */
 int cai_decoder_reset(cai_decoder_t d, int seq);
 int cai_decoder_truncate(cai_decoder_t d, int seq, int n);
-int cai_decoder_len(cai_decoder_t d, int seq, int* len_out);
+int cai_decoder_len(cai_decoder_t d, int seq, int* len_out);   /* tokens streamed so far = the next position */
+/* Eviction for every layer of every sequence of the session (see cai_kv_set_eviction); with it on, positions may run
+ * past max_ctx.  cai_decoder_cache_rows is SDPACacheLength(Index) (neural/neuraldecode.pas:1291-1294). */
+int cai_decoder_set_eviction(cai_decoder_t d, int sink_tokens, int recent_window);
+int cai_decoder_cache_rows(cai_decoder_t d, int seq, int layer, int* rows_out);
+/* EnableInt8KVCache / DisableInt8KVCache (neural/neuraldecode.pas:1277-1290): switches the cache element type; like the
+ * reference only on an empty session (CAI_ERR_STATE once a token has been streamed). */
+int cai_decoder_set_kv_dtype(cai_decoder_t d, int kv_dtype);
 int cai_decoder_snapshot(cai_decoder_t d, int seq, cai_kv_snap_t* out);
 int cai_decoder_restore(cai_decoder_t d, int seq, cai_kv_snap_t snap);
 /* Bytes of weights, biases and gains one decoded token streams (for roofline accounting). */

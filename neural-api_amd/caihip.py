@@ -18,9 +18,9 @@ SYMBOLS = """cai_init cai_shutdown cai_last_error cai_device_name cai_sync cai_g
 cai_dev_alloc cai_dev_free cai_dev_upload cai_dev_download cai_dev_copy
 cai_qw_create cai_qw_create_int8row cai_qw_destroy cai_qw_info cai_qw_dequant_rows cai_qgemv cai_ffn_gateup cai_qgemm
 cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_router_topk
-cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_kv_export_layer cai_kv_import_layer cai_attn_decode
+cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_kv_export_layer cai_kv_import_layer cai_kv_set_eviction cai_kv_rows cai_attn_decode
 cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_generate
-cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_snapshot cai_decoder_restore
+cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_set_eviction cai_decoder_cache_rows cai_decoder_set_kv_dtype cai_decoder_snapshot cai_decoder_restore
 cai_decoder_weight_bytes cai_decoder_get_config cai_decoder_load_gguf
 cai_gguf_open cai_gguf_close cai_gguf_info cai_gguf_meta_int cai_gguf_meta_float cai_gguf_meta_str cai_gguf_meta_array_count
 cai_gguf_meta_array_str cai_gguf_find_tensor cai_gguf_tensor_info cai_gguf_tensor_data cai_gguf_load_qw""".split()
@@ -81,6 +81,8 @@ def load():
         L.cai_kv_snapshot.argtypes = [vp, C.POINTER(vp)]
         L.cai_kv_restore.argtypes = [vp, vp]
         L.cai_kv_snap_destroy.argtypes = [vp]
+        L.cai_kv_set_eviction.argtypes = [vp, C.c_int, C.c_int]
+        L.cai_kv_rows.argtypes = [vp, C.c_int, C.POINTER(C.c_int)]
         L.cai_kv_export_layer.argtypes = [vp, C.c_int, vp, vp, vp, vp]
         L.cai_kv_import_layer.argtypes = [vp, C.c_int, C.c_int, vp, vp, vp, vp]
         L.cai_attn_decode.argtypes = [vp, i32, vp, i32, i32, f32, vp, i32]
@@ -94,6 +96,9 @@ def load():
         L.cai_decoder_reset.argtypes = [vp, i32]
         L.cai_decoder_truncate.argtypes = [vp, i32, i32]
         L.cai_decoder_len.argtypes = [vp, i32, C.POINTER(i32)]
+        L.cai_decoder_set_eviction.argtypes = [vp, i32, i32]
+        L.cai_decoder_set_kv_dtype.argtypes = [vp, i32]
+        L.cai_decoder_cache_rows.argtypes = [vp, i32, i32, C.POINTER(i32)]
         L.cai_decoder_snapshot.argtypes = [vp, i32, C.POINTER(vp)]
         L.cai_decoder_restore.argtypes = [vp, i32, vp]
         L.cai_decoder_weight_bytes.argtypes = [vp, C.POINTER(i64)]
@@ -234,9 +239,17 @@ class KVCache:
     def restore(self, s):
         check(load().cai_kv_restore(self.h, s))
 
+    def set_eviction(self, sinks, recent):
+        check(load().cai_kv_set_eviction(self.h, sinks, recent))
+
+    def rows(self, layer=0):
+        n = C.c_int()
+        check(load().cai_kv_rows(self.h, layer, C.byref(n)))
+        return n.value
+
     def export_layer(self, layer):
         """(k, v, k_scales, v_scales): the live rows in the cache's element type; scales are None unless int8."""
-        n = self.len(layer)
+        n = self.rows(layer)
         et = {KV_F32: np.float32, KV_F16: np.float16, KV_I8: np.int8}[self.dtype]
         k = np.zeros((self.kv_heads, n, self.head_dim), et); v = np.zeros_like(k)
         ks = np.zeros((self.kv_heads, n), np.float32) if self.dtype == KV_I8 else None
@@ -398,6 +411,17 @@ class Decoder:
     def len(self, seq=0):
         n = C.c_int()
         check(load().cai_decoder_len(self.h, seq, C.byref(n)))
+        return n.value
+
+    def set_eviction(self, sinks, recent):
+        check(load().cai_decoder_set_eviction(self.h, sinks, recent))
+
+    def set_kv_dtype(self, dtype):
+        check(load().cai_decoder_set_kv_dtype(self.h, dtype))
+
+    def cache_rows(self, seq=0, layer=0):
+        n = C.c_int()
+        check(load().cai_decoder_cache_rows(self.h, seq, layer, C.byref(n)))
         return n.value
 
     def snapshot(self, seq=0):

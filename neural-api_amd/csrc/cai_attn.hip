@@ -116,7 +116,26 @@ struct AttnParams {
   int* counters;               // [seq][kv_head] arrival counters of the split merge (zero between launches)
   float* ksc; float* vsc;      // int8 caches: row scales [seq][layer][kv_head][max_ctx]
   int64_t seq_rows, layer_row_off;
+  int evict_sinks, evict_cap;  // cap > 0: only the first `sinks` positions and the latest cap - sinks stay cached
 };
+
+// Where the row of stream position `pos` lives and which rows are live.  Without eviction: slot = pos, rows
+// [j_start, pos] (j_start > 0 under a sliding window).  With sink + recent-window eviction (TNNetStreamingDecoder.
+// EnableEviction, neural/neuraldecode.pas:1257-1276) the cache holds positions [0, sinks) and the latest cap - sinks;
+// instead of shifting rows on every token the recent part is a ring: slot = sinks + (pos - sinks) mod (cap - sinks),
+// and all cap rows are live.  Keys keep the rotation of their own position, the query that of `pos`.
+struct LiveRows { int slot, len, j_start; };
+__device__ __forceinline__ LiveRows live_rows(const AttnParams& p, int pos)
+{
+  LiveRows r;
+  if (p.evict_cap > 0 && pos >= p.evict_cap) {
+    r.slot = p.evict_sinks + (pos - p.evict_sinks) % (p.evict_cap - p.evict_sinks); r.len = p.evict_cap; r.j_start = 0;
+  } else {
+    r.slot = pos; r.len = pos + 1;
+    r.j_start = (p.window > 0 && r.len > p.window) ? r.len - p.window : 0;
+  }
+  return r;
+}
 
 // ---- split kernel: RoPE (neural/neural.cl:1517-1542) + KV append (2354-2379) + one slice of the cached decode
 //      (2406-2499), all query heads of a KV head in ONE work-group, so K and V are fetched once.
@@ -175,11 +194,11 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const AttnParams p)
   const int G = p.q_heads / p.kv_heads, n_chunks = (G + HC - 1) / HC;
   const int split = blockIdx.x % p.n_splits, g = blockIdx.x / p.n_splits, seq = blockIdx.y;
   const int pos = p.pos[seq];
-  const int len = pos + 1;
-  const int j_start = (p.window > 0 && len > p.window) ? len - p.window : 0;
+  const LiveRows lr = live_rows(p, pos);
+  const int len = lr.len, j_start = lr.j_start, slot = lr.slot;
   const int s_begin = max(j_start, split * p.split_len), s_end = min(len, (split + 1) * p.split_len);
   if (s_begin >= s_end) return;   // whole work-group leaves together, before any barrier
-  const int s_first = j_start / p.split_len, s_last = pos / p.split_len;
+  const int s_first = j_start / p.split_len, s_last = (len - 1) / p.split_len;
   const int n_active = s_last - s_first + 1;
   const int n_rows = s_end - s_begin, n_pass = (n_rows + 15) >> 4;
 
@@ -213,7 +232,7 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const AttnParams p)
 #pragma unroll
     for (int u = 0; u < NPF; u++) { ring[u] = Row8<KV_T>{}; rsc[u] = 0.0f; if (u < n_pass) issue(base, scales, u, u); }
   };
-  const bool owns_new = !p.appended && pos >= s_begin && pos < s_end;
+  const bool owns_new = !p.appended && slot >= s_begin && slot < s_end;
   if (!owns_new) prime(kc, ksc);            // cached rows are requested before the rotation math
 
   // rotated q of the group's heads -> LDS
@@ -244,12 +263,12 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const AttnParams p)
       }
       v[i] = x0; v[i + 1] = x1;
     }
-    KV_T* dst = (is_v ? vc : kc) + (int64_t)pos * hd;
+    KV_T* dst = (is_v ? vc : kc) + (int64_t)slot * hd;
     if constexpr (I8) {
       const float scale = quantise_row_i8<4>(v);
 #pragma unroll
       for (int i = 0; i < 4; i++) if (e0 + i < hd) dst[e0 + i] = (int8_t)v[i];
-      if (l32 == 0) (is_v ? vsc : ksc)[pos] = scale;
+      if (l32 == 0) (is_v ? vsc : ksc)[slot] = scale;
     } else {
 #pragma unroll
       for (int i = 0; i < 4; i++) if (e0 + i < hd) dst[e0 + i] = kv_from_float<KV_T>(v[i]);
@@ -381,9 +400,8 @@ __global__ __launch_bounds__(128) void attn_merge_kernel(const AttnParams p)
 {
   const int qh = blockIdx.x, seq = blockIdx.y;
   const int hd = p.hd;
-  const int pos = p.pos[seq], len = pos + 1;
-  const int j_start = (p.window > 0 && len > p.window) ? len - p.window : 0;
-  const int s_first = j_start / p.split_len, s_last = pos / p.split_len;
+  const LiveRows lr = live_rows(p, p.pos[seq]);
+  const int s_first = lr.j_start / p.split_len, s_last = (lr.len - 1) / p.split_len;
   const int n_active = s_last - s_first + 1;
   if (n_active == 1) return;                       // the split kernel already wrote the final row
   const float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + s_first) * (hd + 2);
@@ -423,11 +441,11 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
   if (item >= p.n_splits * p.kv_heads) return;
   const int split = item % p.n_splits, g = item / p.n_splits, seq = blockIdx.y;
   const int pos = p.pos[seq];
-  const int len = pos + 1;
-  const int j_start = (p.window > 0 && len > p.window) ? len - p.window : 0;
+  const LiveRows lr = live_rows(p, pos);
+  const int len = lr.len, j_start = lr.j_start, slot = lr.slot;
   const int s_begin = max(j_start, split * p.split_len), s_end = min(len, (split + 1) * p.split_len);
   if (s_begin >= s_end) return;   // whole work-group leaves together, before any barrier
-  const int s_first = j_start / p.split_len, s_last = pos / p.split_len;
+  const int s_first = j_start / p.split_len, s_last = (len - 1) / p.split_len;
   const int n_active = s_last - s_first + 1;
 
   const int tid = threadIdx.x, hw = tid >> 5, l32 = tid & 31;
@@ -491,7 +509,7 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
 #pragma unroll
   for (int i = 0; i < DS; i++) { acc[i] = 0.0f; knew[i] = 0.0f; vnew[i] = 0.0f; }
   // every work-group whose slice holds `pos` keeps the new row in registers; the group's first head appends it
-  const bool owns_new = !p.appended && pos >= s_begin && pos < s_end;
+  const bool owns_new = !p.appended && slot >= s_begin && slot < s_end;
   float knew_s = 1.0f, vnew_s = 1.0f;
   if (owns_new) {
     load_rot(row + qw + g * hd, knew, p.theta != nullptr);
@@ -502,8 +520,8 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
       if (h == 0 && hw == 0) {
 #pragma unroll
         for (int i = 0; i < DS; i++)
-          if (d0 + i < hd) { kc[(int64_t)pos * hd + d0 + i] = (int8_t)knew[i]; vc[(int64_t)pos * hd + d0 + i] = (int8_t)vnew[i]; }
-        if (l32 == 0) { p.ksc[(ksc - p.ksc) + pos] = knew_s; p.vsc[(vsc - p.vsc) + pos] = vnew_s; }
+          if (d0 + i < hd) { kc[(int64_t)slot * hd + d0 + i] = (int8_t)knew[i]; vc[(int64_t)slot * hd + d0 + i] = (int8_t)vnew[i]; }
+        if (l32 == 0) { p.ksc[(ksc - p.ksc) + slot] = knew_s; p.vsc[(vsc - p.vsc) + slot] = vnew_s; }
       }
     } else {
 #pragma unroll
@@ -511,8 +529,8 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
         vnew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(vnew[i]));
         knew[i] = kv_to_float<KV_T>(kv_from_float<KV_T>(knew[i]));
         if (h == 0 && hw == 0 && d0 + i < hd) {
-          kc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(knew[i]);
-          vc[(int64_t)pos * hd + d0 + i] = kv_from_float<KV_T>(vnew[i]);
+          kc[(int64_t)slot * hd + d0 + i] = kv_from_float<KV_T>(knew[i]);
+          vc[(int64_t)slot * hd + d0 + i] = kv_from_float<KV_T>(vnew[i]);
         }
       }
     }
@@ -522,7 +540,7 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
     float sc[PCH], cmax = -1e30f;
 #pragma unroll
     for (int c = 0; c < PCH; c++) {
-      if (owns_new && min(j0 + 8 * c, s_end - 1) == pos) {
+      if (owns_new && min(j0 + 8 * c, s_end - 1) == slot) {
 #pragma unroll
         for (int i = 0; i < DS; i++) { ch.k[c][i] = knew[i]; ch.v[c][i] = vnew[i]; }
         if (I8) { ch.ks[c] = knew_s; ch.vs[c] = vnew_s; }
@@ -628,7 +646,7 @@ __global__ __launch_bounds__(256) void kv_append_rows_kernel(const AttnParams p)
 {
   const int b = blockIdx.x;
   const float* row = p.qkv + (int64_t)b * p.qkv_stride;
-  const int pos = p.pos[b];
+  const int pos = p.pos[b], slot = live_rows(p, pos).slot;
   const int hd = p.hd, qw = p.q_heads * hd, kw = p.kv_heads * hd;
   KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (int64_t)p.seq0 * p.seq_elems + p.layer_off;
   KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (int64_t)p.seq0 * p.seq_elems + p.layer_off;
@@ -641,12 +659,12 @@ __global__ __launch_bounds__(256) void kv_append_rows_kernel(const AttnParams p)
       const float y0 = cs * x0 - sn * x1, y1 = sn * x0 + cs * x1;
       x0 = y0; x1 = y1;
     }
-    KV_T* dst = kc + ((int64_t)g * p.max_ctx + pos) * hd + d;
+    KV_T* dst = kc + ((int64_t)g * p.max_ctx + slot) * hd + d;
     dst[0] = kv_from_float<KV_T>(x0); dst[1] = kv_from_float<KV_T>(x1);
   }
   for (int i = threadIdx.x; i < kw; i += 256) {
     const int g = i / hd, d = i % hd;
-    vc[((int64_t)g * p.max_ctx + pos) * hd + d] = kv_from_float<KV_T>(row[qw + kw + i]);
+    vc[((int64_t)g * p.max_ctx + slot) * hd + d] = kv_from_float<KV_T>(row[qw + kw + i]);
   }
 }
 
@@ -656,7 +674,7 @@ __global__ __launch_bounds__(256) void kv_append_rows_i8_kernel(const AttnParams
 {
   const int b = blockIdx.x, hw = threadIdx.x >> 5, l32 = threadIdx.x & 31;
   const float* row = p.qkv + (int64_t)b * p.qkv_stride;
-  const int pos = p.pos[b];
+  const int pos = p.pos[b], slot = live_rows(p, pos).slot;
   const int hd = p.hd, qw = p.q_heads * hd, kw = p.kv_heads * hd;
   const int d0 = l32 * DS;
   for (int item = hw; item < 2 * p.kv_heads; item += 8) {      // uniform per half-wave; both halves of a wave loop alike
@@ -685,11 +703,11 @@ __global__ __launch_bounds__(256) void kv_append_rows_i8_kernel(const AttnParams
       }
     }
     const float scale = quantise_row_i8<DS>(v);
-    const int64_t slot = (int64_t)p.seq0 * p.seq_rows + p.layer_row_off + (int64_t)g * p.max_ctx + pos;
-    int8_t* dst = reinterpret_cast<int8_t*>(is_v ? p.vc : p.kc) + (int64_t)p.seq0 * p.seq_elems + p.layer_off + ((int64_t)g * p.max_ctx + pos) * hd;
+    const int64_t srow = (int64_t)p.seq0 * p.seq_rows + p.layer_row_off + (int64_t)g * p.max_ctx + slot;
+    int8_t* dst = reinterpret_cast<int8_t*>(is_v ? p.vc : p.kc) + (int64_t)p.seq0 * p.seq_elems + p.layer_off + ((int64_t)g * p.max_ctx + slot) * hd;
 #pragma unroll
     for (int i = 0; i < DS; i++) if (d0 + i < hd) dst[d0 + i] = (int8_t)v[i];
-    if (l32 == 0) (is_v ? p.vsc : p.ksc)[slot] = scale;
+    if (l32 == 0) (is_v ? p.vsc : p.ksc)[srow] = scale;
   }
 }
 
@@ -710,6 +728,7 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   p.theta = theta; p.pos = pos_dev; p.split_len = kv->split_len; p.n_splits = kv->n_splits;
   p.part = prompt_rows ? prompt_part : kv->part; p.out = out; p.out_stride = out_stride; p.seq0 = seq0;
   p.seq_mul = prompt_rows ? 0 : 1; p.appended = prompt_rows ? 1 : 0;
+  p.evict_sinks = kv->evict_sinks; p.evict_cap = kv->evict_cap;
   p.ksc = kv->ks; p.vsc = kv->vs; p.seq_rows = kv->seq_rows(); p.layer_row_off = (int64_t)layer * kv->layer_rows();
   if (prompt_rows && kv->dtype == CAI_KV_I8) {
     if (p.hd <= 32) hipLaunchKernelGGL(kv_append_rows_i8_kernel<1>, dim3(n_seq), dim3(256), 0, c.stream, p);
@@ -790,9 +809,10 @@ int kv_snapshot(cai_kv_s* kv, int seq, cai_kv_snap_s** out)
 {
   cai_kv_snap_s* s = new cai_kv_snap_s();
   s->n_layers = kv->n_layers; s->kv_heads = kv->kv_heads; s->head_dim = kv->head_dim; s->dtype = kv->dtype;
+  s->evict_sinks = kv->evict_sinks; s->evict_cap = kv->evict_cap;
   s->len.resize(kv->n_layers);
   int rows = 0;
-  for (int l = 0; l < kv->n_layers; l++) { s->len[l] = kv->len_at(seq, l); rows = std::max(rows, s->len[l]); }
+  for (int l = 0; l < kv->n_layers; l++) { s->len[l] = kv->len_at(seq, l); rows = std::max(rows, kv->live(s->len[l])); }
   s->rows = rows;
   if (rows > 0) {
     const size_t bytes = (size_t)kv->n_layers * kv->kv_heads * rows * kv->head_dim * kv->elem();
@@ -829,6 +849,8 @@ int kv_restore(cai_kv_s* kv, int seq, const cai_kv_snap_s* s)
   if (s->n_layers != kv->n_layers || s->kv_heads != kv->kv_heads || s->head_dim != kv->head_dim)
     return set_error(CAI_ERR_INVALID, "kv restore: snapshot geometry differs from the cache");
   if (s->dtype != kv->dtype) return set_error(CAI_ERR_INVALID, "kv restore: snapshot element type differs from the cache (mode must match)");
+  if (s->evict_sinks != kv->evict_sinks || s->evict_cap != kv->evict_cap)
+    return set_error(CAI_ERR_INVALID, "kv restore: snapshot was taken under eviction (%d sinks, cap %d), the cache runs (%d, %d)", s->evict_sinks, s->evict_cap, kv->evict_sinks, kv->evict_cap);
   if (s->rows > kv->max_ctx) return set_error(CAI_ERR_INVALID, "kv restore: snapshot holds %d rows, cache %d", s->rows, kv->max_ctx);
   if (s->rows > 0) {
     const size_t row_b = (size_t)kv->head_dim * kv->elem();
@@ -885,7 +907,37 @@ extern "C" int cai_kv_truncate(cai_kv_t kv, int n)
 {
   CAI_REQUIRE(kv, "cai_kv_truncate: null cache");
   CAI_REQUIRE(n >= 0, "cai_kv_truncate: negative length %d", n);
+  for (int l : kv->len)
+    if (l > n && kv->evict_cap > 0 && l > kv->evict_cap) return set_error(CAI_ERR_STATE, "cai_kv_truncate: %d tokens streamed under eviction, the rows before %d are gone", l, l - (kv->evict_cap - kv->evict_sinks));
   for (auto& l : kv->len) if (l > n) l = n;
+  return CAI_OK;
+}
+
+// Sink + recent-window eviction (TNNetStreamingDecoder.EnableEviction / DisableEviction, neural/neuraldecode.pas:5722-5735).
+int cai::kv_set_eviction(cai_kv_s* kv, int sinks, int recent)
+{
+  const int cap = sinks + recent;
+  if (sinks < 0 || recent < 0 || (cap > 0 && recent < 1)) return set_error(CAI_ERR_INVALID, "eviction: %d sink tokens, recent window %d", sinks, recent);
+  if (cap > kv->max_ctx) return set_error(CAI_ERR_INVALID, "eviction: %d sinks + %d recent exceed the cache's %d rows", sinks, recent, kv->max_ctx);
+  // rows sit at slot = position until the stream passes the cap, so the policy may change freely before that
+  const int limit = std::min(kv->evict_cap > 0 ? kv->evict_cap : kv->max_ctx, cap > 0 ? cap : kv->max_ctx);
+  for (int n : kv->len)
+    if (n > limit) return set_error(CAI_ERR_STATE, "eviction: a sequence already holds %d tokens, past the %d the change allows", n, limit);
+  kv->evict_sinks = cap > 0 ? sinks : 0; kv->evict_cap = cap;
+  return CAI_OK;
+}
+
+extern "C" int cai_kv_set_eviction(cai_kv_t kv, int sink_tokens, int recent_window)
+{
+  CAI_REQUIRE(kv, "cai_kv_set_eviction: null cache");
+  return kv_set_eviction(kv, sink_tokens, recent_window);
+}
+
+extern "C" int cai_kv_rows(cai_kv_t kv, int layer, int* rows_out)
+{
+  CAI_REQUIRE(kv && rows_out, "cai_kv_rows: null argument");
+  CAI_REQUIRE(layer >= 0 && layer < kv->n_layers, "cai_kv_rows: layer %d of %d", layer, kv->n_layers);
+  *rows_out = kv->live(kv->len_at(0, layer));
   return CAI_OK;
 }
 
@@ -948,7 +1000,7 @@ extern "C" int cai_kv_export_layer(cai_kv_t kv, int layer, void* k, void* v, flo
   CAI_REQUIRE(kv && k && v, "cai_kv_export_layer: null argument");
   CAI_REQUIRE(layer >= 0 && layer < kv->n_layers, "cai_kv_export_layer: layer %d of %d", layer, kv->n_layers);
   CAI_REQUIRE(kv->dtype != CAI_KV_I8 || (k_scales && v_scales), "cai_kv_export_layer: an int8 cache needs the scale outputs");
-  return kv_layer_copy(kv, layer, kv->len_at(0, layer), k, v, k_scales, v_scales, 0);
+  return kv_layer_copy(kv, layer, kv->live(kv->len_at(0, layer)), k, v, k_scales, v_scales, 0);
 }
 
 extern "C" int cai_kv_import_layer(cai_kv_t kv, int layer, int len, const void* k, const void* v, const float* k_scales, const float* v_scales)
@@ -956,7 +1008,7 @@ extern "C" int cai_kv_import_layer(cai_kv_t kv, int layer, int len, const void* 
   CAI_READY();
   CAI_REQUIRE(kv && (len == 0 || (k && v)), "cai_kv_import_layer: null argument");
   CAI_REQUIRE(layer >= 0 && layer < kv->n_layers, "cai_kv_import_layer: layer %d of %d", layer, kv->n_layers);
-  CAI_REQUIRE(len >= 0 && len <= kv->max_ctx, "cai_kv_import_layer: %d rows, cache holds %d", len, kv->max_ctx);
+  CAI_REQUIRE(len >= 0 && len <= kv->max_ctx && (kv->evict_cap == 0 || len <= kv->evict_cap), "cai_kv_import_layer: %d rows, cache holds %d", len, kv->evict_cap ? kv->evict_cap : kv->max_ctx);
   CAI_REQUIRE(kv->dtype != CAI_KV_I8 || len == 0 || (k_scales && v_scales), "cai_kv_import_layer: an int8 cache needs the row scales");
   const int rc = kv_layer_copy(kv, layer, len, const_cast<void*>(k), const_cast<void*>(v), const_cast<float*>(k_scales), const_cast<float*>(v_scales), 1);
   if (rc) return rc;
@@ -973,7 +1025,7 @@ extern "C" int cai_attn_decode(cai_kv_t kv, int layer, const float* qkv, int q_h
   CAI_REQUIRE(q_heads > 0 && q_heads % kv->kv_heads == 0, "cai_attn_decode: %d query heads vs %d KV heads", q_heads, kv->kv_heads);
   Context& c = ctx();
   const int len = kv->len_at(0, layer);
-  if (len >= kv->max_ctx) return set_error(CAI_ERR_STATE, "cai_attn_decode: cache full (%d rows)", kv->max_ctx);
+  if (len >= kv->max_ctx && kv->evict_cap == 0) return set_error(CAI_ERR_STATE, "cai_attn_decode: cache full (%d rows)", kv->max_ctx);
   const int hd = kv->head_dim;
   const size_t in_b = (size_t)(q_heads + 2 * kv->kv_heads) * hd * sizeof(float), out_b = (size_t)q_heads * hd * sizeof(float);
   // the kernel rotates/append from a mutable row: always work on a private device copy

@@ -437,7 +437,7 @@ extern "C" int cai_decoder_step(cai_decoder_t d, const int32_t* tokens, const in
   for (int b = 0; b < n_b; b++) {
     CAI_REQUIRE(tokens[b] >= 0 && tokens[b] < c.vocab, "cai_decoder_step: token %d outside vocab %d", tokens[b], c.vocab);
     if (pos[b] != d->kv.len_at(b, 0)) return set_error(CAI_ERR_STATE, "cai_decoder_step: sequence %d is at position %d, got %d", b, d->kv.len_at(b, 0), pos[b]);
-    if (pos[b] >= c.max_ctx) return set_error(CAI_ERR_STATE, "cai_decoder_step: sequence %d reached max_ctx %d", b, c.max_ctx);
+    if (pos[b] >= c.max_ctx && d->kv.evict_cap == 0) return set_error(CAI_ERR_STATE, "cai_decoder_step: sequence %d reached max_ctx %d", b, c.max_ctx);
   }
   Context& cx = ctx();
   for (int b = 0; b < n_b; b++) { d->h_io[b] = tokens[b]; d->h_io[8 + b] = pos[b]; }
@@ -461,7 +461,8 @@ extern "C" int cai_decoder_generate(cai_decoder_t d, int32_t first_token, int po
   int rc = check_ready(d); if (rc) return rc;
   CAI_REQUIRE(first_token >= 0 && first_token < c.vocab, "cai_decoder_generate: token %d outside vocab %d", first_token, c.vocab);
   if (pos != d->kv.len_at(0, 0)) return set_error(CAI_ERR_STATE, "cai_decoder_generate: sequence 0 is at position %d, got %d", d->kv.len_at(0, 0), pos);
-  if (pos + n_tokens > c.max_ctx) return set_error(CAI_ERR_STATE, "cai_decoder_generate: %d tokens from %d exceed max_ctx %d", n_tokens, pos, c.max_ctx);
+  if (d->kv.evict_cap == 0 ? pos + n_tokens > c.max_ctx : n_tokens > c.max_ctx)
+    return set_error(CAI_ERR_STATE, "cai_decoder_generate: %d tokens from %d exceed max_ctx %d", n_tokens, pos, c.max_ctx);
   Context& cx = ctx();
   d->h_io[0] = first_token; d->h_io[8] = pos;
   CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
@@ -483,11 +484,12 @@ extern "C" int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* toke
   CAI_REQUIRE(seq >= 0 && seq < c.max_batch, "cai_decoder_prefill: sequence %d of %d", seq, c.max_batch);
   int rc = check_ready(d); if (rc) return rc;
   if (pos0 != d->kv.len_at(seq, 0)) return set_error(CAI_ERR_STATE, "cai_decoder_prefill: sequence %d is at position %d, got %d", seq, d->kv.len_at(seq, 0), pos0);
-  if (pos0 + n > c.max_ctx) return set_error(CAI_ERR_STATE, "cai_decoder_prefill: %d tokens from %d exceed max_ctx %d", n, pos0, c.max_ctx);
+  if (pos0 + n > c.max_ctx && d->kv.evict_cap == 0) return set_error(CAI_ERR_STATE, "cai_decoder_prefill: %d tokens from %d exceed max_ctx %d", n, pos0, c.max_ctx);
   for (int i = 0; i < n; i++) CAI_REQUIRE(tokens[i] >= 0 && tokens[i] < c.vocab, "cai_decoder_prefill: token %d outside vocab %d", tokens[i], c.vocab);
   Context& cx = ctx();
   const char* tok_env = getenv("CAIHIP_PREFILL_TOKENWISE");
-  const bool tokenwise = c.n_experts > 0 || n == 1 || (tok_env && tok_env[0] == '1');
+  // (a prompt that runs past the eviction cap overwrites ring rows its own earlier tokens still need: token by token then)
+  const bool tokenwise = c.n_experts > 0 || n == 1 || (tok_env && tok_env[0] == '1') || (d->kv.evict_cap > 0 && pos0 + n > d->kv.evict_cap);
   if (tokenwise) {
     // Token-at-a-time ingestion, the reference's own prefill (neural/neuralchatengine.pas:1466-1470).
     for (int i = 0; i < n; i++) {
@@ -537,7 +539,49 @@ extern "C" int cai_decoder_truncate(cai_decoder_t d, int seq, int n)
 {
   CAI_REQUIRE(d, "cai_decoder_truncate: null decoder");
   CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch && n >= 0, "cai_decoder_truncate: bad argument");
+  const int have = d->kv.len_at(seq, 0);
+  if (have > n && d->kv.evict_cap > 0 && have > d->kv.evict_cap)
+    return set_error(CAI_ERR_STATE, "cai_decoder_truncate: %d tokens streamed under eviction, the rows before %d are gone", have, have - (d->kv.evict_cap - d->kv.evict_sinks));
   for (int l = 0; l < d->cfg.n_layers; l++) if (d->kv.len_at(seq, l) > n) d->kv.len_at(seq, l) = n;
+  return CAI_OK;
+}
+
+extern "C" int cai_decoder_set_eviction(cai_decoder_t d, int sink_tokens, int recent_window)
+{
+  CAI_REQUIRE(d, "cai_decoder_set_eviction: null decoder");
+  const int rc = kv_set_eviction(&d->kv, sink_tokens, recent_window);
+  if (rc) return rc;
+  (void)hipStreamSynchronize(ctx().stream);
+  invalidate_graphs(d);       // captured steps carry the policy in their kernel arguments
+  return CAI_OK;
+}
+
+// EnableInt8KVCache / DisableInt8KVCache (neural/neuraldecode.pas:1277-1290): the storage mode of an empty session.
+extern "C" int cai_decoder_set_kv_dtype(cai_decoder_t d, int kv_dtype)
+{
+  CAI_READY();
+  CAI_REQUIRE(d, "cai_decoder_set_kv_dtype: null decoder");
+  CAI_REQUIRE(kv_dtype == CAI_KV_F32 || kv_dtype == CAI_KV_F16 || kv_dtype == CAI_KV_I8, "cai_decoder_set_kv_dtype: type %d", kv_dtype);
+  for (int n : d->kv.len)
+    if (n > 0) return set_error(CAI_ERR_STATE, "cai_decoder_set_kv_dtype: the cache holds %d tokens; the storage mode only changes on an empty session", n);
+  if (kv_dtype == d->kv.dtype) return CAI_OK;
+  (void)hipStreamSynchronize(ctx().stream);
+  invalidate_graphs(d);
+  const cai_decoder_config& c = d->cfg;
+  const int sinks = d->kv.evict_sinks, cap = d->kv.evict_cap;
+  kv_free(&d->kv);
+  const int rc = kv_alloc(&d->kv, c.max_batch, c.n_layers, c.n_kv_heads, c.head_dim, c.max_ctx, kv_dtype);
+  if (rc) return rc;
+  d->kv.evict_sinks = sinks; d->kv.evict_cap = cap;
+  d->cfg.kv_dtype = kv_dtype;
+  return CAI_OK;
+}
+
+extern "C" int cai_decoder_cache_rows(cai_decoder_t d, int seq, int layer, int* rows_out)
+{
+  CAI_REQUIRE(d && rows_out, "cai_decoder_cache_rows: null argument");
+  CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch && layer >= 0 && layer < d->cfg.n_layers, "cai_decoder_cache_rows: sequence %d, layer %d", seq, layer);
+  *rows_out = d->kv.live(d->kv.len_at(seq, layer));
   return CAI_OK;
 }
 

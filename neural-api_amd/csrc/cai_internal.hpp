@@ -71,7 +71,9 @@ struct cai_kv_s {
   int n_seq = 1, n_layers = 0, kv_heads = 0, head_dim = 0, max_ctx = 0, dtype = 0;
   void* k = nullptr; void* v = nullptr;   // [seq][layer][kv_head][max_ctx][head_dim]
   float* ks = nullptr; float* vs = nullptr;   // CAI_KV_I8 only: one scale per cached row, [seq][layer][kv_head][max_ctx]
-  std::vector<int> len;                   // [seq][layer] live rows (host mirror)
+  std::vector<int> len;                   // [seq][layer] stream position = tokens appended so far (host mirror)
+  int evict_sinks = 0, evict_cap = 0;     // cap > 0: sink + recent-window eviction, at most cap rows are cached
+  int live(int n) const { return evict_cap > 0 && n > evict_cap ? evict_cap : n; }   // cached rows after n tokens
   int split_len = 64, n_splits = 1;       // split-K geometry of the decode kernel (fixed at creation)
   float* part = nullptr;                  // [seq][q_head][split][head_dim+2] split-K partials
   int part_q_heads = 0;
@@ -87,6 +89,7 @@ struct cai_kv_s {
 
 struct cai_kv_snap_s {
   int n_layers = 0, kv_heads = 0, head_dim = 0, dtype = 0, rows = 0;
+  int evict_sinks = 0, evict_cap = 0;     // the eviction policy the rows were laid out under
   std::vector<int> len;                   // per layer
   void* k = nullptr; void* v = nullptr;   // [layer][kv_head][rows][head_dim]
   float* ks = nullptr; float* vs = nullptr;   // [layer][kv_head][rows] row scales of an int8 cache
@@ -136,6 +139,7 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
                      int prompt_rows = 0, float* prompt_part = nullptr);
 int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, int max_ctx, int dtype);
 void kv_free(cai_kv_s* kv);
+int kv_set_eviction(cai_kv_s* kv, int sinks, int recent);
 int kv_snapshot(cai_kv_s* kv, int seq, cai_kv_snap_s** out);
 int kv_restore(cai_kv_s* kv, int seq, const cai_kv_snap_s* snap);
 // multi-token linear layer (matrix cores for Q4_K, small-batch kernel otherwise); gain != null fuses RMSNorm

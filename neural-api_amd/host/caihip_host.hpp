@@ -7,7 +7,8 @@
 //       FinishAndLoadResult -> block and write NumAs*NumBs floats laid out [b*NumAs + a].
 //       Errors are reported through ErrorProc and the call returns a code; nothing is thrown (957-969).
 //   TNNetStreamingDecoder    (neural/neuraldecode.pas:1210-1333, 5696-5843): session over a whole decoder.
-//       Reset, StepForward(window, AbsPos), TruncateTo, Snapshot / RestoreSnapshot, SDPACacheLength, Output.
+//       Reset, StepForward(window, AbsPos), TruncateTo, Snapshot / RestoreSnapshot, EnableEviction / DisableEviction,
+//       SDPACacheLength, Output.
 //       Importer-level failures raise (EPretrainedImportError / EGGUFError in the reference): here CaiError.
 #pragma once
 #include <caihip.h>
@@ -120,7 +121,13 @@ class TNNetStreamingDecoder {
     else Check(cai_decoder_prefill(d_, 0, Tokens, Count, AbsPos, logits_.data(), &argmax_));
   }
   void TruncateTo(int CommittedLen) { Check(cai_decoder_truncate(d_, 0, CommittedLen)); }
-  int SDPACacheLength(int /*Index*/ = 0) const { int n = 0; Check(cai_decoder_len(d_, 0, &n)); return n; }
+  int SDPACacheLength(int Index = 0) const { int n = 0; Check(cai_decoder_cache_rows(d_, 0, Index, &n)); return n; }
+  // neural/neuraldecode.pas:5722-5735
+  void EnableEviction(int SinkTokens, int RecentWindow) { Check(cai_decoder_set_eviction(d_, SinkTokens, RecentWindow)); }
+  void DisableEviction() { Check(cai_decoder_set_eviction(d_, 0, 0)); }
+  // neural/neuraldecode.pas:1277-1290: only on a fresh session
+  void EnableInt8KVCache() { Check(cai_decoder_set_kv_dtype(d_, CAI_KV_I8)); }
+  void DisableInt8KVCache() { Check(cai_decoder_set_kv_dtype(d_, CAI_KV_F32)); }
   TNNetDecoderSessionSnapshot* Snapshot() { cai_kv_snap_t s = nullptr; Check(cai_decoder_snapshot(d_, 0, &s)); return new TNNetDecoderSessionSnapshot(s); }
   void RestoreSnapshot(const TNNetDecoderSessionSnapshot* Snap) { Check(cai_decoder_restore(d_, 0, Snap->handle())); }
   const std::vector<float>& Output() const { return logits_; }

@@ -77,6 +77,8 @@ function cai_kv_len(kv: TCaiKV; layer: LongInt; len_out: PLongInt): LongInt; cde
 function cai_kv_snapshot(kv: TCaiKV; out_snap: PCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;
 function cai_kv_restore(kv: TCaiKV; snap: TCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;
 function cai_kv_snap_destroy(snap: TCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;
+function cai_kv_set_eviction(kv: TCaiKV; sink_tokens, recent_window: LongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_kv_rows(kv: TCaiKV; layer: LongInt; rows_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_kv_export_layer(kv: TCaiKV; layer: LongInt; k, v: Pointer; k_scales, v_scales: PSingle): LongInt; cdecl; external CAIHIP_LIB;
 function cai_kv_import_layer(kv: TCaiKV; layer, len: LongInt; k, v: Pointer; k_scales, v_scales: PSingle): LongInt; cdecl; external CAIHIP_LIB;
 function cai_attn_decode(kv: TCaiKV; layer: LongInt; qkv: PSingle; q_heads, window: LongInt; softcap: Single; out_f: PSingle; flags: LongInt): LongInt; cdecl; external CAIHIP_LIB;
@@ -91,6 +93,9 @@ function cai_decoder_prefill(d: TCaiDecoder; seq: LongInt; tokens: PLongInt; n, 
 function cai_decoder_reset(d: TCaiDecoder; seq: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_truncate(d: TCaiDecoder; seq, n: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_len(d: TCaiDecoder; seq: LongInt; len_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_decoder_set_eviction(d: TCaiDecoder; sink_tokens, recent_window: LongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_decoder_set_kv_dtype(d: TCaiDecoder; kv_dtype: LongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_decoder_cache_rows(d: TCaiDecoder; seq, layer: LongInt; rows_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_snapshot(d: TCaiDecoder; seq: LongInt; out_snap: PCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_restore(d: TCaiDecoder; seq: LongInt; snap: TCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_weight_bytes(d: TCaiDecoder; algorithmic_bytes_out: PInt64): LongInt; cdecl; external CAIHIP_LIB;

@@ -489,11 +489,24 @@ int orc_argmax(const float* x, int n)
 
 static float round_half(float v) { return orc_f16_to_f32(orc_f32_to_f16(v)); }
 
+/* Live rows after `len` tokens: all of [j0, len) under a sliding window; under sink + recent-window eviction
+ * (neuraldecode.pas:1257-1276: the first `sinks` positions and the latest `recent` are kept, the middle is gone, keys
+ * keep their own rotation) positions [0, sinks) and [len - recent, len) once len exceeds sinks + recent.  The oracle
+ * keeps every row and masks by position, so it states the policy, not a storage scheme.
+ * Pinned by: within the cap identical to the unbounded run, row count pinned at the cap past it
+ * (tests/TestNeuralDecode.pas:3863-3990), brute-force softmax over the stated set. */
+static int row_live(int j, int len, int window, int sinks, int recent)
+{
+  if (sinks + recent > 0 && len > sinks + recent) return j < sinks || j >= len - recent;
+  const int j0 = (window > 0 && len > window) ? len - window : 0;
+  return j >= j0;
+}
+
 /* neural.cl:2354-2379 (append) + 2406-2499 (decode): scores q.K_j/sqrt(dk) (+softcap), max,
  * exp-shift, normaliser, out = (sum_j e_j V_j) * (1/sum).
  * Pinned by: tiny_*_logits.json through orc_model_step; brute-force softmax identity. */
-void orc_attn_decode(const float* qkv, int hq, int hkv, int dk, float* kc, float* vc, int max_ctx,
-                     int cache_len, int window, float softcap, int kv_f16, float* out)
+static void attn_core_f32(const float* qkv, int hq, int hkv, int dk, float* kc, float* vc, int max_ctx,
+                          int cache_len, int window, int sinks, int recent, float softcap, int kv_f16, float* out)
 {
   const int qw = hq * dk, kw = hkv * dk, group = hq / hkv;
   for (int g = 0; g < hkv; g++)
@@ -504,14 +517,14 @@ void orc_attn_decode(const float* qkv, int hq, int hkv, int dk, float* kc, float
       vc[((int64_t)g * max_ctx + cache_len) * dk + d] = v;
     }
   const int len = cache_len + 1;
-  const int j0 = (window > 0 && len > window) ? len - window : 0;
   const float inv_sqrt = 1.0f / sqrtf((float)dk);
   float* sc = (float*)malloc((size_t)len * sizeof(float));
   for (int h = 0; h < hq; h++) {
     const int g = h / group;
     const float* q = qkv + h * dk;
     float m = -1e30f;
-    for (int j = j0; j < len; j++) {
+    for (int j = 0; j < len; j++) {
+      if (!row_live(j, len, window, sinks, recent)) continue;
       const float* kr = kc + ((int64_t)g * max_ctx + j) * dk;
       float acc = 0;
       for (int d = 0; d < dk; d++) acc = fmaf(q[d], kr[d], acc);
@@ -520,15 +533,28 @@ void orc_attn_decode(const float* qkv, int hq, int hkv, int dk, float* kc, float
       sc[j] = s; if (s > m) m = s;
     }
     float sum = 0;
-    for (int j = j0; j < len; j++) { sc[j] = expf(sc[j] - m); sum += sc[j]; }
+    for (int j = 0; j < len; j++) if (row_live(j, len, window, sinks, recent)) { sc[j] = expf(sc[j] - m); sum += sc[j]; }
     const float inv = sum > 0 ? 1.0f / sum : 0;
     for (int d = 0; d < dk; d++) {
       float acc = 0;
-      for (int j = j0; j < len; j++) acc = fmaf(sc[j], vc[((int64_t)g * max_ctx + j) * dk + d], acc);
+      for (int j = 0; j < len; j++)
+        if (row_live(j, len, window, sinks, recent)) acc = fmaf(sc[j], vc[((int64_t)g * max_ctx + j) * dk + d], acc);
       out[h * dk + d] = acc * inv;
     }
   }
   free(sc);
+}
+
+void orc_attn_decode(const float* qkv, int hq, int hkv, int dk, float* kc, float* vc, int max_ctx,
+                     int cache_len, int window, float softcap, int kv_f16, float* out)
+{
+  attn_core_f32(qkv, hq, hkv, dk, kc, vc, max_ctx, cache_len, window, 0, 0, softcap, kv_f16, out);
+}
+
+void orc_attn_decode_evict(const float* qkv, int hq, int hkv, int dk, float* kc, float* vc, int max_ctx,
+                           int cache_len, int sinks, int recent, float softcap, int kv_f16, float* out)
+{
+  attn_core_f32(qkv, hq, hkv, dk, kc, vc, max_ctx, cache_len, 0, sinks, recent, softcap, kv_f16, out);
 }
 
 /* neural.cl:2501-2580 (cai_sdpa_append_kv_int8), the device statement of the host's
@@ -731,7 +757,7 @@ int orc_model_step(orc_model* m, int token, int pos, float* logits)
     orc_rope_interleaved(m->qkv, c->n_q_heads, hd, pos, m->theta);
     orc_rope_interleaved(m->qkv + qw, c->n_kv_heads, hd, pos, m->theta);
     if (c->kv_f16 == 2) orc_attn_decode_i8(m->qkv, c->n_q_heads, c->n_kv_heads, hd, ly->kq, ly->ks, ly->vq, ly->vs, c->max_ctx, pos, c->window, 0.0f, m->att);
-    else orc_attn_decode(m->qkv, c->n_q_heads, c->n_kv_heads, hd, ly->kc, ly->vc, c->max_ctx, pos, c->window, 0.0f, c->kv_f16, m->att);
+    else attn_core_f32(m->qkv, c->n_q_heads, c->n_kv_heads, hd, ly->kc, ly->vc, c->max_ctx, pos, c->window, c->evict_sinks, c->evict_recent, 0.0f, c->kv_f16, m->att);
     lin(m, &ly->w[ORC_W_O], 0, d, m->att, m->tmp);
     for (int i = 0; i < d; i++) m->x[i] += m->tmp[i];
     orc_rmsnorm(m->x, ly->v[ORC_V_MLP_NORM], d, c->eps, m->h);

@@ -78,6 +78,12 @@ void orc_attn_decode(const float* qkv, int q_heads, int kv_heads, int head_dim,
                      float* k_cache, float* v_cache, int max_ctx, int cache_len,
                      int window, float softcap, int kv_f16, float* out);
 
+/* The same under sink + recent-window eviction (neuraldecode.pas:1257-1276); the caches stay unbounded (max_ctx rows
+ * must cover the whole stream), rows outside [0, sinks) u [len - recent, len) are masked once len > sinks + recent. */
+void orc_attn_decode_evict(const float* qkv, int q_heads, int kv_heads, int head_dim,
+                           float* k_cache, float* v_cache, int max_ctx, int cache_len,
+                           int sinks, int recent, float softcap, int kv_f16, float* out);
+
 /* ---- int8 KV cache: per-row symmetric codes + fp32 scale (neural.cl:2501-2687) ----
  * codes [kv_heads][max_ctx][head_dim], scales [kv_heads][max_ctx]. */
 float orc_max_abs_finite(const float* x, int n);                                     /* neuralvolume.pas:12471 */
@@ -97,6 +103,7 @@ typedef struct {
   int32_t n_experts, top_k, norm_topk; /* n_experts == 0 -> dense SwiGLU FFN */
   int32_t kv_f16;         /* cache element model: 0 fp32, 1 rounded to half, 2 int8 codes + row scale */
   int32_t acc64;          /* accumulate linear layers in double */
+  int32_t evict_sinks, evict_recent; /* sink + recent-window eviction (0, 0 = off); max_ctx must still cover the stream */
 } orc_config;
 
 /* tensor slots */

@@ -17,7 +17,7 @@ V_ATTN_NORM, V_MLP_NORM, V_FINAL_NORM, V_Q_NORM, V_K_NORM = range(5)
 class OrcConfig(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("n_layers", "d_model", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab", "max_ctx")] + \
                [("eps", C.c_float), ("rope_theta", C.c_float)] + \
-               [(n, C.c_int32) for n in ("window", "qk_norm_full", "n_experts", "top_k", "norm_topk", "kv_f16", "acc64")]
+               [(n, C.c_int32) for n in ("window", "qk_norm_full", "n_experts", "top_k", "norm_topk", "kv_f16", "acc64", "evict_sinks", "evict_recent")]
 
 
 def _p(a, t=C.c_void_p):
@@ -51,6 +51,8 @@ def lib():
         L.orc_q4k_scale_min.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]; L.orc_q4k_scale_min.restype = None
         L.orc_attn_decode.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int, C.c_void_p]
         L.orc_attn_decode.restype = None
+        L.orc_attn_decode_evict.restype = None
+        L.orc_attn_decode_evict.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int, C.c_void_p]
         L.orc_max_abs_finite.restype = C.c_float; L.orc_max_abs_finite.argtypes = [C.c_void_p, C.c_int]
         L.orc_kv_quant_row.restype = None; L.orc_kv_quant_row.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
         L.orc_attn_decode_i8.restype = None

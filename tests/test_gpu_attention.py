@@ -218,3 +218,69 @@ def test_int8_cache_snapshot_restore_and_layer_import_export():
         b.import_layer(0, *a.export_layer(0)[:2])
         for p in range(12, 20):
             assert np.array_equal(b.attn_decode(0, rows[p], hq), ref[p])
+
+
+def oracle_run_evict(rows, hq, hkv, dk, sinks, recent, kv_f16=0):
+    n = rows.shape[0]
+    kc = np.zeros((hkv, n, dk), np.float32); vc = np.zeros_like(kc)
+    outs = []
+    for pos in range(n):
+        out = np.zeros(hq * dk, np.float32)
+        O.lib().orc_attn_decode_evict(rows[pos].ctypes.data, hq, hkv, dk, kc.ctypes.data, vc.ctypes.data, n, pos, sinks, recent, 0.0, kv_f16, out.ctypes.data)
+        outs.append(out)
+    return np.array(outs)
+
+
+@pytest.mark.parametrize("hq,hkv,dk,ctx,sinks,recent", [(4, 2, 64, 16, 2, 4), (28, 4, 128, 128, 4, 90), (32, 16, 128, 1024, 3, 300), (6, 2, 4, 64, 0, 33)])
+def test_sink_and_window_eviction_matches_oracle_past_max_ctx(hq, hkv, dk, ctx, sinks, recent):
+    """EnableEviction (neural/neuraldecode.pas:1257-1276, tests/TestNeuralDecode.pas:3863-3990): bit-identical to the
+    unbounded cache up to the cap, rows pinned at the cap beyond it, and the stream runs past max_ctx.  The third shape
+    takes the one-work-group-per-KV-head kernel, the others the per-query-head kernel."""
+    from helpers.device import dev
+    cai = dev()
+    rng = np.random.default_rng(ctx + sinks)
+    cap = sinks + recent
+    n = max(ctx + 40, 2 * cap + 7) if ctx <= 128 else cap + 150
+    rows = rng.standard_normal((n, (hq + 2 * hkv) * dk)).astype(np.float32)
+    want = oracle_run_evict(rows, hq, hkv, dk, sinks, recent)
+    plain = cai.KVCache(1, hkv, dk, ctx); ev = cai.KVCache(1, hkv, dk, ctx); ev.set_eviction(sinks, recent)
+    for pos in range(n):
+        got = ev.attn_decode(0, rows[pos], hq)
+        if pos < cap:
+            assert np.array_equal(got, plain.attn_decode(0, rows[pos], hq)), pos
+        assert np.max(np.abs(got - want[pos])) < 1e-5, pos
+        assert ev.rows(0) == min(pos + 1, cap) and ev.len(0) == pos + 1
+    with pytest.raises(cai.CaiError):
+        ev.truncate(cap)                     # the evicted middle cannot come back
+    with pytest.raises(cai.CaiError):
+        ev.set_eviction(0, 0)                # nor can the policy change once the stream is past the cap
+    with pytest.raises(cai.CaiError):
+        plain.set_eviction(ctx, 1)           # sinks + recent must fit the cache
+    # snapshot / restore keeps the ring: the continuation replays exactly
+    snap = ev.snapshot()
+    more = rng.standard_normal((9, rows.shape[1])).astype(np.float32)
+    a = [ev.attn_decode(0, r, hq) for r in more]
+    ev.restore(snap)
+    assert ev.len(0) == n
+    b = [ev.attn_decode(0, r, hq) for r in more]
+    assert all(np.array_equal(x, y) for x, y in zip(a, b))
+    with pytest.raises(cai.CaiError):
+        plain.restore(snap)                  # a snapshot taken under another policy
+    cai.load().cai_kv_snap_destroy(snap)
+
+
+def test_eviction_int8_cache_tracks_fp32_cache():
+    # tests/TestNeuralDecode.pas:3980-4060: both evict the same positions, so the outputs differ by int8 drift only
+    from helpers.device import dev
+    cai = dev()
+    rng = np.random.default_rng(8)
+    hq, hkv, dk, sinks, recent, n = 8, 2, 64, 2, 12, 90
+    rows = rng.standard_normal((n, (hq + 2 * hkv) * dk)).astype(np.float32)
+    f = cai.KVCache(1, hkv, dk, 32); q = cai.KVCache(1, hkv, dk, 32, cai.KV_I8)
+    f.set_eviction(sinks, recent); q.set_eviction(sinks, recent)
+    drift = 0.0
+    for pos in range(n):
+        a = f.attn_decode(0, rows[pos], hq); b = q.attn_decode(0, rows[pos], hq)
+        drift = max(drift, float(np.max(np.abs(a - b))))
+    assert 0 < drift < 5e-2
+    assert q.rows(0) == sinks + recent

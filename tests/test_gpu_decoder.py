@@ -213,3 +213,52 @@ def test_int8_kv_cache_decoder():
     assert all(np.array_equal(x, y) for x, y in zip(a, b))
     assert all(np.array_equal(x, y) for x, y in zip(a, steps[20:30]))
     cai.load().cai_kv_snap_destroy(snap)
+
+
+def test_streaming_eviction_session_runs_past_max_ctx():
+    """TNNetStreamingDecoder.EnableEviction (neural/neuraldecode.pas:1257-1276): logits follow the oracle's position
+    mask while the stream runs to three times max_ctx; generate, prefill and the int8 cache work under it."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    s = SHAPES["llama_like_q4_0"]
+    cfg = dict(s["cfg"]); cfg["max_ctx"] = 48
+    spec = synthetic_spec(cfg, s["qtype"], std=0.05)
+    sinks, recent, n = 4, 36, 150
+    rng = np.random.default_rng(99)
+    toks = rng.integers(0, cfg["vocab"], n).tolist()
+    om = oracle_model(spec, acc64=1, max_ctx=n + 8, evict_sinks=sinks, evict_recent=recent)
+    dec = cai.Decoder(spec, max_batch=2)
+    dec.set_eviction(sinks, recent)
+    worst = 0.0
+    for p, t in enumerate(toks):
+        _, lo = om.step(t, p); _, ld = dec.step(t, p)
+        worst = max(worst, rel_err(ld[0], lo))
+        assert dec.cache_rows(0, 1) == min(p + 1, sinks + recent) and dec.len() == p + 1
+    assert worst < 1e-3, worst
+    # chained greedy generation under eviction == step loop
+    snap = dec.snapshot()
+    gen = dec.generate(toks[-1] % cfg["vocab"], n, 30)
+    dec.restore(snap)
+    tok, seq = toks[-1] % cfg["vocab"], []
+    for i in range(30):
+        am, _ = dec.step(tok, n + i, want_logits=False)
+        tok = int(am[0]); seq.append(tok)
+    assert seq == gen.tolist()
+    cai.load().cai_kv_snap_destroy(snap)
+    # a prompt longer than the cap is ingested token by token and lands on the same logits
+    _, last = dec.prefill(toks[:100], 0, seq=1)
+    om2 = oracle_model(spec, acc64=1, max_ctx=n + 8, evict_sinks=sinks, evict_recent=recent)
+    for p, t in enumerate(toks[:100]):
+        _, lo = om2.step(t, p)
+    assert rel_err(last, lo) < 1e-3
+    # storage mode switch on a fresh session only (EnableInt8KVCache)
+    with pytest.raises(cai.CaiError):
+        dec.set_kv_dtype(cai.KV_I8)
+    dec.reset(0); dec.reset(1)
+    dec.set_kv_dtype(cai.KV_I8)
+    drift = 0.0
+    om3 = oracle_model(spec, acc64=1, max_ctx=n + 8, evict_sinks=sinks, evict_recent=recent)
+    for p, t in enumerate(toks[:80]):
+        _, lo = om3.step(t, p); _, ld = dec.step(t, p)
+        drift = max(drift, rel_err(ld[0], lo))
+    assert drift < 5e-2, drift

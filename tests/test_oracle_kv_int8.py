@@ -125,3 +125,29 @@ def test_int8_decode_brute_force_softmax():
             s = K[g] @ row[h * dk:(h + 1) * dk].astype(np.float64) / np.sqrt(dk)
             w = np.exp(s - s.max()); w /= w.sum()
             np.testing.assert_allclose(out[h * dk:(h + 1) * dk], w @ V[g], rtol=1e-4, atol=1e-5)
+
+
+def test_eviction_mask_within_cap_identical_and_past_cap_brute_force():
+    """Sink + recent-window eviction as the oracle states it (neural/neuraldecode.pas:1257-1276): up to the cap the run
+    is bit-identical to the unbounded one (tests/TestNeuralDecode.pas:3863-3915); past it the output is the softmax over
+    positions [0, sinks) and the latest `recent`."""
+    rng = np.random.default_rng(17)
+    hq, hkv, dk, n, sinks, recent = 4, 2, 8, 20, 2, 4
+    rows = rng.standard_normal((n, (hq + 2 * hkv) * dk)).astype(np.float32)
+    kc = np.zeros((hkv, n, dk), np.float32); vc = np.zeros_like(kc)
+    ke = np.zeros_like(kc); ve = np.zeros_like(kc)
+    for pos in range(n):
+        a = np.zeros(hq * dk, np.float32); b = np.zeros_like(a)
+        O.lib().orc_attn_decode(rows[pos].ctypes.data, hq, hkv, dk, kc.ctypes.data, vc.ctypes.data, n, pos, 0, 0.0, 0, a.ctypes.data)
+        O.lib().orc_attn_decode_evict(rows[pos].ctypes.data, hq, hkv, dk, ke.ctypes.data, ve.ctypes.data, n, pos, sinks, recent, 0.0, 0, b.ctypes.data)
+        if pos + 1 <= sinks + recent:
+            assert np.array_equal(a, b), pos
+        else:
+            live = list(range(sinks)) + list(range(pos + 1 - recent, pos + 1))
+            assert len(live) == sinks + recent
+            for h in range(hq):
+                g = h // (hq // hkv)
+                s = ke[g, live].astype(np.float64) @ rows[pos, h * dk:(h + 1) * dk].astype(np.float64) / np.sqrt(dk)
+                w = np.exp(s - s.max()); w /= w.sum()
+                np.testing.assert_allclose(b[h * dk:(h + 1) * dk], w @ ve[g, live].astype(np.float64), rtol=1e-5, atol=1e-6)
+            assert not np.allclose(a, b)
