@@ -226,6 +226,22 @@ int cai_decoder_generate(cai_decoder_t d, int32_t first_token, int pos, int n_to
 int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* tokens, int n, int pos0,
                         float* last_logits, int32_t* argmax);
 /* Session management (neural/neuraldecode.pas:5714-5843): always safe after a failed step. */
+/* ---- distribution pipeline ahead of the samplers, on the device ----
+ * The non-greedy branch of TChatEngine.GenerateFromIds (neural/neuralchatengine.pas:1374-1396, 1495-1501): RowSoftMax ->
+ * TNNetPenaltyProcessor (ApplyToProbabilities, neural/neuralvolume.pas:5335-5376) -> TNNetTemperatureProcessor
+ * (neural/neuraldecode.pas:4710-4754) -> the candidate prefix the samplers draw from (SelectTopCandidates +
+ * SortTokenArray, neural/neuralvolume.pas:5171-5196): the m <= 1024 most probable tokens, descending, equal
+ * probabilities by token id.  hist_ids / hist_counts: the DISTINCT tokens of the context and how often each occurred
+ * (TNNetTokenHistoryPenalty's FSeen / FCounts); repetition 1, frequency 0, presence 0, temperature 1 are no-ops.
+ * The draw (uniform over the window for TopK / TopP, weighted for WeightedTopK / MinP) stays with the host and its
+ * random generator.  *count_out = min(m, n).  cai_decoder_candidates reads logits row `row` of the session's last
+ * step in place (no read-back of the row); cai_sample_candidates takes any row (CAI_X_DEVICE: a device pointer). */
+int cai_sample_candidates(const float* logits, int n, const int32_t* hist_ids, const int32_t* hist_counts, int n_hist,
+                          float repetition, float frequency, float presence, float temperature, int m,
+                          int32_t* tokens_out, float* probs_out, int* count_out, int flags);
+int cai_decoder_candidates(cai_decoder_t d, int row, const int32_t* hist_ids, const int32_t* hist_counts, int n_hist,
+                           float repetition, float frequency, float presence, float temperature, int m,
+                           int32_t* tokens_out, float* probs_out, int* count_out);
 int cai_decoder_reset(cai_decoder_t d, int seq);
 int cai_decoder_truncate(cai_decoder_t d, int seq, int n);
 int cai_decoder_len(cai_decoder_t d, int seq, int* len_out);   /* tokens streamed so far = the next position */

@@ -20,7 +20,7 @@ cai_qw_create cai_qw_create_int8row cai_qw_destroy cai_qw_info cai_qw_dequant_ro
 cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_router_topk
 cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_kv_export_layer cai_kv_import_layer cai_kv_set_eviction cai_kv_rows cai_attn_decode
 cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_generate
-cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_set_eviction cai_decoder_cache_rows cai_decoder_set_kv_dtype cai_decoder_snapshot cai_decoder_restore
+cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_set_eviction cai_decoder_cache_rows cai_decoder_set_kv_dtype cai_sample_candidates cai_decoder_candidates cai_decoder_snapshot cai_decoder_restore
 cai_decoder_weight_bytes cai_decoder_get_config cai_decoder_load_gguf
 cai_gguf_open cai_gguf_close cai_gguf_info cai_gguf_meta_int cai_gguf_meta_float cai_gguf_meta_str cai_gguf_meta_array_count
 cai_gguf_meta_array_str cai_gguf_find_tensor cai_gguf_tensor_info cai_gguf_tensor_data cai_gguf_load_qw""".split()
@@ -98,6 +98,8 @@ def load():
         L.cai_decoder_len.argtypes = [vp, i32, C.POINTER(i32)]
         L.cai_decoder_set_eviction.argtypes = [vp, i32, i32]
         L.cai_decoder_set_kv_dtype.argtypes = [vp, i32]
+        L.cai_sample_candidates.argtypes = [vp, i32, vp, vp, i32, C.c_float, C.c_float, C.c_float, C.c_float, i32, vp, vp, C.POINTER(i32), i32]
+        L.cai_decoder_candidates.argtypes = [vp, i32, vp, vp, i32, C.c_float, C.c_float, C.c_float, C.c_float, i32, vp, vp, C.POINTER(i32)]
         L.cai_decoder_cache_rows.argtypes = [vp, i32, i32, C.POINTER(i32)]
         L.cai_decoder_snapshot.argtypes = [vp, i32, C.POINTER(vp)]
         L.cai_decoder_restore.argtypes = [vp, i32, vp]
@@ -206,6 +208,21 @@ class QWeight:
             self.close()
         except Exception:
             pass
+
+
+def _history(history):
+    if history is None or len(history) == 0:
+        return np.zeros(0, np.int32), np.zeros(0, np.int32)
+    ids, counts = np.unique(np.asarray(history, np.int32), return_counts=True)
+    return np.ascontiguousarray(ids, np.int32), np.ascontiguousarray(counts, np.int32)
+
+
+def sample_candidates(logits, m, temperature=1.0, history=None, repetition=1.0, frequency=0.0, presence=0.0):
+    logits = np.ascontiguousarray(logits, np.float32)
+    ids, counts = _history(history)
+    tok = np.zeros(m, np.int32); p = np.zeros(m, np.float32); k = C.c_int()
+    check(load().cai_sample_candidates(_ptr(logits), logits.size, _ptr(ids), _ptr(counts), ids.size, repetition, frequency, presence, temperature, m, _ptr(tok), _ptr(p), C.byref(k), 0))
+    return tok[:k.value], p[:k.value]
 
 
 class KVCache:
@@ -415,6 +432,12 @@ class Decoder:
 
     def set_eviction(self, sinks, recent):
         check(load().cai_decoder_set_eviction(self.h, sinks, recent))
+
+    def candidates(self, m, row=0, temperature=1.0, history=None, repetition=1.0, frequency=0.0, presence=0.0):
+        ids, counts = _history(history)
+        tok = np.zeros(m, np.int32); p = np.zeros(m, np.float32); k = C.c_int()
+        check(load().cai_decoder_candidates(self.h, row, _ptr(ids), _ptr(counts), ids.size, repetition, frequency, presence, temperature, m, _ptr(tok), _ptr(p), C.byref(k)))
+        return tok[:k.value], p[:k.value]
 
     def set_kv_dtype(self, dtype):
         check(load().cai_decoder_set_kv_dtype(self.h, dtype))

@@ -527,6 +527,19 @@ extern "C" int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* toke
   return CAI_OK;
 }
 
+// The sampled (non-greedy) branch of the decode loop without the logits read-back (neural/neuralchatengine.pas:1495-1501).
+extern "C" int cai_decoder_candidates(cai_decoder_t d, int row, const int32_t* hist_ids, const int32_t* hist_counts, int n_hist,
+                                      float repetition, float frequency, float presence, float temperature, int m,
+                                      int32_t* tokens_out, float* probs_out, int* count_out)
+{
+  CAI_READY();
+  CAI_REQUIRE(d && tokens_out && probs_out, "cai_decoder_candidates: null argument");
+  CAI_REQUIRE(row >= 0 && row < d->cfg.max_batch, "cai_decoder_candidates: row %d of %d", row, d->cfg.max_batch);
+  CAI_REQUIRE(m >= 1 && m <= 1024, "cai_decoder_candidates: %d candidates (1..1024)", m);
+  return run_candidates(d->logits + (int64_t)row * d->cfg.vocab, d->cfg.vocab, hist_ids, hist_counts, n_hist,
+                        repetition, frequency, presence, temperature, m, tokens_out, probs_out, count_out);
+}
+
 extern "C" int cai_decoder_reset(cai_decoder_t d, int seq)
 {
   CAI_REQUIRE(d, "cai_decoder_reset: null decoder");

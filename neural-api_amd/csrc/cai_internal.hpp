@@ -162,5 +162,10 @@ int prefill_gemm(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride, const
 int prefill_gemm_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, float* y, int64_t y_stride);
 
 void rope_thetas(float base, int head_dim, std::vector<float>& out);
+// softmax -> history penalty -> temperature -> the m most probable tokens (descending) of a device-resident logits row;
+// history and results are host arrays
+int run_candidates(const float* logits_dev, int n, const int32_t* hist_ids, const int32_t* hist_counts, int n_hist,
+                   float repetition, float frequency, float presence, float temperature, int m,
+                   int32_t* tokens_out, float* probs_out, int* count_out);
 
 }  // namespace cai

@@ -13,6 +13,7 @@
 #pragma once
 #include <caihip.h>
 
+#include <algorithm>
 #include <cstdint>
 #include <cstdio>
 #include <functional>
@@ -98,6 +99,75 @@ class TNNetDecoderSessionSnapshot {
   cai_kv_snap_t s_;
 };
 
+// The candidate prefix the device hands back (descending probabilities) and the reference's samplers over it.  The
+// draws are the HOST's: u in [0,1) stands where the reference calls Random, so a host keeps its own generator and seed.
+struct TNNetCandidates {
+  std::vector<int32_t> Token;
+  std::vector<float> Score;
+  int Count() const { return (int)Token.size(); }
+};
+
+// TNNetSamplerTopK (neural/neuralvolume.pas:4716-4731): uniform over the K most probable.
+inline int32_t SampleTopK(const TNNetCandidates& c, int TopK, double u)
+{
+  int n = std::min(std::max(TopK, 1), c.Count());
+  if (n <= 0) return 0;
+  return c.Token[(size_t)std::min(n - 1, (int)(u * n))];
+}
+// TNNetSamplerWeightedTopK (4749-4786): proportional to the kept probabilities; TopK <= 0 keeps the whole prefix.
+inline int32_t SampleWeightedTopK(const TNNetCandidates& c, int TopK, double u)
+{
+  if (c.Count() == 0) return 0;
+  int kept = TopK; if (kept <= 0 || kept > c.Count()) kept = c.Count();
+  float sum = 0; for (int i = 0; i < kept; i++) sum += c.Score[(size_t)i];
+  if (sum <= 0) return c.Token[0];
+  const float roll = (float)u * sum; float cum = 0;
+  for (int i = 0; i < kept; i++) { cum += c.Score[(size_t)i]; if (roll < cum) return c.Token[(size_t)i]; }
+  return c.Token[(size_t)kept - 1];
+}
+// TNNetSamplerTopP (4548-4600): the first index whose cumulative mass exceeds TopP bounds a window that is drawn from
+// UNIFORMLY.  Returns -1 when the prefix does not hold TopP of the mass: ask for a wider prefix (the reference re-sorts
+// the whole row in that case) or fall back to the logits row.
+inline int32_t SampleTopP(const TNNetCandidates& c, float TopP, double u)
+{
+  if (c.Count() == 0) return 0;
+  float cum = 0; int threshold = -1;
+  for (int i = 0; i < c.Count(); i++) { cum += c.Score[(size_t)i]; if (cum > TopP) { threshold = i; break; } }
+  if (threshold < 0) return -1;
+  if (threshold == 0) return c.Token[0];
+  return c.Token[(size_t)std::min(threshold - 1, (int)(u * threshold))];
+}
+// TNNetSamplerMinP (4621-4665): keep p >= MinP * max p, weighted draw.  Returns -1 when the whole prefix passes the cut
+// (the kept set may reach beyond it).
+inline int32_t SampleMinP(const TNNetCandidates& c, float MinP, double u, bool PrefixIsWholeRow = false)
+{
+  if (c.Count() == 0) return 0;
+  const float cut = MinP * c.Score[0];
+  int kept = 0; float sum = 0;
+  for (int i = 0; i < c.Count(); i++) { if (c.Score[(size_t)i] >= cut) { kept++; sum += c.Score[(size_t)i]; } else break; }
+  if (kept == c.Count() && !PrefixIsWholeRow) return -1;
+  if (kept == 0 || sum <= 0) return c.Token[0];
+  const float roll = (float)u * sum; float cum = 0;
+  for (int i = 0; i < kept; i++) { cum += c.Score[(size_t)i]; if (roll < cum) return c.Token[(size_t)i]; }
+  return c.Token[(size_t)kept - 1];
+}
+
+// TNNetTokenHistoryPenalty's bookkeeping (neural/neuralvolume.pas:5266-5292): distinct ids + occurrence counts.
+class TNNetTokenHistory {
+ public:
+  void RegisterToken(int32_t TokenId)
+  {
+    if (TokenId < 0) return;
+    for (size_t i = 0; i < ids_.size(); i++) if (ids_[i] == TokenId) { counts_[i]++; return; }
+    ids_.push_back(TokenId); counts_.push_back(1);
+  }
+  void ResetHistory() { ids_.clear(); counts_.clear(); }
+  const std::vector<int32_t>& Ids() const { return ids_; }
+  const std::vector<int32_t>& Counts() const { return counts_; }
+ private:
+  std::vector<int32_t> ids_, counts_;
+};
+
 class TNNetStreamingDecoder {
  public:
   // BuildLlamaFromGGUF + TNNetStreamingDecoder.Create(pNet, pMaxCacheLen): pMaxCacheLen <= 0 takes the file's context length
@@ -132,6 +202,19 @@ class TNNetStreamingDecoder {
   void RestoreSnapshot(const TNNetDecoderSessionSnapshot* Snap) { Check(cai_decoder_restore(d_, 0, Snap->handle())); }
   const std::vector<float>& Output() const { return logits_; }
   int ArgMaxRow() const { return argmax_; }
+  // RowSoftMax -> penalty -> temperature on the device, over the row of the last StepForward; the m most probable
+  // tokens come back instead of the row (neural/neuralchatengine.pas:1495-1501)
+  TNNetCandidates Candidates(int m, float Temperature = 1.0f, const TNNetTokenHistory* History = nullptr,
+                             float RepetitionPenalty = 1.0f, float FrequencyPenalty = 0.0f, float PresencePenalty = 0.0f)
+  {
+    TNNetCandidates c; c.Token.resize((size_t)m); c.Score.resize((size_t)m);
+    int n = 0;
+    Check(cai_decoder_candidates(d_, 0, History ? History->Ids().data() : nullptr, History ? History->Counts().data() : nullptr,
+                                 History ? (int)History->Ids().size() : 0, RepetitionPenalty, FrequencyPenalty, PresencePenalty,
+                                 Temperature, m, c.Token.data(), c.Score.data(), &n));
+    c.Token.resize((size_t)n); c.Score.resize((size_t)n);
+    return c;
+  }
   // Greedy fast path of the chat engine (neural/neuralchatengine.pas:1493-1494): n tokens chained on the device.
   std::vector<int32_t> GenerateGreedy(int32_t FirstToken, int AbsPos, int n)
   {

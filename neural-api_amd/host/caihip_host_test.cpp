@@ -88,6 +88,60 @@ int main(int argc, char** argv)
       for (int k = 0; k < 6; k++) { dec.StepForward(&t, 1, 4 + k); t = dec.ArgMaxRow(); host_chain.push_back(t); }
       dec.TruncateTo(4);
       EXPECT(dec.GenerateGreedy(first, 4, 6) == host_chain);
+      // sampled decode: the candidate prefix of the resident row is the sorted soft-max head, and the samplers draw from it
+      {
+        dec.Reset();
+        dec.StepForward(seq, 4, 0);
+        const std::vector<float>& lg = dec.Output();
+        caihip::TNNetCandidates c = dec.Candidates(8);
+        EXPECT(c.Count() == 8 && c.Token[0] == dec.ArgMaxRow());
+        double mx = lg[0]; for (float v : lg) mx = std::fmax(mx, (double)v);
+        double sum = 0; for (float v : lg) sum += std::exp((double)v - mx);
+        for (int i = 0; i < c.Count(); i++) {
+          EXPECT(std::fabs(std::exp((double)lg[(size_t)c.Token[(size_t)i]] - mx) / sum - (double)c.Score[(size_t)i]) < 1e-5);
+          if (i) EXPECT(c.Score[(size_t)i] <= c.Score[(size_t)i - 1]);
+        }
+        EXPECT(caihip::SampleTopK(c, 4, 0.0) == c.Token[0] && caihip::SampleTopK(c, 4, 0.99) == c.Token[3]);
+        EXPECT(caihip::SampleWeightedTopK(c, 8, 0.0) == c.Token[0]);
+        EXPECT(caihip::SampleTopP(c, 2.0f, 0.5) == -1);                    // the prefix cannot hold more than all the mass
+        EXPECT(caihip::SampleTopP(c, c.Score[0] * 0.5f, 0.7) == c.Token[0]); // the first token alone exceeds P: fallback to it
+        EXPECT(caihip::SampleMinP(c, 0.999f, 0.3) == c.Token[0] || c.Score[1] >= 0.999f * c.Score[0]);
+        caihip::TNNetTokenHistory hist;
+        for (int i = 0; i < 4; i++) hist.RegisterToken(seq[i]);
+        hist.RegisterToken(c.Token[0]); hist.RegisterToken(c.Token[0]);
+        caihip::TNNetCandidates pen = dec.Candidates(8, 1.0f, &hist, 1.5f, 0.5f, 0.5f);
+        float before = c.Score[0], after = 0;
+        for (int i = 0; i < pen.Count(); i++) if (pen.Token[(size_t)i] == c.Token[0]) after = pen.Score[(size_t)i];
+        EXPECT(after < before);                                            // a repeated token loses mass
+        caihip::TNNetCandidates cold = dec.Candidates(2, 1e-9f);
+        EXPECT(cold.Token[0] == dec.ArgMaxRow() && cold.Score[0] > 0.999f); // T -> 0 is greedy
+      }
+      // streaming past the cache with sink + recent-window eviction (tests/TestNeuralDecode.pas:3930-3975)
+      {
+        dec.Reset();
+        dec.EnableEviction(2, 6);
+        for (int i = 0; i < 40; i++) {
+          dec.StepForward(&seq[i % n], 1, i);
+          EXPECT(dec.SDPACacheLength() == (i + 1 <= 8 ? i + 1 : 8));
+        }
+        bool refused = false;
+        try { dec.DisableEviction(); } catch (const caihip::CaiError&) { refused = true; }
+        EXPECT(refused);                                                   // past the cap the middle is gone
+        dec.Reset();
+        dec.DisableEviction();
+        bool refused2 = false;
+        dec.StepForward(seq, 2, 0);
+        try { dec.EnableInt8KVCache(); } catch (const caihip::CaiError&) { refused2 = true; }
+        EXPECT(refused2);                                                  // only a fresh session switches storage
+        dec.Reset();
+        dec.EnableInt8KVCache();
+        dec.StepForward(seq, n, 0);
+        double drift = 0.0;
+        for (size_t v = 0; v < rows[n - 1].size(); v++) drift = std::fmax(drift, std::fabs((double)rows[n - 1][v] - (double)dec.Output()[v]));
+        EXPECT(drift < 0.1 && dec.SDPACacheLength() == n);
+        dec.Reset();
+        dec.DisableInt8KVCache();
+      }
       // importer errors raise
       bool raised = false;
       try { caihip::TNNetStreamingDecoder bad("/nonexistent/model.gguf"); } catch (const caihip::CaiError& e) { raised = e.code != CAI_OK; }

@@ -92,6 +92,12 @@ function cai_decoder_generate(d: TCaiDecoder; first_token, pos, n_tokens: LongIn
 function cai_decoder_prefill(d: TCaiDecoder; seq: LongInt; tokens: PLongInt; n, pos0: LongInt; last_logits: PSingle; argmax: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_reset(d: TCaiDecoder; seq: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_truncate(d: TCaiDecoder; seq, n: LongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_sample_candidates(logits: PSingle; n: LongInt; hist_ids, hist_counts: PLongInt; n_hist: LongInt;
+  repetition, frequency, presence, temperature: Single; m: LongInt; tokens_out: PLongInt; probs_out: PSingle;
+  count_out: PLongInt; flags: LongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_decoder_candidates(d: TCaiDecoder; row: LongInt; hist_ids, hist_counts: PLongInt; n_hist: LongInt;
+  repetition, frequency, presence, temperature: Single; m: LongInt; tokens_out: PLongInt; probs_out: PSingle;
+  count_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_len(d: TCaiDecoder; seq: LongInt; len_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_set_eviction(d: TCaiDecoder; sink_tokens, recent_window: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_set_kv_dtype(d: TCaiDecoder; kv_dtype: LongInt): LongInt; cdecl; external CAIHIP_LIB;

@@ -483,6 +483,78 @@ int orc_argmax(const float* x, int n)
   return b;
 }
 
+/* The distribution pipeline of TChatEngine.GenerateFromIds (neuralchatengine.pas:1374-1396, 1495-1501):
+ * softmax of the logits row -> history penalty in the probability domain (neuralvolume.pas:5335-5376:
+ * p^repetition, * exp(-(frequency*count + presence)) for every distinct token of the history, then / sum) ->
+ * temperature in the probability domain (neuraldecode.pas:4710-4754: p := exp(ln(max(p,1e-30))/T - ln(max p)/T),
+ * / sum, T clamped to >= 1e-6, T == 1 is a no-op) -> the candidate prefix the samplers draw from: the m most
+ * probable tokens in descending order (TNNetSamplerBase.SelectTopCandidates + SortTokenArray, neuralvolume.pas:
+ * 5171-5196; the reference's nucleus sampler starts from the same 256-wide prefix, 4548-4562).
+ * Equal probabilities: lower token id first (the reference's quicksort leaves that order unspecified).
+ * exp / ln / pow are libm's here; the reference uses its own polynomial versions (tolerance 1e-6, neural.cl:1660-1664).
+ * Pinned by: softmax(logits / T) identity, closed-form penalty cases, sortedness and mass checks
+ * (tests/test_oracle_sampling.py). */
+typedef struct { float p; int32_t id; } orc_cand;
+static int cand_cmp(const void* a, const void* b)
+{
+  const orc_cand* x = (const orc_cand*)a; const orc_cand* y = (const orc_cand*)b;
+  if (x->p != y->p) return x->p > y->p ? -1 : 1;
+  return x->id < y->id ? -1 : (x->id > y->id ? 1 : 0);
+}
+
+int orc_sample_candidates(const float* logits, int n, const int32_t* hist_ids, const int32_t* hist_counts, int n_hist,
+                          float repetition, float frequency, float presence, float temperature, int m,
+                          int32_t* tok_out, float* p_out)
+{
+  /* (row sums are accumulated in double: the reference's vectorised GetSum has its own order, and a sequential
+   * float sum over a 152k row is off by ~1e-4 either way) */
+  float* p = (float*)malloc((size_t)n * sizeof(float));
+  {
+    float mx = logits[0];
+    for (int i = 1; i < n; i++) if (logits[i] > mx) mx = logits[i];
+    double tot = 0;
+    for (int i = 0; i < n; i++) {
+      float a = logits[i] - mx; if (a > 4000) a = 4000; else if (a < -4000) a = -4000;
+      p[i] = expf(a); tot += p[i];
+    }
+    if (tot > 0) { const float inv = (float)(1.0 / tot); for (int i = 0; i < n; i++) p[i] *= inv; }
+  }
+  if (repetition != 1.0f || frequency != 0.0f || presence != 0.0f) {
+    int changed = 0;
+    for (int k = 0; k < n_hist; k++) {
+      const int t = hist_ids[k];
+      if (t < 0 || t >= n) continue;
+      float v = p[t];
+      if (repetition != 1.0f && v > 0) v = powf(v, repetition);
+      if (frequency != 0.0f || presence != 0.0f) v *= expf(-(frequency * (float)hist_counts[k] + presence));
+      p[t] = v; changed = 1;
+    }
+    if (changed) {
+      double tot = 0; for (int i = 0; i < n; i++) tot += p[i];
+      if (tot > 0) for (int i = 0; i < n; i++) p[i] = (float)(p[i] / tot);
+    }
+  }
+  if (temperature != 1.0f) {
+    float T = temperature < 1e-6f ? 1e-6f : temperature;
+    float mx = p[0]; for (int i = 1; i < n; i++) if (p[i] > mx) mx = p[i];
+    if (mx > 0) {
+      const float lm = logf(mx < 1e-30f ? 1e-30f : mx), inv_t = 1.0f / T;
+      double sum = 0;
+      for (int i = 0; i < n; i++) { float v = p[i] < 1e-30f ? 1e-30f : p[i]; v = expf(logf(v) * inv_t - lm * inv_t); p[i] = v; sum += v; }
+      if (sum <= 0) sum = 1.0;
+      const float inv = (float)(1.0 / sum);
+      for (int i = 0; i < n; i++) p[i] *= inv;
+    }
+  }
+  orc_cand* c = (orc_cand*)malloc((size_t)n * sizeof(orc_cand));
+  for (int i = 0; i < n; i++) { c[i].p = p[i]; c[i].id = i; }
+  qsort(c, (size_t)n, sizeof(orc_cand), cand_cmp);
+  if (m > n) m = n;
+  for (int i = 0; i < m; i++) { tok_out[i] = c[i].id; p_out[i] = c[i].p; }
+  free(c); free(p);
+  return m;
+}
+
 /* ------------------------------------------------------------------ */
 /* attention                                                           */
 /* ------------------------------------------------------------------ */

@@ -70,6 +70,13 @@ void orc_softmax(const float* x, int n, float* y);                              
 void orc_topk_gate(const float* probs, int n, int k, int renorm, float* gates_out, int* idx_out); /* tests/TestNeuralNumerical.pas:74997-75042 */
 int  orc_argmax(const float* x, int n);                                              /* neuralchatengine.pas:683-697 */
 
+/* ---- distribution pipeline ahead of the samplers (neuralchatengine.pas:1374-1396, 1495-1501) ----
+ * softmax -> history penalty -> temperature, then the m most probable tokens, descending (ties: lower id first).
+ * hist_ids are the DISTINCT tokens of the context with their occurrence counts.  Returns min(m, n). */
+int orc_sample_candidates(const float* logits, int n, const int32_t* hist_ids, const int32_t* hist_counts, int n_hist,
+                          float repetition, float frequency, float presence, float temperature, int m,
+                          int32_t* tok_out, float* p_out);
+
 /* ---- cached GQA decode attention, fp32, head-major cache (neural.cl:2354-2499) ----
  * k_cache/v_cache: [kv_heads][max_ctx][head_dim]; qkv row = [Q | K | V]. Appends at slot
  * cache_len, then attends over [j_start .. cache_len] where window>0 limits the range.

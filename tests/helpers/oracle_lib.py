@@ -51,6 +51,8 @@ def lib():
         L.orc_q4k_scale_min.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p]; L.orc_q4k_scale_min.restype = None
         L.orc_attn_decode.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int, C.c_void_p]
         L.orc_attn_decode.restype = None
+        L.orc_sample_candidates.restype = C.c_int
+        L.orc_sample_candidates.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, C.c_void_p, C.c_void_p]
         L.orc_attn_decode_evict.restype = None
         L.orc_attn_decode_evict.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int, C.c_void_p]
         L.orc_max_abs_finite.restype = C.c_float; L.orc_max_abs_finite.argtypes = [C.c_void_p, C.c_int]
@@ -159,3 +161,13 @@ class OracleModel:
             lib().orc_model_free(self.h)
         except Exception:
             pass
+
+
+def sample_candidates(logits, m, temperature=1.0, history=None, repetition=1.0, frequency=0.0, presence=0.0):
+    """history: iterable of token ids (the context); returns (tokens, probs) of the m most probable, descending."""
+    logits = np.ascontiguousarray(logits, np.float32)
+    ids, counts = (np.unique(np.asarray(history, np.int32), return_counts=True) if history is not None and len(history) else (np.zeros(0, np.int32), np.zeros(0, np.int64)))
+    ids = np.ascontiguousarray(ids, np.int32); counts = np.ascontiguousarray(counts, np.int32)
+    tok = np.zeros(m, np.int32); p = np.zeros(m, np.float32)
+    k = lib().orc_sample_candidates(_p(logits), logits.size, _p(ids), _p(counts), ids.size, repetition, frequency, presence, temperature, m, _p(tok), _p(p))
+    return tok[:k], p[:k]
