@@ -1,13 +1,13 @@
 // Small-batch (2..8 tokens per pass) Q4_K linear layer on the matrix cores of gfx950: the decode step of a few sequences.
 //
 // At batch 1 the layer is a matrix-vector product and the VALU keeps up with HBM; at batch b the same weights serve
-// b activations, so the contraction goes to v_mfma_f32_32x32x8_f16 while the weights are still streamed once.
+// b activations, so the contraction goes to v_mfma_f32_16x16x32_f16 while the weights are still streamed once.
 //   * A operand = sc_j * q, an integer <= 63 * 15 and therefore EXACT in f16: the 6-bit sub-block scale is folded into
 //     the nibble with one packed fma ((1024 + q) * sc - 1024 * sc, every term exact), so the matrix cores accumulate
 //     across a whole 256-weight super-block and the float scale d is applied once per super-block, not per 32 weights;
 //   * B operand = the activations of up to 8 tokens, scaled per (token, 256-block) by a power of two and split hi + lo
-//     into two f16 (22 significant bits): 8 hi + 8 lo columns of the MFMA tile (the other 16 stay zero);
-//   * the -dmin * mn_j * sum_{k in j} x_k term is one more MFMA step per super-block (k = the 8 sub-blocks).
+//     into two f16 (22 significant bits): 8 hi + 8 lo = the 16 columns of the MFMA tile;
+//   * the -dmin * mn_j * sum_{k in j} x_k term is one more MFMA per row set and super-block (k = the 8 sub-blocks).
 //   Y[t][r] = sum_sb sinv[t][sb] * ( d * P_main - 32 dmin * P_min )   (Q4_K: neural/neuralgguf.pas:472-514)
 //
 // Work layout: grid = (row groups, K slices).  A work-group stages ITS slice of the activations (up to 4 super-blocks)
@@ -25,10 +25,10 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
-constexpr int NB_LDX = 260;      // halfs per staged activation column: 256 + pad (stride = 2 banks mod 64)
+constexpr int NB_LDX = 264;      // halfs per staged activation column: 256 + pad (stride = 4 banks mod 64: 16-byte reads of 16 columns tile the banks)
 constexpr int NB_SC = 16;        // staged columns: 8 tokens x {hi, lo}
 constexpr int NB_TK = 8;         // tokens per pass
-constexpr int NB_SMAX = 4;       // super-blocks per K slice (LDS: 4 x 8.6 KB, so three work-groups share a CU)
+constexpr int NB_SMAX = 5;       // super-blocks per K slice at most (LDS: 8.6 KB each, and three work-groups share a CU)
 
 struct NbSeg { const uint8_t* w; const float* bias; int rows; int y_off; int tile_end; };   // tile_end: cumulative 32-row tiles
 
@@ -54,6 +54,23 @@ __device__ __forceinline__ half4_t bytes_to_half4(uint32_t t)
   return half4_t{a.x, a.y, b.x, b.y};
 }
 
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+// eight nibbles (one per byte of lo, hi) times the sub-block scale -> the eight exact halfs sc * q
+__device__ __forceinline__ half8_t nibbles_times_scale(uint32_t lo, uint32_t hi, half2_t s2, half2_t c2)
+{
+  const half2_t a0 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, lo, 0x04010400u)), s2, c2);   // (1024 + q) * sc - 1024 * sc
+  const half2_t a1 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, lo, 0x04030402u)), s2, c2);
+  const half2_t a2 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04010400u)), s2, c2);
+  const half2_t a3 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, hi, 0x04030402u)), s2, c2);
+  return half8_t{a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+}
+
+// v_mfma_f32_16x16x32_f16: lane (m = lane % 16, kg = lane / 16) supplies 8 consecutive k of row m (A) / column m (B);
+// the 16 x 16 result has rows 4 kg .. 4 kg + 3 of column m in this lane.  Here a tile is 32 weight rows = two row sets,
+// the 16 columns are 8 tokens x {hi, lo}, and lane kg owns quant bytes 32 kg .. 32 kg + 31 of a super-block: sub-block
+// 2 kg in the low nibbles (k steps 0..3), sub-block 2 kg + 1 in the high nibbles (steps 4..7).
 __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
 {
   extern __shared__ __align__(16) unsigned char nb_smem[];
@@ -63,7 +80,7 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
   float* sinv_s = reinterpret_cast<float*>(sxs + S * NB_SC * 8);     // [S][8]
   float* s_d = sinv_s + S * NB_TK;                                   // [4 waves][2][32]: d, 32*dmin per row
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n = lane & 31, kg = lane >> 5;
+  const int n = lane & 15, kg = lane >> 4;
   const int K = p.cols, nsb = K >> 8, nb32 = K >> 5;
   const int slice = blockIdx.y, sb0 = slice * S, nS = min(S, nsb - sb0);
   const int64_t row_bytes = (int64_t)nsb * 144;
@@ -71,22 +88,25 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
   const int n_it = tile0 < p.n_tiles ? (p.n_tiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
   const int nq = n_it * nS;                      // (tile, super-block) items of this wave
 
-  struct WRegs { uint4 h, q[4]; };
+  struct WRegs { uint4 h[2], q[2][2]; };
   auto locate = [&](int tile, const NbSeg*& sg, int& R0) {
     int sgi = 0, t0 = 0;
     if (p.n_seg > 1 && tile >= p.seg[0].tile_end) { sgi = 1; t0 = p.seg[0].tile_end; }
     if (p.n_seg > 2 && tile >= p.seg[1].tile_end) { sgi = 2; t0 = p.seg[1].tile_end; }
     sg = &p.seg[sgi]; R0 = (tile - t0) * 32;
   };
-  // weights of item q: header + this lane's 64 quant bytes (chunks 2kg, 2kg+1) of row R0 + n
+  // weights of item q: for rows R0 + n and R0 + 16 + n the header and this lane's 32 quant bytes
   auto load_w = [&](int q, WRegs& r) {
     if (q < nq) {
       const int tile = tile0 + (q / nS) * p.tile_stride, sb = sb0 + q % nS;
       const NbSeg* sg; int R0; locate(tile, sg, R0);
-      const uint8_t* blk = sg->w + (int64_t)min(R0 + n, sg->rows - 1) * row_bytes + (int64_t)sb * 144;   // tail rows: re-read the last row
-      r.h = *reinterpret_cast<const uint4*>(blk);
 #pragma unroll
-      for (int i = 0; i < 4; i++) r.q[i] = *reinterpret_cast<const uint4*>(blk + 16 + 64 * kg + 16 * i);
+      for (int hh = 0; hh < 2; hh++) {
+        const uint8_t* blk = sg->w + (int64_t)min(R0 + 16 * hh + n, sg->rows - 1) * row_bytes + (int64_t)sb * 144;   // tail rows: re-read the last row
+        r.h[hh] = *reinterpret_cast<const uint4*>(blk);
+        r.q[hh][0] = *reinterpret_cast<const uint4*>(blk + 16 + 32 * kg);
+        r.q[hh][1] = *reinterpret_cast<const uint4*>(blk + 32 + 32 * kg);
+      }
     }
   };
   WRegs wa, wb, wc;
@@ -98,8 +118,7 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
     const int tok = col % NB_TK;
     uint4 v = make_uint4(0, 0, 0, 0);
     if (tok < p.n_tok) v = *reinterpret_cast<const uint4*>(((col / NB_TK) ? p.xlo : p.xhi) + (int64_t)tok * K + (sb0 + s) * 256 + chunk * 8);
-    uint2* dst = reinterpret_cast<uint2*>(xs + (s * NB_SC + col) * NB_LDX + chunk * 8);   // columns are 8-byte aligned
-    dst[0] = make_uint2(v.x, v.y); dst[1] = make_uint2(v.z, v.w);
+    *reinterpret_cast<uint4*>(xs + (s * NB_SC + col) * NB_LDX + chunk * 8) = v;
   }
   for (int idx = threadIdx.x; idx < nS * NB_SC; idx += 256) {
     const int col = idx % NB_SC, s = idx / NB_SC, tok = col % NB_TK;
@@ -110,95 +129,89 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
   }
   __syncthreads();
 
-  float16_t acc;
-#pragma unroll
-  for (int v = 0; v < 16; v++) acc[v] = 0.0f;
-  const bool col_on = n < NB_SC;                 // MFMA columns 16..31 multiply zeros
-  const half4_t zero4 = {(_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f, (_Float16)0.0f};
+  float acc[2][4];
+  const _Float16 k1024 = (_Float16)1024.0f, kz = (_Float16)0.0f;
 
   auto compute = [&](const WRegs& r, int q) {
     const int s = q % nS;
     if (s == 0) {
 #pragma unroll
-      for (int v = 0; v < 16; v++) acc[v] = 0.0f;
+      for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[hh][i] = 0.0f;
     }
-    // 6-bit scales / mins of this lane's four sub-blocks 4kg .. 4kg+3 (neural/neuralgguf.pas:448-464), one per byte
-    const uint32_t sc4 = kg == 0 ? (r.h.y & 0x3f3f3f3fu) : ((r.h.w & 0x0f0f0f0fu) | ((r.h.y >> 2) & 0x30303030u));
-    const uint32_t mn4 = kg == 0 ? (r.h.z & 0x3f3f3f3fu) : (((r.h.w >> 4) & 0x0f0f0f0fu) | ((r.h.z >> 2) & 0x30303030u));
-    const _Float16 k1024 = (_Float16)1024.0f;
-    const half4_t sch = bytes_to_half4(sc4), mnh = bytes_to_half4(mn4);
-    const half4_t scv = half4_t{sch.x - k1024, sch.y - k1024, sch.z - k1024, sch.w - k1024};   // sc as halfs
-    const half4_t mnv = half4_t{mnh.x - k1024, mnh.y - k1024, mnh.z - k1024, mnh.w - k1024};
-    if (kg == 0) {
-      const float d = __half2float(__ushort_as_half((unsigned short)(r.h.x & 0xffffu)));
-      const float dmin = __half2float(__ushort_as_half((unsigned short)(r.h.x >> 16)));
-      s_d[(wave * 2 + 0) * 32 + n] = d; s_d[(wave * 2 + 1) * 32 + n] = dmin * 32.0f;
-    }
-    // two accumulators: consecutive MFMAs do not wait for each other
-    float16_t C0, C1, Cm;
+    float4_t C[2], Cm[2];
+    half2_t s2[2][2], c2[2][2];
 #pragma unroll
-    for (int v = 0; v < 16; v++) { C0[v] = 0.0f; C1[v] = 0.0f; Cm[v] = 0.0f; }
-    const _Float16* xcol = xs + (s * NB_SC + (col_on ? n : 0)) * NB_LDX + 128 * kg;
-#pragma unroll
-    for (int ccl = 0; ccl < 2; ccl++) {
-#pragma unroll
-      for (int hl = 0; hl < 2; hl++) {
-        const int j = 2 * ccl + hl;                                   // sub-block 4kg + j of the super-block
-        const _Float16 sj = j == 0 ? scv.x : (j == 1 ? scv.y : (j == 2 ? scv.z : scv.w));
-        const half2_t s2 = {sj, sj};
-        const half2_t c2 = {(_Float16)(-1024.0f) * sj, (_Float16)(-1024.0f) * sj};   // exact: a multiple of 1024 below 65504
-        const _Float16* xb = xcol + 32 * j;
-#pragma unroll
-        for (int t = 0; t < 8; t++) {
-          const uint4& qq = r.q[2 * ccl + (t >> 2)];
-          const uint32_t qd = (t & 3) == 0 ? qq.x : ((t & 3) == 1 ? qq.y : ((t & 3) == 2 ? qq.z : qq.w));
-          const uint32_t nib = hl ? ((qd >> 4) & 0x0f0f0f0fu) : (qd & 0x0f0f0f0fu);
-          const uint32_t p01 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04010400u);
-          const uint32_t p23 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04030402u);
-          const half2_t a01 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, p01), s2, c2);   // (1024 + q) * sc - 1024 * sc = sc * q
-          const half2_t a23 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, p23), s2, c2);
-          const half4_t A = {a01.x, a01.y, a23.x, a23.y};
-          half4_t B = *reinterpret_cast<const half4_t*>(xb + 4 * t);
-          if (!col_on) B = zero4;
-          if (t & 1) C1 = __builtin_amdgcn_mfma_f32_32x32x8f16(A, B, C1, 0, 0, 0);
-          else C0 = __builtin_amdgcn_mfma_f32_32x32x8f16(A, B, C0, 0, 0, 0);
-        }
+    for (int hh = 0; hh < 2; hh++) {
+      // 6-bit scales / mins (neural/neuralgguf.pas:448-464), one per byte: sub-blocks 0..3 and 4..7; this lane's two
+      const uint4 h = r.h[hh];
+      const uint32_t sc_lo = h.y & 0x3f3f3f3fu, sc_hi = (h.w & 0x0f0f0f0fu) | ((h.y >> 2) & 0x30303030u);
+      const uint32_t mn_lo = h.z & 0x3f3f3f3fu, mn_hi = ((h.w >> 4) & 0x0f0f0f0fu) | ((h.z >> 2) & 0x30303030u);
+      const uint32_t scp = ((kg & 2) ? sc_hi : sc_lo) >> (16 * (kg & 1));     // bytes 0, 1 = sc of sub-blocks 2kg, 2kg+1
+      const uint32_t mnp = ((kg & 2) ? mn_hi : mn_lo) >> (16 * (kg & 1));
+      const half2_t sch = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, scp, 0x04010400u)) - half2_t{k1024, k1024};
+      const half2_t mnh = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, mnp, 0x04010400u)) - half2_t{k1024, k1024};
+      s2[hh][0] = half2_t{sch.x, sch.x}; s2[hh][1] = half2_t{sch.y, sch.y};
+      c2[hh][0] = half2_t{(_Float16)(-1024.0f) * sch.x, (_Float16)(-1024.0f) * sch.x};   // exact: a multiple of 1024 below 65504
+      c2[hh][1] = half2_t{(_Float16)(-1024.0f) * sch.y, (_Float16)(-1024.0f) * sch.y};
+      if (kg == 0) {
+        const float d = __half2float(__ushort_as_half((unsigned short)(h.x & 0xffffu)));
+        const float dmin = __half2float(__ushort_as_half((unsigned short)(h.x >> 16)));
+        s_d[(wave * 2 + 0) * 32 + 16 * hh + n] = d; s_d[(wave * 2 + 1) * 32 + 16 * hh + n] = dmin * 32.0f;
       }
+      // - dmin * mn_j * (sum of the sub-block's activations): k = this lane's two sub-blocks, the other six k stay zero
+      const half2_t bm = *reinterpret_cast<const half2_t*>(sxs + (s * NB_SC + n) * 8 + 2 * kg);
+      const half8_t Am = {mnh.x, mnh.y, kz, kz, kz, kz, kz, kz}, Bm = {bm.x, bm.y, kz, kz, kz, kz, kz, kz};
+      const float4_t z4 = {0.0f, 0.0f, 0.0f, 0.0f};
+      Cm[hh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Am, Bm, z4, 0, 0, 0);
+      C[hh] = z4;
     }
-    {
-      half4_t Bm = *reinterpret_cast<const half4_t*>(sxs + (s * NB_SC + (col_on ? n : 0)) * 8 + 4 * kg);
-      if (!col_on) Bm = zero4;
-      Cm = __builtin_amdgcn_mfma_f32_32x32x8f16(mnv, Bm, Cm, 0, 0, 0);
+    const _Float16* xcol = xs + (s * NB_SC + n) * NB_LDX + 64 * kg;
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      const half8_t B = *reinterpret_cast<const half8_t*>(xcol + 8 * t);
+#pragma unroll
+      for (int hh = 0; hh < 2; hh++) {
+        const uint4& qq = r.q[hh][(t & 3) >> 1];
+        const uint32_t d0 = (t & 1) ? qq.z : qq.x, d1 = (t & 1) ? qq.w : qq.y;       // bytes 8 (t & 3) .. + 7
+        const uint32_t lo = (t < 4) ? (d0 & 0x0f0f0f0fu) : ((d0 >> 4) & 0x0f0f0f0fu);
+        const uint32_t hi = (t < 4) ? (d1 & 0x0f0f0f0fu) : ((d1 >> 4) & 0x0f0f0f0fu);
+        const half8_t A = nibbles_times_scale(lo, hi, s2[hh][t >> 2], c2[hh][t >> 2]);
+        C[hh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, C[hh], 0, 0, 0);
+      }
     }
     const float si = sinv_s[s * NB_TK + (n & (NB_TK - 1))];
     __builtin_amdgcn_wave_barrier();   // s_d was written by this wave's own lanes above; LDS operations of a wave complete in order
 #pragma unroll
-    for (int g = 0; g < 4; g++) {
-      const float4 d4 = *reinterpret_cast<const float4*>(&s_d[(wave * 2 + 0) * 32 + 8 * g + 4 * kg]);
-      const float4 m4 = *reinterpret_cast<const float4*>(&s_d[(wave * 2 + 1) * 32 + 8 * g + 4 * kg]);
-      acc[4 * g + 0] += si * (d4.x * (C0[4 * g + 0] + C1[4 * g + 0]) - m4.x * Cm[4 * g + 0]);
-      acc[4 * g + 1] += si * (d4.y * (C0[4 * g + 1] + C1[4 * g + 1]) - m4.y * Cm[4 * g + 1]);
-      acc[4 * g + 2] += si * (d4.z * (C0[4 * g + 2] + C1[4 * g + 2]) - m4.z * Cm[4 * g + 2]);
-      acc[4 * g + 3] += si * (d4.w * (C0[4 * g + 3] + C1[4 * g + 3]) - m4.w * Cm[4 * g + 3]);
+    for (int hh = 0; hh < 2; hh++) {
+      const float4 d4 = *reinterpret_cast<const float4*>(&s_d[(wave * 2 + 0) * 32 + 16 * hh + 4 * kg]);
+      const float4 m4 = *reinterpret_cast<const float4*>(&s_d[(wave * 2 + 1) * 32 + 16 * hh + 4 * kg]);
+      acc[hh][0] += si * (d4.x * C[hh][0] - m4.x * Cm[hh][0]);
+      acc[hh][1] += si * (d4.y * C[hh][1] - m4.y * Cm[hh][1]);
+      acc[hh][2] += si * (d4.z * C[hh][2] - m4.z * Cm[hh][2]);
+      acc[hh][3] += si * (d4.w * C[hh][3] - m4.w * Cm[hh][3]);
     }
     __builtin_amdgcn_wave_barrier();
     if (s != nS - 1) return;
-    // ---- the slice's contribution of this tile: column t (hi) + column 8 + t (lo); lane t keeps 4 runs of 4 rows ----
+    // ---- the slice's contribution of this tile: column t (hi) + column 8 + t (lo); lane t keeps 2 runs of 4 rows ----
     const int tile = tile0 + (q / nS) * p.tile_stride;
     const NbSeg* sg; int R0; locate(tile, sg, R0);
     const int tok = n & (NB_TK - 1);
-    float tot[16];
+    float tot[2][4];
 #pragma unroll
-    for (int v = 0; v < 16; v++) tot[v] = acc[v] + __shfl_xor(acc[v], NB_TK, 64);
+    for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) tot[hh][i] = acc[hh][i] + __shfl_xor(acc[hh][i], NB_TK, 64);
     if (n < NB_TK && tok < p.n_tok) {
       float* dst = p.part + ((int64_t)slice * p.n_tok + tok) * p.part_stride + sg->y_off;
 #pragma unroll
-      for (int g = 0; g < 4; g++) {
-        const int row = R0 + 8 * g + 4 * kg;
-        if (row + 3 < sg->rows && ((sg->y_off + row) & 3) == 0) *reinterpret_cast<float4*>(dst + row) = make_float4(tot[4 * g], tot[4 * g + 1], tot[4 * g + 2], tot[4 * g + 3]);
+      for (int hh = 0; hh < 2; hh++) {
+        const int row = R0 + 16 * hh + 4 * kg;
+        if (row + 3 < sg->rows && ((sg->y_off + row) & 3) == 0) *reinterpret_cast<float4*>(dst + row) = make_float4(tot[hh][0], tot[hh][1], tot[hh][2], tot[hh][3]);
         else {
 #pragma unroll
-          for (int i = 0; i < 4; i++) if (row + i < sg->rows) dst[row + i] = tot[4 * g + i];
+          for (int i = 0; i < 4; i++) if (row + i < sg->rows) dst[row + i] = tot[hh][i];
         }
       }
     }
@@ -359,22 +372,29 @@ int nb_reserve(int k_max, size_t part_floats)
   return CAI_OK;
 }
 
-// K slices a product over `cols` columns and `tiles` row tiles is cut into
+// How a product over `cols` columns and `tiles` 32-row tiles is cut: S super-blocks per K slice and gx row groups, so
+// that gx * slices work-groups fit the chip in ONE round (three work-groups share a CU) and the waves' shares come out
+// even.  A wave's share is ceil(tiles / (4 gx)) tiles of S items each (item = 32 rows x one super-block) plus the
+// partial result every (tile, slice) writes and its consumer re-reads, priced at 0.45 item.
 static void nb_geometry(int cols, int tiles, int& S, int& n_slices, int& gx, int& tile_stride)
 {
-  const int nsb = cols >> 8, n_cu = ctx().n_cu;
-  S = std::min(NB_SMAX, nsb);
-  { static const int force = []() { const char* e = getenv("CAIHIP_NB_S"); return e ? atoi(e) : 0; }(); if (force >= 1 && force <= 8) S = std::min(force, nsb); }
-  n_slices = (nsb + S - 1) / S;
-  gx = (tiles + 3) / 4;
-  // plenty of row groups: let a wave walk several tiles so the staged slice is reused
-  int per_wave = 1;
-  while (per_wave < 4 && (gx / (per_wave * 2)) * n_slices >= 3 * n_cu) per_wave *= 2;
-  gx = (gx + per_wave - 1) / per_wave;
+  const int nsb = cols >> 8, slots = 3 * ctx().n_cu;
+  static const int force = []() { const char* e = getenv("CAIHIP_NB_S"); return e ? atoi(e) : 0; }();
+  const int s_lo = std::min(2, nsb), s_hi = std::min(NB_SMAX, nsb);
+  float best = 3.0e38f;
+  S = s_lo;
+  for (int s = s_lo; s <= s_hi; s++) {
+    if (force >= 2 && force <= NB_SMAX && s != std::min(force, nsb)) continue;
+    const int ns = (nsb + s - 1) / s;
+    const int g = std::max(1, std::min((tiles + 3) / 4, slots / ns));
+    const int share = (tiles + 4 * g - 1) / (4 * g);
+    const float cost = (float)share * ((float)s + 0.45f);
+    if (cost < best) { best = cost; S = s; gx = g; n_slices = ns; }
+  }
   tile_stride = gx * 4;
 }
-// upper bound of the slice count for a width (sizes the partial buffer): S never drops below min(4, blocks per row)
-int nb_max_slices(int cols) { const int nsb = cols >> 8; return (nsb + std::min(4, nsb) - 1) / std::min(4, std::max(nsb, 1)); }
+// upper bound of the slice count for a width (sizes the partial buffer): S never drops below min(2, blocks per row)
+int nb_max_slices(int cols) { const int nsb = std::max(cols >> 8, 1); const int s = std::min(2, nsb); return (nsb + s - 1) / s; }
 
 static int nb_prep_launch(int src, NbPrepParams& p, int n_tok)
 {
