@@ -711,6 +711,205 @@ __global__ __launch_bounds__(256) void kv_append_rows_i8_kernel(const AttnParams
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Prompt ingestion on the matrix cores: every prompt token attends over the cached rows up to its own position.
+// Work-group = (KV head, four query heads of its group, 32 consecutive tokens); wave w takes head h0 + w.  K and V
+// tiles of 32 cached rows are staged in LDS (V transposed) and shared by the four waves.  Per tile and wave:
+//   S^T[row][token] = K . q^T   on v_mfma_f32_32x32x8_f16: the result lane holds ONE token column, so the running
+//                               maximum, the normaliser and the rescaling of the output are per-lane scalars, and the
+//                               result registers of k-step s are exactly the B operand of step s of the next product;
+//   O^T[dim][token] += V^T . P^T   with P split hi + lo into two f16 (22 bits), like q; a float cache is split too.
+// Same arithmetic as the decode kernels up to the order of the sums (tests: < 1e-4 of token-at-a-time ingestion).
+// ------------------------------------------------------------------------------------------
+typedef _Float16 ph4_t __attribute__((ext_vector_type(4)));
+typedef float pf16_t __attribute__((ext_vector_type(16)));
+
+struct PromptParams {
+  const float* qkv; int64_t qkv_stride;      // rows [Q | K | V], K and V already appended to the cache
+  _Float16* qhi; _Float16* qlo;              // [token][q_heads * 128] rotated q, hi + lo
+  const void* kc; const void* vc;            // this sequence's layer plane: [kv_head][max_ctx][128]
+  int q_heads, kv_heads, max_ctx, n_tok, window;
+  float softcap, inv_sqrt;
+  const float* theta; const int32_t* pos;
+  float* out; int64_t out_stride;
+};
+
+// rotated q (neural/neural.cl:1517-1542) as two f16 planes
+__global__ __launch_bounds__(256) void prompt_q_kernel(const PromptParams p)
+{
+  const int t = blockIdx.x, qw = p.q_heads * 128;
+  const float* row = p.qkv + (int64_t)t * p.qkv_stride;
+  const int pos = p.pos[t];
+  for (int e = threadIdx.x; e < (qw >> 1); e += 256) {
+    const int d = (2 * e) & 127;
+    float x0 = row[2 * e], x1 = row[2 * e + 1];
+    if (p.theta) {
+      float sn, cs; sincosf((float)pos * p.theta[d >> 1], &sn, &cs);
+      const float y0 = cs * x0 - sn * x1, y1 = sn * x0 + cs * x1;
+      x0 = y0; x1 = y1;
+    }
+    const _Float16 h0 = (_Float16)x0, h1 = (_Float16)x1;
+    p.qhi[(int64_t)t * qw + 2 * e] = h0; p.qhi[(int64_t)t * qw + 2 * e + 1] = h1;
+    p.qlo[(int64_t)t * qw + 2 * e] = (_Float16)(x0 - (float)h0); p.qlo[(int64_t)t * qw + 2 * e + 1] = (_Float16)(x1 - (float)h1);
+  }
+}
+
+constexpr int PA_LDK = 132;    // halfs per staged K row (128 + pad: 8-byte reads of 32 rows tile the banks)
+constexpr int PA_LDV = 36;     // halfs per staged V^T row (32 cached rows + pad)
+
+template <typename KV_T>
+__global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
+{
+  constexpr bool F32 = sizeof(KV_T) == 4;
+  constexpr int NP = F32 ? 2 : 1;                 // planes of K and V: a float cache is split hi + lo
+  __shared__ __align__(16) _Float16 sK[NP][32 * PA_LDK];
+  __shared__ __align__(16) _Float16 sV[NP][128 * PA_LDV];
+  const int G = p.q_heads / p.kv_heads, quads = (G + 3) >> 2;
+  const int g = blockIdx.y / quads, h0 = (blockIdx.y % quads) * 4;
+  const int t0 = blockIdx.x * 32;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 31, kg = lane >> 5;
+  const int hq = h0 + wave;                       // head within the group
+  const bool head_on = hq < G;
+  const int head = g * G + (head_on ? hq : 0);
+  const int tok = t0 + n;
+  const bool tok_on = tok < p.n_tok;
+  const int pos_n = tok_on ? p.pos[tok] : -1;
+  const int jstart_n = (p.window > 0 && pos_n + 1 > p.window) ? pos_n + 1 - p.window : 0;
+  // the tile's range of cached rows (tokens are consecutive positions of one sequence)
+  const int pos_first = p.pos[t0], pos_last = p.pos[min(t0 + 31, p.n_tok - 1)];
+  const int j_lo = (p.window > 0 && pos_first + 1 > p.window) ? pos_first + 1 - p.window : 0;
+  const KV_T* kc = reinterpret_cast<const KV_T*>(p.kc) + (int64_t)g * p.max_ctx * 128;
+  const KV_T* vc = reinterpret_cast<const KV_T*>(p.vc) + (int64_t)g * p.max_ctx * 128;
+
+  // this lane's q fragments: token n, dims 8 s + 4 kg .. + 3 of the wave's head
+  ph4_t qh[16], ql[16];
+  {
+    const int64_t qo = (int64_t)min(tok, p.n_tok - 1) * (p.q_heads * 128) + head * 128 + 4 * kg;
+#pragma unroll
+    for (int s = 0; s < 16; s++) {
+      qh[s] = *reinterpret_cast<const ph4_t*>(p.qhi + qo + 8 * s);
+      ql[s] = *reinterpret_cast<const ph4_t*>(p.qlo + qo + 8 * s);
+    }
+  }
+  pf16_t O[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) O[dt][v] = 0.0f;
+  float m_run = -1e30f, l_run = 0.0f;
+
+  const int srow = tid >> 3, sdim = (tid & 7) * 16;         // staging: 16 consecutive elements of one cached row
+  for (int jt = j_lo >> 5; jt * 32 <= pos_last; jt++) {
+    __syncthreads();                                        // the previous tile has been consumed
+    {
+      const int j = min(jt * 32 + srow, p.max_ctx - 1);     // rows past the live range are masked below
+      float kv[16], vv[16];
+      if (F32) {
+#pragma unroll
+        for (int c4 = 0; c4 < 4; c4++) {
+          const float4 a = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(kc) + (int64_t)j * 128 + sdim + 4 * c4);
+          const float4 b = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(vc) + (int64_t)j * 128 + sdim + 4 * c4);
+          kv[4 * c4] = a.x; kv[4 * c4 + 1] = a.y; kv[4 * c4 + 2] = a.z; kv[4 * c4 + 3] = a.w;
+          vv[4 * c4] = b.x; vv[4 * c4 + 1] = b.y; vv[4 * c4 + 2] = b.z; vv[4 * c4 + 3] = b.w;
+        }
+      } else {
+#pragma unroll
+        for (int c8 = 0; c8 < 2; c8++) {
+          const uint4 a = *reinterpret_cast<const uint4*>(reinterpret_cast<const __half*>(kc) + (int64_t)j * 128 + sdim + 8 * c8);
+          const uint4 b = *reinterpret_cast<const uint4*>(reinterpret_cast<const __half*>(vc) + (int64_t)j * 128 + sdim + 8 * c8);
+          const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const __half2 ah = __builtin_bit_cast(__half2, aw[i]), bh = __builtin_bit_cast(__half2, bw[i]);
+            kv[8 * c8 + 2 * i] = __low2float(ah); kv[8 * c8 + 2 * i + 1] = __high2float(ah);
+            vv[8 * c8 + 2 * i] = __low2float(bh); vv[8 * c8 + 2 * i + 1] = __high2float(bh);
+          }
+        }
+      }
+#pragma unroll
+      for (int i4 = 0; i4 < 4; i4++) {                    // K rows stay row-major: 8-byte stores
+        ph4_t kh, kl;
+#pragma unroll
+        for (int i = 0; i < 4; i++) { kh[i] = (_Float16)kv[4 * i4 + i]; kl[i] = (_Float16)(kv[4 * i4 + i] - (float)kh[i]); }
+        *reinterpret_cast<ph4_t*>(&sK[0][srow * PA_LDK + sdim + 4 * i4]) = kh;
+        if (F32) *reinterpret_cast<ph4_t*>(&sK[NP - 1][srow * PA_LDK + sdim + 4 * i4]) = kl;
+      }
+#pragma unroll
+      for (int i = 0; i < 16; i++) {                      // V goes in transposed
+        const _Float16 vh = (_Float16)vv[i];
+        sV[0][(sdim + i) * PA_LDV + srow] = vh;
+        if (F32) sV[NP - 1][(sdim + i) * PA_LDV + srow] = (_Float16)(vv[i] - (float)vh);
+      }
+    }
+    __syncthreads();
+    if (!head_on) continue;                                 // (an idle wave still stages and meets the barriers)
+
+    // ---- S^T = K . q^T ----
+    pf16_t C;
+#pragma unroll
+    for (int v = 0; v < 16; v++) C[v] = 0.0f;
+#pragma unroll
+    for (int s = 0; s < 16; s++) {
+      const ph4_t a = *reinterpret_cast<const ph4_t*>(&sK[0][n * PA_LDK + 8 * s + 4 * kg]);
+      C = __builtin_amdgcn_mfma_f32_32x32x8f16(a, qh[s], C, 0, 0, 0);
+      C = __builtin_amdgcn_mfma_f32_32x32x8f16(a, ql[s], C, 0, 0, 0);
+      if (F32) {
+        const ph4_t al = *reinterpret_cast<const ph4_t*>(&sK[NP - 1][n * PA_LDK + 8 * s + 4 * kg]);
+        C = __builtin_amdgcn_mfma_f32_32x32x8f16(al, qh[s], C, 0, 0, 0);
+      }
+    }
+    // ---- this token's column: mask, running maximum, weights ----
+    float tmax = -1e30f;
+    bool ok[16];
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const int krow = jt * 32 + 8 * (v >> 2) + 4 * kg + (v & 3);
+      float sc = C[v] * p.inv_sqrt;
+      if (p.softcap > 0.0f) sc = p.softcap * tanhf(sc / p.softcap);
+      ok[v] = krow <= pos_n && krow >= jstart_n;
+      C[v] = sc;
+      if (ok[v]) tmax = fmaxf(tmax, sc);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax), corr = expf(m_run - m_new);
+    float psum = 0.0f;
+#pragma unroll
+    for (int v = 0; v < 16; v++) { C[v] = ok[v] ? expf(C[v] - m_new) : 0.0f; psum += C[v]; }
+    psum += __shfl_xor(psum, 32, 64);
+    l_run = l_run * corr + psum; m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) O[dt][v] *= corr;
+    // ---- O^T += V^T . P^T ----
+#pragma unroll
+    for (int s4 = 0; s4 < 4; s4++) {
+      ph4_t ph, pl;
+#pragma unroll
+      for (int i = 0; i < 4; i++) { const _Float16 hv = (_Float16)C[4 * s4 + i]; ph[i] = hv; pl[i] = (_Float16)(C[4 * s4 + i] - (float)hv); }
+#pragma unroll
+      for (int dt = 0; dt < 4; dt++) {
+        const ph4_t a = *reinterpret_cast<const ph4_t*>(&sV[0][(32 * dt + n) * PA_LDV + 8 * s4 + 4 * kg]);
+        O[dt] = __builtin_amdgcn_mfma_f32_32x32x8f16(a, ph, O[dt], 0, 0, 0);
+        O[dt] = __builtin_amdgcn_mfma_f32_32x32x8f16(a, pl, O[dt], 0, 0, 0);
+        if (F32) {
+          const ph4_t al = *reinterpret_cast<const ph4_t*>(&sV[NP - 1][(32 * dt + n) * PA_LDV + 8 * s4 + 4 * kg]);
+          O[dt] = __builtin_amdgcn_mfma_f32_32x32x8f16(al, ph, O[dt], 0, 0, 0);
+        }
+      }
+    }
+  }
+  if (!head_on || !tok_on) return;
+  const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+  float* dst = p.out + (int64_t)tok * p.out_stride + head * 128;
+#pragma unroll
+  for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+    for (int g4 = 0; g4 < 4; g4++)
+      *reinterpret_cast<float4*>(dst + 32 * dt + 8 * g4 + 4 * kg) =
+          make_float4(O[dt][4 * g4] * inv, O[dt][4 * g4 + 1] * inv, O[dt][4 * g4 + 2] * inv, O[dt][4 * g4 + 3] * inv);
+}
+
 int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, int n_seq, int q_heads, int window,
                      float softcap, const float* theta, const int32_t* pos_dev, float* out, int64_t out_stride, int seq0,
                      int prompt_rows, float* prompt_part)
@@ -740,6 +939,32 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   }
   p.counters = kv->d_counters;
   int rc;
+  // prompts over a 128-wide fp32 / fp16 cache: matrix-core kernel, 32 tokens x 4 heads per work-group
+  static const int flash_on = []() { const char* e = getenv("CAIHIP_PROMPT_FLASH"); return e ? atoi(e) : 1; }();
+  if (prompt_rows && flash_on && kv->head_dim == 128 && kv->dtype != CAI_KV_I8 && kv->evict_cap == 0 && n_seq >= 8) {
+    const size_t need = (size_t)n_seq * q_heads * 128;
+    if (need > kv->pq_cap) {
+      CAI_HIP(hipStreamSynchronize(c.stream));
+      if (kv->pq_hi) (void)hipFree(kv->pq_hi);
+      if (kv->pq_lo) (void)hipFree(kv->pq_lo);
+      kv->pq_hi = kv->pq_lo = nullptr; kv->pq_cap = 0;
+      CAI_HIP(hipMalloc(&kv->pq_hi, need * 2));
+      CAI_HIP(hipMalloc(&kv->pq_lo, need * 2));
+      kv->pq_cap = need;
+    }
+    PromptParams pp{};
+    pp.qkv = qkv; pp.qkv_stride = qkv_stride; pp.qhi = (_Float16*)kv->pq_hi; pp.qlo = (_Float16*)kv->pq_lo;
+    const size_t plane = ((size_t)seq0 * kv->seq_elems() + (size_t)layer * kv->layer_elems()) * kv->elem();
+    pp.kc = (const char*)kv->k + plane; pp.vc = (const char*)kv->v + plane;
+    pp.q_heads = q_heads; pp.kv_heads = kv->kv_heads; pp.max_ctx = kv->max_ctx; pp.n_tok = n_seq; pp.window = window;
+    pp.softcap = softcap; pp.inv_sqrt = p.inv_sqrt; pp.theta = theta; pp.pos = pos_dev; pp.out = out; pp.out_stride = out_stride;
+    const int G = q_heads / kv->kv_heads;
+    hipLaunchKernelGGL(prompt_q_kernel, dim3(n_seq), dim3(256), 0, c.stream, pp);
+    const dim3 grid((n_seq + 31) / 32, kv->kv_heads * ((G + 3) / 4));
+    if (kv->dtype == CAI_KV_F16) hipLaunchKernelGGL(attn_prompt_kernel<__half>, grid, dim3(256), 0, c.stream, pp);
+    else hipLaunchKernelGGL(attn_prompt_kernel<float>, grid, dim3(256), 0, c.stream, pp);
+    return CAI_OK;
+  }
   // one work-group per (slice, KV head) serving the whole group of query heads, or one per (slice, query head)
   // (the first fetches K and V once but has G times fewer work-groups: it needs a grid that fills the chip by itself)
   static const int group_min = []() { const char* e = getenv("CAIHIP_ATTN_GROUP_MIN"); return e ? atoi(e) : 256; }();
@@ -797,6 +1022,9 @@ void kv_free(cai_kv_s* kv)
   if (kv->ks) (void)hipFree(kv->ks);
   if (kv->vs) (void)hipFree(kv->vs);
   kv->ks = kv->vs = nullptr;
+  if (kv->pq_hi) (void)hipFree(kv->pq_hi);
+  if (kv->pq_lo) (void)hipFree(kv->pq_lo);
+  kv->pq_hi = kv->pq_lo = nullptr; kv->pq_cap = 0;
   if (kv->part) (void)hipFree(kv->part);
   if (kv->d_len) (void)hipFree(kv->d_len);
   if (kv->d_counters) (void)hipFree(kv->d_counters);
