@@ -93,8 +93,7 @@ struct GemmParams {
   int n_row_groups, n_tok_tiles;
 };
 
-constexpr int PF_LDX = 260;       // halfs per staged token row: 256 + pad (stride = 2 banks mod 64)
-constexpr int PF_TT = 2;          // 32-token MFMA tiles per work-group pass
+constexpr int PF_LDX = 264;       // halfs per staged token row: 256 + pad (stride = 4 banks mod 64: 16-byte reads)
 
 __device__ __forceinline__ half4_t bytes_to_half4_pf(uint32_t t)
 {
@@ -105,20 +104,25 @@ __device__ __forceinline__ half4_t bytes_to_half4_pf(uint32_t t)
   return half4_t{a.x, a.y, b.x, b.y};
 }
 
-// One work-group: 128 rows (wave = 32 rows) x 64 tokens, one super-block (256 columns) per step.
-//   * the weight operand sc_j * q (<= 63 * 15, exact in f16) is built once per super-block per wave and reused by both token
-//     tiles and by the hi and lo activation planes; the matrix cores accumulate across the whole super-block;
+typedef _Float16 half8_pf __attribute__((ext_vector_type(8)));
+
+// One work-group: 128 rows (wave = 32 rows) x TT * 32 tokens, one super-block (256 columns) per step, on
+// v_mfma_f32_32x32x16_f16 (lane (n, kg) supplies 8 consecutive k of row / column n).
+//   * the weight operand sc_j * q (<= 63 * 15, exact in f16) is built once per super-block per wave and reused by the
+//     token tiles and by the hi and lo activation planes; the matrix cores accumulate across the whole super-block, hi
+//     and lo planes into the same accumulator (the chains of the token tiles interleave);
 //   * -dmin * mn_j * sum_{k in j} x_k is one more MFMA step per plane (k = the 8 sub-blocks);
-//   * d and dmin are applied once per super-block (32 FMAs per tile), the token scale once at the end.
-// Work-group ids are laid out so that the token tiles of one row group run on one XCD: the 8 re-reads of its weights (one
-// per 64 tokens) hit that XCD's L2.
+//   * d and dmin are applied once per super-block (2 FMAs per value), the token scale once at the end.
+// Work-group ids are laid out so that the token tiles of one row group run on one XCD: the re-reads of its weights (one
+// per token tile) hit that XCD's L2.  TT = 1 doubles the number of work-groups for matrices with few row groups.
+template <int TT>
 __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
 {
   extern __shared__ __align__(16) unsigned char pf_smem[];
-  constexpr int NTOK = PF_TT * 32;
-  _Float16* xs_hi = reinterpret_cast<_Float16*>(pf_smem);            // [64][PF_LDX]
+  constexpr int NTOK = TT * 32;
+  _Float16* xs_hi = reinterpret_cast<_Float16*>(pf_smem);            // [NTOK][PF_LDX]
   _Float16* xs_lo = xs_hi + NTOK * PF_LDX;
-  _Float16* sx_hi = xs_lo + NTOK * PF_LDX;                            // [64][8]
+  _Float16* sx_hi = xs_lo + NTOK * PF_LDX;                            // [NTOK][8]
   _Float16* sx_lo = sx_hi + NTOK * 8;
   float* s_d = reinterpret_cast<float*>(sx_lo + NTOK * 8);            // [4 waves][2][32]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -140,9 +144,9 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
       for (int i = 0; i < 4; i++) r.q[i] = *reinterpret_cast<const uint4*>(blk + 16 + 64 * kg + 16 * i);
     }
   };
-  float16_t Y[PF_TT];
+  float16_t Y[TT];
 #pragma unroll
-  for (int tt = 0; tt < PF_TT; tt++)
+  for (int tt = 0; tt < TT; tt++)
 #pragma unroll
     for (int v = 0; v < 16; v++) Y[tt][v] = 0.0f;
 
@@ -150,24 +154,38 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
   load_w(0, wcur);
   for (int sb = 0; sb < nsb; sb++) {
     __syncthreads();                       // the previous step's LDS reads are done
-    // ---- stage 64 tokens x 256 columns of both planes, and the block sums ----
-    for (int idx = threadIdx.x; idx < NTOK * 32 * 2; idx += 256) {
-      const int chunk = idx & 31, tok = (idx >> 5) % NTOK, plane = (idx >> 5) / NTOK;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (T0 + tok < p.n_tok) v = *reinterpret_cast<const uint4*>((plane ? p.xlo : p.xhi) + (int64_t)(T0 + tok) * K + sb * 256 + chunk * 8);
-      uint2* dst = reinterpret_cast<uint2*>((plane ? xs_lo : xs_hi) + tok * PF_LDX + chunk * 8);
-      dst[0] = make_uint2(v.x, v.y); dst[1] = make_uint2(v.z, v.w);
+    // ---- stage NTOK tokens x 256 columns of both planes, and the block sums ----
+    {
+      // thread = (token tq + 8 i, 16-byte chunk): offsets from the uniform plane pointers stay 32-bit.  Token rows past
+      // the end repeat the last token (their results are never written), so the loads carry no branch and issue together.
+      const int tq = threadIdx.x >> 5, chunk = threadIdx.x & 31;
+      const uint32_t colo = (uint32_t)(sb * 256 + chunk * 8);
+      constexpr int SB = TT == 2 ? 1 : 4;     // loads in flight per plane (measured: with two token tiles the registers are worth more than the overlap)
+#pragma unroll
+      for (int i0 = 0; i0 < NTOK / 8; i0 += SB) {
+        uint4 vh[SB], vl[SB];
+#pragma unroll
+        for (int i = 0; i < SB; i++) {
+          const uint32_t off = (uint32_t)min(T0 + tq + 8 * (i0 + i), p.n_tok - 1) * (uint32_t)K + colo;
+          vh[i] = *reinterpret_cast<const uint4*>(p.xhi + off);
+          vl[i] = *reinterpret_cast<const uint4*>(p.xlo + off);
+        }
+#pragma unroll
+        for (int i = 0; i < SB; i++) {
+          *reinterpret_cast<uint4*>(xs_hi + (tq + 8 * (i0 + i)) * PF_LDX + chunk * 8) = vh[i];
+          *reinterpret_cast<uint4*>(xs_lo + (tq + 8 * (i0 + i)) * PF_LDX + chunk * 8) = vl[i];
+        }
+      }
     }
     if (threadIdx.x < NTOK * 2) {
       const int tok = threadIdx.x % NTOK, plane = threadIdx.x / NTOK;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (T0 + tok < p.n_tok) v = *reinterpret_cast<const uint4*>((plane ? p.sxlo : p.sxhi) + (int64_t)(T0 + tok) * nb32 + sb * 8);
+      const uint4 v = *reinterpret_cast<const uint4*>((plane ? p.sxlo : p.sxhi) + (int64_t)min(T0 + tok, p.n_tok - 1) * nb32 + sb * 8);
       *reinterpret_cast<uint4*>((plane ? sx_lo : sx_hi) + tok * 8) = v;
     }
     load_w(sb + 1, wnxt);
     __syncthreads();
 
-    // ---- weight operand of this super-block: 32 groups of four sc*q values ----
+    // ---- weight operand of this super-block: 16 groups of eight sc*q values ----
     const WRegs& r = wcur;
     const uint32_t sc4 = kg == 0 ? (r.h.y & 0x3f3f3f3fu) : ((r.h.w & 0x0f0f0f0fu) | ((r.h.y >> 2) & 0x30303030u));
     const uint32_t mn4 = kg == 0 ? (r.h.z & 0x3f3f3f3fu) : (((r.h.w >> 4) & 0x0f0f0f0fu) | ((r.h.z >> 2) & 0x30303030u));
@@ -180,23 +198,24 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
       const float dmin = __half2float(__ushort_as_half((unsigned short)(r.h.x >> 16)));
       s_d[(wave * 2 + 0) * 32 + n] = d; s_d[(wave * 2 + 1) * 32 + n] = dmin * 32.0f;
     }
-    half4_t A[4][8];
+    half8_pf A[4][4];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {                                      // sub-block 4kg + j
+    for (int j = 0; j < 4; j++) {                                      // sub-block 4kg + j: bytes of chunk 2kg + (j >> 1), low or high nibbles
       const int ccl = j >> 1, hl = j & 1;
       const _Float16 sj = j == 0 ? scv.x : (j == 1 ? scv.y : (j == 2 ? scv.z : scv.w));
       const half2_t s2 = {sj, sj};
       const half2_t c2 = {(_Float16)(-1024.0f) * sj, (_Float16)(-1024.0f) * sj};   // exact: a multiple of 1024 below 65504
 #pragma unroll
-      for (int t = 0; t < 8; t++) {
-        const uint4& qq = r.q[2 * ccl + (t >> 2)];
-        const uint32_t qd = (t & 3) == 0 ? qq.x : ((t & 3) == 1 ? qq.y : ((t & 3) == 2 ? qq.z : qq.w));
-        const uint32_t nib = hl ? ((qd >> 4) & 0x0f0f0f0fu) : (qd & 0x0f0f0f0fu);
-        const uint32_t p01 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04010400u);
-        const uint32_t p23 = __builtin_amdgcn_perm(0x64646464u, nib, 0x04030402u);
-        const half2_t a01 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, p01), s2, c2);   // (1024 + q) * sc - 1024 * sc = sc * q
-        const half2_t a23 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, p23), s2, c2);
-        A[j][t] = half4_t{a01.x, a01.y, a23.x, a23.y};
+      for (int t = 0; t < 4; t++) {                                    // weights 8t .. 8t+7 of the sub-block
+        const uint4& qq = r.q[2 * ccl + (t >> 1)];
+        const uint32_t qa = (t & 1) ? qq.z : qq.x, qb = (t & 1) ? qq.w : qq.y;
+        const uint32_t na = hl ? ((qa >> 4) & 0x0f0f0f0fu) : (qa & 0x0f0f0f0fu);
+        const uint32_t nb = hl ? ((qb >> 4) & 0x0f0f0f0fu) : (qb & 0x0f0f0f0fu);
+        const half2_t a0 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, na, 0x04010400u)), s2, c2);   // (1024 + q) * sc - 1024 * sc = sc * q
+        const half2_t a1 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, na, 0x04030402u)), s2, c2);
+        const half2_t a2 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, nb, 0x04010400u)), s2, c2);
+        const half2_t a3 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, nb, 0x04030402u)), s2, c2);
+        A[j][t] = half8_pf{a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
       }
     }
     __builtin_amdgcn_wave_barrier();
@@ -207,34 +226,33 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
       m4[g] = *reinterpret_cast<const float4*>(&s_d[(wave * 2 + 1) * 32 + 8 * g + 4 * kg]);
     }
     __builtin_amdgcn_wave_barrier();
+    float16_t C[TT], Cm[TT];
+    const float16_t zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int tt = 0; tt < PF_TT; tt++) {
-      float16_t C0, C1, Cm;
+    for (int j = 0; j < 4; j++)
 #pragma unroll
-      for (int v = 0; v < 16; v++) { C0[v] = 0.0f; C1[v] = 0.0f; Cm[v] = 0.0f; }
-      const _Float16* bh = xs_hi + (tt * 32 + n) * PF_LDX + 128 * kg;
-      const _Float16* bl = xs_lo + (tt * 32 + n) * PF_LDX + 128 * kg;
+      for (int t = 0; t < 4; t++)
 #pragma unroll
-      for (int j = 0; j < 4; j++)
-#pragma unroll
-        for (int t = 0; t < 8; t++) {
-          const half4_t Bh = *reinterpret_cast<const half4_t*>(bh + 32 * j + 4 * t);
-          const half4_t Bl = *reinterpret_cast<const half4_t*>(bl + 32 * j + 4 * t);
-          C0 = __builtin_amdgcn_mfma_f32_32x32x8f16(A[j][t], Bh, C0, 0, 0, 0);
-          C1 = __builtin_amdgcn_mfma_f32_32x32x8f16(A[j][t], Bl, C1, 0, 0, 0);
+        for (int tt = 0; tt < TT; tt++) {
+          const int off = (tt * 32 + n) * PF_LDX + 128 * kg + 32 * j + 8 * t;
+          const half8_pf Bh = *reinterpret_cast<const half8_pf*>(xs_hi + off);
+          const half8_pf Bl = *reinterpret_cast<const half8_pf*>(xs_lo + off);
+          if (j == 0 && t == 0) C[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[j][t], Bh, zero16, 0, 0, 0);   // a fresh accumulator per super-block
+          else C[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[j][t], Bh, C[tt], 0, 0, 0);
+          C[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[j][t], Bl, C[tt], 0, 0, 0);
         }
-      {
-        const half4_t Bmh = *reinterpret_cast<const half4_t*>(sx_hi + (tt * 32 + n) * 8 + 4 * kg);
-        const half4_t Bml = *reinterpret_cast<const half4_t*>(sx_lo + (tt * 32 + n) * 8 + 4 * kg);
-        Cm = __builtin_amdgcn_mfma_f32_32x32x8f16(mnv, Bmh, Cm, 0, 0, 0);
-        Cm = __builtin_amdgcn_mfma_f32_32x32x8f16(mnv, Bml, Cm, 0, 0, 0);
-      }
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++) {
+      const half4_t Bmh = *reinterpret_cast<const half4_t*>(sx_hi + (tt * 32 + n) * 8 + 4 * kg);
+      const half4_t Bml = *reinterpret_cast<const half4_t*>(sx_lo + (tt * 32 + n) * 8 + 4 * kg);
+      Cm[tt] = __builtin_amdgcn_mfma_f32_32x32x8f16(mnv, Bmh, zero16, 0, 0, 0);
+      Cm[tt] = __builtin_amdgcn_mfma_f32_32x32x8f16(mnv, Bml, Cm[tt], 0, 0, 0);
 #pragma unroll
       for (int g = 0; g < 4; g++) {
-        Y[tt][4 * g + 0] += d4[g].x * (C0[4 * g + 0] + C1[4 * g + 0]) - m4[g].x * Cm[4 * g + 0];
-        Y[tt][4 * g + 1] += d4[g].y * (C0[4 * g + 1] + C1[4 * g + 1]) - m4[g].y * Cm[4 * g + 1];
-        Y[tt][4 * g + 2] += d4[g].z * (C0[4 * g + 2] + C1[4 * g + 2]) - m4[g].z * Cm[4 * g + 2];
-        Y[tt][4 * g + 3] += d4[g].w * (C0[4 * g + 3] + C1[4 * g + 3]) - m4[g].w * Cm[4 * g + 3];
+        Y[tt][4 * g + 0] += d4[g].x * C[tt][4 * g + 0] - m4[g].x * Cm[tt][4 * g + 0];
+        Y[tt][4 * g + 1] += d4[g].y * C[tt][4 * g + 1] - m4[g].y * Cm[tt][4 * g + 1];
+        Y[tt][4 * g + 2] += d4[g].z * C[tt][4 * g + 2] - m4[g].z * Cm[tt][4 * g + 2];
+        Y[tt][4 * g + 3] += d4[g].w * C[tt][4 * g + 3] - m4[g].w * Cm[tt][4 * g + 3];
       }
     }
     wcur = wnxt;
@@ -242,7 +260,7 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
 
   // ---- write: lane holds column (token) n of each tile and rows 8g + 4kg + (0..3) ----
 #pragma unroll
-  for (int tt = 0; tt < PF_TT; tt++) {
+  for (int tt = 0; tt < TT; tt++) {
     const int t = T0 + tt * 32 + n;
     if (t >= p.n_tok) continue;
     const float si = p.sinv[t];
@@ -276,12 +294,23 @@ int launch_gemm_q4k(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo,
   p.w = w->data; p.bias = w->bias; p.rows = (int)w->rows; p.cols = (int)w->cols;
   p.xhi = xhi; p.xlo = xlo; p.sxhi = sxhi; p.sxlo = sxlo; p.sinv = sinv; p.n_tok = n_tok; p.y = y; p.y_stride = y_stride;
   p.residual = residual;
-  p.n_row_groups = (p.rows + 127) / 128; p.n_tok_tiles = (n_tok + PF_TT * 32 - 1) / (PF_TT * 32);
-  const size_t lds = (size_t)PF_TT * 32 * (PF_LDX + 8) * 2 * 2 + 4 * 2 * 32 * 4;
+  p.n_row_groups = (p.rows + 127) / 128;
+  // two token tiles per work-group reuse each weight operand four times; with few row groups one tile per work-group
+  // fills the chip better
+  static const int tt_force = []() { const char* e = getenv("CAIHIP_PF_TT"); return e ? atoi(e) : 0; }();
+  const int wgs2 = p.n_row_groups * ((n_tok + 63) / 64);
+  const int tt = tt_force == 1 || tt_force == 2 ? tt_force : (wgs2 < 2 * ctx().n_cu ? 1 : 2);
+  p.n_tok_tiles = (n_tok + tt * 32 - 1) / (tt * 32);
+  const size_t lds = (size_t)tt * 32 * (PF_LDX + 8) * 2 * 2 + 4 * 2 * 32 * 4;
   static bool attr_done = false;
-  if (!attr_done) { (void)hipFuncSetAttribute((const void*)gemm_q4k_pf, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); attr_done = true; }
+  if (!attr_done) {
+    (void)hipFuncSetAttribute((const void*)gemm_q4k_pf<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    (void)hipFuncSetAttribute((const void*)gemm_q4k_pf<2>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    attr_done = true;
+  }
   const int grid = 8 * p.n_tok_tiles * ((p.n_row_groups + 7) / 8);
-  hipLaunchKernelGGL(gemm_q4k_pf, dim3(grid), dim3(256), lds, ctx().stream, p);
+  if (tt == 1) hipLaunchKernelGGL(gemm_q4k_pf<1>, dim3(grid), dim3(256), lds, ctx().stream, p);
+  else hipLaunchKernelGGL(gemm_q4k_pf<2>, dim3(grid), dim3(256), lds, ctx().stream, p);
   return CAI_OK;
 }
 
