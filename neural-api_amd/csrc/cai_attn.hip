@@ -748,9 +748,10 @@ __global__ __launch_bounds__(256) void prompt_q_kernel(const PromptParams p)
       const float y0 = cs * x0 - sn * x1, y1 = sn * x0 + cs * x1;
       x0 = y0; x1 = y1;
     }
-    const _Float16 h0 = (_Float16)x0, h1 = (_Float16)x1;
+    _Float16 h0, h1, l0, l1;
+    split_f16(x0, h0, l0); split_f16(x1, h1, l1);
     p.qhi[(int64_t)t * qw + 2 * e] = h0; p.qhi[(int64_t)t * qw + 2 * e + 1] = h1;
-    p.qlo[(int64_t)t * qw + 2 * e] = (_Float16)(x0 - (float)h0); p.qlo[(int64_t)t * qw + 2 * e + 1] = (_Float16)(x1 - (float)h1);
+    p.qlo[(int64_t)t * qw + 2 * e] = l0; p.qlo[(int64_t)t * qw + 2 * e + 1] = l1;
   }
 }
 
@@ -830,15 +831,15 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
       for (int i4 = 0; i4 < 4; i4++) {                    // K rows stay row-major: 8-byte stores
         ph4_t kh, kl;
 #pragma unroll
-        for (int i = 0; i < 4; i++) { kh[i] = (_Float16)kv[4 * i4 + i]; kl[i] = (_Float16)(kv[4 * i4 + i] - (float)kh[i]); }
+        for (int i = 0; i < 4; i++) { _Float16 a, b; split_f16(kv[4 * i4 + i], a, b); kh[i] = a; kl[i] = b; }
         *reinterpret_cast<ph4_t*>(&sK[0][srow * PA_LDK + sdim + 4 * i4]) = kh;
         if (F32) *reinterpret_cast<ph4_t*>(&sK[NP - 1][srow * PA_LDK + sdim + 4 * i4]) = kl;
       }
 #pragma unroll
       for (int i = 0; i < 16; i++) {                      // V goes in transposed
-        const _Float16 vh = (_Float16)vv[i];
+        _Float16 vh, vl; split_f16(vv[i], vh, vl);
         sV[0][(sdim + i) * PA_LDV + srow] = vh;
-        if (F32) sV[NP - 1][(sdim + i) * PA_LDV + srow] = (_Float16)(vv[i] - (float)vh);
+        if (F32) sV[NP - 1][(sdim + i) * PA_LDV + srow] = vl;
       }
     }
     __syncthreads();
@@ -886,7 +887,7 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
     for (int s4 = 0; s4 < 4; s4++) {
       ph4_t ph, pl;
 #pragma unroll
-      for (int i = 0; i < 4; i++) { const _Float16 hv = (_Float16)C[4 * s4 + i]; ph[i] = hv; pl[i] = (_Float16)(C[4 * s4 + i] - (float)hv); }
+      for (int i = 0; i < 4; i++) { _Float16 hv, lv; split_f16(C[4 * s4 + i], hv, lv); ph[i] = hv; pl[i] = lv; }
 #pragma unroll
       for (int dt = 0; dt < 4; dt++) {
         const ph4_t a = *reinterpret_cast<const ph4_t*>(&sV[0][(32 * dt + n) * PA_LDV + 8 * s4 + 4 * kg]);

@@ -286,16 +286,16 @@ __global__ __launch_bounds__(256) void nb_prep_kernel(const NbPrepParams p)
   e = max(-60, min(60, e));
   const float s = ldexpf(1.0f, e);
   const float vs = v * s;
-  const _Float16 h = (_Float16)vs;
+  _Float16 h, l; split_f16(vs, h, l);
   const int64_t o = (int64_t)tok * p.K + k;
-  p.hi[o] = h; p.lo[o] = (_Float16)(vs - (float)h);
+  p.hi[o] = h; p.lo[o] = l;
   float sum = vs;
   for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);   // 32-lane groups = the 8 sub-blocks
   if ((threadIdx.x & 31) == 0) {
     const float q = sum * 0.03125f;
-    const _Float16 sh = (_Float16)q;
+    _Float16 sh, sl; split_f16(q, sh, sl);
     const int64_t b = (int64_t)tok * (p.K >> 5) + sb * 8 + (threadIdx.x >> 5);
-    p.sxhi[b] = sh; p.sxlo[b] = (_Float16)(q - (float)sh);
+    p.sxhi[b] = sh; p.sxlo[b] = sl;
   }
   if (threadIdx.x == 0) {
     p.sinvb[(int64_t)tok * (p.K >> 8) + sb] = ldexpf(1.0f, -e);

@@ -47,6 +47,17 @@ int  ensure_stage(void** p, size_t* cap, size_t need);
     if (!cai::ctx().ready) return cai::set_error(CAI_ERR_STATE, "cai_init has not been called"); \
   } while (0)
 
+// x = hi + lo for a pair of f16 operands (22 significant bits).  hi is rounded to 11 significant bits on the float's own
+// bit pattern (nearest even), so its conversion to f16 is exact whichever conversion instruction the compiler picks for
+// the scalar and for the packed use of the value (the two were seen to disagree in rare cases); lo = x - hi is exact in
+// fp32.  NaN and Inf stay what they are (lo of an Inf is NaN: still poison).
+__device__ __forceinline__ void split_f16(float x, _Float16& hi, _Float16& lo)
+{
+  const uint32_t b = __builtin_bit_cast(uint32_t, x);
+  const float h = __builtin_bit_cast(float, (b + 0xFFFu + ((b >> 13) & 1u)) & 0xFFFFE000u);
+  hi = (_Float16)h; lo = (_Float16)(x - h);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Resident weight matrix.  Device layouts (the on-disk block format stays the contract; these are
 // the library's own):

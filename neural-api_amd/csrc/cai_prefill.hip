@@ -68,15 +68,14 @@ __global__ __launch_bounds__(256) void xprep_kernel(const float* x, int64_t x_st
     float v = xr[i];
     if (gain) v = gain[i] * (v * inv);
     const float vs = v * s;
-    const _Float16 h = (_Float16)vs;
-    const _Float16 l = (_Float16)(vs - (float)h);
+    _Float16 h, l; split_f16(vs, h, l);
     hi[(int64_t)t * K + i] = h; lo[(int64_t)t * K + i] = l;
     float sum = v;
     for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
     if (l32 == 0) {   // the block sum in the scaled domain of hi/lo, divided by 32 so that it stays inside the half range
       const float ss = sum * s * 0.03125f;
-      const _Float16 sh = (_Float16)ss;
-      sxhi[(int64_t)t * (K >> 5) + b] = sh; sxlo[(int64_t)t * (K >> 5) + b] = (_Float16)(ss - (float)sh);
+      _Float16 sh, sl; split_f16(ss, sh, sl);
+      sxhi[(int64_t)t * (K >> 5) + b] = sh; sxlo[(int64_t)t * (K >> 5) + b] = sl;
     }
   }
 }

@@ -284,3 +284,29 @@ def test_eviction_int8_cache_tracks_fp32_cache():
         drift = max(drift, float(np.max(np.abs(a - b))))
     assert 0 < drift < 5e-2
     assert q.rows(0) == sinks + recent
+
+
+@pytest.mark.parametrize("hq,hkv,ctx", [(40, 8, 8192), (56, 8, 8192), (32, 16, 1024), (8, 8, 8192)])
+@pytest.mark.parametrize("kv", ["f16", "i8"])
+def test_grouped_decode_attention_fp16_int8(hq, hkv, ctx, kv):
+    """Grids that fill the chip (KV heads x slices >= 256) take the one-work-group-per-KV-head slice kernel (groups of
+    5, 7, 2 and 1 query heads here) with fp16 and int8 caches: same bar as the per-head kernel, int8 codes and scales
+    still exact, with a sliding window and a soft cap."""
+    from helpers.device import dev
+    cai = dev()
+    rng = np.random.default_rng(hq + ctx)
+    dk, n = 128, 150
+    rows = rng.standard_normal((n, (hq + 2 * hkv) * dk)).astype(np.float32)
+    for window, softcap in ((0, 0.0), (70, 25.0)):
+        if kv == "i8":
+            want, (kq, vq, ks, vs) = oracle_run_i8(rows, hq, hkv, dk, n, window, softcap)
+        else:
+            want = oracle_run(rows, hq, hkv, dk, n, window, 1, softcap)
+        cache = cai.KVCache(1, hkv, dk, ctx, cai.KV_I8 if kv == "i8" else cai.KV_F16)
+        for pos in range(n):
+            got = cache.attn_decode(0, rows[pos], hq, window, softcap)
+            assert np.max(np.abs(got - want[pos])) < 1e-5 * max(1.0, np.max(np.abs(want[pos]))), (window, pos)
+        if kv == "i8":
+            k, v, s_k, s_v = cache.export_layer(0)
+            np.testing.assert_array_equal(k, kq); np.testing.assert_array_equal(v, vq)
+            np.testing.assert_array_equal(s_k, ks); np.testing.assert_array_equal(s_v, vs)
