@@ -188,7 +188,7 @@ __device__ __forceinline__ float row16_allsum(float v)
 template <int HC, typename KV_T>
 __global__ __launch_bounds__(256) void attn_group_kernel(const AttnParams p)
 {
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   constexpr bool I8 = sizeof(KV_T) == 1;
   constexpr int NPF = sizeof(KV_T) == 4 ? 4 : 8;     // passes in flight per lane (32 registers either way)
   const int G = p.q_heads / p.kv_heads, n_chunks = (G + HC - 1) / HC;
