@@ -185,12 +185,11 @@ __device__ __forceinline__ float row16_allsum(float v)
   return v;
 }
 
-template <int HC, typename KV_T>
+template <int HC, typename KV_T, int NPF>     // NPF: passes in flight per lane
 __global__ __launch_bounds__(256) void attn_group_kernel(const AttnParams p)
 {
   extern __shared__ __align__(16) float lds[];
   constexpr bool I8 = sizeof(KV_T) == 1;
-  constexpr int NPF = sizeof(KV_T) == 4 ? 4 : 8;     // passes in flight per lane (32 registers either way)
   const int G = p.q_heads / p.kv_heads, n_chunks = (G + HC - 1) / HC;
   const int split = blockIdx.x % p.n_splits, g = blockIdx.x / p.n_splits, seq = blockIdx.y;
   const int pos = p.pos[seq];
@@ -618,6 +617,21 @@ static int launch_split_head(const AttnParams& p, int n_seq, hipStream_t st)
   return CAI_OK;
 }
 
+template <typename KV_T, int NPF>
+static void launch_group_t(const AttnParams& p, const dim3 grid, size_t lds, int hc, hipStream_t st)
+{
+  switch (hc) {
+    case 1: hipLaunchKernelGGL((attn_group_kernel<1, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
+    case 2: hipLaunchKernelGGL((attn_group_kernel<2, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
+    case 3: hipLaunchKernelGGL((attn_group_kernel<3, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
+    case 4: hipLaunchKernelGGL((attn_group_kernel<4, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
+    case 5: hipLaunchKernelGGL((attn_group_kernel<5, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
+    case 6: hipLaunchKernelGGL((attn_group_kernel<6, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
+    case 7: hipLaunchKernelGGL((attn_group_kernel<7, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
+    default: hipLaunchKernelGGL((attn_group_kernel<8, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
+  }
+}
+
 template <typename KV_T>
 static int launch_group(const AttnParams& p, int n_seq, hipStream_t st)
 {
@@ -627,16 +641,11 @@ static int launch_group(const AttnParams& p, int n_seq, hipStream_t st)
   const dim3 grid(p.n_splits * p.kv_heads, n_seq);
   const size_t lds = (size_t)(G * 128 + G * p.split_len + n_chunks * p.split_len * (hc > 4 ? 8 : 4) + 4 * hc * 128 + 2 * G) * sizeof(float);
   if (lds > 64 * 1024) return set_error(CAI_ERR_UNSUPPORTED, "attention: %d query heads per KV head need %zu bytes of LDS", G, lds);
-  switch (hc) {
-    case 1: hipLaunchKernelGGL((attn_group_kernel<1, KV_T>), grid, dim3(256), lds, st, p); break;
-    case 2: hipLaunchKernelGGL((attn_group_kernel<2, KV_T>), grid, dim3(256), lds, st, p); break;
-    case 3: hipLaunchKernelGGL((attn_group_kernel<3, KV_T>), grid, dim3(256), lds, st, p); break;
-    case 4: hipLaunchKernelGGL((attn_group_kernel<4, KV_T>), grid, dim3(256), lds, st, p); break;
-    case 5: hipLaunchKernelGGL((attn_group_kernel<5, KV_T>), grid, dim3(256), lds, st, p); break;
-    case 6: hipLaunchKernelGGL((attn_group_kernel<6, KV_T>), grid, dim3(256), lds, st, p); break;
-    case 7: hipLaunchKernelGGL((attn_group_kernel<7, KV_T>), grid, dim3(256), lds, st, p); break;
-    default: hipLaunchKernelGGL((attn_group_kernel<8, KV_T>), grid, dim3(256), lds, st, p); break;
-  }
+  // Several work-groups per CU: a shallow load ring frees registers for more resident waves (5 instead of 3 per SIMD),
+  // which hides the phase changes of one work-group behind the streaming of the others.  A grid of about one work-group
+  // per CU has nothing to overlap with and keeps the deep ring.
+  if ((int)(grid.x * grid.y) >= 3 * ctx().n_cu) launch_group_t<KV_T, 2>(p, grid, lds, hc, st);
+  else launch_group_t<KV_T, (sizeof(KV_T) == 4 ? 4 : 8)>(p, grid, lds, hc, st);
   return CAI_OK;
 }
 
