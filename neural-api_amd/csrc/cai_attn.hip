@@ -737,6 +737,7 @@ struct PromptParams {
   const float* qkv; int64_t qkv_stride;      // rows [Q | K | V], K and V already appended to the cache
   _Float16* qhi; _Float16* qlo;              // [token][q_heads * 128] rotated q, hi + lo
   const void* kc; const void* vc;            // this sequence's layer plane: [kv_head][max_ctx][128]
+  const float* ksc; const float* vsc;        // int8 cache: row scales of the same plane, [kv_head][max_ctx]
   int q_heads, kv_heads, max_ctx, n_tok, window;
   float softcap, inv_sqrt;
   const float* theta; const int32_t* pos;
@@ -770,8 +771,9 @@ constexpr int PA_LDV = 36;     // halfs per staged V^T row (32 cached rows + pad
 template <typename KV_T>
 __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
 {
-  constexpr bool F32 = sizeof(KV_T) == 4;
-  constexpr int NP = F32 ? 2 : 1;                 // planes of K and V: a float cache is split hi + lo
+  constexpr bool I8P = sizeof(KV_T) == 1;         // int8 rows are dequantised (code * row scale) while they are staged
+  constexpr bool F32 = sizeof(KV_T) != 2;         // ... and, like a float cache, split hi + lo
+  constexpr int NP = F32 ? 2 : 1;                 // planes of K and V
   __shared__ __align__(16) _Float16 sK[NP][32 * PA_LDK];
   __shared__ __align__(16) _Float16 sV[NP][128 * PA_LDV];
   const int G = p.q_heads / p.kv_heads, quads = (G + 3) >> 2;
@@ -814,7 +816,19 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
     {
       const int j = min(jt * 32 + srow, p.max_ctx - 1);     // rows past the live range are masked below
       float kv[16], vv[16];
-      if (F32) {
+      if (I8P) {
+        const uint4 a = *reinterpret_cast<const uint4*>(reinterpret_cast<const int8_t*>(kc) + (int64_t)j * 128 + sdim);
+        const uint4 b = *reinterpret_cast<const uint4*>(reinterpret_cast<const int8_t*>(vc) + (int64_t)j * 128 + sdim);
+        const float ks = p.ksc[(int64_t)g * p.max_ctx + j], vs = p.vsc[(int64_t)g * p.max_ctx + j];
+        const int aw[4] = {(int)a.x, (int)a.y, (int)a.z, (int)a.w}, bw[4] = {(int)b.x, (int)b.y, (int)b.z, (int)b.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          kv[4 * i] = (float)((aw[i] << 24) >> 24) * ks; kv[4 * i + 1] = (float)((aw[i] << 16) >> 24) * ks;
+          kv[4 * i + 2] = (float)((aw[i] << 8) >> 24) * ks; kv[4 * i + 3] = (float)(aw[i] >> 24) * ks;
+          vv[4 * i] = (float)((bw[i] << 24) >> 24) * vs; vv[4 * i + 1] = (float)((bw[i] << 16) >> 24) * vs;
+          vv[4 * i + 2] = (float)((bw[i] << 8) >> 24) * vs; vv[4 * i + 3] = (float)(bw[i] >> 24) * vs;
+        }
+      } else if (sizeof(KV_T) == 4) {
 #pragma unroll
         for (int c4 = 0; c4 < 4; c4++) {
           const float4 a = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(kc) + (int64_t)j * 128 + sdim + 4 * c4);
@@ -949,9 +963,9 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   }
   p.counters = kv->d_counters;
   int rc;
-  // prompts over a 128-wide fp32 / fp16 cache: matrix-core kernel, 32 tokens x 4 heads per work-group
+  // prompts over a 128-wide cache: matrix-core kernel, 32 tokens x 4 heads per work-group
   static const int flash_on = []() { const char* e = getenv("CAIHIP_PROMPT_FLASH"); return e ? atoi(e) : 1; }();
-  if (prompt_rows && flash_on && kv->head_dim == 128 && kv->dtype != CAI_KV_I8 && kv->evict_cap == 0 && n_seq >= 8) {
+  if (prompt_rows && flash_on && kv->head_dim == 128 && kv->evict_cap == 0 && n_seq >= 8) {
     const size_t need = (size_t)n_seq * q_heads * 128;
     if (need > kv->pq_cap) {
       CAI_HIP(hipStreamSynchronize(c.stream));
@@ -966,12 +980,17 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
     pp.qkv = qkv; pp.qkv_stride = qkv_stride; pp.qhi = (_Float16*)kv->pq_hi; pp.qlo = (_Float16*)kv->pq_lo;
     const size_t plane = ((size_t)seq0 * kv->seq_elems() + (size_t)layer * kv->layer_elems()) * kv->elem();
     pp.kc = (const char*)kv->k + plane; pp.vc = (const char*)kv->v + plane;
+    if (kv->dtype == CAI_KV_I8) {
+      const size_t rows0 = (size_t)seq0 * kv->seq_rows() + (size_t)layer * kv->layer_rows();
+      pp.ksc = kv->ks + rows0; pp.vsc = kv->vs + rows0;
+    }
     pp.q_heads = q_heads; pp.kv_heads = kv->kv_heads; pp.max_ctx = kv->max_ctx; pp.n_tok = n_seq; pp.window = window;
     pp.softcap = softcap; pp.inv_sqrt = p.inv_sqrt; pp.theta = theta; pp.pos = pos_dev; pp.out = out; pp.out_stride = out_stride;
     const int G = q_heads / kv->kv_heads;
     hipLaunchKernelGGL(prompt_q_kernel, dim3(n_seq), dim3(256), 0, c.stream, pp);
     const dim3 grid((n_seq + 31) / 32, kv->kv_heads * ((G + 3) / 4));
     if (kv->dtype == CAI_KV_F16) hipLaunchKernelGGL(attn_prompt_kernel<__half>, grid, dim3(256), 0, c.stream, pp);
+    else if (kv->dtype == CAI_KV_I8) hipLaunchKernelGGL(attn_prompt_kernel<int8_t>, grid, dim3(256), 0, c.stream, pp);
     else hipLaunchKernelGGL(attn_prompt_kernel<float>, grid, dim3(256), 0, c.stream, pp);
     return CAI_OK;
   }

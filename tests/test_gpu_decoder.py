@@ -264,26 +264,29 @@ def test_streaming_eviction_session_runs_past_max_ctx():
     assert drift < 5e-2, drift
 
 
-@pytest.mark.parametrize("kv,window", [("f32", 0), ("f16", 0), ("f32", 40), ("f16", 70)])
+@pytest.mark.parametrize("kv,window", [("f32", 0), ("f16", 0), ("f32", 40), ("f16", 70), ("i8", 0), ("i8", 50)])
 def test_prompt_attention_on_matrix_cores_equals_steps(kv, window):
     """Prompt ingestion over a 128-wide cache runs the matrix-core attention kernel (32 tokens x 4 heads per
-    work-group): the last token's logits equal token-at-a-time ingestion for fp32 and fp16 caches, under a sliding
+    work-group): the last token's logits equal token-at-a-time ingestion for fp32, fp16 and int8 caches, under a sliding
     window, for prompt lengths that are not multiples of the tile and for a continuation from position > 0."""
     from helpers.device import dev, rel_err
     cai = dev()
     s = SHAPES["qwen7b_like_q4k"]
     cfg = dict(s["cfg"]); cfg["max_ctx"] = 200; cfg["window"] = window
     spec = synthetic_spec(cfg, s["qtype"], head_qtype=s["head"], qkv_bias=True, std=0.05)
-    dec = cai.Decoder(spec, max_batch=2, kv_dtype=cai.KV_F16 if kv == "f16" else cai.KV_F32)
+    dec = cai.Decoder(spec, max_batch=2, kv_dtype={"f32": cai.KV_F32, "f16": cai.KV_F16, "i8": cai.KV_I8}[kv])
     rng = np.random.default_rng(11)
+    # int8: the two routes compute K and V rows that differ in the last bits, so now and then a code lands one step apart
+    tol = 5e-3 if kv == "i8" else 2e-4
     for n in (33, 97, 160):
         toks = rng.integers(0, cfg["vocab"], n).astype(np.int32)
         dec.reset(0); dec.reset(1)
         for p, t in enumerate(toks):
             am_s, last = dec.step(int(t), p)
         am_p, lg = dec.prefill(toks, 0, seq=1)
-        assert rel_err(lg, last[0]) < 2e-4, (n, rel_err(lg, last[0]))
-        assert am_p == int(am_s[0])
+        assert rel_err(lg, last[0]) < tol, (n, rel_err(lg, last[0]))
+        if kv != "i8":
+            assert am_p == int(am_s[0])
     # a second piece appended at position 50: attends over the rows of the first
     toks = rng.integers(0, cfg["vocab"], 120).astype(np.int32)
     dec.reset(0); dec.reset(1)
@@ -291,4 +294,4 @@ def test_prompt_attention_on_matrix_cores_equals_steps(kv, window):
         _, last = dec.step(int(t), p)
     dec.prefill(toks[:50], 0, seq=1, want_logits=False)
     _, lg = dec.prefill(toks[50:], 50, seq=1)
-    assert rel_err(lg, last[0]) < 2e-4
+    assert rel_err(lg, last[0]) < tol
