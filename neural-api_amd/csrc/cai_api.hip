@@ -293,7 +293,11 @@ extern "C" int cai_qgemv(cai_qw_t w, const float* x, int n_b, float* y, int act,
     dx = (const float*)c.stage_in;
   }
   if (!(flags & CAI_Y_DEVICE)) { if ((rc = ensure_stage(&c.stage_out, &c.stage_out_cap, yb))) return rc; dy = (float*)c.stage_out; }
-  if ((rc = launch_gemv(w, 0, w->rows, dx, n_b, dy, w->rows, act, nullptr))) return rc;
+  // A batch on a matrix too large for the cache: the VALU kernel would be compute-bound, the matrix-core kernel streams
+  // the weights once for the batch.  Small matrices stay on the single-launch kernel (three launches cost more there).
+  if (n_b >= 2 && act == CAI_ACT_NONE && nb_supported(w) && w->data_bytes >= ((int64_t)16 << 20)) {
+    if ((rc = nb_linear(w, dx, w->cols, nullptr, 0.0f, n_b, dy, w->rows, nullptr))) return rc;
+  } else if ((rc = launch_gemv(w, 0, w->rows, dx, n_b, dy, w->rows, act, nullptr))) return rc;
   CAI_HIP(hipGetLastError());
   if (!(flags & CAI_Y_DEVICE)) {
     CAI_HIP(hipMemcpyAsync(y, dy, yb, hipMemcpyDeviceToHost, c.stream));

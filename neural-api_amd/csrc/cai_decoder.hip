@@ -82,12 +82,12 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
   float* ssq_d = d->ssq + 1024;   // written by the down projection, read by the next block's q|k|v
   bool have_ssq_d = false;
   bool down_pending = false;      // small-batch path: the last down product has not been added to x yet
-  // 2..8 sequences on Q4_K weights: every linear layer goes to the matrix cores (weights streamed once for the batch)
+  // 2..8 sequences on block-quantized weights: every linear layer goes to the matrix cores (weights streamed once for the batch)
   auto mma_layer = [&](const cai_decoder_s::Layer& L) {
     if (n_b < 2 || c.n_experts > 0) return false;
     const int slots[6] = {CAI_W_Q, CAI_W_K, CAI_W_V, CAI_W_O, CAI_W_GATEUP, CAI_W_DOWN};
-    for (int sl : slots) if (!gemm_mfma_supported(L.w[sl])) return false;
-    return true;
+    for (int sl : slots) if (!nb_supported(L.w[sl])) return false;
+    return L.w[CAI_W_Q]->qtype == L.w[CAI_W_K]->qtype && L.w[CAI_W_Q]->qtype == L.w[CAI_W_V]->qtype;   // q | k | v share one launch
   };
   for (int l = 0; l < c.n_layers; l++) {
     auto& L = d->layers[l];
@@ -185,7 +185,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
   }
   {
     cai_qw_s* hw = d->head ? d->head : d->embed;   // tied head (neural/neuralpretrained.pas:15555-)
-    if (n_b >= 2 && gemm_mfma_supported(hw)) {
+    if (n_b >= 2 && nb_supported(hw)) {
       const int zero = 0; const cai_qw_s* hwc = hw;
       if (down_pending) rc = nb_prep_residual(d->x, dm, d->final_norm, c.eps, dm, n_b);
       else rc = nb_prep_plain(d->x, dm, d->final_norm, c.eps, dm, n_b);
@@ -230,7 +230,7 @@ static int ensure_prefill_buffers(cai_decoder_s* d, int n)
 static int linear_rows(const cai_qw_s* w, bool prepped, const float* x, int64_t x_stride, const float* gain, float eps, int n,
                        float* y, int64_t y_stride, const float* residual)
 {
-  if (gemm_mfma_supported(w) && n <= 16) return nb_linear(w, x, x_stride, gain, eps, n, y, y_stride, residual);   // bandwidth-bound regime
+  if (nb_supported(w) && (n <= 16 || !gemm_mfma_supported(w))) return nb_linear(w, x, x_stride, gain, eps, n, y, y_stride, residual);   // bandwidth-bound regime, or no prompt kernel for the type
   if (gemm_mfma_supported(w)) {
     int rc;
     if (!prepped && (rc = prefill_prep(x, x_stride, gain, eps, (int)w->cols, n))) return rc;

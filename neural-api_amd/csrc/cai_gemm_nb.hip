@@ -30,7 +30,7 @@ constexpr int NB_SC = 16;        // staged columns: 8 tokens x {hi, lo}
 constexpr int NB_TK = 8;         // tokens per pass
 constexpr int NB_SMAX = 5;       // super-blocks per K slice at most (LDS: 8.6 KB each, and three work-groups share a CU)
 
-struct NbSeg { const uint8_t* w; const float* bias; int rows; int y_off; int tile_end; };   // tile_end: cumulative 32-row tiles
+struct NbSeg { const uint8_t* w; const uint8_t* aux; const float* bias; int rows; int y_off; int tile_end; };   // aux: block scales plane (Q8_0 / Q4_0); tile_end: cumulative 32-row tiles
 
 struct NbParams {
   NbSeg seg[3]; int n_seg;                      // up to three matrices of equal width share one launch (q | k | v)
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
   _Float16* sxs = xs + S * NB_SC * NB_LDX;                           // [S][16][8]
   float* sinv_s = reinterpret_cast<float*>(sxs + S * NB_SC * 8);     // [S][8]
   float* s_d = sinv_s + S * NB_TK;                                   // [4 waves][2][32]: d, 32*dmin per row
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: segment lookups and loop bounds stay scalar
   const int n = lane & 15, kg = lane >> 4;
   const int K = p.cols, nsb = K >> 8, nb32 = K >> 5;
   const int slice = blockIdx.y, sb0 = slice * S, nS = min(S, nsb - sb0);
@@ -96,17 +96,18 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
     sg = &p.seg[sgi]; R0 = (tile - t0) * 32;
   };
   // weights of item q: for rows R0 + n and R0 + 16 + n the header and this lane's 32 quant bytes
+  // Loads are never conditional: past the wave's last item the last one is fetched again (a cache hit).  A load under a
+  // branch would make the compiler wait for ALL outstanding loads at every join.
   auto load_w = [&](int q, WRegs& r) {
-    if (q < nq) {
-      const int tile = tile0 + (q / nS) * p.tile_stride, sb = sb0 + q % nS;
-      const NbSeg* sg; int R0; locate(tile, sg, R0);
+    const int qc = max(min(q, nq - 1), 0);
+    const int tile = min(tile0 + (qc / nS) * p.tile_stride, p.n_tiles - 1), sb = sb0 + qc % nS;
+    const NbSeg* sg; int R0; locate(tile, sg, R0);
 #pragma unroll
-      for (int hh = 0; hh < 2; hh++) {
-        const uint8_t* blk = sg->w + (int64_t)min(R0 + 16 * hh + n, sg->rows - 1) * row_bytes + (int64_t)sb * 144;   // tail rows: re-read the last row
-        r.h[hh] = *reinterpret_cast<const uint4*>(blk);
-        r.q[hh][0] = *reinterpret_cast<const uint4*>(blk + 16 + 32 * kg);
-        r.q[hh][1] = *reinterpret_cast<const uint4*>(blk + 32 + 32 * kg);
-      }
+    for (int hh = 0; hh < 2; hh++) {
+      const uint8_t* blk = sg->w + (int64_t)min(R0 + 16 * hh + n, sg->rows - 1) * row_bytes + (int64_t)sb * 144;   // tail rows: re-read the last row
+      r.h[hh] = *reinterpret_cast<const uint4*>(blk);
+      r.q[hh][0] = *reinterpret_cast<const uint4*>(blk + 16 + 32 * kg);
+      r.q[hh][1] = *reinterpret_cast<const uint4*>(blk + 32 + 32 * kg);
     }
   };
   WRegs wa, wb, wc;
@@ -219,8 +220,212 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
 
   for (int q = 0; q < nq; q += 3) {
     load_w(q + 2, wc); compute(wa, q);
-    if (q + 1 < nq) { load_w(q + 3, wa); compute(wb, q + 1); }
-    if (q + 2 < nq) { load_w(q + 4, wb); compute(wc, q + 2); }
+    load_w(q + 3, wa); if (q + 1 < nq) compute(wb, q + 1);
+    load_w(q + 4, wb); if (q + 2 < nq) compute(wc, q + 2);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Q8_0 / Q4_0 (32-weight blocks, one f16 scale each: neural/neuralgguf.pas:389-441), stored as a quants plane and a
+// scales plane.  The block scale d belongs to a weight ROW, so here the roles of the operands are swapped: the
+// activations are the A operand (16 rows = 8 tokens x {hi, lo}) and 16 weight rows are the B operand.  A lane then
+// holds, for ONE weight row (lane % 16), the results of rows 4 kg .. 4 kg + 3 = four tokens - and d of its own row
+// is a value it loaded itself: result += d * (one MFMA over the 32 weights of the block), no exchange through LDS.
+// The codes are exact in f16: Q8_0 signed bytes, Q4_0 nibble - 8.  Columns are walked in groups of 8 blocks (the
+// granularity of the activation scales); a row's last group may be short (width % 256 != 0): the block index is
+// clamped, the staged activations beyond the width are zero and the scale of such a block counts as zero.
+// ------------------------------------------------------------------------------------------
+struct __attribute__((aligned(4))) Dwords4 { uint32_t x, y, z, w; };   // scale rows are 2-byte items: 4-byte alignment only
+
+template <int QT> __device__ __forceinline__ half8_t codes_to_half8(uint32_t w0, uint32_t w1)
+{
+  uint32_t a, b; _Float16 off;
+  if (QT == CAI_Q8_0) { a = w0 ^ 0x80808080u; b = w1 ^ 0x80808080u; off = (_Float16)(-1152.0f); }   // byte + 128, then 1024 + .. - 1152
+  else { a = w0 & 0x0f0f0f0fu; b = (w0 >> 4) & 0x0f0f0f0fu; off = (_Float16)(-1032.0f); }           // elements e and 16 + e of the block
+  const half2_t o2 = {off, off};
+  const half2_t h0 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, a, 0x04010400u)) + o2;
+  const half2_t h1 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, a, 0x04030402u)) + o2;
+  const half2_t h2 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, b, 0x04010400u)) + o2;
+  const half2_t h3 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, b, 0x04030402u)) + o2;
+  return half8_t{h0.x, h0.y, h1.x, h1.y, h2.x, h2.y, h3.x, h3.y};
+}
+
+// Lane (n = lane % 16, kg = lane / 16) loads 16 contiguous bytes per instruction, so that the four kg lanes of a row
+// fetch 64 contiguous bytes and adjacent instructions finish the cache line; v_permlane{16,32}_swap then hands every
+// MFMA the 8 codes per lane it needs from ONE block:
+//   Q8_0: a load covers two blocks of the row (kg 0, 1: the even one, kg 2, 3: the odd one); swapping the upper 8 bytes
+//         of the lower 32 lanes with the lower 8 bytes of the upper 32 lanes leaves the even block in the first two
+//         dwords of all four lanes and the odd block in the last two; lane kg then holds weights
+//         16 (kg & 1) + 8 (kg >> 1) .. + 7 of its block.
+//   Q4_0: a load is one whole block per lane (16 bytes of nibbles), four blocks per row; a 4 x 4 transposition of dwords
+//         over the kg lanes (swap by 32 lanes, then by 16) leaves dword kg of block c in register c: weights
+//         4 kg .. 4 kg + 3 (low nibbles) and 16 + 4 kg .. + 3 (high nibbles).
+typedef unsigned int uint2_t __attribute__((ext_vector_type(2)));
+
+template <int QT, bool TAIL>   // TAIL: width % 256 != 0
+__global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
+{
+  extern __shared__ __align__(16) unsigned char nb_smem[];
+  const int S = p.sb_per_slice;
+  _Float16* xs = reinterpret_cast<_Float16*>(nb_smem);              // [S][16][NB_LDX]
+  float* sinv_s = reinterpret_cast<float*>(xs + S * NB_SC * NB_LDX);  // [S][8]
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: segment lookups and loop bounds stay scalar
+  const int n = lane & 15, kg = lane >> 4;
+  const int K = p.cols, nsb = (K + 255) >> 8, nb32 = K >> 5;
+  const int slice = blockIdx.y, sb0 = slice * S, nS = min(S, nsb - sb0);
+  const int row_bytes = QT == CAI_Q8_0 ? K : (K >> 1);
+  const int aux_row_bytes = nb32 * 2;
+  const int tile0 = blockIdx.x * 4 + wave;
+  const int n_it = tile0 < p.n_tiles ? (p.n_tiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
+  // an item = 32 rows x 128 bytes of quants: 4 blocks of Q8_0 (half a group) or 8 blocks of Q4_0 (a whole group)
+  constexpr int IB = QT == CAI_Q8_0 ? 4 : 8;     // blocks per item
+  constexpr int IPG = 8 / IB;                    // items per group
+  const int nI = nS * IPG;                       // items per tile
+  const int nq = n_it * nI;
+
+  struct WRegs { uint32_t d[2][IB / 2]; uint4 q[2][2]; };
+  auto locate = [&](int tile, const NbSeg*& sg, int& R0) {
+    int sgi = 0, t0 = 0;
+    if (p.n_seg > 1 && tile >= p.seg[0].tile_end) { sgi = 1; t0 = p.seg[0].tile_end; }
+    if (p.n_seg > 2 && tile >= p.seg[1].tile_end) { sgi = 2; t0 = p.seg[1].tile_end; }
+    sg = &p.seg[sgi]; R0 = (tile - t0) * 32;
+  };
+  // Loads are never conditional: past the wave's last item the last one is fetched again (a cache hit).  A load under a
+  // branch would make the compiler wait for ALL outstanding loads at every join.
+  auto load_w = [&](int q, WRegs& r) {
+    const int qc = max(min(q, nq - 1), 0);
+    const int tile = min(tile0 + (qc / nI) * p.tile_stride, p.n_tiles - 1), it = qc % nI;
+    const int g0 = (sb0 + it / IPG) * 8 + (it % IPG) * IB;                         // first block of the item
+    const NbSeg* sg; int R0; locate(tile, sg, R0);
+#pragma unroll
+    for (int hh = 0; hh < 2; hh++) {
+      const int64_t row = min(R0 + 16 * hh + n, sg->rows - 1);                  // tail rows: re-read the last row
+      const uint8_t* qrow = sg->w + row * row_bytes;
+      const uint8_t* arow = sg->aux + row * aux_row_bytes;
+      if (!TAIL) {
+        if (QT == CAI_Q8_0) { const uint2 t = *reinterpret_cast<const uint2*>(arow + g0 * 2); r.d[hh][0] = t.x; r.d[hh][IB / 2 - 1] = t.y; }
+        else { const uint4 t = *reinterpret_cast<const uint4*>(arow + g0 * 2); r.d[hh][0] = t.x; r.d[hh][1] = t.y; r.d[hh][IB / 2 - 2] = t.z; r.d[hh][IB / 2 - 1] = t.w; }
+      } else {                                                                    // the row may end inside the item: absent blocks get scale 0
+#pragma unroll
+        for (int i = 0; i < IB / 2; i++) {
+          const int b0 = g0 + 2 * i;
+          const uint32_t lo16 = *reinterpret_cast<const uint16_t*>(arow + min(b0, nb32 - 1) * 2);
+          const uint32_t hi16 = *reinterpret_cast<const uint16_t*>(arow + min(b0 + 1, nb32 - 1) * 2);
+          r.d[hh][i] = (b0 < nb32 ? lo16 : 0u) | ((b0 + 1 < nb32 ? hi16 : 0u) << 16);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        int off = g0 * (QT == CAI_Q8_0 ? 32 : 16) + 64 * j + 16 * kg;
+        if (TAIL) off = max(0, min(off, row_bytes - 16));                         // stays inside the row; such codes meet scale 0
+        r.q[hh][j] = *reinterpret_cast<const uint4*>(qrow + off);
+      }
+    }
+  };
+  WRegs w0, w1, w2, w3;
+  load_w(0, w0); load_w(1, w1); load_w(2, w2); load_w(3, w3);   // weights do not depend on the staging below
+
+  // ---- stage this slice of the activations: nS x 16 columns x 256 halfs (zero beyond the width), block scales ----
+  for (int idx = threadIdx.x; idx < nS * NB_SC * 32; idx += 256) {
+    const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC;
+    const int tok = col % NB_TK, k = (sb0 + s) * 256 + chunk * 8;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (tok < p.n_tok && (!TAIL || k < K)) v = *reinterpret_cast<const uint4*>(((col / NB_TK) ? p.xlo : p.xhi) + (int64_t)tok * K + k);
+    *reinterpret_cast<uint4*>(xs + (s * NB_SC + col) * NB_LDX + chunk * 8) = v;
+  }
+  for (int idx = threadIdx.x; idx < nS * NB_TK; idx += 256) {
+    const int tok = idx % NB_TK, s = idx / NB_TK;
+    sinv_s[idx] = tok < p.n_tok ? p.sinvb[(int64_t)tok * nsb + sb0 + s] : 0.0f;
+  }
+  __syncthreads();
+
+  float acc[2][4], g[2][4];
+  const int xoff = QT == CAI_Q8_0 ? 16 * (kg & 1) + 8 * (kg >> 1) : 4 * kg;   // this lane's first weight within a block
+  auto compute = [&](const WRegs& r, int q) {
+    const int it = q % nI, s = it / IPG, part = it % IPG;
+    if (it == 0) {
+#pragma unroll
+      for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[hh][i] = 0.0f;
+    }
+    if (part == 0) {
+#pragma unroll
+      for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) g[hh][i] = 0.0f;
+    }
+    const _Float16* xcol = xs + (s * NB_SC + n) * NB_LDX + part * IB * 32 + xoff;
+    const float4_t z4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    auto block = [&](int hh, int b, uint32_t c0, uint32_t c1) {
+      half8_t X;
+      if (QT == CAI_Q8_0) X = *reinterpret_cast<const half8_t*>(xcol + 32 * b);
+      else {
+        const half4_t x0 = *reinterpret_cast<const half4_t*>(xcol + 32 * b);
+        const half4_t x1 = *reinterpret_cast<const half4_t*>(xcol + 32 * b + 16);
+        X = half8_t{x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+      }
+      const half8_t W = codes_to_half8<QT>(c0, c1);
+      const float4_t C = __builtin_amdgcn_mfma_f32_16x16x32_f16(X, W, z4, 0, 0, 0);
+      const uint32_t dw = r.d[hh][b >> 1];
+      const float d = __half2float(__ushort_as_half((unsigned short)((b & 1) ? (dw >> 16) : (dw & 0xffffu))));
+#pragma unroll
+      for (int i = 0; i < 4; i++) g[hh][i] = fmaf(d, C[i], g[hh][i]);
+    };
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+#pragma unroll
+      for (int hh = 0; hh < 2; hh++) {
+        const uint4 v = r.q[hh][j];
+        if (QT == CAI_Q8_0) {
+          const uint2_t s0 = __builtin_amdgcn_permlane32_swap(v.x, v.z, false, false);   // .x: even block, .y: odd block
+          const uint2_t s1 = __builtin_amdgcn_permlane32_swap(v.y, v.w, false, false);
+          block(hh, 2 * j, s0.x, s1.x);
+          block(hh, 2 * j + 1, s0.y, s1.y);
+        } else {
+          const uint2_t t02 = __builtin_amdgcn_permlane32_swap(v.x, v.z, false, false);
+          const uint2_t t13 = __builtin_amdgcn_permlane32_swap(v.y, v.w, false, false);
+          const uint2_t u01 = __builtin_amdgcn_permlane16_swap(t02.x, t13.x, false, false);  // blocks 4 j, 4 j + 1
+          const uint2_t u23 = __builtin_amdgcn_permlane16_swap(t02.y, t13.y, false, false);  // blocks 4 j + 2, 4 j + 3
+          block(hh, 4 * j, u01.x, 0u); block(hh, 4 * j + 1, u01.y, 0u);
+          block(hh, 4 * j + 2, u23.x, 0u); block(hh, 4 * j + 3, u23.y, 0u);
+        }
+      }
+    }
+    if (part != IPG - 1) return;
+    // result row 4 kg + i of the tile = token (4 kg + i) % 8, its hi (kg < 2) or lo (kg >= 2) part
+    const float4 si = *reinterpret_cast<const float4*>(&sinv_s[s * NB_TK + 4 * (kg & 1)]);
+#pragma unroll
+    for (int hh = 0; hh < 2; hh++) {
+      acc[hh][0] = fmaf(si.x, g[hh][0], acc[hh][0]); acc[hh][1] = fmaf(si.y, g[hh][1], acc[hh][1]);
+      acc[hh][2] = fmaf(si.z, g[hh][2], acc[hh][2]); acc[hh][3] = fmaf(si.w, g[hh][3], acc[hh][3]);
+    }
+    if (it != nI - 1) return;
+    // ---- the slice's contribution of this tile: hi + lo parts meet across kg ^ 2; lanes kg < 2 store four tokens ----
+    const int tile = tile0 + (q / nI) * p.tile_stride;
+    const NbSeg* sg; int R0; locate(tile, sg, R0);
+#pragma unroll
+    for (int hh = 0; hh < 2; hh++) {
+      const int row = R0 + 16 * hh + n;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const float tot = acc[hh][i] + __shfl_xor(acc[hh][i], 32, 64);
+        const int tok = 4 * kg + i;
+        if (kg < 2 && tok < p.n_tok && row < sg->rows)
+          p.part[((int64_t)slice * p.n_tok + tok) * p.part_stride + sg->y_off + row] = tot;
+      }
+    }
+  };
+
+  // ring of four items: three are in flight while one is consumed
+  for (int q = 0; q < nq; q += 4) {
+    compute(w0, q); load_w(q + 4, w0);
+    if (q + 1 < nq) compute(w1, q + 1);
+    load_w(q + 5, w1);
+    if (q + 2 < nq) compute(w2, q + 2);
+    load_w(q + 6, w2);
+    if (q + 3 < nq) compute(w3, q + 3);
+    load_w(q + 7, w3);
   }
 }
 
@@ -256,8 +461,11 @@ __global__ __launch_bounds__(256) void nb_prep_kernel(const NbPrepParams p)
 {
   const int sb = blockIdx.x, tok = blockIdx.y, k = sb * 256 + threadIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float v;
-  if (SRC == 0) v = p.x[(int64_t)tok * p.x_stride + k];
+  const int nsb = (p.K + 255) >> 8;
+  const bool in = k < p.K;                       // the last block of a width that is not a multiple of 256 is short
+  float v = 0.0f;
+  if (!in) {}
+  else if (SRC == 0) v = p.x[(int64_t)tok * p.x_stride + k];
   else if (SRC == 1) {
     v = p.res[(int64_t)tok * p.res_stride + k];
     if (p.bias) v += p.bias[k];
@@ -274,7 +482,7 @@ __global__ __launch_bounds__(256) void nb_prep_kernel(const NbPrepParams p)
     v = silu_mul(up, gate);
   }
   const float raw = v;
-  if (p.gain) v *= p.gain[k];
+  if (in && p.gain) v *= p.gain[k];
   __shared__ float red[8];
   float amax = fabsf(v), ss = raw * raw;
   for (int off = 32; off > 0; off >>= 1) { amax = fmaxf(amax, __shfl_xor(amax, off, 64)); ss += __shfl_xor(ss, off, 64); }
@@ -288,18 +496,18 @@ __global__ __launch_bounds__(256) void nb_prep_kernel(const NbPrepParams p)
   const float vs = v * s;
   _Float16 h, l; split_f16(vs, h, l);
   const int64_t o = (int64_t)tok * p.K + k;
-  p.hi[o] = h; p.lo[o] = l;
+  if (in) { p.hi[o] = h; p.lo[o] = l; }
   float sum = vs;
   for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);   // 32-lane groups = the 8 sub-blocks
-  if ((threadIdx.x & 31) == 0) {
+  if ((threadIdx.x & 31) == 0 && in) {
     const float q = sum * 0.03125f;
     _Float16 sh, sl; split_f16(q, sh, sl);
     const int64_t b = (int64_t)tok * (p.K >> 5) + sb * 8 + (threadIdx.x >> 5);
     p.sxhi[b] = sh; p.sxlo[b] = sl;
   }
   if (threadIdx.x == 0) {
-    p.sinvb[(int64_t)tok * (p.K >> 8) + sb] = ldexpf(1.0f, -e);
-    p.ssq[(int64_t)tok * (p.K >> 8) + sb] = (red[4] + red[5]) + (red[6] + red[7]);
+    p.sinvb[(int64_t)tok * nsb + sb] = ldexpf(1.0f, -e);
+    p.ssq[(int64_t)tok * nsb + sb] = (red[4] + red[5]) + (red[6] + red[7]);
   }
 }
 
@@ -359,8 +567,9 @@ int nb_reserve(int k_max, size_t part_floats)
     for (void* q : old) if (q) (void)hipFree(q);
     CAI_HIP(hipMalloc((void**)&g_nb.hi, need_k * 2)); CAI_HIP(hipMalloc((void**)&g_nb.lo, need_k * 2));
     CAI_HIP(hipMalloc((void**)&g_nb.sxhi, need_k / 32 * 2 + 64)); CAI_HIP(hipMalloc((void**)&g_nb.sxlo, need_k / 32 * 2 + 64));
-    CAI_HIP(hipMalloc((void**)&g_nb.sinvb, need_k / 256 * 4 + 64));
-    CAI_HIP(hipMalloc((void**)&g_nb.ssq[0], need_k / 256 * 4 + 64)); CAI_HIP(hipMalloc((void**)&g_nb.ssq[1], need_k / 256 * 4 + 64));
+    const size_t nblk = (size_t)NB_TK * ((k_max + 255) / 256);
+    CAI_HIP(hipMalloc((void**)&g_nb.sinvb, nblk * 4 + 64));
+    CAI_HIP(hipMalloc((void**)&g_nb.ssq[0], nblk * 4 + 64)); CAI_HIP(hipMalloc((void**)&g_nb.ssq[1], nblk * 4 + 64));
     g_nb.cap_k = need_k; g_nb.generation++;
   }
   if (part_floats > g_nb.cap_part) {
@@ -378,7 +587,7 @@ int nb_reserve(int k_max, size_t part_floats)
 // partial result every (tile, slice) writes and its consumer re-reads, priced at 0.45 item.
 static void nb_geometry(int cols, int tiles, int& S, int& n_slices, int& gx, int& tile_stride)
 {
-  const int nsb = cols >> 8, slots = 3 * ctx().n_cu;
+  const int nsb = (cols + 255) >> 8, slots = 3 * ctx().n_cu;
   static const int force = []() { const char* e = getenv("CAIHIP_NB_S"); return e ? atoi(e) : 0; }();
   const int s_lo = std::min(2, nsb), s_hi = std::min(NB_SMAX, nsb);
   float best = 3.0e38f;
@@ -394,15 +603,15 @@ static void nb_geometry(int cols, int tiles, int& S, int& n_slices, int& gx, int
   tile_stride = gx * 4;
 }
 // upper bound of the slice count for a width (sizes the partial buffer): S never drops below min(2, blocks per row)
-int nb_max_slices(int cols) { const int nsb = std::max(cols >> 8, 1); const int s = std::min(2, nsb); return (nsb + s - 1) / s; }
+int nb_max_slices(int cols) { const int nsb = std::max((cols + 255) >> 8, 1); const int s = std::min(2, nsb); return (nsb + s - 1) / s; }
 
 static int nb_prep_launch(int src, NbPrepParams& p, int n_tok)
 {
-  if (p.K % 256) return set_error(CAI_ERR_UNSUPPORTED, "small-batch pre-pass: width %d is not a multiple of 256", p.K);
+  if (p.K % 32) return set_error(CAI_ERR_UNSUPPORTED, "small-batch pre-pass: width %d is not a multiple of 32", p.K);
   if ((size_t)NB_TK * p.K > g_nb.cap_k || n_tok > NB_TK) return set_error(CAI_ERR_STATE, "small-batch pre-pass: workspace not reserved for %d x %d", n_tok, p.K);
   g_nb.cur ^= 1;
   p.hi = g_nb.hi; p.lo = g_nb.lo; p.sxhi = g_nb.sxhi; p.sxlo = g_nb.sxlo; p.sinvb = g_nb.sinvb; p.ssq = g_nb.ssq[g_nb.cur];
-  const dim3 grid(p.K >> 8, n_tok);
+  const dim3 grid((p.K + 255) >> 8, n_tok);
   if (src == 0) hipLaunchKernelGGL(nb_prep_kernel<0>, grid, dim3(256), 0, ctx().stream, p);
   else if (src == 1) hipLaunchKernelGGL(nb_prep_kernel<1>, grid, dim3(256), 0, ctx().stream, p);
   else hipLaunchKernelGGL(nb_prep_kernel<2>, grid, dim3(256), 0, ctx().stream, p);
@@ -445,17 +654,34 @@ int nb_prep_swiglu(int half, int n_tok)
   return CAI_OK;
 }
 
+// Weight types with a small-batch kernel.  Q4_K super-blocks make the width a multiple of 256 by construction.
+bool nb_supported(const cai_qw_s* w)
+{
+  if (w->qtype == CAI_Q4_K) return w->cols % 256 == 0;
+  return (w->qtype == CAI_Q8_0 || w->qtype == CAI_Q4_0) && w->cols % 32 == 0 && w->cols >= 32;
+}
+
+template <void (*Kernel)(const NbParams)>
+static void nb_launch(const NbParams& p, int gx, int n_slices, size_t lds)
+{
+  static bool attr_done = false;   // one flag per kernel
+  if (!attr_done) { (void)hipFuncSetAttribute((const void*)Kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); attr_done = true; }
+  hipLaunchKernelGGL(Kernel, dim3(gx, n_slices), dim3(256), lds, ctx().stream, p);
+}
+
 // partials <- [W0; W1; W2] . planes
 int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok)
 {
   if (n_w < 1 || n_w > 3 || n_tok < 1 || n_tok > NB_TK) return set_error(CAI_ERR_UNSUPPORTED, "small-batch gemm: %d matrices, %d tokens", n_w, n_tok);
   NbParams p{};
   p.n_seg = n_w; p.cols = (int)ws[0]->cols;
+  const int qt = ws[0]->qtype;
   int tiles = 0, width = 0;
   for (int i = 0; i < n_w; i++) {
-    if (ws[i]->qtype != CAI_Q4_K || ws[i]->cols != ws[0]->cols) return set_error(CAI_ERR_UNSUPPORTED, "small-batch gemm: matrix %d type %d width %lld", i, ws[i]->qtype, (long long)ws[i]->cols);
+    if (!nb_supported(ws[i]) || ws[i]->qtype != qt || ws[i]->cols != ws[0]->cols)
+      return set_error(CAI_ERR_UNSUPPORTED, "small-batch gemm: matrix %d type %d width %lld", i, ws[i]->qtype, (long long)ws[i]->cols);
     tiles += (int)((ws[i]->rows + 31) / 32);
-    p.seg[i].w = ws[i]->data; p.seg[i].bias = ws[i]->bias; p.seg[i].rows = (int)ws[i]->rows; p.seg[i].y_off = y_off[i]; p.seg[i].tile_end = tiles;
+    p.seg[i].w = ws[i]->data; p.seg[i].aux = ws[i]->aux; p.seg[i].bias = ws[i]->bias; p.seg[i].rows = (int)ws[i]->rows; p.seg[i].y_off = y_off[i]; p.seg[i].tile_end = tiles;
     width = std::max(width, y_off[i] + (int)ws[i]->rows);
   }
   p.n_tiles = tiles;
@@ -466,13 +692,18 @@ int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok)
     return set_error(CAI_ERR_STATE, "small-batch gemm: workspace not reserved (%d slices x %d tokens x %lld)", n_slices, n_tok, (long long)stride);
   p.xhi = g_nb.hi; p.xlo = g_nb.lo; p.sxhi = g_nb.sxhi; p.sxlo = g_nb.sxlo; p.sinvb = g_nb.sinvb; p.n_tok = n_tok;
   p.part = g_nb.part; p.part_stride = stride; p.sb_per_slice = S; p.tile_stride = tile_stride;
-  const size_t lds = (size_t)S * NB_SC * (NB_LDX + 8) * 2 + (size_t)S * NB_TK * 4 + 4 * 2 * 32 * 4;
-  static bool attr_done = false;
-  if (!attr_done) { (void)hipFuncSetAttribute((const void*)gemm_q4k_nb, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); attr_done = true; }
-  hipLaunchKernelGGL(gemm_q4k_nb, dim3(gx, n_slices), dim3(256), lds, ctx().stream, p);
+  if (qt == CAI_Q4_K) {
+    const size_t lds = (size_t)S * NB_SC * (NB_LDX + 8) * 2 + (size_t)S * NB_TK * 4 + 4 * 2 * 32 * 4;
+    nb_launch<gemm_q4k_nb>(p, gx, n_slices, lds);
+  } else {
+    const size_t lds = (size_t)S * NB_SC * NB_LDX * 2 + (size_t)S * NB_TK * 4;
+    const bool tail = p.cols % 256 != 0;
+    if (qt == CAI_Q8_0) { if (tail) nb_launch<gemm_blk_nb<CAI_Q8_0, true>>(p, gx, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_Q8_0, false>>(p, gx, n_slices, lds); }
+    else { if (tail) nb_launch<gemm_blk_nb<CAI_Q4_0, true>>(p, gx, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_Q4_0, false>>(p, gx, n_slices, lds); }
+  }
   for (int i = 0; i < 3; i++) g_prod.seg[i] = p.seg[i];
   g_prod.n_seg = n_w; g_prod.n_slices = n_slices; g_prod.n_tok = n_tok; g_prod.part_stride = stride; g_prod.width = width;
-  g_prod.in_ssq = g_pending_ssq; g_prod.in_nsb = g_pending_K >> 8; g_prod.in_K = g_pending_K; g_prod.in_eps = g_pending_eps;
+  g_prod.in_ssq = g_pending_ssq; g_prod.in_nsb = (g_pending_K + 255) >> 8; g_prod.in_K = g_pending_K; g_prod.in_eps = g_pending_eps;
   return CAI_OK;
 }
 
@@ -490,7 +721,7 @@ int nb_reduce(float* y, int64_t y_stride, const float* residual)
   return CAI_OK;
 }
 
-// Whole linear layer for up to 16 tokens (two passes above 8): y = W (gain . x / rms) + bias (+ residual)
+// Whole linear layer, 8 tokens per pass (the weights are streamed once per pass): y = W (gain . x / rms) + bias (+ residual)
 int nb_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok, float* y, int64_t y_stride, const float* residual)
 {
   int rc;

@@ -157,7 +157,8 @@ int kv_restore(cai_kv_s* kv, int seq, const cai_kv_snap_s* snap);
 // multi-token linear layer (matrix cores for Q4_K, small-batch kernel otherwise); gain != null fuses RMSNorm
 int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok,
                    float* y, int64_t y_stride, const float* residual);
-bool gemm_mfma_supported(const cai_qw_s* w);
+bool gemm_mfma_supported(const cai_qw_s* w);   // many-token (prompt) matrix-core kernel
+bool nb_supported(const cai_qw_s* w);          // 2..8-token matrix-core kernel
 // split pre-pass / product form: prep once, then any number of matrices of that width
 // small-batch (<= 8 tokens per pass) matrix-core path: planes <- activations, partials <- product, consumer sums the slices
 int nb_ws_generation();                                        // changes whenever its workspace buffers are reallocated

@@ -365,7 +365,7 @@ int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const fl
                    float* y, int64_t y_stride, const float* residual)
 {
   int rc;
-  if (gemm_mfma_supported(w) && n_tok <= 16) return nb_linear(w, x, x_stride, gain, eps, n_tok, y, y_stride, residual);   // bandwidth-bound regime
+  if (nb_supported(w) && (n_tok <= 16 || !gemm_mfma_supported(w))) return nb_linear(w, x, x_stride, gain, eps, n_tok, y, y_stride, residual);   // bandwidth-bound regime, or no prompt kernel for the type
   if (gemm_mfma_supported(w)) {
     if ((rc = prefill_prep(x, x_stride, gain, eps, (int)w->cols, n_tok))) return rc;
     return prefill_gemm(w, n_tok, y, y_stride, residual);

@@ -116,6 +116,29 @@ def test_generate_equals_step_loop_and_batch_equals_single():
             assert np.max(np.abs(lg[b] - singles[b][p])) <= 1e-5 * np.max(np.abs(singles[b][p]))
 
 
+@pytest.mark.parametrize("name", ["smollm_like_q8", "llama_like_q4_0"])
+def test_batched_decode_of_32_weight_block_models_equals_single(name):
+    """Q8_0 / Q4_0 models stepped as a batch run every linear layer on the matrix cores (width 576 ends in a short block group)."""
+    from helpers.device import dev
+    cai = dev()
+    s = SHAPES[name]
+    spec = synthetic_spec(s["cfg"], s["qtype"], head_qtype=s["head"], qkv_bias=s["bias"], std=0.05)
+    dec = cai.Decoder(spec, max_batch=5)
+    rng = np.random.default_rng(11)
+    toks = rng.integers(0, spec["cfg"]["vocab"], (5, 12))
+    singles = []
+    for b in range(5):
+        dec.reset(0)
+        singles.append([dec.step(int(toks[b, p]), p)[1][0].copy() for p in range(12)])
+    for b in range(5):
+        dec.reset(b)
+    for p in range(12):
+        am, lg = dec.step(toks[:, p], np.full(5, p))
+        for b in range(5):
+            assert np.max(np.abs(lg[b] - singles[b][p])) <= 2e-5 * np.max(np.abs(singles[b][p]))
+            assert int(am[b]) == int(np.argmax(singles[b][p]))
+
+
 def test_prefill_equals_sequential_steps():
     from helpers.device import dev, rel_err
     cai = dev()

@@ -182,3 +182,40 @@ def test_multi_token_gemm_other_types_and_tokens_not_multiple_of_eight():
         x = rng.standard_normal((13, 576)).astype(np.float32)
         got = cai.QWeight(qt, 200, 576, raw).gemm(x)
         assert rel_err(got, O.gemv(qt, raw, 200, 576, x, None, 0, 1)) < TIGHT
+
+
+@pytest.mark.parametrize("qt", [O.Q8_0, O.Q4_0])
+@pytest.mark.parametrize("rows,cols,T", [(128, 256, 2), (33, 512, 3), (1000, 1024, 8), (3584, 3584, 8), (512, 18944, 4), (40000, 2048, 16),
+                                         (5000, 768, 13), (577, 576, 8), (192, 576, 40), (96, 160, 5), (5, 32, 2), (70, 1536, 7)])
+def test_small_batch_gemm_q8_0_q4_0_on_matrix_cores(qt, rows, cols, T):
+    """32-weight block types on the matrix cores: signed codes as exact f16 (activations the A operand, 16 weight rows the B
+    operand, one MFMA per block, the block scale applied to its result) == T single-token layers, bias included.  Widths that
+    are not a multiple of 256 end in a short group of blocks."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    raw, rng = make(qt, rows, cols, T + 200)
+    x = (rng.standard_normal((T, cols)) * rng.uniform(0.01, 30.0, (T, 1))).astype(np.float32)
+    x[0, : cols // 2] = 0.0
+    bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
+    w = cai.QWeight(qt, rows, cols, raw, bias)
+    got = w.gemm(x)
+    want = O.gemv(qt, raw, rows, cols, x, bias, 0, 1)
+    for t in range(T):
+        assert rel_err(got[t], want[t], floor=0.02 * cols ** 0.5 * float(np.abs(x[t]).mean())) < TIGHT, t
+
+
+@pytest.mark.parametrize("qt,rows,cols", [(O.Q8_0, 4101, 4096), (O.Q4_0, 8203, 4096), (O.Q4_K, 8203, 4096)])
+@pytest.mark.parametrize("nb", [2, 4, 8])
+def test_gemv_batch_on_large_matrix_goes_to_matrix_cores(qt, rows, cols, nb):
+    """cai_qgemv with a batch on a matrix of 16 MiB or more takes the matrix-core small-batch path; same contract as batch 1."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    raw, rng = make(qt, rows, cols, nb)
+    x = rng.standard_normal((nb, cols)).astype(np.float32)
+    bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
+    w = cai.QWeight(qt, rows, cols, raw, bias)
+    got = w.gemv(x)
+    want = O.gemv(qt, raw, rows, cols, x, bias, 0, 1)
+    assert rel_err(got, want, floor=0.02 * cols ** 0.5) < TIGHT
+    one = w.gemv(x[:1])
+    assert rel_err(got[:1], one, floor=0.02 * cols ** 0.5) < TIGHT
