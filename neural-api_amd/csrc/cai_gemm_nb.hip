@@ -460,7 +460,7 @@ template <int SRC>
 __global__ __launch_bounds__(256) void nb_prep_kernel(const NbPrepParams p)
 {
   const int sb = blockIdx.x, tok = blockIdx.y, k = sb * 256 + threadIdx.x;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int nsb = (p.K + 255) >> 8;
   const bool in = k < p.K;                       // the last block of a width that is not a multiple of 256 is short
   float v = 0.0f;

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
   extern __shared__ float4 xs4[];          // [NB][kp/4]
   constexpr int UW = QTraits<QT>::UW, T = QTraits<QT>::T;
   constexpr int RR = MODE == 1 ? 2 * R : R;  // weight rows per wave
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int grp = blockIdx.x * 4 + wave;
 
   // segment lookup (groups never straddle segments)
@@ -342,7 +342,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
 template <int QT>
 __global__ __launch_bounds__(256) void gemv_simple(const GemvParams p, int n_b)
 {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int64_t grow = (int64_t)blockIdx.x * 4 + wave;
   int s = 0; int64_t g0 = 0;
   if (p.n_seg > 1 && grow >= p.seg[0].grp_end) { s = 1; g0 = p.seg[0].grp_end; }

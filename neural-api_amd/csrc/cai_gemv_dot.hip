@@ -75,7 +75,8 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
   __shared__ float s_ss[16];
   constexpr int CH = 4;                       // row groups between two meetings of the slice waves
   __shared__ float s_part[2][16][CH][RR];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: group indices, segment lookups and loop bounds stay scalar
   const int step = wave % nsw, gslot = wave / nsw;
   const int cols = p.cols, nsb = cols >> 8;
   const int64_t row_bytes = (int64_t)nsb * 144;
@@ -94,20 +95,21 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
     }
     sg = &p.seg[s]; row0 = (g - g0) * R;
   };
+  // Loads are never conditional: past the last group the last one is fetched again, lanes beyond the row's width fetch
+  // super-block 0 (both cache hits, the values are not used).  A load under a branch would make the compiler wait for
+  // ALL outstanding loads wherever the paths join, i.e. before every new request.
   auto issue = [&](int g, Q4kRegs (&rg)[RR]) {
-    if (g < n_groups && act) {
-      const GemvSeg* sg; int row0; locate(g, sg, row0);
-      const int lim = MODE == 1 ? p.half : sg->rows;
+    const GemvSeg* sg; int row0; locate(min(g, n_groups - 1), sg, row0);
+    const int lim = MODE == 1 ? p.half : sg->rows;
 #pragma unroll
-      for (int r = 0; r < RR; r++) {
-        int row = row0 + (MODE == 1 ? (r >> 1) : r);
-        if (row >= lim) row = lim - 1;               // tail group: re-read the last row, result is not written
-        if (MODE == 1 && (r & 1)) row += p.half;
-        const uint8_t* blk = sg->data + (int64_t)row * row_bytes + lane_off;
-        rg[r].h = *reinterpret_cast<const uint4*>(blk);
-        rg[r].q0 = *reinterpret_cast<const uint4*>(blk + 16 + 32 * cc);
-        rg[r].q1 = *reinterpret_cast<const uint4*>(blk + 32 + 32 * cc);
-      }
+    for (int r = 0; r < RR; r++) {
+      int row = row0 + (MODE == 1 ? (r >> 1) : r);
+      if (row >= lim) row = lim - 1;               // tail group: re-read the last row, result is not written
+      if (MODE == 1 && (r & 1)) row += p.half;
+      const uint8_t* blk = sg->data + (int64_t)row * row_bytes + lane_off;
+      rg[r].h = *reinterpret_cast<const uint4*>(blk);
+      rg[r].q0 = *reinterpret_cast<const uint4*>(blk + 16 + 32 * cc);
+      rg[r].q1 = *reinterpret_cast<const uint4*>(blk + 32 + 32 * cc);
     }
   };
 
@@ -228,7 +230,7 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
     float acc[RR];
 #pragma unroll
     for (int r = 0; r < RR; r++) acc[r] = 0.0f;
-    if (g < n_groups && act) {
+    if (g < n_groups) {   // lanes beyond the row's width hold zero activations: they add exactly 0
 #pragma unroll
       for (int r = 0; r < RR; r++) {
         const uint32_t qw[8] = {cur[r].q0.x, cur[r].q0.y, cur[r].q0.z, cur[r].q0.w, cur[r].q1.x, cur[r].q1.y, cur[r].q1.z, cur[r].q1.w};

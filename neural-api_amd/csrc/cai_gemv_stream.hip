@@ -29,7 +29,7 @@ __global__ __launch_bounds__(512, (MODE == 1 ? 2 * R : R) <= 2 ? 3 : 2) void gem
   __shared__ float s_ss[16];
   constexpr int CH = 4;                       // row groups between two meetings of the slice waves
   __shared__ float s_part[2][8][CH][RR];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int step = wave % nsw, gslot = wave / nsw;
   const int cols = p.cols, nsb = cols >> 8;
   const int64_t row_bytes = (int64_t)nsb * 144;

@@ -28,7 +28,7 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 __global__ __launch_bounds__(256) void xprep_kernel(const float* x, int64_t x_stride, const float* gain, float eps, int K,
                                                     _Float16* hi, _Float16* lo, float* sinv, _Float16* sxhi, _Float16* sxlo)
 {
-  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const float* xr = x + (int64_t)t * x_stride;
   __shared__ float red[4];
   __shared__ float s_scale;
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
   _Float16* sx_hi = xs_lo + NTOK * PF_LDX;                            // [NTOK][8]
   _Float16* sx_lo = sx_hi + NTOK * 8;
   float* s_d = reinterpret_cast<float*>(sx_lo + NTOK * 8);            // [4 waves][2][32]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, kg = lane >> 5;
   // linear id = rg_lo + 8 * (tt + n_tok_tiles * rg_hi): a row group's token tiles share id mod 8
   const int L = blockIdx.x, rg = (L & 7) + 8 * ((L >> 3) / p.n_tok_tiles), ttile = (L >> 3) % p.n_tok_tiles;
