@@ -224,6 +224,9 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
   }
 
   float ssq_acc = 0.0f;   // squares of the outputs this thread wrote (for the consumer's RMSNorm)
+  float keep[RR];         // finished totals of the last row groups, one group per lane
+#pragma unroll
+  for (int r = 0; r < RR; r++) keep[r] = 0.0f;
   auto process = [&](Q4kRegs (&cur)[RR], Q4kRegs (&nxt)[RR], int it) {
     const int g = g_first + it * g_stride;
     issue(g + (NS - 1) * g_stride, nxt);
@@ -292,15 +295,24 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
       }
       return;
     }
-    if (lane != 63 || g >= n_groups) return;
-
-    const GemvSeg* sg; int row0; locate(g, sg, row0);
+    // One wave per row group: the totals of up to 16 groups are parked, one group per lane, and finished together
+    // (bias, activation, residual, store: a single pass of vector code instead of one-lane code after every group).
+    const int slot = it & 15;
+#pragma unroll
+    for (int r = 0; r < RR; r++) {
+      const float tot = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, acc[r]), 63));
+      keep[r] = lane == slot ? tot : keep[r];
+    }
+    if (slot != 15 && it != n_iters - 1) return;
+    const int gg = g_first + (it - slot + lane) * g_stride;
+    if (lane > slot || gg >= n_groups) return;
+    const GemvSeg* sg; int row0; locate(gg, sg, row0);
     if (MODE == 0) {
 #pragma unroll
       for (int r = 0; r < RR; r++) {
         const int row = row0 + r;
         if (row >= sg->rows) break;
-        float v = acc[r];
+        float v = keep[r];
         if (sg->bias) v += sg->bias[row];
         v = act_apply(v, p.act);
         const int o = sg->y_off + row;
@@ -312,7 +324,7 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
       for (int r = 0; r < R; r++) {
         const int row = row0 + r;
         if (row >= p.half) break;
-        float up = acc[2 * r], gate = acc[2 * r + 1];
+        float up = keep[2 * r], gate = keep[2 * r + 1];
         if (sg->bias) { up += sg->bias[row]; gate += sg->bias[p.half + row]; }
         p.y[sg->y_off + row] = silu_mul(up, gate);
       }
@@ -350,7 +362,7 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
   static const int W = []() { const char* e = getenv("CAIHIP_DOT_W"); return e ? atoi(e) : 12; }();   // resident waves per CU
   // row groups in flight per work-group: short rows share one quantised activation among 4 waves; long rows
   // fill the CU with a single work-group
-  const int gwv = nsw >= 3 ? std::max(1, W / nsw) : 4 / nsw;
+  const int gwv = nsw >= 3 ? std::max(1, std::min(W, 12) / nsw) : 4 / nsw;   // the kernel is built for at most 12 waves per work-group
   int64_t total = 0;
   for (int i = 0; i < m.n; i++) total += swiglu_half ? swiglu_half : m.rows[i];
   const int waves_per_wg = nsw * gwv;
