@@ -16,6 +16,7 @@
 //                           sequence with a short cache.
 // Cache element types: fp32, IEEE half, or int8 codes with one fp32 scale per cached row (neural/neural.cl:2501-2687).
 #include "cai_internal.hpp"
+#include "cai_gemv_common.hpp"
 
 namespace cai {
 
@@ -117,6 +118,7 @@ struct AttnParams {
   float* ksc; float* vsc;      // int8 caches: row scales [seq][layer][kv_head][max_ctx]
   int64_t seq_rows, layer_row_off;
   int evict_sinks, evict_cap;  // cap > 0: only the first `sinks` positions and the latest cap - sinks stay cached
+  const float* qn_gain; const float* kn_gain; float qk_eps;   // full-width RMSNorm of q and of k applied while they are read (null: rows are used as they are)
 };
 
 // Where the row of stream position `pos` lives and which rows are live.  Without eviction: slot = pos, rows
@@ -480,6 +482,21 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
   load_chunk(cA, s_begin + hw);      // cached rows are requested before the rotation math
   load_chunk(cB, s_begin + hw + 8 * PCH);
 
+  // Full-width RMSNorm of q and k (neural/neuralpretrained.pas:16511-16530) folded into this kernel: every work-group
+  // sums the squares of the whole q and k rows itself (same order as the stand-alone kernel: strided per thread, wave
+  // totals, (w0 + w1) + (w2 + w3)) and scales the elements it reads.
+  float inv_q = 1.0f, inv_k = 1.0f;
+  if (p.qn_gain) {
+    __shared__ float nred[8];
+    float sq = 0.0f, sk = 0.0f;
+    for (int i = tid; i < qw; i += 256) sq = fmaf(row[i], row[i], sq);
+    for (int i = tid; i < kw; i += 256) sk = fmaf(row[qw + i], row[qw + i], sk);
+    sq = wave_sum(sq); sk = wave_sum(sk);
+    if ((tid & 63) == 63) { nred[tid >> 6] = sq; nred[4 + (tid >> 6)] = sk; }
+    __syncthreads();
+    inv_q = 1.0f / sqrtf(((nred[0] + nred[1]) + (nred[2] + nred[3])) / (float)qw + p.qk_eps);
+    inv_k = 1.0f / sqrtf(((nred[4] + nred[5]) + (nred[6] + nred[7])) / (float)kw + p.qk_eps);
+  }
   float rs[(DS + 1) / 2], rc[(DS + 1) / 2];
 #pragma unroll
   for (int i = 0; i < (DS + 1) / 2; i++) {
@@ -487,32 +504,33 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
     const int d = d0 + 2 * i;
     if (p.theta && d < hd) { const float angle = (float)pos * p.theta[d >> 1]; sincosf(angle, &rs[i], &rc[i]); }
   }
-  auto load_rot = [&](const float* v, float (&o)[DS], bool rotate) {
+  auto load_rot = [&](const float* v, float (&o)[DS], bool rotate, const float* gain, float inv) {
+    auto elem = [&](int d) { return d < hd ? (gain ? gain[d] * (v[d] * inv) : v[d]) : 0.0f; };
     if (DS >= 2) {
 #pragma unroll
       for (int i = 0; i < DS; i += 2) {
         const int d = d0 + i;
-        const float x0 = d < hd ? v[d] : 0.0f, x1 = d + 1 < hd ? v[d + 1] : 0.0f;
+        const float x0 = elem(d), x1 = elem(d + 1);
         if (rotate) { o[i] = rc[i / 2] * x0 - rs[i / 2] * x1; o[i + (DS > 1 ? 1 : 0)] = rs[i / 2] * x0 + rc[i / 2] * x1; }
         else { o[i] = x0; o[i + (DS > 1 ? 1 : 0)] = x1; }
       }
     } else {
       const int d = d0;
-      const float own = d < hd ? v[d] : 0.0f, mate = (d ^ 1) < hd ? v[d ^ 1] : 0.0f;
+      const float own = elem(d), mate = elem(d ^ 1);
       if (rotate) o[0] = (d & 1) ? (rs[0] * mate + rc[0] * own) : (rc[0] * own - rs[0] * mate);
       else o[0] = own;
     }
   };
   float q[DS], knew[DS], vnew[DS], acc[DS];
-  load_rot(row + (g * G + h) * hd, q, p.theta != nullptr);
+  load_rot(row + (g * G + h) * hd, q, p.theta != nullptr, p.qn_gain ? p.qn_gain + (g * G + h) * hd : nullptr, inv_q);
 #pragma unroll
   for (int i = 0; i < DS; i++) { acc[i] = 0.0f; knew[i] = 0.0f; vnew[i] = 0.0f; }
   // every work-group whose slice holds `pos` keeps the new row in registers; the group's first head appends it
   const bool owns_new = !p.appended && slot >= s_begin && slot < s_end;
   float knew_s = 1.0f, vnew_s = 1.0f;
   if (owns_new) {
-    load_rot(row + qw + g * hd, knew, p.theta != nullptr);
-    load_rot(row + qw + kw + g * hd, vnew, false);
+    load_rot(row + qw + g * hd, knew, p.theta != nullptr, p.kn_gain ? p.kn_gain + g * hd : nullptr, inv_k);
+    load_rot(row + qw + kw + g * hd, vnew, false, nullptr, 1.0f);
     if constexpr (I8) {
       knew_s = quantise_row_i8<DS>(knew);
       vnew_s = quantise_row_i8<DS>(vnew);
@@ -936,7 +954,7 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
 
 int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, int n_seq, int q_heads, int window,
                      float softcap, const float* theta, const int32_t* pos_dev, float* out, int64_t out_stride, int seq0,
-                     int prompt_rows, float* prompt_part)
+                     int prompt_rows, float* prompt_part, const float* qn_gain, const float* kn_gain, float qk_eps)
 {
   Context& c = ctx();
   if (layer < 0 || layer >= kv->n_layers) return set_error(CAI_ERR_INVALID, "attention: layer %d of %d", layer, kv->n_layers);
@@ -953,6 +971,16 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   p.seq_mul = prompt_rows ? 0 : 1; p.appended = prompt_rows ? 1 : 0;
   p.evict_sinks = kv->evict_sinks; p.evict_cap = kv->evict_cap;
   p.ksc = kv->ks; p.vsc = kv->vs; p.seq_rows = kv->seq_rows(); p.layer_row_off = (int64_t)layer * kv->layer_rows();
+  int rc;
+  static const int group_min = []() { const char* e = getenv("CAIHIP_ATTN_GROUP_MIN"); return e ? atoi(e) : 256; }();
+  const bool grouped = (kv->head_dim & 7) == 0 && n_seq * kv->kv_heads * kv->n_splits >= group_min;
+  if (qn_gain) {
+    // q and k norms over the whole rows: the per-head decode kernel applies them while it reads its operands; the
+    // other kernels find the rows normalised in place
+    const int qw = q_heads * kv->head_dim, kw = kv->kv_heads * kv->head_dim;
+    if (!prompt_rows && !grouped) { p.qn_gain = qn_gain; p.kn_gain = kn_gain; p.qk_eps = qk_eps; }
+    else if ((rc = launch_rmsnorm_pair(qkv, qn_gain, qw, kn_gain, kw, n_seq, qk_eps, qkv_stride))) return rc;
+  }
   if (prompt_rows && kv->dtype == CAI_KV_I8) {
     if (p.hd <= 32) hipLaunchKernelGGL(kv_append_rows_i8_kernel<1>, dim3(n_seq), dim3(256), 0, c.stream, p);
     else if (p.hd <= 64) hipLaunchKernelGGL(kv_append_rows_i8_kernel<2>, dim3(n_seq), dim3(256), 0, c.stream, p);
@@ -962,7 +990,6 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
     else hipLaunchKernelGGL(kv_append_rows_kernel<float>, dim3(n_seq), dim3(256), 0, c.stream, p);
   }
   p.counters = kv->d_counters;
-  int rc;
   // prompts over a 128-wide cache: matrix-core kernel, 32 tokens x 4 heads per work-group
   static const int flash_on = []() { const char* e = getenv("CAIHIP_PROMPT_FLASH"); return e ? atoi(e) : 1; }();
   if (prompt_rows && flash_on && kv->head_dim == 128 && kv->evict_cap == 0 && n_seq >= 8) {
@@ -996,8 +1023,6 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   }
   // one work-group per (slice, KV head) serving the whole group of query heads, or one per (slice, query head)
   // (the first fetches K and V once but has G times fewer work-groups: it needs a grid that fills the chip by itself)
-  static const int group_min = []() { const char* e = getenv("CAIHIP_ATTN_GROUP_MIN"); return e ? atoi(e) : 256; }();
-  const bool grouped = (kv->head_dim & 7) == 0 && n_seq * kv->kv_heads * kv->n_splits >= group_min;
   if (grouped)
     rc = kv->dtype == CAI_KV_I8 ? launch_group<int8_t>(p, n_seq, c.stream) : kv->dtype == CAI_KV_F16 ? launch_group<__half>(p, n_seq, c.stream) : launch_group<float>(p, n_seq, c.stream);
   else

@@ -101,8 +101,8 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
         const cai_qw_s* qkv3[3] = {L.w[CAI_W_Q], L.w[CAI_W_K], L.w[CAI_W_V]}; const int off3[3] = {0, qw, qw + kw};
         if ((rc = nb_gemm(qkv3, off3, 3, n_b)) || (rc = nb_reduce(d->qkv, qkvw, nullptr))) return rc;
       }
-      if (c.qk_norm_full) launch_rmsnorm_pair(d->qkv, L.v[CAI_V_Q_NORM], qw, L.v[CAI_V_K_NORM], kw, n_b, c.eps, qkvw);
-      if ((rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0))) return rc;
+      if ((rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0, 0, nullptr,
+                                 c.qk_norm_full ? L.v[CAI_V_Q_NORM] : nullptr, c.qk_norm_full ? L.v[CAI_V_K_NORM] : nullptr, c.eps))) return rc;
       const int zero = 0;
       const cai_qw_s* wo = L.w[CAI_W_O]; const cai_qw_s* wgu = L.w[CAI_W_GATEUP]; const cai_qw_s* wdn = L.w[CAI_W_DOWN];
       if ((rc = nb_prep_plain(d->att, qw, nullptr, 0.0f, qw, n_b)) || (rc = nb_gemm(&wo, &zero, 1, n_b))) return rc;
@@ -132,10 +132,8 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
         }
       }
     }
-    if (c.qk_norm_full) {
-      launch_rmsnorm_pair(d->qkv, L.v[CAI_V_Q_NORM], qw, L.v[CAI_V_K_NORM], kw, n_b, c.eps, qkvw);
-    }
-    if ((rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0))) return rc;
+    if ((rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0, 0, nullptr,
+                               c.qk_norm_full ? L.v[CAI_V_Q_NORM] : nullptr, c.qk_norm_full ? L.v[CAI_V_K_NORM] : nullptr, c.eps))) return rc;
     const bool o_hands = gemv_hands_off_ssq(L.w[CAI_W_O], n_b);
     {
       MultiGemv m{}; m.n = 1; m.w[0] = L.w[CAI_W_O]; m.rows[0] = dm;
@@ -254,10 +252,8 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
     if ((rc = linear_rows(wq, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv, qkvw, nullptr))) return rc;
     if ((rc = linear_rows(wk, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw, qkvw, nullptr))) return rc;
     if ((rc = linear_rows(wv, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw + kw, qkvw, nullptr))) return rc;
-    if (c.qk_norm_full) {
-      launch_rmsnorm_pair(d->pqkv, L.v[CAI_V_Q_NORM], qw, L.v[CAI_V_K_NORM], kw, n, c.eps, qkvw);
-    }
-    if ((rc = launch_attn_step(&d->kv, l, d->pqkv, qkvw, n, c.n_q_heads, c.window, 0.0f, d->theta, poss, d->patt, qw, seq, 1, d->ppart))) return rc;
+    if ((rc = launch_attn_step(&d->kv, l, d->pqkv, qkvw, n, c.n_q_heads, c.window, 0.0f, d->theta, poss, d->patt, qw, seq, 1, d->ppart,
+                               c.qk_norm_full ? L.v[CAI_V_Q_NORM] : nullptr, c.qk_norm_full ? L.v[CAI_V_K_NORM] : nullptr, c.eps))) return rc;
     if ((rc = linear_rows(L.w[CAI_W_O], false, d->patt, qw, nullptr, 0.0f, n, d->px, dm, d->px))) return rc;
     if ((rc = linear_rows(L.w[CAI_W_GATEUP], false, d->px, dm, L.v[CAI_V_MLP_NORM], c.eps, n, d->pgu, 2 * I, nullptr))) return rc;
     launch_swiglu(d->pgu, I, n, d->pmid);

@@ -148,7 +148,8 @@ int launch_split_blocks(const uint8_t* raw, int block_bytes, int64_t n_blocks, u
 // hold n_seq * q_heads * n_splits * (head_dim + 2) floats.
 int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, int n_seq, int q_heads, int window,
                      float softcap, const float* theta, const int32_t* pos_dev, float* out, int64_t out_stride, int seq0,
-                     int prompt_rows = 0, float* prompt_part = nullptr);
+                     int prompt_rows = 0, float* prompt_part = nullptr,
+                     const float* qn_gain = nullptr, const float* kn_gain = nullptr, float qk_eps = 0.0f);   // full-width q / k RMSNorm done on the way (null: none)
 int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, int max_ctx, int dtype);
 void kv_free(cai_kv_s* kv);
 int kv_set_eviction(cai_kv_s* kv, int sinks, int recent);

@@ -306,6 +306,24 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float* logits, in
     if (c < n) probs[(int64_t)t * n + c] = v[i]; else v[i] = -1.0f;   // -1 marks "not a candidate"
   }
   float sum = 0.0f, mine = 0.0f;   // lane j keeps the j-th selected gate
+  if (n <= 64) {
+    // One expert per lane: every lane ranks its own probability against the 64 broadcast ones (larger first, lower
+    // index between equals) - a permutation of 0..63 - and the lanes of rank 0..k-1 are the selection, in order.
+    const float pv = v[0];
+    int rank = 0;
+    for (int j = 0; j < 64; j++) {
+      const float o = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pv), j));
+      rank += (o > pv || (o == pv && j < lane)) ? 1 : 0;
+    }
+    for (int j = 0; j < k; j++) {
+      const int src = __ffsll((unsigned long long)__ballot(rank == j)) - 1;
+      const float bv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pv), src));
+      if (lane == j) { mine = bv; expert_out[t * k + j] = src; }
+      sum += bv;
+    }
+    if (lane < k) gate_out[t * k + lane] = renorm ? (sum > 0.0f ? mine * (1.0f / sum) : 0.0f) : mine;
+    return;
+  }
   for (int j = 0; j < k; j++) {
     float bv = -1.0f; int bc = 0x7fffffff;
 #pragma unroll
