@@ -1046,6 +1046,10 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   // while one CU sustains only ~20 GB/s, so a slice should stay under ~100 KB
   static const int sl_max = []() { const char* e = getenv("CAIHIP_ATTN_SPLIT_MAX"); const int v = e ? atoi(e) : 256; return v >= 32 ? v : 256; }();
   int sl = (max_ctx + 15) / 16; sl = (sl + 31) / 32 * 32; if (sl < 32) sl = 32; if (sl > sl_max) sl = sl_max;
+  // a head's whole K (or V) plane of at most 64 KB is one slice: a single work-group streams it in a few microseconds and
+  // the merge launch disappears (small models at short contexts are bound by launches, not by bytes)
+  static const int single_bytes = []() { const char* e = getenv("CAIHIP_ATTN_SINGLE_BYTES"); return e ? atoi(e) : 65536; }();
+  if ((int64_t)max_ctx * head_dim * (dtype == CAI_KV_F16 ? 2 : dtype == CAI_KV_I8 ? 1 : 4) <= single_bytes) sl = (max_ctx + 31) / 32 * 32;
   kv->split_len = sl; kv->n_splits = (max_ctx + sl - 1) / sl;   // the merge stage holds up to 64 splits
   const size_t bytes = (size_t)kv->seq_elems() * n_seq * kv->elem();
   if (kv->n_splits > 64) return set_error(CAI_ERR_UNSUPPORTED, "kv cache: max_ctx %d needs %d splits (limit 64 x 256 rows)", max_ctx, kv->n_splits);
