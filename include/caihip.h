@@ -44,6 +44,7 @@ extern "C" {
 /* ---- pointer-space flags for compute calls ---- */
 #define CAI_X_DEVICE 1  /* input pointer is device memory (a producer's resident buffer; cf. pExternalVBs, neural/neuralopencl.pas:946) */
 #define CAI_Y_DEVICE 2  /* output pointer is device memory (no read-back; cf. ResultBuffer, neural/neuralopencl.pas:383-388) */
+#define CAI_MATRIX_CORES 4  /* cai_qgemm only: take the matrix-core kernels even for a matrix small enough that the dispatcher would keep it on the vector units */
 
 /* ---- KV cache element types ---- */
 #define CAI_KV_F32 0
@@ -116,7 +117,8 @@ int cai_qgemv(cai_qw_t w, const float* x, int n_b, float* y, int act, int flags)
 int cai_ffn_gateup(cai_qw_t gateup, const float* x, const float* gain, float eps, int n_b, float* y, int flags);
 /* Multi-token form on the matrix cores (prefill): x is [n_tokens][cols], y is [n_tokens][rows].
  * No counterpart in the reference, whose prefill is token-at-a-time
- * (neural/neuralchatengine.pas:1466-1470); results equal n_tokens GEMVs within bf16-input tolerance. */
+ * (neural/neuralchatengine.pas:1466-1470); results equal n_tokens GEMVs to about 1e-6 relative (exact integer weight
+ * operands, activations carried as two f16 = 22 significant bits).  flags: CAI_X_DEVICE | CAI_Y_DEVICE | CAI_MATRIX_CORES. */
 int cai_qgemm(cai_qw_t w, const float* x, int n_tokens, float* y, int flags);
 
 /* =====================================================================================

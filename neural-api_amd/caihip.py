@@ -8,7 +8,7 @@ from . import lib_path
 
 F32, F16, Q4_0, Q8_0, Q4_K, Q6_K, I8ROW = 0, 1, 2, 8, 12, 14, 100
 ACT_NONE, ACT_RELU, ACT_SIGMOID, ACT_TANH = 0, 1, 2, 3
-X_DEVICE, Y_DEVICE = 1, 2
+X_DEVICE, Y_DEVICE, MATRIX_CORES = 1, 2, 4
 KV_F32, KV_F16, KV_I8 = 0, 1, 2
 W_EMBED, W_HEAD, W_Q, W_K, W_V, W_O, W_GATEUP, W_DOWN, W_ROUTER = range(9)
 V_ATTN_NORM, V_MLP_NORM, V_FINAL_NORM, V_Q_NORM, V_K_NORM = range(5)
@@ -187,10 +187,10 @@ class QWeight:
         check(load().cai_ffn_gateup(self.h, _ptr(x), _ptr(g), eps, x.shape[0], _ptr(y), 0))
         return y
 
-    def gemm(self, x):
+    def gemm(self, x, matrix_cores=False):
         x = np.ascontiguousarray(x, np.float32).reshape(-1, self.cols)
         y = np.empty((x.shape[0], self.rows), np.float32)
-        check(load().cai_qgemm(self.h, _ptr(x), x.shape[0], _ptr(y), 0))
+        check(load().cai_qgemm(self.h, _ptr(x), x.shape[0], _ptr(y), MATRIX_CORES if matrix_cores else 0))
         return y
 
     def device_bytes(self):

@@ -365,7 +365,9 @@ int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const fl
                    float* y, int64_t y_stride, const float* residual)
 {
   int rc;
-  if (nb_supported(w) && (n_tok <= 16 || !gemm_mfma_supported(w))) return nb_linear(w, x, x_stride, gain, eps, n_tok, y, y_stride, residual);   // bandwidth-bound regime, or no prompt kernel for the type
+  // few tokens (the bandwidth-bound regime) of a Q4_K matrix, or a large matrix of a type without a prompt kernel (a small
+  // one stays in the cache: the single-launch VALU kernel per 8 tokens is cheaper than three launches)
+  if (nb_supported(w) && (gemm_mfma_supported(w) ? n_tok <= 16 : w->data_bytes >= ((int64_t)16 << 20))) return nb_linear(w, x, x_stride, gain, eps, n_tok, y, y_stride, residual);
   if (gemm_mfma_supported(w)) {
     if ((rc = prefill_prep(x, x_stride, gain, eps, (int)w->cols, n_tok))) return rc;
     return prefill_gemm(w, n_tok, y, y_stride, residual);
@@ -397,7 +399,9 @@ extern "C" int cai_qgemm(cai_qw_t w, const float* x, int n_tokens, float* y, int
     dx = (const float*)c.stage_in;
   }
   if (!(flags & CAI_Y_DEVICE)) { if ((rc = ensure_stage(&c.stage_out, &c.stage_out_cap, yb))) return rc; dy = (float*)c.stage_out; }
-  if ((rc = prefill_linear(w, dx, w->cols, nullptr, 0.0f, n_tokens, dy, w->rows, nullptr))) return rc;
+  if ((flags & CAI_MATRIX_CORES) && nb_supported(w) && !gemm_mfma_supported(w)) rc = nb_linear(w, dx, w->cols, nullptr, 0.0f, n_tokens, dy, w->rows, nullptr);
+  else rc = prefill_linear(w, dx, w->cols, nullptr, 0.0f, n_tokens, dy, w->rows, nullptr);
+  if (rc) return rc;
   CAI_HIP(hipGetLastError());
   if (!(flags & CAI_Y_DEVICE)) { CAI_HIP(hipMemcpyAsync(y, dy, yb, hipMemcpyDeviceToHost, c.stream)); CAI_HIP(hipStreamSynchronize(c.stream)); }
   return CAI_OK;

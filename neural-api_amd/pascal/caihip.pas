@@ -23,7 +23,7 @@ const
   CAI_F32 = 0; CAI_F16 = 1; CAI_Q4_0 = 2; CAI_Q8_0 = 8; CAI_Q4_K = 12; CAI_Q6_K = 14; CAI_I8ROW = 100;
   // fused activation opcodes = csAct* of the OpenCL kernels (neural/neural.cl:114-146)
   CAI_ACT_NONE = 0; CAI_ACT_RELU = 1; CAI_ACT_SIGMOID = 2; CAI_ACT_TANH = 3;
-  CAI_X_DEVICE = 1; CAI_Y_DEVICE = 2;
+  CAI_X_DEVICE = 1; CAI_Y_DEVICE = 2; CAI_MATRIX_CORES = 4;
   CAI_KV_F32 = 0; CAI_KV_F16 = 1; CAI_KV_I8 = 2;
   CAI_W_EMBED = 0; CAI_W_HEAD = 1; CAI_W_Q = 2; CAI_W_K = 3; CAI_W_V = 4; CAI_W_O = 5;
   CAI_W_GATEUP = 6; CAI_W_DOWN = 7; CAI_W_ROUTER = 8;

@@ -198,10 +198,11 @@ def test_small_batch_gemm_q8_0_q4_0_on_matrix_cores(qt, rows, cols, T):
     x[0, : cols // 2] = 0.0
     bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
     w = cai.QWeight(qt, rows, cols, raw, bias)
-    got = w.gemm(x)
+    got = w.gemm(x, matrix_cores=True)               # small matrices would otherwise stay on the vector-unit kernel
     want = O.gemv(qt, raw, rows, cols, x, bias, 0, 1)
     for t in range(T):
         assert rel_err(got[t], want[t], floor=0.02 * cols ** 0.5 * float(np.abs(x[t]).mean())) < TIGHT, t
+    assert rel_err(w.gemm(x), want, floor=0.02 * cols ** 0.5 * float(np.abs(x).mean())) < TIGHT   # the dispatcher's own choice
 
 
 @pytest.mark.parametrize("qt,rows,cols", [(O.Q8_0, 4101, 4096), (O.Q4_0, 8203, 4096), (O.Q4_K, 8203, 4096)])
