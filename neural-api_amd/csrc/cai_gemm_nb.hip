@@ -114,19 +114,37 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
   load_w(0, wa); load_w(1, wb);                  // weights do not depend on the staging below
 
   // ---- stage this slice of the activations: nS x 16 columns x 256 halfs, block sums, block scales ----
-  for (int idx = threadIdx.x; idx < nS * NB_SC * 32; idx += 256) {
-    const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC;
-    const int tok = col % NB_TK;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (tok < p.n_tok) v = *reinterpret_cast<const uint4*>(((col / NB_TK) ? p.xlo : p.xhi) + (int64_t)tok * K + (sb0 + s) * 256 + chunk * 8);
-    *reinterpret_cast<uint4*>(xs + (s * NB_SC + col) * NB_LDX + chunk * 8) = v;
-  }
-  for (int idx = threadIdx.x; idx < nS * NB_SC; idx += 256) {
-    const int col = idx % NB_SC, s = idx / NB_SC, tok = col % NB_TK;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (tok < p.n_tok) v = *reinterpret_cast<const uint4*>(((col / NB_TK) ? p.sxlo : p.sxhi) + (int64_t)tok * nb32 + (sb0 + s) * 8);
-    *reinterpret_cast<uint4*>(sxs + idx * 8) = v;
-    if (col < NB_TK) sinv_s[s * NB_TK + tok] = tok < p.n_tok ? p.sinvb[(int64_t)tok * nsb + sb0 + s] : 0.0f;
+  // All requests of a thread are issued before the first value is stored (four at a time for the big array): one memory
+  // round trip per four chunks instead of one per chunk.  Requests are unconditional (clamped token), absent tokens zeroed.
+  {
+    const int n_sx = nS * NB_SC;                   // small arrays: one thread per (super-block, column)
+    const bool sx_on = (int)threadIdx.x < n_sx;
+    const int sx_i = min((int)threadIdx.x, n_sx - 1), sx_col = sx_i % NB_SC, sx_s = sx_i / NB_SC, sx_tok = sx_col % NB_TK;
+    const int sx_tc = min(sx_tok, p.n_tok - 1);
+    const uint4 sxv = *reinterpret_cast<const uint4*>(((sx_col / NB_TK) ? p.sxlo : p.sxhi) + (int64_t)sx_tc * nb32 + (sb0 + sx_s) * 8);
+    const float siv = p.sinvb[(int64_t)sx_tc * nsb + sb0 + sx_s];
+    const int total = nS * NB_SC * 32;
+    for (int base = 0; base < total; base += 4 * 256) {
+      uint4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int idx = min(base + u * 256 + (int)threadIdx.x, total - 1);
+        const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC, tok = min(col % NB_TK, p.n_tok - 1);
+        v[u] = *reinterpret_cast<const uint4*>(((col / NB_TK) ? p.xlo : p.xhi) + (int64_t)tok * K + (sb0 + s) * 256 + chunk * 8);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int idx = base + u * 256 + (int)threadIdx.x;
+        if (idx < total) {
+          const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC;
+          *reinterpret_cast<uint4*>(xs + (s * NB_SC + col) * NB_LDX + chunk * 8) = (col % NB_TK) < p.n_tok ? v[u] : make_uint4(0, 0, 0, 0);
+        }
+      }
+    }
+    if (sx_on) {
+      *reinterpret_cast<uint4*>(sxs + sx_i * 8) = sx_tok < p.n_tok ? sxv : make_uint4(0, 0, 0, 0);
+      if (sx_col < NB_TK) sinv_s[sx_s * NB_TK + sx_tok] = sx_tok < p.n_tok ? siv : 0.0f;
+    }
   }
   __syncthreads();
 
@@ -326,16 +344,34 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
   load_w(0, w0); load_w(1, w1); load_w(2, w2); load_w(3, w3);   // weights do not depend on the staging below
 
   // ---- stage this slice of the activations: nS x 16 columns x 256 halfs (zero beyond the width), block scales ----
-  for (int idx = threadIdx.x; idx < nS * NB_SC * 32; idx += 256) {
-    const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC;
-    const int tok = col % NB_TK, k = (sb0 + s) * 256 + chunk * 8;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (tok < p.n_tok && (!TAIL || k < K)) v = *reinterpret_cast<const uint4*>(((col / NB_TK) ? p.xlo : p.xhi) + (int64_t)tok * K + k);
-    *reinterpret_cast<uint4*>(xs + (s * NB_SC + col) * NB_LDX + chunk * 8) = v;
-  }
-  for (int idx = threadIdx.x; idx < nS * NB_TK; idx += 256) {
-    const int tok = idx % NB_TK, s = idx / NB_TK;
-    sinv_s[idx] = tok < p.n_tok ? p.sinvb[(int64_t)tok * nsb + sb0 + s] : 0.0f;
+  // All requests of a thread are issued before the first value is stored (four at a time): one memory round trip per four
+  // chunks.  Requests are unconditional (clamped token and column), what is absent is zeroed on the way to LDS.
+  {
+    const int n_si = nS * NB_TK;
+    const int si_i = min((int)threadIdx.x, n_si - 1), si_tok = si_i % NB_TK, si_s = si_i / NB_TK;
+    const float siv = p.sinvb[(int64_t)min(si_tok, p.n_tok - 1) * nsb + sb0 + si_s];
+    const int total = nS * NB_SC * 32;
+    for (int base = 0; base < total; base += 4 * 256) {
+      uint4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int idx = min(base + u * 256 + (int)threadIdx.x, total - 1);
+        const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC, tok = min(col % NB_TK, p.n_tok - 1);
+        int k = (sb0 + s) * 256 + chunk * 8;
+        if (TAIL) k = min(k, K - 8);
+        v[u] = *reinterpret_cast<const uint4*>(((col / NB_TK) ? p.xlo : p.xhi) + (int64_t)tok * K + k);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int idx = base + u * 256 + (int)threadIdx.x;
+        if (idx < total) {
+          const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC;
+          const bool present = (col % NB_TK) < p.n_tok && (!TAIL || (sb0 + s) * 256 + chunk * 8 < K);
+          *reinterpret_cast<uint4*>(xs + (s * NB_SC + col) * NB_LDX + chunk * 8) = present ? v[u] : make_uint4(0, 0, 0, 0);
+        }
+      }
+    }
+    if ((int)threadIdx.x < n_si) sinv_s[si_i] = si_tok < p.n_tok ? siv : 0.0f;
   }
   __syncthreads();
 
