@@ -485,10 +485,25 @@ struct NbPrepParams {
   _Float16* hi; _Float16* lo; _Float16* sxhi; _Float16* sxlo; float* sinvb; float* ssq;
 };
 
+// Sums n values `stride` apart in index order; the requests go out eight at a time (the additions stay sequential, so the
+// result does not depend on the batching).
+__device__ __forceinline__ float nb_sum_strided(const float* p, int n, int64_t stride, float acc)
+{
+  int i = 0;
+  for (; i + 8 <= n; i += 8) {
+    float t[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) t[u] = p[(int64_t)(i + u) * stride];
+#pragma unroll
+    for (int u = 0; u < 8; u++) acc += t[u];
+  }
+  for (; i < n; i++) acc += p[(int64_t)i * stride];
+  return acc;
+}
+
 __device__ __forceinline__ float nb_inv_rms(const float* ssq, int nsb, int K, float eps, int tok)
 {
-  float t = 0.0f;
-  for (int i = 0; i < nsb; i++) t += ssq[(int64_t)tok * nsb + i];   // fixed order
+  const float t = nb_sum_strided(ssq + (int64_t)tok * nsb, nsb, 1, 0.0f);   // fixed order
   return 1.0f / sqrtf(t / (float)K + eps);
 }
 
@@ -505,14 +520,13 @@ __global__ __launch_bounds__(256) void nb_prep_kernel(const NbPrepParams p)
   else if (SRC == 1) {
     v = p.res[(int64_t)tok * p.res_stride + k];
     if (p.bias) v += p.bias[k];
-    for (int s = 0; s < p.n_slices; s++) v += p.part[((int64_t)s * p.n_tok + tok) * p.part_stride + k];
+    v = nb_sum_strided(p.part + (int64_t)tok * p.part_stride + k, p.n_slices, (int64_t)p.n_tok * p.part_stride, v);
     p.res[(int64_t)tok * p.res_stride + k] = v;
   } else {
-    float up = 0.0f, gate = 0.0f;
-    for (int s = 0; s < p.n_slices; s++) {
-      const float* row = p.part + ((int64_t)s * p.n_tok + tok) * p.part_stride;
-      up += row[k]; gate += row[p.half + k];
-    }
+    const float* col = p.part + (int64_t)tok * p.part_stride + k;
+    const float up0 = nb_sum_strided(col, p.n_slices, (int64_t)p.n_tok * p.part_stride, 0.0f);
+    const float gate0 = nb_sum_strided(col + p.half, p.n_slices, (int64_t)p.n_tok * p.part_stride, 0.0f);
+    float up = up0, gate = gate0;
     if (p.in_ssq) { const float inv = nb_inv_rms(p.in_ssq, p.in_nsb, p.in_K, p.in_eps, tok); up *= inv; gate *= inv; }
     if (p.bias) { up += p.bias[k]; gate += p.bias[p.half + k]; }
     v = silu_mul(up, gate);
@@ -563,8 +577,7 @@ __global__ __launch_bounds__(256) void nb_reduce_kernel(const NbReduceParams p)
   int sgi = 0;
   if (p.n_seg > 1 && c >= p.seg[1].y_off) sgi = 1;
   if (p.n_seg > 2 && c >= p.seg[2].y_off) sgi = 2;
-  float v = 0.0f;
-  for (int s = 0; s < p.n_slices; s++) v += p.part[((int64_t)s * p.n_tok + tok) * p.part_stride + c];
+  float v = nb_sum_strided(p.part + (int64_t)tok * p.part_stride + c, p.n_slices, (int64_t)p.n_tok * p.part_stride, 0.0f);
   if (p.in_ssq) v *= nb_inv_rms(p.in_ssq, p.in_nsb, p.in_K, p.in_eps, tok);
   if (p.seg[sgi].bias) v += p.seg[sgi].bias[c - p.seg[sgi].y_off];
   const int64_t o = (int64_t)tok * p.y_stride + c;
