@@ -489,8 +489,8 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
   if (p.qn_gain) {
     __shared__ float nred[8];
     float sq = 0.0f, sk = 0.0f;
-    for (int i = tid; i < qw; i += 256) sq = fmaf(row[i], row[i], sq);
-    for (int i = tid; i < kw; i += 256) sk = fmaf(row[qw + i], row[qw + i], sk);
+    for_strided8(row, tid, qw, 256, [&](float v, int) { sq = fmaf(v, v, sq); });
+    for_strided8(row + qw, tid, kw, 256, [&](float v, int) { sk = fmaf(v, v, sk); });
     sq = wave_sum(sq); sk = wave_sum(sk);
     if ((tid & 63) == 63) { nred[tid >> 6] = sq; nred[4 + (tid >> 6)] = sk; }
     __syncthreads();

@@ -96,7 +96,15 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
     for (int b = 0; b < NB; b++) {
       float ss = 0.0f;
       const float* xb = xin + (int64_t)b * cols;
-      for (int i = threadIdx.x; i < cols; i += 256) { const float v = xb[i]; ss = fmaf(v, v, ss); }
+      // eight requests go out before the first square is added (a request per turn would cost a cache round trip per 256
+      // columns); the additions keep their order
+      for (int i0 = threadIdx.x; i0 < cols; i0 += 8 * 256) {
+        float t[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) t[u] = xb[min(i0 + u * 256, cols - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; u++) if (i0 + u * 256 < cols) ss = fmaf(t[u], t[u], ss);
+      }
       ss = wave_sum(ss);
       if (lane == 63) red[b][wave] = ss;
     }
@@ -116,14 +124,26 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
     for (int b = 0; b < NB; b++) {
       const float4* src = reinterpret_cast<const float4*>(xin + (int64_t)b * cols + k0);
       float4* dst = xs4 + b * (p.kp_lds >> 2);
-      for (int n = threadIdx.x; n < n4; n += 256) {
-        float4 v = src[n];
-        if (p.norm_gain) {
-          const float4 g = reinterpret_cast<const float4*>(p.norm_gain + k0)[n];
-          v.x = g.x * (v.x * inv_rms[b]); v.y = g.y * (v.y * inv_rms[b]);
-          v.z = g.z * (v.z * inv_rms[b]); v.w = g.w * (v.w * inv_rms[b]);
+      for (int n0 = threadIdx.x; n0 < n4; n0 += 4 * 256) {     // four requests (and their gains) per turn, then the stores
+        float4 v[4], g[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          const int n = min(n0 + u * 256, n4 - 1);
+          v[u] = src[n];
+          if (p.norm_gain) g[u] = reinterpret_cast<const float4*>(p.norm_gain + k0)[n];
         }
-        dst[lds_slot<QT>(n)] = v;
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+          const int n = n0 + u * 256;
+          if (n < n4) {
+            float4 w = v[u];
+            if (p.norm_gain) {
+              w.x = g[u].x * (w.x * inv_rms[b]); w.y = g[u].y * (w.y * inv_rms[b]);
+              w.z = g[u].z * (w.z * inv_rms[b]); w.w = g[u].w * (w.w * inv_rms[b]);
+            }
+            dst[lds_slot<QT>(n)] = w;
+          }
+        }
       }
     }
     __syncthreads();

@@ -141,9 +141,13 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
         t = wave_sum(t);
         t = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, t), 63));
       } else {
-        for (int k = threadIdx.x; k < n8 * 2; k += nthr) {
-          const float4 v = src[k];
-          t = fmaf(v.x, v.x, t); t = fmaf(v.y, v.y, t); t = fmaf(v.z, v.z, t); t = fmaf(v.w, v.w, t);
+        for (int k0 = threadIdx.x; k0 < n8 * 2; k0 += 4 * nthr) {      // four requests per turn, squares added in index order
+          float4 v[4];
+#pragma unroll
+          for (int u = 0; u < 4; u++) v[u] = src[min(k0 + u * nthr, n8 * 2 - 1)];
+#pragma unroll
+          for (int u = 0; u < 4; u++)
+            if (k0 + u * nthr < n8 * 2) { t = fmaf(v[u].x, v[u].x, t); t = fmaf(v[u].y, v[u].y, t); t = fmaf(v[u].z, v[u].z, t); t = fmaf(v[u].w, v[u].w, t); }
         }
         t = wave_sum(t);
         if (lane == 63) s_ss[wave] = t;

@@ -58,6 +58,33 @@ __device__ __forceinline__ void split_f16(float x, _Float16& hi, _Float16& lo)
   hi = (_Float16)h; lo = (_Float16)(x - h);
 }
 
+// Walks x[i0], x[i0 + step], ... (< n, n >= 1) and hands every value to f(value, index) in index order.  Eight requests go out
+// before the first value is used: a loop that uses each value as it arrives pays one cache round trip per element, which is
+// what a 256-thread work-group reducing a few thousand activations otherwise spends most of its time on.  The second form
+// walks two arrays side by side (g may be null: its values are then 1).
+template <typename F>
+__device__ __forceinline__ void for_strided8(const float* x, int i0, int n, int step, F f)
+{
+  for (int i = i0; i < n; i += 8 * step) {
+    float t[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) t[u] = x[min(i + u * step, n - 1)];
+#pragma unroll
+    for (int u = 0; u < 8; u++) if (i + u * step < n) f(t[u], i + u * step);
+  }
+}
+template <typename F>
+__device__ __forceinline__ void for_strided8(const float* x, const float* g, int i0, int n, int step, F f)
+{
+  for (int i = i0; i < n; i += 8 * step) {
+    float t[8], tg[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) { const int j = min(i + u * step, n - 1); t[u] = x[j]; tg[u] = g ? g[j] : 1.0f; }
+#pragma unroll
+    for (int u = 0; u < 8; u++) if (i + u * step < n) f(t[u], tg[u], i + u * step);
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Resident weight matrix.  Device layouts (the on-disk block format stays the contract; these are
 // the library's own):

@@ -125,13 +125,13 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* x, const floa
   float* yr = y + (int64_t)blockIdx.x * y_stride;
   __shared__ float red[4];
   float ss = 0.0f;
-  for (int i = threadIdx.x; i < n; i += 256) ss = fmaf(xr[i], xr[i], ss);
+  for_strided8(xr, threadIdx.x, n, 256, [&](float v, int) { ss = fmaf(v, v, ss); });
   ss = wave_sum_all(ss);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
   __syncthreads();
   const float tot = (red[0] + red[1]) + (red[2] + red[3]);
   const float inv = 1.0f / sqrtf(tot / (float)n + eps);
-  for (int i = threadIdx.x; i < n; i += 256) yr[i] = gain[i] * (xr[i] * inv);
+  for_strided8(xr, gain, threadIdx.x, n, 256, [&](float v, float g, int i) { yr[i] = g * (v * inv); });
 }
 
 int launch_rmsnorm_strided(const float* x, const float* gain, int n, int n_tokens, float eps, float* y, int64_t x_stride, int64_t y_stride)
@@ -148,13 +148,13 @@ __global__ __launch_bounds__(256) void rmsnorm_pair_kernel(float* x, const float
   const int n = blockIdx.y ? n_b : n_a;
   __shared__ float red[4];
   float ss = 0.0f;
-  for (int i = threadIdx.x; i < n; i += 256) ss = fmaf(xr[i], xr[i], ss);
+  for_strided8(xr, threadIdx.x, n, 256, [&](float v, int) { ss = fmaf(v, v, ss); });
   ss = wave_sum_all(ss);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
   __syncthreads();
   const float tot = (red[0] + red[1]) + (red[2] + red[3]);
   const float inv = 1.0f / sqrtf(tot / (float)n + eps);
-  for (int i = threadIdx.x; i < n; i += 256) xr[i] = gain[i] * (xr[i] * inv);
+  for_strided8(xr, gain, threadIdx.x, n, 256, [&](float v, float g, int i) { xr[i] = g * (v * inv); });
 }
 
 int launch_rmsnorm_pair(float* x, const float* gain_a, int n_a, const float* gain_b, int n_b, int n_tokens, float eps, int64_t stride)

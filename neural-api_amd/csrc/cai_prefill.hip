@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void xprep_kernel(const float* x, int64_t x_st
   float inv = 1.0f;
   if (gain) {
     float ss = 0.0f;
-    for (int i = threadIdx.x; i < K; i += 256) ss = fmaf(xr[i], xr[i], ss);
+    for_strided8(xr, threadIdx.x, K, 256, [&](float v, int) { ss = fmaf(v, v, ss); });
     ss = wave_sum(ss);
     if (lane == 63) red[wave] = ss;
     __syncthreads();
@@ -43,11 +43,10 @@ __global__ __launch_bounds__(256) void xprep_kernel(const float* x, int64_t x_st
     __syncthreads();
   }
   float amax = 0.0f;
-  for (int i = threadIdx.x; i < K; i += 256) {
-    float v = xr[i];
-    if (gain) v = gain[i] * (v * inv);
+  for_strided8(xr, gain, threadIdx.x, K, 256, [&](float v, float g, int) {
+    if (gain) v = g * (v * inv);
     amax = fmaxf(amax, fabsf(v));
-  }
+  });
   for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
   if (lane == 0) red[wave] = amax;
   __syncthreads();
@@ -61,23 +60,20 @@ __global__ __launch_bounds__(256) void xprep_kernel(const float* x, int64_t x_st
   }
   __syncthreads();
   const float s = s_scale;
-  // one 32-block per half-wave pass: 8 blocks per work-group pass
-  const int hw = threadIdx.x >> 5, l32 = threadIdx.x & 31;
-  for (int b = hw; b < (K >> 5); b += 8) {
-    const int i = b * 32 + l32;
-    float v = xr[i];
-    if (gain) v = gain[i] * (v * inv);
+  // one 32-block per half-wave and turn (thread i of a turn takes element turn * 256 + i): 8 blocks per work-group turn
+  for_strided8(xr, gain, threadIdx.x, K, 256, [&](float v, float g, int i) {
+    if (gain) v = g * (v * inv);
     const float vs = v * s;
     _Float16 h, l; split_f16(vs, h, l);
     hi[(int64_t)t * K + i] = h; lo[(int64_t)t * K + i] = l;
     float sum = v;
     for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
-    if (l32 == 0) {   // the block sum in the scaled domain of hi/lo, divided by 32 so that it stays inside the half range
+    if ((i & 31) == 0) {   // the block sum in the scaled domain of hi/lo, divided by 32 so that it stays inside the half range
       const float ss = sum * s * 0.03125f;
       _Float16 sh, sl; split_f16(ss, sh, sl);
-      sxhi[(int64_t)t * (K >> 5) + b] = sh; sxlo[(int64_t)t * (K >> 5) + b] = sl;
+      sxhi[(int64_t)t * (K >> 5) + (i >> 5)] = sh; sxlo[(int64_t)t * (K >> 5) + (i >> 5)] = sl;
     }
-  }
+  });
 }
 
 struct GemmParams {
