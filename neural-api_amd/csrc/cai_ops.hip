@@ -215,8 +215,15 @@ __global__ void moe_combine_kernel(float* x, const float* part, const float* gat
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   float acc = 0.0f;
-  for (int j = 0; j < k; j++) acc = fmaf(gate[t * k + j], part[((int64_t)t * k + j) * n + i], acc);
-  x[(int64_t)t * n + i] += acc;
+  const float xv = x[(int64_t)t * n + i];
+  for (int j0 = 0; j0 < k; j0 += 8) {      // eight experts' values are requested together; the sum keeps the expert order
+    float pv[8], gv[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) { const int j = min(j0 + u, k - 1); pv[u] = part[((int64_t)t * k + j) * n + i]; gv[u] = gate[t * k + j]; }
+#pragma unroll
+    for (int u = 0; u < 8; u++) if (j0 + u < k) acc = fmaf(gv[u], pv[u], acc);
+  }
+  x[(int64_t)t * n + i] = xv + acc;
 }
 int launch_moe_combine(float* x, const float* part, const float* gate, int k, int n, int n_tokens)
 {
@@ -234,7 +241,7 @@ __global__ __launch_bounds__(256) void argmax_stage1(const float* x, int n, floa
   const float* xr = x + (int64_t)row * n;
   float best = 0.0f; int bi = -1;
   const int i0 = slice * 4096, i1 = min(n, i0 + 4096);
-  for (int i = i0 + threadIdx.x; i < i1; i += 256) { const float v = xr[i]; if (bi < 0 || v > best) { best = v; bi = i; } }
+  if (i0 < i1) for_strided8(xr + i0, threadIdx.x, i1 - i0, 256, [&](float v, int i) { if (bi < 0 || v > best) { best = v; bi = i0 + i; } });
   __shared__ float sv[256]; __shared__ int si[256];
   sv[threadIdx.x] = best; si[threadIdx.x] = bi;
   __syncthreads();

@@ -80,16 +80,17 @@ __global__ __launch_bounds__(SMP_T) void candidates_kernel(const SampleParams p)
 
   // ---- softmax (stable; the same clamps as the host row softmax) ----
   float mx = -3.0e38f;
-  for (int i = tid; i < n; i += SMP_T) mx = fmaxf(mx, p.logits[i]);
+  // (every pass over the row requests eight values per thread and turn before it uses the first: see for_strided8)
+  for_strided8(p.logits, tid, n, SMP_T, [&](float v, int) { mx = fmaxf(mx, v); });
   mx = smp_block_max(mx, redf);
   float sum = 0.0f;
-  for (int i = tid; i < n; i += SMP_T) {
-    const float a = fminf(fmaxf(p.logits[i] - mx, -4000.0f), 4000.0f);
+  for_strided8(p.logits, tid, n, SMP_T, [&](float v, int i) {
+    const float a = fminf(fmaxf(v - mx, -4000.0f), 4000.0f);
     const float e = expf(a);
     pr[i] = e; sum += e;
-  }
+  });
   sum = smp_block_sum(sum, redf);
-  if (sum > 0.0f) { const float inv = 1.0f / sum; for (int i = tid; i < n; i += SMP_T) pr[i] *= inv; }
+  if (sum > 0.0f) { const float inv = 1.0f / sum; for_strided8(pr, tid, n, SMP_T, [&](float v, int i) { pr[i] = v * inv; }); }
   __syncthreads();
 
   // ---- history penalty: p^r, * exp(-(f*count + presence)) on the distinct context tokens, renormalise ----
@@ -106,9 +107,9 @@ __global__ __launch_bounds__(SMP_T) void candidates_kernel(const SampleParams p)
     changed = __syncthreads_or(changed);
     if (changed) {
       float tot = 0.0f;
-      for (int i = tid; i < n; i += SMP_T) tot += pr[i];
+      for_strided8(pr, tid, n, SMP_T, [&](float v, int) { tot += v; });
       tot = smp_block_sum(tot, redf);
-      if (tot > 0.0f) for (int i = tid; i < n; i += SMP_T) pr[i] /= tot;
+      if (tot > 0.0f) for_strided8(pr, tid, n, SMP_T, [&](float v, int i) { pr[i] = v / tot; });
       __syncthreads();
     }
   }
@@ -117,19 +118,19 @@ __global__ __launch_bounds__(SMP_T) void candidates_kernel(const SampleParams p)
   if (p.temperature != 1.0f) {
     const float T = fmaxf(p.temperature, 1e-6f);
     float pm = 0.0f;
-    for (int i = tid; i < n; i += SMP_T) pm = fmaxf(pm, pr[i]);
+    for_strided8(pr, tid, n, SMP_T, [&](float v, int) { pm = fmaxf(pm, v); });
     pm = smp_block_max(pm, redf);
     if (pm > 0.0f) {
       const float lm = logf(fmaxf(pm, 1e-30f)), inv_t = 1.0f / T;
       float s2 = 0.0f;
-      for (int i = tid; i < n; i += SMP_T) {
-        const float v = expf(logf(fmaxf(pr[i], 1e-30f)) * inv_t - lm * inv_t);
+      for_strided8(pr, tid, n, SMP_T, [&](float q, int i) {
+        const float v = expf(logf(fmaxf(q, 1e-30f)) * inv_t - lm * inv_t);
         pr[i] = v; s2 += v;
-      }
+      });
       s2 = smp_block_sum(s2, redf);
       if (s2 <= 0.0f) s2 = 1.0f;
       const float inv = 1.0f / s2;
-      for (int i = tid; i < n; i += SMP_T) pr[i] *= inv;
+      for_strided8(pr, tid, n, SMP_T, [&](float v, int i) { pr[i] = v * inv; });
     }
     __syncthreads();
   }
@@ -143,10 +144,10 @@ __global__ __launch_bounds__(SMP_T) void candidates_kernel(const SampleParams p)
   for (int lvl = 0; lvl < 3; lvl++) {
     for (int b = tid; b < 4096; b += SMP_T) hist[b] = 0;
     __syncthreads();
-    for (int i = tid; i < n; i += SMP_T) {
-      const uint32_t u = __float_as_uint(pr[i]);
+    for_strided8(pr, tid, n, SMP_T, [&](float v, int) {
+      const uint32_t u = __float_as_uint(v);
       if ((u & prefix_mask) == prefix) atomicAdd(&hist[(u >> shifts[lvl]) & widths[lvl]], 1);
-    }
+    });
     __syncthreads();
     // thread t owns the four bins 4095-4t .. 4092-4t (top bins first), so a forward scan counts what lies above
     const int b0 = 4095 - 4 * tid;
@@ -171,20 +172,21 @@ __global__ __launch_bounds__(SMP_T) void candidates_kernel(const SampleParams p)
   // ---- survivors: everything above the threshold (any order), then `need` of the equal ones in token order ----
   if (tid == 0) n_gt = 0;
   __syncthreads();
-  for (int i = tid; i < n; i += SMP_T) {
-    const float v = pr[i];
+  for_strided8(pr, tid, n, SMP_T, [&](float v, int i) {
     if (__float_as_uint(v) > thr) { const int s = atomicAdd(&n_gt, 1); cp[s] = v; ct[s] = i; }
-  }
+  });
   __syncthreads();
   const int base = n_gt;                         // = m - need
   {
     const int chunk = (n + SMP_T - 1) / SMP_T, i0 = tid * chunk, i1 = min(n, i0 + chunk);
     int ties = 0;
-    for (int i = i0; i < i1; i++) ties += __float_as_uint(pr[i]) == thr;
+    if (i0 < i1) for_strided8(pr + i0, 0, i1 - i0, 1, [&](float v, int) { ties += __float_as_uint(v) == thr; });
     int total;
     int rank = smp_block_excl_scan(ties, redi, &total);
-    for (int i = i0; i < i1 && rank < need; i++)
-      if (__float_as_uint(pr[i]) == thr) { cp[base + rank] = pr[i]; ct[base + rank] = i; rank++; }
+    if (i0 < i1 && ties > 0 && rank < need)
+      for_strided8(pr + i0, 0, i1 - i0, 1, [&](float v, int i) {
+        if (rank < need && __float_as_uint(v) == thr) { cp[base + rank] = v; ct[base + rank] = i0 + i; rank++; }
+      });
   }
   __syncthreads();
 
