@@ -377,8 +377,18 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
   int wg_per_cu = W / waves_per_wg; if (wg_per_cu < 1) wg_per_cu = 1;
   { const int lds_fit = (int)((160 * 1024 - 4096) / (lds + 1024)); if (wg_per_cu > lds_fit) wg_per_cu = lds_fit < 1 ? 1 : lds_fit; }
   const int max_wgs = c.n_cu * wg_per_cu;
+  static const int r_env = []() { const char* e = getenv("CAIHIP_DOT_R"); return e ? atoi(e) : 0; }();
+  // Two rows per group halve the turns of a wave and double what it has in flight.  With long rows (three or more waves
+  // per row, every wave's lanes full) that only pays when the turns come out even - 7B down projection: 7 turns of one row
+  // beat 4 of two, 570 -> 580 tok/s; with one or two waves per row two rows measured better even at uneven turns (32B
+  // q|k|v and o: 136.9 against 134.1 tok/s).
   int R = 1;
-  if (!swiglu_half && total >= (int64_t)max_wgs * gwv * 4) R = 2;
+  if (!swiglu_half && total >= (int64_t)max_wgs * gwv * 4) {
+    const int64_t slots = (int64_t)max_wgs * gwv;
+    const int64_t turns1 = (total + slots - 1) / slots, turns2 = ((total + 1) / 2 + slots - 1) / slots;
+    if (nsw < 3 || 2 * turns2 <= turns1) R = 2;
+  }
+  if (!swiglu_half && (r_env == 1 || r_env == 2)) R = r_env;
   int cum = 0;
   for (int i = 0; i < m.n; i++) {
     const int64_t rows = swiglu_half ? swiglu_half : m.rows[i];
