@@ -114,7 +114,6 @@ struct AttnParams {
   int seq_mul;                 // 1: activation row s uses cache sequence seq0 + s; 0: all rows share sequence seq0 (prompt)
   int appended;                // 1: the K,V rows of this step are already in the cache (prompt ingestion)
   float* part_override;        // split partials buffer when more rows than cache sequences are in flight
-  int* counters;               // [seq][kv_head] arrival counters of the split merge (zero between launches)
   float* ksc; float* vsc;      // int8 caches: row scales [seq][layer][kv_head][max_ctx]
   int64_t seq_rows, layer_row_off;
   int evict_sinks, evict_cap;  // cap > 0: only the first `sinks` positions and the latest cap - sinks stay cached
@@ -989,7 +988,6 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
     if (kv->dtype == CAI_KV_F16) hipLaunchKernelGGL(kv_append_rows_kernel<__half>, dim3(n_seq), dim3(256), 0, c.stream, p);
     else hipLaunchKernelGGL(kv_append_rows_kernel<float>, dim3(n_seq), dim3(256), 0, c.stream, p);
   }
-  p.counters = kv->d_counters;
   // prompts over a 128-wide cache: matrix-core kernel, 32 tokens x 4 heads per work-group
   static const int flash_on = []() { const char* e = getenv("CAIHIP_PROMPT_FLASH"); return e ? atoi(e) : 1; }();
   if (prompt_rows && flash_on && kv->head_dim == 128 && kv->evict_cap == 0 && n_seq >= 8) {
@@ -1067,8 +1065,6 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   kv->part_q_heads = kv_heads * 8;
   CAI_HIP(hipMalloc(&kv->part, (size_t)n_seq * kv->part_q_heads * kv->n_splits * (head_dim + 2) * sizeof(float)));
   CAI_HIP(hipMalloc(&kv->d_len, sizeof(int32_t) * n_seq));
-  CAI_HIP(hipMalloc(&kv->d_counters, sizeof(int) * n_seq * kv_heads));
-  CAI_HIP(hipMemsetAsync(kv->d_counters, 0, sizeof(int) * n_seq * kv_heads, ctx().stream));
   CAI_HIP(hipStreamSynchronize(ctx().stream));
   return CAI_OK;
 }
@@ -1085,8 +1081,6 @@ void kv_free(cai_kv_s* kv)
   kv->pq_hi = kv->pq_lo = nullptr; kv->pq_cap = 0;
   if (kv->part) (void)hipFree(kv->part);
   if (kv->d_len) (void)hipFree(kv->d_len);
-  if (kv->d_counters) (void)hipFree(kv->d_counters);
-  kv->d_counters = nullptr;
   kv->k = kv->v = nullptr; kv->part = nullptr; kv->d_len = nullptr;
 }
 

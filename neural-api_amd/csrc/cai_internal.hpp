@@ -116,7 +116,6 @@ struct cai_kv_s {
   float* part = nullptr;                  // [seq][q_head][split][head_dim+2] split-K partials
   int part_q_heads = 0;
   int32_t* d_len = nullptr;               // [seq] device scratch: rows live BEFORE the token being decoded
-  int* d_counters = nullptr;              // [seq][kv_head] split-merge arrival counters
   void* pq_hi = nullptr; void* pq_lo = nullptr; size_t pq_cap = 0;   // prompt ingestion: rotated q of a chunk as two f16 planes
   size_t elem() const { return dtype == CAI_KV_F16 ? 2 : dtype == CAI_KV_I8 ? 1 : 4; }
   int64_t layer_rows() const { return (int64_t)kv_heads * max_ctx; }
