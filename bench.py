@@ -131,7 +131,7 @@ def gemv_sweep(cai, synth, torch, with_cpu):
 # HBM bytes per launch of the 7B-shape gate|up kernel from hardware counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000
 # KiB, factors from a 1 GiB copy kernel): profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt.  Not measurable from
 # inside this process; re-collect when the kernel changes.
-GATEUP_TRAFFIC_BYTES = int((37519.7 * 2.000 + 74.7 * 1.000) * 1024)
+GATEUP_TRAFFIC_BYTES = int((37522.5 * 2.000 + 74.2 * 1.000) * 1024)
 
 
 def main():

@@ -405,7 +405,7 @@ __global__ __launch_bounds__(128) void attn_merge_kernel(const AttnParams p)
   const int n_active = s_last - s_first + 1;
   if (n_active == 1) return;                       // the split kernel already wrote the final row
   const float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + s_first) * (hd + 2);
-  __shared__ float mM[64], mL[64];
+  __shared__ float mM[128], mL[128];
   for (int s = threadIdx.x; s < n_active; s += blockDim.x) { mM[s] = pt[(int64_t)s * (hd + 2) + hd]; mL[s] = pt[(int64_t)s * (hd + 2) + hd + 1]; }
   for (int d = threadIdx.x; d < hd; d += blockDim.x) {
     float A = 0.0f, L = 0.0f, M = -1e30f;
@@ -1048,9 +1048,9 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   // the merge launch disappears (small models at short contexts are bound by launches, not by bytes)
   static const int single_bytes = []() { const char* e = getenv("CAIHIP_ATTN_SINGLE_BYTES"); return e ? atoi(e) : 65536; }();
   if ((int64_t)max_ctx * head_dim * (dtype == CAI_KV_F16 ? 2 : dtype == CAI_KV_I8 ? 1 : 4) <= single_bytes) sl = (max_ctx + 31) / 32 * 32;
-  kv->split_len = sl; kv->n_splits = (max_ctx + sl - 1) / sl;   // the merge stage holds up to 64 splits
+  kv->split_len = sl; kv->n_splits = (max_ctx + sl - 1) / sl;   // the merge stage holds up to 128 splits
   const size_t bytes = (size_t)kv->seq_elems() * n_seq * kv->elem();
-  if (kv->n_splits > 64) return set_error(CAI_ERR_UNSUPPORTED, "kv cache: max_ctx %d needs %d splits (limit 64 x 256 rows)", max_ctx, kv->n_splits);
+  if (kv->n_splits > 128) return set_error(CAI_ERR_UNSUPPORTED, "kv cache: max_ctx %d needs %d splits (limit 128 x 256 rows)", max_ctx, kv->n_splits);
   CAI_HIP(hipMalloc(&kv->k, bytes));
   CAI_HIP(hipMalloc(&kv->v, bytes));
   CAI_HIP(hipMemsetAsync(kv->k, 0, bytes, ctx().stream));
