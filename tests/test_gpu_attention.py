@@ -310,3 +310,34 @@ def test_grouped_decode_attention_fp16_int8(hq, hkv, ctx, kv):
             k, v, s_k, s_v = cache.export_layer(0)
             np.testing.assert_array_equal(k, kq); np.testing.assert_array_equal(v, vq)
             np.testing.assert_array_equal(s_k, ks); np.testing.assert_array_equal(s_v, vs)
+
+
+@pytest.mark.parametrize("hq,hkv", [(8, 2), (16, 8)])
+def test_context_beyond_64_slices(hq, hkv):
+    """20k cached rows = 80 slices of 256: more than the 64 the merge stage once held (per-head kernel for 2 KV heads, the
+    per-KV-head kernel for 8).  The cache is filled through the layer import; two decode steps against a float64 soft-max."""
+    from helpers.device import dev
+    cai = dev()
+    rng = np.random.default_rng(hq)
+    dk, n, ctx = 128, 20000, 20480
+    k = rng.standard_normal((hkv, n, dk)).astype(np.float16); v = rng.standard_normal((hkv, n, dk)).astype(np.float16)
+    cache = cai.KVCache(1, hkv, dk, ctx, cai.KV_F16)
+    cache.import_layer(0, k, v)
+    assert cache.len(0) == n
+    kk = [k[h].astype(np.float64) for h in range(hkv)]; vv = [v[h].astype(np.float64) for h in range(hkv)]
+    G = hq // hkv
+    for step in range(2):
+        row = rng.standard_normal((hq + 2 * hkv) * dk).astype(np.float32)
+        got = cache.attn_decode(0, row, hq)
+        q = row[: hq * dk].reshape(hq, dk).astype(np.float64)
+        kn = row[hq * dk: (hq + hkv) * dk].reshape(hkv, dk).astype(np.float16).astype(np.float64)
+        vn = row[(hq + hkv) * dk:].reshape(hkv, dk).astype(np.float16).astype(np.float64)
+        for h in range(hkv):
+            kk[h] = np.vstack([kk[h], kn[h]]); vv[h] = np.vstack([vv[h], vn[h]])
+        want = np.zeros((hq, dk))
+        for qh in range(hq):
+            s = kk[qh // G] @ q[qh] / np.sqrt(dk)
+            w = np.exp(s - s.max()); w /= w.sum()
+            want[qh] = w @ vv[qh // G]
+        assert np.max(np.abs(got.reshape(hq, dk) - want)) < 1e-5, step
+    assert cache.len(0) == n + 2
