@@ -399,7 +399,9 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
   const dim3 block(64 * waves_per_wg);
   auto go = [&](auto kern) {
     static std::set<const void*> raised;   // kernels whose dynamic-LDS limit has been raised
-    if (raised.insert((const void*)kern).second) (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 2048);
+    // (a failing attribute call would leave a sticky error that a later hipGetLastError reports against an innocent launch)
+    if (raised.insert((const void*)kern).second && hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 2048) != hipSuccess)
+      (void)hipGetLastError();
     hipLaunchKernelGGL(kern, dim3(grid), block, lds, st, p, cum, nsw, gwv);
   };
   auto pick = [&](auto ns) {
