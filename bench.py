@@ -77,7 +77,7 @@ def gemv_sweep(cai, synth, torch, with_cpu):
     rotating over enough copies of the matrix to exceed the 256 MB infinity cache (at most 24 copies: the small shapes stay
     cache-resident and are labelled so)."""
     lib = cai.load()
-    QT = {"Q8_0": (cai.Q8_0, 34 / 32), "Q4_0": (cai.Q4_0, 18 / 32), "Q4_K": (cai.Q4_K, 144 / 256)}
+    QT = {"Q8_0": (cai.Q8_0, 34 / 32), "Q4_0": (cai.Q4_0, 18 / 32), "Q4_K": (cai.Q4_K, 144 / 256), "I8ROW": (cai.I8ROW, 1.0)}   # I8ROW: the reference's own per-row int8 format
     shapes = [(2048, 2048), (5632, 2048), (2048, 5632), (18944, 3584), (152064, 3584)]
     gen = torch.Generator(device="cuda"); gen.manual_seed(424242)
     cpu = None
@@ -90,7 +90,7 @@ def gemv_sweep(cai, synth, torch, with_cpu):
         for rows, cols in shapes:
             mat_bytes = rows * cols * bpw
             copies = int(max(1, min(24, -(-320e6 // mat_bytes))))
-            ws = [synth.random_qweight(qt, rows, cols, gen)[0] for _ in range(copies)]
+            ws = [synth.random_int8_rows(rows, cols, gen) if name == "I8ROW" else synth.random_qweight(qt, rows, cols, gen)[0] for _ in range(copies)]
             for nb in (1, 4):
                 x = torch.randn(nb, cols, device="cuda"); y = torch.empty(nb, rows, device="cuda")
                 torch.cuda.synchronize()
@@ -107,7 +107,7 @@ def gemv_sweep(cai, synth, torch, with_cpu):
                 line = {"gemv": name, "rows": rows, "cols": cols, "batch": nb, "us_per_launch": round(us, 2),
                         "algorithmic_bytes": int(algo), "GB_per_s": round(algo / us / 1e3, 1), "frac_of_8TBps": round(algo / us / 1e3 / HBM_PEAK_GBS, 4),
                         "working_set": "hbm" if copies * mat_bytes > 300e6 else "cache-resident (%d x %.1f MB)" % (copies, mat_bytes / 1e6)}
-                if cpu is not None and nb == 1 and name == "Q8_0":
+                if cpu is not None and nb == 1 and name == "I8ROW":
                     # restated reference AVX2 int8-per-row kernel on the same shape (1 B/weight), all host threads
                     import numpy as np
                     thr = min(cpu.cpu_max_threads(), 16)
@@ -144,7 +144,7 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=5)
     ap.add_argument("--kv", choices=["f32", "f16", "i8"], default=None, help="KV cache element type (default: the configuration's own)")
     ap.add_argument("--batch", type=int, default=1, help="independent sequences decoded together (1..8)")
-    ap.add_argument("--gemv-sweep", action="store_true", help="isolated matrix-vector sweep (BASELINE configs[1]): Q8_0 / Q4_0 / Q4_K, five shapes, batch 1 and 4")
+    ap.add_argument("--gemv-sweep", action="store_true", help="isolated matrix-vector sweep (BASELINE configs[1]): Q8_0 / Q4_0 / Q4_K and per-row int8, five shapes, batch 1 and 4")
     ap.add_argument("--copy-calibration", action="store_true", help="only run the 1 GiB device copy kernel 5 times (reference for traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -159,9 +159,11 @@ class QWeight:
         if bias is not None:
             bias = np.ascontiguousarray(bias, np.float32)
         if qtype == I8ROW:
-            codes = np.ascontiguousarray(blocks).view(np.int8)
-            scales = np.ascontiguousarray(scales, np.float32)
-            check(load().cai_qw_create_int8row(rows, cols, _ptr(codes), _ptr(scales), _ptr(bias), C.byref(h)))
+            if not isinstance(blocks, int):            # (an int is a pointer, host or device: taken as it is)
+                blocks = np.ascontiguousarray(blocks).view(np.int8)
+            if not isinstance(scales, int):
+                scales = np.ascontiguousarray(scales, np.float32)
+            check(load().cai_qw_create_int8row(rows, cols, _ptr(blocks), _ptr(scales), _ptr(bias), C.byref(h)))
         else:
             if not isinstance(blocks, int):
                 blocks = np.ascontiguousarray(blocks)

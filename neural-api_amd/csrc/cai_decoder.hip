@@ -86,7 +86,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
   auto mma_layer = [&](const cai_decoder_s::Layer& L) {
     if (n_b < 2 || c.n_experts > 0) return false;
     const int slots[6] = {CAI_W_Q, CAI_W_K, CAI_W_V, CAI_W_O, CAI_W_GATEUP, CAI_W_DOWN};
-    for (int sl : slots) if (!nb_supported(L.w[sl])) return false;
+    for (int sl : slots) if (!nb_supported(L.w[sl]) || L.w[sl]->qtype == CAI_I8ROW) return false;   // (per-row int8 products need the plain reduction for their row scale)
     return L.w[CAI_W_Q]->qtype == L.w[CAI_W_K]->qtype && L.w[CAI_W_Q]->qtype == L.w[CAI_W_V]->qtype;   // q | k | v share one launch
   };
   for (int l = 0; l < c.n_layers; l++) {

@@ -30,7 +30,7 @@ constexpr int NB_SC = 16;        // staged columns: 8 tokens x {hi, lo}
 constexpr int NB_TK = 8;         // tokens per pass
 constexpr int NB_SMAX = 5;       // super-blocks per K slice at most (LDS: 8.6 KB each, and three work-groups share a CU)
 
-struct NbSeg { const uint8_t* w; const uint8_t* aux; const float* bias; int rows; int y_off; int tile_end; };   // aux: block scales plane (Q8_0 / Q4_0); tile_end: cumulative 32-row tiles
+struct NbSeg { const uint8_t* w; const uint8_t* aux; const float* bias; const float* row_scale; int rows; int y_off; int tile_end; };   // aux: block scales plane (Q8_0 / Q4_0); row_scale: per-row int8 matrices; tile_end: cumulative 32-row tiles
 
 struct NbParams {
   NbSeg seg[3]; int n_seg;                      // up to three matrices of equal width share one launch (q | k | v)
@@ -258,7 +258,7 @@ struct __attribute__((aligned(4))) Dwords4 { uint32_t x, y, z, w; };   // scale 
 template <int QT> __device__ __forceinline__ half8_t codes_to_half8(uint32_t w0, uint32_t w1)
 {
   uint32_t a, b; _Float16 off;
-  if (QT == CAI_Q8_0) { a = w0 ^ 0x80808080u; b = w1 ^ 0x80808080u; off = (_Float16)(-1152.0f); }   // byte + 128, then 1024 + .. - 1152
+  if (QT == CAI_Q8_0 || QT == CAI_I8ROW) { a = w0 ^ 0x80808080u; b = w1 ^ 0x80808080u; off = (_Float16)(-1152.0f); }   // byte + 128, then 1024 + .. - 1152
   else { a = w0 & 0x0f0f0f0fu; b = (w0 >> 4) & 0x0f0f0f0fu; off = (_Float16)(-1032.0f); }           // elements e and 16 + e of the block
   const half2_t o2 = {off, off};
   const half2_t h0 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, a, 0x04010400u)) + o2;
@@ -291,12 +291,12 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
   const int n = lane & 15, kg = lane >> 4;
   const int K = p.cols, nsb = (K + 255) >> 8, nb32 = K >> 5;
   const int slice = blockIdx.y, sb0 = slice * S, nS = min(S, nsb - sb0);
-  const int row_bytes = QT == CAI_Q8_0 ? K : (K >> 1);
+  const int row_bytes = QT != CAI_Q4_0 ? K : (K >> 1);
   const int aux_row_bytes = nb32 * 2;
   const int tile0 = blockIdx.x * 4 + wave;
   const int n_it = tile0 < p.n_tiles ? (p.n_tiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
   // an item = 32 rows x 128 bytes of quants: 4 blocks of Q8_0 (half a group) or 8 blocks of Q4_0 (a whole group)
-  constexpr int IB = QT == CAI_Q8_0 ? 4 : 8;     // blocks per item
+  constexpr int IB = QT != CAI_Q4_0 ? 4 : 8;     // blocks per item
   constexpr int IPG = 8 / IB;                    // items per group
   const int nI = nS * IPG;                       // items per tile
   const int nq = n_it * nI;
@@ -320,7 +320,8 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
       const int64_t row = min(R0 + 16 * hh + n, sg->rows - 1);                  // tail rows: re-read the last row
       const uint8_t* qrow = sg->w + row * row_bytes;
       const uint8_t* arow = sg->aux + row * aux_row_bytes;
-      if (!TAIL) {
+      if (QT == CAI_I8ROW) { r.d[hh][0] = 0x3C003C00u; r.d[hh][IB / 2 - 1] = 0x3C003C00u; }   // per-row int8: every block scale is 1
+      else if (!TAIL) {
         if (QT == CAI_Q8_0) { const uint2 t = *reinterpret_cast<const uint2*>(arow + g0 * 2); r.d[hh][0] = t.x; r.d[hh][IB / 2 - 1] = t.y; }
         else { const uint4 t = *reinterpret_cast<const uint4*>(arow + g0 * 2); r.d[hh][0] = t.x; r.d[hh][1] = t.y; r.d[hh][IB / 2 - 2] = t.z; r.d[hh][IB / 2 - 1] = t.w; }
       } else {                                                                    // the row may end inside the item: absent blocks get scale 0
@@ -334,7 +335,7 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
       }
 #pragma unroll
       for (int j = 0; j < 2; j++) {
-        int off = g0 * (QT == CAI_Q8_0 ? 32 : 16) + 64 * j + 16 * kg;
+        int off = g0 * (QT != CAI_Q4_0 ? 32 : 16) + 64 * j + 16 * kg;
         if (TAIL) off = max(0, min(off, row_bytes - 16));                         // stays inside the row; such codes meet scale 0
         r.q[hh][j] = *reinterpret_cast<const uint4*>(qrow + off);
       }
@@ -376,7 +377,7 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
   __syncthreads();
 
   float acc[2][4], g[2][4];
-  const int xoff = QT == CAI_Q8_0 ? 16 * (kg & 1) + 8 * (kg >> 1) : 4 * kg;   // this lane's first weight within a block
+  const int xoff = QT != CAI_Q4_0 ? 16 * (kg & 1) + 8 * (kg >> 1) : 4 * kg;   // this lane's first weight within a block
   auto compute = [&](const WRegs& r, int q) {
     const int it = q % nI, s = it / IPG, part = it % IPG;
     if (it == 0) {
@@ -395,7 +396,7 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
     const float4_t z4 = {0.0f, 0.0f, 0.0f, 0.0f};
     auto block = [&](int hh, int b, uint32_t c0, uint32_t c1) {
       half8_t X;
-      if (QT == CAI_Q8_0) X = *reinterpret_cast<const half8_t*>(xcol + 32 * b);
+      if (QT != CAI_Q4_0) X = *reinterpret_cast<const half8_t*>(xcol + 32 * b);
       else {
         const half4_t x0 = *reinterpret_cast<const half4_t*>(xcol + 32 * b);
         const half4_t x1 = *reinterpret_cast<const half4_t*>(xcol + 32 * b + 16);
@@ -413,7 +414,7 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
 #pragma unroll
       for (int hh = 0; hh < 2; hh++) {
         const uint4 v = r.q[hh][j];
-        if (QT == CAI_Q8_0) {
+        if (QT != CAI_Q4_0) {
           const uint2_t s0 = __builtin_amdgcn_permlane32_swap(v.x, v.z, false, false);   // .x: even block, .y: odd block
           const uint2_t s1 = __builtin_amdgcn_permlane32_swap(v.y, v.w, false, false);
           block(hh, 2 * j, s0.x, s1.x);
@@ -579,6 +580,7 @@ __global__ __launch_bounds__(256) void nb_reduce_kernel(const NbReduceParams p)
   if (p.n_seg > 2 && c >= p.seg[2].y_off) sgi = 2;
   float v = nb_sum_strided(p.part + (int64_t)tok * p.part_stride + c, p.n_slices, (int64_t)p.n_tok * p.part_stride, 0.0f);
   if (p.in_ssq) v *= nb_inv_rms(p.in_ssq, p.in_nsb, p.in_K, p.in_eps, tok);
+  if (p.seg[sgi].row_scale) v *= p.seg[sgi].row_scale[c - p.seg[sgi].y_off];   // per-row int8: (sum code * x) * scale, then bias
   if (p.seg[sgi].bias) v += p.seg[sgi].bias[c - p.seg[sgi].y_off];
   const int64_t o = (int64_t)tok * p.y_stride + c;
   if (p.residual) v += p.residual[o];
@@ -682,7 +684,7 @@ int nb_prep_plain(const float* x, int64_t x_stride, const float* gain, float eps
 // res <- res + last product (+bias); planes <- res (norm as above).  The product must not itself carry a pending norm.
 int nb_prep_residual(float* res, int64_t res_stride, const float* gain, float eps, int K, int n_tok)
 {
-  if (g_prod.n_seg != 1 || g_prod.width != K || g_prod.n_tok != n_tok || g_prod.in_ssq)
+  if (g_prod.n_seg != 1 || g_prod.width != K || g_prod.n_tok != n_tok || g_prod.in_ssq || g_prod.seg[0].row_scale)
     return set_error(CAI_ERR_STATE, "small-batch residual pre-pass: no matching product in flight");
   NbPrepParams p{}; p.res = res; p.res_stride = res_stride; p.part = g_nb.part; p.part_stride = g_prod.part_stride; p.n_slices = g_prod.n_slices; p.n_tok = n_tok;
   p.bias = g_prod.seg[0].bias; p.gain = gain; p.K = K;
@@ -694,7 +696,7 @@ int nb_prep_residual(float* res, int64_t res_stride, const float* gain, float ep
 // planes <- SwiGLU of the last product (rows [0, half) up, [half, 2 half) gate)
 int nb_prep_swiglu(int half, int n_tok)
 {
-  if (g_prod.n_seg != 1 || g_prod.width != 2 * half || g_prod.n_tok != n_tok) return set_error(CAI_ERR_STATE, "small-batch SwiGLU pre-pass: no matching product in flight");
+  if (g_prod.n_seg != 1 || g_prod.width != 2 * half || g_prod.n_tok != n_tok || g_prod.seg[0].row_scale) return set_error(CAI_ERR_STATE, "small-batch SwiGLU pre-pass: no matching product in flight");
   NbPrepParams p{}; p.part = g_nb.part; p.part_stride = g_prod.part_stride; p.n_slices = g_prod.n_slices; p.n_tok = n_tok;
   p.bias = g_prod.seg[0].bias; p.half = half; p.in_ssq = g_prod.in_ssq; p.in_nsb = g_prod.in_nsb; p.in_K = g_prod.in_K; p.in_eps = g_prod.in_eps; p.K = half;
   const int rc = nb_prep_launch(2, p, n_tok); if (rc) return rc;
@@ -707,7 +709,7 @@ int nb_prep_swiglu(int half, int n_tok)
 bool nb_supported(const cai_qw_s* w)
 {
   if (w->qtype == CAI_Q4_K) return w->cols % 256 == 0;
-  return (w->qtype == CAI_Q8_0 || w->qtype == CAI_Q4_0) && w->cols % 32 == 0 && w->cols >= 32;
+  return (w->qtype == CAI_Q8_0 || w->qtype == CAI_Q4_0 || w->qtype == CAI_I8ROW) && w->cols % 32 == 0 && w->cols >= 32;   // per-row int8: unit block scales, the row scale is applied by nb_reduce
 }
 
 template <void (*Kernel)(const NbParams)>
@@ -730,7 +732,7 @@ int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok)
     if (!nb_supported(ws[i]) || ws[i]->qtype != qt || ws[i]->cols != ws[0]->cols)
       return set_error(CAI_ERR_UNSUPPORTED, "small-batch gemm: matrix %d type %d width %lld", i, ws[i]->qtype, (long long)ws[i]->cols);
     tiles += (int)((ws[i]->rows + 31) / 32);
-    p.seg[i].w = ws[i]->data; p.seg[i].aux = ws[i]->aux; p.seg[i].bias = ws[i]->bias; p.seg[i].rows = (int)ws[i]->rows; p.seg[i].y_off = y_off[i]; p.seg[i].tile_end = tiles;
+    p.seg[i].w = ws[i]->data; p.seg[i].aux = ws[i]->aux; p.seg[i].bias = ws[i]->bias; p.seg[i].row_scale = qt == CAI_I8ROW ? reinterpret_cast<const float*>(ws[i]->aux) : nullptr; p.seg[i].rows = (int)ws[i]->rows; p.seg[i].y_off = y_off[i]; p.seg[i].tile_end = tiles;
     width = std::max(width, y_off[i] + (int)ws[i]->rows);
   }
   p.n_tiles = tiles;
@@ -748,6 +750,7 @@ int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok)
     const size_t lds = (size_t)S * NB_SC * NB_LDX * 2 + (size_t)S * NB_TK * 4;
     const bool tail = p.cols % 256 != 0;
     if (qt == CAI_Q8_0) { if (tail) nb_launch<gemm_blk_nb<CAI_Q8_0, true>>(p, gx, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_Q8_0, false>>(p, gx, n_slices, lds); }
+    else if (qt == CAI_I8ROW) { if (tail) nb_launch<gemm_blk_nb<CAI_I8ROW, true>>(p, gx, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_I8ROW, false>>(p, gx, n_slices, lds); }
     else { if (tail) nb_launch<gemm_blk_nb<CAI_Q4_0, true>>(p, gx, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_Q4_0, false>>(p, gx, n_slices, lds); }
   }
   for (int i = 0; i < 3; i++) g_prod.seg[i] = p.seg[i];

@@ -18,6 +18,7 @@ template <int QT> struct QTraits;
 template <> struct QTraits<CAI_Q4_K> { static constexpr int UW = 32, T = 8; };  // weights per unit, float4 per unit
 template <> struct QTraits<CAI_Q4_0> { static constexpr int UW = 32, T = 8; };
 template <> struct QTraits<CAI_Q8_0> { static constexpr int UW = 16, T = 4; };
+template <> struct QTraits<CAI_I8ROW> { static constexpr int UW = 16, T = 4; };   // per-row int8: the Q8_0 walk with one scale per row, applied at the end
 
 // original float4 index n (within the panel) -> LDS float4 slot, unit-transposed in tiles of 16 units
 template <int QT> __device__ __forceinline__ int lds_slot(int n)
@@ -40,7 +41,7 @@ template <int QT> __device__ __forceinline__ int lds_unit_base(int u)
 }
 
 // ------------------------------------------------------------------------------------------
-// Fast kernel: Q4_K / Q4_0 / Q8_0.  MODE 0: plain rows.  MODE 1: SwiGLU pairs (row i and row half+i).
+// Fast kernel: Q4_K / Q4_0 / Q8_0 / per-row int8.  MODE 0: plain rows.  MODE 1: SwiGLU pairs (row i and row half+i).
 // ------------------------------------------------------------------------------------------
 template <int QT, int NB, int R, int MODE>
 __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
@@ -69,6 +70,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
   int64_t row_bytes, aux_row_bytes = 0;
   if (QT == CAI_Q4_K) row_bytes = (int64_t)(cols >> 8) * 144;
   else if (QT == CAI_Q4_0) { row_bytes = cols >> 1; aux_row_bytes = (cols >> 5) * 2; }
+  else if (QT == CAI_I8ROW) row_bytes = cols;
   else { row_bytes = cols; aux_row_bytes = (cols >> 5) * 2; }
 
   const uint8_t* rp[RR]; const uint8_t* ap[RR]; bool live[RR];
@@ -172,7 +174,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
 #pragma unroll
         for (int r = 0; r < RR; r++) {
           q[r] = *reinterpret_cast<const uint4*>(rp[r] + (int64_t)un * 16);
-          dh[r] = *reinterpret_cast<const uint16_t*>(ap[r] + (un >> 1) * 2);
+          dh[r] = QT == CAI_I8ROW ? (uint16_t)0x3C00 : *reinterpret_cast<const uint16_t*>(ap[r] + (un >> 1) * 2);   // per-row int8: block scale 1
         }
       }
       const int xb0 = lds_unit_base<QT>(u);
@@ -250,7 +252,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
 #pragma unroll
         for (int r = 0; r < RR; r++) {
           const uint32_t qw[4] = {q[r].x, q[r].y, q[r].z, q[r].w};
-          if (QT == CAI_Q8_0) {
+          if (QT == CAI_Q8_0 || QT == CAI_I8ROW) {
 #pragma unroll
             for (int w = 0; w < 4; w++) {
               wf[r][4 * w] = (float)(int8_t)(qw[w] & 0xff); wf[r][4 * w + 1] = (float)(int8_t)((qw[w] >> 8) & 0xff);
@@ -281,7 +283,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
             const float4 v = xb[xb0 + t * 16];
             xv[4 * t] = v.x; xv[4 * t + 1] = v.y; xv[4 * t + 2] = v.z; xv[4 * t + 3] = v.w;
           }
-          if (QT == CAI_Q8_0) {
+          if (QT == CAI_Q8_0 || QT == CAI_I8ROW) {
 #pragma unroll
             for (int r = 0; r < RR; r++) {
               float sq = 0.0f;
@@ -332,6 +334,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
 #pragma unroll
         for (int b = 0; b < NB; b++) {
           float v = acc[r][b];
+          if (QT == CAI_I8ROW) v *= reinterpret_cast<const float*>(sg.aux)[bank_row + row];   // (sum code * x) * scale, then bias (neural/neuralvolume.pas:12693-12745)
           if (sg.bias) v += sg.bias[bank_row + row];
           v = act_apply(v, p.act);
           const int64_t o = (int64_t)b * p.y_stride + sg.y_off + row;
@@ -578,6 +581,11 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
     if (qt == CAI_Q4_K) return launch_fast_nb<CAI_Q4_K, 0>(p, m, n_b, c.stream);
     if (qt == CAI_Q4_0) return launch_fast_nb<CAI_Q4_0, 0>(p, m, n_b, c.stream);
     return launch_fast_nb<CAI_Q8_0, 0>(p, m, n_b, c.stream);
+  }
+  if (qt == CAI_I8ROW && p.cols % 32 == 0 && !swiglu_half) {   // per-row int8 of a width the 16-byte walk covers; other widths below
+    p.kp = panel_len(p.cols, n_b);
+    p.kp_lds = (p.kp + 511) / 512 * 512;
+    return launch_fast_nb<CAI_I8ROW, 0>(p, m, n_b, c.stream);
   }
   if (swiglu_half) return set_error(CAI_ERR_UNSUPPORTED, "gemv: fused swiglu needs a block-quantized matrix");
   int64_t cum = 0;

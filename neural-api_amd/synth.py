@@ -91,6 +91,14 @@ def random_qweight(qtype, rows, cols, gen, std=0.02, bias=False, chunk_rows=3276
     return w, (raw if keep_bytes else None), b
 
 
+def random_int8_rows(rows, cols, gen, scale=1e-3):
+    """Resident random matrix in the reference's per-row int8 format (codes in [-127, 127], one float scale per row)."""
+    codes = torch.randint(-127, 128, (rows, cols), device="cuda", dtype=torch.int8, generator=gen)
+    scales = torch.full((rows,), scale, device="cuda", dtype=torch.float32)
+    torch.cuda.synchronize()
+    return cai.QWeight(cai.I8ROW, rows, cols, codes.data_ptr(), None, scales.data_ptr())
+
+
 def random_decoder_spec(cfg, qtype, head_qtype, seed=424242, qkv_bias=False, std=0.02, keep_bytes=False):
     """Backend-neutral spec whose tensors are already resident (entry "qw"); norm gains are 1."""
     import numpy as np

@@ -108,6 +108,23 @@ def test_int8_row_path_scale_then_bias():
     assert rel_err(got, want) < TIGHT
 
 
+@pytest.mark.parametrize("rows,cols", [(128, 512), (1000, 3584), (3, 32), (577, 576), (4096, 18944), (37, 2080)])
+@pytest.mark.parametrize("nb", [1, 3, 8])
+def test_int8_row_widths_of_whole_32_blocks_take_the_vector_kernel(rows, cols, nb):
+    """Per-row int8 matrices whose width is a multiple of 32 run the 16-byte-per-lane kernel of the block types (the row scale
+    applied to the finished sum, then the bias: neuralvolume.pas:12693-12745); same contract and tolerance as other widths."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    rng = np.random.default_rng(rows + cols)
+    wf = (rng.standard_normal((rows, cols)) * 0.05).astype(np.float32)
+    codes, scales = O.quant_int8_rows(wf)
+    bias = rng.standard_normal(rows).astype(np.float32)
+    x = rng.standard_normal((nb, cols)).astype(np.float32)
+    got = cai.QWeight(cai.I8ROW, rows, cols, codes, bias, scales).gemv(x)
+    want = O.gemv(O.I8ROW, codes.view(np.uint8), rows, cols, x, bias, 0, 1, scales)
+    assert rel_err(got, want, floor=0.05 * cols ** 0.5) < TIGHT
+
+
 def test_linearity_and_zero_input():
     # size-independent properties at a full-size shape (18944 x 3584 Q4_K)
     from helpers.device import dev, rel_err
@@ -205,18 +222,23 @@ def test_small_batch_gemm_q8_0_q4_0_on_matrix_cores(qt, rows, cols, T):
     assert rel_err(w.gemm(x), want, floor=0.02 * cols ** 0.5 * float(np.abs(x).mean())) < TIGHT   # the dispatcher's own choice
 
 
-@pytest.mark.parametrize("qt,rows,cols", [(O.Q8_0, 4101, 4096), (O.Q4_0, 8203, 4096), (O.Q4_K, 8203, 4096)])
+@pytest.mark.parametrize("qt,rows,cols", [(O.Q8_0, 4101, 4096), (O.Q4_0, 8203, 4096), (O.Q4_K, 8203, 4096), (O.I8ROW, 4101, 4096), (O.I8ROW, 7001, 2400)])
 @pytest.mark.parametrize("nb", [2, 4, 8])
 def test_gemv_batch_on_large_matrix_goes_to_matrix_cores(qt, rows, cols, nb):
     """cai_qgemv with a batch on a matrix of 16 MiB or more takes the matrix-core small-batch path; same contract as batch 1."""
     from helpers.device import dev, rel_err
     cai = dev()
-    raw, rng = make(qt, rows, cols, nb)
+    scales = None
+    if qt == O.I8ROW:      # the reference's own per-row int8 format (width 2400: a short last block group)
+        rng = np.random.default_rng(nb)
+        raw, scales = O.quant_int8_rows((rng.standard_normal((rows, cols)) * 0.02).astype(np.float32))
+    else:
+        raw, rng = make(qt, rows, cols, nb)
     x = rng.standard_normal((nb, cols)).astype(np.float32)
     bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
-    w = cai.QWeight(qt, rows, cols, raw, bias)
+    w = cai.QWeight(qt, rows, cols, raw, bias, scales)
     got = w.gemv(x)
-    want = O.gemv(qt, raw, rows, cols, x, bias, 0, 1)
+    want = O.gemv(qt, raw.view(np.uint8) if qt == O.I8ROW else raw, rows, cols, x, bias, 0, 1, scales) if qt == O.I8ROW else O.gemv(qt, raw, rows, cols, x, bias, 0, 1)
     assert rel_err(got, want, floor=0.02 * cols ** 0.5) < TIGHT
     one = w.gemv(x[:1])
     assert rel_err(got[:1], one, floor=0.02 * cols ** 0.5) < TIGHT
