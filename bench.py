@@ -77,7 +77,8 @@ def gemv_sweep(cai, synth, torch, with_cpu):
     rotating over enough copies of the matrix to exceed the 256 MB infinity cache (at most 24 copies: the small shapes stay
     cache-resident and are labelled so)."""
     lib = cai.load()
-    QT = {"Q8_0": (cai.Q8_0, 34 / 32), "Q4_0": (cai.Q4_0, 18 / 32), "Q4_K": (cai.Q4_K, 144 / 256), "I8ROW": (cai.I8ROW, 1.0)}   # I8ROW: the reference's own per-row int8 format
+    QT = {"Q8_0": (cai.Q8_0, 34 / 32), "Q4_0": (cai.Q4_0, 18 / 32), "Q4_K": (cai.Q4_K, 144 / 256), "Q6_K": (cai.Q6_K, 210 / 256),
+          "I8ROW": (cai.I8ROW, 1.0)}   # I8ROW: the reference's own per-row int8 format
     shapes = [(2048, 2048), (5632, 2048), (2048, 5632), (18944, 3584), (152064, 3584)]
     gen = torch.Generator(device="cuda"); gen.manual_seed(424242)
     cpu = None

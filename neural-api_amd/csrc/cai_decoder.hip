@@ -87,7 +87,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
     if (n_b < 2 || c.n_experts > 0) return false;
     const int slots[6] = {CAI_W_Q, CAI_W_K, CAI_W_V, CAI_W_O, CAI_W_GATEUP, CAI_W_DOWN};
     for (int sl : slots) if (!nb_supported(L.w[sl]) || L.w[sl]->qtype == CAI_I8ROW) return false;   // (per-row int8 products need the plain reduction for their row scale)
-    return L.w[CAI_W_Q]->qtype == L.w[CAI_W_K]->qtype && L.w[CAI_W_Q]->qtype == L.w[CAI_W_V]->qtype;   // q | k | v share one launch
+    return true;
   };
   for (int l = 0; l < c.n_layers; l++) {
     auto& L = d->layers[l];
@@ -126,9 +126,16 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
       if (same) {
         if ((rc = launch_gemv_multi(m, d->x, n_b, d->qkv, qkvw, CAI_ACT_NONE, nullptr, L.v[CAI_V_ATTN_NORM], c.eps, 0))) return rc;
       } else {
-        for (int i = 0; i < 3; i++) {
-          MultiGemv one{}; one.n = 1; one.w[0] = m.w[i]; one.rows[0] = m.rows[i]; one.y_off[0] = offs[i];
-          if ((rc = launch_gemv_multi(one, d->x, n_b, d->qkv, qkvw, CAI_ACT_NONE, nullptr, L.v[CAI_V_ATTN_NORM], c.eps, 0))) return rc;
+        bool done[3] = {false, false, false};       // one launch per weight type (attn_v of a mixed file differs from attn_q, attn_k)
+        for (int i0 = 0; i0 < 3; i0++) {
+          if (done[i0]) continue;
+          MultiGemv grp{};
+          for (int i = i0; i < 3; i++) {
+            if (m.w[i]->qtype != m.w[i0]->qtype) continue;
+            done[i] = true;
+            grp.w[grp.n] = m.w[i]; grp.rows[grp.n] = m.rows[i]; grp.y_off[grp.n] = offs[i]; grp.n++;
+          }
+          if ((rc = launch_gemv_multi(grp, d->x, n_b, d->qkv, qkvw, CAI_ACT_NONE, nullptr, L.v[CAI_V_ATTN_NORM], c.eps, 0))) return rc;
         }
       }
     }

@@ -467,6 +467,164 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
 }
 
 // ------------------------------------------------------------------------------------------
+// Q6_K (256-weight super-blocks of 210 bytes: 128 of low nibbles, 64 of 2-bit high parts, 16 signed scales, one f16;
+// neural/neuralgguf.pas:639-717).  Scales belong to 16 weights of a ROW, so the operands are swapped as for the 32-weight
+// block types and one v_mfma_f32_16x16x16_f16 covers exactly one scale group: the lane (weight row lane % 16, kg) supplies
+// the codes 4 kg .. 4 kg + 3 of the group (q - 32, exact in f16) and multiplies the four results by d * scale, both values
+// it loaded itself.  Group g = 8 nh + 2 j + h of a super-block lies in bytes 16 (4 nh + 2 (j & 1) + h) .. + 15 of ql
+// (nibble j >> 1) and bytes 16 (2 nh + h) .. + 15 of qh (2-bit field j).  Lane kg loads the 16-byte chunks kg and kg + 4
+// of ql and chunk kg of qh (rows are only 2-byte aligned: the requests are issued unaligned), and a 4 x 4 transposition of
+// dwords over the kg lanes leaves dword kg of chunk c in register c.
+// ------------------------------------------------------------------------------------------
+typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+
+__global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
+{
+  extern __shared__ __align__(16) unsigned char nb_smem[];
+  const int S = p.sb_per_slice;
+  _Float16* xs = reinterpret_cast<_Float16*>(nb_smem);              // [S][16][NB_LDX]
+  float* sinv_s = reinterpret_cast<float*>(xs + S * NB_SC * NB_LDX);  // [S][8]
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n = lane & 15, kg = lane >> 4;
+  const int K = p.cols, nsb = K >> 8;
+  const int slice = blockIdx.y, sb0 = slice * S, nS = min(S, nsb - sb0);
+  const int64_t row_bytes = (int64_t)nsb * 210;
+  const int tile0 = blockIdx.x * 4 + wave;
+  const int n_it = tile0 < p.n_tiles ? (p.n_tiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
+  const int nq = n_it * nS;                      // (tile, super-block) items of this wave
+
+  struct WRegs { u32x4_a2 ql[2][2], qh[2], sc[2]; uint32_t d[2]; };
+  auto locate = [&](int tile, const NbSeg*& sg, int& R0) {
+    int sgi = 0, t0 = 0;
+    if (p.n_seg > 1 && tile >= p.seg[0].tile_end) { sgi = 1; t0 = p.seg[0].tile_end; }
+    if (p.n_seg > 2 && tile >= p.seg[1].tile_end) { sgi = 2; t0 = p.seg[1].tile_end; }
+    sg = &p.seg[sgi]; R0 = (tile - t0) * 32;
+  };
+  // unconditional, clamped: past the wave's last item the last one is fetched again (a cache hit)
+  auto load_w = [&](int q, WRegs& r) {
+    const int qc = max(min(q, nq - 1), 0);
+    const int tile = min(tile0 + (qc / nS) * p.tile_stride, p.n_tiles - 1), sb = sb0 + qc % nS;
+    const NbSeg* sg; int R0; locate(tile, sg, R0);
+#pragma unroll
+    for (int hh = 0; hh < 2; hh++) {
+      const uint8_t* blk = sg->w + (int64_t)min(R0 + 16 * hh + n, sg->rows - 1) * row_bytes + (int64_t)sb * 210;   // tail rows: re-read the last row
+      r.ql[hh][0] = *reinterpret_cast<const u32x4_a2*>(blk + 16 * kg);
+      r.ql[hh][1] = *reinterpret_cast<const u32x4_a2*>(blk + 64 + 16 * kg);
+      r.qh[hh] = *reinterpret_cast<const u32x4_a2*>(blk + 128 + 16 * kg);
+      r.sc[hh] = *reinterpret_cast<const u32x4_a2*>(blk + 192);
+      r.d[hh] = *reinterpret_cast<const uint16_t*>(blk + 208);
+    }
+  };
+  WRegs wa, wb, wc;
+  load_w(0, wa); load_w(1, wb);                  // weights do not depend on the staging below
+
+  // ---- stage this slice of the activations: nS x 16 columns x 256 halfs, block scales (four requests per turn) ----
+  {
+    const int n_si = nS * NB_TK;
+    const int si_i = min((int)threadIdx.x, n_si - 1), si_tok = si_i % NB_TK, si_s = si_i / NB_TK;
+    const float siv = p.sinvb[(int64_t)min(si_tok, p.n_tok - 1) * nsb + sb0 + si_s];
+    const int total = nS * NB_SC * 32;
+    for (int base = 0; base < total; base += 4 * 256) {
+      uint4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int idx = min(base + u * 256 + (int)threadIdx.x, total - 1);
+        const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC, tok = min(col % NB_TK, p.n_tok - 1);
+        v[u] = *reinterpret_cast<const uint4*>(((col / NB_TK) ? p.xlo : p.xhi) + (int64_t)tok * K + (sb0 + s) * 256 + chunk * 8);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) {
+        const int idx = base + u * 256 + (int)threadIdx.x;
+        if (idx < total) {
+          const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC;
+          *reinterpret_cast<uint4*>(xs + (s * NB_SC + col) * NB_LDX + chunk * 8) = (col % NB_TK) < p.n_tok ? v[u] : make_uint4(0, 0, 0, 0);
+        }
+      }
+    }
+    if ((int)threadIdx.x < n_si) sinv_s[si_i] = si_tok < p.n_tok ? siv : 0.0f;
+  }
+  __syncthreads();
+
+  float acc[2][4];
+  auto compute = [&](const WRegs& r, int q) {
+    const int s = q % nS;
+    if (s == 0) {
+#pragma unroll
+      for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[hh][i] = 0.0f;
+    }
+    const _Float16* xcol = xs + (s * NB_SC + n) * NB_LDX + 4 * kg;
+    const float4_t z4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    const half2_t o2 = {(_Float16)(-1056.0f), (_Float16)(-1056.0f)};   // 1024 + q - 1056 = q - 32
+    float g[2][4];
+#pragma unroll
+    for (int hh = 0; hh < 2; hh++) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) g[hh][i] = 0.0f;
+      // dword kg of every chunk: ql chunks 0..7 in lq[0..7], qh chunks 0..3 in hq[0..3]
+      uint32_t lq[8], hq[4];
+#pragma unroll
+      for (int a = 0; a < 3; a++) {
+        const u32x4_a2 v = a < 2 ? r.ql[hh][a] : r.qh[hh];
+        const uint2_t t02 = __builtin_amdgcn_permlane32_swap(v.x, v.z, false, false);
+        const uint2_t t13 = __builtin_amdgcn_permlane32_swap(v.y, v.w, false, false);
+        const uint2_t u01 = __builtin_amdgcn_permlane16_swap(t02.x, t13.x, false, false);
+        const uint2_t u23 = __builtin_amdgcn_permlane16_swap(t02.y, t13.y, false, false);
+        uint32_t* dst = a < 2 ? lq + 4 * a : hq;
+        dst[0] = u01.x; dst[1] = u01.y; dst[2] = u23.x; dst[3] = u23.y;
+      }
+      const float d = __half2float(__ushort_as_half((unsigned short)r.d[hh]));
+      const uint32_t scw[4] = {r.sc[hh].x, r.sc[hh].y, r.sc[hh].z, r.sc[hh].w};
+#pragma unroll
+      for (int gi = 0; gi < 16; gi++) {
+        const int nh = gi >> 3, j = (gi >> 1) & 3, h = gi & 1;
+        const uint32_t lo = (lq[4 * nh + 2 * (j & 1) + h] >> (4 * (j >> 1))) & 0x0f0f0f0fu;
+        const uint32_t hf = hq[2 * nh + h];
+        const uint32_t hi = (j == 0 ? (hf << 4) : j == 1 ? (hf << 2) : j == 2 ? hf : (hf >> 2)) & 0x30303030u;
+        const uint32_t c = lo | hi;
+        const half2_t w01 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, c, 0x04010400u)) + o2;
+        const half2_t w23 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, c, 0x04030402u)) + o2;
+        const half4_t W = {w01.x, w01.y, w23.x, w23.y};
+        const half4_t X = *reinterpret_cast<const half4_t*>(xcol + 16 * gi);
+        const float4_t C = __builtin_amdgcn_mfma_f32_16x16x16f16(X, W, z4, 0, 0, 0);
+        const float ds = d * (float)(int)(int8_t)((scw[gi >> 2] >> (8 * (gi & 3))) & 0xffu);
+#pragma unroll
+        for (int i = 0; i < 4; i++) g[hh][i] = fmaf(ds, C[i], g[hh][i]);
+      }
+    }
+    // result row 4 kg + i of the tile = token (4 kg + i) % 8, its hi (kg < 2) or lo (kg >= 2) part
+    const float4 si = *reinterpret_cast<const float4*>(&sinv_s[s * NB_TK + 4 * (kg & 1)]);
+#pragma unroll
+    for (int hh = 0; hh < 2; hh++) {
+      acc[hh][0] = fmaf(si.x, g[hh][0], acc[hh][0]); acc[hh][1] = fmaf(si.y, g[hh][1], acc[hh][1]);
+      acc[hh][2] = fmaf(si.z, g[hh][2], acc[hh][2]); acc[hh][3] = fmaf(si.w, g[hh][3], acc[hh][3]);
+    }
+    if (s != nS - 1) return;
+    // ---- the slice's contribution of this tile: hi + lo parts meet across kg ^ 2; lanes kg < 2 store four tokens ----
+    const int tile = tile0 + (q / nS) * p.tile_stride;
+    const NbSeg* sg; int R0; locate(tile, sg, R0);
+#pragma unroll
+    for (int hh = 0; hh < 2; hh++) {
+      const int row = R0 + 16 * hh + n;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const float tot = acc[hh][i] + __shfl_xor(acc[hh][i], 32, 64);
+        const int tok = 4 * kg + i;
+        if (kg < 2 && tok < p.n_tok && row < sg->rows)
+          p.part[((int64_t)slice * p.n_tok + tok) * p.part_stride + sg->y_off + row] = tot;
+      }
+    }
+  };
+
+  for (int q = 0; q < nq; q += 3) {
+    load_w(q + 2, wc); compute(wa, q);
+    load_w(q + 3, wa); if (q + 1 < nq) compute(wb, q + 1);
+    load_w(q + 4, wb); if (q + 2 < nq) compute(wc, q + 2);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // Activation pre-pass: one work-group per (256-block, token).  Source of the block:
 //   SRC 0  x[t][k]                                                       (a plain activation row)
 //   SRC 1  res[t][k] + bias[k] + sum_s part[s][t][k], written back to res (a projection added to the residual stream)
@@ -708,7 +866,7 @@ int nb_prep_swiglu(int half, int n_tok)
 // Weight types with a small-batch kernel.  Q4_K super-blocks make the width a multiple of 256 by construction.
 bool nb_supported(const cai_qw_s* w)
 {
-  if (w->qtype == CAI_Q4_K) return w->cols % 256 == 0;
+  if (w->qtype == CAI_Q4_K || w->qtype == CAI_Q6_K) return w->cols % 256 == 0 && w->cols >= 256;
   return (w->qtype == CAI_Q8_0 || w->qtype == CAI_Q4_0 || w->qtype == CAI_I8ROW) && w->cols % 32 == 0 && w->cols >= 32;   // per-row int8: unit block scales, the row scale is applied by nb_reduce
 }
 
@@ -720,40 +878,58 @@ static void nb_launch(const NbParams& p, int gx, int n_slices, size_t lds)
   hipLaunchKernelGGL(Kernel, dim3(gx, n_slices), dim3(256), lds, ctx().stream, p);
 }
 
-// partials <- [W0; W1; W2] . planes
+// partials <- [W0; W1; W2] . planes.  The matrices share the width; those of one type share a launch (a Q4_K_M file keeps
+// attn_v of some blocks in Q6_K beside Q4_K attn_q and attn_k), and every launch cuts the columns into the same slices.
 int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok)
 {
   if (n_w < 1 || n_w > 3 || n_tok < 1 || n_tok > NB_TK) return set_error(CAI_ERR_UNSUPPORTED, "small-batch gemm: %d matrices, %d tokens", n_w, n_tok);
-  NbParams p{};
-  p.n_seg = n_w; p.cols = (int)ws[0]->cols;
-  const int qt = ws[0]->qtype;
+  NbParams base{};
+  base.cols = (int)ws[0]->cols;
+  NbSeg segs[3];
   int tiles = 0, width = 0;
   for (int i = 0; i < n_w; i++) {
-    if (!nb_supported(ws[i]) || ws[i]->qtype != qt || ws[i]->cols != ws[0]->cols)
+    if (!nb_supported(ws[i]) || ws[i]->cols != ws[0]->cols)
       return set_error(CAI_ERR_UNSUPPORTED, "small-batch gemm: matrix %d type %d width %lld", i, ws[i]->qtype, (long long)ws[i]->cols);
+    if (i > 0 && y_off[i] < y_off[i - 1]) return set_error(CAI_ERR_INVALID, "small-batch gemm: output offsets must ascend");
     tiles += (int)((ws[i]->rows + 31) / 32);
-    p.seg[i].w = ws[i]->data; p.seg[i].aux = ws[i]->aux; p.seg[i].bias = ws[i]->bias; p.seg[i].row_scale = qt == CAI_I8ROW ? reinterpret_cast<const float*>(ws[i]->aux) : nullptr; p.seg[i].rows = (int)ws[i]->rows; p.seg[i].y_off = y_off[i]; p.seg[i].tile_end = tiles;
+    segs[i] = NbSeg{ws[i]->data, ws[i]->aux, ws[i]->bias, ws[i]->qtype == CAI_I8ROW ? reinterpret_cast<const float*>(ws[i]->aux) : nullptr, (int)ws[i]->rows, y_off[i], 0};
     width = std::max(width, y_off[i] + (int)ws[i]->rows);
   }
-  p.n_tiles = tiles;
   int S, n_slices, gx, tile_stride;
-  nb_geometry(p.cols, tiles, S, n_slices, gx, tile_stride);
+  nb_geometry(base.cols, tiles, S, n_slices, gx, tile_stride);
   const int64_t stride = (width + 3) / 4 * 4;
-  if ((size_t)NB_TK * p.cols > g_nb.cap_k || (size_t)n_slices * n_tok * stride > g_nb.cap_part)
+  if ((size_t)NB_TK * base.cols > g_nb.cap_k || (size_t)n_slices * n_tok * stride > g_nb.cap_part)
     return set_error(CAI_ERR_STATE, "small-batch gemm: workspace not reserved (%d slices x %d tokens x %lld)", n_slices, n_tok, (long long)stride);
-  p.xhi = g_nb.hi; p.xlo = g_nb.lo; p.sxhi = g_nb.sxhi; p.sxlo = g_nb.sxlo; p.sinvb = g_nb.sinvb; p.n_tok = n_tok;
-  p.part = g_nb.part; p.part_stride = stride; p.sb_per_slice = S; p.tile_stride = tile_stride;
-  if (qt == CAI_Q4_K) {
-    const size_t lds = (size_t)S * NB_SC * (NB_LDX + 8) * 2 + (size_t)S * NB_TK * 4 + 4 * 2 * 32 * 4;
-    nb_launch<gemm_q4k_nb>(p, gx, n_slices, lds);
-  } else {
-    const size_t lds = (size_t)S * NB_SC * NB_LDX * 2 + (size_t)S * NB_TK * 4;
-    const bool tail = p.cols % 256 != 0;
-    if (qt == CAI_Q8_0) { if (tail) nb_launch<gemm_blk_nb<CAI_Q8_0, true>>(p, gx, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_Q8_0, false>>(p, gx, n_slices, lds); }
-    else if (qt == CAI_I8ROW) { if (tail) nb_launch<gemm_blk_nb<CAI_I8ROW, true>>(p, gx, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_I8ROW, false>>(p, gx, n_slices, lds); }
-    else { if (tail) nb_launch<gemm_blk_nb<CAI_Q4_0, true>>(p, gx, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_Q4_0, false>>(p, gx, n_slices, lds); }
+  base.xhi = g_nb.hi; base.xlo = g_nb.lo; base.sxhi = g_nb.sxhi; base.sxlo = g_nb.sxlo; base.sinvb = g_nb.sinvb; base.n_tok = n_tok;
+  base.part = g_nb.part; base.part_stride = stride; base.sb_per_slice = S;
+  bool done[3] = {false, false, false};
+  for (int i0 = 0; i0 < n_w; i0++) {
+    if (done[i0]) continue;
+    const int qt = ws[i0]->qtype;
+    NbParams p = base;
+    int sub = 0;
+    for (int i = i0; i < n_w; i++) {
+      if (ws[i]->qtype != qt) continue;
+      done[i] = true;
+      sub += (segs[i].rows + 31) / 32;
+      p.seg[p.n_seg] = segs[i]; p.seg[p.n_seg].tile_end = sub; p.n_seg++;
+    }
+    p.n_tiles = sub;
+    const int gxs = std::max(1, std::min(gx, (sub + 3) / 4));
+    p.tile_stride = gxs * 4;
+    if (qt == CAI_Q4_K) {
+      const size_t lds = (size_t)S * NB_SC * (NB_LDX + 8) * 2 + (size_t)S * NB_TK * 4 + 4 * 2 * 32 * 4;
+      nb_launch<gemm_q4k_nb>(p, gxs, n_slices, lds);
+    } else {
+      const size_t lds = (size_t)S * NB_SC * NB_LDX * 2 + (size_t)S * NB_TK * 4;
+      const bool tail = p.cols % 256 != 0;
+      if (qt == CAI_Q6_K) nb_launch<gemm_q6k_nb>(p, gxs, n_slices, lds);
+      else if (qt == CAI_Q8_0) { if (tail) nb_launch<gemm_blk_nb<CAI_Q8_0, true>>(p, gxs, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_Q8_0, false>>(p, gxs, n_slices, lds); }
+      else if (qt == CAI_I8ROW) { if (tail) nb_launch<gemm_blk_nb<CAI_I8ROW, true>>(p, gxs, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_I8ROW, false>>(p, gxs, n_slices, lds); }
+      else { if (tail) nb_launch<gemm_blk_nb<CAI_Q4_0, true>>(p, gxs, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_Q4_0, false>>(p, gxs, n_slices, lds); }
+    }
   }
-  for (int i = 0; i < 3; i++) g_prod.seg[i] = p.seg[i];
+  for (int i = 0; i < n_w; i++) g_prod.seg[i] = segs[i];
   g_prod.n_seg = n_w; g_prod.n_slices = n_slices; g_prod.n_tok = n_tok; g_prod.part_stride = stride; g_prod.width = width;
   g_prod.in_ssq = g_pending_ssq; g_prod.in_nsb = (g_pending_K + 255) >> 8; g_prod.in_K = g_pending_K; g_prod.in_eps = g_pending_eps;
   return CAI_OK;

@@ -19,6 +19,12 @@ template <> struct QTraits<CAI_Q4_K> { static constexpr int UW = 32, T = 8; };  
 template <> struct QTraits<CAI_Q4_0> { static constexpr int UW = 32, T = 8; };
 template <> struct QTraits<CAI_Q8_0> { static constexpr int UW = 16, T = 4; };
 template <> struct QTraits<CAI_I8ROW> { static constexpr int UW = 16, T = 4; };   // per-row int8: the Q8_0 walk with one scale per row, applied at the end
+// Q6_K: 16 lanes per 210-byte super-block.  Lane t (half nh = t>>3, byte position l4 = 4*(t&7)) takes four bytes each of the
+// two ql runs and of the qh run of its half, i.e. the 16 weights 128*nh + 32*j + l4 + {0..3}, j = 0..3, which fall in four
+// different 16-weight scale groups (neural/neuralgguf.pas:639-717).  Blocks are only 2-byte aligned in a row; the dword
+// requests are issued unaligned.
+template <> struct QTraits<CAI_Q6_K> { static constexpr int UW = 16, T = 4; };
+typedef uint32_t __attribute__((aligned(2))) u32_a2;
 
 // original float4 index n (within the panel) -> LDS float4 slot, unit-transposed in tiles of 16 units
 template <int QT> __device__ __forceinline__ int lds_slot(int n)
@@ -29,6 +35,7 @@ template <int QT> __device__ __forceinline__ int lds_slot(int n)
     const int sb = n >> 6, cc = (n >> 4) & 3, hi = (n >> 3) & 1, h = (n >> 2) & 1, tt = n & 3;
     u = sb * 8 + cc * 2 + h; t = hi * 4 + tt;
   } else if (QT == CAI_Q4_0) { u = n >> 3; t = n & 7; }
+  else if (QT == CAI_Q6_K) { u = (n >> 6) * 16 + ((n >> 5) & 1) * 8 + (n & 7); t = (n >> 3) & 3; }   // n = [sb][nh:1][j:2][t&7:3]
   else { u = n >> 2; t = n & 3; }
   constexpr int T = QTraits<QT>::T;
   return (u >> 4) * 16 * T + t * 16 + (u & 15);
@@ -38,6 +45,16 @@ template <int QT> __device__ __forceinline__ int lds_unit_base(int u)
 {
   constexpr int T = QTraits<QT>::T;
   return (u >> 4) * 16 * T + (u & 15);   // + t*16
+}
+
+// The four code dwords of a Q6_K lane: cj[j] holds the 6-bit codes (0..63) of weights 32*j + l4 + {0..3} of the half, one per
+// byte: low nibbles from ql (j = 0, 1) or its high nibbles (j = 2, 3), bits 4..5 from the 2-bit field j of the qh bytes.
+__device__ __forceinline__ void q6k_codes(uint32_t ql0, uint32_t ql1, uint32_t qh, uint32_t cj[4])
+{
+  cj[0] = (ql0 & 0x0f0f0f0fu) | ((qh << 4) & 0x30303030u);
+  cj[1] = (ql1 & 0x0f0f0f0fu) | ((qh << 2) & 0x30303030u);
+  cj[2] = ((ql0 >> 4) & 0x0f0f0f0fu) | (qh & 0x30303030u);
+  cj[3] = ((ql1 >> 4) & 0x0f0f0f0fu) | ((qh >> 2) & 0x30303030u);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -69,6 +86,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
   const int cols = p.cols;
   int64_t row_bytes, aux_row_bytes = 0;
   if (QT == CAI_Q4_K) row_bytes = (int64_t)(cols >> 8) * 144;
+  else if (QT == CAI_Q6_K) row_bytes = (int64_t)(cols >> 8) * 210;
   else if (QT == CAI_Q4_0) { row_bytes = cols >> 1; aux_row_bytes = (cols >> 5) * 2; }
   else if (QT == CAI_I8ROW) row_bytes = cols;
   else { row_bytes = cols; aux_row_bytes = (cols >> 5) * 2; }
@@ -162,6 +180,18 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
           hdr[r] = *reinterpret_cast<const uint4*>(blk);
           q[r] = *reinterpret_cast<const uint4*>(blk + 16 + 16 * j);
         }
+      } else if (QT == CAI_Q6_K) {
+        const int sb = (k0 >> 8) + (u >> 4), nh = (u >> 3) & 1, l4 = (u & 7) * 4;
+#pragma unroll
+        for (int r = 0; r < RR; r++) {
+          const uint8_t* blk = rp[r] + (int64_t)sb * 210;
+          q[r].x = *reinterpret_cast<const u32_a2*>(blk + 64 * nh + l4);
+          q[r].y = *reinterpret_cast<const u32_a2*>(blk + 64 * nh + 32 + l4);
+          q[r].z = *reinterpret_cast<const u32_a2*>(blk + 128 + 32 * nh + l4); q[r].w = 0u;
+          hdr[r].x = *reinterpret_cast<const u32_a2*>(blk + 192 + 8 * nh);
+          hdr[r].y = *reinterpret_cast<const u32_a2*>(blk + 196 + 8 * nh);
+          dh[r] = *reinterpret_cast<const uint16_t*>(blk + 208);
+        }
       } else if (QT == CAI_Q4_0) {
         const int blk = (k0 >> 5) + u;
 #pragma unroll
@@ -210,6 +240,25 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
             const float part = d * (cvt_ub0(sc) * slo + cvt_ub1(sc) * shi) - dmin * (cvt_ub0(mn) * sxlo + cvt_ub1(mn) * sxhi);
             acc[r][0] += part;
           }
+        } else if (QT == CAI_Q6_K) {
+          float sx[4];
+#pragma unroll
+          for (int j = 0; j < 4; j++) sx[j] = (xv[4 * j] + xv[4 * j + 1]) + (xv[4 * j + 2] + xv[4 * j + 3]);
+          const int hs = (u & 4) ? 8 : 0;    // positions 16..31 of a 32-run use the odd scale of the pair
+#pragma unroll
+          for (int r = 0; r < RR; r++) {
+            uint32_t cj[4]; q6k_codes(q[r].x, q[r].y, q[r].z, cj);
+            const uint32_t s01 = hdr[r].x >> hs, s23 = hdr[r].y >> hs;
+            const float sc[4] = {(float)(int8_t)(s01 & 0xff), (float)(int8_t)((s01 >> 16) & 0xff), (float)(int8_t)(s23 & 0xff), (float)(int8_t)((s23 >> 16) & 0xff)};
+            float part = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+              float sq = cvt_ub0(cj[j]) * xv[4 * j];
+              sq = fmaf(cvt_ub1(cj[j]), xv[4 * j + 1], sq); sq = fmaf(cvt_ub2(cj[j]), xv[4 * j + 2], sq); sq = fmaf(cvt_ub3(cj[j]), xv[4 * j + 3], sq);
+              part = fmaf(sc[j], fmaf(-32.0f, sx[j], sq), part);
+            }
+            acc[r][0] = fmaf(__half2float(__ushort_as_half(dh[r])), part, acc[r][0]);
+          }
         } else if (QT == CAI_Q4_0) {
           float sx = 0.0f;
 #pragma unroll
@@ -252,7 +301,20 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
 #pragma unroll
         for (int r = 0; r < RR; r++) {
           const uint32_t qw[4] = {q[r].x, q[r].y, q[r].z, q[r].w};
-          if (QT == CAI_Q8_0 || QT == CAI_I8ROW) {
+          if (QT == CAI_Q6_K) {
+            uint32_t cj[4]; q6k_codes(q[r].x, q[r].y, q[r].z, cj);
+            const int hs = (u & 4) ? 8 : 0;
+            const uint32_t s01 = hdr[r].x >> hs, s23 = hdr[r].y >> hs;
+            const float d = __half2float(__ushort_as_half(dh[r]));
+            // the four group scales of the lane travel in s0, s1, m0, m1
+            s0[r] = d * (float)(int8_t)(s01 & 0xff); s1[r] = d * (float)(int8_t)((s01 >> 16) & 0xff);
+            m0[r] = d * (float)(int8_t)(s23 & 0xff); m1[r] = d * (float)(int8_t)((s23 >> 16) & 0xff);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+              wf[r][4 * j] = cvt_ub0(cj[j]) - 32.0f; wf[r][4 * j + 1] = cvt_ub1(cj[j]) - 32.0f;
+              wf[r][4 * j + 2] = cvt_ub2(cj[j]) - 32.0f; wf[r][4 * j + 3] = cvt_ub3(cj[j]) - 32.0f;
+            }
+          } else if (QT == CAI_Q8_0 || QT == CAI_I8ROW) {
 #pragma unroll
             for (int w = 0; w < 4; w++) {
               wf[r][4 * w] = (float)(int8_t)(qw[w] & 0xff); wf[r][4 * w + 1] = (float)(int8_t)((qw[w] >> 8) & 0xff);
@@ -283,7 +345,18 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
             const float4 v = xb[xb0 + t * 16];
             xv[4 * t] = v.x; xv[4 * t + 1] = v.y; xv[4 * t + 2] = v.z; xv[4 * t + 3] = v.w;
           }
-          if (QT == CAI_Q8_0 || QT == CAI_I8ROW) {
+          if (QT == CAI_Q6_K) {
+#pragma unroll
+            for (int r = 0; r < RR; r++) {
+              float g[4];
+#pragma unroll
+              for (int j = 0; j < 4; j++) {
+                g[j] = wf[r][4 * j] * xv[4 * j];
+                g[j] = fmaf(wf[r][4 * j + 1], xv[4 * j + 1], g[j]); g[j] = fmaf(wf[r][4 * j + 2], xv[4 * j + 2], g[j]); g[j] = fmaf(wf[r][4 * j + 3], xv[4 * j + 3], g[j]);
+              }
+              acc[r][b] += (s0[r] * g[0] + s1[r] * g[1]) + (m0[r] * g[2] + m1[r] * g[3]);
+            }
+          } else if (QT == CAI_Q8_0 || QT == CAI_I8ROW) {
 #pragma unroll
             for (int r = 0; r < RR; r++) {
               float sq = 0.0f;
@@ -359,7 +432,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
 }
 
 // ------------------------------------------------------------------------------------------
-// Simple kernel: F32 / F16 / I8ROW and any shape the fast kernel does not take.  One wave per row,
+// Simple kernel: F32 / F16 and the per-row int8 widths the fast kernel does not take.  One wave per row,
 // lanes stride the row with scalar loads (coalesced), fp32 accumulation.
 // ------------------------------------------------------------------------------------------
 template <int QT>
@@ -392,27 +465,6 @@ __global__ __launch_bounds__(256) void gemv_simple(const GemvParams p, int n_b)
       inv = 1.0f / sqrtf(ss / (float)cols + p.norm_eps);
     }
     float acc = 0.0f;
-    if (QT == CAI_Q6_K) {
-      // one super-block (210 B) per pass of the wave: lane = (half n, position ll) owns elements 128n + ll + {0, 32, 64, 96},
-      // i.e. both nibbles of ql bytes 64n + ll and 64n + ll + 32 and the four 2-bit fields of qh byte 32n + ll
-      const uint8_t* rowp = sg.data + wrow * (int64_t)(cols >> 8) * 210;
-      const int n = lane >> 5, ll = lane & 31;
-      for (int sb = 0; sb < (cols >> 8); sb++) {
-        const uint8_t* blk = rowp + (int64_t)sb * 210;
-        const int l0 = blk[64 * n + ll], l1 = blk[64 * n + ll + 32], h = blk[128 + 32 * n + ll];
-        const int8_t* sc = reinterpret_cast<const int8_t*>(blk + 192) + 8 * n + (ll >> 4);
-        const float d = __half2float(__ushort_as_half((unsigned short)(blk[208] | (blk[209] << 8))));
-        const int q[4] = {((l0 & 15) | ((h & 3) << 4)) - 32, ((l1 & 15) | (((h >> 2) & 3) << 4)) - 32,
-                          ((l0 >> 4) | (((h >> 4) & 3) << 4)) - 32, ((l1 >> 4) | (((h >> 6) & 3) << 4)) - 32};
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          const int i = sb * 256 + 128 * n + ll + 32 * j;
-          float xv = xb[i];
-          if (p.norm_gain) xv = p.norm_gain[i] * (xv * inv);
-          acc = fmaf((d * (float)sc[2 * j]) * (float)q[j], xv, acc);
-        }
-      }
-    } else
     for (int i = lane; i < cols; i += 64) {
       float w;
       if (QT == CAI_F32) w = reinterpret_cast<const float*>(sg.data)[wrow * cols + i];
@@ -587,6 +639,11 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
     p.kp_lds = (p.kp + 511) / 512 * 512;
     return launch_fast_nb<CAI_I8ROW, 0>(p, m, n_b, c.stream);
   }
+  if (qt == CAI_Q6_K && !swiglu_half) {
+    p.kp = panel_len(p.cols, n_b);
+    p.kp_lds = (p.kp + 511) / 512 * 512;
+    return launch_fast_nb<CAI_Q6_K, 0>(p, m, n_b, c.stream);
+  }
   if (swiglu_half) return set_error(CAI_ERR_UNSUPPORTED, "gemv: fused swiglu needs a block-quantized matrix");
   int64_t cum = 0;
   for (int i = 0; i < m.n; i++) { cum += m.rows[i]; p.seg[i].grp_end = (int)cum; }
@@ -594,7 +651,6 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
   if (qt == CAI_F32) hipLaunchKernelGGL(gemv_simple<CAI_F32>, grid, dim3(256), 0, c.stream, p, n_b);
   else if (qt == CAI_F16) hipLaunchKernelGGL(gemv_simple<CAI_F16>, grid, dim3(256), 0, c.stream, p, n_b);
   else if (qt == CAI_I8ROW) hipLaunchKernelGGL(gemv_simple<CAI_I8ROW>, grid, dim3(256), 0, c.stream, p, n_b);
-  else if (qt == CAI_Q6_K) hipLaunchKernelGGL(gemv_simple<CAI_Q6_K>, grid, dim3(256), 0, c.stream, p, n_b);
   else return set_error(CAI_ERR_UNSUPPORTED, "gemv: weight type %d", qt);
   return CAI_OK;
 }

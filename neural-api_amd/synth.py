@@ -71,7 +71,30 @@ def pack_q4_k(x):
     return out
 
 
-PACKERS = {cai.Q8_0: pack_q8_0, cai.Q4_0: pack_q4_0, cai.Q4_K: pack_q4_k}
+def pack_q6_k(x):
+    """x: [rows, cols] float32 (cols % 256 == 0) -> uint8 [rows, cols/256, 210]: symmetric fit, one signed scale per 16
+    weights, codes q in 0..63 standing for q - 32 (layout of neural/neuralgguf.pas:639-717)"""
+    rows, cols = x.shape
+    nsb = cols // 256
+    xg = x.view(rows, nsb, 16, 16)
+    step = xg.abs().amax(-1) / 31.0
+    d16 = (step.amax(-1) / 127.0).to(torch.float16)
+    d = d16.float()[..., None]
+    sc = torch.where(d > 0, torch.round(step / d), torch.zeros_like(step)).clamp_(0, 127)
+    ds = (d * sc)[..., None]
+    q = (torch.where(ds > 0, torch.round(xg / ds), torch.zeros_like(xg)).clamp_(-32, 31) + 32).to(torch.uint8)
+    q = q.view(rows, nsb, 2, 4, 32)                       # [half][j][l]: weight 128 half + 32 j + l
+    out = torch.empty(rows, nsb, 210, dtype=torch.uint8, device=x.device)
+    lo = q & 15; hi = q >> 4
+    ql = torch.stack([lo[..., 0, :] | (lo[..., 2, :] << 4), lo[..., 1, :] | (lo[..., 3, :] << 4)], dim=-2)   # [half][2][32]
+    out[..., 0:128] = ql.reshape(rows, nsb, 128)
+    out[..., 128:192] = (hi[..., 0, :] | (hi[..., 1, :] << 2) | (hi[..., 2, :] << 4) | (hi[..., 3, :] << 6)).reshape(rows, nsb, 64)
+    out[..., 192:208] = sc.to(torch.int8).view(torch.uint8)
+    out[..., 208:210] = d16.view(torch.uint8).view(rows, nsb, 2)
+    return out
+
+
+PACKERS = {cai.Q8_0: pack_q8_0, cai.Q4_0: pack_q4_0, cai.Q4_K: pack_q4_k, cai.Q6_K: pack_q6_k}
 
 
 def random_qweight(qtype, rows, cols, gen, std=0.02, bias=False, chunk_rows=32768, keep_bytes=False):

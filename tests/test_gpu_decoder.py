@@ -139,6 +139,40 @@ def test_batched_decode_of_32_weight_block_models_equals_single(name):
             assert int(am[b]) == int(np.argmax(singles[b][p]))
 
 
+def test_batched_decode_and_prompt_of_a_q4k_q6k_mix_equal_single_steps():
+    """The Q4_K_M mix (attn_v and ffn_down of every other block and the head in Q6_K, the rest Q4_K): a batch steps every
+    linear layer on the matrix cores, q | k of one type and v of another sharing the partial buffer; the prompt path takes
+    the Q6_K matrices through the small-batch kernels.  Both equal single-token steps."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    cfg = dict(n_layers=4, d_model=512, n_q_heads=8, n_kv_heads=2, head_dim=64, ffn=1024, vocab=600, max_ctx=64, eps=1e-5, rope_theta=1e4)
+    spec = synthetic_spec(cfg, O.Q4_K, head_qtype=O.Q6_K, seed=5, std=0.05)
+    rng = np.random.default_rng(4)
+    for l in (0, 2):
+        for slot in (O.W_V, O.W_DOWN):
+            t = spec["tensors"][(l, slot)]
+            w = (rng.standard_normal((t["rows"], t["cols"])) * 0.05).astype(np.float32)
+            t.update(type=O.Q6_K, raw=O.quantize(O.Q6_K, w))
+    dec = cai.Decoder(spec, max_batch=4)
+    toks = rng.integers(0, cfg["vocab"], (4, 10))
+    singles = []
+    for b in range(4):
+        dec.reset(0)
+        singles.append([dec.step(int(toks[b, p]), p)[1][0].copy() for p in range(10)])
+    om = oracle_model(spec, acc64=1)
+    want0 = np.array([om.step(int(t), p)[1] for p, t in enumerate(toks[0])])
+    assert rel_err(np.array(singles[0]), want0) < 1e-3
+    for b in range(4):
+        dec.reset(b)
+    for p in range(10):
+        am, lg = dec.step(toks[:, p], np.full(4, p))
+        for b in range(4):
+            assert rel_err(lg[b], singles[b][p]) < 1e-3
+    dec.reset(1)
+    am, lg = dec.prefill([int(t) for t in toks[2]], 0, seq=1)
+    assert rel_err(lg, singles[2][9]) < 1e-3 and am == int(np.argmax(singles[2][9]))
+
+
 def test_prefill_equals_sequential_steps():
     from helpers.device import dev, rel_err
     cai = dev()

@@ -81,9 +81,11 @@ def test_float_weight_types_any_width(qt, rows, cols):
     assert rel_err(got, O.gemv(qt, raw, rows, cols, x, None, 0, 1)) < TIGHT
 
 
-@pytest.mark.parametrize("rows,cols,nb", [(37, 256, 1), (512, 3584, 1), (300, 2048, 3)])
+@pytest.mark.parametrize("rows,cols,nb", [(37, 256, 1), (512, 3584, 1), (300, 2048, 3), (9001, 512, 1), (33001, 256, 1), (70, 18944, 1),
+                                          (66, 18944, 2), (41, 1024, 8), (18000, 256, 5)])
 def test_q6_k_gemv_matches_oracle(rows, cols, nb):
-    """Q6_K (the type real Q4_K_M files use for output.weight and part of ffn_down): functional path, same bar."""
+    """Q6_K (the type real Q4_K_M files use for output.weight and part of ffn_down) on the vector kernel: 16 lanes per
+    210-byte super-block, unaligned dword requests; 1, 2 and 4 rows per wave, several activation panels, batches."""
     from helpers.device import dev, rel_err
     cai = dev()
     raw, rng = make(O.Q6_K, rows, cols, rows + cols)
@@ -222,7 +224,26 @@ def test_small_batch_gemm_q8_0_q4_0_on_matrix_cores(qt, rows, cols, T):
     assert rel_err(w.gemm(x), want, floor=0.02 * cols ** 0.5 * float(np.abs(x).mean())) < TIGHT   # the dispatcher's own choice
 
 
-@pytest.mark.parametrize("qt,rows,cols", [(O.Q8_0, 4101, 4096), (O.Q4_0, 8203, 4096), (O.Q4_K, 8203, 4096), (O.I8ROW, 4101, 4096), (O.I8ROW, 7001, 2400)])
+@pytest.mark.parametrize("rows,cols,T", [(128, 256, 2), (33, 512, 3), (1000, 1024, 8), (3584, 3584, 8), (512, 18944, 4), (20000, 2048, 16), (5000, 768, 13), (70, 1536, 7)])
+def test_small_batch_gemm_q6_k_on_matrix_cores(rows, cols, T):
+    """Q6_K on the matrix cores: one 16-deep MFMA per 16-weight scale group (codes q - 32 exact in f16, d * scale applied to
+    the result by the lane that owns the weight row), unaligned 16-byte requests transposed over the four k lanes
+    == T single-token layers, bias included."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    raw, rng = make(O.Q6_K, rows, cols, T + 300)
+    x = (rng.standard_normal((T, cols)) * rng.uniform(0.01, 30.0, (T, 1))).astype(np.float32)
+    x[0, : cols // 2] = 0.0
+    bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
+    w = cai.QWeight(O.Q6_K, rows, cols, raw, bias)
+    got = w.gemm(x, matrix_cores=True)
+    want = O.gemv(O.Q6_K, raw, rows, cols, x, bias, 0, 1)
+    for t in range(T):
+        assert rel_err(got[t], want[t], floor=0.02 * cols ** 0.5 * float(np.abs(x[t]).mean())) < TIGHT, t
+    assert rel_err(w.gemm(x), want, floor=0.02 * cols ** 0.5 * float(np.abs(x).mean())) < TIGHT   # the dispatcher's own choice
+
+
+@pytest.mark.parametrize("qt,rows,cols", [(O.Q8_0, 4101, 4096), (O.Q4_0, 8203, 4096), (O.Q4_K, 8203, 4096), (O.Q6_K, 5003, 4096), (O.I8ROW, 4101, 4096), (O.I8ROW, 7001, 2400)])
 @pytest.mark.parametrize("nb", [2, 4, 8])
 def test_gemv_batch_on_large_matrix_goes_to_matrix_cores(qt, rows, cols, nb):
     """cai_qgemv with a batch on a matrix of 16 MiB or more takes the matrix-core small-batch path; same contract as batch 1."""
