@@ -101,16 +101,19 @@ __device__ __forceinline__ half4_t bytes_to_half4_pf(uint32_t t)
 
 typedef _Float16 half8_pf __attribute__((ext_vector_type(8)));
 
-// One work-group: 128 rows (wave = 32 rows) x TT * 32 tokens, one super-block (256 columns) per step, on
+// One work-group: 4 waves x RT row tiles of 32 rows x TT * 32 tokens, one super-block (256 columns) per step, on
 // v_mfma_f32_32x32x16_f16 (lane (n, kg) supplies 8 consecutive k of row / column n).
 //   * the weight operand sc_j * q (<= 63 * 15, exact in f16) is built once per super-block per wave and reused by the
 //     token tiles and by the hi and lo activation planes; the matrix cores accumulate across the whole super-block, hi
-//     and lo planes into the same accumulator (the chains of the token tiles interleave);
+//     and lo planes into the same accumulator (the chains of the tiles interleave);
 //   * -dmin * mn_j * sum_{k in j} x_k is one more MFMA step per plane (k = the 8 sub-blocks);
 //   * d and dmin are applied once per super-block (2 FMAs per value), the token scale once at the end.
+// Every MFMA takes its activation operand from LDS (1 KB per wave and instruction): with one row tile per wave the LDS
+// pipe, not the matrix cores, sets the pace.  RT = 2 lets one activation operand serve two row tiles (half the LDS reads
+// per FLOP); it needs 256 rows per work-group and is used for matrices with enough row groups to fill the chip.
 // Work-group ids are laid out so that the token tiles of one row group run on one XCD: the re-reads of its weights (one
 // per token tile) hit that XCD's L2.  TT = 1 doubles the number of work-groups for matrices with few row groups.
-template <int TT>
+template <int TT, int RT>
 __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
 {
   extern __shared__ __align__(16) unsigned char pf_smem[];
@@ -119,33 +122,40 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
   _Float16* xs_lo = xs_hi + NTOK * PF_LDX;
   _Float16* sx_hi = xs_lo + NTOK * PF_LDX;                            // [NTOK][8]
   _Float16* sx_lo = sx_hi + NTOK * 8;
-  float* s_d = reinterpret_cast<float*>(sx_lo + NTOK * 8);            // [4 waves][2][32]
+  float* s_d = reinterpret_cast<float*>(sx_lo + NTOK * 8);            // [4 waves][RT][2][32]
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 31, kg = lane >> 5;
   // linear id = rg_lo + 8 * (tt + n_tok_tiles * rg_hi): a row group's token tiles share id mod 8
   const int L = blockIdx.x, rg = (L & 7) + 8 * ((L >> 3) / p.n_tok_tiles), ttile = (L >> 3) % p.n_tok_tiles;
   if (rg >= p.n_row_groups) return;
-  const int R0 = rg * 128 + wave * 32, T0 = ttile * NTOK;
+  const int R0 = (rg * 4 + wave) * 32 * RT, T0 = ttile * NTOK;
   const int K = p.cols, nsb = K >> 8, nb32 = K >> 5;
   const int64_t row_bytes = (int64_t)nsb * 144;
-  const uint8_t* wrow = p.w + (int64_t)min(R0 + n, p.rows - 1) * row_bytes;   // tail rows: re-read the last row, not written
+  const uint8_t* wrow[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; rt++) wrow[rt] = p.w + (int64_t)min(R0 + 32 * rt + n, p.rows - 1) * row_bytes;   // tail rows: re-read the last row, not written
 
   struct WRegs { uint4 h, q[4]; };
-  auto load_w = [&](int sb, WRegs& r) {
+  auto load_w = [&](int sb, WRegs (&r)[RT]) {
     if (sb < nsb) {
-      const uint8_t* blk = wrow + (int64_t)sb * 144;
-      r.h = *reinterpret_cast<const uint4*>(blk);
 #pragma unroll
-      for (int i = 0; i < 4; i++) r.q[i] = *reinterpret_cast<const uint4*>(blk + 16 + 64 * kg + 16 * i);
+      for (int rt = 0; rt < RT; rt++) {
+        const uint8_t* blk = wrow[rt] + (int64_t)sb * 144;
+        r[rt].h = *reinterpret_cast<const uint4*>(blk);
+#pragma unroll
+        for (int i = 0; i < 4; i++) r[rt].q[i] = *reinterpret_cast<const uint4*>(blk + 16 + 64 * kg + 16 * i);
+      }
     }
   };
-  float16_t Y[TT];
+  float16_t Y[RT][TT];
 #pragma unroll
-  for (int tt = 0; tt < TT; tt++)
+  for (int rt = 0; rt < RT; rt++)
 #pragma unroll
-    for (int v = 0; v < 16; v++) Y[tt][v] = 0.0f;
+    for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) Y[rt][tt][v] = 0.0f;
 
-  WRegs wcur, wnxt;
+  WRegs wcur[RT], wnxt[RT];
   load_w(0, wcur);
   for (int sb = 0; sb < nsb; sb++) {
     __syncthreads();                       // the previous step's LDS reads are done
@@ -155,7 +165,7 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
       // the end repeat the last token (their results are never written), so the loads carry no branch and issue together.
       const int tq = threadIdx.x >> 5, chunk = threadIdx.x & 31;
       const uint32_t colo = (uint32_t)(sb * 256 + chunk * 8);
-      constexpr int SB = TT == 2 ? 1 : 4;     // loads in flight per plane (measured: with two token tiles the registers are worth more than the overlap)
+      constexpr int SB = (TT == 2 || RT == 2) ? 1 : 4;     // loads in flight per plane (measured: with two tiles the registers are worth more than the overlap)
 #pragma unroll
       for (int i0 = 0; i0 < NTOK / 8; i0 += SB) {
         uint4 vh[SB], vl[SB];
@@ -180,48 +190,44 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
     load_w(sb + 1, wnxt);
     __syncthreads();
 
-    // ---- weight operand of this super-block: 16 groups of eight sc*q values ----
-    const WRegs& r = wcur;
-    const uint32_t sc4 = kg == 0 ? (r.h.y & 0x3f3f3f3fu) : ((r.h.w & 0x0f0f0f0fu) | ((r.h.y >> 2) & 0x30303030u));
-    const uint32_t mn4 = kg == 0 ? (r.h.z & 0x3f3f3f3fu) : (((r.h.w >> 4) & 0x0f0f0f0fu) | ((r.h.z >> 2) & 0x30303030u));
+    // ---- weight operand of this super-block: per row tile 16 groups of eight sc*q values ----
     const _Float16 k1024 = (_Float16)1024.0f;
-    const half4_t sch = bytes_to_half4_pf(sc4), mnh = bytes_to_half4_pf(mn4);
-    const half4_t scv = half4_t{sch.x - k1024, sch.y - k1024, sch.z - k1024, sch.w - k1024};
-    const half4_t mnv = half4_t{mnh.x - k1024, mnh.y - k1024, mnh.z - k1024, mnh.w - k1024};
-    if (kg == 0) {
-      const float d = __half2float(__ushort_as_half((unsigned short)(r.h.x & 0xffffu)));
-      const float dmin = __half2float(__ushort_as_half((unsigned short)(r.h.x >> 16)));
-      s_d[(wave * 2 + 0) * 32 + n] = d; s_d[(wave * 2 + 1) * 32 + n] = dmin * 32.0f;
-    }
-    half8_pf A[4][4];
+    half8_pf A[RT][4][4];
+    half4_t mnv[RT];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {                                      // sub-block 4kg + j: bytes of chunk 2kg + (j >> 1), low or high nibbles
-      const int ccl = j >> 1, hl = j & 1;
-      const _Float16 sj = j == 0 ? scv.x : (j == 1 ? scv.y : (j == 2 ? scv.z : scv.w));
-      const half2_t s2 = {sj, sj};
-      const half2_t c2 = {(_Float16)(-1024.0f) * sj, (_Float16)(-1024.0f) * sj};   // exact: a multiple of 1024 below 65504
+    for (int rt = 0; rt < RT; rt++) {
+      const WRegs& r = wcur[rt];
+      const uint32_t sc4 = kg == 0 ? (r.h.y & 0x3f3f3f3fu) : ((r.h.w & 0x0f0f0f0fu) | ((r.h.y >> 2) & 0x30303030u));
+      const uint32_t mn4 = kg == 0 ? (r.h.z & 0x3f3f3f3fu) : (((r.h.w >> 4) & 0x0f0f0f0fu) | ((r.h.z >> 2) & 0x30303030u));
+      const half4_t sch = bytes_to_half4_pf(sc4), mnh = bytes_to_half4_pf(mn4);
+      const half4_t scv = half4_t{sch.x - k1024, sch.y - k1024, sch.z - k1024, sch.w - k1024};
+      mnv[rt] = half4_t{mnh.x - k1024, mnh.y - k1024, mnh.z - k1024, mnh.w - k1024};
+      if (kg == 0) {
+        const float d = __half2float(__ushort_as_half((unsigned short)(r.h.x & 0xffffu)));
+        const float dmin = __half2float(__ushort_as_half((unsigned short)(r.h.x >> 16)));
+        s_d[((wave * RT + rt) * 2 + 0) * 32 + n] = d; s_d[((wave * RT + rt) * 2 + 1) * 32 + n] = dmin * 32.0f;
+      }
 #pragma unroll
-      for (int t = 0; t < 4; t++) {                                    // weights 8t .. 8t+7 of the sub-block
-        const uint4& qq = r.q[2 * ccl + (t >> 1)];
-        const uint32_t qa = (t & 1) ? qq.z : qq.x, qb = (t & 1) ? qq.w : qq.y;
-        const uint32_t na = hl ? ((qa >> 4) & 0x0f0f0f0fu) : (qa & 0x0f0f0f0fu);
-        const uint32_t nb = hl ? ((qb >> 4) & 0x0f0f0f0fu) : (qb & 0x0f0f0f0fu);
-        const half2_t a0 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, na, 0x04010400u)), s2, c2);   // (1024 + q) * sc - 1024 * sc = sc * q
-        const half2_t a1 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, na, 0x04030402u)), s2, c2);
-        const half2_t a2 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, nb, 0x04010400u)), s2, c2);
-        const half2_t a3 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, nb, 0x04030402u)), s2, c2);
-        A[j][t] = half8_pf{a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+      for (int j = 0; j < 4; j++) {                                      // sub-block 4kg + j: bytes of chunk 2kg + (j >> 1), low or high nibbles
+        const int ccl = j >> 1, hl = j & 1;
+        const _Float16 sj = j == 0 ? scv.x : (j == 1 ? scv.y : (j == 2 ? scv.z : scv.w));
+        const half2_t s2 = {sj, sj};
+        const half2_t c2 = {(_Float16)(-1024.0f) * sj, (_Float16)(-1024.0f) * sj};   // exact: a multiple of 1024 below 65504
+#pragma unroll
+        for (int t = 0; t < 4; t++) {                                    // weights 8t .. 8t+7 of the sub-block
+          const uint4& qq = r.q[2 * ccl + (t >> 1)];
+          const uint32_t qa = (t & 1) ? qq.z : qq.x, qb = (t & 1) ? qq.w : qq.y;
+          const uint32_t na = hl ? ((qa >> 4) & 0x0f0f0f0fu) : (qa & 0x0f0f0f0fu);
+          const uint32_t nb = hl ? ((qb >> 4) & 0x0f0f0f0fu) : (qb & 0x0f0f0f0fu);
+          const half2_t a0 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, na, 0x04010400u)), s2, c2);   // (1024 + q) * sc - 1024 * sc = sc * q
+          const half2_t a1 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, na, 0x04030402u)), s2, c2);
+          const half2_t a2 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, nb, 0x04010400u)), s2, c2);
+          const half2_t a3 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, nb, 0x04030402u)), s2, c2);
+          A[rt][j][t] = half8_pf{a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+        }
       }
     }
-    __builtin_amdgcn_wave_barrier();
-    float4 d4[4], m4[4];
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-      d4[g] = *reinterpret_cast<const float4*>(&s_d[(wave * 2 + 0) * 32 + 8 * g + 4 * kg]);
-      m4[g] = *reinterpret_cast<const float4*>(&s_d[(wave * 2 + 1) * 32 + 8 * g + 4 * kg]);
-    }
-    __builtin_amdgcn_wave_barrier();
-    float16_t C[TT], Cm[TT];
+    float16_t C[RT][TT], Cm[RT][TT];
     const float16_t zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int j = 0; j < 4; j++)
@@ -232,43 +238,72 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
           const int off = (tt * 32 + n) * PF_LDX + 128 * kg + 32 * j + 8 * t;
           const half8_pf Bh = *reinterpret_cast<const half8_pf*>(xs_hi + off);
           const half8_pf Bl = *reinterpret_cast<const half8_pf*>(xs_lo + off);
-          if (j == 0 && t == 0) C[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[j][t], Bh, zero16, 0, 0, 0);   // a fresh accumulator per super-block
-          else C[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[j][t], Bh, C[tt], 0, 0, 0);
-          C[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[j][t], Bl, C[tt], 0, 0, 0);
+#pragma unroll
+          for (int rt = 0; rt < RT; rt++) {
+            if (j == 0 && t == 0) C[rt][tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[rt][j][t], Bh, zero16, 0, 0, 0);   // a fresh accumulator per super-block
+            else C[rt][tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[rt][j][t], Bh, C[rt][tt], 0, 0, 0);
+          }
+#pragma unroll
+          for (int rt = 0; rt < RT; rt++) C[rt][tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[rt][j][t], Bl, C[rt][tt], 0, 0, 0);
         }
+    __builtin_amdgcn_wave_barrier();       // s_d was written by this wave's own lanes above; LDS operations of a wave complete in order
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) {
       const half4_t Bmh = *reinterpret_cast<const half4_t*>(sx_hi + (tt * 32 + n) * 8 + 4 * kg);
       const half4_t Bml = *reinterpret_cast<const half4_t*>(sx_lo + (tt * 32 + n) * 8 + 4 * kg);
-      Cm[tt] = __builtin_amdgcn_mfma_f32_32x32x8f16(mnv, Bmh, zero16, 0, 0, 0);
-      Cm[tt] = __builtin_amdgcn_mfma_f32_32x32x8f16(mnv, Bml, Cm[tt], 0, 0, 0);
 #pragma unroll
-      for (int g = 0; g < 4; g++) {
-        Y[tt][4 * g + 0] += d4[g].x * C[tt][4 * g + 0] - m4[g].x * Cm[tt][4 * g + 0];
-        Y[tt][4 * g + 1] += d4[g].y * C[tt][4 * g + 1] - m4[g].y * Cm[tt][4 * g + 1];
-        Y[tt][4 * g + 2] += d4[g].z * C[tt][4 * g + 2] - m4[g].z * Cm[tt][4 * g + 2];
-        Y[tt][4 * g + 3] += d4[g].w * C[tt][4 * g + 3] - m4[g].w * Cm[tt][4 * g + 3];
+      for (int rt = 0; rt < RT; rt++) {
+        Cm[rt][tt] = __builtin_amdgcn_mfma_f32_32x32x8f16(mnv[rt], Bmh, zero16, 0, 0, 0);
+        Cm[rt][tt] = __builtin_amdgcn_mfma_f32_32x32x8f16(mnv[rt], Bml, Cm[rt][tt], 0, 0, 0);
       }
+#pragma unroll
+      for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const float4 d4 = *reinterpret_cast<const float4*>(&s_d[((wave * RT + rt) * 2 + 0) * 32 + 8 * g + 4 * kg]);
+          const float4 m4 = *reinterpret_cast<const float4*>(&s_d[((wave * RT + rt) * 2 + 1) * 32 + 8 * g + 4 * kg]);
+          Y[rt][tt][4 * g + 0] += d4.x * C[rt][tt][4 * g + 0] - m4.x * Cm[rt][tt][4 * g + 0];
+          Y[rt][tt][4 * g + 1] += d4.y * C[rt][tt][4 * g + 1] - m4.y * Cm[rt][tt][4 * g + 1];
+          Y[rt][tt][4 * g + 2] += d4.z * C[rt][tt][4 * g + 2] - m4.z * Cm[rt][tt][4 * g + 2];
+          Y[rt][tt][4 * g + 3] += d4.w * C[rt][tt][4 * g + 3] - m4.w * Cm[rt][tt][4 * g + 3];
+        }
     }
-    wcur = wnxt;
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) wcur[rt] = wnxt[rt];
   }
 
-  // ---- write: lane holds column (token) n of each tile and rows 8g + 4kg + (0..3) ----
+  // ---- write: lane holds column (token) n of each tile and rows 8g + 4kg + (0..3): four consecutive outputs of a token
+  // row go out as one 16-byte store (bias and residual come in the same way) when the addresses allow it ----
+  const bool vec = (p.y_stride & 3) == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 &&
+                   (!p.residual || (reinterpret_cast<uintptr_t>(p.residual) & 15) == 0) && (!p.bias || (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0);
 #pragma unroll
   for (int tt = 0; tt < TT; tt++) {
     const int t = T0 + tt * 32 + n;
     if (t >= p.n_tok) continue;
     const float si = p.sinv[t];
 #pragma unroll
-    for (int v = 0; v < 16; v++) {
-      const int row = R0 + 8 * (v >> 2) + 4 * kg + (v & 3);
-      if (row >= p.rows) continue;
-      const int64_t o = (int64_t)t * p.y_stride + row;
-      float r = Y[tt][v] * si;
-      if (p.bias) r += p.bias[row];
-      if (p.residual) r += p.residual[o];
-      p.y[o] = r;
-    }
+    for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const int row = R0 + 32 * rt + 8 * g + 4 * kg;
+        const int64_t o = (int64_t)t * p.y_stride + row;
+        if (vec && row + 3 < p.rows) {
+          float4 r = make_float4(Y[rt][tt][4 * g] * si, Y[rt][tt][4 * g + 1] * si, Y[rt][tt][4 * g + 2] * si, Y[rt][tt][4 * g + 3] * si);
+          if (p.bias) { const float4 b = *reinterpret_cast<const float4*>(p.bias + row); r.x += b.x; r.y += b.y; r.z += b.z; r.w += b.w; }
+          if (p.residual) { const float4 q = *reinterpret_cast<const float4*>(p.residual + o); r.x += q.x; r.y += q.y; r.z += q.z; r.w += q.w; }
+          *reinterpret_cast<float4*>(p.y + o) = r;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            if (row + i >= p.rows) continue;
+            float r = Y[rt][tt][4 * g + i] * si;
+            if (p.bias) r += p.bias[row + i];
+            if (p.residual) r += p.residual[o + i];
+            p.y[o + i] = r;
+          }
+        }
+      }
   }
 }
 
@@ -289,23 +324,28 @@ int launch_gemm_q4k(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo,
   p.w = w->data; p.bias = w->bias; p.rows = (int)w->rows; p.cols = (int)w->cols;
   p.xhi = xhi; p.xlo = xlo; p.sxhi = sxhi; p.sxlo = sxlo; p.sinv = sinv; p.n_tok = n_tok; p.y = y; p.y_stride = y_stride;
   p.residual = residual;
-  p.n_row_groups = (p.rows + 127) / 128;
-  // two token tiles per work-group reuse each weight operand four times; with few row groups one tile per work-group
-  // fills the chip better
-  static const int tt_force = []() { const char* e = getenv("CAIHIP_PF_TT"); return e ? atoi(e) : 0; }();
-  const int wgs2 = p.n_row_groups * ((n_tok + 63) / 64);
-  const int tt = tt_force == 1 || tt_force == 2 ? tt_force : (wgs2 < 2 * ctx().n_cu ? 1 : 2);
+  // Tiling: two row tiles per wave (256 rows per work-group, 32 tokens) when that still gives every CU several
+  // work-groups; else 128 rows with two token tiles, or with one for matrices with few row groups.
+  static const int tt_force = []() { const char* e = getenv("CAIHIP_PF_TT"); return e ? atoi(e) : 0; }();   // 1, 2: token tiles; 3: two row tiles
+  const int n_cu = ctx().n_cu;
+  const int wgs_rt2 = ((p.rows + 255) / 256) * ((n_tok + 31) / 32);
+  const int wgs_tt2 = ((p.rows + 127) / 128) * ((n_tok + 63) / 64);
+  int mode = wgs_rt2 >= 4 * n_cu ? 3 : (wgs_tt2 < 2 * n_cu ? 1 : 2);
+  if (tt_force >= 1 && tt_force <= 3) mode = tt_force;
+  const int rt = mode == 3 ? 2 : 1, tt = mode == 2 ? 2 : 1;
+  p.n_row_groups = (p.rows + 128 * rt - 1) / (128 * rt);
   p.n_tok_tiles = (n_tok + tt * 32 - 1) / (tt * 32);
-  const size_t lds = (size_t)tt * 32 * (PF_LDX + 8) * 2 * 2 + 4 * 2 * 32 * 4;
+  const size_t lds = (size_t)tt * 32 * (PF_LDX + 8) * 2 * 2 + (size_t)4 * rt * 2 * 32 * 4;
   static bool attr_done = false;
   if (!attr_done) {
-    (void)hipFuncSetAttribute((const void*)gemm_q4k_pf<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-    (void)hipFuncSetAttribute((const void*)gemm_q4k_pf<2>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    const void* ks[3] = {(const void*)gemm_q4k_pf<1, 1>, (const void*)gemm_q4k_pf<2, 1>, (const void*)gemm_q4k_pf<1, 2>};
+    for (const void* k : ks) if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) != hipSuccess) (void)hipGetLastError();
     attr_done = true;
   }
   const int grid = 8 * p.n_tok_tiles * ((p.n_row_groups + 7) / 8);
-  if (tt == 1) hipLaunchKernelGGL(gemm_q4k_pf<1>, dim3(grid), dim3(256), lds, ctx().stream, p);
-  else hipLaunchKernelGGL(gemm_q4k_pf<2>, dim3(grid), dim3(256), lds, ctx().stream, p);
+  if (mode == 3) hipLaunchKernelGGL((gemm_q4k_pf<1, 2>), dim3(grid), dim3(256), lds, ctx().stream, p);
+  else if (mode == 1) hipLaunchKernelGGL((gemm_q4k_pf<1, 1>), dim3(grid), dim3(256), lds, ctx().stream, p);
+  else hipLaunchKernelGGL((gemm_q4k_pf<2, 1>), dim3(grid), dim3(256), lds, ctx().stream, p);
   return CAI_OK;
 }
 
