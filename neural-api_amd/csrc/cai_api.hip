@@ -212,6 +212,17 @@ extern "C" int cai_qw_create(int qtype, int64_t rows, int64_t cols, const void* 
     if (e == hipSuccess) { launch_split_blocks((const uint8_t*)raw, bb, n_blocks, w->data, (uint16_t*)w->aux); e = hipStreamSynchronize(c.stream); }
     (void)hipFree(raw);
     if (e != hipSuccess) return fail(hip_fail(e, "cai_qw_create upload", __FILE__, __LINE__));
+  } else if (qtype == CAI_Q6_K) {
+    const int64_t n_blocks = rows * (cols / 256);
+    w->data_bytes = n_blocks * 192; w->aux_bytes = n_blocks * 18;
+    void* raw = nullptr;
+    if (hipMalloc(&raw, (size_t)raw_bytes) != hipSuccess) return fail(set_error(CAI_ERR_NOMEM, "cai_qw_create: out of device memory (%lld bytes staging)", (long long)raw_bytes));
+    hipError_t e = hipMalloc((void**)&w->data, (size_t)w->data_bytes);
+    if (e == hipSuccess) e = hipMalloc((void**)&w->aux, (size_t)w->aux_bytes);
+    if (e == hipSuccess) e = hipMemcpyAsync(raw, blocks, (size_t)raw_bytes, hipMemcpyDefault, c.stream);
+    if (e == hipSuccess) { launch_split_q6k((const uint8_t*)raw, n_blocks, w->data, w->aux, (uint16_t*)(w->aux + n_blocks * 16)); e = hipStreamSynchronize(c.stream); }
+    (void)hipFree(raw);
+    if (e != hipSuccess) return fail(hip_fail(e, "cai_qw_create upload", __FILE__, __LINE__));
   } else {
     w->data_bytes = raw_bytes;
     hipError_t e = hipMalloc((void**)&w->data, (size_t)raw_bytes);

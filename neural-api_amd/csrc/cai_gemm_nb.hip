@@ -30,7 +30,7 @@ constexpr int NB_SC = 16;        // staged columns: 8 tokens x {hi, lo}
 constexpr int NB_TK = 8;         // tokens per pass
 constexpr int NB_SMAX = 5;       // super-blocks per K slice at most (LDS: 8.6 KB each, and three work-groups share a CU)
 
-struct NbSeg { const uint8_t* w; const uint8_t* aux; const float* bias; const float* row_scale; int rows; int y_off; int tile_end; };   // aux: block scales plane (Q8_0 / Q4_0); row_scale: per-row int8 matrices; tile_end: cumulative 32-row tiles
+struct NbSeg { const uint8_t* w; const uint8_t* aux; const uint8_t* aux2; const float* bias; const float* row_scale; int rows; int y_off; int tile_end; };   // aux: block scales plane (Q8_0 / Q4_0 / Q6_K); aux2: Q6_K plane of d; row_scale: per-row int8 matrices; tile_end: cumulative 32-row tiles
 
 struct NbParams {
   NbSeg seg[3]; int n_seg;                      // up to three matrices of equal width share one launch (q | k | v)
@@ -473,10 +473,11 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
 // the codes 4 kg .. 4 kg + 3 of the group (q - 32, exact in f16) and multiplies the four results by d * scale, both values
 // it loaded itself.  Group g = 8 nh + 2 j + h of a super-block lies in bytes 16 (4 nh + 2 (j & 1) + h) .. + 15 of ql
 // (nibble j >> 1) and bytes 16 (2 nh + h) .. + 15 of qh (2-bit field j).  Lane kg loads the 16-byte chunks kg and kg + 4
-// of ql and chunk kg of qh (rows are only 2-byte aligned: the requests are issued unaligned), and a 4 x 4 transposition of
-// dwords over the kg lanes leaves dword kg of chunk c in register c.
+// of ql and chunk kg of qh, and a 4 x 4 transposition of dwords over the kg lanes leaves dword kg of chunk c in register
+// c.  Resident form: 192-byte ql | qh records, a plane of scales and a plane of d (the file's 210-byte blocks are only
+// 2-byte aligned, and unaligned requests stream at two thirds of the rate).
 // ------------------------------------------------------------------------------------------
-typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
 {
@@ -488,12 +489,12 @@ __global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
   const int n = lane & 15, kg = lane >> 4;
   const int K = p.cols, nsb = K >> 8;
   const int slice = blockIdx.y, sb0 = slice * S, nS = min(S, nsb - sb0);
-  const int64_t row_bytes = (int64_t)nsb * 210;
+  const int64_t row_bytes = (int64_t)nsb * 192;
   const int tile0 = blockIdx.x * 4 + wave;
   const int n_it = tile0 < p.n_tiles ? (p.n_tiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
   const int nq = n_it * nS;                      // (tile, super-block) items of this wave
 
-  struct WRegs { u32x4_a2 ql[2][2], qh[2], sc[2]; uint32_t d[2]; };
+  struct WRegs { u32x4_t ql[2][2], qh[2], sc[2]; uint32_t d[2]; };
   auto locate = [&](int tile, const NbSeg*& sg, int& R0) {
     int sgi = 0, t0 = 0;
     if (p.n_seg > 1 && tile >= p.seg[0].tile_end) { sgi = 1; t0 = p.seg[0].tile_end; }
@@ -507,12 +508,13 @@ __global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
     const NbSeg* sg; int R0; locate(tile, sg, R0);
 #pragma unroll
     for (int hh = 0; hh < 2; hh++) {
-      const uint8_t* blk = sg->w + (int64_t)min(R0 + 16 * hh + n, sg->rows - 1) * row_bytes + (int64_t)sb * 210;   // tail rows: re-read the last row
-      r.ql[hh][0] = *reinterpret_cast<const u32x4_a2*>(blk + 16 * kg);
-      r.ql[hh][1] = *reinterpret_cast<const u32x4_a2*>(blk + 64 + 16 * kg);
-      r.qh[hh] = *reinterpret_cast<const u32x4_a2*>(blk + 128 + 16 * kg);
-      r.sc[hh] = *reinterpret_cast<const u32x4_a2*>(blk + 192);
-      r.d[hh] = *reinterpret_cast<const uint16_t*>(blk + 208);
+      const int64_t b = (int64_t)min(R0 + 16 * hh + n, sg->rows - 1) * nsb + sb;   // tail rows: re-read the last row
+      const uint8_t* blk = sg->w + b * 192;
+      r.ql[hh][0] = *reinterpret_cast<const u32x4_t*>(blk + 16 * kg);
+      r.ql[hh][1] = *reinterpret_cast<const u32x4_t*>(blk + 64 + 16 * kg);
+      r.qh[hh] = *reinterpret_cast<const u32x4_t*>(blk + 128 + 16 * kg);
+      r.sc[hh] = *reinterpret_cast<const u32x4_t*>(sg->aux + b * 16);
+      r.d[hh] = *reinterpret_cast<const uint16_t*>(sg->aux2 + b * 2);
     }
   };
   WRegs wa, wb, wc;
@@ -566,7 +568,7 @@ __global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
       uint32_t lq[8], hq[4];
 #pragma unroll
       for (int a = 0; a < 3; a++) {
-        const u32x4_a2 v = a < 2 ? r.ql[hh][a] : r.qh[hh];
+        const u32x4_t v = a < 2 ? r.ql[hh][a] : r.qh[hh];
         const uint2_t t02 = __builtin_amdgcn_permlane32_swap(v.x, v.z, false, false);
         const uint2_t t13 = __builtin_amdgcn_permlane32_swap(v.y, v.w, false, false);
         const uint2_t u01 = __builtin_amdgcn_permlane16_swap(t02.x, t13.x, false, false);
@@ -892,7 +894,7 @@ int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok)
       return set_error(CAI_ERR_UNSUPPORTED, "small-batch gemm: matrix %d type %d width %lld", i, ws[i]->qtype, (long long)ws[i]->cols);
     if (i > 0 && y_off[i] < y_off[i - 1]) return set_error(CAI_ERR_INVALID, "small-batch gemm: output offsets must ascend");
     tiles += (int)((ws[i]->rows + 31) / 32);
-    segs[i] = NbSeg{ws[i]->data, ws[i]->aux, ws[i]->bias, ws[i]->qtype == CAI_I8ROW ? reinterpret_cast<const float*>(ws[i]->aux) : nullptr, (int)ws[i]->rows, y_off[i], 0};
+    segs[i] = NbSeg{ws[i]->data, ws[i]->aux, qw_aux2(ws[i]), ws[i]->bias, ws[i]->qtype == CAI_I8ROW ? reinterpret_cast<const float*>(ws[i]->aux) : nullptr, (int)ws[i]->rows, y_off[i], 0};
     width = std::max(width, y_off[i] + (int)ws[i]->rows);
   }
   int S, n_slices, gx, tile_stride;

@@ -21,10 +21,9 @@ template <> struct QTraits<CAI_Q8_0> { static constexpr int UW = 16, T = 4; };
 template <> struct QTraits<CAI_I8ROW> { static constexpr int UW = 16, T = 4; };   // per-row int8: the Q8_0 walk with one scale per row, applied at the end
 // Q6_K: 16 lanes per 210-byte super-block.  Lane t (half nh = t>>3, byte position l4 = 4*(t&7)) takes four bytes each of the
 // two ql runs and of the qh run of its half, i.e. the 16 weights 128*nh + 32*j + l4 + {0..3}, j = 0..3, which fall in four
-// different 16-weight scale groups (neural/neuralgguf.pas:639-717).  Blocks are only 2-byte aligned in a row; the dword
-// requests are issued unaligned.
+// different 16-weight scale groups (neural/neuralgguf.pas:639-717).  Resident form: 192-byte ql | qh records, a plane of
+// scales (16 per block) and a plane of d, all aligned.
 template <> struct QTraits<CAI_Q6_K> { static constexpr int UW = 16, T = 4; };
-typedef uint32_t __attribute__((aligned(2))) u32_a2;
 
 // original float4 index n (within the panel) -> LDS float4 slot, unit-transposed in tiles of 16 units
 template <int QT> __device__ __forceinline__ int lds_slot(int n)
@@ -86,12 +85,12 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
   const int cols = p.cols;
   int64_t row_bytes, aux_row_bytes = 0;
   if (QT == CAI_Q4_K) row_bytes = (int64_t)(cols >> 8) * 144;
-  else if (QT == CAI_Q6_K) row_bytes = (int64_t)(cols >> 8) * 210;
+  else if (QT == CAI_Q6_K) { row_bytes = (int64_t)(cols >> 8) * 192; aux_row_bytes = (cols >> 8) * 16; }
   else if (QT == CAI_Q4_0) { row_bytes = cols >> 1; aux_row_bytes = (cols >> 5) * 2; }
   else if (QT == CAI_I8ROW) row_bytes = cols;
   else { row_bytes = cols; aux_row_bytes = (cols >> 5) * 2; }
 
-  const uint8_t* rp[RR]; const uint8_t* ap[RR]; bool live[RR];
+  const uint8_t* rp[RR]; const uint8_t* ap[RR]; const uint8_t* dp[RR]; bool live[RR];
 #pragma unroll
   for (int r = 0; r < RR; r++) {
     int row = row_first + (MODE == 1 ? (r >> 1) : r);
@@ -100,6 +99,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
     if (MODE == 1 && (r & 1)) row += p.half;
     rp[r] = sg.data + (bank_row + row) * row_bytes;
     ap[r] = sg.aux + (bank_row + row) * aux_row_bytes;
+    dp[r] = QT == CAI_Q6_K ? sg.aux2 + (bank_row + row) * (int64_t)(cols >> 8) * 2 : nullptr;
   }
 
   float acc[RR][NB];
@@ -184,13 +184,13 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
         const int sb = (k0 >> 8) + (u >> 4), nh = (u >> 3) & 1, l4 = (u & 7) * 4;
 #pragma unroll
         for (int r = 0; r < RR; r++) {
-          const uint8_t* blk = rp[r] + (int64_t)sb * 210;
-          q[r].x = *reinterpret_cast<const u32_a2*>(blk + 64 * nh + l4);
-          q[r].y = *reinterpret_cast<const u32_a2*>(blk + 64 * nh + 32 + l4);
-          q[r].z = *reinterpret_cast<const u32_a2*>(blk + 128 + 32 * nh + l4); q[r].w = 0u;
-          hdr[r].x = *reinterpret_cast<const u32_a2*>(blk + 192 + 8 * nh);
-          hdr[r].y = *reinterpret_cast<const u32_a2*>(blk + 196 + 8 * nh);
-          dh[r] = *reinterpret_cast<const uint16_t*>(blk + 208);
+          const uint8_t* blk = rp[r] + (int64_t)sb * 192;
+          q[r].x = *reinterpret_cast<const uint32_t*>(blk + 64 * nh + l4);
+          q[r].y = *reinterpret_cast<const uint32_t*>(blk + 64 * nh + 32 + l4);
+          q[r].z = *reinterpret_cast<const uint32_t*>(blk + 128 + 32 * nh + l4); q[r].w = 0u;
+          const uint2 sc2 = *reinterpret_cast<const uint2*>(ap[r] + sb * 16 + 8 * nh);
+          hdr[r].x = sc2.x; hdr[r].y = sc2.y;
+          dh[r] = *reinterpret_cast<const uint16_t*>(dp[r] + sb * 2);
         }
       } else if (QT == CAI_Q4_0) {
         const int blk = (k0 >> 5) + u;
@@ -571,7 +571,7 @@ static int64_t data_row_bytes(const cai_qw_s* w)
 {
   switch (w->qtype) {
     case CAI_Q4_K: return w->cols / 256 * 144;
-    case CAI_Q6_K: return w->cols / 256 * 210;
+    case CAI_Q6_K: return w->cols / 256 * 192;
     case CAI_Q4_0: return w->cols / 2;
     case CAI_Q8_0: case CAI_I8ROW: return w->cols;
     case CAI_F32: return w->cols * 4;
@@ -583,6 +583,7 @@ static int64_t aux_row_bytes(const cai_qw_s* w)
 {
   if (w->qtype == CAI_Q4_0 || w->qtype == CAI_Q8_0) return w->cols / 32 * 2;
   if (w->qtype == CAI_I8ROW) return 4;
+  if (w->qtype == CAI_Q6_K) return w->cols / 256 * 16;
   return 0;
 }
 
@@ -605,6 +606,7 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
       return set_error(CAI_ERR_INVALID, "gemv: row range [%lld,+%lld) outside matrix of %lld rows", (long long)m.row0[i], (long long)m.rows[i], (long long)w->rows);
     p.seg[i].data = w->data + m.row0[i] * data_row_bytes(w);
     p.seg[i].aux = w->aux ? w->aux + m.row0[i] * aux_row_bytes(w) : nullptr;
+    p.seg[i].aux2 = w->qtype == CAI_Q6_K ? qw_aux2(w) + m.row0[i] * (w->cols / 256) * 2 : nullptr;
     p.seg[i].bias = w->bias ? w->bias + m.row0[i] : nullptr;
     p.seg[i].rows = (int)m.rows[i];
     p.seg[i].y_off = m.y_off[i];

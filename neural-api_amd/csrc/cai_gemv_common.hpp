@@ -45,7 +45,7 @@ __device__ __forceinline__ float silu_mul(float up, float gate)
 constexpr int SSQ_PARTS = 1024;   // slots of a sum-of-squares partial array (>= any producer grid)
 
 struct GemvSeg {
-  const uint8_t* data; const uint8_t* aux; const float* bias;
+  const uint8_t* data; const uint8_t* aux; const uint8_t* aux2; const float* bias;   // aux2: Q6_K plane of d
   int rows;       // rows of this segment computed by the launch
   int y_off;      // offset of the segment's first output inside a y row
   int grp_end;    // cumulative row-group count (exclusive)

@@ -99,11 +99,14 @@ struct cai_qw_s {
   int      qtype = 0;
   int64_t  rows = 0, cols = 0;
   uint8_t* data = nullptr;     // quants plane or the raw blocks
-  uint8_t* aux = nullptr;      // half scales plane (Q8_0/Q4_0) or float row scales (I8ROW)
+  uint8_t* aux = nullptr;      // half scales plane (Q8_0/Q4_0), float row scales (I8ROW), or for Q6_K the int8 scales plane (16 per block) followed by the plane of d
   float*   bias = nullptr;
   int64_t  data_bytes = 0, aux_bytes = 0;
   int64_t  algo_bytes = 0;     // bytes of the GGUF form (+bias): what one GEMV must stream
 };
+
+// Q6_K: start of the d plane (behind 16 scale bytes per block); null for the other types
+inline const uint8_t* qw_aux2(const cai_qw_s* w) { return w->qtype == CAI_Q6_K ? w->aux + w->rows * (w->cols >> 8) * 16 : nullptr; }
 
 struct cai_kv_s {
   int n_seq = 1, n_layers = 0, kv_heads = 0, head_dim = 0, max_ctx = 0, dtype = 0;
@@ -167,6 +170,7 @@ void decoder_adopt_weight(cai_decoder_s* d, cai_qw_s* w);   // the decoder destr
 int launch_rmsnorm_pair(float* x, const float* gain_a, int n_a, const float* gain_b, int n_b, int n_tokens, float eps, int64_t stride);
 int launch_moe_combine(float* x, const float* part, const float* gate, int k, int n, int n_tokens);
 int launch_split_blocks(const uint8_t* raw, int block_bytes, int64_t n_blocks, uint8_t* qs, uint16_t* d);
+int launch_split_q6k(const uint8_t* raw, int64_t n_blocks, uint8_t* rec, uint8_t* sc, uint16_t* d);
 // qkv: [n_seq][qkv_stride] rows [Q|K|V]; theta != null applies interleaved RoPE to Q and K first.  pos_dev[s] is
 // both the rotary position and the cache slot the new K,V row goes to; the live range is [.., pos_dev[s]].
 // Activation row s uses cache sequence seq0 + s.  prompt_rows != 0: the n_seq rows are consecutive tokens of ONE
