@@ -32,7 +32,7 @@ extern "C" {
 #define CAI_Q4_0   2
 #define CAI_Q8_0   8
 #define CAI_Q4_K   12
-#define CAI_Q6_K   14  /* 210-byte super-blocks (neural/neuralgguf.pas:639-717); functional path, not bandwidth-tuned */
+#define CAI_Q6_K   14  /* 210-byte super-blocks (neural/neuralgguf.pas:639-717); resident as aligned ql|qh records + planes of scales and d */
 #define CAI_I8ROW  100  /* per-row symmetric int8 + fp32 row scale (neural/neuralvolume.pas:926-987) */
 
 /* ---- activation opcodes fused into the linear layer (neural/neural.cl:114-146) ---- */
