@@ -21,6 +21,9 @@ CONFIGS = {
     # BASELINE.json configs[2]: Qwen2.5-7B shape, Q4_K body, Q8_0 untied head, QKV bias
     "qwen2.5-7b-q4k": dict(cfg=dict(n_layers=28, d_model=3584, n_q_heads=28, n_kv_heads=4, head_dim=128, ffn=18944, vocab=152064,
                                     max_ctx=768, eps=1e-6, rope_theta=1e6), qtype="Q4_K", head="Q8_0", bias=True, prompt=512),
+    # the same shape as llama.cpp's Q4_K_M preset writes it: output.weight and attn_v / ffn_down of about half the blocks in Q6_K
+    "qwen2.5-7b-q4_k_m": dict(cfg=dict(n_layers=28, d_model=3584, n_q_heads=28, n_kv_heads=4, head_dim=128, ffn=18944, vocab=152064,
+                                       max_ctx=768, eps=1e-6, rope_theta=1e6), qtype="Q4_K", head="Q6_K", embed="Q4_K", q6k_mix=True, bias=True, prompt=512),
     # BASELINE.json configs[0] (the reference's own CPU-runnable case): SmolLM2-135M shape, Q8_0, tied head
     "smollm2-135m-q8_0": dict(cfg=dict(n_layers=30, d_model=576, n_q_heads=9, n_kv_heads=3, head_dim=64, ffn=1536, vocab=49152,
                                        max_ctx=256, eps=1e-5, rope_theta=1e5, tied=True), qtype="Q8_0", head="Q8_0", bias=False, prompt=16),
@@ -177,9 +180,10 @@ def main():
     K, W = args.steps, args.warmup
     if prompt_len + W + K > cfg["max_ctx"]:
         cfg["max_ctx"] = prompt_len + W + K
-    QT = {"Q4_K": cai.Q4_K, "Q8_0": cai.Q8_0, "Q4_0": cai.Q4_0}
+    QT = {"Q4_K": cai.Q4_K, "Q8_0": cai.Q8_0, "Q4_0": cai.Q4_0, "Q6_K": cai.Q6_K}
     t0 = time.time()
-    spec = synth.random_decoder_spec(cfg, QT[conf["qtype"]], QT[conf["head"]], seed=424242, qkv_bias=conf["bias"])
+    spec = synth.random_decoder_spec(cfg, QT[conf["qtype"]], QT[conf["head"]], seed=424242, qkv_bias=conf["bias"],
+                                     embed_qtype=QT[conf["embed"]] if "embed" in conf else None, q6k_mix=conf.get("q6k_mix", False))
     B = args.batch
     kv_kind = args.kv or conf.get("kv", "f32")
     dec = cai.Decoder(spec, max_batch=B, kv_dtype={"f32": cai.KV_F32, "f16": cai.KV_F16, "i8": cai.KV_I8}[kv_kind])

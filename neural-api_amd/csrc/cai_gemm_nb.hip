@@ -27,7 +27,8 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 
 constexpr int NB_LDX = 264;      // halfs per staged activation column: 256 + pad (stride = 4 banks mod 64: 16-byte reads of 16 columns tile the banks)
 constexpr int NB_SC = 16;        // staged columns: 8 tokens x {hi, lo}
-constexpr int NB_TK = 8;         // tokens per pass
+constexpr int NB_TK = 8;         // tokens per matrix-core group (8 hi + 8 lo = the 16 rows of an MFMA operand) and per pass of most kernels
+constexpr int NB_TMAX = 32;      // tokens per pass at most (the Q6_K kernel takes four groups); the workspace holds this many
 constexpr int NB_SMAX = 5;       // super-blocks per K slice at most (LDS: 8.6 KB each, and three work-groups share a CU)
 
 struct NbSeg { const uint8_t* w; const uint8_t* aux; const uint8_t* aux2; const float* bias; const float* row_scale; int rows; int y_off; int tile_end; };   // aux: block scales plane (Q8_0 / Q4_0 / Q6_K); aux2: Q6_K plane of d; row_scale: per-row int8 matrices; tile_end: cumulative 32-row tiles
@@ -479,12 +480,15 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
 // ------------------------------------------------------------------------------------------
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
+// NT groups of 8 tokens share every converted weight operand and scale: prompts take 32 tokens per pass (NT = 4).
+template <int NT>
 __global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
 {
   extern __shared__ __align__(16) unsigned char nb_smem[];
   const int S = p.sb_per_slice;
-  _Float16* xs = reinterpret_cast<_Float16*>(nb_smem);              // [S][16][NB_LDX]
-  float* sinv_s = reinterpret_cast<float*>(xs + S * NB_SC * NB_LDX);  // [S][8]
+  constexpr int NC = NT * NB_SC, NTOK = NT * NB_TK;                 // staged columns per super-block: group t holds tokens 8t..8t+7 as 8 hi + 8 lo
+  _Float16* xs = reinterpret_cast<_Float16*>(nb_smem);              // [S][NC][NB_LDX]
+  float* sinv_s = reinterpret_cast<float*>(xs + S * NC * NB_LDX);    // [S][NTOK]
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 15, kg = lane >> 4;
   const int K = p.cols, nsb = K >> 8;
@@ -522,48 +526,55 @@ __global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
 
   // ---- stage this slice of the activations: nS x 16 columns x 256 halfs, block scales (four requests per turn) ----
   {
-    const int n_si = nS * NB_TK;
-    const int si_i = min((int)threadIdx.x, n_si - 1), si_tok = si_i % NB_TK, si_s = si_i / NB_TK;
-    const float siv = p.sinvb[(int64_t)min(si_tok, p.n_tok - 1) * nsb + sb0 + si_s];
-    const int total = nS * NB_SC * 32;
+    const int n_si = nS * NTOK;
+    const int total = nS * NC * 32;
     for (int base = 0; base < total; base += 4 * 256) {
       uint4 v[4];
 #pragma unroll
       for (int u = 0; u < 4; u++) {
         const int idx = min(base + u * 256 + (int)threadIdx.x, total - 1);
-        const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC, tok = min(col % NB_TK, p.n_tok - 1);
-        v[u] = *reinterpret_cast<const uint4*>(((col / NB_TK) ? p.xlo : p.xhi) + (int64_t)tok * K + (sb0 + s) * 256 + chunk * 8);
+        const int chunk = idx & 31, col = (idx >> 5) % NC, s = (idx >> 5) / NC;
+        const int tok = min((col / NB_SC) * NB_TK + col % NB_TK, p.n_tok - 1);
+        v[u] = *reinterpret_cast<const uint4*>((((col % NB_SC) / NB_TK) ? p.xlo : p.xhi) + (int64_t)tok * K + (sb0 + s) * 256 + chunk * 8);
       }
 #pragma unroll
       for (int u = 0; u < 4; u++) {
         const int idx = base + u * 256 + (int)threadIdx.x;
         if (idx < total) {
-          const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC;
-          *reinterpret_cast<uint4*>(xs + (s * NB_SC + col) * NB_LDX + chunk * 8) = (col % NB_TK) < p.n_tok ? v[u] : make_uint4(0, 0, 0, 0);
+          const int chunk = idx & 31, col = (idx >> 5) % NC, s = (idx >> 5) / NC;
+          const int tok = (col / NB_SC) * NB_TK + col % NB_TK;
+          *reinterpret_cast<uint4*>(xs + (s * NC + col) * NB_LDX + chunk * 8) = tok < p.n_tok ? v[u] : make_uint4(0, 0, 0, 0);
         }
       }
     }
-    if ((int)threadIdx.x < n_si) sinv_s[si_i] = si_tok < p.n_tok ? siv : 0.0f;
+    for (int i = threadIdx.x; i < n_si; i += 256) {
+      const int tok = i % NTOK, s = i / NTOK;
+      sinv_s[i] = tok < p.n_tok ? p.sinvb[(int64_t)tok * nsb + sb0 + s] : 0.0f;
+    }
   }
   __syncthreads();
 
-  float acc[2][4];
+  float acc[NT][2][4];
   auto compute = [&](const WRegs& r, int q) {
     const int s = q % nS;
     if (s == 0) {
 #pragma unroll
-      for (int hh = 0; hh < 2; hh++)
+      for (int t = 0; t < NT; t++)
 #pragma unroll
-        for (int i = 0; i < 4; i++) acc[hh][i] = 0.0f;
+        for (int hh = 0; hh < 2; hh++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) acc[t][hh][i] = 0.0f;
     }
-    const _Float16* xcol = xs + (s * NB_SC + n) * NB_LDX + 4 * kg;
+    const _Float16* xcol = xs + (s * NC + n) * NB_LDX + 4 * kg;
     const float4_t z4 = {0.0f, 0.0f, 0.0f, 0.0f};
     const half2_t o2 = {(_Float16)(-1056.0f), (_Float16)(-1056.0f)};   // 1024 + q - 1056 = q - 32
-    float g[2][4];
 #pragma unroll
     for (int hh = 0; hh < 2; hh++) {
+      float g[NT][4];
 #pragma unroll
-      for (int i = 0; i < 4; i++) g[hh][i] = 0.0f;
+      for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) g[t][i] = 0.0f;
       // dword kg of every chunk: ql chunks 0..7 in lq[0..7], qh chunks 0..3 in hq[0..3]
       uint32_t lq[8], hq[4];
 #pragma unroll
@@ -588,35 +599,40 @@ __global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
         const half2_t w01 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, c, 0x04010400u)) + o2;
         const half2_t w23 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, c, 0x04030402u)) + o2;
         const half4_t W = {w01.x, w01.y, w23.x, w23.y};
-        const half4_t X = *reinterpret_cast<const half4_t*>(xcol + 16 * gi);
-        const float4_t C = __builtin_amdgcn_mfma_f32_16x16x16f16(X, W, z4, 0, 0, 0);
         const float ds = d * (float)(int)(int8_t)((scw[gi >> 2] >> (8 * (gi & 3))) & 0xffu);
 #pragma unroll
-        for (int i = 0; i < 4; i++) g[hh][i] = fmaf(ds, C[i], g[hh][i]);
-      }
-    }
-    // result row 4 kg + i of the tile = token (4 kg + i) % 8, its hi (kg < 2) or lo (kg >= 2) part
-    const float4 si = *reinterpret_cast<const float4*>(&sinv_s[s * NB_TK + 4 * (kg & 1)]);
+        for (int t = 0; t < NT; t++) {
+          const half4_t X = *reinterpret_cast<const half4_t*>(xcol + t * NB_SC * NB_LDX + 16 * gi);
+          const float4_t C = __builtin_amdgcn_mfma_f32_16x16x16f16(X, W, z4, 0, 0, 0);
 #pragma unroll
-    for (int hh = 0; hh < 2; hh++) {
-      acc[hh][0] = fmaf(si.x, g[hh][0], acc[hh][0]); acc[hh][1] = fmaf(si.y, g[hh][1], acc[hh][1]);
-      acc[hh][2] = fmaf(si.z, g[hh][2], acc[hh][2]); acc[hh][3] = fmaf(si.w, g[hh][3], acc[hh][3]);
+          for (int i = 0; i < 4; i++) g[t][i] = fmaf(ds, C[i], g[t][i]);
+        }
+      }
+      // result row 4 kg + i of a group = token (4 kg + i) % 8 of the group, its hi (kg < 2) or lo (kg >= 2) part
+#pragma unroll
+      for (int t = 0; t < NT; t++) {
+        const float4 si = *reinterpret_cast<const float4*>(&sinv_s[s * NTOK + t * NB_TK + 4 * (kg & 1)]);
+        acc[t][hh][0] = fmaf(si.x, g[t][0], acc[t][hh][0]); acc[t][hh][1] = fmaf(si.y, g[t][1], acc[t][hh][1]);
+        acc[t][hh][2] = fmaf(si.z, g[t][2], acc[t][hh][2]); acc[t][hh][3] = fmaf(si.w, g[t][3], acc[t][hh][3]);
+      }
     }
     if (s != nS - 1) return;
     // ---- the slice's contribution of this tile: hi + lo parts meet across kg ^ 2; lanes kg < 2 store four tokens ----
     const int tile = tile0 + (q / nS) * p.tile_stride;
     const NbSeg* sg; int R0; locate(tile, sg, R0);
 #pragma unroll
-    for (int hh = 0; hh < 2; hh++) {
-      const int row = R0 + 16 * hh + n;
+    for (int t = 0; t < NT; t++)
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const float tot = acc[hh][i] + __shfl_xor(acc[hh][i], 32, 64);
-        const int tok = 4 * kg + i;
-        if (kg < 2 && tok < p.n_tok && row < sg->rows)
-          p.part[((int64_t)slice * p.n_tok + tok) * p.part_stride + sg->y_off + row] = tot;
+      for (int hh = 0; hh < 2; hh++) {
+        const int row = R0 + 16 * hh + n;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const float tot = acc[t][hh][i] + __shfl_xor(acc[t][hh][i], 32, 64);
+          const int tok = t * NB_TK + 4 * kg + i;
+          if (kg < 2 && tok < p.n_tok && row < sg->rows)
+            p.part[((int64_t)slice * p.n_tok + tok) * p.part_stride + sg->y_off + row] = tot;
+        }
       }
-    }
   };
 
   for (int q = 0; q < nq; q += 3) {
@@ -771,14 +787,14 @@ int nb_ws_generation() { return g_nb.generation; }
 // Reserves planes for k_max columns and a partial buffer of part_floats floats (never inside a stream capture).
 int nb_reserve(int k_max, size_t part_floats)
 {
-  const size_t need_k = (size_t)NB_TK * k_max;
+  const size_t need_k = (size_t)NB_TMAX * k_max;
   if (need_k > g_nb.cap_k) {
     CAI_HIP(hipStreamSynchronize(ctx().stream));
     void* old[] = {g_nb.hi, g_nb.lo, g_nb.sxhi, g_nb.sxlo, g_nb.sinvb, g_nb.ssq[0], g_nb.ssq[1]};
     for (void* q : old) if (q) (void)hipFree(q);
     CAI_HIP(hipMalloc((void**)&g_nb.hi, need_k * 2)); CAI_HIP(hipMalloc((void**)&g_nb.lo, need_k * 2));
     CAI_HIP(hipMalloc((void**)&g_nb.sxhi, need_k / 32 * 2 + 64)); CAI_HIP(hipMalloc((void**)&g_nb.sxlo, need_k / 32 * 2 + 64));
-    const size_t nblk = (size_t)NB_TK * ((k_max + 255) / 256);
+    const size_t nblk = (size_t)NB_TMAX * ((k_max + 255) / 256);
     CAI_HIP(hipMalloc((void**)&g_nb.sinvb, nblk * 4 + 64));
     CAI_HIP(hipMalloc((void**)&g_nb.ssq[0], nblk * 4 + 64)); CAI_HIP(hipMalloc((void**)&g_nb.ssq[1], nblk * 4 + 64));
     g_nb.cap_k = need_k; g_nb.generation++;
@@ -796,11 +812,11 @@ int nb_reserve(int k_max, size_t part_floats)
 // that gx * slices work-groups fit the chip in ONE round (three work-groups share a CU) and the waves' shares come out
 // even.  A wave's share is ceil(tiles / (4 gx)) tiles of S items each (item = 32 rows x one super-block) plus the
 // partial result every (tile, slice) writes and its consumer re-reads, priced at 0.45 item.
-static void nb_geometry(int cols, int tiles, int& S, int& n_slices, int& gx, int& tile_stride)
+static void nb_geometry(int cols, int tiles, int& S, int& n_slices, int& gx, int& tile_stride, int s_max = NB_SMAX)
 {
   const int nsb = (cols + 255) >> 8, slots = 3 * ctx().n_cu;
   static const int force = []() { const char* e = getenv("CAIHIP_NB_S"); return e ? atoi(e) : 0; }();
-  const int s_lo = std::min(2, nsb), s_hi = std::min(NB_SMAX, nsb);
+  const int s_lo = std::min(2, nsb), s_hi = std::min(s_max, nsb);
   float best = 3.0e38f;
   S = s_lo;
   for (int s = s_lo; s <= s_hi; s++) {
@@ -819,7 +835,7 @@ int nb_max_slices(int cols) { const int nsb = std::max((cols + 255) >> 8, 1); co
 static int nb_prep_launch(int src, NbPrepParams& p, int n_tok)
 {
   if (p.K % 32) return set_error(CAI_ERR_UNSUPPORTED, "small-batch pre-pass: width %d is not a multiple of 32", p.K);
-  if ((size_t)NB_TK * p.K > g_nb.cap_k || n_tok > NB_TK) return set_error(CAI_ERR_STATE, "small-batch pre-pass: workspace not reserved for %d x %d", n_tok, p.K);
+  if ((size_t)NB_TMAX * p.K > g_nb.cap_k || n_tok > NB_TMAX) return set_error(CAI_ERR_STATE, "small-batch pre-pass: workspace not reserved for %d x %d", n_tok, p.K);
   g_nb.cur ^= 1;
   p.hi = g_nb.hi; p.lo = g_nb.lo; p.sxhi = g_nb.sxhi; p.sxlo = g_nb.sxlo; p.sinvb = g_nb.sinvb; p.ssq = g_nb.ssq[g_nb.cur];
   const dim3 grid((p.K + 255) >> 8, n_tok);
@@ -880,27 +896,29 @@ static void nb_launch(const NbParams& p, int gx, int n_slices, size_t lds)
   hipLaunchKernelGGL(Kernel, dim3(gx, n_slices), dim3(256), lds, ctx().stream, p);
 }
 
+int nb_pass_tokens(const cai_qw_s* w);
+
 // partials <- [W0; W1; W2] . planes.  The matrices share the width; those of one type share a launch (a Q4_K_M file keeps
 // attn_v of some blocks in Q6_K beside Q4_K attn_q and attn_k), and every launch cuts the columns into the same slices.
 int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok)
 {
-  if (n_w < 1 || n_w > 3 || n_tok < 1 || n_tok > NB_TK) return set_error(CAI_ERR_UNSUPPORTED, "small-batch gemm: %d matrices, %d tokens", n_w, n_tok);
+  if (n_w < 1 || n_w > 3 || n_tok < 1 || n_tok > nb_pass_tokens(ws[0])) return set_error(CAI_ERR_UNSUPPORTED, "small-batch gemm: %d matrices, %d tokens", n_w, n_tok);
   NbParams base{};
   base.cols = (int)ws[0]->cols;
   NbSeg segs[3];
   int tiles = 0, width = 0;
   for (int i = 0; i < n_w; i++) {
-    if (!nb_supported(ws[i]) || ws[i]->cols != ws[0]->cols)
-      return set_error(CAI_ERR_UNSUPPORTED, "small-batch gemm: matrix %d type %d width %lld", i, ws[i]->qtype, (long long)ws[i]->cols);
+    if (!nb_supported(ws[i]) || ws[i]->cols != ws[0]->cols || n_tok > nb_pass_tokens(ws[i]))
+      return set_error(CAI_ERR_UNSUPPORTED, "small-batch gemm: matrix %d type %d width %lld, %d tokens", i, ws[i]->qtype, (long long)ws[i]->cols, n_tok);
     if (i > 0 && y_off[i] < y_off[i - 1]) return set_error(CAI_ERR_INVALID, "small-batch gemm: output offsets must ascend");
     tiles += (int)((ws[i]->rows + 31) / 32);
     segs[i] = NbSeg{ws[i]->data, ws[i]->aux, qw_aux2(ws[i]), ws[i]->bias, ws[i]->qtype == CAI_I8ROW ? reinterpret_cast<const float*>(ws[i]->aux) : nullptr, (int)ws[i]->rows, y_off[i], 0};
     width = std::max(width, y_off[i] + (int)ws[i]->rows);
   }
   int S, n_slices, gx, tile_stride;
-  nb_geometry(base.cols, tiles, S, n_slices, gx, tile_stride);
+  nb_geometry(base.cols, tiles, S, n_slices, gx, tile_stride, n_tok > NB_TK ? 2 : NB_SMAX);
   const int64_t stride = (width + 3) / 4 * 4;
-  if ((size_t)NB_TK * base.cols > g_nb.cap_k || (size_t)n_slices * n_tok * stride > g_nb.cap_part)
+  if ((size_t)NB_TMAX * base.cols > g_nb.cap_k || (size_t)n_slices * n_tok * stride > g_nb.cap_part)
     return set_error(CAI_ERR_STATE, "small-batch gemm: workspace not reserved (%d slices x %d tokens x %lld)", n_slices, n_tok, (long long)stride);
   base.xhi = g_nb.hi; base.xlo = g_nb.lo; base.sxhi = g_nb.sxhi; base.sxlo = g_nb.sxlo; base.sinvb = g_nb.sinvb; base.n_tok = n_tok;
   base.part = g_nb.part; base.part_stride = stride; base.sb_per_slice = S;
@@ -925,7 +943,9 @@ int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok)
     } else {
       const size_t lds = (size_t)S * NB_SC * NB_LDX * 2 + (size_t)S * NB_TK * 4;
       const bool tail = p.cols % 256 != 0;
-      if (qt == CAI_Q6_K) nb_launch<gemm_q6k_nb>(p, gxs, n_slices, lds);
+      if (qt == CAI_Q6_K && n_tok > 2 * NB_TK) nb_launch<gemm_q6k_nb<4>>(p, gxs, n_slices, 4 * lds);
+      else if (qt == CAI_Q6_K && n_tok > NB_TK) nb_launch<gemm_q6k_nb<2>>(p, gxs, n_slices, 2 * lds);
+      else if (qt == CAI_Q6_K) nb_launch<gemm_q6k_nb<1>>(p, gxs, n_slices, lds);
       else if (qt == CAI_Q8_0) { if (tail) nb_launch<gemm_blk_nb<CAI_Q8_0, true>>(p, gxs, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_Q8_0, false>>(p, gxs, n_slices, lds); }
       else if (qt == CAI_I8ROW) { if (tail) nb_launch<gemm_blk_nb<CAI_I8ROW, true>>(p, gxs, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_I8ROW, false>>(p, gxs, n_slices, lds); }
       else { if (tail) nb_launch<gemm_blk_nb<CAI_Q4_0, true>>(p, gxs, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_Q4_0, false>>(p, gxs, n_slices, lds); }
@@ -951,13 +971,21 @@ int nb_reduce(float* y, int64_t y_stride, const float* residual)
   return CAI_OK;
 }
 
+// Tokens one pass of nb_prep / nb_gemm / nb_reduce takes for this weight type
+int nb_pass_tokens(const cai_qw_s* w)
+{
+  static const int q6 = []() { const char* e = getenv("CAIHIP_NB_Q6K_PASS"); const int v = e ? atoi(e) : 16; return v == 8 || v == 16 || v == 32 ? v : 16; }();
+  return w->qtype == CAI_Q6_K ? q6 : NB_TK;
+}
+
 // Whole linear layer, 8 tokens per pass (the weights are streamed once per pass): y = W (gain . x / rms) + bias (+ residual)
 int nb_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok, float* y, int64_t y_stride, const float* residual)
 {
   int rc;
-  if ((rc = nb_reserve((int)w->cols, (size_t)nb_max_slices((int)w->cols) * NB_TK * ((w->rows + 3) / 4 * 4)))) return rc;
-  for (int t0 = 0; t0 < n_tok; t0 += NB_TK) {
-    const int nt = std::min(NB_TK, n_tok - t0); const int zero = 0;
+  const int pass = nb_pass_tokens(w);
+  if ((rc = nb_reserve((int)w->cols, (size_t)nb_max_slices((int)w->cols) * pass * ((w->rows + 3) / 4 * 4)))) return rc;
+  for (int t0 = 0; t0 < n_tok; t0 += pass) {
+    const int nt = std::min(pass, n_tok - t0); const int zero = 0;
     if ((rc = nb_prep_plain(x + (int64_t)t0 * x_stride, x_stride, gain, eps, (int)w->cols, nt))) return rc;
     if ((rc = nb_gemm(&w, &zero, 1, nt))) return rc;
     if ((rc = nb_reduce(y + (int64_t)t0 * y_stride, y_stride, residual ? residual + (int64_t)t0 * y_stride : nullptr))) return rc;

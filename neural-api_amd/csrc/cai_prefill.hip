@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) void xprep_kernel(const float* x, int64_t x_st
 }
 
 struct GemmParams {
-  const uint8_t* w; const float* bias;
+  const uint8_t* w; const uint8_t* aux; const uint8_t* aux2; const float* bias;   // aux, aux2: Q6_K planes of scales and of d
   int rows, cols;
   const _Float16* xhi; const _Float16* xlo;     // [token][cols]
   const _Float16* sxhi; const _Float16* sxlo;   // [token][cols/32]
@@ -307,6 +307,157 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Q6_K on the same tiles (128 rows x TT * 32 tokens per work-group; neural/neuralgguf.pas:639-717).  A weight is
+// d * scale * (q - 32) with one signed 8-bit scale per 16 weights, and scale * (q - 32) reaches 4096: not exact in f16.
+// The scale is split, scale = 16 * (scale >> 4) + (scale & 15), and each weight takes TWO of the k slots of an MFMA:
+// (q - 32) * 16 * (scale >> 4) (a multiple of 16 up to 4096) and (q - 32) * (scale & 15) (at most 480) are both exact,
+// and the activation operand simply holds every value twice.  A lane (row n, half kg of the super-block) owns the 128
+// weights of its half; a step of the chain covers the 4 weights 32 j + l4 .. + 3 of the half: one dword of ql (nibble
+// j >> 1), one of qh (2-bit field j), the scale of group 2 j + (l4 >> 4).  There is no minimum term; d is applied once
+// per super-block.  Resident form: 192-byte ql | qh records, a plane of scales, a plane of d.
+// ------------------------------------------------------------------------------------------
+template <int TT>
+__global__ __launch_bounds__(256, 2) void gemm_q6k_pf(const GemmParams p)
+{
+  extern __shared__ __align__(16) unsigned char pf_smem[];
+  constexpr int NTOK = TT * 32;
+  _Float16* xs_hi = reinterpret_cast<_Float16*>(pf_smem);            // [NTOK][PF_LDX]
+  _Float16* xs_lo = xs_hi + NTOK * PF_LDX;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n = lane & 31, kg = lane >> 5;
+  const int L = blockIdx.x, rg = (L & 7) + 8 * ((L >> 3) / p.n_tok_tiles), ttile = (L >> 3) % p.n_tok_tiles;
+  if (rg >= p.n_row_groups) return;
+  const int R0 = (rg * 4 + wave) * 32, T0 = ttile * NTOK;
+  const int K = p.cols, nsb = K >> 8;
+  const int64_t blk0 = (int64_t)min(R0 + n, p.rows - 1) * nsb;       // tail rows: re-read the last row, not written
+
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+  struct WRegs { u32x4_t ql[4], qh[2]; u32x2_t sc; uint32_t d; };
+  auto load_w = [&](int sb, WRegs& r) {          // unconditional: past the last super-block the last one is fetched again
+    const int64_t b = blk0 + min(sb, nsb - 1);
+    const uint8_t* rec = p.w + b * 192;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r.ql[i] = *reinterpret_cast<const u32x4_t*>(rec + 64 * kg + 16 * i);
+#pragma unroll
+    for (int i = 0; i < 2; i++) r.qh[i] = *reinterpret_cast<const u32x4_t*>(rec + 128 + 32 * kg + 16 * i);
+    r.sc = *reinterpret_cast<const u32x2_t*>(p.aux + b * 16 + 8 * kg);
+    r.d = *reinterpret_cast<const uint16_t*>(p.aux2 + b * 2);
+  };
+  float16_t Y[TT];
+#pragma unroll
+  for (int tt = 0; tt < TT; tt++)
+#pragma unroll
+    for (int v = 0; v < 16; v++) Y[tt][v] = 0.0f;
+
+  WRegs wcur, wnxt;
+  load_w(0, wcur);
+  for (int sb = 0; sb < nsb; sb++) {
+    __syncthreads();                       // the previous step's LDS reads are done
+    {
+      const int tq = threadIdx.x >> 5, chunk = threadIdx.x & 31;
+      const uint32_t colo = (uint32_t)(sb * 256 + chunk * 8);
+      constexpr int SB = TT == 2 ? 1 : 4;
+#pragma unroll
+      for (int i0 = 0; i0 < NTOK / 8; i0 += SB) {
+        uint4 vh[SB], vl[SB];
+#pragma unroll
+        for (int i = 0; i < SB; i++) {
+          const uint32_t off = (uint32_t)min(T0 + tq + 8 * (i0 + i), p.n_tok - 1) * (uint32_t)K + colo;
+          vh[i] = *reinterpret_cast<const uint4*>(p.xhi + off);
+          vl[i] = *reinterpret_cast<const uint4*>(p.xlo + off);
+        }
+#pragma unroll
+        for (int i = 0; i < SB; i++) {
+          *reinterpret_cast<uint4*>(xs_hi + (tq + 8 * (i0 + i)) * PF_LDX + chunk * 8) = vh[i];
+          *reinterpret_cast<uint4*>(xs_lo + (tq + 8 * (i0 + i)) * PF_LDX + chunk * 8) = vl[i];
+        }
+      }
+    }
+    load_w(sb + 1, wnxt);
+    __syncthreads();
+
+    const WRegs& r = wcur;
+    // the 8 scales of this half as exact halfs: 16 * (s >> 4) (from the byte's top nibble, sign kept) and s & 15
+    const uint32_t scw[2] = {r.sc.x, r.sc.y};
+    half2_t s_hi[8], s_lo[8];
+#pragma unroll
+    for (int g = 0; g < 8; g++) {
+      const int sc = (int)(int8_t)((scw[g >> 2] >> (8 * (g & 3))) & 0xffu);
+      const _Float16 h = (_Float16)(float)((sc >> 4) * 16), l = (_Float16)(float)(sc & 15);
+      s_hi[g] = half2_t{h, h}; s_lo[g] = half2_t{l, l};
+    }
+    const half2_t o2 = {(_Float16)(-1056.0f), (_Float16)(-1056.0f)};   // 1024 + q - 1056 = q - 32
+    float16_t C[TT];
+    const float16_t zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int w = 0; w < 8; w++) {                                      // l4 = 4 w
+        const u32x4_t qlv = r.ql[2 * (j & 1) + (w >> 2)], qhv = r.qh[w >> 2];
+        const uint32_t ql = qlv[w & 3], qh = qhv[w & 3];
+        const uint32_t lo = (j >> 1) ? ((ql >> 4) & 0x0f0f0f0fu) : (ql & 0x0f0f0f0fu);
+        const uint32_t hi = (j == 0 ? (qh << 4) : j == 1 ? (qh << 2) : j == 2 ? qh : (qh >> 2)) & 0x30303030u;
+        const uint32_t c = lo | hi;
+        const half2_t c01 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, c, 0x04010400u)) + o2;
+        const half2_t c23 = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, c, 0x04030402u)) + o2;
+        const int g = 2 * j + (w >> 2);
+        const half2_t a0 = c01 * s_hi[g], a1 = c23 * s_hi[g], a2 = c01 * s_lo[g], a3 = c23 * s_lo[g];
+        const half8_pf A = {a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+#pragma unroll
+        for (int tt = 0; tt < TT; tt++) {
+          const int off = (tt * 32 + n) * PF_LDX + 128 * kg + 32 * j + 4 * w;
+          const half4_t xh = *reinterpret_cast<const half4_t*>(xs_hi + off);
+          const half4_t xl = *reinterpret_cast<const half4_t*>(xs_lo + off);
+          const half8_pf Bh = {xh.x, xh.y, xh.z, xh.w, xh.x, xh.y, xh.z, xh.w};
+          const half8_pf Bl = {xl.x, xl.y, xl.z, xl.w, xl.x, xl.y, xl.z, xl.w};
+          if (j == 0 && w == 0) C[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A, Bh, zero16, 0, 0, 0);
+          else C[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A, Bh, C[tt], 0, 0, 0);
+          C[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A, Bl, C[tt], 0, 0, 0);
+        }
+      }
+    // d of result row 8 g + 4 kg + i: held by the lane whose n is that row (both kg copies carry it)
+    const float dmine = __half2float(__ushort_as_half((unsigned short)r.d));
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const float dv = __shfl(dmine, 8 * (v >> 2) + 4 * kg + (v & 3), 64);
+#pragma unroll
+      for (int tt = 0; tt < TT; tt++) Y[tt][v] = fmaf(dv, C[tt][v], Y[tt][v]);
+    }
+    wcur = wnxt;
+  }
+
+  const bool vec = (p.y_stride & 3) == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 &&
+                   (!p.residual || (reinterpret_cast<uintptr_t>(p.residual) & 15) == 0) && (!p.bias || (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0);
+#pragma unroll
+  for (int tt = 0; tt < TT; tt++) {
+    const int t = T0 + tt * 32 + n;
+    if (t >= p.n_tok) continue;
+    const float si = p.sinv[t];
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      const int row = R0 + 8 * g + 4 * kg;
+      const int64_t o = (int64_t)t * p.y_stride + row;
+      if (vec && row + 3 < p.rows) {
+        float4 r = make_float4(Y[tt][4 * g] * si, Y[tt][4 * g + 1] * si, Y[tt][4 * g + 2] * si, Y[tt][4 * g + 3] * si);
+        if (p.bias) { const float4 b = *reinterpret_cast<const float4*>(p.bias + row); r.x += b.x; r.y += b.y; r.z += b.z; r.w += b.w; }
+        if (p.residual) { const float4 q = *reinterpret_cast<const float4*>(p.residual + o); r.x += q.x; r.y += q.y; r.z += q.z; r.w += q.w; }
+        *reinterpret_cast<float4*>(p.y + o) = r;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          if (row + i >= p.rows) continue;
+          float r = Y[tt][4 * g + i] * si;
+          if (p.bias) r += p.bias[row + i];
+          if (p.residual) r += p.residual[o + i];
+          p.y[o + i] = r;
+        }
+      }
+    }
+  }
+}
+
 int launch_xprep(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok,
                  _Float16* hi, _Float16* lo, float* sinv, _Float16* sxhi, _Float16* sxlo)
 {
@@ -314,7 +465,7 @@ int launch_xprep(const float* x, int64_t x_stride, const float* gain, float eps,
   return CAI_OK;
 }
 
-bool gemm_mfma_supported(const cai_qw_s* w) { return w->qtype == CAI_Q4_K; }
+bool gemm_mfma_supported(const cai_qw_s* w) { return (w->qtype == CAI_Q4_K || w->qtype == CAI_Q6_K) && w->cols % 256 == 0; }
 
 int launch_gemm_q4k(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo, const _Float16* sxhi, const _Float16* sxlo, const float* sinv,
                     int n_tok, float* y, int64_t y_stride, const float* residual)
@@ -324,6 +475,23 @@ int launch_gemm_q4k(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo,
   p.w = w->data; p.bias = w->bias; p.rows = (int)w->rows; p.cols = (int)w->cols;
   p.xhi = xhi; p.xlo = xlo; p.sxhi = sxhi; p.sxlo = sxlo; p.sinv = sinv; p.n_tok = n_tok; p.y = y; p.y_stride = y_stride;
   p.residual = residual;
+  if (w->qtype == CAI_Q6_K) {
+    p.aux = w->aux; p.aux2 = qw_aux2(w);
+    const int tt = ((p.rows + 127) / 128) * ((n_tok + 63) / 64) < 2 * ctx().n_cu ? 1 : 2;
+    p.n_row_groups = (p.rows + 127) / 128;
+    p.n_tok_tiles = (n_tok + tt * 32 - 1) / (tt * 32);
+    const size_t lds = (size_t)tt * 32 * PF_LDX * 2 * 2;
+    static bool attr6 = false;
+    if (!attr6) {
+      const void* ks[2] = {(const void*)gemm_q6k_pf<1>, (const void*)gemm_q6k_pf<2>};
+      for (const void* k : ks) if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) != hipSuccess) (void)hipGetLastError();
+      attr6 = true;
+    }
+    const int grid = 8 * p.n_tok_tiles * ((p.n_row_groups + 7) / 8);
+    if (tt == 1) hipLaunchKernelGGL(gemm_q6k_pf<1>, dim3(grid), dim3(256), lds, ctx().stream, p);
+    else hipLaunchKernelGGL(gemm_q6k_pf<2>, dim3(grid), dim3(256), lds, ctx().stream, p);
+    return CAI_OK;
+  }
   // Tiling: two row tiles per wave (256 rows per work-group, 32 tokens) when that still gives every CU several
   // work-groups; else 128 rows with two token tiles, or with one for matrices with few row groups.
   static const int tt_force = []() { const char* e = getenv("CAIHIP_PF_TT"); return e ? atoi(e) : 0; }();   // 1, 2: token tiles; 3: two row tiles
@@ -403,7 +571,7 @@ int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const fl
   int rc;
   // few tokens (the bandwidth-bound regime) of a Q4_K matrix, or a large matrix of a type without a prompt kernel (a small
   // one stays in the cache: the single-launch VALU kernel per 8 tokens is cheaper than three launches)
-  if (nb_supported(w) && (gemm_mfma_supported(w) ? n_tok <= 16 : w->data_bytes >= ((int64_t)16 << 20))) return nb_linear(w, x, x_stride, gain, eps, n_tok, y, y_stride, residual);
+  if (nb_supported(w) && (gemm_mfma_supported(w) ? n_tok <= 16 : (w->data_bytes >= ((int64_t)16 << 20) || (w->qtype == CAI_Q6_K && n_tok >= 16)))) return nb_linear(w, x, x_stride, gain, eps, n_tok, y, y_stride, residual);
   if (gemm_mfma_supported(w)) {
     if ((rc = prefill_prep(x, x_stride, gain, eps, (int)w->cols, n_tok))) return rc;
     return prefill_gemm(w, n_tok, y, y_stride, residual);

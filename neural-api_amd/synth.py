@@ -122,8 +122,14 @@ def random_int8_rows(rows, cols, gen, scale=1e-3):
     return cai.QWeight(cai.I8ROW, rows, cols, codes.data_ptr(), None, scales.data_ptr())
 
 
-def random_decoder_spec(cfg, qtype, head_qtype, seed=424242, qkv_bias=False, std=0.02, keep_bytes=False):
-    """Backend-neutral spec whose tensors are already resident (entry "qw"); norm gains are 1."""
+def more_bits_layer(i, n):
+    """The blocks whose attn_v and ffn_down a Q4_K_M export keeps in Q6_K (the first and last eighth and every third between)."""
+    return i < n // 8 or i >= 7 * n // 8 or (i - n // 8) % 3 == 2
+
+
+def random_decoder_spec(cfg, qtype, head_qtype, seed=424242, qkv_bias=False, std=0.02, keep_bytes=False, embed_qtype=None, q6k_mix=False):
+    """Backend-neutral spec whose tensors are already resident (entry "qw"); norm gains are 1.
+    q6k_mix: attn_v and ffn_down of the more_bits_layer blocks in Q6_K (the Q4_K_M mix)."""
     import numpy as np
     gen = torch.Generator(device="cuda"); gen.manual_seed(seed)
     d, hq, hkv, hd, I, V, L = cfg["d_model"], cfg["n_q_heads"], cfg["n_kv_heads"], cfg["head_dim"], cfg["ffn"], cfg["vocab"], cfg["n_layers"]
@@ -134,14 +140,15 @@ def random_decoder_spec(cfg, qtype, head_qtype, seed=424242, qkv_bias=False, std
         w, raw, b = random_qweight(qt, rows, cols, gen, std, bias, keep_bytes=keep_bytes)
         T[key] = dict(qw=w, type=qt, rows=rows, cols=cols, raw_dev=raw, bias=b)
 
-    put((-1, cai.W_EMBED), head_qtype, V, d)
+    put((-1, cai.W_EMBED), embed_qtype if embed_qtype is not None else head_qtype, V, d)
     if not cfg.get("tied", False):
         put((-1, cai.W_HEAD), head_qtype, V, d)
     Vv[(-1, cai.V_FINAL_NORM)] = np.ones(d, np.float32)
     for l in range(L):
         put((l, cai.W_Q), qtype, hq * hd, d, qkv_bias)
         put((l, cai.W_K), qtype, hkv * hd, d, qkv_bias)
-        put((l, cai.W_V), qtype, hkv * hd, d, qkv_bias)
+        hi = q6k_mix and more_bits_layer(l, L)
+        put((l, cai.W_V), cai.Q6_K if hi else qtype, hkv * hd, d, qkv_bias)
         put((l, cai.W_O), qtype, d, hq * hd)
         Vv[(l, cai.V_ATTN_NORM)] = np.ones(d, np.float32)
         Vv[(l, cai.V_MLP_NORM)] = np.ones(d, np.float32)
@@ -154,6 +161,6 @@ def random_decoder_spec(cfg, qtype, head_qtype, seed=424242, qkv_bias=False, std
             put((l, cai.W_DOWN), qtype, ne * d, I)
         else:
             put((l, cai.W_GATEUP), qtype, 2 * I, d)
-            put((l, cai.W_DOWN), qtype, d, I)
+            put((l, cai.W_DOWN), cai.Q6_K if hi else qtype, d, I)
     c = {k: v for k, v in cfg.items() if k != "tied"}
     return dict(cfg=c, tensors=T, vecs=Vv)

@@ -171,6 +171,15 @@ def test_batched_decode_and_prompt_of_a_q4k_q6k_mix_equal_single_steps():
     dec.reset(1)
     am, lg = dec.prefill([int(t) for t in toks[2]], 0, seq=1)
     assert rel_err(lg, singles[2][9]) < 1e-3 and am == int(np.argmax(singles[2][9]))
+    # a prompt of more than 16 tokens: the Q6_K matrices go through the prompt GEMM with split scales
+    long = [int(t) for t in rng.integers(0, cfg["vocab"], 45)]
+    dec.reset(0)
+    last = None
+    for p, t in enumerate(long):
+        last = dec.step(t, p)[1][0].copy()
+    dec.reset(1)
+    am, lg = dec.prefill(long, 0, seq=1)
+    assert rel_err(lg, last) < 1e-3 and am == int(np.argmax(last))
 
 
 def test_prefill_equals_sequential_steps():

@@ -224,11 +224,13 @@ def test_small_batch_gemm_q8_0_q4_0_on_matrix_cores(qt, rows, cols, T):
     assert rel_err(w.gemm(x), want, floor=0.02 * cols ** 0.5 * float(np.abs(x).mean())) < TIGHT   # the dispatcher's own choice
 
 
-@pytest.mark.parametrize("rows,cols,T", [(128, 256, 2), (33, 512, 3), (1000, 1024, 8), (3584, 3584, 8), (512, 18944, 4), (20000, 2048, 16), (5000, 768, 13), (70, 1536, 7)])
+@pytest.mark.parametrize("rows,cols,T", [(128, 256, 2), (33, 512, 3), (1000, 1024, 8), (3584, 3584, 8), (512, 18944, 4), (20000, 2048, 16), (5000, 768, 13), (70, 1536, 7),
+                                         (1000, 1024, 40), (3584, 3584, 77), (512, 18944, 33), (130, 512, 64), (4099, 256, 129)])
 def test_small_batch_gemm_q6_k_on_matrix_cores(rows, cols, T):
     """Q6_K on the matrix cores: one 16-deep MFMA per 16-weight scale group (codes q - 32 exact in f16, d * scale applied to
-    the result by the lane that owns the weight row), unaligned 16-byte requests transposed over the four k lanes
-    == T single-token layers, bias included."""
+    the result by the lane that owns the weight row), 16-byte requests transposed over the four k lanes
+    == T single-token layers, bias included.  More than 16 tokens take the prompt kernel: the scale split into
+    16 * (s >> 4) and s & 15, two exact f16 operand slots per weight."""
     from helpers.device import dev, rel_err
     cai = dev()
     raw, rng = make(O.Q6_K, rows, cols, T + 300)
