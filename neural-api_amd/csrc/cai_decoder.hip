@@ -235,9 +235,9 @@ static int ensure_prefill_buffers(cai_decoder_s* d, int n)
 static int linear_rows(const cai_qw_s* w, bool prepped, const float* x, int64_t x_stride, const float* gain, float eps, int n,
                        float* y, int64_t y_stride, const float* residual)
 {
-  // few tokens (the bandwidth-bound regime) of a Q4_K matrix, or a large matrix of a type without a prompt kernel (a small
+  // few tokens (the bandwidth-bound regime) of a Q4_K or Q6_K matrix, or a large matrix of a type without a prompt kernel (a small
   // one stays in the cache: the single-launch VALU kernel per 8 tokens is cheaper than three launches)
-  if (nb_supported(w) && (gemm_mfma_supported(w) ? n <= 16 : (w->data_bytes >= ((int64_t)16 << 20) || (w->qtype == CAI_Q6_K && n >= 16)))) return nb_linear(w, x, x_stride, gain, eps, n, y, y_stride, residual);
+  if (nb_supported(w) && (gemm_mfma_supported(w) ? n <= 16 : w->data_bytes >= ((int64_t)16 << 20))) return nb_linear(w, x, x_stride, gain, eps, n, y, y_stride, residual);
   if (gemm_mfma_supported(w)) {
     int rc;
     if (!prepped && (rc = prefill_prep(x, x_stride, gain, eps, (int)w->cols, n))) return rc;

@@ -28,7 +28,7 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 constexpr int NB_LDX = 264;      // halfs per staged activation column: 256 + pad (stride = 4 banks mod 64: 16-byte reads of 16 columns tile the banks)
 constexpr int NB_SC = 16;        // staged columns: 8 tokens x {hi, lo}
 constexpr int NB_TK = 8;         // tokens per matrix-core group (8 hi + 8 lo = the 16 rows of an MFMA operand) and per pass of most kernels
-constexpr int NB_TMAX = 32;      // tokens per pass at most (the Q6_K kernel takes four groups); the workspace holds this many
+constexpr int NB_TMAX = 16;      // tokens per pass at most (the Q6_K kernel takes two groups; four spill its accumulators); the workspace holds this many
 constexpr int NB_SMAX = 5;       // super-blocks per K slice at most (LDS: 8.6 KB each, and three work-groups share a CU)
 
 struct NbSeg { const uint8_t* w; const uint8_t* aux; const uint8_t* aux2; const float* bias; const float* row_scale; int rows; int y_off; int tile_end; };   // aux: block scales plane (Q8_0 / Q4_0 / Q6_K); aux2: Q6_K plane of d; row_scale: per-row int8 matrices; tile_end: cumulative 32-row tiles
@@ -480,7 +480,7 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
 // ------------------------------------------------------------------------------------------
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
-// NT groups of 8 tokens share every converted weight operand and scale: prompts take 32 tokens per pass (NT = 4).
+// NT groups of 8 tokens share every converted weight operand and scale: 9..16 tokens take one pass with NT = 2.
 template <int NT>
 __global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
 {
@@ -943,8 +943,7 @@ int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok)
     } else {
       const size_t lds = (size_t)S * NB_SC * NB_LDX * 2 + (size_t)S * NB_TK * 4;
       const bool tail = p.cols % 256 != 0;
-      if (qt == CAI_Q6_K && n_tok > 2 * NB_TK) nb_launch<gemm_q6k_nb<4>>(p, gxs, n_slices, 4 * lds);
-      else if (qt == CAI_Q6_K && n_tok > NB_TK) nb_launch<gemm_q6k_nb<2>>(p, gxs, n_slices, 2 * lds);
+      if (qt == CAI_Q6_K && n_tok > NB_TK) nb_launch<gemm_q6k_nb<2>>(p, gxs, n_slices, 2 * lds);
       else if (qt == CAI_Q6_K) nb_launch<gemm_q6k_nb<1>>(p, gxs, n_slices, lds);
       else if (qt == CAI_Q8_0) { if (tail) nb_launch<gemm_blk_nb<CAI_Q8_0, true>>(p, gxs, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_Q8_0, false>>(p, gxs, n_slices, lds); }
       else if (qt == CAI_I8ROW) { if (tail) nb_launch<gemm_blk_nb<CAI_I8ROW, true>>(p, gxs, n_slices, lds); else nb_launch<gemm_blk_nb<CAI_I8ROW, false>>(p, gxs, n_slices, lds); }
@@ -972,11 +971,7 @@ int nb_reduce(float* y, int64_t y_stride, const float* residual)
 }
 
 // Tokens one pass of nb_prep / nb_gemm / nb_reduce takes for this weight type
-int nb_pass_tokens(const cai_qw_s* w)
-{
-  static const int q6 = []() { const char* e = getenv("CAIHIP_NB_Q6K_PASS"); const int v = e ? atoi(e) : 16; return v == 8 || v == 16 || v == 32 ? v : 16; }();
-  return w->qtype == CAI_Q6_K ? q6 : NB_TK;
-}
+int nb_pass_tokens(const cai_qw_s* w) { return w->qtype == CAI_Q6_K ? NB_TMAX : NB_TK; }
 
 // Whole linear layer, 8 tokens per pass (the weights are streamed once per pass): y = W (gain . x / rms) + bias (+ residual)
 int nb_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok, float* y, int64_t y_stride, const float* residual)

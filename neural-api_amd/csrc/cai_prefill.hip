@@ -569,15 +569,15 @@ int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const fl
                    float* y, int64_t y_stride, const float* residual)
 {
   int rc;
-  // few tokens (the bandwidth-bound regime) of a Q4_K matrix, or a large matrix of a type without a prompt kernel (a small
+  // few tokens (the bandwidth-bound regime) of a Q4_K or Q6_K matrix, or a large matrix of a type without a prompt kernel (a small
   // one stays in the cache: the single-launch VALU kernel per 8 tokens is cheaper than three launches)
-  if (nb_supported(w) && (gemm_mfma_supported(w) ? n_tok <= 16 : (w->data_bytes >= ((int64_t)16 << 20) || (w->qtype == CAI_Q6_K && n_tok >= 16)))) return nb_linear(w, x, x_stride, gain, eps, n_tok, y, y_stride, residual);
+  if (nb_supported(w) && (gemm_mfma_supported(w) ? n_tok <= 16 : w->data_bytes >= ((int64_t)16 << 20))) return nb_linear(w, x, x_stride, gain, eps, n_tok, y, y_stride, residual);
   if (gemm_mfma_supported(w)) {
     if ((rc = prefill_prep(x, x_stride, gain, eps, (int)w->cols, n_tok))) return rc;
     return prefill_gemm(w, n_tok, y, y_stride, residual);
   }
   // other weight types: groups of up to 8 tokens through the small-batch kernel (x must be contiguous)
-  if (x_stride != w->cols) return set_error(CAI_ERR_UNSUPPORTED, "prefill linear: strided input needs a Q4_K matrix");
+  if (x_stride != w->cols) return set_error(CAI_ERR_UNSUPPORTED, "prefill linear: strided input needs a Q4_K or Q6_K matrix");
   for (int t = 0; t < n_tok; t += 8) {
     const int nb = std::min(8, n_tok - t);
     MultiGemv m{}; m.n = 1; m.w[0] = w; m.rows[0] = w->rows;
