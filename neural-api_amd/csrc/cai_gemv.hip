@@ -612,12 +612,12 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
     p.seg[i].y_off = m.y_off[i];
   }
   const int qt = w0->qtype;
-  if (qt == CAI_Q4_K && n_b == 1 && !m.slot_expert && stream_kernel_enabled()) {
+  if ((qt == CAI_Q4_K || (qt == CAI_Q6_K && m.n == 1 && !swiglu_half)) && n_b == 1 && !m.slot_expert && stream_kernel_enabled()) {
     MultiGemv mm = m;
     if (swiglu_half) { if (m.n != 1) return set_error(CAI_ERR_INVALID, "gemv: swiglu takes one matrix"); p.seg[0].rows = swiglu_half; }
     p.ssq_in = m.ssq_in; p.ssq_out = m.ssq_out;
     static const bool float_x = []() { const char* e = getenv("CAIHIP_GEMV_FLOAT_X"); return e && e[0] == '1'; }();
-    const int rc = float_x ? launch_q4k_stream(p, mm, swiglu_half, c.stream) : launch_q4k_dot(p, mm, swiglu_half, c.stream);
+    const int rc = (float_x && qt == CAI_Q4_K) ? launch_q4k_stream(p, mm, swiglu_half, c.stream) : launch_q4k_dot(p, mm, swiglu_half, c.stream);
     p.ssq_in = nullptr; p.ssq_out = nullptr;
     if (rc != CAI_ERR_UNSUPPORTED) return rc;
   }

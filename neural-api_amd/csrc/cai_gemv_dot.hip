@@ -67,8 +67,15 @@ __device__ __forceinline__ void pack_digits(const float (&f)[4], int (&d)[NL])
 
 }  // namespace
 
-template <int R, int MODE, bool MULTISEG, int NS>
-__global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
+// Q6_K in the same walk (neural/neuralgguf.pas:639-717; resident as 192-byte ql | qh records + planes of scales and d):
+// the lane that owns activations 64 cc .. 64 cc + 63 of a super-block owns, in half nh = cc >> 1, the weights of j = 2 jp
+// (its first 32 activations) and j = 2 jp + 1 (the second 32), jp = cc & 1: the low (jp = 0) or high nibbles of the two
+// 32-byte ql runs and two of the four 2-bit fields of the 32 qh bytes.  Codes 0..63 go to v_dot4 as they are; the - 32
+// offset uses the sums of the lane's integer activations per 16, taken once; each 16 weights have their own scale.
+struct Q6kRegs { uint4 a0, a1, b0, b1, h0, h1; uint2 sc; uint32_t d; };
+
+template <int R, int MODE, bool MULTISEG, int NS, int QT>
+__device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_groups, const int nsw, const int gwv)
 {
   extern __shared__ uint4 xq4[];
   constexpr int RR = MODE == 1 ? 2 * R : R;
@@ -79,12 +86,13 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: group indices, segment lookups and loop bounds stay scalar
   const int step = wave % nsw, gslot = wave / nsw;
   const int cols = p.cols, nsb = cols >> 8;
-  const int64_t row_bytes = (int64_t)nsb * 144;
+  const int64_t row_bytes = (int64_t)nsb * (QT == CAI_Q6_K ? 192 : 144);
   const int sb = step * 16 + (lane >> 2), cc = lane & 3;
   const bool act = sb < nsb;
   const int g_first = blockIdx.x * gwv + gslot, g_stride = gridDim.x * gwv;
   const int n_iters = (n_groups + g_stride - 1) / g_stride;
-  const int64_t lane_off = (int64_t)(act ? sb : 0) * 144;
+  const int64_t lane_off = (int64_t)(act ? sb : 0) * (QT == CAI_Q6_K ? 192 : 144);
+  using WRegs = typename std::conditional<QT == CAI_Q6_K, Q6kRegs, Q4kRegs>::type;
 
   // group -> segment, first row of the group inside the segment
   auto locate = [&](int g, const GemvSeg*& sg, int& row0) {
@@ -98,7 +106,7 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
   // Loads are never conditional: past the last group the last one is fetched again, lanes beyond the row's width fetch
   // super-block 0 (both cache hits, the values are not used).  A load under a branch would make the compiler wait for
   // ALL outstanding loads wherever the paths join, i.e. before every new request.
-  auto issue = [&](int g, Q4kRegs (&rg)[RR]) {
+  auto issue = [&](int g, WRegs (&rg)[RR]) {
     const GemvSeg* sg; int row0; locate(min(g, n_groups - 1), sg, row0);
     const int lim = MODE == 1 ? p.half : sg->rows;
 #pragma unroll
@@ -107,13 +115,23 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
       if (row >= lim) row = lim - 1;               // tail group: re-read the last row, result is not written
       if (MODE == 1 && (r & 1)) row += p.half;
       const uint8_t* blk = sg->data + (int64_t)row * row_bytes + lane_off;
-      rg[r].h = *reinterpret_cast<const uint4*>(blk);
-      rg[r].q0 = *reinterpret_cast<const uint4*>(blk + 16 + 32 * cc);
-      rg[r].q1 = *reinterpret_cast<const uint4*>(blk + 32 + 32 * cc);
+      if constexpr (QT == CAI_Q6_K) {
+        const int nh = cc >> 1;
+        const int64_t b = (int64_t)row * nsb + (act ? sb : 0);
+        rg[r].a0 = *reinterpret_cast<const uint4*>(blk + 64 * nh);      rg[r].a1 = *reinterpret_cast<const uint4*>(blk + 64 * nh + 16);
+        rg[r].b0 = *reinterpret_cast<const uint4*>(blk + 64 * nh + 32); rg[r].b1 = *reinterpret_cast<const uint4*>(blk + 64 * nh + 48);
+        rg[r].h0 = *reinterpret_cast<const uint4*>(blk + 128 + 32 * nh); rg[r].h1 = *reinterpret_cast<const uint4*>(blk + 144 + 32 * nh);
+        rg[r].sc = *reinterpret_cast<const uint2*>(sg->aux + b * 16 + 8 * nh);
+        rg[r].d = *reinterpret_cast<const uint16_t*>(sg->aux2 + b * 2);
+      } else {
+        rg[r].h = *reinterpret_cast<const uint4*>(blk);
+        rg[r].q0 = *reinterpret_cast<const uint4*>(blk + 16 + 32 * cc);
+        rg[r].q1 = *reinterpret_cast<const uint4*>(blk + 32 + 32 * cc);
+      }
     }
   };
 
-  Q4kRegs buf[NS][RR];
+  WRegs buf[NS][RR];
   // weights do not depend on the activation: request the first row groups before anything else
 #pragma unroll
   for (int k = 0; k < NS - 1; k++) issue(g_first + k * g_stride, buf[k]);
@@ -227,11 +245,26 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
       for (int t = 0; t < 16; t++) xq[L][t] = 0;
   }
 
+  float s16[4] = {0.0f, 0.0f, 0.0f, 0.0f};   // Q6_K: the lane's integer activations summed per 16 (first / second 32: groups 0, 1 / 2, 3)
+  if constexpr (QT == CAI_Q6_K) {
+#pragma unroll
+    for (int gq = 0; gq < 4; gq++) {
+      int tot = 0;
+#pragma unroll
+      for (int L = 0; L < NL; L++) {
+        int t = 0;
+#pragma unroll
+        for (int w = 0; w < 4; w++) t = __builtin_amdgcn_sdot4(0x01010101, xq[L][4 * gq + w], t, false);
+        tot += t << (8 * L);
+      }
+      s16[gq] = (float)tot;
+    }
+  }
   float ssq_acc = 0.0f;   // squares of the outputs this thread wrote (for the consumer's RMSNorm)
   float keep[RR];         // finished totals of the last row groups, one group per lane
 #pragma unroll
   for (int r = 0; r < RR; r++) keep[r] = 0.0f;
-  auto process = [&](Q4kRegs (&cur)[RR], Q4kRegs (&nxt)[RR], int it) {
+  auto process = [&](WRegs (&cur)[RR], WRegs (&nxt)[RR], int it) {
     const int g = g_first + it * g_stride;
     issue(g + (NS - 1) * g_stride, nxt);
     float acc[RR];
@@ -240,6 +273,36 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
     if (g < n_groups) {   // lanes beyond the row's width hold zero activations: they add exactly 0
 #pragma unroll
       for (int r = 0; r < RR; r++) {
+        if constexpr (QT == CAI_Q6_K) {
+          const uint32_t qa[8] = {cur[r].a0.x, cur[r].a0.y, cur[r].a0.z, cur[r].a0.w, cur[r].a1.x, cur[r].a1.y, cur[r].a1.z, cur[r].a1.w};
+          const uint32_t qb[8] = {cur[r].b0.x, cur[r].b0.y, cur[r].b0.z, cur[r].b0.w, cur[r].b1.x, cur[r].b1.y, cur[r].b1.z, cur[r].b1.w};
+          const uint32_t qh[8] = {cur[r].h0.x, cur[r].h0.y, cur[r].h0.z, cur[r].h0.w, cur[r].h1.x, cur[r].h1.y, cur[r].h1.z, cur[r].h1.w};
+          const int sh = 4 * (cc & 1);
+          int ig[4][NL];
+#pragma unroll
+          for (int gq = 0; gq < 4; gq++)
+#pragma unroll
+            for (int L = 0; L < NL; L++) ig[gq][L] = 0;
+#pragma unroll
+          for (int w = 0; w < 8; w++) {
+            const uint32_t hw = qh[w] >> sh;
+            const int ca = (int)(((qa[w] >> sh) & 0x0f0f0f0fu) | ((hw << 4) & 0x30303030u));
+            const int cb = (int)(((qb[w] >> sh) & 0x0f0f0f0fu) | ((hw << 2) & 0x30303030u));
+#pragma unroll
+            for (int L = 0; L < NL; L++) {
+              ig[w >> 2][L] = __builtin_amdgcn_sdot4(ca, xq[L][w], ig[w >> 2][L], false);
+              ig[2 + (w >> 2)][L] = __builtin_amdgcn_sdot4(cb, xq[L][8 + w], ig[2 + (w >> 2)][L], false);
+            }
+          }
+          const uint32_t scw = (cc & 1) ? cur[r].sc.y : cur[r].sc.x;   // the four scales of this lane's groups, in order
+          float fg[4];
+#pragma unroll
+          for (int gq = 0; gq < 4; gq++)
+            fg[gq] = (float)(int)(int8_t)((scw >> (8 * gq)) & 0xffu) * fmaf(-32.0f, s16[gq], (float)(ig[gq][0] + (ig[gq][1] << 8) + (ig[gq][2] << 16)));
+          const float d = __half2float(__ushort_as_half((unsigned short)cur[r].d));
+          acc[r] = d * (sA * (fg[0] + fg[1]) + sB * (fg[2] + fg[3]));
+          continue;
+        } else {
         const uint32_t qw[8] = {cur[r].q0.x, cur[r].q0.y, cur[r].q0.z, cur[r].q0.w, cur[r].q1.x, cur[r].q1.y, cur[r].q1.z, cur[r].q1.w};
         int ia[NL], ib[NL];
 #pragma unroll
@@ -258,6 +321,7 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
         const float d = __half2float(__ushort_as_half((unsigned short)(cur[r].h.x & 0xffffu)));
         const float dmin = __half2float(__ushort_as_half((unsigned short)(cur[r].h.x >> 16)));
         acc[r] = d * (cvt_ub0(sc) * (sA * fa) + cvt_ub1(sc) * (sB * fb)) - dmin * (cvt_ub0(mn) * mA + cvt_ub1(mn) * mB);
+        }
       }
     }
 #pragma unroll
@@ -355,6 +419,18 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
   }
 }
 
+template <int R, int MODE, bool MULTISEG, int NS>
+__global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
+{
+  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q4_K>(p, n_groups, nsw, gwv);
+}
+
+template <int R, int NS>
+__global__ __launch_bounds__(768, 3) void gemv_q6k_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
+{
+  gemv_dot_body<R, 0, false, NS, CAI_Q6_K>(p, n_groups, nsw, gwv);
+}
+
 // Host launcher.  Returns CAI_ERR_UNSUPPORTED when the shape does not fit this kernel (caller falls back).
 int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream_t st)
 {
@@ -362,6 +438,8 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
   const int cols = p.cols, nsb = cols >> 8;
   const int nsw = (nsb + 15) >> 4;          // waves along the columns
   if (nsw > 8) return CAI_ERR_UNSUPPORTED;  // rows longer than 32768 columns
+  const bool q6k = m.w[0]->qtype == CAI_Q6_K;
+  if (q6k && (swiglu_half || m.n != 1)) return CAI_ERR_UNSUPPORTED;
   static const int ns_env = []() { const char* e = getenv("CAIHIP_DOT_NS"); return e ? atoi(e) : 2; }();
   static const int W = []() { const char* e = getenv("CAIHIP_DOT_W"); return e ? atoi(e) : 12; }();   // resident waves per CU
   // waves per work-group: short rows (one or two waves span the columns) use ONE work-group of 8 waves per CU - the
@@ -389,6 +467,7 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
     if (nsw < 3 || 2 * turns2 <= turns1) R = 2;
   }
   if (!swiglu_half && (r_env == 1 || r_env == 2)) R = r_env;
+  if (q6k) R = 1;   // (two rows of Q6_K requests in flight twice over do not fit the registers)
   int cum = 0;
   for (int i = 0; i < m.n; i++) {
     const int64_t rows = swiglu_half ? swiglu_half : m.rows[i];
@@ -406,7 +485,8 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
   };
   auto pick = [&](auto ns) {
     constexpr int NSV = decltype(ns)::value;
-    if (swiglu_half) go(gemv_q4k_dot<1, 1, false, NSV>);
+    if (q6k) go(gemv_q6k_dot<1, NSV>);
+    else if (swiglu_half) go(gemv_q4k_dot<1, 1, false, NSV>);
     else if (m.n > 1) { if (R == 2) go(gemv_q4k_dot<2, 0, true, NSV>); else go(gemv_q4k_dot<1, 0, true, NSV>); }
     else { if (R == 2) go(gemv_q4k_dot<2, 0, false, NSV>); else go(gemv_q4k_dot<1, 0, false, NSV>); }
   };
