@@ -612,7 +612,7 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
     p.seg[i].y_off = m.y_off[i];
   }
   const int qt = w0->qtype;
-  if ((qt == CAI_Q4_K || (qt == CAI_Q6_K && m.n == 1 && !swiglu_half)) && n_b == 1 && !m.slot_expert && stream_kernel_enabled()) {
+  if ((qt == CAI_Q4_K || (qt == CAI_Q4_0 && p.cols % 256 == 0) || (qt == CAI_Q6_K && m.n == 1 && !swiglu_half)) && n_b == 1 && !m.slot_expert && stream_kernel_enabled()) {
     MultiGemv mm = m;
     if (swiglu_half) { if (m.n != 1) return set_error(CAI_ERR_INVALID, "gemv: swiglu takes one matrix"); p.seg[0].rows = swiglu_half; }
     p.ssq_in = m.ssq_in; p.ssq_out = m.ssq_out;

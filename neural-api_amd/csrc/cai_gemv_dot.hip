@@ -1,4 +1,5 @@
-// Persistent streaming Q4_K matrix-vector kernel for batch-1 decode on gfx950, integer-dot form.
+// Persistent streaming matrix-vector kernel for batch-1 decode on gfx950, integer-dot form: Q4_K, and with other requests and
+// block arithmetic in the same walk Q4_0 (quants and scales planes) and Q6_K (ql|qh records + planes of scales and d).
 //
 // The weights of a Q4_K sub-block are 4-bit integers with one float scale, so dot(W[a], X) splits into an exact
 // integer part and a handful of float operations per 32 weights once X is held as integers too.  Each
@@ -86,12 +87,12 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: group indices, segment lookups and loop bounds stay scalar
   const int step = wave % nsw, gslot = wave / nsw;
   const int cols = p.cols, nsb = cols >> 8;
-  const int64_t row_bytes = (int64_t)nsb * (QT == CAI_Q6_K ? 192 : 144);
+  const int64_t row_bytes = (int64_t)nsb * (QT == CAI_Q6_K ? 192 : QT == CAI_Q4_0 ? 128 : 144);
   const int sb = step * 16 + (lane >> 2), cc = lane & 3;
   const bool act = sb < nsb;
   const int g_first = blockIdx.x * gwv + gslot, g_stride = gridDim.x * gwv;
   const int n_iters = (n_groups + g_stride - 1) / g_stride;
-  const int64_t lane_off = (int64_t)(act ? sb : 0) * (QT == CAI_Q6_K ? 192 : 144);
+  const int64_t lane_off = (int64_t)(act ? sb : 0) * (QT == CAI_Q6_K ? 192 : QT == CAI_Q4_0 ? 128 : 144);
   using WRegs = typename std::conditional<QT == CAI_Q6_K, Q6kRegs, Q4kRegs>::type;
 
   // group -> segment, first row of the group inside the segment
@@ -123,6 +124,11 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
         rg[r].h0 = *reinterpret_cast<const uint4*>(blk + 128 + 32 * nh); rg[r].h1 = *reinterpret_cast<const uint4*>(blk + 144 + 32 * nh);
         rg[r].sc = *reinterpret_cast<const uint2*>(sg->aux + b * 16 + 8 * nh);
         rg[r].d = *reinterpret_cast<const uint16_t*>(sg->aux2 + b * 2);
+      } else if constexpr (QT == CAI_Q4_0) {
+        // quants plane: the lane's two 32-weight blocks are 32 contiguous bytes; scales plane: their two halfs one dword
+        rg[r].q0 = *reinterpret_cast<const uint4*>(blk + 32 * cc);
+        rg[r].q1 = *reinterpret_cast<const uint4*>(blk + 32 * cc + 16);
+        rg[r].h.x = *reinterpret_cast<const uint32_t*>(sg->aux + ((int64_t)row * nsb + (act ? sb : 0)) * 16 + 4 * cc);
       } else {
         rg[r].h = *reinterpret_cast<const uint4*>(blk);
         rg[r].q0 = *reinterpret_cast<const uint4*>(blk + 16 + 32 * cc);
@@ -302,6 +308,27 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
           const float d = __half2float(__ushort_as_half((unsigned short)cur[r].d));
           acc[r] = d * (sA * (fg[0] + fg[1]) + sB * (fg[2] + fg[3]));
           continue;
+        } else if constexpr (QT == CAI_Q4_0) {
+          // block A = q0 (low nibbles: weights 0..15, high: 16..31), block B = q1; x = d * (nibble - 8) (neural/neuralgguf.pas:811-845)
+          const uint32_t qa[4] = {cur[r].q0.x, cur[r].q0.y, cur[r].q0.z, cur[r].q0.w}, qb[4] = {cur[r].q1.x, cur[r].q1.y, cur[r].q1.z, cur[r].q1.w};
+          int ia[NL], ib[NL];
+#pragma unroll
+          for (int L = 0; L < NL; L++) { ia[L] = 0; ib[L] = 0; }
+#pragma unroll
+          for (int w = 0; w < 4; w++) {
+            const int al = (int)(qa[w] & 0x0f0f0f0fu), ah = (int)((qa[w] >> 4) & 0x0f0f0f0fu);
+            const int bl = (int)(qb[w] & 0x0f0f0f0fu), bh = (int)((qb[w] >> 4) & 0x0f0f0f0fu);
+#pragma unroll
+            for (int L = 0; L < NL; L++) {
+              ia[L] = __builtin_amdgcn_sdot4(al, xq[L][w], ia[L], false);     ia[L] = __builtin_amdgcn_sdot4(ah, xq[L][4 + w], ia[L], false);
+              ib[L] = __builtin_amdgcn_sdot4(bl, xq[L][8 + w], ib[L], false); ib[L] = __builtin_amdgcn_sdot4(bh, xq[L][12 + w], ib[L], false);
+            }
+          }
+          const float fa = (float)(ia[0] + (ia[1] << 8) + (ia[2] << 16)), fb = (float)(ib[0] + (ib[1] << 8) + (ib[2] << 16));
+          const float dA = __half2float(__ushort_as_half((unsigned short)(cur[r].h.x & 0xffffu)));
+          const float dB = __half2float(__ushort_as_half((unsigned short)(cur[r].h.x >> 16)));
+          acc[r] = dA * fmaf(sA, fa, -8.0f * mA) + dB * fmaf(sB, fb, -8.0f * mB);
+          continue;
         } else {
         const uint32_t qw[8] = {cur[r].q0.x, cur[r].q0.y, cur[r].q0.z, cur[r].q0.w, cur[r].q1.x, cur[r].q1.y, cur[r].q1.z, cur[r].q1.w};
         int ia[NL], ib[NL];
@@ -425,6 +452,12 @@ __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const
   gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q4_K>(p, n_groups, nsw, gwv);
 }
 
+template <int R, int MODE, bool MULTISEG, int NS>
+__global__ __launch_bounds__(768, 3) void gemv_q40_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
+{
+  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q4_0>(p, n_groups, nsw, gwv);
+}
+
 template <int R, int NS>
 __global__ __launch_bounds__(768, 3) void gemv_q6k_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
 {
@@ -437,7 +470,7 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
   Context& c = ctx();
   const int cols = p.cols, nsb = cols >> 8;
   const int nsw = (nsb + 15) >> 4;          // waves along the columns
-  if (nsw > 8) return CAI_ERR_UNSUPPORTED;  // rows longer than 32768 columns
+  if (nsw > 8 || cols % 256) return CAI_ERR_UNSUPPORTED;  // rows longer than 32768 columns; Q4_0 widths that are not whole 256-blocks
   const bool q6k = m.w[0]->qtype == CAI_Q6_K;
   if (q6k && (swiglu_half || m.n != 1)) return CAI_ERR_UNSUPPORTED;
   static const int ns_env = []() { const char* e = getenv("CAIHIP_DOT_NS"); return e ? atoi(e) : 2; }();
@@ -486,6 +519,11 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
   auto pick = [&](auto ns) {
     constexpr int NSV = decltype(ns)::value;
     if (q6k) go(gemv_q6k_dot<1, NSV>);
+    else if (m.w[0]->qtype == CAI_Q4_0) {
+      if (swiglu_half) go(gemv_q40_dot<1, 1, false, NSV>);
+      else if (m.n > 1) { if (R == 2) go(gemv_q40_dot<2, 0, true, NSV>); else go(gemv_q40_dot<1, 0, true, NSV>); }
+      else { if (R == 2) go(gemv_q40_dot<2, 0, false, NSV>); else go(gemv_q40_dot<1, 0, false, NSV>); }
+    }
     else if (swiglu_half) go(gemv_q4k_dot<1, 1, false, NSV>);
     else if (m.n > 1) { if (R == 2) go(gemv_q4k_dot<2, 0, true, NSV>); else go(gemv_q4k_dot<1, 0, true, NSV>); }
     else { if (R == 2) go(gemv_q4k_dot<2, 0, false, NSV>); else go(gemv_q4k_dot<1, 0, false, NSV>); }
