@@ -304,7 +304,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
           float fg[4];
 #pragma unroll
           for (int gq = 0; gq < 4; gq++)
-            fg[gq] = (float)(int)(int8_t)((scw >> (8 * gq)) & 0xffu) * fmaf(-32.0f, s16[gq], (float)(ig[gq][0] + (ig[gq][1] << 8) + (ig[gq][2] << 16)));
+            fg[gq] = (float)(int)(int8_t)((scw >> (8 * gq)) & 0xffu) * fmaf(-32.0f, s16[gq], (float)ig[gq][0] + 256.0f * (float)ig[gq][1] + 65536.0f * (float)ig[gq][2]);   // (16 * 63 * 2^22 exceeds 32 bits: the digits are combined in float)
           const float d = __half2float(__ushort_as_half((unsigned short)cur[r].d));
           acc[r] = d * (sA * (fg[0] + fg[1]) + sB * (fg[2] + fg[3]));
           continue;

@@ -96,6 +96,23 @@ def test_q6_k_gemv_matches_oracle(rows, cols, nb):
     assert rel_err(got, want, floor=0.02 * cols ** 0.5) < TIGHT
 
 
+def test_q6_k_largest_codes_on_equal_activations_do_not_overflow_the_integer_sums():
+    """16 codes of 63 against 16 activations at the top of the 23-bit range: 16 * 63 * (2^22 - 1) exceeds 32 bits, so the
+    batch-1 kernel combines its three digit sums in floating point."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    rows, cols = 6, 512
+    blk = np.zeros(210, np.uint8)
+    blk[:192] = 0xFF                                   # every code 63
+    blk[192:208] = np.array([1, 2, 3, 127, 1, 1, 5, 1, 9, 1, 1, 1, 77, 1, 1, 1], np.int8).view(np.uint8)
+    blk[208:210] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    raw = np.tile(blk, rows * cols // 256)
+    for x in (np.ones((1, cols), np.float32), -np.ones((1, cols), np.float32), np.full((1, cols), 3.0e4, np.float32)):
+        got = cai.QWeight(O.Q6_K, rows, cols, raw).gemv(x)
+        want = O.gemv(O.Q6_K, raw, rows, cols, x, None, 0, 1)
+        assert rel_err(got, want) < TIGHT
+
+
 def test_int8_row_path_scale_then_bias():
     # the reference's own fused-quant format: y = scale_a * sum(code*x) + bias_a (neuralvolume.pas:12693-12745)
     from helpers.device import dev, rel_err
