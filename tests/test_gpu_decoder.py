@@ -49,6 +49,11 @@ SHAPES = {
                                      eps=1e-5, rope_theta=1e4), qtype=O.Q4_0, head=None, bias=False),
     "olmoe_like_q8": dict(cfg=dict(n_layers=2, d_model=256, n_q_heads=4, n_kv_heads=4, head_dim=64, ffn=128, vocab=1500, max_ctx=96,
                                    eps=1e-5, rope_theta=1e4, n_experts=16, top_k=4, norm_topk=0, qk_norm_full=1), qtype=O.Q8_0, head=None, bias=False),
+    # expert banks in Q6_K (records, scales and d planes gathered per slot) and a dense Q6_K model on the integer-dot kernel
+    "moe_like_q6k": dict(cfg=dict(n_layers=2, d_model=256, n_q_heads=4, n_kv_heads=2, head_dim=64, ffn=256, vocab=900, max_ctx=96,
+                                  eps=1e-5, rope_theta=1e4, n_experts=8, top_k=2, norm_topk=1), qtype=O.Q6_K, head=None, bias=False),
+    "llama_like_q6k": dict(cfg=dict(n_layers=2, d_model=512, n_q_heads=8, n_kv_heads=2, head_dim=64, ffn=768, vocab=1100, max_ctx=96,
+                                    eps=1e-5, rope_theta=1e4), qtype=O.Q6_K, head=O.Q6_K, bias=True),
 }
 
 
