@@ -71,6 +71,38 @@ static int check_ready(cai_decoder_s* d)
 
 static bool is_block_quant(int qt) { return qt == CAI_Q4_K || qt == CAI_Q4_0 || qt == CAI_Q8_0; }
 
+// Expert half of a block for n_b (<= 8) activation rows x[b][d_model], in place: router -> soft-max -> top-k
+// gates -> gathered gate|up (RMSNorm and SwiGLU fused) -> gathered down -> gate-weighted mixture added to the row
+// (neural/neuralpretrained.pas:15331-15388; neural/neural.cl:2689-2752).
+static int moe_ffn_rows(cai_decoder_s* d, const cai_decoder_s::Layer& L, float* x, int n_b)
+{
+  const cai_decoder_config& c = d->cfg;
+  const int dm = c.d_model, I = c.ffn;
+  int rc;
+  const int E = c.n_experts, K = c.top_k;
+  MultiGemv r{}; r.n = 1; r.w[0] = L.w[CAI_W_ROUTER]; r.rows[0] = E;
+  if ((rc = launch_gemv_multi(r, x, n_b, d->router_logits, E, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;
+  launch_router_topk(d->router_logits, E, K, c.norm_topk, n_b, d->moe_expert, d->moe_gate, d->router_probs);
+  for (int b = 0; b < n_b; b++) {
+    MultiGemv g{}; g.n = 1; g.w[0] = L.w[CAI_W_GATEUP]; g.rows[0] = 2 * I;
+    g.slot_expert = d->moe_expert + b * K; g.n_slots = K; g.expert_rows = 2 * I; g.x_slot_stride = 0;
+    const float* xb = x + (int64_t)b * dm;
+    if (is_block_quant(g.w[0]->qtype)) {
+      g.y_slot_stride = I;
+      if ((rc = launch_gemv_multi(g, xb, 1, d->mid, I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, I))) return rc;
+    } else {
+      g.y_slot_stride = 2 * I;
+      if ((rc = launch_gemv_multi(g, xb, 1, d->gu, 2 * I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;
+      launch_swiglu(d->gu, I, K, d->mid);
+    }
+    MultiGemv dn{}; dn.n = 1; dn.w[0] = L.w[CAI_W_DOWN]; dn.rows[0] = dm;
+    dn.slot_expert = d->moe_expert + b * K; dn.n_slots = K; dn.expert_rows = dm; dn.x_slot_stride = I; dn.y_slot_stride = dm;
+    if ((rc = launch_gemv_multi(dn, d->mid, 1, d->moe_part, dm, CAI_ACT_NONE, nullptr, nullptr, 0.0f, 0))) return rc;
+    launch_moe_combine(x + (int64_t)b * dm, d->moe_part, d->moe_gate + b * K, K, dm, 1);
+  }
+  return CAI_OK;
+}
+
 // Enqueues one whole step for activation rows 0..n_b-1 mapped to cache sequences seq0..seq0+n_b-1.
 static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
 {
@@ -165,27 +197,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
         if ((rc = launch_gemv_multi(dn, d->mid, n_b, d->x, dm, CAI_ACT_NONE, d->x, nullptr, 0.0f, 0))) return rc;
       }
     } else {
-      const int E = c.n_experts, K = c.top_k;
-      MultiGemv r{}; r.n = 1; r.w[0] = L.w[CAI_W_ROUTER]; r.rows[0] = E;
-      if ((rc = launch_gemv_multi(r, d->x, n_b, d->router_logits, E, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;
-      launch_router_topk(d->router_logits, E, K, c.norm_topk, n_b, d->moe_expert, d->moe_gate, d->router_probs);
-      for (int b = 0; b < n_b; b++) {
-        MultiGemv g{}; g.n = 1; g.w[0] = L.w[CAI_W_GATEUP]; g.rows[0] = 2 * I;
-        g.slot_expert = d->moe_expert + b * K; g.n_slots = K; g.expert_rows = 2 * I; g.x_slot_stride = 0;
-        const float* xb = d->x + (int64_t)b * dm;
-        if (is_block_quant(g.w[0]->qtype)) {
-          g.y_slot_stride = I;
-          if ((rc = launch_gemv_multi(g, xb, 1, d->mid, I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, I))) return rc;
-        } else {
-          g.y_slot_stride = 2 * I;
-          if ((rc = launch_gemv_multi(g, xb, 1, d->gu, 2 * I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;
-          launch_swiglu(d->gu, I, K, d->mid);
-        }
-        MultiGemv dn{}; dn.n = 1; dn.w[0] = L.w[CAI_W_DOWN]; dn.rows[0] = dm;
-        dn.slot_expert = d->moe_expert + b * K; dn.n_slots = K; dn.expert_rows = dm; dn.x_slot_stride = I; dn.y_slot_stride = dm;
-        if ((rc = launch_gemv_multi(dn, d->mid, 1, d->moe_part, dm, CAI_ACT_NONE, nullptr, nullptr, 0.0f, 0))) return rc;
-        launch_moe_combine(d->x + (int64_t)b * dm, d->moe_part, d->moe_gate + b * K, K, dm, 1);
-      }
+      if ((rc = moe_ffn_rows(d, L, d->x, n_b))) return rc;
     }
   }
   {
@@ -264,6 +276,14 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
     if ((rc = launch_attn_step(&d->kv, l, d->pqkv, qkvw, n, c.n_q_heads, c.window, 0.0f, d->theta, poss, d->patt, qw, seq, 1, d->ppart,
                                c.qk_norm_full ? L.v[CAI_V_Q_NORM] : nullptr, c.qk_norm_full ? L.v[CAI_V_K_NORM] : nullptr, c.eps))) return rc;
     if ((rc = linear_rows(L.w[CAI_W_O], false, d->patt, qw, nullptr, 0.0f, n, d->px, dm, d->px))) return rc;
+    if (c.n_experts > 0) {
+      // experts differ from token to token: the routed half runs on groups of rows (one router / top-k launch per group,
+      // the gathered products per token), the attention half above on the whole chunk
+      const int grp = 8;
+      for (int t0 = 0; t0 < n; t0 += grp)
+        if ((rc = moe_ffn_rows(d, L, d->px + (int64_t)t0 * dm, std::min(grp, n - t0)))) return rc;
+      continue;
+    }
     if ((rc = linear_rows(L.w[CAI_W_GATEUP], false, d->px, dm, L.v[CAI_V_MLP_NORM], c.eps, n, d->pgu, 2 * I, nullptr))) return rc;
     launch_swiglu(d->pgu, I, n, d->pmid);
     if ((rc = linear_rows(L.w[CAI_W_DOWN], false, d->pmid, I, nullptr, 0.0f, n, d->px, dm, d->px))) return rc;
@@ -332,11 +352,12 @@ extern "C" int cai_decoder_create(const cai_decoder_config* cfg, cai_decoder_t* 
   if (e == hipSuccess) e = alloc_f(&d->mid, (size_t)std::max(B, K) * c.ffn);
   if (e == hipSuccess) e = alloc_f(&d->logits, (size_t)B * c.vocab);
   if (c.n_experts > 0) {
-    if (e == hipSuccess) e = alloc_f(&d->router_logits, (size_t)B * c.n_experts);
-    if (e == hipSuccess) e = alloc_f(&d->router_probs, (size_t)B * c.n_experts);
-    if (e == hipSuccess) e = alloc_f(&d->moe_gate, (size_t)B * K);
+    // (eight rows whatever the batch: a prompt routes its tokens in groups of eight)
+    if (e == hipSuccess) e = alloc_f(&d->router_logits, (size_t)8 * c.n_experts);
+    if (e == hipSuccess) e = alloc_f(&d->router_probs, (size_t)8 * c.n_experts);
+    if (e == hipSuccess) e = alloc_f(&d->moe_gate, (size_t)8 * K);
     if (e == hipSuccess) e = alloc_f(&d->moe_part, (size_t)K * c.d_model);
-    if (e == hipSuccess) e = hipMalloc((void**)&d->moe_expert, (size_t)B * K * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMalloc((void**)&d->moe_expert, (size_t)8 * K * sizeof(int32_t));
   }
   const int ame = argmax_scratch_entries(c.vocab, B);
   if (e == hipSuccess) e = alloc_f(&d->am_v, (size_t)ame);
@@ -494,7 +515,7 @@ extern "C" int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* toke
   Context& cx = ctx();
   const char* tok_env = getenv("CAIHIP_PREFILL_TOKENWISE");
   // (a prompt that runs past the eviction cap overwrites ring rows its own earlier tokens still need: token by token then)
-  const bool tokenwise = c.n_experts > 0 || n == 1 || (tok_env && tok_env[0] == '1') || (d->kv.evict_cap > 0 && pos0 + n > d->kv.evict_cap);
+  const bool tokenwise = n == 1 || (tok_env && tok_env[0] == '1') || (d->kv.evict_cap > 0 && pos0 + n > d->kv.evict_cap);
   if (tokenwise) {
     // Token-at-a-time ingestion, the reference's own prefill (neural/neuralchatengine.pas:1466-1470).
     for (int i = 0; i < n; i++) {

@@ -187,6 +187,31 @@ def test_batched_decode_and_prompt_of_a_q4k_q6k_mix_equal_single_steps():
     assert rel_err(lg, last) < 1e-3 and am == int(np.argmax(last))
 
 
+@pytest.mark.parametrize("name,n", [("olmoe_like_q8", 11), ("olmoe_like_q8", 45), ("moe_like_q6k", 29)])
+def test_moe_prefill_equals_sequential_steps(name, n):
+    """Mixture-of-experts prompts: attention half on the whole chunk, routed half per group of rows (router and top-k once
+    per group, the gathered expert products per token) == token-at-a-time steps."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    s = SHAPES[name]
+    spec = synthetic_spec(s["cfg"], s["qtype"], head_qtype=s["head"], qkv_bias=s["bias"], std=0.05)
+    dec = cai.Decoder(spec, max_batch=3)
+    rng = np.random.default_rng(n)
+    toks = [int(t) for t in rng.integers(0, spec["cfg"]["vocab"], n)]
+    last = None
+    for p, t in enumerate(toks):
+        _, last = dec.step(t, p)
+    am, lg = dec.prefill(toks, 0, seq=1)
+    assert rel_err(lg, last[0]) < 1e-3 and am == int(np.argmax(last[0]))
+    assert dec.len(1) == n
+    # the ingested cache continues like the stepped one
+    a0, l0 = dec.step(7, n)
+    dec2 = cai.Decoder(spec, max_batch=1)
+    dec2.prefill(toks, 0)
+    a1, l1 = dec2.step(7, n)
+    assert rel_err(l1[0], l0[0]) < 1e-3
+
+
 def test_prefill_equals_sequential_steps():
     from helpers.device import dev, rel_err
     cai = dev()
