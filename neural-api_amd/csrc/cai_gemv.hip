@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
     if (MODE == 1 && (r & 1)) row += p.half;
     rp[r] = sg.data + (bank_row + row) * row_bytes;
     ap[r] = sg.aux + (bank_row + row) * aux_row_bytes;
-    dp[r] = QT == CAI_Q6_K ? sg.aux2 + (bank_row + row) * (int64_t)(cols >> 8) * 2 : nullptr;
+    dp[r] = QT == CAI_Q6_K ? p.seg_aux2[s] + (bank_row + row) * (int64_t)(cols >> 8) * 2 : nullptr;
   }
 
   float acc[RR][NB];
@@ -606,7 +606,7 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
       return set_error(CAI_ERR_INVALID, "gemv: row range [%lld,+%lld) outside matrix of %lld rows", (long long)m.row0[i], (long long)m.rows[i], (long long)w->rows);
     p.seg[i].data = w->data + m.row0[i] * data_row_bytes(w);
     p.seg[i].aux = w->aux ? w->aux + m.row0[i] * aux_row_bytes(w) : nullptr;
-    p.seg[i].aux2 = w->qtype == CAI_Q6_K ? qw_aux2(w) + m.row0[i] * (w->cols / 256) * 2 : nullptr;
+    p.seg_aux2[i] = w->qtype == CAI_Q6_K ? qw_aux2(w) + m.row0[i] * (w->cols / 256) * 2 : nullptr;
     p.seg[i].bias = w->bias ? w->bias + m.row0[i] : nullptr;
     p.seg[i].rows = (int)m.rows[i];
     p.seg[i].y_off = m.y_off[i];

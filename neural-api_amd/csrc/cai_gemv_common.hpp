@@ -45,7 +45,7 @@ __device__ __forceinline__ float silu_mul(float up, float gate)
 constexpr int SSQ_PARTS = 1024;   // slots of a sum-of-squares partial array (>= any producer grid)
 
 struct GemvSeg {
-  const uint8_t* data; const uint8_t* aux; const uint8_t* aux2; const float* bias;   // aux2: Q6_K plane of d
+  const uint8_t* data; const uint8_t* aux; const float* bias;
   int rows;       // rows of this segment computed by the launch
   int y_off;      // offset of the segment's first output inside a y row
   int grp_end;    // cumulative row-group count (exclusive)
@@ -68,6 +68,9 @@ struct GemvParams {
   int half;              // swiglu: rows [0,half) are up, [half,2*half) gate
   // expert-bank gather (MoE): blockIdx.y = slot; the slot's expert id selects a row window of the bank
   const int32_t* slot_expert; int64_t expert_rows; int x_slot_stride; int y_slot_stride;
+  // Q6_K: per segment the plane of d (kept behind the fields every launch reads: a wider segment record measured 2 % on the
+  // launch-bound MoE step)
+  const uint8_t* seg_aux2[3];
 };
 
 __device__ __forceinline__ float cvt_ub0(uint32_t v) { return (float)(v & 0xffu); }

@@ -123,7 +123,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
         rg[r].b0 = *reinterpret_cast<const uint4*>(blk + 64 * nh + 32); rg[r].b1 = *reinterpret_cast<const uint4*>(blk + 64 * nh + 48);
         rg[r].h0 = *reinterpret_cast<const uint4*>(blk + 128 + 32 * nh); rg[r].h1 = *reinterpret_cast<const uint4*>(blk + 144 + 32 * nh);
         rg[r].sc = *reinterpret_cast<const uint2*>(sg->aux + b * 16 + 8 * nh);
-        rg[r].d = *reinterpret_cast<const uint16_t*>(sg->aux2 + b * 2);
+        rg[r].d = *reinterpret_cast<const uint16_t*>(p.seg_aux2[0] + b * 2);   // (Q6_K launches hold one segment)
       } else if constexpr (QT == CAI_Q4_0) {
         // quants plane: the lane's two 32-weight blocks are 32 contiguous bytes; scales plane: their two halfs one dword
         rg[r].q0 = *reinterpret_cast<const uint4*>(blk + 32 * cc);
