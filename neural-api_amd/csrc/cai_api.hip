@@ -25,6 +25,7 @@ int set_error(int code, const char* fmt, ...)
 
 int hip_fail(hipError_t e, const char* what, const char* file, int line)
 {
+  (void)hipGetLastError();   // the runtime keeps the error until someone reads it: a later, unrelated launch check would report it again
   return set_error(e == hipErrorOutOfMemory ? CAI_ERR_NOMEM : CAI_ERR_HIP, "%s failed: %s (%s:%d)", what, hipGetErrorString(e), file, line);
 }
 
@@ -205,7 +206,7 @@ extern "C" int cai_qw_create(int qtype, int64_t rows, int64_t cols, const void* 
     const int bb = (int)block_bytes(qtype);
     w->data_bytes = n_blocks * (bb - 2); w->aux_bytes = n_blocks * 2;
     void* raw = nullptr;
-    if (hipMalloc(&raw, (size_t)raw_bytes) != hipSuccess) return fail(set_error(CAI_ERR_NOMEM, "cai_qw_create: out of device memory (%lld bytes staging)", (long long)raw_bytes));
+    if (hipMalloc(&raw, (size_t)raw_bytes) != hipSuccess) return (void)hipGetLastError(), fail(set_error(CAI_ERR_NOMEM, "cai_qw_create: out of device memory (%lld bytes staging)", (long long)raw_bytes));
     hipError_t e = hipMalloc((void**)&w->data, (size_t)w->data_bytes);
     if (e == hipSuccess) e = hipMalloc((void**)&w->aux, (size_t)w->aux_bytes);
     if (e == hipSuccess) e = hipMemcpyAsync(raw, blocks, (size_t)raw_bytes, hipMemcpyDefault, c.stream);
@@ -216,7 +217,7 @@ extern "C" int cai_qw_create(int qtype, int64_t rows, int64_t cols, const void* 
     const int64_t n_blocks = rows * (cols / 256);
     w->data_bytes = n_blocks * 192; w->aux_bytes = n_blocks * 18;
     void* raw = nullptr;
-    if (hipMalloc(&raw, (size_t)raw_bytes) != hipSuccess) return fail(set_error(CAI_ERR_NOMEM, "cai_qw_create: out of device memory (%lld bytes staging)", (long long)raw_bytes));
+    if (hipMalloc(&raw, (size_t)raw_bytes) != hipSuccess) return (void)hipGetLastError(), fail(set_error(CAI_ERR_NOMEM, "cai_qw_create: out of device memory (%lld bytes staging)", (long long)raw_bytes));
     hipError_t e = hipMalloc((void**)&w->data, (size_t)w->data_bytes);
     if (e == hipSuccess) e = hipMalloc((void**)&w->aux, (size_t)w->aux_bytes);
     if (e == hipSuccess) e = hipMemcpyAsync(raw, blocks, (size_t)raw_bytes, hipMemcpyDefault, c.stream);

@@ -82,7 +82,7 @@ static int moe_ffn_rows(cai_decoder_s* d, const cai_decoder_s::Layer& L, float* 
   const int E = c.n_experts, K = c.top_k;
   MultiGemv r{}; r.n = 1; r.w[0] = L.w[CAI_W_ROUTER]; r.rows[0] = E;
   if ((rc = launch_gemv_multi(r, x, n_b, d->router_logits, E, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;
-  launch_router_topk(d->router_logits, E, K, c.norm_topk, n_b, d->moe_expert, d->moe_gate, d->router_probs);
+  if ((rc = launch_router_topk(d->router_logits, E, K, c.norm_topk, n_b, d->moe_expert, d->moe_gate, d->router_probs))) return rc;
   for (int b = 0; b < n_b; b++) {
     MultiGemv g{}; g.n = 1; g.w[0] = L.w[CAI_W_GATEUP]; g.rows[0] = 2 * I;
     g.slot_expert = d->moe_expert + b * K; g.n_slots = K; g.expert_rows = 2 * I; g.x_slot_stride = 0;
@@ -327,7 +327,7 @@ using namespace cai;
 
 extern "C" int cai_decoder_create(const cai_decoder_config* cfg, cai_decoder_t* out)
 {
-  CAI_READY();
+  // (the shape is checked before the device is: a refused configuration is refused on any machine)
   CAI_REQUIRE(cfg && out, "cai_decoder_create: null argument");
   const cai_decoder_config& c = *cfg;
   CAI_REQUIRE(c.n_layers > 0 && c.d_model > 0 && c.n_q_heads > 0 && c.n_kv_heads > 0 && c.head_dim > 0 && c.ffn > 0 && c.vocab > 0 && c.max_ctx > 0,
@@ -335,12 +335,15 @@ extern "C" int cai_decoder_create(const cai_decoder_config* cfg, cai_decoder_t* 
   CAI_REQUIRE(c.n_q_heads % c.n_kv_heads == 0 && c.n_q_heads / c.n_kv_heads <= 8, "cai_decoder_create: %d query heads per %d KV heads unsupported", c.n_q_heads, c.n_kv_heads);
   CAI_REQUIRE(c.max_batch >= 1 && c.max_batch <= 8, "cai_decoder_create: max_batch %d outside 1..8", c.max_batch);
   CAI_REQUIRE(c.n_experts == 0 || (c.top_k >= 1 && c.top_k <= c.n_experts && c.top_k <= 64), "cai_decoder_create: top_k %d of %d experts", c.top_k, c.n_experts);
+  // the router kernel ranks at most 512 experts; a larger bank would leave the gather's expert ids unwritten
+  CAI_REQUIRE(c.n_experts >= 0 && c.n_experts <= 512, "cai_decoder_create: %d experts (supported: up to 512)", c.n_experts);
+  CAI_READY();
   cai_decoder_s* d = new cai_decoder_s();
   d->cfg = c;
   d->layers.resize(c.n_layers);
   const int B = c.max_batch, qw = d->qw(), kw = d->kw();
   int rc = kv_alloc(&d->kv, B, c.n_layers, c.n_kv_heads, c.head_dim, c.max_ctx, c.kv_dtype);
-  if (rc) { delete d; return rc; }
+  if (rc) { kv_free(&d->kv); delete d; return rc; }
   std::vector<float> th; rope_thetas(c.rope_theta, c.head_dim, th);
   auto alloc_f = [&](float** p, size_t n) { return hipMalloc((void**)p, n * sizeof(float)); };
   hipError_t e = alloc_f(&d->theta, th.size());

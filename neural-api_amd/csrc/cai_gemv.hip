@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
   int64_t bank_row = 0;
   const float* xin = p.x; float* yout = p.y;
   if (p.slot_expert) {
-    bank_row = (int64_t)p.slot_expert[blockIdx.y] * p.expert_rows;
+    bank_row = (int64_t)min(max(p.slot_expert[blockIdx.y], 0), p.bank_experts - 1) * p.expert_rows;   // an id outside the bank (a router fed NaN) must not address memory
     xin += (int64_t)blockIdx.y * p.x_slot_stride; yout += (int64_t)blockIdx.y * p.y_slot_stride;
   }
 
@@ -450,7 +450,7 @@ __global__ __launch_bounds__(256) void gemv_simple(const GemvParams p, int n_b)
   int64_t bank_row = 0;
   const float* xin = p.x; float* yout = p.y;
   if (p.slot_expert) {
-    bank_row = (int64_t)p.slot_expert[blockIdx.y] * p.expert_rows;
+    bank_row = (int64_t)min(max(p.slot_expert[blockIdx.y], 0), p.bank_experts - 1) * p.expert_rows;   // an id outside the bank (a router fed NaN) must not address memory
     xin += (int64_t)blockIdx.y * p.x_slot_stride; yout += (int64_t)blockIdx.y * p.y_slot_stride;
   }
   const int64_t wrow = bank_row + row;
@@ -599,6 +599,11 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
   p.ssq_in = nullptr; p.ssq_out = nullptr;
   p.slot_expert = m.slot_expert; p.expert_rows = m.expert_rows; p.x_slot_stride = m.x_slot_stride; p.y_slot_stride = m.y_slot_stride;
   const int n_slots = m.slot_expert ? m.n_slots : 1;
+  if (m.slot_expert) {
+    if (m.n != 1 || m.expert_rows <= 0 || w0->rows % m.expert_rows || m.row0[0] != 0 || m.rows[0] > m.expert_rows)
+      return set_error(CAI_ERR_INVALID, "gemv: expert bank of %lld rows does not divide into windows of %lld", (long long)w0->rows, (long long)m.expert_rows);
+    p.bank_experts = (int)(w0->rows / m.expert_rows);
+  }
   for (int i = 0; i < m.n; i++) {
     const cai_qw_s* w = m.w[i];
     if (w->qtype != w0->qtype || w->cols != w0->cols) return set_error(CAI_ERR_INVALID, "gemv: fused matrices differ in type or width");

@@ -68,6 +68,7 @@ struct GemvParams {
   int half;              // swiglu: rows [0,half) are up, [half,2*half) gate
   // expert-bank gather (MoE): blockIdx.y = slot; the slot's expert id selects a row window of the bank
   const int32_t* slot_expert; int64_t expert_rows; int x_slot_stride; int y_slot_stride;
+  int bank_experts;      // experts in the bank: a slot's id is clamped to [0, bank_experts) before it addresses rows
   // Q6_K: per segment the plane of d (kept behind the fields every launch reads: a wider segment record measured 2 % on the
   // launch-bound MoE step)
   const uint8_t* seg_aux2[3];

@@ -303,6 +303,16 @@ int argmax_scratch_entries(int n, int n_rows) { return (n + 4095) / 4096 * n_row
 // One wave per token; lane i owns experts i, i+64, ...  Selection is k rounds of a wave-wide arg-max in which the
 // larger probability wins and, between equals, the lower expert index (the reference scans upwards with '>').
 constexpr int ROUTER_MAX_PER_LANE = 8;   // up to 512 experts
+// Selection key of a probability: larger key = selected earlier.  A total order whatever the value: lanes that hold no expert
+// get 0, a NaN (a poisoned activation row reaches the router as NaN logits) ranks below every number, and probabilities are
+// non-negative, so their bit patterns order like their values.  With a total order the k selected experts are always k
+// distinct ids inside [0, n); the gates still carry the NaN to the outputs.
+__device__ __forceinline__ uint32_t router_key(float p, bool candidate)
+{
+  if (!candidate) return 0u;
+  if (!(p == p)) return 1u;
+  return __builtin_bit_cast(uint32_t, fmaxf(p, 0.0f)) + 2u;
+}
 __global__ __launch_bounds__(64) void router_topk_kernel(const float* logits, int n, int k, int renorm, int n_tokens, int32_t* expert_out, float* gate_out, float* probs)
 {
   const int t = blockIdx.x, lane = threadIdx.x;
@@ -337,10 +347,11 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float* logits, in
     // One expert per lane: every lane ranks its own probability against the 64 broadcast ones (larger first, lower
     // index between equals) - a permutation of 0..63 - and the lanes of rank 0..k-1 are the selection, in order.
     const float pv = v[0];
+    const uint32_t key = router_key(pv, lane < n);
     int rank = 0;
     for (int j = 0; j < 64; j++) {
-      const float o = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pv), j));
-      rank += (o > pv || (o == pv && j < lane)) ? 1 : 0;
+      const uint32_t o = (uint32_t)__builtin_amdgcn_readlane((int)key, j);
+      rank += (o > key || (o == key && j < lane)) ? 1 : 0;
     }
     for (int j = 0; j < k; j++) {
       const int src = __ffsll((unsigned long long)__ballot(rank == j)) - 1;
@@ -351,18 +362,21 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float* logits, in
     if (lane < k) gate_out[t * k + lane] = renorm ? (sum > 0.0f ? mine * (1.0f / sum) : 0.0f) : mine;
     return;
   }
-  for (int j = 0; j < k; j++) {
-    float bv = -1.0f; int bc = 0x7fffffff;
+  uint32_t key[ROUTER_MAX_PER_LANE];
+#pragma unroll
+  for (int i = 0; i < ROUTER_MAX_PER_LANE; i++) key[i] = router_key(v[i], lane + 64 * i < n);
+  for (int j = 0; j < k; j++) {   // k <= n: an expert that has not been taken (key >= 1) exists in every round
+    uint32_t bk = 0u; float bv = 0.0f; int bc = 0x7fffffff;
 #pragma unroll
     for (int i = 0; i < ROUTER_MAX_PER_LANE; i++)
-      if (v[i] > bv) { bv = v[i]; bc = lane + 64 * i; }   // ascending index inside the lane: '>' keeps the first
+      if (key[i] > bk) { bk = key[i]; bv = v[i]; bc = lane + 64 * i; }   // ascending index inside the lane: '>' keeps the first
     for (int m = 32; m >= 1; m >>= 1) {
-      const float ov = __shfl_xor(bv, m, 64); const int oc = __shfl_xor(bc, m, 64);
-      if (ov > bv || (ov == bv && oc < bc)) { bv = ov; bc = oc; }
+      const uint32_t ok = __shfl_xor(bk, m, 64); const float ov = __shfl_xor(bv, m, 64); const int oc = __shfl_xor(bc, m, 64);
+      if (ok > bk || (ok == bk && oc < bc)) { bk = ok; bv = ov; bc = oc; }
     }
     if ((bc & 63) == lane) {
 #pragma unroll
-      for (int i = 0; i < ROUTER_MAX_PER_LANE; i++) if (bc == lane + 64 * i) v[i] = -1.0f;   // taken
+      for (int i = 0; i < ROUTER_MAX_PER_LANE; i++) if (bc == lane + 64 * i) key[i] = 0u;   // taken
     }
     if (lane == (j & 63)) { mine = bv; expert_out[t * k + j] = bc; }
     sum += bv;
@@ -490,7 +504,7 @@ extern "C" int cai_router_topk(const float* logits, int n, int k, int renorm, in
   if ((rc = stage_input(logits, (size_t)n * 4, flags & CAI_X_DEVICE, &dx))) return rc;
   if ((rc = stage_output(nullptr, (size_t)n * 4, 0, &dscr))) return rc;
   int32_t* d_e = c.d_small; float* d_g = reinterpret_cast<float*>(c.d_small + 64);
-  launch_router_topk((const float*)dx, n, k, renorm, 1, d_e, d_g, (float*)dscr);
+  if ((rc = launch_router_topk((const float*)dx, n, k, renorm, 1, d_e, d_g, (float*)dscr))) return rc;
   CAI_HIP(hipMemcpyAsync(c.h_small, c.d_small, 128 * 4, hipMemcpyDeviceToHost, c.stream));
   CAI_HIP(hipStreamSynchronize(c.stream));
   for (int j = 0; j < k; j++) { expert_out[j] = c.h_small[j]; memcpy(&gate_out[j], &c.h_small[64 + j], 4); }

@@ -38,3 +38,62 @@ def test_header_is_plain_c():
         path = f.name
     subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-fsyntax-only", "-I", os.path.join(ROOT, "include"), path])
     os.unlink(path)
+
+
+def header_arities():
+    with open(os.path.join(ROOT, "include", "caihip.h")) as f:
+        text = re.sub(r"/\*.*?\*/", "", f.read(), flags=re.S)
+    out = {}
+    for name, args in re.findall(r"^\s*int\s+(cai_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text, re.M | re.S):
+        args = args.strip()
+        out[name] = 0 if args in ("", "void") else len(args.split(","))
+    return out
+
+
+def pascal_arities():
+    with open(os.path.join(ROOT, "neural-api_amd", "pascal", "caihip.pas")) as f:
+        text = f.read()
+    out = {}
+    for name, args in re.findall(r"^function\s+(cai_[a-z0-9_]+)\s*\(([^)]*)\)\s*:\s*LongInt\s*;\s*cdecl\s*;\s*external\s+CAIHIP_LIB\s*;", text, re.M | re.S):
+        n = 0
+        for group in args.split(";"):
+            if group.strip():
+                n += len(group.split(":")[0].split(","))
+        out[name] = n
+    return out
+
+
+def test_pascal_unit_declares_the_header_symbols_with_the_same_arities():
+    """The Free Pascal binding cannot be compiled here (no fpc): at least its externals must name exactly the header's
+    entry points, each with the header's number of parameters, every one cdecl and returning a 32-bit integer."""
+    h, p = header_arities(), pascal_arities()
+    assert sorted(h) == header_symbols()
+    assert sorted(p) == sorted(h), "only in header: %s; only in caihip.pas: %s" % (sorted(set(h) - set(p)), sorted(set(p) - set(h)))
+    for name in h:
+        assert p[name] == h[name], "%s: %d parameters in caihip.h, %d in caihip.pas" % (name, h[name], p[name])
+
+
+def test_decoder_config_record_matches_the_struct():
+    """Field order and count of TCaiDecoderConfig against cai_decoder_config (both packed 4-byte fields)."""
+    with open(os.path.join(ROOT, "include", "caihip.h")) as f:
+        body = re.search(r"typedef struct cai_decoder_config \{(.*?)\} cai_decoder_config;", f.read(), re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    c_fields = [n.strip() for decl in body.split(";") if decl.strip() for n in re.sub(r"^\s*(int32_t|float)\s+", "", decl.strip()).split(",")]
+    with open(os.path.join(ROOT, "neural-api_amd", "pascal", "caihip.pas")) as f:
+        rec = re.search(r"TCaiDecoderConfig = packed record(.*?)end;", f.read(), re.S).group(1)
+    p_fields = [n.strip() for decl in rec.split(";") if decl.strip() for n in decl.split(":")[0].split(",")]
+    assert p_fields == c_fields == [n for n, _ in cai.DecoderConfig._fields_]
+
+
+def test_more_experts_than_the_router_ranks_are_refused_without_a_device():
+    """512 experts is what the router kernel ranks; a larger bank is refused when the decoder is created (before any device
+    work, so the answer is the same on a machine without a GPU) instead of leaving expert ids unwritten."""
+    import ctypes as C
+    lib = cai.load()
+    cfg = cai.DecoderConfig(n_layers=1, d_model=256, n_q_heads=2, n_kv_heads=2, head_dim=64, ffn=256, vocab=100, max_ctx=16, eps=1e-5,
+                            rope_theta=1e4, n_experts=1024, top_k=8, max_batch=1)
+    h = C.c_void_p()
+    assert lib.cai_decoder_create(C.byref(cfg), C.byref(h)) == -1
+    assert "1024 experts" in cai.last_error()
+    cfg.n_experts, cfg.top_k = 8, 9
+    assert lib.cai_decoder_create(C.byref(cfg), C.byref(h)) == -1

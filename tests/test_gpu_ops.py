@@ -86,3 +86,28 @@ def test_router_softmax_topk():
     e = np.empty(2, np.int32); g = np.empty(2, np.float32)
     cai.check(cai.load().cai_router_topk(logits.ctypes.data, 4, 2, 1, e.ctypes.data, g.ctypes.data, 0))
     assert list(e) == [0, 2] and np.allclose(g, [0.625, 0.375], atol=1e-5)
+
+
+@pytest.mark.parametrize("n,k", [(64, 8), (16, 4), (200, 8), (512, 64)])
+def test_router_selection_stays_inside_the_bank_on_non_finite_logits(n, k):
+    """A poisoned activation row reaches the router as NaN logits.  The selection must still be k DISTINCT experts inside
+    [0, n) (the ids address rows of the expert bank); the NaN travels on in the gates.  Also checked: the large-expert path
+    (more than 64) against the oracle on ordinary logits, and the refusal of more experts than the kernel ranks."""
+    from helpers.device import dev
+    cai = dev()
+    rng = np.random.default_rng(n + k)
+    e = np.empty(k, np.int32); g = np.empty(k, np.float32)
+    rows = [np.full(n, np.nan, np.float32), np.full(n, np.inf, np.float32), rng.standard_normal(n).astype(np.float32)]
+    rows[2][::3] = np.nan
+    for logits in rows:
+        e[:] = -7
+        cai.check(cai.load().cai_router_topk(logits.ctypes.data, n, k, 0, e.ctypes.data, g.ctypes.data, 0))
+        assert e.min() >= 0 and e.max() < n and len(set(e.tolist())) == k, e
+    logits = rng.standard_normal(n).astype(np.float32) * 2
+    cai.check(cai.load().cai_router_topk(logits.ctypes.data, n, k, 1, e.ctypes.data, g.ctypes.data, 0))
+    p = np.empty(n, np.float32); O.lib().orc_softmax(logits.ctypes.data, n, p.ctypes.data)
+    gw = np.zeros(n, np.float32); iw = np.zeros(k, np.int32)
+    O.lib().orc_topk_gate(p.ctypes.data, n, k, 1, gw.ctypes.data, iw.ctypes.data)
+    assert list(e) == list(iw) and np.allclose(g, gw[iw], rtol=1e-5, atol=1e-7)
+    big = np.zeros(1024, np.float32)
+    assert cai.load().cai_router_topk(big.ctypes.data, 1024, 8, 0, e.ctypes.data, g.ctypes.data, 0) == -4   # CAI_ERR_UNSUPPORTED
