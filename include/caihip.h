@@ -133,6 +133,12 @@ int cai_rope(float* x, int n_heads, int head_dim, int pos, float theta_base, int
 int cai_swiglu(const float* x, int half, int n_tokens, float* y, int flags);
 /* ArgMaxRow (neural/neuralchatengine.pas:683-697): lowest index wins ties. */
 int cai_argmax(const float* x, int n, int32_t* index_out, int flags);
+/* cai_argmax for callers that cannot allocate device memory or wait (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc); it has no counterpart in the reference.  x_dev and index_out_dev are device pointers;
+ * the two launches go to the library stream and the call returns without waiting.  The slice winners between the two
+ * launches live in a fixed 8 KiB array inside the library (one copy per GPU, held until the process ends), which bounds
+ * n at 4 194 304 (CAI_ERR_INVALID beyond).  Calls that overlap on one GPU share that array and race. */
+int cai_argmax_noalloc(const float* x_dev, int n, int32_t* index_out_dev);
 /* TNNetPointwiseSoftMax + TNNetTopKGate (neural/neuralpretrained.pas:15347-15365):
  * softmax over n experts, keep top-k, renormalise iff renorm.  Outputs are host arrays of k. */
 int cai_router_topk(const float* logits, int n, int k, int renorm, int32_t* expert_out, float* gate_out, int flags);

@@ -17,7 +17,7 @@ V_ATTN_NORM, V_MLP_NORM, V_FINAL_NORM, V_Q_NORM, V_K_NORM = range(5)
 SYMBOLS = """cai_init cai_shutdown cai_last_error cai_device_name cai_sync cai_get_stream cai_timer_start cai_timer_stop
 cai_dev_alloc cai_dev_free cai_dev_upload cai_dev_download cai_dev_copy
 cai_qw_create cai_qw_create_int8row cai_qw_destroy cai_qw_info cai_qw_dequant_rows cai_qgemv cai_ffn_gateup cai_qgemm
-cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_router_topk
+cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_argmax_noalloc cai_router_topk
 cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_kv_export_layer cai_kv_import_layer cai_kv_set_eviction cai_kv_rows cai_attn_decode
 cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_generate
 cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_set_eviction cai_decoder_cache_rows cai_decoder_set_kv_dtype cai_sample_candidates cai_decoder_candidates cai_decoder_snapshot cai_decoder_restore
@@ -72,6 +72,7 @@ def load():
         L.cai_rope.argtypes = [vp, i32, i32, i32, f32, i32]
         L.cai_swiglu.argtypes = [vp, i32, i32, vp, i32]
         L.cai_argmax.argtypes = [vp, i32, vp, i32]
+        L.cai_argmax_noalloc.argtypes = [vp, i32, vp]
         L.cai_router_topk.argtypes = [vp, i32, i32, i32, vp, vp, i32]
         L.cai_kv_create.argtypes = [i32, i32, i32, i32, i32, C.POINTER(vp)]
         L.cai_kv_destroy.argtypes = [vp]

@@ -78,6 +78,7 @@ extern "C" int cai_init(int device_ordinal)
   CAI_HIP(hipEventCreate(&c.ev1));
   CAI_HIP(hipMalloc(&c.d_small, 1024 * sizeof(int32_t)));
   CAI_HIP(hipHostMalloc(&c.h_small, 1024 * sizeof(int32_t), hipHostMallocDefault));
+  { const int rc = noalloc_setup(device_ordinal); if (rc) return rc; }
   c.ready = true;
   return CAI_OK;
 }

@@ -163,6 +163,7 @@ int launch_swiglu(const float* x, int half, int n_tokens, float* y);
 int launch_add(float* x, const float* y, int64_t n);
 int launch_argmax(const float* x, int n, int n_rows, int32_t* out, float* scratch_v, int32_t* scratch_i);
 int argmax_scratch_entries(int n, int n_rows);
+int noalloc_setup(int device);   // resolves the device address of the fixed scratch array (cai_init, device current)
 int launch_embed(const cai_qw_s* w, const int32_t* tokens_dev, int n_tokens, float* out);
 int launch_router_topk(const float* logits, int n, int k, int renorm, int n_tokens, int32_t* expert_out, float* gate_out, float* probs_scratch);
 int launch_rmsnorm_strided(const float* x, const float* gain, int n, int n_tokens, float eps, float* y, int64_t x_stride, int64_t y_stride);

@@ -299,6 +299,25 @@ int launch_argmax(const float* x, int n, int n_rows, int32_t* out, float* scratc
 }
 int argmax_scratch_entries(int n, int n_rows) { return (n + 4095) / 4096 * n_rows; }
 
+// ---- arg-max for callers that cannot allocate (cai_argmax_noalloc) ----
+// The slice winners of stage 1 (one float + one index per 4096 elements) go to a file-scope device array instead of the
+// staging buffer cai_argmax grows on demand.  Every GPU holds its own copy of the array at its own address: the address is
+// looked up once per device, with that device current, and host code only ever uses that pointer.
+constexpr int NOALLOC_MAX_SLICES = 1024;                     // rows of up to 4096 * 1024 = 4 194 304 elements
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_MAX_SLICES * 8];
+static void* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {nullptr};
+
+int noalloc_setup(int device)
+{
+  if (device < 0 || device >= NOALLOC_MAX_DEVICES) return set_error(CAI_ERR_INVALID, "device ordinal %d outside 0..%d", device, NOALLOC_MAX_DEVICES - 1);
+  if (g_scratch_ptr[device]) return CAI_OK;
+  void* ptr = nullptr;
+  CAI_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+  g_scratch_ptr[device] = ptr;
+  return CAI_OK;
+}
+
 // ---- router: TNNetPointwiseSoftMax (neural/neural.cl:1594-1647) + TNNetTopKGate ----
 // One wave per token; lane i owns experts i, i+64, ...  Selection is k rounds of a wave-wide arg-max in which the
 // larger probability wins and, between equals, the lower expert index (the reference scans upwards with '>').
@@ -492,6 +511,23 @@ extern "C" int cai_argmax(const float* x, int n, int32_t* index_out, int flags)
   CAI_HIP(hipMemcpyAsync(c.h_small, c.d_small, 4, hipMemcpyDeviceToHost, c.stream));
   CAI_HIP(hipStreamSynchronize(c.stream));
   *index_out = c.h_small[0];
+  return CAI_OK;
+}
+
+// No hipMalloc, no hipFree, no copy, no wait: two launches on the library stream.  Stage 1 writes every slot stage 2 reads
+// (slices 0 .. ceil(n / 4096) - 1), so nothing in the array has to be cleared between calls; calls that overlap on one GPU
+// would share the array and race.
+extern "C" int cai_argmax_noalloc(const float* x_dev, int n, int32_t* index_out_dev)
+{
+  CAI_READY();
+  CAI_REQUIRE(x_dev && index_out_dev && n > 0, "cai_argmax_noalloc: bad argument");
+  if (n > 4096 * NOALLOC_MAX_SLICES)
+    return set_error(CAI_ERR_INVALID, "cai_argmax_noalloc: %d elements exceed the fixed scratch of %d (use cai_argmax)", n, 4096 * NOALLOC_MAX_SLICES);
+  void* ptr = g_scratch_ptr[ctx().device];
+  if (!ptr) return set_error(CAI_ERR_STATE, "cai_argmax_noalloc: scratch address of device %d was not resolved at cai_init", ctx().device);
+  const int ne = argmax_scratch_entries(n, 1);
+  launch_argmax(x_dev, n, 1, index_out_dev, (float*)ptr, (int32_t*)ptr + ne);
+  CAI_HIP(hipGetLastError());
   return CAI_OK;
 }
 

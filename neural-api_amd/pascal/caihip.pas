@@ -67,6 +67,7 @@ function cai_rmsnorm(x, gain_host: PSingle; n, n_tokens: LongInt; eps: Single; y
 function cai_rope(x: PSingle; n_heads, head_dim, pos: LongInt; theta_base: Single; flags: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_swiglu(x: PSingle; half, n_tokens: LongInt; y: PSingle; flags: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_argmax(x: PSingle; n: LongInt; index_out: PLongInt; flags: LongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_argmax_noalloc(x_dev: PSingle; n: LongInt; index_out_dev: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_router_topk(logits: PSingle; n, k, renorm: LongInt; expert_out: PLongInt; gate_out: PSingle; flags: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 
 function cai_kv_create(n_layers, kv_heads, head_dim, max_ctx, kv_dtype: LongInt; out_kv: PCaiKV): LongInt; cdecl; external CAIHIP_LIB;
