@@ -118,7 +118,53 @@ struct AttnParams {
   int64_t seq_rows, layer_row_off;
   int evict_sinks, evict_cap;  // cap > 0: only the first `sinks` positions and the latest cap - sinks stay cached
   const float* qn_gain; const float* kn_gain; float qk_eps;   // full-width RMSNorm of q and of k applied while they are read (null: rows are used as they are)
+  unsigned* merge_cnt;         // decode steps: arrival counters [seq][head]; the work-group that completes the last slice merges (null: a merge launch follows)
 };
+
+// ---- merge of the split partials inside the split kernels ----
+// The slices of a head (or of a KV head's group of heads) finish in any order on any XCD.  Each work-group writes its partial
+// through to memory (agent-scope stores: the XCDs' L2 caches are not coherent with one another inside a launch), waits for the
+// stores to be acknowledged and then counts itself in; the one that counts last reads all partials back at agent scope and
+// writes the finished rows.  The counter wraps to zero on the last arrival, so it needs no clearing between launches.  No
+// cache-wide fence is involved (a __threadfence per work-group measured several times the merge launch it saves).
+__device__ __forceinline__ void part_store(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float part_load(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+// heads qh0 .. qh0 + n_heads - 1 of sequence `seq`; every thread of the work-group calls it after its partial stores
+__device__ __forceinline__ void merge_if_last(const AttnParams& p, int seq, int qh0, int n_heads, int s_first, int n_active, int counter)
+{
+  __shared__ int s_is_last;
+  __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this thread's partial stores have been acknowledged
+  __syncthreads();
+  if (threadIdx.x == 0)
+    s_is_last = __builtin_amdgcn_atomic_inc32(p.merge_cnt + counter, (unsigned)n_active - 1, __ATOMIC_RELAXED, "agent") == (unsigned)n_active - 1;
+  __syncthreads();
+  if (!s_is_last) return;
+  // One round trip: every thread requests, per slice, its value and the slice's maximum and sum together (the latter two
+  // are the same addresses in all threads), then folds the slices in order with a running maximum.
+  const int hd = p.hd;
+  for (int o = threadIdx.x; o < n_heads * hd; o += blockDim.x) {
+    const int qh = qh0 + o / hd, d = o % hd;
+    const float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + s_first) * (hd + 2);
+    float A = 0.0f, L = 0.0f, M = -1e30f;
+    for (int s0 = 0; s0 < n_active; s0 += 8) {
+      float v[8], ms[8], ls[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const float* ps = pt + (int64_t)min(s0 + u, n_active - 1) * (hd + 2);
+        v[u] = part_load(ps + d); ms[u] = part_load(ps + hd); ls[u] = part_load(ps + hd + 1);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        if (s0 + u < n_active && ls[u] > 0.0f) {
+          const float mn = fmaxf(M, ms[u]), c0 = expf(M - mn), c1 = expf(ms[u] - mn);
+          A = fmaf(v[u], c1, A * c0); L = fmaf(ls[u], c1, L * c0); M = mn;
+        }
+      }
+    }
+    p.out[(int64_t)seq * p.out_stride + qh * hd + d] = L > 0.0f ? A * (1.0f / L) : 0.0f;
+  }
+}
 
 // Where the row of stream position `pos` lives and which rows are live.  Without eviction: slot = pos, rows
 // [j_start, pos] (j_start > 0 under a sliding window).  With sink + recent-window eviction (TNNetStreamingDecoder.
@@ -386,13 +432,14 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const AttnParams p)
           p.out[(int64_t)seq * p.out_stride + qh * hd + d] = Ls > 0.0f ? A * (1.0f / Ls) : 0.0f;
         } else {
           float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + split) * (hd + 2);
-          pt[d] = A;
-          if (d == 0) { pt[hd] = M; pt[hd + 1] = Ls; }
+          if (p.merge_cnt) { part_store(pt + d, A); if (d == 0) { part_store(pt + hd, M); part_store(pt + hd + 1, Ls); } }
+          else { pt[d] = A; if (d == 0) { pt[hd] = M; pt[hd + 1] = Ls; } }
         }
       }
     }
     __syncthreads();
   }
+  if (n_active > 1 && p.merge_cnt) merge_if_last(p, seq, g * G, G, s_first, n_active, seq * p.kv_heads * 8 + g);
 }
 
 // ---- merge of the split partials: one work-group per query head; all partial loads are issued together ----
@@ -615,10 +662,11 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
       p.out[(int64_t)seq * p.out_stride + qh * hd + d] = Ls > 0.0f ? A * (1.0f / Ls) : 0.0f;
     } else {
       float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + split) * (hd + 2);
-      pt[d] = A;
-      if (d == 0) { pt[hd] = M; pt[hd + 1] = Ls; }
+      if (p.merge_cnt) { part_store(pt + d, A); if (d == 0) { part_store(pt + hd, M); part_store(pt + hd + 1, Ls); } }
+      else { pt[d] = A; if (d == 0) { pt[hd] = M; pt[hd + 1] = Ls; } }
     }
   }
+  if (n_active > 1 && p.merge_cnt) merge_if_last(p, seq, g * G + h, 1, s_first, n_active, seq * p.kv_heads * 8 + g * G + h);
 }
 
 template <typename KV_T>
@@ -970,6 +1018,7 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   p.seq_mul = prompt_rows ? 0 : 1; p.appended = prompt_rows ? 1 : 0;
   p.evict_sinks = kv->evict_sinks; p.evict_cap = kv->evict_cap;
   p.ksc = kv->ks; p.vsc = kv->vs; p.seq_rows = kv->seq_rows(); p.layer_row_off = (int64_t)layer * kv->layer_rows();
+  p.merge_cnt = prompt_rows ? nullptr : kv->merge_cnt;   // (a prompt has more rows in flight than the counters cover: merge launch)
   int rc;
   static const int group_min = []() { const char* e = getenv("CAIHIP_ATTN_GROUP_MIN"); return e ? atoi(e) : 256; }();
   const bool grouped = (kv->head_dim & 7) == 0 && n_seq * kv->kv_heads * kv->n_splits >= group_min;
@@ -1026,7 +1075,7 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   else
     rc = kv->dtype == CAI_KV_I8 ? launch_split_head<int8_t>(p, n_seq, c.stream) : kv->dtype == CAI_KV_F16 ? launch_split_head<__half>(p, n_seq, c.stream) : launch_split_head<float>(p, n_seq, c.stream);
   if (rc) return rc;
-  if (p.n_splits > 1) hipLaunchKernelGGL(attn_merge_kernel, dim3(q_heads, n_seq), dim3(128), 0, c.stream, p);
+  if (p.n_splits > 1 && !p.merge_cnt) hipLaunchKernelGGL(attn_merge_kernel, dim3(q_heads, n_seq), dim3(128), 0, c.stream, p);
   return CAI_OK;
 }
 
@@ -1065,6 +1114,8 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   kv->part_q_heads = kv_heads * 8;
   CAI_HIP(hipMalloc(&kv->part, (size_t)n_seq * kv->part_q_heads * kv->n_splits * (head_dim + 2) * sizeof(float)));
   CAI_HIP(hipMalloc(&kv->d_len, sizeof(int32_t) * n_seq));
+  CAI_HIP(hipMalloc((void**)&kv->merge_cnt, sizeof(unsigned) * n_seq * kv->part_q_heads));
+  CAI_HIP(hipMemsetAsync(kv->merge_cnt, 0, sizeof(unsigned) * n_seq * kv->part_q_heads, ctx().stream));
   CAI_HIP(hipStreamSynchronize(ctx().stream));
   return CAI_OK;
 }
@@ -1081,6 +1132,8 @@ void kv_free(cai_kv_s* kv)
   kv->pq_hi = kv->pq_lo = nullptr; kv->pq_cap = 0;
   if (kv->part) (void)hipFree(kv->part);
   if (kv->d_len) (void)hipFree(kv->d_len);
+  if (kv->merge_cnt) (void)hipFree(kv->merge_cnt);
+  kv->merge_cnt = nullptr;
   kv->k = kv->v = nullptr; kv->part = nullptr; kv->d_len = nullptr;
 }
 

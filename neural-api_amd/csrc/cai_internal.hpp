@@ -119,6 +119,7 @@ struct cai_kv_s {
   float* part = nullptr;                  // [seq][q_head][split][head_dim+2] split-K partials
   int part_q_heads = 0;
   int32_t* d_len = nullptr;               // [seq] device scratch: rows live BEFORE the token being decoded
+  unsigned* merge_cnt = nullptr;          // [seq][part_q_heads] arrival counters of the in-kernel merge of the split partials (wrap to 0 by themselves)
   void* pq_hi = nullptr; void* pq_lo = nullptr; size_t pq_cap = 0;   // prompt ingestion: rotated q of a chunk as two f16 planes
   size_t elem() const { return dtype == CAI_KV_F16 ? 2 : dtype == CAI_KV_I8 ? 1 : 4; }
   int64_t layer_rows() const { return (int64_t)kv_heads * max_ctx; }
@@ -207,6 +208,7 @@ int prefill_gemm(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride, const
 int prefill_gemm_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, float* y, int64_t y_stride);
 
 void rope_thetas(float base, int head_dim, std::vector<float>& out);
+
 // softmax -> history penalty -> temperature -> the m most probable tokens (descending) of a device-resident logits row;
 // history and results are host arrays
 int run_candidates(const float* logits_dev, int n, const int32_t* hist_ids, const int32_t* hist_counts, int n_hist,
