@@ -40,6 +40,22 @@ CONFIGS = {
 }
 
 
+def host_cpu():
+    """(model name, logical cores of the host, threads the CPU leg uses).  The GPU boxes hand a one-GPU job a 16-core share and
+    set OMP_NUM_THREADS to it; the CPU leg uses what OpenMP reports, which honours that."""
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip(); break
+    except OSError:
+        pass
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from helpers import oracle_lib as O
+    return model, os.cpu_count(), O.lib().cpu_max_threads()
+
+
 def cpu_baseline(cfg, seconds_budget=20.0):
     """Restated reference AVX2 int8-per-row path (oracle/cpu_baseline.c) on a bounded sample of the same workload:
     ONE decoder block's linear layers + the LM head, timed on this host's cores; extrapolated to a full token."""
@@ -47,7 +63,7 @@ def cpu_baseline(cfg, seconds_budget=20.0):
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     from helpers import oracle_lib as O
     L = O.lib()
-    threads = min(L.cpu_max_threads(), 16)
+    model, host_cores, threads = host_cpu()
     d, I, V = cfg["d_model"], cfg["ffn"], cfg["vocab"]
     qw, kw = cfg["n_q_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
     shapes = [(qw, d), (kw, d), (kw, d), (d, qw), (2 * I, d), (d, I)]
@@ -70,9 +86,73 @@ def cpu_baseline(cfg, seconds_budget=20.0):
         t_layer.append(t1 - t0); t_head.append(t2 - t1); reps += 1
     tl, th = sorted(t_layer)[len(t_layer) // 2], sorted(t_head)[len(t_head) // 2]
     tok_s = 1.0 / (cfg["n_layers"] * tl + th)
-    return {"value": round(tok_s, 3), "unit": "tok/s", "cores": threads, "kind": "port",
+    return {"value": round(tok_s, 3), "unit": "tok/s", "cores": threads, "kind": "port", "cpu_model": model, "host_cores": host_cores,
             "sample": "restated AVX2 int8-per-row kernels (reference's default ChatTerminal path): 1 of %d blocks' linear layers + LM head, "
                       "median of %d runs, extrapolated to a full token; attention/norms excluded" % (cfg["n_layers"], reps)}
+
+
+def cpu_baseline_end_to_end(cfg, prompt_len, n_decode, seed=424242):
+    """The whole workload on the CPU port (the plan for the reference's own CPU-runnable configuration): every linear layer
+    through the restated AVX2 int8-per-row kernel on all threads (weights N(0, 0.02) quantised per row like TNNetVolume.QuantizeInt8),
+    norms / rotary / cached attention / SwiGLU / arg-max through the oracle's scalar restatements; prompt_len prompt tokens, then
+    n_decode greedy tokens; tok/s by the reference's --stats definition (first token excluded)."""
+    import numpy as np
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from helpers import oracle_lib as O
+    L = O.lib()
+    model, host_cores, threads = host_cpu()
+    d, I, V, NL = cfg["d_model"], cfg["ffn"], cfg["vocab"], cfg["n_layers"]
+    hq, hkv, hd = cfg["n_q_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    qw, kw = hq * hd, hkv * hd
+    rng = np.random.default_rng(seed)
+
+    def q8(rows, cols):
+        w = rng.standard_normal((rows, cols), dtype=np.float32) * np.float32(0.02)
+        amax = np.abs(w).max(1)
+        scale = np.where(amax > 0, amax / 127.0, 1.0).astype(np.float32)
+        return np.clip(np.rint(w / scale[:, None]), -127, 127).astype(np.int8), scale
+
+    embed = q8(V, d)
+    layers = [dict(qkv=q8(qw + 2 * kw, d), o=q8(d, qw), gu=q8(2 * I, d), dn=q8(d, I)) for _ in range(NL)]
+    ones = np.ones(d, np.float32)
+    theta = np.empty(hd // 2, np.float32); L.orc_rope_thetas(C.c_float(cfg["rope_theta"]), hd, theta.ctypes.data)
+    ctx = prompt_len + n_decode
+    kc = np.zeros((NL, hkv * ctx * hd), np.float32); vc = np.zeros_like(kc)
+    P = lambda a: a.ctypes.data
+
+    def lin(wt, x, y):
+        L.cpu_linear_int8(P(wt[0]), P(wt[1]), wt[0].shape[0], wt[0].shape[1], P(x), 1, None, P(y), threads)
+
+    x = np.empty(d, np.float32); h = np.empty(d, np.float32); qkv = np.empty(qw + 2 * kw, np.float32); att = np.empty(qw, np.float32)
+    gu = np.empty(2 * I, np.float32); mid = np.empty(I, np.float32); t = np.empty(d, np.float32); logits = np.empty(V, np.float32)
+
+    def step(tok, pos):
+        x[:] = embed[0][tok].astype(np.float32) * embed[1][tok]
+        for l, w in enumerate(layers):
+            L.orc_rmsnorm(P(x), P(ones), d, C.c_float(cfg["eps"]), P(h))
+            lin(w["qkv"], h, qkv)
+            L.orc_rope_interleaved(P(qkv), hq + hkv, hd, pos, P(theta))          # q heads, then k heads: one contiguous run
+            L.orc_attn_decode(P(qkv), hq, hkv, hd, P(kc[l]), P(vc[l]), ctx, pos, 0, C.c_float(0.0), 0, P(att))
+            lin(w["o"], att, t); x[:] += t
+            L.orc_rmsnorm(P(x), P(ones), d, C.c_float(cfg["eps"]), P(h))
+            lin(w["gu"], h, gu)
+            L.orc_swiglu(P(gu), I, P(mid))
+            lin(w["dn"], mid, t); x[:] += t
+        L.orc_rmsnorm(P(x), P(ones), d, C.c_float(cfg["eps"]), P(h))
+        lin(embed, h, logits)                                                   # tied head
+        return int(L.orc_argmax(P(logits), V))
+
+    prompt = rng.integers(0, V, prompt_len)
+    tok = 0
+    for p_, t_ in enumerate(prompt):
+        tok = step(int(t_), p_)
+    t_first = time.perf_counter()
+    for i in range(n_decode - 1):
+        tok = step(tok, prompt_len + i)
+    dt = time.perf_counter() - t_first
+    return {"value": round((n_decode - 1) / dt, 2), "unit": "tok/s", "cores": threads, "kind": "port", "cpu_model": model, "host_cores": host_cores,
+            "sample": "whole workload: %d-token prompt + %d greedy tokens, linear layers on the restated AVX2 int8-per-row kernel "
+                      "(all threads), the rest on scalar restatements; first token excluded" % (prompt_len, n_decode)}
 
 
 def gemv_sweep(cai, synth, torch, with_cpu):
@@ -114,7 +194,7 @@ def gemv_sweep(cai, synth, torch, with_cpu):
                 if cpu is not None and nb == 1 and name == "I8ROW":
                     # restated reference AVX2 int8-per-row kernel on the same shape (1 B/weight), all host threads
                     import numpy as np
-                    thr = min(cpu.cpu_max_threads(), 16)
+                    thr = cpu.cpu_max_threads()
                     rng = np.random.default_rng(0)
                     codes = rng.integers(-127, 128, (rows, cols), dtype=np.int8); sc = np.full(rows, 1e-3, np.float32)
                     xv = rng.standard_normal(cols).astype(np.float32); yv = np.empty(rows, np.float32)
@@ -136,6 +216,7 @@ def gemv_sweep(cai, synth, torch, with_cpu):
 # KiB, factors from a 1 GiB copy kernel): profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt.  Not measurable from
 # inside this process; re-collect when the kernel changes.
 GATEUP_TRAFFIC_BYTES = int((37522.5 * 2.000 + 74.2 * 1.000) * 1024)
+GATEUP_TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of gemv_q4k_dot<1,1,false,2>, profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt"
 
 
 def main():
@@ -145,7 +226,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--config", default="qwen2.5-7b-q4k", choices=list(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--kernel-reps", type=int, default=5)
+    ap.add_argument("--reps", type=int, default=5, help="timed repetitions of the K steps (each from the same position); the median is reported")
+    ap.add_argument("--kernel-reps", type=int, default=8, help="repetitions of each kernel class in the per-kernel table")
     ap.add_argument("--kv", choices=["f32", "f16", "i8"], default=None, help="KV cache element type (default: the configuration's own)")
     ap.add_argument("--batch", type=int, default=1, help="independent sequences decoded together (1..8)")
     ap.add_argument("--gemv-sweep", action="store_true", help="isolated matrix-vector sweep (BASELINE configs[1]): Q8_0 / Q4_0 / Q4_K and per-row int8, five shapes, batch 1 and 4")
@@ -218,14 +300,22 @@ def main():
 
     if W > 0:
         tok = decode(tok, pos, W); pos += W
-    cai.check(lib.cai_sync()); torch.cuda.synchronize()
-    ms = C.c_float()
-    t1 = time.perf_counter()
-    cai.check(lib.cai_timer_start())
-    decode(tok, pos, K)
-    cai.check(lib.cai_timer_stop(C.byref(ms)))
-    cai.check(lib.cai_sync()); torch.cuda.synchronize()
-    wall = time.perf_counter() - t1
+    # K steps, timed `reps` times from the same position (the cache is cut back in between); the median repetition is reported
+    walls, evs = [], []
+    for rep in range(max(1, args.reps)):
+        for b in range(B):
+            dec.truncate(pos, seq=b)
+        cai.check(lib.cai_sync()); torch.cuda.synchronize()
+        ms = C.c_float()
+        t1 = time.perf_counter()
+        cai.check(lib.cai_timer_start())
+        decode(tok, pos, K)
+        cai.check(lib.cai_timer_stop(C.byref(ms)))
+        cai.check(lib.cai_sync()); torch.cuda.synchronize()
+        walls.append(time.perf_counter() - t1); evs.append(ms.value)
+    order = sorted(range(len(walls)), key=lambda i: walls[i])
+    mid = order[len(order) // 2]
+    wall = walls[mid]; ms = C.c_float(evs[mid])
     ms_per_step = wall * 1e3 / K
     tok_s = K * B / wall
     ctx_mid = pos + K // 2
@@ -241,23 +331,61 @@ def main():
                           "whole_step_hbm_frac": round(algo_bytes / (wall / K) / 1e9 / HBM_PEAK_GBS, 4),
                           "prefill": {"tokens": prompt_len - 1, "ms": round(pf_ms.value, 2)}}))
         return
-    gu = [spec["tensors"][(l, cai.W_GATEUP)]["qw"] for l in range(L)]
-    d, I = cfg["d_model"], cfg["ffn"]
-    x = torch.randn(d, device="cuda"); g = torch.ones(d, device="cuda"); y = torch.empty(I, device="cuda")
-    torch.cuda.synchronize()
-    for w in gu:  # warm the code path; rotating over all layers keeps the 256 MB infinity cache cold like a real token
-        cai.check(lib.cai_ffn_gateup(w.h, x.data_ptr(), g.data_ptr(), cfg["eps"], 1, y.data_ptr(), cai.X_DEVICE | cai.Y_DEVICE))
-    cai.check(lib.cai_sync())
-    cai.check(lib.cai_timer_start())
-    for _ in range(args.kernel_reps):
-        for w in gu:
-            cai.check(lib.cai_ffn_gateup(w.h, x.data_ptr(), g.data_ptr(), cfg["eps"], 1, y.data_ptr(), cai.X_DEVICE | cai.Y_DEVICE))
-    kms = C.c_float()
-    cai.check(lib.cai_timer_stop(C.byref(kms)))
-    k_avg_us = kms.value * 1e3 / (args.kernel_reps * L)
-    qbytes = {"Q4_K": 144 / 256, "Q8_0": 34 / 32, "Q4_0": 18 / 32}[conf["qtype"]]
+    d, I, V = cfg["d_model"], cfg["ffn"], cfg["vocab"]
+    qw_, kw_ = cfg["n_q_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
+    bpw = {"Q4_K": 144 / 256, "Q8_0": 34 / 32, "Q4_0": 18 / 32, "Q6_K": 210 / 256}
+    qbytes = bpw[conf["qtype"]]
     k_bytes = 2 * I * d * qbytes + 4 * d * 2 + 4 * I     # blocks + x + gain + y
+    # ---- every kernel class of the step, timed in place: the production launches of one class over all blocks, back to
+    #      back between two HIP events on the library's stream (cai_decoder_profile); batch 1 only ----
+    table, k_avg_us = None, None
+    if B == 1:
+        for b in range(B):
+            dec.truncate(pos, seq=b)
+        us = dec.profile(tok, reps=args.kernel_reps)
+        kv_el = {"f32": 4, "f16": 2, "i8": 1}[kv_kind]
+        bias_b = 4 * (qw_ + 2 * kw_) if conf["bias"] else 0
+        head_bpw = bpw[conf["head"]]
+        classes = [
+            ("embedding row", 1, d * bpw[conf.get("embed", conf["head"])] + 4 * d),
+            ("q|k|v (RMSNorm fused)", L, (qw_ + 2 * kw_) * d * qbytes + bias_b + 4 * (2 * d + qw_ + 2 * kw_)),
+            ("attention (rotary + append + cached decode + merge)", L, 2 * kw_ * kv_el * (pos + 1) + 4 * (2 * qw_ + 2 * kw_)),
+            ("o + residual", L, d * qw_ * qbytes + 4 * (qw_ + 2 * d)),
+            ("RMSNorm + gate|up + SwiGLU", L, k_bytes),
+            ("down + residual", L, d * I * qbytes + 4 * (I + 2 * d)),
+            ("final norm + vocabulary projection", 1, V * d * head_bpw + 4 * (2 * d + V)),
+            ("arg-max", 2, 2 * V),
+        ]
+        table = []
+        for (name, n, by), u in zip(classes, us):
+            per = float(u) / n
+            table.append({"class": name, "launches_per_step": n, "us_per_step": round(float(u), 2), "us_per_launch": round(per, 2),
+                          "algorithmic_bytes_per_launch": int(by), "GB_per_s": round(by / per / 1e3, 1), "frac_of_8TBps": round(by / per / 1e3 / HBM_PEAK_GBS, 4)})
+        k_avg_us = float(us[4]) / L
+    else:
+        gu = [spec["tensors"][(l, cai.W_GATEUP)]["qw"] for l in range(L)]
+        x = torch.randn(d, device="cuda"); g = torch.ones(d, device="cuda"); y = torch.empty(I, device="cuda")
+        torch.cuda.synchronize()
+        for w in gu:  # warm the code path; rotating over all layers keeps the 256 MB infinity cache cold like a real token
+            cai.check(lib.cai_ffn_gateup(w.h, x.data_ptr(), g.data_ptr(), cfg["eps"], 1, y.data_ptr(), cai.X_DEVICE | cai.Y_DEVICE))
+        cai.check(lib.cai_sync())
+        cai.check(lib.cai_timer_start())
+        for _ in range(args.kernel_reps):
+            for w in gu:
+                cai.check(lib.cai_ffn_gateup(w.h, x.data_ptr(), g.data_ptr(), cfg["eps"], 1, y.data_ptr(), cai.X_DEVICE | cai.Y_DEVICE))
+        kms = C.c_float()
+        cai.check(lib.cai_timer_stop(C.byref(kms)))
+        k_avg_us = kms.value * 1e3 / (args.kernel_reps * L)
     k_gbs = k_bytes / (k_avg_us * 1e-6) / 1e9
+    # ---- what this machine streams: a 1 GiB device-to-device copy kernel (read + write bytes) ----
+    a = torch.ones(1 << 28, dtype=torch.float32, device="cuda"); bcopy = torch.empty_like(a)
+    cai.check(lib.cai_dev_copy(bcopy.data_ptr(), a.data_ptr(), a.numel() * 4))
+    cai.check(lib.cai_sync()); cai.check(lib.cai_timer_start())
+    for _ in range(5):
+        cai.check(lib.cai_dev_copy(bcopy.data_ptr(), a.data_ptr(), a.numel() * 4))
+    cms = C.c_float(); cai.check(lib.cai_timer_stop(C.byref(cms)))
+    copy_gbs = 5 * 2 * a.numel() * 4 / (cms.value * 1e-3) / 1e9
+    del a, bcopy
 
     res = {
         "metric": "decode tok/s @bs1 (Qwen2.5-7B-shape Q4_K) + % of HBM-bandwidth roofline" if args.config == "qwen2.5-7b-q4k" and B == 1
@@ -278,10 +406,19 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "%s (RMSNorm+gate|up+SwiGLU, %dx%d)" % ("gemv_q4k_dot<1,1,false,2>" if conf["qtype"] == "Q4_K" else "gemv_fast<%s>" % conf["qtype"], 2 * I, d),
                      "achieved": round(k_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(k_gbs / HBM_PEAK_GBS, 4),
                      "avg_launch_us": round(k_avg_us, 2), "algorithmic_bytes_per_launch": int(k_bytes),
-                     "traffic": GATEUP_TRAFFIC_BYTES if args.config == "qwen2.5-7b-q4k" else None, "traffic_unit": "bytes/launch"},
+                     "traffic": GATEUP_TRAFFIC_BYTES if args.config == "qwen2.5-7b-q4k" else None, "traffic_unit": "bytes/launch",
+                     "traffic_source": GATEUP_TRAFFIC_SOURCE if args.config == "qwen2.5-7b-q4k" else None,
+                     "measured_stream_GB_per_s": round(copy_gbs, 1), "frac_of_measured_stream": round(k_gbs / copy_gbs, 4)},
     }
+    res["config"]["timed_repetitions_ms_per_step"] = [round(w * 1e3 / K, 4) for w in walls]
+    if table is not None:
+        total = sum(r["us_per_step"] for r in table)
+        res["kernels"] = {"rows": table, "sum_us_per_step": round(total, 1), "graph_step_us": round(ms.value * 1e3 / K, 1),
+                          "note": "each class timed in place (its production launches over all blocks, back to back, HIP events on the library stream); "
+                                  "the captured graph adds the token hand-over kernel between steps"}
     if not args.no_cpu_baseline:
-        res["cpu_baseline"] = cpu_baseline(cfg)
+        # the reference's own CPU-runnable configuration is small enough to run whole on the host; the others are sampled
+        res["cpu_baseline"] = cpu_baseline_end_to_end(cfg, prompt_len, 128) if args.config == "smollm2-135m-q8_0" else cpu_baseline(cfg)
     print(json.dumps(res))
 
 

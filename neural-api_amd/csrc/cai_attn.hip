@@ -701,7 +701,7 @@ template <typename KV_T>
 static int launch_group(const AttnParams& p, int n_seq, hipStream_t st)
 {
   const int G = p.q_heads / p.kv_heads;
-  static const int hc_max = []() { const char* e = getenv("CAIHIP_ATTN_HC"); const int v = e ? atoi(e) : 8; return v >= 1 && v <= 8 ? v : 8; }();
+  constexpr int hc_max = 8;    // query heads held in registers per pass
   const int n_chunks = (G + hc_max - 1) / hc_max, hc = (G + n_chunks - 1) / n_chunks;
   const dim3 grid(p.n_splits * p.kv_heads, n_seq);
   const size_t lds = (size_t)(G * 128 + G * p.split_len + n_chunks * p.split_len * (hc > 4 ? 8 : 4) + 4 * hc * 128 + 2 * G) * sizeof(float);
@@ -1020,7 +1020,7 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   p.ksc = kv->ks; p.vsc = kv->vs; p.seq_rows = kv->seq_rows(); p.layer_row_off = (int64_t)layer * kv->layer_rows();
   p.merge_cnt = prompt_rows ? nullptr : kv->merge_cnt;   // (a prompt has more rows in flight than the counters cover: merge launch)
   int rc;
-  static const int group_min = []() { const char* e = getenv("CAIHIP_ATTN_GROUP_MIN"); return e ? atoi(e) : 256; }();
+  const int group_min = c.n_cu;   // smallest grid that fills the chip with one work-group per (slice, KV head)
   const bool grouped = (kv->head_dim & 7) == 0 && n_seq * kv->kv_heads * kv->n_splits >= group_min;
   if (qn_gain) {
     // q and k norms over the whole rows: the per-head decode kernel applies them while it reads its operands; the
@@ -1091,11 +1091,11 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   kv->len.assign((size_t)n_seq * n_layers, 0);
   // few, fat splits: every extra split costs the merging work-group another device-coherent load round,
   // while one CU sustains only ~20 GB/s, so a slice should stay under ~100 KB
-  static const int sl_max = []() { const char* e = getenv("CAIHIP_ATTN_SPLIT_MAX"); const int v = e ? atoi(e) : 256; return v >= 32 ? v : 256; }();
+  constexpr int sl_max = 256;
   int sl = (max_ctx + 15) / 16; sl = (sl + 31) / 32 * 32; if (sl < 32) sl = 32; if (sl > sl_max) sl = sl_max;
   // a head's whole K (or V) plane of at most 64 KB is one slice: a single work-group streams it in a few microseconds and
   // the merge launch disappears (small models at short contexts are bound by launches, not by bytes)
-  static const int single_bytes = []() { const char* e = getenv("CAIHIP_ATTN_SINGLE_BYTES"); return e ? atoi(e) : 65536; }();
+  constexpr int single_bytes = 65536;
   if ((int64_t)max_ctx * head_dim * (dtype == CAI_KV_F16 ? 2 : dtype == CAI_KV_I8 ? 1 : 4) <= single_bytes) sl = (max_ctx + 31) / 32 * 32;
   kv->split_len = sl; kv->n_splits = (max_ctx + sl - 1) / sl;   // the merge stage holds up to 128 splits
   const size_t bytes = (size_t)kv->seq_elems() * n_seq * kv->elem();

@@ -104,12 +104,14 @@ static int moe_ffn_rows(cai_decoder_s* d, const cai_decoder_s::Layer& L, float* 
 }
 
 // Enqueues one whole step for activation rows 0..n_b-1 mapped to cache sequences seq0..seq0+n_b-1.
-static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
+// `classes`: bit i set = launch kernel class i (0 embedding, 1 q|k|v, 2 attention, 3 o, 4 gate|up + SwiGLU, 5 down, 6 vocabulary
+// projection, 7 arg-max).  Everything but the per-class timing of cai_decoder_profile passes all bits.
+static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = ~0u)
 {
   const cai_decoder_config& c = d->cfg;
   const int dm = c.d_model, qw = d->qw(), kw = d->kw(), I = c.ffn, qkvw = qw + 2 * kw;
   int rc;
-  if ((rc = launch_embed(d->embed, d->d_tokens, n_b, d->x))) return rc;
+  if ((classes & 1u) && (rc = launch_embed(d->embed, d->d_tokens, n_b, d->x))) return rc;
   float* ssq_o = d->ssq;          // written by the o-projection, read by gate|up
   float* ssq_d = d->ssq + 1024;   // written by the down projection, read by the next block's q|k|v
   bool have_ssq_d = false;
@@ -146,7 +148,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
     }
     if (down_pending) { if ((rc = nb_prep_residual(d->x, dm, nullptr, 0.0f, dm, n_b))) return rc; down_pending = false; }
     // --- attention half ---
-    {
+    if (classes & 2u) {
       MultiGemv m{}; m.n = 3;
       const int slots[3] = {CAI_W_Q, CAI_W_K, CAI_W_V}; const int offs[3] = {0, qw, qw + kw};
       bool same = true;
@@ -171,10 +173,11 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
         }
       }
     }
-    if ((rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0, 0, nullptr,
+    if ((classes & 4u) &&
+        (rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0, 0, nullptr,
                                c.qk_norm_full ? L.v[CAI_V_Q_NORM] : nullptr, c.qk_norm_full ? L.v[CAI_V_K_NORM] : nullptr, c.eps))) return rc;
     const bool o_hands = gemv_hands_off_ssq(L.w[CAI_W_O], n_b);
-    {
+    if (classes & 8u) {
       MultiGemv m{}; m.n = 1; m.w[0] = L.w[CAI_W_O]; m.rows[0] = dm;
       if (o_hands) m.ssq_out = ssq_o;
       if ((rc = launch_gemv_multi(m, d->att, n_b, d->x, dm, CAI_ACT_NONE, d->x, nullptr, 0.0f, 0))) return rc;
@@ -184,23 +187,24 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
     if (c.n_experts == 0) {
       MultiGemv m{}; m.n = 1; m.w[0] = L.w[CAI_W_GATEUP]; m.rows[0] = 2 * I;
       if (o_hands && gemv_hands_off_ssq(m.w[0], n_b)) m.ssq_in = ssq_o;
-      if (is_block_quant(m.w[0]->qtype)) {
+      if (!(classes & 16u)) {
+      } else if (is_block_quant(m.w[0]->qtype)) {
         if ((rc = launch_gemv_multi(m, d->x, n_b, d->mid, I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, I))) return rc;
       } else {
         if ((rc = launch_gemv_multi(m, d->x, n_b, d->gu, 2 * I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;
         launch_swiglu(d->gu, I, n_b, d->mid);
       }
-      {
+      have_ssq_d = gemv_hands_off_ssq(L.w[CAI_W_DOWN], n_b);
+      if (classes & 32u) {
         MultiGemv dn{}; dn.n = 1; dn.w[0] = L.w[CAI_W_DOWN]; dn.rows[0] = dm;
-        have_ssq_d = gemv_hands_off_ssq(dn.w[0], n_b);
         if (have_ssq_d) dn.ssq_out = ssq_d;
         if ((rc = launch_gemv_multi(dn, d->mid, n_b, d->x, dm, CAI_ACT_NONE, d->x, nullptr, 0.0f, 0))) return rc;
       }
     } else {
-      if ((rc = moe_ffn_rows(d, L, d->x, n_b))) return rc;
+      if ((classes & 48u) && (rc = moe_ffn_rows(d, L, d->x, n_b))) return rc;
     }
   }
-  {
+  if (classes & 64u) {
     cai_qw_s* hw = d->head ? d->head : d->embed;   // tied head (neural/neuralpretrained.pas:15555-)
     if (n_b >= 2 && nb_supported(hw)) {
       const int zero = 0; const cai_qw_s* hwc = hw;
@@ -215,7 +219,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0)
     if (have_ssq_d && gemv_hands_off_ssq(hw, n_b)) m.ssq_in = ssq_d;
     if ((rc = launch_gemv_multi(m, d->x, n_b, d->logits, c.vocab, CAI_ACT_NONE, nullptr, d->final_norm, c.eps, 0))) return rc;
   }
-  launch_argmax(d->logits, c.vocab, n_b, d->d_argmax, d->am_v, d->am_i);
+  if (classes & 128u) launch_argmax(d->logits, c.vocab, n_b, d->d_argmax, d->am_v, d->am_i);
   return CAI_OK;
 }
 
@@ -503,6 +507,34 @@ extern "C" int cai_decoder_generate(cai_decoder_t d, int32_t first_token, int po
   CAI_HIP(hipStreamSynchronize(cx.stream));
   for (int l = 0; l < c.n_layers; l++) d->kv.len_at(0, l) = pos + n_tokens;
   return CAI_OK;
+}
+
+// Per-class timing of the batch-1 step: the production launches of one class (all blocks), back to back, between two HIP events.
+extern "C" int cai_decoder_profile(cai_decoder_t d, int32_t token, int reps, float* us_per_step_out, int n_classes)
+{
+  CAI_READY();
+  CAI_REQUIRE(d && us_per_step_out && reps >= 1 && n_classes >= 1 && n_classes <= 8, "cai_decoder_profile: bad argument");
+  const cai_decoder_config& c = d->cfg;
+  int rc = check_ready(d); if (rc) return rc;
+  CAI_REQUIRE(token >= 0 && token < c.vocab, "cai_decoder_profile: token %d outside vocab %d", token, c.vocab);
+  const int pos = d->kv.len_at(0, 0);
+  if (pos >= c.max_ctx && d->kv.evict_cap == 0) return set_error(CAI_ERR_STATE, "cai_decoder_profile: sequence 0 reached max_ctx %d", c.max_ctx);
+  Context& cx = ctx();
+  d->h_io[0] = token; d->h_io[8] = pos;
+  CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
+  if ((rc = enqueue_step(d, 1, 0))) return rc;      // a whole step first: every buffer a class reads holds this step's values
+  for (int k = 0; k < n_classes; k++) {
+    if ((rc = enqueue_step(d, 1, 0, 1u << k))) return rc;   // warm
+    CAI_HIP(hipEventRecord(cx.ev0, cx.stream));
+    for (int r = 0; r < reps; r++) if ((rc = enqueue_step(d, 1, 0, 1u << k))) return rc;
+    CAI_HIP(hipEventRecord(cx.ev1, cx.stream));
+    CAI_HIP(hipEventSynchronize(cx.ev1));
+    float ms = 0.0f;
+    CAI_HIP(hipEventElapsedTime(&ms, cx.ev0, cx.ev1));
+    us_per_step_out[k] = ms * 1e3f / (float)reps;
+  }
+  CAI_HIP(hipGetLastError());
+  return CAI_OK;     // (the session's length is unchanged: the K,V row written at the current position is not counted)
 }
 
 extern "C" int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* tokens, int n, int pos0, float* last_logits, int32_t* argmax)

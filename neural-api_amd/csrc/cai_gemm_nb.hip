@@ -815,12 +815,10 @@ int nb_reserve(int k_max, size_t part_floats)
 static void nb_geometry(int cols, int tiles, int& S, int& n_slices, int& gx, int& tile_stride, int s_max = NB_SMAX)
 {
   const int nsb = (cols + 255) >> 8, slots = 3 * ctx().n_cu;
-  static const int force = []() { const char* e = getenv("CAIHIP_NB_S"); return e ? atoi(e) : 0; }();
   const int s_lo = std::min(2, nsb), s_hi = std::min(s_max, nsb);
   float best = 3.0e38f;
   S = s_lo;
   for (int s = s_lo; s <= s_hi; s++) {
-    if (force >= 2 && force <= NB_SMAX && s != std::min(force, nsb)) continue;
     const int ns = (nsb + s - 1) / s;
     const int g = std::max(1, std::min((tiles + 3) / 4, slots / ns));
     const int share = (tiles + 4 * g - 1) / (4 * g);

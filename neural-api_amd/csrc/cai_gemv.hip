@@ -495,17 +495,11 @@ __global__ void swiglu_rows(const float* x, int half, int n_tokens, float* y)
   y[i] = silu_mul(x[(int64_t)t * 2 * half + d], x[(int64_t)t * 2 * half + half + d]);
 }
 
-int launch_q4k_stream(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream_t st);
 int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream_t st);
-static bool stream_kernel_enabled()
-{
-  static const int on = []() { const char* e = getenv("CAIHIP_GEMV_V1"); return (e && e[0] == '1') ? 0 : 1; }();
-  return on != 0;
-}
 // True when a batch-1 launch on this matrix goes through the streaming kernel (which honours ssq_in / ssq_out).
 bool gemv_hands_off_ssq(const cai_qw_s* w, int n_b)
 {
-  return w->qtype == CAI_Q4_K && n_b == 1 && stream_kernel_enabled() && (((w->cols >> 8) + 15) >> 4) <= 8;
+  return w->qtype == CAI_Q4_K && n_b == 1 && (((w->cols >> 8) + 15) >> 4) <= 8;
 }
 static bool fast_type(int qt) { return qt == CAI_Q4_K || qt == CAI_Q4_0 || qt == CAI_Q8_0; }
 
@@ -617,12 +611,11 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
     p.seg[i].y_off = m.y_off[i];
   }
   const int qt = w0->qtype;
-  if ((qt == CAI_Q4_K || (qt == CAI_Q4_0 && p.cols % 256 == 0) || (qt == CAI_Q6_K && m.n == 1 && !swiglu_half)) && n_b == 1 && !m.slot_expert && stream_kernel_enabled()) {
+  if ((qt == CAI_Q4_K || (qt == CAI_Q4_0 && p.cols % 256 == 0) || (qt == CAI_Q6_K && m.n == 1 && !swiglu_half)) && n_b == 1 && !m.slot_expert) {
     MultiGemv mm = m;
     if (swiglu_half) { if (m.n != 1) return set_error(CAI_ERR_INVALID, "gemv: swiglu takes one matrix"); p.seg[0].rows = swiglu_half; }
     p.ssq_in = m.ssq_in; p.ssq_out = m.ssq_out;
-    static const bool float_x = []() { const char* e = getenv("CAIHIP_GEMV_FLOAT_X"); return e && e[0] == '1'; }();
-    const int rc = (float_x && qt == CAI_Q4_K) ? launch_q4k_stream(p, mm, swiglu_half, c.stream) : launch_q4k_dot(p, mm, swiglu_half, c.stream);
+    const int rc = launch_q4k_dot(p, mm, swiglu_half, c.stream);
     p.ssq_in = nullptr; p.ssq_out = nullptr;
     if (rc != CAI_ERR_UNSUPPORTED) return rc;
   }

@@ -60,6 +60,7 @@ struct GemvParams {
   const float* norm_gain; float norm_eps;  // fused RMSNorm on the input when norm_gain != null
   const float* ssq_in;   // optional: sum(x^2) as SSQ_PARTS partials written by the kernel that produced x
   float* ssq_out;        // optional: this kernel's per-work-group partials of sum(y^2) (SSQ_PARTS slots)
+  int ssq_n;             // slots of the partial arrays in use (a multiple of 64, >= any producer grid on this device: the CU count rounded up)
   int cols;
   int kp;                // panel length in floats (multiple of 256)
   int kp_lds;            // LDS floats reserved per batch row: kp rounded up to whole 16-unit tiles

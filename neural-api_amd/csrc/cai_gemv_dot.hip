@@ -148,20 +148,30 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
     const float4* src = reinterpret_cast<const float4*>(p.x);
     const float4* gsrc = reinterpret_cast<const float4*>(p.norm_gain);
     const int n8 = cols >> 3, nthr = blockDim.x;
-    // one thread = 8 consecutive activations (a quarter of a 32-block: the block's four threads are one DPP quad);
-    // the first eight are requested before the sum of squares is gathered, every later eight one turn ahead
-    int n = threadIdx.x;
-    float4 c0 = {0, 0, 0, 0}, c1 = c0, cg0 = c0, cg1 = c0;
-    if (n < n8) {
-      c0 = src[2 * n]; c1 = src[2 * n + 1];
-      if (p.norm_gain) { cg0 = gsrc[2 * n]; cg1 = gsrc[2 * n + 1]; }
-    }
+    // one thread = 8 consecutive activations (a quarter of a 32-block: the block's four threads are one DPP quad).
+    // A thread's turns (n, n + nthr, ...) are requested SD at a time - a long row (the 18944-wide down projection: four
+    // turns) costs one cache round trip instead of one per turn; the first batch goes out before the sum of squares.
+    constexpr int SD = (MODE == 1 || MULTISEG) ? 1 : 4;   // (the fused-norm walks have rows of one turn; batching only costs them registers)
+    typedef float f4 __attribute__((ext_vector_type(4)));   // (arrays of HIP's float4 struct end up in scratch memory)
+    const f4* src4 = reinterpret_cast<const f4*>(p.x);
+    const f4* gsrc4 = reinterpret_cast<const f4*>(p.norm_gain);
+    f4 c0[SD], c1[SD], cg0[SD], cg1[SD];
+    auto request = [&](int n0) {
+#pragma unroll
+      for (int u = 0; u < SD; u++) {
+        const int nn = min(n0 + u * nthr, n8 - 1);     // past the end: the last eight again (not used)
+        c0[u] = src4[2 * nn]; c1[u] = src4[2 * nn + 1];
+        if (p.norm_gain) { cg0[u] = gsrc4[2 * nn]; cg1[u] = gsrc4[2 * nn + 1]; }
+        else { cg0[u] = (f4)(0.0f); cg1[u] = (f4)(0.0f); }
+      }
+    };
+    request(threadIdx.x);
     if (p.norm_gain) {
       float t = 0.0f;
       if (p.ssq_in) {
         // sum of squares of x delivered by the producing kernel as SSQ_PARTS per-work-group partials (fixed order)
-#pragma unroll
-        for (int i = 0; i < SSQ_PARTS / 64; i++) t += p.ssq_in[i * 64 + lane];
+#pragma unroll 4
+        for (int i = 0; i < p.ssq_n / 64; i++) t += p.ssq_in[i * 64 + lane];
         t = wave_sum(t);
         t = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, t), 63));
       } else {
@@ -182,14 +192,14 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
       }
       inv_rms = 1.0f / sqrtf(t / (float)cols + p.norm_eps);
     }
-    while (n < n8) {
-      float4 v0 = c0, v1 = c1;
-      const float4 g0 = cg0, g1 = cg1;
-      const int nn = n + nthr;
-      if (nn < n8) {
-        c0 = src[2 * nn]; c1 = src[2 * nn + 1];
-        if (p.norm_gain) { cg0 = gsrc[2 * nn]; cg1 = gsrc[2 * nn + 1]; }
-      }
+    for (int n0 = threadIdx.x; n0 < n8; n0 += SD * nthr) {
+     if (n0 != (int)threadIdx.x) request(n0);
+#pragma unroll
+     for (int t = 0; t < SD; t++) {
+      const int n = n0 + t * nthr;
+      if (n < n8) {
+      f4 v0 = c0[t], v1 = c1[t];
+      const f4 g0 = cg0[t], g1 = cg1[t];
       if (p.norm_gain) {
         v0.x = g0.x * (v0.x * inv_rms); v0.y = g0.y * (v0.y * inv_rms); v0.z = g0.z * (v0.z * inv_rms); v0.w = g0.w * (v0.w * inv_rms);
         v1.x = g1.x * (v1.x * inv_rms); v1.y = g1.y * (v1.y * inv_rms); v1.z = g1.z * (v1.z * inv_rms); v1.w = g1.w * (v1.w * inv_rms);
@@ -225,7 +235,8 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
         float* fr = reinterpret_cast<float*>(rec + (size_t)xq_slot(u, NL * 4) * 4);
         fr[hb] = s_blk; fr[2 + hb] = s_blk * (float)isum;
       }
-      n = nn;
+      }
+     }
     }
     __syncthreads();
   }
@@ -442,7 +453,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
       for (int w = 0; w < (int)(blockDim.x >> 6); w++) tot += s_ss[w];
       p.ssq_out[blockIdx.x] = tot;
     }
-    if (blockIdx.x == 0) for (int i = gridDim.x + threadIdx.x; i < SSQ_PARTS; i += blockDim.x) p.ssq_out[i] = 0.0f;
+    if (blockIdx.x == 0) for (int i = gridDim.x + threadIdx.x; i < p.ssq_n; i += blockDim.x) p.ssq_out[i] = 0.0f;
   }
 }
 
@@ -473,14 +484,12 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
   if (nsw > 8 || cols % 256) return CAI_ERR_UNSUPPORTED;  // rows longer than 32768 columns; Q4_0 widths that are not whole 256-blocks
   const bool q6k = m.w[0]->qtype == CAI_Q6_K;
   if (q6k && (swiglu_half || m.n != 1)) return CAI_ERR_UNSUPPORTED;
-  static const int ns_env = []() { const char* e = getenv("CAIHIP_DOT_NS"); return e ? atoi(e) : 2; }();
-  static const int W = []() { const char* e = getenv("CAIHIP_DOT_W"); return e ? atoi(e) : 12; }();   // resident waves per CU
+  constexpr int W = 12;   // resident waves per CU
   // waves per work-group: short rows (one or two waves span the columns) use ONE work-group of 8 waves per CU - the
   // activation is quantised once per CU instead of once per 4 waves, which outweighs the lower wave count (measured:
   // 3 work-groups of 4 waves 537 tok/s, 1 of 12 waves 544, 1 of 8 waves 561 on the 7B shape); long rows fill the CU
   // with a single work-group of up to 12 waves
-  static const int gw_env = []() { const char* e = getenv("CAIHIP_DOT_GWV"); return e ? atoi(e) : 8; }();
-  const int gwv = nsw >= 3 ? std::max(1, std::min(W, 12) / nsw) : std::max(1, std::min(std::max(gw_env, 1), 12) / nsw);   // the kernel is built for at most 12 waves per work-group
+  const int gwv = nsw >= 3 ? std::max(1, W / nsw) : 8 / nsw;   // the kernel is built for at most 12 waves per work-group
   int64_t total = 0;
   for (int i = 0; i < m.n; i++) total += swiglu_half ? swiglu_half : m.rows[i];
   const int waves_per_wg = nsw * gwv;
@@ -488,7 +497,6 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
   int wg_per_cu = W / waves_per_wg; if (wg_per_cu < 1) wg_per_cu = 1;
   { const int lds_fit = (int)((160 * 1024 - 4096) / (lds + 1024)); if (wg_per_cu > lds_fit) wg_per_cu = lds_fit < 1 ? 1 : lds_fit; }
   const int max_wgs = c.n_cu * wg_per_cu;
-  static const int r_env = []() { const char* e = getenv("CAIHIP_DOT_R"); return e ? atoi(e) : 0; }();
   // Two rows per group halve the turns of a wave and double what it has in flight.  With long rows (three or more waves
   // per row, every wave's lanes full) that only pays when the turns come out even - 7B down projection: 7 turns of one row
   // beat 4 of two, 570 -> 580 tok/s; with one or two waves per row two rows measured better even at uneven turns (32B
@@ -499,7 +507,6 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
     const int64_t turns1 = (total + slots - 1) / slots, turns2 = ((total + 1) / 2 + slots - 1) / slots;
     if (nsw < 3 || 2 * turns2 <= turns1) R = 2;
   }
-  if (!swiglu_half && (r_env == 1 || r_env == 2)) R = r_env;
   if (q6k) R = 1;   // (two rows of Q6_K requests in flight twice over do not fit the registers)
   int cum = 0;
   for (int i = 0; i < m.n; i++) {
@@ -507,7 +514,10 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
     cum += (int)((rows + R - 1) / R);
     p.seg[i].grp_end = cum;
   }
-  const int grid = std::min(std::min((cum + gwv - 1) / gwv, max_wgs), SSQ_PARTS);
+  // sum-of-squares hand-off: producer and consumer agree on the slots in use (one work-group per CU is what every geometry
+  // above launches; a larger grid is cut to the slot count)
+  p.ssq_n = std::min(SSQ_PARTS, (c.n_cu + 63) / 64 * 64);
+  const int grid = std::min(std::min((cum + gwv - 1) / gwv, max_wgs), p.ssq_n);
   const dim3 block(64 * waves_per_wg);
   auto go = [&](auto kern) {
     static std::set<const void*> raised;   // kernels whose dynamic-LDS limit has been raised
@@ -528,8 +538,7 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
     else if (m.n > 1) { if (R == 2) go(gemv_q4k_dot<2, 0, true, NSV>); else go(gemv_q4k_dot<1, 0, true, NSV>); }
     else { if (R == 2) go(gemv_q4k_dot<2, 0, false, NSV>); else go(gemv_q4k_dot<1, 0, false, NSV>); }
   };
-  if (ns_env == 3) pick(std::integral_constant<int, 3>());
-  else pick(std::integral_constant<int, 2>());
+  pick(std::integral_constant<int, 2>());   // two row groups per wave: one in flight while one is reduced (three measured slower on every shape)
   return CAI_OK;
 }
 

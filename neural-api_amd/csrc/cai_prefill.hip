@@ -494,12 +494,10 @@ int launch_gemm_q4k(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo,
   }
   // Tiling: two row tiles per wave (256 rows per work-group, 32 tokens) when that still gives every CU several
   // work-groups; else 128 rows with two token tiles, or with one for matrices with few row groups.
-  static const int tt_force = []() { const char* e = getenv("CAIHIP_PF_TT"); return e ? atoi(e) : 0; }();   // 1, 2: token tiles; 3: two row tiles
   const int n_cu = ctx().n_cu;
   const int wgs_rt2 = ((p.rows + 255) / 256) * ((n_tok + 31) / 32);
   const int wgs_tt2 = ((p.rows + 127) / 128) * ((n_tok + 63) / 64);
-  int mode = wgs_rt2 >= 4 * n_cu ? 3 : (wgs_tt2 < 2 * n_cu ? 1 : 2);
-  if (tt_force >= 1 && tt_force <= 3) mode = tt_force;
+  const int mode = wgs_rt2 >= 4 * n_cu ? 3 : (wgs_tt2 < 2 * n_cu ? 1 : 2);   // 1, 2: token tiles; 3: two row tiles
   const int rt = mode == 3 ? 2 : 1, tt = mode == 2 ? 2 : 1;
   p.n_row_groups = (p.rows + 128 * rt - 1) / (128 * rt);
   p.n_tok_tiles = (n_tok + tt * 32 - 1) / (tt * 32);

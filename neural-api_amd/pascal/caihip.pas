@@ -90,6 +90,7 @@ function cai_decoder_set_weight(d: TCaiDecoder; layer, slot: LongInt; w: TCaiQW)
 function cai_decoder_set_vector(d: TCaiDecoder; layer, slot: LongInt; v_host: PSingle; n: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_step(d: TCaiDecoder; tokens, pos: PLongInt; n_b: LongInt; logits: PSingle; argmax: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_generate(d: TCaiDecoder; first_token, pos, n_tokens: LongInt; tokens_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_decoder_profile(d: TCaiDecoder; token, reps: LongInt; us_per_step_out: PSingle; n_classes: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_prefill(d: TCaiDecoder; seq: LongInt; tokens: PLongInt; n, pos0: LongInt; last_logits: PSingle; argmax: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_reset(d: TCaiDecoder; seq: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_truncate(d: TCaiDecoder; seq, n: LongInt): LongInt; cdecl; external CAIHIP_LIB;
