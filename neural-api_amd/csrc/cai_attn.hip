@@ -432,18 +432,19 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const AttnParams p)
           p.out[(int64_t)seq * p.out_stride + qh * hd + d] = Ls > 0.0f ? A * (1.0f / Ls) : 0.0f;
         } else {
           float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + split) * (hd + 2);
-          if (p.merge_cnt) { part_store(pt + d, A); if (d == 0) { part_store(pt + hd, M); part_store(pt + hd + 1, Ls); } }
-          else { pt[d] = A; if (d == 0) { pt[hd] = M; pt[hd + 1] = Ls; } }
+          pt[d] = A;
+          if (d == 0) { pt[hd] = M; pt[hd + 1] = Ls; }
         }
       }
     }
     __syncthreads();
   }
-  if (n_active > 1 && p.merge_cnt) merge_if_last(p, seq, g * G, G, s_first, n_active, seq * p.kv_heads * 8 + g);
 }
 
-// ---- merge of the split partials: one work-group per query head; all partial loads are issued together ----
-__global__ __launch_bounds__(128) void attn_merge_kernel(const AttnParams p)
+// ---- merge of the split partials: one work-group per query head.  Four quarter-groups of head_dim threads each take every
+//      fourth slice (all their loads go out together: one round trip for up to 32 slices per quarter), fold them with a running
+//      maximum, and meet in LDS. ----
+__global__ __launch_bounds__(512) void attn_merge_kernel(const AttnParams p)
 {
   const int qh = blockIdx.x, seq = blockIdx.y;
   const int hd = p.hd;
@@ -452,26 +453,38 @@ __global__ __launch_bounds__(128) void attn_merge_kernel(const AttnParams p)
   const int n_active = s_last - s_first + 1;
   if (n_active == 1) return;                       // the split kernel already wrote the final row
   const float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + s_first) * (hd + 2);
-  __shared__ float mM[128], mL[128];
-  for (int s = threadIdx.x; s < n_active; s += blockDim.x) { mM[s] = pt[(int64_t)s * (hd + 2) + hd]; mL[s] = pt[(int64_t)s * (hd + 2) + hd + 1]; }
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-    float A = 0.0f, L = 0.0f, M = -1e30f;
-    bool first = true;
-    for (int s0 = 0; s0 < n_active; s0 += 16) {
-      float v[16];
+  __shared__ float qA[4][128], qM[4], qL[4];
+  const int quarter = threadIdx.x >> 7, d = threadIdx.x & 127;
+  float A = 0.0f, L = 0.0f, M = -1e30f;
+  if (d < hd) {
+    for (int s0 = quarter; s0 < n_active; s0 += 4 * 8) {
+      float v[8], ms[8], ls[8];
 #pragma unroll
-      for (int u = 0; u < 16; u++) v[u] = s0 + u < n_active ? pt[(int64_t)(s0 + u) * (hd + 2) + d] : 0.0f;
-      if (first) { __syncthreads(); for (int s = 0; s < n_active; s++) M = fmaxf(M, mM[s]); first = false; }
+      for (int u = 0; u < 8; u++) {
+        const float* ps = pt + (int64_t)min(s0 + 4 * u, n_active - 1) * (hd + 2);
+        v[u] = ps[d]; ms[u] = ps[hd]; ls[u] = ps[hd + 1];
+      }
 #pragma unroll
-      for (int u = 0; u < 16; u++) {
-        if (s0 + u < n_active) {
-          const float ls = mL[s0 + u];
-          const float e = ls > 0.0f ? expf(mM[s0 + u] - M) : 0.0f;
-          L = fmaf(ls, e, L); A = fmaf(v[u], e, A);
+      for (int u = 0; u < 8; u++) {
+        if (s0 + 4 * u < n_active && ls[u] > 0.0f) {
+          const float mn = fmaxf(M, ms[u]), c0 = expf(M - mn), c1 = expf(ms[u] - mn);
+          A = fmaf(v[u], c1, A * c0); L = fmaf(ls[u], c1, L * c0); M = mn;
         }
       }
     }
-    p.out[(int64_t)seq * p.out_stride + qh * hd + d] = L > 0.0f ? A * (1.0f / L) : 0.0f;
+    qA[quarter][d] = A;
+    if (d == 0) { qM[quarter] = M; qL[quarter] = L; }
+  }
+  __syncthreads();
+  if (quarter == 0 && d < hd) {
+    const float Mx = fmaxf(fmaxf(qM[0], qM[1]), fmaxf(qM[2], qM[3]));
+    float At = 0.0f, Lt = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+      const float e = qL[k] > 0.0f ? expf(qM[k] - Mx) : 0.0f;
+      At = fmaf(qA[k][d], e, At); Lt = fmaf(qL[k], e, Lt);
+    }
+    p.out[(int64_t)seq * p.out_stride + qh * hd + d] = Lt > 0.0f ? At * (1.0f / Lt) : 0.0f;
   }
 }
 
@@ -1018,10 +1031,13 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   p.seq_mul = prompt_rows ? 0 : 1; p.appended = prompt_rows ? 1 : 0;
   p.evict_sinks = kv->evict_sinks; p.evict_cap = kv->evict_cap;
   p.ksc = kv->ks; p.vsc = kv->vs; p.seq_rows = kv->seq_rows(); p.layer_row_off = (int64_t)layer * kv->layer_rows();
-  p.merge_cnt = prompt_rows ? nullptr : kv->merge_cnt;   // (a prompt has more rows in flight than the counters cover: merge launch)
   int rc;
   const int group_min = c.n_cu;   // smallest grid that fills the chip with one work-group per (slice, KV head)
   const bool grouped = (kv->head_dim & 7) == 0 && n_seq * kv->kv_heads * kv->n_splits >= group_min;
+  // The per-head kernel merges its slices itself (one work-group per head does a head's merge).  A prompt has more rows in
+  // flight than the counters cover, and in the per-KV-head kernel the last arriver would fold a whole group of heads over
+  // many slices alone (32B shape, 33 slices x 5 heads: 37.7 us against 30.7 us with the merge launch): those keep the launch.
+  p.merge_cnt = (prompt_rows || grouped) ? nullptr : kv->merge_cnt;
   if (qn_gain) {
     // q and k norms over the whole rows: the per-head decode kernel applies them while it reads its operands; the
     // other kernels find the rows normalised in place
@@ -1075,7 +1091,7 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   else
     rc = kv->dtype == CAI_KV_I8 ? launch_split_head<int8_t>(p, n_seq, c.stream) : kv->dtype == CAI_KV_F16 ? launch_split_head<__half>(p, n_seq, c.stream) : launch_split_head<float>(p, n_seq, c.stream);
   if (rc) return rc;
-  if (p.n_splits > 1 && !p.merge_cnt) hipLaunchKernelGGL(attn_merge_kernel, dim3(q_heads, n_seq), dim3(128), 0, c.stream, p);
+  if (p.n_splits > 1 && !p.merge_cnt) hipLaunchKernelGGL(attn_merge_kernel, dim3(q_heads, n_seq), dim3(512), 0, c.stream, p);
   return CAI_OK;
 }
 
