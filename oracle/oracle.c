@@ -78,8 +78,8 @@ int64_t orc_block_elems(int type)
 {
   switch (type) {
     case ORC_F32: case ORC_F16: case ORC_I8ROW: return 1;
-    case ORC_Q4_0: case ORC_Q8_0: return 32;
-    case ORC_Q4_K: case ORC_Q6_K: return 256;
+    case ORC_Q4_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: case ORC_Q8_0: return 32;
+    case ORC_Q2_K: case ORC_Q3_K: case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: return 256;
   }
   return -1;
 }
@@ -88,6 +88,8 @@ int64_t orc_block_bytes(int type)
   switch (type) {
     case ORC_F32: return 4; case ORC_F16: return 2; case ORC_I8ROW: return 1;
     case ORC_Q4_0: return 18; case ORC_Q8_0: return 34; case ORC_Q4_K: return 144; case ORC_Q6_K: return 210;
+    case ORC_Q4_1: return 20; case ORC_Q5_0: return 22; case ORC_Q5_1: return 24;    /* neuralgguf.pas:129-138 */
+    case ORC_Q2_K: return 84; case ORC_Q3_K: return 110; case ORC_Q5_K: return 176;  /* neuralgguf.pas:115-125 */
   }
   return -1;
 }
@@ -212,6 +214,105 @@ void orc_quant_q6_k(const float* x, int64_t n, uint8_t* out)
   }
 }
 
+/* neural/neuralgguf.pas:516-587 (DequantizeQ5K): 176-byte super-block = f16 d, f16 dmin, 12 packed scale bytes (the Q4_K
+ * packing), 32 B qh (one bit plane: sub-block j takes bit j of byte i mod 32), 128 B ql (Q4_K's nibble layout);
+ * q = ql | qh_bit << 4 in 0..31, x = (d*sc_j)*q - dmin*mn_j.  d*sc*q has <= 22 significant bits: every product is exact and
+ * the subtraction rounds once, whatever the evaluation order.
+ * Pinned by: bit-exact against tiny_kquant_ref.json["dequant"]["Q5_K"] (gguf-py values), tests/test_oracle_codecs.py. */
+void orc_dequant_q5_k(const uint8_t* raw, int64_t nb, float* out)
+{
+  for (int64_t b = 0; b < nb; b++, raw += 176, out += 256) {
+    uint16_t h; memcpy(&h, raw, 2); const float d = orc_f16_to_f32(h);
+    memcpy(&h, raw + 2, 2); const float dmin = orc_f16_to_f32(h);
+    uint8_t sc[8], mn[8]; orc_q4k_scale_min(raw + 4, sc, mn);
+    const uint8_t* qh = raw + 16; const uint8_t* ql = raw + 48;
+    for (int c = 0; c < 4; c++) {
+      const int jlo = 2 * c;
+      const float dsc_lo = d * (float)sc[jlo], dm_lo = dmin * (float)mn[jlo], dsc_hi = d * (float)sc[jlo + 1], dm_hi = dmin * (float)mn[jlo + 1];
+      for (int i = 0; i < 32; i++) {
+        const uint8_t qlb = ql[32 * c + i], qhb = qh[i];
+        const int q_lo = (qlb & 0x0F) | (((qhb >> jlo) & 1) << 4), q_hi = (qlb >> 4) | (((qhb >> (jlo + 1)) & 1) << 4);
+        out[64 * c + i] = (float)((double)dsc_lo * (double)q_lo - (double)dm_lo);
+        out[64 * c + 32 + i] = (float)((double)dsc_hi * (double)q_hi - (double)dm_hi);
+      }
+    }
+  }
+}
+
+/* neural/neuralgguf.pas:588-648 (DequantizeQ2K): 84-byte super-block = 16 bytes scale | min (low / high nibble, one per
+ * 16-element sub-block), 64 B of 2-bit quants, f16 d, f16 dmin.  Element e: byte (e/128)*32 + e%32, field at shift
+ * 2*((e%128)/32); x = (d*scale)*q - dmin*min.
+ * Pinned by: bit-exact against tiny_kquant_ref.json["dequant"]["Q2_K"]. */
+void orc_dequant_q2_k(const uint8_t* raw, int64_t nb, float* out)
+{
+  for (int64_t b = 0; b < nb; b++, raw += 84, out += 256) {
+    uint16_t h; memcpy(&h, raw + 80, 2); const float d = orc_f16_to_f32(h);
+    memcpy(&h, raw + 82, 2); const float dmin = orc_f16_to_f32(h);
+    for (int e = 0; e < 256; e++) {
+      const uint8_t scb = raw[e >> 4];
+      const float dl = d * (float)(scb & 0x0F), ml = dmin * (float)(scb >> 4);
+      const int q = (raw[16 + (e >> 7) * 32 + (e & 31)] >> (2 * ((e & 127) >> 5))) & 3;
+      out[e] = (float)((double)dl * (double)q - (double)ml);
+    }
+  }
+}
+
+/* neural/neuralgguf.pas:718-806 (DequantizeQ3K): 110-byte super-block = 32 B hmask (third bit plane: bit e/32 of byte e%32),
+ * 64 B qs (2-bit fields laid out like Q2_K), 12 bytes of 6-bit scales (bytes 0..7: low nibble = scale j, high = scale j+8;
+ * bytes 8..11: two high bits of scales b, b+4, b+8, b+12 at shifts 0,2,4,6), f16 d.  scale = 6-bit value - 32;
+ * q = ql - 4 when the hmask bit is CLEAR; x = (d*scale)*q.
+ * Pinned by: the hand-built super-block of tests/TestNeuralPretrained.pas:6238-6299 (scales sb+24, codes e mod 4, hmask bit
+ * (e mod 3) & 1) against its closed form; an independent vectorised restatement on random bytes. */
+void orc_dequant_q3_k(const uint8_t* raw, int64_t nb, float* out)
+{
+  for (int64_t b = 0; b < nb; b++, raw += 110, out += 256) {
+    const uint8_t* hm = raw; const uint8_t* qs = raw + 32; const uint8_t* sp = raw + 96;
+    uint16_t h; memcpy(&h, raw + 108, 2); const float d = orc_f16_to_f32(h);
+    for (int e = 0; e < 256; e++) {
+      const int j = e >> 4;
+      const int lsc = j < 8 ? (sp[j & 7] & 0x0F) : (sp[j & 7] >> 4);
+      const int hsc = (sp[8 + (j & 3)] >> (2 * (j >> 2))) & 3;
+      const float dl = d * (float)((lsc | (hsc << 4)) - 32);
+      const int ql = (qs[(e >> 7) * 32 + (e & 31)] >> (2 * ((e & 127) >> 5))) & 3;
+      const int qh = ((hm[e & 31] >> (e >> 5)) & 1) ^ 1;
+      out[e] = dl * (float)(ql - (qh << 2));
+    }
+  }
+}
+
+/* Legacy 32-element blocks (neural/neuralgguf.pas:846-944); the nibble of element e is LegacyNibble (811-817): low nibble of
+ * byte e for e < 16, high nibble of byte e - 16 otherwise; the fifth bit of Q5_x is bit e of a little-endian 32-bit plane.
+ *   Q4_1 (20 B: f16 d, f16 m, 16 B nibbles):           x = d*nibble + m
+ *   Q5_0 (22 B: f16 d, 4 B qh, 16 B nibbles):           x = d*((nibble | bit<<4) - 16)
+ *   Q5_1 (24 B: f16 d, f16 m, 4 B qh, 16 B nibbles):    x = d*(nibble | bit<<4) + m
+ * Pinned by: the hand-built blocks of tests/TestNeuralPretrained.pas:6145-6236 against their closed forms. */
+static int legacy_nibble(const uint8_t* qs, int e) { return e < 16 ? (qs[e] & 0x0F) : (qs[e - 16] >> 4); }
+void orc_dequant_q4_1(const uint8_t* raw, int64_t nb, float* out)
+{
+  for (int64_t b = 0; b < nb; b++, raw += 20, out += 32) {
+    uint16_t h; memcpy(&h, raw, 2); const float d = orc_f16_to_f32(h);
+    memcpy(&h, raw + 2, 2); const float m = orc_f16_to_f32(h);
+    for (int e = 0; e < 32; e++) out[e] = (float)((double)d * (double)legacy_nibble(raw + 4, e) + (double)m);
+  }
+}
+void orc_dequant_q5_0(const uint8_t* raw, int64_t nb, float* out)
+{
+  for (int64_t b = 0; b < nb; b++, raw += 22, out += 32) {
+    uint16_t h; memcpy(&h, raw, 2); const float d = orc_f16_to_f32(h);
+    uint32_t qh; memcpy(&qh, raw + 2, 4);
+    for (int e = 0; e < 32; e++) out[e] = d * (float)((legacy_nibble(raw + 6, e) | (int)(((qh >> e) & 1u) << 4)) - 16);
+  }
+}
+void orc_dequant_q5_1(const uint8_t* raw, int64_t nb, float* out)
+{
+  for (int64_t b = 0; b < nb; b++, raw += 24, out += 32) {
+    uint16_t h; memcpy(&h, raw, 2); const float d = orc_f16_to_f32(h);
+    memcpy(&h, raw + 2, 2); const float m = orc_f16_to_f32(h);
+    uint32_t qh; memcpy(&qh, raw + 4, 4);
+    for (int e = 0; e < 32; e++) out[e] = (float)((double)d * (double)(legacy_nibble(raw + 8, e) | (int)(((qh >> e) & 1u) << 4)) + (double)m);
+  }
+}
+
 /* neural/neuralgguf.pas:1471-1523 (DecodeGGMLSpan) */
 int orc_dequant(int type, const void* raw, int64_t n, float* out)
 {
@@ -223,6 +324,12 @@ int orc_dequant(int type, const void* raw, int64_t n, float* out)
     case ORC_Q4_0: if (n % 32) return -1; orc_dequant_q4_0(p, n / 32, out); return 0;
     case ORC_Q4_K: if (n % 256) return -1; orc_dequant_q4_k(p, n / 256, out); return 0;
     case ORC_Q6_K: if (n % 256) return -1; orc_dequant_q6_k(p, n / 256, out); return 0;
+    case ORC_Q5_K: if (n % 256) return -1; orc_dequant_q5_k(p, n / 256, out); return 0;
+    case ORC_Q2_K: if (n % 256) return -1; orc_dequant_q2_k(p, n / 256, out); return 0;
+    case ORC_Q3_K: if (n % 256) return -1; orc_dequant_q3_k(p, n / 256, out); return 0;
+    case ORC_Q4_1: if (n % 32) return -1; orc_dequant_q4_1(p, n / 32, out); return 0;
+    case ORC_Q5_0: if (n % 32) return -1; orc_dequant_q5_0(p, n / 32, out); return 0;
+    case ORC_Q5_1: if (n % 32) return -1; orc_dequant_q5_1(p, n / 32, out); return 0;
   }
   return -2;
 }

@@ -10,6 +10,7 @@ ORACLE_DIR = os.path.join(ROOT, "oracle")
 _LIB = None
 
 F32, F16, Q4_0, Q8_0, Q4_K, Q6_K, I8ROW = 0, 1, 2, 8, 12, 14, 100
+Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K = 3, 6, 7, 10, 11, 13   # decoded by the reference too (neural/neuralgguf.pas:1471-1523)
 W_EMBED, W_HEAD, W_Q, W_K, W_V, W_O, W_GATEUP, W_DOWN, W_ROUTER = range(9)
 V_ATTN_NORM, V_MLP_NORM, V_FINAL_NORM, V_Q_NORM, V_K_NORM = range(5)
 
