@@ -30,8 +30,14 @@ extern "C" {
 #define CAI_F32    0
 #define CAI_F16    1
 #define CAI_Q4_0   2
+#define CAI_Q4_1   3   /* the six types below stay resident as the stored block stream (neural/neuralgguf.pas:516-648, 718-944) */
+#define CAI_Q5_0   6
+#define CAI_Q5_1   7
 #define CAI_Q8_0   8
+#define CAI_Q2_K   10
+#define CAI_Q3_K   11
 #define CAI_Q4_K   12
+#define CAI_Q5_K   13
 #define CAI_Q6_K   14  /* 210-byte super-blocks (neural/neuralgguf.pas:639-717); resident as aligned ql|qh records + planes of scales and d */
 #define CAI_I8ROW  100  /* per-row symmetric int8 + fp32 row scale (neural/neuralvolume.pas:926-987) */
 

@@ -7,6 +7,7 @@ import numpy as np
 from . import lib_path
 
 F32, F16, Q4_0, Q8_0, Q4_K, Q6_K, I8ROW = 0, 1, 2, 8, 12, 14, 100
+Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K = 3, 6, 7, 10, 11, 13
 ACT_NONE, ACT_RELU, ACT_SIGMOID, ACT_TANH = 0, 1, 2, 3
 X_DEVICE, Y_DEVICE, MATRIX_CORES = 1, 2, 4
 KV_F32, KV_F16, KV_I8 = 0, 1, 2

@@ -43,11 +43,13 @@ int ensure_stage(void** p, size_t* cap, size_t need)
 int64_t block_elems(int qt)
 {
   switch (qt) { case CAI_F32: case CAI_F16: case CAI_I8ROW: return 1; case CAI_Q4_0: case CAI_Q8_0: return 32; case CAI_Q4_K: case CAI_Q6_K: return 256; }
+  if (raw_block_type(qt)) return raw_block_elems(qt);
   return -1;
 }
 int64_t block_bytes(int qt)
 {
   switch (qt) { case CAI_F32: return 4; case CAI_F16: return 2; case CAI_I8ROW: return 1; case CAI_Q4_0: return 18; case CAI_Q8_0: return 34; case CAI_Q4_K: return 144; case CAI_Q6_K: return 210; }
+  if (raw_block_type(qt)) return raw_block_bytes(qt);
   return -1;
 }
 

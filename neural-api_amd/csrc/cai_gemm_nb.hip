@@ -493,7 +493,6 @@ __global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
   const int n = lane & 15, kg = lane >> 4;
   const int K = p.cols, nsb = K >> 8;
   const int slice = blockIdx.y, sb0 = slice * S, nS = min(S, nsb - sb0);
-  const int64_t row_bytes = (int64_t)nsb * 192;
   const int tile0 = blockIdx.x * 4 + wave;
   const int n_it = tile0 < p.n_tiles ? (p.n_tiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
   const int nq = n_it * nS;                      // (tile, super-block) items of this wave

@@ -10,6 +10,7 @@
 // (reference: neural/neuralvolume.pas:12127-12423, 12693-12745; fused tail neural/neural.cl:111-146).
 #include "cai_internal.hpp"
 #include "cai_gemv_common.hpp"
+#include "cai_blocks_raw.hpp"
 
 namespace cai {
 
@@ -486,6 +487,86 @@ __global__ __launch_bounds__(256) void gemv_simple(const GemvParams p, int n_b)
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Block types resident as the stored stream (Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K).  One wave per row; a lane decodes runs
+// of 16 consecutive weights (run = lane + 64 k, so the 16 lanes of a super-block share its header in cache) and feeds
+// every batch row from the one decode.  fp32 accumulation; fused RMSNorm, bias, activation, residual and the expert-bank
+// gather as in the other kernels.
+// ------------------------------------------------------------------------------------------
+template <int QT>
+__global__ __launch_bounds__(256) void gemv_raw(const GemvParams p, int n_b)
+{
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t grow = (int64_t)blockIdx.x * 4 + wave;
+  int s = 0; int64_t g0 = 0;
+  if (p.n_seg > 1 && grow >= p.seg[0].grp_end) { s = 1; g0 = p.seg[0].grp_end; }
+  if (p.n_seg > 2 && grow >= p.seg[1].grp_end) { s = 2; g0 = p.seg[1].grp_end; }
+  if (grow >= p.seg[p.n_seg - 1].grp_end) return;
+  const GemvSeg sg = p.seg[s];
+  const int row = (int)(grow - g0);
+  const int cols = p.cols;
+  int64_t bank_row = 0;
+  const float* xin = p.x; float* yout = p.y;
+  if (p.slot_expert) {
+    bank_row = (int64_t)min(max(p.slot_expert[blockIdx.y], 0), p.bank_experts - 1) * p.expert_rows;
+    xin += (int64_t)blockIdx.y * p.x_slot_stride; yout += (int64_t)blockIdx.y * p.y_slot_stride;
+  }
+  const int64_t wrow = bank_row + row;
+  const uint8_t* wbase = sg.data + wrow * (int64_t)(cols / raw_block_elems(QT)) * raw_block_bytes(QT);
+  float inv[8];
+#pragma unroll
+  for (int b = 0; b < 8; b++) {
+    inv[b] = 1.0f;
+    if (p.norm_gain && b < n_b) {
+      const float* xb = xin + (int64_t)b * cols;
+      float ss = 0.0f;
+      for (int i = lane * 4; i < cols; i += 256) { const float4 v = *reinterpret_cast<const float4*>(xb + i); ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss); }
+      ss = __shfl(wave_sum(ss), 63);
+      inv[b] = 1.0f / sqrtf(ss / (float)cols + p.norm_eps);
+    }
+  }
+  float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+  const int n_runs = cols >> 4;
+  for (int run = lane; run < n_runs; run += 64) {
+    float w[16];
+    raw_run16<QT>(wbase, run, w);
+    float g[16];
+    if (p.norm_gain) {
+#pragma unroll
+      for (int q = 0; q < 4; q++) { const float4 v = *reinterpret_cast<const float4*>(p.norm_gain + 16 * run + 4 * q); g[4 * q] = v.x; g[4 * q + 1] = v.y; g[4 * q + 2] = v.z; g[4 * q + 3] = v.w; }
+    }
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+      if (b < n_b) {
+        const float* xb = xin + (int64_t)b * cols + 16 * run;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const float4 v = *reinterpret_cast<const float4*>(xb + 4 * q);
+          float xv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int t = 0; t < 4; t++) {
+            const float xn = p.norm_gain ? g[4 * q + t] * (xv[t] * inv[b]) : xv[t];
+            acc[b] = fmaf(w[4 * q + t], xn, acc[b]);
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int b = 0; b < 8; b++) {
+    if (b < n_b) {
+      float a = wave_sum(acc[b]);
+      if (lane == 63) {
+        if (sg.bias) a += sg.bias[wrow];
+        a = act_apply(a, p.act);
+        const int64_t o = (int64_t)b * p.y_stride + sg.y_off + row;
+        if (p.residual) a += p.residual[o];
+        yout[o] = a;
+      }
+    }
+  }
+}
+
 // y[b][i] = x[b][i] * silu(x[b][half+i]) for the simple path (unfused SwiGLU)
 __global__ void swiglu_rows(const float* x, int half, int n_tokens, float* y)
 {
@@ -571,6 +652,7 @@ static int64_t data_row_bytes(const cai_qw_s* w)
     case CAI_F32: return w->cols * 4;
     case CAI_F16: return w->cols * 2;
   }
+  if (raw_block_type(w->qtype)) return w->cols / raw_block_elems(w->qtype) * raw_block_bytes(w->qtype);
   return 0;
 }
 static int64_t aux_row_bytes(const cai_qw_s* w)
@@ -651,6 +733,12 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
   if (qt == CAI_F32) hipLaunchKernelGGL(gemv_simple<CAI_F32>, grid, dim3(256), 0, c.stream, p, n_b);
   else if (qt == CAI_F16) hipLaunchKernelGGL(gemv_simple<CAI_F16>, grid, dim3(256), 0, c.stream, p, n_b);
   else if (qt == CAI_I8ROW) hipLaunchKernelGGL(gemv_simple<CAI_I8ROW>, grid, dim3(256), 0, c.stream, p, n_b);
+  else if (qt == CAI_Q5_K) hipLaunchKernelGGL(gemv_raw<CAI_Q5_K>, grid, dim3(256), 0, c.stream, p, n_b);
+  else if (qt == CAI_Q2_K) hipLaunchKernelGGL(gemv_raw<CAI_Q2_K>, grid, dim3(256), 0, c.stream, p, n_b);
+  else if (qt == CAI_Q3_K) hipLaunchKernelGGL(gemv_raw<CAI_Q3_K>, grid, dim3(256), 0, c.stream, p, n_b);
+  else if (qt == CAI_Q4_1) hipLaunchKernelGGL(gemv_raw<CAI_Q4_1>, grid, dim3(256), 0, c.stream, p, n_b);
+  else if (qt == CAI_Q5_0) hipLaunchKernelGGL(gemv_raw<CAI_Q5_0>, grid, dim3(256), 0, c.stream, p, n_b);
+  else if (qt == CAI_Q5_1) hipLaunchKernelGGL(gemv_raw<CAI_Q5_1>, grid, dim3(256), 0, c.stream, p, n_b);
   else return set_error(CAI_ERR_UNSUPPORTED, "gemv: weight type %d", qt);
   return CAI_OK;
 }

@@ -146,7 +146,6 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
   {
     float inv_rms = 1.0f;
     const float4* src = reinterpret_cast<const float4*>(p.x);
-    const float4* gsrc = reinterpret_cast<const float4*>(p.norm_gain);
     const int n8 = cols >> 3, nthr = blockDim.x;
     // one thread = 8 consecutive activations (a quarter of a 32-block: the block's four threads are one DPP quad).
     // A thread's turns (n, n + nthr, ...) are requested SD at a time - a long row (the 18944-wide down projection: four

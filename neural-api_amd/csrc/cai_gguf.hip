@@ -222,7 +222,7 @@ int read_vector(const cai_gguf_s* g, const std::string& name, int64_t want, std:
   return CAI_OK;
 }
 
-bool uploadable_type(int t) { return t == CAI_F32 || t == CAI_F16 || t == CAI_Q4_0 || t == CAI_Q8_0 || t == CAI_Q4_K || t == CAI_Q6_K; }
+bool uploadable_type(int t) { return t == CAI_F32 || t == CAI_F16 || t == CAI_Q4_0 || t == CAI_Q8_0 || t == CAI_Q4_K || t == CAI_Q6_K || raw_block_type(t); }
 
 // resident weight from one 2-D tensor (or two stacked along the rows) in stored order
 int load_matrix(const cai_gguf_s* g, const std::string& name, const std::string* second, const std::string* bias_name,
@@ -236,7 +236,7 @@ int load_matrix(const cai_gguf_s* g, const std::string& name, const std::string*
   for (const TensorInfo* q : both) {
     if (!q) continue;
     if (q->n_dims != 2) return set_error(CAI_ERR_INVALID, "gguf: tensor \"%s\" has %d dimensions, expected a matrix: %s", q->name.c_str(), q->n_dims, g->path.c_str());
-    if (!uploadable_type(q->ggml_type)) return set_error(CAI_ERR_UNSUPPORTED, "gguf: tensor \"%s\" has ggml type %d; resident types are F32, F16, Q4_0, Q8_0, Q4_K, Q6_K: %s", q->name.c_str(), q->ggml_type, g->path.c_str());
+    if (!uploadable_type(q->ggml_type)) return set_error(CAI_ERR_UNSUPPORTED, "gguf: tensor \"%s\" has ggml type %d; resident types are F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K: %s", q->name.c_str(), q->ggml_type, g->path.c_str());
     if ((want_rows > 0 && q->shape[0] != want_rows) || (want_cols > 0 && q->shape[1] != want_cols))
       return set_error(CAI_ERR_INVALID, "gguf: tensor \"%s\" is [%lld, %lld], expected [%lld, %lld]: %s", q->name.c_str(), (long long)q->shape[0], (long long)q->shape[1], (long long)want_rows, (long long)want_cols, g->path.c_str());
   }

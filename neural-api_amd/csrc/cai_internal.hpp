@@ -105,6 +105,17 @@ struct cai_qw_s {
   int64_t  algo_bytes = 0;     // bytes of the GGUF form (+bias): what one GEMV must stream
 };
 
+// The block types that stay resident as the stored block stream (no repacking at upload)
+__host__ __device__ constexpr bool raw_block_type(int qt)
+{
+  return qt == CAI_Q4_1 || qt == CAI_Q5_0 || qt == CAI_Q5_1 || qt == CAI_Q2_K || qt == CAI_Q3_K || qt == CAI_Q5_K;
+}
+__host__ __device__ constexpr int raw_block_bytes(int qt)
+{
+  return qt == CAI_Q4_1 ? 20 : qt == CAI_Q5_0 ? 22 : qt == CAI_Q5_1 ? 24 : qt == CAI_Q2_K ? 84 : qt == CAI_Q3_K ? 110 : qt == CAI_Q5_K ? 176 : 0;
+}
+__host__ __device__ constexpr int raw_block_elems(int qt) { return (qt == CAI_Q2_K || qt == CAI_Q3_K || qt == CAI_Q5_K) ? 256 : 32; }
+
 // Q6_K: start of the d plane (behind 16 scale bytes per block); null for the other types
 inline const uint8_t* qw_aux2(const cai_qw_s* w) { return w->qtype == CAI_Q6_K ? w->aux + w->rows * (w->cols >> 8) * 16 : nullptr; }
 

@@ -1,5 +1,6 @@
 // Elementwise layer math, block dequantization, embedding gather, arg-max and the MoE router for gfx950.
 #include "cai_internal.hpp"
+#include "cai_blocks_raw.hpp"
 #include <string.h>
 #include <math.h>
 
@@ -64,6 +65,10 @@ __device__ float dequant_elem(int qtype, const uint8_t* data, const uint8_t* aux
       const int hi2 = (blk[128 + (e >> 7) * 32 + (e & 31)] >> (2 * ((e & 127) >> 5))) & 3;
       return dl * (float)((nib | (hi2 << 4)) - 32);
     }
+  }
+  if (raw_block_type(qtype)) {   // resident as stored
+    const int be = raw_block_elems(qtype);
+    return raw_block_elem(qtype, data + (row * (cols / be) + i / be) * raw_block_bytes(qtype), (int)(i % be));
   }
   return 0.0f;
 }

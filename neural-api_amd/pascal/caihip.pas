@@ -21,6 +21,7 @@ const
 
   // ggml tensor type ids (neural/neuralgguf.pas:86-98) + per-row int8
   CAI_F32 = 0; CAI_F16 = 1; CAI_Q4_0 = 2; CAI_Q8_0 = 8; CAI_Q4_K = 12; CAI_Q6_K = 14; CAI_I8ROW = 100;
+  CAI_Q4_1 = 3; CAI_Q5_0 = 6; CAI_Q5_1 = 7; CAI_Q2_K = 10; CAI_Q3_K = 11; CAI_Q5_K = 13;
   // fused activation opcodes = csAct* of the OpenCL kernels (neural/neural.cl:114-146)
   CAI_ACT_NONE = 0; CAI_ACT_RELU = 1; CAI_ACT_SIGMOID = 2; CAI_ACT_TANH = 3;
   CAI_X_DEVICE = 1; CAI_Y_DEVICE = 2; CAI_MATRIX_CORES = 4;

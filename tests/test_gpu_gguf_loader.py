@@ -95,9 +95,8 @@ def test_loader_refuses_what_it_cannot_run(tmp_path):
     m = dict(base); del m["llama.block_count"]; cases.append((m, tens, "llama.block_count"))
     cases.append((dict(base), tens, "missing tensor \"blk.0.attn_q.weight\""))
     m = dict(base); m["llama.rope.scaling.type"] = "yarn"; cases.append((m, tens, "rope.scaling.type"))
-    # a Q5_K embedding: listed by the container, refused by the loader
-    m = dict(base); m["llama.embedding_length"] = 256
-    cases.append((m, [("token_embd.weight", [10, 256], 13, bytes(10 * 176))], "ggml type 13"))
+    # a BF16 embedding: sized by the container, refused by the loader (the reference has no decoder for it either)
+    cases.append((dict(base), [("token_embd.weight", [10, 32], 30, bytes(10 * 64))], "ggml type 30"))
     for i, (meta, tensors, needle) in enumerate(cases):
         p = str(tmp_path / ("c%d.gguf" % i))
         write_gguf(p, meta, tensors)

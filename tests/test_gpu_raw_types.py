@@ -1,0 +1,150 @@
+"""The GGUF block types that stay resident as the stored stream (Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K) through the C ABI:
+dequantisation bit-exact (golden vectors and arbitrary bytes), the matrix-vector kernel against the oracle's
+dequantise-then-dot in double, and a decoder whose file mixes Q5_K and Q6_K the way llama.cpp's Q5_K_M preset does."""
+import numpy as np
+import pytest
+
+from helpers import oracle_lib as O
+from helpers.fixtures_io import GGUFFile, load_json, ref_path
+from helpers.model_build import oracle_model, synthetic_spec
+
+pytestmark = pytest.mark.gpu
+TIGHT = 2e-5
+TOL = 1e-3
+RAW = [O.Q5_K, O.Q2_K, O.Q3_K, O.Q4_1, O.Q5_0, O.Q5_1]
+
+
+@pytest.mark.parametrize("name,qt", [("Q5_K", O.Q5_K), ("Q2_K", O.Q2_K)])
+def test_reference_golden_bit_exact_on_device(name, qt):
+    from helpers.device import dev
+    cai = dev()
+    t, shape, raw = GGUFFile(ref_path("tiny_kquant.gguf")).raw("kq.%s.weight" % name)
+    w = cai.QWeight(qt, 4, 256, raw)
+    want = np.array(load_json("tiny_kquant_ref.json")["dequant"][name], np.float32)
+    assert np.array_equal(w.dequant_rows().reshape(-1).view(np.uint32), want.view(np.uint32))
+    w.close()
+
+
+@pytest.mark.parametrize("qt", RAW)
+def test_random_bytes_bit_exact(qt):
+    """Arbitrary block bytes: every code, packed scale and plane bit; the half fields kept finite."""
+    from helpers.device import dev
+    from test_oracle_codecs_other import random_blocks
+    cai = dev()
+    rows, cols = 37, 1024
+    be = 256 if qt in (O.Q5_K, O.Q2_K, O.Q3_K) else 32
+    raw = random_blocks(qt, rows * cols // be, seed=900 + qt).reshape(-1)
+    w = cai.QWeight(qt, rows, cols, raw)
+    got = w.dequant_rows()
+    want = O.dequant(qt, raw, rows * cols).reshape(rows, cols)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # a window of rows, as the row-streaming loader asks for
+    assert np.array_equal(w.dequant_rows(5, 9).view(np.uint32), want[5:14].view(np.uint32))
+    w.close()
+
+
+@pytest.mark.parametrize("qt", RAW)
+@pytest.mark.parametrize("rows,cols", [(2048, 2048), (3, 256), (1, 9728), (1000, 3584), (64, 18944)])
+def test_gemv_matches_oracle(qt, rows, cols):
+    from helpers.device import dev, rel_err
+    cai = dev()
+    rng = np.random.default_rng(rows * 7 + cols + qt)
+    raw = O.quantize(qt, (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32))
+    bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
+    w = cai.QWeight(qt, rows, cols, raw, bias)
+    for nb in (1, 3, 8):
+        x = rng.standard_normal((nb, cols)).astype(np.float32)
+        got = w.gemv(x)
+        want = O.gemv(qt, raw, rows, cols, x, bias, 0, 1)
+        assert got.shape == want.shape
+        assert rel_err(got, want, floor=0.02 * cols ** 0.5) < TIGHT, nb
+    w.close()
+
+
+@pytest.mark.parametrize("qt,rows,cols", [(O.Q4_1, 96, 160), (O.Q5_0, 576, 576), (O.Q5_1, 5, 32), (O.Q5_0, 192, 1536)])
+def test_gemv_widths_that_are_not_whole_super_blocks(qt, rows, cols):
+    from helpers.device import dev, rel_err
+    cai = dev()
+    rng = np.random.default_rng(cols + qt)
+    raw = O.quantize(qt, (rng.standard_normal((rows, cols)) * 0.05).astype(np.float32))
+    w = cai.QWeight(qt, rows, cols, raw)
+    for nb in (1, 2, 5):
+        x = rng.standard_normal((nb, cols)).astype(np.float32)
+        assert rel_err(w.gemv(x, act=cai.ACT_TANH if nb == 2 else 0), O.gemv(qt, raw, rows, cols, x, None, 3 if nb == 2 else 0, 1)) < TIGHT
+    w.close()
+
+
+def test_width_that_splits_a_block_is_refused():
+    from helpers.device import dev
+    cai = dev()
+    with pytest.raises(cai.CaiError):
+        cai.QWeight(O.Q5_K, 2, 384, np.zeros(2 * 264, np.uint8))
+    with pytest.raises(cai.CaiError):
+        cai.QWeight(O.Q5_0, 2, 48, np.zeros(2 * 33, np.uint8))
+
+
+def q5_k_m_spec(cfg, seed):
+    """Q5_K body; attn_v and ffn_down of every other block and the head in Q6_K (the Q5_K_M preset)."""
+    spec = synthetic_spec(cfg, O.Q5_K, head_qtype=O.Q6_K, seed=seed, std=0.05, qkv_bias=True)
+    rng = np.random.default_rng(seed + 1)
+    for l in range(0, cfg["n_layers"], 2):
+        for slot in (O.W_V, O.W_DOWN):
+            t = spec["tensors"][(l, slot)]
+            w = (rng.standard_normal((t["rows"], t["cols"])) * 0.05).astype(np.float32)
+            t.update(type=O.Q6_K, raw=O.quantize(O.Q6_K, w))
+    return spec
+
+
+def test_q5_k_m_like_decoder_logits_greedy_tokens_batch_and_prompt():
+    from helpers.device import dev, rel_err
+    cai = dev()
+    cfg = dict(n_layers=4, d_model=512, n_q_heads=8, n_kv_heads=2, head_dim=64, ffn=1024, vocab=600, max_ctx=96, eps=1e-5, rope_theta=1e4)
+    spec = q5_k_m_spec(cfg, 21)
+    om = oracle_model(spec, acc64=1)
+    dec = cai.Decoder(spec, max_batch=4)
+    rng = np.random.default_rng(8)
+    prompt = [int(t) for t in rng.integers(0, cfg["vocab"], 6)]
+    tok_o = tok_d = None
+    worst = 0.0
+    singles = []
+    for p, t in enumerate(prompt):
+        tok_o, lo = om.step(t, p); am, ld = dec.step(t, p); tok_d = int(am[0])
+        worst = max(worst, rel_err(ld[0], lo)); singles.append(ld[0].copy())
+    first = tok_d
+    seq_o, seq_d = [], []
+    for i in range(64):                          # 64 greedy tokens identical (the north-star bar)
+        p = len(prompt) + i
+        n_o, lo = om.step(tok_o, p); am, ld = dec.step(tok_d, p)
+        if tok_o == tok_d:
+            worst = max(worst, rel_err(ld[0], lo))
+        tok_o, tok_d = n_o, int(am[0])
+        seq_o.append(tok_o); seq_d.append(tok_d)
+    assert worst < TOL and seq_o == seq_d
+    dec.truncate(len(prompt))
+    assert dec.generate(first, len(prompt), 64).tolist() == seq_o        # the captured-graph path
+    # the prompt path and a batch of 4 equal the single steps
+    dec.reset(1)
+    am, lg = dec.prefill(prompt, 0, seq=1)
+    assert rel_err(lg, singles[-1]) < TOL and am == int(np.argmax(singles[-1]))
+    for b in range(4):
+        dec.reset(b)
+    for p, t in enumerate(prompt):
+        am, lg = dec.step(np.full(4, t), np.full(4, p))
+        for b in range(4):
+            assert rel_err(lg[b], singles[p]) < TOL
+    dec.close()
+
+
+@pytest.mark.parametrize("qt", [O.Q2_K, O.Q3_K, O.Q4_1, O.Q5_0, O.Q5_1])
+def test_decoder_of_each_other_type_against_the_oracle(qt):
+    from helpers.device import dev, rel_err
+    cai = dev()
+    cfg = dict(n_layers=2, d_model=256, n_q_heads=4, n_kv_heads=2, head_dim=64, ffn=512, vocab=300, max_ctx=48, eps=1e-5, rope_theta=1e4)
+    spec = synthetic_spec(cfg, qt, seed=30 + qt, std=0.05)
+    om = oracle_model(spec, acc64=1)
+    dec = cai.Decoder(spec)
+    seq = [3, 299, 17, 17, 250, 9, 1, 0, 44, 120]
+    for p, t in enumerate(seq):
+        n_o, lo = om.step(t, p); am, ld = dec.step(t, p)
+        assert rel_err(ld[0], lo) < TOL and int(am[0]) == n_o
+    dec.close()

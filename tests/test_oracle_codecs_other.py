@@ -135,3 +135,17 @@ def test_random_bytes_against_the_vectorised_restatement(qt):
 def test_row_bytes_of_every_type():
     for qt, be, bb in [(O.Q4_1, 32, 20), (O.Q5_0, 32, 22), (O.Q5_1, 32, 24), (O.Q2_K, 256, 84), (O.Q3_K, 256, 110), (O.Q5_K, 256, 176)]:
         assert O.row_bytes(qt, 4 * be) == 4 * bb and O.row_bytes(qt, be + 1) == -1
+
+
+@pytest.mark.parametrize("qt,rel", [(O.Q5_K, 0.04), (O.Q2_K, 0.4), (O.Q3_K, 0.2), (O.Q4_1, 0.08), (O.Q5_0, 0.05), (O.Q5_1, 0.04)])
+def test_test_side_packers_round_trip_through_the_oracle(qt, rel):
+    """quantize (numpy packers of tests/helpers/quant_other.py) -> oracle decode stays within a format-sized error of the
+    source: pins the packers the model-level tests build their weights with (a wrong plane or shift gives errors ~ 1)."""
+    rng = np.random.default_rng(qt)
+    x = rng.standard_normal((8, 512)).astype(np.float32)
+    raw = O.quantize(qt, x)
+    back = O.dequant(qt, raw, x.size).reshape(x.shape)
+    err = np.sqrt(np.mean((back - x) ** 2)) / np.sqrt(np.mean(x ** 2))
+    assert err < rel, err
+    assert np.array_equal(back.reshape(-1, 256 if qt in (O.Q5_K, O.Q2_K, O.Q3_K) else 32),
+                          vectorised_reference(qt, raw.reshape(-1, O.row_bytes(qt, 512) // (2 if qt in (O.Q5_K, O.Q2_K, O.Q3_K) else 16))))
