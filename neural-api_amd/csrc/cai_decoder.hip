@@ -69,7 +69,6 @@ static int check_ready(cai_decoder_s* d)
   return CAI_OK;
 }
 
-static bool is_block_quant(int qt) { return qt == CAI_Q4_K || qt == CAI_Q4_0 || qt == CAI_Q8_0; }
 
 // Expert half of a block for n_b (<= 8) activation rows x[b][d_model], in place: router -> soft-max -> top-k
 // gates -> gathered gate|up (RMSNorm and SwiGLU fused) -> gathered down -> gate-weighted mixture added to the row
@@ -87,7 +86,7 @@ static int moe_ffn_rows(cai_decoder_s* d, const cai_decoder_s::Layer& L, float* 
     MultiGemv g{}; g.n = 1; g.w[0] = L.w[CAI_W_GATEUP]; g.rows[0] = 2 * I;
     g.slot_expert = d->moe_expert + b * K; g.n_slots = K; g.expert_rows = 2 * I; g.x_slot_stride = 0;
     const float* xb = x + (int64_t)b * dm;
-    if (is_block_quant(g.w[0]->qtype)) {
+    if (gemv_fuses_swiglu(g.w[0], 1, true)) {
       g.y_slot_stride = I;
       if ((rc = launch_gemv_multi(g, xb, 1, d->mid, I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, I))) return rc;
     } else {
@@ -188,7 +187,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = 
       MultiGemv m{}; m.n = 1; m.w[0] = L.w[CAI_W_GATEUP]; m.rows[0] = 2 * I;
       if (o_hands && gemv_hands_off_ssq(m.w[0], n_b)) m.ssq_in = ssq_o;
       if (!(classes & 16u)) {
-      } else if (is_block_quant(m.w[0]->qtype)) {
+      } else if (gemv_fuses_swiglu(m.w[0], n_b, false)) {
         if ((rc = launch_gemv_multi(m, d->x, n_b, d->mid, I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, I))) return rc;
       } else {
         if ((rc = launch_gemv_multi(m, d->x, n_b, d->gu, 2 * I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;

@@ -580,7 +580,13 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
 // True when a batch-1 launch on this matrix goes through the streaming kernel (which honours ssq_in / ssq_out).
 bool gemv_hands_off_ssq(const cai_qw_s* w, int n_b)
 {
-  return w->qtype == CAI_Q4_K && n_b == 1 && (((w->cols >> 8) + 15) >> 4) <= 8;
+  return (w->qtype == CAI_Q4_K || w->qtype == CAI_Q5_K) && n_b == 1 && w->cols % 256 == 0 && (((w->cols >> 8) + 15) >> 4) <= 8;
+}
+// True when launch_gemv_multi takes this matrix with the SwiGLU epilogue (swiglu_half != 0) at this batch width.
+bool gemv_fuses_swiglu(const cai_qw_s* w, int n_b, bool expert_bank)
+{
+  if (w->qtype == CAI_Q4_K || w->qtype == CAI_Q4_0 || w->qtype == CAI_Q8_0) return true;
+  return w->qtype == CAI_Q5_K && n_b == 1 && !expert_bank && gemv_hands_off_ssq(w, 1);   // (integer-dot kernel only)
 }
 static bool fast_type(int qt) { return qt == CAI_Q4_K || qt == CAI_Q4_0 || qt == CAI_Q8_0; }
 
@@ -693,7 +699,7 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
     p.seg[i].y_off = m.y_off[i];
   }
   const int qt = w0->qtype;
-  if ((qt == CAI_Q4_K || (qt == CAI_Q4_0 && p.cols % 256 == 0) || (qt == CAI_Q6_K && m.n == 1 && !swiglu_half)) && n_b == 1 && !m.slot_expert) {
+  if ((qt == CAI_Q4_K || qt == CAI_Q5_K || (qt == CAI_Q4_0 && p.cols % 256 == 0) || (qt == CAI_Q6_K && m.n == 1 && !swiglu_half)) && n_b == 1 && !m.slot_expert) {
     MultiGemv mm = m;
     if (swiglu_half) { if (m.n != 1) return set_error(CAI_ERR_INVALID, "gemv: swiglu takes one matrix"); p.seg[0].rows = swiglu_half; }
     p.ssq_in = m.ssq_in; p.ssq_out = m.ssq_out;

@@ -1,5 +1,6 @@
 // Persistent streaming matrix-vector kernel for batch-1 decode on gfx950, integer-dot form: Q4_K, and with other requests and
-// block arithmetic in the same walk Q4_0 (quants and scales planes) and Q6_K (ql|qh records + planes of scales and d).
+// block arithmetic in the same walk Q5_K (stored super-blocks), Q4_0 (quants and scales planes) and Q6_K (ql|qh records +
+// planes of scales and d).
 //
 // The weights of a Q4_K sub-block are 4-bit integers with one float scale, so dot(W[a], X) splits into an exact
 // integer part and a handful of float operations per 32 weights once X is held as integers too.  Each
@@ -26,6 +27,8 @@ namespace cai {
 namespace {
 
 struct Q4kRegs { uint4 h, q0, q1; };
+struct Q5kRegs { uint4 h, q0, q1, e0, e1; };   // Q5_K: + the 32 bytes of the fifth-bit plane (neural/neuralgguf.pas:516-587)
+template <int QT> constexpr int dot_rec_bytes() { return QT == CAI_Q6_K ? 192 : QT == CAI_Q4_0 ? 128 : QT == CAI_Q5_K ? 176 : 144; }
 
 // LDS slot (in uint4) of the t-th uint4 (t = 0..15) of unit u (64 activations): tiles of 16 units, transposed
 __device__ __forceinline__ int xq_slot(int u, int t) { return (u >> 4) * 256 + t * 16 + (u & 15); }
@@ -87,13 +90,13 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: group indices, segment lookups and loop bounds stay scalar
   const int step = wave % nsw, gslot = wave / nsw;
   const int cols = p.cols, nsb = cols >> 8;
-  const int64_t row_bytes = (int64_t)nsb * (QT == CAI_Q6_K ? 192 : QT == CAI_Q4_0 ? 128 : 144);
+  const int64_t row_bytes = (int64_t)nsb * dot_rec_bytes<QT>();
   const int sb = step * 16 + (lane >> 2), cc = lane & 3;
   const bool act = sb < nsb;
   const int g_first = blockIdx.x * gwv + gslot, g_stride = gridDim.x * gwv;
   const int n_iters = (n_groups + g_stride - 1) / g_stride;
-  const int64_t lane_off = (int64_t)(act ? sb : 0) * (QT == CAI_Q6_K ? 192 : QT == CAI_Q4_0 ? 128 : 144);
-  using WRegs = typename std::conditional<QT == CAI_Q6_K, Q6kRegs, Q4kRegs>::type;
+  const int64_t lane_off = (int64_t)(act ? sb : 0) * dot_rec_bytes<QT>();
+  using WRegs = typename std::conditional<QT == CAI_Q6_K, Q6kRegs, typename std::conditional<QT == CAI_Q5_K, Q5kRegs, Q4kRegs>::type>::type;
 
   // group -> segment, first row of the group inside the segment
   auto locate = [&](int g, const GemvSeg*& sg, int& row0) {
@@ -129,6 +132,12 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
         rg[r].q0 = *reinterpret_cast<const uint4*>(blk + 32 * cc);
         rg[r].q1 = *reinterpret_cast<const uint4*>(blk + 32 * cc + 16);
         rg[r].h.x = *reinterpret_cast<const uint32_t*>(sg->aux + ((int64_t)row * nsb + (act ? sb : 0)) * 16 + 4 * cc);
+      } else if constexpr (QT == CAI_Q5_K) {
+        // header as Q4_K; the lane's 32 nibble bytes sit behind the 32-byte bit plane, which all four lanes of the super-block read
+        rg[r].h = *reinterpret_cast<const uint4*>(blk);
+        rg[r].e0 = *reinterpret_cast<const uint4*>(blk + 16); rg[r].e1 = *reinterpret_cast<const uint4*>(blk + 32);
+        rg[r].q0 = *reinterpret_cast<const uint4*>(blk + 48 + 32 * cc);
+        rg[r].q1 = *reinterpret_cast<const uint4*>(blk + 64 + 32 * cc);
       } else {
         rg[r].h = *reinterpret_cast<const uint4*>(blk);
         rg[r].q0 = *reinterpret_cast<const uint4*>(blk + 16 + 32 * cc);
@@ -339,6 +348,30 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
           const float dB = __half2float(__ushort_as_half((unsigned short)(cur[r].h.x >> 16)));
           acc[r] = dA * fmaf(sA, fa, -8.0f * mA) + dB * fmaf(sB, fb, -8.0f * mB);
           continue;
+        } else if constexpr (QT == CAI_Q5_K) {
+          // code = nibble | bit << 4 (0..31): bit 2 cc of plane byte i belongs to weight i of the first 32, bit 2 cc + 1 to the second
+          const uint32_t qw[8] = {cur[r].q0.x, cur[r].q0.y, cur[r].q0.z, cur[r].q0.w, cur[r].q1.x, cur[r].q1.y, cur[r].q1.z, cur[r].q1.w};
+          const uint32_t qe[8] = {cur[r].e0.x, cur[r].e0.y, cur[r].e0.z, cur[r].e0.w, cur[r].e1.x, cur[r].e1.y, cur[r].e1.z, cur[r].e1.w};
+          int ia[NL], ib[NL];
+#pragma unroll
+          for (int L = 0; L < NL; L++) { ia[L] = 0; ib[L] = 0; }
+#pragma unroll
+          for (int w = 0; w < 8; w++) {
+            const uint32_t ew = qe[w] >> (2 * cc);
+            const int a = (int)((qw[w] & 0x0f0f0f0fu) | ((ew << 4) & 0x10101010u)), b = (int)(((qw[w] >> 4) & 0x0f0f0f0fu) | ((ew << 3) & 0x10101010u));
+#pragma unroll
+            for (int L = 0; L < NL; L++) {
+              ia[L] = __builtin_amdgcn_sdot4(a, xq[L][w], ia[L], false);
+              ib[L] = __builtin_amdgcn_sdot4(b, xq[L][8 + w], ib[L], false);
+            }
+          }
+          // (32 * 31 * 2^22 exceeds 32 bits: the digits are combined in float)
+          const float fa = (float)ia[0] + 256.0f * (float)ia[1] + 65536.0f * (float)ia[2], fb = (float)ib[0] + 256.0f * (float)ib[1] + 65536.0f * (float)ib[2];
+          uint32_t sc, mn; q4k_scale_pair(cur[r].h.y, cur[r].h.z, cur[r].h.w, cc, sc, mn);
+          const float d = __half2float(__ushort_as_half((unsigned short)(cur[r].h.x & 0xffffu)));
+          const float dmin = __half2float(__ushort_as_half((unsigned short)(cur[r].h.x >> 16)));
+          acc[r] = d * (cvt_ub0(sc) * (sA * fa) + cvt_ub1(sc) * (sB * fb)) - dmin * (cvt_ub0(mn) * mA + cvt_ub1(mn) * mB);
+          continue;
         } else {
         const uint32_t qw[8] = {cur[r].q0.x, cur[r].q0.y, cur[r].q0.z, cur[r].q0.w, cur[r].q1.x, cur[r].q1.y, cur[r].q1.z, cur[r].q1.w};
         int ia[NL], ib[NL];
@@ -468,6 +501,12 @@ __global__ __launch_bounds__(768, 3) void gemv_q40_dot(const GemvParams p, const
   gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q4_0>(p, n_groups, nsw, gwv);
 }
 
+template <int R, int MODE, bool MULTISEG, int NS>
+__global__ __launch_bounds__(768, 3) void gemv_q5k_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
+{
+  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q5_K>(p, n_groups, nsw, gwv);
+}
+
 template <int R, int NS>
 __global__ __launch_bounds__(768, 3) void gemv_q6k_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
 {
@@ -532,6 +571,11 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
       if (swiglu_half) go(gemv_q40_dot<1, 1, false, NSV>);
       else if (m.n > 1) { if (R == 2) go(gemv_q40_dot<2, 0, true, NSV>); else go(gemv_q40_dot<1, 0, true, NSV>); }
       else { if (R == 2) go(gemv_q40_dot<2, 0, false, NSV>); else go(gemv_q40_dot<1, 0, false, NSV>); }
+    }
+    else if (m.w[0]->qtype == CAI_Q5_K) {
+      if (swiglu_half) go(gemv_q5k_dot<1, 1, false, NSV>);
+      else if (m.n > 1) { if (R == 2) go(gemv_q5k_dot<2, 0, true, NSV>); else go(gemv_q5k_dot<1, 0, true, NSV>); }
+      else { if (R == 2) go(gemv_q5k_dot<2, 0, false, NSV>); else go(gemv_q5k_dot<1, 0, false, NSV>); }
     }
     else if (swiglu_half) go(gemv_q4k_dot<1, 1, false, NSV>);
     else if (m.n > 1) { if (R == 2) go(gemv_q4k_dot<2, 0, true, NSV>); else go(gemv_q4k_dot<1, 0, true, NSV>); }

@@ -168,6 +168,7 @@ struct MultiGemv {
 int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int64_t y_stride, int act,
                       const float* residual, const float* norm_gain, float norm_eps, int swiglu_half);
 bool gemv_hands_off_ssq(const cai_qw_s* w, int n_b);
+bool gemv_fuses_swiglu(const cai_qw_s* w, int n_b, bool expert_bank);
 int launch_dequant_rows(const cai_qw_s* w, int64_t row0, int64_t n_rows, float* out);
 int launch_rmsnorm(const float* x, const float* gain, int n, int n_tokens, float eps, float* y);
 int launch_rope(float* x, int n_heads, int head_dim, const int32_t* pos_dev, int pos_host, const float* theta, int n_tokens, int64_t token_stride);

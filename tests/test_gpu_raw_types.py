@@ -148,3 +148,41 @@ def test_decoder_of_each_other_type_against_the_oracle(qt):
         n_o, lo = om.step(t, p); am, ld = dec.step(t, p)
         assert rel_err(ld[0], lo) < TOL and int(am[0]) == n_o
     dec.close()
+
+
+def test_q5_k_largest_codes_on_equal_activations_do_not_overflow_the_integer_sums():
+    """Every code 31, every scale 63, all activations equal: the integer sum of a 32-block is 32 * 31 * (2^22 - 1), past
+    32 bits, which is why the batch-1 kernel combines its three digit sums in float."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    rows, cols = 64, 2048
+    blk = np.full(176, 0xff, np.uint8)
+    blk[0:2] = np.array([np.float16(0.01)]).view(np.uint8); blk[2:4] = np.array([np.float16(0.0)]).view(np.uint8)
+    raw = np.tile(blk, rows * cols // 256)
+    w = cai.QWeight(O.Q5_K, rows, cols, raw)
+    for x in (np.ones((1, cols), np.float32), -np.ones((1, cols), np.float32), np.full((1, cols), 3.7e3, np.float32)):
+        assert rel_err(w.gemv(x), O.gemv(O.Q5_K, raw, rows, cols, x, None, 0, 1)) < TIGHT
+    w.close()
+
+
+@pytest.mark.parametrize("rows,cols", [(2048, 512), (37888, 3584), (1024, 5120)])
+def test_q5_k_fused_feed_forward_front_half(rows, cols):
+    """cai_ffn_gateup (RMSNorm -> gate|up -> SwiGLU in one launch) on Q5_K at batch 1, with and without the gain."""
+    import ctypes as C
+    from helpers.device import dev, rel_err
+    cai = dev()
+    rng = np.random.default_rng(rows + cols)
+    raw = O.quantize(O.Q5_K, (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32))
+    w = cai.QWeight(O.Q5_K, rows, cols, raw)
+    x = (rng.standard_normal((1, cols)) * 1.7).astype(np.float32)
+    gain = (1.0 + 0.2 * rng.standard_normal(cols)).astype(np.float32)
+    L = O.lib()
+    for g in (gain, None):
+        h = x[0].copy()
+        if g is not None:
+            L.orc_rmsnorm(C.c_void_p(x[0].ctypes.data), C.c_void_p(g.ctypes.data), cols, C.c_float(1e-6), C.c_void_p(h.ctypes.data))
+        ug = O.gemv(O.Q5_K, raw, rows, cols, h, None, 0, 1)[0]
+        want = np.empty(rows // 2, np.float32)
+        L.orc_swiglu(C.c_void_p(ug.ctypes.data), rows // 2, C.c_void_p(want.ctypes.data))
+        assert rel_err(w.ffn_gateup(x, g, 1e-6)[0], want) < TIGHT
+    w.close()
