@@ -272,6 +272,17 @@ int cai_decoder_cache_rows(cai_decoder_t d, int seq, int layer, int* rows_out);
 /* EnableInt8KVCache / DisableInt8KVCache (neural/neuraldecode.pas:1277-1290): switches the cache element type; like the
  * reference only on an empty session (CAI_ERR_STATE once a token has been streamed). */
 int cai_decoder_set_kv_dtype(cai_decoder_t d, int kv_dtype);
+/* Long-context rules of TNNetRotaryEmbedding as the importers set them from "rope_scaling" (neural/neuralpretrained.pas:633-668,
+ * 13365, 13425): CAI_ROPE_LINEAR = Position Interpolation (theta_k / factor), CAI_ROPE_LLAMA3 = the Llama-3.1 rule
+ * (original_ctx, low_freq_factor, high_freq_factor; no output scale).  Both only change the frequency table, which is rebuilt
+ * in double on the host.  Only on an empty session (CAI_ERR_STATE otherwise: cached keys carry the old rotation). */
+#define CAI_ROPE_NONE   0
+#define CAI_ROPE_LINEAR 1
+#define CAI_ROPE_LLAMA3 2
+int cai_decoder_set_rope_scaling(cai_decoder_t d, int mode, float factor, int original_ctx, float low_freq_factor, float high_freq_factor);
+/* Per-frequency divisors: theta_k = base^(-2k/head_dim) / factors[k], n = head_dim / 2 (the "rope_freqs.weight" tensor llama.cpp
+ * writes for Llama-3.1 exports; the LongFactors table of the reference's record, neural/neuralpretrained.pas:652-655). */
+int cai_decoder_set_rope_freq_factors(cai_decoder_t d, const float* factors, int n);
 int cai_decoder_snapshot(cai_decoder_t d, int seq, cai_kv_snap_t* out);
 int cai_decoder_restore(cai_decoder_t d, int seq, cai_kv_snap_t snap);
 /* Bytes of weights, biases and gains one decoded token streams (for roofline accounting). */

@@ -1157,6 +1157,7 @@ void kv_free(cai_kv_s* kv)
 int kv_snapshot(cai_kv_s* kv, int seq, cai_kv_snap_s** out)
 {
   cai_kv_snap_s* s = new cai_kv_snap_s();
+  auto drop = [&](int code) { cai_kv_snap_destroy(s); return code; };   // every error path releases what the snapshot holds so far
   s->n_layers = kv->n_layers; s->kv_heads = kv->kv_heads; s->head_dim = kv->head_dim; s->dtype = kv->dtype;
   s->evict_sinks = kv->evict_sinks; s->evict_cap = kv->evict_cap;
   s->len.resize(kv->n_layers);
@@ -1165,29 +1166,28 @@ int kv_snapshot(cai_kv_s* kv, int seq, cai_kv_snap_s** out)
   s->rows = rows;
   if (rows > 0) {
     const size_t bytes = (size_t)kv->n_layers * kv->kv_heads * rows * kv->head_dim * kv->elem();
-    if (hipMalloc(&s->k, bytes) != hipSuccess || hipMalloc(&s->v, bytes) != hipSuccess) {
-      if (s->k) (void)hipFree(s->k);
-      delete s; return set_error(CAI_ERR_NOMEM, "kv snapshot: out of device memory (%zu bytes)", 2 * bytes);
-    }
+    if (hipMalloc(&s->k, bytes) != hipSuccess || hipMalloc(&s->v, bytes) != hipSuccess)
+      return (void)hipGetLastError(), drop(set_error(CAI_ERR_NOMEM, "kv snapshot: out of device memory (%zu bytes)", 2 * bytes));
     const size_t row_b = (size_t)kv->head_dim * kv->elem();
     for (int which = 0; which < 2; which++) {
       const char* src = (const char*)(which ? kv->v : kv->k) + (size_t)seq * kv->seq_elems() * kv->elem();
       char* dst = (char*)(which ? s->v : s->k);
       // [layer*kv_heads] planes of max_ctx rows -> planes of `rows` rows
-      CAI_HIP(hipMemcpy2DAsync(dst, (size_t)rows * row_b, src, (size_t)kv->max_ctx * row_b, (size_t)rows * row_b,
-                               (size_t)kv->n_layers * kv->kv_heads, hipMemcpyDeviceToDevice, ctx().stream));
+      const hipError_t e = hipMemcpy2DAsync(dst, (size_t)rows * row_b, src, (size_t)kv->max_ctx * row_b, (size_t)rows * row_b,
+                                            (size_t)kv->n_layers * kv->kv_heads, hipMemcpyDeviceToDevice, ctx().stream);
+      if (e != hipSuccess) return drop(hip_fail(e, "kv snapshot copy", __FILE__, __LINE__));
     }
     if (kv->dtype == CAI_KV_I8) {     // the row scales travel with the codes
       const size_t sb = (size_t)kv->n_layers * kv->kv_heads * rows * sizeof(float);
-      if (hipMalloc(&s->ks, sb) != hipSuccess || hipMalloc(&s->vs, sb) != hipSuccess) {
-        (void)hipFree(s->k); (void)hipFree(s->v); if (s->ks) (void)hipFree(s->ks);
-        delete s; return set_error(CAI_ERR_NOMEM, "kv snapshot: out of device memory (%zu bytes)", 2 * sb);
+      if (hipMalloc(&s->ks, sb) != hipSuccess || hipMalloc(&s->vs, sb) != hipSuccess)
+        return (void)hipGetLastError(), drop(set_error(CAI_ERR_NOMEM, "kv snapshot: out of device memory (%zu bytes)", 2 * sb));
+      for (int which = 0; which < 2; which++) {
+        const hipError_t e = hipMemcpy2DAsync(which ? s->vs : s->ks, (size_t)rows * 4, (which ? kv->vs : kv->ks) + (size_t)seq * kv->seq_rows(), (size_t)kv->max_ctx * 4,
+                                              (size_t)rows * 4, (size_t)kv->n_layers * kv->kv_heads, hipMemcpyDeviceToDevice, ctx().stream);
+        if (e != hipSuccess) return drop(hip_fail(e, "kv snapshot copy", __FILE__, __LINE__));
       }
-      for (int which = 0; which < 2; which++)
-        CAI_HIP(hipMemcpy2DAsync(which ? s->vs : s->ks, (size_t)rows * 4, (which ? kv->vs : kv->ks) + (size_t)seq * kv->seq_rows(), (size_t)kv->max_ctx * 4,
-                                 (size_t)rows * 4, (size_t)kv->n_layers * kv->kv_heads, hipMemcpyDeviceToDevice, ctx().stream));
     }
-    CAI_HIP(hipStreamSynchronize(ctx().stream));
+    { const hipError_t e = hipStreamSynchronize(ctx().stream); if (e != hipSuccess) return drop(hip_fail(e, "kv snapshot sync", __FILE__, __LINE__)); }
   }
   *out = s;
   return CAI_OK;

@@ -34,6 +34,7 @@ struct cai_decoder_s {
   bool use_graph = true;
   int ws_generation = -1;         // activation-workspace generation the captured batch graphs were built against
   std::vector<cai_qw_s*> owned;   // weights created by a loader on the decoder's behalf, destroyed with it
+  bool cache_lost = false;        // a change of cache type ran out of memory twice: the session has no K,V storage
   int qw() const { return cfg.n_q_heads * cfg.head_dim; }
   int kw() const { return cfg.n_kv_heads * cfg.head_dim; }
 };
@@ -56,6 +57,7 @@ static void invalidate_graphs(cai_decoder_s* d)
 static int check_ready(cai_decoder_s* d)
 {
   const cai_decoder_config& c = d->cfg;
+  if (d->cache_lost) return set_error(CAI_ERR_STATE, "decoder: the K,V cache was lost when cai_decoder_set_kv_dtype ran out of device memory; destroy the session");
   if (!d->embed) return set_error(CAI_ERR_STATE, "decoder: embedding weight not set");
   if (!d->final_norm) return set_error(CAI_ERR_STATE, "decoder: final norm gain not set");
   for (int l = 0; l < c.n_layers; l++) {
@@ -642,12 +644,53 @@ extern "C" int cai_decoder_set_kv_dtype(cai_decoder_t d, int kv_dtype)
   invalidate_graphs(d);
   const cai_decoder_config& c = d->cfg;
   const int sinks = d->kv.evict_sinks, cap = d->kv.evict_cap;
+  const int old = d->kv.dtype;
   kv_free(&d->kv);
-  const int rc = kv_alloc(&d->kv, c.max_batch, c.n_layers, c.n_kv_heads, c.head_dim, c.max_ctx, kv_dtype);
-  if (rc) return rc;
+  int rc = kv_alloc(&d->kv, c.max_batch, c.n_layers, c.n_kv_heads, c.head_dim, c.max_ctx, kv_dtype);
+  if (rc) {
+    // back to the type that fitted before; if even that fails the session has no cache and every later call says so
+    kv_free(&d->kv);
+    if (kv_alloc(&d->kv, c.max_batch, c.n_layers, c.n_kv_heads, c.head_dim, c.max_ctx, old)) { kv_free(&d->kv); d->cache_lost = true; }
+    else { d->kv.evict_sinks = sinks; d->kv.evict_cap = cap; }
+    return rc;
+  }
   d->kv.evict_sinks = sinks; d->kv.evict_cap = cap;
   d->cfg.kv_dtype = kv_dtype;
   return CAI_OK;
+}
+
+// Long-context frequency rules of TNNetRotaryEmbedding as the importers configure them (neural/neuralpretrained.pas:633-668):
+// the table is rebuilt on the host in double; captured graphs read it through the same pointer and stay valid.
+static int set_thetas(cai_decoder_s* d, const std::vector<float>& th, const char* who)
+{
+  for (int n : d->kv.len)
+    if (n > 0) return set_error(CAI_ERR_STATE, "%s: the cache holds %d tokens rotated with the old frequencies; set the rule on an empty session", who, n);
+  CAI_HIP(hipMemcpyAsync(d->theta, th.data(), th.size() * 4, hipMemcpyHostToDevice, ctx().stream));
+  CAI_HIP(hipStreamSynchronize(ctx().stream));   // th is the caller's stack
+  return CAI_OK;
+}
+
+extern "C" int cai_decoder_set_rope_scaling(cai_decoder_t d, int mode, float factor, int original_ctx, float low_freq_factor, float high_freq_factor)
+{
+  CAI_READY();
+  CAI_REQUIRE(d, "cai_decoder_set_rope_scaling: null decoder");
+  std::vector<float> th;
+  const int rc = rope_thetas_scaled(d->cfg.rope_theta, d->cfg.head_dim, mode, factor, original_ctx, low_freq_factor, high_freq_factor, th);
+  if (rc) return rc;
+  return set_thetas(d, th, "cai_decoder_set_rope_scaling");
+}
+
+extern "C" int cai_decoder_set_rope_freq_factors(cai_decoder_t d, const float* factors, int n)
+{
+  CAI_READY();
+  CAI_REQUIRE(d && factors, "cai_decoder_set_rope_freq_factors: null argument");
+  CAI_REQUIRE(n == d->cfg.head_dim / 2, "cai_decoder_set_rope_freq_factors: %d factors for %d rotary pairs", n, d->cfg.head_dim / 2);
+  std::vector<float> th(n);
+  for (int k = 0; k < n; k++) {
+    CAI_REQUIRE(factors[k] > 0.0f && factors[k] < 3.0e38f, "cai_decoder_set_rope_freq_factors: factor %d is %g", k, (double)factors[k]);
+    th[k] = (float)(pow((double)d->cfg.rope_theta, -2.0 * k / d->cfg.head_dim) / (double)factors[k]);
+  }
+  return set_thetas(d, th, "cai_decoder_set_rope_freq_factors");
 }
 
 extern "C" int cai_decoder_cache_rows(cai_decoder_t d, int seq, int layer, int* rows_out)

@@ -77,6 +77,8 @@ struct cai_gguf_s {
   std::map<std::string, size_t> meta_index;
   std::vector<TensorInfo> tensors;
   std::map<std::string, size_t> tensor_index;
+  // cai_gguf_meta_array_str: the string array last read, the index after the entry last returned and its byte position
+  const MetaValue* walk_arr = nullptr; int64_t walk_next = 0; size_t walk_pos = 0;
 };
 
 namespace {
@@ -340,9 +342,14 @@ extern "C" int cai_gguf_meta_array_str(cai_gguf_t g, const char* key, int64_t in
   const MetaValue* v = find_meta(g, key);
   if (!v || v->type != GT_ARR || v->elem_type != GT_STR) return set_error(CAI_ERR_INVALID, "gguf: metadata key \"%s\" is missing or not a string array: %s", key, g->path.c_str());
   if (index < 0 || (uint64_t)index >= v->count) return set_error(CAI_ERR_INVALID, "gguf: index %lld outside the %llu entries of \"%s\": %s", (long long)index, (unsigned long long)v->count, key, g->path.c_str());
+  // entries have no fixed size: remember where the last read ended so that walking a vocabulary in order costs one entry per
+  // call instead of a scan from the start (GetMetaArrayString memoises likewise, neural/neuralgguf.pas)
   Cursor c{g->base, g->size}; c.p = v->arr_pos;
+  int64_t k = 0;
+  if (g->walk_arr == v && g->walk_next <= index) { c.p = g->walk_pos; k = g->walk_next; }
   std::string s;
-  for (int64_t k = 0; k <= index; k++) s = c.str();   // entries were validated when the file was opened
+  for (; k <= index; k++) s = c.str();   // entries were validated when the file was opened
+  g->walk_arr = v; g->walk_next = index + 1; g->walk_pos = c.p;
   snprintf(buf, (size_t)n, "%s", s.c_str());
   return CAI_OK;
 }
@@ -392,7 +399,8 @@ extern "C" int cai_gguf_load_qw(cai_gguf_t g, const char* name, const char* bias
 // ------------------------------------------------------------------------------------------
 extern "C" int cai_decoder_load_gguf(const char* path, int max_ctx, int max_batch, int kv_dtype, cai_decoder_t* out)
 {
-  CAI_READY();
+  // (the file's metadata is judged before the device is asked for: a file this path cannot run is refused with the same
+  // message on a host without a GPU)
   CAI_REQUIRE(path && out, "cai_decoder_load_gguf: null argument");
   *out = nullptr;
   cai_gguf_t g = nullptr;
@@ -423,13 +431,37 @@ extern "C" int cai_decoder_load_gguf(const char* path, int max_ctx, int max_batc
     if (dm % hq) return fail(set_error(CAI_ERR_INVALID, "gguf decoder: %s=%lld is not divisible by %s=%lld", key("embedding_length").c_str(), (long long)dm, key("attention.head_count").c_str(), (long long)hq));
     hd = dm / hq;
   }
+  // rope.scaling.type "linear" -> Position Interpolation with rope.scaling.factor; absent / "none" = unscaled; anything else
+  // is refused (neural/neuralpretrained.pas:17539-17557)
+  double rope_linear = 1.0;
   {
     const MetaValue* st = find_meta(g, key("rope.scaling.type").c_str());
     if (st && st->type == GT_STR && st->s != "none") {
       const double f = opt_float("rope.scaling.factor", 1.0);
-      if (!(st->s == "linear" && f == 1.0))
-        return fail(set_error(CAI_ERR_UNSUPPORTED, "gguf decoder: %s \"%s\" (factor %g) is not supported: %s", key("rope.scaling.type").c_str(), st->s.c_str(), f, path));
+      if (st->s != "linear")
+        return fail(set_error(CAI_ERR_UNSUPPORTED, "gguf decoder: %s \"%s\" (factor %g) is not supported (supported: none, linear): %s", key("rope.scaling.type").c_str(), st->s.c_str(), f, path));
+      if (f < 1.0) return fail(set_error(CAI_ERR_INVALID, "gguf decoder: %s must be >= 1, got %g: %s", key("rope.scaling.factor").c_str(), f, path));
+      rope_linear = f;
     }
+  }
+  // per-frequency divisors (llama.cpp's form of the Llama-3.1 rule): one F32 value per rotary pair
+  std::vector<float> rope_factors;
+  if (const TensorInfo* rf = find_tensor(g, "rope_freqs.weight")) {
+    if (rf->ggml_type != CAI_F32 || rf->n_dims != 1 || rf->shape[0] != hd / 2)
+      return fail(set_error(CAI_ERR_INVALID, "gguf decoder: rope_freqs.weight must be %lld F32 values (one per rotary pair): %s", (long long)(hd / 2), path));
+    if (rope_linear != 1.0) return fail(set_error(CAI_ERR_UNSUPPORTED, "gguf decoder: rope_freqs.weight together with linear scaling: %s", path));
+    if ((rc = read_vector(g, "rope_freqs.weight", hd / 2, rope_factors))) return fail(rc);
+  }
+  if (arch == "qwen2") {
+    // the reference refuses sliding-window Qwen2 files rather than run them with full attention (neural/neuralpretrained.pas:17755-17760)
+    const MetaValue* sw = find_meta(g, key("attention.sliding_window").c_str());
+    if (sw && ((sw->type == GT_BOOL && sw->i) || (is_scalar_number(sw) && sw->i > 0)))
+      return fail(set_error(CAI_ERR_UNSUPPORTED, "gguf decoder: %s is set; Qwen2 sliding-window attention is not wired into this loader: %s", key("attention.sliding_window").c_str(), path));
+    for (int l = 0; l < (int)n_layers; l++)
+      for (const char* b : {"attn_q.bias", "attn_k.bias", "attn_v.bias"}) {
+        const std::string nm = "blk." + std::to_string(l) + "." + b;
+        if (!find_tensor(g, nm)) return fail(set_error(CAI_ERR_INVALID, "gguf: missing tensor \"%s\" (qwen2 projections carry biases) in %s", nm.c_str(), path));
+      }
   }
   int64_t vocab = opt_int("vocab_size", 0);
   if (vocab <= 0) {
@@ -442,9 +474,13 @@ extern "C" int cai_decoder_load_gguf(const char* path, int max_ctx, int max_batc
   cai_decoder_config cfg{};
   cfg.n_layers = (int)n_layers; cfg.d_model = (int)dm; cfg.n_q_heads = (int)hq; cfg.n_kv_heads = (int)hkv; cfg.head_dim = (int)hd;
   cfg.ffn = (int)ffn; cfg.vocab = (int)vocab; cfg.max_ctx = max_ctx > 0 ? max_ctx : (int)ctx_len;
-  cfg.eps = (float)opt_float("attention.layer_norm_rms_epsilon", 1e-5); cfg.rope_theta = (float)opt_float("rope.freq_base", 10000.0);
+  // default epsilon: 1e-5 on the llama branch, 1e-6 on the qwen2 branch (neural/neuralpretrained.pas:17533, 17715)
+  cfg.eps = (float)opt_float("attention.layer_norm_rms_epsilon", arch == "qwen2" ? 1e-6 : 1e-5); cfg.rope_theta = (float)opt_float("rope.freq_base", 10000.0);
   cfg.kv_dtype = kv_dtype; cfg.max_batch = max_batch > 0 ? max_batch : 1;
+  { Context& cx = ctx(); if (!cx.ready) return fail(set_error(CAI_ERR_STATE, "cai_init has not been called")); }
   if ((rc = cai_decoder_create(&cfg, &d))) return fail(rc);
+  if (rope_linear != 1.0 && (rc = cai_decoder_set_rope_scaling(d, CAI_ROPE_LINEAR, (float)rope_linear, 0, 0.0f, 0.0f))) return fail(rc);
+  if (!rope_factors.empty() && (rc = cai_decoder_set_rope_freq_factors(d, rope_factors.data(), (int)rope_factors.size()))) return fail(rc);
 
   auto put_w = [&](int layer, int slot, const std::string& name, const std::string* second, const std::string* bias, int64_t rows, int64_t cols) {
     cai_qw_t w = nullptr;

@@ -22,6 +22,7 @@ struct Context {
   // scratch used by calls that take host pointers (grown on demand)
   void*  stage_in = nullptr;  size_t stage_in_cap = 0;
   void*  stage_out = nullptr; size_t stage_out_cap = 0;
+  void*  stage_sample = nullptr; size_t stage_sample_cap = 0;   // a host logits row on its way to cai_sample_candidates
   int32_t* d_small = nullptr;            // 1024 ints of device scratch for small arguments/results
   int32_t* h_small = nullptr;            // 1024 ints of pinned host memory paired with d_small
 };
@@ -220,6 +221,7 @@ int prefill_gemm(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride, const
 int prefill_gemm_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, float* y, int64_t y_stride);
 
 void rope_thetas(float base, int head_dim, std::vector<float>& out);
+int  rope_thetas_scaled(float base, int head_dim, int mode, float factor, int original_ctx, float low_freq_factor, float high_freq_factor, std::vector<float>& out);
 
 // softmax -> history penalty -> temperature -> the m most probable tokens (descending) of a device-resident logits row;
 // history and results are host arrays

@@ -222,6 +222,36 @@ void rope_thetas(float base, int head_dim, std::vector<float>& out)
   for (int k = 0; k < head_dim / 2; k++) out[k] = (float)pow((double)base, -2.0 * k / head_dim);
 }
 
+// The table under a long-context rule (neural/neuralpretrained.pas:633-668, rope_scaling): every rule here only changes the
+// frequencies, so the kernels are the unscaled ones.  In double, rounded once.
+//   linear (Position Interpolation): theta_k / factor
+//   llama3: with r = original_ctx * theta_k / (2 pi) rotations over the training context: r > high_freq_factor keeps theta_k,
+//           r < low_freq_factor takes theta_k / factor, between them the two are blended linearly in r (no output scale)
+int rope_thetas_scaled(float base, int head_dim, int mode, float factor, int original_ctx, float low_freq_factor, float high_freq_factor, std::vector<float>& out)
+{
+  if (mode == CAI_ROPE_NONE) { rope_thetas(base, head_dim, out); return CAI_OK; }
+  if (mode != CAI_ROPE_LINEAR && mode != CAI_ROPE_LLAMA3) return set_error(CAI_ERR_UNSUPPORTED, "rope scaling: mode %d (0 none, 1 linear, 2 llama3)", mode);
+  if (!(factor >= 1.0f)) return set_error(CAI_ERR_INVALID, "rope scaling: factor must be >= 1, got %g", (double)factor);
+  if (mode == CAI_ROPE_LLAMA3 && (original_ctx <= 0 || !(high_freq_factor > low_freq_factor) || !(low_freq_factor > 0.0f)))
+    return set_error(CAI_ERR_INVALID, "rope scaling: llama3 needs original_ctx > 0 and high_freq_factor > low_freq_factor > 0 (got %d, %g, %g)", original_ctx, (double)high_freq_factor, (double)low_freq_factor);
+  out.resize(head_dim / 2);
+  const double two_pi = 6.283185307179586476925286766559;
+  for (int k = 0; k < head_dim / 2; k++) {
+    const double th = pow((double)base, -2.0 * k / head_dim);
+    double v = th / (double)factor;
+    if (mode == CAI_ROPE_LLAMA3) {
+      const double r = (double)original_ctx * th / two_pi;
+      if (r > (double)high_freq_factor) v = th;
+      else if (r >= (double)low_freq_factor) {
+        const double smooth = (r - (double)low_freq_factor) / ((double)high_freq_factor - (double)low_freq_factor);
+        v = (1.0 - smooth) * th / (double)factor + smooth * th;
+      }
+    }
+    out[k] = (float)v;
+  }
+  return CAI_OK;
+}
+
 __global__ void add_kernel(float* x, const float* y, int64_t n)
 {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;

@@ -252,10 +252,9 @@ extern "C" int cai_sample_candidates(const float* logits, int n, const int32_t* 
   const float* row = logits;
   if (!(flags & CAI_X_DEVICE)) {
     // the row travels into a private device buffer behind the scratch areas run_candidates lays out
-    static float* up = nullptr; static size_t up_cap = 0;
-    int rc = ensure_stage((void**)&up, &up_cap, (size_t)n * 4); if (rc) return rc;
-    CAI_HIP(hipMemcpyAsync(up, logits, (size_t)n * 4, hipMemcpyHostToDevice, c.stream));
-    row = up;
+    int rc = ensure_stage(&c.stage_sample, &c.stage_sample_cap, (size_t)n * 4); if (rc) return rc;
+    CAI_HIP(hipMemcpyAsync(c.stage_sample, logits, (size_t)n * 4, hipMemcpyHostToDevice, c.stream));
+    row = (const float*)c.stage_sample;
   }
   return run_candidates(row, n, hist_ids, hist_counts, n_hist, repetition, frequency, presence, temperature, m, tokens_out, probs_out, count_out);
 }

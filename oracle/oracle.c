@@ -527,6 +527,39 @@ void orc_rope_thetas(float base, int head_dim, float* th)
   for (int k = 0; k < head_dim / 2; k++) th[k] = (float)pow((double)base, -2.0 * k / head_dim);
 }
 
+/* Frequency table under a long-context rule (neural/neuralpretrained.pas:633-668: "linear" -> Position Interpolation,
+ * "llama3" -> the Llama-3.1 rule with original_max_position_embeddings, low_freq_factor, high_freq_factor and NO output
+ * scale).  mode 0 none, 1 linear, 2 llama3.  The layer that applies the rule (TNNetRotaryEmbedding) is not among the
+ * reference's files here, so the formulas are the published ones the importer's comments name: PI divides every frequency
+ * by the factor; llama3 keeps pairs that turn more than high_freq_factor times over the original context, divides those
+ * that turn less than low_freq_factor times, and blends linearly in the rotation count between.
+ * Pinned by: the saturating case of tests/TestNeuralNumerical.pas:16008-16028 (d = 8, base 1e4, original 512, low 1,
+ * high 4, factor 8: pairs 0, 1 kept, pairs 2, 3 divided by 8), theta/factor for linear, an independent float64 restatement
+ * of the published rule on a 128-wide head (tests/test_oracle_model.py).  The blend region itself: parity unpinned against
+ * the reference's layer (no fixture exercises it). */
+int orc_rope_thetas_scaled(float base, int head_dim, int mode, float factor, int original_ctx, float low_freq_factor, float high_freq_factor, float* th)
+{
+  if (mode < 0 || mode > 2 || !(factor >= 1.0f)) return -1;
+  if (mode == 2 && (original_ctx <= 0 || !(high_freq_factor > low_freq_factor))) return -1;
+  for (int k = 0; k < head_dim / 2; k++) {
+    const double t = pow((double)base, -2.0 * k / head_dim);
+    double v = t;
+    if (mode == 1) v = t / (double)factor;
+    if (mode == 2) {
+      const double wavelen = 2.0 * M_PI / t;
+      const double lo_wl = (double)original_ctx / (double)low_freq_factor, hi_wl = (double)original_ctx / (double)high_freq_factor;
+      if (wavelen < hi_wl) v = t;
+      else if (wavelen > lo_wl) v = t / (double)factor;
+      else {
+        const double smooth = ((double)original_ctx / wavelen - (double)low_freq_factor) / ((double)high_freq_factor - (double)low_freq_factor);
+        v = (1.0 - smooth) * t / (double)factor + smooth * t;
+      }
+    }
+    th[k] = (float)v;
+  }
+  return 0;
+}
+
 /* neural.cl:1517-1542: pairs (2k,2k+1) per head, angle = (float)pos * theta_k (fp32 product). */
 void orc_rope_interleaved(float* x, int n_heads, int head_dim, int pos, const float* th)
 {
@@ -891,6 +924,12 @@ int orc_model_set_vec(orc_model* m, int layer, int slot, const float* v, int n)
   if (layer < 0 || layer >= m->cfg.n_layers || slot < 0 || slot > 4) return -1;
   m->layers[layer].v[slot] = v;
   return 0;
+}
+
+/* replaces the model's frequency table (head_dim / 2 values): long-context rules only change the table */
+void orc_model_set_thetas(orc_model* m, const float* th, int n)
+{
+  if (n == m->cfg.head_dim / 2) memcpy(m->theta, th, sizeof(float) * (size_t)n);
 }
 
 void orc_model_reset(orc_model* m) { m->len = 0; }

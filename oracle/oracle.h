@@ -65,6 +65,7 @@ int orc_gemv(int type, const void* raw, const float* scales, int64_t rows, int64
 /* ---- elementwise layer math ---- */
 void orc_rmsnorm(const float* x, const float* gain, int n, float eps, float* y);     /* neural.cl:1047-1085 */
 void orc_rope_thetas(float base, int head_dim, float* theta_half);                   /* neural.cl:1510-1515 (host table) */
+int  orc_rope_thetas_scaled(float base, int head_dim, int mode, float factor, int original_ctx, float low_freq_factor, float high_freq_factor, float* theta_half); /* neuralpretrained.pas:633-668 */
 void orc_rope_interleaved(float* x, int n_heads, int head_dim, int pos, const float* theta_half); /* neural.cl:1517-1542 */
 void orc_swiglu(const float* up_gate, int half, float* y);                           /* neural.cl:1213-1263 flag 1 */
 void orc_softmax(const float* x, int n, float* y);                                   /* neural.cl:1594-1647 */
@@ -131,6 +132,7 @@ void orc_model_free(orc_model* m);
 int  orc_model_set_tensor(orc_model* m, int layer, int slot, int type, int64_t rows, int64_t cols,
                           const void* raw, const float* scales, const float* bias);
 int  orc_model_set_vec(orc_model* m, int layer, int slot, const float* v, int n);
+void orc_model_set_thetas(orc_model* m, const float* theta_half, int n);
 void orc_model_reset(orc_model* m);
 void orc_model_truncate(orc_model* m, int n);
 int  orc_model_len(const orc_model* m);

@@ -44,6 +44,8 @@ def lib():
         L.orc_gemv.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         L.orc_rmsnorm.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_void_p]; L.orc_rmsnorm.restype = None
         L.orc_rope_thetas.argtypes = [C.c_float, C.c_int, C.c_void_p]; L.orc_rope_thetas.restype = None
+        L.orc_rope_thetas_scaled.argtypes = [C.c_float, C.c_int, C.c_int, C.c_float, C.c_int, C.c_float, C.c_float, C.c_void_p]
+        L.orc_model_set_thetas.argtypes = [C.c_void_p, C.c_void_p, C.c_int]; L.orc_model_set_thetas.restype = None
         L.orc_rope_interleaved.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]; L.orc_rope_interleaved.restype = None
         L.orc_swiglu.argtypes = [C.c_void_p, C.c_int, C.c_void_p]; L.orc_swiglu.restype = None
         L.orc_softmax.argtypes = [C.c_void_p, C.c_int, C.c_void_p]; L.orc_softmax.restype = None
@@ -150,6 +152,10 @@ class OracleModel:
         v = np.ascontiguousarray(v, np.float32)
         self.keep.append(v)
         assert lib().orc_model_set_vec(self.h, layer, slot, _p(v), v.size) == 0
+
+    def set_thetas(self, th):
+        th = np.ascontiguousarray(th, np.float32)
+        lib().orc_model_set_thetas(self.h, _p(th), th.size)
 
     def reset(self):
         lib().orc_model_reset(self.h)

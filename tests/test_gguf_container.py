@@ -113,3 +113,84 @@ def test_minimal_valid_file_and_missing_file(tmp_path):
     assert np.array_equal(g.tensor_bytes("t").view(np.float32), np.arange(8, dtype=np.float32))
     with pytest.raises(cai.CaiError):
         cai.GGUF(str(tmp_path / "absent.gguf"))
+
+
+def test_string_array_reads_in_any_order_match_the_python_reader(tmp_path):
+    """cai_gguf_meta_array_str remembers where the last read ended (a vocabulary walked in order costs one entry per call);
+    forward, repeated, backward and scattered reads must all return the entry asked for."""
+    words = [("tok%d" % i) * (1 + i % 5) for i in range(300)] + ["", "é✓"]
+    payload = struct.pack("<IQ", 8, len(words)) + b"".join(struct.pack("<Q", len(w.encode())) + w.encode() for w in words)
+    other = struct.pack("<IQ", 8, 2) + b"".join(struct.pack("<Q", 1) + c for c in (b"a", b"b"))
+    p = tmp_path / "v.gguf"
+    p.write_bytes(_gguf(meta=[(b"tokenizer.ggml.tokens", 9, payload), (b"other", 9, other)], pad_to=32))
+    g = cai.GGUF(str(p))
+    n = g.meta_array_count("tokenizer.ggml.tokens")
+    assert n == len(words)
+    order = list(range(n)) + [5, 5, 4, 301, 0, 150, 151, 149, 300] + list(range(n - 1, -1, -7))
+    for i in order:
+        assert g.meta_array_str("tokenizer.ggml.tokens", i) == words[i], i
+        if i % 50 == 0:      # another array in between must not disturb the remembered position
+            assert g.meta_array_str("other", 1) == "b"
+    with pytest.raises(cai.CaiError):
+        g.meta_array_str("tokenizer.ggml.tokens", n)
+
+
+def _tiny_decoder_file(path, arch, extra_meta=(), drop=(), extra_tensors=()):
+    """A one-block decoder file of zeros with the keys the loader requires (written with the tests' GGUF writer)."""
+    from helpers.gguf_write import write_gguf
+    meta = {"general.architecture": arch, arch + ".block_count": 1, arch + ".embedding_length": 32, arch + ".feed_forward_length": 64,
+            arch + ".attention.head_count": 2, arch + ".context_length": 16}
+    meta.update(dict(extra_meta))
+    z = lambda r, c: np.zeros((r, c), np.float32).tobytes()
+    tens = [("token_embd.weight", [10, 32], 0, z(10, 32)), ("output_norm.weight", [32], 0, z(1, 32))]
+    for nm, r, c in [("attn_q", 32, 32), ("attn_k", 32, 32), ("attn_v", 32, 32), ("attn_output", 32, 32), ("ffn_up", 64, 32), ("ffn_gate", 64, 32), ("ffn_down", 32, 64)]:
+        tens.append(("blk.0.%s.weight" % nm, [r, c], 0, z(r, c)))
+    for nm in ("attn_norm", "ffn_norm"):
+        tens.append(("blk.0.%s.weight" % nm, [32], 0, z(1, 32)))
+    if arch == "qwen2":
+        for nm in ("attn_q", "attn_k", "attn_v"):
+            tens.append(("blk.0.%s.bias" % nm, [32], 0, z(1, 32)))
+    tens = [t for t in tens if t[0] not in drop] + list(extra_tensors)
+    write_gguf(path, meta, tens)
+
+
+LOADER_REFUSALS = {
+    # what the reference's importer refuses (neural/neuralpretrained.pas:17539-17557, 17755-17760) is refused here for the same reason
+    "qwen2 sliding window": ("qwen2", {"qwen2.attention.sliding_window": 4096}, (), (), "sliding-window"),
+    "qwen2 without a bias": ("qwen2", {}, ("blk.0.attn_k.bias",), (), "blk.0.attn_k.bias"),
+    "yarn scaling": ("llama", {"llama.rope.scaling.type": "yarn", "llama.rope.scaling.factor": 4.0}, (), (), "supported: none, linear"),
+    "linear factor below one": ("llama", {"llama.rope.scaling.type": "linear", "llama.rope.scaling.factor": 0.5}, (), (), "must be >= 1"),
+    "rope_freqs of the wrong length": ("llama", {}, (), (("rope_freqs.weight", [4], 0, np.ones(4, np.float32).tobytes()),), "one per rotary pair"),
+    "rope_freqs with linear scaling": ("llama", {"llama.rope.scaling.type": "linear", "llama.rope.scaling.factor": 2.0}, (),
+                                       (("rope_freqs.weight", [8], 0, np.ones(8, np.float32).tobytes()),), "together with linear scaling"),
+}
+
+
+@pytest.mark.parametrize("case", list(LOADER_REFUSALS))
+def test_decoder_loader_judges_the_metadata_before_it_needs_a_device(case, tmp_path):
+    """cai_decoder_load_gguf refuses what it cannot run from the file's metadata alone, with the reason, GPU or not."""
+    import ctypes as C
+    arch, meta, drop, extra, needle = LOADER_REFUSALS[case]
+    p = str(tmp_path / "m.gguf")
+    _tiny_decoder_file(p, arch, meta, drop, extra)
+    h = C.c_void_p()
+    rc = cai.load().cai_decoder_load_gguf(p.encode(), 0, 1, 0, C.byref(h))
+    assert rc != 0 and not h.value
+    buf = C.create_string_buffer(2048); cai.load().cai_last_error(buf, 2048)
+    assert needle in buf.value.decode(), buf.value.decode()
+
+
+def test_pascal_binding_and_header_constants_agree():
+    """CAI_* integer constants of the Pascal unit equal the header's."""
+    import os
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    hdr = open(os.path.join(root, "include", "caihip.h")).read()
+    pas = open(os.path.join(root, "neural-api_amd", "pascal", "caihip.pas")).read()
+    h = {m.group(1): int(m.group(2)) for m in re.finditer(r"#define\s+(CAI_[A-Z0-9_]+)\s+\(?(-?\d+)\)?", hdr)}
+    p = {m.group(1): int(m.group(2)) for m in re.finditer(r"\b(CAI_[A-Z0-9_]+)\s*=\s*(-?\d+)\s*;", pas)}
+    assert len(p) >= 20
+    for k, v in p.items():
+        assert h.get(k) == v, (k, v, h.get(k))
+    for k in ("CAI_Q5_K", "CAI_Q2_K", "CAI_Q3_K", "CAI_Q4_1", "CAI_Q5_0", "CAI_Q5_1", "CAI_ROPE_LINEAR", "CAI_ROPE_LLAMA3"):
+        assert k in p, k

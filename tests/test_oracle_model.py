@@ -104,3 +104,41 @@ def test_avx_baseline_kernels_match_scalar():
         c = rng.integers(-127, 128, n).astype(np.int8)
         assert abs(O.lib().cpu_avx_dot_f32(a.ctypes.data, b.ctypes.data, n) - float(a.astype(np.float64) @ b)) < 1e-4 * max(1, n ** 0.5)
         assert abs(O.lib().cpu_avx_dot_int8(c.ctypes.data, b.ctypes.data, n) - float(c.astype(np.float64) @ b)) < 1e-3 * max(1, n ** 0.5)
+
+
+def _scaled(base, hd, mode, factor, orig=0, low=1.0, high=4.0):
+    import ctypes as C
+    th = np.empty(hd // 2, np.float32)
+    assert O.lib().orc_rope_thetas_scaled(C.c_float(base), hd, mode, C.c_float(factor), orig, C.c_float(low), C.c_float(high), th.ctypes.data) == 0
+    return th
+
+
+def test_rope_scaling_tables():
+    """Long-context frequency rules (neural/neuralpretrained.pas:633-668).  Known answers: the saturating case the reference's
+    own test describes (tests/TestNeuralNumerical.pas:16008-16028: d = 8, base 1e4, original 512, low 1, high 4 - pairs 0, 1
+    keep their frequency, pairs 2, 3 are fully interpolated); linear = theta / factor; and the published Llama-3.1 rule
+    written a second way (numpy float64, wavelength masks) on a 128-wide head with the Llama-3.1 constants."""
+    base = np.array([1e4 ** (-2.0 * k / 8) for k in range(4)])
+    th = _scaled(1e4, 8, 2, 8.0, 512, 1.0, 4.0)
+    assert np.array_equal(th, np.array([base[0], base[1], base[2] / 8, base[3] / 8]).astype(np.float32))
+    assert np.array_equal(_scaled(1e4, 8, 1, 4.0), (base / 4).astype(np.float32))
+    assert np.array_equal(_scaled(1e4, 8, 0, 1.0), base.astype(np.float32))
+    # Llama-3.1: rope_theta 5e5, factor 8, original 8192, low 1, high 4
+    hd, factor, orig, low, high = 128, 8.0, 8192, 1.0, 4.0
+    inv = 5e5 ** (-np.arange(0, hd, 2, dtype=np.float64) / hd)
+    wavelen = 2 * np.pi / inv
+    out = np.where(wavelen > orig / low, inv / factor, inv)
+    smooth = (orig / wavelen - low) / (high - low)
+    mid = ~(wavelen < orig / high) & ~(wavelen > orig / low)
+    out = np.where(mid, (1 - smooth) * inv / factor + smooth * inv, out)
+    th = _scaled(5e5, hd, 2, factor, orig, low, high)
+    assert np.array_equal(th, out.astype(np.float32))
+    assert mid.sum() >= 5 and (wavelen < orig / high).sum() >= 20 and (wavelen > orig / low).sum() >= 20   # all three regimes present
+    # between the two limits everywhere, non-increasing in k like the unscaled table
+    assert np.all(th <= inv.astype(np.float32)) and np.all(th >= (inv / factor).astype(np.float32) * (1 - 1e-7))
+    assert np.all(np.diff(th) <= 0)
+    # refused arguments
+    import ctypes as C
+    buf = np.empty(4, np.float32)
+    assert O.lib().orc_rope_thetas_scaled(C.c_float(1e4), 8, 1, C.c_float(0.5), 0, C.c_float(1), C.c_float(4), buf.ctypes.data) != 0
+    assert O.lib().orc_rope_thetas_scaled(C.c_float(1e4), 8, 2, C.c_float(8), 512, C.c_float(4), C.c_float(4), buf.ctypes.data) != 0
