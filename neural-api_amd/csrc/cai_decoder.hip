@@ -28,6 +28,9 @@ struct cai_decoder_s {
   int pf_cap = 0;
   float *px = nullptr, *pqkv = nullptr, *patt = nullptr, *pgu = nullptr, *pmid = nullptr, *ppart = nullptr;
   int32_t* ptokpos = nullptr;                        // [2][pf_cap]: tokens, positions
+  // mixture-of-experts prompt: per chunk the router outputs, the slots grouped by expert and the per-slot activations
+  float *pm_logits = nullptr, *pm_probs = nullptr, *pm_gate = nullptr, *pm_gu = nullptr, *pm_mid = nullptr, *pm_part = nullptr;
+  int32_t *pm_expert = nullptr, *pm_perm = nullptr, *pm_tiles = nullptr;
   int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_argmax = nullptr, *d_gen = nullptr;
   int32_t* h_io = nullptr;   // pinned: tokens[8] pos[8] argmax[8]
   hipGraphExec_t graph[9] = {nullptr};
@@ -228,6 +231,14 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = 
 // Multi-token prompt ingestion of one chunk (n <= pf_cap tokens of sequence `seq` at positions pos0..): every linear
 // layer runs once for the whole chunk (matrix cores for Q4_K), K,V rows are appended, then each token attends up to
 // its own position.  Equals n sequential steps (the reference's prefill, neural/neuralchatengine.pas:1466-1470).
+static void free_moe_prompt(cai_decoder_s* d)
+{
+  void* q[] = {d->pm_logits, d->pm_probs, d->pm_gate, d->pm_gu, d->pm_mid, d->pm_part, d->pm_expert, d->pm_perm, d->pm_tiles};
+  for (void* v : q) if (v) (void)hipFree(v);
+  d->pm_logits = d->pm_probs = d->pm_gate = d->pm_gu = d->pm_mid = d->pm_part = nullptr;
+  d->pm_expert = d->pm_perm = d->pm_tiles = nullptr;
+}
+
 static int ensure_prefill_buffers(cai_decoder_s* d, int n)
 {
   if (d->pf_cap >= n) return CAI_OK;
@@ -237,6 +248,7 @@ static int ensure_prefill_buffers(cai_decoder_s* d, int n)
   { float* pf[] = {d->px, d->pqkv, d->patt, d->pgu, d->pmid, d->ppart}; for (float* q : pf) if (q) (void)hipFree(q); }
   if (d->ptokpos) (void)hipFree(d->ptokpos);
   d->px = d->pqkv = d->patt = d->pgu = d->pmid = d->ppart = nullptr; d->ptokpos = nullptr; d->pf_cap = 0;
+  free_moe_prompt(d);
   const size_t qkvw = d->qw() + 2 * d->kw();
   CAI_HIP(hipMalloc((void**)&d->px, (size_t)cap * c.d_model * 4));
   CAI_HIP(hipMalloc((void**)&d->pqkv, (size_t)cap * qkvw * 4));
@@ -245,17 +257,48 @@ static int ensure_prefill_buffers(cai_decoder_s* d, int n)
   CAI_HIP(hipMalloc((void**)&d->pmid, (size_t)cap * c.ffn * 4));
   CAI_HIP(hipMalloc((void**)&d->ppart, (size_t)cap * c.n_q_heads * d->kv.n_splits * (c.head_dim + 2) * 4));
   CAI_HIP(hipMalloc((void**)&d->ptokpos, (size_t)cap * 2 * sizeof(int32_t)));
+  if (c.n_experts > 0 && c.n_experts <= 512) {
+    const size_t E = c.n_experts, S = (size_t)cap * c.top_k;
+    CAI_HIP(hipMalloc((void**)&d->pm_logits, (size_t)cap * E * 4)); CAI_HIP(hipMalloc((void**)&d->pm_probs, (size_t)cap * E * 4));
+    CAI_HIP(hipMalloc((void**)&d->pm_gate, S * 4)); CAI_HIP(hipMalloc((void**)&d->pm_expert, S * 4)); CAI_HIP(hipMalloc((void**)&d->pm_perm, S * 4));
+    CAI_HIP(hipMalloc((void**)&d->pm_tiles, (size_t)moe_group_max_tiles((int)S, c.n_experts) * 3 * 4));
+    CAI_HIP(hipMalloc((void**)&d->pm_gu, S * 2 * c.ffn * 4)); CAI_HIP(hipMalloc((void**)&d->pm_mid, S * c.ffn * 4)); CAI_HIP(hipMalloc((void**)&d->pm_part, S * c.d_model * 4));
+  }
   d->pf_cap = cap;
   return CAI_OK;
 }
 
 static int linear_rows(const cai_qw_s* w, bool prepped, const float* x, int64_t x_stride, const float* gain, float eps, int n,
+                       float* y, int64_t y_stride, const float* residual);
+
+// Expert half of a block for a whole prompt chunk in px (n tokens), in place (neural/neuralpretrained.pas:15331-15388):
+// router logits -> soft-max / top-k for every token -> the n * top_k slots grouped by expert -> gate|up over the bank in one
+// launch -> SwiGLU -> down over the bank in one launch -> gate-weighted mixture added to each row.
+static int moe_ffn_prompt(cai_decoder_s* d, const cai_decoder_s::Layer& L, int n)
+{
+  const cai_decoder_config& c = d->cfg;
+  const int dm = c.d_model, I = c.ffn, E = c.n_experts, K = c.top_k, slots = n * K;
+  int rc;
+  if ((rc = linear_rows(L.w[CAI_W_ROUTER], false, d->px, dm, L.v[CAI_V_MLP_NORM], c.eps, n, d->pm_logits, E, nullptr))) return rc;
+  if ((rc = launch_router_topk(d->pm_logits, E, K, c.norm_topk, n, d->pm_expert, d->pm_gate, d->pm_probs))) return rc;
+  if ((rc = launch_moe_group(d->pm_expert, slots, E, d->pm_perm, d->pm_tiles))) return rc;
+  const _Float16 *hi, *lo; const float* sinv;
+  if ((rc = prefill_prep(d->px, dm, L.v[CAI_V_MLP_NORM], c.eps, dm, n))) return rc;
+  prefill_planes(&hi, &lo, &sinv);
+  if ((rc = launch_gemm_blk_grouped(L.w[CAI_W_GATEUP], 2 * (int64_t)I, hi, lo, sinv, K, slots, E, d->pm_perm, d->pm_tiles, d->pm_gu, 2 * I))) return rc;
+  launch_swiglu(d->pm_gu, I, slots, d->pm_mid);
+  if ((rc = prefill_prep(d->pm_mid, I, nullptr, 0.0f, I, slots))) return rc;
+  prefill_planes(&hi, &lo, &sinv);
+  if ((rc = launch_gemm_blk_grouped(L.w[CAI_W_DOWN], dm, hi, lo, sinv, 1, slots, E, d->pm_perm, d->pm_tiles, d->pm_part, dm))) return rc;
+  return launch_moe_combine(d->px, d->pm_part, d->pm_gate, K, dm, n);
+}
+
+static int linear_rows(const cai_qw_s* w, bool prepped, const float* x, int64_t x_stride, const float* gain, float eps, int n,
                        float* y, int64_t y_stride, const float* residual)
 {
-  // few tokens (the bandwidth-bound regime) of a Q4_K or Q6_K matrix, or a large matrix of a type without a prompt kernel (a small
-  // one stays in the cache: the single-launch VALU kernel per 8 tokens is cheaper than three launches)
-  if (nb_supported(w) && (gemm_mfma_supported(w) ? n <= 16 : w->data_bytes >= ((int64_t)16 << 20))) return nb_linear(w, x, x_stride, gain, eps, n, y, y_stride, residual);
-  if (gemm_mfma_supported(w)) {
+  const int route = prompt_route(w, n);
+  if (route == 1) return nb_linear(w, x, x_stride, gain, eps, n, y, y_stride, residual);
+  if (route == 2) {
     int rc;
     if (!prepped && (rc = prefill_prep(x, x_stride, gain, eps, (int)w->cols, n))) return rc;
     return prefill_gemm(w, n, y, y_stride, residual);
@@ -273,8 +316,8 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
   for (int l = 0; l < c.n_layers; l++) {
     auto& L = d->layers[l];
     const cai_qw_s* wq = L.w[CAI_W_Q]; const cai_qw_s* wk = L.w[CAI_W_K]; const cai_qw_s* wv = L.w[CAI_W_V];
-    const bool all_mfma = gemm_mfma_supported(wq) && gemm_mfma_supported(wk) && gemm_mfma_supported(wv);
-    if (all_mfma && n > 16 && (rc = prefill_prep(d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, dm, n))) return rc;
+    const bool all_mfma = prompt_route(wq, n) == 2 && prompt_route(wk, n) == 2 && prompt_route(wv, n) == 2;   // one pre-pass serves q, k and v
+    if (all_mfma && (rc = prefill_prep(d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, dm, n))) return rc;
     if ((rc = linear_rows(wq, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv, qkvw, nullptr))) return rc;
     if ((rc = linear_rows(wk, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw, qkvw, nullptr))) return rc;
     if ((rc = linear_rows(wv, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw + kw, qkvw, nullptr))) return rc;
@@ -282,8 +325,13 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
                                c.qk_norm_full ? L.v[CAI_V_Q_NORM] : nullptr, c.qk_norm_full ? L.v[CAI_V_K_NORM] : nullptr, c.eps))) return rc;
     if ((rc = linear_rows(L.w[CAI_W_O], false, d->patt, qw, nullptr, 0.0f, n, d->px, dm, d->px))) return rc;
     if (c.n_experts > 0) {
-      // experts differ from token to token: the routed half runs on groups of rows (one router / top-k launch per group,
-      // the gathered products per token), the attention half above on the whole chunk
+      // experts differ from token to token.  A chunk of more than 16 tokens whose banks the block prompt kernel takes is
+      // sorted by expert and runs each projection as ONE launch over the bank; otherwise the routed half runs on groups of
+      // rows (one router / top-k launch per group, the gathered products per token)
+      if (n > 16 && d->pm_gu && gemm_blk_supported(L.w[CAI_W_GATEUP]) && gemm_blk_supported(L.w[CAI_W_DOWN])) {
+        if ((rc = moe_ffn_prompt(d, L, n))) return rc;
+        continue;
+      }
       const int grp = 8;
       for (int t0 = 0; t0 < n; t0 += grp)
         if ((rc = moe_ffn_rows(d, L, d->px + (int64_t)t0 * dm, std::min(grp, n - t0)))) return rc;
@@ -395,6 +443,7 @@ extern "C" int cai_decoder_destroy(cai_decoder_t d)
   for (auto& L : d->layers) for (float* p : L.v) if (p) (void)hipFree(p);
   { float* pf[] = {d->px, d->pqkv, d->patt, d->pgu, d->pmid, d->ppart}; for (float* q : pf) if (q) (void)hipFree(q); }
   if (d->ptokpos) (void)hipFree(d->ptokpos);
+  free_moe_prompt(d);
   if (d->moe_expert) (void)hipFree(d->moe_expert);
   if (d->am_v) (void)hipFree(d->am_v);
   if (d->am_i) (void)hipFree(d->am_i);

@@ -203,7 +203,17 @@ int kv_restore(cai_kv_s* kv, int seq, const cai_kv_snap_s* snap);
 // multi-token linear layer (matrix cores for Q4_K, small-batch kernel otherwise); gain != null fuses RMSNorm
 int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok,
                    float* y, int64_t y_stride, const float* residual);
-bool gemm_mfma_supported(const cai_qw_s* w);   // many-token (prompt) matrix-core kernel
+bool gemm_mfma_supported(const cai_qw_s* w);   // many-token (prompt) matrix-core kernel of the super-block types (Q4_K, Q6_K)
+bool gemm_blk_supported(const cai_qw_s* w);    // many-token (prompt) matrix-core kernel of the 32-weight block types (Q8_0, Q4_0)
+inline bool prompt_gemm_supported(const cai_qw_s* w) { return gemm_mfma_supported(w) || gemm_blk_supported(w); }
+int launch_gemm_blk(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo, const float* sinv, int n_tok, float* y, int64_t y_stride, const float* residual);
+// mixture-of-experts prompt: slots (token * top_k + rank) grouped by expert, then one launch over the bank per projection
+int moe_group_max_tiles(int n_slots, int n_experts);
+int launch_moe_group(const int32_t* expert, int n_slots, int n_experts, int32_t* perm, int32_t* tile_tab);
+int launch_gemm_blk_grouped(const cai_qw_s* bank, int64_t expert_rows, const _Float16* xhi, const _Float16* xlo, const float* sinv, int x_div,
+                            int n_slots, int n_experts, const int32_t* perm, const int32_t* tile_tab, float* y, int64_t y_stride);
+void prefill_planes(const _Float16** hi, const _Float16** lo, const float** sinv);   // what the last prefill_prep filled
+int  prompt_route(const cai_qw_s* w, int n_tok);   // 0 matrix-vector passes, 1 small-batch kernel, 2 prompt kernel
 bool nb_supported(const cai_qw_s* w);          // 2..8-token matrix-core kernel
 // split pre-pass / product form: prep once, then any number of matrices of that width
 // small-batch (<= 8 tokens per pass) matrix-core path: planes <- activations, partials <- product, consumer sums the slices

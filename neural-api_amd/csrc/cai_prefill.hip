@@ -552,14 +552,30 @@ int prefill_prep(const float* x, int64_t x_stride, const float* gain, float eps,
 int prefill_gemm_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, float* y, int64_t y_stride)
 {
   for (int i = 0; i < n_w; i++) {
-    const int rc = launch_gemm_q4k(ws[i], g_pws.hi, g_pws.lo, g_pws.sxhi, g_pws.sxlo, g_pws.sinv, n_tok, y + y_off[i], y_stride, nullptr);
+    const int rc = prefill_gemm(ws[i], n_tok, y + y_off[i], y_stride, nullptr);
     if (rc) return rc;
   }
   return CAI_OK;
 }
+void prefill_planes(const _Float16** hi, const _Float16** lo, const float** sinv) { *hi = g_pws.hi; *lo = g_pws.lo; *sinv = g_pws.sinv; }
 int prefill_gemm(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride, const float* residual)
 {
+  if (gemm_blk_supported(w)) return launch_gemm_blk(w, g_pws.hi, g_pws.lo, g_pws.sinv, n_tok, y, y_stride, residual);
   return launch_gemm_q4k(w, g_pws.hi, g_pws.lo, g_pws.sxhi, g_pws.sxlo, g_pws.sinv, n_tok, y, y_stride, residual);
+}
+
+// Which kernel family takes n_tok tokens of this matrix: 1 = small-batch matrix-core kernel (passes of up to 8 or 16 tokens;
+// the bandwidth-bound regime), 2 = prompt kernel on prepared activation planes, 0 = matrix-vector kernel in passes of 8.
+//   Q4_K, Q6_K: up to 16 tokens small-batch, above that the prompt kernel;
+//   Q8_0, Q4_0: above 16 tokens the prompt kernel; below, small-batch only for a matrix too large for the cache (a small
+//               one stays resident: one VALU launch per 8 tokens is cheaper than three launches);
+//   per-row int8: small-batch for a large matrix.
+int prompt_route(const cai_qw_s* w, int n_tok)
+{
+  if (gemm_mfma_supported(w)) return n_tok <= 16 && nb_supported(w) ? 1 : 2;
+  if (gemm_blk_supported(w) && n_tok > 16) return 2;
+  if (nb_supported(w) && w->data_bytes >= ((int64_t)16 << 20)) return 1;
+  return 0;
 }
 
 // y[t][rows] = W x[t] (+bias) (+residual) for n_tok tokens; x rows are x_stride apart; gain != null fuses RMSNorm.
@@ -569,13 +585,13 @@ int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const fl
   int rc;
   // few tokens (the bandwidth-bound regime) of a Q4_K or Q6_K matrix, or a large matrix of a type without a prompt kernel (a small
   // one stays in the cache: the single-launch VALU kernel per 8 tokens is cheaper than three launches)
-  if (nb_supported(w) && (gemm_mfma_supported(w) ? n_tok <= 16 : w->data_bytes >= ((int64_t)16 << 20))) return nb_linear(w, x, x_stride, gain, eps, n_tok, y, y_stride, residual);
-  if (gemm_mfma_supported(w)) {
+  if (prompt_route(w, n_tok) == 1) return nb_linear(w, x, x_stride, gain, eps, n_tok, y, y_stride, residual);
+  if (prompt_route(w, n_tok) == 2) {
     if ((rc = prefill_prep(x, x_stride, gain, eps, (int)w->cols, n_tok))) return rc;
     return prefill_gemm(w, n_tok, y, y_stride, residual);
   }
-  // other weight types: groups of up to 8 tokens through the small-batch kernel (x must be contiguous)
-  if (x_stride != w->cols) return set_error(CAI_ERR_UNSUPPORTED, "prefill linear: strided input needs a Q4_K or Q6_K matrix");
+  // other weight types and small matrices at few tokens: groups of up to 8 tokens through the small-batch kernel (x must be contiguous)
+  if (x_stride != w->cols) return set_error(CAI_ERR_UNSUPPORTED, "prefill linear: strided input needs a matrix the matrix-core kernels take");
   for (int t = 0; t < n_tok; t += 8) {
     const int nb = std::min(8, n_tok - t);
     MultiGemv m{}; m.n = 1; m.w[0] = w; m.rows[0] = w->rows;

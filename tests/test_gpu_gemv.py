@@ -282,3 +282,24 @@ def test_gemv_batch_on_large_matrix_goes_to_matrix_cores(qt, rows, cols, nb):
     assert rel_err(got, want, floor=0.02 * cols ** 0.5) < TIGHT
     one = w.gemv(x[:1])
     assert rel_err(got[:1], one, floor=0.02 * cols ** 0.5) < TIGHT
+
+
+@pytest.mark.parametrize("qt", [O.Q8_0, O.Q4_0])
+@pytest.mark.parametrize("rows,cols,T", [(200, 576, 17), (577, 576, 40), (192, 576, 255), (1000, 1024, 33), (3584, 3584, 77), (512, 18944, 64), (130, 512, 129),
+                                         (4099, 256, 96), (96, 160, 31), (5, 32, 100), (9000, 2048, 300), (64, 2048, 255)])
+def test_prompt_gemm_q8_0_q4_0_on_matrix_cores(qt, rows, cols, T):
+    """More than 16 tokens of a 32-weight block type go to the prompt kernel (weights as the B operand of 32x32x16 tiles, the
+    block scale applied to each block's sums): == T single-token layers of the oracle, bias included; widths that end inside a
+    256-column step, row counts that end inside a tile, token counts that end inside a token tile."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    raw, rng = make(qt, rows, cols, T + 300)
+    x = (rng.standard_normal((T, cols)) * rng.uniform(0.01, 30.0, (T, 1))).astype(np.float32)
+    x[0, : cols // 2] = 0.0
+    bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
+    w = cai.QWeight(qt, rows, cols, raw, bias)
+    got = w.gemm(x)
+    want = O.gemv(qt, raw, rows, cols, x, bias, 0, 1)
+    for t in range(T):
+        assert rel_err(got[t], want[t], floor=0.02 * cols ** 0.5 * float(np.abs(x[t]).mean())) < TIGHT, t
+    w.close()
