@@ -161,7 +161,10 @@ def gemv_sweep(cai, synth, torch, with_cpu):
     cache-resident and are labelled so)."""
     lib = cai.load()
     QT = {"Q8_0": (cai.Q8_0, 34 / 32), "Q4_0": (cai.Q4_0, 18 / 32), "Q4_K": (cai.Q4_K, 144 / 256), "Q6_K": (cai.Q6_K, 210 / 256),
-          "I8ROW": (cai.I8ROW, 1.0)}   # I8ROW: the reference's own per-row int8 format
+          "I8ROW": (cai.I8ROW, 1.0),   # I8ROW: the reference's own per-row int8 format
+          # the types kept as the stored block stream (Q5_K at batch 1 on the integer-dot kernel, the rest one wave per row)
+          "Q5_K": (cai.Q5_K, 176 / 256), "Q2_K": (cai.Q2_K, 84 / 256), "Q3_K": (cai.Q3_K, 110 / 256), "Q4_1": (cai.Q4_1, 20 / 32),
+          "Q5_0": (cai.Q5_0, 22 / 32), "Q5_1": (cai.Q5_1, 24 / 32)}
     shapes = [(2048, 2048), (5632, 2048), (2048, 5632), (18944, 3584), (152064, 3584)]
     gen = torch.Generator(device="cuda"); gen.manual_seed(424242)
     cpu = None
@@ -171,10 +174,11 @@ def gemv_sweep(cai, synth, torch, with_cpu):
         from helpers import oracle_lib as O
         cpu = O.lib()
     for name, (qt, bpw) in QT.items():
-        for rows, cols in shapes:
+        for rows, cols in (shapes[3:] if qt in synth.RAW_BLOCKS else shapes):
             mat_bytes = rows * cols * bpw
             copies = int(max(1, min(24, -(-320e6 // mat_bytes))))
-            ws = [synth.random_int8_rows(rows, cols, gen) if name == "I8ROW" else synth.random_qweight(qt, rows, cols, gen)[0] for _ in range(copies)]
+            ws = [synth.random_int8_rows(rows, cols, gen) if name == "I8ROW" else synth.random_raw_qweight(qt, rows, cols, gen) if qt in synth.RAW_BLOCKS
+                  else synth.random_qweight(qt, rows, cols, gen)[0] for _ in range(copies)]
             for nb in (1, 4):
                 x = torch.randn(nb, cols, device="cuda"); y = torch.empty(nb, rows, device="cuda")
                 torch.cuda.synchronize()
@@ -215,7 +219,7 @@ def gemv_sweep(cai, synth, torch, with_cpu):
 # HBM bytes per launch of the 7B-shape gate|up kernel from hardware counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000
 # KiB, factors from a 1 GiB copy kernel): profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt.  Not measurable from
 # inside this process; re-collect when the kernel changes.
-GATEUP_TRAFFIC_BYTES = int((37522.5 * 2.000 + 74.2 * 1.000) * 1024)
+GATEUP_TRAFFIC_BYTES = int((37513.6 * 2.000 + 74.5 * 1.000) * 1024)
 GATEUP_TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of gemv_q4k_dot<1,1,false,2>, profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt"
 
 
@@ -230,7 +234,7 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=8, help="repetitions of each kernel class in the per-kernel table")
     ap.add_argument("--kv", choices=["f32", "f16", "i8"], default=None, help="KV cache element type (default: the configuration's own)")
     ap.add_argument("--batch", type=int, default=1, help="independent sequences decoded together (1..8)")
-    ap.add_argument("--gemv-sweep", action="store_true", help="isolated matrix-vector sweep (BASELINE configs[1]): Q8_0 / Q4_0 / Q4_K and per-row int8, five shapes, batch 1 and 4")
+    ap.add_argument("--gemv-sweep", action="store_true", help="isolated matrix-vector sweep (BASELINE configs[1]): Q8_0 / Q4_0 / Q4_K / Q6_K and per-row int8 on five shapes, the stored-stream types on the two large ones, batch 1 and 4")
     ap.add_argument("--copy-calibration", action="store_true", help="only run the 1 GiB device copy kernel 5 times (reference for traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:

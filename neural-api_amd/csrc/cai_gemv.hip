@@ -488,22 +488,24 @@ __global__ __launch_bounds__(256) void gemv_simple(const GemvParams p, int n_b)
 }
 
 // ------------------------------------------------------------------------------------------
-// Block types resident as the stored stream (Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K).  One wave per row; a lane decodes runs
-// of 16 consecutive weights (run = lane + 64 k, so the 16 lanes of a super-block share its header in cache) and feeds
-// every batch row from the one decode.  fp32 accumulation; fused RMSNorm, bias, activation, residual and the expert-bank
-// gather as in the other kernels.
+// Block types resident as the stored stream (Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K).  A wave takes four consecutive rows; a
+// lane decodes runs of 16 consecutive weights (run = lane + 64 k, so the 16 lanes of a super-block share its header in
+// cache).  The activation values of a run are fetched once for the four rows (one row per wave moved six times the
+// weight bytes through the vector cache), and one decode feeds every batch row.  fp32 accumulation; fused RMSNorm, bias,
+// activation, residual and the expert-bank gather as in the other kernels.
 // ------------------------------------------------------------------------------------------
-template <int QT>
+template <int QT, int NB>   // NB: batch rows the accumulators cover (1 or 8)
 __global__ __launch_bounds__(256) void gemv_raw(const GemvParams p, int n_b)
 {
+  constexpr int R = 4;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int64_t grow = (int64_t)blockIdx.x * 4 + wave;
+  const int64_t grp = (int64_t)blockIdx.x * 4 + wave;
   int s = 0; int64_t g0 = 0;
-  if (p.n_seg > 1 && grow >= p.seg[0].grp_end) { s = 1; g0 = p.seg[0].grp_end; }
-  if (p.n_seg > 2 && grow >= p.seg[1].grp_end) { s = 2; g0 = p.seg[1].grp_end; }
-  if (grow >= p.seg[p.n_seg - 1].grp_end) return;
+  if (p.n_seg > 1 && grp >= p.seg[0].grp_end) { s = 1; g0 = p.seg[0].grp_end; }
+  if (p.n_seg > 2 && grp >= p.seg[1].grp_end) { s = 2; g0 = p.seg[1].grp_end; }
+  if (grp >= p.seg[p.n_seg - 1].grp_end) return;
   const GemvSeg sg = p.seg[s];
-  const int row = (int)(grow - g0);
+  const int row0 = (int)(grp - g0) * R;
   const int cols = p.cols;
   int64_t bank_row = 0;
   const float* xin = p.x; float* yout = p.y;
@@ -511,11 +513,13 @@ __global__ __launch_bounds__(256) void gemv_raw(const GemvParams p, int n_b)
     bank_row = (int64_t)min(max(p.slot_expert[blockIdx.y], 0), p.bank_experts - 1) * p.expert_rows;
     xin += (int64_t)blockIdx.y * p.x_slot_stride; yout += (int64_t)blockIdx.y * p.y_slot_stride;
   }
-  const int64_t wrow = bank_row + row;
-  const uint8_t* wbase = sg.data + wrow * (int64_t)(cols / raw_block_elems(QT)) * raw_block_bytes(QT);
-  float inv[8];
+  const int64_t row_bytes = (int64_t)(cols / raw_block_elems(QT)) * raw_block_bytes(QT);
+  const uint8_t* wbase[R];
 #pragma unroll
-  for (int b = 0; b < 8; b++) {
+  for (int r = 0; r < R; r++) wbase[r] = sg.data + (bank_row + min(row0 + r, sg.rows - 1)) * row_bytes;   // tail group: the last row again, not written
+  float inv[NB];
+#pragma unroll
+  for (int b = 0; b < NB; b++) {
     inv[b] = 1.0f;
     if (p.norm_gain && b < n_b) {
       const float* xb = xin + (int64_t)b * cols;
@@ -525,46 +529,55 @@ __global__ __launch_bounds__(256) void gemv_raw(const GemvParams p, int n_b)
       inv[b] = 1.0f / sqrtf(ss / (float)cols + p.norm_eps);
     }
   }
-  float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+  float acc[R][NB];
+#pragma unroll
+  for (int r = 0; r < R; r++)
+#pragma unroll
+    for (int b = 0; b < NB; b++) acc[r][b] = 0.0f;
   const int n_runs = cols >> 4;
   for (int run = lane; run < n_runs; run += 64) {
-    float w[16];
-    raw_run16<QT>(wbase, run, w);
+    float w[R][16];
+#pragma unroll
+    for (int r = 0; r < R; r++) raw_run16<QT>(wbase[r], run, w[r]);
     float g[16];
     if (p.norm_gain) {
 #pragma unroll
       for (int q = 0; q < 4; q++) { const float4 v = *reinterpret_cast<const float4*>(p.norm_gain + 16 * run + 4 * q); g[4 * q] = v.x; g[4 * q + 1] = v.y; g[4 * q + 2] = v.z; g[4 * q + 3] = v.w; }
     }
 #pragma unroll
-    for (int b = 0; b < 8; b++) {
+    for (int b = 0; b < NB; b++) {
       if (b < n_b) {
         const float* xb = xin + (int64_t)b * cols + 16 * run;
 #pragma unroll
         for (int q = 0; q < 4; q++) {
           const float4 v = *reinterpret_cast<const float4*>(xb + 4 * q);
-          float xv[4] = {v.x, v.y, v.z, v.w};
+          const float xv[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
           for (int t = 0; t < 4; t++) {
             const float xn = p.norm_gain ? g[4 * q + t] * (xv[t] * inv[b]) : xv[t];
-            acc[b] = fmaf(w[4 * q + t], xn, acc[b]);
+#pragma unroll
+            for (int r = 0; r < R; r++) acc[r][b] = fmaf(w[r][4 * q + t], xn, acc[r][b]);
           }
         }
       }
     }
   }
 #pragma unroll
-  for (int b = 0; b < 8; b++) {
-    if (b < n_b) {
-      float a = wave_sum(acc[b]);
-      if (lane == 63) {
-        if (sg.bias) a += sg.bias[wrow];
-        a = act_apply(a, p.act);
-        const int64_t o = (int64_t)b * p.y_stride + sg.y_off + row;
-        if (p.residual) a += p.residual[o];
-        yout[o] = a;
+  for (int r = 0; r < R; r++)
+#pragma unroll
+    for (int b = 0; b < NB; b++) {
+      if (b < n_b) {
+        float a = wave_sum(acc[r][b]);
+        const int row = row0 + r;
+        if (lane == 63 && row < sg.rows) {
+          if (sg.bias) a += sg.bias[bank_row + row];
+          a = act_apply(a, p.act);
+          const int64_t o = (int64_t)b * p.y_stride + sg.y_off + row;
+          if (p.residual) a += p.residual[o];
+          yout[o] = a;
+        }
       }
     }
-  }
 }
 
 // y[b][i] = x[b][i] * silu(x[b][half+i]) for the simple path (unfused SwiGLU)
@@ -733,18 +746,28 @@ int launch_gemv_multi(const MultiGemv& m, const float* x, int n_b, float* y, int
     return launch_fast_nb<CAI_Q6_K, 0>(p, m, n_b, c.stream);
   }
   if (swiglu_half) return set_error(CAI_ERR_UNSUPPORTED, "gemv: fused swiglu needs a block-quantized matrix");
+  if (raw_block_type(qt)) {
+    const int R = 4;
+    int64_t groups = 0;
+    for (int i = 0; i < m.n; i++) { groups += (m.rows[i] + R - 1) / R; p.seg[i].grp_end = (int)groups; }
+    const dim3 grid((unsigned)((groups + 3) / 4), n_slots);
+    auto go = [&](auto k1, auto k8) { if (n_b == 1) hipLaunchKernelGGL(k1, grid, dim3(256), 0, c.stream, p, n_b); else hipLaunchKernelGGL(k8, grid, dim3(256), 0, c.stream, p, n_b); };
+    switch (qt) {
+      case CAI_Q5_K: go(gemv_raw<CAI_Q5_K, 1>, gemv_raw<CAI_Q5_K, 8>); break;
+      case CAI_Q2_K: go(gemv_raw<CAI_Q2_K, 1>, gemv_raw<CAI_Q2_K, 8>); break;
+      case CAI_Q3_K: go(gemv_raw<CAI_Q3_K, 1>, gemv_raw<CAI_Q3_K, 8>); break;
+      case CAI_Q4_1: go(gemv_raw<CAI_Q4_1, 1>, gemv_raw<CAI_Q4_1, 8>); break;
+      case CAI_Q5_0: go(gemv_raw<CAI_Q5_0, 1>, gemv_raw<CAI_Q5_0, 8>); break;
+      default: go(gemv_raw<CAI_Q5_1, 1>, gemv_raw<CAI_Q5_1, 8>); break;
+    }
+    return CAI_OK;
+  }
   int64_t cum = 0;
   for (int i = 0; i < m.n; i++) { cum += m.rows[i]; p.seg[i].grp_end = (int)cum; }
   const dim3 grid((unsigned)((cum + 3) / 4), n_slots);
   if (qt == CAI_F32) hipLaunchKernelGGL(gemv_simple<CAI_F32>, grid, dim3(256), 0, c.stream, p, n_b);
   else if (qt == CAI_F16) hipLaunchKernelGGL(gemv_simple<CAI_F16>, grid, dim3(256), 0, c.stream, p, n_b);
   else if (qt == CAI_I8ROW) hipLaunchKernelGGL(gemv_simple<CAI_I8ROW>, grid, dim3(256), 0, c.stream, p, n_b);
-  else if (qt == CAI_Q5_K) hipLaunchKernelGGL(gemv_raw<CAI_Q5_K>, grid, dim3(256), 0, c.stream, p, n_b);
-  else if (qt == CAI_Q2_K) hipLaunchKernelGGL(gemv_raw<CAI_Q2_K>, grid, dim3(256), 0, c.stream, p, n_b);
-  else if (qt == CAI_Q3_K) hipLaunchKernelGGL(gemv_raw<CAI_Q3_K>, grid, dim3(256), 0, c.stream, p, n_b);
-  else if (qt == CAI_Q4_1) hipLaunchKernelGGL(gemv_raw<CAI_Q4_1>, grid, dim3(256), 0, c.stream, p, n_b);
-  else if (qt == CAI_Q5_0) hipLaunchKernelGGL(gemv_raw<CAI_Q5_0>, grid, dim3(256), 0, c.stream, p, n_b);
-  else if (qt == CAI_Q5_1) hipLaunchKernelGGL(gemv_raw<CAI_Q5_1>, grid, dim3(256), 0, c.stream, p, n_b);
   else return set_error(CAI_ERR_UNSUPPORTED, "gemv: weight type %d", qt);
   return CAI_OK;
 }

@@ -60,6 +60,8 @@ __device__ __forceinline__ half8_b codes8(uint32_t w0, uint32_t w1, int high)
   return half8_b{h0.x, h0.y, h1.x, h1.y, h2.x, h2.y, h3.x, h3.y};
 }
 
+}  // namespace
+
 template <int QT, int TT, int RT>
 __global__ __launch_bounds__(256, 2) void gemm_blk_pf(const BlkGemmParams p)
 {
@@ -264,6 +266,8 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t* expert, 
     perm[off[e] + atomicAdd(&cur[e], 1)] = s;
   }
 }
+
+namespace {
 
 template <int QT>
 int launch_blk(const BlkGemmParams& p0, int n_tiles_grouped)

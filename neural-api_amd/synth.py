@@ -114,6 +114,22 @@ def random_qweight(qtype, rows, cols, gen, std=0.02, bias=False, chunk_rows=3276
     return w, (raw if keep_bytes else None), b
 
 
+# the block types kept as the stored stream: (elements, bytes, offsets of the f16 fields) per block
+RAW_BLOCKS = {cai.Q4_1: (32, 20, (0, 2)), cai.Q5_0: (32, 22, (0,)), cai.Q5_1: (32, 24, (0, 2)),
+              cai.Q2_K: (256, 84, (80, 82)), cai.Q3_K: (256, 110, (108,)), cai.Q5_K: (256, 176, (0, 2))}
+
+
+def random_raw_qweight(qtype, rows, cols, gen):
+    """Resident matrix of a stored-stream block type for timing: random code / scale bytes (every pattern is a valid block),
+    the f16 fields set to a small positive half so that the values stay finite."""
+    be, bb, halfs = RAW_BLOCKS[qtype]
+    raw = torch.randint(0, 256, (rows * (cols // be), bb), device="cuda", dtype=torch.uint8, generator=gen)
+    for h in halfs:
+        raw[:, h] = 0x66; raw[:, h + 1] = 0x10
+    torch.cuda.synchronize()
+    return cai.QWeight(qtype, rows, cols, raw.data_ptr())
+
+
 def random_int8_rows(rows, cols, gen, scale=1e-3):
     """Resident random matrix in the reference's per-row int8 format (codes in [-127, 127], one float scale per row)."""
     codes = torch.randint(-127, 128, (rows, cols), device="cuda", dtype=torch.int8, generator=gen)
