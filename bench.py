@@ -216,6 +216,30 @@ def gemv_sweep(cai, synth, torch, with_cpu):
             torch.cuda.empty_cache()
 
 
+def gemm_sweep(cai, synth, torch):
+    """One JSON line per (type, shape, tokens): the prompt product cai_qgemm with device pointers (activation pre-pass + matrix-core
+    kernel: gemm_q4k_pf / gemm_q6k_pf / gemm_blk_pf), HIP-event time per call over 10 calls."""
+    lib = cai.load()
+    gen = torch.Generator(device="cuda"); gen.manual_seed(424242)
+    for name, qt in (("Q8_0", cai.Q8_0), ("Q4_0", cai.Q4_0), ("Q4_K", cai.Q4_K), ("Q6_K", cai.Q6_K)):
+        for rows, cols in ((37888, 3584), (3584, 18944), (4608, 3584), (2048, 2048)):
+            w = synth.random_qweight(qt, rows, cols, gen)[0]
+            for T in (64, 256, 511, 2048):
+                x = torch.randn(T, cols, device="cuda"); y = torch.empty(T, rows, device="cuda")
+                torch.cuda.synchronize()
+                for _ in range(2):
+                    cai.check(lib.cai_qgemm(w.h, x.data_ptr(), T, y.data_ptr(), cai.X_DEVICE | cai.Y_DEVICE))
+                cai.check(lib.cai_sync()); cai.check(lib.cai_timer_start())
+                for _ in range(10):
+                    cai.check(lib.cai_qgemm(w.h, x.data_ptr(), T, y.data_ptr(), cai.X_DEVICE | cai.Y_DEVICE))
+                ms = C.c_float(); cai.check(lib.cai_timer_stop(C.byref(ms)))
+                us = ms.value * 1e3 / 10
+                print(json.dumps({"gemm": name, "rows": rows, "cols": cols, "tokens": T, "us_per_call": round(us, 1),
+                                  "useful_TFLOP_per_s": round(2.0 * rows * cols * T / us / 1e6, 1), "frac_of_f16_peak": round(2.0 * rows * cols * T / us / 1e6 / 2500.0, 4)}), flush=True)
+            w.close()
+            torch.cuda.empty_cache()
+
+
 # HBM bytes per launch of the 7B-shape gate|up kernel from hardware counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000
 # KiB, factors from a 1 GiB copy kernel): profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt.  Not measurable from
 # inside this process; re-collect when the kernel changes.
@@ -235,6 +259,7 @@ def main():
     ap.add_argument("--kv", choices=["f32", "f16", "i8"], default=None, help="KV cache element type (default: the configuration's own)")
     ap.add_argument("--batch", type=int, default=1, help="independent sequences decoded together (1..8)")
     ap.add_argument("--gemv-sweep", action="store_true", help="isolated matrix-vector sweep (BASELINE configs[1]): Q8_0 / Q4_0 / Q4_K / Q6_K and per-row int8 on five shapes, the stored-stream types on the two large ones, batch 1 and 4")
+    ap.add_argument("--gemm-sweep", action="store_true", help="isolated prompt-product sweep: Q8_0 / Q4_0 / Q4_K / Q6_K, four shapes, 64..2048 tokens (cai_qgemm, device pointers)")
     ap.add_argument("--copy-calibration", action="store_true", help="only run the 1 GiB device copy kernel 5 times (reference for traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -259,6 +284,9 @@ def main():
         return
     if args.gemv_sweep:
         gemv_sweep(cai, synth, torch, not args.no_cpu_baseline)
+        return
+    if args.gemm_sweep:
+        gemm_sweep(cai, synth, torch)
         return
     conf = CONFIGS[args.config]
     cfg = dict(conf["cfg"])
