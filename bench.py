@@ -22,6 +22,9 @@ CONFIGS = {
     "qwen2.5-7b-q4k": dict(cfg=dict(n_layers=28, d_model=3584, n_q_heads=28, n_kv_heads=4, head_dim=128, ffn=18944, vocab=152064,
                                     max_ctx=768, eps=1e-6, rope_theta=1e6), qtype="Q4_K", head="Q8_0", bias=True, prompt=512),
     # the same shape as llama.cpp's Q4_K_M preset writes it: output.weight and attn_v / ffn_down of about half the blocks in Q6_K
+    # the same shape in the Q5_K_M mix (Q5_K body; Q6_K where Q4_K_M has it)
+    "qwen2.5-7b-q5_k_m": dict(cfg=dict(n_layers=28, d_model=3584, n_q_heads=28, n_kv_heads=4, head_dim=128, ffn=18944, vocab=152064,
+                                       max_ctx=768, eps=1e-6, rope_theta=1e6), qtype="Q5_K", head="Q6_K", embed="Q5_K", q6k_mix=True, bias=True, prompt=512),
     "qwen2.5-7b-q4_k_m": dict(cfg=dict(n_layers=28, d_model=3584, n_q_heads=28, n_kv_heads=4, head_dim=128, ffn=18944, vocab=152064,
                                        max_ctx=768, eps=1e-6, rope_theta=1e6), qtype="Q4_K", head="Q6_K", embed="Q4_K", q6k_mix=True, bias=True, prompt=512),
     # BASELINE.json configs[0] (the reference's own CPU-runnable case): SmolLM2-135M shape, Q8_0, tied head
@@ -221,7 +224,7 @@ def gemm_sweep(cai, synth, torch):
     kernel: gemm_q4k_pf / gemm_q6k_pf / gemm_blk_pf), HIP-event time per call over 10 calls."""
     lib = cai.load()
     gen = torch.Generator(device="cuda"); gen.manual_seed(424242)
-    for name, qt in (("Q8_0", cai.Q8_0), ("Q4_0", cai.Q4_0), ("Q4_K", cai.Q4_K), ("Q6_K", cai.Q6_K)):
+    for name, qt in (("Q8_0", cai.Q8_0), ("Q4_0", cai.Q4_0), ("Q4_K", cai.Q4_K), ("Q5_K", cai.Q5_K), ("Q6_K", cai.Q6_K)):
         for rows, cols in ((37888, 3584), (3584, 18944), (4608, 3584), (2048, 2048)):
             w = synth.random_qweight(qt, rows, cols, gen)[0]
             for T in (64, 256, 511, 2048):
@@ -259,7 +262,7 @@ def main():
     ap.add_argument("--kv", choices=["f32", "f16", "i8"], default=None, help="KV cache element type (default: the configuration's own)")
     ap.add_argument("--batch", type=int, default=1, help="independent sequences decoded together (1..8)")
     ap.add_argument("--gemv-sweep", action="store_true", help="isolated matrix-vector sweep (BASELINE configs[1]): Q8_0 / Q4_0 / Q4_K / Q6_K and per-row int8 on five shapes, the stored-stream types on the two large ones, batch 1 and 4")
-    ap.add_argument("--gemm-sweep", action="store_true", help="isolated prompt-product sweep: Q8_0 / Q4_0 / Q4_K / Q6_K, four shapes, 64..2048 tokens (cai_qgemm, device pointers)")
+    ap.add_argument("--gemm-sweep", action="store_true", help="isolated prompt-product sweep: Q8_0 / Q4_0 / Q4_K / Q5_K / Q6_K, four shapes, 64..2048 tokens (cai_qgemm, device pointers)")
     ap.add_argument("--copy-calibration", action="store_true", help="only run the 1 GiB device copy kernel 5 times (reference for traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -294,7 +297,7 @@ def main():
     K, W = args.steps, args.warmup
     if prompt_len + W + K > cfg["max_ctx"]:
         cfg["max_ctx"] = prompt_len + W + K
-    QT = {"Q4_K": cai.Q4_K, "Q8_0": cai.Q8_0, "Q4_0": cai.Q4_0, "Q6_K": cai.Q6_K}
+    QT = {"Q4_K": cai.Q4_K, "Q5_K": cai.Q5_K, "Q8_0": cai.Q8_0, "Q4_0": cai.Q4_0, "Q6_K": cai.Q6_K}
     t0 = time.time()
     spec = synth.random_decoder_spec(cfg, QT[conf["qtype"]], QT[conf["head"]], seed=424242, qkv_bias=conf["bias"],
                                      embed_qtype=QT[conf["embed"]] if "embed" in conf else None, q6k_mix=conf.get("q6k_mix", False))
@@ -365,7 +368,7 @@ def main():
         return
     d, I, V = cfg["d_model"], cfg["ffn"], cfg["vocab"]
     qw_, kw_ = cfg["n_q_heads"] * cfg["head_dim"], cfg["n_kv_heads"] * cfg["head_dim"]
-    bpw = {"Q4_K": 144 / 256, "Q8_0": 34 / 32, "Q4_0": 18 / 32, "Q6_K": 210 / 256}
+    bpw = {"Q4_K": 144 / 256, "Q5_K": 176 / 256, "Q8_0": 34 / 32, "Q4_0": 18 / 32, "Q6_K": 210 / 256}
     qbytes = bpw[conf["qtype"]]
     k_bytes = 2 * I * d * qbytes + 4 * d * 2 + 4 * I     # blocks + x + gain + y
     # ---- every kernel class of the step, timed in place: the production launches of one class over all blocks, back to
@@ -435,7 +438,7 @@ def main():
                                "tok_per_s": round((prompt_len - 1) / max(pf_ms.value, 1e-6) * 1e3, 1),
                                "linear_tflops": round(2.0 * n_lin_weights * (prompt_len - 1) / max(pf_ms.value, 1e-6) / 1e9, 1),
                                "note": "multi-token ingestion: f16 MFMA (exact scale*nibble weight operand, hi/lo-split activations = 2 MFMA passes per useful FLOP) + prompt attention; MFMA f16 dense peak 2500 TFLOP/s"}},
-        "roofline": {"bound": "hbm", "kernel": "%s (RMSNorm+gate|up+SwiGLU, %dx%d)" % ("gemv_q4k_dot<1,1,false,2>" if conf["qtype"] == "Q4_K" else "gemv_fast<%s>" % conf["qtype"], 2 * I, d),
+        "roofline": {"bound": "hbm", "kernel": "%s (RMSNorm+gate|up+SwiGLU, %dx%d)" % ("gemv_q4k_dot<1,1,false,2>" if conf["qtype"] == "Q4_K" else "gemv_q5k_dot<1,1,false,2>" if conf["qtype"] == "Q5_K" else "gemv_fast<%s>" % conf["qtype"], 2 * I, d),
                      "achieved": round(k_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(k_gbs / HBM_PEAK_GBS, 4),
                      "avg_launch_us": round(k_avg_us, 2), "algorithmic_bytes_per_launch": int(k_bytes),
                      "traffic": GATEUP_TRAFFIC_BYTES if args.config == "qwen2.5-7b-q4k" else None, "traffic_unit": "bytes/launch",

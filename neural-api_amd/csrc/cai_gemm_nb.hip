@@ -72,8 +72,12 @@ __device__ __forceinline__ half8_t nibbles_times_scale(uint32_t lo, uint32_t hi,
 // the 16 x 16 result has rows 4 kg .. 4 kg + 3 of column m in this lane.  Here a tile is 32 weight rows = two row sets,
 // the 16 columns are 8 tokens x {hi, lo}, and lane kg owns quant bytes 32 kg .. 32 kg + 31 of a super-block: sub-block
 // 2 kg in the low nibbles (k steps 0..3), sub-block 2 kg + 1 in the high nibbles (steps 4..7).
+// QT = CAI_Q5_K: the same walk over 176-byte super-blocks (neural/neuralgguf.pas:516-587): header as Q4_K, then the 32-byte plane of
+// fifth bits (bit j of byte i belongs to weight i of sub-block j), then the nibbles; sc * (nibble | bit << 4) <= 63 * 31 stays exact in f16.
+template <int QT>
 __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
 {
+  constexpr int BB = QT == CAI_Q5_K ? 176 : 144, QOFF = QT == CAI_Q5_K ? 48 : 16;
   extern __shared__ __align__(16) unsigned char nb_smem[];
   const int S = p.sb_per_slice;
   _Float16* xs = reinterpret_cast<_Float16*>(nb_smem);              // [S][16][NB_LDX]
@@ -84,12 +88,12 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
   const int n = lane & 15, kg = lane >> 4;
   const int K = p.cols, nsb = K >> 8, nb32 = K >> 5;
   const int slice = blockIdx.y, sb0 = slice * S, nS = min(S, nsb - sb0);
-  const int64_t row_bytes = (int64_t)nsb * 144;
+  const int64_t row_bytes = (int64_t)nsb * BB;
   const int tile0 = blockIdx.x * 4 + wave;
   const int n_it = tile0 < p.n_tiles ? (p.n_tiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
   const int nq = n_it * nS;                      // (tile, super-block) items of this wave
 
-  struct WRegs { uint4 h[2], q[2][2]; };
+  struct WRegs { uint4 h[2], q[2][2], e[QT == CAI_Q5_K ? 2 : 1][2]; };   // e: Q5_K's bit plane (all 32 bytes: every lane needs its two bits of each)
   auto locate = [&](int tile, const NbSeg*& sg, int& R0) {
     int sgi = 0, t0 = 0;
     if (p.n_seg > 1 && tile >= p.seg[0].tile_end) { sgi = 1; t0 = p.seg[0].tile_end; }
@@ -105,10 +109,11 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
     const NbSeg* sg; int R0; locate(tile, sg, R0);
 #pragma unroll
     for (int hh = 0; hh < 2; hh++) {
-      const uint8_t* blk = sg->w + (int64_t)min(R0 + 16 * hh + n, sg->rows - 1) * row_bytes + (int64_t)sb * 144;   // tail rows: re-read the last row
+      const uint8_t* blk = sg->w + (int64_t)min(R0 + 16 * hh + n, sg->rows - 1) * row_bytes + (int64_t)sb * BB;   // tail rows: re-read the last row
       r.h[hh] = *reinterpret_cast<const uint4*>(blk);
-      r.q[hh][0] = *reinterpret_cast<const uint4*>(blk + 16 + 32 * kg);
-      r.q[hh][1] = *reinterpret_cast<const uint4*>(blk + 32 + 32 * kg);
+      r.q[hh][0] = *reinterpret_cast<const uint4*>(blk + QOFF + 32 * kg);
+      r.q[hh][1] = *reinterpret_cast<const uint4*>(blk + QOFF + 16 + 32 * kg);
+      if constexpr (QT == CAI_Q5_K) { r.e[hh][0] = *reinterpret_cast<const uint4*>(blk + 16); r.e[hh][1] = *reinterpret_cast<const uint4*>(blk + 32); }
     }
   };
   WRegs wa, wb, wc;
@@ -195,8 +200,14 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
       for (int hh = 0; hh < 2; hh++) {
         const uint4& qq = r.q[hh][(t & 3) >> 1];
         const uint32_t d0 = (t & 1) ? qq.z : qq.x, d1 = (t & 1) ? qq.w : qq.y;       // bytes 8 (t & 3) .. + 7
-        const uint32_t lo = (t < 4) ? (d0 & 0x0f0f0f0fu) : ((d0 >> 4) & 0x0f0f0f0fu);
-        const uint32_t hi = (t < 4) ? (d1 & 0x0f0f0f0fu) : ((d1 >> 4) & 0x0f0f0f0fu);
+        uint32_t lo = (t < 4) ? (d0 & 0x0f0f0f0fu) : ((d0 >> 4) & 0x0f0f0f0fu);
+        uint32_t hi = (t < 4) ? (d1 & 0x0f0f0f0fu) : ((d1 >> 4) & 0x0f0f0f0fu);
+        if constexpr (QT == CAI_Q5_K) {   // plane bytes 8 (t & 3) .. + 7, bit 2 kg (low nibbles' sub-block) or 2 kg + 1
+          const uint4& ee = r.e[hh][(t & 3) >> 1];
+          const uint32_t e0 = (t & 1) ? ee.z : ee.x, e1 = (t & 1) ? ee.w : ee.y;
+          const int bit = 2 * kg + (t >> 2);
+          lo |= ((e0 >> bit) & 0x01010101u) << 4; hi |= ((e1 >> bit) & 0x01010101u) << 4;
+        }
         const half8_t A = nibbles_times_scale(lo, hi, s2[hh][t >> 2], c2[hh][t >> 2]);
         C[hh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, C[hh], 0, 0, 0);
       }
@@ -881,7 +892,7 @@ int nb_prep_swiglu(int half, int n_tok)
 // Weight types with a small-batch kernel.  Q4_K super-blocks make the width a multiple of 256 by construction.
 bool nb_supported(const cai_qw_s* w)
 {
-  if (w->qtype == CAI_Q4_K || w->qtype == CAI_Q6_K) return w->cols % 256 == 0 && w->cols >= 256;
+  if (w->qtype == CAI_Q4_K || w->qtype == CAI_Q5_K || w->qtype == CAI_Q6_K) return w->cols % 256 == 0 && w->cols >= 256;
   return (w->qtype == CAI_Q8_0 || w->qtype == CAI_Q4_0 || w->qtype == CAI_I8ROW) && w->cols % 32 == 0 && w->cols >= 32;   // per-row int8: unit block scales, the row scale is applied by nb_reduce
 }
 
@@ -934,9 +945,9 @@ int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok)
     p.n_tiles = sub;
     const int gxs = std::max(1, std::min(gx, (sub + 3) / 4));
     p.tile_stride = gxs * 4;
-    if (qt == CAI_Q4_K) {
+    if (qt == CAI_Q4_K || qt == CAI_Q5_K) {
       const size_t lds = (size_t)S * NB_SC * (NB_LDX + 8) * 2 + (size_t)S * NB_TK * 4 + 4 * 2 * 32 * 4;
-      nb_launch<gemm_q4k_nb>(p, gxs, n_slices, lds);
+      if (qt == CAI_Q4_K) nb_launch<gemm_q4k_nb<CAI_Q4_K>>(p, gxs, n_slices, lds); else nb_launch<gemm_q4k_nb<CAI_Q5_K>>(p, gxs, n_slices, lds);
     } else {
       const size_t lds = (size_t)S * NB_SC * NB_LDX * 2 + (size_t)S * NB_TK * 4;
       const bool tail = p.cols % 256 != 0;

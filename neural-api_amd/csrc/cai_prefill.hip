@@ -113,9 +113,12 @@ typedef _Float16 half8_pf __attribute__((ext_vector_type(8)));
 // per FLOP); it needs 256 rows per work-group and is used for matrices with enough row groups to fill the chip.
 // Work-group ids are laid out so that the token tiles of one row group run on one XCD: the re-reads of its weights (one
 // per token tile) hit that XCD's L2.  TT = 1 doubles the number of work-groups for matrices with few row groups.
-template <int TT, int RT>
+// QT = CAI_Q5_K: 176-byte super-blocks (neural/neuralgguf.pas:516-587) - the Q4_K header, the 32-byte plane of fifth bits (bit j of byte i
+// belongs to weight i of sub-block j), the nibbles; the weight operand sc * (nibble | bit << 4) <= 63 * 31 stays exact in f16.
+template <int TT, int RT, int QT>
 __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
 {
+  constexpr int BB = QT == CAI_Q5_K ? 176 : 144, QOFF = QT == CAI_Q5_K ? 48 : 16;
   extern __shared__ __align__(16) unsigned char pf_smem[];
   constexpr int NTOK = TT * 32;
   _Float16* xs_hi = reinterpret_cast<_Float16*>(pf_smem);            // [NTOK][PF_LDX]
@@ -130,20 +133,21 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
   if (rg >= p.n_row_groups) return;
   const int R0 = (rg * 4 + wave) * 32 * RT, T0 = ttile * NTOK;
   const int K = p.cols, nsb = K >> 8, nb32 = K >> 5;
-  const int64_t row_bytes = (int64_t)nsb * 144;
+  const int64_t row_bytes = (int64_t)nsb * BB;
   const uint8_t* wrow[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; rt++) wrow[rt] = p.w + (int64_t)min(R0 + 32 * rt + n, p.rows - 1) * row_bytes;   // tail rows: re-read the last row, not written
 
-  struct WRegs { uint4 h, q[4]; };
+  struct WRegs { uint4 h, q[4], e[QT == CAI_Q5_K ? 2 : 1]; };   // e: Q5_K's bit plane (all 32 bytes: the lane needs four bits of each)
   auto load_w = [&](int sb, WRegs (&r)[RT]) {
     if (sb < nsb) {
 #pragma unroll
       for (int rt = 0; rt < RT; rt++) {
-        const uint8_t* blk = wrow[rt] + (int64_t)sb * 144;
+        const uint8_t* blk = wrow[rt] + (int64_t)sb * BB;
         r[rt].h = *reinterpret_cast<const uint4*>(blk);
+        if constexpr (QT == CAI_Q5_K) { r[rt].e[0] = *reinterpret_cast<const uint4*>(blk + 16); r[rt].e[1] = *reinterpret_cast<const uint4*>(blk + 32); }
 #pragma unroll
-        for (int i = 0; i < 4; i++) r[rt].q[i] = *reinterpret_cast<const uint4*>(blk + 16 + 64 * kg + 16 * i);
+        for (int i = 0; i < 4; i++) r[rt].q[i] = *reinterpret_cast<const uint4*>(blk + QOFF + 64 * kg + 16 * i);
       }
     }
   };
@@ -217,8 +221,13 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
         for (int t = 0; t < 4; t++) {                                    // weights 8t .. 8t+7 of the sub-block
           const uint4& qq = r.q[2 * ccl + (t >> 1)];
           const uint32_t qa = (t & 1) ? qq.z : qq.x, qb = (t & 1) ? qq.w : qq.y;
-          const uint32_t na = hl ? ((qa >> 4) & 0x0f0f0f0fu) : (qa & 0x0f0f0f0fu);
-          const uint32_t nb = hl ? ((qb >> 4) & 0x0f0f0f0fu) : (qb & 0x0f0f0f0fu);
+          uint32_t na = hl ? ((qa >> 4) & 0x0f0f0f0fu) : (qa & 0x0f0f0f0fu);
+          uint32_t nb = hl ? ((qb >> 4) & 0x0f0f0f0fu) : (qb & 0x0f0f0f0fu);
+          if constexpr (QT == CAI_Q5_K) {   // plane bytes 8 t .. 8 t + 7, bit 4 kg + j
+            const uint4& ee = r.e[t >> 1];
+            const uint32_t e0 = (t & 1) ? ee.z : ee.x, e1 = (t & 1) ? ee.w : ee.y;
+            na |= ((e0 >> (4 * kg + j)) & 0x01010101u) << 4; nb |= ((e1 >> (4 * kg + j)) & 0x01010101u) << 4;
+          }
           const half2_t a0 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, na, 0x04010400u)), s2, c2);   // (1024 + q) * sc - 1024 * sc = sc * q
           const half2_t a1 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, na, 0x04030402u)), s2, c2);
           const half2_t a2 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, nb, 0x04010400u)), s2, c2);
@@ -465,7 +474,7 @@ int launch_xprep(const float* x, int64_t x_stride, const float* gain, float eps,
   return CAI_OK;
 }
 
-bool gemm_mfma_supported(const cai_qw_s* w) { return (w->qtype == CAI_Q4_K || w->qtype == CAI_Q6_K) && w->cols % 256 == 0; }
+bool gemm_mfma_supported(const cai_qw_s* w) { return (w->qtype == CAI_Q4_K || w->qtype == CAI_Q5_K || w->qtype == CAI_Q6_K) && w->cols % 256 == 0; }
 
 int launch_gemm_q4k(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo, const _Float16* sxhi, const _Float16* sxlo, const float* sinv,
                     int n_tok, float* y, int64_t y_stride, const float* residual)
@@ -504,14 +513,19 @@ int launch_gemm_q4k(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo,
   const size_t lds = (size_t)tt * 32 * (PF_LDX + 8) * 2 * 2 + (size_t)4 * rt * 2 * 32 * 4;
   static bool attr_done = false;
   if (!attr_done) {
-    const void* ks[3] = {(const void*)gemm_q4k_pf<1, 1>, (const void*)gemm_q4k_pf<2, 1>, (const void*)gemm_q4k_pf<1, 2>};
+    const void* ks[6] = {(const void*)gemm_q4k_pf<1, 1, CAI_Q4_K>, (const void*)gemm_q4k_pf<2, 1, CAI_Q4_K>, (const void*)gemm_q4k_pf<1, 2, CAI_Q4_K>,
+                         (const void*)gemm_q4k_pf<1, 1, CAI_Q5_K>, (const void*)gemm_q4k_pf<2, 1, CAI_Q5_K>, (const void*)gemm_q4k_pf<1, 2, CAI_Q5_K>};
     for (const void* k : ks) if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) != hipSuccess) (void)hipGetLastError();
     attr_done = true;
   }
   const int grid = 8 * p.n_tok_tiles * ((p.n_row_groups + 7) / 8);
-  if (mode == 3) hipLaunchKernelGGL((gemm_q4k_pf<1, 2>), dim3(grid), dim3(256), lds, ctx().stream, p);
-  else if (mode == 1) hipLaunchKernelGGL((gemm_q4k_pf<1, 1>), dim3(grid), dim3(256), lds, ctx().stream, p);
-  else hipLaunchKernelGGL((gemm_q4k_pf<2, 1>), dim3(grid), dim3(256), lds, ctx().stream, p);
+  if (w->qtype == CAI_Q5_K) {
+    if (mode == 3) hipLaunchKernelGGL((gemm_q4k_pf<1, 2, CAI_Q5_K>), dim3(grid), dim3(256), lds, ctx().stream, p);
+    else if (mode == 1) hipLaunchKernelGGL((gemm_q4k_pf<1, 1, CAI_Q5_K>), dim3(grid), dim3(256), lds, ctx().stream, p);
+    else hipLaunchKernelGGL((gemm_q4k_pf<2, 1, CAI_Q5_K>), dim3(grid), dim3(256), lds, ctx().stream, p);
+  } else if (mode == 3) hipLaunchKernelGGL((gemm_q4k_pf<1, 2, CAI_Q4_K>), dim3(grid), dim3(256), lds, ctx().stream, p);
+  else if (mode == 1) hipLaunchKernelGGL((gemm_q4k_pf<1, 1, CAI_Q4_K>), dim3(grid), dim3(256), lds, ctx().stream, p);
+  else hipLaunchKernelGGL((gemm_q4k_pf<2, 1, CAI_Q4_K>), dim3(grid), dim3(256), lds, ctx().stream, p);
   return CAI_OK;
 }
 

@@ -71,6 +71,38 @@ def pack_q4_k(x):
     return out
 
 
+def pack_q5_k(x):
+    """x: [rows, cols] float32 (cols % 256 == 0) -> uint8 [rows, cols/256, 176]: the affine fit of pack_q4_k with 32 levels; the
+    fifth bit of weight i of sub-block j is bit j of plane byte i (layout of neural/neuralgguf.pas:516-587)"""
+    rows, cols = x.shape
+    nsb = cols // 256
+    xb = x.view(rows, nsb, 8, 32)
+    lo = xb.amin(-1).clamp(max=0.0)
+    hi = torch.maximum(xb.amax(-1), lo)
+    step = (hi - lo) / 31.0
+    d16 = (step.amax(-1) / 63.0).to(torch.float16)
+    m16 = ((-lo).amax(-1) / 63.0).to(torch.float16)
+    d = d16.float()[..., None]; dm = m16.float()[..., None]
+    sc = torch.where(d > 0, torch.round(step / d), torch.zeros_like(step)).clamp_(0, 63)
+    mn = torch.where(dm > 0, torch.round(-lo / dm), torch.zeros_like(lo)).clamp_(0, 63)
+    ds = (d * sc)[..., None]; off = (dm * mn)[..., None]
+    q = torch.where(ds > 0, torch.round((xb + off) / ds), torch.zeros_like(xb)).clamp_(0, 31).to(torch.uint8)
+    sc = sc.to(torch.uint8); mn = mn.to(torch.uint8)
+    out = torch.empty(rows, nsb, 176, dtype=torch.uint8, device=x.device)
+    out[..., 0:2] = d16.view(torch.uint8).view(rows, nsb, 2)
+    out[..., 2:4] = m16.view(torch.uint8).view(rows, nsb, 2)
+    out[..., 4:8] = (sc[..., :4] & 63) | ((sc[..., 4:] >> 4) << 6)
+    out[..., 8:12] = (mn[..., :4] & 63) | ((mn[..., 4:] >> 4) << 6)
+    out[..., 12:16] = (sc[..., 4:] & 15) | ((mn[..., 4:] & 15) << 4)
+    plane = torch.zeros(rows, nsb, 32, dtype=torch.uint8, device=x.device)
+    for j in range(8):
+        plane |= (q[..., j, :] >> 4) << j
+    out[..., 16:48] = plane
+    qs = (q & 15).view(rows, nsb, 4, 2, 32)
+    out[..., 48:] = (qs[..., 0, :] | (qs[..., 1, :] << 4)).reshape(rows, nsb, 128)
+    return out
+
+
 def pack_q6_k(x):
     """x: [rows, cols] float32 (cols % 256 == 0) -> uint8 [rows, cols/256, 210]: symmetric fit, one signed scale per 16
     weights, codes q in 0..63 standing for q - 32 (layout of neural/neuralgguf.pas:639-717)"""
@@ -94,7 +126,7 @@ def pack_q6_k(x):
     return out
 
 
-PACKERS = {cai.Q8_0: pack_q8_0, cai.Q4_0: pack_q4_0, cai.Q4_K: pack_q4_k, cai.Q6_K: pack_q6_k}
+PACKERS = {cai.Q8_0: pack_q8_0, cai.Q4_0: pack_q4_0, cai.Q4_K: pack_q4_k, cai.Q5_K: pack_q5_k, cai.Q6_K: pack_q6_k}
 
 
 def random_qweight(qtype, rows, cols, gen, std=0.02, bias=False, chunk_rows=32768, keep_bytes=False):

@@ -186,3 +186,65 @@ def test_q5_k_fused_feed_forward_front_half(rows, cols):
         L.orc_swiglu(C.c_void_p(ug.ctypes.data), rows // 2, C.c_void_p(want.ctypes.data))
         assert rel_err(w.ffn_gateup(x, g, 1e-6)[0], want) < TIGHT
     w.close()
+
+
+@pytest.mark.parametrize("rows,cols,T", [(128, 256, 2), (33, 512, 3), (1000, 1024, 8), (3584, 3584, 8), (512, 18944, 4), (5000, 768, 13),
+                                         (1000, 1024, 40), (3584, 3584, 77), (512, 18944, 33), (130, 512, 64), (4099, 256, 129), (9000, 2048, 300)])
+def test_q5_k_on_the_matrix_cores(rows, cols, T):
+    """Q5_K through the small-batch kernel (up to 16 tokens) and the prompt kernel (more): the Q4_K walks with the fifth-bit plane
+    merged into the codes, sc * (nibble | bit << 4) exact in f16; == T single-token layers of the oracle, bias included."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    rng = np.random.default_rng(rows + cols + T)
+    raw = O.quantize(O.Q5_K, (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32))
+    x = (rng.standard_normal((T, cols)) * rng.uniform(0.01, 30.0, (T, 1))).astype(np.float32)
+    x[0, : cols // 2] = 0.0
+    bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
+    w = cai.QWeight(O.Q5_K, rows, cols, raw, bias)
+    got = w.gemm(x, matrix_cores=True)
+    want = O.gemv(O.Q5_K, raw, rows, cols, x, bias, 0, 1)
+    for t in range(T):
+        assert rel_err(got[t], want[t], floor=0.02 * cols ** 0.5 * float(np.abs(x[t]).mean())) < TIGHT, t
+    w.close()
+
+
+def test_q5_k_largest_codes_and_scales_on_the_matrix_cores():
+    """Every code 31 and every scale 63 (the f16 weight operand at its largest, 1953) on both matrix-core kernels."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    rows, cols = 96, 1024
+    blk = np.full(176, 0xff, np.uint8)
+    blk[0:2] = np.array([np.float16(0.01)]).view(np.uint8); blk[2:4] = np.array([np.float16(0.02)]).view(np.uint8)
+    raw = np.tile(blk, rows * cols // 256)
+    w = cai.QWeight(O.Q5_K, rows, cols, raw)
+    rng = np.random.default_rng(3)
+    for T in (5, 40):
+        x = rng.standard_normal((T, cols)).astype(np.float32)
+        assert rel_err(w.gemm(x, matrix_cores=True), O.gemv(O.Q5_K, raw, rows, cols, x, None, 0, 1)) < TIGHT
+    w.close()
+
+
+def test_q5_k_m_like_decoder_long_prompt_and_batched_generation():
+    """A 45-token prompt (prompt kernels for Q5_K and Q6_K) == token-at-a-time steps == the oracle; then a batch of 3 sequences
+    decodes (small-batch kernels) like the single sequence."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    cfg = dict(n_layers=2, d_model=512, n_q_heads=8, n_kv_heads=2, head_dim=64, ffn=1024, vocab=600, max_ctx=96, eps=1e-5, rope_theta=1e4)
+    spec = q5_k_m_spec(cfg, 31)
+    om = oracle_model(spec, acc64=1)
+    dec = cai.Decoder(spec, max_batch=3)
+    rng = np.random.default_rng(9)
+    prompt = [int(t) for t in rng.integers(0, cfg["vocab"], 45)]
+    lo = None
+    for p, t in enumerate(prompt):
+        _, lo = om.step(t, p)
+    for b in range(3):
+        am, lg = dec.prefill(prompt, 0, seq=b)
+        assert rel_err(lg, lo) < TOL and am == int(np.argmax(lo))
+    tok = np.full(3, am)
+    for i in range(6):
+        n_o, lo = om.step(int(tok[0]), len(prompt) + i)
+        tok, lg = dec.step(tok, np.full(3, len(prompt) + i))
+        for b in range(3):
+            assert rel_err(lg[b], lo) < TOL and int(tok[b]) == n_o
+    dec.close()
