@@ -247,7 +247,8 @@ def gemm_sweep(cai, synth, torch):
 # KiB, factors from a 1 GiB copy kernel): profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt.  Not measurable from
 # inside this process; re-collect when the kernel changes.
 GATEUP_TRAFFIC_BYTES = int((37513.6 * 2.000 + 74.5 * 1.000) * 1024)
-GATEUP_TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of gemv_q4k_dot<1,1,false,2>, profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt"
+GATEUP_TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of gemv_q4k_dot<1,1,false,2>, profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt; "
+                         "collected with the tree at commit e3181a8 (cai_gemv_dot.hip last changed in 77da839)")
 
 
 def main():

@@ -794,6 +794,16 @@ const float* g_pending_ssq = nullptr; int g_pending_K = 0; float g_pending_eps =
 
 int nb_ws_generation() { return g_nb.generation; }
 
+// cai_shutdown: the workspace goes back to the device; decoders that captured graphs against it see a new generation
+void nb_release()
+{
+  void* q[] = {g_nb.hi, g_nb.lo, g_nb.sxhi, g_nb.sxlo, g_nb.sinvb, g_nb.ssq[0], g_nb.ssq[1], g_nb.part};
+  for (void* v : q) if (v) (void)hipFree(v);
+  const int gen = g_nb.generation + 1;
+  g_nb = NbWs(); g_nb.generation = gen;
+  g_prod = NbProduct(); g_pending_ssq = nullptr; g_pending_K = 0;
+}
+
 // Reserves planes for k_max columns and a partial buffer of part_floats floats (never inside a stream capture).
 int nb_reserve(int k_max, size_t part_floats)
 {

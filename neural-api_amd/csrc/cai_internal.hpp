@@ -218,6 +218,8 @@ bool nb_supported(const cai_qw_s* w);          // 2..8-token matrix-core kernel
 // split pre-pass / product form: prep once, then any number of matrices of that width
 // small-batch (<= 8 tokens per pass) matrix-core path: planes <- activations, partials <- product, consumer sums the slices
 int nb_ws_generation();                                        // changes whenever its workspace buffers are reallocated
+void nb_release();                                             // frees the small-batch workspace (cai_shutdown)
+void prefill_release();                                        // frees the prompt workspace (cai_shutdown)
 int nb_reserve(int k_max, size_t part_floats);                 // never inside a stream capture
 int nb_max_slices(int cols);
 int nb_prep_plain(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok);

@@ -556,6 +556,13 @@ static int prefill_reserve(int n_tok, int K)
   return CAI_OK;
 }
 
+void prefill_release()   // cai_shutdown
+{
+  void* q[] = {g_pws.hi, g_pws.lo, g_pws.sinv, g_pws.sxhi, g_pws.sxlo};
+  for (void* v : q) if (v) (void)hipFree(v);
+  g_pws = PrefillWs();
+}
+
 int prefill_prep(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok)
 {
   int rc;

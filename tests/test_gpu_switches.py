@@ -44,3 +44,43 @@ def test_switch_selected_path_matches_the_oracle(var, val):
     code = CHILD % dict(root=ROOT, tests=os.path.join(ROOT, "tests"))
     r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0 and "CHILD_OK" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
+
+
+SHUTDOWN_CHILD = r"""
+import sys, importlib
+import numpy as np
+sys.path.insert(0, %(root)r); sys.path.insert(0, %(tests)r)
+from helpers import oracle_lib as O
+from helpers.model_build import synthetic_spec
+from helpers.device import dev, rel_err
+cai = dev()
+cfg = dict(n_layers=2, d_model=512, n_q_heads=8, n_kv_heads=2, head_dim=64, ffn=1024, vocab=600, max_ctx=96, eps=1e-5, rope_theta=1e4)
+spec = synthetic_spec(cfg, O.Q4_K, head_qtype=O.Q8_0, std=0.05)
+prompt = np.random.default_rng(3).integers(0, cfg["vocab"], 40).tolist()
+
+def session():
+    dec = cai.Decoder(spec, max_batch=3)
+    out = [dec.prefill(prompt, 0, seq=b)[1].copy() for b in range(3)]          # prompt workspace
+    tok = np.full(3, 5)
+    for i in range(4):                                                          # small-batch workspace, captured graph
+        tok, lg = dec.step(tok, np.full(3, len(prompt) + i)); out.append(lg.copy())
+    dec.close()
+    return out
+
+a = session()
+cai.check(cai.load().cai_shutdown())          # frees the stream, the staging buffers and both activation workspaces
+cai.init(0)
+b = session()
+for x, y in zip(a, b):
+    assert np.array_equal(np.asarray(x), np.asarray(y))
+cai.check(cai.load().cai_shutdown())
+print("CHILD_OK")
+"""
+
+
+def test_shutdown_frees_the_workspaces_and_a_second_init_runs_the_same():
+    """cai_shutdown followed by cai_init in one process: the matrix-core paths allocate their activation workspaces afresh and
+    every result is bit-identical to the first session's."""
+    code = SHUTDOWN_CHILD % dict(root=ROOT, tests=os.path.join(ROOT, "tests"))
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "CHILD_OK" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
