@@ -279,10 +279,17 @@ int cai_decoder_set_kv_dtype(cai_decoder_t d, int kv_dtype);
 #define CAI_ROPE_NONE   0
 #define CAI_ROPE_LINEAR 1
 #define CAI_ROPE_LLAMA3 2
+#define CAI_ROPE_NTK    3  /* "dynamic" / "ntk": base * factor^(d/(d-2)) */
+#define CAI_ROPE_YARN   4  /* low_freq_factor = beta_slow (YarnAlpha), high_freq_factor = beta_fast (YarnBeta); sets the output scale 0.1 ln(factor) + 1 */
 int cai_decoder_set_rope_scaling(cai_decoder_t d, int mode, float factor, int original_ctx, float low_freq_factor, float high_freq_factor);
 /* Per-frequency divisors: theta_k = base^(-2k/head_dim) / factors[k], n = head_dim / 2 (the "rope_freqs.weight" tensor llama.cpp
  * writes for Llama-3.1 exports; the LongFactors table of the reference's record, neural/neuralpretrained.pas:652-655). */
 int cai_decoder_set_rope_freq_factors(cai_decoder_t d, const float* factors, int n);
+/* The factor the rotary layer puts on its output (YaRN temperature, an explicit attention_factor, LongRoPE's LongAttnFactor:
+ * neural/neuralpretrained.pas:656-667).  The layer sits on q and k, so the session multiplies the attention scores by
+ * scale^2 instead and caches K unscaled.  cai_decoder_set_rope_scaling sets it (YaRN: 0.1 ln(factor) + 1, else 1); call this
+ * afterwards to override.  Empty session only. */
+int cai_decoder_set_rope_out_scale(cai_decoder_t d, float scale);
 int cai_decoder_snapshot(cai_decoder_t d, int seq, cai_kv_snap_t* out);
 int cai_decoder_restore(cai_decoder_t d, int seq, cai_kv_snap_t snap);
 /* Bytes of weights, biases and gains one decoded token streams (for roofline accounting). */

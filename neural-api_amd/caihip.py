@@ -9,7 +9,7 @@ from . import lib_path
 F32, F16, Q4_0, Q8_0, Q4_K, Q6_K, I8ROW = 0, 1, 2, 8, 12, 14, 100
 Q4_1, Q5_0, Q5_1, Q2_K, Q3_K, Q5_K = 3, 6, 7, 10, 11, 13
 ACT_NONE, ACT_RELU, ACT_SIGMOID, ACT_TANH = 0, 1, 2, 3
-ROPE_NONE, ROPE_LINEAR, ROPE_LLAMA3 = 0, 1, 2
+ROPE_NONE, ROPE_LINEAR, ROPE_LLAMA3, ROPE_NTK, ROPE_YARN = 0, 1, 2, 3, 4
 X_DEVICE, Y_DEVICE, MATRIX_CORES = 1, 2, 4
 KV_F32, KV_F16, KV_I8 = 0, 1, 2
 W_EMBED, W_HEAD, W_Q, W_K, W_V, W_O, W_GATEUP, W_DOWN, W_ROUTER = range(9)
@@ -22,7 +22,7 @@ cai_qw_create cai_qw_create_int8row cai_qw_destroy cai_qw_info cai_qw_dequant_ro
 cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_argmax_noalloc cai_router_topk
 cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_kv_export_layer cai_kv_import_layer cai_kv_set_eviction cai_kv_rows cai_attn_decode
 cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_generate cai_decoder_profile
-cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_set_eviction cai_decoder_cache_rows cai_decoder_set_kv_dtype cai_decoder_set_rope_scaling cai_decoder_set_rope_freq_factors cai_sample_candidates cai_decoder_candidates cai_decoder_snapshot cai_decoder_restore
+cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_set_eviction cai_decoder_cache_rows cai_decoder_set_kv_dtype cai_decoder_set_rope_scaling cai_decoder_set_rope_freq_factors cai_decoder_set_rope_out_scale cai_sample_candidates cai_decoder_candidates cai_decoder_snapshot cai_decoder_restore
 cai_decoder_weight_bytes cai_decoder_get_config cai_decoder_load_gguf
 cai_gguf_open cai_gguf_close cai_gguf_info cai_gguf_meta_int cai_gguf_meta_float cai_gguf_meta_str cai_gguf_meta_array_count
 cai_gguf_meta_array_str cai_gguf_find_tensor cai_gguf_tensor_info cai_gguf_tensor_data cai_gguf_load_qw""".split()
@@ -104,6 +104,7 @@ def load():
         L.cai_decoder_set_kv_dtype.argtypes = [vp, i32]
         L.cai_decoder_set_rope_scaling.argtypes = [vp, i32, C.c_float, i32, C.c_float, C.c_float]
         L.cai_decoder_set_rope_freq_factors.argtypes = [vp, vp, i32]
+        L.cai_decoder_set_rope_out_scale.argtypes = [vp, C.c_float]
         L.cai_sample_candidates.argtypes = [vp, i32, vp, vp, i32, C.c_float, C.c_float, C.c_float, C.c_float, i32, vp, vp, C.POINTER(i32), i32]
         L.cai_decoder_candidates.argtypes = [vp, i32, vp, vp, i32, C.c_float, C.c_float, C.c_float, C.c_float, i32, vp, vp, C.POINTER(i32)]
         L.cai_decoder_cache_rows.argtypes = [vp, i32, i32, C.POINTER(i32)]
@@ -459,6 +460,9 @@ class Decoder:
     def set_rope_scaling(self, mode, factor, original_ctx=0, low_freq_factor=1.0, high_freq_factor=4.0):
         """mode: ROPE_NONE / ROPE_LINEAR / ROPE_LLAMA3 (rope_scaling of the importers, neural/neuralpretrained.pas:633-668); empty session only."""
         check(load().cai_decoder_set_rope_scaling(self.h, mode, factor, original_ctx, low_freq_factor, high_freq_factor))
+
+    def set_rope_out_scale(self, scale):
+        check(load().cai_decoder_set_rope_out_scale(self.h, scale))
 
     def set_rope_freq_factors(self, factors):
         f = np.ascontiguousarray(factors, np.float32)

@@ -1025,7 +1025,7 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   p.qkv = qkv; p.qkv_stride = qkv_stride; p.kc = kv->k; p.vc = kv->v;
   p.seq_elems = kv->seq_elems(); p.layer_off = (int64_t)layer * kv->layer_elems();
   p.q_heads = q_heads; p.kv_heads = kv->kv_heads; p.hd = kv->head_dim; p.max_ctx = kv->max_ctx;
-  p.window = window; p.softcap = softcap; p.inv_sqrt = 1.0f / sqrtf((float)kv->head_dim);
+  p.window = window; p.softcap = softcap; p.inv_sqrt = kv->score_mul / sqrtf((float)kv->head_dim);
   p.theta = theta; p.pos = pos_dev; p.split_len = kv->split_len; p.n_splits = kv->n_splits;
   p.part = prompt_rows ? prompt_part : kv->part; p.out = out; p.out_stride = out_stride; p.seq0 = seq0;
   p.seq_mul = prompt_rows ? 0 : 1; p.appended = prompt_rows ? 1 : 0;

@@ -724,9 +724,23 @@ extern "C" int cai_decoder_set_rope_scaling(cai_decoder_t d, int mode, float fac
   CAI_READY();
   CAI_REQUIRE(d, "cai_decoder_set_rope_scaling: null decoder");
   std::vector<float> th;
-  const int rc = rope_thetas_scaled(d->cfg.rope_theta, d->cfg.head_dim, mode, factor, original_ctx, low_freq_factor, high_freq_factor, th);
+  int rc = rope_thetas_scaled(d->cfg.rope_theta, d->cfg.head_dim, mode, factor, original_ctx, low_freq_factor, high_freq_factor, th);
   if (rc) return rc;
-  return set_thetas(d, th, "cai_decoder_set_rope_scaling");
+  if ((rc = set_thetas(d, th, "cai_decoder_set_rope_scaling"))) return rc;
+  const float s = mode == CAI_ROPE_YARN ? (float)(0.1 * log((double)factor) + 1.0) : 1.0f;
+  return cai_decoder_set_rope_out_scale(d, s);
+}
+
+extern "C" int cai_decoder_set_rope_out_scale(cai_decoder_t d, float scale)
+{
+  CAI_READY();
+  CAI_REQUIRE(d, "cai_decoder_set_rope_out_scale: null decoder");
+  CAI_REQUIRE(scale > 0.0f && scale < 3.0e38f, "cai_decoder_set_rope_out_scale: scale %g", (double)scale);
+  for (int n : d->kv.len)
+    if (n > 0) return set_error(CAI_ERR_STATE, "cai_decoder_set_rope_out_scale: the cache holds %d tokens; set the rule on an empty session", n);
+  if (d->kv.score_mul != scale * scale) invalidate_graphs(d);   // the factor is a launch argument of the captured attention kernels
+  d->kv.score_mul = scale * scale;
+  return CAI_OK;
 }
 
 extern "C" int cai_decoder_set_rope_freq_factors(cai_decoder_t d, const float* factors, int n)

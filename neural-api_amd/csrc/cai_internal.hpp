@@ -122,6 +122,7 @@ inline const uint8_t* qw_aux2(const cai_qw_s* w) { return w->qtype == CAI_Q6_K ?
 
 struct cai_kv_s {
   int n_seq = 1, n_layers = 0, kv_heads = 0, head_dim = 0, max_ctx = 0, dtype = 0;
+  float score_mul = 1.0f;                 // on top of 1 / sqrt(head_dim): the square of the rotary layer's output scale
   void* k = nullptr; void* v = nullptr;   // [seq][layer][kv_head][max_ctx][head_dim]
   float* ks = nullptr; float* vs = nullptr;   // CAI_KV_I8 only: one scale per cached row, [seq][layer][kv_head][max_ctx]
   std::vector<int> len;                   // [seq][layer] stream position = tokens appended so far (host mirror)

@@ -227,18 +227,35 @@ void rope_thetas(float base, int head_dim, std::vector<float>& out)
 //   linear (Position Interpolation): theta_k / factor
 //   llama3: with r = original_ctx * theta_k / (2 pi) rotations over the training context: r > high_freq_factor keeps theta_k,
 //           r < low_freq_factor takes theta_k / factor, between them the two are blended linearly in r (no output scale)
+//   ntk:    base' = base * factor^(d / (d - 2)) (the static form of the dynamic rule at the full factor)
+//   yarn:   pair k keeps theta_k below the correction dimension of high_freq_factor (= beta_fast) rotations, takes theta_k / factor
+//           above that of low_freq_factor (= beta_slow), linear in k between (band edges floored / ceiled); the rotated q and k
+//           are also multiplied by 0.1 ln(factor) + 1, which the session applies as its square on the attention scores
 int rope_thetas_scaled(float base, int head_dim, int mode, float factor, int original_ctx, float low_freq_factor, float high_freq_factor, std::vector<float>& out)
 {
   if (mode == CAI_ROPE_NONE) { rope_thetas(base, head_dim, out); return CAI_OK; }
-  if (mode != CAI_ROPE_LINEAR && mode != CAI_ROPE_LLAMA3) return set_error(CAI_ERR_UNSUPPORTED, "rope scaling: mode %d (0 none, 1 linear, 2 llama3)", mode);
+  if (mode < CAI_ROPE_LINEAR || mode > CAI_ROPE_YARN) return set_error(CAI_ERR_UNSUPPORTED, "rope scaling: mode %d (0 none, 1 linear, 2 llama3, 3 ntk, 4 yarn)", mode);
   if (!(factor >= 1.0f)) return set_error(CAI_ERR_INVALID, "rope scaling: factor must be >= 1, got %g", (double)factor);
-  if (mode == CAI_ROPE_LLAMA3 && (original_ctx <= 0 || !(high_freq_factor > low_freq_factor) || !(low_freq_factor > 0.0f)))
-    return set_error(CAI_ERR_INVALID, "rope scaling: llama3 needs original_ctx > 0 and high_freq_factor > low_freq_factor > 0 (got %d, %g, %g)", original_ctx, (double)high_freq_factor, (double)low_freq_factor);
+  if ((mode == CAI_ROPE_LLAMA3 || mode == CAI_ROPE_YARN) && (original_ctx <= 0 || !(high_freq_factor > low_freq_factor) || !(low_freq_factor > 0.0f)))
+    return set_error(CAI_ERR_INVALID, "rope scaling: llama3 / yarn need original_ctx > 0 and high_freq_factor > low_freq_factor > 0 (got %d, %g, %g)", original_ctx, (double)high_freq_factor, (double)low_freq_factor);
+  if (mode == CAI_ROPE_NTK && head_dim <= 2) return set_error(CAI_ERR_INVALID, "rope scaling: ntk needs a head wider than 2");
   out.resize(head_dim / 2);
   const double two_pi = 6.283185307179586476925286766559;
+  double ylow = 0.0, yhigh = 1.0;
+  if (mode == CAI_ROPE_YARN) {
+    const double lb = 2.0 * log((double)base);
+    ylow = std::max(0.0, floor(head_dim * log((double)original_ctx / ((double)high_freq_factor * two_pi)) / lb));
+    yhigh = std::min((double)(head_dim - 1), ceil(head_dim * log((double)original_ctx / ((double)low_freq_factor * two_pi)) / lb));
+    if (yhigh == ylow) yhigh += 0.001;
+  }
   for (int k = 0; k < head_dim / 2; k++) {
     const double th = pow((double)base, -2.0 * k / head_dim);
     double v = th / (double)factor;
+    if (mode == CAI_ROPE_NTK) v = pow((double)base * pow((double)factor, (double)head_dim / (head_dim - 2.0)), -2.0 * k / head_dim);
+    if (mode == CAI_ROPE_YARN) {
+      const double ramp = std::min(1.0, std::max(0.0, ((double)k - ylow) / (yhigh - ylow)));
+      v = (th / (double)factor) * ramp + th * (1.0 - ramp);
+    }
     if (mode == CAI_ROPE_LLAMA3) {
       const double r = (double)original_ctx * th / two_pi;
       if (r > (double)high_freq_factor) v = th;

@@ -22,7 +22,7 @@ const
   // ggml tensor type ids (neural/neuralgguf.pas:86-98) + per-row int8
   CAI_F32 = 0; CAI_F16 = 1; CAI_Q4_0 = 2; CAI_Q8_0 = 8; CAI_Q4_K = 12; CAI_Q6_K = 14; CAI_I8ROW = 100;
   CAI_Q4_1 = 3; CAI_Q5_0 = 6; CAI_Q5_1 = 7; CAI_Q2_K = 10; CAI_Q3_K = 11; CAI_Q5_K = 13;
-  CAI_ROPE_NONE = 0; CAI_ROPE_LINEAR = 1; CAI_ROPE_LLAMA3 = 2;
+  CAI_ROPE_NONE = 0; CAI_ROPE_LINEAR = 1; CAI_ROPE_LLAMA3 = 2; CAI_ROPE_NTK = 3; CAI_ROPE_YARN = 4;
   // fused activation opcodes = csAct* of the OpenCL kernels (neural/neural.cl:114-146)
   CAI_ACT_NONE = 0; CAI_ACT_RELU = 1; CAI_ACT_SIGMOID = 2; CAI_ACT_TANH = 3;
   CAI_X_DEVICE = 1; CAI_Y_DEVICE = 2; CAI_MATRIX_CORES = 4;
@@ -107,6 +107,7 @@ function cai_decoder_set_eviction(d: TCaiDecoder; sink_tokens, recent_window: Lo
 function cai_decoder_set_kv_dtype(d: TCaiDecoder; kv_dtype: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_set_rope_scaling(d: TCaiDecoder; mode: LongInt; factor: Single; original_ctx: LongInt; low_freq_factor, high_freq_factor: Single): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_set_rope_freq_factors(d: TCaiDecoder; factors: PSingle; n: LongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_decoder_set_rope_out_scale(d: TCaiDecoder; scale: Single): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_cache_rows(d: TCaiDecoder; seq, layer: LongInt; rows_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_snapshot(d: TCaiDecoder; seq: LongInt; out_snap: PCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_restore(d: TCaiDecoder; seq: LongInt; snap: TCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;

@@ -529,22 +529,43 @@ void orc_rope_thetas(float base, int head_dim, float* th)
 
 /* Frequency table under a long-context rule (neural/neuralpretrained.pas:633-668: "linear" -> Position Interpolation,
  * "llama3" -> the Llama-3.1 rule with original_max_position_embeddings, low_freq_factor, high_freq_factor and NO output
- * scale).  mode 0 none, 1 linear, 2 llama3.  The layer that applies the rule (TNNetRotaryEmbedding) is not among the
+ * scale; "dynamic"/"ntk" -> NTK-aware base change; "yarn" -> per-pair blend + attention temperature).  mode 0 none, 1 linear,
+ * 2 llama3, 3 ntk, 4 yarn (low_freq_factor = beta_slow / YarnAlpha, high_freq_factor = beta_fast / YarnBeta, band edges
+ * floored / ceiled as HF does by default).  The layer that applies the rule (TNNetRotaryEmbedding) is not among the
  * reference's files here, so the formulas are the published ones the importer's comments name: PI divides every frequency
  * by the factor; llama3 keeps pairs that turn more than high_freq_factor times over the original context, divides those
  * that turn less than low_freq_factor times, and blends linearly in the rotation count between.
  * Pinned by: the saturating case of tests/TestNeuralNumerical.pas:16008-16028 (d = 8, base 1e4, original 512, low 1,
  * high 4, factor 8: pairs 0, 1 kept, pairs 2, 3 divided by 8), theta/factor for linear, an independent float64 restatement
- * of the published rule on a 128-wide head (tests/test_oracle_model.py).  The blend region itself: parity unpinned against
- * the reference's layer (no fixture exercises it). */
+ * of the published rule on a 128-wide head (tests/test_oracle_model.py).  The llama3 blend region itself: parity unpinned
+ * against the reference's layer (no fixture exercises it).  NTK: the exact formula of tests/TestNeuralNumerical.pas:15869-15880
+ * (theta'_k = (base * s^(d/(d-2)))^(-2k/d)).  YaRN: the band case of tests/TestNeuralNumerical.pas:15890-15990 (d = 8, base 1e4,
+ * original 512, s = 2, alpha 1, beta 32: low = floor(0.406) = 0, high = ceil(1.911) = 2, thetas 1, 0.075, 0.005, 0.0005 - the
+ * blend of pair 1 included) and its temperature 0.1 ln(s) + 1 (orc_rope_out_scale). */
 int orc_rope_thetas_scaled(float base, int head_dim, int mode, float factor, int original_ctx, float low_freq_factor, float high_freq_factor, float* th)
 {
-  if (mode < 0 || mode > 2 || !(factor >= 1.0f)) return -1;
-  if (mode == 2 && (original_ctx <= 0 || !(high_freq_factor > low_freq_factor))) return -1;
+  if (mode < 0 || mode > 4 || !(factor >= 1.0f)) return -1;
+  if ((mode == 2 || mode == 4) && (original_ctx <= 0 || !(high_freq_factor > low_freq_factor))) return -1;
+  if (mode == 3 && head_dim <= 2) return -1;
+  double ylow = 0.0, yhigh = 0.0;
+  if (mode == 4) {   /* correction dims of beta_fast (high_freq_factor) and beta_slow (low_freq_factor) rotations */
+    const double lb = 2.0 * log((double)base);
+    ylow = floor(head_dim * log((double)original_ctx / ((double)high_freq_factor * 2.0 * M_PI)) / lb);
+    yhigh = ceil(head_dim * log((double)original_ctx / ((double)low_freq_factor * 2.0 * M_PI)) / lb);
+    if (ylow < 0.0) ylow = 0.0;
+    if (yhigh > head_dim - 1) yhigh = head_dim - 1;
+    if (yhigh == ylow) yhigh += 0.001;
+  }
   for (int k = 0; k < head_dim / 2; k++) {
     const double t = pow((double)base, -2.0 * k / head_dim);
     double v = t;
     if (mode == 1) v = t / (double)factor;
+    if (mode == 3) v = pow((double)base * pow((double)factor, (double)head_dim / (head_dim - 2.0)), -2.0 * k / head_dim);
+    if (mode == 4) {
+      double ramp = ((double)k - ylow) / (yhigh - ylow);
+      ramp = ramp < 0.0 ? 0.0 : (ramp > 1.0 ? 1.0 : ramp);
+      v = (t / (double)factor) * ramp + t * (1.0 - ramp);   /* ramp 0: keep the frequency; ramp 1: fully interpolated */
+    }
     if (mode == 2) {
       const double wavelen = 2.0 * M_PI / t;
       const double lo_wl = (double)original_ctx / (double)low_freq_factor, hi_wl = (double)original_ctx / (double)high_freq_factor;
@@ -559,6 +580,10 @@ int orc_rope_thetas_scaled(float base, int head_dim, int mode, float factor, int
   }
   return 0;
 }
+
+/* The attention temperature a rule puts on the rotated q and k (the kernel's OutScale, neural.cl:1517-1542): YaRN
+ * 0.1 ln(factor) + 1, every other rule 1. */
+float orc_rope_out_scale(int mode, float factor) { return mode == 4 ? (float)(0.1 * log((double)factor) + 1.0) : 1.0f; }
 
 /* neural.cl:1517-1542: pairs (2k,2k+1) per head, angle = (float)pos * theta_k (fp32 product). */
 void orc_rope_interleaved(float* x, int n_heads, int head_dim, int pos, const float* th)
@@ -866,6 +891,7 @@ struct orc_model {
   const float* final_norm;
   orc_layer* layers;
   float* theta;
+  float rope_out_scale;   /* multiplies the rotated q and k (1 unless a rule sets it) */
   int len;
   float *x, *h, *qkv, *att, *gu, *mid, *tmp, *probs, *gates, *logits;
   int* sel;
@@ -887,6 +913,7 @@ orc_model* orc_model_new(const orc_config* cfg)
   }
   m->theta = (float*)malloc(sizeof(float) * (size_t)(cfg->head_dim / 2));
   orc_rope_thetas(cfg->rope_theta, cfg->head_dim, m->theta);
+  m->rope_out_scale = 1.0f;
   int wide = d; if (qw > wide) wide = qw;
   m->x = (float*)calloc((size_t)d, 4); m->h = (float*)calloc((size_t)wide, 4);
   m->qkv = (float*)calloc((size_t)(qw + 2 * kw), 4); m->att = (float*)calloc((size_t)qw, 4);
@@ -932,6 +959,8 @@ void orc_model_set_thetas(orc_model* m, const float* th, int n)
   if (n == m->cfg.head_dim / 2) memcpy(m->theta, th, sizeof(float) * (size_t)n);
 }
 
+void orc_model_set_rope_out_scale(orc_model* m, float s) { m->rope_out_scale = s; }
+
 void orc_model_reset(orc_model* m) { m->len = 0; }
 void orc_model_truncate(orc_model* m, int n) { if (n < m->len) m->len = n < 0 ? 0 : n; }
 int  orc_model_len(const orc_model* m) { return m->len; }
@@ -974,6 +1003,7 @@ int orc_model_step(orc_model* m, int token, int pos, float* logits)
     }
     orc_rope_interleaved(m->qkv, c->n_q_heads, hd, pos, m->theta);
     orc_rope_interleaved(m->qkv + qw, c->n_kv_heads, hd, pos, m->theta);
+    if (m->rope_out_scale != 1.0f) for (int i = 0; i < qw + kw; i++) m->qkv[i] *= m->rope_out_scale;
     if (c->kv_f16 == 2) orc_attn_decode_i8(m->qkv, c->n_q_heads, c->n_kv_heads, hd, ly->kq, ly->ks, ly->vq, ly->vs, c->max_ctx, pos, c->window, 0.0f, m->att);
     else attn_core_f32(m->qkv, c->n_q_heads, c->n_kv_heads, hd, ly->kc, ly->vc, c->max_ctx, pos, c->window, c->evict_sinks, c->evict_recent, 0.0f, c->kv_f16, m->att);
     lin(m, &ly->w[ORC_W_O], 0, d, m->att, m->tmp);

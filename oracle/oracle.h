@@ -133,6 +133,8 @@ int  orc_model_set_tensor(orc_model* m, int layer, int slot, int type, int64_t r
                           const void* raw, const float* scales, const float* bias);
 int  orc_model_set_vec(orc_model* m, int layer, int slot, const float* v, int n);
 void orc_model_set_thetas(orc_model* m, const float* theta_half, int n);
+void orc_model_set_rope_out_scale(orc_model* m, float s);
+float orc_rope_out_scale(int mode, float factor);
 void orc_model_reset(orc_model* m);
 void orc_model_truncate(orc_model* m, int n);
 int  orc_model_len(const orc_model* m);

@@ -46,6 +46,8 @@ def lib():
         L.orc_rope_thetas.argtypes = [C.c_float, C.c_int, C.c_void_p]; L.orc_rope_thetas.restype = None
         L.orc_rope_thetas_scaled.argtypes = [C.c_float, C.c_int, C.c_int, C.c_float, C.c_int, C.c_float, C.c_float, C.c_void_p]
         L.orc_model_set_thetas.argtypes = [C.c_void_p, C.c_void_p, C.c_int]; L.orc_model_set_thetas.restype = None
+        L.orc_model_set_rope_out_scale.argtypes = [C.c_void_p, C.c_float]; L.orc_model_set_rope_out_scale.restype = None
+        L.orc_rope_out_scale.argtypes = [C.c_int, C.c_float]; L.orc_rope_out_scale.restype = C.c_float
         L.orc_rope_interleaved.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]; L.orc_rope_interleaved.restype = None
         L.orc_swiglu.argtypes = [C.c_void_p, C.c_int, C.c_void_p]; L.orc_swiglu.restype = None
         L.orc_softmax.argtypes = [C.c_void_p, C.c_int, C.c_void_p]; L.orc_softmax.restype = None
@@ -156,6 +158,9 @@ class OracleModel:
     def set_thetas(self, th):
         th = np.ascontiguousarray(th, np.float32)
         lib().orc_model_set_thetas(self.h, _p(th), th.size)
+
+    def set_rope_out_scale(self, s):
+        lib().orc_model_set_rope_out_scale(self.h, s)
 
     def reset(self):
         lib().orc_model_reset(self.h)

@@ -30,13 +30,15 @@ def run_both(om, dec, seq, pos0=0):
     return worst
 
 
-@pytest.mark.parametrize("mode,args", [("linear", (1, 4.0, 0, 1.0, 4.0)), ("llama3", (2, 8.0, 16, 1.0, 4.0))])
+@pytest.mark.parametrize("mode,args", [("linear", (1, 4.0, 0, 1.0, 4.0)), ("llama3", (2, 8.0, 16, 1.0, 4.0)), ("ntk", (3, 4.0, 0, 1.0, 4.0)), ("yarn", (4, 4.0, 24, 1.0, 32.0))])
 def test_scaled_decoder_matches_the_oracle_and_differs_from_the_unscaled_one(mode, args):
     from helpers.device import dev, rel_err
     cai = dev()
     spec = synthetic_spec(CFG, O.Q8_0, seed=77, std=0.08)
     th = scaled(CFG["rope_theta"], CFG["head_dim"], *args)
     om = oracle_model(spec, acc64=1); om.set_thetas(th)
+    out_scale = O.lib().orc_rope_out_scale(args[0], C.c_float(args[1]))
+    om.set_rope_out_scale(out_scale)          # the oracle scales the rotated q and k, the device the scores by its square
     dec = cai.Decoder(spec)
     seq = [int(t) for t in np.random.default_rng(5).integers(0, 300, 40)]
     plain = [dec.step(t, p)[1][0].copy() for p, t in enumerate(seq)]
@@ -50,15 +52,20 @@ def test_scaled_decoder_matches_the_oracle_and_differs_from_the_unscaled_one(mod
     dec.reset(0)
     last = [dec.step(t, p)[1][0].copy() for p, t in enumerate(seq)][-1]
     assert rel_err(last, plain[-1]) > 1e-2          # the rule does something at these positions
+    dec.reset(0)
+    am, lg = dec.prefill(seq, 0)                     # the prompt kernels rotate and scale by the same rule
+    assert rel_err(lg, last) < TOL
     # the same table as per-frequency divisors
     base = scaled(CFG["rope_theta"], CFG["head_dim"], 0, 1.0)
     dec.reset(0)
     dec.set_rope_freq_factors(base.astype(np.float64) / th.astype(np.float64))
+    dec.set_rope_out_scale(out_scale)
     again = [dec.step(t, p)[1][0].copy() for p, t in enumerate(seq)][-1]
     assert rel_err(again, last) < 1e-4
     # back to none restores the unscaled logits bit for bit; the captured-graph path follows the table too
     dec.reset(0)
     dec.set_rope_scaling(cai.ROPE_NONE, 1.0)
+    # (none also puts the output scale back to 1)
     back = [dec.step(t, p)[1][0].copy() for p, t in enumerate(seq)][-1]
     assert np.array_equal(back, plain[-1])
     dec.close()
@@ -68,7 +75,7 @@ def test_bad_rules_are_refused():
     from helpers.device import dev
     cai = dev()
     dec = cai.Decoder(synthetic_spec(CFG, O.Q8_0, seed=1))
-    for args in [(1, 0.5, 0, 1.0, 4.0), (2, 8.0, 0, 1.0, 4.0), (2, 8.0, 512, 4.0, 4.0), (3, 2.0, 0, 1.0, 4.0)]:
+    for args in [(1, 0.5, 0, 1.0, 4.0), (2, 8.0, 0, 1.0, 4.0), (2, 8.0, 512, 4.0, 4.0), (4, 2.0, 0, 1.0, 32.0), (7, 2.0, 0, 1.0, 4.0)]:
         with pytest.raises(cai.CaiError):
             dec.set_rope_scaling(*args)
     with pytest.raises(cai.CaiError):

@@ -142,3 +142,28 @@ def test_rope_scaling_tables():
     buf = np.empty(4, np.float32)
     assert O.lib().orc_rope_thetas_scaled(C.c_float(1e4), 8, 1, C.c_float(0.5), 0, C.c_float(1), C.c_float(4), buf.ctypes.data) != 0
     assert O.lib().orc_rope_thetas_scaled(C.c_float(1e4), 8, 2, C.c_float(8), 512, C.c_float(4), C.c_float(4), buf.ctypes.data) != 0
+
+
+def test_rope_scaling_ntk_and_yarn_known_answers():
+    """NTK: theta'_k = (base * s^(d/(d-2)))^(-2k/d) (tests/TestNeuralNumerical.pas:15869-15880, d = 8, s = 4).  YaRN: the band case
+    of tests/TestNeuralNumerical.pas:15890-15990 (d = 8, base 1e4, original 512, s = 2, alpha 1, beta 32): pair 0 keeps its
+    frequency, pair 1 is the half-way blend 0.075, pairs 2 and 3 are fully interpolated; temperature 0.1 ln 2 + 1."""
+    import ctypes as C
+    nb = 1e4 * 4.0 ** (8 / 6)
+    assert np.array_equal(_scaled(1e4, 8, 3, 4.0), np.array([nb ** (-2.0 * k / 8) for k in range(4)]).astype(np.float32))
+    th = _scaled(1e4, 8, 4, 2.0, 512, 1.0, 32.0)
+    assert np.allclose(th, [1.0, 0.075, 0.005, 0.0005], rtol=1e-6, atol=0)
+    assert th[0] == np.float32(1.0) and th[2] == np.float32(0.01 / 2) and th[3] == np.float32(0.001 / 2)
+    L = O.lib()
+    assert abs(L.orc_rope_out_scale(4, C.c_float(2.0)) - (0.1 * np.log(2.0) + 1.0)) < 1e-7
+    assert L.orc_rope_out_scale(2, C.c_float(8.0)) == 1.0 and L.orc_rope_out_scale(0, C.c_float(1.0)) == 1.0
+    # the published YaRN rule written a second way (numpy, the way HF states it) on a 128-wide head: Qwen2.5 long-context constants
+    hd, base, factor, orig, bslow, bfast = 128, 1e6, 4.0, 32768, 1.0, 32.0
+    pos_freqs = base ** (np.arange(0, hd, 2, dtype=np.float64) / hd)
+    corr = lambda rot: hd * np.log(orig / (rot * 2 * np.pi)) / (2 * np.log(base))
+    low, high = max(np.floor(corr(bfast)), 0), min(np.ceil(corr(bslow)), hd - 1)
+    ramp = np.clip((np.arange(hd // 2) - low) / (high - low), 0, 1)
+    extrap_factor = 1 - ramp
+    inv = (1 / (factor * pos_freqs)) * (1 - extrap_factor) + (1 / pos_freqs) * extrap_factor
+    assert np.allclose(_scaled(base, hd, 4, factor, orig, bslow, bfast), inv.astype(np.float32), rtol=3e-7, atol=0)
+    assert 0 < low < high < hd // 2          # a genuine band inside the table
