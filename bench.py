@@ -247,6 +247,15 @@ def gemm_sweep(cai, synth, torch):
 # KiB, factors from a 1 GiB copy kernel): profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt.  Not measurable from
 # inside this process; re-collect when the kernel changes.
 GATEUP_TRAFFIC_BYTES = int((37513.6 * 2.000 + 74.5 * 1.000) * 1024)
+def gateup_kernel_name(qtype, cols):
+    """Name of the batch-1 fused gate|up kernel the library launches for this weight type and width (rows of 17..24
+    super-blocks are packed four to a wave: the fifth template argument)."""
+    if qtype not in ("Q4_K", "Q5_K"):
+        return "gemv_fast<%s>" % qtype
+    packed = cols % 256 == 0 and 16 < cols // 256 <= 24
+    return "gemv_%s_dot<1,1,false,2%s>" % ("q4k" if qtype == "Q4_K" else "q5k", ",4" if packed else "")
+
+
 GATEUP_TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of gemv_q4k_dot<1,1,false,2>, profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt; "
                          "collected with the tree at commit e3181a8 (cai_gemv_dot.hip last changed in 77da839)")
 
@@ -439,7 +448,7 @@ def main():
                                "tok_per_s": round((prompt_len - 1) / max(pf_ms.value, 1e-6) * 1e3, 1),
                                "linear_tflops": round(2.0 * n_lin_weights * (prompt_len - 1) / max(pf_ms.value, 1e-6) / 1e9, 1),
                                "note": "multi-token ingestion: f16 MFMA (exact scale*nibble weight operand, hi/lo-split activations = 2 MFMA passes per useful FLOP) + prompt attention; MFMA f16 dense peak 2500 TFLOP/s"}},
-        "roofline": {"bound": "hbm", "kernel": "%s (RMSNorm+gate|up+SwiGLU, %dx%d)" % ("gemv_q4k_dot<1,1,false,2>" if conf["qtype"] == "Q4_K" else "gemv_q5k_dot<1,1,false,2>" if conf["qtype"] == "Q5_K" else "gemv_fast<%s>" % conf["qtype"], 2 * I, d),
+        "roofline": {"bound": "hbm", "kernel": "%s (RMSNorm+gate|up+SwiGLU, %dx%d)" % (gateup_kernel_name(conf["qtype"], d), 2 * I, d),
                      "achieved": round(k_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(k_gbs / HBM_PEAK_GBS, 4),
                      "avg_launch_us": round(k_avg_us, 2), "algorithmic_bytes_per_launch": int(k_bytes),
                      "traffic": GATEUP_TRAFFIC_BYTES if args.config == "qwen2.5-7b-q4k" else None, "traffic_unit": "bytes/launch",

@@ -13,7 +13,8 @@
 // Work layout (as in the float kernel): a fixed number of work-groups stays resident and strides over the row
 // groups; one lane owns one pair of sub-blocks (64 weights = two 128-bit loads + the 16-byte super-block
 // header); rows longer than 4096 columns are split over `nsw` waves, each keeping its slice of the quantised
-// activation in registers (52 VGPRs).  Weights of the next NS-1 row groups are in flight while one is reduced.
+// activation in registers (52 VGPRs); widths of 17..24 super-blocks pack four rows into a wave instead (slices of four
+// super-blocks), so that no lanes idle.  Weights of the next NS-1 row groups are in flight while one is reduced.
 //
 // Semantics: Out[a] = act(dot(W[a], X) + bias[a]) (+ residual), or for the fused feed-forward front half
 // Out[i] = up_i * silu(gate_i) with up = row i and gate = row half + i
@@ -55,6 +56,18 @@ __device__ __forceinline__ int quad_sum(int v)
   return v;
 }
 
+// sum over each group of 64 / PK lanes, valid in the group's last lane
+template <int PK>
+__device__ __forceinline__ float group_sum(float v)
+{
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, true)); // row_shr:1
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x112, 0xf, 0xf, true)); // row_shr:2
+  if (PK <= 8) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x114, 0xf, 0xf, true)); // row_shr:4
+  if (PK <= 4) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x118, 0xf, 0xf, true)); // row_shr:8
+  if (PK <= 2) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xa, 0xf, true)); // row_bcast:15
+  return v;
+}
+
 // four rounded activations (as float bit patterns of x*inv + 1.5*2^23) -> one dword per digit
 __device__ __forceinline__ void pack_digits(const float (&f)[4], int (&d)[NL])
 {
@@ -78,20 +91,29 @@ __device__ __forceinline__ void pack_digits(const float (&f)[4], int (&d)[NL])
 // offset uses the sums of the lane's integer activations per 16, taken once; each 16 weights have their own scale.
 struct Q6kRegs { uint4 a0, a1, b0, b1, h0, h1; uint2 sc; uint32_t d; };
 
-template <int R, int MODE, bool MULTISEG, int NS, int QT>
+// PK > 1 packs PK rows into one wave: a wave then holds 16 / PK super-blocks of PK different row-group streams (lane
+// quarter-groups of 64 / PK lanes), so a width that is not a multiple of 4096 columns leaves no lanes idle - 5120 columns
+// are five waves of 4 super-blocks x 4 rows instead of two waves of 16 + 4 super-blocks x 1 row.  The row a lane works on
+// then differs inside the wave (addresses and group indices are vector values), sums are taken per lane group and the
+// outputs always finish through LDS.
+template <int R, int MODE, bool MULTISEG, int NS, int QT, int PK = 1>
 __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_groups, const int nsw, const int gwv)
 {
   extern __shared__ uint4 xq4[];
   constexpr int RR = MODE == 1 ? 2 * R : R;
+  constexpr int TS = 16 / PK;                 // super-blocks of a row held by one wave
+  static_assert(PK == 1 || PK == 2 || PK == 4 || PK == 8, "rows packed per wave");
   __shared__ float s_ss[16];
   constexpr int CH = 4;                       // row groups between two meetings of the slice waves
-  __shared__ float s_part[2][16][CH][RR];
+  __shared__ float s_part[2][16][CH][PK * RR];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: group indices, segment lookups and loop bounds stay scalar
-  const int step = wave % nsw, gslot = wave / nsw;
+  const int step = wave % nsw, gquad = wave / nsw;
+  const int prow = PK > 1 ? (lane >> 2) / TS : 0;          // which of the wave's PK row streams this lane belongs to
+  const int gslot = gquad * PK + prow;
   const int cols = p.cols, nsb = cols >> 8;
   const int64_t row_bytes = (int64_t)nsb * dot_rec_bytes<QT>();
-  const int sb = step * 16 + (lane >> 2), cc = lane & 3;
+  const int sb = step * TS + (PK > 1 ? (lane >> 2) % TS : (lane >> 2)), cc = lane & 3;
   const bool act = sb < nsb;
   const int g_first = blockIdx.x * gwv + gslot, g_stride = gridDim.x * gwv;
   const int n_iters = (n_groups + g_stride - 1) / g_stride;
@@ -110,8 +132,25 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
   // Loads are never conditional: past the last group the last one is fetched again, lanes beyond the row's width fetch
   // super-block 0 (both cache hits, the values are not used).  A load under a branch would make the compiler wait for
   // ALL outstanding loads wherever the paths join, i.e. before every new request.
+  // the same with the group index a vector value (packed rows): the segment's fields are selected, not fetched through a
+  // per-lane pointer (that would put a dependent load in front of every weight request)
+  struct SegV { const uint8_t* data; const uint8_t* aux; int rows, row0; };
+  auto locate_v = [&](int g) {
+    SegV v{p.seg[0].data, p.seg[0].aux, p.seg[0].rows, 0};
+    int g0 = 0;
+    if (MULTISEG) {
+      if (p.n_seg > 1 && g >= p.seg[0].grp_end) { v.data = p.seg[1].data; v.aux = p.seg[1].aux; v.rows = p.seg[1].rows; g0 = p.seg[0].grp_end; }
+      if (p.n_seg > 2 && g >= p.seg[1].grp_end) { v.data = p.seg[2].data; v.aux = p.seg[2].aux; v.rows = p.seg[2].rows; g0 = p.seg[1].grp_end; }
+    }
+    v.row0 = (g - g0) * R;
+    return v;
+  };
   auto issue = [&](int g, WRegs (&rg)[RR]) {
-    const GemvSeg* sg; int row0; locate(min(g, n_groups - 1), sg, row0);
+    SegV sv;
+    if constexpr (PK > 1) sv = locate_v(min(g, n_groups - 1));
+    else { const GemvSeg* sg1; int r0; locate(min(g, n_groups - 1), sg1, r0); sv = SegV{sg1->data, sg1->aux, sg1->rows, r0}; }
+    const SegV* sg = &sv;
+    const int row0 = sv.row0;
     const int lim = MODE == 1 ? p.half : sg->rows;
 #pragma unroll
     for (int r = 0; r < RR; r++) {
@@ -295,7 +334,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
     float acc[RR];
 #pragma unroll
     for (int r = 0; r < RR; r++) acc[r] = 0.0f;
-    if (g < n_groups) {   // lanes beyond the row's width hold zero activations: they add exactly 0
+    if (PK > 1 || g < n_groups) {   // lanes beyond the row's width hold zero activations: they add exactly 0; packed rows: groups differ per lane, totals past the end are dropped below
 #pragma unroll
       for (int r = 0; r < RR; r++) {
         if constexpr (QT == CAI_Q6_K) {
@@ -394,6 +433,46 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
         }
       }
     }
+    if constexpr (PK > 1) {
+      // Packed rows: per-lane-group totals (last lane of each group), parked in LDS as the slice waves do, and one lane
+      // per output row of the chunk finishes it.
+      constexpr int SEGL = 64 / PK, RO = MODE == 1 ? R : RR;
+      static_assert(CH * PK * RO <= 64, "one lane per output row of a chunk");
+#pragma unroll
+      for (int r = 0; r < RR; r++) acc[r] = group_sum<PK>(acc[r]);
+      const int slot = it % CH, par = (it / CH) & 1;
+      if ((lane & (SEGL - 1)) == SEGL - 1) {
+#pragma unroll
+        for (int r = 0; r < RR; r++) s_part[par][wave][slot][prow * RR + r] = acc[r];
+      }
+      if (slot != CH - 1 && it != n_iters - 1) return;
+      __syncthreads();
+      if (step != 0) return;
+      const int n_out = (slot + 1) * PK * RO;
+      if (lane >= n_out) return;
+      const int sl = lane / (PK * RO), po = (lane / RO) % PK, r = lane % RO;
+      const int gg = blockIdx.x * gwv + gquad * PK + po + (it - slot + sl) * g_stride;
+      if (gg >= n_groups) return;
+      const GemvSeg* sg; int row0; locate(gg, sg, row0);
+      const int row = row0 + r;
+      if (MODE == 0) {
+        if (row >= sg->rows) return;
+        float v = 0.0f;
+        for (int s2 = 0; s2 < nsw; s2++) v += s_part[par][gquad * nsw + s2][sl][po * RR + r];
+        if (sg->bias) v += sg->bias[row];
+        v = act_apply(v, p.act);
+        const int o = sg->y_off + row;
+        if (p.residual) v += p.residual[o];
+        p.y[o] = v; ssq_acc = fmaf(v, v, ssq_acc);
+      } else {
+        if (row >= p.half) return;
+        float up = 0.0f, gate = 0.0f;
+        for (int s2 = 0; s2 < nsw; s2++) { up += s_part[par][gquad * nsw + s2][sl][po * RR + 2 * r]; gate += s_part[par][gquad * nsw + s2][sl][po * RR + 2 * r + 1]; }
+        if (sg->bias) { up += sg->bias[row]; gate += sg->bias[p.half + row]; }
+        p.y[sg->y_off + row] = silu_mul(up, gate);
+      }
+      return;
+    }
 #pragma unroll
     for (int r = 0; r < RR; r++) acc[r] = wave_sum(acc[r]);   // total in lane 63
 
@@ -418,7 +497,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
       if (MODE == 0) {
         if (row >= sg->rows) return;
         float v = 0.0f;
-        for (int s2 = 0; s2 < nsw; s2++) v += s_part[par][gslot * nsw + s2][sl][r];
+        for (int s2 = 0; s2 < nsw; s2++) v += s_part[par][gquad * nsw + s2][sl][r];
         if (sg->bias) v += sg->bias[row];
         v = act_apply(v, p.act);
         const int o = sg->y_off + row;
@@ -427,7 +506,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
       } else {
         if (row >= p.half) return;
         float up = 0.0f, gate = 0.0f;
-        for (int s2 = 0; s2 < nsw; s2++) { up += s_part[par][gslot * nsw + s2][sl][2 * r]; gate += s_part[par][gslot * nsw + s2][sl][2 * r + 1]; }
+        for (int s2 = 0; s2 < nsw; s2++) { up += s_part[par][gquad * nsw + s2][sl][2 * r]; gate += s_part[par][gquad * nsw + s2][sl][2 * r + 1]; }
         if (sg->bias) { up += sg->bias[row]; gate += sg->bias[p.half + row]; }
         p.y[sg->y_off + row] = silu_mul(up, gate);
       }
@@ -489,22 +568,22 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
   }
 }
 
-template <int R, int MODE, bool MULTISEG, int NS>
+template <int R, int MODE, bool MULTISEG, int NS, int PK = 1>
 __global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
 {
-  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q4_K>(p, n_groups, nsw, gwv);
+  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q4_K, PK>(p, n_groups, nsw, gwv);
 }
 
-template <int R, int MODE, bool MULTISEG, int NS>
+template <int R, int MODE, bool MULTISEG, int NS, int PK = 1>
 __global__ __launch_bounds__(768, 3) void gemv_q40_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
 {
-  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q4_0>(p, n_groups, nsw, gwv);
+  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q4_0, PK>(p, n_groups, nsw, gwv);
 }
 
-template <int R, int MODE, bool MULTISEG, int NS>
+template <int R, int MODE, bool MULTISEG, int NS, int PK = 1>
 __global__ __launch_bounds__(768, 3) void gemv_q5k_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
 {
-  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q5_K>(p, n_groups, nsw, gwv);
+  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q5_K, PK>(p, n_groups, nsw, gwv);
 }
 
 template <int R, int NS>
@@ -518,19 +597,28 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
 {
   Context& c = ctx();
   const int cols = p.cols, nsb = cols >> 8;
-  const int nsw = (nsb + 15) >> 4;          // waves along the columns
+  int nsw = (nsb + 15) >> 4;                // waves along the columns
   if (nsw > 8 || cols % 256) return CAI_ERR_UNSUPPORTED;  // rows longer than 32768 columns; Q4_0 widths that are not whole 256-blocks
   const bool q6k = m.w[0]->qtype == CAI_Q6_K;
   if (q6k && (swiglu_half || m.n != 1)) return CAI_ERR_UNSUPPORTED;
   constexpr int W = 12;   // resident waves per CU
+  // Rows packed per wave: a width of 17..24 super-blocks, whose second 4096-column slice would be mostly empty (5120 columns:
+  // 20 of 32 lane quads at work), is cut into five or six slices of 4 super-blocks instead, four rows to a wave.  Measured
+  // on 55296 x 5120: 40.7 -> 32.5 us, 6144 columns 42.9 -> 38.2; widths that fill one wave lose to the exchange through LDS
+  // (2048 columns: 4.2 -> 4.9 us, 3584: 18.1 -> 19.6) and keep one row per wave.
+  constexpr int PKW = 4;
+  const bool packed = !q6k && nsb > 16 && nsb <= 24;
+  if (packed) nsw = (nsb + 16 / PKW - 1) / (16 / PKW);
   // waves per work-group: short rows (one or two waves span the columns) use ONE work-group of 8 waves per CU - the
   // activation is quantised once per CU instead of once per 4 waves, which outweighs the lower wave count (measured:
   // 3 work-groups of 4 waves 537 tok/s, 1 of 12 waves 544, 1 of 8 waves 561 on the 7B shape); long rows fill the CU
   // with a single work-group of up to 12 waves
-  const int gwv = nsw >= 3 ? std::max(1, W / nsw) : 8 / nsw;   // the kernel is built for at most 12 waves per work-group
+  int gwv = nsw >= 3 ? std::max(1, W / nsw) : 8 / nsw;   // the kernel is built for at most 12 waves per work-group
+  int gquads = gwv;                                        // waves along the rows
+  if (packed) { gquads = W / nsw; gwv = gquads * PKW; }   // two waves along the rows (one measured 6 % slower)
   int64_t total = 0;
   for (int i = 0; i < m.n; i++) total += swiglu_half ? swiglu_half : m.rows[i];
-  const int waves_per_wg = nsw * gwv;
+  const int waves_per_wg = nsw * gquads;
   const size_t lds = (size_t)((cols + 1023) / 1024 * 1024) * 4;   // 16 uint4 per 64 activations
   int wg_per_cu = W / waves_per_wg; if (wg_per_cu < 1) wg_per_cu = 1;
   { const int lds_fit = (int)((160 * 1024 - 4096) / (lds + 1024)); if (wg_per_cu > lds_fit) wg_per_cu = lds_fit < 1 ? 1 : lds_fit; }
@@ -544,6 +632,7 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
     const int64_t slots = (int64_t)max_wgs * gwv;
     const int64_t turns1 = (total + slots - 1) / slots, turns2 = ((total + 1) / 2 + slots - 1) / slots;
     if (nsw < 3 || 2 * turns2 <= turns1) R = 2;
+    if (packed) R = 2;
   }
   if (q6k) R = 1;   // (two rows of Q6_K requests in flight twice over do not fit the registers)
   int cum = 0;
@@ -564,22 +653,27 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
       (void)hipGetLastError();
     hipLaunchKernelGGL(kern, dim3(grid), block, lds, st, p, cum, nsw, gwv);
   };
+  auto pick_pk = [&](auto ns, auto pk) {
+    constexpr int NSV = decltype(ns)::value, PKV = decltype(pk)::value;
+    if (m.w[0]->qtype == CAI_Q4_0) {
+      if (swiglu_half) go(gemv_q40_dot<1, 1, false, NSV, PKV>);
+      else if (m.n > 1) { if (R == 2) go(gemv_q40_dot<2, 0, true, NSV, PKV>); else go(gemv_q40_dot<1, 0, true, NSV, PKV>); }
+      else { if (R == 2) go(gemv_q40_dot<2, 0, false, NSV, PKV>); else go(gemv_q40_dot<1, 0, false, NSV, PKV>); }
+    }
+    else if (m.w[0]->qtype == CAI_Q5_K) {
+      if (swiglu_half) go(gemv_q5k_dot<1, 1, false, NSV, PKV>);
+      else if (m.n > 1) { if (R == 2) go(gemv_q5k_dot<2, 0, true, NSV, PKV>); else go(gemv_q5k_dot<1, 0, true, NSV, PKV>); }
+      else { if (R == 2) go(gemv_q5k_dot<2, 0, false, NSV, PKV>); else go(gemv_q5k_dot<1, 0, false, NSV, PKV>); }
+    }
+    else if (swiglu_half) go(gemv_q4k_dot<1, 1, false, NSV, PKV>);
+    else if (m.n > 1) { if (R == 2) go(gemv_q4k_dot<2, 0, true, NSV, PKV>); else go(gemv_q4k_dot<1, 0, true, NSV, PKV>); }
+    else { if (R == 2) go(gemv_q4k_dot<2, 0, false, NSV, PKV>); else go(gemv_q4k_dot<1, 0, false, NSV, PKV>); }
+  };
   auto pick = [&](auto ns) {
     constexpr int NSV = decltype(ns)::value;
     if (q6k) go(gemv_q6k_dot<1, NSV>);
-    else if (m.w[0]->qtype == CAI_Q4_0) {
-      if (swiglu_half) go(gemv_q40_dot<1, 1, false, NSV>);
-      else if (m.n > 1) { if (R == 2) go(gemv_q40_dot<2, 0, true, NSV>); else go(gemv_q40_dot<1, 0, true, NSV>); }
-      else { if (R == 2) go(gemv_q40_dot<2, 0, false, NSV>); else go(gemv_q40_dot<1, 0, false, NSV>); }
-    }
-    else if (m.w[0]->qtype == CAI_Q5_K) {
-      if (swiglu_half) go(gemv_q5k_dot<1, 1, false, NSV>);
-      else if (m.n > 1) { if (R == 2) go(gemv_q5k_dot<2, 0, true, NSV>); else go(gemv_q5k_dot<1, 0, true, NSV>); }
-      else { if (R == 2) go(gemv_q5k_dot<2, 0, false, NSV>); else go(gemv_q5k_dot<1, 0, false, NSV>); }
-    }
-    else if (swiglu_half) go(gemv_q4k_dot<1, 1, false, NSV>);
-    else if (m.n > 1) { if (R == 2) go(gemv_q4k_dot<2, 0, true, NSV>); else go(gemv_q4k_dot<1, 0, true, NSV>); }
-    else { if (R == 2) go(gemv_q4k_dot<2, 0, false, NSV>); else go(gemv_q4k_dot<1, 0, false, NSV>); }
+    else if (packed) pick_pk(ns, std::integral_constant<int, PKW>());
+    else pick_pk(ns, std::integral_constant<int, 1>());
   };
   pick(std::integral_constant<int, 2>());   // two row groups per wave: one in flight while one is reduced (three measured slower on every shape)
   return CAI_OK;

@@ -64,7 +64,7 @@ def test_ffn_gateup_at_the_benchmarked_shapes(rows, cols):
 
 @pytest.mark.parametrize("rows,cols", [(5120, 5120), (1024, 5120), (5120, 27648), (152064, 5120)])
 def test_q4_k_gemv_at_the_32b_shapes(rows, cols):
-    """Qwen2.5-32B widths: 5120 columns = 20 super-blocks (two waves of 16 + 4 per row), 27648 = 108; batch 1 (integer-dot
+    """Qwen2.5-32B widths: 5120 columns = 20 super-blocks (five waves of 4 super-blocks x 4 rows), 27648 = 108; batch 1 (integer-dot
     kernel) and batch 8 (matrix-core small-batch kernel); bias included."""
     from helpers.device import dev, rel_err
     cai = dev()

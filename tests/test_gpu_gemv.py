@@ -20,7 +20,8 @@ def make(qt, rows, cols, seed):
 
 
 @pytest.mark.parametrize("qt", [O.Q4_K, O.Q8_0, O.Q4_0])
-@pytest.mark.parametrize("rows,cols", [(2048, 2048), (5632, 2048), (2048, 5632), (3, 256), (1, 9728), (1000, 3584), (64, 18944), (40000, 512)])
+@pytest.mark.parametrize("rows,cols", [(2048, 2048), (5632, 2048), (2048, 5632), (3, 256), (1, 9728), (1000, 3584), (64, 18944), (40000, 512),
+                                       (1001, 4352), (77, 6144), (3, 5120), (4099, 5120)])   # 17..24 super-blocks: four rows packed per wave
 @pytest.mark.parametrize("nb", [1, 4])
 def test_gemv_matches_oracle(qt, rows, cols, nb):
     from helpers.device import dev, rel_err

@@ -44,7 +44,7 @@ def test_random_bytes_bit_exact(qt):
 
 
 @pytest.mark.parametrize("qt", RAW)
-@pytest.mark.parametrize("rows,cols", [(2048, 2048), (3, 256), (1, 9728), (1000, 3584), (64, 18944)])
+@pytest.mark.parametrize("rows,cols", [(2048, 2048), (3, 256), (1, 9728), (1000, 3584), (64, 18944), (1001, 5120), (77, 4352)])
 def test_gemv_matches_oracle(qt, rows, cols):
     from helpers.device import dev, rel_err
     cai = dev()
