@@ -322,13 +322,17 @@ def main():
     rng = np.random.default_rng(424242)
     prompt = rng.integers(0, cfg["vocab"], prompt_len).astype(np.int32)
     lib = cai.load()
-    pf_ms = C.c_float(0)
+    pf_ms = C.c_float(0); pf_first_ms = C.c_float(0)
     if prompt_len > 1:
-        dec.prefill(prompt[:min(8, prompt_len - 1)], 0, want_logits=False)   # warm the prefill kernels and buffers
+        dec.prefill(prompt[:min(8, prompt_len - 1)], 0, want_logits=False)   # warm the prefill kernels
         dec.reset()
-        cai.check(lib.cai_sync()); cai.check(lib.cai_timer_start())
-        dec.prefill(prompt[:-1], 0, want_logits=False)
-        cai.check(lib.cai_timer_stop(C.byref(pf_ms)))
+        # the first prompt of this length also grows the library's prompt workspaces (device allocations); the second
+        # pass over the same tokens is the steady state a serving process sees, and the one reported
+        for ms in (pf_first_ms, pf_ms):
+            dec.reset()
+            cai.check(lib.cai_sync()); cai.check(lib.cai_timer_start())
+            dec.prefill(prompt[:-1], 0, want_logits=False)
+            cai.check(lib.cai_timer_stop(C.byref(ms)))
         for b in range(1, B):
             dec.prefill(prompt[:-1], 0, seq=b, want_logits=False)
     tok = int(prompt[-1]); pos = prompt_len - 1
@@ -444,7 +448,7 @@ def main():
                    "algorithmic_bytes_per_step": int(algo_bytes), "hip_event_ms_per_step": round(ms.value / K, 4),
                    "whole_step_hbm_frac": round(algo_bytes / (wall / K) / 1e9 / HBM_PEAK_GBS, 4), "device": cai.device_name(),
                    "build_s": round(t_build, 1),
-                   "prefill": {"tokens": prompt_len - 1, "ms": round(pf_ms.value, 2),
+                   "prefill": {"tokens": prompt_len - 1, "ms": round(pf_ms.value, 2), "first_pass_ms": round(pf_first_ms.value, 2),
                                "tok_per_s": round((prompt_len - 1) / max(pf_ms.value, 1e-6) * 1e3, 1),
                                "linear_tflops": round(2.0 * n_lin_weights * (prompt_len - 1) / max(pf_ms.value, 1e-6) / 1e9, 1),
                                "note": "multi-token ingestion: f16 MFMA (exact scale*nibble weight operand, hi/lo-split activations = 2 MFMA passes per useful FLOP) + prompt attention; MFMA f16 dense peak 2500 TFLOP/s"}},

@@ -29,7 +29,7 @@ struct cai_decoder_s {
   float *px = nullptr, *pqkv = nullptr, *patt = nullptr, *pgu = nullptr, *pmid = nullptr, *ppart = nullptr;
   int32_t* ptokpos = nullptr;                        // [2][pf_cap]: tokens, positions
   // mixture-of-experts prompt: per chunk the router outputs, the slots grouped by expert and the per-slot activations
-  float *pm_logits = nullptr, *pm_probs = nullptr, *pm_gate = nullptr, *pm_gu = nullptr, *pm_mid = nullptr, *pm_part = nullptr;
+  float *pm_logits = nullptr, *pm_probs = nullptr, *pm_gate = nullptr, *pm_gu = nullptr, *pm_part = nullptr;
   int32_t *pm_expert = nullptr, *pm_perm = nullptr, *pm_tiles = nullptr;
   int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_argmax = nullptr, *d_gen = nullptr;
   int32_t* h_io = nullptr;   // pinned: tokens[8] pos[8] argmax[8]
@@ -233,9 +233,9 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = 
 // its own position.  Equals n sequential steps (the reference's prefill, neural/neuralchatengine.pas:1466-1470).
 static void free_moe_prompt(cai_decoder_s* d)
 {
-  void* q[] = {d->pm_logits, d->pm_probs, d->pm_gate, d->pm_gu, d->pm_mid, d->pm_part, d->pm_expert, d->pm_perm, d->pm_tiles};
+  void* q[] = {d->pm_logits, d->pm_probs, d->pm_gate, d->pm_gu, d->pm_part, d->pm_expert, d->pm_perm, d->pm_tiles};
   for (void* v : q) if (v) (void)hipFree(v);
-  d->pm_logits = d->pm_probs = d->pm_gate = d->pm_gu = d->pm_mid = d->pm_part = nullptr;
+  d->pm_logits = d->pm_probs = d->pm_gate = d->pm_gu = d->pm_part = nullptr;
   d->pm_expert = d->pm_perm = d->pm_tiles = nullptr;
 }
 
@@ -262,7 +262,7 @@ static int ensure_prefill_buffers(cai_decoder_s* d, int n)
     CAI_HIP(hipMalloc((void**)&d->pm_logits, (size_t)cap * E * 4)); CAI_HIP(hipMalloc((void**)&d->pm_probs, (size_t)cap * E * 4));
     CAI_HIP(hipMalloc((void**)&d->pm_gate, S * 4)); CAI_HIP(hipMalloc((void**)&d->pm_expert, S * 4)); CAI_HIP(hipMalloc((void**)&d->pm_perm, S * 4));
     CAI_HIP(hipMalloc((void**)&d->pm_tiles, (size_t)moe_group_max_tiles((int)S, c.n_experts) * 3 * 4));
-    CAI_HIP(hipMalloc((void**)&d->pm_gu, S * 2 * c.ffn * 4)); CAI_HIP(hipMalloc((void**)&d->pm_mid, S * c.ffn * 4)); CAI_HIP(hipMalloc((void**)&d->pm_part, S * c.d_model * 4));
+    CAI_HIP(hipMalloc((void**)&d->pm_gu, S * 2 * c.ffn * 4)); CAI_HIP(hipMalloc((void**)&d->pm_part, S * c.d_model * 4));
   }
   d->pf_cap = cap;
   return CAI_OK;
@@ -286,8 +286,7 @@ static int moe_ffn_prompt(cai_decoder_s* d, const cai_decoder_s::Layer& L, int n
   if ((rc = prefill_prep(d->px, dm, L.v[CAI_V_MLP_NORM], c.eps, dm, n))) return rc;
   prefill_planes(&hi, &lo, &sinv);
   if ((rc = launch_gemm_blk_grouped(L.w[CAI_W_GATEUP], 2 * (int64_t)I, hi, lo, sinv, K, slots, E, d->pm_perm, d->pm_tiles, d->pm_gu, 2 * I))) return rc;
-  launch_swiglu(d->pm_gu, I, slots, d->pm_mid);
-  if ((rc = prefill_prep(d->pm_mid, I, nullptr, 0.0f, I, slots))) return rc;
+  if ((rc = prefill_prep_swiglu(d->pm_gu, 2 * I, I, slots))) return rc;   // SwiGLU inside the pre-pass of the down projection
   prefill_planes(&hi, &lo, &sinv);
   if ((rc = launch_gemm_blk_grouped(L.w[CAI_W_DOWN], dm, hi, lo, sinv, 1, slots, E, d->pm_perm, d->pm_tiles, d->pm_part, dm))) return rc;
   return launch_moe_combine(d->px, d->pm_part, d->pm_gate, K, dm, n);
@@ -318,9 +317,14 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
     const cai_qw_s* wq = L.w[CAI_W_Q]; const cai_qw_s* wk = L.w[CAI_W_K]; const cai_qw_s* wv = L.w[CAI_W_V];
     const bool all_mfma = prompt_route(wq, n) == 2 && prompt_route(wk, n) == 2 && prompt_route(wv, n) == 2;   // one pre-pass serves q, k and v
     if (all_mfma && (rc = prefill_prep(d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, dm, n))) return rc;
-    if ((rc = linear_rows(wq, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv, qkvw, nullptr))) return rc;
-    if ((rc = linear_rows(wk, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw, qkvw, nullptr))) return rc;
-    if ((rc = linear_rows(wv, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw + kw, qkvw, nullptr))) return rc;
+    const cai_qw_s* qkv3[3] = {wq, wk, wv}; const int qkv_off[3] = {0, qw, qw + kw};
+    if (all_mfma && gemm_q4k_multi_supported(qkv3, 3)) {   // one launch: the k and v projections alone leave half the chip idle
+      if ((rc = prefill_gemm_multi(qkv3, qkv_off, 3, n, d->pqkv, qkvw))) return rc;
+    } else {
+      if ((rc = linear_rows(wq, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv, qkvw, nullptr))) return rc;
+      if ((rc = linear_rows(wk, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw, qkvw, nullptr))) return rc;
+      if ((rc = linear_rows(wv, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw + kw, qkvw, nullptr))) return rc;
+    }
     if ((rc = launch_attn_step(&d->kv, l, d->pqkv, qkvw, n, c.n_q_heads, c.window, 0.0f, d->theta, poss, d->patt, qw, seq, 1, d->ppart,
                                c.qk_norm_full ? L.v[CAI_V_Q_NORM] : nullptr, c.qk_norm_full ? L.v[CAI_V_K_NORM] : nullptr, c.eps))) return rc;
     if ((rc = linear_rows(L.w[CAI_W_O], false, d->patt, qw, nullptr, 0.0f, n, d->px, dm, d->px))) return rc;
@@ -337,9 +341,21 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
         if ((rc = moe_ffn_rows(d, L, d->px + (int64_t)t0 * dm, std::min(grp, n - t0)))) return rc;
       continue;
     }
+    if (prompt_route(L.w[CAI_W_GATEUP], n) == 2 && prefill_gemm_swiglu_supported(L.w[CAI_W_GATEUP], n)) {
+      // SwiGLU in the epilogue of the gate|up product: a wave holds 32 up rows and their gate rows
+      if ((rc = prefill_prep(d->px, dm, L.v[CAI_V_MLP_NORM], c.eps, dm, n))) return rc;
+      if ((rc = prefill_gemm_swiglu(L.w[CAI_W_GATEUP], n, d->pmid, I))) return rc;
+      if ((rc = linear_rows(L.w[CAI_W_DOWN], false, d->pmid, I, nullptr, 0.0f, n, d->px, dm, d->px))) return rc;
+      continue;
+    }
     if ((rc = linear_rows(L.w[CAI_W_GATEUP], false, d->px, dm, L.v[CAI_V_MLP_NORM], c.eps, n, d->pgu, 2 * I, nullptr))) return rc;
-    launch_swiglu(d->pgu, I, n, d->pmid);
-    if ((rc = linear_rows(L.w[CAI_W_DOWN], false, d->pmid, I, nullptr, 0.0f, n, d->px, dm, d->px))) return rc;
+    if (prompt_route(L.w[CAI_W_DOWN], n) == 2) {   // SwiGLU inside the activation pre-pass of the down projection
+      if ((rc = prefill_prep_swiglu(d->pgu, 2 * I, I, n))) return rc;
+      if ((rc = linear_rows(L.w[CAI_W_DOWN], true, nullptr, I, nullptr, 0.0f, n, d->px, dm, d->px))) return rc;
+    } else {
+      launch_swiglu(d->pgu, I, n, d->pmid);
+      if ((rc = linear_rows(L.w[CAI_W_DOWN], false, d->pmid, I, nullptr, 0.0f, n, d->px, dm, d->px))) return rc;
+    }
   }
   return CAI_OK;
 }

@@ -230,8 +230,14 @@ int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok);
 int nb_reduce(float* y, int64_t y_stride, const float* residual);
 int nb_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok, float* y, int64_t y_stride, const float* residual);
 int prefill_prep(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok);
+int prefill_prep_swiglu(const float* gu, int64_t gu_stride, int half, int n_tok);   // planes <- up * silu(gate)
 int prefill_gemm(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride, const float* residual);
 int prefill_gemm_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, float* y, int64_t y_stride);
+bool gemm_q4k_multi_supported(const cai_qw_s* const* ws, int n_w);
+int launch_gemm_q4k_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, const _Float16* xhi, const _Float16* xlo, const _Float16* sxhi,
+                          const _Float16* sxlo, const float* sinv, int n_tok, float* y, int64_t y_stride, const float* residual, int swiglu_half);
+bool prefill_gemm_swiglu_supported(const cai_qw_s* w, int n_tok);
+int prefill_gemm_swiglu(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride);   // y[t][i] = up_i * silu(gate_i), on the planes of the last prefill_prep
 
 void rope_thetas(float base, int head_dim, std::vector<float>& out);
 int  rope_thetas_scaled(float base, int head_dim, int mode, float factor, int original_ctx, float low_freq_factor, float high_freq_factor, std::vector<float>& out);

@@ -24,34 +24,44 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 // Activation pre-pass (one work-group per token): optional RMSNorm (neural/neural.cl:1047-1085), then
 //   s = 2^e with max|x|*s in [2^13, 2^14),  hi = f16(x*s),  lo = f16(x*s - hi),
 //   sxhi[b] + sxlo[b] = (sum of x over 32-block b) * s / 32 as two halfs (the block sums go to the matrix cores too).
+// SWIGLU: the row holds up | gate (K values each) and the value is up * silu(gate) - the feed-forward's middle step folded into
+// the pre-pass of the down projection (no norm in that case).
 // ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void xprep_kernel(const float* x, int64_t x_stride, const float* gain, float eps, int K,
+template <bool SWIGLU, int NT>     // NT threads per token
+__global__ __launch_bounds__(NT) void xprep_kernel(const float* x, int64_t x_stride, const float* gain, float eps, int K,
                                                     _Float16* hi, _Float16* lo, float* sinv, _Float16* sxhi, _Float16* sxlo)
 {
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const float* xr = x + (int64_t)t * x_stride;
-  __shared__ float red[4];
+  __shared__ float red[NT / 64];
   __shared__ float s_scale;
   float inv = 1.0f;
-  if (gain) {
+  const float* second = SWIGLU ? xr + K : gain;     // the array walked beside x: the gate half, or the norm gain
+  if (!SWIGLU && gain) {
     float ss = 0.0f;
-    for_strided8(xr, threadIdx.x, K, 256, [&](float v, int) { ss = fmaf(v, v, ss); });
+    for_strided8(xr, threadIdx.x, K, NT, [&](float v, int) { ss = fmaf(v, v, ss); });
     ss = wave_sum(ss);
     if (lane == 63) red[wave] = ss;
     __syncthreads();
-    inv = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)K + eps);
+    float tot = 0.0f;
+#pragma unroll
+    for (int w4 = 0; w4 < NT / 64; w4 += 4) tot += (red[w4] + red[w4 + 1]) + (red[w4 + 2] + red[w4 + 3]);
+    inv = 1.0f / sqrtf(tot / (float)K + eps);
     __syncthreads();
   }
   float amax = 0.0f;
-  for_strided8(xr, gain, threadIdx.x, K, 256, [&](float v, float g, int) {
-    if (gain) v = g * (v * inv);
+  for_strided8(xr, second, threadIdx.x, K, NT, [&](float v, float g, int) {
+    if (SWIGLU) v = silu_mul(v, g);
+    else if (gain) v = g * (v * inv);
     amax = fmaxf(amax, fabsf(v));
   });
   for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
   if (lane == 0) red[wave] = amax;
   __syncthreads();
   if (threadIdx.x == 0) {
-    const float a = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float a = 0.0f;
+#pragma unroll
+    for (int w4 = 0; w4 < NT / 64; w4++) a = fmaxf(a, red[w4]);
     int e = 0;
     if (a > 0.0f && a < 3.0e38f) { int ex; frexpf(a, &ex); e = 14 - ex; }   // a = m*2^ex, m in [0.5,1) -> a*2^e in [2^13, 2^14)
     if (e > 60) e = 60; if (e < -60) e = -60;
@@ -61,8 +71,9 @@ __global__ __launch_bounds__(256) void xprep_kernel(const float* x, int64_t x_st
   __syncthreads();
   const float s = s_scale;
   // one 32-block per half-wave and turn (thread i of a turn takes element turn * 256 + i): 8 blocks per work-group turn
-  for_strided8(xr, gain, threadIdx.x, K, 256, [&](float v, float g, int i) {
-    if (gain) v = g * (v * inv);
+  for_strided8(xr, second, threadIdx.x, K, NT, [&](float v, float g, int i) {
+    if (SWIGLU) v = silu_mul(v, g);
+    else if (gain) v = g * (v * inv);
     const float vs = v * s;
     _Float16 h, l; split_f16(vs, h, l);
     hi[(int64_t)t * K + i] = h; lo[(int64_t)t * K + i] = l;
@@ -76,6 +87,88 @@ __global__ __launch_bounds__(256) void xprep_kernel(const float* x, int64_t x_st
   });
 }
 
+// The same pre-pass for rows of at most KE * NT values: every thread keeps its KE values in registers, so the row is read
+// once (the general kernel above reads it for the sum of squares, for the maximum and for the conversion) and SwiGLU is
+// evaluated once.  Thread i takes elements i, i + NT, ...: the order of every sum is that of the general kernel.
+template <bool SWIGLU, int NT, int KE>
+__global__ __launch_bounds__(NT) void xprep_regs_kernel(const float* x, int64_t x_stride, const float* gain, float eps, int K,
+                                                         _Float16* hi, _Float16* lo, float* sinv, _Float16* sxhi, _Float16* sxlo)
+{
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const float* xr = x + (int64_t)t * x_stride;
+  const float* second = SWIGLU ? xr + K : gain;
+  __shared__ float red[NT / 64];
+  __shared__ float s_scale;
+  float v[KE], g[KE];
+#pragma unroll
+  for (int e = 0; e < KE; e++) {                    // requests carry no branch: past the end the last value again (not used)
+    const int j = min((int)threadIdx.x + e * NT, K - 1);
+    v[e] = xr[j]; g[e] = second ? second[j] : 1.0f;
+  }
+  if (!SWIGLU && gain) {
+    float ss = 0.0f;
+#pragma unroll
+    for (int e = 0; e < KE; e++) if ((int)threadIdx.x + e * NT < K) ss = fmaf(v[e], v[e], ss);
+    ss = wave_sum(ss);
+    if (lane == 63) red[wave] = ss;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int w4 = 0; w4 < NT / 64; w4 += 4) tot += (red[w4] + red[w4 + 1]) + (red[w4 + 2] + red[w4 + 3]);
+    const float inv = 1.0f / sqrtf(tot / (float)K + eps);
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < KE; e++) v[e] = g[e] * (v[e] * inv);
+  } else if (SWIGLU) {
+#pragma unroll
+    for (int e = 0; e < KE; e++) v[e] = silu_mul(v[e], g[e]);
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int e = 0; e < KE; e++) if ((int)threadIdx.x + e * NT < K) amax = fmaxf(amax, fabsf(v[e]));
+  for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+  if (lane == 0) red[wave] = amax;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float a = 0.0f;
+#pragma unroll
+    for (int w4 = 0; w4 < NT / 64; w4++) a = fmaxf(a, red[w4]);
+    int ex2 = 0;
+    if (a > 0.0f && a < 3.0e38f) { int ex; frexpf(a, &ex); ex2 = 14 - ex; }
+    if (ex2 > 60) ex2 = 60; if (ex2 < -60) ex2 = -60;
+    s_scale = ldexpf(1.0f, ex2);
+    sinv[t] = ldexpf(1.0f, -ex2);
+  }
+  __syncthreads();
+  const float s = s_scale;
+#pragma unroll
+  for (int e = 0; e < KE; e++) {
+    const int i = (int)threadIdx.x + e * NT;
+    if (i < K) {                                    // K is a multiple of 32: a half-wave is inside or outside together
+      const float vs = v[e] * s;
+      _Float16 h, l; split_f16(vs, h, l);
+      hi[(int64_t)t * K + i] = h; lo[(int64_t)t * K + i] = l;
+      float sum = v[e];
+      for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+      if ((i & 31) == 0) {
+        const float ss = sum * s * 0.03125f;
+        _Float16 sh, sl; split_f16(ss, sh, sl);
+        sxhi[(int64_t)t * (K >> 5) + (i >> 5)] = sh; sxlo[(int64_t)t * (K >> 5) + (i >> 5)] = sl;
+      }
+    }
+  }
+}
+
+template <bool SWIGLU>
+static void xprep_launch(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok,
+                         _Float16* hi, _Float16* lo, float* sinv, _Float16* sxhi, _Float16* sxlo)
+{
+  hipStream_t st = ctx().stream;
+  if (K <= 16 * 256) hipLaunchKernelGGL((xprep_regs_kernel<SWIGLU, 256, 16>), dim3(n_tok), dim3(256), 0, st, x, x_stride, gain, eps, K, hi, lo, sinv, sxhi, sxlo);
+  else if (K <= 24 * 1024) hipLaunchKernelGGL((xprep_regs_kernel<SWIGLU, 1024, 24>), dim3(n_tok), dim3(1024), 0, st, x, x_stride, gain, eps, K, hi, lo, sinv, sxhi, sxlo);
+  else hipLaunchKernelGGL((xprep_kernel<SWIGLU, 1024>), dim3(n_tok), dim3(1024), 0, st, x, x_stride, gain, eps, K, hi, lo, sinv, sxhi, sxlo);
+}
+
 struct GemmParams {
   const uint8_t* w; const uint8_t* aux; const uint8_t* aux2; const float* bias;   // aux, aux2: Q6_K planes of scales and of d
   int rows, cols;
@@ -86,6 +179,13 @@ struct GemmParams {
   float* y; int64_t y_stride;       // y[t*y_stride + row]
   const float* residual;            // same indexing as y, may alias y
   int n_row_groups, n_tok_tiles;
+  // up to two more matrices of the same type and width in the same launch (q | k | v): row groups [seg_end[i], ...) belong to
+  // matrix i + 1, whose rows land y_off2[i] columns into a y row (gemm_q4k_pf only)
+  int n_seg; int seg_end[2];
+  const uint8_t* w2[2]; const float* bias2[2]; int rows2[2]; int y_off2[2];
+  // fused feed-forward front half (gemm_q4k_pf with two row tiles per wave): rows [0, half) are up, [half, 2 half) gate; a wave's
+  // two tiles are 32 up rows and THEIR gate rows, and y[t][i] = up_i * silu(gate_i) is written (y rows are half wide)
+  int swiglu_half;
 };
 
 constexpr int PF_LDX = 264;       // halfs per staged token row: 256 + pad (stride = 4 banks mod 64: 16-byte reads)
@@ -131,12 +231,19 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
   // linear id = rg_lo + 8 * (tt + n_tok_tiles * rg_hi): a row group's token tiles share id mod 8
   const int L = blockIdx.x, rg = (L & 7) + 8 * ((L >> 3) / p.n_tok_tiles), ttile = (L >> 3) % p.n_tok_tiles;
   if (rg >= p.n_row_groups) return;
-  const int R0 = (rg * 4 + wave) * 32 * RT, T0 = ttile * NTOK;
+  const uint8_t* wbase = p.w; const float* bias = p.bias; int rows = p.rows, yo = 0, rgl = rg;   // this work-group's matrix (uniform)
+  if (p.n_seg > 1 && rg >= p.seg_end[0]) { wbase = p.w2[0]; bias = p.bias2[0]; rows = p.rows2[0]; yo = p.y_off2[0]; rgl = rg - p.seg_end[0]; }
+  if (p.n_seg > 2 && rg >= p.seg_end[1]) { wbase = p.w2[1]; bias = p.bias2[1]; rows = p.rows2[1]; yo = p.y_off2[1]; rgl = rg - p.seg_end[1]; }
+  const int half = RT == 2 ? p.swiglu_half : 0;
+  const int R0 = half ? (rgl * 4 + wave) * 32 : (rgl * 4 + wave) * 32 * RT, T0 = ttile * NTOK;
   const int K = p.cols, nsb = K >> 8, nb32 = K >> 5;
   const int64_t row_bytes = (int64_t)nsb * BB;
   const uint8_t* wrow[RT];
 #pragma unroll
-  for (int rt = 0; rt < RT; rt++) wrow[rt] = p.w + (int64_t)min(R0 + 32 * rt + n, p.rows - 1) * row_bytes;   // tail rows: re-read the last row, not written
+  for (int rt = 0; rt < RT; rt++) {     // tail rows: re-read the last row, not written
+    const int row = half ? min(R0 + n, half - 1) + rt * half : min(R0 + 32 * rt + n, rows - 1);
+    wrow[rt] = wbase + (int64_t)row * row_bytes;
+  }
 
   struct WRegs { uint4 h, q[4], e[QT == CAI_Q5_K ? 2 : 1]; };   // e: Q5_K's bit plane (all 32 bytes: the lane needs four bits of each)
   auto load_w = [&](int sb, WRegs (&r)[RT]) {
@@ -284,8 +391,34 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
 
   // ---- write: lane holds column (token) n of each tile and rows 8g + 4kg + (0..3): four consecutive outputs of a token
   // row go out as one 16-byte store (bias and residual come in the same way) when the addresses allow it ----
-  const bool vec = (p.y_stride & 3) == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 &&
-                   (!p.residual || (reinterpret_cast<uintptr_t>(p.residual) & 15) == 0) && (!p.bias || (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0);
+  const bool vec = ((p.y_stride | yo) & 3) == 0 && (reinterpret_cast<uintptr_t>(p.y) & 15) == 0 &&
+                   (!p.residual || (reinterpret_cast<uintptr_t>(p.residual) & 15) == 0) && (!bias || (reinterpret_cast<uintptr_t>(bias) & 15) == 0);
+  if constexpr (RT == 2) if (half) {
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++) {
+      const int t = T0 + tt * 32 + n;
+      if (t >= p.n_tok) continue;
+      const float si = p.sinv[t];
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const int row = R0 + 8 * g + 4 * kg;
+        const int64_t o = (int64_t)t * p.y_stride + row;
+        float r[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          float up = Y[0][tt][4 * g + i] * si, gate = Y[1][tt][4 * g + i] * si;
+          if (bias && row + i < half) { up += bias[row + i]; gate += bias[half + row + i]; }
+          r[i] = silu_mul(up, gate);
+        }
+        if (vec && row + 3 < half) *reinterpret_cast<float4*>(p.y + o) = make_float4(r[0], r[1], r[2], r[3]);
+        else {
+#pragma unroll
+          for (int i = 0; i < 4; i++) if (row + i < half) p.y[o + i] = r[i];
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int tt = 0; tt < TT; tt++) {
     const int t = T0 + tt * 32 + n;
@@ -296,18 +429,18 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_pf(const GemmParams p)
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         const int row = R0 + 32 * rt + 8 * g + 4 * kg;
-        const int64_t o = (int64_t)t * p.y_stride + row;
-        if (vec && row + 3 < p.rows) {
+        const int64_t o = (int64_t)t * p.y_stride + yo + row;
+        if (vec && row + 3 < rows) {
           float4 r = make_float4(Y[rt][tt][4 * g] * si, Y[rt][tt][4 * g + 1] * si, Y[rt][tt][4 * g + 2] * si, Y[rt][tt][4 * g + 3] * si);
-          if (p.bias) { const float4 b = *reinterpret_cast<const float4*>(p.bias + row); r.x += b.x; r.y += b.y; r.z += b.z; r.w += b.w; }
+          if (bias) { const float4 b = *reinterpret_cast<const float4*>(bias + row); r.x += b.x; r.y += b.y; r.z += b.z; r.w += b.w; }
           if (p.residual) { const float4 q = *reinterpret_cast<const float4*>(p.residual + o); r.x += q.x; r.y += q.y; r.z += q.z; r.w += q.w; }
           *reinterpret_cast<float4*>(p.y + o) = r;
         } else {
 #pragma unroll
           for (int i = 0; i < 4; i++) {
-            if (row + i >= p.rows) continue;
+            if (row + i >= rows) continue;
             float r = Y[rt][tt][4 * g + i] * si;
-            if (p.bias) r += p.bias[row + i];
+            if (bias) r += bias[row + i];
             if (p.residual) r += p.residual[o + i];
             p.y[o + i] = r;
           }
@@ -470,7 +603,7 @@ __global__ __launch_bounds__(256, 2) void gemm_q6k_pf(const GemmParams p)
 int launch_xprep(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok,
                  _Float16* hi, _Float16* lo, float* sinv, _Float16* sxhi, _Float16* sxlo)
 {
-  hipLaunchKernelGGL(xprep_kernel, dim3(n_tok), dim3(256), 0, ctx().stream, x, x_stride, gain, eps, K, hi, lo, sinv, sxhi, sxlo);
+  xprep_launch<false>(x, x_stride, gain, eps, K, n_tok, hi, lo, sinv, sxhi, sxlo);
   return CAI_OK;
 }
 
@@ -479,11 +612,34 @@ bool gemm_mfma_supported(const cai_qw_s* w) { return (w->qtype == CAI_Q4_K || w-
 int launch_gemm_q4k(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo, const _Float16* sxhi, const _Float16* sxlo, const float* sinv,
                     int n_tok, float* y, int64_t y_stride, const float* residual)
 {
+  const int zero = 0;
+  return launch_gemm_q4k_multi(&w, &zero, 1, xhi, xlo, sxhi, sxlo, sinv, n_tok, y, y_stride, residual, 0);
+}
+
+// Matrices of one type and width that one launch of the Q4_K / Q5_K prompt kernel can take together
+bool gemm_q4k_multi_supported(const cai_qw_s* const* ws, int n_w)
+{
+  if (n_w < 1 || n_w > 3 || !gemm_mfma_supported(ws[0]) || ws[0]->qtype == CAI_Q6_K) return false;
+  for (int i = 1; i < n_w; i++) if (ws[i]->qtype != ws[0]->qtype || ws[i]->cols != ws[0]->cols) return false;
+  return true;
+}
+
+// y[t][y_off[i] + r] = (W_i x[t])[r] (+ bias_i) for up to three matrices of one type and width; one matrix: y_off[0] = 0, residual allowed.
+// swiglu_half != 0 (one matrix of 2 * swiglu_half rows, no residual): y[t][i] = up_i * silu(gate_i), y rows swiglu_half wide.
+int launch_gemm_q4k_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, const _Float16* xhi, const _Float16* xlo, const _Float16* sxhi,
+                          const _Float16* sxlo, const float* sinv, int n_tok, float* y, int64_t y_stride, const float* residual, int swiglu_half)
+{
+  const cai_qw_s* w = ws[0];
   if (!gemm_mfma_supported(w)) return set_error(CAI_ERR_UNSUPPORTED, "prefill gemm: weight type %d", w->qtype);
+  if (n_w > 1 && (!gemm_q4k_multi_supported(ws, n_w) || residual)) return set_error(CAI_ERR_UNSUPPORTED, "prefill gemm: %d matrices in one launch", n_w);
+  if (swiglu_half && (n_w != 1 || residual || w->qtype == CAI_Q6_K || w->rows != 2 * (int64_t)swiglu_half))
+    return set_error(CAI_ERR_UNSUPPORTED, "prefill gemm: fused SwiGLU needs one Q4_K / Q5_K matrix of 2 x %d rows", swiglu_half);
   GemmParams p{};
   p.w = w->data; p.bias = w->bias; p.rows = (int)w->rows; p.cols = (int)w->cols;
-  p.xhi = xhi; p.xlo = xlo; p.sxhi = sxhi; p.sxlo = sxlo; p.sinv = sinv; p.n_tok = n_tok; p.y = y; p.y_stride = y_stride;
-  p.residual = residual;
+  p.xhi = xhi; p.xlo = xlo; p.sxhi = sxhi; p.sxlo = sxlo; p.sinv = sinv; p.n_tok = n_tok; p.y = y + y_off[0]; p.y_stride = y_stride;
+  p.residual = residual; p.n_seg = n_w;
+  int64_t rows_all = 0;
+  for (int i = 0; i < n_w; i++) rows_all += ws[i]->rows;
   if (w->qtype == CAI_Q6_K) {
     p.aux = w->aux; p.aux2 = qw_aux2(w);
     const int tt = ((p.rows + 127) / 128) * ((n_tok + 63) / 64) < 2 * ctx().n_cu ? 1 : 2;
@@ -504,11 +660,17 @@ int launch_gemm_q4k(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo,
   // Tiling: two row tiles per wave (256 rows per work-group, 32 tokens) when that still gives every CU several
   // work-groups; else 128 rows with two token tiles, or with one for matrices with few row groups.
   const int n_cu = ctx().n_cu;
-  const int wgs_rt2 = ((p.rows + 255) / 256) * ((n_tok + 31) / 32);
-  const int wgs_tt2 = ((p.rows + 127) / 128) * ((n_tok + 63) / 64);
-  const int mode = wgs_rt2 >= 4 * n_cu ? 3 : (wgs_tt2 < 2 * n_cu ? 1 : 2);   // 1, 2: token tiles; 3: two row tiles
+  const int wgs_rt2 = (int)((rows_all + 255) / 256) * ((n_tok + 31) / 32);
+  const int wgs_tt2 = (int)((rows_all + 127) / 128) * ((n_tok + 63) / 64);
+  const int mode = (swiglu_half || wgs_rt2 >= 4 * n_cu) ? 3 : (wgs_tt2 < 2 * n_cu ? 1 : 2);   // 1, 2: token tiles; 3: two row tiles
   const int rt = mode == 3 ? 2 : 1, tt = mode == 2 ? 2 : 1;
-  p.n_row_groups = (p.rows + 128 * rt - 1) / (128 * rt);
+  p.swiglu_half = swiglu_half;
+  p.n_row_groups = 0;
+  for (int i = 0; i < n_w; i++) {       // every matrix starts a row group of its own
+    if (i > 0) { p.seg_end[i - 1] = p.n_row_groups; p.w2[i - 1] = ws[i]->data; p.bias2[i - 1] = ws[i]->bias; p.rows2[i - 1] = (int)ws[i]->rows; p.y_off2[i - 1] = y_off[i] - y_off[0]; }
+    p.n_row_groups += (int)((ws[i]->rows + 128 * rt - 1) / (128 * rt));
+  }
+  if (swiglu_half) p.n_row_groups = (swiglu_half + 127) / 128;   // 128 up rows and their gate rows per work-group
   p.n_tok_tiles = (n_tok + tt * 32 - 1) / (tt * 32);
   const size_t lds = (size_t)tt * 32 * (PF_LDX + 8) * 2 * 2 + (size_t)4 * rt * 2 * 32 * 4;
   static bool attr_done = false;
@@ -569,14 +731,35 @@ int prefill_prep(const float* x, int64_t x_stride, const float* gain, float eps,
   if ((rc = prefill_reserve(n_tok, K))) return rc;
   return launch_xprep(x, x_stride, gain, eps, K, n_tok, g_pws.hi, g_pws.lo, g_pws.sinv, g_pws.sxhi, g_pws.sxlo);
 }
+// planes <- up * silu(gate) of rows holding up | gate (half values each): the pre-pass of the down projection
+int prefill_prep_swiglu(const float* gu, int64_t gu_stride, int half, int n_tok)
+{
+  int rc;
+  if ((rc = prefill_reserve(n_tok, half))) return rc;
+  xprep_launch<true>(gu, gu_stride, nullptr, 0.0f, half, n_tok, g_pws.hi, g_pws.lo, g_pws.sinv, g_pws.sxhi, g_pws.sxlo);
+  return CAI_OK;
+}
 // Several matrices of one width applied to the prepared activations (q | k | v).
 int prefill_gemm_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, float* y, int64_t y_stride)
 {
+  if (n_w > 1 && gemm_q4k_multi_supported(ws, n_w))
+    return launch_gemm_q4k_multi(ws, y_off, n_w, g_pws.hi, g_pws.lo, g_pws.sxhi, g_pws.sxlo, g_pws.sinv, n_tok, y, y_stride, nullptr, 0);
   for (int i = 0; i < n_w; i++) {
     const int rc = prefill_gemm(ws[i], n_tok, y + y_off[i], y_stride, nullptr);
     if (rc) return rc;
   }
   return CAI_OK;
+}
+// y[t][i] = up_i * silu(gate_i) of the prepared activations through a gate|up matrix of 2 * half rows (Q4_K / Q5_K), one launch
+bool prefill_gemm_swiglu_supported(const cai_qw_s* w, int n_tok)
+{
+  // only where the product takes two row tiles per wave anyway (enough work-groups to fill the chip several times over)
+  return gemm_mfma_supported(w) && w->qtype != CAI_Q6_K && w->rows % 2 == 0 && (int)((w->rows + 255) / 256) * ((n_tok + 31) / 32) >= 4 * ctx().n_cu;
+}
+int prefill_gemm_swiglu(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride)
+{
+  const int zero = 0;
+  return launch_gemm_q4k_multi(&w, &zero, 1, g_pws.hi, g_pws.lo, g_pws.sxhi, g_pws.sxlo, g_pws.sinv, n_tok, y, y_stride, nullptr, (int)(w->rows / 2));
 }
 void prefill_planes(const _Float16** hi, const _Float16** lo, const float** sinv) { *hi = g_pws.hi; *lo = g_pws.lo; *sinv = g_pws.sinv; }
 int prefill_gemm(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride, const float* residual)
