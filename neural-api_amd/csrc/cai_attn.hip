@@ -809,6 +809,7 @@ __global__ __launch_bounds__(256) void kv_append_rows_i8_kernel(const AttnParams
 // Same arithmetic as the decode kernels up to the order of the sums (tests: < 1e-4 of token-at-a-time ingestion).
 // ------------------------------------------------------------------------------------------
 typedef _Float16 ph4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 ph8_t __attribute__((ext_vector_type(8)));
 typedef float pf16_t __attribute__((ext_vector_type(16)));
 
 struct PromptParams {
@@ -843,7 +844,7 @@ __global__ __launch_bounds__(256) void prompt_q_kernel(const PromptParams p)
   }
 }
 
-constexpr int PA_LDK = 132;    // halfs per staged K row (128 + pad: 8-byte reads of 32 rows tile the banks)
+constexpr int PA_LDK = 136;    // halfs per staged K row (128 + pad: rows stay 16-byte aligned for the 8-half operand reads)
 constexpr int PA_LDV = 36;     // halfs per staged V^T row (32 cached rows + pad)
 
 template <typename KV_T>
@@ -871,14 +872,14 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
   const KV_T* kc = reinterpret_cast<const KV_T*>(p.kc) + (int64_t)g * p.max_ctx * 128;
   const KV_T* vc = reinterpret_cast<const KV_T*>(p.vc) + (int64_t)g * p.max_ctx * 128;
 
-  // this lane's q fragments: token n, dims 8 s + 4 kg .. + 3 of the wave's head
-  ph4_t qh[16], ql[16];
+  // this lane's q fragments: token n, dims 16 s + 8 kg .. + 7 of the wave's head
+  ph8_t qh[8], ql[8];
   {
-    const int64_t qo = (int64_t)min(tok, p.n_tok - 1) * (p.q_heads * 128) + head * 128 + 4 * kg;
+    const int64_t qo = (int64_t)min(tok, p.n_tok - 1) * (p.q_heads * 128) + head * 128 + 8 * kg;
 #pragma unroll
-    for (int s = 0; s < 16; s++) {
-      qh[s] = *reinterpret_cast<const ph4_t*>(p.qhi + qo + 8 * s);
-      ql[s] = *reinterpret_cast<const ph4_t*>(p.qlo + qo + 8 * s);
+    for (int s = 0; s < 8; s++) {
+      qh[s] = *reinterpret_cast<const ph8_t*>(p.qhi + qo + 16 * s);
+      ql[s] = *reinterpret_cast<const ph8_t*>(p.qlo + qo + 16 * s);
     }
   }
   pf16_t O[4];
@@ -889,15 +890,39 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
   float m_run = -1e30f, l_run = 0.0f;
 
   const int srow = tid >> 3, sdim = (tid & 7) * 16;         // staging: 16 consecutive elements of one cached row
+  // The rows of the NEXT tile are requested before the products of the current one and converted into LDS after them: the
+  // memory round trip runs behind the matrix-core work instead of in front of it.  Requests are unconditional (rows past the
+  // live range are clamped and masked below).
+  struct RawTile { uint4 k[sizeof(KV_T) == 4 ? 4 : 2], v[sizeof(KV_T) == 4 ? 4 : 2]; float ks, vs; };   // (int8: one uint4 each is used)
+  auto fetch = [&](int jt, RawTile& r) {
+    const int j = min(jt * 32 + srow, p.max_ctx - 1);
+    if (I8P) {
+      r.k[0] = *reinterpret_cast<const uint4*>(reinterpret_cast<const int8_t*>(kc) + (int64_t)j * 128 + sdim);
+      r.v[0] = *reinterpret_cast<const uint4*>(reinterpret_cast<const int8_t*>(vc) + (int64_t)j * 128 + sdim);
+      r.ks = p.ksc[(int64_t)g * p.max_ctx + j]; r.vs = p.vsc[(int64_t)g * p.max_ctx + j];
+    } else if (sizeof(KV_T) == 4) {
+#pragma unroll
+      for (int c4 = 0; c4 < 4; c4++) {
+        r.k[c4] = *reinterpret_cast<const uint4*>(reinterpret_cast<const float*>(kc) + (int64_t)j * 128 + sdim + 4 * c4);
+        r.v[c4] = *reinterpret_cast<const uint4*>(reinterpret_cast<const float*>(vc) + (int64_t)j * 128 + sdim + 4 * c4);
+      }
+    } else {
+#pragma unroll
+      for (int c8 = 0; c8 < 2; c8++) {
+        r.k[c8] = *reinterpret_cast<const uint4*>(reinterpret_cast<const __half*>(kc) + (int64_t)j * 128 + sdim + 8 * c8);
+        r.v[c8] = *reinterpret_cast<const uint4*>(reinterpret_cast<const __half*>(vc) + (int64_t)j * 128 + sdim + 8 * c8);
+      }
+    }
+  };
+  RawTile raw;
+  fetch(j_lo >> 5, raw);
   for (int jt = j_lo >> 5; jt * 32 <= pos_last; jt++) {
     __syncthreads();                                        // the previous tile has been consumed
     {
-      const int j = min(jt * 32 + srow, p.max_ctx - 1);     // rows past the live range are masked below
       float kv[16], vv[16];
       if (I8P) {
-        const uint4 a = *reinterpret_cast<const uint4*>(reinterpret_cast<const int8_t*>(kc) + (int64_t)j * 128 + sdim);
-        const uint4 b = *reinterpret_cast<const uint4*>(reinterpret_cast<const int8_t*>(vc) + (int64_t)j * 128 + sdim);
-        const float ks = p.ksc[(int64_t)g * p.max_ctx + j], vs = p.vsc[(int64_t)g * p.max_ctx + j];
+        const uint4 a = raw.k[0], b = raw.v[0];
+        const float ks = raw.ks, vs = raw.vs;
         const int aw[4] = {(int)a.x, (int)a.y, (int)a.z, (int)a.w}, bw[4] = {(int)b.x, (int)b.y, (int)b.z, (int)b.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -909,25 +934,25 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
       } else if (sizeof(KV_T) == 4) {
 #pragma unroll
         for (int c4 = 0; c4 < 4; c4++) {
-          const float4 a = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(kc) + (int64_t)j * 128 + sdim + 4 * c4);
-          const float4 b = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(vc) + (int64_t)j * 128 + sdim + 4 * c4);
-          kv[4 * c4] = a.x; kv[4 * c4 + 1] = a.y; kv[4 * c4 + 2] = a.z; kv[4 * c4 + 3] = a.w;
-          vv[4 * c4] = b.x; vv[4 * c4 + 1] = b.y; vv[4 * c4 + 2] = b.z; vv[4 * c4 + 3] = b.w;
-        }
-      } else {
-#pragma unroll
-        for (int c8 = 0; c8 < 2; c8++) {
-          const uint4 a = *reinterpret_cast<const uint4*>(reinterpret_cast<const __half*>(kc) + (int64_t)j * 128 + sdim + 8 * c8);
-          const uint4 b = *reinterpret_cast<const uint4*>(reinterpret_cast<const __half*>(vc) + (int64_t)j * 128 + sdim + 8 * c8);
-          const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
-#pragma unroll
-          for (int i = 0; i < 4; i++) {
-            const __half2 ah = __builtin_bit_cast(__half2, aw[i]), bh = __builtin_bit_cast(__half2, bw[i]);
-            kv[8 * c8 + 2 * i] = __low2float(ah); kv[8 * c8 + 2 * i + 1] = __high2float(ah);
-            vv[8 * c8 + 2 * i] = __low2float(bh); vv[8 * c8 + 2 * i + 1] = __high2float(bh);
-          }
+          const uint4 a = raw.k[c4], b = raw.v[c4];
+          kv[4 * c4] = __builtin_bit_cast(float, a.x); kv[4 * c4 + 1] = __builtin_bit_cast(float, a.y); kv[4 * c4 + 2] = __builtin_bit_cast(float, a.z); kv[4 * c4 + 3] = __builtin_bit_cast(float, a.w);
+          vv[4 * c4] = __builtin_bit_cast(float, b.x); vv[4 * c4 + 1] = __builtin_bit_cast(float, b.y); vv[4 * c4 + 2] = __builtin_bit_cast(float, b.z); vv[4 * c4 + 3] = __builtin_bit_cast(float, b.w);
         }
       }
+      if constexpr (sizeof(KV_T) == 2) {                  // a half cache goes in as it is
+#pragma unroll
+        for (int c8 = 0; c8 < 2; c8++) {
+          const uint4 a = raw.k[c8], b = raw.v[c8];
+          *reinterpret_cast<uint2*>(&sK[0][srow * PA_LDK + sdim + 8 * c8]) = make_uint2(a.x, a.y);
+          *reinterpret_cast<uint2*>(&sK[0][srow * PA_LDK + sdim + 8 * c8 + 4]) = make_uint2(a.z, a.w);
+          const uint32_t bw[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            sV[0][(sdim + 8 * c8 + 2 * i) * PA_LDV + srow] = __builtin_bit_cast(_Float16, (unsigned short)(bw[i] & 0xffffu));
+            sV[0][(sdim + 8 * c8 + 2 * i + 1) * PA_LDV + srow] = __builtin_bit_cast(_Float16, (unsigned short)(bw[i] >> 16));
+          }
+        }
+      } else {
 #pragma unroll
       for (int i4 = 0; i4 < 4; i4++) {                    // K rows stay row-major: 8-byte stores
         ph4_t kh, kl;
@@ -942,7 +967,9 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
         sV[0][(sdim + i) * PA_LDV + srow] = vh;
         if (F32) sV[NP - 1][(sdim + i) * PA_LDV + srow] = vl;
       }
+      }
     }
+    fetch(jt + 1, raw);                                     // in flight during the products below
     __syncthreads();
     if (!head_on) continue;                                 // (an idle wave still stages and meets the barriers)
 
@@ -951,13 +978,13 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
 #pragma unroll
     for (int v = 0; v < 16; v++) C[v] = 0.0f;
 #pragma unroll
-    for (int s = 0; s < 16; s++) {
-      const ph4_t a = *reinterpret_cast<const ph4_t*>(&sK[0][n * PA_LDK + 8 * s + 4 * kg]);
-      C = __builtin_amdgcn_mfma_f32_32x32x8f16(a, qh[s], C, 0, 0, 0);
-      C = __builtin_amdgcn_mfma_f32_32x32x8f16(a, ql[s], C, 0, 0, 0);
+    for (int s = 0; s < 8; s++) {
+      const ph8_t a = *reinterpret_cast<const ph8_t*>(&sK[0][n * PA_LDK + 16 * s + 8 * kg]);
+      C = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qh[s], C, 0, 0, 0);
+      C = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, ql[s], C, 0, 0, 0);
       if (F32) {
-        const ph4_t al = *reinterpret_cast<const ph4_t*>(&sK[NP - 1][n * PA_LDK + 8 * s + 4 * kg]);
-        C = __builtin_amdgcn_mfma_f32_32x32x8f16(al, qh[s], C, 0, 0, 0);
+        const ph8_t al = *reinterpret_cast<const ph8_t*>(&sK[NP - 1][n * PA_LDK + 16 * s + 8 * kg]);
+        C = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, qh[s], C, 0, 0, 0);
       }
     }
     // ---- this token's column: mask, running maximum, weights ----
@@ -979,24 +1006,33 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
     for (int v = 0; v < 16; v++) { C[v] = ok[v] ? expf(C[v] - m_new) : 0.0f; psum += C[v]; }
     psum += __shfl_xor(psum, 32, 64);
     l_run = l_run * corr + psum; m_run = m_new;
+    if (__builtin_amdgcn_ballot_w64(corr != 1.0f)) {      // (after the first tiles a new maximum is rare: the whole wave skips the rescaling)
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++)
+      for (int dt = 0; dt < 4; dt++)
 #pragma unroll
-      for (int v = 0; v < 16; v++) O[dt][v] *= corr;
+        for (int v = 0; v < 16; v++) O[dt][v] *= corr;
+    }
     // ---- O^T += V^T . P^T ----
+    // The score registers 8 s2 .. 8 s2 + 7 of a lane are cached rows 16 s2 + 4 kg + (0..3) and 16 s2 + 8 + 4 kg + (0..3): taken as
+    // the eight k of a 16-deep step, with the value operand read as the same two groups of four rows (the order of the
+    // rows inside a step is free as long as both operands agree).
 #pragma unroll
-    for (int s4 = 0; s4 < 4; s4++) {
-      ph4_t ph, pl;
+    for (int s2 = 0; s2 < 2; s2++) {
+      ph8_t ph, pl;
 #pragma unroll
-      for (int i = 0; i < 4; i++) { _Float16 hv, lv; split_f16(C[4 * s4 + i], hv, lv); ph[i] = hv; pl[i] = lv; }
+      for (int i = 0; i < 8; i++) { _Float16 hv, lv; split_f16(C[8 * s2 + i], hv, lv); ph[i] = hv; pl[i] = lv; }
 #pragma unroll
       for (int dt = 0; dt < 4; dt++) {
-        const ph4_t a = *reinterpret_cast<const ph4_t*>(&sV[0][(32 * dt + n) * PA_LDV + 8 * s4 + 4 * kg]);
-        O[dt] = __builtin_amdgcn_mfma_f32_32x32x8f16(a, ph, O[dt], 0, 0, 0);
-        O[dt] = __builtin_amdgcn_mfma_f32_32x32x8f16(a, pl, O[dt], 0, 0, 0);
+        const ph4_t a0 = *reinterpret_cast<const ph4_t*>(&sV[0][(32 * dt + n) * PA_LDV + 16 * s2 + 4 * kg]);
+        const ph4_t a1 = *reinterpret_cast<const ph4_t*>(&sV[0][(32 * dt + n) * PA_LDV + 16 * s2 + 8 + 4 * kg]);
+        const ph8_t a = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, ph, O[dt], 0, 0, 0);
+        O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pl, O[dt], 0, 0, 0);
         if (F32) {
-          const ph4_t al = *reinterpret_cast<const ph4_t*>(&sV[NP - 1][(32 * dt + n) * PA_LDV + 8 * s4 + 4 * kg]);
-          O[dt] = __builtin_amdgcn_mfma_f32_32x32x8f16(al, ph, O[dt], 0, 0, 0);
+          const ph4_t b0 = *reinterpret_cast<const ph4_t*>(&sV[NP - 1][(32 * dt + n) * PA_LDV + 16 * s2 + 4 * kg]);
+          const ph4_t b1 = *reinterpret_cast<const ph4_t*>(&sV[NP - 1][(32 * dt + n) * PA_LDV + 16 * s2 + 8 + 4 * kg]);
+          const ph8_t al = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+          O[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, ph, O[dt], 0, 0, 0);
         }
       }
     }
