@@ -31,9 +31,10 @@ struct cai_decoder_s {
   // mixture-of-experts prompt: per chunk the router outputs, the slots grouped by expert and the per-slot activations
   float *pm_logits = nullptr, *pm_probs = nullptr, *pm_gate = nullptr, *pm_gu = nullptr, *pm_part = nullptr;
   int32_t *pm_expert = nullptr, *pm_perm = nullptr, *pm_tiles = nullptr;
-  int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_argmax = nullptr, *d_gen = nullptr;
-  int32_t* h_io = nullptr;   // pinned: tokens[8] pos[8] argmax[8]
+  int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_argmax = nullptr, *d_gen = nullptr, *d_gen_idx = nullptr;
+  int32_t* h_io = nullptr;   // pinned: tokens[8] pos[8] argmax[8] generated-so-far[8]
   hipGraphExec_t graph[9] = {nullptr};
+  hipGraphExec_t gen_graph[2] = {nullptr, nullptr};   // greedy generation: one step + hand-over, GEN_UNROLL steps + hand-overs
   bool use_graph = true;
   int ws_generation = -1;         // activation-workspace generation the captured batch graphs were built against
   std::vector<cai_qw_s*> owned;   // weights created by a loader on the decoder's behalf, destroyed with it
@@ -44,17 +45,23 @@ struct cai_decoder_s {
 
 namespace cai {
 
-__global__ void advance_kernel(int32_t* tokens, int32_t* pos, const int32_t* argmax, int32_t* gen_out, int idx)
+// Greedy hand-over between two steps on the device: the arg-max becomes the next input token, the position advances, and
+// the token is appended to the generated list (its length lives on the device, so the launch has no per-step argument and
+// a captured graph of several steps replays).
+__global__ void advance_kernel(int32_t* tokens, int32_t* pos, const int32_t* argmax, int32_t* gen_out, int32_t* gen_idx)
 {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     const int32_t t = argmax[0];
-    gen_out[idx] = t; tokens[0] = t; pos[0] += 1;
+    const int idx = gen_idx[0];
+    gen_out[idx] = t; gen_idx[0] = idx + 1; tokens[0] = t; pos[0] += 1;
   }
 }
+constexpr int GEN_UNROLL = 8;     // decode steps per launch of the long generation graph
 
 static void invalidate_graphs(cai_decoder_s* d)
 {
   for (auto& g : d->graph) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
+  for (auto& g : d->gen_graph) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
 }
 
 static int check_ready(cai_decoder_s* d)
@@ -390,6 +397,35 @@ static int run_step(cai_decoder_s* d, int n_b)
   return CAI_OK;
 }
 
+// `steps` greedy batch-1 steps of sequence 0, each followed by the hand-over kernel, as ONE graph launch (steps = 1 or
+// GEN_UNROLL): a launch per token costs the stream a gap between graphs and a separate hand-over launch.
+static int run_gen_steps(cai_decoder_s* d, int steps)
+{
+  Context& c = ctx();
+  auto body = [&]() {
+    for (int u = 0; u < steps; u++) {
+      const int rc = enqueue_step(d, 1, 0); if (rc) return rc;
+      hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, c.stream, d->d_tokens, d->d_pos, d->d_argmax, d->d_gen, d->d_gen_idx);
+    }
+    return (int)CAI_OK;
+  };
+  if (!d->use_graph) { const int rc = body(); if (rc) return rc; CAI_HIP(hipGetLastError()); return CAI_OK; }
+  hipGraphExec_t& ge = d->gen_graph[steps == 1 ? 0 : 1];
+  if (!ge) {
+    hipGraph_t g = nullptr;
+    CAI_HIP(hipStreamBeginCapture(c.stream, hipStreamCaptureModeThreadLocal));
+    const int rc = body();
+    const hipError_t e = hipStreamEndCapture(c.stream, &g);
+    if (rc) { if (g) (void)hipGraphDestroy(g); return rc; }
+    if (e != hipSuccess) return hip_fail(e, "hipStreamEndCapture", __FILE__, __LINE__);
+    const hipError_t e2 = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e2 != hipSuccess) return hip_fail(e2, "hipGraphInstantiate", __FILE__, __LINE__);
+  }
+  CAI_HIP(hipGraphLaunch(ge, c.stream));
+  return CAI_OK;
+}
+
 }  // namespace cai
 
 using namespace cai;
@@ -435,13 +471,13 @@ extern "C" int cai_decoder_create(const cai_decoder_config* cfg, cai_decoder_t* 
   if (e == hipSuccess) e = alloc_f(&d->am_v, (size_t)ame);
   if (e == hipSuccess) e = hipMalloc((void**)&d->am_i, (size_t)ame * sizeof(int32_t));
   if (e == hipSuccess) e = alloc_f(&d->ssq, 2 * 1024);
-  if (e == hipSuccess) e = hipMalloc((void**)&d->d_tokens, 3 * 8 * sizeof(int32_t));
+  if (e == hipSuccess) e = hipMalloc((void**)&d->d_tokens, 4 * 8 * sizeof(int32_t));
   if (e == hipSuccess) e = hipMalloc((void**)&d->d_gen, (size_t)c.max_ctx * sizeof(int32_t));
-  if (e == hipSuccess) e = hipHostMalloc((void**)&d->h_io, 3 * 8 * sizeof(int32_t), hipHostMallocDefault);
+  if (e == hipSuccess) e = hipHostMalloc((void**)&d->h_io, 4 * 8 * sizeof(int32_t), hipHostMallocDefault);
   if (e == hipSuccess) e = hipMemcpyAsync(d->theta, th.data(), th.size() * 4, hipMemcpyHostToDevice, ctx().stream);
   if (e == hipSuccess) e = hipStreamSynchronize(ctx().stream);
   if (e != hipSuccess) { cai_decoder_destroy(d); return hip_fail(e, "cai_decoder_create allocation", __FILE__, __LINE__); }
-  d->d_pos = d->d_tokens + 8; d->d_argmax = d->d_tokens + 16;
+  d->d_pos = d->d_tokens + 8; d->d_argmax = d->d_tokens + 16; d->d_gen_idx = d->d_tokens + 24;
   const char* ng = getenv("CAIHIP_NO_GRAPH");
   d->use_graph = !(ng && ng[0] == '1');
   *out = d;
@@ -563,11 +599,13 @@ extern "C" int cai_decoder_generate(cai_decoder_t d, int32_t first_token, int po
   if (d->kv.evict_cap == 0 ? pos + n_tokens > c.max_ctx : n_tokens > c.max_ctx)
     return set_error(CAI_ERR_STATE, "cai_decoder_generate: %d tokens from %d exceed max_ctx %d", n_tokens, pos, c.max_ctx);
   Context& cx = ctx();
-  d->h_io[0] = first_token; d->h_io[8] = pos;
+  d->h_io[0] = first_token; d->h_io[8] = pos; d->h_io[24] = 0;
   CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
-  for (int i = 0; i < n_tokens; i++) {
-    if ((rc = run_step(d, 1))) return rc;
-    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, cx.stream, d->d_tokens, d->d_pos, d->d_argmax, d->d_gen, i);
+  CAI_HIP(hipMemcpyAsync(d->d_gen_idx, d->h_io + 24, sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
+  for (int i = 0; i < n_tokens;) {
+    const int steps = n_tokens - i >= GEN_UNROLL ? GEN_UNROLL : 1;
+    if ((rc = run_gen_steps(d, steps))) return rc;
+    i += steps;
   }
   CAI_HIP(hipMemcpyAsync(tokens_out, d->d_gen, (size_t)n_tokens * sizeof(int32_t), hipMemcpyDeviceToHost, cx.stream));
   CAI_HIP(hipStreamSynchronize(cx.stream));
