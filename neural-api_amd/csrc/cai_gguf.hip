@@ -177,6 +177,8 @@ int parse(cai_gguf_s* g)
                        ti.name.c_str(), ti.ggml_type, (long long)dims[0], be, fn);
     ti.offset = (int64_t)c.get<uint64_t>();
     if (!c.ok) return set_error(CAI_ERR_INVALID, "gguf: truncated tensor table (tensor \"%s\"): %s", ti.name.c_str(), fn);
+    if (known && ti.n_elems / be > (int64_t)(0x7fffffffffffffffll / bb))   // (the product below would wrap and slip past the bounds check)
+      return set_error(CAI_ERR_INVALID, "gguf: tensor \"%s\" byte size overflows: %s", ti.name.c_str(), fn);
     ti.nbytes = known ? ti.n_elems / be * bb : 0;   // unknown types stay listed; loading them is refused
     g->tensor_index[ti.name] = g->tensors.size();
     g->tensors.push_back(std::move(ti));
@@ -470,6 +472,29 @@ extern "C" int cai_decoder_load_gguf(const char* path, int max_ctx, int max_batc
     else { const MetaValue* tk = find_meta(g, "tokenizer.ggml.tokens"); if (tk && tk->type == GT_ARR) vocab = (int64_t)tk->count; }
   }
   if (vocab <= 0) return fail(set_error(CAI_ERR_INVALID, "gguf decoder: cannot determine the vocab size (no %s, no 2-D token_embd.weight, no tokenizer.ggml.tokens) in %s", key("vocab_size").c_str(), path));
+
+  // The metadata is not trusted further than the tensor table bears it out: every block owns tensors, so a block count beyond
+  // the table is a lie, and the first block's matrices and the embedding must have the shapes the keys promise - checked
+  // before anything is sized from these numbers.
+  if (n_layers > (int64_t)g->tensors.size())
+    return fail(set_error(CAI_ERR_INVALID, "gguf decoder: %s=%lld but the file lists %zu tensors: %s", key("block_count").c_str(), (long long)n_layers, g->tensors.size(), path));
+  if (hkv <= 0 || hq % hkv) return fail(set_error(CAI_ERR_INVALID, "gguf decoder: %lld query heads over %lld KV heads: %s", (long long)hq, (long long)hkv, path));
+  const int64_t lim = (int64_t)1 << 24;
+  if (dm > lim || ffn > lim || hq > lim || hd > lim || vocab > ((int64_t)1 << 28) || hq * hd > lim || (max_ctx <= 0 && ctx_len > ((int64_t)1 << 26)))
+    return fail(set_error(CAI_ERR_INVALID, "gguf decoder: implausible dimensions (width %lld, feed-forward %lld, %lld heads of %lld, vocab %lld, context %lld): %s",
+                          (long long)dm, (long long)ffn, (long long)hq, (long long)hd, (long long)vocab, (long long)ctx_len, path));
+  {
+    struct Want { const char* name; int64_t rows, cols; };
+    const Want wants[] = {{"token_embd.weight", vocab, dm}, {"blk.0.attn_q.weight", hq * hd, dm}, {"blk.0.attn_k.weight", hkv * hd, dm},
+                          {"blk.0.attn_output.weight", dm, hq * hd}, {"blk.0.ffn_up.weight", ffn, dm}, {"blk.0.ffn_down.weight", dm, ffn}};
+    for (const Want& w : wants) {
+      const TensorInfo* t = find_tensor(g, w.name);
+      if (!t) return fail(set_error(CAI_ERR_INVALID, "gguf: missing tensor \"%s\" in %s", w.name, path));
+      if (t->n_dims != 2 || t->shape[0] != w.rows || t->shape[1] != w.cols)
+        return fail(set_error(CAI_ERR_INVALID, "gguf: tensor \"%s\" is %lld x %lld, the metadata promises %lld x %lld: %s", w.name,
+                              (long long)t->shape[0], (long long)(t->n_dims > 1 ? t->shape[1] : 1), (long long)w.rows, (long long)w.cols, path));
+    }
+  }
 
   cai_decoder_config cfg{};
   cfg.n_layers = (int)n_layers; cfg.d_model = (int)dm; cfg.n_q_heads = (int)hq; cfg.n_kv_heads = (int)hkv; cfg.head_dim = (int)hd;

@@ -10,13 +10,15 @@ def _s(x):
 
 
 def write_gguf(path, meta, tensors, alignment=32):
-    """meta: {key: int | float | str}; tensors: [(name, row_major_shape, ggml_type, raw_bytes)]."""
+    """meta: {key: int | float | str | list of str}; tensors: [(name, row_major_shape, ggml_type, raw_bytes)]."""
     b = b"GGUF" + struct.pack("<IQQ", 3, len(tensors), len(meta))
     for k, v in meta.items():
         if isinstance(v, str):
             b += _s(k) + struct.pack("<I", 8) + _s(v)
         elif isinstance(v, float):
             b += _s(k) + struct.pack("<If", 6, v)
+        elif isinstance(v, (list, tuple)):      # array of strings
+            b += _s(k) + struct.pack("<IIQ", 9, 8, len(v)) + b"".join(_s(w) for w in v)
         else:
             b += _s(k) + struct.pack("<II", 4, v)
     off, blobs = 0, []

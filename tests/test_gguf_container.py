@@ -87,6 +87,7 @@ CASES = {
     "q8_0 not block multiple": (_gguf(tensors=[(b"t", [33, 2], 8, 0)], pad_to=32, data=b"\0" * 128), "not a multiple of the block size 32"),
     "q4_k not block multiple": (_gguf(tensors=[(b"t", [128, 2], 12, 0)], pad_to=32, data=b"\0" * 512), "not a multiple of the block size 256"),
     "bad alignment": (_gguf(meta=[(b"general.alignment", 4, struct.pack("<I", 24))]), "not a positive power of two"),
+    "byte size wraps": (_gguf(tensors=[(b"t", [0x7fffffff, 0x7fffffff, 2], 0, 0)], pad_to=32, data=b"\0" * 64), "byte size overflows"),
     "tensor outside data": (_gguf(tensors=[(b"t", [64], 0, 0)], pad_to=32, data=b"\0" * 64), "falls outside the data section"),
 }
 
@@ -160,6 +161,10 @@ LOADER_REFUSALS = {
     "qwen2 without a bias": ("qwen2", {}, ("blk.0.attn_k.bias",), (), "blk.0.attn_k.bias"),
     "yarn scaling": ("llama", {"llama.rope.scaling.type": "yarn", "llama.rope.scaling.factor": 4.0}, (), (), "supported: none, linear"),
     "linear factor below one": ("llama", {"llama.rope.scaling.type": "linear", "llama.rope.scaling.factor": 0.5}, (), (), "must be >= 1"),
+    "block count beyond the tensor table": ("llama", {"llama.block_count": 100000}, (), (), "but the file lists"),
+    "width the embedding does not have": ("llama", {"llama.embedding_length": 64}, (), (), "the metadata promises"),
+    "implausible context": ("llama", {"llama.context_length": 1 << 30}, (), (), "implausible dimensions"),
+    "heads that do not divide": ("llama", {"llama.attention.head_count_kv": 3}, (), (), "query heads over"),
     "rope_freqs of the wrong length": ("llama", {}, (), (("rope_freqs.weight", [4], 0, np.ones(4, np.float32).tobytes()),), "one per rotary pair"),
     "rope_freqs with linear scaling": ("llama", {"llama.rope.scaling.type": "linear", "llama.rope.scaling.factor": 2.0}, (),
                                        (("rope_freqs.weight", [8], 0, np.ones(8, np.float32).tobytes()),), "together with linear scaling"),
@@ -194,3 +199,71 @@ def test_pascal_binding_and_header_constants_agree():
         assert h.get(k) == v, (k, v, h.get(k))
     for k in ("CAI_Q5_K", "CAI_Q2_K", "CAI_Q3_K", "CAI_Q4_1", "CAI_Q5_0", "CAI_Q5_1", "CAI_ROPE_LINEAR", "CAI_ROPE_LLAMA3"):
         assert k in p, k
+
+
+FUZZ_CHILD = r'''
+import ctypes as C, importlib, os, sys
+sys.path.insert(0, sys.argv[1])
+cai = importlib.import_module("neural-api_amd.caihip")
+L = cai.load()
+d = sys.argv[2]
+n_ok = 0
+for name in sorted(os.listdir(d)):
+    print(name, flush=True)                      # the last name printed names the file that took the process down
+    path = os.path.join(d, name).encode()
+    g = C.c_void_p()
+    if L.cai_gguf_open(path, C.byref(g)) == 0:
+        n_ok += 1
+        ver, al = C.c_int(), C.c_int(); nt, nm, ds = C.c_int64(), C.c_int64(), C.c_int64()
+        L.cai_gguf_info(g, C.byref(ver), C.byref(al), C.byref(nt), C.byref(nm), C.byref(ds))
+        buf = C.create_string_buffer(256); ty, nd = C.c_int(), C.c_int(); dims = (C.c_int64 * 8)(); off, nb = C.c_int64(), C.c_int64()
+        for i in range(min(nt.value, 64)):
+            if L.cai_gguf_tensor_info(g, i, buf, 256, C.byref(ty), C.byref(nd), dims, C.byref(off), C.byref(nb)) == 0:
+                p = C.c_void_p()
+                if L.cai_gguf_tensor_data(g, i, C.byref(p)) == 0 and nb.value > 0:
+                    C.string_at(p.value, 1); C.string_at(p.value + nb.value - 1, 1)      # first and last byte lie inside the mapping
+        v = C.c_int64(); f = C.c_double()
+        for key in (b"general.architecture", b"llama.block_count", b"llama.context_length", b"tokenizer.ggml.tokens", b"general.alignment"):
+            L.cai_gguf_meta_int(g, key, C.byref(v)); L.cai_gguf_meta_float(g, key, C.byref(f)); L.cai_gguf_meta_str(g, key, buf, 256)
+            if L.cai_gguf_meta_array_count(g, key, C.byref(v)) == 0:
+                for i in (0, v.value - 1, v.value // 2): L.cai_gguf_meta_array_str(g, key, i, buf, 256)
+        L.cai_gguf_close(g)
+    h = C.c_void_p()
+    if L.cai_decoder_load_gguf(path, 0, 1, 0, C.byref(h)) == 0 and h.value: L.cai_decoder_free(h)
+print("done", n_ok, flush=True)
+'''
+
+
+def test_mutated_files_never_take_the_process_down(tmp_path):
+    """Byte flips, overwritten length fields and truncations of a valid decoder file: every one is either refused or read,
+    and every tensor the reader then hands out lies inside the mapping.  Runs in a child process so that a crash is a test
+    failure that names the file; the files come from a fixed seed."""
+    import os, subprocess, sys
+    seed_file = tmp_path / "seed.gguf"
+    _tiny_decoder_file(str(seed_file), "llama", {"tokenizer.ggml.tokens": ["a", "bc", "def"] * 5, "llama.rope.freq_base": 10000.0})
+    blob = seed_file.read_bytes()
+    g = cai.GGUF(str(seed_file)); head = g.info()["data_start"]; del g
+    d = tmp_path / "cases"; d.mkdir()
+    rng = np.random.default_rng(20240611)
+    huge = [0xFFFFFFFFFFFFFFFF, 0xFFFFFFFFFFFFFFF0, 1 << 63, 1 << 40, (1 << 32) - 1, 1 << 31, 0]
+    for i in range(360):
+        b = bytearray(blob)
+        kind = i % 4
+        if kind == 0:                                  # a few flipped bytes in the header / metadata / tensor table
+            for _ in range(int(rng.integers(1, 9))):
+                b[int(rng.integers(0, head))] ^= int(rng.integers(1, 256))
+        elif kind == 1:                                # a length, count, type or offset field replaced by an extreme value
+            at = int(rng.integers(4, head - 8))
+            b[at:at + 8] = struct.pack("<Q", huge[int(rng.integers(0, len(huge)))])
+        elif kind == 2:                                # cut short
+            b = b[:int(rng.integers(0, len(b)))]
+        else:                                          # a run of the table overwritten with noise
+            at = int(rng.integers(0, head - 16)); n = int(rng.integers(1, 16))
+            b[at:at + n] = rng.integers(0, 256, n, dtype=np.uint8).tobytes()
+        (d / ("case_%03d.gguf" % i)).write_bytes(bytes(b))
+    (d / "case_seed.gguf").write_bytes(blob)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", FUZZ_CHILD, root, str(d)], capture_output=True, text=True, timeout=600)
+    lines = r.stdout.strip().splitlines()
+    assert r.returncode == 0, "child ended with %d after %s\n%s" % (r.returncode, lines[-1] if lines else "(nothing)", r.stderr[-2000:])
+    assert lines[-1].startswith("done") and int(lines[-1].split()[1]) >= 1      # at least the unmodified file is read
