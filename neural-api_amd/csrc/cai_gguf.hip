@@ -489,7 +489,7 @@ extern "C" int cai_decoder_load_gguf(const char* path, int max_ctx, int max_batc
                           {"blk.0.attn_output.weight", dm, hq * hd}, {"blk.0.ffn_up.weight", ffn, dm}, {"blk.0.ffn_down.weight", dm, ffn}};
     for (const Want& w : wants) {
       const TensorInfo* t = find_tensor(g, w.name);
-      if (!t) return fail(set_error(CAI_ERR_INVALID, "gguf: missing tensor \"%s\" in %s", w.name, path));
+      if (!t) continue;                        // (reported, in the order of loading, below)
       if (t->n_dims != 2 || t->shape[0] != w.rows || t->shape[1] != w.cols)
         return fail(set_error(CAI_ERR_INVALID, "gguf: tensor \"%s\" is %lld x %lld, the metadata promises %lld x %lld: %s", w.name,
                               (long long)t->shape[0], (long long)(t->n_dims > 1 ? t->shape[1] : 1), (long long)w.rows, (long long)w.cols, path));
