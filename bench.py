@@ -246,18 +246,18 @@ def gemm_sweep(cai, synth, torch):
 # HBM bytes per launch of the 7B-shape gate|up kernel from hardware counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000
 # KiB, factors from a 1 GiB copy kernel): profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt.  Not measurable from
 # inside this process; re-collect when the kernel changes.
-GATEUP_TRAFFIC_BYTES = int((37513.6 * 2.000 + 74.5 * 1.000) * 1024)
+GATEUP_TRAFFIC_BYTES = int((37513.6 * 2.000 + 74.7 * 1.000) * 1024)
 def gateup_kernel_name(qtype, cols):
     """Name of the batch-1 fused gate|up kernel the library launches for this weight type and width (rows of 17..24
-    super-blocks are packed four to a wave: the fifth template argument)."""
+    super-blocks are packed four to a wave: the fifth template argument, else 1)."""
     if qtype not in ("Q4_K", "Q5_K"):
         return "gemv_fast<%s>" % qtype
     packed = cols % 256 == 0 and 16 < cols // 256 <= 24
-    return "gemv_%s_dot<1,1,false,2%s>" % ("q4k" if qtype == "Q4_K" else "q5k", ",4" if packed else "")
+    return "gemv_%s_dot<1,1,false,2,%d>" % ("q4k" if qtype == "Q4_K" else "q5k", 4 if packed else 1)
 
 
-GATEUP_TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of gemv_q4k_dot<1,1,false,2>, profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt; "
-                         "collected with the tree at commit e3181a8 (cai_gemv_dot.hip last changed in 77da839)")
+GATEUP_TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of gemv_q4k_dot<1,1,false,2,1>, profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt; "
+                         "collected with the tree at commit fad3c7b (cai_gemv_dot.hip last changed in 35c29c4)")
 
 
 def main():
