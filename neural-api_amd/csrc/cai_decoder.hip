@@ -325,7 +325,7 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
     const bool all_mfma = prompt_route(wq, n) == 2 && prompt_route(wk, n) == 2 && prompt_route(wv, n) == 2;   // one pre-pass serves q, k and v
     if (all_mfma && (rc = prefill_prep(d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, dm, n))) return rc;
     const cai_qw_s* qkv3[3] = {wq, wk, wv}; const int qkv_off[3] = {0, qw, qw + kw};
-    if (all_mfma && gemm_q4k_multi_supported(qkv3, 3)) {   // one launch: the k and v projections alone leave half the chip idle
+    if (all_mfma && prefill_multi_supported(qkv3, 3)) {   // one launch: the k and v projections alone leave half the chip idle
       if ((rc = prefill_gemm_multi(qkv3, qkv_off, 3, n, d->pqkv, qkvw))) return rc;
     } else {
       if ((rc = linear_rows(wq, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv, qkvw, nullptr))) return rc;

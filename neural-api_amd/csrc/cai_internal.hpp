@@ -234,6 +234,10 @@ int prefill_prep_swiglu(const float* gu, int64_t gu_stride, int half, int n_tok)
 int prefill_gemm(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride, const float* residual);
 int prefill_gemm_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, float* y, int64_t y_stride);
 bool gemm_q4k_multi_supported(const cai_qw_s* const* ws, int n_w);
+bool gemm_blk_multi_supported(const cai_qw_s* const* ws, int n_w);
+int launch_gemm_blk_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, const _Float16* xhi, const _Float16* xlo, const float* sinv,
+                          int n_tok, float* y, int64_t y_stride);
+bool prefill_multi_supported(const cai_qw_s* const* ws, int n_w);   // one launch of a prompt kernel takes these matrices together
 int launch_gemm_q4k_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, const _Float16* xhi, const _Float16* xlo, const _Float16* sxhi,
                           const _Float16* sxlo, const float* sinv, int n_tok, float* y, int64_t y_stride, const float* residual, int swiglu_half);
 bool prefill_gemm_swiglu_supported(const cai_qw_s* w, int n_tok);

@@ -740,10 +740,13 @@ int prefill_prep_swiglu(const float* gu, int64_t gu_stride, int half, int n_tok)
   return CAI_OK;
 }
 // Several matrices of one width applied to the prepared activations (q | k | v).
+bool prefill_multi_supported(const cai_qw_s* const* ws, int n_w) { return gemm_q4k_multi_supported(ws, n_w) || gemm_blk_multi_supported(ws, n_w); }
 int prefill_gemm_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, float* y, int64_t y_stride)
 {
   if (n_w > 1 && gemm_q4k_multi_supported(ws, n_w))
     return launch_gemm_q4k_multi(ws, y_off, n_w, g_pws.hi, g_pws.lo, g_pws.sxhi, g_pws.sxlo, g_pws.sinv, n_tok, y, y_stride, nullptr, 0);
+  if (n_w > 1 && gemm_blk_multi_supported(ws, n_w))
+    return launch_gemm_blk_multi(ws, y_off, n_w, g_pws.hi, g_pws.lo, g_pws.sinv, n_tok, y, y_stride);
   for (int i = 0; i < n_w; i++) {
     const int rc = prefill_gemm(ws[i], n_tok, y + y_off[i], y_stride, nullptr);
     if (rc) return rc;

@@ -43,6 +43,10 @@ struct BlkGemmParams {
   const int32_t* tile_tab; const int32_t* perm;   // perm: sorted position -> slot (token * top_k + rank)
   int x_div;                            // activation row of a slot = slot / x_div; result row = slot
   int64_t expert_rows;
+  // dense launches: up to two more matrices of the same type and width (q | k | v) - row groups [seg_end[i], ...) belong to
+  // matrix i + 1, whose rows land y_off2[i] columns into a y row
+  int n_seg; int seg_end[2];
+  const uint8_t* q2[2]; const uint8_t* d2[2]; const float* bias2[2]; int rows2[2]; int y_off2[2];
 };
 
 // eight codes (two dwords) -> eight exact halfs.  Q8_0: signed bytes; Q4_0: (nibble - 8), low or high nibbles of the bytes
@@ -92,16 +96,19 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_pf(const BlkGemmParams p)
     else { xr = yr = first + m; }
     s_xrow[threadIdx.x] = xr; s_yrow[threadIdx.x] = yr; s_sinv[threadIdx.x] = p.sinv[xr];
   }
-  const int R0 = (rg * 4 + wave) * 32 * RT;
+  const uint8_t* qbase = p.q; const uint8_t* dbase = p.d; const float* bias = p.bias; int rows = p.rows, yo = 0, rgl = rg;   // this work-group's matrix (uniform)
+  if (p.n_seg > 1 && rg >= p.seg_end[0]) { qbase = p.q2[0]; dbase = p.d2[0]; bias = p.bias2[0]; rows = p.rows2[0]; yo = p.y_off2[0]; rgl = rg - p.seg_end[0]; }
+  if (p.n_seg > 2 && rg >= p.seg_end[1]) { qbase = p.q2[1]; dbase = p.d2[1]; bias = p.bias2[1]; rows = p.rows2[1]; yo = p.y_off2[1]; rgl = rg - p.seg_end[1]; }
+  const int R0 = (rgl * 4 + wave) * 32 * RT;
   const int K = p.cols, nb32 = K >> 5, nsb = (K + 255) >> 8;
   constexpr int BQ = QT == CAI_Q8_0 ? 32 : 16;          // quant bytes per block
   const int64_t bank_row = (int64_t)expert * p.expert_rows;
   const uint8_t* qrow[RT]; const uint16_t* drow[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; rt++) {
-    const int64_t r = bank_row + min(R0 + 32 * rt + n, p.rows - 1);     // tail rows: re-read the last row, not written
-    qrow[rt] = p.q + r * (int64_t)nb32 * BQ + (BQ / 2) * kg;
-    drow[rt] = reinterpret_cast<const uint16_t*>(p.d) + r * (int64_t)nb32;
+    const int64_t r = bank_row + min(R0 + 32 * rt + n, rows - 1);     // tail rows: re-read the last row, not written
+    qrow[rt] = qbase + r * (int64_t)nb32 * BQ + (BQ / 2) * kg;
+    drow[rt] = reinterpret_cast<const uint16_t*>(dbase) + r * (int64_t)nb32;
   }
   struct WRegs { uint32_t q[4][BQ / 8]; uint32_t d[2]; };               // per row tile: the lane's piece of 4 blocks, their 4 scales
   // unit u = blocks 4 u .. 4 u + 3 of the row.  Loads carry no branch: past the end the last unit / block is fetched again
@@ -228,11 +235,11 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_pf(const BlkGemmParams p)
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
           const int row = R0 + 32 * rt + n;
-          if (row >= p.rows) continue;
+          if (row >= rows) continue;
           float r = Y[rt][tt][4 * g + i] * si;
-          if (p.bias) r += p.bias[bank_row + row];
-          if (p.residual) r += p.residual[o + row];
-          p.y[o + row] = r;
+          if (bias) r += bias[bank_row + row];
+          if (p.residual) r += p.residual[o + yo + row];
+          p.y[o + yo + row] = r;
         }
       }
 }
@@ -284,10 +291,13 @@ int launch_blk(const BlkGemmParams& p0, int n_tiles_grouped)
   // Tiling: two row tiles per wave (256 rows per work-group) whenever that still gives every CU work; two token tiles on top
   // for long prompts; one row tile for matrices of few rows
   const int tiles32 = p.tile_tab ? n_tiles_grouped : (p.n_tok + 31) / 32;
-  const int wgs_rt2 = ((p.rows + 255) / 256) * tiles32;
+  int rows_all = p.rows;
+  for (int i = 1; i < p.n_seg; i++) rows_all += p.rows2[i - 1];
+  const int wgs_rt2 = ((rows_all + 255) / 256) * tiles32;
   int rt = wgs_rt2 >= n_cu ? 2 : 1, tt = 1;
-  if (!p.tile_tab && rt == 2 && ((p.rows + 255) / 256) * ((p.n_tok + 63) / 64) >= 2 * n_cu) tt = 2;
+  if (!p.tile_tab && rt == 2 && ((rows_all + 255) / 256) * ((p.n_tok + 63) / 64) >= 2 * n_cu) tt = 2;
   p.n_row_groups = (p.rows + 128 * rt - 1) / (128 * rt);
+  for (int i = 1; i < p.n_seg; i++) { p.seg_end[i - 1] = p.n_row_groups; p.n_row_groups += (p.rows2[i - 1] + 128 * rt - 1) / (128 * rt); }   // every matrix starts a row group of its own
   const size_t lds = (size_t)tt * 32 * BL_LDX * 2 * 2;
   int grid;
   if (p.tile_tab) { p.n_tok_tiles = n_tiles_grouped; grid = n_tiles_grouped * p.n_row_groups; }
@@ -312,6 +322,26 @@ int launch_gemm_blk(const cai_qw_s* w, const _Float16* xhi, const _Float16* xlo,
   p.q = w->data; p.d = w->aux; p.bias = w->bias; p.rows = (int)w->rows; p.cols = (int)w->cols;
   p.xhi = xhi; p.xlo = xlo; p.sinv = sinv; p.n_tok = n_tok; p.y = y; p.y_stride = y_stride; p.residual = residual;
   p.x_div = 1; p.expert_rows = 0;
+  return w->qtype == CAI_Q8_0 ? launch_blk<CAI_Q8_0>(p, 0) : launch_blk<CAI_Q4_0>(p, 0);
+}
+
+// Up to three matrices of one type and width in one launch: y[t][y_off[i] + r] = (W_i x[t])[r] (+ bias_i)
+bool gemm_blk_multi_supported(const cai_qw_s* const* ws, int n_w)
+{
+  if (n_w < 1 || n_w > 3 || !gemm_blk_supported(ws[0])) return false;
+  for (int i = 1; i < n_w; i++) if (ws[i]->qtype != ws[0]->qtype || ws[i]->cols != ws[0]->cols) return false;
+  return true;
+}
+int launch_gemm_blk_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, const _Float16* xhi, const _Float16* xlo, const float* sinv,
+                          int n_tok, float* y, int64_t y_stride)
+{
+  if (!gemm_blk_multi_supported(ws, n_w)) return set_error(CAI_ERR_UNSUPPORTED, "prompt gemm: %d matrices in one launch", n_w);
+  const cai_qw_s* w = ws[0];
+  BlkGemmParams p{};
+  p.q = w->data; p.d = w->aux; p.bias = w->bias; p.rows = (int)w->rows; p.cols = (int)w->cols;
+  p.xhi = xhi; p.xlo = xlo; p.sinv = sinv; p.n_tok = n_tok; p.y = y + y_off[0]; p.y_stride = y_stride; p.residual = nullptr;
+  p.x_div = 1; p.expert_rows = 0; p.n_seg = n_w;
+  for (int i = 1; i < n_w; i++) { p.q2[i - 1] = ws[i]->data; p.d2[i - 1] = ws[i]->aux; p.bias2[i - 1] = ws[i]->bias; p.rows2[i - 1] = (int)ws[i]->rows; p.y_off2[i - 1] = y_off[i] - y_off[0]; }
   return w->qtype == CAI_Q8_0 ? launch_blk<CAI_Q8_0>(p, 0) : launch_blk<CAI_Q4_0>(p, 0);
 }
 
