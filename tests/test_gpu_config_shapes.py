@@ -174,3 +174,32 @@ def test_olmoe_width_prompt_grouped_by_expert_against_the_oracle():
         assert rel_err(ld[0], lo) < TOL and int(a[0]) == n_o
         tok_o, am = n_o, int(a[0])
     dec.close()
+
+
+@pytest.mark.parametrize("name,n_tok", [("qwen2.5-7b", 230), ("qwen2.5-32b", 150)])
+def test_full_width_prompt_pass_equals_token_at_a_time(name, n_tok):
+    """A prompt long enough for the full-width prompt pass to take its large-tile forms (q | k | v as one launch with biases,
+    SwiGLU in the epilogue of the gate|up product - engaged from 193 tokens at 37888 rows, from 129 at 55296 -, the
+    register-resident pre-pass of the 18944- / 27648-wide row) against the same tokens ingested one step at a time, whose
+    kernels the test above pins to the oracle at these widths: last-token logits within 2e-4 of the row's largest logit, same
+    arg-max, and the decode step that follows agrees too (the caches hold the same rows)."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    s = TWINS[name]
+    cfg = dict(s["cfg"], max_ctx=256)
+    spec = full_width_spec(cfg, s["qtype"], s["head"], s["bias"], seed=99)
+    kvd = cai.KV_F16 if s["kv_f16"] else cai.KV_F32
+    rng = np.random.default_rng(99)
+    prompt = rng.integers(0, cfg["vocab"], n_tok).tolist()
+    a = cai.Decoder(spec, kv_dtype=kvd)
+    am_s, l_s = None, None
+    for p, t in enumerate(prompt):
+        am_s, l_s = a.step(t, p)
+    nxt_s, l2_s = a.step(int(am_s[0]), n_tok)
+    a.close()
+    b = cai.Decoder(spec, kv_dtype=kvd)
+    am_p, l_p = b.prefill(prompt, 0)
+    assert rel_err(l_p, l_s[0]) < 2e-4 and am_p == int(am_s[0])
+    nxt_p, l2_p = b.step(am_p, n_tok)
+    assert rel_err(l2_p[0], l2_s[0]) < 2e-4 and int(nxt_p[0]) == int(nxt_s[0])
+    b.close()
