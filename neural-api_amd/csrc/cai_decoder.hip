@@ -272,7 +272,9 @@ static int ensure_prefill_buffers(cai_decoder_s* d, int n)
     CAI_HIP(hipMalloc((void**)&d->pm_gu, S * 2 * c.ffn * 4)); CAI_HIP(hipMalloc((void**)&d->pm_part, S * c.d_model * 4));
   }
   d->pf_cap = cap;
-  return CAI_OK;
+  // the activation planes of the prompt products, sized once for the widest row (a mixture-of-experts chunk prepares one row per slot)
+  const int plane_rows = c.n_experts > 0 ? cap * std::max(c.top_k, 1) : cap;
+  return prefill_reserve_rows(plane_rows, std::max(std::max(c.d_model, d->qw()), c.ffn));
 }
 
 static int linear_rows(const cai_qw_s* w, bool prepped, const float* x, int64_t x_stride, const float* gain, float eps, int n,

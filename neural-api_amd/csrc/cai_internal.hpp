@@ -230,6 +230,7 @@ int nb_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok);
 int nb_reduce(float* y, int64_t y_stride, const float* residual);
 int nb_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok, float* y, int64_t y_stride, const float* residual);
 int prefill_prep(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok);
+int prefill_reserve_rows(int n_tok, int K);   // sizes the shared activation planes ahead of the first prefill_prep
 int prefill_prep_swiglu(const float* gu, int64_t gu_stride, int half, int n_tok);   // planes <- up * silu(gate)
 int prefill_gemm(const cai_qw_s* w, int n_tok, float* y, int64_t y_stride, const float* residual);
 int prefill_gemm_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, float* y, int64_t y_stride);

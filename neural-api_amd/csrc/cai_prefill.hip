@@ -718,6 +718,10 @@ static int prefill_reserve(int n_tok, int K)
   return CAI_OK;
 }
 
+// The planes for n_tok rows of up to K columns in one allocation (a decoder knows its widest row before its first prompt;
+// growing width by width would free and allocate, with a stream synchronisation, several times inside that prompt).
+int prefill_reserve_rows(int n_tok, int K) { return prefill_reserve(n_tok, K); }
+
 void prefill_release()   // cai_shutdown
 {
   void* q[] = {g_pws.hi, g_pws.lo, g_pws.sinv, g_pws.sxhi, g_pws.sxlo};
