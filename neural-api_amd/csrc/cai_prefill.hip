@@ -662,7 +662,9 @@ int launch_gemm_q4k_multi(const cai_qw_s* const* ws, const int* y_off, int n_w, 
   const int n_cu = ctx().n_cu;
   const int wgs_rt2 = (int)((rows_all + 255) / 256) * ((n_tok + 31) / 32);
   const int wgs_tt2 = (int)((rows_all + 127) / 128) * ((n_tok + 63) / 64);
-  const int mode = (swiglu_half || wgs_rt2 >= 4 * n_cu) ? 3 : (wgs_tt2 < 2 * n_cu ? 1 : 2);   // 1, 2: token tiles; 3: two row tiles
+  // (measured on 512-token chunks: 7168 rows = 448 work-groups of two row tiles 107 us against 121 us with one tile; 5120 rows = 320
+  // work-groups lose to 640 of one tile, 3584 rows = 224 likewise)
+  const int mode = (swiglu_half || 4 * wgs_rt2 >= 7 * n_cu) ? 3 : (wgs_tt2 < 2 * n_cu ? 1 : 2);   // 1, 2: token tiles; 3: two row tiles
   const int rt = mode == 3 ? 2 : 1, tt = mode == 2 ? 2 : 1;
   p.swiglu_half = swiglu_half;
   p.n_row_groups = 0;
