@@ -821,7 +821,20 @@ struct PromptParams {
   float softcap, inv_sqrt;
   const float* theta; const int32_t* pos;
   float* out; int64_t out_stride;
+  float* part;                               // [token][q_head][K split][128 + 2]: unnormalised sums, maximum, normaliser
 };
+
+constexpr int PA_KT_MIN = 2;     // K tiles (of 32 cached rows) a split takes at least
+constexpr int PA_KS_MAX = 8;     // splits of a token tile's K range at most
+// K tiles a token tile walks and the number of work-groups (blockIdx.z) they are cut over: long ranges are split so that a
+// short prompt (few token tiles, a causal triangle of work) still fills the chip; the merge kernel adds the pieces.
+__device__ __forceinline__ void prompt_k_range(const PromptParams& p, int t0, int n_ks, int& jt0, int& jt1, int& splits)
+{
+  const int pos_first = p.pos[t0], pos_last = p.pos[min(t0 + 31, p.n_tok - 1)];
+  const int j_lo = (p.window > 0 && pos_first + 1 > p.window) ? pos_first + 1 - p.window : 0;
+  jt0 = j_lo >> 5; jt1 = pos_last >> 5;
+  splits = max(1, min(n_ks, (jt1 - jt0 + 1) / PA_KT_MIN));
+}
 
 // rotated q (neural/neural.cl:1517-1542) as two f16 planes
 __global__ __launch_bounds__(256) void prompt_q_kernel(const PromptParams p)
@@ -866,9 +879,16 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
   const bool tok_on = tok < p.n_tok;
   const int pos_n = tok_on ? p.pos[tok] : -1;
   const int jstart_n = (p.window > 0 && pos_n + 1 > p.window) ? pos_n + 1 - p.window : 0;
-  // the tile's range of cached rows (tokens are consecutive positions of one sequence)
-  const int pos_first = p.pos[t0], pos_last = p.pos[min(t0 + 31, p.n_tok - 1)];
-  const int j_lo = (p.window > 0 && pos_first + 1 > p.window) ? pos_first + 1 - p.window : 0;
+  // the tile's range of cached rows (tokens are consecutive positions of one sequence) and this work-group's share of it
+  int jt_first, jt_last, splits;
+  prompt_k_range(p, t0, (int)gridDim.z, jt_first, jt_last, splits);
+  const int ks = blockIdx.z;
+  if (ks >= splits) return;                       // (uniform: the whole work-group leaves before any barrier)
+  {
+    const int per = (jt_last - jt_first + 1 + splits - 1) / splits;
+    const int a = jt_first + ks * per;
+    jt_last = min(jt_last, a + per - 1); jt_first = a;
+  }
   const KV_T* kc = reinterpret_cast<const KV_T*>(p.kc) + (int64_t)g * p.max_ctx * 128;
   const KV_T* vc = reinterpret_cast<const KV_T*>(p.vc) + (int64_t)g * p.max_ctx * 128;
 
@@ -915,8 +935,8 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
     }
   };
   RawTile raw;
-  fetch(j_lo >> 5, raw);
-  for (int jt = j_lo >> 5; jt * 32 <= pos_last; jt++) {
+  fetch(jt_first, raw);
+  for (int jt = jt_first; jt <= jt_last; jt++) {
     __syncthreads();                                        // the previous tile has been consumed
     {
       float kv[16], vv[16];
@@ -1038,6 +1058,18 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
     }
   }
   if (!head_on || !tok_on) return;
+  if (splits > 1) {        // this piece's unnormalised sums, maximum and normaliser; prompt_merge_kernel adds the pieces
+    float* pt = p.part + (((int64_t)tok * p.q_heads + head) * gridDim.z + ks) * 130;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        float* q4 = pt + 32 * dt + 8 * g4 + 4 * kg;       // (130-float records: 8-byte aligned only)
+        q4[0] = O[dt][4 * g4]; q4[1] = O[dt][4 * g4 + 1]; q4[2] = O[dt][4 * g4 + 2]; q4[3] = O[dt][4 * g4 + 3];
+      }
+    if (kg == 0) { pt[128] = m_run; pt[129] = l_run; }
+    return;
+  }
   const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
   float* dst = p.out + (int64_t)tok * p.out_stride + head * 128;
 #pragma unroll
@@ -1046,6 +1078,29 @@ __global__ __launch_bounds__(256) void attn_prompt_kernel(const PromptParams p)
     for (int g4 = 0; g4 < 4; g4++)
       *reinterpret_cast<float4*>(dst + 32 * dt + 8 * g4 + 4 * kg) =
           make_float4(O[dt][4 * g4] * inv, O[dt][4 * g4 + 1] * inv, O[dt][4 * g4 + 2] * inv, O[dt][4 * g4 + 3] * inv);
+}
+
+// out[token][head] = sum of the K splits of a token tile, folded with a running maximum in split order (a tile walked by one
+// work-group was written by it and is left alone)
+__global__ __launch_bounds__(512) void prompt_merge_kernel(const PromptParams p, int n_ks)
+{
+  const int tok = blockIdx.x, head = blockIdx.y * 4 + (threadIdx.x >> 7), d = threadIdx.x & 127;   // four heads per work-group
+  int jt0, jt1, splits;
+  prompt_k_range(p, (tok >> 5) << 5, n_ks, jt0, jt1, splits);
+  if (splits <= 1 || head >= p.q_heads) return;
+  const float* pt = p.part + (((int64_t)tok * p.q_heads + head) * n_ks) * 130;
+  float M = -1e30f, L = 0.0f, A = 0.0f;
+  float ms[PA_KS_MAX], ls[PA_KS_MAX], as[PA_KS_MAX];                     // all requests first (a split past the count repeats the last one; not used)
+#pragma unroll
+  for (int s = 0; s < PA_KS_MAX; s++) { const int sc = min(s, splits - 1); ms[s] = pt[sc * 130 + 128]; ls[s] = pt[sc * 130 + 129]; as[s] = pt[sc * 130 + d]; }
+#pragma unroll
+  for (int s = 0; s < PA_KS_MAX; s++) {
+    if (s < splits && ls[s] > 0.0f) {
+      const float mn = fmaxf(M, ms[s]), c0 = expf(M - mn), c1 = expf(ms[s] - mn);
+      A = A * c0 + as[s] * c1; L = L * c0 + ls[s] * c1; M = mn;
+    }
+  }
+  p.out[(int64_t)tok * p.out_stride + head * 128 + d] = L > 0.0f ? A * (1.0f / L) : 0.0f;
 }
 
 int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, int n_seq, int q_heads, int window,
@@ -1113,11 +1168,28 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
     pp.q_heads = q_heads; pp.kv_heads = kv->kv_heads; pp.max_ctx = kv->max_ctx; pp.n_tok = n_seq; pp.window = window;
     pp.softcap = softcap; pp.inv_sqrt = p.inv_sqrt; pp.theta = theta; pp.pos = pos_dev; pp.out = out; pp.out_stride = out_stride;
     const int G = q_heads / kv->kv_heads;
+    const int wgs = ((n_seq + 31) / 32) * kv->kv_heads * ((G + 3) / 4);
+    // K splits per token tile: as many as keep the launch at one work-group per CU (a tile with few K tiles takes fewer).
+    // Measured on 511 tokens of the 7B shape (128 work-groups unsplit): 67 us -> 38.7 + 11.2 us (merge) with two splits,
+    // 50.8 + 11.6 with three; on 512-token chunks of the 32B shape (256 work-groups) splitting loses (365 -> 373 + 16 us).
+    const int n_ks = std::max(1, std::min(PA_KS_MAX, c.n_cu / wgs));
+    if (n_ks > 1) {
+      const size_t pneed = (size_t)n_seq * q_heads * n_ks * 130;
+      if (pneed > kv->pq_part_cap) {
+        CAI_HIP(hipStreamSynchronize(c.stream));
+        if (kv->pq_part) (void)hipFree(kv->pq_part);
+        kv->pq_part = nullptr; kv->pq_part_cap = 0;
+        CAI_HIP(hipMalloc((void**)&kv->pq_part, pneed * 4));
+        kv->pq_part_cap = pneed;
+      }
+    }
+    pp.part = kv->pq_part;
     hipLaunchKernelGGL(prompt_q_kernel, dim3(n_seq), dim3(256), 0, c.stream, pp);
-    const dim3 grid((n_seq + 31) / 32, kv->kv_heads * ((G + 3) / 4));
+    const dim3 grid((n_seq + 31) / 32, kv->kv_heads * ((G + 3) / 4), n_ks);
     if (kv->dtype == CAI_KV_F16) hipLaunchKernelGGL(attn_prompt_kernel<__half>, grid, dim3(256), 0, c.stream, pp);
     else if (kv->dtype == CAI_KV_I8) hipLaunchKernelGGL(attn_prompt_kernel<int8_t>, grid, dim3(256), 0, c.stream, pp);
     else hipLaunchKernelGGL(attn_prompt_kernel<float>, grid, dim3(256), 0, c.stream, pp);
+    if (n_ks > 1) hipLaunchKernelGGL(prompt_merge_kernel, dim3(n_seq, (q_heads + 3) / 4), dim3(512), 0, c.stream, pp, n_ks);
     return CAI_OK;
   }
   // one work-group per (slice, KV head) serving the whole group of query heads, or one per (slice, query head)
@@ -1181,7 +1253,8 @@ void kv_free(cai_kv_s* kv)
   kv->ks = kv->vs = nullptr;
   if (kv->pq_hi) (void)hipFree(kv->pq_hi);
   if (kv->pq_lo) (void)hipFree(kv->pq_lo);
-  kv->pq_hi = kv->pq_lo = nullptr; kv->pq_cap = 0;
+  if (kv->pq_part) (void)hipFree(kv->pq_part);
+  kv->pq_hi = kv->pq_lo = nullptr; kv->pq_cap = 0; kv->pq_part = nullptr; kv->pq_part_cap = 0;
   if (kv->part) (void)hipFree(kv->part);
   if (kv->d_len) (void)hipFree(kv->d_len);
   if (kv->merge_cnt) (void)hipFree(kv->merge_cnt);

@@ -134,6 +134,7 @@ struct cai_kv_s {
   int32_t* d_len = nullptr;               // [seq] device scratch: rows live BEFORE the token being decoded
   unsigned* merge_cnt = nullptr;          // [seq][part_q_heads] arrival counters of the in-kernel merge of the split partials (wrap to 0 by themselves)
   void* pq_hi = nullptr; void* pq_lo = nullptr; size_t pq_cap = 0;   // prompt ingestion: rotated q of a chunk as two f16 planes
+  float* pq_part = nullptr; size_t pq_part_cap = 0;                     // prompt ingestion: partial results of a token tile's K splits
   size_t elem() const { return dtype == CAI_KV_F16 ? 2 : dtype == CAI_KV_I8 ? 1 : 4; }
   int64_t layer_rows() const { return (int64_t)kv_heads * max_ctx; }
   int64_t seq_rows() const { return layer_rows() * n_layers; }
