@@ -729,7 +729,7 @@ static int launch_group(const AttnParams& p, int n_seq, hipStream_t st)
 
 // Prompt ingestion: rotate the K rows of n_tok tokens at their positions and write K,V into sequence `seq`.
 template <typename KV_T>
-__global__ __launch_bounds__(256) void kv_append_rows_kernel(const AttnParams p)
+__device__ __forceinline__ void kv_append_row(const AttnParams& p)
 {
   const int b = blockIdx.x;
   const float* row = p.qkv + (int64_t)b * p.qkv_stride;
@@ -754,6 +754,8 @@ __global__ __launch_bounds__(256) void kv_append_rows_kernel(const AttnParams p)
     vc[((int64_t)g * p.max_ctx + slot) * hd + d] = kv_from_float<KV_T>(row[qw + kw + i]);
   }
 }
+template <typename KV_T>
+__global__ __launch_bounds__(256) void kv_append_rows_kernel(const AttnParams p) { kv_append_row<KV_T>(p); }
 
 // The same for an int8 cache: one half-wave per (token, KV head, K|V) row, quantised with the decode step's rule.
 template <int DS>
@@ -837,7 +839,7 @@ __device__ __forceinline__ void prompt_k_range(const PromptParams& p, int t0, in
 }
 
 // rotated q (neural/neural.cl:1517-1542) as two f16 planes
-__global__ __launch_bounds__(256) void prompt_q_kernel(const PromptParams p)
+__device__ __forceinline__ void prompt_q_row(const PromptParams& p)
 {
   const int t = blockIdx.x, qw = p.q_heads * 128;
   const float* row = p.qkv + (int64_t)t * p.qkv_stride;
@@ -856,6 +858,10 @@ __global__ __launch_bounds__(256) void prompt_q_kernel(const PromptParams p)
     p.qlo[(int64_t)t * qw + 2 * e] = l0; p.qlo[(int64_t)t * qw + 2 * e + 1] = l1;
   }
 }
+__global__ __launch_bounds__(256) void prompt_q_kernel(const PromptParams p) { prompt_q_row(p); }
+// one launch per chunk for both: the token's K and V rows into the cache, its rotated q into the planes
+template <typename KV_T>
+__global__ __launch_bounds__(256) void prompt_rows_kernel(const AttnParams p, const PromptParams pp) { kv_append_row<KV_T>(p); prompt_q_row(pp); }
 
 constexpr int PA_LDK = 136;    // halfs per staged K row (128 + pad: rows stay 16-byte aligned for the 8-half operand reads)
 constexpr int PA_LDV = 36;     // halfs per staged V^T row (32 cached rows + pad)
@@ -1136,17 +1142,19 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
     if (!prompt_rows && !grouped) { p.qn_gain = qn_gain; p.kn_gain = kn_gain; p.qk_eps = qk_eps; }
     else if ((rc = launch_rmsnorm_pair(qkv, qn_gain, qw, kn_gain, kw, n_seq, qk_eps, qkv_stride))) return rc;
   }
+  // prompts over a 128-wide cache: matrix-core kernel, 32 tokens x 4 heads per work-group
+  static const int flash_on = []() { const char* e = getenv("CAIHIP_PROMPT_FLASH"); return e ? atoi(e) : 1; }();
+  const bool flash = prompt_rows && flash_on && kv->head_dim == 128 && kv->evict_cap == 0 && n_seq >= 8;
+  const bool rows_fused = flash && kv->dtype != CAI_KV_I8;     // the append and the q planes share a launch (below)
   if (prompt_rows && kv->dtype == CAI_KV_I8) {
     if (p.hd <= 32) hipLaunchKernelGGL(kv_append_rows_i8_kernel<1>, dim3(n_seq), dim3(256), 0, c.stream, p);
     else if (p.hd <= 64) hipLaunchKernelGGL(kv_append_rows_i8_kernel<2>, dim3(n_seq), dim3(256), 0, c.stream, p);
     else hipLaunchKernelGGL(kv_append_rows_i8_kernel<4>, dim3(n_seq), dim3(256), 0, c.stream, p);
-  } else if (prompt_rows) {
+  } else if (prompt_rows && !rows_fused) {
     if (kv->dtype == CAI_KV_F16) hipLaunchKernelGGL(kv_append_rows_kernel<__half>, dim3(n_seq), dim3(256), 0, c.stream, p);
     else hipLaunchKernelGGL(kv_append_rows_kernel<float>, dim3(n_seq), dim3(256), 0, c.stream, p);
   }
-  // prompts over a 128-wide cache: matrix-core kernel, 32 tokens x 4 heads per work-group
-  static const int flash_on = []() { const char* e = getenv("CAIHIP_PROMPT_FLASH"); return e ? atoi(e) : 1; }();
-  if (prompt_rows && flash_on && kv->head_dim == 128 && kv->evict_cap == 0 && n_seq >= 8) {
+  if (flash) {
     const size_t need = (size_t)n_seq * q_heads * 128;
     if (need > kv->pq_cap) {
       CAI_HIP(hipStreamSynchronize(c.stream));
@@ -1184,7 +1192,9 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
       }
     }
     pp.part = kv->pq_part;
-    hipLaunchKernelGGL(prompt_q_kernel, dim3(n_seq), dim3(256), 0, c.stream, pp);
+    if (!rows_fused) hipLaunchKernelGGL(prompt_q_kernel, dim3(n_seq), dim3(256), 0, c.stream, pp);
+    else if (kv->dtype == CAI_KV_F16) hipLaunchKernelGGL(prompt_rows_kernel<__half>, dim3(n_seq), dim3(256), 0, c.stream, p, pp);
+    else hipLaunchKernelGGL(prompt_rows_kernel<float>, dim3(n_seq), dim3(256), 0, c.stream, p, pp);
     const dim3 grid((n_seq + 31) / 32, kv->kv_heads * ((G + 3) / 4), n_ks);
     if (kv->dtype == CAI_KV_F16) hipLaunchKernelGGL(attn_prompt_kernel<__half>, grid, dim3(256), 0, c.stream, pp);
     else if (kv->dtype == CAI_KV_I8) hipLaunchKernelGGL(attn_prompt_kernel<int8_t>, grid, dim3(256), 0, c.stream, pp);
