@@ -97,3 +97,44 @@ def test_more_experts_than_the_router_ranks_are_refused_without_a_device():
     assert "1024 experts" in cai.last_error()
     cfg.n_experts, cfg.top_k = 8, 9
     assert lib.cai_decoder_create(C.byref(cfg), C.byref(h)) == -1
+
+
+def pascal_call_sites(path):
+    """(name, number of arguments) of every cai_* call in a Pascal source (comments stripped, parentheses balanced)."""
+    with open(path) as f:
+        text = f.read()
+    text = re.sub(r"\{.*?\}", "", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    calls = []
+    for m in re.finditer(r"\b(cai_[a-z0-9_]+)\s*\(", text):
+        depth, i, n_args, seen = 1, m.end(), 0, False
+        while depth and i < len(text):
+            ch = text[i]
+            if ch in "([":
+                depth += 1; seen = True
+            elif ch in ")]":
+                depth -= 1
+            elif ch == "," and depth == 1:
+                n_args += 1
+            elif not ch.isspace():
+                seen = True
+            i += 1
+        calls.append((m.group(1), n_args + 1 if seen else 0))
+    return calls
+
+
+def test_pascal_session_unit_calls_only_declared_externals_with_their_arities():
+    """caihipsession.pas (the TNNetStreamingDecoder-shaped session over the decoder entry points) cannot be compiled here:
+    every library call it makes must at least name an external of caihip.pas and pass the declared number of arguments,
+    and it must cover the session surface the chat engine uses."""
+    decl = pascal_arities()
+    calls = pascal_call_sites(os.path.join(ROOT, "neural-api_amd", "pascal", "caihipsession.pas"))
+    assert len(calls) >= 15
+    for name, n in calls:
+        assert name in decl, "%s is not declared in caihip.pas" % name
+        assert n == decl[name], "%s called with %d arguments, declared with %d" % (name, n, decl[name])
+    used = {name for name, _ in calls}
+    for need in ("cai_init", "cai_decoder_load_gguf", "cai_decoder_step", "cai_decoder_prefill", "cai_decoder_generate", "cai_decoder_candidates",
+                 "cai_decoder_truncate", "cai_decoder_reset", "cai_decoder_snapshot", "cai_decoder_restore", "cai_decoder_set_kv_dtype",
+                 "cai_decoder_set_eviction", "cai_decoder_cache_rows", "cai_decoder_destroy", "cai_last_error"):
+        assert need in used, need
