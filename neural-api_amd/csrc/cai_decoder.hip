@@ -329,6 +329,9 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
     const cai_qw_s* qkv3[3] = {wq, wk, wv}; const int qkv_off[3] = {0, qw, qw + kw};
     if (all_mfma && prefill_multi_supported(qkv3, 3)) {   // one launch: the k and v projections alone leave half the chip idle
       if ((rc = prefill_gemm_multi(qkv3, qkv_off, 3, n, d->pqkv, qkvw))) return rc;
+    } else if (all_mfma && prefill_multi_supported(qkv3, 2)) {   // attn_v of another type (a Q4_K_M file keeps some in Q6_K): q | k together
+      if ((rc = prefill_gemm_multi(qkv3, qkv_off, 2, n, d->pqkv, qkvw))) return rc;
+      if ((rc = linear_rows(wv, true, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw + kw, qkvw, nullptr))) return rc;
     } else {
       if ((rc = linear_rows(wq, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv, qkvw, nullptr))) return rc;
       if ((rc = linear_rows(wk, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw, qkvw, nullptr))) return rc;
