@@ -304,3 +304,50 @@ def test_prompt_gemm_q8_0_q4_0_on_matrix_cores(qt, rows, cols, T):
     for t in range(T):
         assert rel_err(got[t], want[t], floor=0.02 * cols ** 0.5 * float(np.abs(x[t]).mean())) < TIGHT, t
     w.close()
+
+
+@pytest.mark.parametrize("qt", [O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K])
+@pytest.mark.parametrize("cols", [3584, 5120])
+def test_a_nan_or_inf_activation_reaches_every_output(qt, cols):
+    """The integer-dot kernels hold the activation in block-float form (a maximum and integers): a NaN or an infinity in x
+    must still poison every output row, as it does in the float dot product of the reference (0 * inf = NaN, x + NaN = NaN),
+    and must not leak into rows of a clean batch neighbour."""
+    from helpers.device import dev
+    cai = dev()
+    rows = 300
+    raw, rng = make(qt, rows, cols, cols + qt)
+    w = cai.QWeight(qt, rows, cols, raw)
+    for bad in (np.nan, np.inf, -np.inf):
+        for at in (0, 7, cols - 1, cols // 2 + 33):
+            x = rng.standard_normal((1, cols)).astype(np.float32)
+            x[0, at] = bad
+            got = w.gemv(x)
+            assert not np.isfinite(got).any(), (bad, at, int(np.isfinite(got).sum()))
+    x = rng.standard_normal((3, cols)).astype(np.float32)
+    x[1, 100] = np.nan
+    got = w.gemv(x)
+    assert np.isfinite(got[0]).all() and np.isfinite(got[2]).all() and not np.isfinite(got[1]).any()
+    w.close()
+
+
+@pytest.mark.parametrize("qt,rows,cols", [(O.Q4_K, 8203, 4096), (O.Q8_0, 4101, 4096)])
+def test_a_nan_token_poisons_only_its_own_row_on_the_matrix_cores(qt, rows, cols):
+    """The same through the matrix-core kernels (a batch of 8 on a matrix of 16 MiB or more, and a 40-token prompt product):
+    the poisoned token's outputs are all non-finite, every other token's outputs are finite."""
+    from helpers.device import dev
+    cai = dev()
+    raw, rng = make(qt, rows, cols, 31)
+    w = cai.QWeight(qt, rows, cols, raw)
+    x = rng.standard_normal((8, cols)).astype(np.float32)
+    x[5, 77] = np.nan; x[2, 4000] = np.inf
+    got = w.gemv(x)
+    for t in range(8):
+        assert np.isfinite(got[t]).all() == (t not in (2, 5)), t
+        if t in (2, 5):
+            assert not np.isfinite(got[t]).any(), t
+    x = rng.standard_normal((40, cols)).astype(np.float32)
+    x[33, 1] = np.nan
+    got = w.gemm(x)
+    assert not np.isfinite(got[33]).any()
+    assert np.isfinite(np.delete(got, 33, axis=0)).all()
+    w.close()
