@@ -351,3 +351,26 @@ def test_a_nan_token_poisons_only_its_own_row_on_the_matrix_cores(qt, rows, cols
     assert not np.isfinite(got[33]).any()
     assert np.isfinite(np.delete(got, 33, axis=0)).all()
     w.close()
+
+
+@pytest.mark.parametrize("qt", [O.Q4_K, O.Q4_0, O.Q6_K])
+def test_blocks_of_denormal_and_huge_activations(qt):
+    """Block-float corner cases of the integer-dot kernels: a 32-block holding only denormals (its scale underflows: the block
+    must count as zero, not as NaN), a block of values near 1e30, and a block with one huge and otherwise tiny values (the
+    tiny ones round to zero integers, as 2^-23 of the maximum allows).  The kernels sum quant x activation over a 32-block
+    BEFORE the block's scale (about 1e-3) multiplies it, so their range ends about four decades below the float maximum:
+    activations beyond 1e33 may overflow where a dequantise-first product would not."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    rows, cols = 200, 3584
+    raw, rng = make(qt, rows, cols, 5 + qt)
+    w = cai.QWeight(qt, rows, cols, raw)
+    x = rng.standard_normal((1, cols)).astype(np.float32)
+    x[0, 64:96] = np.float32(1e-40); x[0, 70] = 0.0; x[0, 71] = np.float32(-3e-41)
+    x[0, 512:544] *= np.float32(1e30)
+    x[0, 1024:1056] = np.float32(1e-12); x[0, 1030] = np.float32(5e6)
+    got = w.gemv(x)
+    want = O.gemv(qt, raw, rows, cols, x, None, 0, 1)
+    assert np.isfinite(got).all()
+    assert rel_err(got, want) < TIGHT
+    w.close()
