@@ -5,7 +5,8 @@
  * The library owns all device memory; every create has a destroy; host pointers are never
  * retained after a call returns.  All calls enqueue on one in-order HIP stream owned by the
  * library (the analogue of the reference's single shared in-order OpenCL queue,
- * examples/ChatTerminal/README.md:174-180); calls are not re-entrant.
+ * examples/ChatTerminal/README.md:174-180).  Calls from several host threads are serialised by one
+ * lock inside the library; cai_last_error reports the calling thread's own last failure.
  *
  * Citations are file:line in the reference checkout (joaopauloschuler/neural-api).
  */

@@ -9,17 +9,27 @@
 namespace cai {
 
 static Context g_ctx;
-static std::mutex g_err_mu;
-static std::string g_err;
+static std::recursive_mutex g_api_mu;            // entry points call one another (generate -> step), hence recursive
+static thread_local std::string t_err;           // the message belongs to the thread whose call failed
+static thread_local int t_device = -1;           // HIP's current device is a per-thread setting
 
 Context& ctx() { return g_ctx; }
+
+// One call into the library at a time: the context's stream, staging buffers and scratch are shared by every handle, and
+// all device work is ordered on the one stream anyway.  A thread that enters for the first time (or after cai_init chose
+// another device) makes the library's device its current one.
+ApiLock::ApiLock()
+{
+  g_api_mu.lock();
+  if (g_ctx.ready && t_device != g_ctx.device) { (void)hipSetDevice(g_ctx.device); t_device = g_ctx.device; }
+}
+ApiLock::~ApiLock() { g_api_mu.unlock(); }
 
 int set_error(int code, const char* fmt, ...)
 {
   char buf[512];
   va_list ap; va_start(ap, fmt); vsnprintf(buf, sizeof(buf), fmt, ap); va_end(ap);
-  std::lock_guard<std::mutex> lk(g_err_mu);
-  g_err = buf;
+  t_err = buf;
   return code;
 }
 
@@ -59,6 +69,7 @@ using namespace cai;
 
 extern "C" int cai_init(int device_ordinal)
 {
+  CAI_ENTER();
   Context& c = ctx();
   if (c.ready) {
     if (c.device == device_ordinal) return CAI_OK;
@@ -87,6 +98,7 @@ extern "C" int cai_init(int device_ordinal)
 
 extern "C" int cai_shutdown(void)
 {
+  CAI_ENTER();
   Context& c = ctx();
   if (!c.ready) return CAI_OK;
   (void)hipStreamSynchronize(c.stream);
@@ -105,24 +117,25 @@ extern "C" int cai_shutdown(void)
 extern "C" int cai_last_error(char* buf, int buf_len)
 {
   if (!buf || buf_len <= 0) return CAI_ERR_INVALID;
-  std::lock_guard<std::mutex> lk(g_err_mu);
-  snprintf(buf, (size_t)buf_len, "%s", g_err.c_str());
+  snprintf(buf, (size_t)buf_len, "%s", t_err.c_str());
   return CAI_OK;
 }
 
 extern "C" int cai_device_name(char* buf, int buf_len)
 {
+  CAI_ENTER();
   CAI_READY();
   if (!buf || buf_len <= 0) return CAI_ERR_INVALID;
   snprintf(buf, (size_t)buf_len, "%s", ctx().name);
   return CAI_OK;
 }
 
-extern "C" int cai_sync(void) { CAI_READY(); CAI_HIP(hipStreamSynchronize(ctx().stream)); return CAI_OK; }
-extern "C" int cai_get_stream(void** s) { CAI_READY(); CAI_REQUIRE(s, "cai_get_stream: null out"); *s = (void*)ctx().stream; return CAI_OK; }
-extern "C" int cai_timer_start(void) { CAI_READY(); CAI_HIP(hipEventRecord(ctx().ev0, ctx().stream)); return CAI_OK; }
+extern "C" int cai_sync(void) { CAI_ENTER(); CAI_READY(); CAI_HIP(hipStreamSynchronize(ctx().stream)); return CAI_OK; }
+extern "C" int cai_get_stream(void** s) { CAI_ENTER(); CAI_READY(); CAI_REQUIRE(s, "cai_get_stream: null out"); *s = (void*)ctx().stream; return CAI_OK; }
+extern "C" int cai_timer_start(void) { CAI_ENTER(); CAI_READY(); CAI_HIP(hipEventRecord(ctx().ev0, ctx().stream)); return CAI_OK; }
 extern "C" int cai_timer_stop(float* ms)
 {
+  CAI_ENTER();
   CAI_READY(); CAI_REQUIRE(ms, "cai_timer_stop: null out");
   CAI_HIP(hipEventRecord(ctx().ev1, ctx().stream));
   CAI_HIP(hipEventSynchronize(ctx().ev1));
@@ -132,13 +145,15 @@ extern "C" int cai_timer_stop(float* ms)
 
 extern "C" int cai_dev_alloc(int64_t bytes, void** out)
 {
+  CAI_ENTER();
   CAI_READY(); CAI_REQUIRE(out && bytes > 0, "cai_dev_alloc: bad argument");
   CAI_HIP(hipMalloc(out, (size_t)bytes));
   return CAI_OK;
 }
-extern "C" int cai_dev_free(void* p) { CAI_READY(); if (p) { CAI_HIP(hipStreamSynchronize(ctx().stream)); CAI_HIP(hipFree(p)); } return CAI_OK; }
+extern "C" int cai_dev_free(void* p) { CAI_ENTER(); CAI_READY(); if (p) { CAI_HIP(hipStreamSynchronize(ctx().stream)); CAI_HIP(hipFree(p)); } return CAI_OK; }
 extern "C" int cai_dev_upload(void* d, const void* h, int64_t bytes)
 {
+  CAI_ENTER();
   CAI_READY(); CAI_REQUIRE(d && h && bytes >= 0, "cai_dev_upload: bad argument");
   CAI_HIP(hipMemcpyAsync(d, h, (size_t)bytes, hipMemcpyHostToDevice, ctx().stream));
   CAI_HIP(hipStreamSynchronize(ctx().stream));
@@ -146,6 +161,7 @@ extern "C" int cai_dev_upload(void* d, const void* h, int64_t bytes)
 }
 extern "C" int cai_dev_download(void* h, const void* d, int64_t bytes)
 {
+  CAI_ENTER();
   CAI_READY(); CAI_REQUIRE(d && h && bytes >= 0, "cai_dev_download: bad argument");
   CAI_HIP(hipMemcpyAsync(h, d, (size_t)bytes, hipMemcpyDeviceToHost, ctx().stream));
   CAI_HIP(hipStreamSynchronize(ctx().stream));
@@ -162,6 +178,7 @@ __global__ __launch_bounds__(256) void copy16_kernel(const uint4* src, uint4* ds
 
 extern "C" int cai_dev_copy(void* dst, const void* src, int64_t bytes)
 {
+  CAI_ENTER();
   CAI_READY(); CAI_REQUIRE(dst && src && bytes > 0 && bytes % 16 == 0, "cai_dev_copy: bad argument");
   const size_t n16 = (size_t)bytes / 16;
   const int grid = (int)std::min<size_t>((n16 + 255) / 256, 8192);
@@ -192,6 +209,7 @@ static int qw_set_bias(cai_qw_s* w, const float* bias)
 
 extern "C" int cai_qw_create(int qtype, int64_t rows, int64_t cols, const void* blocks, const float* bias, cai_qw_t* out)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(out && blocks, "cai_qw_create: null argument");
   CAI_REQUIRE(rows > 0 && cols > 0 && rows < (1ll << 31) && cols < (1ll << 31), "cai_qw_create: bad shape %lld x %lld", (long long)rows, (long long)cols);
@@ -243,6 +261,7 @@ extern "C" int cai_qw_create(int qtype, int64_t rows, int64_t cols, const void* 
 
 extern "C" int cai_qw_create_int8row(int64_t rows, int64_t cols, const int8_t* codes, const float* scales, const float* bias, cai_qw_t* out)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(out && codes && scales, "cai_qw_create_int8row: null argument");
   CAI_REQUIRE(rows > 0 && cols > 0 && rows < (1ll << 31) && cols < (1ll << 31), "cai_qw_create_int8row: bad shape");
@@ -264,6 +283,7 @@ extern "C" int cai_qw_create_int8row(int64_t rows, int64_t cols, const int8_t* c
 
 extern "C" int cai_qw_destroy(cai_qw_t w)
 {
+  CAI_ENTER();
   if (!w) return CAI_OK;
   if (ctx().ready) (void)hipStreamSynchronize(ctx().stream);
   qw_free(w);
@@ -272,6 +292,7 @@ extern "C" int cai_qw_destroy(cai_qw_t w)
 
 extern "C" int cai_qw_info(cai_qw_t w, int* qtype, int64_t* rows, int64_t* cols, int64_t* device_bytes)
 {
+  CAI_ENTER();
   CAI_REQUIRE(w, "cai_qw_info: null weight");
   if (qtype) *qtype = w->qtype;
   if (rows) *rows = w->rows;
@@ -282,6 +303,7 @@ extern "C" int cai_qw_info(cai_qw_t w, int* qtype, int64_t* rows, int64_t* cols,
 
 extern "C" int cai_qw_dequant_rows(cai_qw_t w, int64_t row0, int64_t n_rows, float* out, int flags)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(w && out, "cai_qw_dequant_rows: null argument");
   CAI_REQUIRE(row0 >= 0 && n_rows > 0 && row0 + n_rows <= w->rows, "cai_qw_dequant_rows: rows [%lld,+%lld) outside %lld", (long long)row0, (long long)n_rows, (long long)w->rows);
@@ -297,6 +319,7 @@ extern "C" int cai_qw_dequant_rows(cai_qw_t w, int64_t row0, int64_t n_rows, flo
 
 extern "C" int cai_qgemv(cai_qw_t w, const float* x, int n_b, float* y, int act, int flags)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(w && x && y, "cai_qgemv: null argument");
   CAI_REQUIRE(n_b >= 1 && n_b <= 8, "cai_qgemv: n_b %d outside 1..8", n_b);
@@ -325,6 +348,7 @@ extern "C" int cai_qgemv(cai_qw_t w, const float* x, int n_b, float* y, int act,
 
 extern "C" int cai_ffn_gateup(cai_qw_t w, const float* x, const float* gain, float eps, int n_b, float* y, int flags)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(w && x && y, "cai_ffn_gateup: null argument");
   CAI_REQUIRE(n_b >= 1 && n_b <= 8, "cai_ffn_gateup: n_b %d outside 1..8", n_b);

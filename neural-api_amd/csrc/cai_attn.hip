@@ -1347,6 +1347,7 @@ using namespace cai;
 
 extern "C" int cai_kv_create(int n_layers, int kv_heads, int head_dim, int max_ctx, int kv_dtype, cai_kv_t* out)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(out, "cai_kv_create: null out");
   cai_kv_s* kv = new cai_kv_s();
@@ -1358,6 +1359,7 @@ extern "C" int cai_kv_create(int n_layers, int kv_heads, int head_dim, int max_c
 
 extern "C" int cai_kv_destroy(cai_kv_t kv)
 {
+  CAI_ENTER();
   if (!kv) return CAI_OK;
   (void)hipStreamSynchronize(ctx().stream);
   kv_free(kv); delete kv;
@@ -1366,6 +1368,7 @@ extern "C" int cai_kv_destroy(cai_kv_t kv)
 
 extern "C" int cai_kv_reset(cai_kv_t kv)
 {
+  CAI_ENTER();
   CAI_REQUIRE(kv, "cai_kv_reset: null cache");
   std::fill(kv->len.begin(), kv->len.end(), 0);
   return CAI_OK;
@@ -1373,6 +1376,7 @@ extern "C" int cai_kv_reset(cai_kv_t kv)
 
 extern "C" int cai_kv_truncate(cai_kv_t kv, int n)
 {
+  CAI_ENTER();
   CAI_REQUIRE(kv, "cai_kv_truncate: null cache");
   CAI_REQUIRE(n >= 0, "cai_kv_truncate: negative length %d", n);
   for (int l : kv->len)
@@ -1397,12 +1401,14 @@ int cai::kv_set_eviction(cai_kv_s* kv, int sinks, int recent)
 
 extern "C" int cai_kv_set_eviction(cai_kv_t kv, int sink_tokens, int recent_window)
 {
+  CAI_ENTER();
   CAI_REQUIRE(kv, "cai_kv_set_eviction: null cache");
   return kv_set_eviction(kv, sink_tokens, recent_window);
 }
 
 extern "C" int cai_kv_rows(cai_kv_t kv, int layer, int* rows_out)
 {
+  CAI_ENTER();
   CAI_REQUIRE(kv && rows_out, "cai_kv_rows: null argument");
   CAI_REQUIRE(layer >= 0 && layer < kv->n_layers, "cai_kv_rows: layer %d of %d", layer, kv->n_layers);
   *rows_out = kv->live(kv->len_at(0, layer));
@@ -1411,6 +1417,7 @@ extern "C" int cai_kv_rows(cai_kv_t kv, int layer, int* rows_out)
 
 extern "C" int cai_kv_len(cai_kv_t kv, int layer, int* len_out)
 {
+  CAI_ENTER();
   CAI_REQUIRE(kv && len_out, "cai_kv_len: null argument");
   CAI_REQUIRE(layer >= 0 && layer < kv->n_layers, "cai_kv_len: layer %d of %d", layer, kv->n_layers);
   *len_out = kv->len_at(0, layer);
@@ -1419,6 +1426,7 @@ extern "C" int cai_kv_len(cai_kv_t kv, int layer, int* len_out)
 
 extern "C" int cai_kv_snapshot(cai_kv_t kv, cai_kv_snap_t* out)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(kv && out, "cai_kv_snapshot: null argument");
   return kv_snapshot(kv, 0, out);
@@ -1426,6 +1434,7 @@ extern "C" int cai_kv_snapshot(cai_kv_t kv, cai_kv_snap_t* out)
 
 extern "C" int cai_kv_restore(cai_kv_t kv, cai_kv_snap_t snap)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(kv && snap, "cai_kv_restore: null argument");
   return kv_restore(kv, 0, snap);
@@ -1433,6 +1442,7 @@ extern "C" int cai_kv_restore(cai_kv_t kv, cai_kv_snap_t snap)
 
 extern "C" int cai_kv_snap_destroy(cai_kv_snap_t s)
 {
+  CAI_ENTER();
   if (!s) return CAI_OK;
   if (s->k) (void)hipFree(s->k);
   if (s->v) (void)hipFree(s->v);
@@ -1464,6 +1474,7 @@ static int kv_layer_copy(cai_kv_s* kv, int layer, int len, void* k, void* v, flo
 
 extern "C" int cai_kv_export_layer(cai_kv_t kv, int layer, void* k, void* v, float* k_scales, float* v_scales)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(kv && k && v, "cai_kv_export_layer: null argument");
   CAI_REQUIRE(layer >= 0 && layer < kv->n_layers, "cai_kv_export_layer: layer %d of %d", layer, kv->n_layers);
@@ -1473,6 +1484,7 @@ extern "C" int cai_kv_export_layer(cai_kv_t kv, int layer, void* k, void* v, flo
 
 extern "C" int cai_kv_import_layer(cai_kv_t kv, int layer, int len, const void* k, const void* v, const float* k_scales, const float* v_scales)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(kv && (len == 0 || (k && v)), "cai_kv_import_layer: null argument");
   CAI_REQUIRE(layer >= 0 && layer < kv->n_layers, "cai_kv_import_layer: layer %d of %d", layer, kv->n_layers);
@@ -1487,6 +1499,7 @@ extern "C" int cai_kv_import_layer(cai_kv_t kv, int layer, int len, const void* 
 extern "C" int cai_attn_decode(cai_kv_t kv, int layer, const float* qkv, int q_heads, int window, float softcap,
                                float* out, int flags)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(kv && qkv && out, "cai_attn_decode: null argument");
   CAI_REQUIRE(layer >= 0 && layer < kv->n_layers, "cai_attn_decode: layer %d of %d", layer, kv->n_layers);

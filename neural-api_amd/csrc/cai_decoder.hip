@@ -437,6 +437,7 @@ using namespace cai;
 
 extern "C" int cai_decoder_create(const cai_decoder_config* cfg, cai_decoder_t* out)
 {
+  CAI_ENTER();
   // (the shape is checked before the device is: a refused configuration is refused on any machine)
   CAI_REQUIRE(cfg && out, "cai_decoder_create: null argument");
   const cai_decoder_config& c = *cfg;
@@ -491,6 +492,7 @@ extern "C" int cai_decoder_create(const cai_decoder_config* cfg, cai_decoder_t* 
 
 extern "C" int cai_decoder_destroy(cai_decoder_t d)
 {
+  CAI_ENTER();
   if (!d) return CAI_OK;
   if (ctx().ready) (void)hipStreamSynchronize(ctx().stream);
   invalidate_graphs(d);
@@ -518,6 +520,7 @@ void decoder_adopt_weight(cai_decoder_s* d, cai_qw_s* w) { d->owned.push_back(w)
 
 extern "C" int cai_decoder_set_weight(cai_decoder_t d, int layer, int slot, cai_qw_t w)
 {
+  CAI_ENTER();
   CAI_REQUIRE(d && w, "cai_decoder_set_weight: null argument");
   const cai_decoder_config& c = d->cfg;
   const int qw = d->qw(), kw = d->kw();
@@ -547,6 +550,7 @@ extern "C" int cai_decoder_set_weight(cai_decoder_t d, int layer, int slot, cai_
 
 extern "C" int cai_decoder_set_vector(cai_decoder_t d, int layer, int slot, const float* v, int n)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(d && v, "cai_decoder_set_vector: null argument");
   const cai_decoder_config& c = d->cfg;
@@ -569,6 +573,7 @@ extern "C" int cai_decoder_set_vector(cai_decoder_t d, int layer, int slot, cons
 
 extern "C" int cai_decoder_step(cai_decoder_t d, const int32_t* tokens, const int32_t* pos, int n_b, float* logits, int32_t* argmax)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(d && tokens && pos, "cai_decoder_step: null argument");
   const cai_decoder_config& c = d->cfg;
@@ -595,6 +600,7 @@ extern "C" int cai_decoder_step(cai_decoder_t d, const int32_t* tokens, const in
 
 extern "C" int cai_decoder_generate(cai_decoder_t d, int32_t first_token, int pos, int n_tokens, int32_t* tokens_out)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(d && tokens_out && n_tokens >= 1, "cai_decoder_generate: bad argument");
   const cai_decoder_config& c = d->cfg;
@@ -621,6 +627,7 @@ extern "C" int cai_decoder_generate(cai_decoder_t d, int32_t first_token, int po
 // Per-class timing of the batch-1 step: the production launches of one class (all blocks), back to back, between two HIP events.
 extern "C" int cai_decoder_profile(cai_decoder_t d, int32_t token, int reps, float* us_per_step_out, int n_classes)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(d && us_per_step_out && reps >= 1 && n_classes >= 1 && n_classes <= 8, "cai_decoder_profile: bad argument");
   const cai_decoder_config& c = d->cfg;
@@ -648,6 +655,7 @@ extern "C" int cai_decoder_profile(cai_decoder_t d, int32_t token, int reps, flo
 
 extern "C" int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* tokens, int n, int pos0, float* last_logits, int32_t* argmax)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(d && tokens && n >= 1, "cai_decoder_prefill: bad argument");
   const cai_decoder_config& c = d->cfg;
@@ -702,6 +710,7 @@ extern "C" int cai_decoder_candidates(cai_decoder_t d, int row, const int32_t* h
                                       float repetition, float frequency, float presence, float temperature, int m,
                                       int32_t* tokens_out, float* probs_out, int* count_out)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(d && tokens_out && probs_out, "cai_decoder_candidates: null argument");
   CAI_REQUIRE(row >= 0 && row < d->cfg.max_batch, "cai_decoder_candidates: row %d of %d", row, d->cfg.max_batch);
@@ -712,6 +721,7 @@ extern "C" int cai_decoder_candidates(cai_decoder_t d, int row, const int32_t* h
 
 extern "C" int cai_decoder_reset(cai_decoder_t d, int seq)
 {
+  CAI_ENTER();
   CAI_REQUIRE(d, "cai_decoder_reset: null decoder");
   CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch, "cai_decoder_reset: sequence %d of %d", seq, d->cfg.max_batch);
   for (int l = 0; l < d->cfg.n_layers; l++) d->kv.len_at(seq, l) = 0;
@@ -720,6 +730,7 @@ extern "C" int cai_decoder_reset(cai_decoder_t d, int seq)
 
 extern "C" int cai_decoder_truncate(cai_decoder_t d, int seq, int n)
 {
+  CAI_ENTER();
   CAI_REQUIRE(d, "cai_decoder_truncate: null decoder");
   CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch && n >= 0, "cai_decoder_truncate: bad argument");
   const int have = d->kv.len_at(seq, 0);
@@ -731,6 +742,7 @@ extern "C" int cai_decoder_truncate(cai_decoder_t d, int seq, int n)
 
 extern "C" int cai_decoder_set_eviction(cai_decoder_t d, int sink_tokens, int recent_window)
 {
+  CAI_ENTER();
   CAI_REQUIRE(d, "cai_decoder_set_eviction: null decoder");
   const int rc = kv_set_eviction(&d->kv, sink_tokens, recent_window);
   if (rc) return rc;
@@ -742,6 +754,7 @@ extern "C" int cai_decoder_set_eviction(cai_decoder_t d, int sink_tokens, int re
 // EnableInt8KVCache / DisableInt8KVCache (neural/neuraldecode.pas:1277-1290): the storage mode of an empty session.
 extern "C" int cai_decoder_set_kv_dtype(cai_decoder_t d, int kv_dtype)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(d, "cai_decoder_set_kv_dtype: null decoder");
   CAI_REQUIRE(kv_dtype == CAI_KV_F32 || kv_dtype == CAI_KV_F16 || kv_dtype == CAI_KV_I8, "cai_decoder_set_kv_dtype: type %d", kv_dtype);
@@ -780,6 +793,7 @@ static int set_thetas(cai_decoder_s* d, const std::vector<float>& th, const char
 
 extern "C" int cai_decoder_set_rope_scaling(cai_decoder_t d, int mode, float factor, int original_ctx, float low_freq_factor, float high_freq_factor)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(d, "cai_decoder_set_rope_scaling: null decoder");
   std::vector<float> th;
@@ -792,6 +806,7 @@ extern "C" int cai_decoder_set_rope_scaling(cai_decoder_t d, int mode, float fac
 
 extern "C" int cai_decoder_set_rope_out_scale(cai_decoder_t d, float scale)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(d, "cai_decoder_set_rope_out_scale: null decoder");
   CAI_REQUIRE(scale > 0.0f && scale < 3.0e38f, "cai_decoder_set_rope_out_scale: scale %g", (double)scale);
@@ -804,6 +819,7 @@ extern "C" int cai_decoder_set_rope_out_scale(cai_decoder_t d, float scale)
 
 extern "C" int cai_decoder_set_rope_freq_factors(cai_decoder_t d, const float* factors, int n)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(d && factors, "cai_decoder_set_rope_freq_factors: null argument");
   CAI_REQUIRE(n == d->cfg.head_dim / 2, "cai_decoder_set_rope_freq_factors: %d factors for %d rotary pairs", n, d->cfg.head_dim / 2);
@@ -817,6 +833,7 @@ extern "C" int cai_decoder_set_rope_freq_factors(cai_decoder_t d, const float* f
 
 extern "C" int cai_decoder_cache_rows(cai_decoder_t d, int seq, int layer, int* rows_out)
 {
+  CAI_ENTER();
   CAI_REQUIRE(d && rows_out, "cai_decoder_cache_rows: null argument");
   CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch && layer >= 0 && layer < d->cfg.n_layers, "cai_decoder_cache_rows: sequence %d, layer %d", seq, layer);
   *rows_out = d->kv.live(d->kv.len_at(seq, layer));
@@ -825,6 +842,7 @@ extern "C" int cai_decoder_cache_rows(cai_decoder_t d, int seq, int layer, int* 
 
 extern "C" int cai_decoder_len(cai_decoder_t d, int seq, int* len_out)
 {
+  CAI_ENTER();
   CAI_REQUIRE(d && len_out, "cai_decoder_len: null argument");
   CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch, "cai_decoder_len: sequence %d of %d", seq, d->cfg.max_batch);
   *len_out = d->kv.len_at(seq, 0);
@@ -833,6 +851,7 @@ extern "C" int cai_decoder_len(cai_decoder_t d, int seq, int* len_out)
 
 extern "C" int cai_decoder_snapshot(cai_decoder_t d, int seq, cai_kv_snap_t* out)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(d && out, "cai_decoder_snapshot: null argument");
   CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch, "cai_decoder_snapshot: sequence %d of %d", seq, d->cfg.max_batch);
@@ -841,6 +860,7 @@ extern "C" int cai_decoder_snapshot(cai_decoder_t d, int seq, cai_kv_snap_t* out
 
 extern "C" int cai_decoder_restore(cai_decoder_t d, int seq, cai_kv_snap_t snap)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(d && snap, "cai_decoder_restore: null argument");
   CAI_REQUIRE(seq >= 0 && seq < d->cfg.max_batch, "cai_decoder_restore: sequence %d of %d", seq, d->cfg.max_batch);
@@ -849,6 +869,7 @@ extern "C" int cai_decoder_restore(cai_decoder_t d, int seq, cai_kv_snap_t snap)
 
 extern "C" int cai_decoder_get_config(cai_decoder_t d, cai_decoder_config* out)
 {
+  CAI_ENTER();
   CAI_REQUIRE(d && out, "cai_decoder_get_config: null argument");
   *out = d->cfg;
   return CAI_OK;
@@ -856,6 +877,7 @@ extern "C" int cai_decoder_get_config(cai_decoder_t d, cai_decoder_config* out)
 
 extern "C" int cai_decoder_weight_bytes(cai_decoder_t d, int64_t* out)
 {
+  CAI_ENTER();
   CAI_REQUIRE(d && out, "cai_decoder_weight_bytes: null argument");
   const cai_decoder_config& c = d->cfg;
   int rc = check_ready(d); if (rc) return rc;

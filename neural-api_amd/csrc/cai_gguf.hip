@@ -263,6 +263,7 @@ int load_matrix(const cai_gguf_s* g, const std::string& name, const std::string*
 // ------------------------------------------------------------------------------------------
 extern "C" int cai_gguf_open(const char* path, cai_gguf_t* out)
 {
+  CAI_ENTER();
   CAI_REQUIRE(path && out, "cai_gguf_open: null argument");
   *out = nullptr;
   const int fd = open(path, O_RDONLY);
@@ -285,6 +286,7 @@ extern "C" int cai_gguf_open(const char* path, cai_gguf_t* out)
 
 extern "C" int cai_gguf_close(cai_gguf_t g)
 {
+  CAI_ENTER();
   if (!g) return CAI_OK;
   if (g->base) munmap(const_cast<uint8_t*>(g->base), g->size);
   delete g;
@@ -293,6 +295,7 @@ extern "C" int cai_gguf_close(cai_gguf_t g)
 
 extern "C" int cai_gguf_info(cai_gguf_t g, int* version, int* alignment, int64_t* n_tensors, int64_t* n_meta, int64_t* data_start)
 {
+  CAI_ENTER();
   CAI_REQUIRE(g, "cai_gguf_info: null handle");
   if (version) *version = g->version;
   if (alignment) *alignment = g->alignment;
@@ -304,6 +307,7 @@ extern "C" int cai_gguf_info(cai_gguf_t g, int* version, int* alignment, int64_t
 
 extern "C" int cai_gguf_meta_int(cai_gguf_t g, const char* key, int64_t* out)
 {
+  CAI_ENTER();
   CAI_REQUIRE(g && key && out, "cai_gguf_meta_int: null argument");
   const MetaValue* v = find_meta(g, key);
   if (!is_scalar_number(v)) return set_error(CAI_ERR_INVALID, "gguf: metadata key \"%s\" is missing or not a number: %s", key, g->path.c_str());
@@ -313,6 +317,7 @@ extern "C" int cai_gguf_meta_int(cai_gguf_t g, const char* key, int64_t* out)
 
 extern "C" int cai_gguf_meta_float(cai_gguf_t g, const char* key, double* out)
 {
+  CAI_ENTER();
   CAI_REQUIRE(g && key && out, "cai_gguf_meta_float: null argument");
   const MetaValue* v = find_meta(g, key);
   if (!is_scalar_number(v)) return set_error(CAI_ERR_INVALID, "gguf: metadata key \"%s\" is missing or not a number: %s", key, g->path.c_str());
@@ -322,6 +327,7 @@ extern "C" int cai_gguf_meta_float(cai_gguf_t g, const char* key, double* out)
 
 extern "C" int cai_gguf_meta_str(cai_gguf_t g, const char* key, char* buf, int n)
 {
+  CAI_ENTER();
   CAI_REQUIRE(g && key && buf && n > 0, "cai_gguf_meta_str: bad argument");
   const MetaValue* v = find_meta(g, key);
   if (!v || v->type != GT_STR) return set_error(CAI_ERR_INVALID, "gguf: metadata key \"%s\" is missing or not a string: %s", key, g->path.c_str());
@@ -331,6 +337,7 @@ extern "C" int cai_gguf_meta_str(cai_gguf_t g, const char* key, char* buf, int n
 
 extern "C" int cai_gguf_meta_array_count(cai_gguf_t g, const char* key, int64_t* out)
 {
+  CAI_ENTER();
   CAI_REQUIRE(g && key && out, "cai_gguf_meta_array_count: null argument");
   const MetaValue* v = find_meta(g, key);
   if (!v || v->type != GT_ARR) return set_error(CAI_ERR_INVALID, "gguf: metadata key \"%s\" is missing or not an array: %s", key, g->path.c_str());
@@ -340,6 +347,7 @@ extern "C" int cai_gguf_meta_array_count(cai_gguf_t g, const char* key, int64_t*
 
 extern "C" int cai_gguf_meta_array_str(cai_gguf_t g, const char* key, int64_t index, char* buf, int n)
 {
+  CAI_ENTER();
   CAI_REQUIRE(g && key && buf && n > 0, "cai_gguf_meta_array_str: bad argument");
   const MetaValue* v = find_meta(g, key);
   if (!v || v->type != GT_ARR || v->elem_type != GT_STR) return set_error(CAI_ERR_INVALID, "gguf: metadata key \"%s\" is missing or not a string array: %s", key, g->path.c_str());
@@ -358,6 +366,7 @@ extern "C" int cai_gguf_meta_array_str(cai_gguf_t g, const char* key, int64_t in
 
 extern "C" int cai_gguf_find_tensor(cai_gguf_t g, const char* name, int64_t* index)
 {
+  CAI_ENTER();
   CAI_REQUIRE(g && name && index, "cai_gguf_find_tensor: null argument");
   auto it = g->tensor_index.find(name);
   if (it == g->tensor_index.end()) return set_error(CAI_ERR_INVALID, "gguf: missing tensor \"%s\" in %s", name, g->path.c_str());
@@ -368,6 +377,7 @@ extern "C" int cai_gguf_find_tensor(cai_gguf_t g, const char* name, int64_t* ind
 extern "C" int cai_gguf_tensor_info(cai_gguf_t g, int64_t index, char* name_buf, int name_n, int* ggml_type, int* n_dims,
                                     int64_t* shape8, int64_t* data_offset, int64_t* nbytes)
 {
+  CAI_ENTER();
   CAI_REQUIRE(g && index >= 0 && index < (int64_t)g->tensors.size(), "cai_gguf_tensor_info: bad index");
   const TensorInfo& t = g->tensors[(size_t)index];
   if (name_buf && name_n > 0) snprintf(name_buf, (size_t)name_n, "%s", t.name.c_str());
@@ -381,6 +391,7 @@ extern "C" int cai_gguf_tensor_info(cai_gguf_t g, int64_t index, char* name_buf,
 
 extern "C" int cai_gguf_tensor_data(cai_gguf_t g, int64_t index, const void** ptr)
 {
+  CAI_ENTER();
   CAI_REQUIRE(g && ptr && index >= 0 && index < (int64_t)g->tensors.size(), "cai_gguf_tensor_data: bad argument");
   const TensorInfo& t = g->tensors[(size_t)index];
   if (t.nbytes == 0) return set_error(CAI_ERR_UNSUPPORTED, "gguf: tensor \"%s\" has ggml type %d of unknown size: %s", t.name.c_str(), t.ggml_type, g->path.c_str());
@@ -390,6 +401,7 @@ extern "C" int cai_gguf_tensor_data(cai_gguf_t g, int64_t index, const void** pt
 
 extern "C" int cai_gguf_load_qw(cai_gguf_t g, const char* name, const char* bias_name, cai_qw_t* out)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(g && name && out, "cai_gguf_load_qw: null argument");
   const std::string n(name), b(bias_name ? bias_name : "");
@@ -401,6 +413,7 @@ extern "C" int cai_gguf_load_qw(cai_gguf_t g, const char* name, const char* bias
 // ------------------------------------------------------------------------------------------
 extern "C" int cai_decoder_load_gguf(const char* path, int max_ctx, int max_batch, int kv_dtype, cai_decoder_t* out)
 {
+  CAI_ENTER();
   // (the file's metadata is judged before the device is asked for: a file this path cannot run is refused with the same
   // message on a host without a GPU)
   CAI_REQUIRE(path && out, "cai_decoder_load_gguf: null argument");

@@ -28,6 +28,7 @@ struct Context {
 };
 
 Context& ctx();
+struct ApiLock { ApiLock(); ~ApiLock(); ApiLock(const ApiLock&) = delete; ApiLock& operator=(const ApiLock&) = delete; };
 int  set_error(int code, const char* fmt, ...);
 int  hip_fail(hipError_t e, const char* what, const char* file, int line);
 int  ensure_stage(void** p, size_t* cap, size_t need);
@@ -42,6 +43,9 @@ int  ensure_stage(void** p, size_t* cap, size_t need);
   do {                                                                       \
     if (!(cond)) return cai::set_error(CAI_ERR_INVALID, __VA_ARGS__);        \
   } while (0)
+
+// first statement of every exported function: calls from several host threads are serialised
+#define CAI_ENTER() cai::ApiLock api_lock__
 
 #define CAI_READY()                                                          \
   do {                                                                       \

@@ -499,6 +499,7 @@ int finish_output(void* host, const void* dev, size_t bytes, int is_dev)
 
 extern "C" int cai_rmsnorm(const float* x, const float* gain_host, int n, int n_tokens, float eps, float* y, int flags)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(x && gain_host && y && n > 0 && n_tokens > 0, "cai_rmsnorm: bad argument");
   Context& c = ctx();
@@ -517,6 +518,7 @@ extern "C" int cai_rmsnorm(const float* x, const float* gain_host, int n, int n_
 
 extern "C" int cai_rope(float* x, int n_heads, int head_dim, int pos, float theta_base, int flags)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(x && n_heads > 0 && head_dim >= 2 && !(head_dim & 1) && head_dim <= 512, "cai_rope: bad argument");
   Context& c = ctx();
@@ -540,6 +542,7 @@ extern "C" int cai_rope(float* x, int n_heads, int head_dim, int pos, float thet
 
 extern "C" int cai_swiglu(const float* x, int half, int n_tokens, float* y, int flags)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(x && y && half > 0 && n_tokens > 0, "cai_swiglu: bad argument");
   const size_t ob = (size_t)half * n_tokens * 4;
@@ -552,6 +555,7 @@ extern "C" int cai_swiglu(const float* x, int half, int n_tokens, float* y, int 
 
 extern "C" int cai_argmax(const float* x, int n, int32_t* index_out, int flags)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(x && index_out && n > 0, "cai_argmax: bad argument");
   Context& c = ctx();
@@ -571,6 +575,7 @@ extern "C" int cai_argmax(const float* x, int n, int32_t* index_out, int flags)
 // would share the array and race.
 extern "C" int cai_argmax_noalloc(const float* x_dev, int n, int32_t* index_out_dev)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(x_dev && index_out_dev && n > 0, "cai_argmax_noalloc: bad argument");
   if (n > 4096 * NOALLOC_MAX_SLICES)
@@ -585,6 +590,7 @@ extern "C" int cai_argmax_noalloc(const float* x_dev, int n, int32_t* index_out_
 
 extern "C" int cai_router_topk(const float* logits, int n, int k, int renorm, int32_t* expert_out, float* gate_out, int flags)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(logits && expert_out && gate_out && n > 0 && k > 0 && k <= n && k <= 64, "cai_router_topk: bad argument");
   Context& c = ctx();

@@ -819,6 +819,7 @@ using namespace cai;
 
 extern "C" int cai_qgemm(cai_qw_t w, const float* x, int n_tokens, float* y, int flags)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(w && x && y && n_tokens >= 1, "cai_qgemm: bad argument");
   Context& c = ctx();

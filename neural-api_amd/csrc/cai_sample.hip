@@ -245,6 +245,7 @@ extern "C" int cai_sample_candidates(const float* logits, int n, const int32_t* 
                                      float repetition, float frequency, float presence, float temperature, int m,
                                      int32_t* tokens_out, float* probs_out, int* count_out, int flags)
 {
+  CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(logits && tokens_out && probs_out, "cai_sample_candidates: null argument");
   CAI_REQUIRE(n >= 1 && m >= 1 && m <= SMP_MAX_M, "cai_sample_candidates: %d candidates from a row of %d (1..%d)", m, n, SMP_MAX_M);
