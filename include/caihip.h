@@ -232,6 +232,22 @@ int cai_decoder_set_vector(cai_decoder_t d, int layer, int slot, const float* v_
  * sequence's cache length).  logits (host, [n_b][vocab]) and argmax (host, [n_b]) may be NULL. */
 int cai_decoder_step(cai_decoder_t d, const int32_t* tokens, const int32_t* pos, int n_b,
                      float* logits, int32_t* argmax);
+/* Width-n window step of ONE sequence (1 <= n <= 8): tokens[r] is fed at absolute position pos0 + r (pos0 = the cache
+ * length), appended, and attends to everything before it; logits (host, [n][vocab]) and argmax (host, [n]) may be NULL, row r
+ * is the output at position pos0 + r.  This is StepForward on a width-K twin (neural/neuraldecode.pas:1151-1183, 5696-5712),
+ * the verify pass of speculative decoding (examples/SpeculativeDecoding/SpeculativeDecoding.lpr:646-663).  Afterwards the cache
+ * holds pos0 + n rows; cai_decoder_truncate keeps the committed prefix (TruncateTo, neural/neuraldecode.pas:5714).  Sessions
+ * with eviction take windows of one token only. */
+int cai_decoder_step_window(cai_decoder_t d, int seq, const int32_t* tokens, int n, int pos0, float* logits, int32_t* argmax);
+/* PromptLookupDraft (neural/neuraldecode.pas:7742-7765) on token ids: the tokens that followed the most recent earlier
+ * occurrence of the context's last match_len tokens, at most num_draft of them (0: no earlier occurrence).  Host only. */
+int cai_prompt_lookup_draft(const int32_t* context, int n_ctx, int match_len, int num_draft, int32_t* draft_out, int* n_draft_out);
+/* DecodePromptLookup (neural/neuraldecode.pas:7767-7866) on the cached session: greedy continuation of sequence 0 whose passes
+ * verify a prompt-lookup draft of up to min(num_draft, 7) tokens in one window step.  context[0 .. n_ctx-2] must be in the
+ * cache; context[n_ctx-1] is fed first.  Writes n_tokens ids - the ones cai_decoder_generate would write - and the number of
+ * passes taken (may be NULL); the cache ends n_ctx - 1 + n_tokens rows long. */
+int cai_decoder_generate_lookup(cai_decoder_t d, const int32_t* context, int n_ctx, int match_len, int num_draft,
+                                int n_tokens, int32_t* tokens_out, int32_t* passes_out);
 /* Greedy continuation of sequence 0 with no host round trip between tokens: feeds `first_token` at
  * position `pos`, then each argmax as the next token; writes n_tokens ids (the greedy fast path of
  * neural/neuralchatengine.pas:1485-1561 with ArgMaxRow on the device). */

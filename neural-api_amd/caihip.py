@@ -21,7 +21,7 @@ cai_dev_alloc cai_dev_free cai_dev_upload cai_dev_download cai_dev_copy
 cai_qw_create cai_qw_create_int8row cai_qw_destroy cai_qw_info cai_qw_dequant_rows cai_qgemv cai_ffn_gateup cai_qgemm
 cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_argmax_noalloc cai_router_topk
 cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_kv_export_layer cai_kv_import_layer cai_kv_set_eviction cai_kv_rows cai_attn_decode
-cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_generate cai_decoder_profile
+cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_step_window cai_prompt_lookup_draft cai_decoder_generate_lookup cai_decoder_generate cai_decoder_profile
 cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_set_eviction cai_decoder_cache_rows cai_decoder_set_kv_dtype cai_decoder_set_rope_scaling cai_decoder_set_rope_freq_factors cai_decoder_set_rope_out_scale cai_sample_candidates cai_decoder_candidates cai_decoder_snapshot cai_decoder_restore
 cai_decoder_weight_bytes cai_decoder_get_config cai_decoder_load_gguf
 cai_gguf_open cai_gguf_close cai_gguf_info cai_gguf_meta_int cai_gguf_meta_float cai_gguf_meta_str cai_gguf_meta_array_count
@@ -32,6 +32,14 @@ class DecoderConfig(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("n_layers", "d_model", "n_q_heads", "n_kv_heads", "head_dim", "ffn", "vocab", "max_ctx")] + \
                [("eps", C.c_float), ("rope_theta", C.c_float)] + \
                [(n, C.c_int32) for n in ("window", "qk_norm_full", "n_experts", "top_k", "norm_topk", "kv_dtype", "max_batch")]
+
+
+def prompt_lookup_draft(context, match_len, num_draft):
+    """PromptLookupDraft on token ids (host only; the library need not be initialised)"""
+    context = np.ascontiguousarray(context, np.int32)
+    out = np.empty(max(num_draft, 1), np.int32); n = C.c_int32()
+    check(load().cai_prompt_lookup_draft(_ptr(context), context.size, match_len, num_draft, _ptr(out), C.byref(n)))
+    return out[:n.value].tolist()
 
 
 class CaiError(RuntimeError):
@@ -95,6 +103,9 @@ def load():
         L.cai_decoder_set_vector.argtypes = [vp, i32, i32, vp, i32]
         L.cai_decoder_step.argtypes = [vp, vp, vp, i32, vp, vp]
         L.cai_decoder_generate.argtypes = [vp, i32, i32, i32, vp]
+        L.cai_decoder_step_window.argtypes = [vp, i32, vp, i32, i32, vp, vp]
+        L.cai_prompt_lookup_draft.argtypes = [vp, i32, i32, i32, vp, vp]
+        L.cai_decoder_generate_lookup.argtypes = [vp, vp, i32, i32, i32, i32, vp, vp]
         L.cai_decoder_profile.argtypes = [vp, i32, i32, vp, i32]
         L.cai_decoder_prefill.argtypes = [vp, i32, vp, i32, i32, vp, vp]
         L.cai_decoder_reset.argtypes = [vp, i32]
@@ -420,6 +431,22 @@ class Decoder:
         out = np.empty(n, np.int32)
         check(load().cai_decoder_generate(self.h, int(first_token), int(pos), n, _ptr(out)))
         return out
+
+    def step_window(self, tokens, pos0, seq=0, want_logits=True):
+        """width-n window of ONE sequence: row r is the output at position pos0 + r (StepForward on a width-K twin)"""
+        tokens = np.ascontiguousarray(np.atleast_1d(tokens), np.int32)
+        n = tokens.size
+        lg = np.empty((n, self.cfg.vocab), np.float32) if want_logits else None
+        am = np.empty(n, np.int32)
+        check(load().cai_decoder_step_window(self.h, seq, _ptr(tokens), n, int(pos0), _ptr(lg), _ptr(am)))
+        return am, lg
+
+    def generate_lookup(self, context, n, match_len=2, num_draft=4):
+        """greedy continuation with prompt-lookup drafts; returns (tokens, passes).  context[:-1] must be in the cache"""
+        context = np.ascontiguousarray(context, np.int32)
+        out = np.empty(n, np.int32); passes = C.c_int32()
+        check(load().cai_decoder_generate_lookup(self.h, _ptr(context), context.size, match_len, num_draft, n, _ptr(out), C.byref(passes)))
+        return out, passes.value
 
     def profile(self, token, reps=8):
         """microseconds per step in each of the 8 kernel classes of the batch-1 step (see cai_decoder_profile)"""

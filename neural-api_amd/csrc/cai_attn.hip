@@ -1144,7 +1144,7 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   }
   // prompts over a 128-wide cache: matrix-core kernel, 32 tokens x 4 heads per work-group
   static const int flash_on = []() { const char* e = getenv("CAIHIP_PROMPT_FLASH"); return e ? atoi(e) : 1; }();
-  const bool flash = prompt_rows && flash_on && kv->head_dim == 128 && kv->evict_cap == 0 && n_seq >= 8;
+  const bool flash = prompt_rows == 1 && flash_on && kv->head_dim == 128 && kv->evict_cap == 0 && n_seq >= 8;
   const bool rows_fused = flash && kv->dtype != CAI_KV_I8;     // the append and the q planes share a launch (below)
   if (prompt_rows && kv->dtype == CAI_KV_I8) {
     if (p.hd <= 32) hipLaunchKernelGGL(kv_append_rows_i8_kernel<1>, dim3(n_seq), dim3(256), 0, c.stream, p);

@@ -34,6 +34,8 @@ struct cai_decoder_s {
   int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_argmax = nullptr, *d_gen = nullptr, *d_gen_idx = nullptr;
   int32_t* h_io = nullptr;   // pinned: tokens[8] pos[8] argmax[8] generated-so-far[8]
   hipGraphExec_t graph[9] = {nullptr};
+  hipGraphExec_t wgraph[9] = {nullptr};               // width-n window steps of sequence 0 (rows = consecutive positions)
+  float* wpart = nullptr; size_t wpart_elems = 0;     // attention slice results of a window's rows (sized at the first window step)
   hipGraphExec_t gen_graph[2] = {nullptr, nullptr};   // greedy generation: one step + hand-over, GEN_UNROLL steps + hand-overs
   bool use_graph = true;
   int ws_generation = -1;         // activation-workspace generation the captured batch graphs were built against
@@ -61,6 +63,7 @@ constexpr int GEN_UNROLL = 8;     // decode steps per launch of the long generat
 static void invalidate_graphs(cai_decoder_s* d)
 {
   for (auto& g : d->graph) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
+  for (auto& g : d->wgraph) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
   for (auto& g : d->gen_graph) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
 }
 
@@ -117,7 +120,9 @@ static int moe_ffn_rows(cai_decoder_s* d, const cai_decoder_s::Layer& L, float* 
 // Enqueues one whole step for activation rows 0..n_b-1 mapped to cache sequences seq0..seq0+n_b-1.
 // `classes`: bit i set = launch kernel class i (0 embedding, 1 q|k|v, 2 attention, 3 o, 4 gate|up + SwiGLU, 5 down, 6 vocabulary
 // projection, 7 arg-max).  Everything but the per-class timing of cai_decoder_profile passes all bits.
-static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = ~0u)
+// `window`: the rows are n_b CONSECUTIVE tokens of the one sequence seq0 (the width-K window of a speculative verify step,
+// neural/neuraldecode.pas:1151-1183): row r is rotated to and appended at position pos[r] and attends to the rows before it.
+static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = ~0u, bool window = false)
 {
   const cai_decoder_config& c = d->cfg;
   const int dm = c.d_model, qw = d->qw(), kw = d->kw(), I = c.ffn, qkvw = qw + 2 * kw;
@@ -146,7 +151,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = 
         const cai_qw_s* qkv3[3] = {L.w[CAI_W_Q], L.w[CAI_W_K], L.w[CAI_W_V]}; const int off3[3] = {0, qw, qw + kw};
         if ((rc = nb_gemm(qkv3, off3, 3, n_b)) || (rc = nb_reduce(d->qkv, qkvw, nullptr))) return rc;
       }
-      if ((rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0, 0, nullptr,
+      if ((rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0, window ? 2 : 0, window ? d->wpart : nullptr,
                                  c.qk_norm_full ? L.v[CAI_V_Q_NORM] : nullptr, c.qk_norm_full ? L.v[CAI_V_K_NORM] : nullptr, c.eps))) return rc;
       const int zero = 0;
       const cai_qw_s* wo = L.w[CAI_W_O]; const cai_qw_s* wgu = L.w[CAI_W_GATEUP]; const cai_qw_s* wdn = L.w[CAI_W_DOWN];
@@ -185,7 +190,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = 
       }
     }
     if ((classes & 4u) &&
-        (rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0, 0, nullptr,
+        (rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0, window ? 2 : 0, window ? d->wpart : nullptr,
                                c.qk_norm_full ? L.v[CAI_V_Q_NORM] : nullptr, c.qk_norm_full ? L.v[CAI_V_K_NORM] : nullptr, c.eps))) return rc;
     const bool o_hands = gemv_hands_off_ssq(L.w[CAI_W_O], n_b);
     if (classes & 8u) {
@@ -372,7 +377,7 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
   return CAI_OK;
 }
 
-static int run_step(cai_decoder_s* d, int n_b)
+static int run_step(cai_decoder_s* d, int n_b, bool window = false, int seq0 = 0)
 {
   Context& c = ctx();
   if (n_b >= 2) {   // the matrix-core path's activation workspace cannot grow inside a stream capture
@@ -386,19 +391,21 @@ static int run_step(cai_decoder_s* d, int n_b)
     const int rc = nb_reserve(kmax, part); if (rc) return rc;
     if (d->ws_generation != nb_ws_generation()) { invalidate_graphs(d); d->ws_generation = nb_ws_generation(); }
   }
-  if (!d->use_graph) { const int rc = enqueue_step(d, n_b, 0); if (rc) return rc; CAI_HIP(hipGetLastError()); return CAI_OK; }
-  if (!d->graph[n_b]) {
+  // (a captured graph holds the sequence index: only sequence 0 has one)
+  if (!d->use_graph || seq0 != 0) { const int rc = enqueue_step(d, n_b, seq0, ~0u, window); if (rc) return rc; CAI_HIP(hipGetLastError()); return CAI_OK; }
+  hipGraphExec_t& ge = window ? d->wgraph[n_b] : d->graph[n_b];
+  if (!ge) {
     hipGraph_t g = nullptr;
     CAI_HIP(hipStreamBeginCapture(c.stream, hipStreamCaptureModeThreadLocal));
-    const int rc = enqueue_step(d, n_b, 0);
+    const int rc = enqueue_step(d, n_b, 0, ~0u, window);
     const hipError_t e = hipStreamEndCapture(c.stream, &g);
     if (rc) { if (g) (void)hipGraphDestroy(g); return rc; }
     if (e != hipSuccess) return hip_fail(e, "hipStreamEndCapture", __FILE__, __LINE__);
-    const hipError_t e2 = hipGraphInstantiate(&d->graph[n_b], g, nullptr, nullptr, 0);
+    const hipError_t e2 = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
     (void)hipGraphDestroy(g);
     if (e2 != hipSuccess) return hip_fail(e2, "hipGraphInstantiate", __FILE__, __LINE__);
   }
-  CAI_HIP(hipGraphLaunch(d->graph[n_b], c.stream));
+  CAI_HIP(hipGraphLaunch(ge, c.stream));
   return CAI_OK;
 }
 
@@ -431,6 +438,37 @@ static int run_gen_steps(cai_decoder_s* d, int steps)
   return CAI_OK;
 }
 
+// Scratch of a window step's attention: per (row, query head, cache slice) a partial result.
+static int ensure_wpart(cai_decoder_s* d)
+{
+  const size_t need = (size_t)8 * d->kv.part_q_heads * d->kv.n_splits * (d->cfg.head_dim + 2);
+  if (d->wpart && d->wpart_elems >= need) return CAI_OK;
+  CAI_HIP(hipStreamSynchronize(ctx().stream));
+  if (d->wpart) { (void)hipFree(d->wpart); d->wpart = nullptr; }
+  d->wpart_elems = 0;
+  invalidate_graphs(d);                       // captured window steps hold the old pointer
+  CAI_HIP(hipMalloc((void**)&d->wpart, need * sizeof(float)));
+  d->wpart_elems = need;
+  return CAI_OK;
+}
+
+// The most recent earlier occurrence of the context's last match_len tokens; the tokens that followed it (at most num_draft)
+// are the draft (neural/neuraldecode.pas:7742-7765, PromptLookupDraft).  Returns the draft length (0: no match).
+static int lookup_draft(const int32_t* ctx_tok, int n_ctx, int match_len, int num_draft, int32_t* draft)
+{
+  if (match_len < 1 || num_draft < 1 || n_ctx < match_len + 1) return 0;
+  const int32_t* suffix = ctx_tok + n_ctx - match_len;
+  for (int p = n_ctx - match_len - 1; p >= 0; p--) {      // start of a candidate; the suffix itself (p = n_ctx - match_len) is excluded
+    bool same = true;
+    for (int i = 0; i < match_len && same; i++) same = ctx_tok[p + i] == suffix[i];
+    if (!same) continue;
+    const int follow = std::min(n_ctx - (p + match_len), num_draft);
+    for (int i = 0; i < follow; i++) draft[i] = ctx_tok[p + match_len + i];
+    return follow;                                         // the most recent occurrence wins
+  }
+  return 0;
+}
+
 }  // namespace cai
 
 using namespace cai;
@@ -459,12 +497,15 @@ extern "C" int cai_decoder_create(const cai_decoder_config* cfg, cai_decoder_t* 
   auto alloc_f = [&](float** p, size_t n) { return hipMalloc((void**)p, n * sizeof(float)); };
   hipError_t e = alloc_f(&d->theta, th.size());
   const int K = std::max(c.top_k, 1);
-  if (e == hipSuccess) e = alloc_f(&d->x, (size_t)B * c.d_model);
-  if (e == hipSuccess) e = alloc_f(&d->qkv, (size_t)B * (qw + 2 * kw));
-  if (e == hipSuccess) e = alloc_f(&d->att, (size_t)B * qw);
-  if (e == hipSuccess) e = alloc_f(&d->gu, (size_t)std::max(B, K) * 2 * c.ffn);
-  if (e == hipSuccess) e = alloc_f(&d->mid, (size_t)std::max(B, K) * c.ffn);
-  if (e == hipSuccess) e = alloc_f(&d->logits, (size_t)B * c.vocab);
+  // activation rows: eight whatever max_batch is (a window step of ONE sequence is up to eight rows wide; only the K,V
+  // cache grows with the number of sequences)
+  constexpr int RB = 8;
+  if (e == hipSuccess) e = alloc_f(&d->x, (size_t)RB * c.d_model);
+  if (e == hipSuccess) e = alloc_f(&d->qkv, (size_t)RB * (qw + 2 * kw));
+  if (e == hipSuccess) e = alloc_f(&d->att, (size_t)RB * qw);
+  if (e == hipSuccess) e = alloc_f(&d->gu, (size_t)std::max(RB, K) * 2 * c.ffn);
+  if (e == hipSuccess) e = alloc_f(&d->mid, (size_t)std::max(RB, K) * c.ffn);
+  if (e == hipSuccess) e = alloc_f(&d->logits, (size_t)RB * c.vocab);
   if (c.n_experts > 0) {
     // (eight rows whatever the batch: a prompt routes its tokens in groups of eight)
     if (e == hipSuccess) e = alloc_f(&d->router_logits, (size_t)8 * c.n_experts);
@@ -473,7 +514,7 @@ extern "C" int cai_decoder_create(const cai_decoder_config* cfg, cai_decoder_t* 
     if (e == hipSuccess) e = alloc_f(&d->moe_part, (size_t)K * c.d_model);
     if (e == hipSuccess) e = hipMalloc((void**)&d->moe_expert, (size_t)8 * K * sizeof(int32_t));
   }
-  const int ame = argmax_scratch_entries(c.vocab, B);
+  const int ame = argmax_scratch_entries(c.vocab, RB);
   if (e == hipSuccess) e = alloc_f(&d->am_v, (size_t)ame);
   if (e == hipSuccess) e = hipMalloc((void**)&d->am_i, (size_t)ame * sizeof(int32_t));
   if (e == hipSuccess) e = alloc_f(&d->ssq, 2 * 1024);
@@ -497,7 +538,7 @@ extern "C" int cai_decoder_destroy(cai_decoder_t d)
   if (ctx().ready) (void)hipStreamSynchronize(ctx().stream);
   invalidate_graphs(d);
   kv_free(&d->kv);
-  float* fs[] = {d->ssq, d->theta, d->x, d->qkv, d->att, d->gu, d->mid, d->logits, d->router_logits, d->router_probs, d->moe_gate, d->moe_part, d->final_norm};
+  float* fs[] = {d->wpart, d->ssq, d->theta, d->x, d->qkv, d->att, d->gu, d->mid, d->logits, d->router_logits, d->router_probs, d->moe_gate, d->moe_part, d->final_norm};
   for (float* p : fs) if (p) (void)hipFree(p);
   for (auto& L : d->layers) for (float* p : L.v) if (p) (void)hipFree(p);
   { float* pf[] = {d->px, d->pqkv, d->patt, d->pgu, d->pmid, d->ppart}; for (float* q : pf) if (q) (void)hipFree(q); }
@@ -595,6 +636,83 @@ extern "C" int cai_decoder_step(cai_decoder_t d, const int32_t* tokens, const in
     for (int l = 0; l < c.n_layers; l++) d->kv.len_at(b, l) = pos[b] + 1;
     if (argmax) argmax[b] = d->h_io[16 + b];
   }
+  return CAI_OK;
+}
+
+// Width-n window step of ONE sequence (StepForward on a width-K twin, neural/neuraldecode.pas:1151-1183 and 5696-5712; the verify
+// pass of speculative decoding, examples/SpeculativeDecoding/SpeculativeDecoding.lpr:646-663): tokens[r] is fed at position
+// pos0 + r, appended to the cache, and attends to everything before it; row r of the result is the model's output at position
+// pos0 + r.  The cache then holds pos0 + n rows: the caller keeps the prefix it commits with cai_decoder_truncate.
+extern "C" int cai_decoder_step_window(cai_decoder_t d, int seq, const int32_t* tokens, int n, int pos0, float* logits, int32_t* argmax)
+{
+  CAI_ENTER();
+  CAI_READY();
+  CAI_REQUIRE(d && tokens, "cai_decoder_step_window: null argument");
+  const cai_decoder_config& c = d->cfg;
+  CAI_REQUIRE(n >= 1 && n <= 8, "cai_decoder_step_window: width %d outside 1..8", n);
+  CAI_REQUIRE(seq >= 0 && seq < c.max_batch, "cai_decoder_step_window: sequence %d of %d", seq, c.max_batch);
+  int rc = check_ready(d); if (rc) return rc;
+  if (pos0 != d->kv.len_at(seq, 0)) return set_error(CAI_ERR_STATE, "cai_decoder_step_window: sequence %d is at position %d, got %d", seq, d->kv.len_at(seq, 0), pos0);
+  if (d->kv.evict_cap > 0 && n > 1) return set_error(CAI_ERR_UNSUPPORTED, "cai_decoder_step_window: a session with eviction rolls its cache and cannot take back a window; step one token at a time");
+  if (pos0 + n > c.max_ctx && d->kv.evict_cap == 0) return set_error(CAI_ERR_STATE, "cai_decoder_step_window: %d tokens from %d exceed max_ctx %d", n, pos0, c.max_ctx);
+  for (int i = 0; i < n; i++) CAI_REQUIRE(tokens[i] >= 0 && tokens[i] < c.vocab, "cai_decoder_step_window: token %d outside vocab %d", tokens[i], c.vocab);
+  Context& cx = ctx();
+  if (n > 1 && (rc = ensure_wpart(d))) return rc;
+  CAI_HIP(hipStreamSynchronize(cx.stream));   // h_io is reused
+  for (int i = 0; i < n; i++) { d->h_io[i] = tokens[i]; d->h_io[8 + i] = pos0 + i; }
+  CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
+  if ((rc = run_step(d, n, n > 1, seq))) return rc;
+  if (logits) CAI_HIP(hipMemcpyAsync(logits, d->logits, (size_t)n * c.vocab * 4, hipMemcpyDeviceToHost, cx.stream));
+  CAI_HIP(hipMemcpyAsync(d->h_io + 16, d->d_argmax, 8 * sizeof(int32_t), hipMemcpyDeviceToHost, cx.stream));
+  CAI_HIP(hipStreamSynchronize(cx.stream));
+  for (int l = 0; l < c.n_layers; l++) d->kv.len_at(seq, l) = pos0 + n;
+  if (argmax) for (int i = 0; i < n; i++) argmax[i] = d->h_io[16 + i];
+  return CAI_OK;
+}
+
+extern "C" int cai_prompt_lookup_draft(const int32_t* context, int n_ctx, int match_len, int num_draft, int32_t* draft_out, int* n_draft_out)
+{
+  CAI_ENTER();
+  CAI_REQUIRE(context && draft_out && n_draft_out && n_ctx >= 0, "cai_prompt_lookup_draft: bad argument");
+  *n_draft_out = lookup_draft(context, n_ctx, match_len, num_draft, draft_out);
+  return CAI_OK;
+}
+
+// Greedy continuation with prompt-lookup drafts (DecodePromptLookup, neural/neuraldecode.pas:7767-7866, on the cached session):
+// every pass feeds the last committed token plus the draft as ONE window, keeps the drafted tokens the model itself would
+// have produced, and rolls the cache back over the rest.  Every emitted token is the arg-max of a row whose inputs are
+// committed tokens, so the output is that of plain greedy decoding; only the number of passes differs.
+extern "C" int cai_decoder_generate_lookup(cai_decoder_t d, const int32_t* context, int n_ctx, int match_len, int num_draft,
+                                           int n_tokens, int32_t* tokens_out, int32_t* passes_out)
+{
+  CAI_ENTER();
+  CAI_READY();
+  CAI_REQUIRE(d && context && tokens_out && n_ctx >= 1 && n_tokens >= 1, "cai_decoder_generate_lookup: bad argument");
+  const cai_decoder_config& c = d->cfg;
+  if (d->kv.len_at(0, 0) != n_ctx - 1)
+    return set_error(CAI_ERR_STATE, "cai_decoder_generate_lookup: the cache of sequence 0 holds %d tokens, the context's first %d are expected (its last token is fed here)", d->kv.len_at(0, 0), n_ctx - 1);
+  if (n_ctx - 1 + n_tokens > c.max_ctx) return set_error(CAI_ERR_STATE, "cai_decoder_generate_lookup: %d tokens from %d exceed max_ctx %d", n_tokens, n_ctx - 1, c.max_ctx);
+  if (match_len < 1) match_len = 1;                       // (the reference clamps both the same way)
+  if (num_draft < 1) num_draft = 1;
+  const bool can_draft = d->kv.evict_cap == 0;            // a rolling cache cannot take a window back
+  std::vector<int32_t> all(context, context + n_ctx);
+  all.reserve((size_t)n_ctx + n_tokens);
+  int emitted = 0, passes = 0;
+  while (emitted < n_tokens) {
+    const int pos = (int)all.size() - 1;
+    int32_t win[8], am[8];
+    win[0] = all.back();
+    const int room = std::min(std::min(num_draft, 7), std::min(n_tokens - emitted - 1, c.max_ctx - pos - 1));
+    const int nd = can_draft && room > 0 ? lookup_draft(all.data(), (int)all.size(), match_len, room, win + 1) : 0;
+    const int rc = cai_decoder_step_window(d, 0, win, 1 + nd, pos, nullptr, am);
+    if (rc) return rc;
+    passes++;
+    int acc = 0;
+    all.push_back(am[0]); tokens_out[emitted++] = am[0];
+    while (acc < nd && emitted < n_tokens && win[1 + acc] == am[acc]) { acc++; all.push_back(am[acc]); tokens_out[emitted++] = am[acc]; }
+    for (int l = 0; l < c.n_layers; l++) d->kv.len_at(0, l) = pos + 1 + acc;   // rows of rejected drafts are dropped
+  }
+  if (passes_out) *passes_out = passes;
   return CAI_OK;
 }
 
@@ -777,6 +895,8 @@ extern "C" int cai_decoder_set_kv_dtype(cai_decoder_t d, int kv_dtype)
   }
   d->kv.evict_sinks = sinks; d->kv.evict_cap = cap;
   d->cfg.kv_dtype = kv_dtype;
+  // the number of cache slices depends on the storage type, and the prompt and window scratch were sized for the old one
+  d->pf_cap = 0; d->wpart_elems = 0;
   return CAI_OK;
 }
 

@@ -196,7 +196,9 @@ int launch_split_q6k(const uint8_t* raw, int64_t n_blocks, uint8_t* rec, uint8_t
 // both the rotary position and the cache slot the new K,V row goes to; the live range is [.., pos_dev[s]].
 // Activation row s uses cache sequence seq0 + s.  prompt_rows != 0: the n_seq rows are consecutive tokens of ONE
 // sequence (seq0): their K,V rows are appended first, then every row attends up to its own position; prompt_part must
-// hold n_seq * q_heads * n_splits * (head_dim + 2) floats.
+// hold n_seq * q_heads * n_splits * (head_dim + 2) floats.  1 = a prompt chunk (eight rows or more of a 128-wide cache go to the
+// matrix-core kernel, which may grow its operand planes); 2 = a window step inside a captured graph (decode kernels only,
+// nothing is allocated).
 int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, int n_seq, int q_heads, int window,
                      float softcap, const float* theta, const int32_t* pos_dev, float* out, int64_t out_stride, int seq0,
                      int prompt_rows = 0, float* prompt_part = nullptr,

@@ -91,6 +91,9 @@ function cai_decoder_destroy(d: TCaiDecoder): LongInt; cdecl; external CAIHIP_LI
 function cai_decoder_set_weight(d: TCaiDecoder; layer, slot: LongInt; w: TCaiQW): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_set_vector(d: TCaiDecoder; layer, slot: LongInt; v_host: PSingle; n: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_step(d: TCaiDecoder; tokens, pos: PLongInt; n_b: LongInt; logits: PSingle; argmax: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_decoder_step_window(d: TCaiDecoder; seq: LongInt; tokens: PLongInt; n, pos0: LongInt; logits: PSingle; argmax: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_prompt_lookup_draft(context: PLongInt; n_ctx, match_len, num_draft: LongInt; draft_out: PLongInt; n_draft_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_decoder_generate_lookup(d: TCaiDecoder; context: PLongInt; n_ctx, match_len, num_draft, n_tokens: LongInt; tokens_out: PLongInt; passes_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_generate(d: TCaiDecoder; first_token, pos, n_tokens: LongInt; tokens_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_profile(d: TCaiDecoder; token, reps: LongInt; us_per_step_out: PSingle; n_classes: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_prefill(d: TCaiDecoder; seq: LongInt; tokens: PLongInt; n, pos0: LongInt; last_logits: PSingle; argmax: PLongInt): LongInt; cdecl; external CAIHIP_LIB;

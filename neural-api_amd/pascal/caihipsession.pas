@@ -33,6 +33,7 @@ type
     FCfg: TCaiDecoderConfig;
     FSnap: TCaiKVSnap;
     FLogits: TCaiSingleArray;
+    FWindowLogits: TCaiSingleArray;
     procedure Check(rc: LongInt; const Where: string);
     function GetPosition: LongInt;
   public
@@ -52,6 +53,13 @@ type
     function Prefill(const Tokens: TCaiLongIntArray; First, Count: LongInt; WantLogits: Boolean): LongInt;
     // greedy fast path: MaxNew tokens fed back on the device (neural/neuralchatengine.pas:1493-1494)
     function GenerateGreedy(FirstToken, MaxNew: LongInt): TCaiLongIntArray;
+    // width-n window (n <= 8) at the session's position: the verify pass of speculative decoding (StepForward on a width-K
+    // twin, neural/neuraldecode.pas:1151-1183).  ArgMax[r] is the model's token after Tokens[First + r]; the logits rows go
+    // to WindowLogits when WantLogits.  The caller commits a prefix with TruncateTo.
+    procedure StepWindow(const Tokens: TCaiLongIntArray; First, Count: LongInt; WantLogits: Boolean; out ArgMax: TCaiLongIntArray);
+    // DecodePromptLookup on the cached session (neural/neuraldecode.pas:7767-7866): Context[0 .. n-2] must be in the cache;
+    // returns MaxNew greedy tokens, Passes receives the number of window steps taken
+    function GenerateLookup(const Context: TCaiLongIntArray; MatchLen, NumDraft, MaxNew: LongInt; out Passes: LongInt): TCaiLongIntArray;
     // the sampled branch without the logits read-back: the M most probable candidates after the penalties and the
     // temperature, sorted (neural/neuralchatengine.pas:1495-1501); the random draw stays on the host
     function Candidates(const HistIds, HistCounts: TCaiLongIntArray; Repetition, Frequency, Presence, Temperature: Single;
@@ -69,6 +77,7 @@ type
     property Position: LongInt read GetPosition;
     property VocabSize: LongInt read FCfg.vocab;
     property Logits: TCaiSingleArray read FLogits;
+    property WindowLogits: TCaiSingleArray read FWindowLogits;   // [Count][VocabSize] of the last StepWindow
     property Decoder: TCaiDecoder read FDec;
   end;
 
@@ -147,6 +156,32 @@ begin
   SetLength(Result, MaxNew);
   if MaxNew <= 0 then exit;
   Check(cai_decoder_generate(FDec, FirstToken, GetPosition, MaxNew, @Result[0]), 'cai_decoder_generate');
+end;
+
+procedure TCaiHipSession.StepWindow(const Tokens: TCaiLongIntArray; First, Count: LongInt; WantLogits: Boolean;
+  out ArgMax: TCaiLongIntArray);
+var
+  Rows: PSingle;
+begin
+  SetLength(ArgMax, Count);
+  if Count <= 0 then exit;
+  Rows := nil;
+  if WantLogits then
+  begin
+    SetLength(FWindowLogits, Count * FCfg.vocab);
+    Rows := @FWindowLogits[0];
+  end;
+  Check(cai_decoder_step_window(FDec, 0, @Tokens[First], Count, GetPosition, Rows, @ArgMax[0]), 'cai_decoder_step_window');
+end;
+
+function TCaiHipSession.GenerateLookup(const Context: TCaiLongIntArray; MatchLen, NumDraft, MaxNew: LongInt;
+  out Passes: LongInt): TCaiLongIntArray;
+begin
+  Passes := 0;
+  SetLength(Result, MaxNew);
+  if (MaxNew <= 0) or (Length(Context) = 0) then exit;
+  Check(cai_decoder_generate_lookup(FDec, @Context[0], Length(Context), MatchLen, NumDraft, MaxNew, @Result[0], @Passes),
+    'cai_decoder_generate_lookup');
 end;
 
 function TCaiHipSession.Candidates(const HistIds, HistCounts: TCaiLongIntArray; Repetition, Frequency, Presence,

@@ -1037,3 +1037,30 @@ int orc_model_step(orc_model* m, int token, int pos, float* logits)
   m->len = pos + 1;
   return orc_argmax(m->logits, c->vocab);
 }
+
+/* ------------------------------------------------------------------------------------------
+ * Prompt-lookup draft (neural/neuraldecode.pas:7742-7765), kept in the reference's own 1-based terms: the suffix is
+ * Context[CtxLen-MatchLen+1 .. CtxLen]; candidate starts P run from CtxLen-MatchLen down to 1 (P = CtxLen-MatchLen+1 would be
+ * the suffix itself); at the first P whose MatchLen tokens equal the suffix, FollowLen = CtxLen-(P+MatchLen)+1 tokens are
+ * available after the match, of which at most NumDraft are copied; the scan stops there whether or not anything was copied.
+ * Pinned by hand-derived cases and by an exhaustive comparison with the definition restated over all start positions on
+ * short contexts of a two- and three-letter alphabet (tests/test_oracle_lookup.py).
+ * ------------------------------------------------------------------------------------------ */
+int orc_prompt_lookup_draft(const int32_t* ctx, int n_ctx, int match_len, int num_draft, int32_t* draft)
+{
+  const int CtxLen = n_ctx;
+  if (match_len < 1 || num_draft < 1 || CtxLen < match_len + 1) return 0;
+  const int SuffixStart = CtxLen - match_len + 1;             /* 1-based */
+  for (int P = CtxLen - match_len; P >= 1; P--) {
+    int equal = 1;
+    for (int i = 0; i < match_len; i++)
+      if (ctx[P - 1 + i] != ctx[SuffixStart - 1 + i]) { equal = 0; break; }
+    if (!equal) continue;
+    int FollowLen = CtxLen - (P + match_len) + 1;
+    if (FollowLen > num_draft) FollowLen = num_draft;
+    if (FollowLen < 1) return 0;
+    for (int i = 0; i < FollowLen; i++) draft[i] = ctx[P + match_len - 1 + i];
+    return FollowLen;
+  }
+  return 0;
+}

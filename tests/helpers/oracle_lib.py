@@ -72,6 +72,7 @@ def lib():
         L.orc_model_truncate.argtypes = [C.c_void_p, C.c_int]; L.orc_model_truncate.restype = None
         L.orc_model_len.argtypes = [C.c_void_p]
         L.orc_model_step.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p]
+        L.orc_prompt_lookup_draft.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
         L.cpu_avx_dot_f32.restype = C.c_float; L.cpu_avx_dot_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
         L.cpu_avx_dot_int8.restype = C.c_float; L.cpu_avx_dot_int8.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
         L.cpu_linear_f32.argtypes = [C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int]; L.cpu_linear_f32.restype = None
@@ -189,3 +190,10 @@ def sample_candidates(logits, m, temperature=1.0, history=None, repetition=1.0, 
     tok = np.zeros(m, np.int32); p = np.zeros(m, np.float32)
     k = lib().orc_sample_candidates(_p(logits), logits.size, _p(ids), _p(counts), ids.size, repetition, frequency, presence, temperature, m, _p(tok), _p(p))
     return tok[:k], p[:k]
+
+
+def prompt_lookup_draft(context, match_len, num_draft):
+    context = np.ascontiguousarray(context, np.int32)
+    out = np.empty(max(num_draft, 1), np.int32)
+    n = lib().orc_prompt_lookup_draft(context.ctypes.data, context.size, match_len, num_draft, out.ctypes.data)
+    return out[:n].tolist()
