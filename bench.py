@@ -362,6 +362,33 @@ def main():
         cai.check(lib.cai_timer_stop(C.byref(ms)))
         cai.check(lib.cai_sync()); torch.cuda.synchronize()
         walls.append(time.perf_counter() - t1); evs.append(ms.value)
+    # ---- window steps (the verify pass of speculative decoding) and prompt-lookup generation from the same position: not part of
+    #      `value`; every token written equals the greedy one, so the figure depends on how often the continuation repeats earlier text ----
+    spec_info = None
+    if B == 1:
+        dec.truncate(pos)
+        greedy = dec.generate(tok, pos, K)
+        width = 8
+        win = np.concatenate([[tok], greedy[:width - 1]]).astype(np.int32)
+        dec.truncate(pos); dec.step_window(win, pos, want_logits=False)              # captures the window graph
+        cai.check(lib.cai_sync()); t1 = time.perf_counter()
+        n_win = 16
+        for _ in range(n_win):
+            dec.truncate(pos); am, _ = dec.step_window(win, pos, want_logits=False)
+        win_ms = (time.perf_counter() - t1) * 1e3 / n_win
+        dec.truncate(pos)
+        context = np.concatenate([prompt[:-1], [tok]]).astype(np.int32) if W == 0 else None
+        if context is None:
+            # the cache holds prompt + warm-up tokens: rebuild the token history the lookup searches
+            dec.truncate(prompt_len - 1)
+            hist = dec.generate(int(prompt[-1]), prompt_len - 1, W)
+            context = np.concatenate([prompt, hist]).astype(np.int32)
+        cai.check(lib.cai_sync()); t1 = time.perf_counter()
+        got, passes = dec.generate_lookup(context, K, 2, 7)
+        lk_wall = time.perf_counter() - t1
+        spec_info = {"window_width": width, "window_step_ms": round(win_ms, 4), "window_rows_equal_greedy": bool(np.array_equal(am, greedy[:width])),
+                     "lookup": {"match_len": 2, "num_draft": 7, "tokens": K, "passes": int(passes), "tok_per_s": round(K / lk_wall, 1),
+                                "identical_to_greedy": bool(np.array_equal(got, greedy))}}
     order = sorted(range(len(walls)), key=lambda i: walls[i])
     mid = order[len(order) // 2]
     wall = walls[mid]; ms = C.c_float(evs[mid])
@@ -460,6 +487,8 @@ def main():
                      "measured_stream_GB_per_s": round(copy_gbs, 1), "frac_of_measured_stream": round(k_gbs / copy_gbs, 4)},
     }
     res["config"]["timed_repetitions_ms_per_step"] = [round(w * 1e3 / K, 4) for w in walls]
+    if spec_info is not None:
+        res["config"]["speculative"] = spec_info
     if table is not None:
         total = sum(r["us_per_step"] for r in table)
         res["kernels"] = {"rows": table, "sum_us_per_step": round(total, 1), "graph_step_us": round(ms.value * 1e3 / K, 1),

@@ -203,3 +203,30 @@ def test_full_width_prompt_pass_equals_token_at_a_time(name, n_tok):
     nxt_p, l2_p = b.step(am_p, n_tok)
     assert rel_err(l2_p[0], l2_s[0]) < 2e-4 and int(nxt_p[0]) == int(nxt_s[0])
     b.close()
+
+
+@pytest.mark.parametrize("name", ["qwen2.5-7b", "qwen2.5-32b"])
+def test_full_width_window_step_equals_token_at_a_time(name):
+    """A width-8 window of one sequence (the verify pass of speculative decoding, neural/neuraldecode.pas:1151-1183) on the
+    full-width twins, over a cache long enough (4096 rows) for the window's attention to take the grouped multi-slice form:
+    every row within 2e-4 of the width-1 step at the same position (whose kernels the tests above pin to the oracle), same
+    arg-max, and after committing five of the eight rows the next width-1 step agrees as well."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    s = TWINS[name]
+    cfg = dict(s["cfg"], max_ctx=4096)
+    spec = full_width_spec(cfg, s["qtype"], s["head"], s["bias"], seed=123)
+    rng = np.random.default_rng(123)
+    toks = rng.integers(0, cfg["vocab"], 40).tolist()
+    dec = cai.Decoder(spec, kv_dtype=cai.KV_F16 if s["kv_f16"] else cai.KV_F32)
+    dec.prefill(toks[:24], 0, want_logits=False)
+    single = [dec.step(t, 24 + i) for i, t in enumerate(toks[24:33])]
+    dec.truncate(24)
+    am, lg = dec.step_window(toks[24:32], 24)
+    for r in range(8):
+        assert rel_err(lg[r], single[r][1][0]) < 2e-4, r
+        assert int(am[r]) == int(single[r][0][0]), r
+    dec.truncate(29)
+    nxt, l1 = dec.step(toks[29], 29)
+    assert rel_err(l1[0], single[5][1][0]) < 2e-4 and int(nxt[0]) == int(single[5][0][0])
+    dec.close()

@@ -1,7 +1,7 @@
 """The three environment switches the library reads select other code paths (no stream capture; token-by-token prompts;
 prompt attention through the decode kernels).  Each is read once per process, so each case runs in a child process with the
 variable set and is checked against the oracle there: a Q4_K decoder with QKV bias and 7 query heads per KV head, a 40-token
-prompt through cai_decoder_prefill, then 8 greedy tokens through cai_decoder_generate."""
+prompt through cai_decoder_prefill, then 8 greedy tokens through cai_decoder_generate, a window step and the lookup loop."""
 import os
 import subprocess
 import sys
@@ -34,6 +34,13 @@ ref = []
 for i in range(8):
     tok_o, _ = om.step(tok_o, len(prompt) + i); ref.append(tok_o)
 assert gen == ref, (gen, ref)
+# a width-5 window of the same sequence (eager launches under CAIHIP_NO_GRAPH) and the lookup loop built on it
+dec.truncate(len(prompt))
+am, lg = dec.step_window([tok_d] + gen[:4], len(prompt))
+assert am.tolist() == gen[:5], (am.tolist(), gen)
+dec.truncate(len(prompt))
+got, passes = dec.generate_lookup(prompt + [tok_d], 8, 1, 4)
+assert got.tolist() == gen and passes <= 8
 print("CHILD_OK")
 """
 
