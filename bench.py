@@ -368,14 +368,16 @@ def main():
     if B == 1:
         dec.truncate(pos)
         greedy = dec.generate(tok, pos, K)
-        width = 8
-        win = np.concatenate([[tok], greedy[:width - 1]]).astype(np.int32)
-        dec.truncate(pos); dec.step_window(win, pos, want_logits=False)              # captures the window graph
-        cai.check(lib.cai_sync()); t1 = time.perf_counter()
-        n_win = 16
-        for _ in range(n_win):
-            dec.truncate(pos); am, _ = dec.step_window(win, pos, want_logits=False)
-        win_ms = (time.perf_counter() - t1) * 1e3 / n_win
+        win_ms, rows_ok = {}, True
+        for width in (2, 4, 8):
+            win = np.concatenate([[tok], greedy[:width - 1]]).astype(np.int32)
+            dec.truncate(pos); dec.step_window(win, pos, want_logits=False)              # captures the window graph
+            cai.check(lib.cai_sync()); t1 = time.perf_counter()
+            n_win = 16
+            for _ in range(n_win):
+                dec.truncate(pos); am, _ = dec.step_window(win, pos, want_logits=False)
+            win_ms[str(width)] = round((time.perf_counter() - t1) * 1e3 / n_win, 4)
+            rows_ok = rows_ok and bool(np.array_equal(am, greedy[:width]))
         dec.truncate(pos)
         context = np.concatenate([prompt[:-1], [tok]]).astype(np.int32) if W == 0 else None
         if context is None:
@@ -386,7 +388,7 @@ def main():
         cai.check(lib.cai_sync()); t1 = time.perf_counter()
         got, passes = dec.generate_lookup(context, K, 2, 7)
         lk_wall = time.perf_counter() - t1
-        spec_info = {"window_width": width, "window_step_ms": round(win_ms, 4), "window_rows_equal_greedy": bool(np.array_equal(am, greedy[:width])),
+        spec_info = {"window_step_ms_by_width": win_ms, "window_rows_equal_greedy": rows_ok,
                      "lookup": {"match_len": 2, "num_draft": 7, "tokens": K, "passes": int(passes), "tok_per_s": round(K / lk_wall, 1),
                                 "identical_to_greedy": bool(np.array_equal(got, greedy))}}
     order = sorted(range(len(walls)), key=lambda i: walls[i])
