@@ -248,6 +248,10 @@ int cai_prompt_lookup_draft(const int32_t* context, int n_ctx, int match_len, in
  * passes taken (may be NULL); the cache ends n_ctx - 1 + n_tokens rows long. */
 int cai_decoder_generate_lookup(cai_decoder_t d, const int32_t* context, int n_ctx, int match_len, int num_draft,
                                 int n_tokens, int32_t* tokens_out, int32_t* passes_out);
+/* HiddenState of the session (neural/neuraldecode.pas:1314-1321, 5850-5857): the input of the vocabulary projection, i.e. the
+ * final RMSNorm of the residual stream, d_model floats (host), for row `row` (0..7) of the last step or window; row 0 after
+ * cai_decoder_prefill and cai_decoder_generate (the last token fed).  What contrastive search and embedding consumers read. */
+int cai_decoder_hidden_state(cai_decoder_t d, int row, float* hidden_out);
 /* Greedy continuation of sequence 0 with no host round trip between tokens: feeds `first_token` at
  * position `pos`, then each argmax as the next token; writes n_tokens ids (the greedy fast path of
  * neural/neuralchatengine.pas:1485-1561 with ArgMaxRow on the device). */

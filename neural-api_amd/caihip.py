@@ -21,7 +21,7 @@ cai_dev_alloc cai_dev_free cai_dev_upload cai_dev_download cai_dev_copy
 cai_qw_create cai_qw_create_int8row cai_qw_destroy cai_qw_info cai_qw_dequant_rows cai_qgemv cai_ffn_gateup cai_qgemm
 cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_argmax_noalloc cai_router_topk
 cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_kv_export_layer cai_kv_import_layer cai_kv_set_eviction cai_kv_rows cai_attn_decode
-cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_step_window cai_prompt_lookup_draft cai_decoder_generate_lookup cai_decoder_generate cai_decoder_profile
+cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_hidden_state cai_decoder_step_window cai_prompt_lookup_draft cai_decoder_generate_lookup cai_decoder_generate cai_decoder_profile
 cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_set_eviction cai_decoder_cache_rows cai_decoder_set_kv_dtype cai_decoder_set_rope_scaling cai_decoder_set_rope_freq_factors cai_decoder_set_rope_out_scale cai_sample_candidates cai_decoder_candidates cai_decoder_snapshot cai_decoder_restore
 cai_decoder_weight_bytes cai_decoder_get_config cai_decoder_load_gguf
 cai_gguf_open cai_gguf_close cai_gguf_info cai_gguf_meta_int cai_gguf_meta_float cai_gguf_meta_str cai_gguf_meta_array_count
@@ -104,6 +104,7 @@ def load():
         L.cai_decoder_step.argtypes = [vp, vp, vp, i32, vp, vp]
         L.cai_decoder_generate.argtypes = [vp, i32, i32, i32, vp]
         L.cai_decoder_step_window.argtypes = [vp, i32, vp, i32, i32, vp, vp]
+        L.cai_decoder_hidden_state.argtypes = [vp, i32, vp]
         L.cai_prompt_lookup_draft.argtypes = [vp, i32, i32, i32, vp, vp]
         L.cai_decoder_generate_lookup.argtypes = [vp, vp, i32, i32, i32, i32, vp, vp]
         L.cai_decoder_profile.argtypes = [vp, i32, i32, vp, i32]
@@ -430,6 +431,12 @@ class Decoder:
     def generate(self, first_token, pos, n):
         out = np.empty(n, np.int32)
         check(load().cai_decoder_generate(self.h, int(first_token), int(pos), n, _ptr(out)))
+        return out
+
+    def hidden_state(self, row=0):
+        """input of the vocabulary projection for a row of the last step or window (HiddenState of the reference session)"""
+        out = np.empty(self.cfg.d_model, np.float32)
+        check(load().cai_decoder_hidden_state(self.h, row, _ptr(out)))
         return out
 
     def step_window(self, tokens, pos0, seq=0, want_logits=True):

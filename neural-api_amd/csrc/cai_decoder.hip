@@ -812,6 +812,8 @@ extern "C" int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* toke
         MultiGemv hm{}; hm.n = 1; hm.w[0] = hw; hm.rows[0] = c.vocab;
         if ((rc = launch_gemv_multi(hm, d->px + (int64_t)(m - 1) * c.d_model, 1, d->logits, c.vocab, CAI_ACT_NONE, nullptr, d->final_norm, c.eps, 0))) return rc;
         launch_argmax(d->logits, c.vocab, 1, d->d_argmax, d->am_v, d->am_i);
+        // the last token's residual stream goes where a step leaves it (cai_decoder_hidden_state reads row 0)
+        CAI_HIP(hipMemcpyAsync(d->x, d->px + (int64_t)(m - 1) * c.d_model, (size_t)c.d_model * 4, hipMemcpyDeviceToDevice, cx.stream));
       }
     }
   }
@@ -820,6 +822,25 @@ extern "C" int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* toke
   CAI_HIP(hipStreamSynchronize(cx.stream));
   for (int l = 0; l < c.n_layers; l++) d->kv.len_at(seq, l) = pos0 + n;
   if (argmax) *argmax = d->h_io[16];
+  return CAI_OK;
+}
+
+// HiddenState (neural/neuraldecode.pas:1314-1321, 5850-5857): the input of the vocabulary projection - the final RMSNorm of the
+// residual stream - for row `row` of the last step or window (row 0 after cai_decoder_prefill / cai_decoder_generate: the last
+// token fed).  The decode step fuses that norm into the projection, so it is recomputed here from the stream the step left.
+extern "C" int cai_decoder_hidden_state(cai_decoder_t d, int row, float* hidden_out)
+{
+  CAI_ENTER();
+  CAI_READY();
+  CAI_REQUIRE(d && hidden_out, "cai_decoder_hidden_state: null argument");
+  CAI_REQUIRE(row >= 0 && row < 8, "cai_decoder_hidden_state: row %d outside 0..7", row);
+  if (!d->final_norm) return set_error(CAI_ERR_STATE, "cai_decoder_hidden_state: final norm gain not set");
+  Context& cx = ctx();
+  const int dm = d->cfg.d_model;
+  int rc = ensure_stage(&cx.stage_out, &cx.stage_out_cap, (size_t)dm * 4); if (rc) return rc;
+  if ((rc = launch_rmsnorm(d->x + (int64_t)row * dm, d->final_norm, dm, 1, d->cfg.eps, (float*)cx.stage_out))) return rc;
+  CAI_HIP(hipMemcpyAsync(hidden_out, cx.stage_out, (size_t)dm * 4, hipMemcpyDeviceToHost, cx.stream));
+  CAI_HIP(hipStreamSynchronize(cx.stream));
   return CAI_OK;
 }
 

@@ -91,6 +91,7 @@ function cai_decoder_destroy(d: TCaiDecoder): LongInt; cdecl; external CAIHIP_LI
 function cai_decoder_set_weight(d: TCaiDecoder; layer, slot: LongInt; w: TCaiQW): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_set_vector(d: TCaiDecoder; layer, slot: LongInt; v_host: PSingle; n: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_step(d: TCaiDecoder; tokens, pos: PLongInt; n_b: LongInt; logits: PSingle; argmax: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_decoder_hidden_state(d: TCaiDecoder; row: LongInt; hidden_out: PSingle): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_step_window(d: TCaiDecoder; seq: LongInt; tokens: PLongInt; n, pos0: LongInt; logits: PSingle; argmax: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_prompt_lookup_draft(context: PLongInt; n_ctx, match_len, num_draft: LongInt; draft_out: PLongInt; n_draft_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_generate_lookup(d: TCaiDecoder; context: PLongInt; n_ctx, match_len, num_draft, n_tokens: LongInt; tokens_out: PLongInt; passes_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;

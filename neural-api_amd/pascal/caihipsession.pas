@@ -73,6 +73,8 @@ type
     procedure EnableEviction(SinkTokens, RecentWindow: LongInt);
     procedure DisableEviction;
     function CacheRows(LayerIdx: LongInt): LongInt;    // SDPACacheLength(Index)
+    // HiddenState: the input of the vocabulary projection for a row of the last step or window (d_model values)
+    function HiddenState(Row: LongInt = 0): TCaiSingleArray;
 
     property Position: LongInt read GetPosition;
     property VocabSize: LongInt read FCfg.vocab;
@@ -235,6 +237,12 @@ end;
 procedure TCaiHipSession.DisableEviction;
 begin
   Check(cai_decoder_set_eviction(FDec, 0, 0), 'cai_decoder_set_eviction');
+end;
+
+function TCaiHipSession.HiddenState(Row: LongInt): TCaiSingleArray;
+begin
+  SetLength(Result, FCfg.d_model);
+  Check(cai_decoder_hidden_state(FDec, Row, @Result[0]), 'cai_decoder_hidden_state');
 end;
 
 function TCaiHipSession.CacheRows(LayerIdx: LongInt): LongInt;

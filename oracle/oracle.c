@@ -1038,6 +1038,10 @@ int orc_model_step(orc_model* m, int token, int pos, float* logits)
   return orc_argmax(m->logits, c->vocab);
 }
 
+/* HiddenState (neural/neuraldecode.pas:5850-5857): the output of the layer feeding the vocabulary projection, which in the
+ * imported decoders is the final TokenRMSNorm (neuralpretrained.pas:16872-16875).  The step above keeps it in m->h. */
+const float* orc_model_hidden(const orc_model* m) { return m->h; }
+
 /* ------------------------------------------------------------------------------------------
  * Prompt-lookup draft (neural/neuraldecode.pas:7742-7765), kept in the reference's own 1-based terms: the suffix is
  * Context[CtxLen-MatchLen+1 .. CtxLen]; candidate starts P run from CtxLen-MatchLen down to 1 (P = CtxLen-MatchLen+1 would be

@@ -141,6 +141,9 @@ int  orc_model_len(const orc_model* m);
 /* Runs one token at position `pos` (== current cache length). logits may be NULL. Returns argmax. */
 int  orc_model_step(orc_model* m, int token, int pos, float* logits);
 
+/* The input of the vocabulary projection at the last step (final RMSNorm of the residual stream, d_model floats): HiddenState of
+ * the reference session (neural/neuraldecode.pas:5850-5857 with the heuristic of 6794-6807: the layer feeding the head). */
+const float* orc_model_hidden(const orc_model* m);
 /* PromptLookupDraft on token ids (neural/neuraldecode.pas:7742-7765): the (at most num_draft) tokens that followed the most
  * recent STRICTLY EARLIER occurrence of the context's last match_len tokens.  Returns the draft length. */
 int  orc_prompt_lookup_draft(const int32_t* ctx, int n_ctx, int match_len, int num_draft, int32_t* draft);

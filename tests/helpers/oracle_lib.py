@@ -72,6 +72,7 @@ def lib():
         L.orc_model_truncate.argtypes = [C.c_void_p, C.c_int]; L.orc_model_truncate.restype = None
         L.orc_model_len.argtypes = [C.c_void_p]
         L.orc_model_step.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p]
+        L.orc_model_hidden.argtypes = [C.c_void_p]; L.orc_model_hidden.restype = C.POINTER(C.c_float)
         L.orc_prompt_lookup_draft.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
         L.cpu_avx_dot_f32.restype = C.c_float; L.cpu_avx_dot_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
         L.cpu_avx_dot_int8.restype = C.c_float; L.cpu_avx_dot_int8.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
@@ -174,6 +175,10 @@ class OracleModel:
         r = lib().orc_model_step(self.h, int(token), int(pos), _p(lg))
         assert r >= 0, "oracle step failed"
         return r, lg
+
+    def hidden(self):
+        """the input of the vocabulary projection at the last step (a copy)"""
+        return np.ctypeslib.as_array(lib().orc_model_hidden(self.h), shape=(self.cfg.d_model,)).copy()
 
     def __del__(self):
         try:

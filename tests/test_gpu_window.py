@@ -137,3 +137,38 @@ def test_window_and_lookup_refusals():
         dec.step_window([1, 2], 1)
     out, passes = dec.generate_lookup([1, 1], 12, 1, 4)       # drafts are switched off: one token per pass
     assert passes == 12 and len(out) == 12
+
+
+@pytest.mark.parametrize("name", ["qwen7b_like_q4k", "smollm_like_q8", "olmoe_like_q8"])
+def test_hidden_state_after_steps_windows_prompts_and_generation(name):
+    """HiddenState of the reference session (neural/neuraldecode.pas:1314-1321, 5850-5857): the vector the vocabulary projection reads.
+    Pinned two ways: against the oracle's final-norm output at the same position (1e-4 of its largest element), and through the
+    head itself - projecting the returned vector with the oracle's head product gives the step's logits."""
+    from helpers.device import rel_err
+    cai, spec, dec = make(name)
+    rng = np.random.default_rng(21)
+    toks = rng.integers(0, spec["cfg"]["vocab"], 24).tolist()
+    om = oracle_model(spec, acc64=1)
+    hid = []
+    for p, t in enumerate(toks):
+        om.step(t, p); hid.append(om.hidden())
+        _, lg = dec.step(t, p)
+        if p in (0, 7, 23):
+            h = dec.hidden_state()
+            assert rel_err(h, hid[p]) < 1e-4, p
+            head = spec["tensors"].get((-1, O.W_HEAD)) or spec["tensors"][(-1, O.W_EMBED)]
+            proj = O.gemv(head["type"], head["raw"], head["rows"], head["cols"], h[None, :], None, 0, 1)
+            assert rel_err(proj[0], lg[0]) < 1e-4
+    # rows of a window
+    dec.truncate(10)
+    dec.step_window(toks[10:16], 10, want_logits=False)
+    for r in (0, 3, 5):
+        assert rel_err(dec.hidden_state(r), hid[10 + r]) < 1e-4, r
+    # after a prompt pass and after device-side generation: row 0 is the last token fed
+    dec.reset(); dec.prefill(toks[:20], 0, want_logits=False)
+    assert rel_err(dec.hidden_state(), hid[19]) < 1e-4
+    g = dec.generate(toks[20], 20, 3)
+    om.truncate(20); om.step(toks[20], 20); om.step(int(g[0]), 21); om.step(int(g[1]), 22)
+    assert rel_err(dec.hidden_state(), om.hidden()) < 1e-4
+    with pytest.raises(cai.CaiError, match="row 8"):
+        dec.hidden_state(8)
