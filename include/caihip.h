@@ -313,6 +313,10 @@ int cai_decoder_set_rope_freq_factors(cai_decoder_t d, const float* factors, int
 int cai_decoder_set_rope_out_scale(cai_decoder_t d, float scale);
 int cai_decoder_snapshot(cai_decoder_t d, int seq, cai_kv_snap_t* out);
 int cai_decoder_restore(cai_decoder_t d, int seq, cai_kv_snap_t snap);
+/* Sequence dst_seq becomes a copy of src_seq (rows and length), device to device on the library's stream: the cache fork of a
+ * beam search, whose survivors each continue from their parent's cache (DecodeBeamSearchCachedAll, neural/neuraldecode.pas:1436-1453,
+ * keeps one snapshot per hypothesis instead).  The beams of a step are then ONE cai_decoder_step over the sequences. */
+int cai_decoder_fork(cai_decoder_t d, int src_seq, int dst_seq);
 /* Bytes of weights, biases and gains one decoded token streams (for roofline accounting). */
 /* the configuration the decoder was created with (a loader fills it from the file) */
 int cai_decoder_get_config(cai_decoder_t d, cai_decoder_config* out);

@@ -22,7 +22,7 @@ cai_qw_create cai_qw_create_int8row cai_qw_destroy cai_qw_info cai_qw_dequant_ro
 cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_argmax_noalloc cai_router_topk
 cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_kv_export_layer cai_kv_import_layer cai_kv_set_eviction cai_kv_rows cai_attn_decode
 cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_hidden_state cai_decoder_step_window cai_prompt_lookup_draft cai_decoder_generate_lookup cai_decoder_generate cai_decoder_profile
-cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_set_eviction cai_decoder_cache_rows cai_decoder_set_kv_dtype cai_decoder_set_rope_scaling cai_decoder_set_rope_freq_factors cai_decoder_set_rope_out_scale cai_sample_candidates cai_decoder_candidates cai_decoder_snapshot cai_decoder_restore
+cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_set_eviction cai_decoder_cache_rows cai_decoder_set_kv_dtype cai_decoder_set_rope_scaling cai_decoder_set_rope_freq_factors cai_decoder_set_rope_out_scale cai_sample_candidates cai_decoder_candidates cai_decoder_snapshot cai_decoder_restore cai_decoder_fork
 cai_decoder_weight_bytes cai_decoder_get_config cai_decoder_load_gguf
 cai_gguf_open cai_gguf_close cai_gguf_info cai_gguf_meta_int cai_gguf_meta_float cai_gguf_meta_str cai_gguf_meta_array_count
 cai_gguf_meta_array_str cai_gguf_find_tensor cai_gguf_tensor_info cai_gguf_tensor_data cai_gguf_load_qw""".split()
@@ -122,6 +122,7 @@ def load():
         L.cai_decoder_cache_rows.argtypes = [vp, i32, i32, C.POINTER(i32)]
         L.cai_decoder_snapshot.argtypes = [vp, i32, C.POINTER(vp)]
         L.cai_decoder_restore.argtypes = [vp, i32, vp]
+        L.cai_decoder_fork.argtypes = [vp, i32, i32]
         L.cai_decoder_weight_bytes.argtypes = [vp, C.POINTER(i64)]
         L.cai_decoder_get_config.argtypes = [vp, C.POINTER(DecoderConfig)]
         L.cai_decoder_load_gguf.argtypes = [C.c_char_p, i32, i32, i32, C.POINTER(vp)]
@@ -514,6 +515,9 @@ class Decoder:
 
     def restore(self, s, seq=0):
         check(load().cai_decoder_restore(self.h, seq, s))
+
+    def fork(self, src, dst):
+        check(load().cai_decoder_fork(self.h, src, dst))
 
     def weight_bytes(self):
         b = C.c_int64()

@@ -1338,6 +1338,32 @@ int kv_restore(cai_kv_s* kv, int seq, const cai_kv_snap_s* s)
   return CAI_OK;
 }
 
+// Sequence dst becomes a copy of sequence src (the cache-forking step of a beam search: every survivor continues from its
+// parent's rows, neural/neuraldecode.pas:1436-1449): the live rows of every (layer, KV head) plane move device to device, on
+// the library's stream, without a snapshot in between.
+int kv_fork(cai_kv_s* kv, int src, int dst)
+{
+  if (src == dst) return CAI_OK;
+  int rows = 0;
+  for (int l = 0; l < kv->n_layers; l++) rows = std::max(rows, kv->live(kv->len_at(src, l)));
+  if (rows > 0) {
+    const size_t row_b = (size_t)kv->head_dim * kv->elem(), seq_b = (size_t)kv->seq_elems() * kv->elem();
+    for (int which = 0; which < 2; which++) {
+      char* base = (char*)(which ? kv->v : kv->k);
+      CAI_HIP(hipMemcpy2DAsync(base + dst * seq_b, (size_t)kv->max_ctx * row_b, base + src * seq_b, (size_t)kv->max_ctx * row_b, (size_t)rows * row_b,
+                               (size_t)kv->n_layers * kv->kv_heads, hipMemcpyDeviceToDevice, ctx().stream));
+    }
+    if (kv->dtype == CAI_KV_I8)
+      for (int which = 0; which < 2; which++) {
+        float* base = which ? kv->vs : kv->ks;
+        CAI_HIP(hipMemcpy2DAsync(base + (size_t)dst * kv->seq_rows(), (size_t)kv->max_ctx * 4, base + (size_t)src * kv->seq_rows(), (size_t)kv->max_ctx * 4,
+                                 (size_t)rows * 4, (size_t)kv->n_layers * kv->kv_heads, hipMemcpyDeviceToDevice, ctx().stream));
+      }
+  }
+  for (int l = 0; l < kv->n_layers; l++) kv->len_at(dst, l) = kv->len_at(src, l);
+  return CAI_OK;
+}
+
 }  // namespace cai
 
 // ------------------------------------------------------------------------------------------

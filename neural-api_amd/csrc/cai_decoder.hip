@@ -1008,6 +1008,16 @@ extern "C" int cai_decoder_restore(cai_decoder_t d, int seq, cai_kv_snap_t snap)
   return kv_restore(&d->kv, seq, snap);
 }
 
+extern "C" int cai_decoder_fork(cai_decoder_t d, int src_seq, int dst_seq)
+{
+  CAI_ENTER();
+  CAI_READY();
+  CAI_REQUIRE(d, "cai_decoder_fork: null decoder");
+  CAI_REQUIRE(src_seq >= 0 && src_seq < d->cfg.max_batch && dst_seq >= 0 && dst_seq < d->cfg.max_batch,
+              "cai_decoder_fork: sequences %d -> %d of %d", src_seq, dst_seq, d->cfg.max_batch);
+  return kv_fork(&d->kv, src_seq, dst_seq);
+}
+
 extern "C" int cai_decoder_get_config(cai_decoder_t d, cai_decoder_config* out)
 {
   CAI_ENTER();

@@ -208,6 +208,7 @@ void kv_free(cai_kv_s* kv);
 int kv_set_eviction(cai_kv_s* kv, int sinks, int recent);
 int kv_snapshot(cai_kv_s* kv, int seq, cai_kv_snap_s** out);
 int kv_restore(cai_kv_s* kv, int seq, const cai_kv_snap_s* snap);
+int kv_fork(cai_kv_s* kv, int src, int dst);
 // multi-token linear layer (matrix cores for Q4_K, small-batch kernel otherwise); gain != null fuses RMSNorm
 int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok,
                    float* y, int64_t y_stride, const float* residual);

@@ -115,6 +115,7 @@ function cai_decoder_set_rope_out_scale(d: TCaiDecoder; scale: Single): LongInt;
 function cai_decoder_cache_rows(d: TCaiDecoder; seq, layer: LongInt; rows_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_snapshot(d: TCaiDecoder; seq: LongInt; out_snap: PCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_restore(d: TCaiDecoder; seq: LongInt; snap: TCaiKVSnap): LongInt; cdecl; external CAIHIP_LIB;
+function cai_decoder_fork(d: TCaiDecoder; src_seq, dst_seq: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_weight_bytes(d: TCaiDecoder; algorithmic_bytes_out: PInt64): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_get_config(d: TCaiDecoder; out_cfg: Pointer): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_load_gguf(path: PChar; max_ctx, max_batch, kv_dtype: LongInt; out_decoder: PCaiDecoder): LongInt; cdecl; external CAIHIP_LIB;

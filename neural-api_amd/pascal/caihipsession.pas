@@ -70,6 +70,7 @@ type
     procedure Snapshot;
     procedure Restore;
     procedure EnableInt8KVCache;                       // on a fresh session only, like the reference
+    procedure DisableInt8KVCache;                      // back to fp32 rows (neural/neuraldecode.pas:1290), fresh session only
     procedure EnableEviction(SinkTokens, RecentWindow: LongInt);
     procedure DisableEviction;
     function CacheRows(LayerIdx: LongInt): LongInt;    // SDPACacheLength(Index)
@@ -227,6 +228,11 @@ end;
 procedure TCaiHipSession.EnableInt8KVCache;
 begin
   Check(cai_decoder_set_kv_dtype(FDec, CAI_KV_I8), 'cai_decoder_set_kv_dtype');
+end;
+
+procedure TCaiHipSession.DisableInt8KVCache;
+begin
+  Check(cai_decoder_set_kv_dtype(FDec, CAI_KV_F32), 'cai_decoder_set_kv_dtype');
 end;
 
 procedure TCaiHipSession.EnableEviction(SinkTokens, RecentWindow: LongInt);

@@ -172,3 +172,39 @@ def test_hidden_state_after_steps_windows_prompts_and_generation(name):
     assert rel_err(dec.hidden_state(), om.hidden()) < 1e-4
     with pytest.raises(cai.CaiError, match="row 8"):
         dec.hidden_state(8)
+
+
+@pytest.mark.parametrize("kv", [0, 2])
+def test_forked_sequences_step_as_a_batch_like_sequences_built_one_by_one(kv):
+    """The cache fork of a beam search (DecodeBeamSearchCachedAll, neural/neuraldecode.pas:1436-1453: every surviving hypothesis
+    continues from its parent's cache): sequence 0 ingests the prompt, sequences 1..3 are forked from it - directly, and through a
+    snapshot restored into another sequence -, then all four take DIFFERENT tokens in one batched step.  Each row must equal a
+    session that ingested prompt + that token alone."""
+    from helpers.device import rel_err
+    cai, spec, dec = make("qwen7b_like_q4k", max_batch=4, kv_dtype=kv)
+    rng = np.random.default_rng(4)
+    prompt = rng.integers(0, spec["cfg"]["vocab"], 20).tolist()
+    branch = [[5, 9], [17, 3], [900, 41], [2, 2]]
+    want = []
+    for b in range(4):
+        dec.reset(0); dec.prefill(prompt, 0, want_logits=False)
+        dec.step(branch[b][0], 20, want_logits=False)
+        want.append(dec.step(branch[b][1], 21)[1][0].copy())
+    dec.reset(0); dec.prefill(prompt, 0, want_logits=False)
+    dec.fork(0, 1); dec.fork(0, 2)
+    snap = dec.snapshot(0); dec.restore(snap, seq=3); cai.load().cai_kv_snap_destroy(snap)
+    assert [dec.len(b) for b in range(4)] == [20] * 4
+    dec.step([br[0] for br in branch], [20] * 4, want_logits=False)
+    _, lg = dec.step([br[1] for br in branch], [21] * 4)
+    for b in range(4):
+        assert rel_err(lg[b], want[b]) < (2e-3 if kv == 2 else 2e-4), b
+    # a fork overwrites what the target held, and a fork onto itself is a no-op
+    dec.fork(1, 0); dec.fork(2, 2)
+    assert dec.len(0) == 22
+    _, l0 = dec.step([7], [22])
+    dec.truncate(22, seq=1)
+    dec.reset(0); dec.prefill(prompt + branch[1], 0, want_logits=False)
+    _, l1 = dec.step([7], [22])
+    assert rel_err(l0[0], l1[0]) < (2e-3 if kv == 2 else 2e-4)
+    with pytest.raises(cai.CaiError, match="sequences 0 -> 4"):
+        dec.fork(0, 4)
