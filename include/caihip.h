@@ -275,8 +275,9 @@ int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* tokens, int n, 
  * probabilities by token id.  hist_ids / hist_counts: the DISTINCT tokens of the context and how often each occurred
  * (TNNetTokenHistoryPenalty's FSeen / FCounts); repetition 1, frequency 0, presence 0, temperature 1 are no-ops.
  * The draw (uniform over the window for TopK / TopP, weighted for WeightedTopK / MinP) stays with the host and its
- * random generator.  *count_out = min(m, n).  cai_decoder_candidates reads logits row `row` of the session's last
- * step in place (no read-back of the row); cai_sample_candidates takes any row (CAI_X_DEVICE: a device pointer). */
+ * random generator.  *count_out = min(m, n).  cai_decoder_candidates reads logits row `row` (0..7) of the session's last
+ * step (row = sequence) or window (row = position in the window) in place, with no read-back of the row (after a prompt pass
+ * and after cai_decoder_generate: row 0); cai_sample_candidates takes any row (CAI_X_DEVICE: a device pointer). */
 int cai_sample_candidates(const float* logits, int n, const int32_t* hist_ids, const int32_t* hist_counts, int n_hist,
                           float repetition, float frequency, float presence, float temperature, int m,
                           int32_t* tokens_out, float* probs_out, int* count_out, int flags);

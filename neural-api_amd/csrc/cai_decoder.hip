@@ -852,7 +852,7 @@ extern "C" int cai_decoder_candidates(cai_decoder_t d, int row, const int32_t* h
   CAI_ENTER();
   CAI_READY();
   CAI_REQUIRE(d && tokens_out && probs_out, "cai_decoder_candidates: null argument");
-  CAI_REQUIRE(row >= 0 && row < d->cfg.max_batch, "cai_decoder_candidates: row %d of %d", row, d->cfg.max_batch);
+  CAI_REQUIRE(row >= 0 && row < 8, "cai_decoder_candidates: row %d outside 0..7", row);   // a row of the last step (sequence) or window (position)
   CAI_REQUIRE(m >= 1 && m <= 1024, "cai_decoder_candidates: %d candidates (1..1024)", m);
   return run_candidates(d->logits + (int64_t)row * d->cfg.vocab, d->cfg.vocab, hist_ids, hist_counts, n_hist,
                         repetition, frequency, presence, temperature, m, tokens_out, probs_out, count_out);

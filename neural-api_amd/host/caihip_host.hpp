@@ -185,10 +185,39 @@ class TNNetStreamingDecoder {
   void Reset() { Check(cai_decoder_reset(d_, 0)); }
   // One streamed forward of a window of token ids; AbsPos is the absolute position of the FIRST token of the window.
   // After it, Output() holds the logits of the window's last token and ArgMaxRow() their arg-max (lowest index on ties).
+  // A window of 2..8 tokens (the verify pass of speculative decoding, neural/neuraldecode.pas:1151-1183) also keeps every
+  // row: OutputRow(r) / ArgMaxRows()[r] belong to position AbsPos + r.  Longer windows are prompt passes (last row only).
   void StepForward(const int32_t* Tokens, int Count, int AbsPos)
   {
+    rows_ = 0;
     if (Count == 1) { int32_t p = AbsPos; Check(cai_decoder_step(d_, Tokens, &p, 1, logits_.data(), &argmax_)); }
+    else if (Count <= 8) {
+      window_.resize((size_t)Count * (size_t)cfg_.vocab); argmax_rows_.resize((size_t)Count);
+      Check(cai_decoder_step_window(d_, 0, Tokens, Count, AbsPos, window_.data(), argmax_rows_.data()));
+      rows_ = Count;
+      std::copy(window_.end() - cfg_.vocab, window_.end(), logits_.begin());
+      argmax_ = argmax_rows_.back();
+    }
     else Check(cai_decoder_prefill(d_, 0, Tokens, Count, AbsPos, logits_.data(), &argmax_));
+  }
+  int WindowRows() const { return rows_; }
+  const float* OutputRow(int r) const { return window_.data() + (size_t)r * (size_t)cfg_.vocab; }
+  const std::vector<int32_t>& ArgMaxRows() const { return argmax_rows_; }
+  // HiddenState (neural/neuraldecode.pas:1314-1321): the input of the vocabulary projection for a row of the last step or window
+  std::vector<float> HiddenState(int Row = 0)
+  {
+    std::vector<float> h((size_t)cfg_.d_model);
+    Check(cai_decoder_hidden_state(d_, Row, h.data()));
+    return h;
+  }
+  // DecodePromptLookup on the cached session (neural/neuraldecode.pas:7767-7866): Context minus its last token must be in
+  // the cache; returns n greedy tokens, *Passes the number of window steps taken
+  std::vector<int32_t> GenerateLookup(const std::vector<int32_t>& Context, int MatchLen, int NumDraft, int n, int* Passes = nullptr)
+  {
+    std::vector<int32_t> out((size_t)n); int32_t passes = 0;
+    Check(cai_decoder_generate_lookup(d_, Context.data(), (int)Context.size(), MatchLen, NumDraft, n, out.data(), &passes));
+    if (Passes) *Passes = passes;
+    return out;
   }
   void TruncateTo(int CommittedLen) { Check(cai_decoder_truncate(d_, 0, CommittedLen)); }
   int SDPACacheLength(int Index = 0) const { int n = 0; Check(cai_decoder_cache_rows(d_, 0, Index, &n)); return n; }
@@ -202,14 +231,14 @@ class TNNetStreamingDecoder {
   void RestoreSnapshot(const TNNetDecoderSessionSnapshot* Snap) { Check(cai_decoder_restore(d_, 0, Snap->handle())); }
   const std::vector<float>& Output() const { return logits_; }
   int ArgMaxRow() const { return argmax_; }
-  // RowSoftMax -> penalty -> temperature on the device, over the row of the last StepForward; the m most probable
+  // RowSoftMax -> penalty -> temperature on the device, over the (last) row of the last StepForward; the m most probable
   // tokens come back instead of the row (neural/neuralchatengine.pas:1495-1501)
   TNNetCandidates Candidates(int m, float Temperature = 1.0f, const TNNetTokenHistory* History = nullptr,
                              float RepetitionPenalty = 1.0f, float FrequencyPenalty = 0.0f, float PresencePenalty = 0.0f)
   {
     TNNetCandidates c; c.Token.resize((size_t)m); c.Score.resize((size_t)m);
     int n = 0;
-    Check(cai_decoder_candidates(d_, 0, History ? History->Ids().data() : nullptr, History ? History->Counts().data() : nullptr,
+    Check(cai_decoder_candidates(d_, rows_ ? rows_ - 1 : 0, History ? History->Ids().data() : nullptr, History ? History->Counts().data() : nullptr,
                                  History ? (int)History->Ids().size() : 0, RepetitionPenalty, FrequencyPenalty, PresencePenalty,
                                  Temperature, m, c.Token.data(), c.Score.data(), &n));
     c.Token.resize((size_t)n); c.Score.resize((size_t)n);
@@ -226,7 +255,9 @@ class TNNetStreamingDecoder {
  private:
   cai_decoder_t d_ = nullptr;
   cai_decoder_config cfg_{};
-  std::vector<float> logits_;
+  std::vector<float> logits_, window_;
+  std::vector<int32_t> argmax_rows_;
+  int rows_ = 0;
   int32_t argmax_ = -1;
 };
 

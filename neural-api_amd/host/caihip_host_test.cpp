@@ -61,6 +61,14 @@ int main(int argc, char** argv)
       double worst = 0.0;
       for (size_t v = 0; v < rows[n - 1].size(); v++) worst = std::fmax(worst, std::fabs((double)rows[n - 1][v] - (double)dec.Output()[v]));
       EXPECT(worst < 1e-4 && dec.ArgMaxRow() == last_argmax && dec.SDPACacheLength() == n);
+      // a window of up to eight tokens keeps EVERY row (the verify pass of speculative decoding)
+      EXPECT(dec.WindowRows() == n);
+      for (int r = 0; r < n; r++) {
+        double w = 0.0;
+        for (size_t v = 0; v < rows[(size_t)r].size(); v++) w = std::fmax(w, std::fabs((double)rows[(size_t)r][v] - (double)dec.OutputRow(r)[v]));
+        EXPECT(w < 1e-4);
+      }
+      EXPECT((int)dec.HiddenState(n - 1).size() == dec.Config().d_model);
       // speculative rollback: drop 3 tokens, re-feed them, same logits
       dec.TruncateTo(5);
       EXPECT(dec.SDPACacheLength() == 5);
@@ -88,6 +96,10 @@ int main(int argc, char** argv)
       for (int k = 0; k < 6; k++) { dec.StepForward(&t, 1, 4 + k); t = dec.ArgMaxRow(); host_chain.push_back(t); }
       dec.TruncateTo(4);
       EXPECT(dec.GenerateGreedy(first, 4, 6) == host_chain);
+      // prompt-lookup generation writes the same tokens, in at most as many passes
+      dec.TruncateTo(4);
+      { int passes = 0; std::vector<int32_t> ctx(seq, seq + 4); ctx.push_back(first);
+        EXPECT(dec.GenerateLookup(ctx, 1, 4, 6, &passes) == host_chain && passes >= 1 && passes <= 6); }
       // sampled decode: the candidate prefix of the resident row is the sorted soft-max head, and the samplers draw from it
       {
         dec.Reset();

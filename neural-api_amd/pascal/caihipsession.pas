@@ -34,6 +34,7 @@ type
     FSnap: TCaiKVSnap;
     FLogits: TCaiSingleArray;
     FWindowLogits: TCaiSingleArray;
+    FLastRow: LongInt;           // the logits row of the last token fed: 0 after a step, Count - 1 after StepWindow
     procedure Check(rc: LongInt; const Where: string);
     function GetPosition: LongInt;
   public
@@ -61,7 +62,7 @@ type
     // returns MaxNew greedy tokens, Passes receives the number of window steps taken
     function GenerateLookup(const Context: TCaiLongIntArray; MatchLen, NumDraft, MaxNew: LongInt; out Passes: LongInt): TCaiLongIntArray;
     // the sampled branch without the logits read-back: the M most probable candidates after the penalties and the
-    // temperature, sorted (neural/neuralchatengine.pas:1495-1501); the random draw stays on the host
+    // temperature, sorted (neural/neuralchatengine.pas:1495-1501), over the row of the last token fed; the random draw stays on the host
     function Candidates(const HistIds, HistCounts: TCaiLongIntArray; Repetition, Frequency, Presence, Temperature: Single;
       M: LongInt; out Tokens: TCaiLongIntArray; out Probs: TCaiSingleArray): LongInt;
 
@@ -142,6 +143,7 @@ begin
   if WantLogits then Row := @FLogits[0] else Row := nil;
   Result := -1;
   Check(cai_decoder_step(FDec, @Token, @Pos, 1, Row, @Result), 'cai_decoder_step');
+  FLastRow := 0;
 end;
 
 function TCaiHipSession.Prefill(const Tokens: TCaiLongIntArray; First, Count: LongInt; WantLogits: Boolean): LongInt;
@@ -152,6 +154,7 @@ begin
   if Count <= 0 then exit;
   if WantLogits then Row := @FLogits[0] else Row := nil;
   Check(cai_decoder_prefill(FDec, 0, @Tokens[First], Count, GetPosition, Row, @Result), 'cai_decoder_prefill');
+  FLastRow := 0;
 end;
 
 function TCaiHipSession.GenerateGreedy(FirstToken, MaxNew: LongInt): TCaiLongIntArray;
@@ -159,6 +162,7 @@ begin
   SetLength(Result, MaxNew);
   if MaxNew <= 0 then exit;
   Check(cai_decoder_generate(FDec, FirstToken, GetPosition, MaxNew, @Result[0]), 'cai_decoder_generate');
+  FLastRow := 0;
 end;
 
 procedure TCaiHipSession.StepWindow(const Tokens: TCaiLongIntArray; First, Count: LongInt; WantLogits: Boolean;
@@ -175,6 +179,7 @@ begin
     Rows := @FWindowLogits[0];
   end;
   Check(cai_decoder_step_window(FDec, 0, @Tokens[First], Count, GetPosition, Rows, @ArgMax[0]), 'cai_decoder_step_window');
+  FLastRow := Count - 1;
 end;
 
 function TCaiHipSession.GenerateLookup(const Context: TCaiLongIntArray; MatchLen, NumDraft, MaxNew: LongInt;
@@ -197,7 +202,7 @@ begin
   Result := 0;
   if Length(HistIds) > 0 then begin PIds := @HistIds[0]; PCounts := @HistCounts[0]; end
   else begin PIds := nil; PCounts := nil; end;
-  Check(cai_decoder_candidates(FDec, 0, PIds, PCounts, Length(HistIds), Repetition, Frequency, Presence, Temperature, M,
+  Check(cai_decoder_candidates(FDec, FLastRow, PIds, PCounts, Length(HistIds), Repetition, Frequency, Presence, Temperature, M,
     @Tokens[0], @Probs[0], @Result), 'cai_decoder_candidates');
   SetLength(Tokens, Result);
   SetLength(Probs, Result);
