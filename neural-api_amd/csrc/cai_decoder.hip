@@ -691,7 +691,8 @@ extern "C" int cai_decoder_generate_lookup(cai_decoder_t d, const int32_t* conte
   const cai_decoder_config& c = d->cfg;
   if (d->kv.len_at(0, 0) != n_ctx - 1)
     return set_error(CAI_ERR_STATE, "cai_decoder_generate_lookup: the cache of sequence 0 holds %d tokens, the context's first %d are expected (its last token is fed here)", d->kv.len_at(0, 0), n_ctx - 1);
-  if (n_ctx - 1 + n_tokens > c.max_ctx) return set_error(CAI_ERR_STATE, "cai_decoder_generate_lookup: %d tokens from %d exceed max_ctx %d", n_tokens, n_ctx - 1, c.max_ctx);
+  if (d->kv.evict_cap == 0 ? n_ctx - 1 + n_tokens > c.max_ctx : n_tokens > c.max_ctx)   // (a session with eviction runs past max_ctx, like cai_decoder_generate)
+    return set_error(CAI_ERR_STATE, "cai_decoder_generate_lookup: %d tokens from %d exceed max_ctx %d", n_tokens, n_ctx - 1, c.max_ctx);
   if (match_len < 1) match_len = 1;                       // (the reference clamps both the same way)
   if (num_draft < 1) num_draft = 1;
   const bool can_draft = d->kv.evict_cap == 0;            // a rolling cache cannot take a window back
@@ -702,8 +703,8 @@ extern "C" int cai_decoder_generate_lookup(cai_decoder_t d, const int32_t* conte
     const int pos = (int)all.size() - 1;
     int32_t win[8], am[8];
     win[0] = all.back();
-    const int room = std::min(std::min(num_draft, 7), std::min(n_tokens - emitted - 1, c.max_ctx - pos - 1));
-    const int nd = can_draft && room > 0 ? lookup_draft(all.data(), (int)all.size(), match_len, room, win + 1) : 0;
+    const int room = can_draft ? std::min(std::min(num_draft, 7), std::min(n_tokens - emitted - 1, c.max_ctx - pos - 1)) : 0;
+    const int nd = room > 0 ? lookup_draft(all.data(), (int)all.size(), match_len, room, win + 1) : 0;
     const int rc = cai_decoder_step_window(d, 0, win, 1 + nd, pos, nullptr, am);
     if (rc) return rc;
     passes++;

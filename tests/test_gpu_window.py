@@ -137,6 +137,12 @@ def test_window_and_lookup_refusals():
         dec.step_window([1, 2], 1)
     out, passes = dec.generate_lookup([1, 1], 12, 1, 4)       # drafts are switched off: one token per pass
     assert passes == 12 and len(out) == 12
+    # and, like plain generation, the rolling session runs past max_ctx
+    dec.reset(); dec.step_window([1], 0)
+    plain = dec.generate(1, 1, 96).tolist()
+    dec.reset(); dec.step_window([1], 0)
+    out, passes = dec.generate_lookup([1, 1], 96, 1, 4)
+    assert out.tolist() == plain and passes == 96 and dec.len() == 97
 
 
 @pytest.mark.parametrize("name", ["qwen7b_like_q4k", "smollm_like_q8", "olmoe_like_q8"])
