@@ -414,8 +414,8 @@ def main():
     bpw = {"Q4_K": 144 / 256, "Q5_K": 176 / 256, "Q8_0": 34 / 32, "Q4_0": 18 / 32, "Q6_K": 210 / 256}
     qbytes = bpw[conf["qtype"]]
     k_bytes = 2 * I * d * qbytes + 4 * d * 2 + 4 * I     # blocks + x + gain + y
-    # ---- every kernel class of the step, timed in place: the production launches of one class over all blocks, back to
-    #      back between two HIP events on the library's stream (cai_decoder_profile); batch 1 only ----
+    # ---- every kernel class of the step, timed in its place in the chain: whole steps against steps without the class, both
+    #      replayed as captured graphs between two HIP events on the library's stream (cai_decoder_profile); batch 1 only ----
     table, k_avg_us = None, None
     if B == 1:
         for b in range(B):
@@ -494,8 +494,8 @@ def main():
     if table is not None:
         total = sum(r["us_per_step"] for r in table)
         res["kernels"] = {"rows": table, "sum_us_per_step": round(total, 1), "graph_step_us": round(ms.value * 1e3 / K, 1),
-                          "note": "each class timed in place (its production launches over all blocks, back to back, HIP events on the library stream); "
-                                  "the captured graph adds the token hand-over kernel between steps"}
+                          "note": "a class costs what the step gains without its launches: whole steps and steps without the class, each replayed as one "
+                                  "captured graph between two HIP events on the library stream (median of three replays); the generation graph adds the token hand-over kernel between steps"}
     if not args.no_cpu_baseline:
         # the reference's own CPU-runnable configuration is small enough to run whole on the host; the others are sampled
         res["cpu_baseline"] = cpu_baseline_end_to_end(cfg, prompt_len, 128) if args.config == "smollm2-135m-q8_0" else cpu_baseline(cfg)

@@ -257,8 +257,10 @@ int cai_decoder_hidden_state(cai_decoder_t d, int row, float* hidden_out);
  * neural/neuralchatengine.pas:1485-1561 with ArgMaxRow on the device). */
 int cai_decoder_generate(cai_decoder_t d, int32_t first_token, int pos, int n_tokens, int32_t* tokens_out);
 /* Measurement aid (no counterpart in the reference): average microseconds per step spent in each kernel class of the batch-1
- * decode step of sequence 0 at its current position.  Class k's production launches (all blocks) run `reps` times back to back
- * between two HIP events: 0 embedding, 1 q|k|v, 2 attention (rotary + append + cached decode), 3 o + residual,
+ * decode step of sequence 0 at its current position, taken as a difference: `reps` whole steps, and `reps` steps without class
+ * k's launches, each captured and replayed as one graph between two HIP events on the library stream; a class costs what the
+ * step gains without it (the kernel in its place in the chain, dependent-launch gap included; the classes add up to the step).
+ * Classes: 0 embedding, 1 q|k|v, 2 attention (rotary + append + cached decode), 3 o + residual,
  * 4 RMSNorm + gate|up + SwiGLU (expert half of a mixture model: router .. mixture, with 5), 5 down + residual, 6 final norm +
  * vocabulary projection, 7 arg-max.  The session is not advanced (the K,V row of the current position is rewritten). */
 int cai_decoder_profile(cai_decoder_t d, int32_t token, int reps, float* us_per_step_out, int n_classes);
