@@ -391,3 +391,25 @@ def test_prompt_attention_on_matrix_cores_equals_steps(kv, window):
     dec.prefill(toks[:50], 0, seq=1, want_logits=False)
     _, lg = dec.prefill(toks[50:], 50, seq=1)
     assert rel_err(lg, last[0]) < tol
+
+
+@pytest.mark.parametrize("name", ["qwen7b_like_q4k", "olmoe_like_q8"])
+def test_per_class_timing_leaves_the_session_as_it_found_it(name):
+    """cai_decoder_profile (a measurement aid without a counterpart in the reference) replays whole steps and steps without one
+    class of launches at the current position.  It must not advance the session, and the step that follows must give what it
+    gives without the timing pass in between; the classes it reports are finite and the large ones positive."""
+    from helpers.device import dev
+    cai = dev()
+    s = SHAPES[name]
+    spec = synthetic_spec(s["cfg"], s["qtype"], head_qtype=s["head"], qkv_bias=s["bias"], std=0.05)
+    dec = cai.Decoder(spec)
+    toks = [3, 17, 256, 9, 41, 5]
+    for p, t in enumerate(toks[:-1]):
+        dec.step(t, p, want_logits=False)
+    _, want = dec.step(toks[-1], 5)
+    dec.truncate(5)
+    us = dec.profile(toks[-1], reps=4)
+    assert dec.len() == 5
+    assert np.isfinite(us).all() and us[4] > 0 and us[1] > 0 and us.sum() > 0
+    _, got = dec.step(toks[-1], 5)
+    assert np.array_equal(got, want)
