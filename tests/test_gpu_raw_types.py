@@ -132,6 +132,14 @@ def test_q5_k_m_like_decoder_logits_greedy_tokens_batch_and_prompt():
         am, lg = dec.step(np.full(4, t), np.full(4, p))
         for b in range(4):
             assert rel_err(lg[b], singles[p]) < TOL
+    # and as a window of one sequence, followed by lookup generation over the greedy continuation
+    dec.reset(0)
+    am, lg = dec.step_window(prompt, 0)
+    for r in range(len(prompt)):
+        assert rel_err(lg[r], singles[r]) < TOL
+    dec.truncate(len(prompt) - 1)
+    got, passes = dec.generate_lookup(prompt, 65, 1, 5)
+    assert got.tolist() == [first] + seq_o[:64] and passes <= 65
     dec.close()
 
 
@@ -144,9 +152,16 @@ def test_decoder_of_each_other_type_against_the_oracle(qt):
     om = oracle_model(spec, acc64=1)
     dec = cai.Decoder(spec)
     seq = [3, 299, 17, 17, 250, 9, 1, 0, 44, 120]
+    rows = []
     for p, t in enumerate(seq):
         n_o, lo = om.step(t, p); am, ld = dec.step(t, p)
         assert rel_err(ld[0], lo) < TOL and int(am[0]) == n_o
+        rows.append(lo)
+    # the same tokens as one window of five after the first five (the verify pass of speculative decoding)
+    dec.truncate(5)
+    am, lg = dec.step_window(seq[5:], 5)
+    for r in range(5):
+        assert rel_err(lg[r], rows[5 + r]) < TOL and int(am[r]) == int(np.argmax(rows[5 + r]))
     dec.close()
 
 
