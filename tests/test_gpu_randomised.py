@@ -2,8 +2,9 @@
 type, sliding window, q/k norm, mixture of experts, tied head, random norm gains - stepped, windowed, prompt-ingested and batched
 against the oracle; (2) random sequences of session operations (step, window + partial commit, prompt pass, truncate, snapshot /
 restore, fork, reset, device-side generation, lookup generation, batched step over several sequences) with every logits row
-checked against an oracle replaying the same token history, and the session length after every operation.  The same two
-harnesses ran 3000 shapes and 4000 sequences of 60 operations once without a finding (four int8-cache shapes at 5.3e-3 to 6.3e-3
+checked against an oracle replaying the same token history, and the session length after every operation; (3) sessions with
+sink + recent-window eviction run past max_ctx.  The same
+harnesses ran 3000 shapes, 4000 sequences of 60 operations and 3000 eviction sessions once without a finding (four int8-cache shapes at 5.3e-3 to 6.3e-3
 against the 5e-3 bar of that cache type, whose codes may differ by one step between device and oracle)."""
 import numpy as np
 import pytest
@@ -189,6 +190,58 @@ def run_session(cai, rel_err, seed, n_ops=60):
 
 
 
+def run_eviction(cai, rel_err, seed):
+    rng = np.random.default_rng(seed)
+    qtype = int(rng.choice([O.Q4_K, O.Q8_0, O.Q4_0]))
+    hd = int(rng.choice([32, 64, 128])); hkv = int(rng.choice([1, 2])); hq = hkv * int(rng.choice([1, 2, 4]))
+    if (hq * hd) % 256: hq, hkv, hd = 4, 2, 64
+    sinks = int(rng.choice([0, 1, 4])); recent = int(rng.integers(6, 48))
+    T = int(rng.integers(sinks + recent + 5, 220))
+    mc = sinks + recent + int(rng.integers(0, 40))
+    cfg = dict(n_layers=2, d_model=int(rng.choice([256, 512])), n_q_heads=hq, n_kv_heads=hkv, head_dim=hd, ffn=256,
+               vocab=int(rng.integers(100, 900)), max_ctx=mc, eps=1e-5, rope_theta=1e4)
+    kv = int(rng.choice([0, 0, 1]))
+    spec = synthetic_spec(cfg, qtype, qkv_bias=bool(rng.random() < 0.5), std=0.05, seed=seed)
+    dec = cai.Decoder(spec, kv_dtype=kv)
+    dec.set_eviction(sinks, recent)
+    om = oracle_model(spec, acc64=1, kv_f16=kv, max_ctx=T + 16, evict_sinks=sinks, evict_recent=recent)
+    V = cfg["vocab"]; pos = 0; tol = 1e-3; log = []
+    while pos < T:
+        op = rng.choice(["step", "prefill", "generate", "window1", "snaprestore"])
+        log.append((op, pos))
+        if op == "step":
+            t = int(rng.integers(0, V)); _, lo = om.step(t, pos); _, ld = dec.step(t, pos); pos += 1
+            e = rel_err(ld[0], lo); assert e < tol, (op, pos, e, sinks, recent, mc, log[-5:])
+        elif op == "window1":
+            t = int(rng.integers(0, V)); _, lo = om.step(t, pos); _, ld = dec.step_window([t], pos); pos += 1
+            e = rel_err(ld[0], lo); assert e < tol, (op, pos, e, sinks, recent, mc, log[-5:])
+        elif op == "prefill":
+            n = int(min(rng.integers(1, 60), T - pos)); ts = rng.integers(0, V, n).tolist()
+            for i, t in enumerate(ts): _, lo = om.step(t, pos + i)
+            _, ld = dec.prefill(ts, pos); pos += n
+            e = rel_err(ld, lo); assert e < tol, (op, n, pos, e, sinks, recent, mc, log[-5:])
+        elif op == "generate" and pos >= 1:
+            n = int(min(rng.integers(1, 12), T - pos, mc))
+            if n < 1: continue
+            t = int(rng.integers(0, V)); out = dec.generate(t, pos, n).tolist()
+            cur = t
+            for i, g in enumerate(out):
+                am, lo = om.step(cur, pos + i)
+                if am != g:
+                    top2 = np.sort(lo)[-2:]
+                    assert top2[1] - top2[0] < 2 * tol * np.max(np.abs(lo)), (op, i, g, am, sinks, recent, mc, log[-5:])
+                cur = g
+            pos += n
+        elif op == "snaprestore":
+            s = dec.snapshot(); 
+            if pos < T - 3:
+                for i in range(3): dec.step(int(rng.integers(0, V)), pos + i, want_logits=False)
+            dec.restore(s); cai.load().cai_kv_snap_destroy(s)
+        assert dec.len() == pos, ("len", dec.len(), pos, log[-4:])
+        assert dec.cache_rows(0, 0) == min(pos, sinks + recent), ("rows", dec.cache_rows(0, 0), pos, sinks, recent)
+    dec.close()
+
+
 @pytest.mark.parametrize("seed0", [1000, 1010, 1020, 1030])
 def test_random_model_shapes_against_the_oracle(seed0):
     from helpers.device import dev, rel_err
@@ -207,5 +260,18 @@ def test_random_session_operation_sequences_against_the_oracle(seed0):
     for seed in range(seed0, seed0 + 10):
         try:
             run_session(cai, rel_err, seed)
+        except AssertionError as e:
+            raise AssertionError((seed,) + e.args)
+
+
+@pytest.mark.parametrize("seed0", [1, 16])
+def test_random_sessions_with_eviction_against_the_oracle(seed0):
+    """sink + recent-window sessions (neural/neuraldecode.pas:1257-1276) run past max_ctx through steps, prompt passes of any
+    length, device-side generation and snapshot / restore; every logits row against the oracle's evicting cache"""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    for seed in range(seed0, seed0 + 15):
+        try:
+            run_eviction(cai, rel_err, seed)
         except AssertionError as e:
             raise AssertionError((seed,) + e.args)
