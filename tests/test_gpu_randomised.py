@@ -3,8 +3,8 @@ type, sliding window, q/k norm, mixture of experts, tied head, random norm gains
 against the oracle; (2) random sequences of session operations (step, window + partial commit, prompt pass, truncate, snapshot /
 restore, fork, reset, device-side generation, lookup generation, batched step over several sequences) with every logits row
 checked against an oracle replaying the same token history, and the session length after every operation; (3) sessions with
-sink + recent-window eviction run past max_ctx.  The same
-harnesses ran 3000 shapes, 4000 sequences of 60 operations and 3000 eviction sessions once without a finding (four int8-cache shapes at 5.3e-3 to 6.3e-3
+sink + recent-window eviction run past max_ctx; (4) the stand-alone products on random shapes.  The same
+harnesses ran 3000 model shapes, 4000 sequences of 60 operations, 3000 eviction sessions and 4000 product shapes once without a finding (four int8-cache shapes at 5.3e-3 to 6.3e-3
 against the 5e-3 bar of that cache type, whose codes may differ by one step between device and oracle)."""
 import numpy as np
 import pytest
@@ -242,6 +242,55 @@ def run_eviction(cai, rel_err, seed):
     dec.close()
 
 
+TYPES = [O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_K, O.F32, O.Q2_K, O.Q3_K, O.Q4_1, O.Q5_0, O.Q5_1]
+
+def run_products(cai, rel_err, seed):
+    rng = np.random.default_rng(seed)
+    qt = int(rng.choice(TYPES))
+    k256 = qt in (O.Q4_K, O.Q6_K, O.Q5_K, O.Q2_K, O.Q3_K)
+    cols = int(rng.integers(1, 33)) * 256 if k256 else int(rng.integers(1, 200)) * 32
+    if rng.random() < 0.1: cols = int(rng.choice([18944, 27648 if k256 else 11008, 14336]))
+    rows = int(rng.choice([rng.integers(1, 40), rng.integers(40, 700), rng.integers(700, 6000)]))
+    if cols > 12000: rows = min(rows, 600)
+    w = (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32)
+    raw = O.quantize(qt, w)
+    bias = (rng.standard_normal(rows) * 0.1).astype(np.float32) if rng.random() < 0.4 else None
+    W = cai.QWeight(qt, rows, cols, raw, bias=bias)
+    what = ("type", qt, "rows", rows, "cols", cols, "bias", bias is not None)
+    # matrix-vector, batch 1..8
+    nb = int(rng.integers(1, 9)); act = int(rng.choice([0, 0, 1, 2, 3]))
+    x = rng.standard_normal((nb, cols)).astype(np.float32)
+    got = W.gemv(x, act=act); want = O.gemv(qt, raw, rows, cols, x, bias, act, 1)
+    e = rel_err(got, want); assert e < 1e-4, ("gemv", nb, act, e) + what
+    # prompt product
+    T = int(rng.choice([rng.integers(1, 9), rng.integers(9, 70), rng.integers(70, 300)]))
+    if rows * cols > 3e7: T = min(T, 40)
+    xt = rng.standard_normal((T, cols)).astype(np.float32)
+    want = O.gemv(qt, raw, rows, cols, xt, bias, 0, 1)
+    for mc in (False, True):
+        got = W.gemm(xt, matrix_cores=mc)
+        e = rel_err(got, want); assert e < 1e-4, ("gemm", T, mc, e) + what
+    # fused feed-forward front half on even row counts of block types the fused kernels take
+    if rows % 2 == 0 and bias is None and qt in (O.Q4_K, O.Q8_0, O.Q4_0, O.Q5_K):
+        half = rows // 2
+        gain = (1.0 + 0.2 * rng.standard_normal(cols)).astype(np.float32) if rng.random() < 0.7 else None
+        xb = rng.standard_normal((1, cols)).astype(np.float32)
+        try:
+            got = W.ffn_gateup(xb, gain, 1e-6)
+        except cai.CaiError as ex:
+            if "unsupported" in str(ex).lower() or "needs" in str(ex).lower(): got = None
+            else: raise
+        if got is not None:
+            xn = xb.astype(np.float64)
+            if gain is not None:
+                xn = gain.astype(np.float64) * (xn / np.sqrt(np.mean(xn * xn) + 1e-6))
+            y = O.gemv(qt, raw, rows, cols, xn.astype(np.float32), None, 0, 1).astype(np.float64)[0]
+            up, gate = y[:half], y[half:]
+            ref = up * (gate / (1.0 + np.exp(-gate)))
+            e = rel_err(got[0], ref.astype(np.float32)); assert e < 2e-4, ("gateup", gain is not None, e) + what
+    W.close()
+
+
 @pytest.mark.parametrize("seed0", [1000, 1010, 1020, 1030])
 def test_random_model_shapes_against_the_oracle(seed0):
     from helpers.device import dev, rel_err
@@ -273,5 +322,18 @@ def test_random_sessions_with_eviction_against_the_oracle(seed0):
     for seed in range(seed0, seed0 + 15):
         try:
             run_eviction(cai, rel_err, seed)
+        except AssertionError as e:
+            raise AssertionError((seed,) + e.args)
+
+
+@pytest.mark.parametrize("seed0", [1, 21])
+def test_random_product_shapes_against_the_oracle(seed0):
+    """cai_qgemv (batch 1..8, bias, activation), cai_qgemm (1..300 tokens, with and without the matrix-core flag) and
+    cai_ffn_gateup on random row counts and widths of all eleven weight types"""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    for seed in range(seed0, seed0 + 20):
+        try:
+            run_products(cai, rel_err, seed)
         except AssertionError as e:
             raise AssertionError((seed,) + e.args)
