@@ -1231,9 +1231,11 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   // the merge launch disappears (small models at short contexts are bound by launches, not by bytes)
   constexpr int single_bytes = 65536;
   if ((int64_t)max_ctx * head_dim * (dtype == CAI_KV_F16 ? 2 : dtype == CAI_KV_I8 ? 1 : 4) <= single_bytes) sl = (max_ctx + 31) / 32 * 32;
-  kv->split_len = sl; kv->n_splits = (max_ctx + sl - 1) / sl;   // the merge stage holds up to 128 splits
+  kv->split_len = sl; kv->n_splits = (max_ctx + sl - 1) / sl;
   const size_t bytes = (size_t)kv->seq_elems() * n_seq * kv->elem();
-  if (kv->n_splits > 128) return set_error(CAI_ERR_UNSUPPORTED, "kv cache: max_ctx %d needs %d splits (limit 128 x 256 rows)", max_ctx, kv->n_splits);
+  // (the kernels index slices generically; the bound keeps the per-row scratch of prompts and windows - one partial result per
+  // slice and query head - within reason: 131072 rows are 512 slices)
+  if (kv->n_splits > 512) return set_error(CAI_ERR_UNSUPPORTED, "kv cache: max_ctx %d needs %d slices of %d rows (limit 512: 131072 rows)", max_ctx, kv->n_splits, sl);
   CAI_HIP(hipMalloc(&kv->k, bytes));
   CAI_HIP(hipMalloc(&kv->v, bytes));
   CAI_HIP(hipMemsetAsync(kv->k, 0, bytes, ctx().stream));

@@ -341,3 +341,45 @@ def test_context_beyond_64_slices(hq, hkv):
             want[qh] = w @ vv[qh // G]
         assert np.max(np.abs(got.reshape(hq, dk) - want)) < 1e-5, step
     assert cache.len(0) == n + 2
+
+
+@pytest.mark.parametrize("kvt,hq,hkv,ctx,n", [("f16", 10, 2, 131072, 100003), ("f32", 4, 1, 65536, 65530), ("i8", 8, 8, 40000, 39000)])
+def test_very_long_caches_many_slices(kvt, hq, hkv, ctx, n):
+    """Caches beyond 32768 rows (up to 512 slices of 256 rows): the cache is filled from the host (cai_kv_import_layer), then
+    three tokens are decoded on top of it and compared with the oracle's kernel over the same rows.  One KV head with 256 slices
+    takes the per-head kernels and their in-kernel merge, the others the grouped kernel and the merge launch."""
+    from helpers.device import dev
+    cai = dev()
+    dk = 128
+    rng = np.random.default_rng(ctx)
+    dtype = {"f32": cai.KV_F32, "f16": cai.KV_F16, "i8": cai.KV_I8}[kvt]
+    kv = cai.KVCache(1, hkv, dk, ctx, dtype)
+    k = rng.standard_normal((hkv, n, dk)).astype(np.float32); v = rng.standard_normal((hkv, n, dk)).astype(np.float32)
+    rows = rng.standard_normal((3, (hq + 2 * hkv) * dk)).astype(np.float32)
+    if kvt == "i8":
+        kq = np.zeros((hkv, ctx, dk), np.int8); vq = np.zeros_like(kq); ks = np.zeros((hkv, ctx), np.float32); vs = np.zeros_like(ks)
+        for g in range(hkv):        # per-row codes and scales as the append kernel makes them (neural/neural.cl:2501-2580)
+            for src, q, s in ((k[g], kq[g], ks[g]), (v[g], vq[g], vs[g])):
+                m = np.max(np.abs(src), axis=1); sc = np.where(m > 0, m / 127.0, 1.0).astype(np.float32)
+                q[:n] = np.clip(np.rint(src / sc[:, None]), -127, 127).astype(np.int8); s[:n] = np.where(m > 0, sc, 0.0)
+        kv.import_layer(0, kq[:, :n], vq[:, :n], ks[:, :n], vs[:, :n])
+        for i in range(3):
+            out = np.zeros(hq * dk, np.float32)
+            O.lib().orc_attn_decode_i8(rows[i].ctypes.data, hq, hkv, dk, kq.ctypes.data, ks.ctypes.data, vq.ctypes.data, vs.ctypes.data,
+                                       ctx, n + i, 0, 0.0, out.ctypes.data)
+            got = kv.attn_decode(0, rows[i], hq)
+            assert np.max(np.abs(got - out)) < 2e-5 * max(1.0, np.max(np.abs(out))), i
+    else:
+        f16 = kvt == "f16"
+        if f16:
+            k = k.astype(np.float16).astype(np.float32); v = v.astype(np.float16).astype(np.float32)
+        kc = np.zeros((hkv, ctx, dk), np.float32); vc = np.zeros_like(kc); kc[:, :n] = k; vc[:, :n] = v
+        kv.import_layer(0, k.astype(np.float16) if f16 else k, v.astype(np.float16) if f16 else v)
+        for i in range(3):
+            out = np.zeros(hq * dk, np.float32)
+            O.lib().orc_attn_decode(rows[i].ctypes.data, hq, hkv, dk, kc.ctypes.data, vc.ctypes.data, ctx, n + i, 0, 0.0, 1 if f16 else 0, out.ctypes.data)
+            got = kv.attn_decode(0, rows[i], hq)
+            assert np.max(np.abs(got - out)) < 2e-5 * max(1.0, np.max(np.abs(out))), i
+    assert kv.len(0) == n + 3
+    with pytest.raises(cai.CaiError, match="limit 512"):
+        cai.KVCache(1, 1, 128, 131072 + 256, cai.KV_F16)

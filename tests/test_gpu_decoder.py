@@ -413,3 +413,25 @@ def test_per_class_timing_leaves_the_session_as_it_found_it(name):
     assert np.isfinite(us).all() and us[4] > 0 and us[1] > 0 and us.sum() > 0
     _, got = dec.step(toks[-1], 5)
     assert np.array_equal(got, want)
+
+
+def test_session_beyond_32768_rows_prompt_pass_and_decode_step_agree():
+    """A 66 000-token session (258 cache slices): the prompt pass ingests the history through the matrix-core attention kernel,
+    the decode step then walks the 66 000 cached rows with the split kernels; the same last token taken both ways must give the
+    same logits.  (The stand-alone attention test pins such caches to the oracle; this covers the session plumbing: chunked
+    ingestion, positions, captured step graph at that length.)"""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    cfg = dict(n_layers=1, d_model=256, n_q_heads=2, n_kv_heads=1, head_dim=128, ffn=256, vocab=300, max_ctx=66100, eps=1e-5, rope_theta=1e6)
+    spec = synthetic_spec(cfg, O.Q8_0, std=0.05)
+    dec = cai.Decoder(spec, max_batch=2, kv_dtype=cai.KV_F16)
+    rng = np.random.default_rng(66)
+    toks = rng.integers(0, cfg["vocab"], 66000).astype(np.int32)
+    dec.prefill(toks[:-1], 0, seq=0, want_logits=False)
+    am_a, la = dec.step_window([int(toks[-1])], 65999, seq=0)
+    am_b, lb = dec.prefill(toks, 0, seq=1)
+    assert dec.len(0) == 66000 and dec.len(1) == 66000
+    assert rel_err(la[0], lb) < 2e-4 and int(am_a[0]) == am_b
+    g = dec.generate(int(am_a[0]), 66000, 4)
+    assert dec.len(0) == 66004 and len(g) == 4
+    dec.close()
