@@ -1123,14 +1123,22 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   p.seq_elems = kv->seq_elems(); p.layer_off = (int64_t)layer * kv->layer_elems();
   p.q_heads = q_heads; p.kv_heads = kv->kv_heads; p.hd = kv->head_dim; p.max_ctx = kv->max_ctx;
   p.window = window; p.softcap = softcap; p.inv_sqrt = kv->score_mul / sqrtf((float)kv->head_dim);
-  p.theta = theta; p.pos = pos_dev; p.split_len = kv->split_len; p.n_splits = kv->n_splits;
+  p.theta = theta; p.pos = pos_dev;
+  if (kv->geo_rows > 0) {   // the caller chose a length bucket: it must cover the rows the host knows to be in use
+    int needed = 0;
+    for (int s0 = 0; s0 < (prompt_rows ? 1 : n_seq); s0++) needed = std::max(needed, kv->len_at(seq0 + s0, layer) + (prompt_rows ? n_seq : 1));
+    if (needed > kv->geo_rows) return set_error(CAI_ERR_STATE, "attention: launch geometry covers %d rows, %d are in use", kv->geo_rows, needed);
+  }
+  kv_geometry(kv, kv->geo_rows, &p.split_len, &p.n_splits);
   p.part = prompt_rows ? prompt_part : kv->part; p.out = out; p.out_stride = out_stride; p.seq0 = seq0;
   p.seq_mul = prompt_rows ? 0 : 1; p.appended = prompt_rows ? 1 : 0;
   p.evict_sinks = kv->evict_sinks; p.evict_cap = kv->evict_cap;
   p.ksc = kv->ks; p.vsc = kv->vs; p.seq_rows = kv->seq_rows(); p.layer_row_off = (int64_t)layer * kv->layer_rows();
   int rc;
   const int group_min = c.n_cu;   // smallest grid that fills the chip with one work-group per (slice, KV head)
-  const bool grouped = (kv->head_dim & 7) == 0 && n_seq * kv->kv_heads * kv->n_splits >= group_min;
+  // (a cache short enough to be ONE slice may be up to 2048 rows long: the grouped kernel's per-slice score arrays in LDS are
+  // sized for ordinary slices, the per-head kernel keeps its state in registers)
+  const bool grouped = (kv->head_dim & 7) == 0 && p.split_len <= 256 && n_seq * kv->kv_heads * p.n_splits >= group_min;
   // The per-head kernel merges its slices itself (one work-group per head does a head's merge).  A prompt has more rows in
   // flight than the counters cover, and in the per-KV-head kernel the last arriver would fold a whole group of heads over
   // many slices alone (32B shape, 33 slices x 5 heads: 37.7 us against 30.7 us with the merge launch): those keep the launch.
@@ -1216,6 +1224,28 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
 // ------------------------------------------------------------------------------------------
 // cache lifetime
 // ------------------------------------------------------------------------------------------
+int kv_bucket_rows(const cai_kv_s* kv, int needed_rows)
+{
+  if (kv->evict_cap > 0) return 0;                       // a rolling cache is short by construction: its own geometry
+  int rows = 1024;
+  while (rows < needed_rows && rows < kv->max_ctx) rows *= 2;
+  return rows >= kv->max_ctx ? 0 : rows;
+}
+
+void kv_geometry(const cai_kv_s* kv, int rows, int* split_len, int* n_splits)
+{
+  if (rows <= 0 || rows > kv->max_ctx) rows = kv->max_ctx;
+  // few, fat slices: every extra slice costs the merging work-group another device-coherent load round,
+  // while one CU sustains only ~20 GB/s, so a slice should stay under ~100 KB
+  constexpr int sl_max = 256;
+  int sl = (rows + 15) / 16; sl = (sl + 31) / 32 * 32; if (sl < 32) sl = 32; if (sl > sl_max) sl = sl_max;
+  // a head's whole K (or V) plane of at most 64 KB is one slice: a single work-group streams it in a few microseconds and
+  // the merge launch disappears (small models at short contexts are bound by launches, not by bytes)
+  constexpr int single_bytes = 65536;
+  if ((int64_t)rows * kv->head_dim * (kv->dtype == CAI_KV_F16 ? 2 : kv->dtype == CAI_KV_I8 ? 1 : 4) <= single_bytes) sl = (rows + 31) / 32 * 32;
+  *split_len = sl; *n_splits = (rows + sl - 1) / sl;
+}
+
 int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, int max_ctx, int dtype)
 {
   if (n_seq < 1 || n_layers < 1 || kv_heads < 1 || head_dim < 2 || (head_dim & 1) || (head_dim > 64 && (head_dim & 3)) || head_dim > 128 || max_ctx < 1)
@@ -1223,19 +1253,14 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
   if (dtype != CAI_KV_F32 && dtype != CAI_KV_F16 && dtype != CAI_KV_I8) return set_error(CAI_ERR_INVALID, "kv cache: dtype %d", dtype);
   kv->n_seq = n_seq; kv->n_layers = n_layers; kv->kv_heads = kv_heads; kv->head_dim = head_dim; kv->max_ctx = max_ctx; kv->dtype = dtype;
   kv->len.assign((size_t)n_seq * n_layers, 0);
-  // few, fat splits: every extra split costs the merging work-group another device-coherent load round,
-  // while one CU sustains only ~20 GB/s, so a slice should stay under ~100 KB
-  constexpr int sl_max = 256;
-  int sl = (max_ctx + 15) / 16; sl = (sl + 31) / 32 * 32; if (sl < 32) sl = 32; if (sl > sl_max) sl = sl_max;
-  // a head's whole K (or V) plane of at most 64 KB is one slice: a single work-group streams it in a few microseconds and
-  // the merge launch disappears (small models at short contexts are bound by launches, not by bytes)
-  constexpr int single_bytes = 65536;
-  if ((int64_t)max_ctx * head_dim * (dtype == CAI_KV_F16 ? 2 : dtype == CAI_KV_I8 ? 1 : 4) <= single_bytes) sl = (max_ctx + 31) / 32 * 32;
-  kv->split_len = sl; kv->n_splits = (max_ctx + sl - 1) / sl;
+  kv->geo_rows = 0;
+  kv_geometry(kv, 0, &kv->split_len, &kv->n_splits);
+  kv->n_splits_alloc = kv->n_splits;
+  for (int rows = 1024; rows < max_ctx; rows *= 2) { int sl, ns; kv_geometry(kv, rows, &sl, &ns); kv->n_splits_alloc = std::max(kv->n_splits_alloc, ns); }
   const size_t bytes = (size_t)kv->seq_elems() * n_seq * kv->elem();
   // (the kernels index slices generically; the bound keeps the per-row scratch of prompts and windows - one partial result per
   // slice and query head - within reason: 131072 rows are 512 slices)
-  if (kv->n_splits > 512) return set_error(CAI_ERR_UNSUPPORTED, "kv cache: max_ctx %d needs %d slices of %d rows (limit 512: 131072 rows)", max_ctx, kv->n_splits, sl);
+  if (kv->n_splits > 512) return set_error(CAI_ERR_UNSUPPORTED, "kv cache: max_ctx %d needs %d slices of %d rows (limit 512: 131072 rows)", max_ctx, kv->n_splits, kv->split_len);
   CAI_HIP(hipMalloc(&kv->k, bytes));
   CAI_HIP(hipMalloc(&kv->v, bytes));
   CAI_HIP(hipMemsetAsync(kv->k, 0, bytes, ctx().stream));
@@ -1248,7 +1273,7 @@ int kv_alloc(cai_kv_s* kv, int n_seq, int n_layers, int kv_heads, int head_dim, 
     CAI_HIP(hipMemsetAsync(kv->vs, 0, sb, ctx().stream));
   }
   kv->part_q_heads = kv_heads * 8;
-  CAI_HIP(hipMalloc(&kv->part, (size_t)n_seq * kv->part_q_heads * kv->n_splits * (head_dim + 2) * sizeof(float)));
+  CAI_HIP(hipMalloc(&kv->part, (size_t)n_seq * kv->part_q_heads * kv->n_splits_alloc * (head_dim + 2) * sizeof(float)));
   CAI_HIP(hipMalloc(&kv->d_len, sizeof(int32_t) * n_seq));
   CAI_HIP(hipMalloc((void**)&kv->merge_cnt, sizeof(unsigned) * n_seq * kv->part_q_heads));
   CAI_HIP(hipMemsetAsync(kv->merge_cnt, 0, sizeof(unsigned) * n_seq * kv->part_q_heads, ctx().stream));
@@ -1544,6 +1569,7 @@ extern "C" int cai_attn_decode(cai_kv_t kv, int layer, const float* qkv, int q_h
   if (!(flags & CAI_Y_DEVICE)) { rc = ensure_stage(&c.stage_out, &c.stage_out_cap, out_b); if (rc) return rc; d_out = (float*)c.stage_out; }
   c.h_small[0] = len;
   CAI_HIP(hipMemcpyAsync(kv->d_len, c.h_small, sizeof(int32_t), hipMemcpyHostToDevice, c.stream));
+  kv->geo_rows = kv_bucket_rows(kv, len + 1);
   rc = launch_attn_step(kv, layer, (float*)c.stage_in, 0, 1, q_heads, window, softcap, nullptr, kv->d_len, d_out, 0, 0, 0, nullptr);
   if (rc) return rc;
   if (!(flags & CAI_Y_DEVICE)) CAI_HIP(hipMemcpyAsync(out, d_out, out_b, hipMemcpyDeviceToHost, c.stream));

@@ -10,6 +10,7 @@
 #include "cai_internal.hpp"
 
 #include <algorithm>
+#include <map>
 
 struct cai_decoder_s {
   cai_decoder_config cfg{};
@@ -33,10 +34,11 @@ struct cai_decoder_s {
   int32_t *pm_expert = nullptr, *pm_perm = nullptr, *pm_tiles = nullptr;
   int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_argmax = nullptr, *d_gen = nullptr, *d_gen_idx = nullptr;
   int32_t* h_io = nullptr;   // pinned: tokens[8] pos[8] argmax[8] generated-so-far[8]
-  hipGraphExec_t graph[9] = {nullptr};
-  hipGraphExec_t wgraph[9] = {nullptr};               // width-n window steps of sequence 0 (rows = consecutive positions)
+  // captured launch sequences of sequence 0, keyed by kind (0 batched step, 1 window step of one sequence, 2 greedy steps with
+  // their hand-overs), width (rows or steps) and the cache-length bucket whose slice geometry the attention launches hold
+  std::map<int, hipGraphExec_t> graphs;
+  static int graph_key(int kind, int width, int bucket_rows) { return (kind << 28) | (width << 20) | (bucket_rows >> 8); }
   float* wpart = nullptr; size_t wpart_elems = 0;     // attention slice results of a window's rows (sized at the first window step)
-  hipGraphExec_t gen_graph[2] = {nullptr, nullptr};   // greedy generation: one step + hand-over, GEN_UNROLL steps + hand-overs
   bool use_graph = true;
   int ws_generation = -1;         // activation-workspace generation the captured batch graphs were built against
   std::vector<cai_qw_s*> owned;   // weights created by a loader on the decoder's behalf, destroyed with it
@@ -62,9 +64,8 @@ constexpr int GEN_UNROLL = 8;     // decode steps per launch of the long generat
 
 static void invalidate_graphs(cai_decoder_s* d)
 {
-  for (auto& g : d->graph) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
-  for (auto& g : d->wgraph) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
-  for (auto& g : d->gen_graph) if (g) { (void)hipGraphExecDestroy(g); g = nullptr; }
+  for (auto& kvp : d->graphs) if (kvp.second) (void)hipGraphExecDestroy(kvp.second);
+  d->graphs.clear();
 }
 
 static int check_ready(cai_decoder_s* d)
@@ -267,7 +268,7 @@ static int ensure_prefill_buffers(cai_decoder_s* d, int n)
   CAI_HIP(hipMalloc((void**)&d->patt, (size_t)cap * d->qw() * 4));
   CAI_HIP(hipMalloc((void**)&d->pgu, (size_t)cap * 2 * c.ffn * 4));
   CAI_HIP(hipMalloc((void**)&d->pmid, (size_t)cap * c.ffn * 4));
-  CAI_HIP(hipMalloc((void**)&d->ppart, (size_t)cap * c.n_q_heads * d->kv.n_splits * (c.head_dim + 2) * 4));
+  CAI_HIP(hipMalloc((void**)&d->ppart, (size_t)cap * c.n_q_heads * d->kv.n_splits_alloc * (c.head_dim + 2) * 4));
   CAI_HIP(hipMalloc((void**)&d->ptokpos, (size_t)cap * 2 * sizeof(int32_t)));
   if (c.n_experts > 0 && c.n_experts <= 512) {
     const size_t E = c.n_experts, S = (size_t)cap * c.top_k;
@@ -377,7 +378,8 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
   return CAI_OK;
 }
 
-static int run_step(cai_decoder_s* d, int n_b, bool window = false, int seq0 = 0)
+// `rows_needed`: cache rows the step's attention must cover (largest position + 1 over its rows)
+static int run_step(cai_decoder_s* d, int n_b, int rows_needed, bool window = false, int seq0 = 0)
 {
   Context& c = ctx();
   if (n_b >= 2) {   // the matrix-core path's activation workspace cannot grow inside a stream capture
@@ -391,9 +393,11 @@ static int run_step(cai_decoder_s* d, int n_b, bool window = false, int seq0 = 0
     const int rc = nb_reserve(kmax, part); if (rc) return rc;
     if (d->ws_generation != nb_ws_generation()) { invalidate_graphs(d); d->ws_generation = nb_ws_generation(); }
   }
+  const int bucket = kv_bucket_rows(&d->kv, rows_needed);
+  d->kv.geo_rows = bucket;
   // (a captured graph holds the sequence index: only sequence 0 has one)
   if (!d->use_graph || seq0 != 0) { const int rc = enqueue_step(d, n_b, seq0, ~0u, window); if (rc) return rc; CAI_HIP(hipGetLastError()); return CAI_OK; }
-  hipGraphExec_t& ge = window ? d->wgraph[n_b] : d->graph[n_b];
+  hipGraphExec_t& ge = d->graphs[cai_decoder_s::graph_key(window ? 1 : 0, n_b, bucket)];
   if (!ge) {
     hipGraph_t g = nullptr;
     CAI_HIP(hipStreamBeginCapture(c.stream, hipStreamCaptureModeThreadLocal));
@@ -411,9 +415,11 @@ static int run_step(cai_decoder_s* d, int n_b, bool window = false, int seq0 = 0
 
 // `steps` greedy batch-1 steps of sequence 0, each followed by the hand-over kernel, as ONE graph launch (steps = 1 or
 // GEN_UNROLL): a launch per token costs the stream a gap between graphs and a separate hand-over launch.
-static int run_gen_steps(cai_decoder_s* d, int steps)
+static int run_gen_steps(cai_decoder_s* d, int steps, int rows_needed)
 {
   Context& c = ctx();
+  const int bucket = kv_bucket_rows(&d->kv, rows_needed);
+  d->kv.geo_rows = bucket;
   auto body = [&]() {
     for (int u = 0; u < steps; u++) {
       const int rc = enqueue_step(d, 1, 0); if (rc) return rc;
@@ -422,7 +428,7 @@ static int run_gen_steps(cai_decoder_s* d, int steps)
     return (int)CAI_OK;
   };
   if (!d->use_graph) { const int rc = body(); if (rc) return rc; CAI_HIP(hipGetLastError()); return CAI_OK; }
-  hipGraphExec_t& ge = d->gen_graph[steps == 1 ? 0 : 1];
+  hipGraphExec_t& ge = d->graphs[cai_decoder_s::graph_key(2, steps, bucket)];
   if (!ge) {
     hipGraph_t g = nullptr;
     CAI_HIP(hipStreamBeginCapture(c.stream, hipStreamCaptureModeThreadLocal));
@@ -441,7 +447,7 @@ static int run_gen_steps(cai_decoder_s* d, int steps)
 // Scratch of a window step's attention: per (row, query head, cache slice) a partial result.
 static int ensure_wpart(cai_decoder_s* d)
 {
-  const size_t need = (size_t)8 * d->kv.part_q_heads * d->kv.n_splits * (d->cfg.head_dim + 2);
+  const size_t need = (size_t)8 * d->kv.part_q_heads * d->kv.n_splits_alloc * (d->cfg.head_dim + 2);
   if (d->wpart && d->wpart_elems >= need) return CAI_OK;
   CAI_HIP(hipStreamSynchronize(ctx().stream));
   if (d->wpart) { (void)hipFree(d->wpart); d->wpart = nullptr; }
@@ -628,7 +634,9 @@ extern "C" int cai_decoder_step(cai_decoder_t d, const int32_t* tokens, const in
   Context& cx = ctx();
   for (int b = 0; b < n_b; b++) { d->h_io[b] = tokens[b]; d->h_io[8 + b] = pos[b]; }
   CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
-  if ((rc = run_step(d, n_b))) return rc;
+  int rows_needed = 0;
+  for (int b = 0; b < n_b; b++) rows_needed = std::max(rows_needed, pos[b] + 1);
+  if ((rc = run_step(d, n_b, rows_needed))) return rc;
   if (logits) CAI_HIP(hipMemcpyAsync(logits, d->logits, (size_t)n_b * c.vocab * 4, hipMemcpyDeviceToHost, cx.stream));
   CAI_HIP(hipMemcpyAsync(d->h_io + 16, d->d_argmax, 8 * sizeof(int32_t), hipMemcpyDeviceToHost, cx.stream));
   CAI_HIP(hipStreamSynchronize(cx.stream));
@@ -661,7 +669,7 @@ extern "C" int cai_decoder_step_window(cai_decoder_t d, int seq, const int32_t* 
   CAI_HIP(hipStreamSynchronize(cx.stream));   // h_io is reused
   for (int i = 0; i < n; i++) { d->h_io[i] = tokens[i]; d->h_io[8 + i] = pos0 + i; }
   CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
-  if ((rc = run_step(d, n, n > 1, seq))) return rc;
+  if ((rc = run_step(d, n, pos0 + n, n > 1, seq))) return rc;
   if (logits) CAI_HIP(hipMemcpyAsync(logits, d->logits, (size_t)n * c.vocab * 4, hipMemcpyDeviceToHost, cx.stream));
   CAI_HIP(hipMemcpyAsync(d->h_io + 16, d->d_argmax, 8 * sizeof(int32_t), hipMemcpyDeviceToHost, cx.stream));
   CAI_HIP(hipStreamSynchronize(cx.stream));
@@ -734,7 +742,7 @@ extern "C" int cai_decoder_generate(cai_decoder_t d, int32_t first_token, int po
   CAI_HIP(hipMemcpyAsync(d->d_gen_idx, d->h_io + 24, sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
   for (int i = 0; i < n_tokens;) {
     const int steps = n_tokens - i >= GEN_UNROLL ? GEN_UNROLL : 1;
-    if ((rc = run_gen_steps(d, steps))) return rc;
+    if ((rc = run_gen_steps(d, steps, pos + i + steps))) return rc;
     i += steps;
   }
   CAI_HIP(hipMemcpyAsync(tokens_out, d->d_gen, (size_t)n_tokens * sizeof(int32_t), hipMemcpyDeviceToHost, cx.stream));
@@ -757,6 +765,7 @@ extern "C" int cai_decoder_profile(cai_decoder_t d, int32_t token, int reps, flo
   Context& cx = ctx();
   d->h_io[0] = token; d->h_io[8] = pos;
   CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
+  d->kv.geo_rows = kv_bucket_rows(&d->kv, pos + 1);
   if ((rc = enqueue_step(d, 1, 0))) return rc;      // a whole step first: every buffer a class reads holds this step's values
   // `reps` steps restricted to `classes`, as ONE captured graph replayed between two events (the way the decode step itself runs;
   // launches enqueued one by one are paced by the host thread, 17.6 to 20.1 us for the same 17.4 us kernel from machine to machine)
@@ -833,8 +842,7 @@ extern "C" int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* toke
       CAI_HIP(hipStreamSynchronize(cx.stream));   // h_io is reused
       d->h_io[0] = tokens[i]; d->h_io[8] = pos0 + i;
       CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
-      if (seq == 0) { if ((rc = run_step(d, 1))) return rc; }
-      else { if ((rc = enqueue_step(d, 1, seq))) return rc; }
+      if ((rc = run_step(d, 1, pos0 + i + 1, false, seq))) return rc;
     }
   } else {
     const int chunk = 512;
@@ -845,6 +853,7 @@ extern "C" int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* toke
       for (int i = 0; i < m; i++) { tp[i] = tokens[t0 + i]; tp[d->pf_cap + i] = pos0 + t0 + i; }
       CAI_HIP(hipMemcpyAsync(d->ptokpos, tp.data(), tp.size() * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
       CAI_HIP(hipStreamSynchronize(cx.stream));
+      d->kv.geo_rows = kv_bucket_rows(&d->kv, pos0 + t0 + m);
       if ((rc = enqueue_prefill_chunk(d, seq, m))) return rc;
       CAI_HIP(hipGetLastError());
       if (t0 + chunk >= n) {

@@ -132,7 +132,9 @@ struct cai_kv_s {
   std::vector<int> len;                   // [seq][layer] stream position = tokens appended so far (host mirror)
   int evict_sinks = 0, evict_cap = 0;     // cap > 0: sink + recent-window eviction, at most cap rows are cached
   int live(int n) const { return evict_cap > 0 && n > evict_cap ? evict_cap : n; }   // cached rows after n tokens
-  int split_len = 64, n_splits = 1;       // split-K geometry of the decode kernel (fixed at creation)
+  int split_len = 64, n_splits = 1;       // slice geometry of the decode kernels for a cache filled up to max_ctx
+  int n_splits_alloc = 1;                 // most slices any length bucket uses (sizes the per-slice scratch)
+  int geo_rows = 0;                       // rows the launches being enqueued must cover (0: max_ctx); see kv_geometry
   float* part = nullptr;                  // [seq][q_head][split][head_dim+2] split-K partials
   int part_q_heads = 0;
   int32_t* d_len = nullptr;               // [seq] device scratch: rows live BEFORE the token being decoded
@@ -209,6 +211,12 @@ int kv_set_eviction(cai_kv_s* kv, int sinks, int recent);
 int kv_snapshot(cai_kv_s* kv, int seq, cai_kv_snap_s** out);
 int kv_restore(cai_kv_s* kv, int seq, const cai_kv_snap_s* snap);
 int kv_fork(cai_kv_s* kv, int src, int dst);
+// Slice geometry by the rows in use, not by max_ctx: a session created for 32768 rows that holds 600 would otherwise cut them
+// into 3 slices of 256 (12 busy work-groups on the 7B shape; 463 against 597 tok/s).  Lengths fall into buckets of 1024 * 2^b rows
+// (a captured graph holds its launch geometry, so the decoder keeps one graph per bucket); kv_bucket_rows gives the bucket's
+// upper bound for a needed row count (max_ctx for the last one), kv_geometry the slice length and count for it.
+int kv_bucket_rows(const cai_kv_s* kv, int needed_rows);
+void kv_geometry(const cai_kv_s* kv, int rows, int* split_len, int* n_splits);
 // multi-token linear layer (matrix cores for Q4_K, small-batch kernel otherwise); gain != null fuses RMSNorm
 int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok,
                    float* y, int64_t y_stride, const float* residual);

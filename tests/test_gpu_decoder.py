@@ -435,3 +435,52 @@ def test_session_beyond_32768_rows_prompt_pass_and_decode_step_agree():
     g = dec.generate(int(am_a[0]), 66000, 4)
     assert dec.len(0) == 66004 and len(g) == 4
     dec.close()
+
+
+@pytest.mark.parametrize("kv", [0, 1])
+def test_attention_geometry_follows_the_session_length_across_bucket_boundaries(kv):
+    """The slice geometry of the decode attention follows the rows in use (buckets of 1024 * 2^b rows, one captured graph per
+    bucket), not max_ctx.  A session created for 5000 rows is walked across the 1024- and 2048-row boundaries by single steps,
+    by the eight-step generation graph, by windows and by a batch whose sequences sit in different buckets; every logits row
+    against the oracle."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    cfg = dict(n_layers=2, d_model=256, n_q_heads=4, n_kv_heads=2, head_dim=64, ffn=256, vocab=400, max_ctx=5000, eps=1e-5, rope_theta=1e4)
+    spec = synthetic_spec(cfg, O.Q8_0, std=0.05)
+    om = oracle_model(spec, acc64=1, kv_f16=kv)
+    dec = cai.Decoder(spec, max_batch=2, kv_dtype=kv)
+    rng = np.random.default_rng(12)
+    toks = rng.integers(0, cfg["vocab"], 2100).tolist()
+    ref = [om.step(t, p) for p, t in enumerate(toks)]
+    # 1010 tokens by a prompt pass, then single steps over the first boundary
+    dec.prefill(toks[:1010], 0, want_logits=False)
+    for p in range(1010, 1030):
+        _, lg = dec.step(toks[p], p)
+        assert rel_err(lg[0], ref[p][1]) < 1e-3, p
+    # back to 1018 and on with the generation graph (eight steps per launch straddle row 1024)
+    dec.truncate(1018)
+    g = dec.generate(toks[1018], 1018, 20).tolist()
+    cur, p = toks[1018], 1018
+    om.truncate(1018)
+    for t in g:
+        am, lg = om.step(cur, p)
+        if am != t:
+            top2 = np.sort(lg)[-2:]; assert top2[1] - top2[0] < 2e-3 * np.max(np.abs(lg)), p
+        cur, p = t, p + 1
+    # windows over the boundary, on fresh history
+    dec.truncate(1010); om.truncate(1010)
+    for p in range(1010, 1018): om.step(toks[p], p)
+    dec.step_window(toks[1010:1018], 1010, want_logits=False)
+    am, lg = dec.step_window(toks[1018:1026], 1018)
+    for r in range(8):
+        assert rel_err(lg[r], ref[1018 + r][1]) < 1e-3, r
+    # second boundary by a prompt pass that ends behind it, then steps
+    dec.prefill(toks[1026:2060], 1026, want_logits=False)
+    for p in range(2060, 2070):
+        _, lg = dec.step(toks[p], p)
+        assert rel_err(lg[0], ref[p][1]) < 1e-3, p
+    # a batch whose sequences are in different buckets: the longer one decides the geometry
+    dec.prefill(toks[:300], 0, seq=1, want_logits=False)
+    _, lg = dec.step([toks[2070], toks[300]], [2070, 300])
+    assert rel_err(lg[0], ref[2070][1]) < 1e-3 and rel_err(lg[1], ref[300][1]) < 1e-3
+    dec.close()
