@@ -729,14 +729,14 @@ static float round_half(float v) { return orc_f16_to_f32(orc_f32_to_f16(v)); }
 /* Live rows after `len` tokens: all of [j0, len) under a sliding window; under sink + recent-window eviction
  * (neuraldecode.pas:1257-1276: the first `sinks` positions and the latest `recent` are kept, the middle is gone, keys
  * keep their own rotation) positions [0, sinks) and [len - recent, len) once len exceeds sinks + recent.  The oracle
- * keeps every row and masks by position, so it states the policy, not a storage scheme.
+ * keeps every row and walks the live positions in order, so it states the policy, not a storage scheme.
  * Pinned by: within the cap identical to the unbounded run, row count pinned at the cap past it
  * (tests/TestNeuralDecode.pas:3863-3990), brute-force softmax over the stated set. */
-static int row_live(int j, int len, int window, int sinks, int recent)
+static void live_runs(int len, int window, int sinks, int recent, int run0[2], int run1[2])
 {
-  if (sinks + recent > 0 && len > sinks + recent) return j < sinks || j >= len - recent;
-  const int j0 = (window > 0 && len > window) ? len - window : 0;
-  return j >= j0;
+  /* at most two runs of consecutive positions, in ascending order */
+  if (sinks + recent > 0 && len > sinks + recent) { run0[0] = 0; run1[0] = sinks; run0[1] = len - recent; run1[1] = len; }
+  else { run0[0] = (window > 0 && len > window) ? len - window : 0; run1[0] = len; run0[1] = 0; run1[1] = 0; }
 }
 
 /* neural.cl:2354-2379 (append) + 2406-2499 (decode): scores q.K_j/sqrt(dk) (+softcap), max,
@@ -756,26 +756,30 @@ static void attn_core_f32(const float* qkv, int hq, int hkv, int dk, float* kc, 
   const int len = cache_len + 1;
   const float inv_sqrt = 1.0f / sqrtf((float)dk);
   float* sc = (float*)malloc((size_t)len * sizeof(float));
+  /* the live rows are walked run by run, so a stream far past the cap costs what its live rows cost */
+  int run0[2], run1[2];
+  live_runs(len, window, sinks, recent, run0, run1);
   for (int h = 0; h < hq; h++) {
     const int g = h / group;
     const float* q = qkv + h * dk;
     float m = -1e30f;
-    for (int j = 0; j < len; j++) {
-      if (!row_live(j, len, window, sinks, recent)) continue;
-      const float* kr = kc + ((int64_t)g * max_ctx + j) * dk;
-      float acc = 0;
-      for (int d = 0; d < dk; d++) acc = fmaf(q[d], kr[d], acc);
-      float s = acc * inv_sqrt;
-      if (softcap > 0) s = softcap * tanhf(s / softcap);
-      sc[j] = s; if (s > m) m = s;
-    }
+    for (int r = 0; r < 2; r++)
+      for (int j = run0[r]; j < run1[r]; j++) {
+        const float* kr = kc + ((int64_t)g * max_ctx + j) * dk;
+        float acc = 0;
+        for (int d = 0; d < dk; d++) acc = fmaf(q[d], kr[d], acc);
+        float s = acc * inv_sqrt;
+        if (softcap > 0) s = softcap * tanhf(s / softcap);
+        sc[j] = s; if (s > m) m = s;
+      }
     float sum = 0;
-    for (int j = 0; j < len; j++) if (row_live(j, len, window, sinks, recent)) { sc[j] = expf(sc[j] - m); sum += sc[j]; }
+    for (int r = 0; r < 2; r++)
+      for (int j = run0[r]; j < run1[r]; j++) { sc[j] = expf(sc[j] - m); sum += sc[j]; }
     const float inv = sum > 0 ? 1.0f / sum : 0;
     for (int d = 0; d < dk; d++) {
       float acc = 0;
-      for (int j = 0; j < len; j++)
-        if (row_live(j, len, window, sinks, recent)) acc = fmaf(sc[j], vc[((int64_t)g * max_ctx + j) * dk + d], acc);
+      for (int r = 0; r < 2; r++)
+        for (int j = run0[r]; j < run1[r]; j++) acc = fmaf(sc[j], vc[((int64_t)g * max_ctx + j) * dk + d], acc);
       out[h * dk + d] = acc * inv;
     }
   }

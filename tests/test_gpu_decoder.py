@@ -484,3 +484,34 @@ def test_attention_geometry_follows_the_session_length_across_bucket_boundaries(
     _, lg = dec.step([toks[2070], toks[300]], [2070, 300])
     assert rel_err(lg[0], ref[2070][1]) < 1e-3 and rel_err(lg[1], ref[300][1]) < 1e-3
     dec.close()
+
+
+def test_rotary_positions_far_beyond_32768_in_a_rolling_session():
+    """Positions up to 70 000 through the kernels that rotate q and k inside attention (a session with eviction keeps only sinks +
+    recent rows, so the stream runs far past max_ctx): the device generates 70 000 greedy tokens, the oracle is fed the same tokens
+    and the logits of steps at positions 40 000, 69 990.. are compared (angle = fp32 position x frequency as in
+    neural/neural.cl:1517-1542; an inaccurate sine / cosine at large arguments would show here)."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    cfg = dict(n_layers=1, d_model=256, n_q_heads=2, n_kv_heads=1, head_dim=128, ffn=256, vocab=300, max_ctx=64, eps=1e-5, rope_theta=1e4)
+    spec = synthetic_spec(cfg, O.Q8_0, std=0.05)
+    dec = cai.Decoder(spec)
+    dec.set_eviction(2, 30)
+    om = oracle_model(spec, acc64=1, max_ctx=70100, evict_sinks=2, evict_recent=30)
+    toks = [7]
+    pos = 0
+    for target in (40000, 69990):
+        out = []
+        while pos + len(out) < target:                    # cai_decoder_generate takes at most max_ctx tokens per call
+            n = min(64, target - pos - len(out))
+            out += dec.generate(toks[-1] if not out else out[-1], pos + len(out), n).tolist()
+        # the oracle takes the device's tokens as inputs (greedy ties would otherwise fork the two histories)
+        for i, t in enumerate([toks[-1]] + out[:-1]):
+            om.step(t, pos + i, want_logits=False)
+        pos += len(out); toks.append(out[-1])
+        for i in range(5):
+            t = int(toks[-1])
+            _, lo = om.step(t, pos); am, ld = dec.step(t, pos)
+            assert rel_err(ld[0], lo) < 1e-3, (pos, rel_err(ld[0], lo))
+            pos += 1; toks.append(int(am[0]))
+    dec.close()

@@ -23,7 +23,7 @@ def test_rmsnorm():
         assert np.max(np.abs(y - want)) < 2e-6 * np.max(np.abs(want))
 
 
-@pytest.mark.parametrize("pos", [0, 1, 17, 511, 8319])
+@pytest.mark.parametrize("pos", [0, 1, 17, 511, 8319, 32767, 65535, 131071])   # (angles up to 131071 rad: the fp32 product of the reference, accurate sine / cosine)
 @pytest.mark.parametrize("base,hd", [(10000.0, 64), (1e6, 128), (10000.0, 4)])
 def test_rope_interleaved(pos, base, hd):
     from helpers.device import dev
