@@ -28,6 +28,7 @@ struct cai_decoder_s {
   // prompt ingestion (multi-token) buffers, allocated at the first prefill: rows of up to pf_cap tokens
   int pf_cap = 0;
   float *px = nullptr, *pqkv = nullptr, *patt = nullptr, *pgu = nullptr, *pmid = nullptr, *ppart = nullptr;
+  size_t ppart_elems = 0;                            // (per row, query head and cache slice: sized for the length bucket in use)
   int32_t* ptokpos = nullptr;                        // [2][pf_cap]: tokens, positions
   // mixture-of-experts prompt: per chunk the router outputs, the slots grouped by expert and the per-slot activations
   float *pm_logits = nullptr, *pm_probs = nullptr, *pm_gate = nullptr, *pm_gu = nullptr, *pm_part = nullptr;
@@ -260,7 +261,7 @@ static int ensure_prefill_buffers(cai_decoder_s* d, int n)
   CAI_HIP(hipStreamSynchronize(ctx().stream));
   { float* pf[] = {d->px, d->pqkv, d->patt, d->pgu, d->pmid, d->ppart}; for (float* q : pf) if (q) (void)hipFree(q); }
   if (d->ptokpos) (void)hipFree(d->ptokpos);
-  d->px = d->pqkv = d->patt = d->pgu = d->pmid = d->ppart = nullptr; d->ptokpos = nullptr; d->pf_cap = 0;
+  d->px = d->pqkv = d->patt = d->pgu = d->pmid = d->ppart = nullptr; d->ptokpos = nullptr; d->pf_cap = 0; d->ppart_elems = 0;
   free_moe_prompt(d);
   const size_t qkvw = d->qw() + 2 * d->kw();
   CAI_HIP(hipMalloc((void**)&d->px, (size_t)cap * c.d_model * 4));
@@ -268,7 +269,6 @@ static int ensure_prefill_buffers(cai_decoder_s* d, int n)
   CAI_HIP(hipMalloc((void**)&d->patt, (size_t)cap * d->qw() * 4));
   CAI_HIP(hipMalloc((void**)&d->pgu, (size_t)cap * 2 * c.ffn * 4));
   CAI_HIP(hipMalloc((void**)&d->pmid, (size_t)cap * c.ffn * 4));
-  CAI_HIP(hipMalloc((void**)&d->ppart, (size_t)cap * c.n_q_heads * d->kv.n_splits_alloc * (c.head_dim + 2) * 4));
   CAI_HIP(hipMalloc((void**)&d->ptokpos, (size_t)cap * 2 * sizeof(int32_t)));
   if (c.n_experts > 0 && c.n_experts <= 512) {
     const size_t E = c.n_experts, S = (size_t)cap * c.top_k;
@@ -281,6 +281,23 @@ static int ensure_prefill_buffers(cai_decoder_s* d, int n)
   // the activation planes of the prompt products, sized once for the widest row (a mixture-of-experts chunk prepares one row per slot)
   const int plane_rows = c.n_experts > 0 ? cap * std::max(c.top_k, 1) : cap;
   return prefill_reserve_rows(plane_rows, std::max(std::max(c.d_model, d->qw()), c.ffn));
+}
+
+// Partial results of the prompt rows' attention when it runs on the decode kernels (rows x query heads x cache slices): sized
+// for the slice count of the length bucket in use, so a session created for 131072 rows does not hold 512 slices' worth for a
+// prompt at its start.  Grown on demand; prompt passes are not captured, so the pointer may change between them.
+static int ensure_ppart(cai_decoder_s* d, int rows_needed)
+{
+  int sl, ns;
+  kv_geometry(&d->kv, kv_bucket_rows(&d->kv, rows_needed), &sl, &ns);
+  const size_t need = (size_t)d->pf_cap * d->cfg.n_q_heads * ns * (d->cfg.head_dim + 2);
+  if (d->ppart && d->ppart_elems >= need) return CAI_OK;
+  CAI_HIP(hipStreamSynchronize(ctx().stream));
+  if (d->ppart) { (void)hipFree(d->ppart); d->ppart = nullptr; }
+  d->ppart_elems = 0;
+  CAI_HIP(hipMalloc((void**)&d->ppart, need * sizeof(float)));
+  d->ppart_elems = need;
+  return CAI_OK;
 }
 
 static int linear_rows(const cai_qw_s* w, bool prepped, const float* x, int64_t x_stride, const float* gain, float eps, int n,
@@ -854,6 +871,7 @@ extern "C" int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* toke
       CAI_HIP(hipMemcpyAsync(d->ptokpos, tp.data(), tp.size() * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
       CAI_HIP(hipStreamSynchronize(cx.stream));
       d->kv.geo_rows = kv_bucket_rows(&d->kv, pos0 + t0 + m);
+      if ((rc = ensure_ppart(d, pos0 + t0 + m))) return rc;
       if ((rc = enqueue_prefill_chunk(d, seq, m))) return rc;
       CAI_HIP(hipGetLastError());
       if (t0 + chunk >= n) {
