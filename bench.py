@@ -271,6 +271,7 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=8, help="repetitions of each kernel class in the per-kernel table")
     ap.add_argument("--kv", choices=["f32", "f16", "i8"], default=None, help="KV cache element type (default: the configuration's own)")
     ap.add_argument("--batch", type=int, default=1, help="independent sequences decoded together (1..8)")
+    ap.add_argument("--prompt", type=int, default=0, help="prompt length in tokens (default: the configuration's own)")
     ap.add_argument("--max-ctx", type=int, default=0, help="cache rows per sequence (default: the configuration's own; the cache geometry - slice count, attention grid - follows it)")
     ap.add_argument("--gemv-sweep", action="store_true", help="isolated matrix-vector sweep (BASELINE configs[1]): Q8_0 / Q4_0 / Q4_K / Q6_K and per-row int8 on five shapes, the stored-stream types on the two large ones, batch 1 and 4")
     ap.add_argument("--gemm-sweep", action="store_true", help="isolated prompt-product sweep: Q8_0 / Q4_0 / Q4_K / Q5_K / Q6_K, four shapes, 64..2048 tokens (cai_qgemm, device pointers)")
@@ -304,7 +305,7 @@ def main():
         return
     conf = CONFIGS[args.config]
     cfg = dict(conf["cfg"])
-    prompt_len = conf["prompt"]
+    prompt_len = args.prompt if args.prompt > 0 else conf["prompt"]
     K, W = args.steps, args.warmup
     if args.max_ctx > 0:
         cfg["max_ctx"] = args.max_ctx
