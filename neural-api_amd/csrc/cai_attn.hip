@@ -1239,6 +1239,12 @@ void kv_geometry(const cai_kv_s* kv, int rows, int* split_len, int* n_splits)
   // while one CU sustains only ~20 GB/s, so a slice should stay under ~100 KB
   constexpr int sl_max = 256;
   int sl = (rows + 15) / 16; sl = (sl + 31) / 32 * 32; if (sl < 32) sl = 32; if (sl > sl_max) sl = sl_max;
+  // From 8192 rows on the grouped kernel (K and V fetched once for all query heads of a KV head) is the fast one, but it needs
+  // about one work-group per CU: with few KV heads the slices are halved until slices x KV heads fill the chip.  7B shape, 4 KV
+  // heads, 7000 rows: 256-row slices take the per-head kernel at 31.8 us per launch, 128-row slices the grouped one at 23.3
+  // (445 -> 494 tok/s); at 4096 rows both forms take the same time and the longer slices stay.
+  if (rows >= 8192 && (kv->head_dim & 7) == 0)
+    while (sl > 64 && kv->kv_heads * ((rows + sl - 1) / sl) < ctx().n_cu) sl /= 2;
   // a head's whole K (or V) plane of at most 64 KB is one slice: a single work-group streams it in a few microseconds and
   // the merge launch disappears (small models at short contexts are bound by launches, not by bytes)
   constexpr int single_bytes = 65536;

@@ -343,9 +343,10 @@ def test_context_beyond_64_slices(hq, hkv):
     assert cache.len(0) == n + 2
 
 
-@pytest.mark.parametrize("kvt,hq,hkv,ctx,n", [("f16", 10, 2, 131072, 100003), ("f32", 4, 1, 65536, 65530), ("i8", 8, 8, 40000, 39000)])
+@pytest.mark.parametrize("kvt,hq,hkv,ctx,n", [("f16", 10, 2, 131072, 100003), ("f32", 4, 1, 65536, 65530), ("i8", 8, 8, 40000, 39000),
+                                             ("f16", 4, 1, 12000, 11990), ("f32", 6, 2, 9000, 8990)])   # (few KV heads from 8192 rows: slices halved for the grouped kernel)
 def test_very_long_caches_many_slices(kvt, hq, hkv, ctx, n):
-    """Caches beyond 32768 rows (up to 512 slices of 256 rows): the cache is filled from the host (cai_kv_import_layer), then
+    """Long caches (up to 512 slices of 256 rows; 64- and 128-row slices where few KV heads would leave the grouped kernel short of work-groups): the cache is filled from the host (cai_kv_import_layer), then
     three tokens are decoded on top of it and compared with the oracle's kernel over the same rows.  One KV head with 256 slices
     takes the per-head kernels and their in-kernel merge, the others the grouped kernel and the merge launch."""
     from helpers.device import dev
