@@ -768,7 +768,7 @@ extern "C" int cai_decoder_generate(cai_decoder_t d, int32_t first_token, int po
   return CAI_OK;
 }
 
-// Per-class timing of the batch-1 step: the production launches of one class (all blocks), back to back, between two HIP events.
+// Per-class timing of the batch-1 step: what the captured step gains when one class of launches is left out (see below).
 extern "C" int cai_decoder_profile(cai_decoder_t d, int32_t token, int reps, float* us_per_step_out, int n_classes)
 {
   CAI_ENTER();
