@@ -247,6 +247,47 @@ def gemm_sweep(cai, synth, torch):
 # KiB, factors from a 1 GiB copy kernel): profiles/gemv_q4k_gateup_qwen7b_hbm_traffic.txt.  Not measurable from
 # inside this process; re-collect when the kernel changes.
 GATEUP_TRAFFIC_BYTES = int((37513.6 * 2.000 + 74.7 * 1.000) * 1024)
+def step_timeline(dec, tok, np):
+    """Where one decode step spends its time, from stamps taken inside the kernels (100 MHz wall clock, 10 ns resolution).
+    Per launch: gap = first work-group entry minus the last exit of the launch before it (what the hardware needs between two
+    dependent kernels: end-of-kernel cache write-back, packet processing, dispatch), skew = last entry minus first entry, then
+    medians over work-groups of the in-kernel phases (issue: entry to first requests out; arrive: until the activation values
+    are there; quant: until the block-float form is in LDS; lift: until it is in registers; loop; tail: loop end to exit) and
+    the slowest work-group's loop and tail; span = last exit minus first entry."""
+    names = ["embedding", "q|k|v", "attention", "o", "gate|up", "down", "head", "arg-max"]
+    recs = dec.timeline(tok)
+    rows, prev_end = [], None
+    nm = lambda a: float(np.nanmedian(a)) if np.isfinite(a).any() else float("nan")
+    for cls, st in recs:
+        live = ~np.isnan(st[:, 7])
+        if not live.any():
+            prev_end = None; continue
+        s = st[live]
+        first, last_in, end = s[:, 0].min(), s[:, 0].max(), s[:, 7].max()
+        r = {"cls": cls, "wgs": int(live.sum()), "gap": float("nan") if prev_end is None else first - prev_end, "skew": last_in - first,
+             "stage": nm(s[:, 4] - s[:, 0]), "loop": nm(s[:, 5] - s[:, 4]), "tail": nm(s[:, 7] - s[:, 5]),
+             "loop_max": float((s[:, 5] - s[:, 4]).max()), "tail_max": float((s[:, 7] - s[:, 5]).max()), "span": end - first, "start": first}
+        if cls == 2:   # attention: 1 position known, 6 arrival counted
+            r.update(issue=nm(s[:, 1] - s[:, 0]), arrive=nm(s[:, 4] - s[:, 1]), quant=float("nan"), lift=float("nan"),
+                     count=nm(s[:, 6] - s[:, 5]), merge=float(np.nanmax(s[:, 7] - s[:, 6])))
+        else:
+            r.update(issue=nm(s[:, 1] - s[:, 0]), arrive=nm(s[:, 2] - s[:, 1]), quant=nm(s[:, 3] - s[:, 2]), lift=nm(s[:, 4] - s[:, 3]),
+                     count=float("nan"), merge=float("nan"))
+        rows.append(r); prev_end = end
+    print("one captured decode step, %d instrumented launches, %.1f us from the first entry to the last exit" % (len(rows), rows[-1]["start"] + rows[-1]["span"] - rows[0]["start"]))
+    cols = ("gap", "skew", "issue", "arrive", "quant", "lift", "stage", "loop", "tail", "loop_max", "tail_max", "count", "merge", "span")
+    print("%-10s %3s %5s |" % ("class", "n", "wgs") + "".join(" %8s" % c for c in cols))
+    out = {}
+    for k in range(8):
+        sel = [r for r in rows[2:] if r["cls"] == k and np.isfinite(r["gap"])] or [r for r in rows if r["cls"] == k and np.isfinite(r["gap"])]
+        if not sel:
+            continue
+        m = {f: float(np.mean([r[f] for r in sel])) for f in cols}
+        out[names[k]] = dict({f: round(v, 2) for f, v in m.items() if np.isfinite(v)}, n=len(sel), wgs=sel[0]["wgs"])
+        print("%-10s %3d %5d |" % (names[k], len(sel), sel[0]["wgs"]) + "".join(" %8.2f" % m[c] for c in cols))
+    print(json.dumps({"step_timeline_us": out}))
+
+
 def gateup_kernel_name(qtype, cols):
     """Name of the batch-1 fused gate|up kernel the library launches for this weight type and width (rows of 17..24
     super-blocks are packed four to a wave: the fifth template argument, else 1)."""
@@ -275,6 +316,7 @@ def main():
     ap.add_argument("--max-ctx", type=int, default=0, help="cache rows per sequence (default: the configuration's own; the cache geometry - slice count, attention grid - follows it)")
     ap.add_argument("--gemv-sweep", action="store_true", help="isolated matrix-vector sweep (BASELINE configs[1]): Q8_0 / Q4_0 / Q4_K / Q6_K and per-row int8 on five shapes, the stored-stream types on the two large ones, batch 1 and 4")
     ap.add_argument("--gemm-sweep", action="store_true", help="isolated prompt-product sweep: Q8_0 / Q4_0 / Q4_K / Q5_K / Q6_K, four shapes, 64..2048 tokens (cai_qgemm, device pointers)")
+    ap.add_argument("--step-timeline", action="store_true", help="device-side timeline of one captured batch-1 step (cai_decoder_timeline): per kernel class the gap to the previous launch, dispatch skew, staging, loop and tail times from wall-clock stamps taken inside the kernels")
     ap.add_argument("--copy-calibration", action="store_true", help="only run the 1 GiB device copy kernel 5 times (reference for traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -353,6 +395,9 @@ def main():
 
     if W > 0:
         tok = decode(tok, pos, W); pos += W
+    if args.step_timeline:
+        step_timeline(dec, tok, np)
+        return
     # K steps, timed `reps` times from the same position (the cache is cut back in between); the median repetition is reported
     walls, evs = [], []
     for rep in range(max(1, args.reps)):

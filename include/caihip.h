@@ -264,6 +264,17 @@ int cai_decoder_generate(cai_decoder_t d, int32_t first_token, int pos, int n_to
  * 4 RMSNorm + gate|up + SwiGLU (expert half of a mixture model: router .. mixture, with 5), 5 down + residual, 6 final norm +
  * vocabulary projection, 7 arg-max.  The session is not advanced (the K,V row of the current position is rewritten). */
 int cai_decoder_profile(cai_decoder_t d, int32_t token, int reps, float* us_per_step_out, int n_classes);
+/* Measurement aid (no counterpart in the reference): device-side timeline of ONE batch-1 decode step of sequence 0 at its current
+ * position.  The step is captured with timeline records armed and replayed as a graph three times; the stamps of the last
+ * replay come back.  Instrumented launches (the integer-dot and block matrix-vector kernels, the per-head attention kernel)
+ * store eight wall-clock stamps per work-group (thread 0): 0 entry, 7 exit (after the result stores were issued), 4 inputs
+ * staged (activation in registers / query rotated), 5 main loop done; matrix-vector kernels also 1 first requests issued,
+ * 2 activation values arrived, 3 block-float form complete in LDS; attention also 1 position known, 6 arrival counted.  A stamp a
+ * work-group never reached stays zero.  launches_out[3 i ..] = class of launch i (as in cai_decoder_profile), its
+ * work-groups, index of its first stamp; stamps_out[first + 8 wg + k].  ticks_per_us_out: wall-clock ticks per microsecond.
+ * The session is not advanced. */
+int cai_decoder_timeline(cai_decoder_t d, int32_t token, uint64_t* stamps_out, int64_t stamps_cap, int32_t* launches_out,
+                         int launches_cap, int* n_launches_out, int64_t* n_stamps_out, float* ticks_per_us_out);
 /* Multi-token prompt ingestion for sequence `seq` on the matrix cores: equals n sequential steps
  * within tolerance.  last_logits (host, [vocab]) and argmax may be NULL. */
 int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* tokens, int n, int pos0,

@@ -8,7 +8,7 @@ import os
 import subprocess
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(PKG_DIR, "libcaihip.so")
+LIB_PATH = os.environ.get("CAIHIP_LIB") or os.path.join(PKG_DIR, "libcaihip.so")   # (CAIHIP_LIB: another build of the library)
 CSRC_DIR = os.path.join(PKG_DIR, "csrc")
 
 

@@ -21,7 +21,7 @@ cai_dev_alloc cai_dev_free cai_dev_upload cai_dev_download cai_dev_copy
 cai_qw_create cai_qw_create_int8row cai_qw_destroy cai_qw_info cai_qw_dequant_rows cai_qgemv cai_ffn_gateup cai_qgemm
 cai_rmsnorm cai_rope cai_swiglu cai_argmax cai_argmax_noalloc cai_router_topk
 cai_kv_create cai_kv_destroy cai_kv_reset cai_kv_truncate cai_kv_len cai_kv_snapshot cai_kv_restore cai_kv_snap_destroy cai_kv_export_layer cai_kv_import_layer cai_kv_set_eviction cai_kv_rows cai_attn_decode
-cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_hidden_state cai_decoder_step_window cai_prompt_lookup_draft cai_decoder_generate_lookup cai_decoder_generate cai_decoder_profile
+cai_decoder_create cai_decoder_destroy cai_decoder_set_weight cai_decoder_set_vector cai_decoder_step cai_decoder_hidden_state cai_decoder_step_window cai_prompt_lookup_draft cai_decoder_generate_lookup cai_decoder_generate cai_decoder_profile cai_decoder_timeline
 cai_decoder_prefill cai_decoder_reset cai_decoder_truncate cai_decoder_len cai_decoder_set_eviction cai_decoder_cache_rows cai_decoder_set_kv_dtype cai_decoder_set_rope_scaling cai_decoder_set_rope_freq_factors cai_decoder_set_rope_out_scale cai_sample_candidates cai_decoder_candidates cai_decoder_snapshot cai_decoder_restore cai_decoder_fork
 cai_decoder_weight_bytes cai_decoder_get_config cai_decoder_load_gguf
 cai_gguf_open cai_gguf_close cai_gguf_info cai_gguf_meta_int cai_gguf_meta_float cai_gguf_meta_str cai_gguf_meta_array_count
@@ -108,6 +108,7 @@ def load():
         L.cai_prompt_lookup_draft.argtypes = [vp, i32, i32, i32, vp, vp]
         L.cai_decoder_generate_lookup.argtypes = [vp, vp, i32, i32, i32, i32, vp, vp]
         L.cai_decoder_profile.argtypes = [vp, i32, i32, vp, i32]
+        L.cai_decoder_timeline.argtypes = [vp, i32, vp, C.c_int64, vp, i32, vp, vp, vp]
         L.cai_decoder_prefill.argtypes = [vp, i32, vp, i32, i32, vp, vp]
         L.cai_decoder_reset.argtypes = [vp, i32]
         L.cai_decoder_truncate.argtypes = [vp, i32, i32]
@@ -461,6 +462,21 @@ class Decoder:
         us = np.zeros(8, np.float32)
         check(load().cai_decoder_profile(self.h, int(token), reps, _ptr(us), 8))
         return us
+
+    def timeline(self, token, stamps_cap=1 << 20, launches_cap=4096):
+        """device-side stamps of one captured batch-1 step (see cai_decoder_timeline): a list of (class, stamps[work-groups][8]
+        in microseconds from the earliest stamp; NaN where a work-group never took the stamp)"""
+        st = np.zeros(stamps_cap, np.uint64); la = np.zeros(3 * launches_cap, np.int32)
+        n_l = C.c_int32(); n_s = C.c_int64(); tpu = C.c_float()
+        check(load().cai_decoder_timeline(self.h, int(token), _ptr(st), stamps_cap, _ptr(la), launches_cap, C.byref(n_l), C.byref(n_s), C.byref(tpu)))
+        st = st[:n_s.value]
+        t0 = st[st > 0].min() if (st > 0).any() else 0
+        us = np.where(st > 0, (st.astype(np.int64) - np.int64(t0)).astype(np.float64) / tpu.value, np.nan)
+        out = []
+        for i in range(n_l.value):
+            cls, wgs, first = (int(v) for v in la[3 * i: 3 * i + 3])
+            out.append((cls, us[first: first + 8 * wgs].reshape(wgs, 8)))
+        return out
 
     def prefill(self, tokens, pos0=0, seq=0, want_logits=True):
         tokens = np.ascontiguousarray(tokens, np.int32)

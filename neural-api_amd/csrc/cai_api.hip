@@ -39,6 +39,16 @@ int hip_fail(hipError_t e, const char* what, const char* file, int line)
   return set_error(e == hipErrorOutOfMemory ? CAI_ERR_NOMEM : CAI_ERR_HIP, "%s failed: %s (%s:%d)", what, hipGetErrorString(e), file, line);
 }
 
+unsigned long long* timeline_next(int n_wg)
+{
+  Context::Timeline& t = g_ctx.tl;
+  if (!t.armed || t.used + (size_t)n_wg * TL_STAMPS > t.cap) return nullptr;
+  unsigned long long* r = t.buf + t.used;
+  t.launches.push_back(t.cls); t.launches.push_back(n_wg); t.launches.push_back((int32_t)t.used);
+  t.used += (size_t)n_wg * TL_STAMPS;
+  return r;
+}
+
 int ensure_stage(void** p, size_t* cap, size_t need)
 {
   if (*cap >= need) return CAI_OK;
@@ -108,6 +118,7 @@ extern "C" int cai_shutdown(void)
   nb_release(); prefill_release();
   if (c.d_small) (void)hipFree(c.d_small);
   if (c.h_small) (void)hipHostFree(c.h_small);
+  if (c.tl.buf) (void)hipFree(c.tl.buf);
   (void)hipEventDestroy(c.ev0); (void)hipEventDestroy(c.ev1);
   (void)hipStreamDestroy(c.stream);
   c = Context();

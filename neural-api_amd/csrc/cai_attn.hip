@@ -119,6 +119,7 @@ struct AttnParams {
   int evict_sinks, evict_cap;  // cap > 0: only the first `sinks` positions and the latest cap - sinks stay cached
   const float* qn_gain; const float* kn_gain; float qk_eps;   // full-width RMSNorm of q and of k applied while they are read (null: rows are used as they are)
   unsigned* merge_cnt;         // decode steps: arrival counters [seq][head]; the work-group that completes the last slice merges (null: a merge launch follows)
+  unsigned long long* timeline; // stamps of this launch's work-groups (null: none)
 };
 
 // ---- merge of the split partials inside the split kernels ----
@@ -139,23 +140,25 @@ __device__ __forceinline__ void merge_if_last(const AttnParams& p, int seq, int 
   if (threadIdx.x == 0)
     s_is_last = __builtin_amdgcn_atomic_inc32(p.merge_cnt + counter, (unsigned)n_active - 1, __ATOMIC_RELAXED, "agent") == (unsigned)n_active - 1;
   __syncthreads();
+  timeline_stamp(p.timeline, 6);
   if (!s_is_last) return;
-  // One round trip: every thread requests, per slice, its value and the slice's maximum and sum together (the latter two
-  // are the same addresses in all threads), then folds the slices in order with a running maximum.
+  // One round trip per MB slices: every thread requests, per slice, its value and the slice's maximum and sum together (the
+  // latter two are the same addresses in all threads), then folds the slices in order with a running maximum.
+  constexpr int MB = 12;
   const int hd = p.hd;
   for (int o = threadIdx.x; o < n_heads * hd; o += blockDim.x) {
     const int qh = qh0 + o / hd, d = o % hd;
     const float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + s_first) * (hd + 2);
     float A = 0.0f, L = 0.0f, M = -1e30f;
-    for (int s0 = 0; s0 < n_active; s0 += 8) {
-      float v[8], ms[8], ls[8];
+    for (int s0 = 0; s0 < n_active; s0 += MB) {
+      float v[MB], ms[MB], ls[MB];
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
+      for (int u = 0; u < MB; u++) {
         const float* ps = pt + (int64_t)min(s0 + u, n_active - 1) * (hd + 2);
         v[u] = part_load(ps + d); ms[u] = part_load(ps + hd); ls[u] = part_load(ps + hd + 1);
       }
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
+      for (int u = 0; u < MB; u++) {
         if (s0 + u < n_active && ls[u] > 0.0f) {
           const float mn = fmaxf(M, ms[u]), c0 = expf(M - mn), c1 = expf(ms[u] - mn);
           A = fmaf(v[u], c1, A * c0); L = fmaf(ls[u], c1, L * c0); M = mn;
@@ -495,6 +498,7 @@ __global__ __launch_bounds__(512) void attn_merge_kernel(const AttnParams p)
 template <int DS, typename KV_T>
 __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p)
 {
+  timeline_stamp(p.timeline, 0);
   const int G = p.q_heads / p.kv_heads;
   // linear id = item_lo + 8 * (h + G * item_hi), item = split + n_splits * kv_head: consecutive ids rotate over the XCDs
   const int L = blockIdx.x, item = (L & 7) + 8 * ((L >> 3) / G), h = (L >> 3) % G;
@@ -507,6 +511,7 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
   if (s_begin >= s_end) return;   // whole work-group leaves together, before any barrier
   const int s_first = j_start / p.split_len, s_last = (len - 1) / p.split_len;
   const int n_active = s_last - s_first + 1;
+  timeline_stamp(p.timeline, 1);
 
   const int tid = threadIdx.x, hw = tid >> 5, l32 = tid & 31;
   const int hd = p.hd, qw = p.q_heads * hd, kw = p.kv_heads * hd;
@@ -538,7 +543,23 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
       if (I8) { ch.ks[c] = ksc[j]; ch.vs[c] = vsc[j]; }
     }
   };
-  load_chunk(cA, s_begin + hw);      // cached rows are requested before the rotation math
+  // Requests return in the order they were issued: the step's own q, k, v elements and the rotary frequencies go out first, the
+  // cached rows behind them, so that the rotation (sine and cosine of an exact angle) runs while the rows are on their way
+  // instead of after them.
+  const bool owns_new = !p.appended && slot >= s_begin && slot < s_end;
+  float qraw[DS], kraw[DS], vraw[DS], qmate = 0.0f, kmate = 0.0f, th[(DS + 1) / 2];
+  {
+    const float* qp = row + (g * G + h) * hd; const float* kp = row + qw + g * hd; const float* vp = row + qw + kw + g * hd;
+#pragma unroll
+    for (int i = 0; i < DS; i++) {
+      const int d = min(d0 + i, hd - 1);          // (lanes beyond the head width read its last element; the values are dropped)
+      qraw[i] = qp[d]; kraw[i] = owns_new ? kp[d] : 0.0f; vraw[i] = owns_new ? vp[d] : 0.0f;
+    }
+    if (DS == 1) { const int dm = min(d0 ^ 1, hd - 1); qmate = qp[dm]; kmate = owns_new ? kp[dm] : 0.0f; }
+#pragma unroll
+    for (int i = 0; i < (DS + 1) / 2; i++) th[i] = p.theta ? p.theta[min(d0 + 2 * i, hd - 1) >> 1] : 0.0f;
+  }
+  load_chunk(cA, s_begin + hw);
   load_chunk(cB, s_begin + hw + 8 * PCH);
 
   // Full-width RMSNorm of q and k (neural/neuralpretrained.pas:16511-16530) folded into this kernel: every work-group
@@ -561,35 +582,35 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
   for (int i = 0; i < (DS + 1) / 2; i++) {
     rs[i] = 0.0f; rc[i] = 1.0f;
     const int d = d0 + 2 * i;
-    if (p.theta && d < hd) { const float angle = (float)pos * p.theta[d >> 1]; sincosf(angle, &rs[i], &rc[i]); }
+    if (p.theta && d < hd) { const float angle = (float)pos * th[i]; sincosf(angle, &rs[i], &rc[i]); }
   }
-  auto load_rot = [&](const float* v, float (&o)[DS], bool rotate, const float* gain, float inv) {
-    auto elem = [&](int d) { return d < hd ? (gain ? gain[d] * (v[d] * inv) : v[d]) : 0.0f; };
+  // raw elements (own DS, for DS = 1 also the pair's other element) -> optional RMSNorm gain -> optional rotation
+  auto finish_rot = [&](const float (&raw)[DS], float mate_raw, float (&o)[DS], bool rotate, const float* gain, float inv) {
+    auto elem = [&](float v, int d) { return d < hd ? (gain ? gain[d] * (v * inv) : v) : 0.0f; };
     if (DS >= 2) {
 #pragma unroll
       for (int i = 0; i < DS; i += 2) {
         const int d = d0 + i;
-        const float x0 = elem(d), x1 = elem(d + 1);
+        const float x0 = elem(raw[i], d), x1 = elem(raw[i + (DS > 1 ? 1 : 0)], d + 1);
         if (rotate) { o[i] = rc[i / 2] * x0 - rs[i / 2] * x1; o[i + (DS > 1 ? 1 : 0)] = rs[i / 2] * x0 + rc[i / 2] * x1; }
         else { o[i] = x0; o[i + (DS > 1 ? 1 : 0)] = x1; }
       }
     } else {
       const int d = d0;
-      const float own = elem(d), mate = elem(d ^ 1);
+      const float own = elem(raw[0], d), mate = elem(mate_raw, d ^ 1);
       if (rotate) o[0] = (d & 1) ? (rs[0] * mate + rc[0] * own) : (rc[0] * own - rs[0] * mate);
       else o[0] = own;
     }
   };
   float q[DS], knew[DS], vnew[DS], acc[DS];
-  load_rot(row + (g * G + h) * hd, q, p.theta != nullptr, p.qn_gain ? p.qn_gain + (g * G + h) * hd : nullptr, inv_q);
+  finish_rot(qraw, qmate, q, p.theta != nullptr, p.qn_gain ? p.qn_gain + (g * G + h) * hd : nullptr, inv_q);
 #pragma unroll
   for (int i = 0; i < DS; i++) { acc[i] = 0.0f; knew[i] = 0.0f; vnew[i] = 0.0f; }
   // every work-group whose slice holds `pos` keeps the new row in registers; the group's first head appends it
-  const bool owns_new = !p.appended && slot >= s_begin && slot < s_end;
   float knew_s = 1.0f, vnew_s = 1.0f;
   if (owns_new) {
-    load_rot(row + qw + g * hd, knew, p.theta != nullptr, p.kn_gain ? p.kn_gain + g * hd : nullptr, inv_k);
-    load_rot(row + qw + kw + g * hd, vnew, false, nullptr, 1.0f);
+    finish_rot(kraw, kmate, knew, p.theta != nullptr, p.kn_gain ? p.kn_gain + g * hd : nullptr, inv_k);
+    finish_rot(vraw, 0.0f, vnew, false, nullptr, 1.0f);
     if constexpr (I8) {
       knew_s = quantise_row_i8<DS>(knew);
       vnew_s = quantise_row_i8<DS>(vnew);
@@ -612,6 +633,7 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
     }
   }
   float m = -1e30f, l = 0.0f;
+  timeline_stamp_after(p.timeline, 4, q[0]);
   auto reduce_chunk = [&](Chunk& ch, int j0) {
     float sc[PCH], cmax = -1e30f;
 #pragma unroll
@@ -653,6 +675,7 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
   }
 
   // ---- meeting of the 8 half-waves ----
+  timeline_stamp(p.timeline, 5);
   __shared__ float sm[8], sl[8];
   __shared__ float sacc[8][32 * DS];
   if (l32 == 0) { sm[hw] = m; sl[hw] = l; }
@@ -680,14 +703,17 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
     }
   }
   if (n_active > 1 && p.merge_cnt) merge_if_last(p, seq, g * G + h, 1, s_first, n_active, seq * p.kv_heads * 8 + g * G + h);
+  timeline_stamp(p.timeline, 7);
 }
 
 template <typename KV_T>
-static int launch_split_head(const AttnParams& p, int n_seq, hipStream_t st)
+static int launch_split_head(const AttnParams& p0, int n_seq, hipStream_t st)
 {
+  AttnParams p = p0;
   const int G = p.q_heads / p.kv_heads;
   const int items = p.n_splits * p.kv_heads;
   const dim3 grid(8 * G * ((items + 7) / 8), n_seq);
+  p.timeline = timeline_next((int)(grid.x * grid.y));
   if (p.hd <= 32) hipLaunchKernelGGL((attn_split_head_kernel<1, KV_T>), grid, dim3(256), 0, st, p);
   else if (p.hd <= 64) hipLaunchKernelGGL((attn_split_head_kernel<2, KV_T>), grid, dim3(256), 0, st, p);
   else if (p.hd <= 128) hipLaunchKernelGGL((attn_split_head_kernel<4, KV_T>), grid, dim3(256), 0, st, p);

@@ -129,6 +129,8 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = 
   const cai_decoder_config& c = d->cfg;
   const int dm = c.d_model, qw = d->qw(), kw = d->kw(), I = c.ffn, qkvw = qw + 2 * kw;
   int rc;
+  int& tl_cls = ctx().tl.cls;    // class of the launches that follow (timeline records)
+  tl_cls = 0;
   if ((classes & 1u) && (rc = launch_embed(d->embed, d->d_tokens, n_b, d->x))) return rc;
   float* ssq_o = d->ssq;          // written by the o-projection, read by gate|up
   float* ssq_d = d->ssq + 1024;   // written by the down projection, read by the next block's q|k|v
@@ -166,6 +168,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = 
     }
     if (down_pending) { if ((rc = nb_prep_residual(d->x, dm, nullptr, 0.0f, dm, n_b))) return rc; down_pending = false; }
     // --- attention half ---
+    tl_cls = 1;
     if (classes & 2u) {
       MultiGemv m{}; m.n = 3;
       const int slots[3] = {CAI_W_Q, CAI_W_K, CAI_W_V}; const int offs[3] = {0, qw, qw + kw};
@@ -191,10 +194,12 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = 
         }
       }
     }
+    tl_cls = 2;
     if ((classes & 4u) &&
         (rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0, window ? 2 : 0, window ? d->wpart : nullptr,
                                c.qk_norm_full ? L.v[CAI_V_Q_NORM] : nullptr, c.qk_norm_full ? L.v[CAI_V_K_NORM] : nullptr, c.eps))) return rc;
     const bool o_hands = gemv_hands_off_ssq(L.w[CAI_W_O], n_b);
+    tl_cls = 3;
     if (classes & 8u) {
       MultiGemv m{}; m.n = 1; m.w[0] = L.w[CAI_W_O]; m.rows[0] = dm;
       if (o_hands) m.ssq_out = ssq_o;
@@ -202,6 +207,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = 
     }
     have_ssq_d = false;
     // --- feed-forward half ---
+    tl_cls = 4;
     if (c.n_experts == 0) {
       MultiGemv m{}; m.n = 1; m.w[0] = L.w[CAI_W_GATEUP]; m.rows[0] = 2 * I;
       if (o_hands && gemv_hands_off_ssq(m.w[0], n_b)) m.ssq_in = ssq_o;
@@ -213,6 +219,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = 
         launch_swiglu(d->gu, I, n_b, d->mid);
       }
       have_ssq_d = gemv_hands_off_ssq(L.w[CAI_W_DOWN], n_b);
+      tl_cls = 5;
       if (classes & 32u) {
         MultiGemv dn{}; dn.n = 1; dn.w[0] = L.w[CAI_W_DOWN]; dn.rows[0] = dm;
         if (have_ssq_d) dn.ssq_out = ssq_d;
@@ -222,6 +229,7 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = 
       if ((classes & 48u) && (rc = moe_ffn_rows(d, L, d->x, n_b))) return rc;
     }
   }
+  tl_cls = 6;
   if (classes & 64u) {
     cai_qw_s* hw = d->head ? d->head : d->embed;   // tied head (neural/neuralpretrained.pas:15555-)
     if (n_b >= 2 && nb_supported(hw)) {
@@ -835,6 +843,61 @@ extern "C" int cai_decoder_profile(cai_decoder_t d, int32_t token, int reps, flo
   }
   if ((rc = enqueue_step(d, 1, 0))) return rc;      // leave the buffers as a whole step leaves them
   CAI_HIP(hipGetLastError());
+  return CAI_OK;     // (the session's length is unchanged: the K,V row written at the current position is not counted)
+}
+
+// Device-side timeline of one captured batch-1 step (see the header): stamps of the third replay.
+extern "C" int cai_decoder_timeline(cai_decoder_t d, int32_t token, uint64_t* stamps_out, int64_t stamps_cap, int32_t* launches_out,
+                                    int launches_cap, int* n_launches_out, int64_t* n_stamps_out, float* ticks_per_us_out)
+{
+  CAI_ENTER();
+  CAI_READY();
+  CAI_REQUIRE(d && stamps_out && launches_out && n_launches_out && n_stamps_out && ticks_per_us_out && stamps_cap > 0 && launches_cap > 0, "cai_decoder_timeline: bad argument");
+  const cai_decoder_config& c = d->cfg;
+  int rc = check_ready(d); if (rc) return rc;
+  CAI_REQUIRE(token >= 0 && token < c.vocab, "cai_decoder_timeline: token %d outside vocab %d", token, c.vocab);
+  const int pos = d->kv.len_at(0, 0);
+  if (pos >= c.max_ctx && d->kv.evict_cap == 0) return set_error(CAI_ERR_STATE, "cai_decoder_timeline: sequence 0 reached max_ctx %d", c.max_ctx);
+#ifndef CAI_TIMELINE
+  return set_error(CAI_ERR_UNSUPPORTED, "cai_decoder_timeline: this build carries no stamps (build libcaihip_timeline.so: make -C neural-api_amd/csrc timeline)");
+#endif
+  Context& cx = ctx();
+  Context::Timeline& tl = cx.tl;
+  if ((size_t)stamps_cap > tl.cap) {
+    CAI_HIP(hipStreamSynchronize(cx.stream));
+    if (tl.buf) { (void)hipFree(tl.buf); tl.buf = nullptr; tl.cap = 0; }
+    CAI_HIP(hipMalloc((void**)&tl.buf, (size_t)stamps_cap * sizeof(unsigned long long)));
+    tl.cap = (size_t)stamps_cap;
+  }
+  d->h_io[0] = token; d->h_io[8] = pos;
+  CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
+  d->kv.geo_rows = kv_bucket_rows(&d->kv, pos + 1);
+  tl.used = 0; tl.launches.clear(); tl.armed = true;
+  hipGraph_t g = nullptr; hipGraphExec_t ge = nullptr;
+  hipError_t e = hipStreamBeginCapture(cx.stream, hipStreamCaptureModeThreadLocal);
+  if (e != hipSuccess) { tl.armed = false; return hip_fail(e, "hipStreamBeginCapture", __FILE__, __LINE__); }
+  rc = enqueue_step(d, 1, 0);
+  tl.armed = false;
+  e = hipStreamEndCapture(cx.stream, &g);
+  if (rc) { if (g) (void)hipGraphDestroy(g); return rc; }
+  if (e != hipSuccess) return hip_fail(e, "hipStreamEndCapture", __FILE__, __LINE__);
+  e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(g);
+  if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate", __FILE__, __LINE__);
+  for (int i = 0; i < 3 && e == hipSuccess; i++) {
+    if (i == 2) e = hipMemsetAsync(tl.buf, 0, tl.used * sizeof(unsigned long long), cx.stream);
+    if (e == hipSuccess) e = hipGraphLaunch(ge, cx.stream);
+  }
+  if (e == hipSuccess) e = hipMemcpyAsync(stamps_out, tl.buf, tl.used * sizeof(unsigned long long), hipMemcpyDeviceToHost, cx.stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(cx.stream);
+  (void)hipGraphExecDestroy(ge);
+  if (e != hipSuccess) return hip_fail(e, "cai_decoder_timeline replay", __FILE__, __LINE__);
+  const int n = std::min((int)(tl.launches.size() / 3), launches_cap);
+  for (int i = 0; i < 3 * n; i++) launches_out[i] = tl.launches[i];
+  *n_launches_out = n; *n_stamps_out = (int64_t)tl.used;
+  int khz = 100000;
+  (void)hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, cx.device);
+  *ticks_per_us_out = (float)khz * 1e-3f;
   return CAI_OK;     // (the session's length is unchanged: the K,V row written at the current position is not counted)
 }
 

@@ -64,6 +64,7 @@ template <int QT, int NB, int R, int MODE>
 __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
 {
   extern __shared__ float4 xs4[];          // [NB][kp/4]
+  timeline_stamp(p.timeline, 0);
   constexpr int UW = QTraits<QT>::UW, T = QTraits<QT>::T;
   constexpr int RR = MODE == 1 ? 2 * R : R;  // weight rows per wave
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -168,6 +169,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
       }
     }
     __syncthreads();
+    if (k0 == 0) timeline_stamp(p.timeline, 4);
 
     const int n_units = kp / UW;
     for (int u = lane; u < n_units; u += 64) {
@@ -394,6 +396,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
   }
 
   // ---- reduce across the wave and write ----
+  timeline_stamp(p.timeline, 5);
 #pragma unroll
   for (int r = 0; r < RR; r++)
 #pragma unroll
@@ -430,6 +433,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
       }
     }
   }
+  timeline_stamp(p.timeline, 7);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -613,10 +617,12 @@ static int panel_len(int cols, int nb)
 }
 
 template <int QT, int NB, int MODE>
-static int launch_fast_r(const GemvParams& p, int n_groups_r, int R, int n_slots, hipStream_t st)
+static int launch_fast_r(const GemvParams& p0, int n_groups_r, int R, int n_slots, hipStream_t st)
 {
+  GemvParams p = p0;
   const size_t lds = (size_t)NB * p.kp_lds * 4;
   const dim3 grid((n_groups_r + 3) / 4, n_slots);
+  p.timeline = timeline_next((int)(grid.x * grid.y));
   if constexpr (NB == 1 && MODE == 0) {
     if (R == 4) { hipLaunchKernelGGL((gemv_fast<QT, NB, 4, MODE>), grid, dim3(256), lds, st, p); return CAI_OK; }
   }

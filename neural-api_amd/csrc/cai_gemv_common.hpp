@@ -73,6 +73,7 @@ struct GemvParams {
   // Q6_K: per segment the plane of d (kept behind the fields every launch reads: a wider segment record measured 2 % on the
   // launch-bound MoE step)
   const uint8_t* seg_aux2[3];
+  unsigned long long* timeline;   // stamps of this launch's work-groups (null: none)
 };
 
 __device__ __forceinline__ float cvt_ub0(uint32_t v) { return (float)(v & 0xffu); }

@@ -100,6 +100,7 @@ template <int R, int MODE, bool MULTISEG, int NS, int QT, int PK = 1>
 __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_groups, const int nsw, const int gwv)
 {
   extern __shared__ uint4 xq4[];
+  timeline_stamp(p.timeline, 0);
   constexpr int RR = MODE == 1 ? 2 * R : R;
   constexpr int TS = 16 / PK;                 // super-blocks of a row held by one wave
   static_assert(PK == 1 || PK == 2 || PK == 4 || PK == 8, "rows packed per wave");
@@ -186,9 +187,6 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
   };
 
   WRegs buf[NS][RR];
-  // weights do not depend on the activation: request the first row groups before anything else
-#pragma unroll
-  for (int k = 0; k < NS - 1; k++) issue(g_first + k * g_stride, buf[k]);
 
   // ---- activation -> block-float integers, once per work-group, through LDS ----
   {
@@ -213,10 +211,27 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
       }
     };
     request(threadIdx.x);
+    // Requests return in the order they were issued: the activation (and the producer's sum-of-squares partials) go out
+    // BEFORE the first weight requests, so that their arrival does not queue behind the first burst of weights from HBM
+    // and the block-float conversion runs while that burst is on its way (weights first: 605 tok/s on the 7B shape, this
+    // order 618).
+    float tq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const bool ssq_short = p.norm_gain && p.ssq_in && p.ssq_n <= 256;
+    if (ssq_short) {
+#pragma unroll
+      for (int u = 0; u < 4; u++) tq[u] = p.ssq_in[min(u * 64 + lane, p.ssq_n - 1)];
+    }
+#pragma unroll
+    for (int k = 0; k < NS - 1; k++) issue(g_first + k * g_stride, buf[k]);
+    timeline_stamp(p.timeline, 1);
     if (p.norm_gain) {
       float t = 0.0f;
       if (p.ssq_in) {
         // sum of squares of x delivered by the producing kernel as SSQ_PARTS per-work-group partials (fixed order)
+        if (ssq_short) {
+#pragma unroll
+          for (int u = 0; u < 4; u++) t += u * 64 < p.ssq_n ? tq[u] : 0.0f;
+        } else
 #pragma unroll 4
         for (int i = 0; i < p.ssq_n / 64; i++) t += p.ssq_in[i * 64 + lane];
         t = wave_sum(t);
@@ -239,6 +254,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
       }
       inv_rms = 1.0f / sqrtf(t / (float)cols + p.norm_eps);
     }
+    timeline_stamp_after(p.timeline, 2, c0[0].x + inv_rms);
     for (int n0 = threadIdx.x; n0 < n8; n0 += SD * nthr) {
      if (n0 != (int)threadIdx.x) request(n0);
 #pragma unroll
@@ -286,6 +302,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
      }
     }
     __syncthreads();
+    timeline_stamp(p.timeline, 3);
   }
   int xq[NL][16];
   float sA = 0.0f, sB = 0.0f, mA = 0.0f, mB = 0.0f;
@@ -324,6 +341,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
       s16[gq] = (float)tot;
     }
   }
+  timeline_stamp(p.timeline, 4);
   float ssq_acc = 0.0f;   // squares of the outputs this thread wrote (for the consumer's RMSNorm)
   float keep[RR];         // finished totals of the last row groups, one group per lane
 #pragma unroll
@@ -553,6 +571,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
     for (int k = 0; k < NS; k++)
       if (it + k < n_iters) process(buf[k], buf[(k + NS - 1) % NS], it + k);
   }
+  timeline_stamp(p.timeline, 5);
 
   if (p.ssq_out) {   // per-work-group partial of sum(y^2), summed in a fixed order; unused slots are zeroed by group 0
     __syncthreads();
@@ -566,6 +585,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
     }
     if (blockIdx.x == 0) for (int i = gridDim.x + threadIdx.x; i < p.ssq_n; i += blockDim.x) p.ssq_out[i] = 0.0f;
   }
+  timeline_stamp(p.timeline, 7);
 }
 
 template <int R, int MODE, bool MULTISEG, int NS, int PK = 1>
@@ -646,6 +666,7 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
   p.ssq_n = std::min(SSQ_PARTS, (c.n_cu + 63) / 64 * 64);
   const int grid = std::min(std::min((cum + gwv - 1) / gwv, max_wgs), p.ssq_n);
   const dim3 block(64 * waves_per_wg);
+  p.timeline = timeline_next(grid);
   auto go = [&](auto kern) {
     static std::set<const void*> raised;   // kernels whose dynamic-LDS limit has been raised
     // (a failing attribute call would leave a sticky error that a later hipGetLastError reports against an innocent launch)
@@ -675,7 +696,7 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
     else if (packed) pick_pk(ns, std::integral_constant<int, PKW>());
     else pick_pk(ns, std::integral_constant<int, 1>());
   };
-  pick(std::integral_constant<int, 2>());   // two row groups per wave: one in flight while one is reduced (three measured slower on every shape)
+  pick(std::integral_constant<int, 2>());   // two row groups per wave: one in flight while one is reduced (three or four, also for the one-row walks alone, measured slower on every shape)
   return CAI_OK;
 }
 

@@ -25,7 +25,34 @@ struct Context {
   void*  stage_sample = nullptr; size_t stage_sample_cap = 0;   // a host logits row on its way to cai_sample_candidates
   int32_t* d_small = nullptr;            // 1024 ints of device scratch for small arguments/results
   int32_t* h_small = nullptr;            // 1024 ints of pinned host memory paired with d_small
+  // Step timeline (measurement aid, cai_decoder_timeline): while armed, every instrumented launch gets a record of eight
+  // wall-clock stamps per work-group (0 entry .. 7 exit, the ones between are the kernel's own) and a descriptor (class,
+  // work-groups, offset)
+  struct Timeline {
+    bool armed = false; int cls = 0;
+    unsigned long long* buf = nullptr; size_t cap = 0, used = 0;   // stamps (device)
+    std::vector<int32_t> launches;                                  // [n][3]: class, work-groups, first stamp
+  } tl;
 };
+// record of the launch being enqueued (null unless a timeline is armed): TL_STAMPS stamps per work-group.  The stamps exist
+// only in a build with -DCAI_TIMELINE (make timeline -> libcaihip_timeline.so): even a never-taken stamp costs the streaming
+// kernels 3 % (the branch around it makes the compiler wait for every outstanding request where the paths join).
+constexpr int TL_STAMPS = 8;
+unsigned long long* timeline_next(int n_wg);
+#ifdef CAI_TIMELINE
+__device__ __forceinline__ void timeline_stamp(unsigned long long* t, int k)
+{
+  if (t && threadIdx.x == 0) t[(size_t)(blockIdx.x + gridDim.x * blockIdx.y) * TL_STAMPS + k] = wall_clock64();
+}
+// the same once `dep` has arrived (a stamp the compiler may not move in front of the wait for a loaded value)
+__device__ __forceinline__ void timeline_stamp_after(unsigned long long* t, int k, float dep)
+{
+  if (t) { asm volatile("" :: "v"(dep)); timeline_stamp(t, k); }
+}
+#else
+__device__ __forceinline__ void timeline_stamp(unsigned long long*, int) {}
+__device__ __forceinline__ void timeline_stamp_after(unsigned long long*, int, float) {}
+#endif
 
 Context& ctx();
 struct ApiLock { ApiLock(); ~ApiLock(); ApiLock(const ApiLock&) = delete; ApiLock& operator=(const ApiLock&) = delete; };

@@ -97,6 +97,7 @@ function cai_prompt_lookup_draft(context: PLongInt; n_ctx, match_len, num_draft:
 function cai_decoder_generate_lookup(d: TCaiDecoder; context: PLongInt; n_ctx, match_len, num_draft, n_tokens: LongInt; tokens_out: PLongInt; passes_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_generate(d: TCaiDecoder; first_token, pos, n_tokens: LongInt; tokens_out: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_profile(d: TCaiDecoder; token, reps: LongInt; us_per_step_out: PSingle; n_classes: LongInt): LongInt; cdecl; external CAIHIP_LIB;
+function cai_decoder_timeline(d: TCaiDecoder; token: LongInt; stamps_out: PQWord; stamps_cap: Int64; launches_out: PLongInt; launches_cap: LongInt; n_launches_out: PLongInt; n_stamps_out: PInt64; ticks_per_us_out: PSingle): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_prefill(d: TCaiDecoder; seq: LongInt; tokens: PLongInt; n, pos0: LongInt; last_logits: PSingle; argmax: PLongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_reset(d: TCaiDecoder; seq: LongInt): LongInt; cdecl; external CAIHIP_LIB;
 function cai_decoder_truncate(d: TCaiDecoder; seq, n: LongInt): LongInt; cdecl; external CAIHIP_LIB;
