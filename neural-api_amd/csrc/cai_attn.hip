@@ -495,16 +495,36 @@ __global__ __launch_bounds__(512) void attn_merge_kernel(const AttnParams p)
 //      L2: their work-groups are numbered so that they land on the same XCD), but no work-group loops over heads:
 //      with one wave per SIMD that loop is a chain of dependent DPP/exp/LDS latencies and dominated the step.
 //      Running state lives in registers; LDS is used once, for the meeting of the 8 half-waves. ----
+// The leading scalar arguments are the ones the first requests need (position, the step's q | k | v row, rotary frequencies,
+// grid geometry): they arrive preloaded in scalar registers (see the Makefile), so the position request leaves at once and the
+// rest of the parameter block is fetched while it is on its way.  hheads = query heads | KV heads << 16, hgeo = slices | head
+// width << 16.
 template <int DS, typename KV_T>
-__global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p)
+__global__ __launch_bounds__(256) void attn_split_head_kernel(const int32_t* hpos, const float* hqkv, const float* htheta, const long long hqkv_stride,
+                                                              const int hheads, const int hgeo, const AttnParams p)
 {
   timeline_stamp(p.timeline, 0);
-  const int G = p.q_heads / p.kv_heads;
+  const int q_heads = hheads & 0xffff, kv_heads = hheads >> 16, n_splits = hgeo & 0xffff, hd = hgeo >> 16;
+  const int G = q_heads / kv_heads;
   // linear id = item_lo + 8 * (h + G * item_hi), item = split + n_splits * kv_head: consecutive ids rotate over the XCDs
   const int L = blockIdx.x, item = (L & 7) + 8 * ((L >> 3) / G), h = (L >> 3) % G;
-  if (item >= p.n_splits * p.kv_heads) return;
-  const int split = item % p.n_splits, g = item / p.n_splits, seq = blockIdx.y;
-  const int pos = p.pos[seq];
+  if (item >= n_splits * kv_heads) return;
+  const int split = item % n_splits, g = item / n_splits, seq = blockIdx.y;
+  const int pos = hpos[seq];
+  // the query elements and the frequencies do not depend on the position: requested behind it, before anything waits
+  const int tid = threadIdx.x, hw = tid >> 5, l32 = tid & 31;
+  const int qw = q_heads * hd, kw = kv_heads * hd;
+  const int d0 = l32 * DS;
+  const float* row = hqkv + (int64_t)seq * hqkv_stride;
+  float qraw[DS], qmate = 0.0f, th[(DS + 1) / 2];
+  {
+    const float* qp = row + (g * G + h) * hd;
+#pragma unroll
+    for (int i = 0; i < DS; i++) qraw[i] = qp[min(d0 + i, hd - 1)];          // (lanes beyond the head width read its last element; the values are dropped)
+    if (DS == 1) qmate = qp[min(d0 ^ 1, hd - 1)];
+#pragma unroll
+    for (int i = 0; i < (DS + 1) / 2; i++) th[i] = htheta ? htheta[min(d0 + 2 * i, hd - 1) >> 1] : 0.0f;
+  }
   const LiveRows lr = live_rows(p, pos);
   const int len = lr.len, j_start = lr.j_start, slot = lr.slot;
   const int s_begin = max(j_start, split * p.split_len), s_end = min(len, (split + 1) * p.split_len);
@@ -513,10 +533,6 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
   const int n_active = s_last - s_first + 1;
   timeline_stamp(p.timeline, 1);
 
-  const int tid = threadIdx.x, hw = tid >> 5, l32 = tid & 31;
-  const int hd = p.hd, qw = p.q_heads * hd, kw = p.kv_heads * hd;
-  const int d0 = l32 * DS;
-  const float* row = p.qkv + (int64_t)seq * p.qkv_stride;
   KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (seq * p.seq_mul + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
   KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + (seq * p.seq_mul + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
 
@@ -547,17 +563,15 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const AttnParams p
   // cached rows behind them, so that the rotation (sine and cosine of an exact angle) runs while the rows are on their way
   // instead of after them.
   const bool owns_new = !p.appended && slot >= s_begin && slot < s_end;
-  float qraw[DS], kraw[DS], vraw[DS], qmate = 0.0f, kmate = 0.0f, th[(DS + 1) / 2];
+  float kraw[DS], vraw[DS], kmate = 0.0f;
   {
-    const float* qp = row + (g * G + h) * hd; const float* kp = row + qw + g * hd; const float* vp = row + qw + kw + g * hd;
+    const float* kp = row + qw + g * hd; const float* vp = row + qw + kw + g * hd;
 #pragma unroll
     for (int i = 0; i < DS; i++) {
-      const int d = min(d0 + i, hd - 1);          // (lanes beyond the head width read its last element; the values are dropped)
-      qraw[i] = qp[d]; kraw[i] = owns_new ? kp[d] : 0.0f; vraw[i] = owns_new ? vp[d] : 0.0f;
+      const int d = min(d0 + i, hd - 1);
+      kraw[i] = owns_new ? kp[d] : 0.0f; vraw[i] = owns_new ? vp[d] : 0.0f;
     }
-    if (DS == 1) { const int dm = min(d0 ^ 1, hd - 1); qmate = qp[dm]; kmate = owns_new ? kp[dm] : 0.0f; }
-#pragma unroll
-    for (int i = 0; i < (DS + 1) / 2; i++) th[i] = p.theta ? p.theta[min(d0 + 2 * i, hd - 1) >> 1] : 0.0f;
+    if (DS == 1) kmate = owns_new ? kp[min(d0 ^ 1, hd - 1)] : 0.0f;
   }
   load_chunk(cA, s_begin + hw);
   load_chunk(cB, s_begin + hw + 8 * PCH);
@@ -714,9 +728,12 @@ static int launch_split_head(const AttnParams& p0, int n_seq, hipStream_t st)
   const int items = p.n_splits * p.kv_heads;
   const dim3 grid(8 * G * ((items + 7) / 8), n_seq);
   p.timeline = timeline_next((int)(grid.x * grid.y));
-  if (p.hd <= 32) hipLaunchKernelGGL((attn_split_head_kernel<1, KV_T>), grid, dim3(256), 0, st, p);
-  else if (p.hd <= 64) hipLaunchKernelGGL((attn_split_head_kernel<2, KV_T>), grid, dim3(256), 0, st, p);
-  else if (p.hd <= 128) hipLaunchKernelGGL((attn_split_head_kernel<4, KV_T>), grid, dim3(256), 0, st, p);
+  const int hheads = p.q_heads | p.kv_heads << 16, hgeo = p.n_splits | p.hd << 16;
+  if (p.q_heads > 0xffff || p.kv_heads > 0x7fff || p.n_splits > 0xffff) return set_error(CAI_ERR_UNSUPPORTED, "attention: %d query heads, %d slices", p.q_heads, p.n_splits);
+  const long long qs = (long long)p.qkv_stride;
+  if (p.hd <= 32) hipLaunchKernelGGL((attn_split_head_kernel<1, KV_T>), grid, dim3(256), 0, st, p.pos, (const float*)p.qkv, p.theta, qs, hheads, hgeo, p);
+  else if (p.hd <= 64) hipLaunchKernelGGL((attn_split_head_kernel<2, KV_T>), grid, dim3(256), 0, st, p.pos, (const float*)p.qkv, p.theta, qs, hheads, hgeo, p);
+  else if (p.hd <= 128) hipLaunchKernelGGL((attn_split_head_kernel<4, KV_T>), grid, dim3(256), 0, st, p.pos, (const float*)p.qkv, p.theta, qs, hheads, hgeo, p);
   else return set_error(CAI_ERR_UNSUPPORTED, "attention: head_dim %d > 128", p.hd);
   return CAI_OK;
 }

@@ -96,9 +96,22 @@ struct Q6kRegs { uint4 a0, a1, b0, b1, h0, h1; uint2 sc; uint32_t d; };
 // are five waves of 4 super-blocks x 4 rows instead of two waves of 16 + 4 super-blocks x 1 row.  The row a lane works on
 // then differs inside the wave (addresses and group indices are vector values), sums are taken per lane group and the
 // outputs always finish through LDS.
+// The arguments every work-group needs before it can issue its first requests travel as leading scalar kernel arguments:
+// the compiler is told to have the first 14 dwords of the argument block preloaded into scalar registers at wave launch
+// (-mllvm -amdgpu-kernarg-preload-count), so neither the activation requests nor the first weight requests wait for a round
+// trip to the argument block (fields of the parameter struct are fetched where they are first used, one round trip each).
+// rows0: rows of segment 0 (the fused feed-forward walk: the half); geo = waves along a row | waves (row streams) along the
+// rows << 8 | slots of the sum-of-squares hand-off / 64 << 16.
+struct DotHot { const float* x; const uint8_t* w0; const float* gain; const float* ssq_in; int cols, n_groups, geo, grid, rows0; };
+#define DOT_HOT_ARGS const float* hx, const uint8_t* hw0, const float* hgain, const float* hssq, const int hcols, const int hgroups, const int hgeo, const int hgrid, const int hrows0
+#define DOT_HOT_PACK DotHot{hx, hw0, hgain, hssq, hcols, hgroups, hgeo, hgrid, hrows0}
+
 template <int R, int MODE, bool MULTISEG, int NS, int QT, int PK = 1>
-__device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_groups, const int nsw, const int gwv)
+__device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const DotHot a)
 {
+  const int n_groups = a.n_groups, nsw = a.geo & 0xff, gwv = (a.geo >> 8) & 0xff, ssq_n = (a.geo >> 16) << 6;
+  const int half = MODE == 1 ? a.rows0 : 0;
+  const int nthr_wg = 64 * nsw * (gwv / PK);     // threads of the work-group (the launcher's geometry)
   extern __shared__ uint4 xq4[];
   timeline_stamp(p.timeline, 0);
   constexpr int RR = MODE == 1 ? 2 * R : R;
@@ -112,11 +125,11 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
   const int step = wave % nsw, gquad = wave / nsw;
   const int prow = PK > 1 ? (lane >> 2) / TS : 0;          // which of the wave's PK row streams this lane belongs to
   const int gslot = gquad * PK + prow;
-  const int cols = p.cols, nsb = cols >> 8;
+  const int cols = a.cols, nsb = cols >> 8;
   const int64_t row_bytes = (int64_t)nsb * dot_rec_bytes<QT>();
   const int sb = step * TS + (PK > 1 ? (lane >> 2) % TS : (lane >> 2)), cc = lane & 3;
   const bool act = sb < nsb;
-  const int g_first = blockIdx.x * gwv + gslot, g_stride = gridDim.x * gwv;
+  const int g_first = blockIdx.x * gwv + gslot, g_stride = a.grid * gwv;
   const int n_iters = (n_groups + g_stride - 1) / g_stride;
   const int64_t lane_off = (int64_t)(act ? sb : 0) * dot_rec_bytes<QT>();
   using WRegs = typename std::conditional<QT == CAI_Q6_K, Q6kRegs, typename std::conditional<QT == CAI_Q5_K, Q5kRegs, Q4kRegs>::type>::type;
@@ -129,6 +142,18 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
       if (p.n_seg > 2 && g >= p.seg[1].grp_end) { s = 2; g0 = p.seg[1].grp_end; }
     }
     sg = &p.seg[s]; row0 = (g - g0) * R;
+  };
+  // the same, with the weight pointer of segment 0 taken from the preloaded arguments
+  auto locate_w = [&](int g, const uint8_t*& data, const uint8_t*& aux, int& rows, int& row0) {
+    int s = 0, g0 = 0;
+    if (MULTISEG) {
+      if (p.n_seg > 1 && g >= p.seg[0].grp_end) { s = 1; g0 = p.seg[0].grp_end; }
+      if (p.n_seg > 2 && g >= p.seg[1].grp_end) { s = 2; g0 = p.seg[1].grp_end; }
+    }
+    data = (!MULTISEG || s == 0) ? a.w0 : p.seg[s].data;
+    if (QT == CAI_Q4_K || QT == CAI_Q5_K) aux = nullptr; else aux = p.seg[s].aux;
+    rows = (!MULTISEG || s == 0) ? a.rows0 : p.seg[s].rows;
+    row0 = (g - g0) * R;
   };
   // Loads are never conditional: past the last group the last one is fetched again, lanes beyond the row's width fetch
   // super-block 0 (both cache hits, the values are not used).  A load under a branch would make the compiler wait for
@@ -149,15 +174,15 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
   auto issue = [&](int g, WRegs (&rg)[RR]) {
     SegV sv;
     if constexpr (PK > 1) sv = locate_v(min(g, n_groups - 1));
-    else { const GemvSeg* sg1; int r0; locate(min(g, n_groups - 1), sg1, r0); sv = SegV{sg1->data, sg1->aux, sg1->rows, r0}; }
+    else locate_w(min(g, n_groups - 1), sv.data, sv.aux, sv.rows, sv.row0);
     const SegV* sg = &sv;
     const int row0 = sv.row0;
-    const int lim = MODE == 1 ? p.half : sg->rows;
+    const int lim = MODE == 1 ? half : sg->rows;
 #pragma unroll
     for (int r = 0; r < RR; r++) {
       int row = row0 + (MODE == 1 ? (r >> 1) : r);
       if (row >= lim) row = lim - 1;               // tail group: re-read the last row, result is not written
-      if (MODE == 1 && (r & 1)) row += p.half;
+      if (MODE == 1 && (r & 1)) row += half;
       const uint8_t* blk = sg->data + (int64_t)row * row_bytes + lane_off;
       if constexpr (QT == CAI_Q6_K) {
         const int nh = cc >> 1;
@@ -191,22 +216,22 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
   // ---- activation -> block-float integers, once per work-group, through LDS ----
   {
     float inv_rms = 1.0f;
-    const float4* src = reinterpret_cast<const float4*>(p.x);
-    const int n8 = cols >> 3, nthr = blockDim.x;
+    const float4* src = reinterpret_cast<const float4*>(a.x);
+    const int n8 = cols >> 3, nthr = nthr_wg;
     // one thread = 8 consecutive activations (a quarter of a 32-block: the block's four threads are one DPP quad).
     // A thread's turns (n, n + nthr, ...) are requested SD at a time - a long row (the 18944-wide down projection: four
     // turns) costs one cache round trip instead of one per turn; the first batch goes out before the sum of squares.
     constexpr int SD = (MODE == 1 || MULTISEG) ? 1 : 4;   // (the fused-norm walks have rows of one turn; batching only costs them registers)
     typedef float f4 __attribute__((ext_vector_type(4)));   // (arrays of HIP's float4 struct end up in scratch memory)
-    const f4* src4 = reinterpret_cast<const f4*>(p.x);
-    const f4* gsrc4 = reinterpret_cast<const f4*>(p.norm_gain);
+    const f4* src4 = reinterpret_cast<const f4*>(a.x);
+    const f4* gsrc4 = reinterpret_cast<const f4*>(a.gain);
     f4 c0[SD], c1[SD], cg0[SD], cg1[SD];
     auto request = [&](int n0) {
 #pragma unroll
       for (int u = 0; u < SD; u++) {
         const int nn = min(n0 + u * nthr, n8 - 1);     // past the end: the last eight again (not used)
         c0[u] = src4[2 * nn]; c1[u] = src4[2 * nn + 1];
-        if (p.norm_gain) { cg0[u] = gsrc4[2 * nn]; cg1[u] = gsrc4[2 * nn + 1]; }
+        if (a.gain) { cg0[u] = gsrc4[2 * nn]; cg1[u] = gsrc4[2 * nn + 1]; }
         else { cg0[u] = (f4)(0.0f); cg1[u] = (f4)(0.0f); }
       }
     };
@@ -216,24 +241,24 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
     // and the block-float conversion runs while that burst is on its way (weights first: 605 tok/s on the 7B shape, this
     // order 618).
     float tq[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    const bool ssq_short = p.norm_gain && p.ssq_in && p.ssq_n <= 256;
+    const bool ssq_short = a.gain && a.ssq_in && ssq_n <= 256;
     if (ssq_short) {
 #pragma unroll
-      for (int u = 0; u < 4; u++) tq[u] = p.ssq_in[min(u * 64 + lane, p.ssq_n - 1)];
+      for (int u = 0; u < 4; u++) tq[u] = a.ssq_in[min(u * 64 + lane, ssq_n - 1)];
     }
 #pragma unroll
     for (int k = 0; k < NS - 1; k++) issue(g_first + k * g_stride, buf[k]);
     timeline_stamp(p.timeline, 1);
-    if (p.norm_gain) {
+    if (a.gain) {
       float t = 0.0f;
-      if (p.ssq_in) {
+      if (a.ssq_in) {
         // sum of squares of x delivered by the producing kernel as SSQ_PARTS per-work-group partials (fixed order)
         if (ssq_short) {
 #pragma unroll
-          for (int u = 0; u < 4; u++) t += u * 64 < p.ssq_n ? tq[u] : 0.0f;
+          for (int u = 0; u < 4; u++) t += u * 64 < ssq_n ? tq[u] : 0.0f;
         } else
 #pragma unroll 4
-        for (int i = 0; i < p.ssq_n / 64; i++) t += p.ssq_in[i * 64 + lane];
+        for (int i = 0; i < ssq_n / 64; i++) t += a.ssq_in[i * 64 + lane];
         t = wave_sum(t);
         t = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, t), 63));
       } else {
@@ -249,7 +274,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
         if (lane == 63) s_ss[wave] = t;
         __syncthreads();
         t = 0.0f;
-        for (int w = 0; w < (int)(blockDim.x >> 6); w++) t += s_ss[w];
+        for (int w = 0; w < (nthr_wg >> 6); w++) t += s_ss[w];
         __syncthreads();                                 // s_ss is reused by the output sum of squares
       }
       inv_rms = 1.0f / sqrtf(t / (float)cols + p.norm_eps);
@@ -263,7 +288,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
       if (n < n8) {
       f4 v0 = c0[t], v1 = c1[t];
       const f4 g0 = cg0[t], g1 = cg1[t];
-      if (p.norm_gain) {
+      if (a.gain) {
         v0.x = g0.x * (v0.x * inv_rms); v0.y = g0.y * (v0.y * inv_rms); v0.z = g0.z * (v0.z * inv_rms); v0.w = g0.w * (v0.w * inv_rms);
         v1.x = g1.x * (v1.x * inv_rms); v1.y = g1.y * (v1.y * inv_rms); v1.z = g1.z * (v1.z * inv_rms); v1.w = g1.w * (v1.w * inv_rms);
       }
@@ -580,36 +605,36 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const int n_g
     __syncthreads();
     if (threadIdx.x == 0) {
       float tot = 0.0f;
-      for (int w = 0; w < (int)(blockDim.x >> 6); w++) tot += s_ss[w];
+      for (int w = 0; w < (nthr_wg >> 6); w++) tot += s_ss[w];
       p.ssq_out[blockIdx.x] = tot;
     }
-    if (blockIdx.x == 0) for (int i = gridDim.x + threadIdx.x; i < p.ssq_n; i += blockDim.x) p.ssq_out[i] = 0.0f;
+    if (blockIdx.x == 0) for (int i = a.grid + threadIdx.x; i < ssq_n; i += nthr_wg) p.ssq_out[i] = 0.0f;
   }
   timeline_stamp(p.timeline, 7);
 }
 
 template <int R, int MODE, bool MULTISEG, int NS, int PK = 1>
-__global__ __launch_bounds__(768, 3) void gemv_q4k_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
+__global__ __launch_bounds__(768, 3) void gemv_q4k_dot(DOT_HOT_ARGS, const GemvParams p)
 {
-  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q4_K, PK>(p, n_groups, nsw, gwv);
+  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q4_K, PK>(p, DOT_HOT_PACK);
 }
 
 template <int R, int MODE, bool MULTISEG, int NS, int PK = 1>
-__global__ __launch_bounds__(768, 3) void gemv_q40_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
+__global__ __launch_bounds__(768, 3) void gemv_q40_dot(DOT_HOT_ARGS, const GemvParams p)
 {
-  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q4_0, PK>(p, n_groups, nsw, gwv);
+  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q4_0, PK>(p, DOT_HOT_PACK);
 }
 
 template <int R, int MODE, bool MULTISEG, int NS, int PK = 1>
-__global__ __launch_bounds__(768, 3) void gemv_q5k_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
+__global__ __launch_bounds__(768, 3) void gemv_q5k_dot(DOT_HOT_ARGS, const GemvParams p)
 {
-  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q5_K, PK>(p, n_groups, nsw, gwv);
+  gemv_dot_body<R, MODE, MULTISEG, NS, CAI_Q5_K, PK>(p, DOT_HOT_PACK);
 }
 
 template <int R, int NS>
-__global__ __launch_bounds__(768, 3) void gemv_q6k_dot(const GemvParams p, const int n_groups, const int nsw, const int gwv)
+__global__ __launch_bounds__(768, 3) void gemv_q6k_dot(DOT_HOT_ARGS, const GemvParams p)
 {
-  gemv_dot_body<R, 0, false, NS, CAI_Q6_K>(p, n_groups, nsw, gwv);
+  gemv_dot_body<R, 0, false, NS, CAI_Q6_K>(p, DOT_HOT_PACK);
 }
 
 // Host launcher.  Returns CAI_ERR_UNSUPPORTED when the shape does not fit this kernel (caller falls back).
@@ -672,7 +697,8 @@ int launch_q4k_dot(GemvParams& p, const MultiGemv& m, int swiglu_half, hipStream
     // (a failing attribute call would leave a sticky error that a later hipGetLastError reports against an innocent launch)
     if (raised.insert((const void*)kern).second && hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 2048) != hipSuccess)
       (void)hipGetLastError();
-    hipLaunchKernelGGL(kern, dim3(grid), block, lds, st, p, cum, nsw, gwv);
+    hipLaunchKernelGGL(kern, dim3(grid), block, lds, st, p.x, p.seg[0].data, p.norm_gain, p.ssq_in, p.cols, cum, nsw | gwv << 8 | (p.ssq_n >> 6) << 16,
+                       grid, swiglu_half ? swiglu_half : p.seg[0].rows, p);
   };
   auto pick_pk = [&](auto ns, auto pk) {
     constexpr int NSV = decltype(ns)::value, PKV = decltype(pk)::value;
