@@ -325,7 +325,12 @@ def main():
 
     import numpy as np
     import torch
-    importlib.import_module("neural-api_amd")
+    pkg = importlib.import_module("neural-api_amd")
+    if args.step_timeline:
+        # the stamps live in a build of their own (make -C neural-api_amd/csrc timeline): they cost the product kernels 3 %
+        pkg.LIB_PATH = os.path.join(pkg.PKG_DIR, "libcaihip_timeline.so")
+        if not os.path.exists(pkg.LIB_PATH):
+            print("bench.py: --step-timeline needs libcaihip_timeline.so (make -C neural-api_amd/csrc timeline)", file=sys.stderr); sys.exit(2)
     cai = importlib.import_module("neural-api_amd.caihip")
     synth = importlib.import_module("neural-api_amd.synth")
     if not torch.cuda.is_available():

@@ -503,7 +503,7 @@ template <int DS, typename KV_T>
 __global__ __launch_bounds__(256) void attn_split_head_kernel(const int32_t* hpos, const float* hqkv, const float* htheta, const long long hqkv_stride,
                                                               const int hheads, const int hgeo, const AttnParams p)
 {
-  timeline_stamp(p.timeline, 0);
+  const unsigned long long tl0 = timeline_now();
   const int q_heads = hheads & 0xffff, kv_heads = hheads >> 16, n_splits = hgeo & 0xffff, hd = hgeo >> 16;
   const int G = q_heads / kv_heads;
   // linear id = item_lo + 8 * (h + G * item_hi), item = split + n_splits * kv_head: consecutive ids rotate over the XCDs
@@ -531,6 +531,7 @@ __global__ __launch_bounds__(256) void attn_split_head_kernel(const int32_t* hpo
   if (s_begin >= s_end) return;   // whole work-group leaves together, before any barrier
   const int s_first = j_start / p.split_len, s_last = (len - 1) / p.split_len;
   const int n_active = s_last - s_first + 1;
+  timeline_put(p.timeline, 0, tl0);
   timeline_stamp(p.timeline, 1);
 
   KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + (seq * p.seq_mul + p.seq0) * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;

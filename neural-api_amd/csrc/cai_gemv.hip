@@ -64,7 +64,7 @@ template <int QT, int NB, int R, int MODE>
 __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
 {
   extern __shared__ float4 xs4[];          // [NB][kp/4]
-  timeline_stamp(p.timeline, 0);
+  const unsigned long long tl0 = timeline_now();
   constexpr int UW = QTraits<QT>::UW, T = QTraits<QT>::T;
   constexpr int RR = MODE == 1 ? 2 * R : R;  // weight rows per wave
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -169,7 +169,7 @@ __global__ __launch_bounds__(256) void gemv_fast(const GemvParams p)
       }
     }
     __syncthreads();
-    if (k0 == 0) timeline_stamp(p.timeline, 4);
+    if (k0 == 0) { timeline_put(p.timeline, 0, tl0); timeline_stamp(p.timeline, 4); }
 
     const int n_units = kp / UW;
     for (int u = lane; u < n_units; u += 64) {

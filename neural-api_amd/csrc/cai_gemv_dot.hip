@@ -113,7 +113,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const DotHot 
   const int half = MODE == 1 ? a.rows0 : 0;
   const int nthr_wg = 64 * nsw * (gwv / PK);     // threads of the work-group (the launcher's geometry)
   extern __shared__ uint4 xq4[];
-  timeline_stamp(p.timeline, 0);
+  const unsigned long long tl0 = timeline_now();
   constexpr int RR = MODE == 1 ? 2 * R : R;
   constexpr int TS = 16 / PK;                 // super-blocks of a row held by one wave
   static_assert(PK == 1 || PK == 2 || PK == 4 || PK == 8, "rows packed per wave");
@@ -248,6 +248,7 @@ __device__ __forceinline__ void gemv_dot_body(const GemvParams& p, const DotHot 
     }
 #pragma unroll
     for (int k = 0; k < NS - 1; k++) issue(g_first + k * g_stride, buf[k]);
+    timeline_put(p.timeline, 0, tl0);
     timeline_stamp(p.timeline, 1);
     if (a.gain) {
       float t = 0.0f;

@@ -44,6 +44,13 @@ __device__ __forceinline__ void timeline_stamp(unsigned long long* t, int k)
 {
   if (t && threadIdx.x == 0) t[(size_t)(blockIdx.x + gridDim.x * blockIdx.y) * TL_STAMPS + k] = wall_clock64();
 }
+// entry stamp: taken into a register before anything is fetched (the record's address comes from the argument block, which
+// is a memory round trip away at that point) and stored with timeline_put once the first requests are out
+__device__ __forceinline__ unsigned long long timeline_now() { return wall_clock64(); }
+__device__ __forceinline__ void timeline_put(unsigned long long* t, int k, unsigned long long v)
+{
+  if (t && threadIdx.x == 0) t[(size_t)(blockIdx.x + gridDim.x * blockIdx.y) * TL_STAMPS + k] = v;
+}
 // the same once `dep` has arrived (a stamp the compiler may not move in front of the wait for a loaded value)
 __device__ __forceinline__ void timeline_stamp_after(unsigned long long* t, int k, float dep)
 {
@@ -51,6 +58,8 @@ __device__ __forceinline__ void timeline_stamp_after(unsigned long long* t, int 
 }
 #else
 __device__ __forceinline__ void timeline_stamp(unsigned long long*, int) {}
+__device__ __forceinline__ unsigned long long timeline_now() { return 0; }
+__device__ __forceinline__ void timeline_put(unsigned long long*, int, unsigned long long) {}
 __device__ __forceinline__ void timeline_stamp_after(unsigned long long*, int, float) {}
 #endif
 
