@@ -898,6 +898,8 @@ struct orc_model {
   float rope_out_scale;   /* multiplies the rotated q and k (1 unless a rule sets it) */
   int len;
   float *x, *h, *qkv, *att, *gu, *mid, *tmp, *probs, *gates, *logits;
+  float *probs_all;   /* router probabilities of every block at the last step (a test's view of how close a selection was) */
+  int swap_layer, swap_pos;   /* test hook: at this block and position the k-th and (k+1)-th expert trade places (-1: never) */
   int* sel;
 };
 
@@ -924,6 +926,8 @@ orc_model* orc_model_new(const orc_config* cfg)
   m->gu = (float*)calloc((size_t)2 * cfg->ffn, 4); m->mid = (float*)calloc((size_t)cfg->ffn, 4);
   m->tmp = (float*)calloc((size_t)wide, 4);
   int ne = cfg->n_experts > 0 ? cfg->n_experts : 1;
+  m->swap_layer = -1; m->swap_pos = -1;
+  m->probs_all = (float*)calloc((size_t)ne * (size_t)(cfg->n_layers > 0 ? cfg->n_layers : 1), 4);
   m->probs = (float*)calloc((size_t)ne, 4); m->gates = (float*)calloc((size_t)ne, 4); m->sel = (int*)calloc((size_t)ne, sizeof(int));
   m->logits = (float*)calloc((size_t)cfg->vocab, 4);
   return m;
@@ -934,6 +938,7 @@ void orc_model_free(orc_model* m)
   if (!m) return;
   for (int l = 0; l < m->cfg.n_layers; l++) { orc_layer* y = &m->layers[l]; free(y->kc); free(y->vc); free(y->kq); free(y->vq); free(y->ks); free(y->vs); }
   free(m->layers); free(m->theta); free(m->x); free(m->h); free(m->qkv); free(m->att); free(m->gu); free(m->mid);
+  free(m->probs_all);
   free(m->tmp); free(m->probs); free(m->gates); free(m->sel); free(m->logits); free(m);
 }
 
@@ -1016,6 +1021,19 @@ int orc_model_step(orc_model* m, int token, int pos, float* logits)
     if (c->n_experts > 0) {
       lin(m, &ly->w[ORC_W_ROUTER], 0, c->n_experts, m->h, m->tmp);
       orc_softmax(m->tmp, c->n_experts, m->probs);
+      memcpy(m->probs_all + (size_t)l * c->n_experts, m->probs, (size_t)c->n_experts * 4);
+      if (l == m->swap_layer && pos == m->swap_pos && c->top_k < c->n_experts) {
+        /* the selection a rounding-level change of the router sums would make: rank top_k and rank top_k + 1 trade their
+         * probabilities (ranks by value, lower index first on equal values, as orc_topk_gate orders them) */
+        int ik = -1, ik1 = -1;
+        for (int i = 0; i < c->n_experts; i++) {
+          int rank = 0;
+          for (int j = 0; j < c->n_experts; j++) if (m->probs[j] > m->probs[i] || (m->probs[j] == m->probs[i] && j < i)) rank++;
+          if (rank == c->top_k - 1) ik = i;
+          if (rank == c->top_k) ik1 = i;
+        }
+        if (ik >= 0 && ik1 >= 0) { float t = m->probs[ik]; m->probs[ik] = m->probs[ik1]; m->probs[ik1] = t; }
+      }
       orc_topk_gate(m->probs, c->n_experts, c->top_k, c->norm_topk, m->gates, m->sel);
       float* acc = (float*)calloc((size_t)d, 4);
       for (int j = 0; j < c->top_k; j++) {
@@ -1045,6 +1063,15 @@ int orc_model_step(orc_model* m, int token, int pos, float* logits)
 /* HiddenState (neural/neuraldecode.pas:5850-5857): the output of the layer feeding the vocabulary projection, which in the
  * imported decoders is the final TokenRMSNorm (neuralpretrained.pas:16872-16875).  The step above keeps it in m->h. */
 const float* orc_model_hidden(const orc_model* m) { return m->h; }
+/* test hook: the step at position `pos` selects, in block `layer`, the (k+1)-th most probable expert instead of the k-th
+ * (what the other side of a near tie looks like); layer -1 switches it off */
+void orc_model_swap_selection(orc_model* m, int layer, int pos) { m->swap_layer = layer; m->swap_pos = pos; }
+/* router probabilities (soft-max over all experts) of block `layer` at the last step; null for a dense model */
+const float* orc_model_router_probs(const orc_model* m, int layer)
+{
+  if (m->cfg.n_experts <= 0 || layer < 0 || layer >= m->cfg.n_layers) return 0;
+  return m->probs_all + (size_t)layer * m->cfg.n_experts;
+}
 
 /* ------------------------------------------------------------------------------------------
  * Prompt-lookup draft (neural/neuraldecode.pas:7742-7765), kept in the reference's own 1-based terms: the suffix is

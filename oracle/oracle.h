@@ -144,6 +144,8 @@ int  orc_model_step(orc_model* m, int token, int pos, float* logits);
 /* The input of the vocabulary projection at the last step (final RMSNorm of the residual stream, d_model floats): HiddenState of
  * the reference session (neural/neuraldecode.pas:5850-5857 with the heuristic of 6794-6807: the layer feeding the head). */
 const float* orc_model_hidden(const orc_model* m);
+void orc_model_swap_selection(orc_model* m, int layer, int pos);       /* test hook: rank k and k + 1 trade places there */
+const float* orc_model_router_probs(const orc_model* m, int layer);   /* block `layer`'s router soft-max at the last step */
 /* PromptLookupDraft on token ids (neural/neuraldecode.pas:7742-7765): the (at most num_draft) tokens that followed the most
  * recent STRICTLY EARLIER occurrence of the context's last match_len tokens.  Returns the draft length. */
 int  orc_prompt_lookup_draft(const int32_t* ctx, int n_ctx, int match_len, int num_draft, int32_t* draft);

@@ -73,6 +73,8 @@ def lib():
         L.orc_model_len.argtypes = [C.c_void_p]
         L.orc_model_step.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         L.orc_model_hidden.argtypes = [C.c_void_p]; L.orc_model_hidden.restype = C.POINTER(C.c_float)
+        L.orc_model_swap_selection.argtypes = [C.c_void_p, C.c_int, C.c_int]; L.orc_model_swap_selection.restype = None
+        L.orc_model_router_probs.argtypes = [C.c_void_p, C.c_int]; L.orc_model_router_probs.restype = C.POINTER(C.c_float)
         L.orc_prompt_lookup_draft.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
         L.cpu_avx_dot_f32.restype = C.c_float; L.cpu_avx_dot_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
         L.cpu_avx_dot_int8.restype = C.c_float; L.cpu_avx_dot_int8.argtypes = [C.c_void_p, C.c_void_p, C.c_int]
@@ -179,6 +181,14 @@ class OracleModel:
     def hidden(self):
         """the input of the vocabulary projection at the last step (a copy)"""
         return np.ctypeslib.as_array(lib().orc_model_hidden(self.h), shape=(self.cfg.d_model,)).copy()
+
+    def swap_selection(self, layer, pos):
+        """the step at `pos` takes, in block `layer`, the (k+1)-th most probable expert instead of the k-th (-1: off)"""
+        lib().orc_model_swap_selection(self.h, layer, pos)
+
+    def router_probs(self, layer):
+        """router soft-max of block `layer` at the last step (a copy)"""
+        return np.ctypeslib.as_array(lib().orc_model_router_probs(self.h, layer), shape=(self.cfg.n_experts,)).copy()
 
     def __del__(self):
         try:
