@@ -236,27 +236,31 @@ __device__ __forceinline__ float row16_allsum(float v)
 }
 
 template <int HC, typename KV_T, int NPF>     // NPF: passes in flight per lane
-__global__ __launch_bounds__(256) void attn_group_kernel(const AttnParams p)
+__global__ __launch_bounds__(256) void attn_group_kernel(const int32_t* hpos, const float* hqkv, const float* htheta, const long long hqkv_stride,
+                                                         const int hheads, const int hgeo, const int hsl, const AttnParams p)
 {
+  // (leading scalar arguments arrive preloaded in scalar registers: position, q | k | v row and frequencies are requested without
+  //  a round trip to the argument block; hheads = query heads | KV heads << 16, hgeo = slices | head width << 16, hsl = slice length)
+  const int h_q_heads = hheads & 0xffff, h_kv_heads = hheads >> 16, h_n_splits = hgeo & 0xffff, h_hd = hgeo >> 16;
   extern __shared__ __align__(16) float lds[];
   constexpr bool I8 = sizeof(KV_T) == 1;
-  const int G = p.q_heads / p.kv_heads, n_chunks = (G + HC - 1) / HC;
-  const int split = blockIdx.x % p.n_splits, g = blockIdx.x / p.n_splits, seq = blockIdx.y;
-  const int pos = p.pos[seq];
+  const int G = h_q_heads / h_kv_heads, n_chunks = (G + HC - 1) / HC;
+  const int split = blockIdx.x % h_n_splits, g = blockIdx.x / h_n_splits, seq = blockIdx.y;
+  const int pos = hpos[seq];
   const LiveRows lr = live_rows(p, pos);
   const int len = lr.len, j_start = lr.j_start, slot = lr.slot;
-  const int s_begin = max(j_start, split * p.split_len), s_end = min(len, (split + 1) * p.split_len);
+  const int s_begin = max(j_start, split * hsl), s_end = min(len, (split + 1) * hsl);
   if (s_begin >= s_end) return;   // whole work-group leaves together, before any barrier
-  const int s_first = j_start / p.split_len, s_last = (len - 1) / p.split_len;
+  const int s_first = j_start / hsl, s_last = (len - 1) / hsl;
   const int n_active = s_last - s_first + 1;
   const int n_rows = s_end - s_begin, n_pass = (n_rows + 15) >> 4;
 
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, r = lane >> 4, c = lane & 15, rr = 4 * w + r;
-  const int hd = p.hd, qw = p.q_heads * hd, kw = p.kv_heads * hd, SL = p.split_len;
+  const int hd = h_hd, qw = h_q_heads * hd, kw = h_kv_heads * hd, SL = hsl;
   const int d0 = 8 * c;
   const bool lane_on = d0 < hd;
   const int dl = lane_on ? d0 : 0;
-  const float* row = p.qkv + (int64_t)seq * p.qkv_stride;
+  const float* row = hqkv + (int64_t)seq * hqkv_stride;
   const int64_t cache_seq = seq * p.seq_mul + p.seq0;
   KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + cache_seq * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
   KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + cache_seq * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
@@ -279,18 +283,30 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const AttnParams p)
   };
   auto prime = [&](const KV_T* base, const float* scales) {
 #pragma unroll
-    for (int u = 0; u < NPF; u++) { ring[u] = Row8<KV_T>{}; rsc[u] = 0.0f; if (u < n_pass) issue(base, scales, u, u); }
+    for (int u = 0; u < NPF; u++) { rsc[u] = 0.0f; issue(base, scales, u, u); }   // (never conditional: passes beyond the slice re-read its last row, unused)
   };
   const bool owns_new = !p.appended && slot >= s_begin && slot < s_end;
-  if (!owns_new) prime(kc, ksc);            // cached rows are requested before the rotation math
+  // Requests return in the order they were issued: the group's q pairs and frequencies (two turns of the work-group cover up to
+  // eight 128-wide heads) go out first, the cached rows behind them, so that the rotation runs while the rows are on their way.
+  const int n_qp = G * (hd >> 1);
+  float qx0[2], qx1[2], qth[2];
+#pragma unroll
+  for (int u = 0; u < 2; u++) {
+    const int e = min(tid + 256 * u, n_qp - 1), h = e / (hd >> 1), i = e % (hd >> 1);
+    const float* qh = row + (g * G + h) * hd;
+    qx0[u] = qh[2 * i]; qx1[u] = qh[2 * i + 1]; qth[u] = htheta ? htheta[i] : 0.0f;
+  }
+  if (!owns_new) prime(kc, ksc);
 
   // rotated q of the group's heads -> LDS
-  for (int e = tid; e < G * (hd >> 1); e += 256) {
+  for (int e = tid; e < n_qp; e += 256) {
     const int h = e / (hd >> 1), i = e % (hd >> 1);
-    const float* qh = row + (g * G + h) * hd;
-    float x0 = qh[2 * i], x1 = qh[2 * i + 1];
-    if (p.theta) {
-      float sn, cs; sincosf((float)pos * p.theta[i], &sn, &cs);
+    const int u = (e - tid) >> 8;
+    float x0, x1, th;
+    if (u < 2) { x0 = u ? qx0[1] : qx0[0]; x1 = u ? qx1[1] : qx1[0]; th = u ? qth[1] : qth[0]; }
+    else { const float* qh = row + (g * G + h) * hd; x0 = qh[2 * i]; x1 = qh[2 * i + 1]; th = htheta ? htheta[i] : 0.0f; }
+    if (htheta) {
+      float sn, cs; sincosf((float)pos * th, &sn, &cs);
       const float y0 = cs * x0 - sn * x1, y1 = sn * x0 + cs * x1;
       x0 = y0; x1 = y1;
     }
@@ -305,8 +321,8 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const AttnParams p)
     for (int i = 0; i < 4; i += 2) {
       const int d = e0 + i;
       float x0 = d < hd ? src[d] : 0.0f, x1 = d + 1 < hd ? src[d + 1] : 0.0f;
-      if (p.theta && !is_v && d < hd) {
-        float sn, cs; sincosf((float)pos * p.theta[d >> 1], &sn, &cs);
+      if (htheta && !is_v && d < hd) {
+        float sn, cs; sincosf((float)pos * htheta[d >> 1], &sn, &cs);
         const float y0 = cs * x0 - sn * x1, y1 = sn * x0 + cs * x1;
         x0 = y0; x1 = y1;
       }
@@ -434,7 +450,7 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const AttnParams p)
         if (n_active == 1) {
           p.out[(int64_t)seq * p.out_stride + qh * hd + d] = Ls > 0.0f ? A * (1.0f / Ls) : 0.0f;
         } else {
-          float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + split) * (hd + 2);
+          float* pt = p.part + (((int64_t)seq * h_q_heads + qh) * h_n_splits + split) * (hd + 2);
           pt[d] = A;
           if (d == 0) { pt[hd] = M; pt[hd + 1] = Ls; }
         }
@@ -447,15 +463,17 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const AttnParams p)
 // ---- merge of the split partials: one work-group per query head.  Four quarter-groups of head_dim threads each take every
 //      fourth slice (all their loads go out together: one round trip for up to 32 slices per quarter), fold them with a running
 //      maximum, and meet in LDS. ----
-__global__ __launch_bounds__(512) void attn_merge_kernel(const AttnParams p)
+__global__ __launch_bounds__(512) void attn_merge_kernel(const int32_t* hpos, const float* hpart, float* hout, const long long hout_stride,
+                                                         const int hheads, const int hgeo, const int hsl, const AttnParams p)
 {
+  const int h_q_heads = hheads & 0xffff, h_n_splits = hgeo & 0xffff, h_hd = hgeo >> 16;     // (preloaded leading arguments, as in the split kernels)
   const int qh = blockIdx.x, seq = blockIdx.y;
-  const int hd = p.hd;
-  const LiveRows lr = live_rows(p, p.pos[seq]);
-  const int s_first = lr.j_start / p.split_len, s_last = (lr.len - 1) / p.split_len;
+  const int hd = h_hd;
+  const LiveRows lr = live_rows(p, hpos[seq]);
+  const int s_first = lr.j_start / hsl, s_last = (lr.len - 1) / hsl;
   const int n_active = s_last - s_first + 1;
   if (n_active == 1) return;                       // the split kernel already wrote the final row
-  const float* pt = p.part + (((int64_t)seq * p.q_heads + qh) * p.n_splits + s_first) * (hd + 2);
+  const float* pt = hpart + (((int64_t)seq * h_q_heads + qh) * h_n_splits + s_first) * (hd + 2);
   __shared__ float qA[4][128], qM[4], qL[4];
   const int quarter = threadIdx.x >> 7, d = threadIdx.x & 127;
   float A = 0.0f, L = 0.0f, M = -1e30f;
@@ -487,7 +505,7 @@ __global__ __launch_bounds__(512) void attn_merge_kernel(const AttnParams p)
       const float e = qL[k] > 0.0f ? expf(qM[k] - Mx) : 0.0f;
       At = fmaf(qA[k][d], e, At); Lt = fmaf(qL[k], e, Lt);
     }
-    p.out[(int64_t)seq * p.out_stride + qh * hd + d] = Lt > 0.0f ? At * (1.0f / Lt) : 0.0f;
+    hout[(int64_t)seq * hout_stride + qh * hd + d] = Lt > 0.0f ? At * (1.0f / Lt) : 0.0f;
   }
 }
 
@@ -743,14 +761,16 @@ template <typename KV_T, int NPF>
 static void launch_group_t(const AttnParams& p, const dim3 grid, size_t lds, int hc, hipStream_t st)
 {
   switch (hc) {
-    case 1: hipLaunchKernelGGL((attn_group_kernel<1, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
-    case 2: hipLaunchKernelGGL((attn_group_kernel<2, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
-    case 3: hipLaunchKernelGGL((attn_group_kernel<3, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
-    case 4: hipLaunchKernelGGL((attn_group_kernel<4, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
-    case 5: hipLaunchKernelGGL((attn_group_kernel<5, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
-    case 6: hipLaunchKernelGGL((attn_group_kernel<6, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
-    case 7: hipLaunchKernelGGL((attn_group_kernel<7, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
-    default: hipLaunchKernelGGL((attn_group_kernel<8, KV_T, NPF>), grid, dim3(256), lds, st, p); break;
+#define CAI_GROUP_ARGS p.pos, (const float*)p.qkv, p.theta, (long long)p.qkv_stride, p.q_heads | p.kv_heads << 16, p.n_splits | p.hd << 16, p.split_len, p
+    case 1: hipLaunchKernelGGL((attn_group_kernel<1, KV_T, NPF>), grid, dim3(256), lds, st, CAI_GROUP_ARGS); break;
+    case 2: hipLaunchKernelGGL((attn_group_kernel<2, KV_T, NPF>), grid, dim3(256), lds, st, CAI_GROUP_ARGS); break;
+    case 3: hipLaunchKernelGGL((attn_group_kernel<3, KV_T, NPF>), grid, dim3(256), lds, st, CAI_GROUP_ARGS); break;
+    case 4: hipLaunchKernelGGL((attn_group_kernel<4, KV_T, NPF>), grid, dim3(256), lds, st, CAI_GROUP_ARGS); break;
+    case 5: hipLaunchKernelGGL((attn_group_kernel<5, KV_T, NPF>), grid, dim3(256), lds, st, CAI_GROUP_ARGS); break;
+    case 6: hipLaunchKernelGGL((attn_group_kernel<6, KV_T, NPF>), grid, dim3(256), lds, st, CAI_GROUP_ARGS); break;
+    case 7: hipLaunchKernelGGL((attn_group_kernel<7, KV_T, NPF>), grid, dim3(256), lds, st, CAI_GROUP_ARGS); break;
+    default: hipLaunchKernelGGL((attn_group_kernel<8, KV_T, NPF>), grid, dim3(256), lds, st, CAI_GROUP_ARGS); break;
+#undef CAI_GROUP_ARGS
   }
 }
 
@@ -1261,7 +1281,9 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   else
     rc = kv->dtype == CAI_KV_I8 ? launch_split_head<int8_t>(p, n_seq, c.stream) : kv->dtype == CAI_KV_F16 ? launch_split_head<__half>(p, n_seq, c.stream) : launch_split_head<float>(p, n_seq, c.stream);
   if (rc) return rc;
-  if (p.n_splits > 1 && !p.merge_cnt) hipLaunchKernelGGL(attn_merge_kernel, dim3(q_heads, n_seq), dim3(512), 0, c.stream, p);
+  if (p.n_splits > 1 && !p.merge_cnt)
+    hipLaunchKernelGGL(attn_merge_kernel, dim3(q_heads, n_seq), dim3(512), 0, c.stream, p.pos, (const float*)p.part, p.out, (long long)p.out_stride,
+                       p.q_heads | p.kv_heads << 16, p.n_splits | p.hd << 16, p.split_len, p);
   return CAI_OK;
 }
 

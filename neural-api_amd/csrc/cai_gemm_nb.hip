@@ -75,22 +75,22 @@ __device__ __forceinline__ half8_t nibbles_times_scale(uint32_t lo, uint32_t hi,
 // QT = CAI_Q5_K: the same walk over 176-byte super-blocks (neural/neuralgguf.pas:516-587): header as Q4_K, then the 32-byte plane of
 // fifth bits (bit j of byte i belongs to weight i of sub-block j), then the nibbles; sc * (nibble | bit << 4) <= 63 * 31 stays exact in f16.
 template <int QT>
-__global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
+__global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const _Float16* hxhi, const _Float16* hxlo, const _Float16* hsxhi, const _Float16* hsxlo, const float* hsinvb, const int hcols, const int hntok, const int hS, const int hntiles, const NbParams p)
 {
   constexpr int BB = QT == CAI_Q5_K ? 176 : 144, QOFF = QT == CAI_Q5_K ? 48 : 16;
   extern __shared__ __align__(16) unsigned char nb_smem[];
-  const int S = p.sb_per_slice;
+  const int S = hS;
   _Float16* xs = reinterpret_cast<_Float16*>(nb_smem);              // [S][16][NB_LDX]
   _Float16* sxs = xs + S * NB_SC * NB_LDX;                           // [S][16][8]
   float* sinv_s = reinterpret_cast<float*>(sxs + S * NB_SC * 8);     // [S][8]
   float* s_d = sinv_s + S * NB_TK;                                   // [4 waves][2][32]: d, 32*dmin per row
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: segment lookups and loop bounds stay scalar
   const int n = lane & 15, kg = lane >> 4;
-  const int K = p.cols, nsb = K >> 8, nb32 = K >> 5;
+  const int K = hcols, nsb = K >> 8, nb32 = K >> 5;
   const int slice = blockIdx.y, sb0 = slice * S, nS = min(S, nsb - sb0);
   const int64_t row_bytes = (int64_t)nsb * BB;
   const int tile0 = blockIdx.x * 4 + wave;
-  const int n_it = tile0 < p.n_tiles ? (p.n_tiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
+  const int n_it = tile0 < hntiles ? (hntiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
   const int nq = n_it * nS;                      // (tile, super-block) items of this wave
 
   struct WRegs { uint4 h[2], q[2][2], e[QT == CAI_Q5_K ? 2 : 1][2]; };   // e: Q5_K's bit plane (all 32 bytes: every lane needs its two bits of each)
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
   // branch would make the compiler wait for ALL outstanding loads at every join.
   auto load_w = [&](int q, WRegs& r) {
     const int qc = max(min(q, nq - 1), 0);
-    const int tile = min(tile0 + (qc / nS) * p.tile_stride, p.n_tiles - 1), sb = sb0 + qc % nS;
+    const int tile = min(tile0 + (qc / nS) * p.tile_stride, hntiles - 1), sb = sb0 + qc % nS;
     const NbSeg* sg; int R0; locate(tile, sg, R0);
 #pragma unroll
     for (int hh = 0; hh < 2; hh++) {
@@ -117,39 +117,41 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
     }
   };
   WRegs wa, wb, wc;
-  load_w(0, wa); load_w(1, wb);                  // weights do not depend on the staging below
 
   // ---- stage this slice of the activations: nS x 16 columns x 256 halfs, block sums, block scales ----
+  // Requests return in the order they were issued: the first batch of activation requests goes out BEFORE the first weight
+  // requests (which do not depend on the staging), so that the staged values do not queue behind the first burst of weights.
   // All requests of a thread are issued before the first value is stored (four at a time for the big array): one memory
   // round trip per four chunks instead of one per chunk.  Requests are unconditional (clamped token), absent tokens zeroed.
   {
     const int n_sx = nS * NB_SC;                   // small arrays: one thread per (super-block, column)
     const bool sx_on = (int)threadIdx.x < n_sx;
     const int sx_i = min((int)threadIdx.x, n_sx - 1), sx_col = sx_i % NB_SC, sx_s = sx_i / NB_SC, sx_tok = sx_col % NB_TK;
-    const int sx_tc = min(sx_tok, p.n_tok - 1);
-    const uint4 sxv = *reinterpret_cast<const uint4*>(((sx_col / NB_TK) ? p.sxlo : p.sxhi) + (int64_t)sx_tc * nb32 + (sb0 + sx_s) * 8);
-    const float siv = p.sinvb[(int64_t)sx_tc * nsb + sb0 + sx_s];
+    const int sx_tc = min(sx_tok, hntok - 1);
+    const uint4 sxv = *reinterpret_cast<const uint4*>(((sx_col / NB_TK) ? hsxlo : hsxhi) + (int64_t)sx_tc * nb32 + (sb0 + sx_s) * 8);
+    const float siv = hsinvb[(int64_t)sx_tc * nsb + sb0 + sx_s];
     const int total = nS * NB_SC * 32;
     for (int base = 0; base < total; base += 4 * 256) {
       uint4 v[4];
 #pragma unroll
       for (int u = 0; u < 4; u++) {
         const int idx = min(base + u * 256 + (int)threadIdx.x, total - 1);
-        const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC, tok = min(col % NB_TK, p.n_tok - 1);
-        v[u] = *reinterpret_cast<const uint4*>(((col / NB_TK) ? p.xlo : p.xhi) + (int64_t)tok * K + (sb0 + s) * 256 + chunk * 8);
+        const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC, tok = min(col % NB_TK, hntok - 1);
+        v[u] = *reinterpret_cast<const uint4*>(((col / NB_TK) ? hxlo : hxhi) + (int64_t)tok * K + (sb0 + s) * 256 + chunk * 8);
       }
+      if (base == 0) { load_w(0, wa); load_w(1, wb); }
 #pragma unroll
       for (int u = 0; u < 4; u++) {
         const int idx = base + u * 256 + (int)threadIdx.x;
         if (idx < total) {
           const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC;
-          *reinterpret_cast<uint4*>(xs + (s * NB_SC + col) * NB_LDX + chunk * 8) = (col % NB_TK) < p.n_tok ? v[u] : make_uint4(0, 0, 0, 0);
+          *reinterpret_cast<uint4*>(xs + (s * NB_SC + col) * NB_LDX + chunk * 8) = (col % NB_TK) < hntok ? v[u] : make_uint4(0, 0, 0, 0);
         }
       }
     }
     if (sx_on) {
-      *reinterpret_cast<uint4*>(sxs + sx_i * 8) = sx_tok < p.n_tok ? sxv : make_uint4(0, 0, 0, 0);
-      if (sx_col < NB_TK) sinv_s[sx_s * NB_TK + sx_tok] = sx_tok < p.n_tok ? siv : 0.0f;
+      *reinterpret_cast<uint4*>(sxs + sx_i * 8) = sx_tok < hntok ? sxv : make_uint4(0, 0, 0, 0);
+      if (sx_col < NB_TK) sinv_s[sx_s * NB_TK + sx_tok] = sx_tok < hntok ? siv : 0.0f;
     }
   }
   __syncthreads();
@@ -234,8 +236,8 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const NbParams p)
     for (int hh = 0; hh < 2; hh++)
 #pragma unroll
       for (int i = 0; i < 4; i++) tot[hh][i] = acc[hh][i] + __shfl_xor(acc[hh][i], NB_TK, 64);
-    if (n < NB_TK && tok < p.n_tok) {
-      float* dst = p.part + ((int64_t)slice * p.n_tok + tok) * p.part_stride + sg->y_off;
+    if (n < NB_TK && tok < hntok) {
+      float* dst = p.part + ((int64_t)slice * hntok + tok) * p.part_stride + sg->y_off;
 #pragma unroll
       for (int hh = 0; hh < 2; hh++) {
         const int row = R0 + 16 * hh + 4 * kg;
@@ -293,20 +295,20 @@ template <int QT> __device__ __forceinline__ half8_t codes_to_half8(uint32_t w0,
 typedef unsigned int uint2_t __attribute__((ext_vector_type(2)));
 
 template <int QT, bool TAIL>   // TAIL: width % 256 != 0
-__global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
+__global__ __launch_bounds__(256, 2) void gemm_blk_nb(const _Float16* hxhi, const _Float16* hxlo, const _Float16* hsxhi, const _Float16* hsxlo, const float* hsinvb, const int hcols, const int hntok, const int hS, const int hntiles, const NbParams p)
 {
   extern __shared__ __align__(16) unsigned char nb_smem[];
-  const int S = p.sb_per_slice;
+  const int S = hS;
   _Float16* xs = reinterpret_cast<_Float16*>(nb_smem);              // [S][16][NB_LDX]
   float* sinv_s = reinterpret_cast<float*>(xs + S * NB_SC * NB_LDX);  // [S][8]
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // uniform: segment lookups and loop bounds stay scalar
   const int n = lane & 15, kg = lane >> 4;
-  const int K = p.cols, nsb = (K + 255) >> 8, nb32 = K >> 5;
+  const int K = hcols, nsb = (K + 255) >> 8, nb32 = K >> 5;
   const int slice = blockIdx.y, sb0 = slice * S, nS = min(S, nsb - sb0);
   const int row_bytes = QT != CAI_Q4_0 ? K : (K >> 1);
   const int aux_row_bytes = nb32 * 2;
   const int tile0 = blockIdx.x * 4 + wave;
-  const int n_it = tile0 < p.n_tiles ? (p.n_tiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
+  const int n_it = tile0 < hntiles ? (hntiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
   // an item = 32 rows x 128 bytes of quants: 4 blocks of Q8_0 (half a group) or 8 blocks of Q4_0 (a whole group)
   constexpr int IB = QT != CAI_Q4_0 ? 4 : 8;     // blocks per item
   constexpr int IPG = 8 / IB;                    // items per group
@@ -324,7 +326,7 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
   // branch would make the compiler wait for ALL outstanding loads at every join.
   auto load_w = [&](int q, WRegs& r) {
     const int qc = max(min(q, nq - 1), 0);
-    const int tile = min(tile0 + (qc / nI) * p.tile_stride, p.n_tiles - 1), it = qc % nI;
+    const int tile = min(tile0 + (qc / nI) * p.tile_stride, hntiles - 1), it = qc % nI;
     const int g0 = (sb0 + it / IPG) * 8 + (it % IPG) * IB;                         // first block of the item
     const NbSeg* sg; int R0; locate(tile, sg, R0);
 #pragma unroll
@@ -354,7 +356,6 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
     }
   };
   WRegs w0, w1, w2, w3;
-  load_w(0, w0); load_w(1, w1); load_w(2, w2); load_w(3, w3);   // weights do not depend on the staging below
 
   // ---- stage this slice of the activations: nS x 16 columns x 256 halfs (zero beyond the width), block scales ----
   // All requests of a thread are issued before the first value is stored (four at a time): one memory round trip per four
@@ -362,29 +363,30 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
   {
     const int n_si = nS * NB_TK;
     const int si_i = min((int)threadIdx.x, n_si - 1), si_tok = si_i % NB_TK, si_s = si_i / NB_TK;
-    const float siv = p.sinvb[(int64_t)min(si_tok, p.n_tok - 1) * nsb + sb0 + si_s];
+    const float siv = hsinvb[(int64_t)min(si_tok, hntok - 1) * nsb + sb0 + si_s];
     const int total = nS * NB_SC * 32;
     for (int base = 0; base < total; base += 4 * 256) {
       uint4 v[4];
 #pragma unroll
       for (int u = 0; u < 4; u++) {
         const int idx = min(base + u * 256 + (int)threadIdx.x, total - 1);
-        const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC, tok = min(col % NB_TK, p.n_tok - 1);
+        const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC, tok = min(col % NB_TK, hntok - 1);
         int k = (sb0 + s) * 256 + chunk * 8;
         if (TAIL) k = min(k, K - 8);
-        v[u] = *reinterpret_cast<const uint4*>(((col / NB_TK) ? p.xlo : p.xhi) + (int64_t)tok * K + k);
+        v[u] = *reinterpret_cast<const uint4*>(((col / NB_TK) ? hxlo : hxhi) + (int64_t)tok * K + k);
       }
+      if (base == 0) { load_w(0, w0); load_w(1, w1); load_w(2, w2); load_w(3, w3); }   // (behind the first activation requests: see gemm_q4k_nb)
 #pragma unroll
       for (int u = 0; u < 4; u++) {
         const int idx = base + u * 256 + (int)threadIdx.x;
         if (idx < total) {
           const int chunk = idx & 31, col = (idx >> 5) % NB_SC, s = (idx >> 5) / NB_SC;
-          const bool present = (col % NB_TK) < p.n_tok && (!TAIL || (sb0 + s) * 256 + chunk * 8 < K);
+          const bool present = (col % NB_TK) < hntok && (!TAIL || (sb0 + s) * 256 + chunk * 8 < K);
           *reinterpret_cast<uint4*>(xs + (s * NB_SC + col) * NB_LDX + chunk * 8) = present ? v[u] : make_uint4(0, 0, 0, 0);
         }
       }
     }
-    if ((int)threadIdx.x < n_si) sinv_s[si_i] = si_tok < p.n_tok ? siv : 0.0f;
+    if ((int)threadIdx.x < n_si) sinv_s[si_i] = si_tok < hntok ? siv : 0.0f;
   }
   __syncthreads();
 
@@ -460,8 +462,8 @@ __global__ __launch_bounds__(256, 2) void gemm_blk_nb(const NbParams p)
       for (int i = 0; i < 4; i++) {
         const float tot = acc[hh][i] + __shfl_xor(acc[hh][i], 32, 64);
         const int tok = 4 * kg + i;
-        if (kg < 2 && tok < p.n_tok && row < sg->rows)
-          p.part[((int64_t)slice * p.n_tok + tok) * p.part_stride + sg->y_off + row] = tot;
+        if (kg < 2 && tok < hntok && row < sg->rows)
+          p.part[((int64_t)slice * hntok + tok) * p.part_stride + sg->y_off + row] = tot;
       }
     }
   };
@@ -493,19 +495,19 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 // NT groups of 8 tokens share every converted weight operand and scale: 9..16 tokens take one pass with NT = 2.
 template <int NT>
-__global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
+__global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const _Float16* hxhi, const _Float16* hxlo, const _Float16* hsxhi, const _Float16* hsxlo, const float* hsinvb, const int hcols, const int hntok, const int hS, const int hntiles, const NbParams p)
 {
   extern __shared__ __align__(16) unsigned char nb_smem[];
-  const int S = p.sb_per_slice;
+  const int S = hS;
   constexpr int NC = NT * NB_SC, NTOK = NT * NB_TK;                 // staged columns per super-block: group t holds tokens 8t..8t+7 as 8 hi + 8 lo
   _Float16* xs = reinterpret_cast<_Float16*>(nb_smem);              // [S][NC][NB_LDX]
   float* sinv_s = reinterpret_cast<float*>(xs + S * NC * NB_LDX);    // [S][NTOK]
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n = lane & 15, kg = lane >> 4;
-  const int K = p.cols, nsb = K >> 8;
+  const int K = hcols, nsb = K >> 8;
   const int slice = blockIdx.y, sb0 = slice * S, nS = min(S, nsb - sb0);
   const int tile0 = blockIdx.x * 4 + wave;
-  const int n_it = tile0 < p.n_tiles ? (p.n_tiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
+  const int n_it = tile0 < hntiles ? (hntiles - tile0 + p.tile_stride - 1) / p.tile_stride : 0;
   const int nq = n_it * nS;                      // (tile, super-block) items of this wave
 
   struct WRegs { u32x4_t ql[2][2], qh[2], sc[2]; uint32_t d[2]; };
@@ -518,7 +520,7 @@ __global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
   // unconditional, clamped: past the wave's last item the last one is fetched again (a cache hit)
   auto load_w = [&](int q, WRegs& r) {
     const int qc = max(min(q, nq - 1), 0);
-    const int tile = min(tile0 + (qc / nS) * p.tile_stride, p.n_tiles - 1), sb = sb0 + qc % nS;
+    const int tile = min(tile0 + (qc / nS) * p.tile_stride, hntiles - 1), sb = sb0 + qc % nS;
     const NbSeg* sg; int R0; locate(tile, sg, R0);
 #pragma unroll
     for (int hh = 0; hh < 2; hh++) {
@@ -532,7 +534,6 @@ __global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
     }
   };
   WRegs wa, wb, wc;
-  load_w(0, wa); load_w(1, wb);                  // weights do not depend on the staging below
 
   // ---- stage this slice of the activations: nS x 16 columns x 256 halfs, block scales (four requests per turn) ----
   {
@@ -544,22 +545,23 @@ __global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
       for (int u = 0; u < 4; u++) {
         const int idx = min(base + u * 256 + (int)threadIdx.x, total - 1);
         const int chunk = idx & 31, col = (idx >> 5) % NC, s = (idx >> 5) / NC;
-        const int tok = min((col / NB_SC) * NB_TK + col % NB_TK, p.n_tok - 1);
-        v[u] = *reinterpret_cast<const uint4*>((((col % NB_SC) / NB_TK) ? p.xlo : p.xhi) + (int64_t)tok * K + (sb0 + s) * 256 + chunk * 8);
+        const int tok = min((col / NB_SC) * NB_TK + col % NB_TK, hntok - 1);
+        v[u] = *reinterpret_cast<const uint4*>((((col % NB_SC) / NB_TK) ? hxlo : hxhi) + (int64_t)tok * K + (sb0 + s) * 256 + chunk * 8);
       }
+      if (base == 0) { load_w(0, wa); load_w(1, wb); }   // (behind the first activation requests: see gemm_q4k_nb)
 #pragma unroll
       for (int u = 0; u < 4; u++) {
         const int idx = base + u * 256 + (int)threadIdx.x;
         if (idx < total) {
           const int chunk = idx & 31, col = (idx >> 5) % NC, s = (idx >> 5) / NC;
           const int tok = (col / NB_SC) * NB_TK + col % NB_TK;
-          *reinterpret_cast<uint4*>(xs + (s * NC + col) * NB_LDX + chunk * 8) = tok < p.n_tok ? v[u] : make_uint4(0, 0, 0, 0);
+          *reinterpret_cast<uint4*>(xs + (s * NC + col) * NB_LDX + chunk * 8) = tok < hntok ? v[u] : make_uint4(0, 0, 0, 0);
         }
       }
     }
     for (int i = threadIdx.x; i < n_si; i += 256) {
       const int tok = i % NTOK, s = i / NTOK;
-      sinv_s[i] = tok < p.n_tok ? p.sinvb[(int64_t)tok * nsb + sb0 + s] : 0.0f;
+      sinv_s[i] = tok < hntok ? hsinvb[(int64_t)tok * nsb + sb0 + s] : 0.0f;
     }
   }
   __syncthreads();
@@ -639,8 +641,8 @@ __global__ __launch_bounds__(256, 2) void gemm_q6k_nb(const NbParams p)
         for (int i = 0; i < 4; i++) {
           const float tot = acc[t][hh][i] + __shfl_xor(acc[t][hh][i], 32, 64);
           const int tok = t * NB_TK + 4 * kg + i;
-          if (kg < 2 && tok < p.n_tok && row < sg->rows)
-            p.part[((int64_t)slice * p.n_tok + tok) * p.part_stride + sg->y_off + row] = tot;
+          if (kg < 2 && tok < hntok && row < sg->rows)
+            p.part[((int64_t)slice * hntok + tok) * p.part_stride + sg->y_off + row] = tot;
         }
       }
   };
@@ -694,8 +696,10 @@ __device__ __forceinline__ float nb_inv_rms(const float* ssq, int nsb, int K, fl
   return 1.0f / sqrtf(t / (float)K + eps);
 }
 
+// (what the first requests need travels as leading scalar arguments, preloaded in scalar registers: hsrc = x (SRC 0) or res (SRC 1))
 template <int SRC>
-__global__ __launch_bounds__(256) void nb_prep_kernel(const NbPrepParams p)
+__global__ __launch_bounds__(256) void nb_prep_kernel(const float* hsrc, const long long hstride, const float* hpart, const long long hpstride, const float* hbias,
+                                                      const float* hgain, const int hns, const int hntok, const NbPrepParams p)
 {
   const int sb = blockIdx.x, tok = blockIdx.y, k = sb * 256 + threadIdx.x;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -703,23 +707,23 @@ __global__ __launch_bounds__(256) void nb_prep_kernel(const NbPrepParams p)
   const bool in = k < p.K;                       // the last block of a width that is not a multiple of 256 is short
   float v = 0.0f;
   if (!in) {}
-  else if (SRC == 0) v = p.x[(int64_t)tok * p.x_stride + k];
+  else if (SRC == 0) v = hsrc[(int64_t)tok * hstride + k];
   else if (SRC == 1) {
-    v = p.res[(int64_t)tok * p.res_stride + k];
-    if (p.bias) v += p.bias[k];
-    v = nb_sum_strided(p.part + (int64_t)tok * p.part_stride + k, p.n_slices, (int64_t)p.n_tok * p.part_stride, v);
+    v = hsrc[(int64_t)tok * hstride + k];
+    if (hbias) v += hbias[k];
+    v = nb_sum_strided(hpart + (int64_t)tok * hpstride + k, hns, (int64_t)hntok * hpstride, v);
     p.res[(int64_t)tok * p.res_stride + k] = v;
   } else {
-    const float* col = p.part + (int64_t)tok * p.part_stride + k;
-    const float up0 = nb_sum_strided(col, p.n_slices, (int64_t)p.n_tok * p.part_stride, 0.0f);
-    const float gate0 = nb_sum_strided(col + p.half, p.n_slices, (int64_t)p.n_tok * p.part_stride, 0.0f);
+    const float* col = hpart + (int64_t)tok * hpstride + k;
+    const float up0 = nb_sum_strided(col, hns, (int64_t)hntok * hpstride, 0.0f);
+    const float gate0 = nb_sum_strided(col + p.half, hns, (int64_t)hntok * hpstride, 0.0f);
     float up = up0, gate = gate0;
     if (p.in_ssq) { const float inv = nb_inv_rms(p.in_ssq, p.in_nsb, p.in_K, p.in_eps, tok); up *= inv; gate *= inv; }
-    if (p.bias) { up += p.bias[k]; gate += p.bias[p.half + k]; }
+    if (hbias) { up += hbias[k]; gate += hbias[p.half + k]; }
     v = silu_mul(up, gate);
   }
   const float raw = v;
-  if (in && p.gain) v *= p.gain[k];
+  if (in && hgain) v *= hgain[k];
   __shared__ float red[8];
   float amax = fabsf(v), ss = raw * raw;
   for (int off = 32; off > 0; off >>= 1) { amax = fmaxf(amax, __shfl_xor(amax, off, 64)); ss += __shfl_xor(ss, off, 64); }
@@ -756,15 +760,15 @@ struct NbReduceParams {
   float* y; int64_t y_stride; const float* residual;
   int width;                                    // columns covered (sum of the segments)
 };
-__global__ __launch_bounds__(256) void nb_reduce_kernel(const NbReduceParams p)
+__global__ __launch_bounds__(256) void nb_reduce_kernel(const float* hpart, const long long hpstride, const int hns, const int hntok, const int hwidth, const NbReduceParams p)
 {
   const int tok = blockIdx.y;
   const int c = blockIdx.x * 256 + threadIdx.x;
-  if (c >= p.width) return;
+  if (c >= hwidth) return;
   int sgi = 0;
   if (p.n_seg > 1 && c >= p.seg[1].y_off) sgi = 1;
   if (p.n_seg > 2 && c >= p.seg[2].y_off) sgi = 2;
-  float v = nb_sum_strided(p.part + (int64_t)tok * p.part_stride + c, p.n_slices, (int64_t)p.n_tok * p.part_stride, 0.0f);
+  float v = nb_sum_strided(hpart + (int64_t)tok * hpstride + c, hns, (int64_t)hntok * hpstride, 0.0f);
   if (p.in_ssq) v *= nb_inv_rms(p.in_ssq, p.in_nsb, p.in_K, p.in_eps, tok);
   if (p.seg[sgi].row_scale) v *= p.seg[sgi].row_scale[c - p.seg[sgi].y_off];   // per-row int8: (sum code * x) * scale, then bias
   if (p.seg[sgi].bias) v += p.seg[sgi].bias[c - p.seg[sgi].y_off];
@@ -857,9 +861,11 @@ static int nb_prep_launch(int src, NbPrepParams& p, int n_tok)
   g_nb.cur ^= 1;
   p.hi = g_nb.hi; p.lo = g_nb.lo; p.sxhi = g_nb.sxhi; p.sxlo = g_nb.sxlo; p.sinvb = g_nb.sinvb; p.ssq = g_nb.ssq[g_nb.cur];
   const dim3 grid((p.K + 255) >> 8, n_tok);
-  if (src == 0) hipLaunchKernelGGL(nb_prep_kernel<0>, grid, dim3(256), 0, ctx().stream, p);
-  else if (src == 1) hipLaunchKernelGGL(nb_prep_kernel<1>, grid, dim3(256), 0, ctx().stream, p);
-  else hipLaunchKernelGGL(nb_prep_kernel<2>, grid, dim3(256), 0, ctx().stream, p);
+  const float* hsrc = src == 0 ? p.x : src == 1 ? p.res : nullptr;
+  const long long hstride = src == 0 ? p.x_stride : p.res_stride, hps = p.part_stride;
+  if (src == 0) hipLaunchKernelGGL(nb_prep_kernel<0>, grid, dim3(256), 0, ctx().stream, hsrc, hstride, p.part, hps, p.bias, p.gain, p.n_slices, p.n_tok, p);
+  else if (src == 1) hipLaunchKernelGGL(nb_prep_kernel<1>, grid, dim3(256), 0, ctx().stream, hsrc, hstride, p.part, hps, p.bias, p.gain, p.n_slices, p.n_tok, p);
+  else hipLaunchKernelGGL(nb_prep_kernel<2>, grid, dim3(256), 0, ctx().stream, hsrc, hstride, p.part, hps, p.bias, p.gain, p.n_slices, p.n_tok, p);
   return CAI_OK;
 }
 static void nb_set_pending_norm(const float* gain, int K, float eps)
@@ -906,12 +912,14 @@ bool nb_supported(const cai_qw_s* w)
   return (w->qtype == CAI_Q8_0 || w->qtype == CAI_Q4_0 || w->qtype == CAI_I8ROW) && w->cols % 32 == 0 && w->cols >= 32;   // per-row int8: unit block scales, the row scale is applied by nb_reduce
 }
 
-template <void (*Kernel)(const NbParams)>
+// (the activation planes, the width and the slice geometry travel as leading scalar arguments: they arrive preloaded in scalar
+//  registers, so the first requests do not wait for a round trip to the argument block; see the Makefile)
+template <void (*Kernel)(const _Float16*, const _Float16*, const _Float16*, const _Float16*, const float*, int, int, int, int, const NbParams)>
 static void nb_launch(const NbParams& p, int gx, int n_slices, size_t lds)
 {
   static bool attr_done = false;   // one flag per kernel
   if (!attr_done) { (void)hipFuncSetAttribute((const void*)Kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); attr_done = true; }
-  hipLaunchKernelGGL(Kernel, dim3(gx, n_slices), dim3(256), lds, ctx().stream, p);
+  hipLaunchKernelGGL(Kernel, dim3(gx, n_slices), dim3(256), lds, ctx().stream, p.xhi, p.xlo, p.sxhi, p.sxlo, p.sinvb, p.cols, p.n_tok, p.sb_per_slice, p.n_tiles, p);
 }
 
 int nb_pass_tokens(const cai_qw_s* w);
@@ -983,7 +991,7 @@ int nb_reduce(float* y, int64_t y_stride, const float* residual)
   p.n_seg = g_prod.n_seg; p.part = g_nb.part; p.part_stride = g_prod.part_stride; p.n_slices = g_prod.n_slices; p.n_tok = g_prod.n_tok;
   p.in_ssq = g_prod.in_ssq; p.in_nsb = g_prod.in_nsb; p.in_K = g_prod.in_K; p.in_eps = g_prod.in_eps;
   p.y = y; p.y_stride = y_stride; p.residual = residual; p.width = g_prod.width;
-  hipLaunchKernelGGL(nb_reduce_kernel, dim3((p.width + 255) / 256, p.n_tok), dim3(256), 0, ctx().stream, p);
+  hipLaunchKernelGGL(nb_reduce_kernel, dim3((p.width + 255) / 256, p.n_tok), dim3(256), 0, ctx().stream, p.part, (long long)p.part_stride, p.n_slices, p.n_tok, p.width, p);
   g_prod.n_seg = 0;
   return CAI_OK;
 }
