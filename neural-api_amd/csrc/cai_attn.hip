@@ -131,6 +131,18 @@ struct AttnParams {
 __device__ __forceinline__ void part_store(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ float part_load(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
+// Hand-over of the partial results.  The form built by default relies on what gfx942 / gfx950 do, not on the language's
+// memory model: the partials are stored with agent-scope atomic stores (written through to memory, bypassing the
+// non-coherent caches), vmcnt(0) returns only when those stores have been acknowledged, the work-group barrier orders every
+// wave's acknowledgement before thread 0's agent-scope increment, and the last arriver reads with agent-scope atomic loads
+// issued after the barrier that publishes s_is_last (atomic loads are not moved above it by the compiler).  It breaks if
+// the partials are accessed with ordinary loads or stores, or on a target where an acknowledged agent-scope store may still
+// be invisible to another compute unit.  -DCAI_MERGE_RELACQ builds the form the memory model guarantees (release increment,
+// acquire fence in the last arriver); it writes back and invalidates the L2 of the XCD on every hand-over and takes the
+// 7B batch-1 step from 1.52 to 1.60 ms.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(CAI_MERGE_RELACQ) && !defined(__gfx950__) && !defined(__gfx942__)
+#error "merge_if_last: the relaxed hand-over is only valid on gfx942 / gfx950; build with -DCAI_MERGE_RELACQ"
+#endif
 // heads qh0 .. qh0 + n_heads - 1 of sequence `seq`; every thread of the work-group calls it after its partial stores
 __device__ __forceinline__ void merge_if_last(const AttnParams& p, int seq, int qh0, int n_heads, int s_first, int n_active, int counter)
 {
@@ -138,10 +150,17 @@ __device__ __forceinline__ void merge_if_last(const AttnParams& p, int seq, int 
   __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this thread's partial stores have been acknowledged
   __syncthreads();
   if (threadIdx.x == 0)
+#ifdef CAI_MERGE_RELACQ
+    s_is_last = __builtin_amdgcn_atomic_inc32(p.merge_cnt + counter, (unsigned)n_active - 1, __ATOMIC_RELEASE, "agent") == (unsigned)n_active - 1;
+#else
     s_is_last = __builtin_amdgcn_atomic_inc32(p.merge_cnt + counter, (unsigned)n_active - 1, __ATOMIC_RELAXED, "agent") == (unsigned)n_active - 1;
+#endif
   __syncthreads();
   timeline_stamp(p.timeline, 6);
   if (!s_is_last) return;
+#ifdef CAI_MERGE_RELACQ
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#endif
   // One round trip per MB slices: every thread requests, per slice, its value and the slice's maximum and sum together (the
   // latter two are the same addresses in all threads), then folds the slices in order with a running maximum.
   constexpr int MB = 12;
@@ -1173,6 +1192,13 @@ __global__ __launch_bounds__(512) void prompt_merge_kernel(const PromptParams p,
   p.out[(int64_t)tok * p.out_stride + head * 128 + d] = L > 0.0f ? A * (1.0f / L) : 0.0f;
 }
 
+// Whether n prompt rows of this cache go to the matrix-core prompt kernel (it needs no per-slice partial results).
+bool attn_prompt_is_flash(const cai_kv_s* kv, int n)
+{
+  static const int flash_on = []() { const char* e = getenv("CAIHIP_PROMPT_FLASH"); return e ? atoi(e) : 1; }();
+  return flash_on && kv->head_dim == 128 && kv->evict_cap == 0 && n >= 8;
+}
+
 int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, int n_seq, int q_heads, int window,
                      float softcap, const float* theta, const int32_t* pos_dev, float* out, int64_t out_stride, int seq0,
                      int prompt_rows, float* prompt_part, const float* qn_gain, const float* kn_gain, float qk_eps)
@@ -1215,8 +1241,7 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
     else if ((rc = launch_rmsnorm_pair(qkv, qn_gain, qw, kn_gain, kw, n_seq, qk_eps, qkv_stride))) return rc;
   }
   // prompts over a 128-wide cache: matrix-core kernel, 32 tokens x 4 heads per work-group
-  static const int flash_on = []() { const char* e = getenv("CAIHIP_PROMPT_FLASH"); return e ? atoi(e) : 1; }();
-  const bool flash = prompt_rows == 1 && flash_on && kv->head_dim == 128 && kv->evict_cap == 0 && n_seq >= 8;
+  const bool flash = prompt_rows == 1 && attn_prompt_is_flash(kv, n_seq);
   const bool rows_fused = flash && kv->dtype != CAI_KV_I8;     // the append and the q planes share a launch (below)
   if (prompt_rows && kv->dtype == CAI_KV_I8) {
     if (p.hd <= 32) hipLaunchKernelGGL(kv_append_rows_i8_kernel<1>, dim3(n_seq), dim3(256), 0, c.stream, p);

@@ -29,6 +29,7 @@ struct cai_decoder_s {
   int pf_cap = 0;
   float *px = nullptr, *pqkv = nullptr, *patt = nullptr, *pgu = nullptr, *pmid = nullptr, *ppart = nullptr;
   size_t ppart_elems = 0;                            // (per row, query head and cache slice: sized for the length bucket in use)
+  int ppart_rows = 1;                                // prompt rows per attention launch that ppart holds (ensure_ppart)
   int32_t* ptokpos = nullptr;                        // [2][pf_cap]: tokens, positions
   // mixture-of-experts prompt: per chunk the router outputs, the slots grouped by expert and the per-slot activations
   float *pm_logits = nullptr, *pm_probs = nullptr, *pm_gate = nullptr, *pm_gu = nullptr, *pm_part = nullptr;
@@ -293,12 +294,24 @@ static int ensure_prefill_buffers(cai_decoder_s* d, int n)
 
 // Partial results of the prompt rows' attention when it runs on the decode kernels (rows x query heads x cache slices): sized
 // for the slice count of the length bucket in use, so a session created for 131072 rows does not hold 512 slices' worth for a
-// prompt at its start.  Grown on demand; prompt passes are not captured, so the pointer may change between them.
-static int ensure_ppart(cai_decoder_s* d, int rows_needed)
+// prompt at its start, and for at most 256 MiB: a chunk whose rows need more (512 slices x 32 heads x 66 floats are 4.3 MB
+// per row) attends in groups of ppart_rows rows, one attention launch per group.  A chunk the matrix-core prompt kernel
+// takes needs none.  Grown on demand; prompt passes are not captured, so the pointer may change between them.
+// (CAIHIP_PROMPT_PART_KB: another bound, read once per process; the tests use it to reach the grouped form with small models)
+static size_t ppart_bytes()
 {
+  static const size_t b = []() { const char* e = getenv("CAIHIP_PROMPT_PART_KB"); return e && atoll(e) > 0 ? (size_t)atoll(e) << 10 : (size_t)256 << 20; }();
+  return b;
+}
+static int ensure_ppart(cai_decoder_s* d, int rows_needed, int n)
+{
+  if (attn_prompt_is_flash(&d->kv, n)) { d->ppart_rows = n; return CAI_OK; }
   int sl, ns;
   kv_geometry(&d->kv, kv_bucket_rows(&d->kv, rows_needed), &sl, &ns);
-  const size_t need = (size_t)d->pf_cap * d->cfg.n_q_heads * ns * (d->cfg.head_dim + 2);
+  const size_t per_row = (size_t)d->cfg.n_q_heads * ns * (d->cfg.head_dim + 2);
+  const int rows = (int)std::max<size_t>(1, std::min<size_t>((size_t)n, ppart_bytes() / (per_row * sizeof(float))));
+  const size_t need = per_row * rows;
+  d->ppart_rows = rows;
   if (d->ppart && d->ppart_elems >= need) return CAI_OK;
   CAI_HIP(hipStreamSynchronize(ctx().stream));
   if (d->ppart) { (void)hipFree(d->ppart); d->ppart = nullptr; }
@@ -368,8 +381,11 @@ static int enqueue_prefill_chunk(cai_decoder_s* d, int seq, int n)
       if ((rc = linear_rows(wk, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw, qkvw, nullptr))) return rc;
       if ((rc = linear_rows(wv, all_mfma, d->px, dm, L.v[CAI_V_ATTN_NORM], c.eps, n, d->pqkv + qw + kw, qkvw, nullptr))) return rc;
     }
-    if ((rc = launch_attn_step(&d->kv, l, d->pqkv, qkvw, n, c.n_q_heads, c.window, 0.0f, d->theta, poss, d->patt, qw, seq, 1, d->ppart,
-                               c.qk_norm_full ? L.v[CAI_V_Q_NORM] : nullptr, c.qk_norm_full ? L.v[CAI_V_K_NORM] : nullptr, c.eps))) return rc;
+    // (rows attend to the cache rows up to their own position, so a later group may be appended after an earlier one has attended)
+    for (int r0 = 0; r0 < n; r0 += d->ppart_rows)
+      if ((rc = launch_attn_step(&d->kv, l, d->pqkv + (int64_t)r0 * qkvw, qkvw, std::min(d->ppart_rows, n - r0), c.n_q_heads, c.window, 0.0f, d->theta,
+                                 poss + r0, d->patt + (int64_t)r0 * qw, qw, seq, 1, d->ppart,
+                                 c.qk_norm_full ? L.v[CAI_V_Q_NORM] : nullptr, c.qk_norm_full ? L.v[CAI_V_K_NORM] : nullptr, c.eps))) return rc;
     if ((rc = linear_rows(L.w[CAI_W_O], false, d->patt, qw, nullptr, 0.0f, n, d->px, dm, d->px))) return rc;
     if (c.n_experts > 0) {
       // experts differ from token to token.  A chunk of more than 16 tokens whose banks the block prompt kernel takes is
@@ -934,7 +950,7 @@ extern "C" int cai_decoder_prefill(cai_decoder_t d, int seq, const int32_t* toke
       CAI_HIP(hipMemcpyAsync(d->ptokpos, tp.data(), tp.size() * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
       CAI_HIP(hipStreamSynchronize(cx.stream));
       d->kv.geo_rows = kv_bucket_rows(&d->kv, pos0 + t0 + m);
-      if ((rc = ensure_ppart(d, pos0 + t0 + m))) return rc;
+      if ((rc = ensure_ppart(d, pos0 + t0 + m, m))) return rc;
       if ((rc = enqueue_prefill_chunk(d, seq, m))) return rc;
       CAI_HIP(hipGetLastError());
       if (t0 + chunk >= n) {

@@ -446,10 +446,11 @@ extern "C" int cai_decoder_load_gguf(const char* path, int max_ctx, int max_batc
     if (dm % hq) return fail(set_error(CAI_ERR_INVALID, "gguf decoder: %s=%lld is not divisible by %s=%lld", key("embedding_length").c_str(), (long long)dm, key("attention.head_count").c_str(), (long long)hq));
     hd = dm / hq;
   }
-  // rope.scaling.type "linear" -> Position Interpolation with rope.scaling.factor; absent / "none" = unscaled; anything else
-  // is refused (neural/neuralpretrained.pas:17539-17557)
+  // llama files: rope.scaling.type "linear" -> Position Interpolation with rope.scaling.factor; absent / "none" = unscaled;
+  // anything else is refused (neural/neuralpretrained.pas:17539-17557).  qwen2 files: the key is not read and the rotation
+  // stays unscaled, as the reference's qwen2 import leaves it (neural/neuralpretrained.pas:17720).
   double rope_linear = 1.0;
-  {
+  if (arch == "llama") {
     const MetaValue* st = find_meta(g, key("rope.scaling.type").c_str());
     if (st && st->type == GT_STR && st->s != "none") {
       const double f = opt_float("rope.scaling.factor", 1.0);
@@ -459,7 +460,9 @@ extern "C" int cai_decoder_load_gguf(const char* path, int max_ctx, int max_batc
       rope_linear = f;
     }
   }
-  // per-frequency divisors (llama.cpp's form of the Llama-3.1 rule): one F32 value per rotary pair
+  // per-frequency divisors (llama.cpp's form of the Llama-3.1 rule): one F32 value per rotary pair.  The reference's import
+  // never reads this tensor and rotates such a file with the plain frequencies; a caller that wants exactly that resets the
+  // divisors to 1 after loading (cai_decoder_set_rope_freq_factors).
   std::vector<float> rope_factors;
   if (const TensorInfo* rf = find_tensor(g, "rope_freqs.weight")) {
     if (rf->ggml_type != CAI_F32 || rf->n_dims != 1 || rf->shape[0] != hd / 2)

@@ -252,6 +252,7 @@ int kv_fork(cai_kv_s* kv, int src, int dst);
 // (a captured graph holds its launch geometry, so the decoder keeps one graph per bucket); kv_bucket_rows gives the bucket's
 // upper bound for a needed row count (max_ctx for the last one), kv_geometry the slice length and count for it.
 int kv_bucket_rows(const cai_kv_s* kv, int needed_rows);
+bool attn_prompt_is_flash(const cai_kv_s* kv, int n);
 void kv_geometry(const cai_kv_s* kv, int rows, int* split_len, int* n_splits);
 // multi-token linear layer (matrix cores for Q4_K, small-batch kernel otherwise); gain != null fuses RMSNorm
 int prefill_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok,

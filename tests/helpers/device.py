@@ -7,6 +7,11 @@ ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# torch first: it brings its own copy of the HIP runtime, and a process that has started the system's copy through the
+# product library before torch's is loaded finds no device from torch afterwards (tests that make weights with torch on
+# the device would then depend on which test file ran first)
+import torch  # noqa: E402,F401
+
 pkg = importlib.import_module("neural-api_amd")
 cai = importlib.import_module("neural-api_amd.caihip")
 _inited = False

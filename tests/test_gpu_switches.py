@@ -1,5 +1,5 @@
-"""The three environment switches the library reads select other code paths (no stream capture; token-by-token prompts;
-prompt attention through the decode kernels).  Each is read once per process, so each case runs in a child process with the
+"""The environment switches the library reads select other code paths (no stream capture; token-by-token prompts;
+prompt attention through the decode kernels, and the bound of its partial-result buffer).  Each is read once per process, so each case runs in a child process with the
 variable set and is checked against the oracle there: a Q4_K decoder with QKV bias and 7 query heads per KV head, a 40-token
 prompt through cai_decoder_prefill, then 8 greedy tokens through cai_decoder_generate, a window step and the lookup loop."""
 import os
@@ -45,9 +45,12 @@ print("CHILD_OK")
 """
 
 
-@pytest.mark.parametrize("var,val", [("CAIHIP_NO_GRAPH", "1"), ("CAIHIP_PREFILL_TOKENWISE", "1"), ("CAIHIP_PROMPT_FLASH", "0")])
-def test_switch_selected_path_matches_the_oracle(var, val):
-    env = dict(os.environ); env[var] = val
+@pytest.mark.parametrize("switches", [{"CAIHIP_NO_GRAPH": "1"}, {"CAIHIP_PREFILL_TOKENWISE": "1"}, {"CAIHIP_PROMPT_FLASH": "0"},
+                                      # prompt attention on the decode kernels with room for 4 rows' partial results per launch
+                                      # (14 heads x 1 slice x 130 floats a row): the 40-token prompt attends in 10 groups
+                                      {"CAIHIP_PROMPT_FLASH": "0", "CAIHIP_PROMPT_PART_KB": "32"}])
+def test_switch_selected_path_matches_the_oracle(switches):
+    env = dict(os.environ); env.update(switches)
     code = CHILD % dict(root=ROOT, tests=os.path.join(ROOT, "tests"))
     r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0 and "CHILD_OK" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
@@ -90,4 +93,40 @@ def test_shutdown_frees_the_workspaces_and_a_second_init_runs_the_same():
     every result is bit-identical to the first session's."""
     code = SHUTDOWN_CHILD % dict(root=ROOT, tests=os.path.join(ROOT, "tests"))
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "CHILD_OK" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
+
+
+LATE_PROMPT_CHILD = r"""
+import sys, importlib
+import numpy as np
+sys.path.insert(0, %(root)r); sys.path.insert(0, %(tests)r)
+from helpers import oracle_lib as O
+from helpers.model_build import synthetic_spec
+from helpers.device import dev, rel_err
+cai = dev()
+cfg = dict(n_layers=1, d_model=128, n_q_heads=2, n_kv_heads=1, head_dim=64, ffn=256, vocab=512, max_ctx=36864, eps=1e-5, rope_theta=1e4)
+spec = synthetic_spec(cfg, O.Q8_0, head_qtype=O.Q8_0, std=0.08)
+dec = cai.Decoder(spec)
+toks = np.random.default_rng(11).integers(0, cfg["vocab"], 33000).tolist()
+head, tail = toks[:-96], toks[-96:]
+dec.prefill(head, 0)
+tok_a, la = dec.prefill(tail, len(head))          # 288 slices x 2 heads x 66 floats = 152 KB a row: groups of 13 rows under the 2 MB bound
+dec.truncate(len(head))
+for i, t in enumerate(tail):
+    am, lb = dec.step(t, len(head) + i)
+assert rel_err(la, lb[0]) < 1e-4, rel_err(la, lb[0])
+assert tok_a == int(am[0])
+print("CHILD_OK")
+"""
+
+
+def test_prompt_late_in_a_long_cache_on_the_decode_kernels_attends_in_bounded_groups():
+    """A head_dim-64 model (its prompts attend through the decode kernels) with a 36864-row cache: 96 prompt tokens at position
+    32904 need 288 slices of partial results per row and head; with the buffer bounded to 2 MB they attend in groups of 13 rows.
+    The result equals stepping the same 96 tokens one at a time (the reference's own prompt order,
+    neural/neuralchatengine.pas:1466-1470; that path is compared with the oracle elsewhere - the oracle itself would need
+    minutes for 33000 positions)."""
+    env = dict(os.environ); env["CAIHIP_PROMPT_PART_KB"] = "2048"
+    code = LATE_PROMPT_CHILD % dict(root=ROOT, tests=os.path.join(ROOT, "tests"))
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0 and "CHILD_OK" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
