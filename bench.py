@@ -401,7 +401,9 @@ def main():
     if W > 0:
         tok = decode(tok, pos, W); pos += W
     if args.step_timeline:
-        step_timeline(dec, tok, np)
+        if B > 1:
+            os.environ["CAIHIP_TL_BATCH"] = str(B)      # (read by the stamped build: the step of all B sequences)
+        step_timeline(dec, int(np.asarray(tok).ravel()[0]), np)
         return
     # K steps, timed `reps` times from the same position (the cache is cut back in between); the median repetition is reported
     walls, evs = [], []

@@ -115,7 +115,7 @@ extern "C" int cai_shutdown(void)
   if (c.stage_in) (void)hipFree(c.stage_in);
   if (c.stage_out) (void)hipFree(c.stage_out);
   if (c.stage_sample) (void)hipFree(c.stage_sample);
-  nb_release(); prefill_release();
+  nb_release(); ra_release(); prefill_release();
   if (c.d_small) (void)hipFree(c.d_small);
   if (c.h_small) (void)hipHostFree(c.h_small);
   if (c.tl.buf) (void)hipFree(c.tl.buf);

@@ -144,8 +144,37 @@ static int enqueue_step(cai_decoder_s* d, int n_b, int seq0, unsigned classes = 
     for (int sl : slots) if (!nb_supported(L.w[sl]) || L.w[sl]->qtype == CAI_I8ROW) return false;   // (per-row int8 products need the plain reduction for their row scale)
     return true;
   };
+  // ... and when all six are Q4_K of widths the register-resident form takes, a linear layer is ONE launch: activations
+  // quantised by the product itself, norm factor, bias, residual and SwiGLU in its epilogue (CAIHIP_SMALL_BATCH_PLANES=1
+  // keeps the form with activation planes and slice partials)
+  static const bool ra_on = []() { const char* e = getenv("CAIHIP_SMALL_BATCH_PLANES"); return !(e && e[0] == '1'); }();
+  auto ra_layer = [&](const cai_decoder_s::Layer& L) {
+    if (!ra_on || n_b < 2 || n_b > 8 || c.n_experts > 0) return false;
+    const cai_qw_s* qkv3[3] = {L.w[CAI_W_Q], L.w[CAI_W_K], L.w[CAI_W_V]};
+    const cai_qw_s* wo = L.w[CAI_W_O]; const cai_qw_s* wgu = L.w[CAI_W_GATEUP]; const cai_qw_s* wdn = L.w[CAI_W_DOWN];
+    return ra_supported(qkv3, 3, true, 0) && ra_supported(&wo, 1, false, 0) && ra_supported(&wgu, 1, true, I) && ra_supported(&wdn, 1, false, 0);
+  };
   for (int l = 0; l < c.n_layers; l++) {
     auto& L = d->layers[l];
+    if (ra_layer(L)) {
+      if (down_pending) { if ((rc = nb_prep_residual(d->x, dm, nullptr, 0.0f, dm, n_b))) return rc; down_pending = false; }
+      const cai_qw_s* qkv3[3] = {L.w[CAI_W_Q], L.w[CAI_W_K], L.w[CAI_W_V]}; const int off3[3] = {0, qw, qw + kw};
+      tl_cls = 1;
+      if ((rc = ra_gemm(qkv3, off3, 3, n_b, d->x, dm, L.v[CAI_V_ATTN_NORM], c.eps, 0, d->qkv, qkvw, nullptr))) return rc;
+      tl_cls = 2;
+      if ((rc = launch_attn_step(&d->kv, l, d->qkv, qkvw, n_b, c.n_q_heads, c.window, 0.0f, d->theta, d->d_pos, d->att, qw, seq0, window ? 2 : 0, window ? d->wpart : nullptr,
+                                 c.qk_norm_full ? L.v[CAI_V_Q_NORM] : nullptr, c.qk_norm_full ? L.v[CAI_V_K_NORM] : nullptr, c.eps))) return rc;
+      const int zero = 0;
+      const cai_qw_s* wo = L.w[CAI_W_O]; const cai_qw_s* wgu = L.w[CAI_W_GATEUP]; const cai_qw_s* wdn = L.w[CAI_W_DOWN];
+      tl_cls = 3;
+      if ((rc = ra_gemm(&wo, &zero, 1, n_b, d->att, qw, nullptr, 0.0f, 0, d->x, dm, d->x))) return rc;
+      tl_cls = 4;
+      if ((rc = ra_gemm(&wgu, &zero, 1, n_b, d->x, dm, L.v[CAI_V_MLP_NORM], c.eps, I, d->mid, I, nullptr))) return rc;
+      tl_cls = 5;
+      if ((rc = ra_gemm(&wdn, &zero, 1, n_b, d->mid, I, nullptr, 0.0f, 0, d->x, dm, d->x))) return rc;
+      have_ssq_d = false;
+      continue;
+    }
     if (mma_layer(L)) {
       // the down product of the previous block is still in slices: the pre-pass adds it to the residual stream
       if (down_pending) rc = nb_prep_residual(d->x, dm, L.v[CAI_V_ATTN_NORM], c.eps, dm, n_b);
@@ -431,8 +460,10 @@ static int run_step(cai_decoder_s* d, int n_b, int rows_needed, bool window = fa
     size_t part = std::max(std::max((size_t)nb_max_slices(dm) * al4(qkvw), (size_t)nb_max_slices(d->qw()) * al4(dm)),
                            std::max((size_t)nb_max_slices(dm) * al4(2 * (int64_t)cf.ffn), (size_t)nb_max_slices(cf.ffn) * al4(dm)));
     part = std::max(part, (size_t)nb_max_slices(dm) * al4(cf.vocab)) * 8;
-    const int rc = nb_reserve(kmax, part); if (rc) return rc;
-    if (d->ws_generation != nb_ws_generation()) { invalidate_graphs(d); d->ws_generation = nb_ws_generation(); }
+    int rc = nb_reserve(kmax, part); if (rc) return rc;
+    if ((rc = ra_reserve(std::max(ra_part_floats(dm, cf.ffn), ra_part_floats(dm, d->qw()))))) return rc;   // (the sliced products: down and o)
+    const int gen = nb_ws_generation() + ra_ws_generation();      // (both only ever grow)
+    if (d->ws_generation != gen) { invalidate_graphs(d); d->ws_generation = gen; }
   }
   const int bucket = kv_bucket_rows(&d->kv, rows_needed);
   d->kv.geo_rows = bucket;
@@ -885,14 +916,18 @@ extern "C" int cai_decoder_timeline(cai_decoder_t d, int32_t token, uint64_t* st
     CAI_HIP(hipMalloc((void**)&tl.buf, (size_t)stamps_cap * sizeof(unsigned long long)));
     tl.cap = (size_t)stamps_cap;
   }
-  d->h_io[0] = token; d->h_io[8] = pos;
+  // (CAIHIP_TL_BATCH = b: the step of sequences 0 .. b - 1, each at its own position, all fed `token`)
+  const char* tb = getenv("CAIHIP_TL_BATCH");
+  const int n_b = tb ? std::max(1, std::min(atoi(tb), std::min(c.max_batch, 8))) : 1;
+  int rows_needed = pos + 1;
+  for (int b = 0; b < n_b; b++) { d->h_io[b] = token; d->h_io[8 + b] = d->kv.len_at(b, 0); rows_needed = std::max(rows_needed, d->kv.len_at(b, 0) + 1); }
   CAI_HIP(hipMemcpyAsync(d->d_tokens, d->h_io, 16 * sizeof(int32_t), hipMemcpyHostToDevice, cx.stream));
-  d->kv.geo_rows = kv_bucket_rows(&d->kv, pos + 1);
+  d->kv.geo_rows = kv_bucket_rows(&d->kv, rows_needed);
   tl.used = 0; tl.launches.clear(); tl.armed = true;
   hipGraph_t g = nullptr; hipGraphExec_t ge = nullptr;
   hipError_t e = hipStreamBeginCapture(cx.stream, hipStreamCaptureModeThreadLocal);
   if (e != hipSuccess) { tl.armed = false; return hip_fail(e, "hipStreamBeginCapture", __FILE__, __LINE__); }
-  rc = enqueue_step(d, 1, 0);
+  rc = enqueue_step(d, n_b, 0);
   tl.armed = false;
   e = hipStreamEndCapture(cx.stream, &g);
   if (rc) { if (g) (void)hipGraphDestroy(g); return rc; }

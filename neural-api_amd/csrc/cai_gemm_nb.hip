@@ -70,8 +70,11 @@ __device__ __forceinline__ half8_t nibbles_times_scale(uint32_t lo, uint32_t hi,
 
 // v_mfma_f32_16x16x32_f16: lane (m = lane % 16, kg = lane / 16) supplies 8 consecutive k of row m (A) / column m (B);
 // the 16 x 16 result has rows 4 kg .. 4 kg + 3 of column m in this lane.  Here a tile is 32 weight rows = two row sets,
-// the 16 columns are 8 tokens x {hi, lo}, and lane kg owns quant bytes 32 kg .. 32 kg + 31 of a super-block: sub-block
-// 2 kg in the low nibbles (k steps 0..3), sub-block 2 kg + 1 in the high nibbles (steps 4..7).
+// the 16 columns are 8 tokens x {hi, lo}.  The order of k inside a super-block is free (both operands follow it), so it is
+// chosen for the requests: the four kg lanes of a row ask for 64 CONTIGUOUS quant bytes per request (bytes 16 kg .. + 15,
+// then 64 + 16 kg .. + 15), which touches each 64-byte sector of the 144-byte blocks once per request; with 32 contiguous
+// bytes per lane every request touched the pieces of all sectors of a block.  Lane kg therefore owns weights
+// 16 (kg & 1) .. + 15 of sub-blocks 2 g, 2 g + 1 (low, high nibbles) for g = kg / 2 and for g = 2 + kg / 2.
 // QT = CAI_Q5_K: the same walk over 176-byte super-blocks (neural/neuralgguf.pas:516-587): header as Q4_K, then the 32-byte plane of
 // fifth bits (bit j of byte i belongs to weight i of sub-block j), then the nibbles; sc * (nibble | bit << 4) <= 63 * 31 stays exact in f16.
 template <int QT>
@@ -111,8 +114,8 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const _Float16* hxhi, cons
     for (int hh = 0; hh < 2; hh++) {
       const uint8_t* blk = sg->w + (int64_t)min(R0 + 16 * hh + n, sg->rows - 1) * row_bytes + (int64_t)sb * BB;   // tail rows: re-read the last row
       r.h[hh] = *reinterpret_cast<const uint4*>(blk);
-      r.q[hh][0] = *reinterpret_cast<const uint4*>(blk + QOFF + 32 * kg);
-      r.q[hh][1] = *reinterpret_cast<const uint4*>(blk + QOFF + 16 + 32 * kg);
+      r.q[hh][0] = *reinterpret_cast<const uint4*>(blk + QOFF + 16 * kg);
+      r.q[hh][1] = *reinterpret_cast<const uint4*>(blk + QOFF + 64 + 16 * kg);
       if constexpr (QT == CAI_Q5_K) { r.e[hh][0] = *reinterpret_cast<const uint4*>(blk + 16); r.e[hh][1] = *reinterpret_cast<const uint4*>(blk + 32); }
     }
   };
@@ -168,20 +171,25 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const _Float16* hxhi, cons
         for (int i = 0; i < 4; i++) acc[hh][i] = 0.0f;
     }
     float4_t C[2], Cm[2];
-    half2_t s2[2][2], c2[2][2];
+    half2_t s2[2][4], c2[2][4];
 #pragma unroll
     for (int hh = 0; hh < 2; hh++) {
       // 6-bit scales / mins (neural/neuralgguf.pas:448-464), one per byte: sub-blocks 0..3 and 4..7; this lane's two
       const uint4 h = r.h[hh];
       const uint32_t sc_lo = h.y & 0x3f3f3f3fu, sc_hi = (h.w & 0x0f0f0f0fu) | ((h.y >> 2) & 0x30303030u);
       const uint32_t mn_lo = h.z & 0x3f3f3f3fu, mn_hi = ((h.w >> 4) & 0x0f0f0f0fu) | ((h.z >> 2) & 0x30303030u);
-      const uint32_t scp = ((kg & 2) ? sc_hi : sc_lo) >> (16 * (kg & 1));     // bytes 0, 1 = sc of sub-blocks 2kg, 2kg+1
+      // the lane's quant bytes are those of byte groups kg / 2 (first request) and 2 + kg / 2 (second): sub-blocks
+      // 2 (kg / 2), + 1 (low, high nibbles) and 4 + 2 (kg / 2), + 1; the min term below keeps sub-blocks 2 kg, 2 kg + 1
+      const uint32_t scq[2] = {sc_lo >> (16 * (kg >> 1)), sc_hi >> (16 * (kg >> 1))};
       const uint32_t mnp = ((kg & 2) ? mn_hi : mn_lo) >> (16 * (kg & 1));
-      const half2_t sch = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, scp, 0x04010400u)) - half2_t{k1024, k1024};
       const half2_t mnh = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, mnp, 0x04010400u)) - half2_t{k1024, k1024};
-      s2[hh][0] = half2_t{sch.x, sch.x}; s2[hh][1] = half2_t{sch.y, sch.y};
-      c2[hh][0] = half2_t{(_Float16)(-1024.0f) * sch.x, (_Float16)(-1024.0f) * sch.x};   // exact: a multiple of 1024 below 65504
-      c2[hh][1] = half2_t{(_Float16)(-1024.0f) * sch.y, (_Float16)(-1024.0f) * sch.y};
+#pragma unroll
+      for (int c = 0; c < 2; c++) {
+        const half2_t sch = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, scq[c], 0x04010400u)) - half2_t{k1024, k1024};
+        s2[hh][2 * c] = half2_t{sch.x, sch.x}; s2[hh][2 * c + 1] = half2_t{sch.y, sch.y};
+        c2[hh][2 * c] = half2_t{(_Float16)(-1024.0f) * sch.x, (_Float16)(-1024.0f) * sch.x};   // exact: a multiple of 1024 below 65504
+        c2[hh][2 * c + 1] = half2_t{(_Float16)(-1024.0f) * sch.y, (_Float16)(-1024.0f) * sch.y};
+      }
       if (kg == 0) {
         const float d = __half2float(__ushort_as_half((unsigned short)(h.x & 0xffffu)));
         const float dmin = __half2float(__ushort_as_half((unsigned short)(h.x >> 16)));
@@ -194,23 +202,30 @@ __global__ __launch_bounds__(256, 2) void gemm_q4k_nb(const _Float16* hxhi, cons
       Cm[hh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Am, Bm, z4, 0, 0, 0);
       C[hh] = z4;
     }
-    const _Float16* xcol = xs + (s * NB_SC + n) * NB_LDX + 64 * kg;
+    // step t = 4 c + 2 nib + j: request c, low or high nibbles, bytes 8 j .. 8 j + 7 of the lane's 16 = weights
+    // 16 (kg & 1) + 8 j .. + 7 of sub-block 2 (kg / 2 + 2 c) + nib
+    const _Float16* xcol = xs + (s * NB_SC + n) * NB_LDX + 64 * (kg >> 1) + 16 * (kg & 1);
+    uint4 ee[2];
+    if constexpr (QT == CAI_Q5_K) {
+#pragma unroll
+      for (int hh = 0; hh < 2; hh++) ee[hh] = (kg & 1) ? r.e[hh][1] : r.e[hh][0];   // plane bytes 16 (kg & 1) .. + 15
+    }
 #pragma unroll
     for (int t = 0; t < 8; t++) {
-      const half8_t B = *reinterpret_cast<const half8_t*>(xcol + 8 * t);
+      const int c = t >> 2, nib = (t >> 1) & 1, j = t & 1;
+      const half8_t B = *reinterpret_cast<const half8_t*>(xcol + 128 * c + 32 * nib + 8 * j);
 #pragma unroll
       for (int hh = 0; hh < 2; hh++) {
-        const uint4& qq = r.q[hh][(t & 3) >> 1];
-        const uint32_t d0 = (t & 1) ? qq.z : qq.x, d1 = (t & 1) ? qq.w : qq.y;       // bytes 8 (t & 3) .. + 7
-        uint32_t lo = (t < 4) ? (d0 & 0x0f0f0f0fu) : ((d0 >> 4) & 0x0f0f0f0fu);
-        uint32_t hi = (t < 4) ? (d1 & 0x0f0f0f0fu) : ((d1 >> 4) & 0x0f0f0f0fu);
-        if constexpr (QT == CAI_Q5_K) {   // plane bytes 8 (t & 3) .. + 7, bit 2 kg (low nibbles' sub-block) or 2 kg + 1
-          const uint4& ee = r.e[hh][(t & 3) >> 1];
-          const uint32_t e0 = (t & 1) ? ee.z : ee.x, e1 = (t & 1) ? ee.w : ee.y;
-          const int bit = 2 * kg + (t >> 2);
+        const uint4& qq = r.q[hh][c];
+        const uint32_t d0 = j ? qq.z : qq.x, d1 = j ? qq.w : qq.y;
+        uint32_t lo = nib ? ((d0 >> 4) & 0x0f0f0f0fu) : (d0 & 0x0f0f0f0fu);
+        uint32_t hi = nib ? ((d1 >> 4) & 0x0f0f0f0fu) : (d1 & 0x0f0f0f0fu);
+        if constexpr (QT == CAI_Q5_K) {   // bit (sub-block) of the plane bytes of these weights
+          const uint32_t e0 = j ? ee[hh].z : ee[hh].x, e1 = j ? ee[hh].w : ee[hh].y;
+          const int bit = 2 * ((kg >> 1) + 2 * c) + nib;
           lo |= ((e0 >> bit) & 0x01010101u) << 4; hi |= ((e1 >> bit) & 0x01010101u) << 4;
         }
-        const half8_t A = nibbles_times_scale(lo, hi, s2[hh][t >> 2], c2[hh][t >> 2]);
+        const half8_t A = nibbles_times_scale(lo, hi, s2[hh][2 * c + nib], c2[hh][2 * c + nib]);
         C[hh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, C[hh], 0, 0, 0);
       }
     }

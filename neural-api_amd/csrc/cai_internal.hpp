@@ -275,6 +275,14 @@ int nb_ws_generation();                                        // changes whenev
 void nb_release();                                             // frees the small-batch workspace (cai_shutdown)
 void prefill_release();                                        // frees the prompt workspace (cai_shutdown)
 int nb_reserve(int k_max, size_t part_floats);                 // never inside a stream capture
+// small-batch Q4_K products with the activations held in registers (cai_gemm_ra.hip): one launch per linear layer
+bool ra_supported(const cai_qw_s* const* ws, int n_w, bool normed, int swiglu_half);
+size_t ra_part_floats(int64_t rows, int64_t cols);
+int ra_reserve(size_t part_floats);                            // never inside a stream capture
+int ra_ws_generation();
+void ra_release();
+int ra_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, const float* x, int64_t x_stride, const float* gain, float eps,
+            int swiglu_half, float* y, int64_t y_stride, const float* residual);
 int nb_max_slices(int cols);
 int nb_prep_plain(const float* x, int64_t x_stride, const float* gain, float eps, int K, int n_tok);
 int nb_prep_residual(float* res, int64_t res_stride, const float* gain, float eps, int K, int n_tok);   // res += last product
