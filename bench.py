@@ -272,7 +272,7 @@ def step_timeline(dec, tok, np):
                      count=nm(s[:, 6] - s[:, 5]), merge=float(np.nanmax(s[:, 7] - s[:, 6])))
         else:
             r.update(issue=nm(s[:, 1] - s[:, 0]), arrive=nm(s[:, 2] - s[:, 1]), quant=nm(s[:, 3] - s[:, 2]), lift=nm(s[:, 4] - s[:, 3]),
-                     count=float("nan"), merge=float("nan"))
+                     count=nm(s[:, 6] - s[:, 4]), merge=float("nan"))
         rows.append(r); prev_end = end
     print("one captured decode step, %d instrumented launches, %.1f us from the first entry to the last exit" % (len(rows), rows[-1]["start"] + rows[-1]["span"] - rows[0]["start"]))
     cols = ("gap", "skew", "issue", "arrive", "quant", "lift", "stage", "loop", "tail", "loop_max", "tail_max", "count", "merge", "span")

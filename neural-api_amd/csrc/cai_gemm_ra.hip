@@ -101,6 +101,9 @@ __device__ __forceinline__ uint32_t ra_ror8(uint32_t v) { return (uint32_t)__bui
 // the 8 of them at 8 j (in the order 0, 2, 1, 3, 4, 6, 5, 7: see ra_weights).  For the min term lane kg stands for the two sub-blocks 2 g + 4 c1, + 1 (each lane pair kg, kg ^ 1
 // holds the halves of four sub-blocks' activations, so their sums are one exchange away).
 // (what the first requests need travels as leading scalar arguments, preloaded in scalar registers)
+// HH: 16-row sets per unit of rows (2: pairs - what SwiGLU needs and what long walks take; 1 halves the unit, for products
+// with fewer pairs than compute units or an uneven number per work-group).  GAIN: the activations carry an RMSNorm gain.
+template <int HH, bool GAIN>
 __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, const long long hstride, const float* hgain, const int hcols, const int hntok,
                                                           const int hnpairs, const int hS, const RaParams p)
 {
@@ -133,10 +136,10 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
     if (p.n_seg > 2 && pair >= p.seg[1].pair_end) { sgi = 2; t0 = p.seg[1].pair_end; }
     sg = &p.seg[sgi];
     if (p.swiglu_half > 0) { r0 = 16 * pair; r1 = p.swiglu_half + 16 * pair; }
-    else { r0 = (pair - t0) * 32; r1 = r0 + 16; }
+    else { r0 = (pair - t0) * 16 * HH; r1 = r0 + 16; }
   };
 
-  struct WRegs { uint4 h[2], q[2][2]; };
+  struct WRegs { uint4 h[HH], q[HH][2]; };
   // weights of item q = (pair q / 2, super-block q % 2 of this wave): for the rows n of both row sets the header and this
   // lane's 2 x 16 quant bytes.  Loads are never conditional: past the last item the last one is fetched again (a cache hit).
   auto load_w = [&](int q, WRegs& r) __attribute__((always_inline)) {
@@ -144,7 +147,7 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
     const int pair = min((int)blockIdx.x + (qc >> 1) * (int)gridDim.x, hnpairs - 1), sb = sbw0 + min(qc & 1, max(nsw, 1) - 1);
     const RaSeg* sg; int r0, r1; locate(pair, sg, r0, r1);
 #pragma unroll
-    for (int hh = 0; hh < 2; hh++) {
+    for (int hh = 0; hh < HH; hh++) {
       const uint8_t* blk = sg->w + (int64_t)min((hh ? r1 : r0) + n, sg->rows - 1) * row_bytes + (int64_t)sb * RA_BB;   // tail rows: re-read the last row
       r.h[hh] = *reinterpret_cast<const uint4*>(blk);
       r.q[hh][0] = *reinterpret_cast<const uint4*>(blk + 16 + 16 * kg);
@@ -174,7 +177,7 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
   float4 gr[RA_SBW][4];
 #pragma unroll
   for (int j = 0; j < RA_SBW; j++) {
-    const float* pg = (hgain ? hgain : hsrc) + (int64_t)(sbw0 + min(j, max(nsw, 1) - 1)) * 256 + 4 * ii;    // (no gain: any readable address, the values are not used)
+    const float* pg = (GAIN ? hgain : hsrc) + (int64_t)(sbw0 + min(j, max(nsw, 1) - 1)) * 256 + 4 * ii;    // (no gain: any readable address, the values are not used)
 #pragma unroll
     for (int m = 0; m < 4; m++) gr[j][m] = *reinterpret_cast<const float4*>(pg + 64 * m);
   }
@@ -193,7 +196,7 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
         const float4 a = xr[j][hq][m], gq = gr[j][m];
         const float raw[4] = {a.x, a.y, a.z, a.w}, gg[4] = {gq.x, gq.y, gq.z, gq.w};
 #pragma unroll
-        for (int u = 0; u < 4; u++) { v[m][u] = hgain ? raw[u] * gg[u] : raw[u]; amax = fmaxf(amax, fabsf(v[m][u])); ss = fmaf(raw[u], raw[u], ss); }
+        for (int u = 0; u < 4; u++) { v[m][u] = GAIN ? raw[u] * gg[u] : raw[u]; amax = fmaxf(amax, fabsf(v[m][u])); ss = fmaf(raw[u], raw[u], ss); }
       }
       amax = ra_row_max(amax); ss = ra_row_sum(ss);
       if (j == 0 && hq == 0) timeline_stamp_after(p.timeline, 2, amax);
@@ -243,12 +246,12 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
   timeline_stamp(p.timeline, 4);
   // what the finishing wave of a pair adds to the rows (bias, residual) is requested when the pair starts: by every wave, so
   // that the requests stay unconditional (a kilobyte per wave and pair), and from a harmless address when there is none
-  struct Extra { float4 bias[2], res[2]; };
+  struct Extra { float4 bias[HH], res[HH]; };
   auto prefetch = [&](int i, Extra& f) __attribute__((always_inline)) {
     const int pair = min((int)blockIdx.x + min(i, max(npw, 1) - 1) * (int)gridDim.x, hnpairs - 1);
     const RaSeg* sg; int r0, r1; locate(pair, sg, r0, r1);
 #pragma unroll
-    for (int hh = 0; hh < 2; hh++) {
+    for (int hh = 0; hh < HH; hh++) {
       const int row = (hh ? r1 : r0) + 4 * kg;
       const float* bp = sg->bias ? sg->bias + row : reinterpret_cast<const float*>(sg->w);
       const float* rp = p.residual ? p.residual + (int64_t)tokc * p.y_stride + sg->y_off + row : p.y;
@@ -257,7 +260,7 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
     }
   };
   Extra ea, eb;
-  float acc[2][4];
+  float acc[HH][4];
   const _Float16 k1024 = (_Float16)1024.0f, kz = (_Float16)0.0f;
   uint32_t kreg = 0x64006400u;                 // 1024.0 twice, kept in a register the compiler cannot fold (see ra_weights)
   asm volatile("" : "+v"(kreg));
@@ -265,15 +268,15 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
   auto compute = [&](const WRegs& r, const int j) __attribute__((always_inline)) {
     if (j == 0) {
 #pragma unroll
-      for (int hh = 0; hh < 2; hh++)
+      for (int hh = 0; hh < HH; hh++)
 #pragma unroll
         for (int i = 0; i < 4; i++) acc[hh][i] = 0.0f;
     }
     if (j >= nsw) return;
-    float4_t C[2], Cm[2];
-    half2_t s2[2][4], c2[2][4];
+    float4_t C[HH], Cm[HH];
+    half2_t s2[HH][4], c2[HH][4];
 #pragma unroll
-    for (int hh = 0; hh < 2; hh++) {
+    for (int hh = 0; hh < HH; hh++) {
       // 6-bit scales / mins (neural/neuralgguf.pas:448-464), one per byte: sub-blocks 0..3 and 4..7
       const uint4 h = r.h[hh];
       const uint32_t sc_lo = h.y & 0x3f3f3f3fu, sc_hi = (h.w & 0x0f0f0f0fu) | ((h.y >> 2) & 0x30303030u);
@@ -304,7 +307,7 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
     for (int t = 0; t < 8; t++) {
       const int c = t >> 2, nib = (t >> 1) & 1, jj = t & 1;      // request, nibble, dword pair
 #pragma unroll
-      for (int hh = 0; hh < 2; hh++) {
+      for (int hh = 0; hh < HH; hh++) {
         const uint4& qq = r.q[hh][c];
         const uint32_t d0 = jj ? qq.z : qq.x, d1 = jj ? qq.w : qq.y;
         const half8_t A = nib ? ra_weights<true>(d0, d1, s2[hh][2 * c + 1], c2[hh][2 * c + 1], kreg) : ra_weights<false>(d0, d1, s2[hh][2 * c], c2[hh][2 * c], kreg);
@@ -313,7 +316,7 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
     }
     __builtin_amdgcn_wave_barrier();   // s_d was written by this wave's own lanes above; LDS operations of a wave complete in order
 #pragma unroll
-    for (int hh = 0; hh < 2; hh++) {
+    for (int hh = 0; hh < HH; hh++) {
       const float4 d4 = *reinterpret_cast<const float4*>(&s_d[wave][0][16 * hh + 4 * kg]);
       const float4 m4 = *reinterpret_cast<const float4*>(&s_d[wave][1][16 * hh + 4 * kg]);
       acc[hh][0] += sinv[j] * (d4.x * C[hh][0] - m4.x * Cm[hh][0]);
@@ -328,15 +331,15 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
   auto pair_end = [&](int i, const Extra& f) __attribute__((always_inline)) {
     const int slot = i & 1;
     if (nsw > 0) {
-      float tot[8];
+      float tot[4 * HH];
 #pragma unroll
-      for (int hh = 0; hh < 2; hh++)
+      for (int hh = 0; hh < HH; hh++)
 #pragma unroll
         for (int k = 0; k < 4; k++) tot[4 * hh + k] = acc[hh][k] + ra_ror8(acc[hh][k]);
       if (!lo_col) {
         float* dst = reinterpret_cast<float*>(wl) + (slot * 32 + kg * 8 + n) * 8;
         *reinterpret_cast<float4*>(dst) = make_float4(tot[0], tot[1], tot[2], tot[3]);
-        *reinterpret_cast<float4*>(dst + 4) = make_float4(tot[4], tot[5], tot[6], tot[7]);
+        if constexpr (HH == 2) *reinterpret_cast<float4*>(dst + 4) = make_float4(tot[4], tot[5], tot[6], tot[7]);
       }
     }
     __syncthreads();     // (the slot is written again two pairs on: after the next barrier, which the finishing wave reaches after its reads)
@@ -344,21 +347,22 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
     float t8[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     for (int w = 0; w < nwa; w++) {       // wave order: fixed
       const float* src = reinterpret_cast<const float*>(ra_dyn + (size_t)w * RA_WAVE_LDS) + (slot * 32 + kg * 8 + n) * 8;
-      const float4 a = *reinterpret_cast<const float4*>(src), b = *reinterpret_cast<const float4*>(src + 4);
-      t8[0] += a.x; t8[1] += a.y; t8[2] += a.z; t8[3] += a.w; t8[4] += b.x; t8[5] += b.y; t8[6] += b.z; t8[7] += b.w;
+      const float4 a = *reinterpret_cast<const float4*>(src);
+      t8[0] += a.x; t8[1] += a.y; t8[2] += a.z; t8[3] += a.w;
+      if constexpr (HH == 2) { const float4 b = *reinterpret_cast<const float4*>(src + 4); t8[4] += b.x; t8[5] += b.y; t8[6] += b.z; t8[7] += b.w; }
     }
     if (!tok_on) return;
     float inv = 1.0f;
-    if (hgain) {   // (a product with a gain is one slice: the work-group has seen the whole row; every wave has passed this pair's barrier)
+    if (GAIN) {   // (a product with a gain is one slice: the work-group has seen the whole row; every wave has passed this pair's barrier)
       float t = 0.0f;
       for (int sb = 0; sb < nS; sb++) t += ssq_s[sb][tok];     // fixed order
       inv = 1.0f / sqrtf(t / (float)K + p.eps);
     }
     const int pair = (int)blockIdx.x + i * (int)gridDim.x;
     const RaSeg* sg; int r0, r1; locate(pair, sg, r0, r1);
-    if (p.swiglu_half > 0) {
+    if (HH == 2 && p.swiglu_half > 0) {
       const int col = 16 * pair + 4 * kg;       // rows r0 + 4 kg .. + 3 (up) and r1 + 4 kg .. + 3 (gate)
-      const float bu[4] = {f.bias[0].x, f.bias[0].y, f.bias[0].z, f.bias[0].w}, bg[4] = {f.bias[1].x, f.bias[1].y, f.bias[1].z, f.bias[1].w};
+      const float bu[4] = {f.bias[0].x, f.bias[0].y, f.bias[0].z, f.bias[0].w}, bg[4] = {f.bias[HH - 1].x, f.bias[HH - 1].y, f.bias[HH - 1].z, f.bias[HH - 1].w};
       float o[4];
 #pragma unroll
       for (int k = 0; k < 4; k++) {
@@ -370,7 +374,7 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
       return;
     }
 #pragma unroll
-    for (int hh = 0; hh < 2; hh++) {
+    for (int hh = 0; hh < HH; hh++) {
       const int row = (hh ? r1 : r0) + 4 * kg;
       if (p.n_slices > 1) {
         float* dst = p.part + ((int64_t)slice * hntok + tok) * p.part_stride + sg->y_off + row;
@@ -394,6 +398,7 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
     prefetch(q >> 1, ea);
     load_w(q + 3, wd); compute(wa, 0);
     load_w(q + 4, wa); compute(wb, 1);
+    if (q == 0 && p.n_slices == 1) timeline_stamp_after(p.timeline, 6, acc[0][0]);
     pair_end(q >> 1, ea);
     prefetch((q >> 1) + 1, eb);
     load_w(q + 5, wb); if (q + 2 < nq) compute(wc, 0);      // (requests stay unconditional)
@@ -410,9 +415,9 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
     __syncthreads();
     timeline_stamp(p.timeline, 6);
     if (!s_is_last) { timeline_stamp(p.timeline, 7); return; }
-    const int total = npw * 32 * hntok;
+    const int total = npw * 16 * HH * hntok;
     for (int e = threadIdx.x; e < total; e += blockDim.x) {
-      const int r32 = e & 31, t = (e >> 5) % hntok, i = (e >> 5) / hntok;
+      const int r32 = e % (16 * HH), t = (e / (16 * HH)) % hntok, i = (e / (16 * HH)) / hntok;
       const RaSeg* sg; int r0, r1; locate((int)blockIdx.x + i * (int)gridDim.x, sg, r0, r1);
       const int row = r0 + r32;
       if (row >= sg->rows) continue;
@@ -503,14 +508,14 @@ size_t ra_part_floats(int64_t rows, int64_t cols)
   return (size_t)ns_max * RA_TK * (size_t)((rows + 3) / 4 * 4);
 }
 
-// Whether ra_gemm takes these matrices: Q4_K, one width of whole super-blocks, whole 16-row sets (32 for plain products),
+// Whether ra_gemm takes these matrices: Q4_K, one width of whole super-blocks, whole 16-row sets,
 // one column slice when the product carries an RMSNorm or SwiGLU.
 bool ra_supported(const cai_qw_s* const* ws, int n_w, bool normed, int swiglu_half)
 {
   if (n_w < 1 || n_w > 3 || (swiglu_half > 0 && n_w != 1)) return false;
   for (int i = 0; i < n_w; i++) {
     const cai_qw_s* w = ws[i];
-    if (w->qtype != CAI_Q4_K || w->cols != ws[0]->cols || w->cols % 256 || w->cols < 256 || w->rows % 32) return false;
+    if (w->qtype != CAI_Q4_K || w->cols != ws[0]->cols || w->cols % 256 || w->cols < 256 || w->rows % 16) return false;
   }
   if (swiglu_half > 0 && (ws[0]->rows != 2 * (int64_t)swiglu_half || swiglu_half % 16)) return false;
   const int nsb = (int)(ws[0]->cols >> 8);
@@ -532,17 +537,28 @@ int ra_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, con
     if ((y_off[i] & 3) || (ws[i]->bias && (reinterpret_cast<uintptr_t>(ws[i]->bias) & 15)))
       return set_error(CAI_ERR_INVALID, "small-batch product (register form): output offsets and biases must be 16-byte aligned");
   RaParams p{};
-  int pairs = 0; int64_t width = 0;
-  for (int i = 0; i < n_w; i++) {
-    pairs += swiglu_half > 0 ? swiglu_half / 16 : (int)(ws[i]->rows / 32);
-    p.seg[i] = RaSeg{ws[i]->data, ws[i]->bias, (int)ws[i]->rows, y_off[i], pairs};
-    width = std::max<int64_t>(width, y_off[i] + ws[i]->rows);
-  }
   p.n_seg = n_w; p.eps = eps; p.swiglu_half = swiglu_half; p.y = y; p.y_stride = y_stride; p.residual = residual;
   const int cols = (int)ws[0]->cols, nsb = cols >> 8;
-  int S = 0, n_slices = 0, gx = 0;
-  if (!ra_geometry(nsb, pairs, gain != nullptr || swiglu_half > 0, S, n_slices, gx))
-    return set_error(CAI_ERR_UNSUPPORTED, "small-batch product (register form): width %d", cols);
+  const bool one_slice = gain != nullptr || swiglu_half > 0;
+  // units of 32 rows (pairs of row sets), or of 16 where that shortens the longest walk (a wave takes 2 x HH items per unit)
+  int HH = 2, S = 0, n_slices = 0, gx = 0, units = 0;
+  {
+    int u2 = 0, u1 = 0;
+    for (int i = 0; i < n_w; i++) { u2 += swiglu_half > 0 ? swiglu_half / 16 : (int)(ws[i]->rows / 32); u1 += (int)(ws[i]->rows / 16); }
+    bool whole_pairs = true;
+    for (int i = 0; i < n_w; i++) whole_pairs = whole_pairs && ws[i]->rows % 32 == 0;
+    int S2 = 0, ns2 = 0, g2 = 0, S1 = 0, ns1 = 0, g1 = 0;
+    if (!ra_geometry(nsb, u2, one_slice, S2, ns2, g2) || !ra_geometry(nsb, u1, one_slice, S1, ns1, g1))
+      return set_error(CAI_ERR_UNSUPPORTED, "small-batch product (register form): width %d", cols);
+    units = u2; S = S2; n_slices = ns2; gx = g2;
+    if (swiglu_half == 0 && (!whole_pairs || (u1 + g1 - 1) / g1 < 2 * ((u2 + g2 - 1) / g2))) { HH = 1; units = u1; S = S1; n_slices = ns1; gx = g1; }
+  }
+  int cum = 0; int64_t width = 0;
+  for (int i = 0; i < n_w; i++) {
+    cum += swiglu_half > 0 ? swiglu_half / 16 : (int)(ws[i]->rows / (16 * HH));
+    p.seg[i] = RaSeg{ws[i]->data, ws[i]->bias, (int)ws[i]->rows, y_off[i], cum};
+    width = std::max<int64_t>(width, y_off[i] + ws[i]->rows);
+  }
   p.n_slices = n_slices;
   if (n_slices > 1) {
     p.part_stride = (width + 3) / 4 * 4;
@@ -552,9 +568,17 @@ int ra_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, con
   }
   const int nw = (S + RA_SBW - 1) / RA_SBW;
   p.timeline = timeline_next(gx * n_slices);
-  static bool attr_done = false;
-  if (!attr_done) { CAI_HIP(hipFuncSetAttribute((const void*)gemm_q4k_ra, hipFuncAttributeMaxDynamicSharedMemorySize, RA_NW * RA_WAVE_LDS)); attr_done = true; }
-  hipLaunchKernelGGL(gemm_q4k_ra, dim3(gx, n_slices), dim3(64 * nw), (size_t)nw * RA_WAVE_LDS, ctx().stream, x, (long long)x_stride, gain, cols, n_tok, pairs, S, p);
+  const dim3 grid(gx, n_slices), block(64 * nw);
+  const size_t lds = (size_t)nw * RA_WAVE_LDS;
+#define RA_LAUNCH(HHv, GAINv) do { \
+    static bool attr_done = false; \
+    if (!attr_done) { CAI_HIP(hipFuncSetAttribute((const void*)gemm_q4k_ra<HHv, GAINv>, hipFuncAttributeMaxDynamicSharedMemorySize, RA_NW * RA_WAVE_LDS)); attr_done = true; } \
+    hipLaunchKernelGGL((gemm_q4k_ra<HHv, GAINv>), grid, block, lds, ctx().stream, x, (long long)x_stride, gain, cols, n_tok, units, S, p); } while (0)
+  if (HH == 2 && gain) RA_LAUNCH(2, true);
+  else if (HH == 2) RA_LAUNCH(2, false);
+  else if (gain) RA_LAUNCH(1, true);
+  else RA_LAUNCH(1, false);
+#undef RA_LAUNCH
   return CAI_OK;
 }
 
