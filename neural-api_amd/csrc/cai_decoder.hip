@@ -461,7 +461,7 @@ static int run_step(cai_decoder_s* d, int n_b, int rows_needed, bool window = fa
                            std::max((size_t)nb_max_slices(dm) * al4(2 * (int64_t)cf.ffn), (size_t)nb_max_slices(cf.ffn) * al4(dm)));
     part = std::max(part, (size_t)nb_max_slices(dm) * al4(cf.vocab)) * 8;
     int rc = nb_reserve(kmax, part); if (rc) return rc;
-    if ((rc = ra_reserve(std::max(ra_part_floats(dm, cf.ffn), ra_part_floats(dm, d->qw()))))) return rc;   // (the sliced products: down and o)
+    if ((rc = ra_reserve(std::max(std::max(ra_part_floats(qkvw, dm), ra_part_floats(dm, d->qw())), std::max(ra_part_floats(2 * (int64_t)cf.ffn, dm), ra_part_floats(dm, cf.ffn)))))) return rc;   // (products of more than 16 super-blocks are sliced)
     const int gen = nb_ws_generation() + ra_ws_generation();      // (both only ever grow)
     if (d->ws_generation != gen) { invalidate_graphs(d); d->ws_generation = gen; }
   }

@@ -1018,6 +1018,17 @@ int nb_pass_tokens(const cai_qw_s* w) { return w->qtype == CAI_Q6_K ? NB_TMAX : 
 int nb_linear(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int n_tok, float* y, int64_t y_stride, const float* residual)
 {
   int rc;
+  // Q4_K matrices of whole row sets: the one-launch form (cai_gemm_ra.hip), 8 tokens per launch
+  if (ra_supported(&w, 1, gain != nullptr, 0) && !(x_stride & 3) && !(y_stride & 3) && !(reinterpret_cast<uintptr_t>(x) & 15) && !(reinterpret_cast<uintptr_t>(y) & 15) &&
+      !(residual && (reinterpret_cast<uintptr_t>(residual) & 15)) && !(gain && (reinterpret_cast<uintptr_t>(gain) & 15)) && !(w->bias && (reinterpret_cast<uintptr_t>(w->bias) & 15))) {
+    if ((rc = ra_reserve(ra_part_floats(w->rows, w->cols)))) return rc;
+    for (int t0 = 0; t0 < n_tok; t0 += 8) {
+      const int zero = 0;
+      if ((rc = ra_gemm(&w, &zero, 1, std::min(8, n_tok - t0), x + (int64_t)t0 * x_stride, x_stride, gain, eps, 0, y + (int64_t)t0 * y_stride, y_stride,
+                        residual ? residual + (int64_t)t0 * y_stride : nullptr))) return rc;
+    }
+    return CAI_OK;
+  }
   const int pass = nb_pass_tokens(w);
   if ((rc = nb_reserve((int)w->cols, (size_t)nb_max_slices((int)w->cols) * pass * ((w->rows + 3) / 4 * 4)))) return rc;
   for (int t0 = 0; t0 < n_tok; t0 += pass) {

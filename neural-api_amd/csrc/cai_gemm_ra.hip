@@ -33,7 +33,7 @@ constexpr int RA_NW = 8;         // waves per work-group at most
 constexpr int RA_SBW = 2;        // super-blocks of a row per wave
 constexpr int RA_SMAX = RA_NW * RA_SBW;   // super-blocks per column slice at most
 constexpr int RA_BB = 144;       // bytes of a Q4_K super-block
-constexpr int RA_PART_BATCH = 8; // slices the last arriver requests at once
+constexpr int RA_PART_BATCH = 8; // slices of an element the last arriver requests at once (times 2 elements, times 2 for SwiGLU)
 constexpr int RA_XLD = RA_SBW * 256 + 8;          // halfs per operand column in LDS (+8: 16 columns x 16-byte reads tile the banks)
 constexpr int RA_WAVE_LDS = 16 * RA_XLD * 2 + 16 * 16 * 2 + RA_SBW * RA_TK * 4 + 192;   // = 17408 bytes per wave
 
@@ -352,14 +352,23 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
       if constexpr (HH == 2) { const float4 b = *reinterpret_cast<const float4*>(src + 4); t8[4] += b.x; t8[5] += b.y; t8[6] += b.z; t8[7] += b.w; }
     }
     if (!tok_on) return;
+    const int pair = (int)blockIdx.x + i * (int)gridDim.x;
+    const RaSeg* sg; int r0, r1; locate(pair, sg, r0, r1);
+    if (p.n_slices > 1) {     // a slice's share of the rows (finished by the last slice to arrive, below)
+#pragma unroll
+      for (int hh = 0; hh < HH; hh++) {
+        float* dst = p.part + ((int64_t)slice * hntok + tok) * p.part_stride + sg->y_off + (hh ? r1 : r0) + 4 * kg;
+#pragma unroll
+        for (int k = 0; k < 4; k++) ra_part_store(dst + k, t8[4 * hh + k]);
+      }
+      return;
+    }
     float inv = 1.0f;
     if (GAIN) {   // (a product with a gain is one slice: the work-group has seen the whole row; every wave has passed this pair's barrier)
       float t = 0.0f;
       for (int sb = 0; sb < nS; sb++) t += ssq_s[sb][tok];     // fixed order
       inv = 1.0f / sqrtf(t / (float)K + p.eps);
     }
-    const int pair = (int)blockIdx.x + i * (int)gridDim.x;
-    const RaSeg* sg; int r0, r1; locate(pair, sg, r0, r1);
     if (HH == 2 && p.swiglu_half > 0) {
       const int col = 16 * pair + 4 * kg;       // rows r0 + 4 kg .. + 3 (up) and r1 + 4 kg .. + 3 (gate)
       const float bu[4] = {f.bias[0].x, f.bias[0].y, f.bias[0].z, f.bias[0].w}, bg[4] = {f.bias[HH - 1].x, f.bias[HH - 1].y, f.bias[HH - 1].z, f.bias[HH - 1].w};
@@ -376,12 +385,6 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
 #pragma unroll
     for (int hh = 0; hh < HH; hh++) {
       const int row = (hh ? r1 : r0) + 4 * kg;
-      if (p.n_slices > 1) {
-        float* dst = p.part + ((int64_t)slice * hntok + tok) * p.part_stride + sg->y_off + row;
-#pragma unroll
-        for (int k = 0; k < 4; k++) ra_part_store(dst + k, t8[4 * hh + k]);
-        continue;
-      }
       const float bb[4] = {f.bias[hh].x, f.bias[hh].y, f.bias[hh].z, f.bias[hh].w}, rr[4] = {f.res[hh].x, f.res[hh].y, f.res[hh].z, f.res[hh].w};
       float vv[4];
 #pragma unroll
@@ -406,8 +409,8 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
   }
   timeline_stamp(p.timeline, 5);
   if (p.n_slices > 1) {
-    // the slices of a row group meet: shares stored with agent-scope stores and acknowledged (vmcnt(0)) before the barrier
-    // and the work-group's arrival; the last arriver reads them with agent-scope loads, in slice order
+    // the slices of a row group meet: shares stored with agent-scope stores and acknowledged (vmcnt(0)) before the barrier and
+    // the work-group's arrival; the last arriver reads them with agent-scope loads, in slice order
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
     if (threadIdx.x == 0)
@@ -415,26 +418,39 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
     __syncthreads();
     timeline_stamp(p.timeline, 6);
     if (!s_is_last) { timeline_stamp(p.timeline, 7); return; }
-    const int total = npw * 16 * HH * hntok;
-    for (int e = threadIdx.x; e < total; e += blockDim.x) {
-      const int r32 = e % (16 * HH), t = (e / (16 * HH)) % hntok, i = (e / (16 * HH)) / hntok;
-      const RaSeg* sg; int r0, r1; locate((int)blockIdx.x + i * (int)gridDim.x, sg, r0, r1);
-      const int row = r0 + r32;
-      if (row >= sg->rows) continue;
-      const float* src = p.part + (int64_t)t * p.part_stride + sg->y_off + row;
-      const int64_t o = (int64_t)t * p.y_stride + sg->y_off + row;
-      // all requests of the element first (the slices, bias, residual), then the additions in slice order
-      float ps[RA_PART_BATCH];
-      const float bv = sg->bias ? sg->bias[row] : 0.0f, rv = p.residual ? p.residual[o] : 0.0f;
-      float v = 0.0f;
-      for (int s0 = 0; s0 < p.n_slices; s0 += RA_PART_BATCH) {
+    // the elements EB at a time: all slices' shares of a batch of elements (and their bias and residual) are requested before
+    // the first addition; the additions run in slice order
+    const int rpu = 16 * HH;                                  // rows per unit
+    const int total = npw * rpu * hntok;
+    const int64_t sstep = (int64_t)hntok * p.part_stride;     // from one slice's share of an element to the next
+    constexpr int EB = 2;
+    for (int e0 = threadIdx.x; e0 < total; e0 += EB * blockDim.x) {
+      const float* src[EB]; float bias[EB], res[EB], sum[EB]; int64_t out[EB]; bool on[EB];
 #pragma unroll
-        for (int u = 0; u < RA_PART_BATCH; u++) ps[u] = ra_part_load(src + (int64_t)min(s0 + u, p.n_slices - 1) * hntok * p.part_stride);
-#pragma unroll
-        for (int u = 0; u < RA_PART_BATCH; u++) if (s0 + u < p.n_slices) v += ps[u];
+      for (int b = 0; b < EB; b++) {
+        const int e = min(e0 + b * (int)blockDim.x, total - 1);
+        on[b] = e0 + b * (int)blockDim.x < total;
+        const int rl = e % rpu, t = (e / rpu) % hntok, i = (e / rpu) / hntok;
+        const RaSeg* sg; int r0, r1; locate((int)blockIdx.x + i * (int)gridDim.x, sg, r0, r1);
+        src[b] = p.part + (int64_t)t * p.part_stride + sg->y_off + r0 + rl;
+        out[b] = (int64_t)t * p.y_stride + sg->y_off + r0 + rl;
+        bias[b] = sg->bias ? sg->bias[r0 + rl] : 0.0f;
+        res[b] = p.residual ? p.residual[out[b]] : 0.0f;
+        sum[b] = 0.0f;
       }
-      v += bv; v += rv;
-      p.y[o] = v;
+      for (int s0 = 0; s0 < p.n_slices; s0 += RA_PART_BATCH) {
+        float ps[EB][RA_PART_BATCH];
+#pragma unroll
+        for (int b = 0; b < EB; b++)
+#pragma unroll
+          for (int u = 0; u < RA_PART_BATCH; u++) ps[b][u] = ra_part_load(src[b] + (int64_t)min(s0 + u, p.n_slices - 1) * sstep);
+#pragma unroll
+        for (int b = 0; b < EB; b++)
+#pragma unroll
+          for (int u = 0; u < RA_PART_BATCH; u++) if (s0 + u < p.n_slices) sum[b] += ps[b][u];
+      }
+#pragma unroll
+      for (int b = 0; b < EB; b++) if (on[b]) p.y[out[b]] = sum[b] + bias[b] + res[b];
     }
   }
   timeline_stamp(p.timeline, 7);
@@ -450,14 +466,14 @@ constexpr int RA_COUNTERS = 1024;
 
 // How a product over nsb super-blocks and `pairs` row pairs is cut: column slices of S super-blocks (work-groups of
 // ceil(S / 2) waves; a CU holds 8 such waves) and gx row groups, so that all work-groups are resident at once and the
-// longest walk (pairs of a work-group) is shortest; fewer slices at equal length.  A product that needs 1/rms or SwiGLU must stay one slice.
-bool ra_geometry(int nsb, int pairs, bool one_slice, int& S, int& n_slices, int& gx)
+// longest walk (pairs of a work-group) is shortest; fewer slices at equal length.
+bool ra_geometry(int nsb, int pairs, int& S, int& n_slices, int& gx)
 {
   const int n_cu = ctx().n_cu;
   const int ns_min = (nsb + RA_SMAX - 1) / RA_SMAX;
-  if (one_slice && ns_min > 1) return false;
   float best = 3.0e38f;
-  for (int ns = ns_min; ns <= (one_slice ? 1 : std::min(nsb, ns_min + 8)); ns++) {
+  // (a width that fits one slice stays one: no partial results at all)
+  for (int ns = ns_min; ns <= (ns_min == 1 ? 1 : std::min(nsb, ns_min + 8)); ns++) {
     const int s = (nsb + ns - 1) / ns;
     if ((nsb + s - 1) / s != ns) continue;
     const int nw = (s + RA_SBW - 1) / RA_SBW;
@@ -518,6 +534,8 @@ bool ra_supported(const cai_qw_s* const* ws, int n_w, bool normed, int swiglu_ha
     if (w->qtype != CAI_Q4_K || w->cols != ws[0]->cols || w->cols % 256 || w->cols < 256 || w->rows % 16) return false;
   }
   if (swiglu_half > 0 && (ws[0]->rows != 2 * (int64_t)swiglu_half || swiglu_half % 16)) return false;
+  // a product with an RMSNorm or SwiGLU must be one column slice (its finishing wave needs the whole row's sum of squares and
+  // both halves' rows); measured on 5120 columns a sliced form with those exchanged through memory lost to the plane form
   const int nsb = (int)(ws[0]->cols >> 8);
   return !((normed || swiglu_half > 0) && nsb > RA_SMAX);
 }
@@ -539,7 +557,6 @@ int ra_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, con
   RaParams p{};
   p.n_seg = n_w; p.eps = eps; p.swiglu_half = swiglu_half; p.y = y; p.y_stride = y_stride; p.residual = residual;
   const int cols = (int)ws[0]->cols, nsb = cols >> 8;
-  const bool one_slice = gain != nullptr || swiglu_half > 0;
   // units of 32 rows (pairs of row sets), or of 16 where that shortens the longest walk (a wave takes 2 x HH items per unit)
   int HH = 2, S = 0, n_slices = 0, gx = 0, units = 0;
   {
@@ -548,7 +565,7 @@ int ra_gemm(const cai_qw_s* const* ws, const int* y_off, int n_w, int n_tok, con
     bool whole_pairs = true;
     for (int i = 0; i < n_w; i++) whole_pairs = whole_pairs && ws[i]->rows % 32 == 0;
     int S2 = 0, ns2 = 0, g2 = 0, S1 = 0, ns1 = 0, g1 = 0;
-    if (!ra_geometry(nsb, u2, one_slice, S2, ns2, g2) || !ra_geometry(nsb, u1, one_slice, S1, ns1, g1))
+    if (!ra_geometry(nsb, u2, S2, ns2, g2) || !ra_geometry(nsb, u1, S1, ns1, g1))
       return set_error(CAI_ERR_UNSUPPORTED, "small-batch product (register form): width %d", cols);
     units = u2; S = S2; n_slices = ns2; gx = g2;
     if (swiglu_half == 0 && (!whole_pairs || (u1 + g1 - 1) / g1 < 2 * ((u2 + g2 - 1) / g2))) { HH = 1; units = u1; S = S1; n_slices = ns1; gx = g1; }
