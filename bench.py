@@ -253,7 +253,8 @@ def step_timeline(dec, tok, np):
     dependent kernels: end-of-kernel cache write-back, packet processing, dispatch), skew = last entry minus first entry, then
     medians over work-groups of the in-kernel phases (issue: entry to first requests out; arrive: until the activation values
     are there; quant: until the block-float form is in LDS; lift: until it is in registers; loop; tail: loop end to exit) and
-    the slowest work-group's loop and tail; span = last exit minus first entry."""
+    the slowest work-group's loop and tail; span = last exit minus first entry.  count: the attention launch's wait for the
+    arrival counter; in the one-launch small-batch products (a batched step: --batch) the first unit's products in the first wave."""
     names = ["embedding", "q|k|v", "attention", "o", "gate|up", "down", "head", "arg-max"]
     recs = dec.timeline(tok)
     rows, prev_end = [], None

@@ -1,5 +1,5 @@
 """The environment switches the library reads select other code paths (no stream capture; token-by-token prompts;
-prompt attention through the decode kernels, and the bound of its partial-result buffer).  Each is read once per process, so each case runs in a child process with the
+prompt attention through the decode kernels and the bound of its partial-result buffer; the older form of the small-batch step).  Each is read once per process, so each case runs in a child process with the
 variable set and is checked against the oracle there: a Q4_K decoder with QKV bias and 7 query heads per KV head, a 40-token
 prompt through cai_decoder_prefill, then 8 greedy tokens through cai_decoder_generate, a window step and the lookup loop."""
 import os
@@ -48,7 +48,10 @@ print("CHILD_OK")
 @pytest.mark.parametrize("switches", [{"CAIHIP_NO_GRAPH": "1"}, {"CAIHIP_PREFILL_TOKENWISE": "1"}, {"CAIHIP_PROMPT_FLASH": "0"},
                                       # prompt attention on the decode kernels with room for 4 rows' partial results per launch
                                       # (14 heads x 1 slice x 130 floats a row): the 40-token prompt attends in 10 groups
-                                      {"CAIHIP_PROMPT_FLASH": "0", "CAIHIP_PROMPT_PART_KB": "32"}])
+                                      {"CAIHIP_PROMPT_FLASH": "0", "CAIHIP_PROMPT_PART_KB": "32"},
+                                      # batched / window steps of a Q4_K model through the form with activation planes and slice
+                                      # partials (the one-launch form takes them otherwise)
+                                      {"CAIHIP_SMALL_BATCH_PLANES": "1"}])
 def test_switch_selected_path_matches_the_oracle(switches):
     env = dict(os.environ); env.update(switches)
     code = CHILD % dict(root=ROOT, tests=os.path.join(ROOT, "tests"))
