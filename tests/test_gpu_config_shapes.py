@@ -81,6 +81,30 @@ def test_q4_k_gemv_at_the_32b_shapes(rows, cols):
     w.close()
 
 
+@pytest.mark.parametrize("rows,cols", [(38864, 768), (6864, 4352), (3152, 9472), (17456, 1792)])
+def test_q4_k_one_launch_small_batch_form_on_awkward_shapes(rows, cols):
+    """The one-launch small-batch form of Q4_K (a batch of cai_qgemv on a matrix of 16 MiB or more) where its geometry has
+    remainders: an odd number of super-blocks (768 = 3: the last wave of a work-group covers one, not two), widths cut into
+    column slices that the last work-group to arrive adds up (4352 = 17 super-blocks: two slices, 9472 = 37: three), row counts
+    that are an odd number of 16-row sets (units of 16 rows), 2, 3, 5 and 8 tokens; against the float64-accumulated oracle,
+    with bias."""
+    from helpers.device import dev, rel_err
+    cai = dev()
+    assert rows % 16 == 0 and (rows // 16) % 2 == 1 and rows * cols * 144 // 256 >= 16 << 20
+    raw, rng = big_matrix(O.Q4_K, rows, cols, rows + 7 * cols)
+    bias = (rng.standard_normal(rows) * 0.1).astype(np.float32)
+    w = cai.QWeight(O.Q4_K, rows, cols, raw, bias)
+    x = rng.standard_normal((8, cols)).astype(np.float32)
+    x[3] *= 40.0                       # tokens of different magnitude: the block scales are per token
+    x[5, : cols // 2] = 0.0            # whole zero blocks
+    want = O.gemv(O.Q4_K, raw, rows, cols, x, bias, 0, 1)
+    for nb in (2, 3, 5, 8):
+        got = w.gemv(x[:nb])
+        for b in range(nb):
+            assert rel_err(got[b], want[b], floor=0.02 * cols ** 0.5 * (40.0 if b == 3 else 1.0)) < TIGHT, (nb, b)
+    w.close()
+
+
 @pytest.mark.parametrize("qt", [O.Q8_0, O.Q4_0])
 @pytest.mark.parametrize("rows,cols", [(18944, 3584), (152064, 3584)])
 def test_q8_0_q4_0_gemv_at_the_large_sweep_shapes(qt, rows, cols):
