@@ -260,6 +260,7 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const int32_t* hpos, co
 {
   // (leading scalar arguments arrive preloaded in scalar registers: position, q | k | v row and frequencies are requested without
   //  a round trip to the argument block; hheads = query heads | KV heads << 16, hgeo = slices | head width << 16, hsl = slice length)
+  const unsigned long long tl0 = timeline_now();
   const int h_q_heads = hheads & 0xffff, h_kv_heads = hheads >> 16, h_n_splits = hgeo & 0xffff, h_hd = hgeo >> 16;
   extern __shared__ __align__(16) float lds[];
   constexpr bool I8 = sizeof(KV_T) == 1;
@@ -316,6 +317,8 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const int32_t* hpos, co
     qx0[u] = qh[2 * i]; qx1[u] = qh[2 * i + 1]; qth[u] = htheta ? htheta[i] : 0.0f;
   }
   if (!owns_new) prime(kc, ksc);
+  timeline_put(p.timeline, 0, tl0);
+  timeline_stamp(p.timeline, 1);
 
   // rotated q of the group's heads -> LDS
   for (int e = tid; e < n_qp; e += 256) {
@@ -360,6 +363,7 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const int32_t* hpos, co
   }
   __syncthreads();      // q is staged; the appended row is visible to this work-group's loads
   if (owns_new) prime(kc, ksc);
+  timeline_stamp(p.timeline, 4);
 
   // ---- phase 1: scores of the slice ----
   for (int ch = 0; ch < n_chunks; ch++) {
@@ -398,6 +402,7 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const int32_t* hpos, co
   }
   prime(vc, vsc);        // the first value rows travel while the softmax runs
   __syncthreads();
+  timeline_stamp(p.timeline, 5);
 
   // ---- phase 2: slice maximum, exp-shift and sum per head (wave w takes heads w, w+4, ..) ----
   for (int h = w; h < G; h += 4) {
@@ -417,6 +422,7 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const int32_t* hpos, co
   }
   __syncthreads();
 
+  timeline_stamp(p.timeline, 6);
   // ---- phase 3: value sums ----
   for (int ch = 0; ch < n_chunks; ch++) {
     const int h0 = ch * HC;
@@ -477,6 +483,288 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const int32_t* hpos, co
     }
     __syncthreads();
   }
+  timeline_stamp(p.timeline, 7);
+}
+
+// ---- the same split on the matrix cores: half-precision cache, 128-wide heads, groups of up to 16 query heads.
+//      The VALU form above spends its time on instructions (8 conversions, 8 fused multiply-adds per head and a 4-step lane
+//      reduction per head for every 16 bytes of K), one wave per SIMD.  Here a wave requests ALL its rows of the slice at once
+//      (16-row tiles w, w + NW, ..: TPW tiles of K and of V, 16 KB in flight per wave) and the products are
+//        S[row][head]  = K . q^T      v_mfma_f32_16x16x32_f16, K rows straight from memory as the A operand (lane = row,
+//                                     16 bytes = 8 of the 32 contraction slots), q split hi + lo into two f16 planes in LDS;
+//        O[head][dim] += P^T . V      the result registers of the first product (lane = head, 4 rows each of two tiles) ARE
+//                                     the A operand of a 32-row step; P is scaled by 1024 and split hi + lo (its low part
+//                                     stays clear of the f16 subnormal range); V goes through LDS as it arrives (row-major,
+//                                     16-byte stores) and comes back as 32-bit words = two neighbouring dims of one row, so
+//                                     that one byte permute per word pair builds the operand of the even and of the odd dims.
+//      Every wave keeps its own maximum and sum per head; the four waves meet once, in LDS, and the slice partial has the
+//      same form as above.  Same contract and tolerance as the VALU kernels (1e-5 against the oracle). ----
+typedef _Float16 ph4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 ph8_t __attribute__((ext_vector_type(8)));
+constexpr int GM_LD = 136;                         // halfs per staged row (128 + pad: 16-byte aligned, 4 rows apart = 16 banks apart)
+constexpr int GM_FIXED = 2 * 16 * GM_LD * 2 + 512 + 1024;  // q hi | q lo | new K,V row | per-wave maximum and sum
+constexpr int gm_lds_bytes(int tpw, int nw) { return GM_FIXED + nw * tpw * 16 * GM_LD * 2; }
+
+// TPW 16-row tiles per wave, NW waves: 2 x 4 (slices of up to 128 rows) or 2 x 8 (up to 256: two waves per SIMD overlap each
+// other's dependent LDS / matrix-core / soft-max chains)
+template <int TPW, int NW>
+__global__ __launch_bounds__(64 * NW) void attn_group_mfma_kernel(const int32_t* hpos, const float* hqkv, const float* htheta, const long long hqkv_stride,
+                                                              const int hheads, const int hgeo, const int hsl, const AttnParams p)
+{
+  const unsigned long long tl0 = timeline_now();
+  const int h_q_heads = hheads & 0xffff, h_kv_heads = hheads >> 16, h_n_splits = hgeo & 0xffff;
+  constexpr int hd = 128;
+  extern __shared__ __align__(16) unsigned char glds[];
+  _Float16* sqh = reinterpret_cast<_Float16*>(glds);
+  _Float16* sql = sqh + 16 * GM_LD;
+  _Float16* snew = sql + 16 * GM_LD;                           // [K | V][128]
+  float* sML = reinterpret_cast<float*>(snew + 256);           // [wave][head][maximum, sum]
+  constexpr int REGION = TPW * 16 * GM_LD * 2;                 // bytes of a wave's V tiles (later: its [head][128] float sums)
+  const int G = h_q_heads / h_kv_heads;
+  const int split = blockIdx.x % h_n_splits, g = blockIdx.x / h_n_splits, seq = blockIdx.y;
+  const int pos = hpos[seq];
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, n16 = lane & 15, kg = lane >> 4;
+  const int qw = h_q_heads * hd, kw = h_kv_heads * hd;
+  const float* row = hqkv + (int64_t)seq * hqkv_stride;
+  // the group's q pairs and frequencies do not depend on the position: requested behind it, before anything waits
+  float qx0[2], qx1[2], qth[2];
+#pragma unroll
+  for (int u = 0; u < 2; u++) {
+    const int e = tid + 64 * NW * u, h = min(e >> 6, G - 1), i = e & 63;
+    const float* qh = row + (g * G + h) * hd;
+    qx0[u] = qh[2 * i]; qx1[u] = qh[2 * i + 1]; qth[u] = htheta ? htheta[i] : 0.0f;
+  }
+  const int SL = hsl, base = split * SL;
+  const int64_t cache_seq = seq * p.seq_mul + p.seq0;
+  __half* kc = reinterpret_cast<__half*>(p.kc) + cache_seq * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  __half* vc = reinterpret_cast<__half*>(p.vc) + cache_seq * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  // The wave's first K tile is requested before the position is known (its rows exist whatever the position: the slice lies
+  // inside the cache; rows past the live range are masked), so the stream starts while the position is still on its way.
+  uint4 kreg[TPW][4], vreg[TPW][4];
+  {
+    const int j = min(base + 16 * w + n16, p.max_ctx - 1);
+#pragma unroll
+    for (int s4 = 0; s4 < 4; s4++) kreg[0][s4] = *reinterpret_cast<const uint4*>(kc + (int64_t)j * hd + 32 * s4 + 8 * kg);
+  }
+  const LiveRows lr = live_rows(p, pos);
+  const int len = lr.len, j_start = lr.j_start, slot = lr.slot;
+  const int s_begin = max(j_start, base), s_end = min(len, base + SL);
+  if (s_begin >= s_end) return;   // whole work-group leaves together, before any barrier
+  const int s_first = j_start / SL, s_last = (len - 1) / SL;
+  const int n_active = s_last - s_first + 1;
+
+  // the work-group whose slice holds `pos` appends the new row (wave 0, one half-wave each for K and V): its raw elements are
+  // requested here, in front of the cached rows (requests return in order)
+  const bool owns_new = !p.appended && slot >= s_begin && slot < s_end;
+  float nraw[4] = {0.0f, 0.0f, 0.0f, 0.0f}, nth[2] = {0.0f, 0.0f};
+  if (owns_new && w == 0) {
+    const int l32 = lane & 31, is_v = lane >> 5, e0 = 4 * l32;
+    const float* src = row + qw + (is_v ? kw : 0) + g * hd + e0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) nraw[i] = src[i];
+    if (htheta) { nth[0] = htheta[e0 >> 1]; nth[1] = htheta[(e0 >> 1) + 1]; }
+  }
+  // every other row of the wave's tiles, K first (the first product starts while V is still on its way).
+  // Rows past the live range repeat its last row and are masked below.
+#pragma unroll
+  for (int t = 1; t < TPW; t++) {
+    const int j = min(base + 16 * (w + NW * t) + n16, s_end - 1);
+#pragma unroll
+    for (int s4 = 0; s4 < 4; s4++) kreg[t][s4] = *reinterpret_cast<const uint4*>(kc + (int64_t)j * hd + 32 * s4 + 8 * kg);
+  }
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int j = min(base + 16 * (w + NW * t) + 4 * i + kg, s_end - 1);
+      vreg[t][i] = *reinterpret_cast<const uint4*>(vc + (int64_t)j * hd + 8 * n16);
+    }
+  timeline_put(p.timeline, 0, tl0);
+  timeline_stamp(p.timeline, 1);
+
+  // rotated q of the group's heads as two f16 planes in LDS (wave w takes heads w, w + NW, ..; rows G .. 15 are zero)
+#pragma unroll
+  for (int u = 0; u < 16 / NW; u++) {
+    const int h = w + NW * u, i = lane;
+    _Float16 h0 = 0, h1 = 0, l0 = 0, l1 = 0;
+    if (h < G) {
+      float x0, x1, th;
+      if (u < 2) { x0 = qx0[u]; x1 = qx1[u]; th = qth[u]; }
+      else { const float* qh = row + (g * G + h) * hd; x0 = qh[2 * i]; x1 = qh[2 * i + 1]; th = htheta ? htheta[i] : 0.0f; }
+      if (htheta) {
+        float sn, cs; sincosf((float)pos * th, &sn, &cs);
+        const float y0 = cs * x0 - sn * x1, y1 = sn * x0 + cs * x1;
+        x0 = y0; x1 = y1;
+      }
+      split_f16(x0, h0, l0); split_f16(x1, h1, l1);
+    }
+    sqh[h * GM_LD + 2 * i] = h0; sqh[h * GM_LD + 2 * i + 1] = h1;
+    sql[h * GM_LD + 2 * i] = l0; sql[h * GM_LD + 2 * i + 1] = l1;
+  }
+  // the new row: rotated, rounded to the cache's precision, stored, and kept in LDS for this work-group's own products (its
+  // requests for that row went out before the store)
+  if (owns_new && w == 0) {
+    const int l32 = lane & 31, is_v = lane >> 5, e0 = 4 * l32;
+    __half* dst = (is_v ? vc : kc) + (int64_t)slot * hd;
+#pragma unroll
+    for (int i = 0; i < 4; i += 2) {
+      const int d = e0 + i;
+      float x0 = nraw[i], x1 = nraw[i + 1];
+      if (htheta && !is_v) {
+        float sn, cs; sincosf((float)pos * nth[i >> 1], &sn, &cs);
+        const float y0 = cs * x0 - sn * x1, y1 = sn * x0 + cs * x1;
+        x0 = y0; x1 = y1;
+      }
+      const __half r0 = __float2half_rn(x0), r1 = __float2half_rn(x1);
+      dst[d] = r0; dst[d + 1] = r1;
+      snew[is_v * 128 + d] = __builtin_bit_cast(_Float16, r0); snew[is_v * 128 + d + 1] = __builtin_bit_cast(_Float16, r1);
+    }
+  }
+  __syncthreads();
+  timeline_stamp(p.timeline, 4);
+
+  ph8_t qh8[4], ql8[4];
+#pragma unroll
+  for (int s4 = 0; s4 < 4; s4++) {
+    qh8[s4] = *reinterpret_cast<const ph8_t*>(sqh + n16 * GM_LD + 32 * s4 + 8 * kg);
+    ql8[s4] = *reinterpret_cast<const ph8_t*>(sql + n16 * GM_LD + 32 * s4 + 8 * kg);
+  }
+  if (owns_new) {
+    // the new row from LDS in place of what memory held; rows past the live range may be memory that was never written (the
+    // new row's slot before this step): their V registers are cleared, 0 x NaN would poison the sums
+    const int rs = slot - base;
+#pragma unroll
+    for (int t = 0; t < TPW; t++) {
+      const int r0 = 16 * (w + NW * t);
+      if (rs >= r0 && rs < r0 + 16) {
+        if (n16 == rs - r0) {
+#pragma unroll
+          for (int s4 = 0; s4 < 4; s4++) kreg[t][s4] = *reinterpret_cast<const uint4*>(snew + 32 * s4 + 8 * kg);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+          if (4 * i + kg == rs - r0) vreg[t][i] = *reinterpret_cast<const uint4*>(snew + 128 + 8 * n16);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        if (base + r0 + 4 * i + kg >= s_end) vreg[t][i] = make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+
+  // ---- scores of the wave's rows, maximum, weights ----
+  typedef float gf4_t __attribute__((ext_vector_type(4)));
+  gf4_t C[TPW];
+#pragma unroll
+  for (int t = 0; t < TPW; t++) {
+    C[t] = gf4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int s4 = 0; s4 < 4; s4++) {
+      const ph8_t a = __builtin_bit_cast(ph8_t, kreg[t][s4]);
+      C[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qh8[s4], C[t], 0, 0, 0);
+      C[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, ql8[s4], C[t], 0, 0, 0);
+    }
+  }
+  // lane (n16, kg) holds head n16 of rows 4 kg .. 4 kg + 3 of every tile
+  float m_w = -1e30f;
+  bool ok[TPW][4];
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int j = base + 16 * (w + NW * t) + 4 * kg + i;
+      float sc = C[t][i] * p.inv_sqrt;
+      if (p.softcap > 0.0f) sc = p.softcap * tanhf(sc / p.softcap);
+      ok[t][i] = j >= s_begin && j < s_end;
+      C[t][i] = sc;
+      if (ok[t][i]) m_w = fmaxf(m_w, sc);
+    }
+  m_w = fmaxf(m_w, __shfl_xor(m_w, 16, 64));
+  m_w = fmaxf(m_w, __shfl_xor(m_w, 32, 64));
+  float l_w = 0.0f;
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) { C[t][i] = ok[t][i] ? expf(C[t][i] - m_w) : 0.0f; l_w += C[t][i]; }
+  l_w += __shfl_xor(l_w, 16, 64);
+  l_w += __shfl_xor(l_w, 32, 64);
+  timeline_stamp(p.timeline, 5);
+
+  // ---- value sums ----
+  unsigned char* region = glds + GM_FIXED + w * REGION;
+  _Float16* sV = reinterpret_cast<_Float16*>(region);
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) *reinterpret_cast<uint4*>(sV + (16 * t + 4 * i + kg) * GM_LD + 8 * n16) = vreg[t][i];
+  gf4_t Oe[4], Oo[4];
+#pragma unroll
+  for (int u = 0; u < 4; u++) { Oe[u] = gf4_t{0.0f, 0.0f, 0.0f, 0.0f}; Oo[u] = gf4_t{0.0f, 0.0f, 0.0f, 0.0f}; }
+#pragma unroll
+  for (int b = 0; b < TPW / 2; b++) {
+    // contraction slot e of this lane group = row 4 kg + (e & 3) of tile 2 b + (e >> 2), in both operands
+    ph8_t ph, pl;
+#pragma unroll
+    for (int e = 0; e < 8; e++) { _Float16 hv, lv; split_f16(C[2 * b + (e >> 2)][e & 3] * 1024.0f, hv, lv); ph[e] = hv; pl[e] = lv; }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+      uint32_t wv[8];
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        wv[e] = *reinterpret_cast<const uint32_t*>(sV + (16 * (2 * b + (e >> 2)) + 4 * kg + (e & 3)) * GM_LD + 32 * u + 2 * n16);
+      uint4 va, vb;       // column n16 of the even dims 32 u + 2 n16 and of the odd dims 32 u + 2 n16 + 1
+      va.x = __builtin_amdgcn_perm(wv[1], wv[0], 0x05040100u); vb.x = __builtin_amdgcn_perm(wv[1], wv[0], 0x07060302u);
+      va.y = __builtin_amdgcn_perm(wv[3], wv[2], 0x05040100u); vb.y = __builtin_amdgcn_perm(wv[3], wv[2], 0x07060302u);
+      va.z = __builtin_amdgcn_perm(wv[5], wv[4], 0x05040100u); vb.z = __builtin_amdgcn_perm(wv[5], wv[4], 0x07060302u);
+      va.w = __builtin_amdgcn_perm(wv[7], wv[6], 0x05040100u); vb.w = __builtin_amdgcn_perm(wv[7], wv[6], 0x07060302u);
+      const ph8_t a8 = __builtin_bit_cast(ph8_t, va), b8 = __builtin_bit_cast(ph8_t, vb);
+      Oe[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ph, a8, Oe[u], 0, 0, 0);
+      Oe[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl, a8, Oe[u], 0, 0, 0);
+      Oo[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ph, b8, Oo[u], 0, 0, 0);
+      Oo[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl, b8, Oo[u], 0, 0, 0);
+    }
+  }
+  timeline_stamp(p.timeline, 6);
+  // ---- meeting of the waves: lane (n16, kg) holds heads 4 kg .. 4 kg + 3, dims 32 u + 2 n16 (+ 1) ----
+  float* sO = reinterpret_cast<float*>(region);       // [head][128], over the wave's own V tiles (all read by now)
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+    if (4 * kg + i < G) {
+#pragma unroll
+      for (int u = 0; u < 4; u++) *reinterpret_cast<float2*>(sO + (4 * kg + i) * 128 + 32 * u + 2 * n16) = make_float2(Oe[u][i], Oo[u][i]);
+    }
+  if (kg == 0) { sML[(w * 16 + n16) * 2] = m_w; sML[(w * 16 + n16) * 2 + 1] = l_w; }
+  __syncthreads();
+  for (int o = tid; o < G * hd; o += 64 * NW) {
+    const int h = o >> 7, d = o & 127;
+    float mw[NW], lw[NW], ow[NW];
+#pragma unroll
+    for (int k = 0; k < NW; k++) {
+      mw[k] = sML[(k * 16 + h) * 2]; lw[k] = sML[(k * 16 + h) * 2 + 1];
+      ow[k] = reinterpret_cast<const float*>(glds + GM_FIXED + k * REGION)[h * 128 + d];
+    }
+    float M = mw[0];
+#pragma unroll
+    for (int k = 1; k < NW; k++) M = fmaxf(M, mw[k]);
+    float A = 0.0f, Ls = 0.0f;
+#pragma unroll
+    for (int k4 = 0; k4 < NW; k4 += 4) {      // fixed order: groups of four waves
+      float e[4];
+#pragma unroll
+      for (int k = 0; k < 4; k++) e[k] = lw[k4 + k] > 0.0f ? expf(mw[k4 + k] - M) : 0.0f;
+      A += (ow[k4] * e[0] + ow[k4 + 1] * e[1]) + (ow[k4 + 2] * e[2] + ow[k4 + 3] * e[3]);
+      Ls += (lw[k4] * e[0] + lw[k4 + 1] * e[1]) + (lw[k4 + 2] * e[2] + lw[k4 + 3] * e[3]);
+    }
+    A *= 1.0f / 1024.0f;
+    const int qh = g * G + h;
+    if (n_active == 1) {
+      p.out[(int64_t)seq * p.out_stride + qh * hd + d] = Ls > 0.0f ? A * (1.0f / Ls) : 0.0f;
+    } else {
+      float* pt = p.part + (((int64_t)seq * h_q_heads + qh) * h_n_splits + split) * (hd + 2);
+      pt[d] = A;
+      if (d == 0) { pt[hd] = M; pt[hd + 1] = Ls; }
+    }
+  }
+  timeline_stamp(p.timeline, 7);
 }
 
 // ---- merge of the split partials: one work-group per query head.  Four quarter-groups of head_dim threads each take every
@@ -488,24 +776,39 @@ __global__ __launch_bounds__(512) void attn_merge_kernel(const int32_t* hpos, co
   const int h_q_heads = hheads & 0xffff, h_n_splits = hgeo & 0xffff, h_hd = hgeo >> 16;     // (preloaded leading arguments, as in the split kernels)
   const int qh = blockIdx.x, seq = blockIdx.y;
   const int hd = h_hd;
+  __shared__ float qA[4][128], qM[4], qL[4];
+  const int quarter = threadIdx.x >> 7, d = threadIdx.x & 127;
+  constexpr int MR = 12;                           // slices per quarter and round trip
+  // Without a sliding window the first live slice is slice 0 whatever the position: the first round of partials (48 slices) is
+  // requested before the position has arrived and masked by the slice count afterwards (a partial past the live range is
+  // whatever an earlier step left there: it is selected away, never used in arithmetic).
+  const bool ahead = p.window <= 0 && d < hd;
+  const float* pt0 = hpart + ((int64_t)seq * h_q_heads + qh) * h_n_splits * (hd + 2);
+  float v[MR], ms[MR], ls[MR];
+  if (ahead) {
+#pragma unroll
+    for (int u = 0; u < MR; u++) {
+      const float* ps = pt0 + (int64_t)min(quarter + 4 * u, h_n_splits - 1) * (hd + 2);
+      v[u] = ps[d]; ms[u] = ps[hd]; ls[u] = ps[hd + 1];
+    }
+  }
   const LiveRows lr = live_rows(p, hpos[seq]);
   const int s_first = lr.j_start / hsl, s_last = (lr.len - 1) / hsl;
   const int n_active = s_last - s_first + 1;
   if (n_active == 1) return;                       // the split kernel already wrote the final row
-  const float* pt = hpart + (((int64_t)seq * h_q_heads + qh) * h_n_splits + s_first) * (hd + 2);
-  __shared__ float qA[4][128], qM[4], qL[4];
-  const int quarter = threadIdx.x >> 7, d = threadIdx.x & 127;
+  const float* pt = pt0 + (int64_t)s_first * (hd + 2);
   float A = 0.0f, L = 0.0f, M = -1e30f;
   if (d < hd) {
-    for (int s0 = quarter; s0 < n_active; s0 += 4 * 8) {
-      float v[8], ms[8], ls[8];
+    for (int s0 = quarter; s0 < n_active; s0 += 4 * MR) {
+      if (!(ahead && s0 == quarter)) {
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
-        const float* ps = pt + (int64_t)min(s0 + 4 * u, n_active - 1) * (hd + 2);
-        v[u] = ps[d]; ms[u] = ps[hd]; ls[u] = ps[hd + 1];
+        for (int u = 0; u < MR; u++) {
+          const float* ps = pt + (int64_t)min(s0 + 4 * u, n_active - 1) * (hd + 2);
+          v[u] = ps[d]; ms[u] = ps[hd]; ls[u] = ps[hd + 1];
+        }
       }
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
+      for (int u = 0; u < MR; u++) {
         if (s0 + 4 * u < n_active && ls[u] > 0.0f) {
           const float mn = fmaxf(M, ms[u]), c0 = expf(M - mn), c1 = expf(ms[u] - mn);
           A = fmaf(v[u], c1, A * c0); L = fmaf(ls[u], c1, L * c0); M = mn;
@@ -777,8 +1080,10 @@ static int launch_split_head(const AttnParams& p0, int n_seq, hipStream_t st)
 }
 
 template <typename KV_T, int NPF>
-static void launch_group_t(const AttnParams& p, const dim3 grid, size_t lds, int hc, hipStream_t st)
+static void launch_group_t(const AttnParams& p0, const dim3 grid, size_t lds, int hc, hipStream_t st)
 {
+  AttnParams p = p0;
+  p.timeline = timeline_next((int)(grid.x * grid.y));
   switch (hc) {
 #define CAI_GROUP_ARGS p.pos, (const float*)p.qkv, p.theta, (long long)p.qkv_stride, p.q_heads | p.kv_heads << 16, p.n_splits | p.hd << 16, p.split_len, p
     case 1: hipLaunchKernelGGL((attn_group_kernel<1, KV_T, NPF>), grid, dim3(256), lds, st, CAI_GROUP_ARGS); break;
@@ -807,6 +1112,31 @@ static int launch_group(const AttnParams& p, int n_seq, hipStream_t st)
   // per CU has nothing to overlap with and keeps the deep ring.
   if ((int)(grid.x * grid.y) >= 3 * ctx().n_cu) launch_group_t<KV_T, 2>(p, grid, lds, hc, st);
   else launch_group_t<KV_T, (sizeof(KV_T) == 4 ? 4 : 8)>(p, grid, lds, hc, st);
+  return CAI_OK;
+}
+
+// Whether the grouped launch of this cache takes the matrix-core kernel (CAIHIP_ATTN_GROUP_MFMA=0 keeps the VALU form).
+static bool group_takes_mfma(const AttnParams& p, int dtype)
+{
+  static const bool on = []() { const char* e = getenv("CAIHIP_ATTN_GROUP_MFMA"); return !(e && e[0] == '0'); }();
+  return on && dtype == CAI_KV_F16 && p.hd == 128 && p.q_heads / p.kv_heads <= 16 && p.split_len <= 256;
+}
+static int launch_group_mfma(const AttnParams& p0, int n_seq, hipStream_t st)
+{
+  AttnParams p = p0;
+  const dim3 grid(p.n_splits * p.kv_heads, n_seq);
+  p.timeline = timeline_next((int)(grid.x * grid.y));
+  if (p.q_heads > 0xffff || p.kv_heads > 0x7fff || p.n_splits > 0xffff) return set_error(CAI_ERR_UNSUPPORTED, "attention: %d query heads, %d slices", p.q_heads, p.n_splits);
+  const int hheads = p.q_heads | p.kv_heads << 16, hgeo = p.n_splits | p.hd << 16;
+#define CAI_GM_LAUNCH(TPWv, NWv) do { \
+    static bool attr_done = false;      /* up to 80 KB of dynamic LDS */ \
+    if (!attr_done) { CAI_HIP(hipFuncSetAttribute((const void*)attn_group_mfma_kernel<TPWv, NWv>, hipFuncAttributeMaxDynamicSharedMemorySize, gm_lds_bytes(TPWv, NWv))); attr_done = true; } \
+    hipLaunchKernelGGL((attn_group_mfma_kernel<TPWv, NWv>), grid, dim3(64 * NWv), gm_lds_bytes(TPWv, NWv), st, p.pos, (const float*)p.qkv, p.theta, (long long)p.qkv_stride, hheads, hgeo, p.split_len, p); } while (0)
+  // slices of up to 128 rows: four waves; longer ones: eight (32B shape at 8.2k rows, slices of 256: 177.5 tok/s with four waves
+  // of four tiles, 180.8 with eight waves of two at batch 1; 693.7 against 698.0 at batch 8)
+  if (p.split_len <= 128) CAI_GM_LAUNCH(2, 4);
+  else CAI_GM_LAUNCH(2, 8);
+#undef CAI_GM_LAUNCH
   return CAI_OK;
 }
 
@@ -893,8 +1223,6 @@ __global__ __launch_bounds__(256) void kv_append_rows_i8_kernel(const AttnParams
 //   O^T[dim][token] += V^T . P^T   with P split hi + lo into two f16 (22 bits), like q; a float cache is split too.
 // Same arithmetic as the decode kernels up to the order of the sums (tests: < 1e-4 of token-at-a-time ingestion).
 // ------------------------------------------------------------------------------------------
-typedef _Float16 ph4_t __attribute__((ext_vector_type(4)));
-typedef _Float16 ph8_t __attribute__((ext_vector_type(8)));
 typedef float pf16_t __attribute__((ext_vector_type(16)));
 
 struct PromptParams {
@@ -1301,7 +1629,9 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   }
   // one work-group per (slice, KV head) serving the whole group of query heads, or one per (slice, query head)
   // (the first fetches K and V once but has G times fewer work-groups: it needs a grid that fills the chip by itself)
-  if (grouped)
+  if (grouped && group_takes_mfma(p, kv->dtype))
+    rc = launch_group_mfma(p, n_seq, c.stream);
+  else if (grouped)
     rc = kv->dtype == CAI_KV_I8 ? launch_group<int8_t>(p, n_seq, c.stream) : kv->dtype == CAI_KV_F16 ? launch_group<__half>(p, n_seq, c.stream) : launch_group<float>(p, n_seq, c.stream);
   else
     rc = kv->dtype == CAI_KV_I8 ? launch_split_head<int8_t>(p, n_seq, c.stream) : kv->dtype == CAI_KV_F16 ? launch_split_head<__half>(p, n_seq, c.stream) : launch_split_head<float>(p, n_seq, c.stream);

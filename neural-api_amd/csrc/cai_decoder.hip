@@ -97,9 +97,13 @@ static int moe_ffn_rows(cai_decoder_s* d, const cai_decoder_s::Layer& L, float* 
   const int dm = c.d_model, I = c.ffn;
   int rc;
   const int E = c.n_experts, K = c.top_k;
-  MultiGemv r{}; r.n = 1; r.w[0] = L.w[CAI_W_ROUTER]; r.rows[0] = E;
-  if ((rc = launch_gemv_multi(r, x, n_b, d->router_logits, E, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;
-  if ((rc = launch_router_topk(d->router_logits, E, K, c.norm_topk, n_b, d->moe_expert, d->moe_gate, d->router_probs))) return rc;
+  if (router_fused_supported(L.w[CAI_W_ROUTER], K) && L.w[CAI_W_ROUTER]->rows == E && dm % 4 == 0) {
+    if ((rc = launch_router_fused(L.w[CAI_W_ROUTER], x, dm, L.v[CAI_V_MLP_NORM], c.eps, K, c.norm_topk, n_b, d->router_logits, d->moe_expert, d->moe_gate, d->router_probs, reinterpret_cast<unsigned*>(d->moe_expert + 8 * K)))) return rc;
+  } else {
+    MultiGemv r{}; r.n = 1; r.w[0] = L.w[CAI_W_ROUTER]; r.rows[0] = E;
+    if ((rc = launch_gemv_multi(r, x, n_b, d->router_logits, E, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;
+    if ((rc = launch_router_topk(d->router_logits, E, K, c.norm_topk, n_b, d->moe_expert, d->moe_gate, d->router_probs))) return rc;
+  }
   for (int b = 0; b < n_b; b++) {
     MultiGemv g{}; g.n = 1; g.w[0] = L.w[CAI_W_GATEUP]; g.rows[0] = 2 * I;
     g.slot_expert = d->moe_expert + b * K; g.n_slots = K; g.expert_rows = 2 * I; g.x_slot_stride = 0;
@@ -111,6 +115,10 @@ static int moe_ffn_rows(cai_decoder_s* d, const cai_decoder_s::Layer& L, float* 
       g.y_slot_stride = 2 * I;
       if ((rc = launch_gemv_multi(g, xb, 1, d->gu, 2 * I, CAI_ACT_NONE, nullptr, L.v[CAI_V_MLP_NORM], c.eps, 0))) return rc;
       launch_swiglu(d->gu, I, K, d->mid);
+    }
+    if (moe_down_mix_supported(L.w[CAI_W_DOWN], dm, K) && I % 4 == 0) {
+      if ((rc = launch_moe_down_mix(L.w[CAI_W_DOWN], dm, d->mid, d->moe_expert + b * K, d->moe_gate + b * K, K, x + (int64_t)b * dm))) return rc;
+      continue;
     }
     MultiGemv dn{}; dn.n = 1; dn.w[0] = L.w[CAI_W_DOWN]; dn.rows[0] = dm;
     dn.slot_expert = d->moe_expert + b * K; dn.n_slots = K; dn.expert_rows = dm; dn.x_slot_stride = I; dn.y_slot_stride = dm;
@@ -590,7 +598,9 @@ extern "C" int cai_decoder_create(const cai_decoder_config* cfg, cai_decoder_t* 
     if (e == hipSuccess) e = alloc_f(&d->router_probs, (size_t)8 * c.n_experts);
     if (e == hipSuccess) e = alloc_f(&d->moe_gate, (size_t)8 * K);
     if (e == hipSuccess) e = alloc_f(&d->moe_part, (size_t)K * c.d_model);
-    if (e == hipSuccess) e = hipMalloc((void**)&d->moe_expert, (size_t)8 * K * sizeof(int32_t));
+    // (+ eight arrival counters of the one-launch router behind the selections: zero once, they wrap back to zero)
+    if (e == hipSuccess) e = hipMalloc((void**)&d->moe_expert, (size_t)(8 * K + 8) * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMemsetAsync(d->moe_expert, 0, (size_t)(8 * K + 8) * sizeof(int32_t), ctx().stream);
   }
   const int ame = argmax_scratch_entries(c.vocab, RB);
   if (e == hipSuccess) e = alloc_f(&d->am_v, (size_t)ame);

@@ -224,10 +224,17 @@ int argmax_scratch_entries(int n, int n_rows);
 int noalloc_setup(int device);   // resolves the device address of the fixed scratch array (cai_init, device current)
 int launch_embed(const cai_qw_s* w, const int32_t* tokens_dev, int n_tokens, float* out);
 int launch_router_topk(const float* logits, int n, int k, int renorm, int n_tokens, int32_t* expert_out, float* gate_out, float* probs_scratch);
+// ... and the router's matrix-vector product, RMSNorm and selection in one launch (Q8_0 router rows, up to 64 experts)
+bool router_fused_supported(const cai_qw_s* w, int k);
+int launch_router_fused(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int k, int renorm, int n_tokens,
+                        float* logits_out, int32_t* expert_out, float* gate_out, float* probs_scratch, unsigned* counters);   // counters: one per token, zero before the first launch (they wrap back to zero)
 int launch_rmsnorm_strided(const float* x, const float* gain, int n, int n_tokens, float eps, float* y, int64_t x_stride, int64_t y_stride);
 void decoder_adopt_weight(cai_decoder_s* d, cai_qw_s* w);   // the decoder destroys w with itself
 int launch_rmsnorm_pair(float* x, const float* gain_a, int n_a, const float* gain_b, int n_b, int n_tokens, float eps, int64_t stride);
 int launch_moe_combine(float* x, const float* part, const float* gate, int k, int n, int n_tokens);
+// gathered down projection of one token's k experts and the mixture into x[dm] in one launch (Q8_0 bank, k <= 8; mid: [k][cols])
+bool moe_down_mix_supported(const cai_qw_s* w, int dm, int k);
+int launch_moe_down_mix(const cai_qw_s* w, int dm, const float* mid, const int32_t* experts, const float* gates, int k, float* x);
 int launch_split_blocks(const uint8_t* raw, int block_bytes, int64_t n_blocks, uint8_t* qs, uint16_t* d);
 int launch_split_q6k(const uint8_t* raw, int64_t n_blocks, uint8_t* rec, uint8_t* sc, uint16_t* d);
 // qkv: [n_seq][qkv_stride] rows [Q|K|V]; theta != null applies interleaved RoPE to Q and K first.  pos_dev[s] is

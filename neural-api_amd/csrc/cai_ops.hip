@@ -303,6 +303,82 @@ int launch_moe_combine(float* x, const float* part, const float* gate, int k, in
   return CAI_OK;
 }
 
+// Gathered down projection and the gate-weighted mixture of a token in ONE launch (Q8_0 expert bank, up to 8 selected experts):
+// a wave takes R output rows for ALL selected experts - the R x k weight rows (a lane 16 values of each per 1024 columns), the
+// k SwiGLU rows and the gates are requested together, one round trip behind the expert ids - and adds
+// sum_j gate_j * (row of expert j . mid_j) to the residual row in place (neural/neuralpretrained.pas:15372-15388).  Takes the
+// place of the gathered matrix-vector launch, its k partial rows and the mixture launch.
+template <int R>
+__global__ __launch_bounds__(256) void moe_down_mix_kernel(const int8_t* wq, const __half* wsc, const int bank_experts, const int dm, const int cols,
+                                                           const float* mid, const int32_t* experts, const float* gates, const int k, float* x)
+{
+  const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+  const int row0 = (blockIdx.x * 4 + w) * R;
+  if (row0 >= dm) return;               // (no barrier in this kernel)
+  int e[8]; float g[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    const int jj = min(j, k - 1);
+    e[j] = min(max(experts[jj], 0), bank_experts - 1);      // an id outside the bank (a router fed NaN) must not address memory
+    g[j] = j < k ? gates[jj] : 0.0f;
+  }
+  const int nblk = cols >> 5;
+  float acc[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) acc[r] = 0.0f;
+  for (int c0 = 0; c0 < cols; c0 += 1024) {
+    const bool on = c0 + 16 * lane < cols;
+    const int col = on ? c0 + 16 * lane : 0;
+    uint4 q[8][R]; float sc[8][R]; float4 xv[8][4];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+#pragma unroll
+      for (int r = 0; r < R; r++) {
+        const int64_t row = (int64_t)e[j] * dm + min(row0 + r, dm - 1);
+        q[j][r] = *reinterpret_cast<const uint4*>(wq + row * cols + col);
+        sc[j][r] = __half2float(wsc[row * nblk + (col >> 5)]);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; u++) xv[j][u] = reinterpret_cast<const float4*>(mid + (int64_t)min(j, k - 1) * cols + col)[u];
+    }
+    if (on) {
+#pragma unroll
+      for (int j = 0; j < 8; j++)
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          const int c4[4] = {(int)q[j][r].x, (int)q[j][r].y, (int)q[j][r].z, (int)q[j][r].w};
+          float d = 0.0f;
+#pragma unroll
+          for (int u = 0; u < 4; u++) {
+            d = fmaf(xv[j][u].x, (float)((c4[u] << 24) >> 24), d); d = fmaf(xv[j][u].y, (float)((c4[u] << 16) >> 24), d);
+            d = fmaf(xv[j][u].z, (float)((c4[u] << 8) >> 24), d); d = fmaf(xv[j][u].w, (float)(c4[u] >> 24), d);
+          }
+          acc[r] = fmaf(g[j] * sc[j][r], d, acc[r]);
+        }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    float a = acc[r];
+    for (int m = 32; m >= 1; m >>= 1) a += __shfl_xor(a, m, 64);
+    if (lane == 0 && row0 + r < dm) x[row0 + r] += a;
+  }
+}
+bool moe_down_mix_supported(const cai_qw_s* w, int dm, int k)
+{
+  static const bool off = []() { const char* e = getenv("CAIHIP_MOE_DOWN_LAUNCHES"); return e && e[0] == '1'; }();   // keep the two launches
+  return !off && w->qtype == CAI_Q8_0 && !w->bias && k >= 1 && k <= 8 && dm > 0 && w->rows % dm == 0 && w->cols % 32 == 0;
+}
+int launch_moe_down_mix(const cai_qw_s* w, int dm, const float* mid, const int32_t* experts, const float* gates, int k, float* x)
+{
+  if (!moe_down_mix_supported(w, dm, k)) return set_error(CAI_ERR_UNSUPPORTED, "moe: the one-launch down projection takes a Q8_0 bank and up to 8 selected experts");
+  if ((reinterpret_cast<uintptr_t>(mid) | reinterpret_cast<uintptr_t>(w->data)) & 15) return set_error(CAI_ERR_INVALID, "moe: rows must be 16-byte aligned");
+  constexpr int R = 2;
+  hipLaunchKernelGGL(moe_down_mix_kernel<R>, dim3((unsigned)((dm + 4 * R - 1) / (4 * R))), dim3(256), 0, ctx().stream, (const int8_t*)w->data, (const __half*)w->aux,
+                     (int)(w->rows / dm), dm, (int)w->cols, mid, experts, gates, k, x);
+  return CAI_OK;
+}
+
 // ---- ArgMaxRow (neural/neuralchatengine.pas:683-697): strict >, lowest index wins ties ----
 // Two stages: work-groups scan 4096-element slices, then one work-group folds the slice winners.
 __device__ __forceinline__ bool argmax_better(float v, int i, float bv, int bi) { return bi < 0 || v > bv || (v == bv && i < bi); }
@@ -384,10 +460,50 @@ __device__ __forceinline__ uint32_t router_key(float p, bool candidate)
   if (!(p == p)) return 1u;
   return __builtin_bit_cast(uint32_t, fmaxf(p, 0.0f)) + 2u;
 }
+// Soft-max over n <= 64 logits and the k largest probabilities, by ONE wave (lane i owns expert i and brings its logit): every lane ranks its own
+// probability against the 64 broadcast ones (larger first, lower index between equals) - a permutation of 0..63 - and the lanes
+// of rank 0..k-1 are the selection, in order.  Returns the probability of the lane's expert; lane j < k gets the j-th selected
+// expert and its gate (divided by the sum of the k selected when renorm is set).
+__device__ __forceinline__ float router_select64(float logit, int n, int k, int renorm, int lane, int& expert_j, float& gate_j)
+{
+  float v = lane < n ? logit : -3.0e38f;
+  float mx = v;
+  for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+  float a = v - mx; a = a > 4000.0f ? 4000.0f : (a < -4000.0f ? -4000.0f : a);
+  v = lane < n ? expf(a) : 0.0f;
+  float tot = v;
+  for (int m = 32; m >= 1; m >>= 1) tot += __shfl_xor(tot, m, 64);
+  const float inv = tot > 0.0f ? 1.0f / tot : 1.0f;
+  v *= inv;
+  const float pv = lane < n ? v : -1.0f;      // -1 marks "not a candidate"
+  const uint32_t key = router_key(pv, lane < n);
+  int rank = 0;
+  for (int j = 0; j < 64; j++) {
+    const uint32_t o = (uint32_t)__builtin_amdgcn_readlane((int)key, j);
+    rank += (o > key || (o == key && j < lane)) ? 1 : 0;
+  }
+  float sum = 0.0f, mine = 0.0f;
+  expert_j = 0;
+  for (int j = 0; j < k; j++) {
+    const int src = __ffsll((unsigned long long)__ballot(rank == j)) - 1;
+    const float bv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pv), src));
+    if (lane == j) { mine = bv; expert_j = src; }
+    sum += bv;
+  }
+  gate_j = renorm ? (sum > 0.0f ? mine * (1.0f / sum) : 0.0f) : mine;
+  return v;
+}
 __global__ __launch_bounds__(64) void router_topk_kernel(const float* logits, int n, int k, int renorm, int n_tokens, int32_t* expert_out, float* gate_out, float* probs)
 {
   const int t = blockIdx.x, lane = threadIdx.x;
   const float* x = logits + (int64_t)t * n;
+  if (n <= 64) {     // one expert per lane
+    int ej; float gj;
+    const float pr = router_select64(lane < n ? x[lane] : 0.0f, n, k, renorm, lane, ej, gj);
+    if (lane < n) probs[(int64_t)t * n + lane] = pr;
+    if (lane < k) { expert_out[t * k + lane] = ej; gate_out[t * k + lane] = gj; }
+    return;
+  }
   float v[ROUTER_MAX_PER_LANE];
   float mx = -3.0e38f;
 #pragma unroll
@@ -414,25 +530,6 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float* logits, in
     if (c < n) probs[(int64_t)t * n + c] = v[i]; else v[i] = -1.0f;   // -1 marks "not a candidate"
   }
   float sum = 0.0f, mine = 0.0f;   // lane j keeps the j-th selected gate
-  if (n <= 64) {
-    // One expert per lane: every lane ranks its own probability against the 64 broadcast ones (larger first, lower
-    // index between equals) - a permutation of 0..63 - and the lanes of rank 0..k-1 are the selection, in order.
-    const float pv = v[0];
-    const uint32_t key = router_key(pv, lane < n);
-    int rank = 0;
-    for (int j = 0; j < 64; j++) {
-      const uint32_t o = (uint32_t)__builtin_amdgcn_readlane((int)key, j);
-      rank += (o > key || (o == key && j < lane)) ? 1 : 0;
-    }
-    for (int j = 0; j < k; j++) {
-      const int src = __ffsll((unsigned long long)__ballot(rank == j)) - 1;
-      const float bv = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, pv), src));
-      if (lane == j) { mine = bv; expert_out[t * k + j] = src; }
-      sum += bv;
-    }
-    if (lane < k) gate_out[t * k + lane] = renorm ? (sum > 0.0f ? mine * (1.0f / sum) : 0.0f) : mine;
-    return;
-  }
   uint32_t key[ROUTER_MAX_PER_LANE];
 #pragma unroll
   for (int i = 0; i < ROUTER_MAX_PER_LANE; i++) key[i] = router_key(v[i], lane + 64 * i < n);
@@ -459,6 +556,84 @@ int launch_router_topk(const float* logits, int n, int k, int renorm, int n_toke
 {
   if (n < 1 || n > 64 * ROUTER_MAX_PER_LANE || k < 1 || k > 64 || k > n) return set_error(CAI_ERR_UNSUPPORTED, "router: %d experts, top-%d (supported: up to %d experts, k <= 64)", n, k, 64 * ROUTER_MAX_PER_LANE);
   hipLaunchKernelGGL(router_topk_kernel, dim3(n_tokens), dim3(64), 0, ctx().stream, logits, n, k, renorm, n_tokens, expert_out, gate_out, probs_scratch);
+  return CAI_OK;
+}
+
+// The router of up to 64 experts in ONE launch: a work-group of four waves per four experts and token (one work-group for all
+// the rows measured slower than the two launches it replaced: a single CU streams the 128 KB of a 64 x 2048 router at about
+// 20 GB/s).  Every wave sums the squares of the row itself (no meeting before the products), takes one Q8_0 router row (a lane
+// one 32-value block per 2048 columns; the factor 1 / rms multiplies the finished sum) and stores its logit at agent scope; the
+// work-group that arrives last (wrapping counter per token, the hand-over of the attention merge: agent-scope stores
+// acknowledged under vmcnt(0), work-group barrier, agent-scope increment, agent-scope loads) selects (router_select64).  Takes the
+// place of the matrix-vector launch and the selection launch of a decode step (TNNetPointwiseSoftMax + TNNetTopKGate behind the
+// router's TNNetPointwiseConvLinear, neural/neuralpretrained.pas:15331-15348).
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(CAI_MERGE_RELACQ) && !defined(__gfx950__) && !defined(__gfx942__)
+#error "router_fused_kernel: the relaxed hand-over is only valid on gfx942 / gfx950; build with -DCAI_MERGE_RELACQ"
+#endif
+__global__ __launch_bounds__(256) void router_fused_kernel(const float* x, const long long x_stride, const float* gain, const float eps,
+                                                           const int8_t* wq, const __half* wsc, const int n, const int cols, const int k, const int renorm,
+                                                           float* logits_out, int32_t* expert_out, float* gate_out, float* probs, unsigned* counters)
+{
+  __shared__ int s_is_last;
+  const int t = blockIdx.y, tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int r_own = blockIdx.x * 4 + w, r = min(r_own, n - 1);
+  const float* xb = x + (int64_t)t * x_stride;
+  const int nblk = cols >> 5;
+  float acc = 0.0f, ss = 0.0f;
+  for (int c0 = 0; c0 < nblk; c0 += 64) {
+    const bool on = c0 + lane < nblk;
+    const int blk = on ? c0 + lane : nblk - 1;
+    const uint4* src = reinterpret_cast<const uint4*>(wq + (int64_t)r * cols + 32 * blk);
+    const uint4 q0 = src[0], q1 = src[1];
+    const float sc = __half2float(wsc[(int64_t)r * nblk + blk]);
+    const uint32_t wd[8] = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+    float d = 0.0f;
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+      const float4 v = reinterpret_cast<const float4*>(xb + 32 * blk)[q], g = reinterpret_cast<const float4*>(gain + 32 * blk)[q];
+      const float xv[4] = {on ? v.x : 0.0f, on ? v.y : 0.0f, on ? v.z : 0.0f, on ? v.w : 0.0f};
+      const int c4 = (int)wd[q];
+      ss = fmaf(xv[0], xv[0], ss); ss = fmaf(xv[1], xv[1], ss); ss = fmaf(xv[2], xv[2], ss); ss = fmaf(xv[3], xv[3], ss);
+      d = fmaf(g.x * xv[0], (float)((c4 << 24) >> 24), d); d = fmaf(g.y * xv[1], (float)((c4 << 16) >> 24), d);
+      d = fmaf(g.z * xv[2], (float)((c4 << 8) >> 24), d); d = fmaf(g.w * xv[3], (float)(c4 >> 24), d);
+    }
+    acc = fmaf(d, sc, acc);
+  }
+  for (int m = 32; m >= 1; m >>= 1) { ss += __shfl_xor(ss, m, 64); acc += __shfl_xor(acc, m, 64); }
+  const float logit = acc * (1.0f / sqrtf(ss / (float)cols + eps));
+  if (lane == 0 && r_own < n) __hip_atomic_store(logits_out + (int64_t)t * n + r_own, logit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): the logit store has been acknowledged
+  __syncthreads();
+  if (tid == 0)
+#ifdef CAI_MERGE_RELACQ
+    s_is_last = __builtin_amdgcn_atomic_inc32(counters + t, gridDim.x - 1, __ATOMIC_RELEASE, "agent") == gridDim.x - 1;
+#else
+    s_is_last = __builtin_amdgcn_atomic_inc32(counters + t, gridDim.x - 1, __ATOMIC_RELAXED, "agent") == gridDim.x - 1;
+#endif
+  __syncthreads();
+  if (!s_is_last || w != 0) return;
+#ifdef CAI_MERGE_RELACQ
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#endif
+  const float lg = __hip_atomic_load(logits_out + (int64_t)t * n + min(lane, n - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  int ej; float gj;
+  const float pr = router_select64(lg, n, k, renorm, lane, ej, gj);
+  if (lane < n) probs[(int64_t)t * n + lane] = pr;
+  if (lane < k) { expert_out[t * k + lane] = ej; gate_out[t * k + lane] = gj; }
+}
+
+bool router_fused_supported(const cai_qw_s* w, int k)
+{
+  static const bool off = []() { const char* e = getenv("CAIHIP_ROUTER_LAUNCHES"); return e && e[0] == '1'; }();   // keep the two launches
+  return !off && w->qtype == CAI_Q8_0 && !w->bias && w->rows >= 1 && w->rows <= 64 && k >= 1 && k <= w->rows && w->cols % 32 == 0;
+}
+int launch_router_fused(const cai_qw_s* w, const float* x, int64_t x_stride, const float* gain, float eps, int k, int renorm, int n_tokens,
+                        float* logits_out, int32_t* expert_out, float* gate_out, float* probs_scratch, unsigned* counters)
+{
+  if (!router_fused_supported(w, k) || !gain || !counters) return set_error(CAI_ERR_UNSUPPORTED, "router: the one-launch form takes a Q8_0 router of up to 64 experts with a norm gain");
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gain) | (uintptr_t)(x_stride * 4)) & 15) return set_error(CAI_ERR_INVALID, "router: activation rows and gain must be 16-byte aligned");
+  hipLaunchKernelGGL(router_fused_kernel, dim3((unsigned)((w->rows + 3) / 4), n_tokens), dim3(256), 0, ctx().stream, x, (long long)x_stride, gain, eps, (const int8_t*)w->data, (const __half*)w->aux,
+                     (int)w->rows, (int)w->cols, k, renorm, logits_out, expert_out, gate_out, probs_scratch, counters);
   return CAI_OK;
 }
 

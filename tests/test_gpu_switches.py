@@ -59,6 +59,41 @@ def test_switch_selected_path_matches_the_oracle(switches):
     assert r.returncode == 0 and "CHILD_OK" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
 
 
+MOE_CHILD = r"""
+import sys
+import numpy as np
+sys.path.insert(0, %(root)r); sys.path.insert(0, %(tests)r)
+from helpers import oracle_lib as O
+from helpers.model_build import oracle_model, synthetic_spec
+from helpers.device import dev, rel_err
+cai = dev()
+# 16 KV heads x 16 slices of 64 rows = 256 work-groups: the decode attention of this cache is the one-work-group-per-KV-head kernel
+cfg = dict(n_layers=2, d_model=256, n_q_heads=32, n_kv_heads=16, head_dim=128, ffn=96, vocab=512, max_ctx=1024, eps=1e-5, rope_theta=1e4,
+           n_experts=8, top_k=3, norm_topk=1)
+spec = synthetic_spec(cfg, O.Q8_0, std=0.05)
+om, dec = oracle_model(spec, kv_f16=1), cai.Decoder(spec, kv_dtype=cai.KV_F16)
+prompt = np.random.default_rng(11).integers(0, cfg["vocab"], 70).tolist()      # crosses a slice boundary
+for p, t in enumerate(prompt):
+    tok_o, lo = om.step(t, p)
+    tok_d, ld = dec.step(np.array([t]), np.array([p]))
+    assert rel_err(ld[0], lo) < 1e-3, (p, rel_err(ld[0], lo))
+    assert int(tok_d[0]) == tok_o, p
+print("CHILD_OK")
+"""
+
+
+@pytest.mark.parametrize("switches", [{}, {"CAIHIP_ATTN_GROUP_MFMA": "0"}, {"CAIHIP_ROUTER_LAUNCHES": "1"}, {"CAIHIP_MOE_DOWN_LAUNCHES": "1"}])
+def test_moe_fp16_cache_paths_match_the_oracle(switches):
+    """A Q8_0 mixture-of-experts decoder over a half-precision cache, token by token against the oracle: by default the grouped
+    decode attention runs on the matrix cores, the router is one launch (products, soft-max and top-k; the last work-group to
+    arrive selects) and the gathered down projection adds the gate-weighted mixture itself; each switch puts one of the three back
+    on its separate launches."""
+    env = dict(os.environ); env.update(switches)
+    code = MOE_CHILD % dict(root=ROOT, tests=os.path.join(ROOT, "tests"))
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "CHILD_OK" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
+
+
 SHUTDOWN_CHILD = r"""
 import sys, importlib
 import numpy as np
