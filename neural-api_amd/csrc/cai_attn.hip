@@ -244,6 +244,29 @@ __device__ __forceinline__ void unpack8(const Row8<int8_t>& r, float (&v)[8])
   }
 }
 
+// wave64 maximum / sum in every lane: DPP steps inside the vector unit (row_shr within rows of 16, row_bcast15 / row_bcast31,
+// total in lane 63, broadcast through a scalar register) instead of six trips through the LDS crossbar
+__device__ __forceinline__ float wave_allmax(float v)
+{
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, false)));
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x112, 0xf, 0xf, false)));
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x114, 0xf, 0xf, false)));
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x118, 0xf, 0xf, false)));
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x142, 0xa, 0xf, false)));
+  v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v), 0x143, 0xc, 0xf, false)));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+__device__ __forceinline__ float wave_allsum(float v)
+{
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wave_sum(v)), 63));
+}
+// gfx950 row swaps (a row = 16 lanes).  row_swap16: rows 1, 3 of x change places with rows 0, 2 of y, i.e. x = (x0 y0 x2 y2),
+// y = (x1 y1 x3 y3); row_swap32: the upper half of x with the lower half of y, i.e. x = (x0 x1 y0 y1), y = (x2 x3 y2 y3).
+// Written as instructions: through the builtins this compiler read BOTH results from the first register (sums came out as
+// 2 x the first result).  The instruction needs two idle cycles after a vector write of its operands, which the compiler
+// cannot see inside the statement: the s_nop provides them.
+__device__ __forceinline__ void row_swap16(float& x, float& y) { asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x), "+v"(y)); }
+__device__ __forceinline__ void row_swap32(float& x, float& y) { asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x), "+v"(y)); }
 // sum over each aligned group of 16 lanes, result in every lane of the group
 __device__ __forceinline__ float row16_allsum(float v)
 {
@@ -410,14 +433,14 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const int32_t* hpos, co
     if (p.softcap > 0.0f)
       for (int rl = lane; rl < n_rows; rl += 64) sS[h * SL + rl] = p.softcap * tanhf(sS[h * SL + rl] / p.softcap);
     for (int rl = lane; rl < n_rows; rl += 64) m = fmaxf(m, sS[h * SL + rl]);
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    m = wave_allmax(m);
     float l = 0.0f;
     for (int rl = lane; rl < n_rows; rl += 64) {
       const float e = expf(sS[h * SL + rl] - m);
       l += e;
       sP[((h / HC) * SL + rl) * PW + h % HC] = I8 ? e * vsc[s_begin + rl] : e;
     }
-    for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
+    l = wave_allsum(l);
     if (lane == 0) { sML[h] = m; sML[G + h] = l; }
   }
   __syncthreads();
@@ -455,16 +478,26 @@ __global__ __launch_bounds__(256) void attn_group_kernel(const int32_t* hpos, co
         }
       }
     }
-    // the wave's 4 row groups, then the 4 waves
+    // The wave's 4 row groups (rows of 16 lanes), then the 4 waves.  A transposing sum: the row-swap instructions of gfx950 turn
+    // two registers into (row 0+1 | 2+3 of the first, of the second), then four into one whose row r holds the total of value
+    // 4 q + r - (r0 + r1) + (r2 + r3) as a butterfly over lanes ^16, ^32 would give, in 1.5 instructions per value instead of
+    // two LDS-crossbar permutes and two additions, and with one store per four values (the butterfly form took 3.8 of the
+    // launch's 15 us at batch 8).
 #pragma unroll
-    for (int hh = 0; hh < HC; hh++)
+    for (int q4 = 0; q4 < 2 * HC; q4++) {
+      float s2[2];
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        float a = acc[hh][i];
-        a += __shfl_xor(a, 16, 64);
-        a += __shfl_xor(a, 32, 64);
-        if (r == 0 && lane_on) sred[(w * HC + hh) * 128 + d0 + i] = a;
+      for (int hf = 0; hf < 2; hf++) {
+        const int n = 4 * q4 + 2 * hf;
+        float x = acc[n >> 3][n & 7], y = acc[(n + 1) >> 3][(n + 1) & 7];
+        row_swap16(x, y);
+        s2[hf] = x + y;                 // rows: x0+x1 | y0+y1 | x2+x3 | y2+y3
       }
+      row_swap32(s2[0], s2[1]);
+      const float tot = s2[0] + s2[1];  // row r: total of value 4 q4 + r
+      const int n = 4 * q4 + r;
+      if (lane_on) sred[(w * HC + (n >> 3)) * 128 + d0 + (n & 7)] = tot;
+    }
     __syncthreads();
     for (int o = tid; o < HC * hd; o += 256) {
       const int hh = o / hd, d = o % hd, h = h0 + hh;
