@@ -540,17 +540,30 @@ constexpr int gm_lds_bytes(int tpw, int nw) { return GM_FIXED + nw * tpw * 16 * 
 
 // TPW 16-row tiles per wave, NW waves: 2 x 4 (slices of up to 128 rows) or 2 x 8 (up to 256: two waves per SIMD overlap each
 // other's dependent LDS / matrix-core / soft-max chains)
-template <int TPW, int NW>
+// KV_T = int8_t: the codes become f16 exactly on their way into the operands (byte ^ 0x80 under a 0x64 exponent byte = 1152 + code,
+// one packed subtraction: 1.25 instructions per element), the K row scale multiplies the finished score and the V row scale the
+// soft-max weight before its hi + lo split, as in the VALU kernels (neural/neural.cl:2639-2640, 2683-2684).
+__device__ __forceinline__ ph8_t gm_codes_to_halfs(uint32_t w0, uint32_t w1)
+{
+  typedef _Float16 gh2_t __attribute__((ext_vector_type(2)));
+  const uint32_t x0 = w0 ^ 0x80808080u, x1 = w1 ^ 0x80808080u, K = 0x64646464u;
+  const gh2_t off = {(_Float16)1152.0f, (_Float16)1152.0f};
+  const gh2_t a = __builtin_bit_cast(gh2_t, __builtin_amdgcn_perm(K, x0, 0x04010400u)) - off, b = __builtin_bit_cast(gh2_t, __builtin_amdgcn_perm(K, x0, 0x04030402u)) - off;
+  const gh2_t c = __builtin_bit_cast(gh2_t, __builtin_amdgcn_perm(K, x1, 0x04010400u)) - off, d = __builtin_bit_cast(gh2_t, __builtin_amdgcn_perm(K, x1, 0x04030402u)) - off;
+  return ph8_t{a.x, a.y, b.x, b.y, c.x, c.y, d.x, d.y};
+}
+template <int TPW, int NW, typename KV_T>
 __global__ __launch_bounds__(64 * NW) void attn_group_mfma_kernel(const int32_t* hpos, const float* hqkv, const float* htheta, const long long hqkv_stride,
                                                               const int hheads, const int hgeo, const int hsl, const AttnParams p)
 {
   const unsigned long long tl0 = timeline_now();
   const int h_q_heads = hheads & 0xffff, h_kv_heads = hheads >> 16, h_n_splits = hgeo & 0xffff;
   constexpr int hd = 128;
+  constexpr bool I8 = sizeof(KV_T) == 1;
   extern __shared__ __align__(16) unsigned char glds[];
   _Float16* sqh = reinterpret_cast<_Float16*>(glds);
   _Float16* sql = sqh + 16 * GM_LD;
-  _Float16* snew = sql + 16 * GM_LD;                           // [K | V][128]
+  _Float16* snew = sql + 16 * GM_LD;                           // [K | V][128] (int8: the codes as bytes, then the two row scales at byte 256)
   float* sML = reinterpret_cast<float*>(snew + 256);           // [wave][head][maximum, sum]
   constexpr int REGION = TPW * 16 * GM_LD * 2;                 // bytes of a wave's V tiles (later: its [head][128] float sums)
   const int G = h_q_heads / h_kv_heads;
@@ -569,15 +582,20 @@ __global__ __launch_bounds__(64 * NW) void attn_group_mfma_kernel(const int32_t*
   }
   const int SL = hsl, base = split * SL;
   const int64_t cache_seq = seq * p.seq_mul + p.seq0;
-  __half* kc = reinterpret_cast<__half*>(p.kc) + cache_seq * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
-  __half* vc = reinterpret_cast<__half*>(p.vc) + cache_seq * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  KV_T* kc = reinterpret_cast<KV_T*>(p.kc) + cache_seq * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  KV_T* vc = reinterpret_cast<KV_T*>(p.vc) + cache_seq * p.seq_elems + p.layer_off + (int64_t)g * p.max_ctx * hd;
+  float* ksc = nullptr; float* vsc = nullptr;
+  if (I8) { const int64_t r0 = cache_seq * p.seq_rows + p.layer_row_off + (int64_t)g * p.max_ctx; ksc = p.ksc + r0; vsc = p.vsc + r0; }
+  // contraction slots of a lane group: half cache dims 32 s + 8 kg .., int8 cache dims 32 kg + 8 s .. (a lane's 32 codes of a row are
+  // two 16-byte requests)
+  constexpr int KCH = I8 ? 2 : 4;          // 16-byte requests per lane and K tile
   // The wave's first K tile is requested before the position is known (its rows exist whatever the position: the slice lies
   // inside the cache; rows past the live range are masked), so the stream starts while the position is still on its way.
   uint4 kreg[TPW][4], vreg[TPW][4];
   {
     const int j = min(base + 16 * w + n16, p.max_ctx - 1);
 #pragma unroll
-    for (int s4 = 0; s4 < 4; s4++) kreg[0][s4] = *reinterpret_cast<const uint4*>(kc + (int64_t)j * hd + 32 * s4 + 8 * kg);
+    for (int s4 = 0; s4 < KCH; s4++) kreg[0][s4] = *reinterpret_cast<const uint4*>(kc + (int64_t)j * hd + (I8 ? 32 * kg + 16 * s4 : 32 * s4 + 8 * kg));
   }
   const LiveRows lr = live_rows(p, pos);
   const int len = lr.len, j_start = lr.j_start, slot = lr.slot;
@@ -597,20 +615,32 @@ __global__ __launch_bounds__(64 * NW) void attn_group_mfma_kernel(const int32_t*
     for (int i = 0; i < 4; i++) nraw[i] = src[i];
     if (htheta) { nth[0] = htheta[e0 >> 1]; nth[1] = htheta[(e0 >> 1) + 1]; }
   }
+  // int8: the scales of the rows whose scores this lane will hold (rows 4 kg .. 4 kg + 3 of every tile), in front of the rows
+  float ks4[TPW][4], vs4[TPW][4];
+#pragma unroll
+  for (int t = 0; t < TPW; t++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int j = min(base + 16 * (w + NW * t) + 4 * kg + i, s_end - 1);
+      ks4[t][i] = I8 ? ksc[j] : 1.0f; vs4[t][i] = I8 ? vsc[j] : 1.0f;
+    }
   // every other row of the wave's tiles, K first (the first product starts while V is still on its way).
   // Rows past the live range repeat its last row and are masked below.
 #pragma unroll
   for (int t = 1; t < TPW; t++) {
     const int j = min(base + 16 * (w + NW * t) + n16, s_end - 1);
 #pragma unroll
-    for (int s4 = 0; s4 < 4; s4++) kreg[t][s4] = *reinterpret_cast<const uint4*>(kc + (int64_t)j * hd + 32 * s4 + 8 * kg);
+    for (int s4 = 0; s4 < KCH; s4++) kreg[t][s4] = *reinterpret_cast<const uint4*>(kc + (int64_t)j * hd + (I8 ? 32 * kg + 16 * s4 : 32 * s4 + 8 * kg));
   }
+  // V rows as they lie in memory: half cache 4 rows x 256 bytes per request, int8 cache 8 rows x 128 bytes
+  constexpr int VCH = I8 ? 2 : 4, VROWS = I8 ? 8 : 4;
+  const int vrow = I8 ? lane >> 3 : kg, vcol = I8 ? 16 * (lane & 7) : 8 * n16;
 #pragma unroll
   for (int t = 0; t < TPW; t++)
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int j = min(base + 16 * (w + NW * t) + 4 * i + kg, s_end - 1);
-      vreg[t][i] = *reinterpret_cast<const uint4*>(vc + (int64_t)j * hd + 8 * n16);
+    for (int i = 0; i < VCH; i++) {
+      const int j = min(base + 16 * (w + NW * t) + VROWS * i + vrow, s_end - 1);
+      vreg[t][i] = *reinterpret_cast<const uint4*>(vc + (int64_t)j * hd + vcol);
     }
   timeline_put(p.timeline, 0, tl0);
   timeline_stamp(p.timeline, 1);
@@ -634,23 +664,34 @@ __global__ __launch_bounds__(64 * NW) void attn_group_mfma_kernel(const int32_t*
     sqh[h * GM_LD + 2 * i] = h0; sqh[h * GM_LD + 2 * i + 1] = h1;
     sql[h * GM_LD + 2 * i] = l0; sql[h * GM_LD + 2 * i + 1] = l1;
   }
-  // the new row: rotated, rounded to the cache's precision, stored, and kept in LDS for this work-group's own products (its
-  // requests for that row went out before the store)
+  // the new row: rotated, rounded to the cache's precision (int8: quantised, neural/neural.cl:2501-2580), stored, and kept in LDS for
+  // this work-group's own products (its requests for that row went out before the store)
   if (owns_new && w == 0) {
     const int l32 = lane & 31, is_v = lane >> 5, e0 = 4 * l32;
-    __half* dst = (is_v ? vc : kc) + (int64_t)slot * hd;
+    KV_T* dst = (is_v ? vc : kc) + (int64_t)slot * hd;
+    float v4[4];
 #pragma unroll
     for (int i = 0; i < 4; i += 2) {
-      const int d = e0 + i;
       float x0 = nraw[i], x1 = nraw[i + 1];
       if (htheta && !is_v) {
         float sn, cs; sincosf((float)pos * nth[i >> 1], &sn, &cs);
         const float y0 = cs * x0 - sn * x1, y1 = sn * x0 + cs * x1;
         x0 = y0; x1 = y1;
       }
-      const __half r0 = __float2half_rn(x0), r1 = __float2half_rn(x1);
-      dst[d] = r0; dst[d + 1] = r1;
-      snew[is_v * 128 + d] = __builtin_bit_cast(_Float16, r0); snew[is_v * 128 + d + 1] = __builtin_bit_cast(_Float16, r1);
+      v4[i] = x0; v4[i + 1] = x1;
+    }
+    if constexpr (I8) {
+      const float scale = quantise_row_i8<4>(v4);
+      int8_t* sb = reinterpret_cast<int8_t*>(snew);
+#pragma unroll
+      for (int i = 0; i < 4; i++) { dst[e0 + i] = (int8_t)v4[i]; sb[is_v * 128 + e0 + i] = (int8_t)v4[i]; }
+      if (l32 == 0) { (is_v ? vsc : ksc)[slot] = scale; reinterpret_cast<float*>(snew + 128)[is_v] = scale; }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const __half r = __float2half_rn(v4[i]);
+        dst[e0 + i] = r; snew[is_v * 128 + e0 + i] = __builtin_bit_cast(_Float16, r);
+      }
     }
   }
   __syncthreads();
@@ -659,8 +700,8 @@ __global__ __launch_bounds__(64 * NW) void attn_group_mfma_kernel(const int32_t*
   ph8_t qh8[4], ql8[4];
 #pragma unroll
   for (int s4 = 0; s4 < 4; s4++) {
-    qh8[s4] = *reinterpret_cast<const ph8_t*>(sqh + n16 * GM_LD + 32 * s4 + 8 * kg);
-    ql8[s4] = *reinterpret_cast<const ph8_t*>(sql + n16 * GM_LD + 32 * s4 + 8 * kg);
+    qh8[s4] = *reinterpret_cast<const ph8_t*>(sqh + n16 * GM_LD + (I8 ? 32 * kg + 8 * s4 : 32 * s4 + 8 * kg));
+    ql8[s4] = *reinterpret_cast<const ph8_t*>(sql + n16 * GM_LD + (I8 ? 32 * kg + 8 * s4 : 32 * s4 + 8 * kg));
   }
   if (owns_new) {
     // the new row from LDS in place of what memory held; rows past the live range may be memory that was never written (the
@@ -670,17 +711,23 @@ __global__ __launch_bounds__(64 * NW) void attn_group_mfma_kernel(const int32_t*
     for (int t = 0; t < TPW; t++) {
       const int r0 = 16 * (w + NW * t);
       if (rs >= r0 && rs < r0 + 16) {
+        const unsigned char* sb = reinterpret_cast<const unsigned char*>(snew);
         if (n16 == rs - r0) {
 #pragma unroll
-          for (int s4 = 0; s4 < 4; s4++) kreg[t][s4] = *reinterpret_cast<const uint4*>(snew + 32 * s4 + 8 * kg);
+          for (int s4 = 0; s4 < KCH; s4++) kreg[t][s4] = *reinterpret_cast<const uint4*>(sb + (I8 ? 32 * kg + 16 * s4 : 2 * (32 * s4 + 8 * kg)));
         }
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-          if (4 * i + kg == rs - r0) vreg[t][i] = *reinterpret_cast<const uint4*>(snew + 128 + 8 * n16);
+        for (int i = 0; i < VCH; i++)
+          if (VROWS * i + vrow == rs - r0) vreg[t][i] = *reinterpret_cast<const uint4*>(sb + (I8 ? 128 + vcol : 2 * (128 + vcol)));
+        if (I8) {
+#pragma unroll
+          for (int i = 0; i < 4; i++)
+            if (4 * kg + i == rs - r0) { ks4[t][i] = reinterpret_cast<const float*>(snew + 128)[0]; vs4[t][i] = reinterpret_cast<const float*>(snew + 128)[1]; }
+        }
       }
 #pragma unroll
-      for (int i = 0; i < 4; i++)
-        if (base + r0 + 4 * i + kg >= s_end) vreg[t][i] = make_uint4(0u, 0u, 0u, 0u);
+      for (int i = 0; i < VCH; i++)
+        if (base + r0 + VROWS * i + vrow >= s_end) vreg[t][i] = make_uint4(0u, 0u, 0u, 0u);
     }
   }
 
@@ -692,7 +739,11 @@ __global__ __launch_bounds__(64 * NW) void attn_group_mfma_kernel(const int32_t*
     C[t] = gf4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int s4 = 0; s4 < 4; s4++) {
-      const ph8_t a = __builtin_bit_cast(ph8_t, kreg[t][s4]);
+      ph8_t a;
+      if constexpr (I8) {
+        const uint4 kq = kreg[t][s4 >> 1];
+        a = (s4 & 1) ? gm_codes_to_halfs(kq.z, kq.w) : gm_codes_to_halfs(kq.x, kq.y);
+      } else a = __builtin_bit_cast(ph8_t, kreg[t][s4]);
       C[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qh8[s4], C[t], 0, 0, 0);
       C[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, ql8[s4], C[t], 0, 0, 0);
     }
@@ -705,7 +756,7 @@ __global__ __launch_bounds__(64 * NW) void attn_group_mfma_kernel(const int32_t*
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int j = base + 16 * (w + NW * t) + 4 * kg + i;
-      float sc = C[t][i] * p.inv_sqrt;
+      float sc = C[t][i] * (I8 ? ks4[t][i] * p.inv_sqrt : p.inv_sqrt);
       if (p.softcap > 0.0f) sc = p.softcap * tanhf(sc / p.softcap);
       ok[t][i] = j >= s_begin && j < s_end;
       C[t][i] = sc;
@@ -728,7 +779,14 @@ __global__ __launch_bounds__(64 * NW) void attn_group_mfma_kernel(const int32_t*
 #pragma unroll
   for (int t = 0; t < TPW; t++)
 #pragma unroll
-    for (int i = 0; i < 4; i++) *reinterpret_cast<uint4*>(sV + (16 * t + 4 * i + kg) * GM_LD + 8 * n16) = vreg[t][i];
+    for (int i = 0; i < VCH; i++) {
+      if constexpr (I8) {
+        const uint4 vq = vreg[t][i];
+        _Float16* dstv = sV + (16 * t + 8 * i + vrow) * GM_LD + vcol;
+        *reinterpret_cast<ph8_t*>(dstv) = gm_codes_to_halfs(vq.x, vq.y);
+        *reinterpret_cast<ph8_t*>(dstv + 8) = gm_codes_to_halfs(vq.z, vq.w);
+      } else *reinterpret_cast<uint4*>(sV + (16 * t + 4 * i + kg) * GM_LD + 8 * n16) = vreg[t][i];
+    }
   gf4_t Oe[4], Oo[4];
 #pragma unroll
   for (int u = 0; u < 4; u++) { Oe[u] = gf4_t{0.0f, 0.0f, 0.0f, 0.0f}; Oo[u] = gf4_t{0.0f, 0.0f, 0.0f, 0.0f}; }
@@ -737,7 +795,11 @@ __global__ __launch_bounds__(64 * NW) void attn_group_mfma_kernel(const int32_t*
     // contraction slot e of this lane group = row 4 kg + (e & 3) of tile 2 b + (e >> 2), in both operands
     ph8_t ph, pl;
 #pragma unroll
-    for (int e = 0; e < 8; e++) { _Float16 hv, lv; split_f16(C[2 * b + (e >> 2)][e & 3] * 1024.0f, hv, lv); ph[e] = hv; pl[e] = lv; }
+    for (int e = 0; e < 8; e++) {
+      const int t = 2 * b + (e >> 2), i = e & 3;
+      const float pe = I8 ? (ok[t][i] ? C[t][i] * vs4[t][i] : 0.0f) : C[t][i];      // (a dead row's scale is whatever memory holds)
+      _Float16 hv, lv; split_f16(pe * 1024.0f, hv, lv); ph[e] = hv; pl[e] = lv;
+    }
 #pragma unroll
     for (int u = 0; u < 4; u++) {
       uint32_t wv[8];
@@ -1152,8 +1214,9 @@ static int launch_group(const AttnParams& p, int n_seq, hipStream_t st)
 static bool group_takes_mfma(const AttnParams& p, int dtype)
 {
   static const bool on = []() { const char* e = getenv("CAIHIP_ATTN_GROUP_MFMA"); return !(e && e[0] == '0'); }();
-  return on && dtype == CAI_KV_F16 && p.hd == 128 && p.q_heads / p.kv_heads <= 16 && p.split_len <= 256;
+  return on && (dtype == CAI_KV_F16 || dtype == CAI_KV_I8) && p.hd == 128 && p.q_heads / p.kv_heads <= 16 && p.split_len <= 256;
 }
+template <typename KV_T>
 static int launch_group_mfma(const AttnParams& p0, int n_seq, hipStream_t st)
 {
   AttnParams p = p0;
@@ -1163,8 +1226,8 @@ static int launch_group_mfma(const AttnParams& p0, int n_seq, hipStream_t st)
   const int hheads = p.q_heads | p.kv_heads << 16, hgeo = p.n_splits | p.hd << 16;
 #define CAI_GM_LAUNCH(TPWv, NWv) do { \
     static bool attr_done = false;      /* up to 80 KB of dynamic LDS */ \
-    if (!attr_done) { CAI_HIP(hipFuncSetAttribute((const void*)attn_group_mfma_kernel<TPWv, NWv>, hipFuncAttributeMaxDynamicSharedMemorySize, gm_lds_bytes(TPWv, NWv))); attr_done = true; } \
-    hipLaunchKernelGGL((attn_group_mfma_kernel<TPWv, NWv>), grid, dim3(64 * NWv), gm_lds_bytes(TPWv, NWv), st, p.pos, (const float*)p.qkv, p.theta, (long long)p.qkv_stride, hheads, hgeo, p.split_len, p); } while (0)
+    if (!attr_done) { CAI_HIP(hipFuncSetAttribute((const void*)attn_group_mfma_kernel<TPWv, NWv, KV_T>, hipFuncAttributeMaxDynamicSharedMemorySize, gm_lds_bytes(TPWv, NWv))); attr_done = true; } \
+    hipLaunchKernelGGL((attn_group_mfma_kernel<TPWv, NWv, KV_T>), grid, dim3(64 * NWv), gm_lds_bytes(TPWv, NWv), st, p.pos, (const float*)p.qkv, p.theta, (long long)p.qkv_stride, hheads, hgeo, p.split_len, p); } while (0)
   // slices of up to 128 rows: four waves; longer ones: eight (32B shape at 8.2k rows, slices of 256: 177.5 tok/s with four waves
   // of four tiles, 180.8 with eight waves of two at batch 1; 693.7 against 698.0 at batch 8)
   if (p.split_len <= 128) CAI_GM_LAUNCH(2, 4);
@@ -1663,7 +1726,7 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
   // one work-group per (slice, KV head) serving the whole group of query heads, or one per (slice, query head)
   // (the first fetches K and V once but has G times fewer work-groups: it needs a grid that fills the chip by itself)
   if (grouped && group_takes_mfma(p, kv->dtype))
-    rc = launch_group_mfma(p, n_seq, c.stream);
+    rc = kv->dtype == CAI_KV_I8 ? launch_group_mfma<int8_t>(p, n_seq, c.stream) : launch_group_mfma<__half>(p, n_seq, c.stream);
   else if (grouped)
     rc = kv->dtype == CAI_KV_I8 ? launch_group<int8_t>(p, n_seq, c.stream) : kv->dtype == CAI_KV_F16 ? launch_group<__half>(p, n_seq, c.stream) : launch_group<float>(p, n_seq, c.stream);
   else

@@ -94,6 +94,41 @@ def test_moe_fp16_cache_paths_match_the_oracle(switches):
     assert r.returncode == 0 and "CHILD_OK" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
 
 
+ATTN_CHILD = r"""
+import sys
+import numpy as np
+sys.path.insert(0, %(root)r); sys.path.insert(0, %(tests)r)
+from helpers.device import dev
+from test_gpu_attention import oracle_run, oracle_run_i8
+cai = dev()
+hq, hkv, dk, ctx, n = 40, 8, 128, 8192, 90          # 8 KV heads x 33 slices: the one-work-group-per-KV-head kernel
+rows = np.random.default_rng(5).standard_normal((n, (hq + 2 * hkv) * dk)).astype(np.float32)
+for kv, window, softcap in (("f16", 0, 0.0), ("i8", 70, 25.0)):
+    if kv == "i8":
+        want, (kq, vq, ks, vs) = oracle_run_i8(rows, hq, hkv, dk, n, window, softcap)
+    else:
+        want = oracle_run(rows, hq, hkv, dk, n, window, 1, softcap)
+    cache = cai.KVCache(1, hkv, dk, ctx, cai.KV_I8 if kv == "i8" else cai.KV_F16)
+    for pos in range(n):
+        got = cache.attn_decode(0, rows[pos], hq, window, softcap)
+        assert np.max(np.abs(got - want[pos])) < 1e-5 * max(1.0, np.max(np.abs(want[pos]))), (kv, pos)
+    if kv == "i8":
+        k, v, s_k, s_v = cache.export_layer(0)
+        np.testing.assert_array_equal(k, kq); np.testing.assert_array_equal(v, vq)
+        np.testing.assert_array_equal(s_k, ks); np.testing.assert_array_equal(s_v, vs)
+print("CHILD_OK")
+"""
+
+
+def test_grouped_attention_valu_form_under_its_switch():
+    """CAIHIP_ATTN_GROUP_MFMA=0: half-precision and int8 caches of 128-wide heads go back to the VALU form of the per-KV-head
+    decode kernel (the default takes them to the matrix-core form, tests/test_gpu_attention.py): same bar, int8 codes and scales exact."""
+    env = dict(os.environ); env["CAIHIP_ATTN_GROUP_MFMA"] = "0"
+    code = ATTN_CHILD % dict(root=ROOT, tests=os.path.join(ROOT, "tests"))
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "CHILD_OK" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
+
+
 SHUTDOWN_CHILD = r"""
 import sys, importlib
 import numpy as np
