@@ -384,3 +384,70 @@ def test_very_long_caches_many_slices(kvt, hq, hkv, ctx, n):
     assert kv.len(0) == n + 3
     with pytest.raises(cai.CaiError, match="limit 512"):
         cai.KVCache(1, 1, 128, 131072 + 256, cai.KV_F16)
+
+
+def _quantise_rows_i8(src):
+    """per-row codes and scales as the append kernel makes them (neural/neural.cl:2501-2580)"""
+    m = np.max(np.abs(src), axis=1); sc = np.where(m > 0, m / 127.0, 1.0).astype(np.float32)
+    return np.clip(np.rint(src / sc[:, None]), -127, 127).astype(np.int8), np.where(m > 0, sc, 0.0).astype(np.float32)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_grouped_matrix_core_attention_random_geometry(seed):
+    """The one-work-group-per-KV-head kernel on the matrix cores (fp16 and int8 caches of 128-wide heads) over random geometries:
+    8 / 16 / 32 KV heads, 1..8 query heads per KV head, caches of 1024..12000 rows filled to a random length from the host (so the
+    live range ends anywhere inside a slice, in any of its 16-row tiles), window, soft cap; a few tokens decoded on top against the
+    oracle's kernel over the same rows."""
+    from helpers.device import dev
+    cai = dev()
+    rng = np.random.default_rng(5000 + seed)
+    dk = 128
+    hkv = int(rng.choice([8, 16, 32])); G = int(rng.choice([1, 2, 3, 4, 5, 6, 7, 8])); hq = hkv * G
+    need = (256 + hkv - 1) // hkv                       # slices for a grid that takes this kernel
+    ctx = int(rng.choice([c for c in (1024, 2048, 4096, 8192, 8448, 12000) if (c + 255) // 256 >= need or (c <= 4096 and 16 >= need)]))
+    kvt = "i8" if seed % 2 else "f16"
+    n0, steps = int(rng.integers(0, ctx - 30)), int(rng.integers(2, 6))
+    window, softcap = int(rng.choice([0, 0, 70, 300])), float(rng.choice([0.0, 0.0, 25.0]))
+    k = rng.standard_normal((hkv, n0, dk)).astype(np.float32); v = rng.standard_normal((hkv, n0, dk)).astype(np.float32)
+    rows = rng.standard_normal((steps, (hq + 2 * hkv) * dk)).astype(np.float32)
+    kv = cai.KVCache(1, hkv, dk, ctx, cai.KV_I8 if kvt == "i8" else cai.KV_F16)
+    what = (hq, hkv, ctx, kvt, n0, window, softcap)
+    if kvt == "i8":
+        kq = np.zeros((hkv, ctx, dk), np.int8); vq = np.zeros_like(kq); ks = np.zeros((hkv, ctx), np.float32); vs = np.zeros_like(ks)
+        for g in range(hkv):
+            if n0:
+                kq[g, :n0], ks[g, :n0] = _quantise_rows_i8(k[g]); vq[g, :n0], vs[g, :n0] = _quantise_rows_i8(v[g])
+        if n0:
+            kv.import_layer(0, kq[:, :n0], vq[:, :n0], ks[:, :n0], vs[:, :n0])
+    else:
+        k = k.astype(np.float16).astype(np.float32); v = v.astype(np.float16).astype(np.float32)
+        kc = np.zeros((hkv, ctx, dk), np.float32); vc = np.zeros_like(kc); kc[:, :n0] = k; vc[:, :n0] = v
+        if n0:
+            kv.import_layer(0, k.astype(np.float16), v.astype(np.float16))
+    for i in range(steps):
+        out = np.zeros(hq * dk, np.float32)
+        if kvt == "i8":
+            O.lib().orc_attn_decode_i8(rows[i].ctypes.data, hq, hkv, dk, kq.ctypes.data, ks.ctypes.data, vq.ctypes.data, vs.ctypes.data,
+                                       ctx, n0 + i, window, softcap, out.ctypes.data)
+        else:
+            O.lib().orc_attn_decode(rows[i].ctypes.data, hq, hkv, dk, kc.ctypes.data, vc.ctypes.data, ctx, n0 + i, window, softcap, 1, out.ctypes.data)
+        got = kv.attn_decode(0, rows[i], hq, window, softcap)
+        assert np.max(np.abs(got - out)) < 2e-5 * max(1.0, np.max(np.abs(out))), (i,) + what
+
+
+@pytest.mark.parametrize("hkv,G,sinks,recent", [(16, 2, 3, 130), (32, 1, 0, 300), (16, 3, 17, 40)])
+def test_grouped_matrix_core_attention_rolling_eviction(hkv, G, sinks, recent):
+    """Sink + recent-window eviction on a half-precision cache through the same kernel: the appended row's slot lies in the middle of the
+    ring, every cached row stays live."""
+    from helpers.device import dev
+    cai = dev()
+    rng = np.random.default_rng(hkv + sinks)
+    dk, ctx, hq = 128, 1024, hkv * G
+    n = sinks + recent + 40
+    rows = rng.standard_normal((n, (hq + 2 * hkv) * dk)).astype(np.float32)
+    want = oracle_run_evict(rows, hq, hkv, dk, sinks, recent, 1)
+    kv = cai.KVCache(1, hkv, dk, ctx, cai.KV_F16); kv.set_eviction(sinks, recent)
+    for pos in range(n):
+        got = kv.attn_decode(0, rows[pos], hq)
+        assert np.max(np.abs(got - want[pos])) < 2e-5 * max(1.0, np.max(np.abs(want[pos]))), pos
+
