@@ -865,6 +865,7 @@ __global__ __launch_bounds__(64 * NW) void attn_group_mfma_kernel(const int32_t*
 // ---- merge of the split partials: one work-group per query head.  Four quarter-groups of head_dim threads each take every
 //      fourth slice (all their loads go out together: one round trip for up to 32 slices per quarter), fold them with a running
 //      maximum, and meet in LDS. ----
+template <int MR>      // slices per quarter and round trip: 12, or 32 for long caches (130k rows = 508 slices: 4 dependent rounds instead of 11)
 __global__ __launch_bounds__(512) void attn_merge_kernel(const int32_t* hpos, const float* hpart, float* hout, const long long hout_stride,
                                                          const int hheads, const int hgeo, const int hsl, const AttnParams p)
 {
@@ -873,8 +874,7 @@ __global__ __launch_bounds__(512) void attn_merge_kernel(const int32_t* hpos, co
   const int hd = h_hd;
   __shared__ float qA[4][128], qM[4], qL[4];
   const int quarter = threadIdx.x >> 7, d = threadIdx.x & 127;
-  constexpr int MR = 12;                           // slices per quarter and round trip
-  // Without a sliding window the first live slice is slice 0 whatever the position: the first round of partials (48 slices) is
+  // Without a sliding window the first live slice is slice 0 whatever the position: the first round of partials (4 MR slices) is
   // requested before the position has arrived and masked by the slice count afterwards (a partial past the live range is
   // whatever an earlier step left there: it is selected away, never used in arithmetic).
   const bool ahead = p.window <= 0 && d < hd;
@@ -1733,8 +1733,14 @@ int launch_attn_step(cai_kv_s* kv, int layer, float* qkv, int64_t qkv_stride, in
     rc = kv->dtype == CAI_KV_I8 ? launch_split_head<int8_t>(p, n_seq, c.stream) : kv->dtype == CAI_KV_F16 ? launch_split_head<__half>(p, n_seq, c.stream) : launch_split_head<float>(p, n_seq, c.stream);
   if (rc) return rc;
   if (p.n_splits > 1 && !p.merge_cnt)
-    hipLaunchKernelGGL(attn_merge_kernel, dim3(q_heads, n_seq), dim3(512), 0, c.stream, p.pos, (const float*)p.part, p.out, (long long)p.out_stride,
-                       p.q_heads | p.kv_heads << 16, p.n_splits | p.hd << 16, p.split_len, p);
+  {
+    if (p.n_splits > 96)
+      hipLaunchKernelGGL(attn_merge_kernel<32>, dim3(q_heads, n_seq), dim3(512), 0, c.stream, p.pos, (const float*)p.part, p.out, (long long)p.out_stride,
+                         p.q_heads | p.kv_heads << 16, p.n_splits | p.hd << 16, p.split_len, p);
+    else
+      hipLaunchKernelGGL(attn_merge_kernel<12>, dim3(q_heads, n_seq), dim3(512), 0, c.stream, p.pos, (const float*)p.part, p.out, (long long)p.out_stride,
+                         p.q_heads | p.kv_heads << 16, p.n_splits | p.hd << 16, p.split_len, p);
+  }
   return CAI_OK;
 }
 
