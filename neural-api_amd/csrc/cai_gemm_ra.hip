@@ -207,18 +207,17 @@ __global__ __launch_bounds__(64 * RA_NW) void gemm_q4k_ra(const float* hsrc, con
       const float s = on ? ldexpf(1.0f, e) : 0.0f;      // (an absent token's columns: zeros)
 #pragma unroll
       for (int m = 0; m < 4; m++) {
-        _Float16 h[4], l[4];
-        float sm = 0.0f;
+        // vs = h + l to 21 bits, both parts converted two at a time towards zero (v_cvt_pkrtz_f16_f32: the pair comes out packed, and
+        // in the operand's order - inside a group of 8 that order is 0, 2, 1, 3, 4, 6, 5, 7 (ra_weights): the middle two of every four
+        // swap); l = vs - h is exact in fp32 and has the sign of vs
+        float vs[4], sm = 0.0f;
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-          const float vs = v[m][u] * s;
-          h[u] = (_Float16)vs; l[u] = (_Float16)(vs - (float)h[u]);      // vs = h + l to 22 bits
-          sm += vs;
-        }
-        // inside a group of 8 the operand order is 0, 2, 1, 3, 4, 6, 5, 7 (ra_weights): the middle two of every four swap
-        typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-        *reinterpret_cast<half4_t*>(xw + t8 * RA_XLD + j * 256 + 64 * m + 4 * ii) = half4_t{h[0], h[2], h[1], h[3]};
-        *reinterpret_cast<half4_t*>(xw + (8 + t8) * RA_XLD + j * 256 + 64 * m + 4 * ii) = half4_t{l[0], l[2], l[1], l[3]};
+        for (int u = 0; u < 4; u++) { vs[u] = v[m][u] * s; sm += vs[u]; }
+        typedef __fp16 pk2_t __attribute__((ext_vector_type(2)));
+        const pk2_t h02 = __builtin_amdgcn_cvt_pkrtz(vs[0], vs[2]), h13 = __builtin_amdgcn_cvt_pkrtz(vs[1], vs[3]);
+        const pk2_t l02 = __builtin_amdgcn_cvt_pkrtz(vs[0] - (float)h02.x, vs[2] - (float)h02.y), l13 = __builtin_amdgcn_cvt_pkrtz(vs[1] - (float)h13.x, vs[3] - (float)h13.y);
+        *reinterpret_cast<uint2*>(xw + t8 * RA_XLD + j * 256 + 64 * m + 4 * ii) = make_uint2(__builtin_bit_cast(uint32_t, h02), __builtin_bit_cast(uint32_t, h13));
+        *reinterpret_cast<uint2*>(xw + (8 + t8) * RA_XLD + j * 256 + 64 * m + 4 * ii) = make_uint2(__builtin_bit_cast(uint32_t, l02), __builtin_bit_cast(uint32_t, l13));
         // sub-block 2 m + i / 8 of the block: the sum of 8 lanes' values, / 32, hi + lo
         sm = ra_oct_sum(sm) * 0.03125f;
         const _Float16 qh = (_Float16)sm, ql = (_Float16)(sm - (float)qh);
